@@ -1,0 +1,66 @@
+"""Loads libclblast_hip.so (the C-ABI drop-in library) and declares its entry points for ctypes.
+
+The library is built in-tree by ``make -C clblast_amd/csrc`` (or ``__graft_entry__.build()``). There
+is no CPU fallback: if the shared object is missing, importing this module's ``load()`` raises.
+"""
+import ctypes
+import os
+from ctypes import c_char_p, c_double, c_float, c_int, c_size_t, c_ushort, c_void_p, POINTER
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libclblast_hip.so")
+CSRC_DIR = os.path.join(_HERE, "csrc")
+
+_lib = None
+
+_SCALAR = {"S": c_float, "D": c_double, "H": c_ushort}
+
+
+def _declare(lib):
+    sz, vp = c_size_t, c_void_p
+    for prefix, scalar in _SCALAR.items():
+        gemm_args = [c_int, c_int, c_int, sz, sz, sz, scalar, vp, sz, sz, vp, sz, sz, scalar, vp, sz, sz, vp, vp]
+        f = getattr(lib, "CLBlast%sgemm" % prefix)
+        f.argtypes, f.restype = gemm_args, c_int
+        f = getattr(lib, "CLBlast%sgemmWithTempBuffer" % prefix)
+        f.argtypes, f.restype = gemm_args + [vp], c_int
+        f = getattr(lib, "CLBlast%sgemmBatched" % prefix)
+        f.argtypes = [c_int, c_int, c_int, sz, sz, sz, POINTER(scalar), vp, POINTER(sz), sz, vp, POINTER(sz), sz,
+                      POINTER(scalar), vp, POINTER(sz), sz, sz, vp, vp]
+        f.restype = c_int
+        f = getattr(lib, "CLBlast%sgemmStridedBatched" % prefix)
+        f.argtypes = [c_int, c_int, c_int, sz, sz, sz, scalar, vp, sz, sz, sz, vp, sz, sz, sz, scalar, vp, sz, sz, sz,
+                      sz, vp, vp]
+        f.restype = c_int
+        f = getattr(lib, "CLBlast%sGemmTempBufferSize" % prefix)
+        f.argtypes = [c_int, c_int, c_int, sz, sz, sz, sz, sz, sz, sz, sz, sz, vp, POINTER(sz)]
+        f.restype = c_int
+    lib.CLBlastClearCache.argtypes, lib.CLBlastClearCache.restype = [], c_int
+    lib.CLBlastOverrideParameters.argtypes = [c_int, c_char_p, c_int, sz, POINTER(c_char_p), POINTER(sz)]
+    lib.CLBlastOverrideParameters.restype = c_int
+    lib.CLBlastFloatToHalf.argtypes, lib.CLBlastFloatToHalf.restype = [c_float], c_ushort
+    lib.CLBlastHalfToFloat.argtypes, lib.CLBlastHalfToFloat.restype = [c_ushort], c_float
+
+
+def load():
+    """Returns the ctypes handle of libclblast_hip.so, loading it on first use."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                "%s is missing: build it with `make -C %s` (needs hipcc); there is no fallback path" %
+                (LIB_PATH, CSRC_DIR))
+        lib = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+        _declare(lib)
+        _lib = lib
+    return _lib
+
+
+# Every symbol the public C headers declare, for the export test.
+C_API_SYMBOLS = (
+    ["CLBlast%sgemm%s" % (p, s) for p in "SDH" for s in ("", "Batched", "StridedBatched", "WithTempBuffer")] +
+    ["CLBlast%sGemmTempBufferSize" % p for p in "SDH"] +
+    ["CLBlastClearCache", "CLBlastOverrideParameters", "CLBlastFloatToHalf", "CLBlastHalfToFloat"])
+DEVICE_LAYER_SYMBOLS = [
+    "clbh_gemm_launch", "clbh_gemm_workspace_bytes", "clbh_buffer_extent", "clbh_alloc_async", "clbh_free_async",
+    "clbh_upload_async", "clbh_event_record", "clbh_stream_device", "clbh_error_string"]

@@ -1,0 +1,181 @@
+"""Python host-side mirror of the reference's Python binding for the GEMM family.
+
+``gemm``, ``gemmBatched`` and ``gemmStridedBatched`` keep the argument names, order and defaults of
+pyclblast (reference: src/pyclblast/src/pyclblast.pyx:1891-1915 gemm, :2360 gemmBatched, :2452
+gemmStridedBatched): row-major layout, element offsets, leading dimensions, booleans for the
+transposes. Where pyclblast takes a PyOpenCL queue and ``pyopencl.array.Array`` operands, these take a
+``torch.cuda.Stream`` (or None for the current stream) and CUDA/HIP torch tensors; only the device
+pointer and the dtype of a tensor are used, its shape is not interpreted. Errors raise
+``CLBlastError`` carrying the status code, like pyclblast's RuntimeError with the status name.
+
+``raw_*`` functions are the thin ctypes calls on plain integers (device pointers, stream handle);
+everything in the package goes through them and therefore through the C ABI.
+"""
+import ctypes
+
+from . import _lib
+
+ROW_MAJOR, COL_MAJOR = 101, 102
+TRANS_NO, TRANS_YES, TRANS_CONJ = 111, 112, 113
+
+STATUS_NAMES = {
+    0: "kSuccess", -4: "kTempBufferAllocFailure", -30: "kInvalidValue", -36: "kInvalidCommandQueue",
+    -1024: "kNotImplemented", -1022: "kInvalidMatrixA", -1021: "kInvalidMatrixB", -1020: "kInvalidMatrixC",
+    -1017: "kInvalidDimension", -1016: "kInvalidLeadDimA", -1015: "kInvalidLeadDimB", -1014: "kInvalidLeadDimC",
+    -1011: "kInsufficientMemoryA", -1010: "kInsufficientMemoryB", -1009: "kInsufficientMemoryC",
+    -2050: "kInsufficientMemoryTemp", -2049: "kInvalidBatchCount", -2048: "kInvalidOverrideKernel",
+    -2047: "kMissingOverrideParameter", -2045: "kNoHalfPrecision", -2044: "kNoDoublePrecision",
+    -2040: "kUnknownError", -2039: "kUnexpectedError",
+}
+
+
+class CLBlastError(RuntimeError):
+    def __init__(self, routine, status):
+        self.status = status
+        RuntimeError.__init__(self, "PyCLBlast: '%s' failed: %s (%d)" %
+                              (routine, STATUS_NAMES.get(status, "status"), status))
+
+
+def float_to_half_bits(value):
+    """fp32 -> binary16 bit pattern with the reference's truncating conversion."""
+    return int(_lib.load().CLBlastFloatToHalf(ctypes.c_float(value)))
+
+
+def half_bits_to_float(bits):
+    return float(_lib.load().CLBlastHalfToFloat(ctypes.c_ushort(bits)))
+
+
+def _prefix_of(dtype_name):
+    try:
+        return {"float32": "S", "float64": "D", "float16": "H"}[dtype_name]
+    except KeyError:
+        raise ValueError("PyCLBlast: unrecognized data-type '%s'" % dtype_name)
+
+
+def _scalar(prefix, value):
+    return float_to_half_bits(value) if prefix == "H" else value
+
+
+def _stream_ref(stream_handle):
+    """The C API takes a pointer to the stream handle (reference: cl_command_queue* queue)."""
+    return ctypes.byref(ctypes.c_void_p(stream_handle))
+
+
+# ---- raw calls on integers ---------------------------------------------------------------------------
+
+def raw_gemm(prefix, layout, a_transpose, b_transpose, m, n, k, alpha, a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld,
+             beta, c_ptr, c_offset, c_ld, stream_handle=0, event_handle=None, temp_ptr=None):
+    lib = _lib.load()
+    event_ref = None if event_handle is None else ctypes.byref(ctypes.c_void_p(event_handle))
+    args = [layout, a_transpose, b_transpose, m, n, k, _scalar(prefix, alpha), a_ptr, a_offset, a_ld, b_ptr, b_offset,
+            b_ld, _scalar(prefix, beta), c_ptr, c_offset, c_ld, _stream_ref(stream_handle), event_ref]
+    if temp_ptr is None:
+        return getattr(lib, "CLBlast%sgemm" % prefix)(*args)
+    return getattr(lib, "CLBlast%sgemmWithTempBuffer" % prefix)(*(args + [temp_ptr]))
+
+
+def raw_gemm_batched(prefix, layout, a_transpose, b_transpose, m, n, k, alphas, a_ptr, a_offsets, a_ld, b_ptr,
+                     b_offsets, b_ld, betas, c_ptr, c_offsets, c_ld, batch_count, stream_handle=0):
+    lib = _lib.load()
+    scalar_t = _lib._SCALAR[prefix]
+    count = len(alphas)
+    mk_s = lambda xs: (scalar_t * max(len(xs), 1))(*[_scalar(prefix, x) for x in xs])
+    mk_z = lambda xs: (ctypes.c_size_t * max(len(xs), 1))(*xs)
+    assert len(betas) == count and len(a_offsets) == count and len(b_offsets) == count and len(c_offsets) == count
+    return getattr(lib, "CLBlast%sgemmBatched" % prefix)(
+        layout, a_transpose, b_transpose, m, n, k, mk_s(alphas), a_ptr, mk_z(a_offsets), a_ld, b_ptr,
+        mk_z(b_offsets), b_ld, mk_s(betas), c_ptr, mk_z(c_offsets), c_ld, batch_count, _stream_ref(stream_handle),
+        None)
+
+
+def raw_gemm_strided_batched(prefix, layout, a_transpose, b_transpose, m, n, k, alpha, a_ptr, a_offset, a_ld,
+                             a_stride, b_ptr, b_offset, b_ld, b_stride, beta, c_ptr, c_offset, c_ld, c_stride,
+                             batch_count, stream_handle=0):
+    lib = _lib.load()
+    return getattr(lib, "CLBlast%sgemmStridedBatched" % prefix)(
+        layout, a_transpose, b_transpose, m, n, k, _scalar(prefix, alpha), a_ptr, a_offset, a_ld, a_stride, b_ptr,
+        b_offset, b_ld, b_stride, _scalar(prefix, beta), c_ptr, c_offset, c_ld, c_stride, batch_count,
+        _stream_ref(stream_handle), None)
+
+
+def raw_gemm_temp_buffer_size(prefix, layout, a_transpose, b_transpose, m, n, k, a_offset, a_ld, b_offset, b_ld,
+                              c_offset, c_ld, stream_handle=0):
+    lib = _lib.load()
+    size = ctypes.c_size_t(0)
+    status = getattr(lib, "CLBlast%sGemmTempBufferSize" % prefix)(
+        layout, a_transpose, b_transpose, m, n, k, a_offset, a_ld, b_offset, b_ld, c_offset, c_ld,
+        _stream_ref(stream_handle), ctypes.byref(size))
+    return status, size.value
+
+
+def override_parameters(device, kernel_name, precision_bits, parameters):
+    """Reference: pyclblast.override_parameters (src/pyclblast/src/pyclblast.pyx:2555-2594)."""
+    lib = _lib.load()
+    names = [key.encode() for key in parameters]
+    values = [parameters[key] for key in parameters]
+    status = lib.CLBlastOverrideParameters(
+        device, kernel_name.encode(), precision_bits, len(names), (ctypes.c_char_p * max(len(names), 1))(*names),
+        (ctypes.c_size_t * max(len(values), 1))(*values))
+    if status != 0:
+        raise CLBlastError("CLBlastOverrideParameters", status)
+
+
+def clear_cache():
+    return _lib.load().CLBlastClearCache()
+
+
+# ---- pyclblast-shaped calls on torch tensors ---------------------------------------------------------
+
+def _tensor_info(*tensors):
+    names = {str(t.dtype).replace("torch.", "") for t in tensors}
+    if len(names) != 1:
+        raise ValueError("PyCLBlast: All arrays have to be of the same data-type, got: %s" % ", ".join(sorted(names)))
+    for t in tensors:
+        if not t.is_cuda:
+            raise ValueError("PyCLBlast: operands must live on the GPU")
+    return _prefix_of(names.pop())
+
+
+def _stream_handle(queue):
+    import torch
+    stream = torch.cuda.current_stream() if queue is None else queue
+    return stream.cuda_stream
+
+
+def gemm(queue, m, n, k, a, b, c, a_ld, b_ld, c_ld, alpha=1.0, beta=0.0, a_transp=False, b_transp=False, a_offset=0,
+         b_offset=0, c_offset=0):
+    """xGEMM: General matrix-matrix multiplication (row-major, like pyclblast.gemm)."""
+    prefix = _tensor_info(a, b, c)
+    status = raw_gemm(prefix, ROW_MAJOR, TRANS_YES if a_transp else TRANS_NO, TRANS_YES if b_transp else TRANS_NO, m,
+                      n, k, alpha, a.data_ptr(), a_offset, a_ld, b.data_ptr(), b_offset, b_ld, beta, c.data_ptr(),
+                      c_offset, c_ld, _stream_handle(queue))
+    if status != 0:
+        raise CLBlastError("CLBlast%sgemm" % prefix, status)
+
+
+def gemmBatched(queue, m, n, k, a, b, c, alphas, betas, a_ld, b_ld, c_ld, a_offsets, b_offsets, c_offsets,
+                a_transp=False, b_transp=False):
+    """xGEMMBATCHED: Batched version of GEMM (row-major, like pyclblast.gemmBatched)."""
+    prefix = _tensor_info(a, b, c)
+    batch_count = len(a_offsets)
+    if not (len(b_offsets) == len(c_offsets) == len(alphas) == len(betas) == batch_count):
+        raise RuntimeError("PyCLBlast: 'CLBlastXgemmBatched' failed: length of batch-sized arguments a_offsets, "
+                           "b_offsets, c_offsets, alphas, betas should be equal")
+    status = raw_gemm_batched(prefix, ROW_MAJOR, TRANS_YES if a_transp else TRANS_NO,
+                              TRANS_YES if b_transp else TRANS_NO, m, n, k, list(alphas), a.data_ptr(),
+                              list(a_offsets), a_ld, b.data_ptr(), list(b_offsets), b_ld, list(betas), c.data_ptr(),
+                              list(c_offsets), c_ld, batch_count, _stream_handle(queue))
+    if status != 0:
+        raise CLBlastError("CLBlast%sgemmBatched" % prefix, status)
+
+
+def gemmStridedBatched(queue, m, n, k, batch_count, a, b, c, a_ld, b_ld, c_ld, a_stride, b_stride, c_stride,
+                       alpha=1.0, beta=0.0, a_transp=False, b_transp=False, a_offset=0, b_offset=0, c_offset=0):
+    """xGEMMSTRIDEDBATCHED: StridedBatched version of GEMM (row-major, like pyclblast.gemmStridedBatched)."""
+    prefix = _tensor_info(a, b, c)
+    status = raw_gemm_strided_batched(prefix, ROW_MAJOR, TRANS_YES if a_transp else TRANS_NO,
+                                      TRANS_YES if b_transp else TRANS_NO, m, n, k, alpha, a.data_ptr(), a_offset,
+                                      a_ld, a_stride, b.data_ptr(), b_offset, b_ld, b_stride, beta, c.data_ptr(),
+                                      c_offset, c_ld, c_stride, batch_count, _stream_handle(queue))
+    if status != 0:
+        raise CLBlastError("CLBlast%sgemmStridedBatched" % prefix, status)

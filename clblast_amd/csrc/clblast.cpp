@@ -1,0 +1,150 @@
+// =================================================================================================
+// Bodies of the C++ API (include/clblast_hip.h): build the routine object, run it, and translate every
+// exception into a status code so that nothing is thrown across the library boundary. Mirrors the
+// structure of the reference's src/clblast.cpp:1066-1084 (Gemm), :1573-1601 (GemmBatched),
+// :1630-1647 (GemmStridedBatched), :1682-1708 (GemmTempBufferSize) and src/api_common.cpp:25-33,
+// 140-221 (ClearCache, RetrieveParameters, OverrideParameters).
+// =================================================================================================
+#include <vector>
+
+#include "clblast_hip.h"
+#include "routines/xgemm.hpp"
+#include "routines/xgemmbatched.hpp"
+
+#define CLBLAST_HIP_PUBLIC __attribute__((visibility("default")))
+
+namespace clblast {
+// =================================================================================================
+
+template <typename T>
+StatusCode Gemm(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
+                const size_t n, const size_t k, const T alpha, const void* a_buffer, const size_t a_offset,
+                const size_t a_ld, const void* b_buffer, const size_t b_offset, const size_t b_ld, const T beta,
+                void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event,
+                void* temp_buffer) {
+  try {
+    auto routine = Xgemm<T>(queue, event);
+    const auto temp_buffer_provided = (temp_buffer != nullptr);
+    routine.DoGemm(layout, a_transpose, b_transpose, m, n, k, alpha, Buffer<T>(a_buffer), a_offset, a_ld,
+                   Buffer<T>(b_buffer), b_offset, b_ld, beta, Buffer<T>(c_buffer), c_offset, c_ld,
+                   Buffer<T>(temp_buffer), temp_buffer_provided);
+    return StatusCode::kSuccess;
+  } catch (...) {
+    return DispatchException();
+  }
+}
+
+template <typename T>
+StatusCode GemmBatched(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
+                       const size_t n, const size_t k, const T* alphas, const void* a_buffer, const size_t* a_offsets,
+                       const size_t a_ld, const void* b_buffer, const size_t* b_offsets, const size_t b_ld,
+                       const T* betas, void* c_buffer, const size_t* c_offsets, const size_t c_ld,
+                       const size_t batch_count, hipStream_t* queue, hipEvent_t* event) {
+  try {
+    auto routine = XgemmBatched<T>(queue, event);
+    if (batch_count > 0 && (alphas == nullptr || betas == nullptr || a_offsets == nullptr || b_offsets == nullptr ||
+                            c_offsets == nullptr)) {
+      throw BLASError(StatusCode::kInvalidBatchCount, "null per-batch array");
+    }
+    const auto alphas_cpp = std::vector<T>(alphas, alphas + batch_count);
+    const auto betas_cpp = std::vector<T>(betas, betas + batch_count);
+    const auto a_offsets_cpp = std::vector<size_t>(a_offsets, a_offsets + batch_count);
+    const auto b_offsets_cpp = std::vector<size_t>(b_offsets, b_offsets + batch_count);
+    const auto c_offsets_cpp = std::vector<size_t>(c_offsets, c_offsets + batch_count);
+    routine.DoGemmBatched(layout, a_transpose, b_transpose, m, n, k, alphas_cpp, Buffer<T>(a_buffer), a_offsets_cpp,
+                          a_ld, Buffer<T>(b_buffer), b_offsets_cpp, b_ld, betas_cpp, Buffer<T>(c_buffer),
+                          c_offsets_cpp, c_ld, batch_count);
+    return StatusCode::kSuccess;
+  } catch (...) {
+    return DispatchException();
+  }
+}
+
+template <typename T>
+StatusCode GemmStridedBatched(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
+                              const size_t m, const size_t n, const size_t k, const T alpha, const void* a_buffer,
+                              const size_t a_offset, const size_t a_ld, const size_t a_stride, const void* b_buffer,
+                              const size_t b_offset, const size_t b_ld, const size_t b_stride, const T beta,
+                              void* c_buffer, const size_t c_offset, const size_t c_ld, const size_t c_stride,
+                              const size_t batch_count, hipStream_t* queue, hipEvent_t* event) {
+  try {
+    auto routine = XgemmStridedBatched<T>(queue, event);
+    routine.DoGemmStridedBatched(layout, a_transpose, b_transpose, m, n, k, alpha, Buffer<T>(a_buffer), a_offset,
+                                 a_ld, a_stride, Buffer<T>(b_buffer), b_offset, b_ld, b_stride, beta,
+                                 Buffer<T>(c_buffer), c_offset, c_ld, c_stride, batch_count);
+    return StatusCode::kSuccess;
+  } catch (...) {
+    return DispatchException();
+  }
+}
+
+template <typename T>
+StatusCode GemmTempBufferSize(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
+                              const size_t m, const size_t n, const size_t k, const size_t a_offset, const size_t a_ld,
+                              const size_t b_offset, const size_t b_ld, const size_t c_offset, const size_t c_ld,
+                              hipStream_t* queue, size_t& temp_buffer_size) {
+  try {
+    (void)a_offset; (void)a_ld; (void)b_offset; (void)b_ld; (void)c_offset; (void)c_ld;  // operands are read in place
+    if (queue == nullptr) {
+      throw RuntimeErrorCode(StatusCode::kInvalidCommandQueue, "queue is a null pointer");
+    }
+    auto device = 0;
+    CheckDevice(clbh_stream_device(*queue, &device), "clbh_stream_device");
+    temp_buffer_size = Xgemm<T>::TempBytes(layout, a_transpose, b_transpose, m, n, k,
+                                           MinIndirectSize(device, PrecisionValue<T>()));
+    return StatusCode::kSuccess;
+  } catch (...) {
+    return DispatchException();
+  }
+}
+
+#define CLBLAST_HIP_INSTANTIATE(T)                                                                                  \
+  template StatusCode CLBLAST_HIP_PUBLIC Gemm<T>(const Layout, const Transpose, const Transpose, const size_t,      \
+                                                 const size_t, const size_t, const T, const void*, const size_t,    \
+                                                 const size_t, const void*, const size_t, const size_t, const T,    \
+                                                 void*, const size_t, const size_t, hipStream_t*, hipEvent_t*,      \
+                                                 void*);                                                            \
+  template StatusCode CLBLAST_HIP_PUBLIC GemmBatched<T>(                                                            \
+      const Layout, const Transpose, const Transpose, const size_t, const size_t, const size_t, const T*,           \
+      const void*, const size_t*, const size_t, const void*, const size_t*, const size_t, const T*, void*,          \
+      const size_t*, const size_t, const size_t, hipStream_t*, hipEvent_t*);                                        \
+  template StatusCode CLBLAST_HIP_PUBLIC GemmStridedBatched<T>(                                                     \
+      const Layout, const Transpose, const Transpose, const size_t, const size_t, const size_t, const T,            \
+      const void*, const size_t, const size_t, const size_t, const void*, const size_t, const size_t, const size_t, \
+      const T, void*, const size_t, const size_t, const size_t, const size_t, hipStream_t*, hipEvent_t*);           \
+  template StatusCode CLBLAST_HIP_PUBLIC GemmTempBufferSize<T>(                                                     \
+      const Layout, const Transpose, const Transpose, const size_t, const size_t, const size_t, const size_t,       \
+      const size_t, const size_t, const size_t, const size_t, const size_t, hipStream_t*, size_t&);
+CLBLAST_HIP_INSTANTIATE(half)
+CLBLAST_HIP_INSTANTIATE(float)
+CLBLAST_HIP_INSTANTIATE(double)
+#undef CLBLAST_HIP_INSTANTIATE
+
+// =================================================================================================
+
+// Kernels are compiled ahead of time: there is no program or binary cache to drop. Parameter
+// overrides survive, as they do in the reference (api_common.cpp:25-33 leaves the database cache alone).
+CLBLAST_HIP_PUBLIC StatusCode ClearCache() { return StatusCode::kSuccess; }
+
+CLBLAST_HIP_PUBLIC StatusCode OverrideParameters(const int device, const std::string& kernel_name,
+                                                 const Precision precision,
+                                                 const std::unordered_map<std::string, size_t>& parameters) {
+  try {
+    return OverrideRoutineParameters(device, kernel_name, precision, parameters);
+  } catch (...) {
+    return DispatchException();
+  }
+}
+
+CLBLAST_HIP_PUBLIC StatusCode RetrieveParameters(const int device, const std::string& kernel_name,
+                                                 const Precision precision,
+                                                 std::unordered_map<std::string, size_t>& parameters) {
+  try {
+    return RetrieveRoutineParameters(device, kernel_name, precision, parameters);
+  } catch (...) {
+    return DispatchException();
+  }
+}
+
+// =================================================================================================
+}  // namespace clblast

@@ -1,0 +1,261 @@
+// =================================================================================================
+// extern "C" wrappers (include/clblast_hip_c.h) over the C++ API: cast the enums, forward, and turn any
+// exception that still escapes into kUnexpectedError. Mirrors the reference's src/clblast_c.cpp
+// (GEMM family: :1800-1874, :2723-3084; cache and override functions: :3089-3127).
+// =================================================================================================
+#include "clblast_hip_c.h"
+
+#include <string>
+#include <unordered_map>
+
+#include "clblast_half.h"
+#include "clblast_hip.h"
+#include "routines/routine_common.hpp"
+
+namespace {
+inline clblast::Layout L(const CLBlastLayout v) { return static_cast<clblast::Layout>(v); }
+inline clblast::Transpose Tr(const CLBlastTranspose v) { return static_cast<clblast::Transpose>(v); }
+template <typename F>
+CLBlastStatusCode Guarded(F&& body) {
+  try {
+    return static_cast<CLBlastStatusCode>(body());
+  } catch (...) {
+    return static_cast<CLBlastStatusCode>(clblast::DispatchExceptionForC());
+  }
+}
+}  // namespace
+
+extern "C" {
+
+// ---- SGEMM family ------------------------------------------------------------------------------
+CLBlastStatusCode CLBlastSgemm(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                               const CLBlastTranspose b_transpose, const size_t m, const size_t n, const size_t k,
+                               const float alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+                               const void* b_buffer, const size_t b_offset, const size_t b_ld, const float beta,
+                               void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                               hipEvent_t* event) {
+  return Guarded([&]() {
+    return clblast::Gemm<float>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, alpha, a_buffer, a_offset, a_ld,
+                              b_buffer, b_offset, b_ld, beta, c_buffer, c_offset, c_ld, queue, event, nullptr);
+  });
+}
+
+CLBlastStatusCode CLBlastSgemmWithTempBuffer(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                             const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                             const size_t k, const float alpha, const void* a_buffer,
+                                             const size_t a_offset, const size_t a_ld, const void* b_buffer,
+                                             const size_t b_offset, const size_t b_ld, const float beta,
+                                             void* c_buffer, const size_t c_offset, const size_t c_ld,
+                                             hipStream_t* queue, hipEvent_t* event, void* temp_buffer) {
+  return Guarded([&]() {
+    return clblast::Gemm<float>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, alpha, a_buffer, a_offset, a_ld,
+                              b_buffer, b_offset, b_ld, beta, c_buffer, c_offset, c_ld, queue, event, temp_buffer);
+  });
+}
+
+CLBlastStatusCode CLBlastSgemmBatched(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                      const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                      const size_t k, const float* alphas, const void* a_buffer,
+                                      const size_t* a_offsets, const size_t a_ld, const void* b_buffer,
+                                      const size_t* b_offsets, const size_t b_ld, const float* betas, void* c_buffer,
+                                      const size_t* c_offsets, const size_t c_ld, const size_t batch_count,
+                                      hipStream_t* queue, hipEvent_t* event) {
+  return Guarded([&]() {
+    return clblast::GemmBatched<float>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, alphas, a_buffer,
+                                     a_offsets, a_ld, b_buffer, b_offsets, b_ld, betas, c_buffer, c_offsets, c_ld,
+                                     batch_count, queue, event);
+  });
+}
+
+CLBlastStatusCode CLBlastSgemmStridedBatched(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                             const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                             const size_t k, const float alpha, const void* a_buffer,
+                                             const size_t a_offset, const size_t a_ld, const size_t a_stride,
+                                             const void* b_buffer, const size_t b_offset, const size_t b_ld,
+                                             const size_t b_stride, const float beta, void* c_buffer,
+                                             const size_t c_offset, const size_t c_ld, const size_t c_stride,
+                                             const size_t batch_count, hipStream_t* queue, hipEvent_t* event) {
+  return Guarded([&]() {
+    return clblast::GemmStridedBatched<float>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, alpha, a_buffer,
+                                            a_offset, a_ld, a_stride, b_buffer, b_offset, b_ld, b_stride, beta,
+                                            c_buffer, c_offset, c_ld, c_stride, batch_count, queue, event);
+  });
+}
+
+CLBlastStatusCode CLBlastSGemmTempBufferSize(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                             const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                             const size_t k, const size_t a_offset, const size_t a_ld,
+                                             const size_t b_offset, const size_t b_ld, const size_t c_offset,
+                                             const size_t c_ld, hipStream_t* queue, size_t* temp_buffer_size) {
+  return Guarded([&]() {
+    if (temp_buffer_size == nullptr) {
+      return clblast::StatusCode::kInvalidValue;
+    }
+    return clblast::GemmTempBufferSize<float>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, a_offset, a_ld,
+                                            b_offset, b_ld, c_offset, c_ld, queue, *temp_buffer_size);
+  });
+}
+
+// ---- DGEMM family ------------------------------------------------------------------------------
+CLBlastStatusCode CLBlastDgemm(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                               const CLBlastTranspose b_transpose, const size_t m, const size_t n, const size_t k,
+                               const double alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+                               const void* b_buffer, const size_t b_offset, const size_t b_ld, const double beta,
+                               void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                               hipEvent_t* event) {
+  return Guarded([&]() {
+    return clblast::Gemm<double>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, alpha, a_buffer, a_offset, a_ld,
+                              b_buffer, b_offset, b_ld, beta, c_buffer, c_offset, c_ld, queue, event, nullptr);
+  });
+}
+
+CLBlastStatusCode CLBlastDgemmWithTempBuffer(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                             const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                             const size_t k, const double alpha, const void* a_buffer,
+                                             const size_t a_offset, const size_t a_ld, const void* b_buffer,
+                                             const size_t b_offset, const size_t b_ld, const double beta,
+                                             void* c_buffer, const size_t c_offset, const size_t c_ld,
+                                             hipStream_t* queue, hipEvent_t* event, void* temp_buffer) {
+  return Guarded([&]() {
+    return clblast::Gemm<double>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, alpha, a_buffer, a_offset, a_ld,
+                              b_buffer, b_offset, b_ld, beta, c_buffer, c_offset, c_ld, queue, event, temp_buffer);
+  });
+}
+
+CLBlastStatusCode CLBlastDgemmBatched(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                      const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                      const size_t k, const double* alphas, const void* a_buffer,
+                                      const size_t* a_offsets, const size_t a_ld, const void* b_buffer,
+                                      const size_t* b_offsets, const size_t b_ld, const double* betas, void* c_buffer,
+                                      const size_t* c_offsets, const size_t c_ld, const size_t batch_count,
+                                      hipStream_t* queue, hipEvent_t* event) {
+  return Guarded([&]() {
+    return clblast::GemmBatched<double>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, alphas, a_buffer,
+                                     a_offsets, a_ld, b_buffer, b_offsets, b_ld, betas, c_buffer, c_offsets, c_ld,
+                                     batch_count, queue, event);
+  });
+}
+
+CLBlastStatusCode CLBlastDgemmStridedBatched(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                             const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                             const size_t k, const double alpha, const void* a_buffer,
+                                             const size_t a_offset, const size_t a_ld, const size_t a_stride,
+                                             const void* b_buffer, const size_t b_offset, const size_t b_ld,
+                                             const size_t b_stride, const double beta, void* c_buffer,
+                                             const size_t c_offset, const size_t c_ld, const size_t c_stride,
+                                             const size_t batch_count, hipStream_t* queue, hipEvent_t* event) {
+  return Guarded([&]() {
+    return clblast::GemmStridedBatched<double>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, alpha, a_buffer,
+                                            a_offset, a_ld, a_stride, b_buffer, b_offset, b_ld, b_stride, beta,
+                                            c_buffer, c_offset, c_ld, c_stride, batch_count, queue, event);
+  });
+}
+
+CLBlastStatusCode CLBlastDGemmTempBufferSize(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                             const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                             const size_t k, const size_t a_offset, const size_t a_ld,
+                                             const size_t b_offset, const size_t b_ld, const size_t c_offset,
+                                             const size_t c_ld, hipStream_t* queue, size_t* temp_buffer_size) {
+  return Guarded([&]() {
+    if (temp_buffer_size == nullptr) {
+      return clblast::StatusCode::kInvalidValue;
+    }
+    return clblast::GemmTempBufferSize<double>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, a_offset, a_ld,
+                                            b_offset, b_ld, c_offset, c_ld, queue, *temp_buffer_size);
+  });
+}
+
+// ---- HGEMM family ------------------------------------------------------------------------------
+CLBlastStatusCode CLBlastHgemm(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                               const CLBlastTranspose b_transpose, const size_t m, const size_t n, const size_t k,
+                               const cl_half alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+                               const void* b_buffer, const size_t b_offset, const size_t b_ld, const cl_half beta,
+                               void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                               hipEvent_t* event) {
+  return Guarded([&]() {
+    return clblast::Gemm<clblast::half>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, alpha, a_buffer, a_offset, a_ld,
+                              b_buffer, b_offset, b_ld, beta, c_buffer, c_offset, c_ld, queue, event, nullptr);
+  });
+}
+
+CLBlastStatusCode CLBlastHgemmWithTempBuffer(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                             const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                             const size_t k, const cl_half alpha, const void* a_buffer,
+                                             const size_t a_offset, const size_t a_ld, const void* b_buffer,
+                                             const size_t b_offset, const size_t b_ld, const cl_half beta,
+                                             void* c_buffer, const size_t c_offset, const size_t c_ld,
+                                             hipStream_t* queue, hipEvent_t* event, void* temp_buffer) {
+  return Guarded([&]() {
+    return clblast::Gemm<clblast::half>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, alpha, a_buffer, a_offset, a_ld,
+                              b_buffer, b_offset, b_ld, beta, c_buffer, c_offset, c_ld, queue, event, temp_buffer);
+  });
+}
+
+CLBlastStatusCode CLBlastHgemmBatched(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                      const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                      const size_t k, const cl_half* alphas, const void* a_buffer,
+                                      const size_t* a_offsets, const size_t a_ld, const void* b_buffer,
+                                      const size_t* b_offsets, const size_t b_ld, const cl_half* betas, void* c_buffer,
+                                      const size_t* c_offsets, const size_t c_ld, const size_t batch_count,
+                                      hipStream_t* queue, hipEvent_t* event) {
+  return Guarded([&]() {
+    return clblast::GemmBatched<clblast::half>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, alphas, a_buffer,
+                                     a_offsets, a_ld, b_buffer, b_offsets, b_ld, betas, c_buffer, c_offsets, c_ld,
+                                     batch_count, queue, event);
+  });
+}
+
+CLBlastStatusCode CLBlastHgemmStridedBatched(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                             const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                             const size_t k, const cl_half alpha, const void* a_buffer,
+                                             const size_t a_offset, const size_t a_ld, const size_t a_stride,
+                                             const void* b_buffer, const size_t b_offset, const size_t b_ld,
+                                             const size_t b_stride, const cl_half beta, void* c_buffer,
+                                             const size_t c_offset, const size_t c_ld, const size_t c_stride,
+                                             const size_t batch_count, hipStream_t* queue, hipEvent_t* event) {
+  return Guarded([&]() {
+    return clblast::GemmStridedBatched<clblast::half>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, alpha, a_buffer,
+                                            a_offset, a_ld, a_stride, b_buffer, b_offset, b_ld, b_stride, beta,
+                                            c_buffer, c_offset, c_ld, c_stride, batch_count, queue, event);
+  });
+}
+
+CLBlastStatusCode CLBlastHGemmTempBufferSize(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                             const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                             const size_t k, const size_t a_offset, const size_t a_ld,
+                                             const size_t b_offset, const size_t b_ld, const size_t c_offset,
+                                             const size_t c_ld, hipStream_t* queue, size_t* temp_buffer_size) {
+  return Guarded([&]() {
+    if (temp_buffer_size == nullptr) {
+      return clblast::StatusCode::kInvalidValue;
+    }
+    return clblast::GemmTempBufferSize<clblast::half>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, a_offset, a_ld,
+                                            b_offset, b_ld, c_offset, c_ld, queue, *temp_buffer_size);
+  });
+}
+
+// ---- cache, overrides, half conversion -----------------------------------------------------------
+CLBlastStatusCode CLBlastClearCache(void) {
+  return Guarded([]() { return clblast::ClearCache(); });
+}
+
+CLBlastStatusCode CLBlastOverrideParameters(const int device, const char* kernel_name,
+                                            const CLBlastPrecision precision, const size_t num_parameters,
+                                            const char** parameters_names, const size_t* parameters_values) {
+  return Guarded([&]() {
+    if (kernel_name == nullptr || (num_parameters > 0 && (parameters_names == nullptr || parameters_values == nullptr))) {
+      return clblast::StatusCode::kInvalidValue;
+    }
+    auto parameters = std::unordered_map<std::string, size_t>();
+    for (auto i = size_t{0}; i < num_parameters; ++i) {
+      parameters[std::string(parameters_names[i])] = parameters_values[i];
+    }
+    return clblast::OverrideParameters(device, std::string(kernel_name), static_cast<clblast::Precision>(precision),
+                                       parameters);
+  });
+}
+
+cl_half CLBlastFloatToHalf(const float value) { return FloatToHalf(value); }
+float CLBlastHalfToFloat(const cl_half value) { return HalfToFloat(value); }
+
+}  // extern "C"

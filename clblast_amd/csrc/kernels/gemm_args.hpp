@@ -1,0 +1,71 @@
+// =================================================================================================
+// Kernel-side view of one canonical GEMM launch (see include/clbh_device.h for the index formulas) and
+// small device helpers shared by all gfx950 GEMM kernels.
+// =================================================================================================
+#ifndef CLBLAST_HIP_KERNELS_GEMM_ARGS_HPP_
+#define CLBLAST_HIP_KERNELS_GEMM_ARGS_HPP_
+
+#include <hip/hip_runtime.h>
+
+namespace clbh {
+
+// Storage type -> type the kernels accumulate and scale in. fp16 accumulates in fp32.
+template <typename T> struct ComputeType { using type = T; };
+template <> struct ComputeType<_Float16> { using type = float; };
+
+template <typename CT>
+struct GemmArgs {
+  const void* a;
+  const void* b;
+  void* c;
+  long long a_offset, b_offset, c_offset;
+  long long a_ld, b_ld, c_ld;
+  long long a_stride, b_stride, c_stride;
+  int m, n, k;
+  int batch_count;
+  CT alpha, beta;
+  const CT* alphas;  // per-batch scalars and offsets, or nullptr
+  const CT* betas;
+  const long long* a_offsets;
+  const long long* b_offsets;
+  const long long* c_offsets;
+};
+
+// Resolves the operand bases and scalars of batch `batch`.
+template <typename T, typename CT>
+__device__ __forceinline__ void ResolveBatch(const GemmArgs<CT>& p, const int batch, const T*& a, const T*& b, T*& c,
+                                             CT& alpha, CT& beta) {
+  long long a_off = p.a_offset, b_off = p.b_offset, c_off = p.c_offset;
+  alpha = p.alpha;
+  beta = p.beta;
+  if (p.alphas != nullptr) {
+    a_off += p.a_offsets[batch];
+    b_off += p.b_offsets[batch];
+    c_off += p.c_offsets[batch];
+    alpha = p.alphas[batch];
+    beta = p.betas[batch];
+  } else {
+    a_off += p.a_stride * batch;
+    b_off += p.b_stride * batch;
+    c_off += p.c_stride * batch;
+  }
+  a = static_cast<const T*>(p.a) + a_off;
+  b = static_cast<const T*>(p.b) + b_off;
+  c = static_cast<T*>(p.c) + c_off;
+}
+
+// Epilogue rule of the reference kernels: with beta == 0 the old C is never read, so NaN/Inf in it do
+// not propagate (reference: src/kernels/level3/xgemm_part2.opencl:84-165,
+// xgemm_direct_part1.opencl:178-187). alpha == 0 is not special-cased.
+template <typename T, typename CT>
+__device__ __forceinline__ void StoreResult(T* c, const long long index, const CT acc, const CT alpha, const CT beta) {
+  if (beta == CT(0)) {
+    c[index] = static_cast<T>(alpha * acc);
+  } else {
+    c[index] = static_cast<T>(alpha * acc + beta * static_cast<CT>(c[index]));
+  }
+}
+
+}  // namespace clbh
+
+#endif  // CLBLAST_HIP_KERNELS_GEMM_ARGS_HPP_

@@ -1,0 +1,111 @@
+// =================================================================================================
+// Error dispatch and matrix validation shared by the GEMM routines (see routine_common.hpp).
+// =================================================================================================
+#include "routines/routine_common.hpp"
+
+#include <cstdio>
+
+namespace clblast {
+// =================================================================================================
+
+StatusCode DispatchException(const bool silent) {
+  const char* message = nullptr;
+  auto status = StatusCode::kUnknownError;
+  try {
+    throw;
+  } catch (const BLASError& e) {
+    status = e.status();  // argument errors stay silent
+  } catch (const RuntimeErrorCode& e) {
+    message = e.what();
+    status = e.status();
+  } catch (const DeviceError& e) {
+    message = e.what();
+    status = StatusCode::kUnknownError;
+  } catch (const std::runtime_error& e) {
+    message = e.what();
+    status = StatusCode::kUnknownError;
+  }
+  // anything else propagates to the caller's catch-all (the C wrappers turn it into kUnexpectedError)
+  if (message != nullptr && !silent) {
+    fprintf(stderr, "CLBlast: %s\n", message);
+  }
+  return status;
+}
+
+StatusCode DispatchExceptionForC() {
+  const char* message = nullptr;
+  try {
+    throw;
+  } catch (const std::exception& e) {
+    message = e.what();
+  } catch (...) {
+    message = "unknown exception";
+  }
+  fprintf(stderr, "CLBlast (unexpected): %s\n", message);
+  return StatusCode::kUnexpectedError;
+}
+
+// =================================================================================================
+
+template <typename T>
+size_t Buffer<T>::GetSize() const {
+  auto bytes = size_t{0};
+  if (pointer_ == nullptr || clbh_buffer_extent(pointer_, &bytes) != 0) {
+    throw std::runtime_error("not a device allocation");
+  }
+  return bytes;
+}
+
+namespace {
+template <typename T>
+void TestMatrix(const size_t one, const size_t two, const Buffer<T>& buffer, const size_t offset, const size_t ld,
+                const bool test_lead_dim, const StatusCode bad_ld, const StatusCode too_small,
+                const StatusCode bad_buffer) {
+  if (test_lead_dim && ld < one) {
+    throw BLASError(bad_ld);
+  }
+  auto available = size_t{0};
+  try {
+    available = buffer.GetSize();
+  } catch (const std::runtime_error& e) {
+    throw BLASError(bad_buffer, e.what());
+  }
+  const auto required_size = (ld * (two - 1) + one + offset) * sizeof(T);
+  if (available < required_size) {
+    throw BLASError(too_small);
+  }
+}
+}  // namespace
+
+template <typename T>
+void TestMatrixA(const size_t one, const size_t two, const Buffer<T>& buffer, const size_t offset, const size_t ld,
+                 const bool test_lead_dim) {
+  TestMatrix(one, two, buffer, offset, ld, test_lead_dim, StatusCode::kInvalidLeadDimA,
+             StatusCode::kInsufficientMemoryA, StatusCode::kInvalidMatrixA);
+}
+template <typename T>
+void TestMatrixB(const size_t one, const size_t two, const Buffer<T>& buffer, const size_t offset, const size_t ld,
+                 const bool test_lead_dim) {
+  TestMatrix(one, two, buffer, offset, ld, test_lead_dim, StatusCode::kInvalidLeadDimB,
+             StatusCode::kInsufficientMemoryB, StatusCode::kInvalidMatrixB);
+}
+template <typename T>
+void TestMatrixC(const size_t one, const size_t two, const Buffer<T>& buffer, const size_t offset, const size_t ld) {
+  TestMatrix(one, two, buffer, offset, ld, true, StatusCode::kInvalidLeadDimC, StatusCode::kInsufficientMemoryC,
+             StatusCode::kInvalidMatrixC);
+}
+
+#define CLBLAST_HIP_INSTANTIATE(T)                                                                            \
+  template class Buffer<T>;                                                                                   \
+  template void TestMatrixA<T>(const size_t, const size_t, const Buffer<T>&, const size_t, const size_t,      \
+                               const bool);                                                                   \
+  template void TestMatrixB<T>(const size_t, const size_t, const Buffer<T>&, const size_t, const size_t,      \
+                               const bool);                                                                   \
+  template void TestMatrixC<T>(const size_t, const size_t, const Buffer<T>&, const size_t, const size_t);
+CLBLAST_HIP_INSTANTIATE(half)
+CLBLAST_HIP_INSTANTIATE(float)
+CLBLAST_HIP_INSTANTIATE(double)
+#undef CLBLAST_HIP_INSTANTIATE
+
+// =================================================================================================
+}  // namespace clblast

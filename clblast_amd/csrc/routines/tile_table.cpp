@@ -1,0 +1,81 @@
+// =================================================================================================
+// Kernel selection for gfx950 (see tile_table.hpp).
+// =================================================================================================
+#include "routines/tile_table.hpp"
+
+#include <map>
+#include <mutex>
+#include <tuple>
+
+#include "clbh_device.h"
+
+namespace clblast {
+namespace {
+
+std::mutex override_mutex;
+std::map<std::tuple<int, int>, size_t> min_indirect_overrides;  // (device, precision bits) -> threshold
+
+}  // namespace
+
+// The MFMA kernels predicate their edge tiles, so they are correct for every shape; the threshold only
+// marks where a 128x128 (or larger) macro tile stops paying for itself against the 64x64 FMA kernel.
+size_t DefaultMinIndirectSize(const Precision precision) {
+  switch (precision) {
+    case Precision::kHalf: return 96;
+    case Precision::kDouble: return 96;
+    default: return 96;
+  }
+}
+
+size_t MinIndirectSize(const int device, const Precision precision) {
+  std::lock_guard<std::mutex> lock(override_mutex);
+  const auto found = min_indirect_overrides.find(std::make_tuple(device, static_cast<int>(precision)));
+  return (found != min_indirect_overrides.end()) ? found->second : DefaultMinIndirectSize(precision);
+}
+
+bool UseDirectKernel(const size_t m, const size_t n, const size_t k, const size_t min_indirect_size) {
+  const auto m_n_k =
+      static_cast<unsigned long long>(m) * static_cast<unsigned long long>(n) * static_cast<unsigned long long>(k);
+  const auto threshold = static_cast<unsigned long long>(min_indirect_size);
+  return m_n_k < threshold * threshold * threshold;
+}
+
+KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const bool b_kcontig, const size_t m,
+                          const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,
+                          const size_t min_indirect_size) {
+  (void)precision; (void)a_kcontig; (void)b_kcontig; (void)batch_count; (void)per_batch_scalars;
+  if (UseDirectKernel(m, n, k, min_indirect_size)) {
+    return KernelChoice{CLBH_KERNEL_GENERAL, 0};
+  }
+  return KernelChoice{CLBH_KERNEL_MFMA, 0};
+}
+
+StatusCode OverrideRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,
+                                     const std::unordered_map<std::string, size_t>& parameters) {
+  if (kernel_name != "GemmRoutine") {
+    return StatusCode::kInvalidOverrideKernel;
+  }
+  const auto found = parameters.find("XGEMM_MIN_INDIRECT_SIZE");
+  if (found == parameters.end()) {
+    return StatusCode::kMissingOverrideParameter;
+  }
+  std::lock_guard<std::mutex> lock(override_mutex);
+  min_indirect_overrides[std::make_tuple(device, static_cast<int>(precision))] = found->second;
+  return StatusCode::kSuccess;
+}
+
+StatusCode RetrieveRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,
+                                     std::unordered_map<std::string, size_t>& parameters) {
+  if (kernel_name != "GemmRoutine") {
+    return StatusCode::kInvalidOverrideKernel;
+  }
+  parameters["XGEMM_MIN_INDIRECT_SIZE"] = MinIndirectSize(device, precision);
+  return StatusCode::kSuccess;
+}
+
+void ClearOverrides() {
+  std::lock_guard<std::mutex> lock(override_mutex);
+  min_indirect_overrides.clear();
+}
+
+}  // namespace clblast

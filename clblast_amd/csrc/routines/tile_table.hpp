@@ -1,0 +1,47 @@
+// =================================================================================================
+// The CDNA4 tile table: which kernel family and which tile shape a GEMM problem gets on gfx950. It
+// replaces the reference's per-device tuning database (src/database/, parameters MWG/NWG/KWG/...,
+// XGEMM_MIN_INDIRECT_SIZE in src/database/kernels/gemm_routine/) with a handful of fixed choices.
+// The only run-time knob kept is the direct/indirect threshold, because the reference's own tests
+// use it to force either kernel family (test/routines/level3/xgemm.hpp:62-70).
+// =================================================================================================
+#ifndef CLBLAST_HIP_TILE_TABLE_HPP_
+#define CLBLAST_HIP_TILE_TABLE_HPP_
+
+#include <cstddef>
+#include <string>
+#include <unordered_map>
+
+#include "clblast_hip.h"
+
+namespace clblast {
+
+struct KernelChoice {
+  int kernel_class;  // enum clbh_kernel_class
+  int tile_variant;  // index into the variant list of that class
+};
+
+// Default direct/indirect thresholds per precision (see tile_table.cpp for the reasoning).
+size_t DefaultMinIndirectSize(const Precision precision);
+
+// Threshold currently in force for (device, precision): the default or an OverrideParameters value.
+size_t MinIndirectSize(const int device, const Precision precision);
+
+// Same decision rule as the reference (src/routines/level3/xgemm.hpp:63-69): m*n*k < threshold^3.
+bool UseDirectKernel(const size_t m, const size_t n, const size_t k, const size_t min_indirect_size);
+
+// Picks the kernel family and tile for a canonical problem (m, n, k per matrix).
+KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const bool b_kcontig, const size_t m,
+                          const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,
+                          const size_t min_indirect_size);
+
+// Parameter override store behind clblast::OverrideParameters / RetrieveParameters / ClearCache.
+StatusCode OverrideRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,
+                                     const std::unordered_map<std::string, size_t>& parameters);
+StatusCode RetrieveRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,
+                                     std::unordered_map<std::string, size_t>& parameters);
+void ClearOverrides();
+
+}  // namespace clblast
+
+#endif  // CLBLAST_HIP_TILE_TABLE_HPP_

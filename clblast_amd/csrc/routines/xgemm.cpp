@@ -1,0 +1,166 @@
+// =================================================================================================
+// Xgemm<T> host logic (see xgemm.hpp).
+// =================================================================================================
+#include "routines/xgemm.hpp"
+
+#include <climits>
+
+namespace clblast {
+// =================================================================================================
+
+GemmRoutineBase::GemmRoutineBase(hipStream_t* queue, hipEvent_t* event, const Precision precision)
+    : stream_(nullptr), event_(event), device_(0), min_indirect_size_(0) {
+  if (queue == nullptr) {
+    throw RuntimeErrorCode(StatusCode::kInvalidCommandQueue, "queue is a null pointer");
+  }
+  stream_ = *queue;
+  CheckDevice(clbh_stream_device(stream_, &device_), "clbh_stream_device");
+  min_indirect_size_ = MinIndirectSize(device_, precision);
+}
+
+void GemmRoutineBase::Finish() const {
+  if (event_ != nullptr && *event_ != nullptr) {
+    CheckDevice(clbh_event_record(*event_, stream_), "clbh_event_record");
+  }
+}
+
+// =================================================================================================
+
+template <typename T>
+Xgemm<T>::Xgemm(hipStream_t* queue, hipEvent_t* event) : GemmRoutineBase(queue, event, PrecisionValue<T>()) {}
+
+template <typename T>
+GemmShape Xgemm<T>::ProcessArguments(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
+                                     const size_t m, const size_t n, const size_t k) {
+  if ((m == 0) || (n == 0) || (k == 0)) {
+    throw BLASError(StatusCode::kInvalidDimension);
+  }
+  // For the real types handled here a conjugate transpose is a plain transpose
+  // (reference: src/kernels/common.opencl:247-251).
+  auto shape = GemmShape{};
+  const auto col_major = (layout == Layout::kColMajor);
+  shape.a_rotated = col_major ? (a_transpose != Transpose::kNo) : (a_transpose == Transpose::kNo);
+  shape.b_rotated = col_major ? (b_transpose != Transpose::kNo) : (b_transpose == Transpose::kNo);
+  shape.c_rotated = !col_major;
+  shape.a_one = shape.a_rotated ? k : m;
+  shape.a_two = shape.a_rotated ? m : k;
+  shape.b_one = shape.b_rotated ? n : k;
+  shape.b_two = shape.b_rotated ? k : n;
+  shape.c_one = shape.c_rotated ? n : m;
+  shape.c_two = shape.c_rotated ? m : n;
+  return shape;
+}
+
+template <typename T>
+clbh_gemm_desc Xgemm<T>::Canonicalise(const GemmShape& shape, const Layout layout, const size_t m, const size_t n,
+                                      const size_t k, const void* a, const size_t a_offset, const size_t a_ld,
+                                      const void* b, const size_t b_offset, const size_t b_ld, void* c,
+                                      const size_t c_offset, const size_t c_ld) {
+  if (m > static_cast<size_t>(INT_MAX) || n > static_cast<size_t>(INT_MAX) || k > static_cast<size_t>(INT_MAX)) {
+    throw BLASError(StatusCode::kInvalidDimension, "dimension exceeds 2^31-1");
+  }
+  auto desc = clbh_gemm_desc{};
+  desc.precision = static_cast<int>(PrecisionValue<T>());
+  desc.k = static_cast<int>(k);
+  desc.batch_count = 1;
+  desc.c = c;
+  desc.c_offset = static_cast<long long>(c_offset);
+  desc.c_ld = static_cast<long long>(c_ld);
+  if (layout == Layout::kColMajor) {
+    // A(i,p): rotated -> i*lda + p (k contiguous). B(p,j): rotated -> p*ldb + j (n contiguous).
+    desc.m = static_cast<int>(m);
+    desc.n = static_cast<int>(n);
+    desc.a = a;
+    desc.a_offset = static_cast<long long>(a_offset);
+    desc.a_ld = static_cast<long long>(a_ld);
+    desc.a_kcontig = shape.a_rotated ? 1 : 0;
+    desc.b = b;
+    desc.b_offset = static_cast<long long>(b_offset);
+    desc.b_ld = static_cast<long long>(b_ld);
+    desc.b_kcontig = shape.b_rotated ? 0 : 1;
+  } else {
+    // Row-major C (m x n) is column-major C^T (n x m) = op(B)^T * op(A)^T: the user's B becomes the
+    // canonical A (its n index is the canonical row index), the user's A the canonical B.
+    desc.m = static_cast<int>(n);
+    desc.n = static_cast<int>(m);
+    desc.a = b;
+    desc.a_offset = static_cast<long long>(b_offset);
+    desc.a_ld = static_cast<long long>(b_ld);
+    desc.a_kcontig = shape.b_rotated ? 0 : 1;
+    desc.b = a;
+    desc.b_offset = static_cast<long long>(a_offset);
+    desc.b_ld = static_cast<long long>(a_ld);
+    desc.b_kcontig = shape.a_rotated ? 1 : 0;
+  }
+  return desc;
+}
+
+template <typename T>
+size_t Xgemm<T>::TempBytes(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
+                           const size_t m, const size_t n, const size_t k, const size_t min_indirect_size) {
+  const auto shape = ProcessArguments(layout, a_transpose, b_transpose, m, n, k);
+  auto desc = Canonicalise(shape, layout, m, n, k, nullptr, 0, shape.a_one, nullptr, 0, shape.b_one, nullptr, 0,
+                           shape.c_one);
+  const auto choice = SelectKernel(PrecisionValue<T>(), desc.a_kcontig != 0, desc.b_kcontig != 0,
+                                   static_cast<size_t>(desc.m), static_cast<size_t>(desc.n), k, 1, false,
+                                   min_indirect_size);
+  desc.kernel_class = choice.kernel_class;
+  desc.tile_variant = choice.tile_variant;
+  return clbh_gemm_workspace_bytes(&desc);
+}
+
+// =================================================================================================
+
+template <typename T>
+void Xgemm<T>::DoGemm(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
+                      const size_t n, const size_t k, const T alpha, const Buffer<T>& a_buffer, const size_t a_offset,
+                      const size_t a_ld, const Buffer<T>& b_buffer, const size_t b_offset, const size_t b_ld,
+                      const T beta, const Buffer<T>& c_buffer, const size_t c_offset, const size_t c_ld,
+                      const Buffer<T>& temp_buffer, const bool temp_buffer_provided) {
+  // Same order as the reference: dimensions, then A (ld, size), B, C, then the temporary buffer
+  const auto shape = ProcessArguments(layout, a_transpose, b_transpose, m, n, k);
+  TestMatrixA(shape.a_one, shape.a_two, a_buffer, a_offset, a_ld);
+  TestMatrixB(shape.b_one, shape.b_two, b_buffer, b_offset, b_ld);
+  TestMatrixC(shape.c_one, shape.c_two, c_buffer, c_offset, c_ld);
+
+  auto desc = Canonicalise(shape, layout, m, n, k, a_buffer(), a_offset, a_ld, b_buffer(), b_offset, b_ld,
+                           const_cast<void*>(c_buffer()), c_offset, c_ld);
+  const auto choice = SelectKernel(PrecisionValue<T>(), desc.a_kcontig != 0, desc.b_kcontig != 0,
+                                   static_cast<size_t>(desc.m), static_cast<size_t>(desc.n), k, 1, false,
+                                   min_indirect_size());
+  desc.kernel_class = choice.kernel_class;
+  desc.tile_variant = choice.tile_variant;
+  desc.alpha = ScalarToDouble(alpha);
+  desc.beta = ScalarToDouble(beta);
+
+  // Temporary memory: only split-K launches want any. A caller-provided buffer must be large enough
+  // (reference: xgemm.cpp:146-151), otherwise stream-ordered scratch is taken for the call.
+  const auto temp_bytes = clbh_gemm_workspace_bytes(&desc);
+  void* scratch = nullptr;
+  if (temp_buffer_provided) {
+    if (temp_bytes > 0 && temp_buffer.GetSize() < temp_bytes) {
+      throw BLASError(StatusCode::kInsufficientMemoryTemp);
+    }
+    desc.workspace = const_cast<void*>(temp_buffer());
+  } else if (temp_bytes > 0) {
+    if (clbh_alloc_async(&scratch, temp_bytes, stream()) != 0) {
+      throw RuntimeErrorCode(StatusCode::kTempBufferAllocFailure, "temporary buffer");
+    }
+    desc.workspace = scratch;
+  }
+  desc.workspace_bytes = temp_bytes;
+
+  const auto launch_status = clbh_gemm_launch(&desc, stream());
+  if (scratch != nullptr) {
+    clbh_free_async(scratch, stream());
+  }
+  CheckDevice(launch_status, "clbh_gemm_launch");
+  Finish();
+}
+
+template class Xgemm<half>;
+template class Xgemm<float>;
+template class Xgemm<double>;
+
+// =================================================================================================
+}  // namespace clblast

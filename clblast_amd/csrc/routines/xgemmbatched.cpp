@@ -1,0 +1,159 @@
+// =================================================================================================
+// Batched and strided-batched GEMM host logic (see xgemmbatched.hpp).
+// =================================================================================================
+#include "routines/xgemmbatched.hpp"
+
+#include <algorithm>
+#include <climits>
+#include <cstring>
+
+namespace clblast {
+// =================================================================================================
+
+template <typename T>
+XgemmBatched<T>::XgemmBatched(hipStream_t* queue, hipEvent_t* event)
+    : GemmRoutineBase(queue, event, PrecisionValue<T>()) {}
+
+template <typename T>
+void XgemmBatched<T>::DoGemmBatched(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
+                                    const size_t m, const size_t n, const size_t k, const std::vector<T>& alphas,
+                                    const Buffer<T>& a_buffer, const std::vector<size_t>& a_offsets,
+                                    const size_t a_ld, const Buffer<T>& b_buffer,
+                                    const std::vector<size_t>& b_offsets, const size_t b_ld,
+                                    const std::vector<T>& betas, const Buffer<T>& c_buffer,
+                                    const std::vector<size_t>& c_offsets, const size_t c_ld,
+                                    const size_t batch_count) {
+  // Batch count and array lengths first (reference: xgemmbatched.cpp:66-69)
+  if ((batch_count < 1) || (alphas.size() != batch_count) || (betas.size() != batch_count) ||
+      (a_offsets.size() != batch_count) || (b_offsets.size() != batch_count) || (c_offsets.size() != batch_count)) {
+    throw BLASError(StatusCode::kInvalidBatchCount);
+  }
+  if (batch_count > static_cast<size_t>(INT_MAX)) {
+    throw BLASError(StatusCode::kInvalidBatchCount, "batch count exceeds 2^31-1");
+  }
+  const auto shape = Xgemm<T>::ProcessArguments(layout, a_transpose, b_transpose, m, n, k);
+
+  // The largest offset decides; the leading dimensions of A and B are not tested, that of C is
+  // (reference: xgemmbatched.cpp:82-84, buffer_test.hpp:169-190)
+  const auto a_max = *std::max_element(a_offsets.begin(), a_offsets.end());
+  const auto b_max = *std::max_element(b_offsets.begin(), b_offsets.end());
+  const auto c_max = *std::max_element(c_offsets.begin(), c_offsets.end());
+  TestMatrixA(shape.a_one, shape.a_two, a_buffer, a_max, a_ld, false);
+  TestMatrixB(shape.b_one, shape.b_two, b_buffer, b_max, b_ld, false);
+  TestMatrixC(shape.c_one, shape.c_two, c_buffer, c_max, c_ld);
+
+  auto desc = Xgemm<T>::Canonicalise(shape, layout, m, n, k, a_buffer(), 0, a_ld, b_buffer(), 0, b_ld,
+                                     const_cast<void*>(c_buffer()), 0, c_ld);
+  const auto choice = SelectKernel(PrecisionValue<T>(), desc.a_kcontig != 0, desc.b_kcontig != 0,
+                                   static_cast<size_t>(desc.m), static_cast<size_t>(desc.n), k, batch_count, true,
+                                   min_indirect_size());
+  desc.kernel_class = choice.kernel_class;
+  desc.tile_variant = choice.tile_variant;
+  desc.batch_count = static_cast<int>(batch_count);
+
+  // Packs [alphas | betas | a_offsets | b_offsets | c_offsets] into one host block. Scalars are stored
+  // in the kernels' compute type: float for fp16/fp32 (half scalars are widened on the host as in
+  // utilities.cpp:480-483), double for fp64. After the row-major fold the canonical A is the user's B.
+  const auto scalar_bytes = (PrecisionValue<T>() == Precision::kDouble) ? sizeof(double) : sizeof(float);
+  const auto scalars_block = Ceil(batch_count * scalar_bytes, 8);
+  const auto offsets_block = batch_count * sizeof(long long);
+  const auto total_bytes = 2 * scalars_block + 3 * offsets_block;
+  auto packed = std::vector<unsigned char>(total_bytes);
+  for (auto batch = size_t{0}; batch < batch_count; ++batch) {
+    if (PrecisionValue<T>() == Precision::kDouble) {
+      const auto alpha = ScalarToDouble(alphas[batch]);
+      const auto beta = ScalarToDouble(betas[batch]);
+      std::memcpy(&packed[batch * sizeof(double)], &alpha, sizeof(double));
+      std::memcpy(&packed[scalars_block + batch * sizeof(double)], &beta, sizeof(double));
+    } else {
+      const auto alpha = static_cast<float>(ScalarToDouble(alphas[batch]));
+      const auto beta = static_cast<float>(ScalarToDouble(betas[batch]));
+      std::memcpy(&packed[batch * sizeof(float)], &alpha, sizeof(float));
+      std::memcpy(&packed[scalars_block + batch * sizeof(float)], &beta, sizeof(float));
+    }
+    const auto col_major = (layout == Layout::kColMajor);
+    const auto a_off = static_cast<long long>(col_major ? a_offsets[batch] : b_offsets[batch]);
+    const auto b_off = static_cast<long long>(col_major ? b_offsets[batch] : a_offsets[batch]);
+    const auto c_off = static_cast<long long>(c_offsets[batch]);
+    std::memcpy(&packed[2 * scalars_block + batch * sizeof(long long)], &a_off, sizeof(long long));
+    std::memcpy(&packed[2 * scalars_block + offsets_block + batch * sizeof(long long)], &b_off, sizeof(long long));
+    std::memcpy(&packed[2 * scalars_block + 2 * offsets_block + batch * sizeof(long long)], &c_off,
+                sizeof(long long));
+  }
+
+  void* device_block = nullptr;
+  if (clbh_alloc_async(&device_block, total_bytes, stream()) != 0) {
+    throw RuntimeErrorCode(StatusCode::kTempBufferAllocFailure, "batch metadata");
+  }
+  auto status = clbh_upload_async(device_block, packed.data(), total_bytes, stream());
+  if (status == 0) {
+    const auto base = static_cast<unsigned char*>(device_block);
+    desc.batch.alphas = base;
+    desc.batch.betas = base + scalars_block;
+    desc.batch.a_offsets = reinterpret_cast<const long long*>(base + 2 * scalars_block);
+    desc.batch.b_offsets = reinterpret_cast<const long long*>(base + 2 * scalars_block + offsets_block);
+    desc.batch.c_offsets = reinterpret_cast<const long long*>(base + 2 * scalars_block + 2 * offsets_block);
+    status = clbh_gemm_launch(&desc, stream());
+  }
+  clbh_free_async(device_block, stream());
+  CheckDevice(status, "batched GEMM launch");
+  Finish();
+}
+
+// =================================================================================================
+
+template <typename T>
+XgemmStridedBatched<T>::XgemmStridedBatched(hipStream_t* queue, hipEvent_t* event)
+    : GemmRoutineBase(queue, event, PrecisionValue<T>()) {}
+
+template <typename T>
+void XgemmStridedBatched<T>::DoGemmStridedBatched(
+    const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m, const size_t n,
+    const size_t k, const T alpha, const Buffer<T>& a_buffer, const size_t a_offset, const size_t a_ld,
+    const size_t a_stride, const Buffer<T>& b_buffer, const size_t b_offset, const size_t b_ld, const size_t b_stride,
+    const T beta, const Buffer<T>& c_buffer, const size_t c_offset, const size_t c_ld, const size_t c_stride,
+    const size_t batch_count) {
+  // reference: xgemmstridedbatched.cpp:68-75
+  if (batch_count < 1) {
+    throw BLASError(StatusCode::kInvalidBatchCount);
+  }
+  if (c_stride == 0) {
+    throw BLASError(StatusCode::kInvalidDimension);
+  }
+  if (batch_count > static_cast<size_t>(INT_MAX)) {
+    throw BLASError(StatusCode::kInvalidBatchCount, "batch count exceeds 2^31-1");
+  }
+  const auto shape = Xgemm<T>::ProcessArguments(layout, a_transpose, b_transpose, m, n, k);
+
+  // The last matrix of the batch decides (reference: buffer_test.hpp:195-218)
+  TestMatrixA(shape.a_one, shape.a_two, a_buffer, a_offset + (batch_count - 1) * a_stride, a_ld);
+  TestMatrixB(shape.b_one, shape.b_two, b_buffer, b_offset + (batch_count - 1) * b_stride, b_ld);
+  TestMatrixC(shape.c_one, shape.c_two, c_buffer, c_offset + (batch_count - 1) * c_stride, c_ld);
+
+  auto desc = Xgemm<T>::Canonicalise(shape, layout, m, n, k, a_buffer(), a_offset, a_ld, b_buffer(), b_offset, b_ld,
+                                     const_cast<void*>(c_buffer()), c_offset, c_ld);
+  const auto col_major = (layout == Layout::kColMajor);
+  desc.a_stride = static_cast<long long>(col_major ? a_stride : b_stride);
+  desc.b_stride = static_cast<long long>(col_major ? b_stride : a_stride);
+  desc.c_stride = static_cast<long long>(c_stride);
+  desc.batch_count = static_cast<int>(batch_count);
+  desc.alpha = ScalarToDouble(alpha);
+  desc.beta = ScalarToDouble(beta);
+  const auto choice = SelectKernel(PrecisionValue<T>(), desc.a_kcontig != 0, desc.b_kcontig != 0,
+                                   static_cast<size_t>(desc.m), static_cast<size_t>(desc.n), k, batch_count, false,
+                                   min_indirect_size());
+  desc.kernel_class = choice.kernel_class;
+  desc.tile_variant = choice.tile_variant;
+  CheckDevice(clbh_gemm_launch(&desc, stream()), "strided-batched GEMM launch");
+  Finish();
+}
+
+template class XgemmBatched<half>;
+template class XgemmBatched<float>;
+template class XgemmBatched<double>;
+template class XgemmStridedBatched<half>;
+template class XgemmStridedBatched<float>;
+template class XgemmStridedBatched<double>;
+
+// =================================================================================================
+}  // namespace clblast

@@ -1,0 +1,99 @@
+// =================================================================================================
+// Thin C-ABI device layer: the only place of the library that touches the HIP runtime. The C++ host
+// routines (routines/xgemm*.cpp) describe one canonical GEMM launch in a plain struct and hand it to
+// clbh_gemm_launch; they never include HIP headers.
+//
+// It takes the place of the reference's kernel-launch plumbing: `Kernel::SetArgument/Launch`
+// (reference: src/clpp11.hpp:816-879), `RunKernel` (src/routines/common.cpp:24-85), `Buffer::GetSize`
+// (src/clpp11.hpp:763-768) and the blocking scalar/offset uploads of the batched routines
+// (src/routines/levelx/xgemmbatched.cpp:87-100, 262-267).
+//
+// Canonical problem: column-major C (m x n, leading dimension c_ld) = alpha * A * B + beta * C with
+//   A(i,p) at a[a_offset + (a_kcontig ? i*a_ld + p : p*a_ld + i)]   i < m, p < k
+//   B(p,j) at b[b_offset + (b_kcontig ? j*b_ld + p : p*b_ld + j)]   p < k, j < n
+//   C(i,j) at c[c_offset + j*c_ld + i]
+// Row-major problems are folded into this form on the host by exchanging the roles of A and B.
+// Batch b adds b*stride (strided) or the b-th entry of the offset arrays (batched) to each offset.
+// =================================================================================================
+#ifndef CLBH_DEVICE_H_
+#define CLBH_DEVICE_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* hipStream_t;
+typedef struct ihipEvent_t* hipEvent_t;
+
+#define CLBH_API __attribute__((visibility("default")))
+
+// Kernel families of the engine (what the reference's tuning database selected by parameter sets).
+enum clbh_kernel_class {
+  CLBH_KERNEL_GENERAL = 0,  // bounds-checked LDS-tiled FMA kernel, any shape (reference analogue: XgemmDirect)
+  CLBH_KERNEL_MFMA = 1,     // large-tile MFMA kernel with LDS double buffering (analogue: Xgemm indirect)
+  CLBH_KERNEL_SMALL_BATCHED = 2,  // one wavefront per small matrix, bandwidth bound
+  CLBH_KERNEL_SKINNY = 3          // split-K streaming kernel for problems with a tiny m or n
+};
+
+// Per-batch metadata of GemmBatched, all device pointers (NULL for plain and strided launches).
+typedef struct clbh_batch_arrays_ {
+  const void* alphas;           // element type = compute scalar type (float for fp16/fp32, double for fp64)
+  const void* betas;
+  const long long* a_offsets;   // element offsets
+  const long long* b_offsets;
+  const long long* c_offsets;
+} clbh_batch_arrays;
+
+typedef struct clbh_gemm_desc_ {
+  int precision;      // 16, 32 or 64 (bits of the storage type)
+  int kernel_class;   // enum clbh_kernel_class
+  int tile_variant;   // index into the tile table of that class (0 = default)
+  int a_kcontig;      // see header comment
+  int b_kcontig;
+  int m, n, k;
+  int batch_count;    // >= 1
+  const void* a;
+  const void* b;
+  void* c;
+  long long a_offset, b_offset, c_offset;  // elements
+  long long a_ld, b_ld, c_ld;              // elements
+  long long a_stride, b_stride, c_stride;  // elements; used when batch.alphas == NULL
+  double alpha, beta;                      // used when batch.alphas == NULL
+  clbh_batch_arrays batch;
+  void* workspace;          // optional device scratch (split-K partial sums), may be NULL
+  size_t workspace_bytes;
+} clbh_gemm_desc;
+
+// Enqueues the kernel(s) for one descriptor on `stream`. Returns 0 on success, otherwise the HIP
+// error code (positive). Never synchronises.
+CLBH_API int clbh_gemm_launch(const clbh_gemm_desc* desc, hipStream_t stream);
+
+// Bytes of device scratch the given descriptor needs in `workspace` (0 for most launches).
+CLBH_API size_t clbh_gemm_workspace_bytes(const clbh_gemm_desc* desc);
+
+// Number of bytes addressable from `ptr` to the end of the device allocation that contains it.
+// Returns 0 on success, non-zero if `ptr` is not inside a device allocation.
+CLBH_API int clbh_buffer_extent(const void* ptr, size_t* bytes_available);
+
+// Stream-ordered scratch memory.
+CLBH_API int clbh_alloc_async(void** ptr, size_t bytes, hipStream_t stream);
+CLBH_API int clbh_free_async(void* ptr, hipStream_t stream);
+
+// Stream-ordered host-to-device copy of a small array; the host memory may be reused on return.
+CLBH_API int clbh_upload_async(void* dst_device, const void* src_host, size_t bytes, hipStream_t stream);
+
+CLBH_API int clbh_event_record(hipEvent_t event, hipStream_t stream);
+
+// Ordinal of the device `stream` belongs to (the current device for the null stream).
+CLBH_API int clbh_stream_device(hipStream_t stream, int* device);
+
+// Human-readable text for a code returned by the functions above.
+CLBH_API const char* clbh_error_string(int code);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif  // CLBH_DEVICE_H_

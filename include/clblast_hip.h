@@ -1,0 +1,161 @@
+// =================================================================================================
+// C++ interface of the MI355X (gfx950) GEMM engine behind the CLBlast GEMM API.
+//
+// The argument surface is the one of CLBlast's `include/clblast.h` (reference: Gemm :427-432,
+// GemmBatched :538-543, GemmStridedBatched :547-553, GemmTempBufferSize :558-562, StatusCode :61-129,
+// Layout/Transpose/Precision :132-147, OverrideParameters :620-624, ClearCache :568). Only the handle
+// types differ: `cl_mem` becomes a raw device pointer (`void*`, as returned by hipMalloc or
+// `tensor.data_ptr()`), `cl_command_queue*` becomes `hipStream_t*` and `cl_event*` becomes
+// `hipEvent_t*`. Offsets and leading dimensions are in elements, exactly as in the reference.
+//
+// Differences a caller can observe:
+//   * `event`: the OpenCL flavour hands back a new event; here a non-null `*event` must be an
+//     existing hipEvent_t which is recorded on `*queue` after the last kernel of the call.
+//   * All work is stream-ordered on `*queue`; the call returns after enqueueing.
+//   * GemmTempBufferSize reports what this engine needs (normally 0), not the reference's figure.
+// =================================================================================================
+#ifndef CLBLAST_HIP_H_
+#define CLBLAST_HIP_H_
+
+#include <cstddef>
+#include <string>
+#include <unordered_map>
+
+// HIP handle types, declared the way <hip/hip_runtime_api.h> declares them so that this header can be
+// used with or without the HIP headers in the same translation unit.
+typedef struct ihipStream_t* hipStream_t;
+typedef struct ihipEvent_t* hipEvent_t;
+
+namespace clblast {
+// =================================================================================================
+
+// Status codes: numeric values are ABI and equal the reference's (include/clblast.h:61-129).
+enum class StatusCode {
+  kSuccess = 0,
+  kOpenCLCompilerNotAvailable = -3,
+  kTempBufferAllocFailure = -4,
+  kOpenCLOutOfResources = -5,
+  kOpenCLOutOfHostMemory = -6,
+  kOpenCLBuildProgramFailure = -11,
+  kInvalidValue = -30,
+  kInvalidCommandQueue = -36,
+  kInvalidMemObject = -38,
+  kInvalidBinary = -42,
+  kInvalidBuildOptions = -43,
+  kInvalidProgram = -44,
+  kInvalidProgramExecutable = -45,
+  kInvalidKernelName = -46,
+  kInvalidKernelDefinition = -47,
+  kInvalidKernel = -48,
+  kInvalidArgIndex = -49,
+  kInvalidArgValue = -50,
+  kInvalidArgSize = -51,
+  kInvalidKernelArgs = -52,
+  kInvalidLocalNumDimensions = -53,
+  kInvalidLocalThreadsTotal = -54,
+  kInvalidLocalThreadsDim = -55,
+  kInvalidGlobalOffset = -56,
+  kInvalidEventWaitList = -57,
+  kInvalidEvent = -58,
+  kInvalidOperation = -59,
+  kInvalidBufferSize = -61,
+  kInvalidGlobalWorkSize = -63,
+
+  kNotImplemented = -1024,
+  kInvalidMatrixA = -1022,
+  kInvalidMatrixB = -1021,
+  kInvalidMatrixC = -1020,
+  kInvalidVectorX = -1019,
+  kInvalidVectorY = -1018,
+  kInvalidDimension = -1017,
+  kInvalidLeadDimA = -1016,
+  kInvalidLeadDimB = -1015,
+  kInvalidLeadDimC = -1014,
+  kInvalidIncrementX = -1013,
+  kInvalidIncrementY = -1012,
+  kInsufficientMemoryA = -1011,
+  kInsufficientMemoryB = -1010,
+  kInsufficientMemoryC = -1009,
+  kInsufficientMemoryX = -1008,
+  kInsufficientMemoryY = -1007,
+
+  kInsufficientMemoryTemp = -2050,
+  kInvalidBatchCount = -2049,
+  kInvalidOverrideKernel = -2048,
+  kMissingOverrideParameter = -2047,
+  kInvalidLocalMemUsage = -2046,
+  kNoHalfPrecision = -2045,
+  kNoDoublePrecision = -2044,
+  kInvalidVectorScalar = -2043,
+  kInsufficientMemoryScalar = -2042,
+  kDatabaseError = -2041,
+  kUnknownError = -2040,
+  kUnexpectedError = -2039,
+  kInvalidVectorZ = -2038,
+  kInvalidIncrementZ = -2037,
+  kInsufficientMemoryZ = -2036,
+};
+
+enum class Layout { kRowMajor = 101, kColMajor = 102 };
+enum class Transpose { kNo = 111, kYes = 112, kConjugate = 113 };
+enum class Precision { kHalf = 16, kSingle = 32, kDouble = 64, kComplexSingle = 3232, kComplexDouble = 6464, kAny = -1 };
+
+// Host type of fp16 scalars and data: the IEEE binary16 bit pattern (reference: clblast_half.h:21).
+using half = unsigned short;
+
+// =================================================================================================
+
+// C = alpha * op(A) * op(B) + beta * C. T is float, double or half.
+template <typename T>
+StatusCode Gemm(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
+                const size_t n, const size_t k, const T alpha, const void* a_buffer, const size_t a_offset,
+                const size_t a_ld, const void* b_buffer, const size_t b_offset, const size_t b_ld, const T beta,
+                void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                hipEvent_t* event = nullptr, void* temp_buffer = nullptr);
+
+// Per-batch scalars and element offsets (host arrays of length batch_count).
+template <typename T>
+StatusCode GemmBatched(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
+                       const size_t n, const size_t k, const T* alphas, const void* a_buffer, const size_t* a_offsets,
+                       const size_t a_ld, const void* b_buffer, const size_t* b_offsets, const size_t b_ld,
+                       const T* betas, void* c_buffer, const size_t* c_offsets, const size_t c_ld,
+                       const size_t batch_count, hipStream_t* queue, hipEvent_t* event = nullptr);
+
+// One alpha/beta; matrix b of the batch lives at offset + b * stride.
+template <typename T>
+StatusCode GemmStridedBatched(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
+                              const size_t m, const size_t n, const size_t k, const T alpha, const void* a_buffer,
+                              const size_t a_offset, const size_t a_ld, const size_t a_stride, const void* b_buffer,
+                              const size_t b_offset, const size_t b_ld, const size_t b_stride, const T beta,
+                              void* c_buffer, const size_t c_offset, const size_t c_ld, const size_t c_stride,
+                              const size_t batch_count, hipStream_t* queue, hipEvent_t* event = nullptr);
+
+// Bytes this engine wants in `temp_buffer` for the given arguments (0 when none is needed).
+template <typename T>
+StatusCode GemmTempBufferSize(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
+                              const size_t m, const size_t n, const size_t k, const size_t a_offset, const size_t a_ld,
+                              const size_t b_offset, const size_t b_ld, const size_t c_offset, const size_t c_ld,
+                              hipStream_t* queue, size_t& temp_buffer_size);
+
+// =================================================================================================
+
+// Drops per-process cached state (device properties, buffer-extent cache). Kernels are compiled ahead
+// of time, so there is no program cache to clear.
+StatusCode ClearCache();
+
+// Overrides engine parameters for one device ordinal and precision. Accepted kernel names:
+//   "GemmRoutine": {"XGEMM_MIN_INDIRECT_SIZE": s} - problems with m*n*k < s^3 take the general
+//                  (direct) kernel, all others the MFMA-tiled kernels (reference:
+//                  src/routines/level3/xgemm.hpp:63-69, test/routines/level3/xgemm.hpp:62-70).
+// Any other kernel name returns kInvalidOverrideKernel, a missing parameter kMissingOverrideParameter.
+StatusCode OverrideParameters(const int device, const std::string& kernel_name, const Precision precision,
+                              const std::unordered_map<std::string, size_t>& parameters);
+
+// Reads back the parameters currently in force for (device, kernel_name, precision).
+StatusCode RetrieveParameters(const int device, const std::string& kernel_name, const Precision precision,
+                              std::unordered_map<std::string, size_t>& parameters);
+
+// =================================================================================================
+}  // namespace clblast
+
+#endif  // CLBLAST_HIP_H_

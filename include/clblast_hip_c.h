@@ -1,0 +1,200 @@
+// =================================================================================================
+// C interface (extern "C") of the MI355X (gfx950) GEMM engine behind the CLBlast GEMM API.
+//
+// These are the entry points a foreign-function binding (ctypes, cgo, JNI, N-API) binds. They carry
+// plain pointers and sizes only. Names, argument order and meaning follow CLBlast's
+// `include/clblast_c.h`; each declaration cites the reference declaration it replaces. Handle types:
+// `cl_mem` -> `void*` device pointer, `cl_command_queue*` -> `hipStream_t*`, `cl_event*` ->
+// `hipEvent_t*` (a non-null `*event` is an existing event that is recorded after the last kernel).
+// Offsets, strides and leading dimensions are in elements. Half-precision scalars travel as IEEE
+// binary16 bit patterns (`cl_half` = unsigned short).
+// =================================================================================================
+#ifndef CLBLAST_HIP_C_H_
+#define CLBLAST_HIP_C_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+// HIP handle types, declared as <hip/hip_runtime_api.h> declares them.
+typedef struct ihipStream_t* hipStream_t;
+typedef struct ihipEvent_t* hipEvent_t;
+
+#ifndef CLBLAST_HIP_CL_HALF_DEFINED
+#define CLBLAST_HIP_CL_HALF_DEFINED
+typedef unsigned short cl_half;
+#endif
+
+#define CLBLAST_HIP_API __attribute__((visibility("default")))
+
+// Status codes (reference: include/clblast_c.h:62-130). Only the codes this path can return are
+// named; every other value of the reference's enum keeps its numeric meaning.
+typedef enum CLBlastStatusCode_ {
+  CLBlastSuccess = 0,
+  CLBlastTempBufferAllocFailure = -4,
+  CLBlastInvalidValue = -30,
+  CLBlastInvalidCommandQueue = -36,
+  CLBlastNotImplemented = -1024,
+  CLBlastInvalidMatrixA = -1022,
+  CLBlastInvalidMatrixB = -1021,
+  CLBlastInvalidMatrixC = -1020,
+  CLBlastInvalidDimension = -1017,
+  CLBlastInvalidLeadDimA = -1016,
+  CLBlastInvalidLeadDimB = -1015,
+  CLBlastInvalidLeadDimC = -1014,
+  CLBlastInsufficientMemoryA = -1011,
+  CLBlastInsufficientMemoryB = -1010,
+  CLBlastInsufficientMemoryC = -1009,
+  CLBlastInsufficientMemoryTemp = -2050,
+  CLBlastInvalidBatchCount = -2049,
+  CLBlastInvalidOverrideKernel = -2048,
+  CLBlastMissingOverrideParameter = -2047,
+  CLBlastNoHalfPrecision = -2045,
+  CLBlastNoDoublePrecision = -2044,
+  CLBlastUnknownError = -2040,
+  CLBlastUnexpectedError = -2039
+} CLBlastStatusCode;
+
+// reference: include/clblast_c.h:133-138, 148-154
+typedef enum CLBlastLayout_ { CLBlastLayoutRowMajor = 101, CLBlastLayoutColMajor = 102 } CLBlastLayout;
+typedef enum CLBlastTranspose_ {
+  CLBlastTransposeNo = 111,
+  CLBlastTransposeYes = 112,
+  CLBlastTransposeConjugate = 113
+} CLBlastTranspose;
+typedef enum CLBlastPrecision_ {
+  CLBlastPrecisionHalf = 16,
+  CLBlastPrecisionSingle = 32,
+  CLBlastPrecisionDouble = 64
+} CLBlastPrecision;
+
+
+// =================================================================================================
+// General matrix-matrix multiplication C = alpha*op(A)*op(B) + beta*C
+// replaces CLBlastSgemm/CLBlastDgemm/CLBlastHgemm (reference: include/clblast_c.h:885-919, src/clblast_c.cpp:1800-1874)
+CLBlastStatusCode CLBLAST_HIP_API CLBlastSgemm(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                               const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                               const size_t k, const float alpha, const void* a_buffer,
+                                               const size_t a_offset, const size_t a_ld, const void* b_buffer,
+                                               const size_t b_offset, const size_t b_ld, const float beta,
+                                               void* c_buffer, const size_t c_offset, const size_t c_ld,
+                                               hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastDgemm(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                               const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                               const size_t k, const double alpha, const void* a_buffer,
+                                               const size_t a_offset, const size_t a_ld, const void* b_buffer,
+                                               const size_t b_offset, const size_t b_ld, const double beta,
+                                               void* c_buffer, const size_t c_offset, const size_t c_ld,
+                                               hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastHgemm(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                               const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                               const size_t k, const cl_half alpha, const void* a_buffer,
+                                               const size_t a_offset, const size_t a_ld, const void* b_buffer,
+                                               const size_t b_offset, const size_t b_ld, const cl_half beta,
+                                               void* c_buffer, const size_t c_offset, const size_t c_ld,
+                                               hipStream_t* queue, hipEvent_t* event);
+
+// =================================================================================================
+// Batched GEMM with per-batch alpha, beta and element offsets (host arrays of length batch_count)
+// replaces CLBlast{S,D,H}gemmBatched (reference: include/clblast_c.h:1303-1337, src/clblast_c.cpp:2723-2833)
+CLBlastStatusCode CLBLAST_HIP_API CLBlastSgemmBatched(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const float* alphas, const void* a_buffer, const size_t* a_offsets,
+    const size_t a_ld, const void* b_buffer, const size_t* b_offsets, const size_t b_ld, const float* betas,
+    void* c_buffer, const size_t* c_offsets, const size_t c_ld, const size_t batch_count, hipStream_t* queue,
+    hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastDgemmBatched(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const double* alphas, const void* a_buffer, const size_t* a_offsets,
+    const size_t a_ld, const void* b_buffer, const size_t* b_offsets, const size_t b_ld, const double* betas,
+    void* c_buffer, const size_t* c_offsets, const size_t c_ld, const size_t batch_count, hipStream_t* queue,
+    hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastHgemmBatched(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const cl_half* alphas, const void* a_buffer, const size_t* a_offsets,
+    const size_t a_ld, const void* b_buffer, const size_t* b_offsets, const size_t b_ld, const cl_half* betas,
+    void* c_buffer, const size_t* c_offsets, const size_t c_ld, const size_t batch_count, hipStream_t* queue,
+    hipEvent_t* event);
+
+// =================================================================================================
+// Strided-batched GEMM: matrix i of the batch lives at offset + i*stride
+// replaces CLBlast{S,D,H}gemmStridedBatched (reference: include/clblast_c.h:1341-1370, src/clblast_c.cpp:2835-2924)
+CLBlastStatusCode CLBLAST_HIP_API CLBlastSgemmStridedBatched(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const float alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+    const size_t a_stride, const void* b_buffer, const size_t b_offset, const size_t b_ld, const size_t b_stride,
+    const float beta, void* c_buffer, const size_t c_offset, const size_t c_ld, const size_t c_stride,
+    const size_t batch_count, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastDgemmStridedBatched(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const double alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+    const size_t a_stride, const void* b_buffer, const size_t b_offset, const size_t b_ld, const size_t b_stride,
+    const double beta, void* c_buffer, const size_t c_offset, const size_t c_ld, const size_t c_stride,
+    const size_t batch_count, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastHgemmStridedBatched(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const cl_half alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+    const size_t a_stride, const void* b_buffer, const size_t b_offset, const size_t b_ld, const size_t b_stride,
+    const cl_half beta, void* c_buffer, const size_t c_offset, const size_t c_ld, const size_t c_stride,
+    const size_t batch_count, hipStream_t* queue, hipEvent_t* event);
+
+// =================================================================================================
+// GEMM with a caller-provided temporary buffer (may be NULL)
+// replaces CLBlast{S,D,H}gemmWithTempBuffer (reference: include/clblast_c.h:1375-1408, src/clblast_c.cpp:2926-3009)
+CLBlastStatusCode CLBLAST_HIP_API CLBlastSgemmWithTempBuffer(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const float alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+    const void* b_buffer, const size_t b_offset, const size_t b_ld, const float beta, void* c_buffer,
+    const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event, void* temp_buffer);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastDgemmWithTempBuffer(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const double alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+    const void* b_buffer, const size_t b_offset, const size_t b_ld, const double beta, void* c_buffer,
+    const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event, void* temp_buffer);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastHgemmWithTempBuffer(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const cl_half alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+    const void* b_buffer, const size_t b_offset, const size_t b_ld, const cl_half beta, void* c_buffer,
+    const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event, void* temp_buffer);
+
+// =================================================================================================
+// Bytes wanted in temp_buffer for these arguments (0 when none is needed)
+// replaces CLBlast{S,D,H}GemmTempBufferSize (reference: include/clblast_c.h:1412-1445, src/clblast_c.cpp:3011-3084)
+CLBlastStatusCode CLBLAST_HIP_API CLBlastSGemmTempBufferSize(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const size_t a_offset, const size_t a_ld, const size_t b_offset, const size_t b_ld,
+    const size_t c_offset, const size_t c_ld, hipStream_t* queue, size_t* temp_buffer_size);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastDGemmTempBufferSize(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const size_t a_offset, const size_t a_ld, const size_t b_offset, const size_t b_ld,
+    const size_t c_offset, const size_t c_ld, hipStream_t* queue, size_t* temp_buffer_size);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastHGemmTempBufferSize(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const size_t a_offset, const size_t a_ld, const size_t b_offset, const size_t b_ld,
+    const size_t c_offset, const size_t c_ld, hipStream_t* queue, size_t* temp_buffer_size);
+
+// =================================================================================================
+// replaces CLBlastClearCache (reference: include/clblast_c.h:1451, src/clblast_c.cpp:3089-3095)
+CLBlastStatusCode CLBLAST_HIP_API CLBlastClearCache(void);
+
+// replaces CLBlastOverrideParameters (reference: include/clblast_c.h:1461-1463, src/clblast_c.cpp:3109-3127);
+// `device` is a HIP device ordinal. Accepted: kernel_name "GemmRoutine", parameter
+// "XGEMM_MIN_INDIRECT_SIZE" (problems with m*n*k below its cube run the general direct kernel).
+CLBlastStatusCode CLBLAST_HIP_API CLBlastOverrideParameters(const int device, const char* kernel_name,
+                                                            const CLBlastPrecision precision,
+                                                            const size_t num_parameters,
+                                                            const char** parameters_names,
+                                                            const size_t* parameters_values);
+
+// Host fp16 conversions with the reference's semantics (reference: include/clblast_half.h:34-97 truncating
+// FloatToHalf, :101-347 HalfToFloat), exported for bindings that cannot include clblast_half.h.
+cl_half CLBLAST_HIP_API CLBlastFloatToHalf(const float value);
+float CLBLAST_HIP_API CLBlastHalfToFloat(const cl_half value);
+
+#ifdef __cplusplus
+}  // extern "C"
+#endif
+
+#endif  // CLBLAST_HIP_C_H_

@@ -1,0 +1,123 @@
+"""Parity of Gemm<T> through the C ABI against the CPU oracle, on a real MI355X.
+
+The sweep follows the reference's own (test/correctness/testblas.hpp:134-144: every dimension and leading
+dimension in {7, 64}, both layouts, all transposes; tester.cpp:346-353 offsets {0, 10}; tester.cpp:645-684
+alpha/beta in {0, 1, 3.14}), run once per kernel family (test/correctness/routines/level3/xgemm.cpp:15-30
+forces indirect and direct in turn). The bar is the relative Frobenius error versus the fp64 oracle:
+1e-5 (fp32), 1e-12 (fp64), 1e-2 (fp16), plus "nothing outside the logical C region changes".
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+from oracle import COL_MAJOR, CONJ, NO, ROW_MAJOR, YES
+
+pytestmark = pytest.mark.gpu
+
+LAYOUTS = (ROW_MAJOR, COL_MAJOR)
+TRANSPOSES = (NO, YES)
+BITS = (32, 64, 16)
+PATHS = ("direct", "indirect")
+
+
+@pytest.fixture(params=PATHS)
+def path(request):
+    return request.param
+
+
+@pytest.mark.parametrize("bits", BITS)
+def test_reference_sweep_dims_and_leading_dims(gpu, bits, path):
+    """m, n, k, lda, ldb, ldc in {7, 64} x layouts x transposes; invalid ld combinations must return the
+    reference's error code (and leave C alone), valid ones must match the oracle."""
+    gpu.force_path(bits, path)
+    try:
+        seed = 0
+        for layout, ta, tb in itertools.product(LAYOUTS, TRANSPOSES, TRANSPOSES):
+            for m, n, k, a_ld, b_ld, c_ld in itertools.product((7, 64), repeat=6):
+                seed += 1
+                problem = gpu.Problem(bits, layout, ta, tb, m, n, k, 3.14, 3.14, a_ld, b_ld, c_ld, seed=seed)
+                status, c_after = problem.run()
+                assert status == problem.expected_status(), problem.describe()
+                if status == 0:
+                    problem.check(c_after)
+                else:
+                    assert np.array_equal(c_after.view(np.uint8), problem.c.view(np.uint8))
+    finally:
+        gpu.force_path(bits, None)
+
+
+@pytest.mark.parametrize("bits", BITS)
+def test_reference_sweep_offsets_and_scalars(gpu, bits, path):
+    gpu.force_path(bits, path)
+    try:
+        seed = 1000
+        for layout, ta, tb in itertools.product(LAYOUTS, (NO, YES, CONJ), (NO, YES, CONJ)):
+            for offsets in ((0, 0, 0), (10, 10, 10), (3, 0, 17)):
+                for alpha, beta in itertools.product((0.0, 1.0, 3.14), repeat=2):
+                    seed += 1
+                    problem = gpu.Problem(bits, layout, ta, tb, 64, 7, 33, alpha, beta, a_offset=offsets[0],
+                                          b_offset=offsets[1], c_offset=offsets[2], seed=seed, extra_ld=(2, 0, 5))
+                    status, c_after = problem.run()
+                    assert status == 0, problem.describe()
+                    problem.check(c_after)
+    finally:
+        gpu.force_path(bits, None)
+
+
+@pytest.mark.parametrize("bits", BITS)
+def test_edge_tiles(gpu, bits, path):
+    """Ragged shapes around the tile sizes, odd offsets and padded leading dimensions."""
+    gpu.force_path(bits, path)
+    try:
+        seed = 5000
+        shapes = [(1, 1, 1), (15, 17, 3), (16, 16, 127), (17, 15, 129), (31, 33, 1), (33, 31, 64), (255, 257, 65),
+                  (257, 255, 31), (129, 2, 260), (2, 130, 259), (300, 200, 100)]
+        for (m, n, k), (ta, tb), layout in itertools.product(shapes, itertools.product(TRANSPOSES, TRANSPOSES),
+                                                            LAYOUTS):
+            seed += 1
+            extra = ((0, 0, 0), (1, 1, 1), (3, 5, 7))[seed % 3]
+            offsets = ((0, 0, 0), (1, 3, 5), (11, 13, 19))[(seed // 3) % 3]
+            problem = gpu.Problem(bits, layout, ta, tb, m, n, k, -0.75, 2.0, a_offset=offsets[0],
+                                  b_offset=offsets[1], c_offset=offsets[2], seed=seed, extra_ld=extra)
+            status, c_after = problem.run()
+            assert status == 0, problem.describe()
+            problem.check(c_after)
+    finally:
+        gpu.force_path(bits, None)
+
+
+@pytest.mark.parametrize("bits", BITS)
+def test_beta_zero_never_reads_c(gpu, bits, path):
+    """Reference kernels skip the C load when beta == 0 (xgemm_part2.opencl:84): NaN/Inf in C vanish."""
+    gpu.force_path(bits, path)
+    try:
+        problem = gpu.Problem(bits, COL_MAJOR, NO, NO, 70, 65, 40, 1.5, 0.0, seed=7)
+        index = __import__("oracle").c_indices(problem.layout, problem.m, problem.n, problem.c_offset, problem.c_ld)
+        problem.c[index.ravel()[::2]] = np.nan
+        problem.c[index.ravel()[1::2]] = np.inf
+        status, c_after = problem.run()
+        assert status == 0
+        assert np.all(np.isfinite(c_after[index]))
+        problem.check(c_after)
+    finally:
+        gpu.force_path(bits, None)
+
+
+@pytest.mark.parametrize("bits", BITS)
+def test_alpha_zero_is_not_special(gpu, bits, path):
+    """Unlike CBLAS, alpha == 0 still forms A*B, so a NaN in A reaches C (common.opencl:215-244: the
+    epilogue is alpha*acc + beta*C with no shortcut)."""
+    gpu.force_path(bits, path)
+    try:
+        problem = gpu.Problem(bits, COL_MAJOR, NO, NO, 40, 30, 20, 0.0, 1.0, seed=8)
+        problem.a[problem.a_offset + 3] = np.nan  # A(3, 0): poisons row 3 of the product
+        status, c_after = problem.run()
+        assert status == 0
+        index = __import__("oracle").c_indices(problem.layout, problem.m, problem.n, problem.c_offset, problem.c_ld)
+        got = c_after[index]
+        assert np.all(np.isnan(got[3, :]))
+        rest = np.delete(got, 3, axis=0)
+        assert np.array_equal(rest, np.delete(problem.c[index], 3, axis=0))
+    finally:
+        gpu.force_path(bits, None)
