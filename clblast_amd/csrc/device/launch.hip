@@ -10,6 +10,7 @@
 #include "clbh_device.h"
 #include "kernels/gemm_args.hpp"
 #include "kernels/gemm_general.hpp"
+#include "kernels/gemm_mfma.hpp"
 
 namespace clbh {
 namespace {
@@ -66,9 +67,79 @@ int LaunchGeneral(const clbh_gemm_desc& d, hipStream_t stream) {
   return static_cast<int>(hipGetLastError());
 }
 
+// ---- MFMA kernels (fp32, fp64) ----------------------------------------------------------------------
+// True when every 16-byte access of the tile loaders and of the epilogue is naturally aligned.
+template <typename T>
+bool Aligned16(const clbh_gemm_desc& d) {
+  constexpr long long VEC = 16 / sizeof(T);
+  const auto address = [](const void* base, long long offset) {
+    return reinterpret_cast<unsigned long long>(base) + static_cast<unsigned long long>(offset) * sizeof(T);
+  };
+  if (address(d.a, d.a_offset) % 16 || address(d.b, d.b_offset) % 16 || address(d.c, d.c_offset) % 16) { return false; }
+  if (d.a_ld % VEC || d.b_ld % VEC || d.c_ld % VEC) { return false; }
+  if (d.batch_count > 1) {
+    if (d.batch.alphas != nullptr) { return false; }  // per-batch offsets are only known on the device
+    if (d.a_stride % VEC || d.b_stride % VEC || d.c_stride % VEC) { return false; }
+  }
+  return true;
+}
+
+template <typename T, typename Config, bool A_KC, bool B_KC, bool ALIGNED>
+int LaunchMfmaVariant(const clbh_gemm_desc& d, hipStream_t stream) {
+  const auto args = MakeArgs<T>(d);
+  const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
+  const long long tiles_n = (d.n + Config::TILE_N - 1) / Config::TILE_N;
+  if (tiles_m * tiles_n > INT_MAX) { return hipErrorInvalidConfiguration; }
+  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
+  constexpr size_t lds_bytes = Config::LDS_ELEMS * sizeof(T);
+  auto kernel = GemmMfmaKernel<T, Config, A_KC, B_KC, ALIGNED>;
+  if (lds_bytes > 48 * 1024) {
+    static const hipError_t attribute_status = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+    if (attribute_status != hipSuccess) { return static_cast<int>(attribute_status); }
+  }
+  kernel<<<grid, dim3(kMfmaThreads), lds_bytes, stream>>>(args, static_cast<int>(tiles_m), static_cast<int>(tiles_n));
+  return static_cast<int>(hipGetLastError());
+}
+
+template <typename T, typename Config>
+int LaunchMfmaConfig(const clbh_gemm_desc& d, hipStream_t stream) {
+  const bool aligned = Aligned16<T>(d);
+  const int variant = (d.a_kcontig ? 4 : 0) | (d.b_kcontig ? 2 : 0) | (aligned ? 1 : 0);
+  switch (variant) {
+    case 0: return LaunchMfmaVariant<T, Config, false, false, false>(d, stream);
+    case 1: return LaunchMfmaVariant<T, Config, false, false, true>(d, stream);
+    case 2: return LaunchMfmaVariant<T, Config, false, true, false>(d, stream);
+    case 3: return LaunchMfmaVariant<T, Config, false, true, true>(d, stream);
+    case 4: return LaunchMfmaVariant<T, Config, true, false, false>(d, stream);
+    case 5: return LaunchMfmaVariant<T, Config, true, false, true>(d, stream);
+    case 6: return LaunchMfmaVariant<T, Config, true, true, false>(d, stream);
+    default: return LaunchMfmaVariant<T, Config, true, true, true>(d, stream);
+  }
+}
+
+template <typename T>
+int LaunchMfma(const clbh_gemm_desc& d, hipStream_t stream);
+
+template <>
+int LaunchMfma<float>(const clbh_gemm_desc& d, hipStream_t stream) {
+  return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16>>(d, stream);  // 128 x 128 x 16
+}
+
+template <>
+int LaunchMfma<double>(const clbh_gemm_desc& d, hipStream_t stream) {
+  return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 4, 8>>(d, stream);  // 128 x 128 x 8
+}
+
+template <>
+int LaunchMfma<_Float16>(const clbh_gemm_desc& d, hipStream_t stream) {
+  return LaunchGeneral<_Float16>(d, stream);
+}
+
 template <typename T>
 int LaunchTyped(const clbh_gemm_desc& d, hipStream_t stream) {
   switch (d.kernel_class) {
+    case CLBH_KERNEL_MFMA: return LaunchMfma<T>(d, stream);
     default: return LaunchGeneral<T>(d, stream);
   }
 }

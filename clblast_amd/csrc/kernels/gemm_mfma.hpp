@@ -1,0 +1,335 @@
+// =================================================================================================
+// Large-tile MFMA GEMM kernel for gfx950, fp32 and fp64. It stands where the reference has its
+// "indirect" path (src/routines/level3/xgemm.cpp:102-222 with the kernels of
+// src/kernels/level3/xgemm_part1-4.opencl, copy_pad/transpose_pad.opencl), but needs none of that
+// path's pre- and post-kernels: both operand orientations, arbitrary leading dimensions and offsets
+// and ragged edges are handled by the tile loaders and the epilogue of this one kernel.
+//
+// Structure (one work-group = 256 threads = 4 wavefronts):
+//   * the work-group owns a TILE_M x TILE_N block of C; K is walked in slabs of TILE_K;
+//   * global -> registers -> LDS staging with two LDS buffers, so that the loads of slab t+1 are in
+//     flight while slab t feeds the matrix cores, with one barrier per slab;
+//   * both operands sit in LDS as [k][x] (x = m for A, n for B; x contiguous) whatever their layout in
+//     memory: x-contiguous operands are copied with 16-byte loads and stores, k-contiguous ones are
+//     loaded with 16-byte loads along k and scattered into LDS (a transpose on the fly);
+//   * each wavefront computes a (MF*FM) x (MF*FN) block with v_mfma_f32_32x32x2_f32 (MF = 32) or
+//     v_mfma_f64_16x16x4_f64 (MF = 16). The n-indexed values are fed as the MFMA's A operand and the
+//     m-indexed ones as its B operand, so the lanes of a result register run along m: stores to the
+//     column-major C are contiguous per lane group. A lane owns FM consecutive m (one LDS read of
+//     FM elements, one vector store of FM elements);
+//   * the blockIdx -> tile mapping first makes the work-groups that the hardware deals round-robin to
+//     one XCD (blockIdx % 8) logically contiguous, then walks C in groups of GROUP_M tile rows, so
+//     the tiles in flight on one XCD share A and B panels in that XCD's L2.
+// =================================================================================================
+#ifndef CLBLAST_HIP_KERNELS_GEMM_MFMA_HPP_
+#define CLBLAST_HIP_KERNELS_GEMM_MFMA_HPP_
+
+#include "kernels/gemm_args.hpp"
+
+namespace clbh {
+
+constexpr int kMfmaThreads = 256;
+constexpr int kNumXcd = 8;
+
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef double double4_t __attribute__((ext_vector_type(4)));
+
+// ---- per-precision MFMA traits ---------------------------------------------------------------------
+template <typename T> struct MfmaTraits;
+
+template <> struct MfmaTraits<float> {
+  static constexpr int MF = 32;       // the instruction computes an MF x MF block
+  static constexpr int KP = 2;        // k extent of one instruction
+  static constexpr int ACC = 16;      // accumulator elements per lane and block
+  using Acc = float16_t;
+  static __device__ __forceinline__ Acc Zero() { return Acc(0.0f); }
+  static __device__ __forceinline__ Acc Mfma(const float rows, const float cols, const Acc acc) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(rows, cols, acc, 0, 0, 0);
+  }
+  // row of the MF x MF block held by accumulator element r of a lane in k-group g
+  static __device__ __forceinline__ int Row(const int r, const int g) { return 8 * (r / 4) + 4 * g + (r % 4); }
+};
+
+template <> struct MfmaTraits<double> {
+  static constexpr int MF = 16;
+  static constexpr int KP = 4;
+  static constexpr int ACC = 4;
+  using Acc = double4_t;
+  static __device__ __forceinline__ Acc Zero() { return Acc(0.0); }
+  static __device__ __forceinline__ Acc Mfma(const double rows, const double cols, const Acc acc) {
+    return __builtin_amdgcn_mfma_f64_16x16x4f64(rows, cols, acc, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int Row(const int r, const int g) { return 4 * r + g; }
+};
+
+// ---- tile configuration ----------------------------------------------------------------------------
+// WM x WN wavefronts per work-group (WM * WN == 4), each owning FM x FN MFMA blocks.
+template <typename T, int WM_, int WN_, int FM_, int FN_, int TILE_K_>
+struct MfmaConfig {
+  using Traits = MfmaTraits<T>;
+  static constexpr int WM = WM_, WN = WN_, FM = FM_, FN = FN_;
+  static constexpr int TILE_M = WM * FM * Traits::MF;
+  static constexpr int TILE_N = WN * FN * Traits::MF;
+  static constexpr int TILE_K = TILE_K_;
+  static constexpr int VEC = 16 / sizeof(T);  // elements per 16-byte access
+  // Row pitch of the LDS tiles in elements. pitch % (64 / VEC... ) is chosen so that the scattered
+  // 4-byte (fp32) or 8-byte (fp64) stores of the k-contiguous loader fall into distinct banks: the 64
+  // lanes of a wavefront write (TILE_K / VEC) different k rows, which must be (64 * 4 / sizeof(T)) /
+  // (TILE_K / VEC) elements apart modulo the bank window.
+  static constexpr int PAD = VEC;
+  static constexpr int PITCH_M = TILE_M + PAD;
+  static constexpr int PITCH_N = TILE_N + PAD;
+  static constexpr int LDS_ELEMS = 2 * TILE_K * (PITCH_M + PITCH_N);  // two buffers
+  static constexpr int CHUNKS_A = TILE_M * TILE_K / VEC / kMfmaThreads;  // 16-byte chunks per thread and slab
+  static constexpr int CHUNKS_B = TILE_N * TILE_K / VEC / kMfmaThreads;
+  static_assert(WM * WN * 64 == kMfmaThreads, "four wavefronts per work-group");
+  static_assert(TILE_M * TILE_K % (VEC * kMfmaThreads) == 0 && TILE_N * TILE_K % (VEC * kMfmaThreads) == 0,
+                "slab must divide evenly over the threads");
+  static_assert(TILE_K % Traits::KP == 0 && TILE_K % VEC == 0, "slab depth");
+};
+
+// Vector types for LDS and global accesses; never assumed to be aligned beyond 16 bytes.
+template <typename T, int N> struct VecType { typedef T type __attribute__((ext_vector_type(N), aligned(N * sizeof(T) < 16 ? N * sizeof(T) : 16))); };
+template <typename T> struct VecType<T, 1> { typedef T type; };
+
+template <typename V, typename T, int N>
+__device__ __forceinline__ T VecGet(const V v, const int i) {
+  if constexpr (N == 1) { return v; } else { return v[i]; }
+}
+template <typename V, typename T, int N>
+__device__ __forceinline__ V VecWith(V v, const int i, const T value) {
+  if constexpr (N == 1) { v = value; } else { v[i] = value; }
+  return v;
+}
+
+// ---- slab loaders ----------------------------------------------------------------------------------
+// One operand slab is TILE_X x TILE_K elements. `base` points at element (x = 0, k = 0) of the matrix of
+// this batch; the element (x, k) lives at base[KC ? x*ld + k : k*ld + x]. Every thread moves PIECES
+// pieces of VL elements (VL = 16 bytes' worth when every address is 16-byte aligned, else 1). The
+// piece -> (x, k) mapping puts consecutive threads along the contiguous index of the operand in
+// memory, so a wavefront's accesses coalesce for either orientation.
+template <int TILE_X, int TILE_K, int VL, bool KC>
+struct PieceMap {
+  static constexpr int ALONG = (KC ? TILE_K : TILE_X) / VL;  // pieces per contiguous line of the slab
+  static __device__ __forceinline__ void Get(const int piece, int& x, int& k) {
+    const int line = piece / ALONG, pos = (piece % ALONG) * VL;
+    x = KC ? line : pos;
+    k = KC ? pos : line;
+  }
+};
+
+// Fast path: the whole slab is inside the matrix.
+template <typename T, int TILE_X, int TILE_K, int PIECES, int VL, bool KC>
+__device__ __forceinline__ void LoadSlab(const T* __restrict__ base, const long long ld, const int x0, const int k0,
+                                         const int tid, T (&regs)[PIECES][VL]) {
+  using Map = PieceMap<TILE_X, TILE_K, VL, KC>;
+  using V = typename VecType<T, VL>::type;
+#pragma unroll
+  for (int c = 0; c < PIECES; ++c) {
+    int x, k;
+    Map::Get(tid + c * kMfmaThreads, x, k);
+    const T* src = KC ? base + (x0 + x) * ld + (k0 + k) : base + (k0 + k) * ld + (x0 + x);
+    const V v = *reinterpret_cast<const V*>(src);
+#pragma unroll
+    for (int e = 0; e < VL; ++e) { regs[c][e] = VecGet<V, T, VL>(v, e); }
+  }
+}
+
+// Checked path for edge tiles and the K tail: elements outside the matrix read as zero.
+template <typename T, int TILE_X, int TILE_K, int PIECES, int VL, bool KC>
+__device__ __forceinline__ void LoadSlabChecked(const T* __restrict__ base, const long long ld, const int x0,
+                                                const int k0, const int x_end, const int k_end, const int tid,
+                                                T (&regs)[PIECES][VL]) {
+  using Map = PieceMap<TILE_X, TILE_K, VL, KC>;
+#pragma unroll
+  for (int c = 0; c < PIECES; ++c) {
+    int x, k;
+    Map::Get(tid + c * kMfmaThreads, x, k);
+#pragma unroll
+    for (int e = 0; e < VL; ++e) {
+      const int gx = x0 + x + (KC ? 0 : e), gk = k0 + k + (KC ? e : 0);
+      T value = T(0);
+      if (gx < x_end && gk < k_end) { value = KC ? base[gx * ld + gk] : base[gk * ld + gx]; }
+      regs[c][e] = value;
+    }
+  }
+}
+
+// Registers -> LDS tile [k][x] with row pitch PITCH.
+template <typename T, int TILE_X, int TILE_K, int PITCH, int PIECES, int VL, bool KC>
+__device__ __forceinline__ void StoreSlab(T* __restrict__ tile, const int tid, const T (&regs)[PIECES][VL]) {
+  using Map = PieceMap<TILE_X, TILE_K, VL, KC>;
+  using V = typename VecType<T, VL>::type;
+#pragma unroll
+  for (int c = 0; c < PIECES; ++c) {
+    int x, k;
+    Map::Get(tid + c * kMfmaThreads, x, k);
+    if (KC) {
+#pragma unroll
+      for (int e = 0; e < VL; ++e) { tile[(k + e) * PITCH + x] = regs[c][e]; }
+    } else {
+      V v;
+#pragma unroll
+      for (int e = 0; e < VL; ++e) { v = VecWith<V, T, VL>(v, e, regs[c][e]); }
+      *reinterpret_cast<V*>(&tile[k * PITCH + x]) = v;
+    }
+  }
+}
+
+// ---- blockIdx -> tile ------------------------------------------------------------------------------
+__device__ __forceinline__ void TileOfBlock(const int block, const int num_blocks, const int tiles_m,
+                                            const int tiles_n, int& tile_m, int& tile_n) {
+  // (1) work-groups are dealt to the XCDs round-robin: give each XCD a contiguous logical range
+  const int per_xcd = (num_blocks + kNumXcd - 1) / kNumXcd;
+  const int remainder = num_blocks % kNumXcd;
+  const int tall = (remainder == 0) ? kNumXcd : remainder;  // XCDs that own per_xcd blocks
+  const int xcd = block % kNumXcd, local = block / kNumXcd;
+  const int logical = (xcd < tall) ? xcd * per_xcd + local
+                                   : tall * per_xcd + (xcd - tall) * (per_xcd - 1) + local;
+  // (2) grouped walk: GROUP_M tile rows at a time, column by column inside a group
+  constexpr int GROUP_M = 8;
+  const int in_group = GROUP_M * tiles_n;
+  const int group = logical / in_group;
+  const int first_m = group * GROUP_M;
+  const int group_rows = min(tiles_m - first_m, GROUP_M);
+  tile_m = first_m + (logical % in_group) % group_rows;
+  tile_n = (logical % in_group) / group_rows;
+}
+
+// ---- the kernel ------------------------------------------------------------------------------------
+template <typename T, typename Config, bool A_KC, bool B_KC, bool ALIGNED>
+__global__ __launch_bounds__(kMfmaThreads) void GemmMfmaKernel(const GemmArgs<T> p, const int tiles_m,
+                                                               const int tiles_n) {
+  using Traits = typename Config::Traits;
+  using Acc = typename Traits::Acc;
+  constexpr int MF = Traits::MF, KP = Traits::KP, ACC = Traits::ACC;
+  constexpr int TILE_M = Config::TILE_M, TILE_N = Config::TILE_N, TILE_K = Config::TILE_K;
+  constexpr int FM = Config::FM, FN = Config::FN, VEC = Config::VEC;
+  constexpr int PITCH_M = Config::PITCH_M, PITCH_N = Config::PITCH_N;
+  constexpr int VL = ALIGNED ? VEC : 1;  // elements per global access
+  constexpr int PIECES_A = Config::CHUNKS_A * VEC / VL, PIECES_B = Config::CHUNKS_B * VEC / VL;
+  using VM = typename VecType<T, FM>::type;
+  using VN = typename VecType<T, FN>::type;
+
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+  T* a_tiles = lds;                             // [2][TILE_K][PITCH_M]
+  T* b_tiles = lds + 2 * TILE_K * PITCH_M;      // [2][TILE_K][PITCH_N]
+
+  const int tid = threadIdx.x;
+  const int lane = tid % 64, wave = tid / 64;
+  const int wave_m = wave % Config::WM, wave_n = wave / Config::WM;
+  const int lane_x = lane % MF;  // position along the lane dimension of the MFMA block
+  const int lane_g = lane / MF;  // k-group of the lane inside one instruction
+
+  int tile_m, tile_n;
+  TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
+  const bool interior = (m0 + TILE_M <= p.m) && (n0 + TILE_N <= p.n);
+  const int full_slabs = p.k / TILE_K;
+  const int slabs = (p.k + TILE_K - 1) / TILE_K;
+
+  // LDS read offsets of this lane: FM consecutive m and FN consecutive n per k row
+  const int a_read = wave_m * (FM * MF) + lane_x * FM;
+  const int b_read = wave_n * (FN * MF) + lane_x * FN;
+
+  for (int batch = blockIdx.y; batch < p.batch_count; batch += gridDim.y) {
+    const T* a;
+    const T* b;
+    T* c;
+    T alpha, beta;
+    ResolveBatch<T, T>(p, batch, a, b, c, alpha, beta);
+
+    Acc acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+#pragma unroll
+      for (int j = 0; j < FN; ++j) { acc[i][j] = Traits::Zero(); }
+    }
+
+    T a_regs[PIECES_A][VL];
+    T b_regs[PIECES_B][VL];
+
+    auto load = [&](const int slab) {
+      const int k0 = slab * TILE_K;
+      if (interior && slab < full_slabs) {
+        LoadSlab<T, TILE_M, TILE_K, PIECES_A, VL, A_KC>(a, p.a_ld, m0, k0, tid, a_regs);
+        LoadSlab<T, TILE_N, TILE_K, PIECES_B, VL, B_KC>(b, p.b_ld, n0, k0, tid, b_regs);
+      } else {
+        LoadSlabChecked<T, TILE_M, TILE_K, PIECES_A, VL, A_KC>(a, p.a_ld, m0, k0, p.m, p.k, tid, a_regs);
+        LoadSlabChecked<T, TILE_N, TILE_K, PIECES_B, VL, B_KC>(b, p.b_ld, n0, k0, p.n, p.k, tid, b_regs);
+      }
+    };
+    auto store = [&](const int buffer) {
+      StoreSlab<T, TILE_M, TILE_K, PITCH_M, PIECES_A, VL, A_KC>(a_tiles + buffer * TILE_K * PITCH_M, tid, a_regs);
+      StoreSlab<T, TILE_N, TILE_K, PITCH_N, PIECES_B, VL, B_KC>(b_tiles + buffer * TILE_K * PITCH_N, tid, b_regs);
+    };
+
+    load(0);
+    store(0);
+    __syncthreads();
+
+    for (int slab = 0; slab < slabs; ++slab) {
+      const int buffer = slab & 1;
+      if (slab + 1 < slabs) { load(slab + 1); }
+
+      const T* a_tile = a_tiles + buffer * TILE_K * PITCH_M + a_read;
+      const T* b_tile = b_tiles + buffer * TILE_K * PITCH_N + b_read;
+#pragma unroll
+      for (int ks = 0; ks < TILE_K / KP; ++ks) {
+        const int k = ks * KP + lane_g;
+        const VM av = *reinterpret_cast<const VM*>(&a_tile[k * PITCH_M]);
+        const VN bv = *reinterpret_cast<const VN*>(&b_tile[k * PITCH_N]);
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+#pragma unroll
+          for (int j = 0; j < FN; ++j) {
+            acc[i][j] = Traits::Mfma(VecGet<VN, T, FN>(bv, j), VecGet<VM, T, FM>(av, i), acc[i][j]);
+          }
+        }
+      }
+
+      if (slab + 1 < slabs) { store(buffer ^ 1); }
+      __syncthreads();
+    }
+
+    // Epilogue. Lane owns m = m_base + i (i < FM); accumulator element r of block (i, j) is the
+    // column n = n_base + FN * Row(r) + j.
+    const int m_base = m0 + a_read;
+    const int n_base = n0 + wave_n * (FN * MF);
+    const bool vector_store = ALIGNED && (FM > 1) && (m_base + FM <= p.m);
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+#pragma unroll
+      for (int r = 0; r < ACC; ++r) {
+        const int n = n_base + FN * Traits::Row(r, lane_g) + j;
+        if (n >= p.n) { continue; }
+        T* dst = c + n * p.c_ld + m_base;
+        if (vector_store) {
+          VM out;
+          if (beta == T(0)) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i) { out = VecWith<VM, T, FM>(out, i, alpha * acc[i][j][r]); }
+          } else {
+            const VM old = *reinterpret_cast<const VM*>(dst);
+#pragma unroll
+            for (int i = 0; i < FM; ++i) {
+              out = VecWith<VM, T, FM>(out, i, alpha * acc[i][j][r] + beta * VecGet<VM, T, FM>(old, i));
+            }
+          }
+          *reinterpret_cast<VM*>(dst) = out;
+        } else {
+#pragma unroll
+          for (int i = 0; i < FM; ++i) {
+            if (m_base + i < p.m) { StoreResult<T, T>(dst, i, acc[i][j][r], alpha, beta); }
+          }
+        }
+      }
+    }
+    __syncthreads();  // the next batch reuses the LDS buffers
+  }
+}
+
+}  // namespace clbh
+
+#endif  // CLBLAST_HIP_KERNELS_GEMM_MFMA_HPP_
