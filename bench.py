@@ -1,0 +1,278 @@
+#!/usr/bin/env python3
+"""Benchmark of the GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+A "step" is one GEMM call through the C ABI of libclblast_hip.so on operands that are already resident in
+HBM. The headline workload is BASELINE.json configs[1], fp32 variant: SGEMM, row-major, A transposed, B
+not, m = n = k = 8192, leading dimensions 8192, alpha = 1, beta = 0, inputs uniform[-1, 1) from a fixed
+seed. The script prints ONE JSON line: whole-job GFLOPS (2*m*n*k per step), the roofline of the dominant
+kernel measured with events on the launch stream, a CPU baseline on the host cores (the reference's
+indirect path restated in C, from oracle/), and - unless --no-extras - the other BASELINE configs
+(DGEMM and HGEMM 8192^3, SGEMM 1024^3, strided-batched 8192 x 32^3, the irregular shapes) as extra entries.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+ROW, COL, NO, YES = 101, 102, 111, 112
+# MI355X datasheet peaks (dense): TFLOP/s per storage type, HBM3E TB/s
+PEAK_TFLOPS = {"S": 157.3, "D": 78.6, "H": 2516.6}
+PEAK_HBM_GBS = 8000.0
+BITS = {"S": 32, "D": 64, "H": 16}
+DTYPE_NAME = {"S": "f32", "D": "f64", "H": "f16"}
+
+
+def parse_args():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=20)
+    parser.add_argument("--warmup", type=int, default=3)
+    parser.add_argument("--no-extras", action="store_true", help="only the headline workload")
+    parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    parser.add_argument("--only", default=None, help="run a single extra workload by name and exit (for profiling)")
+    return parser.parse_args()
+
+
+class Workload:
+    """One GEMM configuration with device-resident operands."""
+
+    def __init__(self, name, prefix, layout, ta, tb, m, n, k, alpha, beta, lda=None, ldb=None, ldc=None, offsets=(0, 0, 0),
+                 batch=1, ab_range=(-1.0, 1.0), c_range=(-1.0, 1.0), seed=2024):
+        import torch
+        self.name, self.prefix, self.layout, self.ta, self.tb = name, prefix, layout, ta, tb
+        self.m, self.n, self.k, self.alpha, self.beta, self.batch = m, n, k, alpha, beta, batch
+        col = (layout == COL)
+        a_rot = (col and ta != NO) or (not col and ta == NO)
+        b_rot = (col and tb != NO) or (not col and tb == NO)
+        self.a_one, self.a_two = (k, m) if a_rot else (m, k)
+        self.b_one, self.b_two = (n, k) if b_rot else (k, n)
+        self.c_one, self.c_two = (n, m) if not col else (m, n)
+        self.lda = self.a_one if lda is None else lda
+        self.ldb = self.b_one if ldb is None else ldb
+        self.ldc = self.c_one if ldc is None else ldc
+        self.offsets = offsets
+        self.a_stride, self.b_stride, self.c_stride = self.lda * self.a_two, self.ldb * self.b_two, self.ldc * self.c_two
+        dtype = {"S": torch.float32, "D": torch.float64, "H": torch.float16}[prefix]
+        generator = torch.Generator(device="cuda")
+        generator.manual_seed(seed)
+
+        def make(count, low, high):
+            values = torch.rand(count, device="cuda", dtype=torch.float64 if prefix == "D" else torch.float32,
+                                generator=generator)
+            return (values * (high - low) + low).to(dtype)
+
+        self.a = make(self.a_stride * batch + offsets[0], *ab_range)
+        self.b = make(self.b_stride * batch + offsets[1], *ab_range)
+        self.c = make(self.c_stride * batch + offsets[2], *c_range)
+        self.c_initial = self.c.clone() if beta != 0 else None
+
+    @property
+    def flops(self):
+        return 2.0 * self.m * self.n * self.k * self.batch
+
+    @property
+    def algorithmic_bytes(self):
+        """Bytes a perfect implementation moves: A and B read once, C written once (and read when beta != 0)."""
+        element = BITS[self.prefix] // 8
+        c_passes = 2 if self.beta != 0 else 1
+        return element * self.batch * (self.m * self.k + self.k * self.n + c_passes * self.m * self.n)
+
+    def call(self, stream_handle):
+        from clblast_amd.api import raw_gemm, raw_gemm_strided_batched
+        if self.batch == 1:
+            status = raw_gemm(self.prefix, self.layout, self.ta, self.tb, self.m, self.n, self.k, self.alpha,
+                              self.a.data_ptr(), self.offsets[0], self.lda, self.b.data_ptr(), self.offsets[1], self.ldb,
+                              self.beta, self.c.data_ptr(), self.offsets[2], self.ldc, stream_handle)
+        else:
+            status = raw_gemm_strided_batched(self.prefix, self.layout, self.ta, self.tb, self.m, self.n, self.k,
+                                              self.alpha, self.a.data_ptr(), self.offsets[0], self.lda, self.a_stride,
+                                              self.b.data_ptr(), self.offsets[1], self.ldb, self.b_stride, self.beta,
+                                              self.c.data_ptr(), self.offsets[2], self.ldc, self.c_stride, self.batch,
+                                              stream_handle)
+        if status != 0:
+            raise RuntimeError("%s: status %d" % (self.name, status))
+
+    def logical(self, which):
+        """op(A) (m x k), op(B) (k x n) or C (m x n) of batch 0 as strided views of the device buffers."""
+        import torch
+        buffer, offset, ld, rows, cols, rotated = {
+            "a": (self.a, self.offsets[0], self.lda, self.m, self.k, self._a_rot()),
+            "b": (self.b, self.offsets[1], self.ldb, self.k, self.n, self._b_rot()),
+            "c": (self.c, self.offsets[2], self.ldc, self.m, self.n, self.layout == ROW),
+        }[which]
+        strides = (ld, 1) if rotated else (1, ld)
+        return torch.as_strided(buffer, (rows, cols), strides, offset)
+
+    def _a_rot(self):
+        col = (self.layout == COL)
+        return (col and self.ta != NO) or (not col and self.ta == NO)
+
+    def _b_rot(self):
+        col = (self.layout == COL)
+        return (col and self.tb != NO) or (not col and self.tb == NO)
+
+    def freivalds_error(self):
+        """||C x - (alpha op(A) (op(B) x) + beta C0 x)|| / ||...|| in fp64 on the GPU for a random x: an
+        O(n^2) check that the timed output is a GEMM result (batch 0)."""
+        import torch
+        x = torch.rand(self.n, 1, device="cuda", dtype=torch.float64) - 0.5
+        a, b, c = self.logical("a").double(), self.logical("b").double(), self.logical("c").double()
+        expected = self.alpha * (a @ (b @ x))
+        if self.beta != 0:
+            c0 = torch.as_strided(self.c_initial, c.shape, self.logical("c").stride(), self.offsets[2]).double()
+            expected = expected + self.beta * (c0 @ x)
+        return float(((c @ x) - expected).norm() / expected.norm())
+
+
+def time_workload(workload, steps, warmup):
+    """Returns (wall seconds for `steps` calls, average device milliseconds per call from stream events)."""
+    import torch
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(warmup):
+            workload.call(stream.cuda_stream)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        wall_start = time.perf_counter()
+        start.record(stream)
+        for _ in range(steps):
+            workload.call(stream.cuda_stream)
+        stop.record(stream)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - wall_start
+    return wall, start.elapsed_time(stop) / steps
+
+
+def verified_error(workload):
+    """One fresh call on the initial C, then the Freivalds check."""
+    import torch
+    if workload.c_initial is not None:
+        workload.c.copy_(workload.c_initial)
+    workload.call(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return workload.freivalds_error()
+
+
+def roofline_of(workload, device_ms):
+    seconds = device_ms * 1e-3
+    intensity = workload.flops / workload.algorithmic_bytes
+    ridge = PEAK_TFLOPS[workload.prefix] * 1e12 / (PEAK_HBM_GBS * 1e9)
+    if intensity >= ridge:
+        achieved = workload.flops / seconds / 1e12
+        peak = PEAK_TFLOPS[workload.prefix]
+        return {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(achieved / peak, 4), "traffic": None}
+    achieved = workload.algorithmic_bytes / seconds / 1e9
+    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": None}
+
+
+def cpu_baseline(target_seconds=15.0):
+    """The reference's indirect path restated on the CPU (oracle/gemm_oracle.c: xgemm_port_f32), timed on a
+    row slab of the headline problem sized to take about `target_seconds` on this host."""
+    import numpy as np
+    import oracle
+    n = k = 8192
+    threads = oracle.num_threads()
+
+    def run(m):
+        # row-major, A transposed: A is stored k x m, B k x n, C m x n
+        a = oracle.uniform(1, k * m, -1.0, 1.0, 32)
+        b = oracle.uniform(2, k * n, -1.0, 1.0, 32)
+        c = np.zeros(m * n, dtype=np.float32)
+        begin = time.perf_counter()
+        oracle.xgemm_port(ROW, YES, NO, m, n, k, 1.0, a, 0, m, b, 0, n, 0.0, c, 0, n)
+        return time.perf_counter() - begin
+
+    probe_m = 256
+    probe_seconds = run(probe_m)
+    rate = 2.0 * probe_m * n * k / probe_seconds
+    m = int(min(8192, max(256, (rate * target_seconds / (2.0 * n * k)) // 256 * 256)))
+    seconds = run(m) if m != probe_m else probe_seconds
+    return {"value": round(2.0 * m * n * k / seconds / 1e9, 1), "unit": "GFLOPS", "cores": threads, "kind": "port",
+            "sample": "rows 0..%d of C of the same SGEMM (m=%d, n=k=8192, row-major, A^T): %.1f s; CPU restatement "
+                      "of the reference's Xgemm indirect path with its default 32x32x32 tiles, OpenMP over tiles, not "
+                      "CLBlast on PoCL (no CPU OpenCL device on this host)" % (m - 1, m, seconds)}
+
+
+EXTRA_WORKLOADS = {
+    "cfg1_sgemm_1024_colNN": lambda: Workload("cfg1", "S", COL, NO, NO, 1024, 1024, 1024, 1.5, 0.5),
+    "cfg2_dgemm_8192_rowTN": lambda: Workload("cfg2d", "D", ROW, YES, NO, 8192, 8192, 8192, 1.0, 0.0),
+    "cfg3_hgemm_8192_colNT": lambda: Workload("cfg3", "H", COL, NO, YES, 8192, 8192, 8192, 1.0, 1.0,
+                                               ab_range=(-0.5, 0.5)),
+    "cfg4_sgemm_strided_batched_8192x32": lambda: Workload("cfg4", "S", COL, NO, NO, 32, 32, 32, 1.0, 0.0, batch=8192),
+    "cfg5_sgemm_1000_colNN": lambda: Workload("cfg5a", "S", COL, NO, NO, 1000, 1000, 1000, -0.75, 2.0, 1003, 1005, 1007,
+                                               (11, 13, 19)),
+    "cfg5_sgemm_4099x17x4096_colNN": lambda: Workload("cfg5b", "S", COL, NO, NO, 4099, 17, 4096, -0.75, 2.0, 4102, 4101,
+                                                       4106, (11, 13, 19)),
+    "cfg5_sgemm_17x4099x4096_colNN": lambda: Workload("cfg5c", "S", COL, NO, NO, 17, 4099, 4096, -0.75, 2.0, 20, 4101,
+                                                       24, (11, 13, 19)),
+    "cfg5_sgemm_8191x8191x127_colNN": lambda: Workload("cfg5d", "S", COL, NO, NO, 8191, 8191, 127, -0.75, 2.0, 8194,
+                                                        132, 8198, (11, 13, 19)),
+}
+
+
+def run_extra(name, steps, warmup):
+    import torch
+    workload = EXTRA_WORKLOADS[name]()
+    error = verified_error(workload)
+    _, device_ms = time_workload(workload, steps, warmup)
+    roofline = roofline_of(workload, device_ms)
+    entry = {"ms": round(device_ms, 4), "gflops": round(workload.flops / (device_ms * 1e-3) / 1e9, 1),
+             "gbs": round(workload.algorithmic_bytes / (device_ms * 1e-3) / 1e9, 1), "dtype": DTYPE_NAME[workload.prefix],
+             "frac_of_peak": round(workload.flops / (device_ms * 1e-3) / 1e12 / PEAK_TFLOPS[workload.prefix], 4),
+             "roofline": roofline, "freivalds_rel_error": float("%.3g" % error)}
+    del workload
+    torch.cuda.empty_cache()
+    return entry
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (every box has one MI355X); --gpus %d is not run" % args.gpus)
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    from clblast_amd import _lib
+    _lib.load()  # fails loudly when the HIP library is missing: there is no fallback
+
+    if args.only is not None:
+        print(json.dumps({args.only: run_extra(args.only, args.steps, args.warmup)}))
+        return
+
+    headline = Workload("cfg2s", "S", ROW, YES, NO, 8192, 8192, 8192, 1.0, 0.0)
+    error = verified_error(headline)
+    wall, device_ms = time_workload(headline, args.steps, args.warmup)
+    gflops = headline.flops * args.steps / wall / 1e9
+    result = {
+        "metric": "SGEMM 8192^3 GFLOPS (2*m*n*k/s)", "value": round(gflops, 1), "unit": "GFLOPS", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall / args.steps * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1] fp32: SGEMM row-major, A transposed, B not, m=n=k=8192, "
+                               "lda=ldb=ldc=8192, alpha=1, beta=0, uniform[-1,1) seed 2024; inputs resident in HBM",
+                   "api": "CLBlastSgemm via the C ABI", "frac_of_fp32_peak": round(gflops / 1e3 / PEAK_TFLOPS["S"], 4)},
+        "freivalds_rel_error": float("%.3g" % error),
+        "roofline": roofline_of(headline, device_ms),
+    }
+    del headline
+    torch.cuda.empty_cache()
+    if not args.no_extras:
+        extras = {}
+        for name in EXTRA_WORKLOADS:
+            extras[name] = run_extra(name, max(3, args.steps // 2), args.warmup)
+        result["other_configs"] = extras
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
