@@ -11,6 +11,7 @@
 #include "kernels/gemm_args.hpp"
 #include "kernels/gemm_general.hpp"
 #include "kernels/gemm_mfma.hpp"
+#include "kernels/gemm_mfma_f16.hpp"
 
 namespace clbh {
 namespace {
@@ -123,17 +124,65 @@ int LaunchMfma(const clbh_gemm_desc& d, hipStream_t stream);
 
 template <>
 int LaunchMfma<float>(const clbh_gemm_desc& d, hipStream_t stream) {
-  return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16>>(d, stream);  // 128 x 128 x 16
+  switch (d.tile_variant) {
+    case 1: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16, 3>>(d, stream);
+    case 2: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16, 4>>(d, stream);
+    case 3: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 4, 2, 16, 2>>(d, stream);  // 256 x 128 x 16
+    case 4: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 32, 2>>(d, stream);  // 128 x 128 x 32
+    default: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16, 2>>(d, stream);  // 128 x 128 x 16
+  }
 }
 
 template <>
 int LaunchMfma<double>(const clbh_gemm_desc& d, hipStream_t stream) {
-  return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 4, 8>>(d, stream);  // 128 x 128 x 8
+  switch (d.tile_variant) {
+    case 1: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 2, 8, 2>>(d, stream);   // 128 x 64 x 8
+    case 2: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 2, 16, 2>>(d, stream);  // 128 x 64 x 16
+    case 3: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 2, 16, 3>>(d, stream);  // 128 x 64 x 16
+    case 4: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 4, 16, 2>>(d, stream);  // 128 x 128 x 16
+    default: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 4, 8, 2>>(d, stream);  // 128 x 128 x 8
+  }
+}
+
+// ---- MFMA kernel, fp16 ---------------------------------------------------------------------------
+template <typename Config, bool A_KC, bool B_KC, bool ALIGNED>
+int LaunchHgemmVariant(const clbh_gemm_desc& d, hipStream_t stream) {
+  const auto args = MakeArgs<float>(d);
+  const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
+  const long long tiles_n = (d.n + Config::TILE_N - 1) / Config::TILE_N;
+  if (tiles_m * tiles_n > INT_MAX) { return hipErrorInvalidConfiguration; }
+  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
+  constexpr size_t lds_bytes = Config::LDS_BYTES;
+  auto kernel = HgemmMfmaKernel<Config, A_KC, B_KC, ALIGNED>;
+  if (lds_bytes > 48 * 1024) {
+    static const hipError_t attribute_status = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+    if (attribute_status != hipSuccess) { return static_cast<int>(attribute_status); }
+  }
+  kernel<<<grid, dim3(kMfmaThreads), lds_bytes, stream>>>(args, static_cast<int>(tiles_m), static_cast<int>(tiles_n));
+  return static_cast<int>(hipGetLastError());
+}
+
+template <typename Config, bool ALIGNED>
+int LaunchHgemmConfig(const clbh_gemm_desc& d, hipStream_t stream) {
+  const int variant = (d.a_kcontig ? 2 : 0) | (d.b_kcontig ? 1 : 0);
+  switch (variant) {
+    case 0: return LaunchHgemmVariant<Config, false, false, ALIGNED>(d, stream);
+    case 1: return LaunchHgemmVariant<Config, false, true, ALIGNED>(d, stream);
+    case 2: return LaunchHgemmVariant<Config, true, false, ALIGNED>(d, stream);
+    default: return LaunchHgemmVariant<Config, true, true, ALIGNED>(d, stream);
+  }
 }
 
 template <>
 int LaunchMfma<_Float16>(const clbh_gemm_desc& d, hipStream_t stream) {
-  return LaunchGeneral<_Float16>(d, stream);
+  // The 256 x 256 tiles exist for 16-byte aligned operands only; everything else takes 128 x 128.
+  if (!Aligned16<_Float16>(d)) { return LaunchHgemmConfig<HgemmConfig<2, 2, 32>, false>(d, stream); }
+  switch (d.tile_variant) {
+    case 1: return LaunchHgemmConfig<HgemmConfig<4, 4, 32>, true>(d, stream);   // 256 x 256 x 32
+    case 2: return LaunchHgemmConfig<HgemmConfig<4, 4, 64>, true>(d, stream);   // 256 x 256 x 64
+    default: return LaunchHgemmConfig<HgemmConfig<2, 2, 32>, true>(d, stream);  // 128 x 128 x 32
+  }
 }
 
 template <typename T>

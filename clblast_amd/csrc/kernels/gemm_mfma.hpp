@@ -64,8 +64,9 @@ template <> struct MfmaTraits<double> {
 
 // ---- tile configuration ----------------------------------------------------------------------------
 // WM x WN wavefronts per work-group (WM * WN == 4), each owning FM x FN MFMA blocks.
-template <typename T, int WM_, int WN_, int FM_, int FN_, int TILE_K_>
+template <typename T, int WM_, int WN_, int FM_, int FN_, int TILE_K_, int MIN_WAVES_ = 2>
 struct MfmaConfig {
+  static constexpr int MIN_WAVES = MIN_WAVES_;  // wavefronts per SIMD the register budget must allow
   using Traits = MfmaTraits<T>;
   static constexpr int WM = WM_, WN = WN_, FM = FM_, FN = FN_;
   static constexpr int TILE_M = WM * FM * Traits::MF;
@@ -135,23 +136,21 @@ __device__ __forceinline__ void LoadSlab(const T* __restrict__ base, const long 
   }
 }
 
-// Checked path for edge tiles and the K tail: elements outside the matrix read as zero.
-template <typename T, int TILE_X, int TILE_K, int PIECES, int VL, bool KC>
-__device__ __forceinline__ void LoadSlabChecked(const T* __restrict__ base, const long long ld, const int x0,
-                                                const int k0, const int x_end, const int k_end, const int tid,
-                                                T (&regs)[PIECES][VL]) {
-  using Map = PieceMap<TILE_X, TILE_K, VL, KC>;
-#pragma unroll
-  for (int c = 0; c < PIECES; ++c) {
+// Edge tiles and the K tail: element-wise, bounds-checked copy straight into the LDS tile [k][x] (no
+// register staging, no overlap with the multiplication). Elements outside the matrix become zero.
+template <typename T, int TILE_X, int TILE_K, int PITCH, bool KC>
+__device__ __forceinline__ void FillSlabChecked(T* __restrict__ tile, const T* __restrict__ base, const long long ld,
+                                                const int x0, const int k0, const int x_end, const int k_end,
+                                                const int tid) {
+  using Map = PieceMap<TILE_X, TILE_K, 1, KC>;
+#pragma unroll 4
+  for (int piece = tid; piece < TILE_X * TILE_K; piece += kMfmaThreads) {
     int x, k;
-    Map::Get(tid + c * kMfmaThreads, x, k);
-#pragma unroll
-    for (int e = 0; e < VL; ++e) {
-      const int gx = x0 + x + (KC ? 0 : e), gk = k0 + k + (KC ? e : 0);
-      T value = T(0);
-      if (gx < x_end && gk < k_end) { value = KC ? base[gx * ld + gk] : base[gk * ld + gx]; }
-      regs[c][e] = value;
-    }
+    Map::Get(piece, x, k);
+    const int gx = x0 + x, gk = k0 + k;
+    T value = T(0);
+    if (gx < x_end && gk < k_end) { value = KC ? base[gx * ld + gk] : base[gk * ld + gx]; }
+    tile[k * PITCH + x] = value;
   }
 }
 
@@ -198,7 +197,7 @@ __device__ __forceinline__ void TileOfBlock(const int block, const int num_block
 
 // ---- the kernel ------------------------------------------------------------------------------------
 template <typename T, typename Config, bool A_KC, bool B_KC, bool ALIGNED>
-__global__ __launch_bounds__(kMfmaThreads) void GemmMfmaKernel(const GemmArgs<T> p, const int tiles_m,
+__global__ __launch_bounds__(kMfmaThreads, Config::MIN_WAVES) void GemmMfmaKernel(const GemmArgs<T> p, const int tiles_m,
                                                                const int tiles_n) {
   using Traits = typename Config::Traits;
   using Acc = typename Traits::Acc;
@@ -251,28 +250,14 @@ __global__ __launch_bounds__(kMfmaThreads) void GemmMfmaKernel(const GemmArgs<T>
     T b_regs[PIECES_B][VL];
 
     auto load = [&](const int slab) {
-      const int k0 = slab * TILE_K;
-      if (interior && slab < full_slabs) {
-        LoadSlab<T, TILE_M, TILE_K, PIECES_A, VL, A_KC>(a, p.a_ld, m0, k0, tid, a_regs);
-        LoadSlab<T, TILE_N, TILE_K, PIECES_B, VL, B_KC>(b, p.b_ld, n0, k0, tid, b_regs);
-      } else {
-        LoadSlabChecked<T, TILE_M, TILE_K, PIECES_A, VL, A_KC>(a, p.a_ld, m0, k0, p.m, p.k, tid, a_regs);
-        LoadSlabChecked<T, TILE_N, TILE_K, PIECES_B, VL, B_KC>(b, p.b_ld, n0, k0, p.n, p.k, tid, b_regs);
-      }
+      LoadSlab<T, TILE_M, TILE_K, PIECES_A, VL, A_KC>(a, p.a_ld, m0, slab * TILE_K, tid, a_regs);
+      LoadSlab<T, TILE_N, TILE_K, PIECES_B, VL, B_KC>(b, p.b_ld, n0, slab * TILE_K, tid, b_regs);
     };
     auto store = [&](const int buffer) {
       StoreSlab<T, TILE_M, TILE_K, PITCH_M, PIECES_A, VL, A_KC>(a_tiles + buffer * TILE_K * PITCH_M, tid, a_regs);
       StoreSlab<T, TILE_N, TILE_K, PITCH_N, PIECES_B, VL, B_KC>(b_tiles + buffer * TILE_K * PITCH_N, tid, b_regs);
     };
-
-    load(0);
-    store(0);
-    __syncthreads();
-
-    for (int slab = 0; slab < slabs; ++slab) {
-      const int buffer = slab & 1;
-      if (slab + 1 < slabs) { load(slab + 1); }
-
+    auto multiply = [&](const int buffer) {
       const T* a_tile = a_tiles + buffer * TILE_K * PITCH_M + a_read;
       const T* b_tile = b_tiles + buffer * TILE_K * PITCH_N + b_read;
 #pragma unroll
@@ -288,8 +273,28 @@ __global__ __launch_bounds__(kMfmaThreads) void GemmMfmaKernel(const GemmArgs<T>
           }
         }
       }
+    };
 
-      if (slab + 1 < slabs) { store(buffer ^ 1); }
+    // Interior tiles: software-pipelined walk over the full slabs.
+    const int fast_slabs = interior ? full_slabs : 0;
+    if (fast_slabs > 0) {
+      load(0);
+      store(0);
+      __syncthreads();
+      for (int slab = 0; slab < fast_slabs; ++slab) {
+        const int buffer = slab & 1;
+        if (slab + 1 < fast_slabs) { load(slab + 1); }
+        multiply(buffer);
+        if (slab + 1 < fast_slabs) { store(buffer ^ 1); }
+        __syncthreads();
+      }
+    }
+    // Edge tiles (all slabs) and the K tail of interior tiles: checked, unpipelined.
+    for (int slab = fast_slabs; slab < slabs; ++slab) {
+      FillSlabChecked<T, TILE_M, TILE_K, PITCH_M, A_KC>(a_tiles, a, p.a_ld, m0, slab * TILE_K, p.m, p.k, tid);
+      FillSlabChecked<T, TILE_N, TILE_K, PITCH_N, B_KC>(b_tiles, b, p.b_ld, n0, slab * TILE_K, p.n, p.k, tid);
+      __syncthreads();
+      multiply(0);
       __syncthreads();
     }
 
@@ -326,7 +331,6 @@ __global__ __launch_bounds__(kMfmaThreads) void GemmMfmaKernel(const GemmArgs<T>
         }
       }
     }
-    __syncthreads();  // the next batch reuses the LDS buffers
   }
 }
 

@@ -1,0 +1,245 @@
+// =================================================================================================
+// Large-tile MFMA GEMM kernel for gfx950, fp16 storage with fp32 accumulation (HGEMM). Like the
+// fp32/fp64 kernel (gemm_mfma.hpp) it replaces the reference's whole "indirect" chain
+// (src/routines/level3/xgemm.cpp:102-222, src/kernels/level3/xgemm_part1-4.opencl) with one launch
+// that reads the caller's operands in place. Unlike the reference, which accumulates in fp16
+// (src/kernels/common.opencl:44-45), products are accumulated in fp32 by v_mfma_f32_32x32x16_f16 and
+// rounded to fp16 once, in the epilogue.
+//
+// Structure (one work-group = 256 threads = 4 wavefronts in a 2 x 2 arrangement):
+//   * work-group tile (64*FM) x (64*FN), K walked in slabs of TILE_K, two LDS buffers, global loads
+//     of slab t+1 in flight while slab t is multiplied, one barrier per slab;
+//   * the MFMA wants 8 consecutive k per lane. A k-contiguous operand is kept in LDS as [x][k]
+//     (pitch TILE_K + 8 halfs: conflict-free 16-byte reads) and read with one ds_read_b128 per
+//     operand block. An x-contiguous operand (x = m for A, n for B) is kept as [k][x] (pitch
+//     tile + 32 halfs) and read with the CDNA4 transposing LDS read ds_read_b64_tr_b16, which hands
+//     each lane four consecutive k of its own x: the transpose costs no VALU work and no extra pass;
+//   * the n-indexed fragment is the MFMA's A operand and the m-indexed one its B operand, so the
+//     lanes of every accumulator register run along m, the contiguous index of the column-major C.
+// =================================================================================================
+#ifndef CLBLAST_HIP_KERNELS_GEMM_MFMA_F16_HPP_
+#define CLBLAST_HIP_KERNELS_GEMM_MFMA_F16_HPP_
+
+#include "kernels/gemm_args.hpp"
+#include "kernels/gemm_mfma.hpp"
+
+namespace clbh {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef short short4_t __attribute__((ext_vector_type(4)));
+
+// FM x FN MFMA blocks (32 x 32) per wavefront, 2 x 2 wavefronts.
+template <int FM_, int FN_, int TILE_K_>
+struct HgemmConfig {
+  static constexpr int FM = FM_, FN = FN_;
+  static constexpr int TILE_M = 2 * FM * 32;
+  static constexpr int TILE_N = 2 * FN * 32;
+  static constexpr int TILE_K = TILE_K_;
+  static constexpr int PITCH_KC = TILE_K + 8;    // halfs per x row of a [x][k] tile
+  static constexpr int PITCH_XM = TILE_M + 32;   // halfs per k row of a [k][m] tile
+  static constexpr int PITCH_XN = TILE_N + 32;
+  static constexpr int A_ELEMS_KC = TILE_M * PITCH_KC, A_ELEMS_XC = TILE_K * PITCH_XM;
+  static constexpr int B_ELEMS_KC = TILE_N * PITCH_KC, B_ELEMS_XC = TILE_K * PITCH_XN;
+  static constexpr int A_ELEMS = A_ELEMS_KC > A_ELEMS_XC ? A_ELEMS_KC : A_ELEMS_XC;
+  static constexpr int B_ELEMS = B_ELEMS_KC > B_ELEMS_XC ? B_ELEMS_KC : B_ELEMS_XC;
+  static constexpr int LDS_BYTES = 2 * (A_ELEMS + B_ELEMS) * 2;
+  static_assert(TILE_K % 16 == 0, "slab depth is a multiple of the MFMA k extent");
+};
+
+// ---- slab movement ---------------------------------------------------------------------------------
+// Slab of TILE_X x TILE_K halfs; element (x, k) at base[KC ? x*ld + k : k*ld + x]. Threads move pieces
+// of VL halfs (8 when every address is 16-byte aligned, else 1), consecutive threads along the
+// contiguous index.
+template <int TILE_X, int TILE_K, int PIECES, int VL, bool KC>
+__device__ __forceinline__ void HLoadSlab(const _Float16* __restrict__ base, const long long ld, const int x0,
+                                          const int k0, const int tid,
+                                          typename VecType<_Float16, VL>::type (&regs)[PIECES]) {
+  using Map = PieceMap<TILE_X, TILE_K, VL, KC>;
+  using V = typename VecType<_Float16, VL>::type;
+#pragma unroll
+  for (int c = 0; c < PIECES; ++c) {
+    int x, k;
+    Map::Get(tid + c * kMfmaThreads, x, k);
+    const _Float16* src = KC ? base + (x0 + x) * ld + (k0 + k) : base + (k0 + k) * ld + (x0 + x);
+    regs[c] = *reinterpret_cast<const V*>(src);
+  }
+}
+
+// Edge tiles and the K tail: element-wise, bounds-checked copy straight into LDS (no register staging, no
+// overlap with the multiplication). Elements outside the matrix become zero.
+template <int TILE_X, int TILE_K, int PITCH, bool KC>
+__device__ __forceinline__ void HFillSlabChecked(_Float16* __restrict__ tile, const _Float16* __restrict__ base,
+                                                 const long long ld, const int x0, const int k0, const int x_end,
+                                                 const int k_end, const int tid) {
+  using Map = PieceMap<TILE_X, TILE_K, 1, KC>;
+#pragma unroll 4
+  for (int piece = tid; piece < TILE_X * TILE_K; piece += kMfmaThreads) {
+    int x, k;
+    Map::Get(piece, x, k);
+    const int gx = x0 + x, gk = k0 + k;
+    _Float16 value = _Float16(0);
+    if (gx < x_end && gk < k_end) { value = KC ? base[gx * ld + gk] : base[gk * ld + gx]; }
+    tile[KC ? x * PITCH + k : k * PITCH + x] = value;
+  }
+}
+
+// Registers -> LDS in the same orientation as memory: [x][k] for KC, [k][x] otherwise.
+template <int TILE_X, int TILE_K, int PITCH, int PIECES, int VL, bool KC>
+__device__ __forceinline__ void HStoreSlab(_Float16* __restrict__ tile, const int tid,
+                                           const typename VecType<_Float16, VL>::type (&regs)[PIECES]) {
+  using Map = PieceMap<TILE_X, TILE_K, VL, KC>;
+  using V = typename VecType<_Float16, VL>::type;
+#pragma unroll
+  for (int c = 0; c < PIECES; ++c) {
+    int x, k;
+    Map::Get(tid + c * kMfmaThreads, x, k);
+    _Float16* dst = KC ? &tile[x * PITCH + k] : &tile[k * PITCH + x];
+    *reinterpret_cast<V*>(dst) = regs[c];
+  }
+}
+
+// One MFMA operand fragment: the 8 halfs of k = k16 + 8*(lane/32) .. +8 for x = x32 + lane%32.
+template <int PITCH, bool KC>
+__device__ __forceinline__ half8_t HReadFragment(const _Float16* __restrict__ tile, const int x32, const int k16,
+                                                 const int lane) {
+  if (KC) {
+    return *reinterpret_cast<const half8_t*>(&tile[(x32 + lane % 32) * PITCH + k16 + 8 * (lane / 32)]);
+  } else {
+    // Transposing read: within each group of 16 lanes, lane q addresses 4 halfs at row k + q/4, columns
+    // 4*(q%4)..+3, and receives the 4 halfs of rows k..k+3 at column q. Groups 0/1 take x 0-15/16-31
+    // of k 0-7, groups 2/3 the same x of k 8-15; two reads give the 8 consecutive k of a lane.
+    const int group = lane / 16, q = lane % 16;
+    const int x = x32 + 16 * (group % 2) + 4 * (q % 4);
+    const int k = k16 + 8 * (group / 2) + q / 4;
+    typedef __attribute__((address_space(3))) short4_t* LdsPtr;
+    const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(&tile[k * PITCH + x]));
+    const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(&tile[(k + 4) * PITCH + x]));
+    half8_t out;
+    const half4_t lo_h = __builtin_bit_cast(half4_t, lo), hi_h = __builtin_bit_cast(half4_t, hi);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { out[e] = lo_h[e]; out[4 + e] = hi_h[e]; }
+    return out;
+  }
+}
+
+// ---- the kernel ------------------------------------------------------------------------------------
+template <typename Config, bool A_KC, bool B_KC, bool ALIGNED>
+__global__ __launch_bounds__(kMfmaThreads) void HgemmMfmaKernel(const GemmArgs<float> p, const int tiles_m,
+                                                                const int tiles_n) {
+  using T = _Float16;
+  constexpr int TILE_M = Config::TILE_M, TILE_N = Config::TILE_N, TILE_K = Config::TILE_K;
+  constexpr int FM = Config::FM, FN = Config::FN;
+  constexpr int PITCH_A = A_KC ? Config::PITCH_KC : Config::PITCH_XM;
+  constexpr int PITCH_B = B_KC ? Config::PITCH_KC : Config::PITCH_XN;
+  constexpr int VL = ALIGNED ? 8 : 1;
+  constexpr int PIECES_A = TILE_M * TILE_K / VL / kMfmaThreads, PIECES_B = TILE_N * TILE_K / VL / kMfmaThreads;
+
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+  T* a_tiles = lds;                          // two buffers of A_ELEMS
+  T* b_tiles = lds + 2 * Config::A_ELEMS;    // two buffers of B_ELEMS
+
+  const int tid = threadIdx.x;
+  const int lane = tid % 64, wave = tid / 64;
+  const int wave_m = wave % 2, wave_n = wave / 2;
+
+  int tile_m, tile_n;
+  TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
+  const bool interior = (m0 + TILE_M <= p.m) && (n0 + TILE_N <= p.n);
+  const int full_slabs = p.k / TILE_K;
+  const int slabs = (p.k + TILE_K - 1) / TILE_K;
+
+  for (int batch = blockIdx.y; batch < p.batch_count; batch += gridDim.y) {
+    const T* a;
+    const T* b;
+    T* c;
+    float alpha, beta;
+    ResolveBatch<T, float>(p, batch, a, b, c, alpha, beta);
+
+    float16_t acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+#pragma unroll
+      for (int j = 0; j < FN; ++j) { acc[i][j] = float16_t(0.0f); }
+    }
+
+    typename VecType<T, VL>::type a_regs[PIECES_A];
+    typename VecType<T, VL>::type b_regs[PIECES_B];
+
+    auto load = [&](const int slab) {
+      HLoadSlab<TILE_M, TILE_K, PIECES_A, VL, A_KC>(a, p.a_ld, m0, slab * TILE_K, tid, a_regs);
+      HLoadSlab<TILE_N, TILE_K, PIECES_B, VL, B_KC>(b, p.b_ld, n0, slab * TILE_K, tid, b_regs);
+    };
+    auto store = [&](const int buffer) {
+      HStoreSlab<TILE_M, TILE_K, PITCH_A, PIECES_A, VL, A_KC>(a_tiles + buffer * Config::A_ELEMS, tid, a_regs);
+      HStoreSlab<TILE_N, TILE_K, PITCH_B, PIECES_B, VL, B_KC>(b_tiles + buffer * Config::B_ELEMS, tid, b_regs);
+    };
+    auto multiply = [&](const int buffer) {
+      const T* a_tile = a_tiles + buffer * Config::A_ELEMS;
+      const T* b_tile = b_tiles + buffer * Config::B_ELEMS;
+#pragma unroll
+      for (int ks = 0; ks < TILE_K / 16; ++ks) {
+        half8_t a_frag[FM], b_frag[FN];
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          a_frag[i] = HReadFragment<PITCH_A, A_KC>(a_tile, (wave_m * FM + i) * 32, ks * 16, lane);
+        }
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+          b_frag[j] = HReadFragment<PITCH_B, B_KC>(b_tile, (wave_n * FN + j) * 32, ks * 16, lane);
+        }
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+#pragma unroll
+          for (int j = 0; j < FN; ++j) {
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b_frag[j], a_frag[i], acc[i][j], 0, 0, 0);
+          }
+        }
+      }
+    };
+
+    // Interior tiles: software-pipelined walk over the full slabs.
+    const int fast_slabs = interior ? full_slabs : 0;
+    if (fast_slabs > 0) {
+      load(0);
+      store(0);
+      __syncthreads();
+      for (int slab = 0; slab < fast_slabs; ++slab) {
+        const int buffer = slab & 1;
+        if (slab + 1 < fast_slabs) { load(slab + 1); }
+        multiply(buffer);
+        if (slab + 1 < fast_slabs) { store(buffer ^ 1); }
+        __syncthreads();
+      }
+    }
+    // Edge tiles (all slabs) and the K tail of interior tiles: checked, unpipelined.
+    for (int slab = fast_slabs; slab < slabs; ++slab) {
+      HFillSlabChecked<TILE_M, TILE_K, PITCH_A, A_KC>(a_tiles, a, p.a_ld, m0, slab * TILE_K, p.m, p.k, tid);
+      HFillSlabChecked<TILE_N, TILE_K, PITCH_B, B_KC>(b_tiles, b, p.b_ld, n0, slab * TILE_K, p.n, p.k, tid);
+      __syncthreads();
+      multiply(0);
+      __syncthreads();
+    }
+
+    // Epilogue: lane owns m = m_blk + lane%32; accumulator element r is the column n_blk + Row(r).
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      const int m = m0 + (wave_m * FM + i) * 32 + lane % 32;
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+        const int n_blk = n0 + (wave_n * FN + j) * 32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int n = n_blk + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+          if (m < p.m && n < p.n) { StoreResult<T, float>(c, n * p.c_ld + m, acc[i][j][r], alpha, beta); }
+        }
+      }
+    }
+  }
+}
+
+}  // namespace clbh
+
+#endif  // CLBLAST_HIP_KERNELS_GEMM_MFMA_F16_HPP_

@@ -14,6 +14,13 @@ namespace {
 
 std::mutex override_mutex;
 std::map<std::tuple<int, int>, size_t> min_indirect_overrides;  // (device, precision bits) -> threshold
+std::map<int, size_t> tile_variant_overrides;                   // precision bits -> forced MFMA tile (0 = automatic)
+
+size_t ForcedTileVariant(const Precision precision) {
+  std::lock_guard<std::mutex> lock(override_mutex);
+  const auto found = tile_variant_overrides.find(static_cast<int>(precision));
+  return (found != tile_variant_overrides.end()) ? found->second : 0;
+}
 
 }  // namespace
 
@@ -33,6 +40,10 @@ size_t MinIndirectSize(const int device, const Precision precision) {
   return (found != min_indirect_overrides.end()) ? found->second : DefaultMinIndirectSize(precision);
 }
 
+namespace {
+size_t CeilDivide(const size_t x, const size_t y) { return (x + y - 1) / y; }
+}  // namespace
+
 bool UseDirectKernel(const size_t m, const size_t n, const size_t k, const size_t min_indirect_size) {
   const auto m_n_k =
       static_cast<unsigned long long>(m) * static_cast<unsigned long long>(n) * static_cast<unsigned long long>(k);
@@ -43,15 +54,39 @@ bool UseDirectKernel(const size_t m, const size_t n, const size_t k, const size_
 KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const bool b_kcontig, const size_t m,
                           const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,
                           const size_t min_indirect_size) {
-  (void)precision; (void)a_kcontig; (void)b_kcontig; (void)batch_count; (void)per_batch_scalars;
+  (void)a_kcontig; (void)b_kcontig; (void)batch_count; (void)per_batch_scalars;
   if (UseDirectKernel(m, n, k, min_indirect_size)) {
     return KernelChoice{CLBH_KERNEL_GENERAL, 0};
+  }
+  const auto forced = ForcedTileVariant(precision);
+  if (forced != 0) {
+    return KernelChoice{CLBH_KERNEL_MFMA, static_cast<int>(forced) - 1};
+  }
+  if (precision == Precision::kHalf) {
+    // 256 x 256 tiles once they fill the 256 CUs at least twice over, else 128 x 128
+    const auto big_tiles = CeilDivide(m, 256) * CeilDivide(n, 256);
+    return KernelChoice{CLBH_KERNEL_MFMA, (big_tiles >= 512) ? 2 : 0};
+  }
+  if (precision == Precision::kSingle) {
+    // 256 x 128 tiles (index 3) while they give every CU at least two work-groups, else 128 x 128
+    // with the tighter register budget (index 1)
+    const auto big_tiles = CeilDivide(m, 256) * CeilDivide(n, 128);
+    return KernelChoice{CLBH_KERNEL_MFMA, (big_tiles >= 512) ? 3 : 1};
   }
   return KernelChoice{CLBH_KERNEL_MFMA, 0};
 }
 
 StatusCode OverrideRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,
                                      const std::unordered_map<std::string, size_t>& parameters) {
+  if (kernel_name == "Xgemm") {  // forces one tile of the MFMA family: TILE_VARIANT = 1 + index, 0 = automatic
+    const auto variant = parameters.find("TILE_VARIANT");
+    if (variant == parameters.end()) {
+      return StatusCode::kMissingOverrideParameter;
+    }
+    std::lock_guard<std::mutex> lock(override_mutex);
+    tile_variant_overrides[static_cast<int>(precision)] = variant->second;
+    return StatusCode::kSuccess;
+  }
   if (kernel_name != "GemmRoutine") {
     return StatusCode::kInvalidOverrideKernel;
   }
@@ -66,6 +101,10 @@ StatusCode OverrideRoutineParameters(const int device, const std::string& kernel
 
 StatusCode RetrieveRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,
                                      std::unordered_map<std::string, size_t>& parameters) {
+  if (kernel_name == "Xgemm") {
+    parameters["TILE_VARIANT"] = ForcedTileVariant(precision);
+    return StatusCode::kSuccess;
+  }
   if (kernel_name != "GemmRoutine") {
     return StatusCode::kInvalidOverrideKernel;
   }
@@ -76,6 +115,7 @@ StatusCode RetrieveRoutineParameters(const int device, const std::string& kernel
 void ClearOverrides() {
   std::lock_guard<std::mutex> lock(override_mutex);
   min_indirect_overrides.clear();
+  tile_variant_overrides.clear();
 }
 
 }  // namespace clblast
