@@ -159,7 +159,7 @@ int LaunchHgemmVariant(const clbh_gemm_desc& d, hipStream_t stream) {
         reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (attribute_status != hipSuccess) { return static_cast<int>(attribute_status); }
   }
-  kernel<<<grid, dim3(kMfmaThreads), lds_bytes, stream>>>(args, static_cast<int>(tiles_m), static_cast<int>(tiles_n));
+  kernel<<<grid, dim3(Config::THREADS), lds_bytes, stream>>>(args, static_cast<int>(tiles_m), static_cast<int>(tiles_n));
   return static_cast<int>(hipGetLastError());
 }
 
@@ -176,12 +176,16 @@ int LaunchHgemmConfig(const clbh_gemm_desc& d, hipStream_t stream) {
 
 template <>
 int LaunchMfma<_Float16>(const clbh_gemm_desc& d, hipStream_t stream) {
-  // The 256 x 256 tiles exist for 16-byte aligned operands only; everything else takes 128 x 128.
-  if (!Aligned16<_Float16>(d)) { return LaunchHgemmConfig<HgemmConfig<2, 2, 32>, false>(d, stream); }
+  // The large tiles exist for 16-byte aligned operands only; everything else takes 128 x 128.
+  using Small = HgemmConfig<2, 2, 2, 2, 32, 2, false>;  // 128 x 128 x 32, 4 waves
+  if (!Aligned16<_Float16>(d)) { return LaunchHgemmConfig<Small, false>(d, stream); }
   switch (d.tile_variant) {
-    case 1: return LaunchHgemmConfig<HgemmConfig<4, 4, 32>, true>(d, stream);   // 256 x 256 x 32
-    case 2: return LaunchHgemmConfig<HgemmConfig<4, 4, 64>, true>(d, stream);   // 256 x 256 x 64
-    default: return LaunchHgemmConfig<HgemmConfig<2, 2, 32>, true>(d, stream);  // 128 x 128 x 32
+    case 1: return LaunchHgemmConfig<HgemmConfig<2, 2, 4, 4, 32, 1, true>, true>(d, stream);   // 256 x 256 x 32, 4 waves, pipelined
+    case 2: return LaunchHgemmConfig<HgemmConfig<2, 2, 4, 4, 64, 1, true>, true>(d, stream);   // 256 x 256 x 64, 4 waves, pipelined
+    case 3: return LaunchHgemmConfig<HgemmConfig<2, 4, 4, 2, 32, 2, false>, true>(d, stream);  // 256 x 256 x 32, 8 waves
+    case 4: return LaunchHgemmConfig<HgemmConfig<2, 4, 4, 2, 32, 2, true>, true>(d, stream);   // 256 x 256 x 32, 8 waves, pipelined
+    case 5: return LaunchHgemmConfig<HgemmConfig<2, 4, 4, 2, 64, 2, true>, true>(d, stream);   // 256 x 256 x 64, 8 waves, pipelined
+    default: return LaunchHgemmConfig<Small, true>(d, stream);
   }
 }
 

@@ -20,6 +20,8 @@
 #ifndef CLBLAST_HIP_KERNELS_GEMM_MFMA_F16_HPP_
 #define CLBLAST_HIP_KERNELS_GEMM_MFMA_F16_HPP_
 
+#include <type_traits>
+
 #include "kernels/gemm_args.hpp"
 #include "kernels/gemm_mfma.hpp"
 
@@ -29,12 +31,16 @@ typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef short short4_t __attribute__((ext_vector_type(4)));
 
-// FM x FN MFMA blocks (32 x 32) per wavefront, 2 x 2 wavefronts.
-template <int FM_, int FN_, int TILE_K_>
+// WM x WN wavefronts per work-group, each owning FM x FN MFMA blocks of 32 x 32. MIN_WAVES is the number
+// of wavefronts per SIMD the register budget must allow. PIPELINED selects the explicitly scheduled main
+// loop (see HgemmMfmaKernel); it needs FM >= FN and an even number of k-steps per slab.
+template <int WM_, int WN_, int FM_, int FN_, int TILE_K_, int MIN_WAVES_, bool PIPELINED_>
 struct HgemmConfig {
-  static constexpr int FM = FM_, FN = FN_;
-  static constexpr int TILE_M = 2 * FM * 32;
-  static constexpr int TILE_N = 2 * FN * 32;
+  static constexpr int WM = WM_, WN = WN_, FM = FM_, FN = FN_, MIN_WAVES = MIN_WAVES_;
+  static constexpr bool PIPELINED = PIPELINED_;
+  static constexpr int THREADS = 64 * WM * WN;
+  static constexpr int TILE_M = WM * FM * 32;
+  static constexpr int TILE_N = WN * FN * 32;
   static constexpr int TILE_K = TILE_K_;
   static constexpr int PITCH_KC = TILE_K + 8;    // halfs per x row of a [x][k] tile
   static constexpr int PITCH_XM = TILE_M + 32;   // halfs per k row of a [k][m] tile
@@ -45,13 +51,15 @@ struct HgemmConfig {
   static constexpr int B_ELEMS = B_ELEMS_KC > B_ELEMS_XC ? B_ELEMS_KC : B_ELEMS_XC;
   static constexpr int LDS_BYTES = 2 * (A_ELEMS + B_ELEMS) * 2;
   static_assert(TILE_K % 16 == 0, "slab depth is a multiple of the MFMA k extent");
+  static_assert((TILE_M * TILE_K) % (8 * THREADS) == 0 && (TILE_N * TILE_K) % (8 * THREADS) == 0, "slab split");
+  static_assert(!PIPELINED || (FM >= FN && (TILE_K / 16) % 2 == 0), "pipelined loop shape");
 };
 
 // ---- slab movement ---------------------------------------------------------------------------------
 // Slab of TILE_X x TILE_K halfs; element (x, k) at base[KC ? x*ld + k : k*ld + x]. Threads move pieces
 // of VL halfs (8 when every address is 16-byte aligned, else 1), consecutive threads along the
 // contiguous index.
-template <int TILE_X, int TILE_K, int PIECES, int VL, bool KC>
+template <int THREADS, int TILE_X, int TILE_K, int PIECES, int VL, bool KC>
 __device__ __forceinline__ void HLoadSlab(const _Float16* __restrict__ base, const long long ld, const int x0,
                                           const int k0, const int tid,
                                           typename VecType<_Float16, VL>::type (&regs)[PIECES]) {
@@ -60,7 +68,7 @@ __device__ __forceinline__ void HLoadSlab(const _Float16* __restrict__ base, con
 #pragma unroll
   for (int c = 0; c < PIECES; ++c) {
     int x, k;
-    Map::Get(tid + c * kMfmaThreads, x, k);
+    Map::Get(tid + c * THREADS, x, k);
     const _Float16* src = KC ? base + (x0 + x) * ld + (k0 + k) : base + (k0 + k) * ld + (x0 + x);
     regs[c] = *reinterpret_cast<const V*>(src);
   }
@@ -68,13 +76,13 @@ __device__ __forceinline__ void HLoadSlab(const _Float16* __restrict__ base, con
 
 // Edge tiles and the K tail: element-wise, bounds-checked copy straight into LDS (no register staging, no
 // overlap with the multiplication). Elements outside the matrix become zero.
-template <int TILE_X, int TILE_K, int PITCH, bool KC>
+template <int THREADS, int TILE_X, int TILE_K, int PITCH, bool KC>
 __device__ __forceinline__ void HFillSlabChecked(_Float16* __restrict__ tile, const _Float16* __restrict__ base,
                                                  const long long ld, const int x0, const int k0, const int x_end,
                                                  const int k_end, const int tid) {
   using Map = PieceMap<TILE_X, TILE_K, 1, KC>;
 #pragma unroll 4
-  for (int piece = tid; piece < TILE_X * TILE_K; piece += kMfmaThreads) {
+  for (int piece = tid; piece < TILE_X * TILE_K; piece += THREADS) {
     int x, k;
     Map::Get(piece, x, k);
     const int gx = x0 + x, gk = k0 + k;
@@ -85,7 +93,7 @@ __device__ __forceinline__ void HFillSlabChecked(_Float16* __restrict__ tile, co
 }
 
 // Registers -> LDS in the same orientation as memory: [x][k] for KC, [k][x] otherwise.
-template <int TILE_X, int TILE_K, int PITCH, int PIECES, int VL, bool KC>
+template <int THREADS, int TILE_X, int TILE_K, int PITCH, int PIECES, int VL, bool KC>
 __device__ __forceinline__ void HStoreSlab(_Float16* __restrict__ tile, const int tid,
                                            const typename VecType<_Float16, VL>::type (&regs)[PIECES]) {
   using Map = PieceMap<TILE_X, TILE_K, VL, KC>;
@@ -93,10 +101,28 @@ __device__ __forceinline__ void HStoreSlab(_Float16* __restrict__ tile, const in
 #pragma unroll
   for (int c = 0; c < PIECES; ++c) {
     int x, k;
-    Map::Get(tid + c * kMfmaThreads, x, k);
+    Map::Get(tid + c * THREADS, x, k);
     _Float16* dst = KC ? &tile[x * PITCH + k] : &tile[k * PITCH + x];
     *reinterpret_cast<V*>(dst) = regs[c];
   }
+}
+
+// Single pieces of a slab (16 bytes), for the explicitly scheduled loop.
+template <int THREADS, int TILE_X, int TILE_K, bool KC>
+__device__ __forceinline__ half8_t HLoadPiece(const _Float16* __restrict__ base, const long long ld, const int x0,
+                                              const int k0, const int tid, const int c) {
+  int x, k;
+  PieceMap<TILE_X, TILE_K, 8, KC>::Get(tid + c * THREADS, x, k);
+  const _Float16* src = KC ? base + (x0 + x) * ld + (k0 + k) : base + (k0 + k) * ld + (x0 + x);
+  return *reinterpret_cast<const half8_t*>(src);
+}
+
+template <int THREADS, int TILE_X, int TILE_K, int PITCH, bool KC>
+__device__ __forceinline__ void HStorePiece(_Float16* __restrict__ tile, const int tid, const int c,
+                                            const half8_t value) {
+  int x, k;
+  PieceMap<TILE_X, TILE_K, 8, KC>::Get(tid + c * THREADS, x, k);
+  *reinterpret_cast<half8_t*>(KC ? &tile[x * PITCH + k] : &tile[k * PITCH + x]) = value;
 }
 
 // One MFMA operand fragment: the 8 halfs of k = k16 + 8*(lane/32) .. +8 for x = x32 + lane%32.
@@ -125,7 +151,7 @@ __device__ __forceinline__ half8_t HReadFragment(const _Float16* __restrict__ ti
 
 // ---- the kernel ------------------------------------------------------------------------------------
 template <typename Config, bool A_KC, bool B_KC, bool ALIGNED>
-__global__ __launch_bounds__(kMfmaThreads) void HgemmMfmaKernel(const GemmArgs<float> p, const int tiles_m,
+__global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaKernel(const GemmArgs<float> p, const int tiles_m,
                                                                 const int tiles_n) {
   using T = _Float16;
   constexpr int TILE_M = Config::TILE_M, TILE_N = Config::TILE_N, TILE_K = Config::TILE_K;
@@ -133,7 +159,8 @@ __global__ __launch_bounds__(kMfmaThreads) void HgemmMfmaKernel(const GemmArgs<f
   constexpr int PITCH_A = A_KC ? Config::PITCH_KC : Config::PITCH_XM;
   constexpr int PITCH_B = B_KC ? Config::PITCH_KC : Config::PITCH_XN;
   constexpr int VL = ALIGNED ? 8 : 1;
-  constexpr int PIECES_A = TILE_M * TILE_K / VL / kMfmaThreads, PIECES_B = TILE_N * TILE_K / VL / kMfmaThreads;
+  constexpr int THREADS = Config::THREADS;
+  constexpr int PIECES_A = TILE_M * TILE_K / VL / THREADS, PIECES_B = TILE_N * TILE_K / VL / THREADS;
 
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
@@ -142,7 +169,7 @@ __global__ __launch_bounds__(kMfmaThreads) void HgemmMfmaKernel(const GemmArgs<f
 
   const int tid = threadIdx.x;
   const int lane = tid % 64, wave = tid / 64;
-  const int wave_m = wave % 2, wave_n = wave / 2;
+  const int wave_m = wave % Config::WM, wave_n = wave / Config::WM;
 
   int tile_m, tile_n;
   TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
@@ -169,12 +196,32 @@ __global__ __launch_bounds__(kMfmaThreads) void HgemmMfmaKernel(const GemmArgs<f
     typename VecType<T, VL>::type b_regs[PIECES_B];
 
     auto load = [&](const int slab) {
-      HLoadSlab<TILE_M, TILE_K, PIECES_A, VL, A_KC>(a, p.a_ld, m0, slab * TILE_K, tid, a_regs);
-      HLoadSlab<TILE_N, TILE_K, PIECES_B, VL, B_KC>(b, p.b_ld, n0, slab * TILE_K, tid, b_regs);
+      HLoadSlab<THREADS, TILE_M, TILE_K, PIECES_A, VL, A_KC>(a, p.a_ld, m0, slab * TILE_K, tid, a_regs);
+      HLoadSlab<THREADS, TILE_N, TILE_K, PIECES_B, VL, B_KC>(b, p.b_ld, n0, slab * TILE_K, tid, b_regs);
     };
     auto store = [&](const int buffer) {
-      HStoreSlab<TILE_M, TILE_K, PITCH_A, PIECES_A, VL, A_KC>(a_tiles + buffer * Config::A_ELEMS, tid, a_regs);
-      HStoreSlab<TILE_N, TILE_K, PITCH_B, PIECES_B, VL, B_KC>(b_tiles + buffer * Config::B_ELEMS, tid, b_regs);
+      HStoreSlab<THREADS, TILE_M, TILE_K, PITCH_A, PIECES_A, VL, A_KC>(a_tiles + buffer * Config::A_ELEMS, tid, a_regs);
+      HStoreSlab<THREADS, TILE_N, TILE_K, PITCH_B, PIECES_B, VL, B_KC>(b_tiles + buffer * Config::B_ELEMS, tid, b_regs);
+    };
+    auto read_fragments = [&](const T* a_tile, const T* b_tile, const int ks, half8_t (&a_frag)[FM],
+                              half8_t (&b_frag)[FN]) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        a_frag[i] = HReadFragment<PITCH_A, A_KC>(a_tile, (wave_m * FM + i) * 32, ks * 16, lane);
+      }
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+        b_frag[j] = HReadFragment<PITCH_B, B_KC>(b_tile, (wave_n * FN + j) * 32, ks * 16, lane);
+      }
+    };
+    auto multiply_fragments = [&](const half8_t (&a_frag)[FM], const half8_t (&b_frag)[FN]) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b_frag[j], a_frag[i], acc[i][j], 0, 0, 0);
+        }
+      }
     };
     auto multiply = [&](const int buffer) {
       const T* a_tile = a_tiles + buffer * Config::A_ELEMS;
@@ -182,27 +229,87 @@ __global__ __launch_bounds__(kMfmaThreads) void HgemmMfmaKernel(const GemmArgs<f
 #pragma unroll
       for (int ks = 0; ks < TILE_K / 16; ++ks) {
         half8_t a_frag[FM], b_frag[FN];
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-          a_frag[i] = HReadFragment<PITCH_A, A_KC>(a_tile, (wave_m * FM + i) * 32, ks * 16, lane);
-        }
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-          b_frag[j] = HReadFragment<PITCH_B, B_KC>(b_tile, (wave_n * FN + j) * 32, ks * 16, lane);
-        }
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-#pragma unroll
-          for (int j = 0; j < FN; ++j) {
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b_frag[j], a_frag[i], acc[i][j], 0, 0, 0);
-          }
-        }
+        read_fragments(a_tile, b_tile, ks, a_frag, b_frag);
+        multiply_fragments(a_frag, b_frag);
       }
     };
 
     // Interior tiles: software-pipelined walk over the full slabs.
     const int fast_slabs = interior ? full_slabs : 0;
-    if (fast_slabs > 0) {
+    if constexpr (Config::PIPELINED && ALIGNED) {
+      // Explicit schedule for one wavefront per SIMD, where nothing but the instruction order inside the
+      // wavefront can hide latency. Per slab (KSTEPS k-steps of FM quarters each):
+      //   quarter q of k-step s:  LDS reads of the a/b fragments q of k-step s+1 (other register set),
+      //                           then the FN MFMAs of block row q of k-step s,
+      //                           then a share of: store staged slab t+1 into the other LDS buffer and
+      //                           refill the staging registers with slab t+2 from global memory.
+      //   One barrier per slab, before the last k-step: by then every wavefront has issued all its reads
+      //   of the current buffer and all its stores to the other one, so the last k-step can already
+      //   fetch the first fragments of slab t+1. Scheduling fences pin this order for the compiler.
+      constexpr int KSTEPS = TILE_K / 16;
+      constexpr int SLOTS = (KSTEPS - 1) * FM;                       // quarters before the barrier
+      constexpr int PER_SLOT = (PIECES_A + PIECES_B + SLOTS - 1) / SLOTS;
+      if (fast_slabs > 0) {
+        load(0);
+        store(0);
+        if (fast_slabs > 1) { load(1); }
+        __syncthreads();
+        half8_t a_frag[2][FM], b_frag[2][FN];
+        read_fragments(a_tiles, b_tiles, 0, a_frag[0], b_frag[0]);
+        // One slab. STORE: the staging registers hold slab+1 and go to the other LDS buffer; LOAD: they are
+        // refilled with slab+2. Both are compile-time so that the steady state has no branches.
+        auto slab_body = [&](const int slab, auto store_tag, auto load_tag) {
+          constexpr bool STORE = decltype(store_tag)::value, LOAD = decltype(load_tag)::value;
+          const int cur = slab & 1;
+          const T* a_cur = a_tiles + cur * Config::A_ELEMS;
+          const T* b_cur = b_tiles + cur * Config::B_ELEMS;
+          T* a_nxt = a_tiles + (cur ^ 1) * Config::A_ELEMS;
+          T* b_nxt = b_tiles + (cur ^ 1) * Config::B_ELEMS;
+          const int k_load = (slab + 2) * TILE_K;
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) {
+            const int set = ks % 2;
+            const T* a_src = (ks + 1 < KSTEPS) ? a_cur : a_nxt;
+            const T* b_src = (ks + 1 < KSTEPS) ? b_cur : b_nxt;
+            const int ks_src = (ks + 1 < KSTEPS) ? ks + 1 : 0;
+#pragma unroll
+            for (int q = 0; q < FM; ++q) {
+              a_frag[set ^ 1][q] = HReadFragment<PITCH_A, A_KC>(a_src, (wave_m * FM + q) * 32, ks_src * 16, lane);
+              if (q < FN) {
+                b_frag[set ^ 1][q] = HReadFragment<PITCH_B, B_KC>(b_src, (wave_n * FN + q) * 32, ks_src * 16, lane);
+              }
+              __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+              for (int j = 0; j < FN; ++j) {
+                acc[q][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b_frag[set][j], a_frag[set][q], acc[q][j], 0, 0, 0);
+              }
+              if (ks < KSTEPS - 1) {
+                const int slot = ks * FM + q;
+#pragma unroll
+                for (int u = 0; u < PER_SLOT; ++u) {
+                  const int piece = slot * PER_SLOT + u;
+                  if (piece < PIECES_A) {
+                    if (STORE) { HStorePiece<THREADS, TILE_M, TILE_K, PITCH_A, A_KC>(a_nxt, tid, piece, a_regs[piece]); }
+                    if (LOAD) { a_regs[piece] = HLoadPiece<THREADS, TILE_M, TILE_K, A_KC>(a, p.a_ld, m0, k_load, tid, piece); }
+                  } else if (piece < PIECES_A + PIECES_B) {
+                    const int pb = piece - PIECES_A;
+                    if (STORE) { HStorePiece<THREADS, TILE_N, TILE_K, PITCH_B, B_KC>(b_nxt, tid, pb, b_regs[pb]); }
+                    if (LOAD) { b_regs[pb] = HLoadPiece<THREADS, TILE_N, TILE_K, B_KC>(b, p.b_ld, n0, k_load, tid, pb); }
+                  }
+                }
+              }
+              __builtin_amdgcn_sched_barrier(0);
+            }
+            if (ks == KSTEPS - 2) { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+          }
+        };
+        int slab = 0;
+        for (; slab + 2 < fast_slabs; ++slab) { slab_body(slab, std::true_type{}, std::true_type{}); }
+        if (slab + 1 < fast_slabs) { slab_body(slab, std::true_type{}, std::false_type{}); ++slab; }
+        slab_body(slab, std::false_type{}, std::false_type{});
+        __syncthreads();
+      }
+    } else if (fast_slabs > 0) {
       load(0);
       store(0);
       __syncthreads();
@@ -216,8 +323,8 @@ __global__ __launch_bounds__(kMfmaThreads) void HgemmMfmaKernel(const GemmArgs<f
     }
     // Edge tiles (all slabs) and the K tail of interior tiles: checked, unpipelined.
     for (int slab = fast_slabs; slab < slabs; ++slab) {
-      HFillSlabChecked<TILE_M, TILE_K, PITCH_A, A_KC>(a_tiles, a, p.a_ld, m0, slab * TILE_K, p.m, p.k, tid);
-      HFillSlabChecked<TILE_N, TILE_K, PITCH_B, B_KC>(b_tiles, b, p.b_ld, n0, slab * TILE_K, p.n, p.k, tid);
+      HFillSlabChecked<THREADS, TILE_M, TILE_K, PITCH_A, A_KC>(a_tiles, a, p.a_ld, m0, slab * TILE_K, p.m, p.k, tid);
+      HFillSlabChecked<THREADS, TILE_N, TILE_K, PITCH_B, B_KC>(b_tiles, b, p.b_ld, n0, slab * TILE_K, p.n, p.k, tid);
       __syncthreads();
       multiply(0);
       __syncthreads();
