@@ -8,7 +8,8 @@ import os
 from ctypes import c_char_p, c_double, c_float, c_int, c_size_t, c_ushort, c_void_p, POINTER
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libclblast_hip.so")
+# CLBLAST_HIP_LIBRARY points at another build of the same library (e.g. an experimental one).
+LIB_PATH = os.environ.get("CLBLAST_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libclblast_hip.so")
 CSRC_DIR = os.path.join(_HERE, "csrc")
 
 _lib = None

@@ -25,6 +25,20 @@
 #include "kernels/gemm_args.hpp"
 #include "kernels/gemm_mfma.hpp"
 
+// Timing experiments only (results are wrong when set): never defined by the product build.
+#ifndef CLBH_EXPERIMENT_NO_LOADS
+#define CLBH_EXPERIMENT_NO_LOADS 0
+#endif
+#ifndef CLBH_EXPERIMENT_NO_BARRIER
+#define CLBH_EXPERIMENT_NO_BARRIER 0
+#endif
+#ifndef CLBH_EXPERIMENT_NO_STORES
+#define CLBH_EXPERIMENT_NO_STORES 0
+#endif
+#ifndef CLBH_EXPERIMENT_NO_READS
+#define CLBH_EXPERIMENT_NO_READS 0
+#endif
+
 namespace clbh {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -290,17 +304,20 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
                   const int piece = slot * PER_SLOT + u;
                   if (piece < PIECES_A) {
                     if (STORE) { HStorePiece<THREADS, TILE_M, TILE_K, PITCH_A, A_KC>(a_nxt, tid, piece, a_regs[piece]); }
-                    if (LOAD) { a_regs[piece] = HLoadPiece<THREADS, TILE_M, TILE_K, A_KC>(a, p.a_ld, m0, k_load, tid, piece); }
+                    if (LOAD && !CLBH_EXPERIMENT_NO_LOADS) { a_regs[piece] = HLoadPiece<THREADS, TILE_M, TILE_K, A_KC>(a, p.a_ld, m0, k_load, tid, piece); }
                   } else if (piece < PIECES_A + PIECES_B) {
                     const int pb = piece - PIECES_A;
                     if (STORE) { HStorePiece<THREADS, TILE_N, TILE_K, PITCH_B, B_KC>(b_nxt, tid, pb, b_regs[pb]); }
-                    if (LOAD) { b_regs[pb] = HLoadPiece<THREADS, TILE_N, TILE_K, B_KC>(b, p.b_ld, n0, k_load, tid, pb); }
+                    if (LOAD && !CLBH_EXPERIMENT_NO_LOADS) { b_regs[pb] = HLoadPiece<THREADS, TILE_N, TILE_K, B_KC>(b, p.b_ld, n0, k_load, tid, pb); }
                   }
                 }
               }
               __builtin_amdgcn_sched_barrier(0);
             }
-            if (ks == KSTEPS - 2) { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+            if (ks == KSTEPS - 2) {
+              if (CLBH_EXPERIMENT_NO_BARRIER) { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+              else { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+            }
           }
         };
         int slab = 0;
