@@ -1,227 +1,22 @@
 // =================================================================================================
-// Implementation of the thin C-ABI device layer (include/clbh_device.h): the one translation unit that
-// calls the HIP runtime and launches the gfx950 kernels.
+// Implementation of the thin C-ABI device layer (include/clbh_device.h): runtime services and the
+// dispatch of a launch descriptor to the per-precision translation units (launch_f16/f32/f64/small.hip),
+// which are the only other files that touch the HIP runtime.
 // =================================================================================================
-#include <hip/hip_runtime.h>
-
-#include <algorithm>
-#include <climits>
-
-#include "clbh_device.h"
-#include "kernels/gemm_args.hpp"
-#include "kernels/gemm_general.hpp"
-#include "kernels/gemm_mfma.hpp"
-#include "kernels/gemm_mfma_f16.hpp"
-#include "kernels/gemm_mfma_f16_big.hpp"
+#include "device/launch_common.hpp"
 
 namespace clbh {
 namespace {
 
-constexpr int kMaxGridY = 65535;
-
-template <typename CT>
-GemmArgs<CT> MakeArgs(const clbh_gemm_desc& d) {
-  GemmArgs<CT> p;
-  p.a = d.a;
-  p.b = d.b;
-  p.c = d.c;
-  p.a_offset = d.a_offset;
-  p.b_offset = d.b_offset;
-  p.c_offset = d.c_offset;
-  p.a_ld = d.a_ld;
-  p.b_ld = d.b_ld;
-  p.c_ld = d.c_ld;
-  p.a_stride = d.a_stride;
-  p.b_stride = d.b_stride;
-  p.c_stride = d.c_stride;
-  p.m = d.m;
-  p.n = d.n;
-  p.k = d.k;
-  p.batch_count = d.batch_count;
-  p.alpha = static_cast<CT>(d.alpha);
-  p.beta = static_cast<CT>(d.beta);
-  p.alphas = static_cast<const CT*>(d.batch.alphas);
-  p.betas = static_cast<const CT*>(d.batch.betas);
-  p.a_offsets = d.batch.a_offsets;
-  p.b_offsets = d.batch.b_offsets;
-  p.c_offsets = d.batch.c_offsets;
-  return p;
-}
-
-// ---- general kernel -------------------------------------------------------------------------------
-template <typename T>
-int LaunchGeneral(const clbh_gemm_desc& d, hipStream_t stream) {
-  using CT = typename ComputeType<T>::type;
-  const auto args = MakeArgs<CT>(d);
-  const long long tiles_m = (d.m + kGeneralTileM - 1) / kGeneralTileM;
-  const long long tiles_n = (d.n + kGeneralTileN - 1) / kGeneralTileN;
-  if (tiles_m * tiles_n > INT_MAX) { return hipErrorInvalidConfiguration; }
-  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
-  const dim3 block(kGeneralThreads);
-  const int tm = static_cast<int>(tiles_m);
-  if (d.a_kcontig) {
-    if (d.b_kcontig) { GemmGeneralKernel<T, true, true><<<grid, block, 0, stream>>>(args, tm); }
-    else { GemmGeneralKernel<T, true, false><<<grid, block, 0, stream>>>(args, tm); }
-  } else {
-    if (d.b_kcontig) { GemmGeneralKernel<T, false, true><<<grid, block, 0, stream>>>(args, tm); }
-    else { GemmGeneralKernel<T, false, false><<<grid, block, 0, stream>>>(args, tm); }
-  }
-  return static_cast<int>(hipGetLastError());
-}
-
-// ---- MFMA kernels (fp32, fp64) ----------------------------------------------------------------------
-// True when every 16-byte access of the tile loaders and of the epilogue is naturally aligned.
-template <typename T>
-bool Aligned16(const clbh_gemm_desc& d) {
-  constexpr long long VEC = 16 / sizeof(T);
-  const auto address = [](const void* base, long long offset) {
-    return reinterpret_cast<unsigned long long>(base) + static_cast<unsigned long long>(offset) * sizeof(T);
-  };
-  if (address(d.a, d.a_offset) % 16 || address(d.b, d.b_offset) % 16 || address(d.c, d.c_offset) % 16) { return false; }
-  if (d.a_ld % VEC || d.b_ld % VEC || d.c_ld % VEC) { return false; }
-  if (d.batch_count > 1) {
-    if (d.batch.alphas != nullptr) { return false; }  // per-batch offsets are only known on the device
-    if (d.a_stride % VEC || d.b_stride % VEC || d.c_stride % VEC) { return false; }
-  }
-  return true;
-}
-
-template <typename T, typename Config, bool A_KC, bool B_KC, bool ALIGNED>
-int LaunchMfmaVariant(const clbh_gemm_desc& d, hipStream_t stream) {
-  const auto args = MakeArgs<T>(d);
-  const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
-  const long long tiles_n = (d.n + Config::TILE_N - 1) / Config::TILE_N;
-  if (tiles_m * tiles_n > INT_MAX) { return hipErrorInvalidConfiguration; }
-  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
-  constexpr size_t lds_bytes = Config::LDS_ELEMS * sizeof(T);
-  auto kernel = GemmMfmaKernel<T, Config, A_KC, B_KC, ALIGNED>;
-  if (lds_bytes > 48 * 1024) {
-    static const hipError_t attribute_status = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
-    if (attribute_status != hipSuccess) { return static_cast<int>(attribute_status); }
-  }
-  kernel<<<grid, dim3(kMfmaThreads), lds_bytes, stream>>>(args, static_cast<int>(tiles_m), static_cast<int>(tiles_n));
-  return static_cast<int>(hipGetLastError());
-}
-
-template <typename T, typename Config>
-int LaunchMfmaConfig(const clbh_gemm_desc& d, hipStream_t stream) {
-  const bool aligned = Aligned16<T>(d);
-  const int variant = (d.a_kcontig ? 4 : 0) | (d.b_kcontig ? 2 : 0) | (aligned ? 1 : 0);
-  switch (variant) {
-    case 0: return LaunchMfmaVariant<T, Config, false, false, false>(d, stream);
-    case 1: return LaunchMfmaVariant<T, Config, false, false, true>(d, stream);
-    case 2: return LaunchMfmaVariant<T, Config, false, true, false>(d, stream);
-    case 3: return LaunchMfmaVariant<T, Config, false, true, true>(d, stream);
-    case 4: return LaunchMfmaVariant<T, Config, true, false, false>(d, stream);
-    case 5: return LaunchMfmaVariant<T, Config, true, false, true>(d, stream);
-    case 6: return LaunchMfmaVariant<T, Config, true, true, false>(d, stream);
-    default: return LaunchMfmaVariant<T, Config, true, true, true>(d, stream);
-  }
-}
-
-template <typename T>
-int LaunchMfma(const clbh_gemm_desc& d, hipStream_t stream);
-
-template <>
-int LaunchMfma<float>(const clbh_gemm_desc& d, hipStream_t stream) {
-  switch (d.tile_variant) {
-    case 1: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16, 3>>(d, stream);
-    case 2: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16, 4>>(d, stream);
-    case 3: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 4, 2, 16, 2>>(d, stream);  // 256 x 128 x 16
-    case 4: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 32, 2>>(d, stream);  // 128 x 128 x 32
-    default: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16, 2>>(d, stream);  // 128 x 128 x 16
-  }
-}
-
-template <>
-int LaunchMfma<double>(const clbh_gemm_desc& d, hipStream_t stream) {
-  switch (d.tile_variant) {
-    case 1: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 2, 8, 2>>(d, stream);   // 128 x 64 x 8
-    case 2: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 2, 16, 2>>(d, stream);  // 128 x 64 x 16
-    case 3: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 2, 16, 3>>(d, stream);  // 128 x 64 x 16
-    case 4: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 4, 16, 2>>(d, stream);  // 128 x 128 x 16
-    default: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 4, 8, 2>>(d, stream);  // 128 x 128 x 8
-  }
-}
-
-// ---- MFMA kernel, fp16 ---------------------------------------------------------------------------
-template <typename Config, bool A_KC, bool B_KC, bool ALIGNED>
-int LaunchHgemmVariant(const clbh_gemm_desc& d, hipStream_t stream) {
-  const auto args = MakeArgs<float>(d);
-  const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
-  const long long tiles_n = (d.n + Config::TILE_N - 1) / Config::TILE_N;
-  if (tiles_m * tiles_n > INT_MAX) { return hipErrorInvalidConfiguration; }
-  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
-  constexpr size_t lds_bytes = Config::LDS_BYTES;
-  auto kernel = HgemmMfmaKernel<Config, A_KC, B_KC, ALIGNED>;
-  if (lds_bytes > 48 * 1024) {
-    static const hipError_t attribute_status = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
-    if (attribute_status != hipSuccess) { return static_cast<int>(attribute_status); }
-  }
-  kernel<<<grid, dim3(Config::THREADS), lds_bytes, stream>>>(args, static_cast<int>(tiles_m), static_cast<int>(tiles_n));
-  return static_cast<int>(hipGetLastError());
-}
-
-template <typename Config, bool ALIGNED>
-int LaunchHgemmConfig(const clbh_gemm_desc& d, hipStream_t stream) {
-  const int variant = (d.a_kcontig ? 2 : 0) | (d.b_kcontig ? 1 : 0);
-  switch (variant) {
-    case 0: return LaunchHgemmVariant<Config, false, false, ALIGNED>(d, stream);
-    case 1: return LaunchHgemmVariant<Config, false, true, ALIGNED>(d, stream);
-    case 2: return LaunchHgemmVariant<Config, true, false, ALIGNED>(d, stream);
-    default: return LaunchHgemmVariant<Config, true, true, ALIGNED>(d, stream);
-  }
-}
-
-template <typename Config, bool A_KC, bool B_KC>
-int LaunchHgemmBigVariant(const clbh_gemm_desc& d, hipStream_t stream) {
-  const auto args = MakeArgs<float>(d);
-  const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
-  const long long tiles_n = (d.n + Config::TILE_N - 1) / Config::TILE_N;
-  if (tiles_m * tiles_n > INT_MAX) { return hipErrorInvalidConfiguration; }
-  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
-  constexpr size_t lds_bytes = Config::LDS_BYTES;
-  auto kernel = HgemmBigKernel<Config, A_KC, B_KC>;
-  static const hipError_t attribute_status = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
-  if (attribute_status != hipSuccess) { return static_cast<int>(attribute_status); }
-  kernel<<<grid, dim3(Config::THREADS), lds_bytes, stream>>>(args, static_cast<int>(tiles_m), static_cast<int>(tiles_n));
-  return static_cast<int>(hipGetLastError());
-}
-
-// Needs 16-byte aligned operands (checked by the caller).
-template <typename Config>
-int LaunchHgemmBig(const clbh_gemm_desc& d, hipStream_t stream) {
-  const int variant = (d.a_kcontig ? 2 : 0) | (d.b_kcontig ? 1 : 0);
-  switch (variant) {
-    case 0: return LaunchHgemmBigVariant<Config, false, false>(d, stream);
-    case 1: return LaunchHgemmBigVariant<Config, false, true>(d, stream);
-    case 2: return LaunchHgemmBigVariant<Config, true, false>(d, stream);
-    default: return LaunchHgemmBigVariant<Config, true, true>(d, stream);
-  }
-}
-
-template <>
-int LaunchMfma<_Float16>(const clbh_gemm_desc& d, hipStream_t stream) {
-  // The large tiles exist for 16-byte aligned operands only; everything else takes 128 x 128.
-  using Small = HgemmConfig<2, 2, 2, 2, 32, 2, false>;  // 128 x 128 x 32, 4 waves
-  if (!Aligned16<_Float16>(d)) { return LaunchHgemmConfig<Small, false>(d, stream); }
-  switch (d.tile_variant) {
-    case 1: return LaunchHgemmConfig<HgemmConfig<2, 4, 4, 2, 32, 2, false>, true>(d, stream);  // 256 x 256 x 32, 8 waves
-    case 2: return LaunchHgemmConfig<HgemmConfig<2, 4, 4, 2, 32, 2, true>, true>(d, stream);   // 256 x 256 x 32, 8 waves, pipelined
-    case 3: return LaunchHgemmBig<HgemmBigConfig<2, 2, 4, 4, 1>>(d, stream);                   // 256 x 256 x 64 swizzled, 4 waves
-    case 4: return LaunchHgemmBig<HgemmBigConfig<2, 4, 4, 2, 2>>(d, stream);                   // 256 x 256 x 64 swizzled, 8 waves
-    default: return LaunchHgemmConfig<Small, true>(d, stream);
-  }
-}
-
-template <typename T>
 int LaunchTyped(const clbh_gemm_desc& d, hipStream_t stream) {
-  switch (d.kernel_class) {
-    case CLBH_KERNEL_MFMA: return LaunchMfma<T>(d, stream);
-    default: return LaunchGeneral<T>(d, stream);
+  const bool mfma = (d.kernel_class == CLBH_KERNEL_MFMA);
+  switch (d.precision) {
+    case 16: return mfma ? LaunchMfmaF16(d, stream) : LaunchGeneralF16(d, stream);
+    case 32:
+      if (d.kernel_class == CLBH_KERNEL_SMALL_BATCHED) { return LaunchSmallBatched(d, stream); }
+      return mfma ? LaunchMfmaF32(d, stream) : LaunchGeneralF32(d, stream);
+    case 64: return mfma ? LaunchMfmaF64(d, stream) : LaunchGeneralF64(d, stream);
+    default: return hipErrorInvalidValue;
   }
 }
 
@@ -247,17 +42,14 @@ extern "C" {
 
 int clbh_gemm_launch(const clbh_gemm_desc* desc, hipStream_t stream) {
   if (desc == nullptr || !clbh::ValidDescriptor(*desc)) { return hipErrorInvalidValue; }
-  switch (desc->precision) {
-    case 16: return clbh::LaunchTyped<_Float16>(*desc, stream);
-    case 32: return clbh::LaunchTyped<float>(*desc, stream);
-    case 64: return clbh::LaunchTyped<double>(*desc, stream);
-    default: return hipErrorInvalidValue;
-  }
+  return clbh::LaunchTyped(*desc, stream);
 }
 
 size_t clbh_gemm_workspace_bytes(const clbh_gemm_desc* desc) {
-  (void)desc;
-  return 0;
+  if (desc == nullptr || desc->kernel_class != CLBH_KERNEL_MFMA) { return 0; }
+  const auto plan = clbh::PlanSplit(*desc);
+  if (plan.splits <= 1) { return 0; }
+  return static_cast<size_t>(desc->precision / 8) * plan.splits * plan.ld * static_cast<size_t>(desc->n);
 }
 
 int clbh_buffer_extent(const void* ptr, size_t* bytes_available) {

@@ -1,0 +1,93 @@
+// =================================================================================================
+// Helpers shared by the translation units that instantiate and launch the gfx950 GEMM kernels.
+// =================================================================================================
+#ifndef CLBLAST_HIP_DEVICE_LAUNCH_COMMON_HPP_
+#define CLBLAST_HIP_DEVICE_LAUNCH_COMMON_HPP_
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <climits>
+
+#include "clbh_device.h"
+#include "kernels/gemm_args.hpp"
+
+namespace clbh {
+
+// Entry points of the per-precision translation units.
+int LaunchGeneralF16(const clbh_gemm_desc& d, hipStream_t stream);
+int LaunchGeneralF32(const clbh_gemm_desc& d, hipStream_t stream);
+int LaunchGeneralF64(const clbh_gemm_desc& d, hipStream_t stream);
+int LaunchMfmaF16(const clbh_gemm_desc& d, hipStream_t stream);
+int LaunchMfmaF32(const clbh_gemm_desc& d, hipStream_t stream);
+int LaunchMfmaF64(const clbh_gemm_desc& d, hipStream_t stream);
+int LaunchSmallBatched(const clbh_gemm_desc& d, hipStream_t stream);
+
+constexpr int kMaxGridY = 65535;
+
+template <typename CT>
+GemmArgs<CT> MakeArgs(const clbh_gemm_desc& d) {
+  GemmArgs<CT> p;
+  p.a = d.a;
+  p.b = d.b;
+  p.c = d.c;
+  p.a_offset = d.a_offset;
+  p.b_offset = d.b_offset;
+  p.c_offset = d.c_offset;
+  p.a_ld = d.a_ld;
+  p.b_ld = d.b_ld;
+  p.c_ld = d.c_ld;
+  p.a_stride = d.a_stride;
+  p.b_stride = d.b_stride;
+  p.c_stride = d.c_stride;
+  p.m = d.m;
+  p.n = d.n;
+  p.k = d.k;
+  p.batch_count = d.batch_count;
+  p.alpha = static_cast<CT>(d.alpha);
+  p.beta = static_cast<CT>(d.beta);
+  p.alphas = static_cast<const CT*>(d.batch.alphas);
+  p.betas = static_cast<const CT*>(d.batch.betas);
+  p.a_offsets = d.batch.a_offsets;
+  p.b_offsets = d.batch.b_offsets;
+  p.c_offsets = d.batch.c_offsets;
+  p.split_chunk = 0;
+  p.split_ld = 0;
+  p.split_workspace = nullptr;
+  return p;
+}
+
+
+// True when every 16-byte access of the tile loaders and of the epilogue is naturally aligned.
+template <typename T>
+inline bool Aligned16(const clbh_gemm_desc& d) {
+  constexpr long long VEC = 16 / sizeof(T);
+  const auto address = [](const void* base, long long offset) {
+    return reinterpret_cast<unsigned long long>(base) + static_cast<unsigned long long>(offset) * sizeof(T);
+  };
+  if (address(d.a, d.a_offset) % 16 || address(d.b, d.b_offset) % 16 || address(d.c, d.c_offset) % 16) { return false; }
+  if (d.a_ld % VEC || d.b_ld % VEC || d.c_ld % VEC) { return false; }
+  if (d.batch_count > 1) {
+    if (d.batch.alphas != nullptr) { return false; }  // per-batch offsets are only known on the device
+    if (d.a_stride % VEC || d.b_stride % VEC || d.c_stride % VEC) { return false; }
+  }
+  return true;
+}
+
+// Split-K geometry of a descriptor: K range per split (a multiple of 64) and the workspace leading dimension.
+struct SplitPlan {
+  int splits, chunk, ld;
+};
+inline SplitPlan PlanSplit(const clbh_gemm_desc& d) {
+  SplitPlan plan{1, 0, 0};
+  if (d.split_k > 1 && d.batch_count == 1 && d.batch.alphas == nullptr && d.precision != 16) {
+    const int chunk = ((d.k + d.split_k - 1) / d.split_k + 63) / 64 * 64;
+    const int splits = (d.k + chunk - 1) / chunk;
+    if (splits > 1) { plan = SplitPlan{splits, chunk, (d.m + 3) / 4 * 4}; }
+  }
+  return plan;
+}
+
+}  // namespace clbh
+
+#endif  // CLBLAST_HIP_DEVICE_LAUNCH_COMMON_HPP_

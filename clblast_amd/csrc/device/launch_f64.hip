@@ -1,0 +1,23 @@
+// =================================================================================================
+// fp64 instantiations of the general and MFMA GEMM kernels and the fp64 tile table.
+// =================================================================================================
+#include "device/launch_mfma.hpp"
+
+namespace clbh {
+namespace {
+}  // namespace
+
+int LaunchMfmaF64(const clbh_gemm_desc& d, hipStream_t stream) {
+  switch (d.tile_variant) {
+    case 1: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 2, 8, 2>>(d, stream);   // 128 x 64 x 8
+    case 2: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 2, 16, 2>>(d, stream);  // 128 x 64 x 16
+    case 3: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 2, 16, 3>>(d, stream);  // 128 x 64 x 16
+    case 4: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 4, 16, 2>>(d, stream);  // 128 x 128 x 16
+    default: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 4, 8, 2>>(d, stream);  // 128 x 128 x 8
+  }
+}
+
+
+int LaunchGeneralF64(const clbh_gemm_desc& d, hipStream_t stream) { return LaunchGeneral<double>(d, stream); }
+
+}  // namespace clbh

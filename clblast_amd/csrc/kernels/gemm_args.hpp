@@ -29,6 +29,12 @@ struct GemmArgs {
   const long long* a_offsets;
   const long long* b_offsets;
   const long long* c_offsets;
+  // Split-K launches (split_chunk > 0): "batch" s multiplies the k range [s*split_chunk, (s+1)*split_chunk)
+  // of ONE problem into slab s of the workspace (column-major m x n, leading dimension split_ld); a
+  // second kernel adds the slabs up and applies alpha and beta.
+  int split_chunk;
+  int split_ld;
+  void* split_workspace;
 };
 
 // Resolves the operand bases and scalars of batch `batch`.

@@ -136,6 +136,24 @@ __device__ __forceinline__ void LoadSlab(const T* __restrict__ base, const long 
   }
 }
 
+// Register-staged load of a slab whose x range sticks out of the matrix (the k range is complete):
+// elements beyond x_end read as zero. Keeps edge tiles on the pipelined path.
+template <typename T, int TILE_X, int TILE_K, int PIECES, int VL, bool KC>
+__device__ __forceinline__ void LoadSlabEdge(const T* __restrict__ base, const long long ld, const int x0, const int k0,
+                                             const int x_end, const int tid, T (&regs)[PIECES][VL]) {
+  using Map = PieceMap<TILE_X, TILE_K, VL, KC>;
+#pragma unroll
+  for (int c = 0; c < PIECES; ++c) {
+    int x, k;
+    Map::Get(tid + c * kMfmaThreads, x, k);
+#pragma unroll
+    for (int e = 0; e < VL; ++e) {
+      const int gx = x0 + x + (KC ? 0 : e), gk = k0 + k + (KC ? e : 0);
+      regs[c][e] = (gx < x_end) ? (KC ? base[gx * ld + gk] : base[gk * ld + gx]) : T(0);
+    }
+  }
+}
+
 // Edge tiles and the K tail: element-wise, bounds-checked copy straight into the LDS tile [k][x] (no
 // register staging, no overlap with the multiplication). Elements outside the matrix become zero.
 template <typename T, int TILE_X, int TILE_K, int PITCH, bool KC>
@@ -197,7 +215,7 @@ __device__ __forceinline__ void TileOfBlock(const int block, const int num_block
 
 // ---- the kernel ------------------------------------------------------------------------------------
 template <typename T, typename Config, bool A_KC, bool B_KC, bool ALIGNED>
-__global__ __launch_bounds__(kMfmaThreads, Config::MIN_WAVES) void GemmMfmaKernel(const GemmArgs<T> p, const int tiles_m,
+__global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void GemmMfmaKernel(const GemmArgs<T> p, const int tiles_m,
                                                                const int tiles_n) {
   using Traits = typename Config::Traits;
   using Acc = typename Traits::Acc;
@@ -224,12 +242,13 @@ __global__ __launch_bounds__(kMfmaThreads, Config::MIN_WAVES) void GemmMfmaKerne
   int tile_m, tile_n;
   TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
   const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
-  const bool interior = (m0 + TILE_M <= p.m) && (n0 + TILE_N <= p.n);
-  const int full_slabs = p.k / TILE_K;
-  const int slabs = (p.k + TILE_K - 1) / TILE_K;
+  const bool a_full = (m0 + TILE_M <= p.m), b_full = (n0 + TILE_N <= p.n);
 
-  // LDS read offsets of this lane: FM consecutive m and FN consecutive n per k row
-  const int a_read = wave_m * (FM * MF) + lane_x * FM;
+  // LDS read offsets of this lane. Aligned operands: the lane owns FM consecutive m (one vector LDS read,
+  // one vector store to C). Otherwise C is stored element-wise, and the lane owns m = lane_x, lane_x + MF,
+  // ... so that the lanes of each scalar store cover consecutive addresses.
+  constexpr bool M_INTERLEAVED = ALIGNED;
+  const int a_read = wave_m * (FM * MF) + (M_INTERLEAVED ? lane_x * FM : lane_x);
   const int b_read = wave_n * (FN * MF) + lane_x * FN;
 
   for (int batch = blockIdx.y; batch < p.batch_count; batch += gridDim.y) {
@@ -238,6 +257,22 @@ __global__ __launch_bounds__(kMfmaThreads, Config::MIN_WAVES) void GemmMfmaKerne
     T* c;
     T alpha, beta;
     ResolveBatch<T, T>(p, batch, a, b, c, alpha, beta);
+    int k_len = p.k;
+    long long c_ld = p.c_ld;
+    bool c_aligned = ALIGNED;
+    if (p.split_chunk > 0) {  // this "batch" is one K range of a single problem
+      const int k_begin = batch * p.split_chunk;
+      k_len = min(p.split_chunk, p.k - k_begin);
+      a = static_cast<const T*>(p.a) + p.a_offset + (A_KC ? k_begin : k_begin * p.a_ld);
+      b = static_cast<const T*>(p.b) + p.b_offset + (B_KC ? k_begin : k_begin * p.b_ld);
+      c_ld = p.split_ld;
+      c = static_cast<T*>(p.split_workspace) + static_cast<long long>(batch) * p.split_ld * p.n;
+      alpha = T(1);
+      beta = T(0);
+      c_aligned = true;  // the workspace is 256-byte aligned and split_ld a multiple of 4
+    }
+    const int full_slabs = k_len / TILE_K;
+    const int slabs = (k_len + TILE_K - 1) / TILE_K;
 
     Acc acc[FM][FN];
 #pragma unroll
@@ -250,8 +285,10 @@ __global__ __launch_bounds__(kMfmaThreads, Config::MIN_WAVES) void GemmMfmaKerne
     T b_regs[PIECES_B][VL];
 
     auto load = [&](const int slab) {
-      LoadSlab<T, TILE_M, TILE_K, PIECES_A, VL, A_KC>(a, p.a_ld, m0, slab * TILE_K, tid, a_regs);
-      LoadSlab<T, TILE_N, TILE_K, PIECES_B, VL, B_KC>(b, p.b_ld, n0, slab * TILE_K, tid, b_regs);
+      if (a_full) { LoadSlab<T, TILE_M, TILE_K, PIECES_A, VL, A_KC>(a, p.a_ld, m0, slab * TILE_K, tid, a_regs); }
+      else { LoadSlabEdge<T, TILE_M, TILE_K, PIECES_A, VL, A_KC>(a, p.a_ld, m0, slab * TILE_K, p.m, tid, a_regs); }
+      if (b_full) { LoadSlab<T, TILE_N, TILE_K, PIECES_B, VL, B_KC>(b, p.b_ld, n0, slab * TILE_K, tid, b_regs); }
+      else { LoadSlabEdge<T, TILE_N, TILE_K, PIECES_B, VL, B_KC>(b, p.b_ld, n0, slab * TILE_K, p.n, tid, b_regs); }
     };
     auto store = [&](const int buffer) {
       StoreSlab<T, TILE_M, TILE_K, PITCH_M, PIECES_A, VL, A_KC>(a_tiles + buffer * TILE_K * PITCH_M, tid, a_regs);
@@ -263,7 +300,13 @@ __global__ __launch_bounds__(kMfmaThreads, Config::MIN_WAVES) void GemmMfmaKerne
 #pragma unroll
       for (int ks = 0; ks < TILE_K / KP; ++ks) {
         const int k = ks * KP + lane_g;
-        const VM av = *reinterpret_cast<const VM*>(&a_tile[k * PITCH_M]);
+        VM av;
+        if constexpr (M_INTERLEAVED) {
+          av = *reinterpret_cast<const VM*>(&a_tile[k * PITCH_M]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < FM; ++i) { av = VecWith<VM, T, FM>(av, i, a_tile[k * PITCH_M + i * MF]); }
+        }
         const VN bv = *reinterpret_cast<const VN*>(&b_tile[k * PITCH_N]);
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
@@ -275,8 +318,8 @@ __global__ __launch_bounds__(kMfmaThreads, Config::MIN_WAVES) void GemmMfmaKerne
       }
     };
 
-    // Interior tiles: software-pipelined walk over the full slabs.
-    const int fast_slabs = interior ? full_slabs : 0;
+    // Software-pipelined walk over the full slabs (edge tiles load with x predication).
+    const int fast_slabs = full_slabs;
     if (fast_slabs > 0) {
       load(0);
       store(0);
@@ -289,10 +332,10 @@ __global__ __launch_bounds__(kMfmaThreads, Config::MIN_WAVES) void GemmMfmaKerne
         __syncthreads();
       }
     }
-    // Edge tiles (all slabs) and the K tail of interior tiles: checked, unpipelined.
+    // The K tail: checked, unpipelined.
     for (int slab = fast_slabs; slab < slabs; ++slab) {
-      FillSlabChecked<T, TILE_M, TILE_K, PITCH_M, A_KC>(a_tiles, a, p.a_ld, m0, slab * TILE_K, p.m, p.k, tid);
-      FillSlabChecked<T, TILE_N, TILE_K, PITCH_N, B_KC>(b_tiles, b, p.b_ld, n0, slab * TILE_K, p.n, p.k, tid);
+      FillSlabChecked<T, TILE_M, TILE_K, PITCH_M, A_KC>(a_tiles, a, p.a_ld, m0, slab * TILE_K, p.m, k_len, tid);
+      FillSlabChecked<T, TILE_N, TILE_K, PITCH_N, B_KC>(b_tiles, b, p.b_ld, n0, slab * TILE_K, p.n, k_len, tid);
       __syncthreads();
       multiply(0);
       __syncthreads();
@@ -302,14 +345,15 @@ __global__ __launch_bounds__(kMfmaThreads, Config::MIN_WAVES) void GemmMfmaKerne
     // column n = n_base + FN * Row(r) + j.
     const int m_base = m0 + a_read;
     const int n_base = n0 + wave_n * (FN * MF);
-    const bool vector_store = ALIGNED && (FM > 1) && (m_base + FM <= p.m);
+    constexpr int M_STEP = M_INTERLEAVED ? 1 : MF;  // distance in m between the lane's accumulator blocks
+    const bool vector_store = M_INTERLEAVED && c_aligned && (FM > 1) && (m_base + FM <= p.m);
 #pragma unroll
     for (int j = 0; j < FN; ++j) {
 #pragma unroll
       for (int r = 0; r < ACC; ++r) {
         const int n = n_base + FN * Traits::Row(r, lane_g) + j;
         if (n >= p.n) { continue; }
-        T* dst = c + n * p.c_ld + m_base;
+        T* dst = c + n * c_ld + m_base;
         if (vector_store) {
           VM out;
           if (beta == T(0)) {
@@ -326,12 +370,27 @@ __global__ __launch_bounds__(kMfmaThreads, Config::MIN_WAVES) void GemmMfmaKerne
         } else {
 #pragma unroll
           for (int i = 0; i < FM; ++i) {
-            if (m_base + i < p.m) { StoreResult<T, T>(dst, i, acc[i][j][r], alpha, beta); }
+            if (m_base + i * M_STEP < p.m) { StoreResult<T, T>(dst, i * M_STEP, acc[i][j][r], alpha, beta); }
           }
         }
       }
     }
   }
+}
+
+// Second pass of a split-K launch: C = alpha * (sum of the workspace slabs) + beta * C.
+template <typename T>
+__global__ __launch_bounds__(256) void GemmSplitReduceKernel(const T* __restrict__ workspace, const int splits,
+                                                             const int split_ld, T* __restrict__ c, const long long c_ld,
+                                                             const int m, const int n, const T alpha, const T beta) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int j = blockIdx.y;
+  if (i >= m) { return; }
+  const long long slab = static_cast<long long>(split_ld) * n;
+  const T* src = workspace + static_cast<long long>(j) * split_ld + i;
+  T sum = T(0);
+  for (int s = 0; s < splits; ++s) { sum += src[s * slab]; }
+  StoreResult<T, T>(c, j * c_ld + i, sum, alpha, beta);
 }
 
 }  // namespace clbh

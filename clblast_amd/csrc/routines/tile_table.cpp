@@ -3,6 +3,7 @@
 // =================================================================================================
 #include "routines/tile_table.hpp"
 
+#include <algorithm>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -51,29 +52,57 @@ bool UseDirectKernel(const size_t m, const size_t n, const size_t k, const size_
   return m_n_k < threshold * threshold * threshold;
 }
 
+// fp32 tile table (index -> work-group tile), see device/launch.hip:
+//   1: 128 x 128 x 16   3: 256 x 128 x 16   5: 128 x 32 x 32   6: 32 x 128 x 32   7: 64 x 64 x 16
+namespace {
+struct Tile {
+  int index;
+  size_t tile_m, tile_n;
+};
+
+// Number of K ranges that brings the launch to about two work-groups per CU, keeping ranges >= 128.
+int SplitFor(const size_t tiles, const size_t k) {
+  constexpr size_t kWantedGroups = 512;
+  if (tiles >= 256 || k < 512) { return 1; }
+  const auto wanted = CeilDivide(kWantedGroups, tiles);
+  const auto allowed = k / 128;
+  return static_cast<int>(std::max<size_t>(1, std::min<size_t>({wanted, allowed, 64})));
+}
+}  // namespace
+
 KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const bool b_kcontig, const size_t m,
                           const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,
                           const size_t min_indirect_size) {
-  (void)a_kcontig; (void)b_kcontig; (void)batch_count; (void)per_batch_scalars;
+  (void)a_kcontig; (void)b_kcontig; (void)per_batch_scalars;
+  // Many small fp32 matrices: one wavefront per matrix, bandwidth bound
+  if (precision == Precision::kSingle && batch_count >= 16 && m <= 32 && n <= 32 && k <= 32) {
+    return KernelChoice{CLBH_KERNEL_SMALL_BATCHED, 0, 1};
+  }
   if (UseDirectKernel(m, n, k, min_indirect_size)) {
-    return KernelChoice{CLBH_KERNEL_GENERAL, 0};
+    return KernelChoice{CLBH_KERNEL_GENERAL, 0, 1};
   }
   const auto forced = ForcedTileVariant(precision);
   if (forced != 0) {
-    return KernelChoice{CLBH_KERNEL_MFMA, static_cast<int>(forced) - 1};
+    return KernelChoice{CLBH_KERNEL_MFMA, static_cast<int>(forced) - 1, 1};
   }
   if (precision == Precision::kHalf) {
     // 256 x 256 tiles (8 wavefronts, index 2) once there are at least two per CU, else 128 x 128
     const auto big_tiles = CeilDivide(m, 256) * CeilDivide(n, 256);
-    return KernelChoice{CLBH_KERNEL_MFMA, (big_tiles >= 512) ? 2 : 0};
+    return KernelChoice{CLBH_KERNEL_MFMA, (big_tiles >= 512) ? 2 : 0, 1};
   }
   if (precision == Precision::kSingle) {
-    // 256 x 128 tiles (index 3) while they give every CU at least two work-groups, else 128 x 128
-    // with the tighter register budget (index 1)
-    const auto big_tiles = CeilDivide(m, 256) * CeilDivide(n, 128);
-    return KernelChoice{CLBH_KERNEL_MFMA, (big_tiles >= 512) ? 3 : 1};
+    auto tile = Tile{1, 128, 128};
+    if (CeilDivide(m, 256) * CeilDivide(n, 128) >= 512) { tile = Tile{3, 256, 128}; }
+    else if (n <= 32 && m >= 256) { tile = Tile{5, 128, 32}; }   // skinny: stream A
+    else if (m <= 32 && n >= 256) { tile = Tile{6, 32, 128}; }   // skinny: stream B
+    else if (CeilDivide(m, 128) * CeilDivide(n, 128) < 128) { tile = Tile{7, 64, 64}; }
+    const auto tiles = CeilDivide(m, tile.tile_m) * CeilDivide(n, tile.tile_n) * batch_count;
+    const auto split = (batch_count == 1) ? SplitFor(tiles, k) : 1;
+    return KernelChoice{CLBH_KERNEL_MFMA, tile.index, split};
   }
-  return KernelChoice{CLBH_KERNEL_MFMA, 0};
+  // fp64: 128 x 128 x 8 tiles, split K when they cannot fill the chip
+  const auto tiles = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
+  return KernelChoice{CLBH_KERNEL_MFMA, 0, (batch_count == 1) ? SplitFor(tiles, k) : 1};
 }
 
 StatusCode OverrideRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,

@@ -19,6 +19,7 @@ namespace clblast {
 struct KernelChoice {
   int kernel_class;  // enum clbh_kernel_class
   int tile_variant;  // index into the variant list of that class
+  int split_k;       // number of K ranges to spread over extra work-groups (1 = none)
 };
 
 // Default direct/indirect thresholds per precision (see tile_table.cpp for the reasoning).

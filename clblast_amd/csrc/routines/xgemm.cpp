@@ -106,6 +106,7 @@ size_t Xgemm<T>::TempBytes(const Layout layout, const Transpose a_transpose, con
                                    min_indirect_size);
   desc.kernel_class = choice.kernel_class;
   desc.tile_variant = choice.tile_variant;
+  desc.split_k = choice.split_k;
   return clbh_gemm_workspace_bytes(&desc);
 }
 
@@ -130,6 +131,7 @@ void Xgemm<T>::DoGemm(const Layout layout, const Transpose a_transpose, const Tr
                                    min_indirect_size());
   desc.kernel_class = choice.kernel_class;
   desc.tile_variant = choice.tile_variant;
+  desc.split_k = choice.split_k;
   desc.alpha = ScalarToDouble(alpha);
   desc.beta = ScalarToDouble(beta);
 

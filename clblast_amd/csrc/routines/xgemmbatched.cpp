@@ -49,6 +49,7 @@ void XgemmBatched<T>::DoGemmBatched(const Layout layout, const Transpose a_trans
                                    min_indirect_size());
   desc.kernel_class = choice.kernel_class;
   desc.tile_variant = choice.tile_variant;
+  desc.split_k = choice.split_k;
   desc.batch_count = static_cast<int>(batch_count);
 
   // Packs [alphas | betas | a_offsets | b_offsets | c_offsets] into one host block. Scalars are stored
@@ -144,6 +145,7 @@ void XgemmStridedBatched<T>::DoGemmStridedBatched(
                                    min_indirect_size());
   desc.kernel_class = choice.kernel_class;
   desc.tile_variant = choice.tile_variant;
+  desc.split_k = choice.split_k;
   CheckDevice(clbh_gemm_launch(&desc, stream()), "strided-batched GEMM launch");
   Finish();
 }

@@ -224,8 +224,8 @@ def float_to_half_truncate_numpy(values):
     """Vectorised statement of the truncating conversion for finite fp32 inputs: round toward zero onto
     the binary16 grid, magnitudes >= 65536 -> infinity (overflow rule of clblast_half.h:31-34)."""
     values = np.asarray(values, dtype=np.float32)
-    nearest = values.astype(np.float16)
     with np.errstate(over="ignore", invalid="ignore"):
+        nearest = values.astype(np.float16)
         too_big = np.abs(nearest.astype(np.float32)) > np.abs(values)
     bits = nearest.view(np.uint16).copy()
     # stepping one ulp toward zero is "bits - 1" for both signs in sign-magnitude binary16

@@ -1,0 +1,150 @@
+"""Parity of GemmBatched<T> and GemmStridedBatched<T> through the C ABI against the CPU oracle (per batch).
+
+Cases follow the reference's batched test descriptors (test/routines/levelx/xgemmbatched.hpp:21-212,
+xgemmstridedbatched.hpp:21-194: batch counts {1, 3}, the {7, 64} dimension sweep) plus what the kernels here
+add: the 32-cubed shape of the one-wavefront-per-matrix kernel, shared and overlapping input offsets
+(samples/sgemm_batched.cpp:53-59), zero input strides (broadcast), per-batch alpha and beta."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import clblast_amd
+import oracle
+from oracle import COL_MAJOR, NO, ROW_MAJOR, YES
+
+pytestmark = pytest.mark.gpu
+
+TOL = {16: 1e-2, 32: 1e-5, 64: 1e-12}
+PREFIX = {16: "H", 32: "S", 64: "D"}
+
+
+def run_strided(gpu, bits, layout, ta, tb, m, n, k, alpha, beta, batch, a_stride=None, b_stride=None, offsets=(0, 0, 0),
+                extra_ld=(0, 0, 0), seed=1):
+    _, shape = oracle.process_arguments(layout, ta, tb, m, n, k)
+    a_ld, b_ld, c_ld = shape.a_one + extra_ld[0], shape.b_one + extra_ld[1], shape.c_one + extra_ld[2]
+    a_need = oracle.required_elements(shape.a_one, shape.a_two, a_ld, 0)
+    b_need = oracle.required_elements(shape.b_one, shape.b_two, b_ld, 0)
+    c_stride = oracle.required_elements(shape.c_one, shape.c_two, c_ld, 0) + 5
+    a_stride = a_need + 3 if a_stride is None else a_stride
+    b_stride = b_need + 1 if b_stride is None else b_stride
+    a = oracle.uniform(seed, offsets[0] + a_stride * (batch - 1) + a_need + gpu.CANARY, -1, 1, bits)
+    b = oracle.uniform(seed + 1, offsets[1] + b_stride * (batch - 1) + b_need + gpu.CANARY, -1, 1, bits)
+    c = oracle.uniform(seed + 2, offsets[2] + c_stride * batch + gpu.CANARY, -1, 1, bits)
+    a_dev, b_dev, c_dev = gpu.to_device(a), gpu.to_device(b), gpu.to_device(c)
+    status = clblast_amd.raw_gemm_strided_batched(PREFIX[bits], layout, ta, tb, m, n, k, alpha, a_dev.data_ptr(),
+                                                  offsets[0], a_ld, a_stride, b_dev.data_ptr(), offsets[1], b_ld,
+                                                  b_stride, beta, c_dev.data_ptr(), offsets[2], c_ld, c_stride, batch,
+                                                  gpu.stream_handle())
+    torch.cuda.synchronize()
+    assert status == 0
+    c_after = c_dev.cpu().numpy()
+    untouched = np.ones(c.size, dtype=bool)
+    for index in range(batch):
+        expected = oracle.gemm(layout, ta, tb, m, n, k, alpha, a, offsets[0] + index * a_stride, a_ld, b,
+                               offsets[1] + index * b_stride, b_ld, beta, c, offsets[2] + index * c_stride, c_ld)
+        where = oracle.c_indices(layout, m, n, offsets[2] + index * c_stride, c_ld)
+        error = oracle.rel_frobenius(c_after[where], expected)
+        assert error <= TOL[bits], "batch %d: rel. Frobenius error %.2e" % (index, error)
+        untouched[where.ravel()] = False
+    assert np.array_equal(c_after[untouched].view(np.uint8), c[untouched].view(np.uint8))
+
+
+@pytest.mark.parametrize("bits", [32, 64, 16])
+def test_strided_batched_reference_sweep(gpu, bits):
+    seed = 0
+    for layout, ta, tb in itertools.product((ROW_MAJOR, COL_MAJOR), (NO, YES), (NO, YES)):
+        for m, n, k in itertools.product((7, 64), repeat=3):
+            for batch in (1, 3):
+                seed += 3
+                run_strided(gpu, bits, layout, ta, tb, m, n, k, 3.14, 3.14, batch, seed=seed,
+                            offsets=((0, 0, 0), (10, 10, 10))[seed % 2], extra_ld=((0, 0, 0), (1, 2, 3))[(seed // 2) % 2])
+
+
+@pytest.mark.parametrize("layout", [ROW_MAJOR, COL_MAJOR])
+def test_strided_batched_small_matrix_kernel(gpu, layout):
+    """m, n, k <= 32 with many batches takes the one-wavefront-per-matrix kernel: dense 32^3 (16-byte loads)
+    and ragged / padded / offset variants (element-wise loads)."""
+    seed = 100
+    for ta, tb in itertools.product((NO, YES), (NO, YES)):
+        for (m, n, k), extra, offsets, strides in [((32, 32, 32), (0, 0, 0), (0, 0, 0), (1024, 1024)),
+                                                   ((32, 32, 32), (0, 0, 0), (4, 8, 12), (1024, 1024)),
+                                                   ((32, 32, 32), (1, 0, 2), (3, 1, 5), (None, None)),
+                                                   ((17, 31, 9), (0, 0, 0), (0, 0, 0), (None, None)),
+                                                   ((1, 32, 32), (2, 2, 2), (1, 1, 1), (None, None)),
+                                                   ((32, 32, 32), (0, 0, 0), (0, 0, 0), (0, 0))]:  # broadcast A and B
+            for alpha, beta in ((1.0, 0.0), (-0.75, 2.0)):
+                seed += 3
+                run_strided(gpu, 32, layout, ta, tb, m, n, k, alpha, beta, 67, strides[0], strides[1], offsets, extra, seed)
+
+
+@pytest.mark.parametrize("bits", [32, 64, 16])
+def test_batched_with_per_batch_scalars_and_offsets(gpu, bits):
+    seed = 500
+    for layout, ta, tb in itertools.product((ROW_MAJOR, COL_MAJOR), (NO, YES), (NO, YES)):
+        for (m, n, k), batch in (((7, 64, 7), 3), ((64, 7, 64), 1), ((32, 32, 32), 40), ((9, 5, 33), 17)):
+            seed += 3
+            _, shape = oracle.process_arguments(layout, ta, tb, m, n, k)
+            a_ld, b_ld, c_ld = shape.a_one + 1, shape.b_one, shape.c_one + 2
+            a_need = oracle.required_elements(shape.a_one, shape.a_two, a_ld, 0)
+            b_need = oracle.required_elements(shape.b_one, shape.b_two, b_ld, 0)
+            c_need = oracle.required_elements(shape.c_one, shape.c_two, c_ld, 0)
+            rng = np.random.Generator(np.random.PCG64(seed))
+            # inputs may share or overlap; outputs must be disjoint
+            a_offsets = [int(v) for v in rng.integers(0, a_need, batch)]
+            b_offsets = [0] * batch
+            c_offsets = [7 + index * (c_need + 3) for index in rng.permutation(batch)]
+            alphas = [float(v) for v in rng.uniform(-2, 2, batch)]
+            betas = [float(v) if index % 3 else 0.0 for index, v in enumerate(rng.uniform(-2, 2, batch))]
+            a = oracle.uniform(seed, max(a_offsets) + a_need + gpu.CANARY, -1, 1, bits)
+            b = oracle.uniform(seed + 1, b_need + gpu.CANARY, -1, 1, bits)
+            c = oracle.uniform(seed + 2, max(c_offsets) + c_need + gpu.CANARY, -1, 1, bits)
+            a_dev, b_dev, c_dev = gpu.to_device(a), gpu.to_device(b), gpu.to_device(c)
+            status = clblast_amd.raw_gemm_batched(PREFIX[bits], layout, ta, tb, m, n, k, alphas, a_dev.data_ptr(),
+                                                  a_offsets, a_ld, b_dev.data_ptr(), b_offsets, b_ld, betas,
+                                                  c_dev.data_ptr(), c_offsets, c_ld, batch, gpu.stream_handle())
+            torch.cuda.synchronize()
+            assert status == 0
+            c_after = c_dev.cpu().numpy()
+            untouched = np.ones(c.size, dtype=bool)
+            for index in range(batch):
+                # fp16 scalars reach the kernels through the reference's truncating FloatToHalf
+                alpha = clblast_amd.half_bits_to_float(clblast_amd.float_to_half_bits(alphas[index])) if bits == 16 else alphas[index]
+                beta = clblast_amd.half_bits_to_float(clblast_amd.float_to_half_bits(betas[index])) if bits == 16 else betas[index]
+                if bits == 32:
+                    alpha, beta = float(np.float32(alpha)), float(np.float32(beta))
+                expected = oracle.gemm(layout, ta, tb, m, n, k, alpha, a, a_offsets[index], a_ld, b, 0, b_ld, beta, c,
+                                       c_offsets[index], c_ld)
+                where = oracle.c_indices(layout, m, n, c_offsets[index], c_ld)
+                assert oracle.rel_frobenius(c_after[where], expected) <= TOL[bits]
+                untouched[where.ravel()] = False
+            assert np.array_equal(c_after[untouched].view(np.uint8), c[untouched].view(np.uint8))
+
+
+def test_python_binding_mirrors_pyclblast(gpu):
+    """np.dot versus gemm for m, n, k in {1, 7, 32}, three decimals (reference:
+    src/pyclblast/test/test_pyclblast.py:65-81), through the pyclblast-shaped functions on torch tensors."""
+    for m, n, k in itertools.product((1, 7, 32), repeat=3):
+        a = np.random.default_rng(m * 100 + n * 10 + k).random((m, k)).astype(np.float32)
+        b = np.random.default_rng(7).random((k, n)).astype(np.float32)
+        c = np.zeros((m, n), dtype=np.float32)
+        a_dev, b_dev, c_dev = gpu.to_device(a), gpu.to_device(b), gpu.to_device(c)
+        clblast_amd.gemm(None, m, n, k, a_dev, b_dev, c_dev, a_ld=k, b_ld=n, c_ld=n)
+        torch.cuda.synchronize()
+        np.testing.assert_array_almost_equal(c_dev.cpu().numpy(), np.dot(a, b), 3)
+    a = np.random.default_rng(1).random((3, 8, 4)).astype(np.float64)
+    b = np.random.default_rng(2).random((3, 4, 6)).astype(np.float64)
+    c_dev = gpu.to_device(np.zeros((3, 8, 6)))
+    clblast_amd.gemmStridedBatched(None, 8, 6, 4, 3, gpu.to_device(a), gpu.to_device(b), c_dev, 4, 6, 6, 32, 24, 48)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(c_dev.cpu().numpy(), a @ b, rtol=1e-12)
+    c_dev = gpu.to_device(np.ones((3, 8, 6)))
+    clblast_amd.gemmBatched(None, 8, 6, 4, gpu.to_device(a), gpu.to_device(b), c_dev, [1.0, 2.0, 3.0], [0.0, 1.0, -1.0],
+                            4, 6, 6, [0, 32, 64], [0, 24, 48], [0, 48, 96])
+    torch.cuda.synchronize()
+    expected = np.stack([1.0 * a[0] @ b[0], 2.0 * a[1] @ b[1] + 1.0, 3.0 * a[2] @ b[2] - 1.0])
+    np.testing.assert_allclose(c_dev.cpu().numpy(), expected, rtol=1e-12)
+    with pytest.raises(clblast_amd.CLBlastError) as info:
+        clblast_amd.gemm(None, 0, 4, 4, a_dev, b_dev, c_dev.float(), 4, 4, 4)
+    assert info.value.status == -1017
