@@ -27,6 +27,10 @@ PEAK_TFLOPS = {"S": 157.3, "D": 78.6, "H": 2516.6}
 PEAK_HBM_GBS = 8000.0
 BITS = {"S": 32, "D": 64, "H": 16}
 DTYPE_NAME = {"S": "f32", "D": "f64", "H": "f16"}
+# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
+# the readings of a plain 1 GiB copy (profiles/<workload>.md holds the commands and the raw readings). A bench run
+# cannot collect counters itself, so these are the figures of the committed profiles.
+MEASURED_TRAFFIC_BYTES = {"cfg2s": 5.717e9, "cfg3": 2.291e9, "cfg4": 1.007e8}
 
 
 def parse_args():
@@ -37,6 +41,9 @@ def parse_args():
     parser.add_argument("--no-extras", action="store_true", help="only the headline workload")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     parser.add_argument("--only", default=None, help="run a single extra workload by name and exit (for profiling)")
+    parser.add_argument("--copy-calibration", action="store_true",
+                        help="also run one plain 1 GiB device-to-device copy (reads 2^30 bytes, writes 2^30 bytes): the "
+                             "known-size kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
     return parser.parse_args()
 
 
@@ -168,10 +175,10 @@ def roofline_of(workload, device_ms):
         achieved = workload.flops / seconds / 1e12
         peak = PEAK_TFLOPS[workload.prefix]
         return {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(achieved / peak, 4), "traffic": None}
+                "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(workload.name)}
     achieved = workload.algorithmic_bytes / seconds / 1e9
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-            "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": None}
+            "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(workload.name)}
 
 
 def cpu_baseline(target_seconds=15.0):
@@ -243,6 +250,14 @@ def main():
         sys.exit("bench.py: no GPU visible")
     from clblast_amd import _lib
     _lib.load()  # fails loudly when the HIP library is missing: there is no fallback
+
+    if args.copy_calibration:
+        source = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
+        target = torch.empty_like(source)
+        target.copy_(source)
+        torch.cuda.synchronize()
+        del source, target
+        torch.cuda.empty_cache()
 
     if args.only is not None:
         print(json.dumps({args.only: run_extra(args.only, args.steps, args.warmup)}))
