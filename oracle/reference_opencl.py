@@ -1,0 +1,186 @@
+"""TEST INFRASTRUCTURE ONLY: runs the REAL reference library on an OpenCL device of this machine.
+
+oracle/_ref/libclblast_ref.so is CLBlast itself (OpenCL flavour), compiled by oracle/Makefile (`make -C oracle
+ref-full`) from the reference tree where it lies. Where the OpenCL runtime exposes a device (the ROCm OpenCL
+runtime of the GPU box exposes the MI355X), this module calls the reference's own `CLBlast{S,D,H}gemm`,
+`...gemmStridedBatched` (reference: include/clblast_c.h:885-919, 1341-1370) on seeded inputs and returns the
+result and the time, so that tests can compare the HIP library with the reference on identical inputs and
+bench.py can quote the reference's speed on the same GPU. It must run in a process that has not initialised
+HIP (both runtimes in one process were seen to lose the device), hence the command-line interface:
+
+    python -m oracle.reference_opencl --spec spec.json --out result.npz
+
+spec.json: {"routine": "gemm"|"strided", "bits": 16|32|64, "layout", "ta", "tb", "m", "n", "k", "alpha", "beta",
+"a_ld", "b_ld", "c_ld", "offsets": [a, b, c], "seed": s, "low"/"high", "ab_low"/"ab_high", "batch", "strides",
+"runs": r, "sizes": [a, b, c] element counts}. Inputs are oracle.uniform(seed*3 + {0,1,2}, ...), exactly what
+tests/harness.py and the callers generate. The OpenCL host code here is a minimal ctypes binding of the
+standard OpenCL 1.2 C API; nothing of the reference is copied.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+REF_LIBRARY = os.path.join(HERE, "_ref", "libclblast_ref.so")
+CL_DEVICE_TYPE_ALL = 0xFFFFFFFF
+CL_MEM_READ_WRITE = 1
+CL_TRUE = 1
+CL_DEVICE_NAME = 0x102B
+SCALAR = {16: ctypes.c_ushort, 32: ctypes.c_float, 64: ctypes.c_double}
+PREFIX = {16: "H", 32: "S", 64: "D"}
+
+
+def available():
+    return os.path.exists(REF_LIBRARY)
+
+
+class OpenCL:
+    def __init__(self):
+        self.cl = ctypes.CDLL("libOpenCL.so.1")
+        vp, u32, sz = ctypes.c_void_p, ctypes.c_uint, ctypes.c_size_t
+        self.cl.clCreateContext.restype = vp
+        self.cl.clCreateCommandQueue.restype = vp
+        self.cl.clCreateCommandQueue.argtypes = [vp, vp, ctypes.c_ulong, ctypes.POINTER(ctypes.c_int)]
+        self.cl.clCreateBuffer.restype = vp
+        self.cl.clCreateBuffer.argtypes = [vp, ctypes.c_ulong, sz, vp, ctypes.POINTER(ctypes.c_int)]
+        self.cl.clEnqueueWriteBuffer.argtypes = [vp, vp, u32, sz, sz, vp, u32, vp, vp]
+        self.cl.clEnqueueReadBuffer.argtypes = [vp, vp, u32, sz, sz, vp, u32, vp, vp]
+        self.cl.clFinish.argtypes = [vp]
+        self.cl.clReleaseMemObject.argtypes = [vp]
+        self.cl.clWaitForEvents.argtypes = [u32, ctypes.POINTER(vp)]
+        self.cl.clReleaseEvent.argtypes = [vp]
+        count = u32(0)
+        platforms = (vp * 8)()
+        if self.cl.clGetPlatformIDs(8, platforms, ctypes.byref(count)) != 0 or count.value == 0:
+            raise RuntimeError("no OpenCL platform")
+        self.device = None
+        for index in range(count.value):
+            devices = (vp * 8)()
+            found = u32(0)
+            status = self.cl.clGetDeviceIDs(vp(platforms[index]), ctypes.c_ulong(CL_DEVICE_TYPE_ALL), 8, devices,
+                                            ctypes.byref(found))
+            if status == 0 and found.value > 0:
+                self.device = vp(devices[0])
+                break
+        if self.device is None:
+            raise RuntimeError("no OpenCL device")
+        name = ctypes.create_string_buffer(256)
+        self.cl.clGetDeviceInfo(self.device, CL_DEVICE_NAME, 256, name, None)
+        self.device_name = name.value.decode()
+        error = ctypes.c_int(0)
+        device_array = (vp * 1)(self.device)
+        self.context = vp(self.cl.clCreateContext(None, 1, device_array, None, None, ctypes.byref(error)))
+        assert error.value == 0, "clCreateContext %d" % error.value
+        self.queue = vp(self.cl.clCreateCommandQueue(self.context, self.device, 0, ctypes.byref(error)))
+        assert error.value == 0, "clCreateCommandQueue %d" % error.value
+
+    def buffer_from(self, array):
+        error = ctypes.c_int(0)
+        handle = ctypes.c_void_p(self.cl.clCreateBuffer(self.context, CL_MEM_READ_WRITE, array.nbytes, None,
+                                                        ctypes.byref(error)))
+        assert error.value == 0, "clCreateBuffer %d" % error.value
+        self.write(handle, array)
+        return handle
+
+    def write(self, handle, array):
+        status = self.cl.clEnqueueWriteBuffer(self.queue, handle, CL_TRUE, 0, array.nbytes, array.ctypes.data, 0, None, None)
+        assert status == 0, "clEnqueueWriteBuffer %d" % status
+
+    def read(self, handle, array):
+        status = self.cl.clEnqueueReadBuffer(self.queue, handle, CL_TRUE, 0, array.nbytes, array.ctypes.data, 0, None, None)
+        assert status == 0, "clEnqueueReadBuffer %d" % status
+
+    def finish(self):
+        self.cl.clFinish(self.queue)
+
+
+def scalar_argument(bits, value, reference):
+    if bits == 16:  # cl_half bit pattern; the test scalars are exactly representable
+        return ctypes.c_ushort(int(np.array([value], dtype=np.float32).astype(np.float16).view(np.uint16)[0]))
+    return SCALAR[bits](value)
+
+
+def run(spec):
+    sys.path.insert(0, os.path.dirname(HERE))
+    import oracle
+    bits = spec["bits"]
+    opencl = OpenCL()
+    reference = ctypes.CDLL(REF_LIBRARY)
+    seed = spec["seed"]
+    sizes = spec["sizes"]
+    ab_low, ab_high = spec.get("ab_low", spec.get("low", -1.0)), spec.get("ab_high", spec.get("high", 1.0))
+    a = oracle.uniform(seed * 3 + 0, sizes[0], ab_low, ab_high, bits)
+    b = oracle.uniform(seed * 3 + 1, sizes[1], ab_low, ab_high, bits)
+    c = oracle.uniform(seed * 3 + 2, sizes[2], spec.get("low", -1.0), spec.get("high", 1.0), bits)
+    a_buffer, b_buffer, c_buffer = opencl.buffer_from(a), opencl.buffer_from(b), opencl.buffer_from(c)
+    sz, vp = ctypes.c_size_t, ctypes.c_void_p
+    queue = vp(opencl.queue.value)
+    alpha, beta = scalar_argument(bits, spec["alpha"], reference), scalar_argument(bits, spec["beta"], reference)
+    offsets = spec.get("offsets", [0, 0, 0])
+    m, n, k = sz(spec["m"]), sz(spec["n"]), sz(spec["k"])
+
+    def call():
+        event = vp(None)
+        if spec["routine"] == "gemm":
+            function = getattr(reference, "CLBlast%sgemm" % PREFIX[bits])
+            status = function(ctypes.c_int(spec["layout"]), ctypes.c_int(spec["ta"]), ctypes.c_int(spec["tb"]), m, n, k,
+                              alpha, a_buffer, sz(offsets[0]), sz(spec["a_ld"]), b_buffer, sz(offsets[1]),
+                              sz(spec["b_ld"]), beta, c_buffer, sz(offsets[2]), sz(spec["c_ld"]), ctypes.byref(queue),
+                              ctypes.byref(event))
+        else:
+            strides = spec["strides"]
+            function = getattr(reference, "CLBlast%sgemmStridedBatched" % PREFIX[bits])
+            status = function(ctypes.c_int(spec["layout"]), ctypes.c_int(spec["ta"]), ctypes.c_int(spec["tb"]), m, n, k,
+                              alpha, a_buffer, sz(offsets[0]), sz(spec["a_ld"]), sz(strides[0]), b_buffer,
+                              sz(offsets[1]), sz(spec["b_ld"]), sz(strides[1]), beta, c_buffer, sz(offsets[2]),
+                              sz(spec["c_ld"]), sz(strides[2]), sz(spec["batch"]), ctypes.byref(queue),
+                              ctypes.byref(event))
+        if status == 0 and event.value:
+            events = (vp * 1)(event.value)
+            opencl.cl.clWaitForEvents(1, events)
+            opencl.cl.clReleaseEvent(event)
+        return status
+
+    status = call()  # first call: includes the reference's run-time kernel compilation
+    opencl.finish()
+    result = np.empty_like(c)
+    opencl.read(c_buffer, result)
+    times = []
+    for _ in range(spec.get("runs", 0)):  # the reference's client reports the minimum over runs, wall clock
+        opencl.write(c_buffer, c)
+        opencl.finish()
+        begin = time.perf_counter()
+        call()
+        opencl.finish()
+        times.append(time.perf_counter() - begin)
+    for handle in (a_buffer, b_buffer, c_buffer):
+        opencl.cl.clReleaseMemObject(handle)
+    return status, result, times, opencl.device_name
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--spec", required=True)
+    parser.add_argument("--out", required=True)
+    args = parser.parse_args()
+    with open(args.spec) as handle:
+        specs = json.load(handle)
+    outputs = {}
+    summary = []
+    for index, spec in enumerate(specs):
+        status, result, times, device_name = run(spec)
+        outputs["c_%d" % index] = result
+        summary.append({"status": status, "times": times, "device": device_name})
+        print("reference_opencl: case %d status %d min time %s on %s" %
+              (index, status, ("%.3f ms" % (min(times) * 1e3)) if times else "-", device_name), flush=True)
+    outputs["summary"] = np.array(json.dumps(summary))
+    np.savez(args.out, **outputs)
+
+
+if __name__ == "__main__":
+    main()
