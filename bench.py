@@ -17,6 +17,8 @@ import os
 import sys
 import time
 
+import numpy as np
+
 ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
@@ -209,6 +211,51 @@ def cpu_baseline(target_seconds=15.0):
                       "CLBlast on PoCL (no CPU OpenCL device on this host)" % (m - 1, m, seconds)}
 
 
+def reference_on_this_gpu(runs=3):
+    """Part of the baseline leg: the real reference library (oracle/_ref/libclblast_ref.so, CLBlast built from its
+    own sources, untuned for this device as upstream has no gfx950 database entry) timed on this GPU through the
+    OpenCL runtime, in a child process that never touches HIP. Wall clock around call + clFinish, minimum over
+    runs, as the reference's own client reports it (reference: test/performance/client.cpp:300-330). Returns None
+    when the library or an OpenCL device is missing."""
+    import subprocess
+    import tempfile
+    from oracle import reference_opencl
+    if not reference_opencl.available():
+        return None
+    full = lambda bits, layout, ta, tb, lo: dict(
+        routine="gemm", bits=bits, layout=layout, ta=ta, tb=tb, m=8192, n=8192, k=8192, alpha=1.0, beta=0.0, a_ld=8192,
+        b_ld=8192, c_ld=8192, offsets=[0, 0, 0], seed=7, ab_low=-lo, ab_high=lo, runs=runs, sizes=[8192 * 8192] * 3)
+    specs = {"sgemm_8192_rowTN": full(32, ROW, YES, NO, 1.0), "dgemm_8192_rowTN": full(64, ROW, YES, NO, 1.0),
+             "hgemm_8192_colNT": dict(full(16, COL, NO, YES, 0.5), beta=1.0),
+             "sgemm_1024_colNN": dict(routine="gemm", bits=32, layout=COL, ta=NO, tb=NO, m=1024, n=1024, k=1024, alpha=1.5,
+                                      beta=0.5, a_ld=1024, b_ld=1024, c_ld=1024, offsets=[0, 0, 0], seed=8, runs=10,
+                                      sizes=[1024 * 1024] * 3),
+             "sgemm_strided_batched_8192x32": dict(routine="strided", bits=32, layout=COL, ta=NO, tb=NO, m=32, n=32, k=32,
+                                                   alpha=1.0, beta=0.0, a_ld=32, b_ld=32, c_ld=32, offsets=[0, 0, 0],
+                                                   strides=[1024] * 3, batch=8192, seed=9, runs=10,
+                                                   sizes=[1024 * 8192] * 3)}
+    flops = {name: 2.0 * spec["m"] * spec["n"] * spec["k"] * spec.get("batch", 1) for name, spec in specs.items()}
+    root = os.path.dirname(os.path.abspath(__file__))
+    with tempfile.TemporaryDirectory() as folder:
+        spec_file, out_file = os.path.join(folder, "spec.json"), os.path.join(folder, "out.npz")
+        with open(spec_file, "w") as handle:
+            json.dump(list(specs.values()), handle)
+        done = subprocess.run([sys.executable, "-m", "oracle.reference_opencl", "--spec", spec_file, "--out", out_file,
+                               "--no-results"], cwd=root, capture_output=True, text=True, timeout=600)
+        if done.returncode != 0:
+            return {"error": (done.stderr or done.stdout)[-300:]}
+        summary = json.loads(str(np.load(out_file, allow_pickle=False)["summary"]))
+    report = {"what": "reference CLBlast (OpenCL, default parameters) on this GPU: min wall clock of %d runs" % runs,
+              "device": summary[0]["device"]}
+    for (name, _), entry in zip(specs.items(), summary):
+        if entry["status"] == 0 and entry["times"]:
+            seconds = min(entry["times"])
+            report[name] = {"ms": round(seconds * 1e3, 4), "gflops": round(flops[name] / seconds / 1e9, 1)}
+        else:
+            report[name] = {"status": entry["status"]}
+    return report
+
+
 EXTRA_WORKLOADS = {
     "cfg1_sgemm_1024_colNN": lambda: Workload("cfg1", "S", COL, NO, NO, 1024, 1024, 1024, 1.5, 0.5),
     "cfg2_dgemm_8192_rowTN": lambda: Workload("cfg2d", "D", ROW, YES, NO, 8192, 8192, 8192, 1.0, 0.0),
@@ -286,6 +333,7 @@ def main():
         result["other_configs"] = extras
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
+        result["cpu_baseline"]["reference_opencl_on_this_gpu"] = reference_on_this_gpu()
     print(json.dumps(result))
 
 
