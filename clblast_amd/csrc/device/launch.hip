@@ -3,6 +3,10 @@
 // dispatch of a launch descriptor to the per-precision translation units (launch_f16/f32/f64/small.hip),
 // which are the only other files that touch the HIP runtime.
 // =================================================================================================
+#include <cstring>
+#include <mutex>
+#include <vector>
+
 #include "device/launch_common.hpp"
 
 namespace clbh {
@@ -33,6 +37,52 @@ bool ValidDescriptor(const clbh_gemm_desc& d) {
   }
   if (d.a_offset < 0 || d.b_offset < 0 || d.c_offset < 0) { return false; }
   return true;
+}
+
+// Pinned staging blocks for small host-to-device uploads. The caller's memory is copied into a block
+// at once (so it may be reused on return), the block feeds a truly asynchronous copy, and an event
+// recorded behind the copy says when the block is free again. Blocks live until the process ends;
+// their number is bounded by the uploads that were ever in flight together.
+struct PinnedBlock {
+  void* host;
+  size_t bytes;
+  hipEvent_t done;
+  int device;
+  bool in_flight;
+};
+std::mutex pinned_mutex;
+std::vector<PinnedBlock> pinned_blocks;
+
+int StagedUpload(void* dst_device, const void* src_host, size_t bytes, hipStream_t stream, int device) {
+  std::lock_guard<std::mutex> lock(pinned_mutex);
+  PinnedBlock* block = nullptr;
+  for (auto& candidate : pinned_blocks) {
+    if (candidate.device != device || candidate.bytes < bytes) { continue; }
+    if (candidate.in_flight && hipEventQuery(candidate.done) == hipSuccess) { candidate.in_flight = false; }
+    if (!candidate.in_flight) { block = &candidate; break; }
+  }
+  (void)hipGetLastError();  // hipEventQuery reports "not ready" as an error code
+  if (block == nullptr) {
+    auto fresh = PinnedBlock{nullptr, size_t{64} << 10, nullptr, device, false};
+    while (fresh.bytes < bytes) { fresh.bytes *= 2; }
+    auto status = hipHostMalloc(&fresh.host, fresh.bytes, hipHostMallocDefault);
+    if (status != hipSuccess) { return static_cast<int>(status); }
+    status = hipEventCreateWithFlags(&fresh.done, hipEventDisableTiming);
+    if (status != hipSuccess) { (void)hipHostFree(fresh.host); return static_cast<int>(status); }
+    pinned_blocks.push_back(fresh);
+    block = &pinned_blocks.back();
+  }
+  std::memcpy(block->host, src_host, bytes);
+  auto status = hipMemcpyAsync(dst_device, block->host, bytes, hipMemcpyHostToDevice, stream);
+  if (status != hipSuccess) { return static_cast<int>(status); }
+  status = hipEventRecord(block->done, stream);
+  if (status != hipSuccess) {
+    // without the event the block's reuse cannot be ordered: wait here, once, and keep it free
+    (void)hipStreamSynchronize(stream);
+    return static_cast<int>(status);
+  }
+  block->in_flight = true;
+  return 0;
 }
 
 }  // namespace
@@ -73,7 +123,12 @@ int clbh_alloc_async(void** ptr, size_t bytes, hipStream_t stream) {
 int clbh_free_async(void* ptr, hipStream_t stream) { return static_cast<int>(hipFreeAsync(ptr, stream)); }
 
 int clbh_upload_async(void* dst_device, const void* src_host, size_t bytes, hipStream_t stream) {
-  return static_cast<int>(hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, stream));
+  if (dst_device == nullptr || src_host == nullptr) { return hipErrorInvalidValue; }
+  if (bytes == 0) { return 0; }
+  int device = 0;
+  auto status = clbh_stream_device(stream, &device);
+  if (status != 0) { return status; }
+  return clbh::StagedUpload(dst_device, src_host, bytes, stream, device);
 }
 
 int clbh_event_record(hipEvent_t event, hipStream_t stream) {

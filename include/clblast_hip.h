@@ -139,14 +139,16 @@ StatusCode GemmTempBufferSize(const Layout layout, const Transpose a_transpose, 
 
 // =================================================================================================
 
-// Drops per-process cached state (device properties, buffer-extent cache). Kernels are compiled ahead
-// of time, so there is no program cache to clear.
+// Kept for source compatibility: kernels are compiled ahead of time, so there is no program cache to
+// clear. Returns kSuccess and leaves parameter overrides in place.
 StatusCode ClearCache();
 
 // Overrides engine parameters for one device ordinal and precision. Accepted kernel names:
 //   "GemmRoutine": {"XGEMM_MIN_INDIRECT_SIZE": s} - problems with m*n*k < s^3 take the general
 //                  (direct) kernel, all others the MFMA-tiled kernels (reference:
 //                  src/routines/level3/xgemm.hpp:63-69, test/routines/level3/xgemm.hpp:62-70).
+//   "Xgemm":       {"TILE_VARIANT": v} - v > 0 forces tile variant v of the MFMA-tiled kernels for
+//                  that precision (for measurements and tests), 0 restores the automatic choice.
 // Any other kernel name returns kInvalidOverrideKernel, a missing parameter kMissingOverrideParameter.
 StatusCode OverrideParameters(const int device, const std::string& kernel_name, const Precision precision,
                               const std::unordered_map<std::string, size_t>& parameters);
