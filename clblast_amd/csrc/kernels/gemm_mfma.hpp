@@ -24,6 +24,8 @@
 #ifndef CLBLAST_HIP_KERNELS_GEMM_MFMA_HPP_
 #define CLBLAST_HIP_KERNELS_GEMM_MFMA_HPP_
 
+#include <type_traits>
+
 #include "kernels/gemm_args.hpp"
 
 namespace clbh {
@@ -193,6 +195,48 @@ __device__ __forceinline__ void StoreSlab(T* __restrict__ tile, const int tid, c
   }
 }
 
+// One piece of a full slab: global memory -> register vector, and register vector -> LDS tile [k][x].
+// Thread t moves the pieces t, t + THREADS, ... of the slab; with LINES = THREADS / ALONG whole lines per
+// round, piece c of a thread lies c * LINES lines after its piece 0. The address is split into a part that
+// is uniform over the work-group (64-bit, scalar registers) and the thread's byte offset inside the slab
+// (32-bit, one vector register for all pieces of an operand): a global load takes exactly this pair.
+template <int TILE_X, int TILE_K, int VL, bool KC>
+struct PieceRounds {
+  static constexpr int ALONG = PieceMap<TILE_X, TILE_K, VL, KC>::ALONG;
+  static_assert(kMfmaThreads % ALONG == 0, "whole lines per round of pieces");
+  static constexpr int LINES = kMfmaThreads / ALONG;
+};
+
+template <typename T, int TILE_X, int TILE_K, int VL, bool KC>
+__device__ __forceinline__ unsigned int PieceLaneBytes(const long long ld, const int tid) {
+  using Rounds = PieceRounds<TILE_X, TILE_K, VL, KC>;
+  const int line = tid / Rounds::ALONG, pos = (tid % Rounds::ALONG) * VL;
+  return static_cast<unsigned int>((line * ld + pos) * static_cast<long long>(sizeof(T)));
+}
+
+// `slab` points at the slab's first element (x0, k0) and must be uniform over the work-group.
+template <typename T, int TILE_X, int TILE_K, int VL, bool KC>
+__device__ __forceinline__ typename VecType<T, VL>::type LoadPiece(const T* __restrict__ slab, const long long ld,
+                                                                   const unsigned int lane_bytes, const int c) {
+  using Rounds = PieceRounds<TILE_X, TILE_K, VL, KC>;
+  const char* round = reinterpret_cast<const char*>(slab + static_cast<long long>(c * Rounds::LINES) * ld);
+  return *reinterpret_cast<const typename VecType<T, VL>::type*>(round + lane_bytes);
+}
+
+template <typename T, int TILE_X, int TILE_K, int PITCH, int VL, bool KC>
+__device__ __forceinline__ void StorePiece(T* __restrict__ tile, const int tid, const int c,
+                                           const typename VecType<T, VL>::type v) {
+  using V = typename VecType<T, VL>::type;
+  int x, k;
+  PieceMap<TILE_X, TILE_K, VL, KC>::Get(tid + c * kMfmaThreads, x, k);
+  if (KC) {
+#pragma unroll
+    for (int e = 0; e < VL; ++e) { tile[(k + e) * PITCH + x] = VecGet<V, T, VL>(v, e); }
+  } else {
+    *reinterpret_cast<V*>(&tile[k * PITCH + x]) = v;
+  }
+}
+
 // ---- blockIdx -> tile ------------------------------------------------------------------------------
 __device__ __forceinline__ void TileOfBlock(const int block, const int num_blocks, const int tiles_m,
                                             const int tiles_n, int& tile_m, int& tile_n) {
@@ -318,9 +362,112 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
       }
     };
 
-    // Software-pipelined walk over the full slabs (edge tiles load with x predication).
+    // Software-pipelined walk over the full slabs.
     const int fast_slabs = full_slabs;
-    if (fast_slabs > 0) {
+    if (a_full && b_full && fast_slabs > 0) {
+      // Interior tiles: explicit schedule, so that the matrix pipe never waits at a slab boundary even
+      // with one wavefront per SIMD. Per k-step: LDS reads of the fragments of the NEXT k-step (other
+      // register set), the FM x FN MFMAs of this k-step, then a share of "store staged slab t+1 into
+      // the other LDS buffer, refill the staging registers with slab t+2". One barrier per slab, before
+      // its last k-step: by then every wavefront has finished its reads of the current buffer and its
+      // stores to the other one, so the last k-step already fetches the first fragments of slab t+1.
+      constexpr int KSTEPS = TILE_K / KP;
+      static_assert(KSTEPS % 2 == 0, "fragment register sets alternate per k-step");
+      constexpr int SLOTS = KSTEPS - 1;
+      constexpr int PER_SLOT = (PIECES_A + PIECES_B + SLOTS - 1) / SLOTS;
+      using VP = typename VecType<T, VL>::type;
+      VP a_stage[PIECES_A], b_stage[PIECES_B];
+      const unsigned int a_lane_bytes = PieceLaneBytes<T, TILE_M, TILE_K, VL, A_KC>(p.a_ld, tid);
+      const unsigned int b_lane_bytes = PieceLaneBytes<T, TILE_N, TILE_K, VL, B_KC>(p.b_ld, tid);
+      const T* a_tile0 = a + (A_KC ? m0 * p.a_ld : static_cast<long long>(m0));  // element (m0, k = 0), uniform
+      const T* b_tile0 = b + (B_KC ? n0 * p.b_ld : static_cast<long long>(n0));
+      auto load_piece = [&](const int piece, const int k0) {
+        if (piece < PIECES_A) {
+          a_stage[piece] = LoadPiece<T, TILE_M, TILE_K, VL, A_KC>(a_tile0 + (A_KC ? static_cast<long long>(k0) : k0 * p.a_ld),
+                                                                 p.a_ld, a_lane_bytes, piece);
+        } else {
+          b_stage[piece - PIECES_A] = LoadPiece<T, TILE_N, TILE_K, VL, B_KC>(
+              b_tile0 + (B_KC ? static_cast<long long>(k0) : k0 * p.b_ld), p.b_ld, b_lane_bytes, piece - PIECES_A);
+        }
+      };
+      auto store_piece = [&](const int piece, T* a_dst, T* b_dst) {
+        if (piece < PIECES_A) { StorePiece<T, TILE_M, TILE_K, PITCH_M, VL, A_KC>(a_dst, tid, piece, a_stage[piece]); }
+        else { StorePiece<T, TILE_N, TILE_K, PITCH_N, VL, B_KC>(b_dst, tid, piece - PIECES_A, b_stage[piece - PIECES_A]); }
+      };
+      auto read_a = [&](const T* tile, const int ks) {
+        const int k = ks * KP + lane_g;
+        VM av;
+        if constexpr (M_INTERLEAVED) {
+          av = *reinterpret_cast<const VM*>(&tile[k * PITCH_M + a_read]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < FM; ++i) { av = VecWith<VM, T, FM>(av, i, tile[k * PITCH_M + a_read + i * MF]); }
+        }
+        return av;
+      };
+      auto read_b = [&](const T* tile, const int ks) {
+        return *reinterpret_cast<const VN*>(&tile[(ks * KP + lane_g) * PITCH_N + b_read]);
+      };
+#pragma unroll
+      for (int piece = 0; piece < PIECES_A + PIECES_B; ++piece) { load_piece(piece, 0); }
+#pragma unroll
+      for (int piece = 0; piece < PIECES_A + PIECES_B; ++piece) { store_piece(piece, a_tiles, b_tiles); }
+      if (fast_slabs > 1) {
+#pragma unroll
+        for (int piece = 0; piece < PIECES_A + PIECES_B; ++piece) { load_piece(piece, TILE_K); }
+      }
+      __syncthreads();
+      VM av[2];
+      VN bv[2];
+      av[0] = read_a(a_tiles, 0);
+      bv[0] = read_b(b_tiles, 0);
+      auto slab_body = [&](const int slab, auto store_tag, auto load_tag) {
+        constexpr bool STORE = decltype(store_tag)::value, LOAD = decltype(load_tag)::value;
+        const int cur = slab & 1;
+        const T* a_cur = a_tiles + cur * TILE_K * PITCH_M;
+        const T* b_cur = b_tiles + cur * TILE_K * PITCH_N;
+        T* a_nxt = a_tiles + (cur ^ 1) * TILE_K * PITCH_M;
+        T* b_nxt = b_tiles + (cur ^ 1) * TILE_K * PITCH_N;
+        const int k_load = (slab + 2) * TILE_K;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const int set = ks % 2;
+          if (ks + 1 < KSTEPS) {
+            av[set ^ 1] = read_a(a_cur, ks + 1);
+            bv[set ^ 1] = read_b(b_cur, ks + 1);
+          } else {
+            av[set ^ 1] = read_a(a_nxt, 0);
+            bv[set ^ 1] = read_b(b_nxt, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int i = 0; i < FM; ++i) {
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+              acc[i][j] = Traits::Mfma(VecGet<VN, T, FN>(bv[set], j), VecGet<VM, T, FM>(av[set], i), acc[i][j]);
+            }
+          }
+          if (ks < KSTEPS - 1) {
+#pragma unroll
+            for (int u = 0; u < PER_SLOT; ++u) {
+              const int piece = ks * PER_SLOT + u;
+              if (piece < PIECES_A + PIECES_B) {
+                if (STORE) { store_piece(piece, a_nxt, b_nxt); }
+                if (LOAD) { load_piece(piece, k_load); }
+              }
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if (ks == KSTEPS - 2) { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+        }
+      };
+      int slab = 0;
+      for (; slab + 2 < fast_slabs; ++slab) { slab_body(slab, std::true_type{}, std::true_type{}); }
+      if (slab + 1 < fast_slabs) { slab_body(slab, std::true_type{}, std::false_type{}); ++slab; }
+      slab_body(slab, std::false_type{}, std::false_type{});
+      __syncthreads();
+    } else if (fast_slabs > 0) {
+      // Edge tiles: same double buffering, loads predicated along x, order left to the compiler.
       load(0);
       store(0);
       __syncthreads();
