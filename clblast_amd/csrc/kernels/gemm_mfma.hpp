@@ -26,6 +26,10 @@
 
 #include <type_traits>
 
+#ifndef CLBH_EXP_NO_DIRECT
+#define CLBH_EXP_NO_DIRECT 0
+#endif
+
 #include "kernels/gemm_args.hpp"
 
 namespace clbh {
@@ -237,6 +241,51 @@ __device__ __forceinline__ void StorePiece(T* __restrict__ tile, const int tid, 
   }
 }
 
+// ---- direct global -> LDS loads (x-contiguous, 16-byte aligned operands on interior tiles) ----------
+// One `buffer_load_dwordx4 ... lds` moves 16 bytes per lane straight into LDS, lane l landing at
+// base + 16 * l: a wavefront fills 1 KiB of contiguous LDS per instruction and no vector register or
+// LDS store instruction is spent on staging. A slab [k][x] is therefore kept as groups of R whole rows
+// (R * TILE_X * sizeof(T) == 1 KiB, or one row in several instructions when a row is longer), groups
+// GROUP_PITCH elements apart. An operand that is staged through registers uses the same description
+// with R == 1, i.e. plain rows of pitch TILE_X + PAD.
+template <typename T, int TILE_X, int TILE_K, bool DIRECT>
+struct SlabLayout {
+  static constexpr int VEC = 16 / sizeof(T);
+  static constexpr int WAVE_ELEMS = 1024 / sizeof(T);                       // elements per wavefront-wide load
+  static constexpr int R = (DIRECT && TILE_X < WAVE_ELEMS) ? WAVE_ELEMS / TILE_X : 1;  // rows per group
+  static constexpr int PARTS = (DIRECT && TILE_X > WAVE_ELEMS) ? TILE_X / WAVE_ELEMS : 1;  // loads per row
+  static constexpr int GROUPS = TILE_K / R;
+  static constexpr int GROUP_PITCH = R * TILE_X + VEC;
+  static constexpr int ELEMS = GROUPS * GROUP_PITCH;                         // one stage
+  static constexpr int LOADS = GROUPS * PARTS;                               // wavefront-wide loads per slab
+  static constexpr int LOADS_PER_WAVE = (LOADS + 3) / 4;
+  static_assert(TILE_K % R == 0, "whole groups per slab");
+  // offset of element (k, 0)
+  static __device__ __forceinline__ int Row(const int k) { return (k / R) * GROUP_PITCH + (k % R) * TILE_X; }
+};
+
+// Issues the `round`-th direct load of this wavefront for one slab. `slab` points at the slab's first
+// element (x0, k0), `stage` at the LDS stage; both are uniform over the work-group.
+template <typename T, int TILE_X, int TILE_K>
+__device__ __forceinline__ void DirectLoad(const T* __restrict__ slab, const long long ld, T* stage, const int wave,
+                                           const int lane, const int round) {
+  using L = SlabLayout<T, TILE_X, TILE_K, true>;
+  const int index = wave + 4 * round;
+  if (L::LOADS % 4 != 0 && index >= L::LOADS) { return; }
+  const int group = index / L::PARTS, part = index % L::PARTS;
+  const int in_group = lane * L::VEC;                                      // element of the 1 KiB chunk
+  const int row = (L::R > 1) ? in_group / TILE_X : 0, x = (L::R > 1) ? in_group % TILE_X : in_group;
+  const int lane_bytes = static_cast<int>((row * ld + x) * static_cast<long long>(sizeof(T)));
+  const T* chunk = slab + static_cast<long long>(group * L::R) * ld + part * L::WAVE_ELEMS;
+  // Buffer form of the load (untyped raw buffer over the rest of the address space, no range check
+  // needed on interior tiles): unlike the flat-encoded global form it leaves the LDS counter alone, so
+  // waits on LDS reads stay counted instead of draining the queue.
+  const __amdgpu_buffer_rsrc_t resource = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(chunk), 0, -1, 0x00020000);
+  typedef __attribute__((address_space(3))) void* LdsPtr;
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(resource, (LdsPtr)(stage + group * L::GROUP_PITCH + part * L::WAVE_ELEMS), 16,
+                                           lane_bytes, 0, 0, 0);
+}
+
 // ---- blockIdx -> tile ------------------------------------------------------------------------------
 __device__ __forceinline__ void TileOfBlock(const int block, const int num_blocks, const int tiles_m,
                                             const int tiles_n, int& tile_m, int& tile_n) {
@@ -367,67 +416,90 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
     if (a_full && b_full && fast_slabs > 0) {
       // Interior tiles: explicit schedule, so that the matrix pipe never waits at a slab boundary even
       // with one wavefront per SIMD. Per k-step: LDS reads of the fragments of the NEXT k-step (other
-      // register set), the FM x FN MFMAs of this k-step, then a share of "store staged slab t+1 into
-      // the other LDS buffer, refill the staging registers with slab t+2". One barrier per slab, before
-      // its last k-step: by then every wavefront has finished its reads of the current buffer and its
-      // stores to the other one, so the last k-step already fetches the first fragments of slab t+1.
+      // register set), the FM x FN MFMAs of this k-step, then a share of the data movement for the
+      // coming slabs. An x-contiguous aligned operand goes global -> LDS directly (slab t+1, issued in
+      // the first k-step of slab t); any other operand is staged through registers ("store staged slab
+      // t+1 into the other LDS buffer, refill the staging registers with slab t+2"). One barrier per
+      // slab, before its last k-step: by then every wavefront has finished its reads of the current
+      // buffer and its writes to the other one, so the last k-step already fetches the first fragments
+      // of slab t+1.
       constexpr int KSTEPS = TILE_K / KP;
       static_assert(KSTEPS % 2 == 0, "fragment register sets alternate per k-step");
+      constexpr bool A_DIRECT = !A_KC && ALIGNED && !CLBH_EXP_NO_DIRECT, B_DIRECT = !B_KC && ALIGNED && !CLBH_EXP_NO_DIRECT;
+      using LA = SlabLayout<T, TILE_M, TILE_K, A_DIRECT>;
+      using LB = SlabLayout<T, TILE_N, TILE_K, B_DIRECT>;
+      static_assert(2 * (LA::ELEMS + LB::ELEMS) <= Config::LDS_ELEMS, "LDS allocation covers both layouts");
+      constexpr int STAGED_A = A_DIRECT ? 0 : PIECES_A, STAGED_B = B_DIRECT ? 0 : PIECES_B;
+      constexpr int STAGED = STAGED_A + STAGED_B;
       constexpr int SLOTS = KSTEPS - 1;
-      constexpr int PER_SLOT = (PIECES_A + PIECES_B + SLOTS - 1) / SLOTS;
+      constexpr int PER_SLOT = (STAGED + SLOTS - 1) / SLOTS;
+      T* a_stages = lds;                        // [2][LA::ELEMS]
+      T* b_stages = lds + 2 * LA::ELEMS;        // [2][LB::ELEMS]
+      const int wave_u = __builtin_amdgcn_readfirstlane(wave);
       using VP = typename VecType<T, VL>::type;
-      VP a_stage[PIECES_A], b_stage[PIECES_B];
+      VP a_stage[STAGED_A > 0 ? STAGED_A : 1], b_stage[STAGED_B > 0 ? STAGED_B : 1];
       const unsigned int a_lane_bytes = PieceLaneBytes<T, TILE_M, TILE_K, VL, A_KC>(p.a_ld, tid);
       const unsigned int b_lane_bytes = PieceLaneBytes<T, TILE_N, TILE_K, VL, B_KC>(p.b_ld, tid);
       const T* a_tile0 = a + (A_KC ? m0 * p.a_ld : static_cast<long long>(m0));  // element (m0, k = 0), uniform
       const T* b_tile0 = b + (B_KC ? n0 * p.b_ld : static_cast<long long>(n0));
+      auto a_slab = [&](const int k0) { return a_tile0 + (A_KC ? static_cast<long long>(k0) : k0 * p.a_ld); };
+      auto b_slab = [&](const int k0) { return b_tile0 + (B_KC ? static_cast<long long>(k0) : k0 * p.b_ld); };
       auto load_piece = [&](const int piece, const int k0) {
-        if (piece < PIECES_A) {
-          a_stage[piece] = LoadPiece<T, TILE_M, TILE_K, VL, A_KC>(a_tile0 + (A_KC ? static_cast<long long>(k0) : k0 * p.a_ld),
-                                                                 p.a_ld, a_lane_bytes, piece);
-        } else {
-          b_stage[piece - PIECES_A] = LoadPiece<T, TILE_N, TILE_K, VL, B_KC>(
-              b_tile0 + (B_KC ? static_cast<long long>(k0) : k0 * p.b_ld), p.b_ld, b_lane_bytes, piece - PIECES_A);
-        }
+        if (piece < STAGED_A) { a_stage[piece] = LoadPiece<T, TILE_M, TILE_K, VL, A_KC>(a_slab(k0), p.a_ld, a_lane_bytes, piece); }
+        else { b_stage[piece - STAGED_A] = LoadPiece<T, TILE_N, TILE_K, VL, B_KC>(b_slab(k0), p.b_ld, b_lane_bytes, piece - STAGED_A); }
       };
       auto store_piece = [&](const int piece, T* a_dst, T* b_dst) {
-        if (piece < PIECES_A) { StorePiece<T, TILE_M, TILE_K, PITCH_M, VL, A_KC>(a_dst, tid, piece, a_stage[piece]); }
-        else { StorePiece<T, TILE_N, TILE_K, PITCH_N, VL, B_KC>(b_dst, tid, piece - PIECES_A, b_stage[piece - PIECES_A]); }
+        if (piece < STAGED_A) { StorePiece<T, TILE_M, TILE_K, LA::GROUP_PITCH, VL, A_KC>(a_dst, tid, piece, a_stage[piece]); }
+        else { StorePiece<T, TILE_N, TILE_K, LB::GROUP_PITCH, VL, B_KC>(b_dst, tid, piece - STAGED_A, b_stage[piece - STAGED_A]); }
       };
-      auto read_a = [&](const T* tile, const int ks) {
-        const int k = ks * KP + lane_g;
+      auto direct_loads = [&](const int k0, T* a_dst, T* b_dst) {
+        if constexpr (A_DIRECT) {
+#pragma unroll
+          for (int round = 0; round < LA::LOADS_PER_WAVE; ++round) { DirectLoad<T, TILE_M, TILE_K>(a_slab(k0), p.a_ld, a_dst, wave_u, lane, round); }
+        }
+        if constexpr (B_DIRECT) {
+#pragma unroll
+          for (int round = 0; round < LB::LOADS_PER_WAVE; ++round) { DirectLoad<T, TILE_N, TILE_K>(b_slab(k0), p.b_ld, b_dst, wave_u, lane, round); }
+        }
+      };
+      const int a_lane_row = LA::Row(lane_g) + a_read, b_lane_row = LB::Row(lane_g) + b_read;
+      auto read_a = [&](const T* stage, const int ks) {
+        const T* src = stage + LA::Row(ks * KP) + a_lane_row;
         VM av;
         if constexpr (M_INTERLEAVED) {
-          av = *reinterpret_cast<const VM*>(&tile[k * PITCH_M + a_read]);
+          av = *reinterpret_cast<const VM*>(src);
         } else {
 #pragma unroll
-          for (int i = 0; i < FM; ++i) { av = VecWith<VM, T, FM>(av, i, tile[k * PITCH_M + a_read + i * MF]); }
+          for (int i = 0; i < FM; ++i) { av = VecWith<VM, T, FM>(av, i, src[i * MF]); }
         }
         return av;
       };
-      auto read_b = [&](const T* tile, const int ks) {
-        return *reinterpret_cast<const VN*>(&tile[(ks * KP + lane_g) * PITCH_N + b_read]);
+      auto read_b = [&](const T* stage, const int ks) {
+        return *reinterpret_cast<const VN*>(stage + LB::Row(ks * KP) + b_lane_row);
       };
+      static_assert((KP % LA::R == 0 || LA::R % KP == 0) && (KP % LB::R == 0 || LB::R % KP == 0), "row offsets add up");
+      direct_loads(0, a_stages, b_stages);
 #pragma unroll
-      for (int piece = 0; piece < PIECES_A + PIECES_B; ++piece) { load_piece(piece, 0); }
+      for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, 0); }
 #pragma unroll
-      for (int piece = 0; piece < PIECES_A + PIECES_B; ++piece) { store_piece(piece, a_tiles, b_tiles); }
+      for (int piece = 0; piece < STAGED; ++piece) { store_piece(piece, a_stages, b_stages); }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       if (fast_slabs > 1) {
 #pragma unroll
-        for (int piece = 0; piece < PIECES_A + PIECES_B; ++piece) { load_piece(piece, TILE_K); }
+        for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, TILE_K); }
       }
       __syncthreads();
       VM av[2];
       VN bv[2];
-      av[0] = read_a(a_tiles, 0);
-      bv[0] = read_b(b_tiles, 0);
+      av[0] = read_a(a_stages, 0);
+      bv[0] = read_b(b_stages, 0);
       auto slab_body = [&](const int slab, auto store_tag, auto load_tag) {
         constexpr bool STORE = decltype(store_tag)::value, LOAD = decltype(load_tag)::value;
         const int cur = slab & 1;
-        const T* a_cur = a_tiles + cur * TILE_K * PITCH_M;
-        const T* b_cur = b_tiles + cur * TILE_K * PITCH_N;
-        T* a_nxt = a_tiles + (cur ^ 1) * TILE_K * PITCH_M;
-        T* b_nxt = b_tiles + (cur ^ 1) * TILE_K * PITCH_N;
+        const T* a_cur = a_stages + cur * LA::ELEMS;
+        const T* b_cur = b_stages + cur * LB::ELEMS;
+        T* a_nxt = a_stages + (cur ^ 1) * LA::ELEMS;
+        T* b_nxt = b_stages + (cur ^ 1) * LB::ELEMS;
         const int k_load = (slab + 2) * TILE_K;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
@@ -447,18 +519,27 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
               acc[i][j] = Traits::Mfma(VecGet<VN, T, FN>(bv[set], j), VecGet<VM, T, FM>(av[set], i), acc[i][j]);
             }
           }
+          // the other buffer is free since the barrier of the previous slab
+          if (ks == 0 && STORE) { direct_loads((slab + 1) * TILE_K, a_nxt, b_nxt); }
           if (ks < KSTEPS - 1) {
 #pragma unroll
             for (int u = 0; u < PER_SLOT; ++u) {
               const int piece = ks * PER_SLOT + u;
-              if (piece < PIECES_A + PIECES_B) {
+              if (piece < STAGED) {
                 if (STORE) { store_piece(piece, a_nxt, b_nxt); }
                 if (LOAD) { load_piece(piece, k_load); }
               }
             }
           }
           __builtin_amdgcn_sched_barrier(0);
-          if (ks == KSTEPS - 2) { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+          if (ks == KSTEPS - 2) {
+            // direct loads of this slab are older than its register loads: all but those must have landed
+            if ((A_DIRECT || B_DIRECT) && STORE) {
+              if (LOAD && STAGED > 0) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(STAGED) : "memory"); }
+              else { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+          }
         }
       };
       int slab = 0;
