@@ -14,8 +14,8 @@
 //     operand block. An x-contiguous operand (x = m for A, n for B) is kept as [k][x] (pitch
 //     tile + 32 halfs) and read with the CDNA4 transposing LDS read ds_read_b64_tr_b16, which hands
 //     each lane four consecutive k of its own x: the transpose costs no VALU work and no extra pass;
-//   * the n-indexed fragment is the MFMA's A operand and the m-indexed one its B operand, so the
-//     lanes of every accumulator register run along m, the contiguous index of the column-major C.
+//   * the m-indexed fragment is the MFMA's A operand, so a lane holds runs of four consecutive m; the
+//     epilogue stages each block column through LDS and moves C in whole 16-byte pieces along m.
 // =================================================================================================
 #ifndef CLBLAST_HIP_KERNELS_GEMM_MFMA_F16_HPP_
 #define CLBLAST_HIP_KERNELS_GEMM_MFMA_F16_HPP_
@@ -233,7 +233,7 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
       for (int i = 0; i < FM; ++i) {
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b_frag[j], a_frag[i], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag[i], b_frag[j], acc[i][j], 0, 0, 0);
         }
       }
     };
@@ -295,7 +295,7 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
               __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
               for (int j = 0; j < FN; ++j) {
-                acc[q][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b_frag[set][j], a_frag[set][q], acc[q][j], 0, 0, 0);
+                acc[q][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag[set][q], b_frag[set][j], acc[q][j], 0, 0, 0);
               }
               if (ks < KSTEPS - 1) {
                 const int slot = ks * FM + q;
@@ -347,19 +347,86 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
       __syncthreads();
     }
 
-    // Epilogue: lane owns m = m_blk + lane%32; accumulator element r is the column n_blk + Row(r).
+    // Epilogue, staged through LDS so that global memory sees whole lines. The m-indexed fragment is the
+    // MFMA's A operand: accumulator elements 4g..4g+3 of a lane are the rows m = 8g + 4*(lane/32) + 0..3 of
+    // column n = lane%32 of the 32 x 32 block. Per block column j a wavefront owns a [32 n][WAVE_M m] fp16
+    // staging tile of its own: C (when beta != 0) comes in with 16-byte accesses along m, every lane
+    // combines its four consecutive m in fp32 and rounds once, and the finished rows leave with 16-byte
+    // stores. Only wavefront-local ordering is needed (LDS operations of a wavefront complete in order).
+    {
+      constexpr int WAVE_M = FM * 32, STAGE_PITCH = WAVE_M + 8;
+      constexpr int LANES_PER_ROW = WAVE_M / 8, ROWS_PER_PASS = 64 / LANES_PER_ROW, PASSES = 32 / ROWS_PER_PASS;
+      static_assert((THREADS / 64) * 32 * STAGE_PITCH * 2 <= Config::LDS_BYTES, "staging tiles fit the slab buffers");
+      T* stage = lds + wave * (32 * STAGE_PITCH);
+      const int wave_m0 = m0 + wave_m * WAVE_M;
+      const bool vector_rows = ALIGNED && (wave_m0 + WAVE_M <= p.m) && (p.c_ld % 8 == 0) &&
+                               ((reinterpret_cast<unsigned long long>(c) & 15) == 0);
+      auto wave_fence = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      };
+      // moves the staging tile's rows from (LOAD) or to (!LOAD) the block column starting at n_blk
+      auto rows = [&](const int n_blk, auto load_tag) {
+        constexpr bool LOAD = decltype(load_tag)::value;
+        if (vector_rows) {
 #pragma unroll
-    for (int i = 0; i < FM; ++i) {
-      const int m = m0 + (wave_m * FM + i) * 32 + lane % 32;
+          for (int pass = 0; pass < PASSES; ++pass) {
+            const int row = pass * ROWS_PER_PASS + lane / LANES_PER_ROW, col = 8 * (lane % LANES_PER_ROW);
+            if (n_blk + row < p.n) {
+              T* global = c + (n_blk + row) * p.c_ld + wave_m0 + col;
+              half8_t* local = reinterpret_cast<half8_t*>(&stage[row * STAGE_PITCH + col]);
+              if (LOAD) { *local = *reinterpret_cast<const half8_t*>(global); }
+              else { *reinterpret_cast<half8_t*>(global) = *local; }
+            }
+          }
+        } else {
+#pragma unroll 1
+          for (int row = 0; row < 32; ++row) {
+            if (n_blk + row >= p.n) { break; }
+#pragma unroll
+            for (int col = lane; col < WAVE_M; col += 64) {
+              if (wave_m0 + col < p.m) {
+                T* global = c + (n_blk + row) * p.c_ld + wave_m0 + col;
+                if (LOAD) { stage[row * STAGE_PITCH + col] = *global; }
+                else { *global = stage[row * STAGE_PITCH + col]; }
+              }
+            }
+          }
+        }
+      };
+      __syncthreads();  // every wavefront is done with the slab buffers
 #pragma unroll
       for (int j = 0; j < FN; ++j) {
         const int n_blk = n0 + (wave_n * FN + j) * 32;
+        if (n_blk < p.n && wave_m0 < p.m) {
+          if (beta != 0.0f) {
+            rows(n_blk, std::true_type{});
+            wave_fence();
+          }
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int n = n_blk + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-          if (m < p.m && n < p.n) { StoreResult<T, float>(c, n * p.c_ld + m, acc[i][j][r], alpha, beta); }
+          for (int i = 0; i < FM; ++i) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              half4_t* cell = reinterpret_cast<half4_t*>(&stage[(lane % 32) * STAGE_PITCH + 32 * i + 8 * g + 4 * (lane / 32)]);
+              half4_t out;
+              if (beta != 0.0f) {
+                const half4_t old = *cell;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { out[e] = static_cast<T>(alpha * acc[i][j][4 * g + e] + beta * static_cast<float>(old[e])); }
+              } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { out[e] = static_cast<T>(alpha * acc[i][j][4 * g + e]); }
+              }
+              *cell = out;
+            }
+          }
+          wave_fence();
+          rows(n_blk, std::false_type{});
+          wave_fence();
         }
       }
+      __syncthreads();  // the next batch entry refills the slab buffers
     }
   }
 }
