@@ -4,7 +4,6 @@
 #include "device/launch_common.hpp"
 #include "kernels/gemm_general.hpp"
 #include "kernels/gemm_mfma_f16.hpp"
-#include "kernels/gemm_mfma_f16_big.hpp"
 
 namespace clbh {
 namespace {
@@ -60,34 +59,6 @@ int LaunchHgemmConfig(const clbh_gemm_desc& d, hipStream_t stream) {
   }
 }
 
-template <typename Config, bool A_KC, bool B_KC>
-int LaunchHgemmBigVariant(const clbh_gemm_desc& d, hipStream_t stream) {
-  const auto args = MakeArgs<float>(d);
-  const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
-  const long long tiles_n = (d.n + Config::TILE_N - 1) / Config::TILE_N;
-  if (tiles_m * tiles_n > INT_MAX) { return hipErrorInvalidConfiguration; }
-  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
-  constexpr size_t lds_bytes = Config::LDS_BYTES;
-  auto kernel = HgemmBigKernel<Config, A_KC, B_KC>;
-  static const hipError_t attribute_status = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
-  if (attribute_status != hipSuccess) { return static_cast<int>(attribute_status); }
-  kernel<<<grid, dim3(Config::THREADS), lds_bytes, stream>>>(args, static_cast<int>(tiles_m), static_cast<int>(tiles_n));
-  return static_cast<int>(hipGetLastError());
-}
-
-// Needs 16-byte aligned operands (checked by the caller).
-template <typename Config>
-int LaunchHgemmBig(const clbh_gemm_desc& d, hipStream_t stream) {
-  const int variant = (d.a_kcontig ? 2 : 0) | (d.b_kcontig ? 1 : 0);
-  switch (variant) {
-    case 0: return LaunchHgemmBigVariant<Config, false, false>(d, stream);
-    case 1: return LaunchHgemmBigVariant<Config, false, true>(d, stream);
-    case 2: return LaunchHgemmBigVariant<Config, true, false>(d, stream);
-    default: return LaunchHgemmBigVariant<Config, true, true>(d, stream);
-  }
-}
-
 }  // namespace
 
 int LaunchMfmaF16(const clbh_gemm_desc& d, hipStream_t stream) {
@@ -96,9 +67,10 @@ int LaunchMfmaF16(const clbh_gemm_desc& d, hipStream_t stream) {
   if (!Aligned16<_Float16>(d)) { return LaunchHgemmConfig<Small, false>(d, stream); }
   switch (d.tile_variant) {
     case 1: return LaunchHgemmConfig<HgemmConfig<2, 4, 4, 2, 32, 2, false>, true>(d, stream);  // 256 x 256 x 32, 8 waves
-    case 2: return LaunchHgemmConfig<HgemmConfig<2, 4, 4, 2, 32, 2, true>, true>(d, stream);   // 256 x 256 x 32, 8 waves, pipelined
-    case 3: return LaunchHgemmBig<HgemmBigConfig<2, 2, 4, 4, 1>>(d, stream);                   // 256 x 256 x 64 swizzled, 4 waves
-    case 4: return LaunchHgemmBig<HgemmBigConfig<2, 4, 4, 2, 2>>(d, stream);                   // 256 x 256 x 64 swizzled, 8 waves
+    // 256 x 256 x 32, 8 waves, explicitly scheduled, direct global -> LDS loads into a ring of 4 / 3 / 2 slabs
+    case 2: return LaunchHgemmConfig<HgemmConfig<2, 4, 4, 2, 32, 2, true, 4>, true>(d, stream);
+    case 3: return LaunchHgemmConfig<HgemmConfig<2, 4, 4, 2, 32, 2, true, 3>, true>(d, stream);
+    case 4: return LaunchHgemmConfig<HgemmConfig<2, 4, 4, 2, 32, 2, true, 2>, true>(d, stream);
     default: return LaunchHgemmConfig<Small, true>(d, stream);
   }
 }

@@ -25,20 +25,6 @@
 #include "kernels/gemm_args.hpp"
 #include "kernels/gemm_mfma.hpp"
 
-// Timing experiments only (results are wrong when set): never defined by the product build.
-#ifndef CLBH_EXPERIMENT_NO_LOADS
-#define CLBH_EXPERIMENT_NO_LOADS 0
-#endif
-#ifndef CLBH_EXPERIMENT_NO_BARRIER
-#define CLBH_EXPERIMENT_NO_BARRIER 0
-#endif
-#ifndef CLBH_EXPERIMENT_NO_STORES
-#define CLBH_EXPERIMENT_NO_STORES 0
-#endif
-#ifndef CLBH_EXPERIMENT_NO_READS
-#define CLBH_EXPERIMENT_NO_READS 0
-#endif
-
 namespace clbh {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -48,8 +34,9 @@ typedef short short4_t __attribute__((ext_vector_type(4)));
 // WM x WN wavefronts per work-group, each owning FM x FN MFMA blocks of 32 x 32. MIN_WAVES is the number
 // of wavefronts per SIMD the register budget must allow. PIPELINED selects the explicitly scheduled main
 // loop (see HgemmMfmaKernel); it needs FM >= FN and an even number of k-steps per slab.
-template <int WM_, int WN_, int FM_, int FN_, int TILE_K_, int MIN_WAVES_, bool PIPELINED_>
+template <int WM_, int WN_, int FM_, int FN_, int TILE_K_, int MIN_WAVES_, bool PIPELINED_, int STAGES_ = 2>
 struct HgemmConfig {
+  static constexpr int STAGES = STAGES_;  // LDS slab buffers of the pipelined loop
   static constexpr int WM = WM_, WN = WN_, FM = FM_, FN = FN_, MIN_WAVES = MIN_WAVES_;
   static constexpr bool PIPELINED = PIPELINED_;
   static constexpr int THREADS = 64 * WM * WN;
@@ -63,10 +50,16 @@ struct HgemmConfig {
   static constexpr int B_ELEMS_KC = TILE_N * PITCH_KC, B_ELEMS_XC = TILE_K * PITCH_XN;
   static constexpr int A_ELEMS = A_ELEMS_KC > A_ELEMS_XC ? A_ELEMS_KC : A_ELEMS_XC;
   static constexpr int B_ELEMS = B_ELEMS_KC > B_ELEMS_XC ? B_ELEMS_KC : B_ELEMS_XC;
-  static constexpr int LDS_BYTES = 2 * (A_ELEMS + B_ELEMS) * 2;
+  // the pipelined loop keeps STAGES slabs per operand in the direct-load layouts (HDirectLayout, <= 544 halfs
+  // per KiB of slab)
+  static constexpr int DIRECT_ELEMS = (TILE_M + TILE_N) * TILE_K / 512 * 544;
+  static constexpr int PLAIN_BYTES = 2 * (A_ELEMS + B_ELEMS) * 2;
+  static constexpr int DIRECT_BYTES = PIPELINED_ ? STAGES_ * DIRECT_ELEMS * 2 : 0;
+  static constexpr int LDS_BYTES = PLAIN_BYTES > DIRECT_BYTES ? PLAIN_BYTES : DIRECT_BYTES;
   static_assert(TILE_K % 16 == 0, "slab depth is a multiple of the MFMA k extent");
   static_assert((TILE_M * TILE_K) % (8 * THREADS) == 0 && (TILE_N * TILE_K) % (8 * THREADS) == 0, "slab split");
-  static_assert(!PIPELINED || (FM >= FN && (TILE_K / 16) % 2 == 0), "pipelined loop shape");
+  static_assert(!PIPELINED || (FM >= FN && TILE_K == 32 && TILE_M == 256 && TILE_N == 256 && THREADS == 512 && STAGES >= 2),
+                "pipelined loop shape");
 };
 
 // ---- slab movement ---------------------------------------------------------------------------------
@@ -163,6 +156,79 @@ __device__ __forceinline__ half8_t HReadFragment(const _Float16* __restrict__ ti
   }
 }
 
+// ---- direct global -> LDS slabs for the pipelined loop (256 x 32 halfs per operand and slab) ---------
+// `buffer_load_dwordx4 ... lds` puts lane l's 16 bytes at base + 16 * l, so LDS is filled in 1 KiB pieces
+// whose inner layout is fixed; which 16 bytes of global memory a lane fetches is free, and that freedom
+// carries the bank swizzle.
+//   x-contiguous operand: a piece is two k rows of 256 halfs; in the odd row the 16-byte chunk t of the
+//     row sits at position t ^ 2. Pieces are 544 halfs apart. The transposing read of a 16-lane group then
+//     touches rows k..k+3 in four different 32-byte bank windows.
+//   k-contiguous operand: a piece is 16 x rows of 32 halfs (4 chunks); chunk c of row r sits at position
+//     c ^ ((r >> 2) & 3), so the 16-byte reads of 16 consecutive rows cover all 64 banks once.
+template <bool KC>
+struct HDirectLayout {
+  static constexpr int PIECE_PITCH = KC ? 512 : 544;  // halfs
+  static constexpr int PIECES = 16;                   // per operand and slab
+  static constexpr int ELEMS = PIECES * PIECE_PITCH;
+};
+
+// Issues the round-th (0 or 1) piece load of this wavefront; `slab` points at element (x0, k0), uniform.
+template <bool KC>
+__device__ __forceinline__ void HDirectLoad(const _Float16* __restrict__ slab, const long long ld, _Float16* stage,
+                                            const int wave, const int lane, const int round) {
+  const int piece = wave + 8 * round;
+  const _Float16* source;
+  int lane_elems;
+  if (KC) {
+    const int row = lane / 4, chunk = (lane % 4) ^ ((row >> 2) & 3);
+    source = slab + static_cast<long long>(16 * piece) * ld;
+    lane_elems = static_cast<int>(row * ld) + 8 * chunk;
+  } else {
+    const int row = lane / 32, chunk = (lane % 32) ^ (2 * row);
+    source = slab + static_cast<long long>(2 * piece) * ld;
+    lane_elems = static_cast<int>(row * ld) + 8 * chunk;
+  }
+  const __amdgpu_buffer_rsrc_t resource = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(source), 0, -1, 0x00020000);
+  typedef __attribute__((address_space(3))) void* LdsPtr;
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(resource, (LdsPtr)(stage + piece * HDirectLayout<KC>::PIECE_PITCH), 16,
+                                           lane_elems * 2, 0, 0, 0);
+}
+
+// Lane-constant part of a fragment address in a direct-layout stage, for the block starting at x32 = 0 and
+// k-step 0; HDirectFragment adds the block and k-step.
+template <bool KC>
+__device__ __forceinline__ int HDirectLaneOffset(const int lane) {
+  if (KC) {
+    const int row = lane % 16;
+    return ((lane % 32) / 16) * 512 + row * 32 + 8 * ((lane / 32) ^ ((row >> 2) & 3));
+  } else {
+    const int group = lane / 16, q = lane % 16, parity = (q / 4) % 2;
+    const int x = (16 * (group % 2) + 4 * (q % 4)) ^ (16 * parity);
+    return (4 * (group / 2) + (q / 4) / 2) * 544 + parity * 256 + x;
+  }
+}
+
+// Fragment of block x32 (a multiple of 32) and k-step ks (0 or 1) of a direct-layout stage.
+template <bool KC>
+__device__ __forceinline__ half8_t HDirectFragment(const _Float16* __restrict__ stage, const int lane_offset, const int x32,
+                                                   const int ks) {
+  if (KC) {
+    // chunk index of the k-step is 2*ks + lane/32; the swizzle is an XOR, so k-step 1 flips bit 1 of it
+    const int offset = (x32 / 16) * 512 + (lane_offset ^ (ks * 16));
+    return *reinterpret_cast<const half8_t*>(&stage[offset]);
+  } else {
+    typedef __attribute__((address_space(3))) short4_t* LdsPtr;
+    const _Float16* src = stage + ks * 8 * 544 + x32 + lane_offset;
+    const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(src));
+    const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(src + 2 * 544));
+    half8_t out;
+    const half4_t lo_h = __builtin_bit_cast(half4_t, lo), hi_h = __builtin_bit_cast(half4_t, hi);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { out[e] = lo_h[e]; out[4 + e] = hi_h[e]; }
+    return out;
+  }
+}
+
 // ---- the kernel ------------------------------------------------------------------------------------
 template <typename Config, bool A_KC, bool B_KC, bool ALIGNED>
 __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaKernel(const GemmArgs<float> p, const int tiles_m,
@@ -251,35 +317,59 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
     // Interior tiles: software-pipelined walk over the full slabs.
     const int fast_slabs = interior ? full_slabs : 0;
     if constexpr (Config::PIPELINED && ALIGNED) {
-      // Explicit schedule for one wavefront per SIMD, where nothing but the instruction order inside the
-      // wavefront can hide latency. Per slab (KSTEPS k-steps of FM quarters each):
+      // Explicit schedule for few wavefronts per SIMD, where little but the instruction order inside the
+      // wavefront hides latency. Slabs go global -> LDS directly into a ring of STAGES buffers: the loads
+      // of slab t+STAGES-1 are issued at the start of slab t (its buffer was released by the barrier of
+      // slab t-1) and have STAGES-2 slabs plus one k-step to land. Per slab (2 k-steps of FM quarters):
       //   quarter q of k-step s:  LDS reads of the a/b fragments q of k-step s+1 (other register set),
-      //                           then the FN MFMAs of block row q of k-step s,
-      //                           then a share of: store staged slab t+1 into the other LDS buffer and
-      //                           refill the staging registers with slab t+2 from global memory.
+      //                           then the FN MFMAs of block row q of k-step s.
       //   One barrier per slab, before the last k-step: by then every wavefront has issued all its reads
-      //   of the current buffer and all its stores to the other one, so the last k-step can already
+      //   of the current buffer, and slab t+1 has landed for everybody, so the last k-step can already
       //   fetch the first fragments of slab t+1. Scheduling fences pin this order for the compiler.
-      constexpr int KSTEPS = TILE_K / 16;
-      constexpr int SLOTS = (KSTEPS - 1) * FM;                       // quarters before the barrier
-      constexpr int PER_SLOT = (PIECES_A + PIECES_B + SLOTS - 1) / SLOTS;
+      constexpr int KSTEPS = TILE_K / 16, STAGES = Config::STAGES;
+      constexpr int LOADS_PER_SLAB = 4;  // per wavefront: two pieces of A, two of B
+      using LA = HDirectLayout<A_KC>;
+      using LB = HDirectLayout<B_KC>;
+      static_assert(STAGES * (LA::ELEMS + LB::ELEMS) * 2 <= Config::LDS_BYTES, "LDS allocation covers the ring");
       if (fast_slabs > 0) {
-        load(0);
-        store(0);
-        if (fast_slabs > 1) { load(1); }
+        T* a_ring = lds;
+        T* b_ring = lds + STAGES * LA::ELEMS;
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+        const T* a_tile0 = a + (A_KC ? m0 * p.a_ld : static_cast<long long>(m0));  // element (m0, k = 0), uniform
+        const T* b_tile0 = b + (B_KC ? n0 * p.b_ld : static_cast<long long>(n0));
+        auto issue = [&](const int slab, const int buffer) {
+          const int k0 = slab * TILE_K;
+          const T* a_slab = a_tile0 + (A_KC ? static_cast<long long>(k0) : k0 * p.a_ld);
+          const T* b_slab = b_tile0 + (B_KC ? static_cast<long long>(k0) : k0 * p.b_ld);
+#pragma unroll
+          for (int round = 0; round < 2; ++round) {
+            HDirectLoad<A_KC>(a_slab, p.a_ld, a_ring + buffer * LA::ELEMS, wave_u, lane, round);
+            HDirectLoad<B_KC>(b_slab, p.b_ld, b_ring + buffer * LB::ELEMS, wave_u, lane, round);
+          }
+        };
+        const int a_lane = HDirectLaneOffset<A_KC>(lane), b_lane = HDirectLaneOffset<B_KC>(lane);
+#pragma unroll
+        for (int s = 0; s < STAGES - 1; ++s) {
+          if (s < fast_slabs) { issue(s, s); }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         half8_t a_frag[2][FM], b_frag[2][FN];
-        read_fragments(a_tiles, b_tiles, 0, a_frag[0], b_frag[0]);
-        // One slab. STORE: the staging registers hold slab+1 and go to the other LDS buffer; LOAD: they are
-        // refilled with slab+2. Both are compile-time so that the steady state has no branches.
-        auto slab_body = [&](const int slab, auto store_tag, auto load_tag) {
-          constexpr bool STORE = decltype(store_tag)::value, LOAD = decltype(load_tag)::value;
-          const int cur = slab & 1;
-          const T* a_cur = a_tiles + cur * Config::A_ELEMS;
-          const T* b_cur = b_tiles + cur * Config::B_ELEMS;
-          T* a_nxt = a_tiles + (cur ^ 1) * Config::A_ELEMS;
-          T* b_nxt = b_tiles + (cur ^ 1) * Config::B_ELEMS;
-          const int k_load = (slab + 2) * TILE_K;
+#pragma unroll
+        for (int q = 0; q < FM; ++q) { a_frag[0][q] = HDirectFragment<A_KC>(a_ring, a_lane, (wave_m * FM + q) * 32, 0); }
+#pragma unroll
+        for (int q = 0; q < FN; ++q) { b_frag[0][q] = HDirectFragment<B_KC>(b_ring, b_lane, (wave_n * FN + q) * 32, 0); }
+        int cur = 0;  // buffer of the current slab; the next slab is in cur + 1, the free one is cur - 1 (mod STAGES)
+        // One slab. ISSUE: slab + STAGES - 1 exists and is requested; compile-time, so that the steady state has
+        // no branches.
+        auto slab_body = [&](const int slab, auto issue_tag) {
+          constexpr bool ISSUE = decltype(issue_tag)::value;
+          const int nxt = (cur + 1 == STAGES) ? 0 : cur + 1;
+          const int free_buffer = (cur == 0) ? STAGES - 1 : cur - 1;
+          const T* a_cur = a_ring + cur * LA::ELEMS;
+          const T* b_cur = b_ring + cur * LB::ELEMS;
+          const T* a_nxt = a_ring + nxt * LA::ELEMS;
+          const T* b_nxt = b_ring + nxt * LB::ELEMS;
 #pragma unroll
           for (int ks = 0; ks < KSTEPS; ++ks) {
             const int set = ks % 2;
@@ -288,42 +378,29 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
             const int ks_src = (ks + 1 < KSTEPS) ? ks + 1 : 0;
 #pragma unroll
             for (int q = 0; q < FM; ++q) {
-              a_frag[set ^ 1][q] = HReadFragment<PITCH_A, A_KC>(a_src, (wave_m * FM + q) * 32, ks_src * 16, lane);
-              if (q < FN) {
-                b_frag[set ^ 1][q] = HReadFragment<PITCH_B, B_KC>(b_src, (wave_n * FN + q) * 32, ks_src * 16, lane);
-              }
+              a_frag[set ^ 1][q] = HDirectFragment<A_KC>(a_src, a_lane, (wave_m * FM + q) * 32, ks_src);
+              if (q < FN) { b_frag[set ^ 1][q] = HDirectFragment<B_KC>(b_src, b_lane, (wave_n * FN + q) * 32, ks_src); }
               __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
               for (int j = 0; j < FN; ++j) {
                 acc[q][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag[set][q], b_frag[set][j], acc[q][j], 0, 0, 0);
               }
-              if (ks < KSTEPS - 1) {
-                const int slot = ks * FM + q;
-#pragma unroll
-                for (int u = 0; u < PER_SLOT; ++u) {
-                  const int piece = slot * PER_SLOT + u;
-                  if (piece < PIECES_A) {
-                    if (STORE) { HStorePiece<THREADS, TILE_M, TILE_K, PITCH_A, A_KC>(a_nxt, tid, piece, a_regs[piece]); }
-                    if (LOAD && !CLBH_EXPERIMENT_NO_LOADS) { a_regs[piece] = HLoadPiece<THREADS, TILE_M, TILE_K, A_KC>(a, p.a_ld, m0, k_load, tid, piece); }
-                  } else if (piece < PIECES_A + PIECES_B) {
-                    const int pb = piece - PIECES_A;
-                    if (STORE) { HStorePiece<THREADS, TILE_N, TILE_K, PITCH_B, B_KC>(b_nxt, tid, pb, b_regs[pb]); }
-                    if (LOAD && !CLBH_EXPERIMENT_NO_LOADS) { b_regs[pb] = HLoadPiece<THREADS, TILE_N, TILE_K, B_KC>(b, p.b_ld, n0, k_load, tid, pb); }
-                  }
-                }
-              }
+              if (ISSUE && ks == 0 && q == 0) { issue(slab + STAGES - 1, free_buffer); }
               __builtin_amdgcn_sched_barrier(0);
             }
             if (ks == KSTEPS - 2) {
-              if (CLBH_EXPERIMENT_NO_BARRIER) { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-              else { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+              // slab + 1 must have landed; in the steady state the loads of the STAGES - 2 slabs after it may
+              // still be in flight (loads complete in order)
+              if (ISSUE) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * LOADS_PER_SLAB) : "memory"); }
+              else { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+              asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
             }
           }
+          cur = nxt;
         };
         int slab = 0;
-        for (; slab + 2 < fast_slabs; ++slab) { slab_body(slab, std::true_type{}, std::true_type{}); }
-        if (slab + 1 < fast_slabs) { slab_body(slab, std::true_type{}, std::false_type{}); ++slab; }
-        slab_body(slab, std::false_type{}, std::false_type{});
+        for (; slab + STAGES - 1 < fast_slabs; ++slab) { slab_body(slab, std::true_type{}); }
+        for (; slab < fast_slabs; ++slab) { slab_body(slab, std::false_type{}); }
         __syncthreads();
       }
     } else if (fast_slabs > 0) {

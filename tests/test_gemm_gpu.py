@@ -121,3 +121,34 @@ def test_alpha_zero_is_not_special(gpu, bits, path):
         assert np.array_equal(rest, np.delete(problem.c[index], 3, axis=0))
     finally:
         gpu.force_path(bits, None)
+
+
+TILE_VARIANTS = {32: range(1, 9), 64: range(1, 6), 16: range(1, 5)}
+
+
+@pytest.mark.parametrize("bits", BITS)
+def test_every_tile_variant(gpu, bits):
+    """Each tile of the MFMA family (normally picked by shape) is forced in turn on shapes that reach its
+    interior tiles, its edge tiles, its K tail and its unaligned instance, for all four operand
+    orientations."""
+    import clblast_amd
+    gpu.force_path(bits, "indirect")
+    try:
+        seed = 7000
+        for variant in TILE_VARIANTS[bits]:
+            clblast_amd.override_parameters(0, "Xgemm", bits, {"TILE_VARIANT": variant})
+            for (ta, tb) in itertools.product(TRANSPOSES, TRANSPOSES):
+                for (m, n, k), extra, offsets in (((512, 512, 256), (0, 0, 0), (0, 0, 0)),
+                                                  ((520, 264, 200), (8, 8, 8), (8, 16, 24)),
+                                                  ((300, 270, 100), (3, 5, 7), (11, 13, 19))):
+                    seed += 1
+                    problem = gpu.Problem(bits, COL_MAJOR, ta, tb, m, n, k, 0.5, 2.0 if seed % 2 else 0.0,
+                                          a_offset=offsets[0], b_offset=offsets[1], c_offset=offsets[2], seed=seed,
+                                          extra_ld=extra)
+                    status, c_after = problem.run()
+                    assert status == 0, (variant, problem.describe())
+                    problem.check(c_after)
+    finally:
+        import clblast_amd
+        clblast_amd.override_parameters(0, "Xgemm", bits, {"TILE_VARIANT": 0})
+        gpu.force_path(bits, None)
