@@ -50,9 +50,9 @@ struct HgemmConfig {
   static constexpr int B_ELEMS_KC = TILE_N * PITCH_KC, B_ELEMS_XC = TILE_K * PITCH_XN;
   static constexpr int A_ELEMS = A_ELEMS_KC > A_ELEMS_XC ? A_ELEMS_KC : A_ELEMS_XC;
   static constexpr int B_ELEMS = B_ELEMS_KC > B_ELEMS_XC ? B_ELEMS_KC : B_ELEMS_XC;
-  // the pipelined loop keeps STAGES slabs per operand in the direct-load layouts (HDirectLayout, <= 544 halfs
+  // the pipelined loop keeps STAGES slabs per operand in the direct-load layouts (HDirectLayout, <= 576 halfs
   // per KiB of slab)
-  static constexpr int DIRECT_ELEMS = (TILE_M + TILE_N) * TILE_K / 512 * 544;
+  static constexpr int DIRECT_ELEMS = (TILE_M + TILE_N) * TILE_K / 512 * 576;
   static constexpr int PLAIN_BYTES = 2 * (A_ELEMS + B_ELEMS) * 2;
   static constexpr int DIRECT_BYTES = PIPELINED_ ? STAGES_ * DIRECT_ELEMS * 2 : 0;
   static constexpr int LDS_BYTES = PLAIN_BYTES > DIRECT_BYTES ? PLAIN_BYTES : DIRECT_BYTES;
@@ -161,13 +161,13 @@ __device__ __forceinline__ half8_t HReadFragment(const _Float16* __restrict__ ti
 // whose inner layout is fixed; which 16 bytes of global memory a lane fetches is free, and that freedom
 // carries the bank swizzle.
 //   x-contiguous operand: a piece is two k rows of 256 halfs; in the odd row the 16-byte chunk t of the
-//     row sits at position t ^ 2. Pieces are 544 halfs apart. The transposing read of a 16-lane group then
-//     touches rows k..k+3 in four different 32-byte bank windows.
+//     row sits at position t ^ 4. Pieces are 576 halfs apart. LDS serves 32 lanes of a transposing read per
+//     cycle: rows k..k+3, 64 bytes each, which this layout spreads over eight different 32-byte bank windows.
 //   k-contiguous operand: a piece is 16 x rows of 32 halfs (4 chunks); chunk c of row r sits at position
 //     c ^ ((r >> 2) & 3), so the 16-byte reads of 16 consecutive rows cover all 64 banks once.
 template <bool KC>
 struct HDirectLayout {
-  static constexpr int PIECE_PITCH = KC ? 512 : 544;  // halfs
+  static constexpr int PIECE_PITCH = KC ? 512 : 576;  // halfs
   static constexpr int PIECES = 16;                   // per operand and slab
   static constexpr int ELEMS = PIECES * PIECE_PITCH;
 };
@@ -184,7 +184,7 @@ __device__ __forceinline__ void HDirectLoad(const _Float16* __restrict__ slab, c
     source = slab + static_cast<long long>(16 * piece) * ld;
     lane_elems = static_cast<int>(row * ld) + 8 * chunk;
   } else {
-    const int row = lane / 32, chunk = (lane % 32) ^ (2 * row);
+    const int row = lane / 32, chunk = (lane % 32) ^ (4 * row);
     source = slab + static_cast<long long>(2 * piece) * ld;
     lane_elems = static_cast<int>(row * ld) + 8 * chunk;
   }
@@ -194,33 +194,31 @@ __device__ __forceinline__ void HDirectLoad(const _Float16* __restrict__ slab, c
                                            lane_elems * 2, 0, 0, 0);
 }
 
-// Lane-constant part of a fragment address in a direct-layout stage, for the block starting at x32 = 0 and
-// k-step 0; HDirectFragment adds the block and k-step.
+// Offset of a lane's fragment data for the block starting at x32 (a multiple of 32), k-step 0, in a
+// direct-layout stage; constant over the whole K walk.
 template <bool KC>
-__device__ __forceinline__ int HDirectLaneOffset(const int lane) {
+__device__ __forceinline__ int HDirectLaneOffset(const int lane, const int x32) {
   if (KC) {
     const int row = lane % 16;
-    return ((lane % 32) / 16) * 512 + row * 32 + 8 * ((lane / 32) ^ ((row >> 2) & 3));
+    return (x32 / 16 + (lane % 32) / 16) * 512 + row * 32 + 8 * ((lane / 32) ^ ((row >> 2) & 3));
   } else {
     const int group = lane / 16, q = lane % 16, parity = (q / 4) % 2;
-    const int x = (16 * (group % 2) + 4 * (q % 4)) ^ (16 * parity);
-    return (4 * (group / 2) + (q / 4) / 2) * 544 + parity * 256 + x;
+    const int x = (x32 + 16 * (group % 2) + 4 * (q % 4)) ^ (32 * parity);  // odd rows hold chunk t at t ^ 4
+    return (4 * (group / 2) + (q / 4) / 2) * 576 + parity * 256 + x;
   }
 }
 
-// Fragment of block x32 (a multiple of 32) and k-step ks (0 or 1) of a direct-layout stage.
+// Fragment of k-step ks (0 or 1) of a direct-layout stage, for the lane offset of its block.
 template <bool KC>
-__device__ __forceinline__ half8_t HDirectFragment(const _Float16* __restrict__ stage, const int lane_offset, const int x32,
-                                                   const int ks) {
+__device__ __forceinline__ half8_t HDirectFragment(const _Float16* __restrict__ stage, const int lane_offset, const int ks) {
   if (KC) {
     // chunk index of the k-step is 2*ks + lane/32; the swizzle is an XOR, so k-step 1 flips bit 1 of it
-    const int offset = (x32 / 16) * 512 + (lane_offset ^ (ks * 16));
-    return *reinterpret_cast<const half8_t*>(&stage[offset]);
+    return *reinterpret_cast<const half8_t*>(&stage[lane_offset ^ (ks * 16)]);
   } else {
     typedef __attribute__((address_space(3))) short4_t* LdsPtr;
-    const _Float16* src = stage + ks * 8 * 544 + x32 + lane_offset;
+    const _Float16* src = stage + ks * 8 * 576 + lane_offset;
     const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(src));
-    const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(src + 2 * 544));
+    const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(src + 2 * 576));
     half8_t out;
     const half4_t lo_h = __builtin_bit_cast(half4_t, lo), hi_h = __builtin_bit_cast(half4_t, hi);
 #pragma unroll
@@ -347,7 +345,11 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
             HDirectLoad<B_KC>(b_slab, p.b_ld, b_ring + buffer * LB::ELEMS, wave_u, lane, round);
           }
         };
-        const int a_lane = HDirectLaneOffset<A_KC>(lane), b_lane = HDirectLaneOffset<B_KC>(lane);
+        int a_lane[FM], b_lane[FN];
+#pragma unroll
+        for (int q = 0; q < FM; ++q) { a_lane[q] = HDirectLaneOffset<A_KC>(lane, (wave_m * FM + q) * 32); }
+#pragma unroll
+        for (int q = 0; q < FN; ++q) { b_lane[q] = HDirectLaneOffset<B_KC>(lane, (wave_n * FN + q) * 32); }
 #pragma unroll
         for (int s = 0; s < STAGES - 1; ++s) {
           if (s < fast_slabs) { issue(s, s); }
@@ -356,9 +358,9 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
         __syncthreads();
         half8_t a_frag[2][FM], b_frag[2][FN];
 #pragma unroll
-        for (int q = 0; q < FM; ++q) { a_frag[0][q] = HDirectFragment<A_KC>(a_ring, a_lane, (wave_m * FM + q) * 32, 0); }
+        for (int q = 0; q < FM; ++q) { a_frag[0][q] = HDirectFragment<A_KC>(a_ring, a_lane[q], 0); }
 #pragma unroll
-        for (int q = 0; q < FN; ++q) { b_frag[0][q] = HDirectFragment<B_KC>(b_ring, b_lane, (wave_n * FN + q) * 32, 0); }
+        for (int q = 0; q < FN; ++q) { b_frag[0][q] = HDirectFragment<B_KC>(b_ring, b_lane[q], 0); }
         int cur = 0;  // buffer of the current slab; the next slab is in cur + 1, the free one is cur - 1 (mod STAGES)
         // One slab. ISSUE: slab + STAGES - 1 exists and is requested; compile-time, so that the steady state has
         // no branches.
@@ -378,8 +380,8 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
             const int ks_src = (ks + 1 < KSTEPS) ? ks + 1 : 0;
 #pragma unroll
             for (int q = 0; q < FM; ++q) {
-              a_frag[set ^ 1][q] = HDirectFragment<A_KC>(a_src, a_lane, (wave_m * FM + q) * 32, ks_src);
-              if (q < FN) { b_frag[set ^ 1][q] = HDirectFragment<B_KC>(b_src, b_lane, (wave_n * FN + q) * 32, ks_src); }
+              a_frag[set ^ 1][q] = HDirectFragment<A_KC>(a_src, a_lane[q], ks_src);
+              if (q < FN) { b_frag[set ^ 1][q] = HDirectFragment<B_KC>(b_src, b_lane[q], ks_src); }
               __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
               for (int j = 0; j < FN; ++j) {

@@ -86,9 +86,10 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     return KernelChoice{CLBH_KERNEL_MFMA, static_cast<int>(forced) - 1, 1};
   }
   if (precision == Precision::kHalf) {
-    // 256 x 256 tiles (8 wavefronts, index 2) once there are at least two per CU, else 128 x 128
+    // 256 x 256 tiles (8 wavefronts, ring of 3 direct-loaded slabs: index 3) once there are at least two per CU,
+    // else 128 x 128
     const auto big_tiles = CeilDivide(m, 256) * CeilDivide(n, 256);
-    return KernelChoice{CLBH_KERNEL_MFMA, (big_tiles >= 512) ? 2 : 0, 1};
+    return KernelChoice{CLBH_KERNEL_MFMA, (big_tiles >= 512) ? 3 : 0, 1};
   }
   if (precision == Precision::kSingle) {
     auto tile = Tile{1, 128, 128};
