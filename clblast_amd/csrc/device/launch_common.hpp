@@ -74,6 +74,15 @@ inline bool Aligned16(const clbh_gemm_desc& d) {
   return true;
 }
 
+// The tiled kernels address a slab with 32-bit byte offsets from a per-load base: up to 64 lines of a
+// k-contiguous operand, up to 8 rows of an x-contiguous one. Operands whose leading dimension is too
+// large for that take the general kernel.
+template <typename T>
+inline bool LeadingDimsFitTiles(const clbh_gemm_desc& d) {
+  const auto limit = [](bool kcontig) { return static_cast<long long>((1ull << 32) / ((kcontig ? 64 : 8) * sizeof(T))); };
+  return d.a_ld < limit(d.a_kcontig != 0) && d.b_ld < limit(d.b_kcontig != 0);
+}
+
 // Split-K geometry of a descriptor: K range per split (a multiple of 64) and the workspace leading dimension.
 struct SplitPlan {
   int splits, chunk, ld;

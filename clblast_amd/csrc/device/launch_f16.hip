@@ -62,6 +62,7 @@ int LaunchHgemmConfig(const clbh_gemm_desc& d, hipStream_t stream) {
 }  // namespace
 
 int LaunchMfmaF16(const clbh_gemm_desc& d, hipStream_t stream) {
+  if (!LeadingDimsFitTiles<_Float16>(d)) { return LaunchGeneral<_Float16>(d, stream); }
   // The large tiles exist for 16-byte aligned operands only; everything else takes 128 x 128.
   using Small = HgemmConfig<2, 2, 2, 2, 32, 2, false>;  // 128 x 128 x 32, 4 waves
   if (!Aligned16<_Float16>(d)) { return LaunchHgemmConfig<Small, false>(d, stream); }

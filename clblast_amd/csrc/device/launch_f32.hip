@@ -8,6 +8,7 @@ namespace {
 }  // namespace
 
 int LaunchMfmaF32(const clbh_gemm_desc& d, hipStream_t stream) {
+  if (!LeadingDimsFitTiles<float>(d)) { return LaunchGeneral<float>(d, stream); }
   switch (d.tile_variant) {
     case 1: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16, 3>>(d, stream);
     case 2: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16, 4>>(d, stream);

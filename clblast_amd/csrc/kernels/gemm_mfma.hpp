@@ -24,11 +24,8 @@
 #ifndef CLBLAST_HIP_KERNELS_GEMM_MFMA_HPP_
 #define CLBLAST_HIP_KERNELS_GEMM_MFMA_HPP_
 
+#include <tuple>
 #include <type_traits>
-
-#ifndef CLBH_EXP_NO_DIRECT
-#define CLBH_EXP_NO_DIRECT 0
-#endif
 
 #include "kernels/gemm_args.hpp"
 
@@ -109,181 +106,131 @@ __device__ __forceinline__ V VecWith(V v, const int i, const T value) {
   return v;
 }
 
-// ---- slab loaders ----------------------------------------------------------------------------------
-// One operand slab is TILE_X x TILE_K elements. `base` points at element (x = 0, k = 0) of the matrix of
-// this batch; the element (x, k) lives at base[KC ? x*ld + k : k*ld + x]. Every thread moves PIECES
-// pieces of VL elements (VL = 16 bytes' worth when every address is 16-byte aligned, else 1). The
-// piece -> (x, k) mapping puts consecutive threads along the contiguous index of the operand in
-// memory, so a wavefront's accesses coalesce for either orientation.
-template <int TILE_X, int TILE_K, int VL, bool KC>
-struct PieceMap {
-  static constexpr int ALONG = (KC ? TILE_K : TILE_X) / VL;  // pieces per contiguous line of the slab
-  static __device__ __forceinline__ void Get(const int piece, int& x, int& k) {
-    const int line = piece / ALONG, pos = (piece % ALONG) * VL;
-    x = KC ? line : pos;
-    k = KC ? pos : line;
-  }
-};
-
-// Fast path: the whole slab is inside the matrix.
-template <typename T, int TILE_X, int TILE_K, int PIECES, int VL, bool KC>
-__device__ __forceinline__ void LoadSlab(const T* __restrict__ base, const long long ld, const int x0, const int k0,
-                                         const int tid, T (&regs)[PIECES][VL]) {
-  using Map = PieceMap<TILE_X, TILE_K, VL, KC>;
-  using V = typename VecType<T, VL>::type;
-#pragma unroll
-  for (int c = 0; c < PIECES; ++c) {
-    int x, k;
-    Map::Get(tid + c * kMfmaThreads, x, k);
-    const T* src = KC ? base + (x0 + x) * ld + (k0 + k) : base + (k0 + k) * ld + (x0 + x);
-    const V v = *reinterpret_cast<const V*>(src);
-#pragma unroll
-    for (int e = 0; e < VL; ++e) { regs[c][e] = VecGet<V, T, VL>(v, e); }
-  }
-}
-
-// Register-staged load of a slab whose x range sticks out of the matrix (the k range is complete):
-// elements beyond x_end read as zero. Keeps edge tiles on the pipelined path.
-template <typename T, int TILE_X, int TILE_K, int PIECES, int VL, bool KC>
-__device__ __forceinline__ void LoadSlabEdge(const T* __restrict__ base, const long long ld, const int x0, const int k0,
-                                             const int x_end, const int tid, T (&regs)[PIECES][VL]) {
-  using Map = PieceMap<TILE_X, TILE_K, VL, KC>;
-#pragma unroll
-  for (int c = 0; c < PIECES; ++c) {
-    int x, k;
-    Map::Get(tid + c * kMfmaThreads, x, k);
-#pragma unroll
-    for (int e = 0; e < VL; ++e) {
-      const int gx = x0 + x + (KC ? 0 : e), gk = k0 + k + (KC ? e : 0);
-      regs[c][e] = (gx < x_end) ? (KC ? base[gx * ld + gk] : base[gk * ld + gx]) : T(0);
-    }
-  }
-}
-
-// Edge tiles and the K tail: element-wise, bounds-checked copy straight into the LDS tile [k][x] (no
-// register staging, no overlap with the multiplication). Elements outside the matrix become zero.
-template <typename T, int TILE_X, int TILE_K, int PITCH, bool KC>
-__device__ __forceinline__ void FillSlabChecked(T* __restrict__ tile, const T* __restrict__ base, const long long ld,
-                                                const int x0, const int k0, const int x_end, const int k_end,
-                                                const int tid) {
-  using Map = PieceMap<TILE_X, TILE_K, 1, KC>;
-#pragma unroll 4
-  for (int piece = tid; piece < TILE_X * TILE_K; piece += kMfmaThreads) {
-    int x, k;
-    Map::Get(piece, x, k);
-    const int gx = x0 + x, gk = k0 + k;
-    T value = T(0);
-    if (gx < x_end && gk < k_end) { value = KC ? base[gx * ld + gk] : base[gk * ld + gx]; }
-    tile[k * PITCH + x] = value;
-  }
-}
-
-// Registers -> LDS tile [k][x] with row pitch PITCH.
-template <typename T, int TILE_X, int TILE_K, int PITCH, int PIECES, int VL, bool KC>
-__device__ __forceinline__ void StoreSlab(T* __restrict__ tile, const int tid, const T (&regs)[PIECES][VL]) {
-  using Map = PieceMap<TILE_X, TILE_K, VL, KC>;
-  using V = typename VecType<T, VL>::type;
-#pragma unroll
-  for (int c = 0; c < PIECES; ++c) {
-    int x, k;
-    Map::Get(tid + c * kMfmaThreads, x, k);
-    if (KC) {
-#pragma unroll
-      for (int e = 0; e < VL; ++e) { tile[(k + e) * PITCH + x] = regs[c][e]; }
-    } else {
-      V v;
-#pragma unroll
-      for (int e = 0; e < VL; ++e) { v = VecWith<V, T, VL>(v, e, regs[c][e]); }
-      *reinterpret_cast<V*>(&tile[k * PITCH + x]) = v;
-    }
-  }
-}
-
-// One piece of a full slab: global memory -> register vector, and register vector -> LDS tile [k][x].
-// Thread t moves the pieces t, t + THREADS, ... of the slab; with LINES = THREADS / ALONG whole lines per
-// round, piece c of a thread lies c * LINES lines after its piece 0. The address is split into a part that
-// is uniform over the work-group (64-bit, scalar registers) and the thread's byte offset inside the slab
-// (32-bit, one vector register for all pieces of an operand): a global load takes exactly this pair.
-template <int TILE_X, int TILE_K, int VL, bool KC>
-struct PieceRounds {
-  static constexpr int ALONG = PieceMap<TILE_X, TILE_K, VL, KC>::ALONG;
-  static_assert(kMfmaThreads % ALONG == 0, "whole lines per round of pieces");
-  static constexpr int LINES = kMfmaThreads / ALONG;
-};
-
-template <typename T, int TILE_X, int TILE_K, int VL, bool KC>
-__device__ __forceinline__ unsigned int PieceLaneBytes(const long long ld, const int tid) {
-  using Rounds = PieceRounds<TILE_X, TILE_K, VL, KC>;
-  const int line = tid / Rounds::ALONG, pos = (tid % Rounds::ALONG) * VL;
-  return static_cast<unsigned int>((line * ld + pos) * static_cast<long long>(sizeof(T)));
-}
-
-// `slab` points at the slab's first element (x0, k0) and must be uniform over the work-group.
-template <typename T, int TILE_X, int TILE_K, int VL, bool KC>
-__device__ __forceinline__ typename VecType<T, VL>::type LoadPiece(const T* __restrict__ slab, const long long ld,
-                                                                   const unsigned int lane_bytes, const int c) {
-  using Rounds = PieceRounds<TILE_X, TILE_K, VL, KC>;
-  const char* round = reinterpret_cast<const char*>(slab + static_cast<long long>(c * Rounds::LINES) * ld);
-  return *reinterpret_cast<const typename VecType<T, VL>::type*>(round + lane_bytes);
-}
-
-template <typename T, int TILE_X, int TILE_K, int PITCH, int VL, bool KC>
-__device__ __forceinline__ void StorePiece(T* __restrict__ tile, const int tid, const int c,
-                                           const typename VecType<T, VL>::type v) {
-  using V = typename VecType<T, VL>::type;
-  int x, k;
-  PieceMap<TILE_X, TILE_K, VL, KC>::Get(tid + c * kMfmaThreads, x, k);
-  if (KC) {
-#pragma unroll
-    for (int e = 0; e < VL; ++e) { tile[(k + e) * PITCH + x] = VecGet<V, T, VL>(v, e); }
-  } else {
-    *reinterpret_cast<V*>(&tile[k * PITCH + x]) = v;
-  }
-}
-
-// ---- direct global -> LDS loads (x-contiguous, 16-byte aligned operands on interior tiles) ----------
-// One `buffer_load_dwordx4 ... lds` moves 16 bytes per lane straight into LDS, lane l landing at
-// base + 16 * l: a wavefront fills 1 KiB of contiguous LDS per instruction and no vector register or
-// LDS store instruction is spent on staging. A slab [k][x] is therefore kept as groups of R whole rows
-// (R * TILE_X * sizeof(T) == 1 KiB, or one row in several instructions when a row is longer), groups
-// GROUP_PITCH elements apart. An operand that is staged through registers uses the same description
-// with R == 1, i.e. plain rows of pitch TILE_X + PAD.
-template <typename T, int TILE_X, int TILE_K, bool DIRECT>
+// ---- slab movement ---------------------------------------------------------------------------------
+// One operand slab is TILE_X x TILE_K elements; element (x, k) of the operand lives at
+// base[KC ? x*ld + k : k*ld + x]. In LDS a slab is always [k][x]. All global reads are buffer loads: the
+// resource of every load is cut off at the end of the operand's valid region, so elements outside the
+// matrix are never touched and read as zero (the hardware checks the range per dword), and rows or
+// columns of a tile that lie outside the matrix but inside that linear range read finite garbage that
+// only reaches results nobody stores. No tile needs a special path.
+//
+// x-contiguous operand ("direct"): `buffer_load_dword[x4] ... lds` moves LANE_BYTES per lane straight
+// into LDS, lane l landing at base + LANE_BYTES * l, so a wavefront fills WAVE_BYTES of contiguous LDS per
+// instruction and no vector register or LDS store is spent on staging. A slab is kept as groups of R
+// whole rows (R * row bytes == WAVE_BYTES; R == 1 with PARTS loads per row when a row is longer), groups
+// GROUP_PITCH elements apart. LANE_BYTES is 16 when every address is 16-byte aligned, else 4.
+// k-contiguous operand ("staged"): loaded into registers (16 bytes per piece when aligned, else one
+// element) and scattered into LDS transposed; the same description with R == 1, i.e. plain rows.
+template <typename T, int TILE_X, int TILE_K, bool DIRECT, int LANE_BYTES>
 struct SlabLayout {
   static constexpr int VEC = 16 / sizeof(T);
-  static constexpr int WAVE_ELEMS = 1024 / sizeof(T);                       // elements per wavefront-wide load
-  static constexpr int R = (DIRECT && TILE_X < WAVE_ELEMS) ? WAVE_ELEMS / TILE_X : 1;  // rows per group
-  static constexpr int PARTS = (DIRECT && TILE_X > WAVE_ELEMS) ? TILE_X / WAVE_ELEMS : 1;  // loads per row
+  static constexpr int ROW_BYTES = TILE_X * sizeof(T), WAVE_BYTES = 64 * LANE_BYTES;
+  static constexpr int WAVE_ELEMS = WAVE_BYTES / sizeof(T);
+  static constexpr int R = (DIRECT && ROW_BYTES < WAVE_BYTES) ? WAVE_BYTES / ROW_BYTES : 1;      // rows per group
+  static constexpr int PARTS = (DIRECT && ROW_BYTES > WAVE_BYTES) ? ROW_BYTES / WAVE_BYTES : 1;  // loads per row
   static constexpr int GROUPS = TILE_K / R;
   static constexpr int GROUP_PITCH = R * TILE_X + VEC;
-  static constexpr int ELEMS = GROUPS * GROUP_PITCH;                         // one stage
-  static constexpr int LOADS = GROUPS * PARTS;                               // wavefront-wide loads per slab
+  static constexpr int ELEMS = GROUPS * GROUP_PITCH;  // one stage
+  static constexpr int LOADS = GROUPS * PARTS;        // wavefront-wide loads per slab
   static constexpr int LOADS_PER_WAVE = (LOADS + 3) / 4;
   static_assert(TILE_K % R == 0, "whole groups per slab");
+  static_assert(PARTS == 1 || PARTS == 2 || PARTS == 4, "a wavefront always loads the same part of a row");
   // offset of element (k, 0)
   static __device__ __forceinline__ int Row(const int k) { return (k / R) * GROUP_PITCH + (k % R) * TILE_X; }
 };
 
-// Issues the `round`-th direct load of this wavefront for one slab. `slab` points at the slab's first
-// element (x0, k0), `stage` at the LDS stage; both are uniform over the work-group.
-template <typename T, int TILE_X, int TILE_K>
-__device__ __forceinline__ void DirectLoad(const T* __restrict__ slab, const long long ld, T* stage, const int wave,
-                                           const int lane, const int round) {
-  using L = SlabLayout<T, TILE_X, TILE_K, true>;
-  const int index = wave + 4 * round;
-  if (L::LOADS % 4 != 0 && index >= L::LOADS) { return; }
-  const int group = index / L::PARTS, part = index % L::PARTS;
-  const int in_group = lane * L::VEC;                                      // element of the 1 KiB chunk
-  const int row = (L::R > 1) ? in_group / TILE_X : 0, x = (L::R > 1) ? in_group % TILE_X : in_group;
-  const int lane_bytes = static_cast<int>((row * ld + x) * static_cast<long long>(sizeof(T)));
-  const T* chunk = slab + static_cast<long long>(group * L::R) * ld + part * L::WAVE_ELEMS;
-  // Buffer form of the load (untyped raw buffer over the rest of the address space, no range check
-  // needed on interior tiles): unlike the flat-encoded global form it leaves the LDS counter alone, so
-  // waits on LDS reads stay counted instead of draining the queue.
-  const __amdgpu_buffer_rsrc_t resource = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(chunk), 0, -1, 0x00020000);
-  typedef __attribute__((address_space(3))) void* LdsPtr;
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(resource, (LdsPtr)(stage + group * L::GROUP_PITCH + part * L::WAVE_ELEMS), 16,
-                                           lane_bytes, 0, 0, 0);
+// Bytes from `from` to `end`, clamped to what a buffer resource can hold; both pointers are uniform.
+__device__ __forceinline__ int RecordsUpTo(const void* from, const void* end) {
+  const long long bytes = static_cast<const char*>(end) - static_cast<const char*>(from);
+  // clamp to [0, 2^32 - 1] on the two 32-bit halves: stays on the scalar unit (it has no 64-bit compares)
+  int high = static_cast<int>(bytes >> 32);
+  const unsigned int low = static_cast<unsigned int>(bytes);
+  asm("" : "+s"(high));  // opaque, or the halves are fused back into 64-bit vector compares
+  return static_cast<int>(high < 0 ? 0u : (high != 0 ? 0xffffffffu : low));
+}
+
+constexpr int kRawBufferFlags = 0x00020000;  // untyped raw buffer (stride 0), range-checked against its byte count
+
+// Byte offset of this lane inside the chunk a direct load moves.
+template <typename T, int TILE_X, int TILE_K, int LANE_BYTES>
+__device__ __forceinline__ int DirectLaneBytes(const long long ld, const int lane) {
+  using L = SlabLayout<T, TILE_X, TILE_K, true, LANE_BYTES>;
+  const int position = lane * LANE_BYTES;
+  const int row = (L::R > 1) ? position / L::ROW_BYTES : 0, in_row = (L::R > 1) ? position % L::ROW_BYTES : position;
+  return static_cast<int>(row * ld * static_cast<long long>(sizeof(T))) + in_row;
+}
+
+// Issues this wavefront's direct loads for one slab (nothing for a staged operand). Tag only makes the
+// instantiation unique per kernel: the host pass of hipcc 7.2 rejects a second kernel reusing a
+// specialization of this function ("no matching function"), while the device pass accepts it. `slab` points at the slab's first
+// element (x0, k0), `valid_end` behind the last element of the operand, `stage` at the LDS stage; all
+// three are uniform over the work-group.
+template <typename T, int TILE_X, int TILE_K, int LANE_BYTES, bool DIRECT, typename Tag>
+__device__ __forceinline__ void DirectLoads(const T* __restrict__ slab, const T* valid_end, const long long ld, T* stage,
+                                            const int wave, const int lane_bytes) {
+  if constexpr (DIRECT) {
+    using L = SlabLayout<T, TILE_X, TILE_K, true, LANE_BYTES>;
+#pragma unroll
+    for (int round = 0; round < L::LOADS_PER_WAVE; ++round) {
+      const int index = wave + 4 * round;
+      if (L::LOADS % 4 == 0 || index < L::LOADS) {
+        const int group = index / L::PARTS, part = index % L::PARTS;
+        const T* chunk = slab + static_cast<long long>(group * L::R) * ld + part * L::WAVE_ELEMS;
+        typedef __attribute__((address_space(3))) void* LdsPtr;
+        // (the buffer form, unlike the flat-encoded global form, leaves the LDS counter alone, so waits on
+        // LDS reads stay counted instead of draining the queue)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(__builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(chunk), 0, RecordsUpTo(chunk, valid_end), kRawBufferFlags),
+                                                 (LdsPtr)(stage + group * L::GROUP_PITCH + part * L::WAVE_ELEMS),
+                                                 LANE_BYTES, lane_bytes, 0, 0, 0);
+      }
+    }
+  }
+}
+
+// Staged operand: thread t moves the pieces t, t + 256, ... of the slab (VL elements each, consecutive
+// threads along k); with LINES whole x lines per round, piece c lies c * LINES lines after piece 0.
+template <int TILE_X, int TILE_K, int VL>
+struct StagedPieces {
+  static constexpr int ALONG = TILE_K / VL;  // pieces per x line
+  static_assert(kMfmaThreads % ALONG == 0, "whole lines per round of pieces");
+  static constexpr int LINES = kMfmaThreads / ALONG;
+  static constexpr int PIECES = TILE_X * TILE_K / VL / kMfmaThreads;
+  static __device__ __forceinline__ int Line(const int tid) { return tid / ALONG; }
+  static __device__ __forceinline__ int K(const int tid) { return (tid % ALONG) * VL; }
+};
+
+template <typename T, int VL, typename Resource>
+__device__ __forceinline__ typename VecType<T, VL>::type BufferLoad(const Resource resource, const int offset) {
+  using V = typename VecType<T, VL>::type;
+  constexpr int BYTES = VL * sizeof(T);
+  if constexpr (BYTES == 4) { return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b32(resource, offset, 0, 0)); }
+  else if constexpr (BYTES == 8) { return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b64(resource, offset, 0, 0)); }
+  else { static_assert(BYTES == 16, "piece size"); return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b128(resource, offset, 0, 0)); }
+}
+
+// Piece c of this thread for the slab at `slab` (element (x0, k0), uniform).
+template <typename T, int TILE_X, int TILE_K, int VL>
+__device__ __forceinline__ typename VecType<T, VL>::type LoadPiece(const T* __restrict__ slab, const T* valid_end,
+                                                                   const long long ld, const int lane_bytes, const int c) {
+  using P = StagedPieces<TILE_X, TILE_K, VL>;
+  const T* round = slab + static_cast<long long>(c * P::LINES) * ld;
+  return BufferLoad<T, VL>(__builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(round), 0, RecordsUpTo(round, valid_end), kRawBufferFlags), lane_bytes);
+}
+
+// Registers -> LDS tile [k][x] of row pitch PITCH. CHECK zeroes the elements at k >= k_valid (the K tail:
+// such elements lie inside the operand's linear range and hold the next line's data).
+template <typename T, int TILE_X, int TILE_K, int PITCH, int VL, bool CHECK>
+__device__ __forceinline__ void StorePiece(T* __restrict__ tile, const int tid, const int c,
+                                           const typename VecType<T, VL>::type v, const int k_valid) {
+  using P = StagedPieces<TILE_X, TILE_K, VL>;
+  using V = typename VecType<T, VL>::type;
+  const int x = P::Line(tid) + c * P::LINES, k = P::K(tid);
+#pragma unroll
+  for (int e = 0; e < VL; ++e) {
+    T value = VecGet<V, T, VL>(v, e);
+    if (CHECK && k + e >= k_valid) { value = T(0); }
+    tile[(k + e) * PITCH + x] = value;
+  }
 }
 
 // ---- blockIdx -> tile ------------------------------------------------------------------------------
@@ -315,19 +262,33 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
   constexpr int MF = Traits::MF, KP = Traits::KP, ACC = Traits::ACC;
   constexpr int TILE_M = Config::TILE_M, TILE_N = Config::TILE_N, TILE_K = Config::TILE_K;
   constexpr int FM = Config::FM, FN = Config::FN, VEC = Config::VEC;
-  constexpr int PITCH_M = Config::PITCH_M, PITCH_N = Config::PITCH_N;
-  constexpr int VL = ALIGNED ? VEC : 1;  // elements per global access
-  constexpr int PIECES_A = Config::CHUNKS_A * VEC / VL, PIECES_B = Config::CHUNKS_B * VEC / VL;
+  constexpr int VL = ALIGNED ? VEC : 1;         // elements per staged global access
+  constexpr int LANE_BYTES = ALIGNED ? 16 : 4;  // bytes per lane of a direct load
+  constexpr bool A_DIRECT = !A_KC, B_DIRECT = !B_KC;
+  using LA = SlabLayout<T, TILE_M, TILE_K, A_DIRECT, LANE_BYTES>;
+  using LB = SlabLayout<T, TILE_N, TILE_K, B_DIRECT, LANE_BYTES>;
+  using PA = StagedPieces<TILE_M, TILE_K, VL>;
+  using PB = StagedPieces<TILE_N, TILE_K, VL>;
+  static_assert(2 * (LA::ELEMS + LB::ELEMS) <= Config::LDS_ELEMS, "LDS allocation covers the layouts");
+  constexpr int STAGED_A = A_DIRECT ? 0 : PA::PIECES, STAGED_B = B_DIRECT ? 0 : PB::PIECES;
+  constexpr int STAGED = STAGED_A + STAGED_B;
+  constexpr int KSTEPS = TILE_K / KP;
+  static_assert(KSTEPS % 2 == 0, "fragment register sets alternate per k-step");
+  constexpr int SLOTS = KSTEPS - 1;
+  constexpr int PER_SLOT = (STAGED + SLOTS - 1) / SLOTS;
   using VM = typename VecType<T, FM>::type;
   using VN = typename VecType<T, FN>::type;
+  using VP = typename VecType<T, VL>::type;
+  using KernelTag = std::tuple<Config, std::integral_constant<int, (A_KC ? 4 : 0) | (B_KC ? 2 : 0) | (ALIGNED ? 1 : 0)>>;
 
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
-  T* a_tiles = lds;                             // [2][TILE_K][PITCH_M]
-  T* b_tiles = lds + 2 * TILE_K * PITCH_M;      // [2][TILE_K][PITCH_N]
+  T* a_stages = lds;                  // [2][LA::ELEMS]
+  T* b_stages = lds + 2 * LA::ELEMS;  // [2][LB::ELEMS]
 
   const int tid = threadIdx.x;
   const int lane = tid % 64, wave = tid / 64;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int wave_m = wave % Config::WM, wave_n = wave / Config::WM;
   const int lane_x = lane % MF;  // position along the lane dimension of the MFMA block
   const int lane_g = lane / MF;  // k-group of the lane inside one instruction
@@ -335,7 +296,6 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
   int tile_m, tile_n;
   TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
   const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
-  const bool a_full = (m0 + TILE_M <= p.m), b_full = (n0 + TILE_N <= p.n);
 
   // LDS read offsets of this lane. Aligned operands: the lane owns FM consecutive m (one vector LDS read,
   // one vector store to C). Otherwise C is stored element-wise, and the lane owns m = lane_x, lane_x + MF,
@@ -343,6 +303,8 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
   constexpr bool M_INTERLEAVED = ALIGNED;
   const int a_read = wave_m * (FM * MF) + (M_INTERLEAVED ? lane_x * FM : lane_x);
   const int b_read = wave_n * (FN * MF) + lane_x * FN;
+  static_assert((KP % LA::R == 0 || LA::R % KP == 0) && (KP % LB::R == 0 || LB::R % KP == 0), "row offsets add up");
+  const int a_lane_row = LA::Row(lane_g) + a_read, b_lane_row = LB::Row(lane_g) + b_read;
 
   for (int batch = blockIdx.y; batch < p.batch_count; batch += gridDim.y) {
     const T* a;
@@ -364,7 +326,6 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
       beta = T(0);
       c_aligned = true;  // the workspace is 256-byte aligned and split_ld a multiple of 4
     }
-    const int full_slabs = k_len / TILE_K;
     const int slabs = (k_len + TILE_K - 1) / TILE_K;
 
     Acc acc[FM][FN];
@@ -374,200 +335,129 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
       for (int j = 0; j < FN; ++j) { acc[i][j] = Traits::Zero(); }
     }
 
-    T a_regs[PIECES_A][VL];
-    T b_regs[PIECES_B][VL];
+    // Walk over the slabs, explicitly scheduled so that the matrix pipe never waits at a slab boundary even
+    // with one wavefront per SIMD. Per k-step: LDS reads of the fragments of the NEXT k-step (other
+    // register set), the FM x FN MFMAs of this k-step, then a share of the data movement for the coming
+    // slabs: a direct operand's slab t+1 is requested in the first k-step of slab t; a staged operand
+    // stores its slab t+1 into the other LDS buffer and refills the staging registers with slab t+2. One
+    // barrier per slab, before its last k-step: by then every wavefront has finished its reads of the
+    // current buffer and its writes to the other one, so the last k-step already fetches the first
+    // fragments of slab t+1.
+    const T* a_tile0 = a + (A_KC ? m0 * p.a_ld : static_cast<long long>(m0));  // element (m0, k = 0), uniform
+    const T* b_tile0 = b + (B_KC ? n0 * p.b_ld : static_cast<long long>(n0));
+    // behind the last element of the operand: (x = extent - 1, k = k_len - 1) + 1
+    const T* a_end = a + (A_KC ? (p.m - 1) * p.a_ld + k_len : (k_len - 1) * p.a_ld + p.m);
+    const T* b_end = b + (B_KC ? (p.n - 1) * p.b_ld + k_len : (k_len - 1) * p.b_ld + p.n);
+    const int a_lane_bytes = A_DIRECT ? DirectLaneBytes<T, TILE_M, TILE_K, LANE_BYTES>(p.a_ld, lane)
+                                      : static_cast<int>((PA::Line(tid) * p.a_ld + PA::K(tid)) * static_cast<long long>(sizeof(T)));
+    const int b_lane_bytes = B_DIRECT ? DirectLaneBytes<T, TILE_N, TILE_K, LANE_BYTES>(p.b_ld, lane)
+                                      : static_cast<int>((PB::Line(tid) * p.b_ld + PB::K(tid)) * static_cast<long long>(sizeof(T)));
+    auto a_slab = [&](const int k0) { return a_tile0 + (A_KC ? static_cast<long long>(k0) : k0 * p.a_ld); };
+    auto b_slab = [&](const int k0) { return b_tile0 + (B_KC ? static_cast<long long>(k0) : k0 * p.b_ld); };
+    VP a_stage[STAGED_A > 0 ? STAGED_A : 1], b_stage[STAGED_B > 0 ? STAGED_B : 1];
+    auto load_piece = [&](const int piece, const int k0) {
+      if (piece < STAGED_A) { a_stage[piece] = LoadPiece<T, TILE_M, TILE_K, VL>(a_slab(k0), a_end, p.a_ld, a_lane_bytes, piece); }
+      else { b_stage[piece - STAGED_A] = LoadPiece<T, TILE_N, TILE_K, VL>(b_slab(k0), b_end, p.b_ld, b_lane_bytes, piece - STAGED_A); }
+    };
+    auto store_piece = [&](const int piece, T* a_dst, T* b_dst, const int k0, auto check_tag) {
+      constexpr bool CHECK = decltype(check_tag)::value;
+      if (piece < STAGED_A) {
+        StorePiece<T, TILE_M, TILE_K, LA::GROUP_PITCH, VL, CHECK>(a_dst, tid, piece, a_stage[piece], k_len - k0);
+      } else {
+        StorePiece<T, TILE_N, TILE_K, LB::GROUP_PITCH, VL, CHECK>(b_dst, tid, piece - STAGED_A, b_stage[piece - STAGED_A], k_len - k0);
+      }
+    };
+    auto direct_loads = [&](const int k0, auto* a_dst, auto* b_dst) {
+      DirectLoads<T, TILE_M, TILE_K, LANE_BYTES, A_DIRECT, KernelTag>(a_slab(k0), a_end, p.a_ld, a_dst, wave_u, a_lane_bytes);
+      DirectLoads<T, TILE_N, TILE_K, LANE_BYTES, B_DIRECT, KernelTag>(b_slab(k0), b_end, p.b_ld, b_dst, wave_u, b_lane_bytes);
+    };
+    auto read_a = [&](const T* stage, const int ks) {
+      const T* src = stage + LA::Row(ks * KP) + a_lane_row;
+      VM av;
+      if constexpr (M_INTERLEAVED) {
+        av = *reinterpret_cast<const VM*>(src);
+      } else {
+#pragma unroll
+        for (int i = 0; i < FM; ++i) { av = VecWith<VM, T, FM>(av, i, src[i * MF]); }
+      }
+      return av;
+    };
+    auto read_b = [&](const T* stage, const int ks) {
+      return *reinterpret_cast<const VN*>(stage + LB::Row(ks * KP) + b_lane_row);
+    };
 
-    auto load = [&](const int slab) {
-      if (a_full) { LoadSlab<T, TILE_M, TILE_K, PIECES_A, VL, A_KC>(a, p.a_ld, m0, slab * TILE_K, tid, a_regs); }
-      else { LoadSlabEdge<T, TILE_M, TILE_K, PIECES_A, VL, A_KC>(a, p.a_ld, m0, slab * TILE_K, p.m, tid, a_regs); }
-      if (b_full) { LoadSlab<T, TILE_N, TILE_K, PIECES_B, VL, B_KC>(b, p.b_ld, n0, slab * TILE_K, tid, b_regs); }
-      else { LoadSlabEdge<T, TILE_N, TILE_K, PIECES_B, VL, B_KC>(b, p.b_ld, n0, slab * TILE_K, p.n, tid, b_regs); }
-    };
-    auto store = [&](const int buffer) {
-      StoreSlab<T, TILE_M, TILE_K, PITCH_M, PIECES_A, VL, A_KC>(a_tiles + buffer * TILE_K * PITCH_M, tid, a_regs);
-      StoreSlab<T, TILE_N, TILE_K, PITCH_N, PIECES_B, VL, B_KC>(b_tiles + buffer * TILE_K * PITCH_N, tid, b_regs);
-    };
-    auto multiply = [&](const int buffer) {
-      const T* a_tile = a_tiles + buffer * TILE_K * PITCH_M + a_read;
-      const T* b_tile = b_tiles + buffer * TILE_K * PITCH_N + b_read;
+    direct_loads(0, a_stages, b_stages);
 #pragma unroll
-      for (int ks = 0; ks < TILE_K / KP; ++ks) {
-        const int k = ks * KP + lane_g;
-        VM av;
-        if constexpr (M_INTERLEAVED) {
-          av = *reinterpret_cast<const VM*>(&a_tile[k * PITCH_M]);
+    for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, 0); }
+#pragma unroll
+    for (int piece = 0; piece < STAGED; ++piece) { store_piece(piece, a_stages, b_stages, 0, std::true_type{}); }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (slabs > 1) {
+#pragma unroll
+      for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, TILE_K); }
+    }
+    __syncthreads();
+    VM av[2];
+    VN bv[2];
+    av[0] = read_a(a_stages, 0);
+    bv[0] = read_b(b_stages, 0);
+    // One slab. STORE: slab + 1 exists (direct operands request it, staged ones store it); LOAD: slab + 2
+    // exists (staged operands fetch it). Compile-time, so that the steady state has no branches; the slab
+    // stored without a following load is the last one, the only one that can hold a K tail.
+    auto slab_body = [&](const int slab, auto store_tag, auto load_tag) {
+      constexpr bool STORE = decltype(store_tag)::value, LOAD = decltype(load_tag)::value;
+      const int cur = slab & 1;
+      const T* a_cur = a_stages + cur * LA::ELEMS;
+      const T* b_cur = b_stages + cur * LB::ELEMS;
+      T* a_nxt = a_stages + (cur ^ 1) * LA::ELEMS;
+      T* b_nxt = b_stages + (cur ^ 1) * LB::ELEMS;
+      const int k_store = (slab + 1) * TILE_K, k_load = (slab + 2) * TILE_K;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int set = ks % 2;
+        if (ks + 1 < KSTEPS) {
+          av[set ^ 1] = read_a(a_cur, ks + 1);
+          bv[set ^ 1] = read_b(b_cur, ks + 1);
         } else {
-#pragma unroll
-          for (int i = 0; i < FM; ++i) { av = VecWith<VM, T, FM>(av, i, a_tile[k * PITCH_M + i * MF]); }
+          av[set ^ 1] = read_a(a_nxt, 0);
+          bv[set ^ 1] = read_b(b_nxt, 0);
         }
-        const VN bv = *reinterpret_cast<const VN*>(&b_tile[k * PITCH_N]);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
 #pragma unroll
           for (int j = 0; j < FN; ++j) {
-            acc[i][j] = Traits::Mfma(VecGet<VN, T, FN>(bv, j), VecGet<VM, T, FM>(av, i), acc[i][j]);
+            acc[i][j] = Traits::Mfma(VecGet<VN, T, FN>(bv[set], j), VecGet<VM, T, FM>(av[set], i), acc[i][j]);
           }
+        }
+        // the other buffer is free since the barrier of the previous slab
+        if (ks == 0 && STORE) { direct_loads(k_store, a_nxt, b_nxt); }
+        if (ks < KSTEPS - 1) {
+#pragma unroll
+          for (int u = 0; u < PER_SLOT; ++u) {
+            const int piece = ks * PER_SLOT + u;
+            if (piece < STAGED) {
+              if (STORE) { store_piece(piece, a_nxt, b_nxt, k_store, std::integral_constant<bool, !LOAD>{}); }
+              if (LOAD) { load_piece(piece, k_load); }
+            }
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (ks == KSTEPS - 2) {
+          // direct loads of this slab are older than its register loads: all but those must have landed
+          if ((A_DIRECT || B_DIRECT) && STORE) {
+            if (LOAD && STAGED > 0) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(STAGED) : "memory"); }
+            else { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+          }
+          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         }
       }
     };
-
-    // Software-pipelined walk over the full slabs.
-    const int fast_slabs = full_slabs;
-    if (a_full && b_full && fast_slabs > 0) {
-      // Interior tiles: explicit schedule, so that the matrix pipe never waits at a slab boundary even
-      // with one wavefront per SIMD. Per k-step: LDS reads of the fragments of the NEXT k-step (other
-      // register set), the FM x FN MFMAs of this k-step, then a share of the data movement for the
-      // coming slabs. An x-contiguous aligned operand goes global -> LDS directly (slab t+1, issued in
-      // the first k-step of slab t); any other operand is staged through registers ("store staged slab
-      // t+1 into the other LDS buffer, refill the staging registers with slab t+2"). One barrier per
-      // slab, before its last k-step: by then every wavefront has finished its reads of the current
-      // buffer and its writes to the other one, so the last k-step already fetches the first fragments
-      // of slab t+1.
-      constexpr int KSTEPS = TILE_K / KP;
-      static_assert(KSTEPS % 2 == 0, "fragment register sets alternate per k-step");
-      constexpr bool A_DIRECT = !A_KC && ALIGNED && !CLBH_EXP_NO_DIRECT, B_DIRECT = !B_KC && ALIGNED && !CLBH_EXP_NO_DIRECT;
-      using LA = SlabLayout<T, TILE_M, TILE_K, A_DIRECT>;
-      using LB = SlabLayout<T, TILE_N, TILE_K, B_DIRECT>;
-      static_assert(2 * (LA::ELEMS + LB::ELEMS) <= Config::LDS_ELEMS, "LDS allocation covers both layouts");
-      constexpr int STAGED_A = A_DIRECT ? 0 : PIECES_A, STAGED_B = B_DIRECT ? 0 : PIECES_B;
-      constexpr int STAGED = STAGED_A + STAGED_B;
-      constexpr int SLOTS = KSTEPS - 1;
-      constexpr int PER_SLOT = (STAGED + SLOTS - 1) / SLOTS;
-      T* a_stages = lds;                        // [2][LA::ELEMS]
-      T* b_stages = lds + 2 * LA::ELEMS;        // [2][LB::ELEMS]
-      const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-      using VP = typename VecType<T, VL>::type;
-      VP a_stage[STAGED_A > 0 ? STAGED_A : 1], b_stage[STAGED_B > 0 ? STAGED_B : 1];
-      const unsigned int a_lane_bytes = PieceLaneBytes<T, TILE_M, TILE_K, VL, A_KC>(p.a_ld, tid);
-      const unsigned int b_lane_bytes = PieceLaneBytes<T, TILE_N, TILE_K, VL, B_KC>(p.b_ld, tid);
-      const T* a_tile0 = a + (A_KC ? m0 * p.a_ld : static_cast<long long>(m0));  // element (m0, k = 0), uniform
-      const T* b_tile0 = b + (B_KC ? n0 * p.b_ld : static_cast<long long>(n0));
-      auto a_slab = [&](const int k0) { return a_tile0 + (A_KC ? static_cast<long long>(k0) : k0 * p.a_ld); };
-      auto b_slab = [&](const int k0) { return b_tile0 + (B_KC ? static_cast<long long>(k0) : k0 * p.b_ld); };
-      auto load_piece = [&](const int piece, const int k0) {
-        if (piece < STAGED_A) { a_stage[piece] = LoadPiece<T, TILE_M, TILE_K, VL, A_KC>(a_slab(k0), p.a_ld, a_lane_bytes, piece); }
-        else { b_stage[piece - STAGED_A] = LoadPiece<T, TILE_N, TILE_K, VL, B_KC>(b_slab(k0), p.b_ld, b_lane_bytes, piece - STAGED_A); }
-      };
-      auto store_piece = [&](const int piece, T* a_dst, T* b_dst) {
-        if (piece < STAGED_A) { StorePiece<T, TILE_M, TILE_K, LA::GROUP_PITCH, VL, A_KC>(a_dst, tid, piece, a_stage[piece]); }
-        else { StorePiece<T, TILE_N, TILE_K, LB::GROUP_PITCH, VL, B_KC>(b_dst, tid, piece - STAGED_A, b_stage[piece - STAGED_A]); }
-      };
-      auto direct_loads = [&](const int k0, T* a_dst, T* b_dst) {
-        if constexpr (A_DIRECT) {
-#pragma unroll
-          for (int round = 0; round < LA::LOADS_PER_WAVE; ++round) { DirectLoad<T, TILE_M, TILE_K>(a_slab(k0), p.a_ld, a_dst, wave_u, lane, round); }
-        }
-        if constexpr (B_DIRECT) {
-#pragma unroll
-          for (int round = 0; round < LB::LOADS_PER_WAVE; ++round) { DirectLoad<T, TILE_N, TILE_K>(b_slab(k0), p.b_ld, b_dst, wave_u, lane, round); }
-        }
-      };
-      const int a_lane_row = LA::Row(lane_g) + a_read, b_lane_row = LB::Row(lane_g) + b_read;
-      auto read_a = [&](const T* stage, const int ks) {
-        const T* src = stage + LA::Row(ks * KP) + a_lane_row;
-        VM av;
-        if constexpr (M_INTERLEAVED) {
-          av = *reinterpret_cast<const VM*>(src);
-        } else {
-#pragma unroll
-          for (int i = 0; i < FM; ++i) { av = VecWith<VM, T, FM>(av, i, src[i * MF]); }
-        }
-        return av;
-      };
-      auto read_b = [&](const T* stage, const int ks) {
-        return *reinterpret_cast<const VN*>(stage + LB::Row(ks * KP) + b_lane_row);
-      };
-      static_assert((KP % LA::R == 0 || LA::R % KP == 0) && (KP % LB::R == 0 || LB::R % KP == 0), "row offsets add up");
-      direct_loads(0, a_stages, b_stages);
-#pragma unroll
-      for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, 0); }
-#pragma unroll
-      for (int piece = 0; piece < STAGED; ++piece) { store_piece(piece, a_stages, b_stages); }
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      if (fast_slabs > 1) {
-#pragma unroll
-        for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, TILE_K); }
-      }
-      __syncthreads();
-      VM av[2];
-      VN bv[2];
-      av[0] = read_a(a_stages, 0);
-      bv[0] = read_b(b_stages, 0);
-      auto slab_body = [&](const int slab, auto store_tag, auto load_tag) {
-        constexpr bool STORE = decltype(store_tag)::value, LOAD = decltype(load_tag)::value;
-        const int cur = slab & 1;
-        const T* a_cur = a_stages + cur * LA::ELEMS;
-        const T* b_cur = b_stages + cur * LB::ELEMS;
-        T* a_nxt = a_stages + (cur ^ 1) * LA::ELEMS;
-        T* b_nxt = b_stages + (cur ^ 1) * LB::ELEMS;
-        const int k_load = (slab + 2) * TILE_K;
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          const int set = ks % 2;
-          if (ks + 1 < KSTEPS) {
-            av[set ^ 1] = read_a(a_cur, ks + 1);
-            bv[set ^ 1] = read_b(b_cur, ks + 1);
-          } else {
-            av[set ^ 1] = read_a(a_nxt, 0);
-            bv[set ^ 1] = read_b(b_nxt, 0);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int i = 0; i < FM; ++i) {
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-              acc[i][j] = Traits::Mfma(VecGet<VN, T, FN>(bv[set], j), VecGet<VM, T, FM>(av[set], i), acc[i][j]);
-            }
-          }
-          // the other buffer is free since the barrier of the previous slab
-          if (ks == 0 && STORE) { direct_loads((slab + 1) * TILE_K, a_nxt, b_nxt); }
-          if (ks < KSTEPS - 1) {
-#pragma unroll
-            for (int u = 0; u < PER_SLOT; ++u) {
-              const int piece = ks * PER_SLOT + u;
-              if (piece < STAGED) {
-                if (STORE) { store_piece(piece, a_nxt, b_nxt); }
-                if (LOAD) { load_piece(piece, k_load); }
-              }
-            }
-          }
-          __builtin_amdgcn_sched_barrier(0);
-          if (ks == KSTEPS - 2) {
-            // direct loads of this slab are older than its register loads: all but those must have landed
-            if ((A_DIRECT || B_DIRECT) && STORE) {
-              if (LOAD && STAGED > 0) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(STAGED) : "memory"); }
-              else { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-          }
-        }
-      };
-      int slab = 0;
-      for (; slab + 2 < fast_slabs; ++slab) { slab_body(slab, std::true_type{}, std::true_type{}); }
-      if (slab + 1 < fast_slabs) { slab_body(slab, std::true_type{}, std::false_type{}); ++slab; }
-      slab_body(slab, std::false_type{}, std::false_type{});
-      __syncthreads();
-    } else if (fast_slabs > 0) {
-      // Edge tiles: same double buffering, loads predicated along x, order left to the compiler.
-      load(0);
-      store(0);
-      __syncthreads();
-      for (int slab = 0; slab < fast_slabs; ++slab) {
-        const int buffer = slab & 1;
-        if (slab + 1 < fast_slabs) { load(slab + 1); }
-        multiply(buffer);
-        if (slab + 1 < fast_slabs) { store(buffer ^ 1); }
-        __syncthreads();
-      }
-    }
-    // The K tail: checked, unpipelined.
-    for (int slab = fast_slabs; slab < slabs; ++slab) {
-      FillSlabChecked<T, TILE_M, TILE_K, PITCH_M, A_KC>(a_tiles, a, p.a_ld, m0, slab * TILE_K, p.m, k_len, tid);
-      FillSlabChecked<T, TILE_N, TILE_K, PITCH_N, B_KC>(b_tiles, b, p.b_ld, n0, slab * TILE_K, p.n, k_len, tid);
-      __syncthreads();
-      multiply(0);
-      __syncthreads();
-    }
+    int slab = 0;
+    for (; slab + 2 < slabs; ++slab) { slab_body(slab, std::true_type{}, std::true_type{}); }
+    if (slab + 1 < slabs) { slab_body(slab, std::true_type{}, std::false_type{}); ++slab; }
+    slab_body(slab, std::false_type{}, std::false_type{});
+    __syncthreads();
 
     // Epilogue. Lane owns m = m_base + i (i < FM); accumulator element r of block (i, j) is the
     // column n = n_base + FN * Row(r) + j.

@@ -63,6 +63,18 @@ struct HgemmConfig {
 };
 
 // ---- slab movement ---------------------------------------------------------------------------------
+// piece -> (x, k) of a slab moved in pieces of VL elements: consecutive threads run along the contiguous
+// index of the operand in memory, so a wavefront's accesses coalesce for either orientation.
+template <int TILE_X, int TILE_K, int VL, bool KC>
+struct PieceMap {
+  static constexpr int ALONG = (KC ? TILE_K : TILE_X) / VL;  // pieces per contiguous line of the slab
+  static __device__ __forceinline__ void Get(const int piece, int& x, int& k) {
+    const int line = piece / ALONG, pos = (piece % ALONG) * VL;
+    x = KC ? line : pos;
+    k = KC ? pos : line;
+  }
+};
+
 // Slab of TILE_X x TILE_K halfs; element (x, k) at base[KC ? x*ld + k : k*ld + x]. Threads move pieces
 // of VL halfs (8 when every address is 16-byte aligned, else 1), consecutive threads along the
 // contiguous index.

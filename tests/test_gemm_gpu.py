@@ -152,3 +152,31 @@ def test_every_tile_variant(gpu, bits):
         import clblast_amd
         clblast_amd.override_parameters(0, "Xgemm", bits, {"TILE_VARIANT": 0})
         gpu.force_path(bits, None)
+
+
+@pytest.mark.parametrize("bits", BITS)
+def test_padding_and_neighbouring_memory_never_reach_the_result(gpu, bits, path):
+    """Every element of the A and B buffers outside the logical matrices (leading-dimension padding, the
+    offset prefix, the tail) is NaN: edge tiles and the K tail may read such memory but must not let it
+    into C. (The reference pads into zero-filled temporaries, src/routines/level3/xgemm.cpp:160-189.)"""
+    import oracle
+    gpu.force_path(bits, path)
+    try:
+        seed = 9000
+        shapes = [(33, 31, 17), (130, 70, 45), (257, 129, 100), (64, 64, 64), (200, 300, 127)]
+        for (m, n, k), (ta, tb), layout in itertools.product(shapes, itertools.product(TRANSPOSES, TRANSPOSES), LAYOUTS):
+            seed += 1
+            extra = ((4, 4, 4), (1, 2, 3), (8, 0, 8))[seed % 3]
+            offsets = ((0, 0, 0), (4, 8, 12), (5, 3, 1))[(seed // 3) % 3]
+            problem = gpu.Problem(bits, layout, ta, tb, m, n, k, 1.25, 0.5, a_offset=offsets[0], b_offset=offsets[1],
+                                  c_offset=offsets[2], seed=seed, extra_ld=extra)
+            for buffer, transpose, rows, cols, offset, ld in ((problem.a, ta, m, k, problem.a_offset, problem.a_ld),
+                                                              (problem.b, tb, k, n, problem.b_offset, problem.b_ld)):
+                keep = np.zeros(buffer.size, dtype=bool)
+                keep[oracle.operand_indices(layout, transpose, rows, cols, offset, ld).ravel()] = True
+                buffer[~keep] = np.nan
+            status, c_after = problem.run()
+            assert status == 0, problem.describe()
+            problem.check(c_after)
+    finally:
+        gpu.force_path(bits, None)
