@@ -165,7 +165,7 @@ __device__ __forceinline__ int DirectLaneBytes(const long long ld, const int lan
 // specialization of this function ("no matching function"), while the device pass accepts it. `slab` points at the slab's first
 // element (x0, k0), `valid_end` behind the last element of the operand, `stage` at the LDS stage; all
 // three are uniform over the work-group.
-template <typename T, int TILE_X, int TILE_K, int LANE_BYTES, bool DIRECT, typename Tag>
+template <typename T, int TILE_X, int TILE_K, int LANE_BYTES, bool DIRECT, bool RANGE, typename Tag>
 __device__ __forceinline__ void DirectLoads(const T* __restrict__ slab, const T* valid_end, const long long ld, T* stage,
                                             const int wave, const int lane_bytes) {
   if constexpr (DIRECT) {
@@ -179,7 +179,7 @@ __device__ __forceinline__ void DirectLoads(const T* __restrict__ slab, const T*
         typedef __attribute__((address_space(3))) void* LdsPtr;
         // (the buffer form, unlike the flat-encoded global form, leaves the LDS counter alone, so waits on
         // LDS reads stay counted instead of draining the queue)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(__builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(chunk), 0, RecordsUpTo(chunk, valid_end), kRawBufferFlags),
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(__builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(chunk), 0, RANGE ? RecordsUpTo(chunk, valid_end) : -1, kRawBufferFlags),
                                                  (LdsPtr)(stage + group * L::GROUP_PITCH + part * L::WAVE_ELEMS),
                                                  LANE_BYTES, lane_bytes, 0, 0, 0);
       }
@@ -209,12 +209,12 @@ __device__ __forceinline__ typename VecType<T, VL>::type BufferLoad(const Resour
 }
 
 // Piece c of this thread for the slab at `slab` (element (x0, k0), uniform).
-template <typename T, int TILE_X, int TILE_K, int VL>
+template <typename T, int TILE_X, int TILE_K, int VL, bool RANGE>
 __device__ __forceinline__ typename VecType<T, VL>::type LoadPiece(const T* __restrict__ slab, const T* valid_end,
                                                                    const long long ld, const int lane_bytes, const int c) {
   using P = StagedPieces<TILE_X, TILE_K, VL>;
   const T* round = slab + static_cast<long long>(c * P::LINES) * ld;
-  return BufferLoad<T, VL>(__builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(round), 0, RecordsUpTo(round, valid_end), kRawBufferFlags), lane_bytes);
+  return BufferLoad<T, VL>(__builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(round), 0, RANGE ? RecordsUpTo(round, valid_end) : -1, kRawBufferFlags), lane_bytes);
 }
 
 // Registers -> LDS tile [k][x] of row pitch PITCH. CHECK zeroes the elements at k >= k_valid (the K tail:
@@ -354,110 +354,119 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
                                       : static_cast<int>((PB::Line(tid) * p.b_ld + PB::K(tid)) * static_cast<long long>(sizeof(T)));
     auto a_slab = [&](const int k0) { return a_tile0 + (A_KC ? static_cast<long long>(k0) : k0 * p.a_ld); };
     auto b_slab = [&](const int k0) { return b_tile0 + (B_KC ? static_cast<long long>(k0) : k0 * p.b_ld); };
-    VP a_stage[STAGED_A > 0 ? STAGED_A : 1], b_stage[STAGED_B > 0 ? STAGED_B : 1];
-    auto load_piece = [&](const int piece, const int k0) {
-      if (piece < STAGED_A) { a_stage[piece] = LoadPiece<T, TILE_M, TILE_K, VL>(a_slab(k0), a_end, p.a_ld, a_lane_bytes, piece); }
-      else { b_stage[piece - STAGED_A] = LoadPiece<T, TILE_N, TILE_K, VL>(b_slab(k0), b_end, p.b_ld, b_lane_bytes, piece - STAGED_A); }
-    };
-    auto store_piece = [&](const int piece, T* a_dst, T* b_dst, const int k0, auto check_tag) {
-      constexpr bool CHECK = decltype(check_tag)::value;
-      if (piece < STAGED_A) {
-        StorePiece<T, TILE_M, TILE_K, LA::GROUP_PITCH, VL, CHECK>(a_dst, tid, piece, a_stage[piece], k_len - k0);
-      } else {
-        StorePiece<T, TILE_N, TILE_K, LB::GROUP_PITCH, VL, CHECK>(b_dst, tid, piece - STAGED_A, b_stage[piece - STAGED_A], k_len - k0);
-      }
-    };
-    auto direct_loads = [&](const int k0, auto* a_dst, auto* b_dst) {
-      DirectLoads<T, TILE_M, TILE_K, LANE_BYTES, A_DIRECT, KernelTag>(a_slab(k0), a_end, p.a_ld, a_dst, wave_u, a_lane_bytes);
-      DirectLoads<T, TILE_N, TILE_K, LANE_BYTES, B_DIRECT, KernelTag>(b_slab(k0), b_end, p.b_ld, b_dst, wave_u, b_lane_bytes);
-    };
-    auto read_a = [&](const T* stage, const int ks) {
-      const T* src = stage + LA::Row(ks * KP) + a_lane_row;
-      VM av;
-      if constexpr (M_INTERLEAVED) {
-        av = *reinterpret_cast<const VM*>(src);
-      } else {
-#pragma unroll
-        for (int i = 0; i < FM; ++i) { av = VecWith<VM, T, FM>(av, i, src[i * MF]); }
-      }
-      return av;
-    };
-    auto read_b = [&](const T* stage, const int ks) {
-      return *reinterpret_cast<const VN*>(stage + LB::Row(ks * KP) + b_lane_row);
-    };
-
-    direct_loads(0, a_stages, b_stages);
-#pragma unroll
-    for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, 0); }
-#pragma unroll
-    for (int piece = 0; piece < STAGED; ++piece) { store_piece(piece, a_stages, b_stages, 0, std::true_type{}); }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (slabs > 1) {
-#pragma unroll
-      for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, TILE_K); }
-    }
-    __syncthreads();
-    VM av[2];
-    VN bv[2];
-    av[0] = read_a(a_stages, 0);
-    bv[0] = read_b(b_stages, 0);
-    // One slab. STORE: slab + 1 exists (direct operands request it, staged ones store it); LOAD: slab + 2
-    // exists (staged operands fetch it). Compile-time, so that the steady state has no branches; the slab
-    // stored without a following load is the last one, the only one that can hold a K tail.
-    auto slab_body = [&](const int slab, auto store_tag, auto load_tag) {
-      constexpr bool STORE = decltype(store_tag)::value, LOAD = decltype(load_tag)::value;
-      const int cur = slab & 1;
-      const T* a_cur = a_stages + cur * LA::ELEMS;
-      const T* b_cur = b_stages + cur * LB::ELEMS;
-      T* a_nxt = a_stages + (cur ^ 1) * LA::ELEMS;
-      T* b_nxt = b_stages + (cur ^ 1) * LB::ELEMS;
-      const int k_store = (slab + 1) * TILE_K, k_load = (slab + 2) * TILE_K;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        const int set = ks % 2;
-        if (ks + 1 < KSTEPS) {
-          av[set ^ 1] = read_a(a_cur, ks + 1);
-          bv[set ^ 1] = read_b(b_cur, ks + 1);
+    // The walk exists twice: with range-checked loads (tiles that touch an edge of the matrix, or a K
+    // tail), and without (the resources then cover "everything", which saves the scalar arithmetic of one
+    // byte count per load).
+    auto walk = [&](auto range_tag) {
+      constexpr bool RANGE = decltype(range_tag)::value;
+      VP a_stage[STAGED_A > 0 ? STAGED_A : 1], b_stage[STAGED_B > 0 ? STAGED_B : 1];
+      auto load_piece = [&](const int piece, const int k0) {
+        if (piece < STAGED_A) { a_stage[piece] = LoadPiece<T, TILE_M, TILE_K, VL, RANGE>(a_slab(k0), a_end, p.a_ld, a_lane_bytes, piece); }
+        else { b_stage[piece - STAGED_A] = LoadPiece<T, TILE_N, TILE_K, VL, RANGE>(b_slab(k0), b_end, p.b_ld, b_lane_bytes, piece - STAGED_A); }
+      };
+      auto store_piece = [&](const int piece, T* a_dst, T* b_dst, const int k0, auto check_tag) {
+        constexpr bool CHECK = RANGE && decltype(check_tag)::value;
+        if (piece < STAGED_A) {
+          StorePiece<T, TILE_M, TILE_K, LA::GROUP_PITCH, VL, CHECK>(a_dst, tid, piece, a_stage[piece], k_len - k0);
         } else {
-          av[set ^ 1] = read_a(a_nxt, 0);
-          bv[set ^ 1] = read_b(b_nxt, 0);
+          StorePiece<T, TILE_N, TILE_K, LB::GROUP_PITCH, VL, CHECK>(b_dst, tid, piece - STAGED_A, b_stage[piece - STAGED_A], k_len - k0);
         }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-#pragma unroll
-          for (int j = 0; j < FN; ++j) {
-            acc[i][j] = Traits::Mfma(VecGet<VN, T, FN>(bv[set], j), VecGet<VM, T, FM>(av[set], i), acc[i][j]);
+      };
+      auto direct_loads = [&](const int k0, auto* a_dst, auto* b_dst) {
+        DirectLoads<T, TILE_M, TILE_K, LANE_BYTES, A_DIRECT, RANGE, KernelTag>(a_slab(k0), a_end, p.a_ld, a_dst, wave_u, a_lane_bytes);
+        DirectLoads<T, TILE_N, TILE_K, LANE_BYTES, B_DIRECT, RANGE, KernelTag>(b_slab(k0), b_end, p.b_ld, b_dst, wave_u, b_lane_bytes);
+      };
+      auto read_a = [&](const T* stage, const int ks) {
+        const T* src = stage + LA::Row(ks * KP) + a_lane_row;
+        VM av;
+        if constexpr (M_INTERLEAVED) {
+          av = *reinterpret_cast<const VM*>(src);
+        } else {
+  #pragma unroll
+          for (int i = 0; i < FM; ++i) { av = VecWith<VM, T, FM>(av, i, src[i * MF]); }
+        }
+        return av;
+      };
+      auto read_b = [&](const T* stage, const int ks) {
+        return *reinterpret_cast<const VN*>(stage + LB::Row(ks * KP) + b_lane_row);
+      };
+
+      direct_loads(0, a_stages, b_stages);
+  #pragma unroll
+      for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, 0); }
+  #pragma unroll
+      for (int piece = 0; piece < STAGED; ++piece) { store_piece(piece, a_stages, b_stages, 0, std::true_type{}); }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (slabs > 1) {
+  #pragma unroll
+        for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, TILE_K); }
+      }
+      __syncthreads();
+      VM av[2];
+      VN bv[2];
+      av[0] = read_a(a_stages, 0);
+      bv[0] = read_b(b_stages, 0);
+      // One slab. STORE: slab + 1 exists (direct operands request it, staged ones store it); LOAD: slab + 2
+      // exists (staged operands fetch it). Compile-time, so that the steady state has no branches; the slab
+      // stored without a following load is the last one, the only one that can hold a K tail.
+      auto slab_body = [&](const int slab, auto store_tag, auto load_tag) {
+        constexpr bool STORE = decltype(store_tag)::value, LOAD = decltype(load_tag)::value;
+        const int cur = slab & 1;
+        const T* a_cur = a_stages + cur * LA::ELEMS;
+        const T* b_cur = b_stages + cur * LB::ELEMS;
+        T* a_nxt = a_stages + (cur ^ 1) * LA::ELEMS;
+        T* b_nxt = b_stages + (cur ^ 1) * LB::ELEMS;
+        const int k_store = (slab + 1) * TILE_K, k_load = (slab + 2) * TILE_K;
+  #pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const int set = ks % 2;
+          if (ks + 1 < KSTEPS) {
+            av[set ^ 1] = read_a(a_cur, ks + 1);
+            bv[set ^ 1] = read_b(b_cur, ks + 1);
+          } else {
+            av[set ^ 1] = read_a(a_nxt, 0);
+            bv[set ^ 1] = read_b(b_nxt, 0);
           }
-        }
-        // the other buffer is free since the barrier of the previous slab
-        if (ks == 0 && STORE) { direct_loads(k_store, a_nxt, b_nxt); }
-        if (ks < KSTEPS - 1) {
-#pragma unroll
-          for (int u = 0; u < PER_SLOT; ++u) {
-            const int piece = ks * PER_SLOT + u;
-            if (piece < STAGED) {
-              if (STORE) { store_piece(piece, a_nxt, b_nxt, k_store, std::integral_constant<bool, !LOAD>{}); }
-              if (LOAD) { load_piece(piece, k_load); }
+          __builtin_amdgcn_sched_barrier(0);
+  #pragma unroll
+          for (int i = 0; i < FM; ++i) {
+  #pragma unroll
+            for (int j = 0; j < FN; ++j) {
+              acc[i][j] = Traits::Mfma(VecGet<VN, T, FN>(bv[set], j), VecGet<VM, T, FM>(av[set], i), acc[i][j]);
             }
           }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (ks == KSTEPS - 2) {
-          // direct loads of this slab are older than its register loads: all but those must have landed
-          if ((A_DIRECT || B_DIRECT) && STORE) {
-            if (LOAD && STAGED > 0) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(STAGED) : "memory"); }
-            else { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+          // the other buffer is free since the barrier of the previous slab
+          if (ks == 0 && STORE) { direct_loads(k_store, a_nxt, b_nxt); }
+          if (ks < KSTEPS - 1) {
+  #pragma unroll
+            for (int u = 0; u < PER_SLOT; ++u) {
+              const int piece = ks * PER_SLOT + u;
+              if (piece < STAGED) {
+                if (STORE) { store_piece(piece, a_nxt, b_nxt, k_store, std::integral_constant<bool, !LOAD>{}); }
+                if (LOAD) { load_piece(piece, k_load); }
+              }
+            }
           }
-          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+          __builtin_amdgcn_sched_barrier(0);
+          if (ks == KSTEPS - 2) {
+            // direct loads of this slab are older than its register loads: all but those must have landed
+            if ((A_DIRECT || B_DIRECT) && STORE) {
+              if (LOAD && STAGED > 0) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(STAGED) : "memory"); }
+              else { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+          }
         }
-      }
+      };
+      int slab = 0;
+      for (; slab + 2 < slabs; ++slab) { slab_body(slab, std::true_type{}, std::true_type{}); }
+      if (slab + 1 < slabs) { slab_body(slab, std::true_type{}, std::false_type{}); ++slab; }
+      slab_body(slab, std::false_type{}, std::false_type{});
+      __syncthreads();
+
     };
-    int slab = 0;
-    for (; slab + 2 < slabs; ++slab) { slab_body(slab, std::true_type{}, std::true_type{}); }
-    if (slab + 1 < slabs) { slab_body(slab, std::true_type{}, std::false_type{}); ++slab; }
-    slab_body(slab, std::false_type{}, std::false_type{});
-    __syncthreads();
+    if (m0 + TILE_M <= p.m && n0 + TILE_N <= p.n && k_len % TILE_K == 0) { walk(std::false_type{}); }
+    else { walk(std::true_type{}); }
 
     // Epilogue. Lane owns m = m_base + i (i < FM); accumulator element r of block (i, j) is the
     // column n = n_base + FN * Row(r) + j.
