@@ -72,16 +72,12 @@ int LaunchMfmaVariant(const clbh_gemm_desc& d, hipStream_t stream) {
 
 template <typename T, typename Config>
 int LaunchMfmaConfig(const clbh_gemm_desc& d, hipStream_t stream) {
-  const bool aligned = Aligned16<T>(d);
-  const int variant = (d.a_kcontig ? 4 : 0) | (d.b_kcontig ? 2 : 0) | (aligned ? 1 : 0);
+  // fp32 / fp64: every address is dword aligned, which is all the 16-byte accesses of the kernel need
+  const int variant = (d.a_kcontig ? 2 : 0) | (d.b_kcontig ? 1 : 0);
   switch (variant) {
-    case 0: return LaunchMfmaVariant<T, Config, false, false, false>(d, stream);
-    case 1: return LaunchMfmaVariant<T, Config, false, false, true>(d, stream);
-    case 2: return LaunchMfmaVariant<T, Config, false, true, false>(d, stream);
-    case 3: return LaunchMfmaVariant<T, Config, false, true, true>(d, stream);
-    case 4: return LaunchMfmaVariant<T, Config, true, false, false>(d, stream);
-    case 5: return LaunchMfmaVariant<T, Config, true, false, true>(d, stream);
-    case 6: return LaunchMfmaVariant<T, Config, true, true, false>(d, stream);
+    case 0: return LaunchMfmaVariant<T, Config, false, false, true>(d, stream);
+    case 1: return LaunchMfmaVariant<T, Config, false, true, true>(d, stream);
+    case 2: return LaunchMfmaVariant<T, Config, true, false, true>(d, stream);
     default: return LaunchMfmaVariant<T, Config, true, true, true>(d, stream);
   }
 }

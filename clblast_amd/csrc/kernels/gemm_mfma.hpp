@@ -262,6 +262,8 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
   constexpr int MF = Traits::MF, KP = Traits::KP, ACC = Traits::ACC;
   constexpr int TILE_M = Config::TILE_M, TILE_N = Config::TILE_N, TILE_K = Config::TILE_K;
   constexpr int FM = Config::FM, FN = Config::FN, VEC = Config::VEC;
+  // ALIGNED: 16-byte global accesses. fp32 and fp64 operands always qualify: the memory system wants dword
+  // alignment only, whatever the offsets and leading dimensions are.
   constexpr int VL = ALIGNED ? VEC : 1;         // elements per staged global access
   constexpr int LANE_BYTES = ALIGNED ? 16 : 4;  // bytes per lane of a direct load
   constexpr bool A_DIRECT = !A_KC, B_DIRECT = !B_KC;
@@ -314,7 +316,6 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
     ResolveBatch<T, T>(p, batch, a, b, c, alpha, beta);
     int k_len = p.k;
     long long c_ld = p.c_ld;
-    bool c_aligned = ALIGNED;
     if (p.split_chunk > 0) {  // this "batch" is one K range of a single problem
       const int k_begin = batch * p.split_chunk;
       k_len = min(p.split_chunk, p.k - k_begin);
@@ -324,7 +325,6 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
       c = static_cast<T*>(p.split_workspace) + static_cast<long long>(batch) * p.split_ld * p.n;
       alpha = T(1);
       beta = T(0);
-      c_aligned = true;  // the workspace is 256-byte aligned and split_ld a multiple of 4
     }
     const int slabs = (k_len + TILE_K - 1) / TILE_K;
 
@@ -473,7 +473,9 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
     const int m_base = m0 + a_read;
     const int n_base = n0 + wave_n * (FN * MF);
     constexpr int M_STEP = M_INTERLEAVED ? 1 : MF;  // distance in m between the lane's accumulator blocks
-    const bool vector_store = M_INTERLEAVED && c_aligned && (FM > 1) && (m_base + FM <= p.m);
+    // 16-byte accesses to C need dword alignment only, which every fp32/fp64 address has
+    typedef T VMG __attribute__((ext_vector_type(FM > 1 ? FM : 2), aligned(sizeof(T))));
+    const bool vector_store = M_INTERLEAVED && (FM > 1) && (m_base + FM <= p.m);
 #pragma unroll
     for (int j = 0; j < FN; ++j) {
 #pragma unroll
@@ -482,18 +484,16 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
         if (n >= p.n) { continue; }
         T* dst = c + n * c_ld + m_base;
         if (vector_store) {
-          VM out;
+          VMG out;
           if (beta == T(0)) {
 #pragma unroll
-            for (int i = 0; i < FM; ++i) { out = VecWith<VM, T, FM>(out, i, alpha * acc[i][j][r]); }
+            for (int i = 0; i < FM; ++i) { out[i] = alpha * acc[i][j][r]; }
           } else {
-            const VM old = *reinterpret_cast<const VM*>(dst);
+            const VMG old = *reinterpret_cast<const VMG*>(dst);
 #pragma unroll
-            for (int i = 0; i < FM; ++i) {
-              out = VecWith<VM, T, FM>(out, i, alpha * acc[i][j][r] + beta * VecGet<VM, T, FM>(old, i));
-            }
+            for (int i = 0; i < FM; ++i) { out[i] = alpha * acc[i][j][r] + beta * old[i]; }
           }
-          *reinterpret_cast<VM*>(dst) = out;
+          *reinterpret_cast<VMG*>(dst) = out;
         } else {
 #pragma unroll
           for (int i = 0; i < FM; ++i) {
