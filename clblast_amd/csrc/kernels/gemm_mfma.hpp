@@ -83,7 +83,8 @@ struct MfmaConfig {
   static constexpr int PAD = VEC;
   static constexpr int PITCH_M = TILE_M + PAD;
   static constexpr int PITCH_N = TILE_N + PAD;
-  static constexpr int LDS_ELEMS = 2 * TILE_K * (PITCH_M + PITCH_N);  // two buffers
+  static constexpr int STAGES = 3;                                         // LDS slab buffers (a ring)
+  static constexpr int LDS_ELEMS = STAGES * TILE_K * (PITCH_M + PITCH_N);
   static constexpr int CHUNKS_A = TILE_M * TILE_K / VEC / kMfmaThreads;  // 16-byte chunks per thread and slab
   static constexpr int CHUNKS_B = TILE_N * TILE_K / VEC / kMfmaThreads;
   static_assert(WM * WN * 64 == kMfmaThreads, "four wavefronts per work-group");
@@ -160,31 +161,25 @@ __device__ __forceinline__ int DirectLaneBytes(const long long ld, const int lan
   return static_cast<int>(row * ld * static_cast<long long>(sizeof(T))) + in_row;
 }
 
-// Issues this wavefront's direct loads for one slab (nothing for a staged operand). Tag only makes the
+// Issues the round-th direct load of this wavefront for one slab. Tag only makes the
 // instantiation unique per kernel: the host pass of hipcc 7.2 rejects a second kernel reusing a
 // specialization of this function ("no matching function"), while the device pass accepts it. `slab` points at the slab's first
 // element (x0, k0), `valid_end` behind the last element of the operand, `stage` at the LDS stage; all
 // three are uniform over the work-group.
-template <typename T, int TILE_X, int TILE_K, int LANE_BYTES, bool DIRECT, bool RANGE, typename Tag>
-__device__ __forceinline__ void DirectLoads(const T* __restrict__ slab, const T* valid_end, const long long ld, T* stage,
-                                            const int wave, const int lane_bytes) {
-  if constexpr (DIRECT) {
-    using L = SlabLayout<T, TILE_X, TILE_K, true, LANE_BYTES>;
-#pragma unroll
-    for (int round = 0; round < L::LOADS_PER_WAVE; ++round) {
-      const int index = wave + 4 * round;
-      if (L::LOADS % 4 == 0 || index < L::LOADS) {
-        const int group = index / L::PARTS, part = index % L::PARTS;
-        const T* chunk = slab + static_cast<long long>(group * L::R) * ld + part * L::WAVE_ELEMS;
-        typedef __attribute__((address_space(3))) void* LdsPtr;
-        // (the buffer form, unlike the flat-encoded global form, leaves the LDS counter alone, so waits on
-        // LDS reads stay counted instead of draining the queue)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(__builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(chunk), 0, RANGE ? RecordsUpTo(chunk, valid_end) : -1, kRawBufferFlags),
-                                                 (LdsPtr)(stage + group * L::GROUP_PITCH + part * L::WAVE_ELEMS),
-                                                 LANE_BYTES, lane_bytes, 0, 0, 0);
-      }
-    }
-  }
+template <typename T, int TILE_X, int TILE_K, int LANE_BYTES, bool RANGE, typename Tag>
+__device__ __forceinline__ void DirectLoad(const T* __restrict__ slab, const T* valid_end, const long long ld, T* stage,
+                                           const int wave, const int lane_bytes, const int round) {
+  using L = SlabLayout<T, TILE_X, TILE_K, true, LANE_BYTES>;
+  static_assert(L::LOADS % 4 == 0, "every wavefront issues the same number of loads (the waits count them)");
+  const int index = wave + 4 * round;
+  const int group = index / L::PARTS, part = index % L::PARTS;
+  const T* chunk = slab + static_cast<long long>(group * L::R) * ld + part * L::WAVE_ELEMS;
+  typedef __attribute__((address_space(3))) void* LdsPtr;
+  // (the buffer form, unlike the flat-encoded global form, leaves the LDS counter alone, so waits on LDS
+  // reads stay counted instead of draining the queue)
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(chunk), 0, RANGE ? RecordsUpTo(chunk, valid_end) : -1, kRawBufferFlags),
+      (LdsPtr)(stage + group * L::GROUP_PITCH + part * L::WAVE_ELEMS), LANE_BYTES, lane_bytes, 0, 0, 0);
 }
 
 // Staged operand: thread t moves the pieces t, t + 256, ... of the slab (VL elements each, consecutive
@@ -271,7 +266,9 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
   using LB = SlabLayout<T, TILE_N, TILE_K, B_DIRECT, LANE_BYTES>;
   using PA = StagedPieces<TILE_M, TILE_K, VL>;
   using PB = StagedPieces<TILE_N, TILE_K, VL>;
-  static_assert(2 * (LA::ELEMS + LB::ELEMS) <= Config::LDS_ELEMS, "LDS allocation covers the layouts");
+  constexpr int STAGES = Config::STAGES;
+  static_assert(STAGES == 3, "the tags of the slab walk assume a ring of three");
+  static_assert(STAGES * (LA::ELEMS + LB::ELEMS) <= Config::LDS_ELEMS, "LDS allocation covers the layouts");
   constexpr int STAGED_A = A_DIRECT ? 0 : PA::PIECES, STAGED_B = B_DIRECT ? 0 : PB::PIECES;
   constexpr int STAGED = STAGED_A + STAGED_B;
   constexpr int KSTEPS = TILE_K / KP;
@@ -285,8 +282,8 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
 
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
-  T* a_stages = lds;                  // [2][LA::ELEMS]
-  T* b_stages = lds + 2 * LA::ELEMS;  // [2][LB::ELEMS]
+  T* a_stages = lds;                       // [STAGES][LA::ELEMS]
+  T* b_stages = lds + STAGES * LA::ELEMS;  // [STAGES][LB::ELEMS]
 
   const int tid = threadIdx.x;
   const int lane = tid % 64, wave = tid / 64;
@@ -372,9 +369,17 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
           StorePiece<T, TILE_N, TILE_K, LB::GROUP_PITCH, VL, CHECK>(b_dst, tid, piece - STAGED_A, b_stage[piece - STAGED_A], k_len - k0);
         }
       };
-      auto direct_loads = [&](const int k0, auto* a_dst, auto* b_dst) {
-        DirectLoads<T, TILE_M, TILE_K, LANE_BYTES, A_DIRECT, RANGE, KernelTag>(a_slab(k0), a_end, p.a_ld, a_dst, wave_u, a_lane_bytes);
-        DirectLoads<T, TILE_N, TILE_K, LANE_BYTES, B_DIRECT, RANGE, KernelTag>(b_slab(k0), b_end, p.b_ld, b_dst, wave_u, b_lane_bytes);
+      // direct loads of one slab, numbered over both operands: A's rounds first
+      constexpr int DIRECT_A = A_DIRECT ? LA::LOADS_PER_WAVE : 0, DIRECT_B = B_DIRECT ? LB::LOADS_PER_WAVE : 0;
+      constexpr int DIRECT = DIRECT_A + DIRECT_B;
+      constexpr int DIRECT_PER_SLOT = (DIRECT + SLOTS - 1) / SLOTS;
+      auto direct_load = [&](const int load, const int k0, auto* a_dst, auto* b_dst) {
+        if constexpr (DIRECT_A > 0) {
+          if (load < DIRECT_A) { DirectLoad<T, TILE_M, TILE_K, LANE_BYTES, RANGE, KernelTag>(a_slab(k0), a_end, p.a_ld, a_dst, wave_u, a_lane_bytes, load); }
+        }
+        if constexpr (DIRECT_B > 0) {
+          if (load >= DIRECT_A) { DirectLoad<T, TILE_N, TILE_K, LANE_BYTES, RANGE, KernelTag>(b_slab(k0), b_end, p.b_ld, b_dst, wave_u, b_lane_bytes, load - DIRECT_A); }
+        }
       };
       auto read_a = [&](const T* stage, const int ks) {
         const T* src = stage + LA::Row(ks * KP) + a_lane_row;
@@ -382,7 +387,7 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
         if constexpr (M_INTERLEAVED) {
           av = *reinterpret_cast<const VM*>(src);
         } else {
-  #pragma unroll
+#pragma unroll
           for (int i = 0; i < FM; ++i) { av = VecWith<VM, T, FM>(av, i, src[i * MF]); }
         }
         return av;
@@ -391,14 +396,19 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
         return *reinterpret_cast<const VN*>(stage + LB::Row(ks * KP) + b_lane_row);
       };
 
-      direct_loads(0, a_stages, b_stages);
-  #pragma unroll
+      // Prologue: slab 0 lands in buffer 0 (the staged registers' wait also covers the older direct loads),
+      // slab 1 is requested.
+#pragma unroll
+      for (int load = 0; load < DIRECT; ++load) { direct_load(load, 0, a_stages, b_stages); }
+#pragma unroll
       for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, 0); }
-  #pragma unroll
+#pragma unroll
       for (int piece = 0; piece < STAGED; ++piece) { store_piece(piece, a_stages, b_stages, 0, std::true_type{}); }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       if (slabs > 1) {
-  #pragma unroll
+#pragma unroll
+        for (int load = 0; load < DIRECT; ++load) { direct_load(load, TILE_K, a_stages + LA::ELEMS, b_stages + LB::ELEMS); }
+#pragma unroll
         for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, TILE_K); }
       }
       __syncthreads();
@@ -406,18 +416,22 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
       VN bv[2];
       av[0] = read_a(a_stages, 0);
       bv[0] = read_b(b_stages, 0);
-      // One slab. STORE: slab + 1 exists (direct operands request it, staged ones store it); LOAD: slab + 2
-      // exists (staged operands fetch it). Compile-time, so that the steady state has no branches; the slab
-      // stored without a following load is the last one, the only one that can hold a K tail.
+      int cur = 0;  // ring position of the current slab; slab + 1 is in the next buffer, slab + 2 goes into the one before
+      // One slab. STORE: slab + 1 exists (staged operands store it); LOAD: slab + 2 exists (direct operands
+      // request it into the buffer that the barrier of the previous slab released, staged operands fetch it
+      // into registers). Compile-time, so that the steady state has no branches; the slab stored without a
+      // following load is the last one, the only one that can hold a K tail.
       auto slab_body = [&](const int slab, auto store_tag, auto load_tag) {
         constexpr bool STORE = decltype(store_tag)::value, LOAD = decltype(load_tag)::value;
-        const int cur = slab & 1;
+        const int nxt = (cur == STAGES - 1) ? 0 : cur + 1, prv = (cur == 0) ? STAGES - 1 : cur - 1;
         const T* a_cur = a_stages + cur * LA::ELEMS;
         const T* b_cur = b_stages + cur * LB::ELEMS;
-        T* a_nxt = a_stages + (cur ^ 1) * LA::ELEMS;
-        T* b_nxt = b_stages + (cur ^ 1) * LB::ELEMS;
+        T* a_nxt = a_stages + nxt * LA::ELEMS;
+        T* b_nxt = b_stages + nxt * LB::ELEMS;
+        T* a_prv = a_stages + prv * LA::ELEMS;
+        T* b_prv = b_stages + prv * LB::ELEMS;
         const int k_store = (slab + 1) * TILE_K, k_load = (slab + 2) * TILE_K;
-  #pragma unroll
+#pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
           const int set = ks % 2;
           if (ks + 1 < KSTEPS) {
@@ -428,17 +442,15 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
             bv[set ^ 1] = read_b(b_nxt, 0);
           }
           __builtin_amdgcn_sched_barrier(0);
-  #pragma unroll
+#pragma unroll
           for (int i = 0; i < FM; ++i) {
-  #pragma unroll
+#pragma unroll
             for (int j = 0; j < FN; ++j) {
               acc[i][j] = Traits::Mfma(VecGet<VN, T, FN>(bv[set], j), VecGet<VM, T, FM>(av[set], i), acc[i][j]);
             }
           }
-          // the other buffer is free since the barrier of the previous slab
-          if (ks == 0 && STORE) { direct_loads(k_store, a_nxt, b_nxt); }
           if (ks < KSTEPS - 1) {
-  #pragma unroll
+#pragma unroll
             for (int u = 0; u < PER_SLOT; ++u) {
               const int piece = ks * PER_SLOT + u;
               if (piece < STAGED) {
@@ -446,24 +458,28 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
                 if (LOAD) { load_piece(piece, k_load); }
               }
             }
+#pragma unroll
+            for (int u = 0; u < DIRECT_PER_SLOT; ++u) {
+              const int load = ks * DIRECT_PER_SLOT + u;
+              if (LOAD && load < DIRECT) { direct_load(load, k_load, a_prv, b_prv); }
+            }
           }
           __builtin_amdgcn_sched_barrier(0);
           if (ks == KSTEPS - 2) {
-            // direct loads of this slab are older than its register loads: all but those must have landed
-            if ((A_DIRECT || B_DIRECT) && STORE) {
-              if (LOAD && STAGED > 0) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(STAGED) : "memory"); }
-              else { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-            }
+            // slab + 1 must have landed for everybody: everything requested before this slab has to be
+            // complete, this slab's own requests (slab + 2) may stay in flight (loads complete in order)
+            if (LOAD) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DIRECT + STAGED) : "memory"); }
+            else { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
           }
         }
+        cur = nxt;
       };
       int slab = 0;
       for (; slab + 2 < slabs; ++slab) { slab_body(slab, std::true_type{}, std::true_type{}); }
       if (slab + 1 < slabs) { slab_body(slab, std::true_type{}, std::false_type{}); ++slab; }
       slab_body(slab, std::false_type{}, std::false_type{});
       __syncthreads();
-
     };
     if (m0 + TILE_M <= p.m && n0 + TILE_N <= p.n && k_len % TILE_K == 0) { walk(std::false_type{}); }
     else { walk(std::true_type{}); }
