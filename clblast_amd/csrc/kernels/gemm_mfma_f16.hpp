@@ -341,20 +341,22 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
       using LA = HDirectLayout<A_KC>;
       using LB = HDirectLayout<B_KC>;
       static_assert(STAGES * (LA::ELEMS + LB::ELEMS) * 2 <= Config::LDS_BYTES, "LDS allocation covers the ring");
+      static_assert(LOADS_PER_SLAB <= FM, "one request per quarter of the first k-step");
       if (fast_slabs > 0) {
         T* a_ring = lds;
         T* b_ring = lds + STAGES * LA::ELEMS;
         const int wave_u = __builtin_amdgcn_readfirstlane(wave);
         const T* a_tile0 = a + (A_KC ? m0 * p.a_ld : static_cast<long long>(m0));  // element (m0, k = 0), uniform
         const T* b_tile0 = b + (B_KC ? n0 * p.b_ld : static_cast<long long>(n0));
-        auto issue = [&](const int slab, const int buffer) {
+        // load 0..3 of a slab: piece rounds A0, B0, A1, B1 of this wavefront
+        auto issue = [&](const int load, const int slab, const int buffer) {
           const int k0 = slab * TILE_K;
-          const T* a_slab = a_tile0 + (A_KC ? static_cast<long long>(k0) : k0 * p.a_ld);
-          const T* b_slab = b_tile0 + (B_KC ? static_cast<long long>(k0) : k0 * p.b_ld);
-#pragma unroll
-          for (int round = 0; round < 2; ++round) {
-            HDirectLoad<A_KC>(a_slab, p.a_ld, a_ring + buffer * LA::ELEMS, wave_u, lane, round);
-            HDirectLoad<B_KC>(b_slab, p.b_ld, b_ring + buffer * LB::ELEMS, wave_u, lane, round);
+          if (load % 2 == 0) {
+            HDirectLoad<A_KC>(a_tile0 + (A_KC ? static_cast<long long>(k0) : k0 * p.a_ld), p.a_ld, a_ring + buffer * LA::ELEMS,
+                              wave_u, lane, load / 2);
+          } else {
+            HDirectLoad<B_KC>(b_tile0 + (B_KC ? static_cast<long long>(k0) : k0 * p.b_ld), p.b_ld, b_ring + buffer * LB::ELEMS,
+                              wave_u, lane, load / 2);
           }
         };
         int a_lane[FM], b_lane[FN];
@@ -364,7 +366,10 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
         for (int q = 0; q < FN; ++q) { b_lane[q] = HDirectLaneOffset<B_KC>(lane, (wave_n * FN + q) * 32); }
 #pragma unroll
         for (int s = 0; s < STAGES - 1; ++s) {
-          if (s < fast_slabs) { issue(s, s); }
+          if (s < fast_slabs) {
+#pragma unroll
+            for (int load = 0; load < LOADS_PER_SLAB; ++load) { issue(load, s, s); }
+          }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -399,7 +404,8 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
               for (int j = 0; j < FN; ++j) {
                 acc[q][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag[set][q], b_frag[set][j], acc[q][j], 0, 0, 0);
               }
-              if (ISSUE && ks == 0 && q == 0) { issue(slab + STAGES - 1, free_buffer); }
+              // one request per quarter: a burst of identical requests from all work-groups defeats the L2
+              if (ISSUE && ks == 0 && q < LOADS_PER_SLAB) { issue(q, slab + STAGES - 1, free_buffer); }
               __builtin_amdgcn_sched_barrier(0);
             }
             if (ks == KSTEPS - 2) {
