@@ -36,9 +36,12 @@
  *     code compiled from /root/reference into oracle/_ref (see oracle/Makefile) where that exists,
  *     and against committed fixtures produced from it (tests/golden/).
  *   - oracle_gemm: against hand-computed fixtures, numpy float64 matmul, and library CBLAS-style
- *     identities (tests/test_oracle.py); xgemm_port_* against oracle_gemm.
- *   - status functions: pinned by reading the reference source only; the reference's own tests never
- *     pin them without clBLAS. Stated as such in the tests.
+ *     identities (tests/test_oracle.py); xgemm_port_* against oracle_gemm; and against the results of
+ *     the real reference library run on an OpenCL device (tests/test_reference_opencl_gpu.py).
+ *   - gemm and strided-batched status functions: against the status codes the real reference library
+ *     returns for a 1000-case validation sweep per precision, executed on an OpenCL device
+ *     (tests/test_reference_opencl_gpu.py); the batched variant (per-batch offset arrays) by reading the
+ *     reference source only.
  * ================================================================================================= */
 #include <stddef.h>
 #include <stdint.h>

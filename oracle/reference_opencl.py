@@ -163,6 +163,50 @@ def run(spec):
     return status, result, times, opencl.device_name
 
 
+def status_sweep(spec):
+    """Calls the reference's gemm (or strided-batched gemm) once per case with buffers of exact byte sizes and
+    returns only the status codes: {"routine": "status_sweep", "bits", "strided": bool, "cases": [[layout, ta, tb,
+    m, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes] (+ [a_stride, b_stride, c_stride, batch] when strided)]}."""
+    bits = spec["bits"]
+    opencl = OpenCL()
+    reference = ctypes.CDLL(REF_LIBRARY)
+    sz, vp = ctypes.c_size_t, ctypes.c_void_p
+    queue = vp(opencl.queue.value)
+    pool = {}
+
+    def buffer_of(size_bytes, position):
+        key = (size_bytes, position)
+        if key not in pool:
+            pool[key] = opencl.buffer_from(np.zeros(max(size_bytes, 1), dtype=np.uint8))
+        return pool[key]
+
+    alpha, beta = scalar_argument(bits, 1.0, reference), scalar_argument(bits, 0.0, reference)
+    statuses = []
+    for case in spec["cases"]:
+        layout, ta, tb, m, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes = case[:12]
+        a, b, c = buffer_of(a_bytes, 0), buffer_of(b_bytes, 1), buffer_of(c_bytes, 2)
+        event = vp(None)
+        if spec.get("strided"):
+            a_stride, b_stride, c_stride, batch = case[12:16]
+            function = getattr(reference, "CLBlast%sgemmStridedBatched" % PREFIX[bits])
+            status = function(ctypes.c_int(layout), ctypes.c_int(ta), ctypes.c_int(tb), sz(m), sz(n), sz(k), alpha, a, sz(0),
+                              sz(a_ld), sz(a_stride), b, sz(0), sz(b_ld), sz(b_stride), beta, c, sz(0), sz(c_ld), sz(c_stride),
+                              sz(batch), ctypes.byref(queue), ctypes.byref(event))
+        else:
+            function = getattr(reference, "CLBlast%sgemm" % PREFIX[bits])
+            status = function(ctypes.c_int(layout), ctypes.c_int(ta), ctypes.c_int(tb), sz(m), sz(n), sz(k), alpha, a, sz(0),
+                              sz(a_ld), b, sz(0), sz(b_ld), beta, c, sz(0), sz(c_ld), ctypes.byref(queue), ctypes.byref(event))
+        if status == 0 and event.value:
+            events = (vp * 1)(event.value)
+            opencl.cl.clWaitForEvents(1, events)
+            opencl.cl.clReleaseEvent(event)
+        statuses.append(int(status))
+    opencl.finish()
+    for handle in pool.values():
+        opencl.cl.clReleaseMemObject(handle)
+    return statuses, opencl.device_name
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--spec", required=True)
@@ -174,6 +218,11 @@ def main():
     outputs = {}
     summary = []
     for index, spec in enumerate(specs):
+        if spec.get("routine") == "status_sweep":
+            statuses, device_name = status_sweep(spec)
+            summary.append({"statuses": statuses, "device": device_name})
+            print("reference_opencl: case %d: %d status codes on %s" % (index, len(statuses), device_name), flush=True)
+            continue
         status, result, times, device_name = run(spec)
         if not args.no_results:
             outputs["c_%d" % index] = result

@@ -132,3 +132,36 @@ def test_baseline_shapes_against_the_reference(gpu, tmp_path):
     data, summary = run_reference(specs, tmp_path)
     for index, spec in enumerate(specs):
         compare(gpu, spec, data["c_%d" % index], summary[index]["status"])
+
+
+def status_cases(bits):
+    eb = bits // 8
+    full = 64 * 64 * eb
+    cases = []
+    for layout, ta, tb in itertools.product((ROW_MAJOR, COL_MAJOR), (NO, YES), (NO, YES)):
+        for m, n, k in ((64, 64, 64), (7, 64, 7), (0, 64, 64), (64, 0, 64), (64, 64, 0)):
+            for lds in ((64, 64, 64), (7, 64, 64), (64, 7, 64), (64, 64, 7), (7, 7, 7)):
+                for sizes in ((full, full, full), (full - eb, full, full), (full, full - eb, full),
+                              (full, full, full - eb), (eb, eb, eb)):
+                    cases.append([layout, ta, tb, m, n, k, lds[0], lds[1], lds[2], sizes[0], sizes[1], sizes[2]])
+    return cases
+
+
+@pytest.mark.parametrize("bits", (32, 64, 16))
+def test_status_codes_of_the_real_reference(gpu, tmp_path, bits):
+    """The argument checks of the reference, executed: its status for every case of the validation sweep (zero
+    dimensions, short leading dimensions, short buffers, in all orders) must be the one the oracle's restatement
+    predicts - the same sweep that tests/test_status_gpu.py runs against this library."""
+    cases = status_cases(bits)
+    strided = [case + [64 * 64, 64 * 64, 64 * 64, batch] for case in cases[::7] for batch in (1, 0, 2)]
+    _, summary = run_reference([dict(routine="status_sweep", bits=bits, cases=cases),
+                                dict(routine="status_sweep", bits=bits, strided=True, cases=strided)], tmp_path)
+    for case, status in zip(cases, summary[0]["statuses"]):
+        layout, ta, tb, m, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes = case
+        expected = oracle.gemm_status(bits, layout, ta, tb, m, n, k, 0, a_ld, a_bytes, 0, b_ld, b_bytes, 0, c_ld, c_bytes)
+        assert status == expected, (case, status, expected)
+    for case, status in zip(strided, summary[1]["statuses"]):
+        layout, ta, tb, m, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes, a_stride, b_stride, c_stride, batch = case
+        expected = oracle.strided_status(bits, layout, ta, tb, m, n, k, 0, a_ld, a_stride, a_bytes, 0, b_ld,
+                                          b_stride, b_bytes, 0, c_ld, c_stride, c_bytes, batch)
+        assert status == expected, (case, status, expected)
