@@ -38,10 +38,9 @@
  *   - oracle_gemm: against hand-computed fixtures, numpy float64 matmul, and library CBLAS-style
  *     identities (tests/test_oracle.py); xgemm_port_* against oracle_gemm; and against the results of
  *     the real reference library run on an OpenCL device (tests/test_reference_opencl_gpu.py).
- *   - gemm and strided-batched status functions: against the status codes the real reference library
- *     returns for a 1000-case validation sweep per precision, executed on an OpenCL device
- *     (tests/test_reference_opencl_gpu.py); the batched variant (per-batch offset arrays) by reading the
- *     reference source only.
+ *   - status functions (gemm, batched, strided-batched): against the status codes the real reference
+ *     library returns for a validation sweep per precision (1000 + 455 + 430 cases), executed on an
+ *     OpenCL device (tests/test_reference_opencl_gpu.py).
  * ================================================================================================= */
 #include <stddef.h>
 #include <stdint.h>

@@ -166,7 +166,8 @@ def run(spec):
 def status_sweep(spec):
     """Calls the reference's gemm (or strided-batched gemm) once per case with buffers of exact byte sizes and
     returns only the status codes: {"routine": "status_sweep", "bits", "strided": bool, "cases": [[layout, ta, tb,
-    m, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes] (+ [a_stride, b_stride, c_stride, batch] when strided)]}."""
+    m, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes] (+ [a_stride, b_stride, c_stride, batch] when "strided",
+    + [a_offsets, b_offsets, c_offsets] (lists, one entry per batch) when "batched")]}."""
     bits = spec["bits"]
     opencl = OpenCL()
     reference = ctypes.CDLL(REF_LIBRARY)
@@ -186,7 +187,17 @@ def status_sweep(spec):
         layout, ta, tb, m, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes = case[:12]
         a, b, c = buffer_of(a_bytes, 0), buffer_of(b_bytes, 1), buffer_of(c_bytes, 2)
         event = vp(None)
-        if spec.get("strided"):
+        if spec.get("batched"):
+            offsets = case[12:15]  # three lists of element offsets, one entry per batch
+            count = len(offsets[0])
+            scalars = (SCALAR[bits] * max(count, 1))(*([alpha.value] * count))
+            zeros = (SCALAR[bits] * max(count, 1))(*([beta.value] * count))
+            arrays = [(sz * max(count, 1))(*values) for values in offsets]
+            function = getattr(reference, "CLBlast%sgemmBatched" % PREFIX[bits])
+            status = function(ctypes.c_int(layout), ctypes.c_int(ta), ctypes.c_int(tb), sz(m), sz(n), sz(k), scalars, a,
+                              arrays[0], sz(a_ld), b, arrays[1], sz(b_ld), zeros, c, arrays[2], sz(c_ld), sz(count),
+                              ctypes.byref(queue), ctypes.byref(event))
+        elif spec.get("strided"):
             a_stride, b_stride, c_stride, batch = case[12:16]
             function = getattr(reference, "CLBlast%sgemmStridedBatched" % PREFIX[bits])
             status = function(ctypes.c_int(layout), ctypes.c_int(ta), ctypes.c_int(tb), sz(m), sz(n), sz(k), alpha, a, sz(0),

@@ -154,8 +154,16 @@ def test_status_codes_of_the_real_reference(gpu, tmp_path, bits):
     predicts - the same sweep that tests/test_status_gpu.py runs against this library."""
     cases = status_cases(bits)
     strided = [case + [64 * 64, 64 * 64, 64 * 64, batch] for case in cases[::7] for batch in (1, 0, 2)]
+    offset_sets = ([[0], [0], [0]], [[0, 8], [0, 8], [0, 8]], [[], [], []], [[0, 4096], [0, 0], [0, 0]], [[0, 0], [0, 0], [0, 4096]])
+    batched = [case + [list(o) for o in offsets] for case in cases[::11] for offsets in offset_sets]
     _, summary = run_reference([dict(routine="status_sweep", bits=bits, cases=cases),
-                                dict(routine="status_sweep", bits=bits, strided=True, cases=strided)], tmp_path)
+                                dict(routine="status_sweep", bits=bits, strided=True, cases=strided),
+                                dict(routine="status_sweep", bits=bits, batched=True, cases=batched)], tmp_path)
+    for case, status in zip(batched, summary[2]["statuses"]):
+        layout, ta, tb, m, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes, a_offsets, b_offsets, c_offsets = case
+        expected = oracle.batched_status(bits, layout, ta, tb, m, n, k, a_offsets, a_ld, a_bytes, b_offsets, b_ld, b_bytes,
+                                         c_offsets, c_ld, c_bytes, len(a_offsets))
+        assert status == expected, (case, status, expected)
     for case, status in zip(cases, summary[0]["statuses"]):
         layout, ta, tb, m, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes = case
         expected = oracle.gemm_status(bits, layout, ta, tb, m, n, k, 0, a_ld, a_bytes, 0, b_ld, b_bytes, 0, c_ld, c_bytes)
