@@ -10,8 +10,8 @@ namespace {
 int LaunchMfmaF32(const clbh_gemm_desc& d, hipStream_t stream) {
   if (!LeadingDimsFitTiles<float>(d)) { return LaunchGeneral<float>(d, stream); }
   switch (d.tile_variant) {
-    case 1: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16, 3>>(d, stream);
-    case 2: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16, 4>>(d, stream);
+    case 1: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 1, 1, 32, 4>>(d, stream);  // 64 x 64 x 32
+    case 2: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 1, 1, 64, 4>>(d, stream);  // 64 x 64 x 64
     case 3: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 4, 2, 16, 2>>(d, stream);  // 256 x 128 x 16
     case 4: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 32, 2>>(d, stream);  // 128 x 128 x 32
     case 5: return LaunchMfmaConfig<float, MfmaConfig<float, 4, 1, 1, 1, 32, 4>>(d, stream);  // 128 x 32 x 32 (skinny n)

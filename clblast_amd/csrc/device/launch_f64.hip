@@ -10,7 +10,7 @@ namespace {
 int LaunchMfmaF64(const clbh_gemm_desc& d, hipStream_t stream) {
   if (!LeadingDimsFitTiles<double>(d)) { return LaunchGeneral<double>(d, stream); }
   switch (d.tile_variant) {
-    case 1: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 2, 8, 2>>(d, stream);   // 128 x 64 x 8
+    case 1: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 2, 2, 16, 3>>(d, stream);  // 64 x 64 x 16
     case 2: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 2, 16, 2>>(d, stream);  // 128 x 64 x 16
     case 3: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 2, 16, 3>>(d, stream);  // 128 x 64 x 16
     case 4: return LaunchMfmaConfig<double, MfmaConfig<double, 2, 2, 4, 4, 16, 2>>(d, stream);  // 128 x 128 x 16

@@ -16,11 +16,18 @@ namespace {
 std::mutex override_mutex;
 std::map<std::tuple<int, int>, size_t> min_indirect_overrides;  // (device, precision bits) -> threshold
 std::map<int, size_t> tile_variant_overrides;                   // precision bits -> forced MFMA tile (0 = automatic)
+std::map<int, size_t> split_overrides;                          // precision bits -> K ranges of a forced tile
 
 size_t ForcedTileVariant(const Precision precision) {
   std::lock_guard<std::mutex> lock(override_mutex);
   const auto found = tile_variant_overrides.find(static_cast<int>(precision));
   return (found != tile_variant_overrides.end()) ? found->second : 0;
+}
+
+size_t ForcedSplit(const Precision precision) {
+  std::lock_guard<std::mutex> lock(override_mutex);
+  const auto found = split_overrides.find(static_cast<int>(precision));
+  return (found != split_overrides.end() && found->second > 0) ? found->second : 1;
 }
 
 }  // namespace
@@ -53,20 +60,22 @@ bool UseDirectKernel(const size_t m, const size_t n, const size_t k, const size_
 }
 
 // fp32 tile table (index -> work-group tile), see device/launch.hip:
-//   1: 128 x 128 x 16   3: 256 x 128 x 16   5: 128 x 32 x 32   6: 32 x 128 x 32   7: 64 x 64 x 16
+//   0: 128 x 128 x 16   3: 256 x 128 x 16   5: 128 x 32 x 32   6: 32 x 128 x 32   7: 64 x 64 x 16
 namespace {
 struct Tile {
   int index;
   size_t tile_m, tile_n;
 };
 
-// Number of K ranges that brings the launch to about two work-groups per CU, keeping ranges >= 128.
+// Number of K ranges for a launch of `tiles` work-groups. Splitting costs a second launch (the reduction, about
+// 8 us) and pays only when most CUs would idle through a long K walk (about 16 ns per unit of k and work-group):
+// ranges stay >= 512 deep and bring the launch to about two work-groups per CU.
 int SplitFor(const size_t tiles, const size_t k) {
   constexpr size_t kWantedGroups = 512;
-  if (tiles >= 256 || k < 512) { return 1; }
+  if (tiles >= 192 || k < 2048) { return 1; }
   const auto wanted = CeilDivide(kWantedGroups, tiles);
-  const auto allowed = k / 128;
-  return static_cast<int>(std::max<size_t>(1, std::min<size_t>({wanted, allowed, 64})));
+  const auto allowed = k / 512;
+  return static_cast<int>(std::max<size_t>(1, std::min<size_t>({wanted, allowed, 32})));
 }
 }  // namespace
 
@@ -83,7 +92,10 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   }
   const auto forced = ForcedTileVariant(precision);
   if (forced != 0) {
-    return KernelChoice{CLBH_KERNEL_MFMA, static_cast<int>(forced) - 1, 1};
+    // a forced tile takes the forced number of K ranges (fp32/fp64, unbatched calls only), never more than k / 16
+    const auto ranges = (precision != Precision::kHalf && batch_count == 1)
+                            ? std::max<size_t>(1, std::min<size_t>(ForcedSplit(precision), k / 16)) : 1;
+    return KernelChoice{CLBH_KERNEL_MFMA, static_cast<int>(forced) - 1, static_cast<int>(ranges)};
   }
   if (precision == Precision::kHalf) {
     // 256 x 256 tiles (8 wavefronts, ring of 3 direct-loaded slabs: index 3) once there are at least two per CU,
@@ -92,18 +104,22 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     return KernelChoice{CLBH_KERNEL_MFMA, (big_tiles >= 512) ? 3 : 0, 1};
   }
   if (precision == Precision::kSingle) {
-    auto tile = Tile{1, 128, 128};
-    if (CeilDivide(m, 256) * CeilDivide(n, 128) >= 512) { tile = Tile{3, 256, 128}; }
-    else if (n <= 32 && m >= 256) { tile = Tile{5, 128, 32}; }   // skinny: stream A
+    // Measured on the MI355X (tile x split sweep over 18 shapes): 64 x 64 tiles (several work-groups per CU hide
+    // each other's latencies) win up to about 3072^3 and whenever k is short (C traffic dominates); 256 x 128 needs
+    // two full rounds of tiles and a long K walk; the skinny tiles stream the one large operand.
+    auto tile = Tile{7, 64, 64};
+    if (n <= 32 && m >= 256) { tile = Tile{5, 128, 32}; }        // skinny: stream A
     else if (m <= 32 && n >= 256) { tile = Tile{6, 32, 128}; }   // skinny: stream B
-    else if (CeilDivide(m, 128) * CeilDivide(n, 128) < 128) { tile = Tile{7, 64, 64}; }
+    else if (CeilDivide(m, 256) * CeilDivide(n, 128) >= 512 && k >= 1024) { tile = Tile{3, 256, 128}; }
     const auto tiles = CeilDivide(m, tile.tile_m) * CeilDivide(n, tile.tile_n) * batch_count;
     const auto split = (batch_count == 1) ? SplitFor(tiles, k) : 1;
     return KernelChoice{CLBH_KERNEL_MFMA, tile.index, split};
   }
-  // fp64: 128 x 128 x 8 tiles, split K when they cannot fill the chip
-  const auto tiles = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
-  return KernelChoice{CLBH_KERNEL_MFMA, 0, (batch_count == 1) ? SplitFor(tiles, k) : 1};
+  // fp64 (same sweep): 64 x 64 x 16 tiles (index 1) up to about 3072^3, 128 x 128 x 8 (index 0) beyond
+  const bool large = CeilDivide(m, 128) * CeilDivide(n, 128) >= 1024 && k >= 1024;
+  const auto tile_size = large ? size_t{128} : size_t{64};
+  const auto tiles = CeilDivide(m, tile_size) * CeilDivide(n, tile_size) * batch_count;
+  return KernelChoice{CLBH_KERNEL_MFMA, large ? 0 : 1, (batch_count == 1) ? SplitFor(tiles, k) : 1};
 }
 
 StatusCode OverrideRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,
@@ -113,8 +129,10 @@ StatusCode OverrideRoutineParameters(const int device, const std::string& kernel
     if (variant == parameters.end()) {
       return StatusCode::kMissingOverrideParameter;
     }
+    const auto split = parameters.find("SPLIT_K");
     std::lock_guard<std::mutex> lock(override_mutex);
     tile_variant_overrides[static_cast<int>(precision)] = variant->second;
+    split_overrides[static_cast<int>(precision)] = (split != parameters.end()) ? split->second : 1;
     return StatusCode::kSuccess;
   }
   if (kernel_name != "GemmRoutine") {
@@ -133,6 +151,7 @@ StatusCode RetrieveRoutineParameters(const int device, const std::string& kernel
                                      std::unordered_map<std::string, size_t>& parameters) {
   if (kernel_name == "Xgemm") {
     parameters["TILE_VARIANT"] = ForcedTileVariant(precision);
+    parameters["SPLIT_K"] = ForcedSplit(precision);
     return StatusCode::kSuccess;
   }
   if (kernel_name != "GemmRoutine") {
@@ -146,6 +165,7 @@ void ClearOverrides() {
   std::lock_guard<std::mutex> lock(override_mutex);
   min_indirect_overrides.clear();
   tile_variant_overrides.clear();
+  split_overrides.clear();
 }
 
 }  // namespace clblast
