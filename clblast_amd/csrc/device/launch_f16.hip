@@ -1,8 +1,9 @@
 // =================================================================================================
-// fp16 instantiations: general kernel, the two HGEMM MFMA kernels and the fp16 tile table.
+// fp16 instantiations: general kernel, the direct-load HGEMM kernel and its element-wise fallback.
 // =================================================================================================
 #include "device/launch_common.hpp"
 #include "kernels/gemm_general.hpp"
+#include "kernels/gemm_direct_f16.hpp"
 #include "kernels/gemm_mfma_f16.hpp"
 
 namespace clbh {
@@ -59,20 +60,62 @@ int LaunchHgemmConfig(const clbh_gemm_desc& d, hipStream_t stream) {
   }
 }
 
+// ---- direct-load MFMA kernel, fp16 (dword-aligned operands) ---------------------------------------
+template <typename Config, bool A_KC, bool B_KC>
+int LaunchHdirectVariant(const clbh_gemm_desc& d, hipStream_t stream) {
+  const auto args = MakeArgs<float>(d);
+  const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
+  const long long tiles_n = (d.n + Config::TILE_N - 1) / Config::TILE_N;
+  if (tiles_m * tiles_n > INT_MAX) { return hipErrorInvalidConfiguration; }
+  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
+  constexpr size_t lds_bytes = Config::LDS_BYTES;
+  auto kernel = HgemmDirectKernel<Config, A_KC, B_KC>;
+  if (lds_bytes > 48 * 1024) {
+    static const hipError_t attribute_status = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+    if (attribute_status != hipSuccess) { return static_cast<int>(attribute_status); }
+  }
+  kernel<<<grid, dim3(Config::THREADS), lds_bytes, stream>>>(args, static_cast<int>(tiles_m), static_cast<int>(tiles_n));
+  return static_cast<int>(hipGetLastError());
+}
+
+template <typename Config>
+int LaunchHdirectConfig(const clbh_gemm_desc& d, hipStream_t stream) {
+  const int variant = (d.a_kcontig ? 2 : 0) | (d.b_kcontig ? 1 : 0);
+  switch (variant) {
+    case 0: return LaunchHdirectVariant<Config, false, false>(d, stream);
+    case 1: return LaunchHdirectVariant<Config, false, true>(d, stream);
+    case 2: return LaunchHdirectVariant<Config, true, false>(d, stream);
+    default: return LaunchHdirectVariant<Config, true, true>(d, stream);
+  }
+}
+
+// True when the direct global -> LDS loads of the fp16 kernel are possible: they move dwords.
+bool DwordAlignedHalf(const clbh_gemm_desc& d) {
+  const auto address = [](const void* base, long long offset) {
+    return reinterpret_cast<unsigned long long>(base) + static_cast<unsigned long long>(offset) * 2;
+  };
+  if (address(d.a, d.a_offset) % 4 || address(d.b, d.b_offset) % 4) { return false; }
+  if (d.a_ld % 2 || d.b_ld % 2) { return false; }
+  if (d.batch_count > 1) {
+    if (d.batch.alphas != nullptr) { return false; }  // per-batch offsets are only known on the device
+    if (d.a_stride % 2 || d.b_stride % 2) { return false; }
+  }
+  return true;
+}
+
 }  // namespace
 
 int LaunchMfmaF16(const clbh_gemm_desc& d, hipStream_t stream) {
   if (!LeadingDimsFitTiles<_Float16>(d)) { return LaunchGeneral<_Float16>(d, stream); }
-  // The large tiles exist for 16-byte aligned operands only; everything else takes 128 x 128.
-  using Small = HgemmConfig<2, 2, 2, 2, 32, 2, false>;  // 128 x 128 x 32, 4 waves
-  if (!Aligned16<_Float16>(d)) { return LaunchHgemmConfig<Small, false>(d, stream); }
+  // operands at odd element offsets or with odd leading dimensions: element-wise 128 x 128 kernel
+  if (!DwordAlignedHalf(d)) { return LaunchHgemmConfig<HgemmConfig<2, 2, 2, 2, 32, 2>, false>(d, stream); }
   switch (d.tile_variant) {
-    case 1: return LaunchHgemmConfig<HgemmConfig<2, 4, 4, 2, 32, 2, false>, true>(d, stream);  // 256 x 256 x 32, 8 waves
-    // 256 x 256 x 32, 8 waves, explicitly scheduled, direct global -> LDS loads into a ring of 4 / 3 / 2 slabs
-    case 2: return LaunchHgemmConfig<HgemmConfig<2, 4, 4, 2, 32, 2, true, 4>, true>(d, stream);
-    case 3: return LaunchHgemmConfig<HgemmConfig<2, 4, 4, 2, 32, 2, true, 3>, true>(d, stream);
-    case 4: return LaunchHgemmConfig<HgemmConfig<2, 4, 4, 2, 32, 2, true, 2>, true>(d, stream);
-    default: return LaunchHgemmConfig<Small, true>(d, stream);
+    case 1: return LaunchHdirectConfig<HdirectConfig<2, 2, 1, 1, 4>>(d, stream);  // 64 x 64, 4 wavefronts
+    case 2: return LaunchHdirectConfig<HdirectConfig<2, 4, 4, 2, 2>>(d, stream);  // 256 x 256, 8 wavefronts
+    case 3: return LaunchHdirectConfig<HdirectConfig<4, 1, 1, 1, 4>>(d, stream);  // 128 x 32 (skinny n)
+    case 4: return LaunchHdirectConfig<HdirectConfig<1, 4, 1, 1, 4>>(d, stream);  // 32 x 128 (skinny m)
+    default: return LaunchHdirectConfig<HdirectConfig<2, 2, 2, 2, 2>>(d, stream);  // 128 x 128, 4 wavefronts
   }
 }
 

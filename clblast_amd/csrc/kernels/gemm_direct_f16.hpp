@@ -1,0 +1,384 @@
+// =================================================================================================
+// MFMA GEMM kernel for gfx950, fp16 storage with fp32 accumulation (HGEMM), for operands whose
+// addresses are dword aligned (base and offsets multiples of 4 bytes, even leading dimensions). It
+// replaces the reference's whole "indirect" chain (src/routines/level3/xgemm.cpp:102-222,
+// src/kernels/level3/xgemm_part1-4.opencl) and its direct kernels (xgemm_direct_part1-3.opencl) with
+// one launch that reads the caller's operands in place. Unlike the reference, which accumulates in
+// fp16 (src/kernels/common.opencl:44-45), products are accumulated in fp32 by
+// v_mfma_f32_32x32x16_f16 and rounded to fp16 once, in the epilogue.
+//
+// Structure:
+//   * work-group tile (32*WM*FM) x (32*WN*FN), one wavefront per FM x FN blocks of 32 x 32; K is walked
+//     in slabs of 32 that live in a ring of three LDS buffers;
+//   * every slab goes global -> LDS directly (`buffer_load_dwordx4 ... lds`: lane l's 16 bytes land at
+//     base + 16 * l, so LDS is filled in 1 KiB pieces whose inner order is fixed, while which 16 bytes of
+//     global memory a lane fetches is free - that freedom carries the bank swizzles). The resources
+//     are cut off at the end of the operand: loads beyond it touch no memory and deliver zero, so edge
+//     tiles and the K tail of an x-contiguous operand need nothing special; the K tail of a
+//     k-contiguous operand (whose out-of-range elements are the next line's data) is zeroed in LDS by
+//     the wavefront that requested the piece;
+//   * the MFMA wants 8 consecutive k per lane. A k-contiguous operand is kept as [x][32] (16-byte chunk c
+//     of row x at position c ^ ((x >> 2) & 3): the 16-byte reads of 16 consecutive rows cover all 64 banks
+//     once) and read with one ds_read_b128 per fragment. An x-contiguous operand is kept as [k][W] (chunk t
+//     of row k at t ^ swizzle(k)) and read with the CDNA4 transposing LDS read ds_read_b64_tr_b16. LDS
+//     serves 32 lanes of such a read per cycle: rows k..k+3, 64 bytes each, which the swizzle spreads
+//     over four different 16-dword bank windows;
+//   * explicit schedule, fenced for the compiler: per quarter of a k-step "LDS reads of the fragments of
+//     the next k-step (other register set), FN MFMAs, a share of the requests for slab t+2"; one barrier
+//     per slab, before its last k-step, so that the last k-step already fetches the first fragments of
+//     slab t+1 and the matrix pipe never drains at a slab boundary;
+//   * the m-indexed fragment is the MFMA's A operand, so a lane holds runs of four consecutive m; the
+//     epilogue stages each block column through LDS and moves C in 16-byte pieces along m.
+// =================================================================================================
+#ifndef CLBLAST_HIP_KERNELS_GEMM_DIRECT_F16_HPP_
+#define CLBLAST_HIP_KERNELS_GEMM_DIRECT_F16_HPP_
+
+#include <type_traits>
+
+#include "kernels/gemm_args.hpp"
+#include "kernels/gemm_mfma.hpp"
+#include "kernels/gemm_mfma_f16.hpp"
+
+namespace clbh {
+
+// WM x WN wavefronts per work-group, each owning FM x FN MFMA blocks of 32 x 32 (FM >= FN). MIN_WAVES is the
+// number of wavefronts per SIMD the register budget must allow.
+template <int WM_, int WN_, int FM_, int FN_, int MIN_WAVES_>
+struct HdirectConfig {
+  static constexpr int WM = WM_, WN = WN_, FM = FM_, FN = FN_, MIN_WAVES = MIN_WAVES_;
+  static constexpr int WAVES = WM * WN, THREADS = 64 * WAVES;
+  static constexpr int TILE_M = WM * FM * 32, TILE_N = WN * FN * 32, TILE_K = 32, STAGES = 3;
+  static constexpr int PIECES_A = TILE_M / 16, PIECES_B = TILE_N / 16;  // 1 KiB pieces of a slab
+  static constexpr int ROUNDS = (PIECES_A + PIECES_B + WAVES - 1) / WAVES;  // requests per wavefront and slab
+  static constexpr bool DUMMY = (PIECES_A + PIECES_B) % WAVES != 0;  // some requests go to a scratch piece
+  static constexpr int A_ELEMS = PIECES_A * 512, B_ELEMS = PIECES_B * 512;  // halfs per stage
+  static constexpr int RING_BYTES = (STAGES * (A_ELEMS + B_ELEMS) + (DUMMY ? 512 : 0)) * 2;
+  static constexpr int EPILOGUE_BYTES = WAVES * 32 * (FM * 32 + 8) * 2;
+  static constexpr int LDS_BYTES = RING_BYTES > EPILOGUE_BYTES ? RING_BYTES : EPILOGUE_BYTES;
+  static_assert(FM >= FN, "the quarters of a k-step run over the m blocks");
+};
+
+// Chunk swizzle of row k of an x-contiguous slab [k][W]: rows k..k+3 must fall into different 16-dword
+// bank windows for a 64-byte read per row.
+template <int W>
+__device__ __forceinline__ int HSwizzle(const int k) {
+  return (W >= 128) ? 4 * (k & 3) : (W == 64) ? 4 * ((k >> 1) & 1) : 0;
+}
+
+// Byte count from `from` to `end`, rounded up to whole dwords (the range check works per dword; the last
+// one may hold a single valid half) and clamped to what a resource can hold.
+__device__ __forceinline__ int HRecordsUpTo(const void* from, const void* end) {
+  const long long bytes = (static_cast<const char*>(end) - static_cast<const char*>(from) + 3) & ~3ll;
+  int high = static_cast<int>(bytes >> 32);
+  const unsigned int low = static_cast<unsigned int>(bytes);
+  asm("" : "+s"(high));  // opaque, or the halves are fused back into 64-bit vector compares
+  return static_cast<int>(high < 0 ? 0u : (high != 0 ? 0xffffffffu : low));
+}
+
+// Requests piece `piece` (1 KiB) of the slab at `slab` (element (x0, k0), uniform) into `stage`.
+// KC: the piece is x rows 16*piece..+15 of 32 halfs; XC: k rows (512/W)*piece.. of W halfs.
+template <int W, bool KC, bool RANGE, typename Tag>
+__device__ __forceinline__ void HRequestPiece(const _Float16* __restrict__ slab, const _Float16* valid_end, const long long ld,
+                                              _Float16* stage, const int piece, const int lane) {
+  constexpr int ROWS = KC ? 16 : 512 / W, CHUNKS = KC ? 4 : W / 8;  // rows of the piece, 16-byte chunks per row
+  const int row = lane / CHUNKS, position = lane % CHUNKS;
+  const int chunk = KC ? position ^ ((row >> 2) & 3) : position ^ HSwizzle<W>(ROWS * piece + row);
+  const _Float16* source = slab + static_cast<long long>(ROWS * piece) * ld;
+  const int lane_bytes = static_cast<int>((row * ld + 8 * chunk) * 2);
+  typedef __attribute__((address_space(3))) void* LdsPtr;
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(source), 0, RANGE ? HRecordsUpTo(source, valid_end) : -1,
+                                        kRawBufferFlags),
+      (LdsPtr)(stage + piece * 512), 16, lane_bytes, 0, 0, 0);
+}
+
+// After its own request for a k-contiguous piece has landed, the wavefront zeroes the elements k >= k_valid.
+__device__ __forceinline__ void HZeroTail(_Float16* stage, const int piece, const int lane, const int k_valid) {
+  const int row = lane / 4, chunk = (lane % 4) ^ ((row >> 2) & 3);
+  half8_t* cell = reinterpret_cast<half8_t*>(stage + piece * 512 + lane * 8);
+  if (8 * chunk + 7 >= k_valid) {
+    half8_t value = *cell;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { if (8 * chunk + e >= k_valid) { value[e] = _Float16(0); } }
+    *cell = value;
+  }
+}
+
+// Offset (halfs) of a lane's fragment data for the block starting at x32 (a multiple of 32), k-step 0.
+template <int W, bool KC>
+__device__ __forceinline__ int HFragmentOffset(const int lane, const int x32) {
+  if (KC) {
+    const int x = x32 + lane % 32;
+    return x * 32 + 8 * ((lane / 32) ^ ((x >> 2) & 3));
+  } else {
+    const int group = lane / 16, q = lane % 16;
+    const int k = 8 * (group / 2) + q / 4;
+    const int x = x32 + 16 * (group % 2) + 4 * (q % 4);
+    return k * W + 8 * ((x / 8) ^ HSwizzle<W>(k)) + x % 8;
+  }
+}
+
+// Fragment of k-step ks (0 or 1) of a stage.
+template <int W, bool KC>
+__device__ __forceinline__ half8_t HFragment(const _Float16* __restrict__ stage, const int offset, const int ks) {
+  if (KC) {
+    // chunk index of the k-step is 2*ks + lane/32; the swizzle is an XOR, so k-step 1 flips bit 1 of it
+    return *reinterpret_cast<const half8_t*>(&stage[offset ^ (ks * 16)]);
+  } else {
+    typedef __attribute__((address_space(3))) short4_t* LdsPtr;
+    const _Float16* src = stage + ks * 16 * W + offset;  // rows k + 16 * ks: the swizzle depends on k % 4 only
+    const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(src));
+    const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(src + 4 * W));
+    half8_t out;
+    const half4_t lo_h = __builtin_bit_cast(half4_t, lo), hi_h = __builtin_bit_cast(half4_t, hi);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { out[e] = lo_h[e]; out[4 + e] = hi_h[e]; }
+    return out;
+  }
+}
+
+// ---- the kernel ------------------------------------------------------------------------------------
+template <typename Config, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirectKernel(const GemmArgs<float> p, const int tiles_m,
+                                                                  const int tiles_n) {
+  using T = _Float16;
+  constexpr int TILE_M = Config::TILE_M, TILE_N = Config::TILE_N, TILE_K = Config::TILE_K;
+  constexpr int FM = Config::FM, FN = Config::FN, WAVES = Config::WAVES, STAGES = Config::STAGES, ROUNDS = Config::ROUNDS;
+  constexpr int KSTEPS = TILE_K / 16;
+  static_assert(KSTEPS == 2 && STAGES == 3, "schedule below: one barrier after the first of two k-steps, ring of three");
+  using KernelTag = std::tuple<Config, std::integral_constant<int, (A_KC ? 2 : 0) | (B_KC ? 1 : 0)>>;
+
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+  T* a_ring = lds;                               // [STAGES][A_ELEMS]
+  T* b_ring = lds + STAGES * Config::A_ELEMS;    // [STAGES][B_ELEMS]
+  T* scratch_piece = lds + STAGES * (Config::A_ELEMS + Config::B_ELEMS);
+
+  const int tid = threadIdx.x;
+  const int lane = tid % 64, wave = tid / 64;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int wave_m = wave % Config::WM, wave_n = wave / Config::WM;
+
+  int tile_m, tile_n;
+  TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
+
+  int a_offset[FM], b_offset[FN];
+#pragma unroll
+  for (int q = 0; q < FM; ++q) { a_offset[q] = HFragmentOffset<TILE_M, A_KC>(lane, (wave_m * FM + q) * 32); }
+#pragma unroll
+  for (int q = 0; q < FN; ++q) { b_offset[q] = HFragmentOffset<TILE_N, B_KC>(lane, (wave_n * FN + q) * 32); }
+
+  for (int batch = blockIdx.y; batch < p.batch_count; batch += gridDim.y) {
+    const T* a;
+    const T* b;
+    T* c;
+    float alpha, beta;
+    ResolveBatch<T, float>(p, batch, a, b, c, alpha, beta);
+    const int k_len = p.k;
+    const int slabs = (k_len + TILE_K - 1) / TILE_K;
+    const int k_tail = k_len % TILE_K;  // valid depth of the last slab when it is partial
+
+    float16_t acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+#pragma unroll
+      for (int j = 0; j < FN; ++j) { acc[i][j] = float16_t(0.0f); }
+    }
+
+    const T* a_tile0 = a + (A_KC ? m0 * p.a_ld : static_cast<long long>(m0));  // element (m0, k = 0), uniform
+    const T* b_tile0 = b + (B_KC ? n0 * p.b_ld : static_cast<long long>(n0));
+    // behind the last element of the operand: (x = extent - 1, k = k_len - 1) + 1
+    const T* a_end = a + (A_KC ? (p.m - 1) * p.a_ld + k_len : (k_len - 1) * p.a_ld + p.m);
+    const T* b_end = b + (B_KC ? (p.n - 1) * p.b_ld + k_len : (k_len - 1) * p.b_ld + p.n);
+
+    // The walk exists twice: with range-checked requests (tiles that touch an edge of the matrix, or a K
+    // tail), and without (saves the scalar arithmetic of one byte count per request).
+    auto walk = [&](auto range_tag) {
+      constexpr bool RANGE = decltype(range_tag)::value;
+      // request `round` of this wavefront for slab `slab` into ring position `buffer`
+      auto request = [&](const int round, const int slab, const int buffer) {
+        const int k0 = slab * TILE_K;
+        const int piece = wave_u + WAVES * round;
+        if (piece < Config::PIECES_A) {
+          HRequestPiece<TILE_M, A_KC, RANGE, KernelTag>(a_tile0 + (A_KC ? static_cast<long long>(k0) : k0 * p.a_ld), a_end, p.a_ld,
+                                                        a_ring + buffer * Config::A_ELEMS, piece, lane);
+        } else if (!Config::DUMMY || piece < Config::PIECES_A + Config::PIECES_B) {
+          HRequestPiece<TILE_N, B_KC, RANGE, KernelTag>(b_tile0 + (B_KC ? static_cast<long long>(k0) : k0 * p.b_ld), b_end, p.b_ld,
+                                                        b_ring + buffer * Config::B_ELEMS, piece - Config::PIECES_A, lane);
+        } else {
+          // keeps the number of outstanding requests equal in all wavefronts (the waits count them): an
+          // empty resource moves nothing but zeros, into a piece nobody reads
+          typedef __attribute__((address_space(3))) void* LdsPtr;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(__builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a_tile0), 0, 0, kRawBufferFlags),
+                                                   (LdsPtr)(scratch_piece), 16, lane * 16, 0, 0, 0);
+        }
+      };
+      // zeroes the K tail of the k-contiguous pieces this wavefront requested for the slab in `buffer`
+      auto zero_tail = [&](const int buffer) {
+        if (!RANGE || k_tail == 0 || !(A_KC || B_KC)) { return; }
+#pragma unroll
+        for (int round = 0; round < ROUNDS; ++round) {
+          const int piece = wave_u + WAVES * round;
+          if (piece < Config::PIECES_A) {
+            if (A_KC) { HZeroTail(a_ring + buffer * Config::A_ELEMS, piece, lane, k_tail); }
+          } else if (piece < Config::PIECES_A + Config::PIECES_B) {
+            if (B_KC) { HZeroTail(b_ring + buffer * Config::B_ELEMS, piece - Config::PIECES_A, lane, k_tail); }
+          }
+        }
+      };
+
+      // Prologue: slab 0 lands in ring position 0, slab 1 is requested.
+#pragma unroll
+      for (int round = 0; round < ROUNDS; ++round) { request(round, 0, 0); }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (slabs == 1) { zero_tail(0); }
+      if (slabs > 1) {
+#pragma unroll
+        for (int round = 0; round < ROUNDS; ++round) { request(round, 1, 1); }
+      }
+      __syncthreads();
+      half8_t a_frag[2][FM], b_frag[2][FN];
+#pragma unroll
+      for (int q = 0; q < FM; ++q) { a_frag[0][q] = HFragment<TILE_M, A_KC>(a_ring, a_offset[q], 0); }
+#pragma unroll
+      for (int q = 0; q < FN; ++q) { b_frag[0][q] = HFragment<TILE_N, B_KC>(b_ring, b_offset[q], 0); }
+      int cur = 0;  // ring position of the current slab; slab + 1 is in the next one, slab + 2 goes into the one before
+      // One slab. NEXT: slab + 1 exists; LOAD: slab + 2 exists and is requested into the buffer that the barrier of
+      // the previous slab released. Compile-time, so that the steady state has no branches.
+      constexpr int PER_QUARTER = (ROUNDS + FM - 1) / FM;
+      auto slab_body = [&](const int slab, auto next_tag, auto load_tag) {
+        constexpr bool NEXT = decltype(next_tag)::value, LOAD = decltype(load_tag)::value;
+        const int nxt = (cur == STAGES - 1) ? 0 : cur + 1, prv = (cur == 0) ? STAGES - 1 : cur - 1;
+        const T* a_cur = a_ring + cur * Config::A_ELEMS;
+        const T* b_cur = b_ring + cur * Config::B_ELEMS;
+        const T* a_nxt = a_ring + nxt * Config::A_ELEMS;
+        const T* b_nxt = b_ring + nxt * Config::B_ELEMS;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const int set = ks % 2;
+          const T* a_src = (ks + 1 < KSTEPS) ? a_cur : a_nxt;
+          const T* b_src = (ks + 1 < KSTEPS) ? b_cur : b_nxt;
+          const int ks_src = (ks + 1 < KSTEPS) ? ks + 1 : 0;
+#pragma unroll
+          for (int q = 0; q < FM; ++q) {
+            a_frag[set ^ 1][q] = HFragment<TILE_M, A_KC>(a_src, a_offset[q], ks_src);
+            if (q < FN) { b_frag[set ^ 1][q] = HFragment<TILE_N, B_KC>(b_src, b_offset[q], ks_src); }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+              acc[q][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag[set][q], b_frag[set][j], acc[q][j], 0, 0, 0);
+            }
+            // spread over the quarters: a burst of identical requests from all work-groups defeats the L2
+            if (LOAD && ks == 0) {
+#pragma unroll
+              for (int u = 0; u < PER_QUARTER; ++u) {
+                if (q * PER_QUARTER + u < ROUNDS) { request(q * PER_QUARTER + u, slab + 2, prv); }
+              }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          if (ks == KSTEPS - 2) {
+            // slab + 1 must have landed for everybody; this slab's own requests (slab + 2) may stay in flight
+            if (LOAD) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(ROUNDS) : "memory"); }
+            else { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+            if (NEXT && !LOAD) { zero_tail(nxt); }  // slab + 1 is the last one
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+          }
+        }
+        cur = nxt;
+      };
+      int slab = 0;
+      for (; slab + 2 < slabs; ++slab) { slab_body(slab, std::true_type{}, std::true_type{}); }
+      if (slab + 1 < slabs) { slab_body(slab, std::true_type{}, std::false_type{}); ++slab; }
+      slab_body(slab, std::false_type{}, std::false_type{});
+    };
+    if (m0 + TILE_M <= p.m && n0 + TILE_N <= p.n && k_tail == 0) { walk(std::false_type{}); }
+    else { walk(std::true_type{}); }
+
+    // Epilogue, staged through LDS so that global memory sees whole lines. Accumulator elements 4g..4g+3 of a
+    // lane are the rows m = 8g + 4*(lane/32) + 0..3 of column n = lane%32 of the 32 x 32 block. Per block
+    // column j a wavefront owns a [32 n][WAVE_M m] fp16 staging tile of its own: C (when beta != 0) comes in
+    // with 16-byte accesses along m, every lane combines its four consecutive m in fp32 and rounds once, and
+    // the finished rows leave with 16-byte stores. Only wavefront-local ordering is needed (LDS operations of
+    // a wavefront complete in order).
+    {
+      constexpr int WAVE_M = FM * 32, STAGE_PITCH = WAVE_M + 8;
+      constexpr int LANES_PER_ROW = WAVE_M / 8, ROWS_PER_PASS = 64 / LANES_PER_ROW, PASSES = 32 / ROWS_PER_PASS;
+      typedef _Float16 half8u_t __attribute__((ext_vector_type(8), aligned(4)));  // C needs dword alignment only
+      T* stage = lds + wave * (32 * STAGE_PITCH);
+      const int wave_m0 = m0 + wave_m * WAVE_M;
+      const bool vector_rows = (wave_m0 + WAVE_M <= p.m) && (p.c_ld % 2 == 0) && ((reinterpret_cast<unsigned long long>(c) & 3) == 0);
+      auto wave_fence = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      };
+      // moves the staging tile's rows from (LOAD) or to (!LOAD) the block column starting at n_blk
+      auto rows = [&](const int n_blk, auto load_tag) {
+        constexpr bool LOAD = decltype(load_tag)::value;
+        if (vector_rows) {
+#pragma unroll
+          for (int pass = 0; pass < PASSES; ++pass) {
+            const int row = pass * ROWS_PER_PASS + lane / LANES_PER_ROW, col = 8 * (lane % LANES_PER_ROW);
+            if (n_blk + row < p.n) {
+              T* global = c + (n_blk + row) * p.c_ld + wave_m0 + col;
+              half8_t* local = reinterpret_cast<half8_t*>(&stage[row * STAGE_PITCH + col]);
+              if (LOAD) { *local = *reinterpret_cast<const half8u_t*>(global); }
+              else { *reinterpret_cast<half8u_t*>(global) = *local; }
+            }
+          }
+        } else {
+#pragma unroll 1
+          for (int row = 0; row < 32; ++row) {
+            if (n_blk + row >= p.n) { break; }
+#pragma unroll
+            for (int col = lane; col < WAVE_M; col += 64) {
+              if (wave_m0 + col < p.m) {
+                T* global = c + (n_blk + row) * p.c_ld + wave_m0 + col;
+                if (LOAD) { stage[row * STAGE_PITCH + col] = *global; }
+                else { *global = stage[row * STAGE_PITCH + col]; }
+              }
+            }
+          }
+        }
+      };
+      __syncthreads();  // every wavefront is done with the slab buffers
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+        const int n_blk = n0 + (wave_n * FN + j) * 32;
+        if (n_blk < p.n && wave_m0 < p.m) {
+          if (beta != 0.0f) {
+            rows(n_blk, std::true_type{});
+            wave_fence();
+          }
+#pragma unroll
+          for (int i = 0; i < FM; ++i) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              half4_t* cell = reinterpret_cast<half4_t*>(&stage[(lane % 32) * STAGE_PITCH + 32 * i + 8 * g + 4 * (lane / 32)]);
+              half4_t out;
+              if (beta != 0.0f) {
+                const half4_t old = *cell;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { out[e] = static_cast<T>(alpha * acc[i][j][4 * g + e] + beta * static_cast<float>(old[e])); }
+              } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { out[e] = static_cast<T>(alpha * acc[i][j][4 * g + e]); }
+              }
+              *cell = out;
+            }
+          }
+          wave_fence();
+          rows(n_blk, std::false_type{});
+          wave_fence();
+        }
+      }
+      __syncthreads();  // the next batch entry refills the slab buffers
+    }
+  }
+}
+
+}  // namespace clbh
+
+#endif  // CLBLAST_HIP_KERNELS_GEMM_DIRECT_F16_HPP_

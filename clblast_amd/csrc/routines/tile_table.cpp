@@ -98,10 +98,13 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     return KernelChoice{CLBH_KERNEL_MFMA, static_cast<int>(forced) - 1, static_cast<int>(ranges)};
   }
   if (precision == Precision::kHalf) {
-    // 256 x 256 tiles (8 wavefronts, ring of 3 direct-loaded slabs: index 3) once there are at least two per CU,
-    // else 128 x 128
-    const auto big_tiles = CeilDivide(m, 256) * CeilDivide(n, 256);
-    return KernelChoice{CLBH_KERNEL_MFMA, (big_tiles >= 512) ? 3 : 0, 1};
+    // direct-load tiles: 0: 128 x 128, 1: 64 x 64, 2: 256 x 256 (8 wavefronts), 3: 128 x 32, 4: 32 x 128
+    int tile = 1;
+    if (n <= 32 && m >= 256) { tile = 3; }
+    else if (m <= 32 && n >= 256) { tile = 4; }
+    else if (CeilDivide(m, 256) * CeilDivide(n, 256) >= 128 && k >= 512) { tile = 2; }
+    else if (CeilDivide(m, 128) * CeilDivide(n, 128) >= 256) { tile = 0; }
+    return KernelChoice{CLBH_KERNEL_MFMA, tile, 1};
   }
   if (precision == Precision::kSingle) {
     // Measured on the MI355X (tile x split sweep over 18 shapes): 64 x 64 tiles (several work-groups per CU hide
