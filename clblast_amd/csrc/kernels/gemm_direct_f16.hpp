@@ -75,21 +75,27 @@ __device__ __forceinline__ int HRecordsUpTo(const void* from, const void* end) {
   return static_cast<int>(high < 0 ? 0u : (high != 0 ? 0xffffffffu : low));
 }
 
-// Requests piece `piece` (1 KiB) of the slab at `slab` (element (x0, k0), uniform) into `stage`.
-// KC: the piece is x rows 16*piece..+15 of 32 halfs; XC: k rows (512/W)*piece.. of W halfs.
-template <int W, bool KC, bool RANGE, typename Tag>
-__device__ __forceinline__ void HRequestPiece(const _Float16* __restrict__ slab, const _Float16* valid_end, const long long ld,
-                                              _Float16* stage, const int piece, const int lane) {
-  constexpr int ROWS = KC ? 16 : 512 / W, CHUNKS = KC ? 4 : W / 8;  // rows of the piece, 16-byte chunks per row
-  const int row = lane / CHUNKS, position = lane % CHUNKS;
-  const int chunk = KC ? position ^ ((row >> 2) & 3) : position ^ HSwizzle<W>(ROWS * piece + row);
-  const _Float16* source = slab + static_cast<long long>(ROWS * piece) * ld;
-  const int lane_bytes = static_cast<int>((row * ld + 8 * chunk) * 2);
+// Requests one 1 KiB piece: `source` points at its first row (uniform), `lane_bytes` is the lane's byte offset
+// from there (HPieceLaneBytes), `destination` the piece's place in the LDS stage (uniform).
+template <bool RANGE, typename Tag>
+__device__ __forceinline__ void HRequestPiece(const _Float16* __restrict__ source, const _Float16* valid_end,
+                                              _Float16* destination, const int lane_bytes) {
   typedef __attribute__((address_space(3))) void* LdsPtr;
   __builtin_amdgcn_raw_ptr_buffer_load_lds(
       __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(source), 0, RANGE ? HRecordsUpTo(source, valid_end) : -1,
                                         kRawBufferFlags),
-      (LdsPtr)(stage + piece * 512), 16, lane_bytes, 0, 0, 0);
+      (LdsPtr)(destination), 16, lane_bytes, 0, 0, 0);
+}
+
+// Byte offset of a lane's 16 bytes from the first row of piece `piece`. KC: the piece is x rows
+// 16*piece..+15 of 32 halfs; XC: k rows (512/W)*piece.. of W halfs. The lane's LDS position is fixed
+// (16 * lane), the chunk it fetches carries the swizzle.
+template <int W, bool KC>
+__device__ __forceinline__ int HPieceLaneBytes(const long long ld, const int piece, const int lane) {
+  constexpr int ROWS = KC ? 16 : 512 / W, CHUNKS = KC ? 4 : W / 8;  // rows of the piece, 16-byte chunks per row
+  const int row = lane / CHUNKS, position = lane % CHUNKS;
+  const int chunk = KC ? position ^ ((row >> 2) & 3) : position ^ HSwizzle<W>(ROWS * piece + row);
+  return static_cast<int>((row * ld + 8 * chunk) * 2);
 }
 
 // After its own request for a k-contiguous piece has landed, the wavefront zeroes the elements k >= k_valid.
@@ -196,16 +202,42 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
     // tail), and without (saves the scalar arithmetic of one byte count per request).
     auto walk = [&](auto range_tag) {
       constexpr bool RANGE = decltype(range_tag)::value;
-      // request `round` of this wavefront for slab `slab` into ring position `buffer`
-      auto request = [&](const int round, const int slab, const int buffer) {
-        const int k0 = slab * TILE_K;
+      // Request `round` of this wavefront: which piece, where its rows start inside a slab (elements), the
+      // lane's byte offset and the piece's place inside a stage; all constant over the K walk.
+      const T* a_request = a_tile0;  // first row of the slab to be requested next
+      const T* b_request = b_tile0;
+      const long long a_step = A_KC ? static_cast<long long>(TILE_K) : TILE_K * p.a_ld;
+      const long long b_step = B_KC ? static_cast<long long>(TILE_K) : TILE_K * p.b_ld;
+      long long piece_start[ROUNDS];
+      int piece_lane_bytes[ROUNDS], piece_place[ROUNDS];
+#pragma unroll
+      for (int round = 0; round < ROUNDS; ++round) {
         const int piece = wave_u + WAVES * round;
-        if (piece < Config::PIECES_A) {
-          HRequestPiece<TILE_M, A_KC, RANGE, KernelTag>(a_tile0 + (A_KC ? static_cast<long long>(k0) : k0 * p.a_ld), a_end, p.a_ld,
-                                                        a_ring + buffer * Config::A_ELEMS, piece, lane);
+        if ((Config::PIECES_A % WAVES == 0) ? (round < Config::PIECES_A / WAVES) : (piece < Config::PIECES_A)) {
+          piece_start[round] = static_cast<long long>((A_KC ? 16 : 512 / TILE_M) * piece) * p.a_ld;
+          piece_lane_bytes[round] = HPieceLaneBytes<TILE_M, A_KC>(p.a_ld, piece, lane);
+          piece_place[round] = piece * 512;
+        } else {
+          const int b_piece = piece - Config::PIECES_A;
+          piece_start[round] = static_cast<long long>((B_KC ? 16 : 512 / TILE_N) * b_piece) * p.b_ld;
+          piece_lane_bytes[round] = HPieceLaneBytes<TILE_N, B_KC>(p.b_ld, b_piece, lane);
+          piece_place[round] = b_piece * 512;
+        }
+      }
+      // requests piece `round` of the slab at a_request / b_request into ring position `buffer`
+      // (when the pieces of A fill whole rounds, the operand of a round is known at compile time: no branch
+      // stands between the MFMAs)
+      auto is_a = [&](const int round, const int piece) {
+        return (Config::PIECES_A % WAVES == 0) ? (round < Config::PIECES_A / WAVES) : (piece < Config::PIECES_A);
+      };
+      auto request = [&](const int round, const int buffer) {
+        const int piece = wave_u + WAVES * round;
+        if (is_a(round, piece)) {
+          HRequestPiece<RANGE, KernelTag>(a_request + piece_start[round], a_end,
+                                          a_ring + buffer * Config::A_ELEMS + piece_place[round], piece_lane_bytes[round]);
         } else if (!Config::DUMMY || piece < Config::PIECES_A + Config::PIECES_B) {
-          HRequestPiece<TILE_N, B_KC, RANGE, KernelTag>(b_tile0 + (B_KC ? static_cast<long long>(k0) : k0 * p.b_ld), b_end, p.b_ld,
-                                                        b_ring + buffer * Config::B_ELEMS, piece - Config::PIECES_A, lane);
+          HRequestPiece<RANGE, KernelTag>(b_request + piece_start[round], b_end,
+                                          b_ring + buffer * Config::B_ELEMS + piece_place[round], piece_lane_bytes[round]);
         } else {
           // keeps the number of outstanding requests equal in all wavefronts (the waits count them): an
           // empty resource moves nothing but zeros, into a piece nobody reads
@@ -214,6 +246,7 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
                                                    (LdsPtr)(scratch_piece), 16, lane * 16, 0, 0, 0);
         }
       };
+      auto next_request_slab = [&]() { a_request += a_step; b_request += b_step; };
       // zeroes the K tail of the k-contiguous pieces this wavefront requested for the slab in `buffer`
       auto zero_tail = [&](const int buffer) {
         if (!RANGE || k_tail == 0 || !(A_KC || B_KC)) { return; }
@@ -230,12 +263,14 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
 
       // Prologue: slab 0 lands in ring position 0, slab 1 is requested.
 #pragma unroll
-      for (int round = 0; round < ROUNDS; ++round) { request(round, 0, 0); }
+      for (int round = 0; round < ROUNDS; ++round) { request(round, 0); }
+      next_request_slab();
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       if (slabs == 1) { zero_tail(0); }
       if (slabs > 1) {
 #pragma unroll
-        for (int round = 0; round < ROUNDS; ++round) { request(round, 1, 1); }
+        for (int round = 0; round < ROUNDS; ++round) { request(round, 1); }
+        next_request_slab();
       }
       __syncthreads();
       half8_t a_frag[2][FM], b_frag[2][FN];
@@ -273,7 +308,7 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
             if (LOAD && ks == 0) {
 #pragma unroll
               for (int u = 0; u < PER_QUARTER; ++u) {
-                if (q * PER_QUARTER + u < ROUNDS) { request(q * PER_QUARTER + u, slab + 2, prv); }
+                if (q * PER_QUARTER + u < ROUNDS) { request(q * PER_QUARTER + u, prv); }
               }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -287,6 +322,7 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
           }
         }
         cur = nxt;
+        if (LOAD) { next_request_slab(); }
       };
       int slab = 0;
       for (; slab + 2 < slabs; ++slab) { slab_body(slab, std::true_type{}, std::true_type{}); }

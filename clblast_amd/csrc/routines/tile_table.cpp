@@ -98,12 +98,14 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     return KernelChoice{CLBH_KERNEL_MFMA, static_cast<int>(forced) - 1, static_cast<int>(ranges)};
   }
   if (precision == Precision::kHalf) {
-    // direct-load tiles: 0: 128 x 128, 1: 64 x 64, 2: 256 x 256 (8 wavefronts), 3: 128 x 32, 4: 32 x 128
+    // Direct-load tiles, 0: 128 x 128, 1: 64 x 64, 2: 256 x 256 (8 wavefronts), 3: 128 x 32, 4: 32 x 128. Measured
+    // (tile sweep over 15 shapes): 256 x 256 when its tiles fill whole rounds of the 256 CUs, 128 x 128 from 256
+    // tiles on, else 64 x 64 - also for skinny shapes (there is no split-K for fp16, occupancy does the hiding).
+    const auto big = CeilDivide(m, 256) * CeilDivide(n, 256) * batch_count;
+    const auto rounds = CeilDivide(big, 256);
     int tile = 1;
-    if (n <= 32 && m >= 256) { tile = 3; }
-    else if (m <= 32 && n >= 256) { tile = 4; }
-    else if (CeilDivide(m, 256) * CeilDivide(n, 256) >= 128 && k >= 512) { tile = 2; }
-    else if (CeilDivide(m, 128) * CeilDivide(n, 128) >= 256) { tile = 0; }
+    if (5 * big >= 4 * rounds * 256 && k >= 512) { tile = 2; }
+    else if (CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count >= 256) { tile = 0; }
     return KernelChoice{CLBH_KERNEL_MFMA, tile, 1};
   }
   if (precision == Precision::kSingle) {
