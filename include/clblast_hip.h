@@ -147,8 +147,9 @@ StatusCode ClearCache();
 //   "GemmRoutine": {"XGEMM_MIN_INDIRECT_SIZE": s} - problems with m*n*k < s^3 take the general
 //                  (direct) kernel, all others the MFMA-tiled kernels (reference:
 //                  src/routines/level3/xgemm.hpp:63-69, test/routines/level3/xgemm.hpp:62-70).
-//   "Xgemm":       {"TILE_VARIANT": v} - v > 0 forces tile variant v of the MFMA-tiled kernels for
-//                  that precision (for measurements and tests), 0 restores the automatic choice.
+//   "Xgemm":       {"TILE_VARIANT": v, "SPLIT_K": s} - v > 0 forces tile variant v of the MFMA-tiled
+//                  kernels for that precision, walked in s K ranges (optional; fp32/fp64), for
+//                  measurements and tests; 0 restores the automatic choice.
 // Any other kernel name returns kInvalidOverrideKernel, a missing parameter kMissingOverrideParameter.
 StatusCode OverrideParameters(const int device, const std::string& kernel_name, const Precision precision,
                               const std::unordered_map<std::string, size_t>& parameters);
