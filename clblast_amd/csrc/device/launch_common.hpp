@@ -68,8 +68,11 @@ inline bool Aligned16(const clbh_gemm_desc& d) {
   if (address(d.a, d.a_offset) % 16 || address(d.b, d.b_offset) % 16 || address(d.c, d.c_offset) % 16) { return false; }
   if (d.a_ld % VEC || d.b_ld % VEC || d.c_ld % VEC) { return false; }
   if (d.batch_count > 1) {
-    if (d.batch.alphas != nullptr) { return false; }  // per-batch offsets are only known on the device
-    if (d.a_stride % VEC || d.b_stride % VEC || d.c_stride % VEC) { return false; }
+    if (d.batch.alphas != nullptr) {  // per-batch offsets: the host side says what divides them all
+      if (d.batch.offset_multiple < VEC || d.batch.offset_multiple % VEC) { return false; }
+    } else if (d.a_stride % VEC || d.b_stride % VEC || d.c_stride % VEC) {
+      return false;
+    }
   }
   return true;
 }

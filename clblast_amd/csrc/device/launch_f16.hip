@@ -98,8 +98,11 @@ bool DwordAlignedHalf(const clbh_gemm_desc& d) {
   if (address(d.a, d.a_offset) % 4 || address(d.b, d.b_offset) % 4) { return false; }
   if (d.a_ld % 2 || d.b_ld % 2) { return false; }
   if (d.batch_count > 1) {
-    if (d.batch.alphas != nullptr) { return false; }  // per-batch offsets are only known on the device
-    if (d.a_stride % 2 || d.b_stride % 2) { return false; }
+    if (d.batch.alphas != nullptr) {  // per-batch offsets: the host side says what divides them all
+      if (d.batch.offset_multiple < 2 || d.batch.offset_multiple % 2) { return false; }
+    } else if (d.a_stride % 2 || d.b_stride % 2) {
+      return false;
+    }
   }
   return true;
 }

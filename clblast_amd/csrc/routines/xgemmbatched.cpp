@@ -82,6 +82,14 @@ void XgemmBatched<T>::DoGemmBatched(const Layout layout, const Transpose a_trans
                 sizeof(long long));
   }
 
+  // what the launcher may assume about the alignment of the per-batch offsets (elements): the largest power
+  // of two up to 8 that divides all of them
+  auto multiple = size_t{8};
+  for (auto batch = size_t{0}; batch < batch_count; ++batch) {
+    while (multiple > 1 && ((a_offsets[batch] | b_offsets[batch] | c_offsets[batch]) % multiple) != 0) { multiple /= 2; }
+  }
+  desc.batch.offset_multiple = static_cast<int>(multiple);
+
   void* device_block = nullptr;
   if (clbh_alloc_async(&device_block, total_bytes, stream()) != 0) {
     throw RuntimeErrorCode(StatusCode::kTempBufferAllocFailure, "batch metadata");

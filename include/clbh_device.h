@@ -44,6 +44,7 @@ typedef struct clbh_batch_arrays_ {
   const long long* a_offsets;   // element offsets
   const long long* b_offsets;
   const long long* c_offsets;
+  int offset_multiple;          // every entry of the three offset arrays is a multiple of this (0 or 1: unknown)
 } clbh_batch_arrays;
 
 typedef struct clbh_gemm_desc_ {
