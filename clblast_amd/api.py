@@ -17,6 +17,8 @@ from . import _lib
 
 ROW_MAJOR, COL_MAJOR = 101, 102
 TRANS_NO, TRANS_YES, TRANS_CONJ = 111, 112, 113
+TRIANGLE_UPPER, TRIANGLE_LOWER = 121, 122
+SIDE_LEFT, SIDE_RIGHT = 141, 142
 
 STATUS_NAMES = {
     0: "kSuccess", -4: "kTempBufferAllocFailure", -30: "kInvalidValue", -36: "kInvalidCommandQueue",
@@ -72,6 +74,16 @@ def raw_gemm(prefix, layout, a_transpose, b_transpose, m, n, k, alpha, a_ptr, a_
     if temp_ptr is None:
         return getattr(lib, "CLBlast%sgemm" % prefix)(*args)
     return getattr(lib, "CLBlast%sgemmWithTempBuffer" % prefix)(*(args + [temp_ptr]))
+
+
+def raw_symm(prefix, layout, side, triangle, m, n, alpha, a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld, beta, c_ptr,
+             c_offset, c_ld, stream_handle=0, event_handle=None):
+    """CLBlast{S,D,H}symm through the C ABI (reference: include/clblast_c.h:921-945)."""
+    lib = _lib.load()
+    event_ref = None if event_handle is None else ctypes.byref(ctypes.c_void_p(event_handle))
+    return getattr(lib, "CLBlast%ssymm" % prefix)(layout, side, triangle, m, n, _scalar(prefix, alpha), a_ptr, a_offset, a_ld,
+                                                  b_ptr, b_offset, b_ld, _scalar(prefix, beta), c_ptr, c_offset, c_ld,
+                                                  _stream_ref(stream_handle), event_ref)
 
 
 def raw_gemm_batched(prefix, layout, a_transpose, b_transpose, m, n, k, alphas, a_ptr, a_offsets, a_ld, b_ptr,
@@ -151,6 +163,17 @@ def gemm(queue, m, n, k, a, b, c, a_ld, b_ld, c_ld, alpha=1.0, beta=0.0, a_trans
                       c_offset, c_ld, _stream_handle(queue))
     if status != 0:
         raise CLBlastError("CLBlast%sgemm" % prefix, status)
+
+
+def symm(queue, m, n, a, b, c, a_ld, b_ld, c_ld, alpha=1.0, beta=0.0, right_side=False, lower_triangle=False, a_offset=0,
+         b_offset=0, c_offset=0):
+    """xSYMM: Symmetric matrix-matrix multiplication (row-major, like pyclblast.symm; pyclblast.pyx:1939-1974)."""
+    prefix = _tensor_info(a, b, c)
+    status = raw_symm(prefix, ROW_MAJOR, SIDE_RIGHT if right_side else SIDE_LEFT,
+                      TRIANGLE_LOWER if lower_triangle else TRIANGLE_UPPER, m, n, alpha, a.data_ptr(), a_offset, a_ld,
+                      b.data_ptr(), b_offset, b_ld, beta, c.data_ptr(), c_offset, c_ld, _stream_handle(queue))
+    if status != 0:
+        raise CLBlastError("CLBlast%ssymm" % prefix, status)
 
 
 def gemmBatched(queue, m, n, k, a, b, c, alphas, betas, a_ld, b_ld, c_ld, a_offsets, b_offsets, c_offsets,

@@ -10,6 +10,7 @@
 #include "clblast_hip.h"
 #include "routines/xgemm.hpp"
 #include "routines/xgemmbatched.hpp"
+#include "routines/xsymm.hpp"
 
 #define CLBLAST_HIP_PUBLIC __attribute__((visibility("default")))
 
@@ -28,6 +29,21 @@ StatusCode Gemm(const Layout layout, const Transpose a_transpose, const Transpos
     routine.DoGemm(layout, a_transpose, b_transpose, m, n, k, alpha, Buffer<T>(a_buffer), a_offset, a_ld,
                    Buffer<T>(b_buffer), b_offset, b_ld, beta, Buffer<T>(c_buffer), c_offset, c_ld,
                    Buffer<T>(temp_buffer), temp_buffer_provided);
+    return StatusCode::kSuccess;
+  } catch (...) {
+    return DispatchException();
+  }
+}
+
+template <typename T>
+StatusCode Symm(const Layout layout, const Side side, const Triangle triangle, const size_t m, const size_t n,
+                const T alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld, const void* b_buffer,
+                const size_t b_offset, const size_t b_ld, const T beta, void* c_buffer, const size_t c_offset,
+                const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {
+  try {
+    auto routine = Xsymm<T>(queue, event);
+    routine.DoSymm(layout, side, triangle, m, n, alpha, Buffer<T>(a_buffer), a_offset, a_ld, Buffer<T>(b_buffer), b_offset,
+                   b_ld, beta, Buffer<T>(c_buffer), c_offset, c_ld);
     return StatusCode::kSuccess;
   } catch (...) {
     return DispatchException();
@@ -114,7 +130,11 @@ StatusCode GemmTempBufferSize(const Layout layout, const Transpose a_transpose, 
       const T, void*, const size_t, const size_t, const size_t, const size_t, hipStream_t*, hipEvent_t*);           \
   template StatusCode CLBLAST_HIP_PUBLIC GemmTempBufferSize<T>(                                                     \
       const Layout, const Transpose, const Transpose, const size_t, const size_t, const size_t, const size_t,       \
-      const size_t, const size_t, const size_t, const size_t, const size_t, hipStream_t*, size_t&);
+      const size_t, const size_t, const size_t, const size_t, const size_t, hipStream_t*, size_t&);         \
+  template StatusCode CLBLAST_HIP_PUBLIC Symm<T>(const Layout, const Side, const Triangle, const size_t, const size_t,  \
+                                                 const T, const void*, const size_t, const size_t, const void*,     \
+                                                 const size_t, const size_t, const T, void*, const size_t,          \
+                                                 const size_t, hipStream_t*, hipEvent_t*);
 CLBLAST_HIP_INSTANTIATE(half)
 CLBLAST_HIP_INSTANTIATE(float)
 CLBLAST_HIP_INSTANTIATE(double)

@@ -258,4 +258,41 @@ CLBlastStatusCode CLBlastOverrideParameters(const int device, const char* kernel
 cl_half CLBlastFloatToHalf(const float value) { return FloatToHalf(value); }
 float CLBlastHalfToFloat(const cl_half value) { return HalfToFloat(value); }
 
+// ---- SYMM ---------------------------------------------------------------------------------------
+CLBlastStatusCode CLBlastSsymm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,
+                               const size_t m, const size_t n, const float alpha, const void* a_buffer,
+                               const size_t a_offset, const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                               const size_t b_ld, const float beta, void* c_buffer, const size_t c_offset,
+                               const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {
+  return Guarded([&]() {
+    return clblast::Symm<float>(L(layout), static_cast<clblast::Side>(side), static_cast<clblast::Triangle>(triangle), m, n,
+                             alpha, a_buffer, a_offset, a_ld, b_buffer, b_offset, b_ld, beta, c_buffer, c_offset, c_ld,
+                             queue, event);
+  });
+}
+
+CLBlastStatusCode CLBlastDsymm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,
+                               const size_t m, const size_t n, const double alpha, const void* a_buffer,
+                               const size_t a_offset, const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                               const size_t b_ld, const double beta, void* c_buffer, const size_t c_offset,
+                               const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {
+  return Guarded([&]() {
+    return clblast::Symm<double>(L(layout), static_cast<clblast::Side>(side), static_cast<clblast::Triangle>(triangle), m, n,
+                             alpha, a_buffer, a_offset, a_ld, b_buffer, b_offset, b_ld, beta, c_buffer, c_offset, c_ld,
+                             queue, event);
+  });
+}
+
+CLBlastStatusCode CLBlastHsymm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,
+                               const size_t m, const size_t n, const unsigned short alpha, const void* a_buffer,
+                               const size_t a_offset, const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                               const size_t b_ld, const unsigned short beta, void* c_buffer, const size_t c_offset,
+                               const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {
+  return Guarded([&]() {
+    return clblast::Symm<clblast::half>(L(layout), static_cast<clblast::Side>(side), static_cast<clblast::Triangle>(triangle), m, n,
+                             alpha, a_buffer, a_offset, a_ld, b_buffer, b_offset, b_ld, beta, c_buffer, c_offset, c_ld,
+                             queue, event);
+  });
+}
+
 }  // extern "C"

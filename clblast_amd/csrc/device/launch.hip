@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "device/launch_common.hpp"
+#include "kernels/symmetric_to_square.hpp"
 
 namespace clbh {
 namespace {
@@ -100,6 +101,29 @@ size_t clbh_gemm_workspace_bytes(const clbh_gemm_desc* desc) {
   const auto plan = clbh::PlanSplit(*desc);
   if (plan.splits <= 1) { return 0; }
   return static_cast<size_t>(desc->precision / 8) * plan.splits * plan.ld * static_cast<size_t>(desc->n);
+}
+
+int clbh_symmetric_to_square(int precision, int upper, int k, const void* src, long long src_offset, long long src_ld,
+                             void* dst, hipStream_t stream) {
+  if (k <= 0 || src == nullptr || dst == nullptr || src_ld < k || src_offset < 0) { return hipErrorInvalidValue; }
+  const unsigned tiles = static_cast<unsigned>((k + clbh::kSymmetricTile - 1) / clbh::kSymmetricTile);
+  const dim3 grid(tiles, tiles);
+  switch (precision) {
+    case 16:
+      clbh::SymmetricToSquareKernel<_Float16><<<grid, dim3(256), 0, stream>>>(
+          k, upper != 0, static_cast<const _Float16*>(src) + src_offset, src_ld, static_cast<_Float16*>(dst), k);
+      break;
+    case 32:
+      clbh::SymmetricToSquareKernel<float><<<grid, dim3(256), 0, stream>>>(
+          k, upper != 0, static_cast<const float*>(src) + src_offset, src_ld, static_cast<float*>(dst), k);
+      break;
+    case 64:
+      clbh::SymmetricToSquareKernel<double><<<grid, dim3(256), 0, stream>>>(
+          k, upper != 0, static_cast<const double*>(src) + src_offset, src_ld, static_cast<double*>(dst), k);
+      break;
+    default: return hipErrorInvalidValue;
+  }
+  return static_cast<int>(hipGetLastError());
 }
 
 int clbh_buffer_extent(const void* ptr, size_t* bytes_available) {

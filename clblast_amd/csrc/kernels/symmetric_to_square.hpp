@@ -1,0 +1,52 @@
+// =================================================================================================
+// Expands a symmetric matrix of which one triangle is stored into a dense square matrix, the first step
+// of SYMM (reference: kernels SymmLowerToSquared / SymmUpperToSquared,
+// src/kernels/level3/convert_symmetric.opencl:24-92). Both matrices are addressed as
+// buffer[two * ld + one]; "upper" means the stored elements are those with one <= two.
+//
+// One work-group moves a 64 x 64 tile of the result. Whatever the triangle, it reads source tiles along
+// their contiguous index only: the tile itself when it lies in the stored triangle, its mirror image
+// otherwise (transposed through LDS), and for the tiles on the diagonal one tile serves both halves.
+// HBM bound: k*k elements written, as many read.
+// =================================================================================================
+#ifndef CLBLAST_HIP_KERNELS_SYMMETRIC_TO_SQUARE_HPP_
+#define CLBLAST_HIP_KERNELS_SYMMETRIC_TO_SQUARE_HPP_
+
+#include <hip/hip_runtime.h>
+
+namespace clbh {
+
+constexpr int kSymmetricTile = 64;
+
+template <typename T>
+__global__ __launch_bounds__(256) void SymmetricToSquareKernel(const int k, const bool upper, const T* __restrict__ src,
+                                                               const long long src_ld, T* __restrict__ dst,
+                                                               const long long dst_ld) {
+  __shared__ T tile[kSymmetricTile][kSymmetricTile + 1];
+  const int one0 = blockIdx.x * kSymmetricTile, two0 = blockIdx.y * kSymmetricTile;  // tile of the result
+  // the stored tile that holds this tile's data: itself when stored, else its mirror image
+  const bool stored = upper ? (one0 <= two0) : (two0 <= one0);
+  const int s_one0 = stored ? one0 : two0, s_two0 = stored ? two0 : one0;
+  const int lane_one = threadIdx.x % kSymmetricTile, first_two = threadIdx.x / kSymmetricTile;
+  // source tile -> LDS as [two][one], reading along `one`
+  for (int two = first_two; two < kSymmetricTile; two += 256 / kSymmetricTile) {
+    const int g_one = s_one0 + lane_one, g_two = s_two0 + two;
+    T value = T(0);
+    if (g_one < k && g_two < k) { value = src[g_two * src_ld + g_one]; }
+    tile[two][lane_one] = value;
+  }
+  __syncthreads();
+  const bool diagonal = (one0 == two0);
+  for (int two = first_two; two < kSymmetricTile; two += 256 / kSymmetricTile) {
+    const int g_one = one0 + lane_one, g_two = two0 + two;
+    if (g_one < k && g_two < k) {
+      // element (one, two) of the result: taken as stored, or from the mirrored position
+      const bool as_stored = diagonal ? (upper ? (lane_one <= two) : (two <= lane_one)) : stored;
+      dst[g_two * dst_ld + g_one] = as_stored ? tile[two][lane_one] : tile[lane_one][two];
+    }
+  }
+}
+
+}  // namespace clbh
+
+#endif  // CLBLAST_HIP_KERNELS_SYMMETRIC_TO_SQUARE_HPP_

@@ -49,6 +49,7 @@ StatusCode DispatchExceptionForC() {
 
 template <typename T>
 size_t Buffer<T>::GetSize() const {
+  if (size_known_) { return known_bytes_; }
   auto bytes = size_t{0};
   if (pointer_ == nullptr || clbh_buffer_extent(pointer_, &bytes) != 0) {
     throw std::runtime_error("not a device allocation");

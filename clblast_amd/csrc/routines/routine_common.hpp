@@ -30,11 +30,13 @@ class BLASError : public std::invalid_argument {
   explicit BLASError(const StatusCode status, const std::string& detail = std::string{})
       : std::invalid_argument("BLAS error: " + std::to_string(static_cast<int>(status)) +
                               (detail.empty() ? "" : " (" + detail + ")")),
-        status_(status) {}
+        status_(status), details_(detail) {}
   StatusCode status() const { return status_; }
+  const std::string& details() const { return details_; }
 
  private:
   StatusCode status_;
+  std::string details_;
 };
 
 // Failures that are not the caller's fault: reported on stderr as "CLBlast: ..." and mapped to their
@@ -109,7 +111,9 @@ constexpr size_t ElementBytes() { return sizeof(T); }
 template <typename T>
 class Buffer {
  public:
-  explicit Buffer(const void* pointer) : pointer_(pointer) {}
+  explicit Buffer(const void* pointer) : pointer_(pointer), known_bytes_(0), size_known_(false) {}
+  // for memory the library allocated itself (the driver is not asked about it)
+  Buffer(const void* pointer, const size_t bytes) : pointer_(pointer), known_bytes_(bytes), size_known_(true) {}
   const void* operator()() const { return pointer_; }
   // Bytes addressable from the pointer to the end of its allocation. Throws std::runtime_error if
   // the pointer is not device memory, which the matrix tests turn into kInvalidMatrix{A,B,C}.
@@ -117,6 +121,8 @@ class Buffer {
 
  private:
   const void* pointer_;
+  size_t known_bytes_;
+  bool size_known_;
 };
 
 // Argument-validation contract; check order: leading dimension first, then the buffer size.

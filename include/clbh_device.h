@@ -75,6 +75,12 @@ CLBH_API int clbh_gemm_launch(const clbh_gemm_desc* desc, hipStream_t stream);
 // Bytes of device scratch the given descriptor needs in `workspace` (0 for most launches).
 CLBH_API size_t clbh_gemm_workspace_bytes(const clbh_gemm_desc* desc);
 
+// Expands the symmetric k x k matrix at src + src_offset (elements; one triangle stored, addressed as
+// [two * src_ld + one], `upper`: the stored elements have one <= two) into the dense k x k matrix `dst`
+// (leading dimension k). precision: 16, 32 or 64.
+CLBH_API int clbh_symmetric_to_square(int precision, int upper, int k, const void* src, long long src_offset,
+                                      long long src_ld, void* dst, hipStream_t stream);
+
 // Number of bytes addressable from `ptr` to the end of the device allocation that contains it.
 // Returns 0 on success, non-zero if `ptr` is not inside a device allocation.
 CLBH_API int clbh_buffer_extent(const void* ptr, size_t* bytes_available);

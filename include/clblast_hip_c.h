@@ -64,6 +64,8 @@ typedef enum CLBlastTranspose_ {
   CLBlastTransposeYes = 112,
   CLBlastTransposeConjugate = 113
 } CLBlastTranspose;
+typedef enum CLBlastTriangle_ { CLBlastTriangleUpper = 121, CLBlastTriangleLower = 122 } CLBlastTriangle;
+typedef enum CLBlastSide_ { CLBlastSideLeft = 141, CLBlastSideRight = 142 } CLBlastSide;
 typedef enum CLBlastPrecision_ {
   CLBlastPrecisionHalf = 16,
   CLBlastPrecisionSingle = 32,
@@ -95,6 +97,31 @@ CLBlastStatusCode CLBLAST_HIP_API CLBlastHgemm(const CLBlastLayout layout, const
                                                const size_t b_offset, const size_t b_ld, const cl_half beta,
                                                void* c_buffer, const size_t c_offset, const size_t c_ld,
                                                hipStream_t* queue, hipEvent_t* event);
+
+// =================================================================================================
+// Symmetric matrix-matrix multiplication C = alpha*A*B + beta*C (side left) or alpha*B*A + beta*C (side right)
+// replaces CLBlastSsymm/CLBlastDsymm/CLBlastHsymm (reference: include/clblast_c.h:921-945, src/clblast_c.cpp:1876-1960)
+CLBlastStatusCode CLBLAST_HIP_API CLBlastSsymm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const size_t m, const size_t n,
+                                               const float alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, const float beta, void* c_buffer,
+                                               const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                                               hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastDsymm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const size_t m, const size_t n,
+                                               const double alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, const double beta, void* c_buffer,
+                                               const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                                               hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastHsymm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const size_t m, const size_t n,
+                                               const unsigned short alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, const unsigned short beta, void* c_buffer,
+                                               const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                                               hipEvent_t* event);
 
 // =================================================================================================
 // Batched GEMM with per-batch alpha, beta and element offsets (host arrays of length batch_count)

@@ -49,6 +49,10 @@ def lib():
         sz, vp, dbl, ci = ctypes.c_size_t, ctypes.c_void_p, ctypes.c_double, ctypes.c_int
         handle.oracle_gemm.argtypes = [ci, ci, ci, ci, sz, sz, sz, dbl, vp, sz, sz, vp, sz, sz, dbl, vp, sz, sz, vp]
         handle.oracle_gemm.restype = ci
+        handle.oracle_symm.argtypes = [ci, ci, ci, ci, sz, sz, dbl, vp, sz, sz, vp, sz, sz, dbl, vp, sz, sz, vp]
+        handle.oracle_symm.restype = ci
+        handle.oracle_symm_status.argtypes = [ci, ci, ci] + [sz] * 11
+        handle.oracle_symm_status.restype = ci
         handle.oracle_process_arguments.argtypes = [ci, ci, ci, sz, sz, sz, ctypes.POINTER(Shape)]
         handle.oracle_process_arguments.restype = ci
         handle.oracle_gemm_status.argtypes = [ci, ci, ci, ci] + [sz] * 12
@@ -122,6 +126,44 @@ def gemm(layout, a_transpose, b_transpose, m, n, k, alpha, a, a_offset, a_ld, b,
     if status != 0:
         raise ValueError("oracle_gemm status %d" % status)
     return result
+
+
+LEFT, RIGHT, UPPER, LOWER = 141, 142, 121, 122
+
+
+def symm(layout, side, triangle, m, n, alpha, a, a_offset, a_ld, b, b_offset, b_ld, beta, c, c_offset, c_ld):
+    """New logical C (m x n, float64, unrounded) of SYMM computed by the C oracle from flat numpy buffers."""
+    bits = _bits(a)
+    assert _bits(b) == bits and _bits(c) == bits
+    a, b, c = np.ascontiguousarray(a), np.ascontiguousarray(b), np.ascontiguousarray(c)
+    result = np.empty((m, n), dtype=np.float64)
+    status = lib().oracle_symm(bits, layout, side, triangle, m, n, float(alpha), a.ctypes.data, a_offset, a_ld,
+                               b.ctypes.data, b_offset, b_ld, float(beta), c.ctypes.data, c_offset, c_ld, result.ctypes.data)
+    if status != 0:
+        raise ValueError("oracle_symm status %d" % status)
+    return result
+
+
+def symm_status(bits, layout, side, m, n, a_offset, a_ld, a_bytes, b_offset, b_ld, b_bytes, c_offset, c_ld, c_bytes):
+    return lib().oracle_symm_status(bits, layout, side, m, n, a_offset, a_ld, a_bytes, b_offset, b_ld, b_bytes, c_offset,
+                                    c_ld, c_bytes)
+
+
+def symm_numpy(layout, side, triangle, m, n, alpha, a, a_offset, a_ld, b, b_offset, b_ld, beta, c, c_offset, c_ld):
+    """Independent float64 statement of SYMM: symmetrise the named triangle with numpy, then matmul."""
+    k = m if side == LEFT else n
+    col_major = (layout == COL_MAJOR)
+    i = np.arange(k, dtype=np.int64)[:, None]
+    j = np.arange(k, dtype=np.int64)[None, :]
+    stored = a[a_offset + (j * a_ld + i if col_major else i * a_ld + j)].astype(np.float64)  # [i, j] = A(i, j) as laid out
+    half_matrix = np.triu(stored) if triangle == UPPER else np.tril(stored)
+    full = half_matrix + half_matrix.T - np.diag(np.diag(stored))
+    r = np.arange(m, dtype=np.int64)[:, None]
+    q = np.arange(n, dtype=np.int64)[None, :]
+    b_full = b[b_offset + (q * b_ld + r if col_major else r * b_ld + q)].astype(np.float64)
+    c_full = c[c_offset + (q * c_ld + r if col_major else r * c_ld + q)].astype(np.float64)
+    product = full @ b_full if side == LEFT else b_full @ full
+    return alpha * product + (beta * c_full if beta != 0 else 0.0)
 
 
 def operand_indices(layout, transpose, rows, cols, offset, ld, is_c=False):

@@ -334,6 +334,73 @@ EXPORT int oracle_gemm(int precision_bits, int layout, int a_transpose, int b_tr
   return kSuccess;
 }
 
+/* ---- SYMM ---------------------------------------------------------------------------------------
+ * BLAS definition restated (reference: src/routines/level3/xsymm.cpp:33-114, which expands the stored
+ * triangle with SymmUpperToSquared / SymmLowerToSquared, src/kernels/level3/convert_symmetric.opencl:24-92,
+ * and calls DoGemm): A is k x k symmetric (k = m for side left, n for side right); element A(i, j) of the
+ * named triangle (upper: i <= j) lives at layout index (col-major: j*ld + i, row-major: i*ld + j), the other
+ * triangle is never read. result (m x n, row i contiguous) = alpha * A * B + beta * C or alpha * B * A + beta * C. */
+enum { kSideLeft = 141, kSideRight = 142, kTriangleUpper = 121, kTriangleLower = 122 };
+
+static double symmetric_element(const void* a, int bits, int layout, int triangle, size_t a_offset, size_t a_ld, size_t i,
+                                size_t j) {
+  const int in_triangle = (triangle == kTriangleUpper) ? (i <= j) : (i >= j);
+  const size_t r = in_triangle ? i : j, q = in_triangle ? j : i; /* the stored twin */
+  const size_t index = (layout == kColMajor) ? (a_offset + q * a_ld + r) : (a_offset + r * a_ld + q);
+  return load_as_double(a, bits, index);
+}
+
+EXPORT int oracle_symm(int precision_bits, int layout, int side, int triangle, size_t m, size_t n, double alpha,
+                       const void* a, size_t a_offset, size_t a_ld, const void* b, size_t b_offset, size_t b_ld,
+                       double beta, const void* c, size_t c_offset, size_t c_ld, double* result) {
+  if (m == 0 || n == 0) return kInvalidDimension;
+  const int col_major = (layout == kColMajor);
+#pragma omp parallel for schedule(static)
+  for (long long ii = 0; ii < (long long)m; ++ii) {
+    const size_t i = (size_t)ii;
+    for (size_t j = 0; j < n; ++j) {
+      long double sum = 0.0L;
+      if (side == kSideLeft) { /* sum_p A(i, p) B(p, j) */
+        for (size_t p = 0; p < m; ++p) {
+          const size_t b_index = col_major ? (b_offset + j * b_ld + p) : (b_offset + p * b_ld + j);
+          sum += (long double)symmetric_element(a, precision_bits, layout, triangle, a_offset, a_ld, i, p) *
+                 (long double)load_as_double(b, precision_bits, b_index);
+        }
+      } else { /* sum_p B(i, p) A(p, j) */
+        for (size_t p = 0; p < n; ++p) {
+          const size_t b_index = col_major ? (b_offset + p * b_ld + i) : (b_offset + i * b_ld + p);
+          sum += (long double)load_as_double(b, precision_bits, b_index) *
+                 (long double)symmetric_element(a, precision_bits, layout, triangle, a_offset, a_ld, p, j);
+        }
+      }
+      double value = alpha * (double)sum;
+      if (beta != 0.0) {
+        const size_t index = col_major ? (c_offset + j * c_ld + i) : (c_offset + i * c_ld + j);
+        value += beta * load_as_double(c, precision_bits, index);
+      }
+      result[i * n + j] = value;
+    }
+  }
+  return kSuccess;
+}
+
+/* Status of Symm<T> (xsymm.cpp:39-49 and the DoGemm it ends in; for side right the GEMM's A is the caller's B
+ * and the codes are swapped back, xsymm.cpp:88-109). All handles valid. */
+EXPORT int oracle_symm_status(int precision_bits, int layout, int side, size_t m, size_t n, size_t a_offset, size_t a_ld,
+                              size_t a_bytes, size_t b_offset, size_t b_ld, size_t b_bytes, size_t c_offset, size_t c_ld,
+                              size_t c_bytes) {
+  if (m == 0 || n == 0) return kInvalidDimension;
+  const size_t eb = (size_t)precision_bits / 8;
+  const size_t k = (side == kSideLeft) ? m : n;
+  int status = test_matrix(k, k, a_bytes, a_offset, a_ld, eb, 1, kInvalidLeadDimA, kInsufficientMemoryA);
+  if (status != kSuccess) return status;
+  /* B and C are m x n in the given layout */
+  const size_t one = (layout == kColMajor) ? m : n, two = (layout == kColMajor) ? n : m;
+  status = test_matrix(one, two, b_bytes, b_offset, b_ld, eb, 1, kInvalidLeadDimB, kInsufficientMemoryB);
+  if (status != kSuccess) return status;
+  return test_matrix(one, two, c_bytes, c_offset, c_ld, eb, 1, kInvalidLeadDimC, kInsufficientMemoryC);
+}
+
 /* ---- the reference's indirect path restated on the CPU (the "port" baseline) -------------------- */
 
 #define DEFINE_XGEMM_PORT(NAME, REAL)                                                                              \

@@ -3,14 +3,14 @@
 oracle/_ref/libclblast_ref.so is CLBlast itself (OpenCL flavour), compiled by oracle/Makefile (`make -C oracle
 ref-full`) from the reference tree where it lies. Where the OpenCL runtime exposes a device (the ROCm OpenCL
 runtime of the GPU box exposes the MI355X), this module calls the reference's own `CLBlast{S,D,H}gemm`,
-`...gemmStridedBatched` (reference: include/clblast_c.h:885-919, 1341-1370) on seeded inputs and returns the
+`...gemmStridedBatched`, `...symm` (reference: include/clblast_c.h:885-945, 1341-1370) on seeded inputs and returns the
 result and the time, so that tests can compare the HIP library with the reference on identical inputs and
 bench.py can quote the reference's speed on the same GPU. It must run in a process that has not initialised
 HIP (both runtimes in one process were seen to lose the device), hence the command-line interface:
 
     python -m oracle.reference_opencl --spec spec.json --out result.npz
 
-spec.json: {"routine": "gemm"|"strided", "bits": 16|32|64, "layout", "ta", "tb", "m", "n", "k", "alpha", "beta",
+spec.json: {"routine": "gemm"|"strided"|"symm" (then "side", "triangle" instead of "ta", "tb", "k"), "bits": 16|32|64, "layout", "ta", "tb", "m", "n", "k", "alpha", "beta",
 "a_ld", "b_ld", "c_ld", "offsets": [a, b, c], "seed": s, "low"/"high", "ab_low"/"ab_high", "batch", "strides",
 "runs": r, "sizes": [a, b, c] element counts}. Inputs are oracle.uniform(seed*3 + {0,1,2}, ...), exactly what
 tests/harness.py and the callers generate. The OpenCL host code here is a minimal ctypes binding of the
@@ -122,11 +122,17 @@ def run(spec):
     queue = vp(opencl.queue.value)
     alpha, beta = scalar_argument(bits, spec["alpha"], reference), scalar_argument(bits, spec["beta"], reference)
     offsets = spec.get("offsets", [0, 0, 0])
-    m, n, k = sz(spec["m"]), sz(spec["n"]), sz(spec["k"])
+    m, n, k = sz(spec["m"]), sz(spec["n"]), sz(spec.get("k", 0))
 
     def call():
         event = vp(None)
-        if spec["routine"] == "gemm":
+        if spec["routine"] == "symm":
+            function = getattr(reference, "CLBlast%ssymm" % PREFIX[bits])
+            status = function(ctypes.c_int(spec["layout"]), ctypes.c_int(spec["side"]), ctypes.c_int(spec["triangle"]), m,
+                              n, alpha, a_buffer, sz(offsets[0]), sz(spec["a_ld"]), b_buffer, sz(offsets[1]),
+                              sz(spec["b_ld"]), beta, c_buffer, sz(offsets[2]), sz(spec["c_ld"]), ctypes.byref(queue),
+                              ctypes.byref(event))
+        elif spec["routine"] == "gemm":
             function = getattr(reference, "CLBlast%sgemm" % PREFIX[bits])
             status = function(ctypes.c_int(spec["layout"]), ctypes.c_int(spec["ta"]), ctypes.c_int(spec["tb"]), m, n, k,
                               alpha, a_buffer, sz(offsets[0]), sz(spec["a_ld"]), b_buffer, sz(offsets[1]),
@@ -184,10 +190,17 @@ def status_sweep(spec):
     alpha, beta = scalar_argument(bits, 1.0, reference), scalar_argument(bits, 0.0, reference)
     statuses = []
     for case in spec["cases"]:
-        layout, ta, tb, m, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes = case[:12]
+        if spec.get("symm"):  # [layout, side, triangle, m, n, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes]
+            layout, side, triangle, m, n, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes = case
+        else:
+            layout, ta, tb, m, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes = case[:12]
         a, b, c = buffer_of(a_bytes, 0), buffer_of(b_bytes, 1), buffer_of(c_bytes, 2)
         event = vp(None)
-        if spec.get("batched"):
+        if spec.get("symm"):
+            function = getattr(reference, "CLBlast%ssymm" % PREFIX[bits])
+            status = function(ctypes.c_int(layout), ctypes.c_int(side), ctypes.c_int(triangle), sz(m), sz(n), alpha, a, sz(0),
+                              sz(a_ld), b, sz(0), sz(b_ld), beta, c, sz(0), sz(c_ld), ctypes.byref(queue), ctypes.byref(event))
+        elif spec.get("batched"):
             offsets = case[12:15]  # three lists of element offsets, one entry per batch
             count = len(offsets[0])
             scalars = (SCALAR[bits] * max(count, 1))(*([alpha.value] * count))
