@@ -32,7 +32,7 @@ DTYPE_NAME = {"S": "f32", "D": "f64", "H": "f16"}
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
 # the readings of a plain 1 GiB copy (profiles/<workload>.md holds the commands and the raw readings). A bench run
 # cannot collect counters itself, so these are the figures of the committed profiles.
-MEASURED_TRAFFIC_BYTES = {"cfg2s": 4.870e9, "cfg2d": 9.157e9, "cfg3": 1.888e9, "cfg4": 1.007e8, "cfg5d": 5.927e8}
+MEASURED_TRAFFIC_BYTES = {"cfg2s": 4.815e9, "cfg2d": 9.140e9, "cfg3": 1.883e9, "cfg4": 1.007e8, "cfg5d": 6.319e8}
 
 
 def parse_args():
@@ -140,6 +140,32 @@ class Workload:
         return float(((c @ x) - expected).norm() / expected.norm())
 
 
+class SymmWorkload(Workload):
+    """SYMM, C := alpha A B + beta C with A symmetric m x m on the left and only one triangle of it valid (the
+    other one holds NaN): a symmetric-to-square pass over A followed by the GEMM of the same shape."""
+
+    def __init__(self, name, prefix, layout, upper, m, n, alpha, beta):
+        import torch
+        super().__init__(name, prefix, layout, NO, NO, m, n, m, alpha, beta)
+        self.triangle = 121 if upper else 122
+        square = self.a.view(m, m)  # memory position [r, q]: A(r, q) in row-major, A(q, r) in column-major
+        memory_upper = upper == (layout == ROW)
+        valid = torch.triu(square) if memory_upper else torch.tril(square)
+        self.full = (valid + valid.T - torch.diag(torch.diag(square))).contiguous()
+        mask = torch.ones(m, m, device="cuda", dtype=torch.bool)
+        square[torch.tril(mask, -1) if memory_upper else torch.triu(mask, 1)] = float("nan")
+
+    def call(self, stream_handle):
+        from clblast_amd.api import raw_symm
+        status = raw_symm(self.prefix, self.layout, 141, self.triangle, self.m, self.n, self.alpha, self.a.data_ptr(), 0,
+                          self.lda, self.b.data_ptr(), 0, self.ldb, self.beta, self.c.data_ptr(), 0, self.ldc, stream_handle)
+        if status != 0:
+            raise RuntimeError("%s: status %d" % (self.name, status))
+
+    def logical(self, which):
+        return self.full.view(self.m, self.m) if which == "a" else super().logical(which)
+
+
 def time_workload(workload, steps, warmup):
     """Returns (wall seconds for `steps` calls, average device milliseconds per call from stream events)."""
     import torch
@@ -233,7 +259,10 @@ def reference_on_this_gpu(runs=3):
              "sgemm_strided_batched_8192x32": dict(routine="strided", bits=32, layout=COL, ta=NO, tb=NO, m=32, n=32, k=32,
                                                    alpha=1.0, beta=0.0, a_ld=32, b_ld=32, c_ld=32, offsets=[0, 0, 0],
                                                    strides=[1024] * 3, batch=8192, seed=9, runs=10,
-                                                   sizes=[1024 * 8192] * 3)}
+                                                   sizes=[1024 * 8192] * 3),
+             "ssymm_4096_colLeftUpper": dict(routine="symm", bits=32, layout=COL, side=141, triangle=121, m=4096, n=4096,
+                                             k=4096, alpha=1.0, beta=0.0, a_ld=4096, b_ld=4096, c_ld=4096,
+                                             offsets=[0, 0, 0], seed=10, runs=5, sizes=[4096 * 4096] * 3)}
     flops = {name: 2.0 * spec["m"] * spec["n"] * spec["k"] * spec.get("batch", 1) for name, spec in specs.items()}
     root = os.path.dirname(os.path.abspath(__file__))
     with tempfile.TemporaryDirectory() as folder:
@@ -270,6 +299,8 @@ EXTRA_WORKLOADS = {
                                                        24, (11, 13, 19)),
     "cfg5_sgemm_8191x8191x127_colNN": lambda: Workload("cfg5d", "S", COL, NO, NO, 8191, 8191, 127, -0.75, 2.0, 8194,
                                                         132, 8198, (11, 13, 19)),
+    "next_ssymm_4096_colLeftUpper": lambda: SymmWorkload("symm_s", "S", COL, True, 4096, 4096, 1.0, 0.0),
+    "next_hsymm_4096_rowLeftLower": lambda: SymmWorkload("symm_h", "H", ROW, False, 4096, 4096, 1.0, 0.0),
 }
 
 

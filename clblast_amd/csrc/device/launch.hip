@@ -89,6 +89,25 @@ int StagedUpload(void* dst_device, const void* src_host, size_t bytes, hipStream
 }  // namespace
 }  // namespace clbh
 
+namespace {
+template <typename T>
+int LaunchSymmetricToSquare(const int upper, const int k, const void* src, const long long src_offset,
+                            const long long src_ld, void* dst, hipStream_t stream) {
+  const unsigned tiles = static_cast<unsigned>((k + clbh::kSymmetricTile - 1) / clbh::kSymmetricTile);
+  const dim3 grid(tiles, tiles);
+  const T* source = static_cast<const T*>(src) + src_offset;
+  constexpr int VEC = 8 / sizeof(T);  // 8 bytes per lane and access when everything is a multiple of that
+  const bool vector = VEC > 1 && k % VEC == 0 && src_ld % VEC == 0 && reinterpret_cast<unsigned long long>(source) % 8 == 0 &&
+                      reinterpret_cast<unsigned long long>(dst) % 8 == 0;
+  if (vector) {
+    clbh::SymmetricToSquareKernel<T, VEC><<<grid, dim3(256), 0, stream>>>(k, upper != 0, source, src_ld, static_cast<T*>(dst), k);
+  } else {
+    clbh::SymmetricToSquareKernel<T, 1><<<grid, dim3(256), 0, stream>>>(k, upper != 0, source, src_ld, static_cast<T*>(dst), k);
+  }
+  return static_cast<int>(hipGetLastError());
+}
+}  // namespace
+
 extern "C" {
 
 int clbh_gemm_launch(const clbh_gemm_desc* desc, hipStream_t stream) {
@@ -106,24 +125,12 @@ size_t clbh_gemm_workspace_bytes(const clbh_gemm_desc* desc) {
 int clbh_symmetric_to_square(int precision, int upper, int k, const void* src, long long src_offset, long long src_ld,
                              void* dst, hipStream_t stream) {
   if (k <= 0 || src == nullptr || dst == nullptr || src_ld < k || src_offset < 0) { return hipErrorInvalidValue; }
-  const unsigned tiles = static_cast<unsigned>((k + clbh::kSymmetricTile - 1) / clbh::kSymmetricTile);
-  const dim3 grid(tiles, tiles);
   switch (precision) {
-    case 16:
-      clbh::SymmetricToSquareKernel<_Float16><<<grid, dim3(256), 0, stream>>>(
-          k, upper != 0, static_cast<const _Float16*>(src) + src_offset, src_ld, static_cast<_Float16*>(dst), k);
-      break;
-    case 32:
-      clbh::SymmetricToSquareKernel<float><<<grid, dim3(256), 0, stream>>>(
-          k, upper != 0, static_cast<const float*>(src) + src_offset, src_ld, static_cast<float*>(dst), k);
-      break;
-    case 64:
-      clbh::SymmetricToSquareKernel<double><<<grid, dim3(256), 0, stream>>>(
-          k, upper != 0, static_cast<const double*>(src) + src_offset, src_ld, static_cast<double*>(dst), k);
-      break;
+    case 16: return LaunchSymmetricToSquare<_Float16>(upper, k, src, src_offset, src_ld, dst, stream);
+    case 32: return LaunchSymmetricToSquare<float>(upper, k, src, src_offset, src_ld, dst, stream);
+    case 64: return LaunchSymmetricToSquare<double>(upper, k, src, src_offset, src_ld, dst, stream);
     default: return hipErrorInvalidValue;
   }
-  return static_cast<int>(hipGetLastError());
 }
 
 int clbh_buffer_extent(const void* ptr, size_t* bytes_available) {
