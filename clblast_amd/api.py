@@ -19,6 +19,7 @@ ROW_MAJOR, COL_MAJOR = 101, 102
 TRANS_NO, TRANS_YES, TRANS_CONJ = 111, 112, 113
 TRIANGLE_UPPER, TRIANGLE_LOWER = 121, 122
 SIDE_LEFT, SIDE_RIGHT = 141, 142
+DIAGONAL_NON_UNIT, DIAGONAL_UNIT = 131, 132
 
 STATUS_NAMES = {
     0: "kSuccess", -4: "kTempBufferAllocFailure", -30: "kInvalidValue", -36: "kInvalidCommandQueue",
@@ -84,6 +85,16 @@ def raw_symm(prefix, layout, side, triangle, m, n, alpha, a_ptr, a_offset, a_ld,
     return getattr(lib, "CLBlast%ssymm" % prefix)(layout, side, triangle, m, n, _scalar(prefix, alpha), a_ptr, a_offset, a_ld,
                                                   b_ptr, b_offset, b_ld, _scalar(prefix, beta), c_ptr, c_offset, c_ld,
                                                   _stream_ref(stream_handle), event_ref)
+
+
+def raw_trmm(prefix, layout, side, triangle, a_transpose, diagonal, m, n, alpha, a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld,
+             stream_handle=0, event_handle=None):
+    """CLBlast{S,D,H}trmm through the C ABI (reference: include/clblast_c.h:1062-1092)."""
+    lib = _lib.load()
+    event_ref = None if event_handle is None else ctypes.byref(ctypes.c_void_p(event_handle))
+    return getattr(lib, "CLBlast%strmm" % prefix)(layout, side, triangle, a_transpose, diagonal, m, n, _scalar(prefix, alpha),
+                                                  a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld, _stream_ref(stream_handle),
+                                                  event_ref)
 
 
 def raw_gemm_batched(prefix, layout, a_transpose, b_transpose, m, n, k, alphas, a_ptr, a_offsets, a_ld, b_ptr,
@@ -174,6 +185,18 @@ def symm(queue, m, n, a, b, c, a_ld, b_ld, c_ld, alpha=1.0, beta=0.0, right_side
                       b.data_ptr(), b_offset, b_ld, beta, c.data_ptr(), c_offset, c_ld, _stream_handle(queue))
     if status != 0:
         raise CLBlastError("CLBlast%ssymm" % prefix, status)
+
+
+def trmm(queue, m, n, a, b, a_ld, b_ld, alpha=1.0, right_side=False, lower_triangle=False, a_transp=False,
+         unit_diagonal=False, a_offset=0, b_offset=0):
+    """xTRMM: Triangular matrix-matrix multiplication (row-major, like pyclblast.trmm; pyclblast.pyx:2196-2232)."""
+    prefix = _tensor_info(a, b)
+    status = raw_trmm(prefix, ROW_MAJOR, SIDE_RIGHT if right_side else SIDE_LEFT,
+                      TRIANGLE_LOWER if lower_triangle else TRIANGLE_UPPER, TRANS_YES if a_transp else TRANS_NO,
+                      DIAGONAL_UNIT if unit_diagonal else DIAGONAL_NON_UNIT, m, n, alpha, a.data_ptr(), a_offset, a_ld,
+                      b.data_ptr(), b_offset, b_ld, _stream_handle(queue))
+    if status != 0:
+        raise CLBlastError("CLBlast%strmm" % prefix, status)
 
 
 def gemmBatched(queue, m, n, k, a, b, c, alphas, betas, a_ld, b_ld, c_ld, a_offsets, b_offsets, c_offsets,

@@ -11,6 +11,7 @@
 #include "routines/xgemm.hpp"
 #include "routines/xgemmbatched.hpp"
 #include "routines/xsymm.hpp"
+#include "routines/xtrmm.hpp"
 
 #define CLBLAST_HIP_PUBLIC __attribute__((visibility("default")))
 
@@ -44,6 +45,21 @@ StatusCode Symm(const Layout layout, const Side side, const Triangle triangle, c
     auto routine = Xsymm<T>(queue, event);
     routine.DoSymm(layout, side, triangle, m, n, alpha, Buffer<T>(a_buffer), a_offset, a_ld, Buffer<T>(b_buffer), b_offset,
                    b_ld, beta, Buffer<T>(c_buffer), c_offset, c_ld);
+    return StatusCode::kSuccess;
+  } catch (...) {
+    return DispatchException();
+  }
+}
+
+template <typename T>
+StatusCode Trmm(const Layout layout, const Side side, const Triangle triangle, const Transpose a_transpose,
+                const Diagonal diagonal, const size_t m, const size_t n, const T alpha, const void* a_buffer,
+                const size_t a_offset, const size_t a_ld, void* b_buffer, const size_t b_offset, const size_t b_ld,
+                hipStream_t* queue, hipEvent_t* event) {
+  try {
+    auto routine = Xtrmm<T>(queue, event);
+    routine.DoTrmm(layout, side, triangle, a_transpose, diagonal, m, n, alpha, Buffer<T>(a_buffer), a_offset, a_ld,
+                   Buffer<T>(b_buffer), b_offset, b_ld);
     return StatusCode::kSuccess;
   } catch (...) {
     return DispatchException();
@@ -134,7 +150,11 @@ StatusCode GemmTempBufferSize(const Layout layout, const Transpose a_transpose, 
   template StatusCode CLBLAST_HIP_PUBLIC Symm<T>(const Layout, const Side, const Triangle, const size_t, const size_t,  \
                                                  const T, const void*, const size_t, const size_t, const void*,     \
                                                  const size_t, const size_t, const T, void*, const size_t,          \
-                                                 const size_t, hipStream_t*, hipEvent_t*);
+                                                 const size_t, hipStream_t*, hipEvent_t*);                          \
+  template StatusCode CLBLAST_HIP_PUBLIC Trmm<T>(const Layout, const Side, const Triangle, const Transpose,         \
+                                                 const Diagonal, const size_t, const size_t, const T, const void*,  \
+                                                 const size_t, const size_t, void*, const size_t, const size_t,     \
+                                                 hipStream_t*, hipEvent_t*);
 CLBLAST_HIP_INSTANTIATE(half)
 CLBLAST_HIP_INSTANTIATE(float)
 CLBLAST_HIP_INSTANTIATE(double)

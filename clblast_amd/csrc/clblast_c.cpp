@@ -295,4 +295,22 @@ CLBlastStatusCode CLBlastHsymm(const CLBlastLayout layout, const CLBlastSide sid
   });
 }
 
+// ---- TRMM ---------------------------------------------------------------------------------------
+#define CLBLAST_HIP_TRMM(NAME, ROUTINE, CTYPE, TYPE)                                                                \
+  CLBlastStatusCode NAME(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,         \
+                         const CLBlastTranspose a_transpose, const CLBlastDiagonal diagonal, const size_t m,         \
+                         const size_t n, const CTYPE alpha, const void* a_buffer, const size_t a_offset,             \
+                         const size_t a_ld, void* b_buffer, const size_t b_offset, const size_t b_ld,                \
+                         hipStream_t* queue, hipEvent_t* event) {                                                    \
+    return Guarded([&]() {                                                                                           \
+      return clblast::ROUTINE<TYPE>(L(layout), static_cast<clblast::Side>(side),                                     \
+                                    static_cast<clblast::Triangle>(triangle), Tr(a_transpose),                       \
+                                    static_cast<clblast::Diagonal>(diagonal), m, n, alpha, a_buffer, a_offset, a_ld, \
+                                    b_buffer, b_offset, b_ld, queue, event);                                         \
+    });                                                                                                              \
+  }
+CLBLAST_HIP_TRMM(CLBlastStrmm, Trmm, float, float)
+CLBLAST_HIP_TRMM(CLBlastDtrmm, Trmm, double, double)
+CLBLAST_HIP_TRMM(CLBlastHtrmm, Trmm, unsigned short, clblast::half)
+
 }  // extern "C"

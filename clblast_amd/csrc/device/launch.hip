@@ -9,6 +9,7 @@
 
 #include "device/launch_common.hpp"
 #include "kernels/symmetric_to_square.hpp"
+#include "kernels/triangular_to_square.hpp"
 
 namespace clbh {
 namespace {
@@ -108,6 +109,49 @@ int LaunchSymmetricToSquare(const int upper, const int k, const void* src, const
 }
 }  // namespace
 
+namespace {
+bool MultipleOf8Bytes(const void* pointer) { return reinterpret_cast<unsigned long long>(pointer) % 8 == 0; }
+
+template <typename T>
+int LaunchTriangularToSquare(const int upper, const int unit, const int k, const void* src, const long long src_offset,
+                             const long long src_ld, void* dst, const long long dst_ld, hipStream_t stream) {
+  const T* source = static_cast<const T*>(src) + src_offset;
+  constexpr int VEC = 8 / sizeof(T);
+  const bool vector = VEC > 1 && k % VEC == 0 && src_ld % VEC == 0 && dst_ld % VEC == 0 && MultipleOf8Bytes(source) &&
+                      MultipleOf8Bytes(dst);
+  const int lanes = vector ? (k + VEC - 1) / VEC : k;
+  const dim3 grid(static_cast<unsigned>((lanes + clbh::kCopyThreads - 1) / clbh::kCopyThreads),
+                  static_cast<unsigned>(std::min(k, clbh::kCopyMaxGridY)));
+  if (vector) {
+    clbh::TriangularToSquareKernel<T, VEC><<<grid, dim3(clbh::kCopyThreads), 0, stream>>>(
+        k, upper != 0, unit != 0, source, src_ld, static_cast<T*>(dst), dst_ld);
+  } else {
+    clbh::TriangularToSquareKernel<T, 1><<<grid, dim3(clbh::kCopyThreads), 0, stream>>>(
+        k, upper != 0, unit != 0, source, src_ld, static_cast<T*>(dst), dst_ld);
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
+template <typename T>
+int LaunchCopyMatrix(const int one, const int two, const void* src, const long long src_offset, const long long src_ld,
+                     void* dst, const long long dst_offset, const long long dst_ld, hipStream_t stream) {
+  const T* source = static_cast<const T*>(src) + src_offset;
+  T* target = static_cast<T*>(dst) + dst_offset;
+  constexpr int VEC = 8 / sizeof(T);
+  const bool vector = VEC > 1 && one % VEC == 0 && src_ld % VEC == 0 && dst_ld % VEC == 0 && MultipleOf8Bytes(source) &&
+                      MultipleOf8Bytes(target);
+  const int lanes = vector ? one / VEC : one;
+  const dim3 grid(static_cast<unsigned>((lanes + clbh::kCopyThreads - 1) / clbh::kCopyThreads),
+                  static_cast<unsigned>(std::min(two, clbh::kCopyMaxGridY)));
+  if (vector) {
+    clbh::CopyMatrixKernel<T, VEC><<<grid, dim3(clbh::kCopyThreads), 0, stream>>>(one, two, source, src_ld, target, dst_ld);
+  } else {
+    clbh::CopyMatrixKernel<T, 1><<<grid, dim3(clbh::kCopyThreads), 0, stream>>>(one, two, source, src_ld, target, dst_ld);
+  }
+  return static_cast<int>(hipGetLastError());
+}
+}  // namespace
+
 extern "C" {
 
 int clbh_gemm_launch(const clbh_gemm_desc* desc, hipStream_t stream) {
@@ -129,6 +173,31 @@ int clbh_symmetric_to_square(int precision, int upper, int k, const void* src, l
     case 16: return LaunchSymmetricToSquare<_Float16>(upper, k, src, src_offset, src_ld, dst, stream);
     case 32: return LaunchSymmetricToSquare<float>(upper, k, src, src_offset, src_ld, dst, stream);
     case 64: return LaunchSymmetricToSquare<double>(upper, k, src, src_offset, src_ld, dst, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+int clbh_triangular_to_square(int precision, int upper, int unit_diagonal, int k, const void* src, long long src_offset,
+                              long long src_ld, void* dst, long long dst_ld, hipStream_t stream) {
+  if (k <= 0 || src == nullptr || dst == nullptr || src_ld < k || dst_ld < k || src_offset < 0) { return hipErrorInvalidValue; }
+  switch (precision) {
+    case 16: return LaunchTriangularToSquare<_Float16>(upper, unit_diagonal, k, src, src_offset, src_ld, dst, dst_ld, stream);
+    case 32: return LaunchTriangularToSquare<float>(upper, unit_diagonal, k, src, src_offset, src_ld, dst, dst_ld, stream);
+    case 64: return LaunchTriangularToSquare<double>(upper, unit_diagonal, k, src, src_offset, src_ld, dst, dst_ld, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+int clbh_copy_matrix(int precision, int one_extent, int two_extent, const void* src, long long src_offset, long long src_ld,
+                     void* dst, long long dst_offset, long long dst_ld, hipStream_t stream) {
+  if (one_extent <= 0 || two_extent <= 0 || src == nullptr || dst == nullptr || src_ld < one_extent || dst_ld < one_extent ||
+      src_offset < 0 || dst_offset < 0) {
+    return hipErrorInvalidValue;
+  }
+  switch (precision) {
+    case 16: return LaunchCopyMatrix<_Float16>(one_extent, two_extent, src, src_offset, src_ld, dst, dst_offset, dst_ld, stream);
+    case 32: return LaunchCopyMatrix<float>(one_extent, two_extent, src, src_offset, src_ld, dst, dst_offset, dst_ld, stream);
+    case 64: return LaunchCopyMatrix<double>(one_extent, two_extent, src, src_offset, src_ld, dst, dst_offset, dst_ld, stream);
     default: return hipErrorInvalidValue;
   }
 }

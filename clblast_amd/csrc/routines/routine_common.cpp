@@ -32,6 +32,30 @@ StatusCode DispatchException(const bool silent) {
   return status;
 }
 
+BLASError SwappedOperands(const BLASError& error) {
+  switch (error.status()) {
+    case StatusCode::kInvalidMatrixA: return BLASError(StatusCode::kInvalidMatrixB, error.details());
+    case StatusCode::kInvalidMatrixB: return BLASError(StatusCode::kInvalidMatrixA, error.details());
+    case StatusCode::kInvalidLeadDimA: return BLASError(StatusCode::kInvalidLeadDimB, error.details());
+    case StatusCode::kInvalidLeadDimB: return BLASError(StatusCode::kInvalidLeadDimA, error.details());
+    case StatusCode::kInsufficientMemoryA: return BLASError(StatusCode::kInsufficientMemoryB, error.details());
+    case StatusCode::kInsufficientMemoryB: return BLASError(StatusCode::kInsufficientMemoryA, error.details());
+    default: return error;
+  }
+}
+
+StreamScratch::StreamScratch(const size_t bytes, hipStream_t stream, const char* what)
+    : pointer_(nullptr), bytes_(bytes), stream_(stream) {
+  if (clbh_alloc_async(&pointer_, bytes, stream) != 0) {
+    pointer_ = nullptr;
+    throw RuntimeErrorCode(StatusCode::kTempBufferAllocFailure, what);
+  }
+}
+
+StreamScratch::~StreamScratch() {
+  if (pointer_ != nullptr) { clbh_free_async(pointer_, stream_); }
+}
+
 StatusCode DispatchExceptionForC() {
   const char* message = nullptr;
   try {

@@ -107,6 +107,14 @@ constexpr size_t ElementBytes() { return sizeof(T); }
 
 // =================================================================================================
 
+// The constants 0, 1 and -1 in the host type of a precision (fp16: the binary16 bit patterns)
+template <typename T> inline T ConstantZero() { return T(0); }
+template <typename T> inline T ConstantOne() { return T(1); }
+template <typename T> inline T ConstantNegOne() { return T(-1); }
+template <> inline half ConstantZero<half>() { return 0x0000; }
+template <> inline half ConstantOne<half>() { return 0x3C00; }
+template <> inline half ConstantNegOne<half>() { return 0xBC00; }
+
 // Non-owning view of a caller's device allocation (reference: Buffer<T>(cl_mem), clpp11.hpp:650).
 template <typename T>
 class Buffer {
@@ -123,6 +131,27 @@ class Buffer {
   const void* pointer_;
   size_t known_bytes_;
   bool size_known_;
+};
+
+// The error of a GEMM whose A and B were the caller's B and A, in the caller's terms (reference:
+// src/routines/level3/xsymm.cpp:92-109, xtrmm.cpp:110-127).
+BLASError SwappedOperands(const BLASError& error);
+
+// Stream-ordered scratch memory of one call: allocated on the caller's stream, freed on it when the object goes
+// out of scope (after the kernels that use it have been enqueued), also when an error unwinds the call.
+class StreamScratch {
+ public:
+  StreamScratch(const size_t bytes, hipStream_t stream, const char* what);
+  ~StreamScratch();
+  StreamScratch(const StreamScratch&) = delete;
+  StreamScratch& operator=(const StreamScratch&) = delete;
+  void* get() const { return pointer_; }
+  size_t bytes() const { return bytes_; }
+
+ private:
+  void* pointer_;
+  size_t bytes_;
+  hipStream_t stream_;
 };
 
 // Argument-validation contract; check order: leading dimension first, then the buffer size.

@@ -30,42 +30,25 @@ void Xsymm<T>::DoSymm(const Layout layout, const Side side, const Triangle trian
   // column-major lower one (xsymm.cpp:53-55)
   const auto is_upper = ((triangle == Triangle::kUpper && layout != Layout::kRowMajor) ||
                          (triangle == Triangle::kLower && layout == Layout::kRowMajor));
-  void* square = nullptr;
   const auto square_bytes = k * k * sizeof(T);
-  if (clbh_alloc_async(&square, square_bytes, this->stream()) != 0) {
-    throw RuntimeErrorCode(StatusCode::kTempBufferAllocFailure, "square copy of the symmetric matrix");
-  }
-  try {
-    CheckDevice(clbh_symmetric_to_square(static_cast<int>(PrecisionValue<T>()), is_upper ? 1 : 0, static_cast<int>(k),
-                                         a_buffer(), static_cast<long long>(a_offset), static_cast<long long>(a_ld), square,
-                                         this->stream()),
-                "clbh_symmetric_to_square");
-    const auto square_buffer = Buffer<T>(square, square_bytes);
-    const auto no_temp = Buffer<T>(nullptr);
-    if (side == Side::kLeft) {  // C := A B + C
-      this->DoGemm(layout, Transpose::kNo, Transpose::kNo, m, n, k, alpha, square_buffer, 0, k, b_buffer, b_offset, b_ld, beta,
+  const StreamScratch square(square_bytes, this->stream(), "square copy of the symmetric matrix");
+  CheckDevice(clbh_symmetric_to_square(static_cast<int>(PrecisionValue<T>()), is_upper ? 1 : 0, static_cast<int>(k),
+                                       a_buffer(), static_cast<long long>(a_offset), static_cast<long long>(a_ld),
+                                       square.get(), this->stream()),
+              "clbh_symmetric_to_square");
+  const auto square_buffer = Buffer<T>(square.get(), square_bytes);
+  const auto no_temp = Buffer<T>(nullptr);
+  if (side == Side::kLeft) {  // C := A B + C
+    this->DoGemm(layout, Transpose::kNo, Transpose::kNo, m, n, k, alpha, square_buffer, 0, k, b_buffer, b_offset, b_ld, beta,
+                 c_buffer, c_offset, c_ld, no_temp, false);
+  } else {  // C := B A + C: the GEMM's A is the caller's B, so its error codes are swapped back (xsymm.cpp:88-109)
+    try {
+      this->DoGemm(layout, Transpose::kNo, Transpose::kNo, m, n, k, alpha, b_buffer, b_offset, b_ld, square_buffer, 0, k, beta,
                    c_buffer, c_offset, c_ld, no_temp, false);
-    } else {  // C := B A + C: the GEMM's A is the caller's B, so its error codes are swapped back (xsymm.cpp:88-109)
-      try {
-        this->DoGemm(layout, Transpose::kNo, Transpose::kNo, m, n, k, alpha, b_buffer, b_offset, b_ld, square_buffer, 0, k, beta,
-                     c_buffer, c_offset, c_ld, no_temp, false);
-      } catch (BLASError& e) {
-        switch (e.status()) {
-          case StatusCode::kInvalidMatrixA: throw BLASError(StatusCode::kInvalidMatrixB, e.details());
-          case StatusCode::kInvalidMatrixB: throw BLASError(StatusCode::kInvalidMatrixA, e.details());
-          case StatusCode::kInvalidLeadDimA: throw BLASError(StatusCode::kInvalidLeadDimB, e.details());
-          case StatusCode::kInvalidLeadDimB: throw BLASError(StatusCode::kInvalidLeadDimA, e.details());
-          case StatusCode::kInsufficientMemoryA: throw BLASError(StatusCode::kInsufficientMemoryB, e.details());
-          case StatusCode::kInsufficientMemoryB: throw BLASError(StatusCode::kInsufficientMemoryA, e.details());
-          default: throw;
-        }
-      }
+    } catch (BLASError& e) {
+      throw SwappedOperands(e);
     }
-  } catch (...) {
-    clbh_free_async(square, this->stream());
-    throw;
   }
-  clbh_free_async(square, this->stream());
 }
 
 template class Xsymm<half>;

@@ -81,6 +81,16 @@ CLBH_API size_t clbh_gemm_workspace_bytes(const clbh_gemm_desc* desc);
 CLBH_API int clbh_symmetric_to_square(int precision, int upper, int k, const void* src, long long src_offset,
                                       long long src_ld, void* dst, hipStream_t stream);
 
+// Dense k x k copy (leading dimension dst_ld >= k) of the triangular matrix at src + src_offset: the stored triangle
+// as it is, zeros in the other one, ones on the diagonal when `unit_diagonal` (the stored diagonal is then not read).
+CLBH_API int clbh_triangular_to_square(int precision, int upper, int unit_diagonal, int k, const void* src,
+                                       long long src_offset, long long src_ld, void* dst, long long dst_ld,
+                                       hipStream_t stream);
+
+// dst[dst_offset + two * dst_ld + one] = src[src_offset + two * src_ld + one] for one < one_extent, two < two_extent.
+CLBH_API int clbh_copy_matrix(int precision, int one_extent, int two_extent, const void* src, long long src_offset,
+                              long long src_ld, void* dst, long long dst_offset, long long dst_ld, hipStream_t stream);
+
 // Number of bytes addressable from `ptr` to the end of the device allocation that contains it.
 // Returns 0 on success, non-zero if `ptr` is not inside a device allocation.
 CLBH_API int clbh_buffer_extent(const void* ptr, size_t* bytes_available);

@@ -2,7 +2,7 @@
 // C++ interface of the MI355X (gfx950) GEMM engine behind the CLBlast GEMM API.
 //
 // The argument surface is the one of CLBlast's `include/clblast.h` (reference: Gemm :427-432,
-// GemmBatched :538-543, GemmStridedBatched :547-553, Symm :459-464, GemmTempBufferSize :558-562, StatusCode :61-129,
+// GemmBatched :538-543, GemmStridedBatched :547-553, Symm :459-464, Trmm :476-481, GemmTempBufferSize :558-562, StatusCode :61-129,
 // Layout/Transpose/Precision :132-147, OverrideParameters :620-624, ClearCache :568). Only the handle
 // types differ: `cl_mem` becomes a raw device pointer (`void*`, as returned by hipMalloc or
 // `tensor.data_ptr()`), `cl_command_queue*` becomes `hipStream_t*` and `cl_event*` becomes
@@ -99,6 +99,7 @@ enum class StatusCode {
 enum class Layout { kRowMajor = 101, kColMajor = 102 };
 enum class Transpose { kNo = 111, kYes = 112, kConjugate = 113 };
 enum class Triangle { kUpper = 121, kLower = 122 };
+enum class Diagonal { kNonUnit = 131, kUnit = 132 };
 enum class Side { kLeft = 141, kRight = 142 };
 enum class Precision { kHalf = 16, kSingle = 32, kDouble = 64, kComplexSingle = 3232, kComplexDouble = 6464, kAny = -1 };
 
@@ -140,6 +141,15 @@ StatusCode Symm(const Layout layout, const Side side, const Triangle triangle, c
                 const T alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld, const void* b_buffer,
                 const size_t b_offset, const size_t b_ld, const T beta, void* c_buffer, const size_t c_offset,
                 const size_t c_ld, hipStream_t* queue, hipEvent_t* event = nullptr);
+
+// Triangular matrix-matrix multiplication in place, B = alpha * op(A) * B (side left, A is m x m) or
+// B = alpha * B * op(A) (side right, A is n x n); only the named triangle of A is read, and not its diagonal when
+// that is `kUnit` (reference: include/clblast.h:476-481, src/routines/level3/xtrmm.cpp:33-130).
+template <typename T>
+StatusCode Trmm(const Layout layout, const Side side, const Triangle triangle, const Transpose a_transpose,
+                const Diagonal diagonal, const size_t m, const size_t n, const T alpha, const void* a_buffer,
+                const size_t a_offset, const size_t a_ld, void* b_buffer, const size_t b_offset, const size_t b_ld,
+                hipStream_t* queue, hipEvent_t* event = nullptr);
 
 // Bytes this engine wants in `temp_buffer` for the given arguments (0 when none is needed).
 template <typename T>

@@ -65,6 +65,7 @@ typedef enum CLBlastTranspose_ {
   CLBlastTransposeConjugate = 113
 } CLBlastTranspose;
 typedef enum CLBlastTriangle_ { CLBlastTriangleUpper = 121, CLBlastTriangleLower = 122 } CLBlastTriangle;
+typedef enum CLBlastDiagonal_ { CLBlastDiagonalNonUnit = 131, CLBlastDiagonalUnit = 132 } CLBlastDiagonal;
 typedef enum CLBlastSide_ { CLBlastSideLeft = 141, CLBlastSideRight = 142 } CLBlastSide;
 typedef enum CLBlastPrecision_ {
   CLBlastPrecisionHalf = 16,
@@ -122,6 +123,27 @@ CLBlastStatusCode CLBLAST_HIP_API CLBlastHsymm(const CLBlastLayout layout, const
                                                const size_t b_ld, const unsigned short beta, void* c_buffer,
                                                const size_t c_offset, const size_t c_ld, hipStream_t* queue,
                                                hipEvent_t* event);
+
+// Triangular matrix-matrix multiplication in place: B = alpha*op(A)*B (side left) or alpha*B*op(A) (side right)
+// replaces CLBlastStrmm/CLBlastDtrmm/CLBlastHtrmm (reference: include/clblast_c.h:1062-1092, src/clblast_c.cpp:2300-2400)
+CLBlastStatusCode CLBLAST_HIP_API CLBlastStrmm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const CLBlastTranspose a_transpose,
+                                               const CLBlastDiagonal diagonal, const size_t m, const size_t n,
+                                               const float alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastDtrmm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const CLBlastTranspose a_transpose,
+                                               const CLBlastDiagonal diagonal, const size_t m, const size_t n,
+                                               const double alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastHtrmm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const CLBlastTranspose a_transpose,
+                                               const CLBlastDiagonal diagonal, const size_t m, const size_t n,
+                                               const unsigned short alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, hipStream_t* queue, hipEvent_t* event);
 
 // =================================================================================================
 // Batched GEMM with per-batch alpha, beta and element offsets (host arrays of length batch_count)

@@ -53,6 +53,16 @@ def lib():
         handle.oracle_symm.restype = ci
         handle.oracle_symm_status.argtypes = [ci, ci, ci] + [sz] * 11
         handle.oracle_symm_status.restype = ci
+        handle.oracle_trmm.argtypes = [ci] * 6 + [sz, sz, dbl, vp, sz, sz, vp, sz, sz, vp]
+        handle.oracle_trmm.restype = ci
+        handle.oracle_trsm.argtypes = [ci] * 6 + [sz, sz, dbl, vp, sz, sz, vp, sz, sz, vp]
+        handle.oracle_trsm.restype = ci
+        handle.oracle_trmm_status.argtypes = [ci, ci, ci] + [sz] * 8
+        handle.oracle_trmm_status.restype = ci
+        handle.oracle_syr2k.argtypes = [ci] * 5 + [sz, sz, dbl, vp, sz, sz, vp, sz, sz, dbl, vp, sz, sz, vp]
+        handle.oracle_syr2k.restype = ci
+        handle.oracle_syr2k_status.argtypes = [ci, ci, ci] + [sz] * 11
+        handle.oracle_syr2k_status.restype = ci
         handle.oracle_process_arguments.argtypes = [ci, ci, ci, sz, sz, sz, ctypes.POINTER(Shape)]
         handle.oracle_process_arguments.restype = ci
         handle.oracle_gemm_status.argtypes = [ci, ci, ci, ci] + [sz] * 12
@@ -164,6 +174,86 @@ def symm_numpy(layout, side, triangle, m, n, alpha, a, a_offset, a_ld, b, b_offs
     c_full = c[c_offset + (q * c_ld + r if col_major else r * c_ld + q)].astype(np.float64)
     product = full @ b_full if side == LEFT else b_full @ full
     return alpha * product + (beta * c_full if beta != 0 else 0.0)
+
+
+NON_UNIT, UNIT = 131, 132
+
+
+def _triangular(function, name, layout, side, triangle, a_transpose, diagonal, m, n, alpha, a, a_offset, a_ld, b, b_offset,
+                b_ld):
+    bits = _bits(a)
+    assert _bits(b) == bits
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    result = np.empty((m, n), dtype=np.float64)
+    status = function(bits, layout, side, triangle, a_transpose, diagonal, m, n, float(alpha), a.ctypes.data, a_offset, a_ld,
+                      b.ctypes.data, b_offset, b_ld, result.ctypes.data)
+    if status != 0:
+        raise ValueError("%s status %d" % (name, status))
+    return result
+
+
+def trmm(layout, side, triangle, a_transpose, diagonal, m, n, alpha, a, a_offset, a_ld, b, b_offset, b_ld):
+    """New logical B (m x n, float64, unrounded) of TRMM computed by the C oracle from flat numpy buffers."""
+    return _triangular(lib().oracle_trmm, "oracle_trmm", layout, side, triangle, a_transpose, diagonal, m, n, alpha, a,
+                       a_offset, a_ld, b, b_offset, b_ld)
+
+
+def trsm(layout, side, triangle, a_transpose, diagonal, m, n, alpha, a, a_offset, a_ld, b, b_offset, b_ld):
+    """The solution X (m x n, float64) of op(A) X = alpha B (left) or X op(A) = alpha B (right) by the C oracle."""
+    return _triangular(lib().oracle_trsm, "oracle_trsm", layout, side, triangle, a_transpose, diagonal, m, n, alpha, a,
+                       a_offset, a_ld, b, b_offset, b_ld)
+
+
+def trmm_status(bits, layout, side, m, n, a_offset, a_ld, a_bytes, b_offset, b_ld, b_bytes):
+    """Status of Trmm and of Trsm (the same tests in the same order)."""
+    return lib().oracle_trmm_status(bits, layout, side, m, n, a_offset, a_ld, a_bytes, b_offset, b_ld, b_bytes)
+
+
+def syr2k(layout, triangle, transpose, n, k, alpha, a, a_offset, a_ld, b, b_offset, b_ld, beta, c, c_offset, c_ld,
+          two_sided=True):
+    """The whole logical n x n C (float64) after SYR2K (or, with b = a and two_sided False, SYRK): updated inside the
+    triangle, the old values outside."""
+    bits = _bits(a)
+    assert _bits(b) == bits and _bits(c) == bits
+    a, b, c = np.ascontiguousarray(a), np.ascontiguousarray(b), np.ascontiguousarray(c)
+    result = np.empty((n, n), dtype=np.float64)
+    status = lib().oracle_syr2k(bits, layout, triangle, transpose, 1 if two_sided else 0, n, k, float(alpha), a.ctypes.data,
+                                a_offset, a_ld, b.ctypes.data, b_offset, b_ld, float(beta), c.ctypes.data, c_offset, c_ld,
+                                result.ctypes.data)
+    if status != 0:
+        raise ValueError("oracle_syr2k status %d" % status)
+    return result
+
+
+def syrk(layout, triangle, transpose, n, k, alpha, a, a_offset, a_ld, beta, c, c_offset, c_ld):
+    return syr2k(layout, triangle, transpose, n, k, alpha, a, a_offset, a_ld, a, a_offset, a_ld, beta, c, c_offset, c_ld,
+                 two_sided=False)
+
+
+def syr2k_status(bits, layout, transpose, n, k, a_offset, a_ld, a_bytes, b_offset, b_ld, b_bytes, c_offset, c_ld, c_bytes):
+    return lib().oracle_syr2k_status(bits, layout, transpose, n, k, a_offset, a_ld, a_bytes, b_offset, b_ld, b_bytes,
+                                     c_offset, c_ld, c_bytes)
+
+
+def syrk_status(bits, layout, transpose, n, k, a_offset, a_ld, a_bytes, c_offset, c_ld, c_bytes):
+    return syr2k_status(bits, layout, transpose, n, k, a_offset, a_ld, a_bytes, a_offset, a_ld, a_bytes, c_offset, c_ld,
+                        c_bytes)
+
+
+def matrix_view(layout, buffer, offset, ld, rows, cols):
+    """The logical rows x cols matrix stored at `offset` with leading dimension `ld`, gathered as float64."""
+    r = np.arange(rows, dtype=np.int64)[:, None]
+    q = np.arange(cols, dtype=np.int64)[None, :]
+    return buffer[offset + (q * ld + r if layout == COL_MAJOR else r * ld + q)].astype(np.float64)
+
+
+def triangular_numpy(layout, triangle, a_transpose, diagonal, k, a, a_offset, a_ld):
+    """op(A) as a dense float64 k x k matrix: the named triangle, zeros elsewhere, ones on a unit diagonal."""
+    stored = matrix_view(layout, a, a_offset, a_ld, k, k)
+    dense = np.triu(stored) if triangle == UPPER else np.tril(stored)
+    if diagonal == UNIT:
+        np.fill_diagonal(dense, 1.0)
+    return dense if a_transpose == NO else dense.T
 
 
 def operand_indices(layout, transpose, rows, cols, offset, ld, is_c=False):

@@ -31,6 +31,10 @@
  *                              acc += a*b in the storage precision) and copy/transpose C back. This is
  *                              the "port" CPU baseline, parallelised over tiles with OpenMP.
  *
+ *   oracle_symm, oracle_trmm,  the Level-3 routines the reference builds on its GEMM (src/routines/level3/xsymm.cpp,
+ *   oracle_trsm, oracle_syr2k  xtrmm.cpp, xtrsm.cpp, xsyrk.cpp, xsyr2k.cpp) stated from their definitions in long
+ *   and their *_status         double arithmetic, with the check order of those files.
+ *
  * How each part is pinned (the reference ships no golden vectors for this path):
  *   - process_arguments/use_direct/temp_size/half conversions: compared against the reference's own
  *     code compiled from /root/reference into oracle/_ref (see oracle/Makefile) where that exists,
@@ -41,6 +45,9 @@
  *   - status functions (gemm, batched, strided-batched): against the status codes the real reference
  *     library returns for a validation sweep per precision (1000 + 455 + 430 cases), executed on an
  *     OpenCL device (tests/test_reference_opencl_gpu.py).
+ *   - symm/trmm/trsm/syrk/syr2k: against independent numpy statements, the BLAS routines of scipy
+ *     (dsymm, dtrmm, dtrsm, dsyrk, dsyr2k), algebraic identities, and the real reference library on an OpenCL
+ *     device, status codes included (tests/test_level3_oracle.py, tests/test_symm_oracle.py, tests/test_*_gpu.py).
  * ================================================================================================= */
 #include <stddef.h>
 #include <stdint.h>
@@ -399,6 +406,162 @@ EXPORT int oracle_symm_status(int precision_bits, int layout, int side, size_t m
   status = test_matrix(one, two, b_bytes, b_offset, b_ld, eb, 1, kInvalidLeadDimB, kInsufficientMemoryB);
   if (status != kSuccess) return status;
   return test_matrix(one, two, c_bytes, c_offset, c_ld, eb, 1, kInvalidLeadDimC, kInsufficientMemoryC);
+}
+
+/* ---- the other Level-3 routines built on the GEMM path ------------------------------------------ */
+
+enum { kDiagonalNonUnit = 131, kDiagonalUnit = 132 };
+
+static size_t matrix_index(int layout, size_t offset, size_t ld, size_t row, size_t col) {
+  return (layout == kColMajor) ? (offset + col * ld + row) : (offset + row * ld + col);
+}
+
+/* Element (i, j) of op(A) for a triangular A of which only `triangle` is stored; a unit diagonal is implied,
+ * not read (src/kernels/level3/convert_triangular.opencl:41-48, 80-87). */
+static double triangular_element(const void* a, int bits, int layout, int triangle, int transpose, int diagonal,
+                                 size_t a_offset, size_t a_ld, size_t i, size_t j) {
+  const size_t r = (transpose == kNo) ? i : j, q = (transpose == kNo) ? j : i;
+  if (r == q && diagonal == kDiagonalUnit) return 1.0;
+  const int stored = (triangle == kTriangleUpper) ? (r <= q) : (r >= q);
+  return stored ? load_as_double(a, bits, matrix_index(layout, a_offset, a_ld, r, q)) : 0.0;
+}
+
+/* TRMM (src/routines/level3/xtrmm.cpp:33-130): result (m x n, row-major array) = alpha * op(A) * B (left) or
+ * alpha * B * op(A) (right). */
+EXPORT int oracle_trmm(int bits, int layout, int side, int triangle, int a_transpose, int diagonal, size_t m, size_t n,
+                       double alpha, const void* a, size_t a_offset, size_t a_ld, const void* b, size_t b_offset,
+                       size_t b_ld, double* result) {
+  if (m == 0 || n == 0) return kInvalidDimension;
+#pragma omp parallel for schedule(static)
+  for (long long ii = 0; ii < (long long)m; ++ii) {
+    const size_t i = (size_t)ii;
+    for (size_t j = 0; j < n; ++j) {
+      long double sum = 0.0L;
+      if (side == kSideLeft) {
+        for (size_t p = 0; p < m; ++p)
+          sum += (long double)triangular_element(a, bits, layout, triangle, a_transpose, diagonal, a_offset, a_ld, i, p) *
+                 (long double)load_as_double(b, bits, matrix_index(layout, b_offset, b_ld, p, j));
+      } else {
+        for (size_t p = 0; p < n; ++p)
+          sum += (long double)load_as_double(b, bits, matrix_index(layout, b_offset, b_ld, i, p)) *
+                 (long double)triangular_element(a, bits, layout, triangle, a_transpose, diagonal, a_offset, a_ld, p, j);
+      }
+      result[i * n + j] = alpha * (double)sum;
+    }
+  }
+  return kSuccess;
+}
+
+/* TRSM (src/routines/level3/xtrsm.cpp:38-60 for the meaning): result X (m x n) solves op(A) * X = alpha * B (left)
+ * or X * op(A) = alpha * B (right), by substitution in long double. */
+EXPORT int oracle_trsm(int bits, int layout, int side, int triangle, int a_transpose, int diagonal, size_t m, size_t n,
+                       double alpha, const void* a, size_t a_offset, size_t a_ld, const void* b, size_t b_offset,
+                       size_t b_ld, double* result) {
+  if (m == 0 || n == 0) return kInvalidDimension;
+  const size_t k = (side == kSideLeft) ? m : n;
+  /* op(A) as a dense k x k matrix t; op(A) is lower triangular when (lower, not transposed) or (upper, transposed) */
+  long double* t = (long double*)malloc(sizeof(long double) * k * k);
+  if (t == NULL) return -4;
+  for (size_t i = 0; i < k; ++i)
+    for (size_t j = 0; j < k; ++j)
+      t[i * k + j] = (long double)triangular_element(a, bits, layout, triangle, a_transpose, diagonal, a_offset, a_ld, i, j);
+  const int op_lower = ((triangle == kTriangleLower) == (a_transpose == kNo));
+  if (side == kSideLeft) { /* column j of X: t x = alpha b */
+#pragma omp parallel for schedule(static)
+    for (long long jj = 0; jj < (long long)n; ++jj) {
+      const size_t j = (size_t)jj;
+      long double* x = (long double*)malloc(sizeof(long double) * m);
+      for (size_t step = 0; step < m; ++step) {
+        const size_t i = op_lower ? step : (m - 1 - step);
+        long double value = (long double)alpha * (long double)load_as_double(b, bits, matrix_index(layout, b_offset, b_ld, i, j));
+        if (op_lower) { for (size_t p = 0; p < i; ++p) value -= t[i * k + p] * x[p]; }
+        else { for (size_t p = i + 1; p < m; ++p) value -= t[i * k + p] * x[p]; }
+        x[i] = value / t[i * k + i];
+      }
+      for (size_t i = 0; i < m; ++i) result[i * n + j] = (double)x[i];
+      free(x);
+    }
+  } else { /* row i of X: x t = alpha b, i.e. t^T x^T = alpha b^T; t^T is lower when t is upper */
+#pragma omp parallel for schedule(static)
+    for (long long ii = 0; ii < (long long)m; ++ii) {
+      const size_t i = (size_t)ii;
+      long double* x = (long double*)malloc(sizeof(long double) * n);
+      for (size_t step = 0; step < n; ++step) {
+        const size_t j = op_lower ? (n - 1 - step) : step;
+        long double value = (long double)alpha * (long double)load_as_double(b, bits, matrix_index(layout, b_offset, b_ld, i, j));
+        if (op_lower) { for (size_t p = j + 1; p < n; ++p) value -= x[p] * t[p * k + j]; }
+        else { for (size_t p = 0; p < j; ++p) value -= x[p] * t[p * k + j]; }
+        x[j] = value / t[j * k + j];
+      }
+      for (size_t j = 0; j < n; ++j) result[i * n + j] = (double)x[j];
+      free(x);
+    }
+  }
+  free(t);
+  return kSuccess;
+}
+
+/* Status of Trmm<T> and Trsm<T>: dimensions, A (k x k), B (m x n in the given layout) (xtrmm.cpp:38-52;
+ * xtrsm.cpp:49-56 after its row-major -> column-major exchange, 73-89: the same tests). All handles valid. */
+EXPORT int oracle_trmm_status(int bits, int layout, int side, size_t m, size_t n, size_t a_offset, size_t a_ld,
+                              size_t a_bytes, size_t b_offset, size_t b_ld, size_t b_bytes) {
+  if (m == 0 || n == 0) return kInvalidDimension;
+  const size_t eb = (size_t)bits / 8;
+  const size_t k = (side == kSideLeft) ? m : n;
+  const int status = test_matrix(k, k, a_bytes, a_offset, a_ld, eb, 1, kInvalidLeadDimA, kInsufficientMemoryA);
+  if (status != kSuccess) return status;
+  const size_t one = (layout == kColMajor) ? m : n, two = (layout == kColMajor) ? n : m;
+  return test_matrix(one, two, b_bytes, b_offset, b_ld, eb, 1, kInvalidLeadDimB, kInsufficientMemoryB);
+}
+
+/* SYRK and SYR2K (src/routines/level3/xsyrk.cpp:50-61,63-166, xsyr2k.cpp:30-48): the full n x n logical C after the
+ * call: inside `triangle` alpha * op(A) * op(B)^T [+ alpha * op(B) * op(A)^T] + beta * C, outside it the old C.
+ * op(X) is n x k: X itself (transpose == no) or X^T. For SYRK pass b = a and two_sided = 0. */
+EXPORT int oracle_syr2k(int bits, int layout, int triangle, int transpose, int two_sided, size_t n, size_t k, double alpha,
+                        const void* a, size_t a_offset, size_t a_ld, const void* b, size_t b_offset, size_t b_ld,
+                        double beta, const void* c, size_t c_offset, size_t c_ld, double* result) {
+  if (n == 0 || k == 0) return kInvalidDimension;
+#pragma omp parallel for schedule(static)
+  for (long long ii = 0; ii < (long long)n; ++ii) {
+    const size_t i = (size_t)ii;
+    for (size_t j = 0; j < n; ++j) {
+      const double old = load_as_double(c, bits, matrix_index(layout, c_offset, c_ld, i, j));
+      const int inside = (triangle == kTriangleUpper) ? (i <= j) : (i >= j);
+      if (!inside) { result[i * n + j] = old; continue; }
+      long double sum = 0.0L;
+      for (size_t p = 0; p < k; ++p) {
+        /* op(X)(row, p) = X(row, p) or X(p, row) */
+        const size_t ai = (transpose == kNo) ? matrix_index(layout, a_offset, a_ld, i, p) : matrix_index(layout, a_offset, a_ld, p, i);
+        const size_t bj = (transpose == kNo) ? matrix_index(layout, b_offset, b_ld, j, p) : matrix_index(layout, b_offset, b_ld, p, j);
+        sum += (long double)load_as_double(a, bits, ai) * (long double)load_as_double(b, bits, bj);
+        if (two_sided) {
+          const size_t bi = (transpose == kNo) ? matrix_index(layout, b_offset, b_ld, i, p) : matrix_index(layout, b_offset, b_ld, p, i);
+          const size_t aj = (transpose == kNo) ? matrix_index(layout, a_offset, a_ld, j, p) : matrix_index(layout, a_offset, a_ld, p, j);
+          sum += (long double)load_as_double(b, bits, bi) * (long double)load_as_double(a, bits, aj);
+        }
+      }
+      double value = alpha * (double)sum;
+      if (beta != 0.0) value += beta * old;
+      result[i * n + j] = value;
+    }
+  }
+  return kSuccess;
+}
+
+/* Status of Syrk<T> (b_* = a_*) and Syr2k<T>: ProcessArguments with m = n, then A, B, C (xsyrk.cpp:69-83). */
+EXPORT int oracle_syr2k_status(int bits, int layout, int transpose, size_t n, size_t k, size_t a_offset, size_t a_ld,
+                               size_t a_bytes, size_t b_offset, size_t b_ld, size_t b_bytes, size_t c_offset, size_t c_ld,
+                               size_t c_bytes) {
+  if (n == 0 || k == 0) return kInvalidDimension;
+  const size_t eb = (size_t)bits / 8;
+  /* A and B are stored n x k (not transposed) or k x n; "one" is the contiguous extent */
+  const int rotated = (layout == kColMajor) ? (transpose != kNo) : (transpose == kNo);
+  const size_t one = rotated ? k : n, two = rotated ? n : k;
+  int status = test_matrix(one, two, a_bytes, a_offset, a_ld, eb, 1, kInvalidLeadDimA, kInsufficientMemoryA);
+  if (status != kSuccess) return status;
+  status = test_matrix(one, two, b_bytes, b_offset, b_ld, eb, 1, kInvalidLeadDimB, kInsufficientMemoryB);
+  if (status != kSuccess) return status;
+  return test_matrix(n, n, c_bytes, c_offset, c_ld, eb, 1, kInvalidLeadDimC, kInsufficientMemoryC);
 }
 
 /* ---- the reference's indirect path restated on the CPU (the "port" baseline) -------------------- */

@@ -10,7 +10,8 @@ HIP (both runtimes in one process were seen to lose the device), hence the comma
 
     python -m oracle.reference_opencl --spec spec.json --out result.npz
 
-spec.json: {"routine": "gemm"|"strided"|"symm" (then "side", "triangle" instead of "ta", "tb", "k"), "bits": 16|32|64, "layout", "ta", "tb", "m", "n", "k", "alpha", "beta",
+spec.json: {"routine": "gemm"|"strided"|"symm" (then "side", "triangle" instead of "ta", "tb", "k")|"trmm"|"trsm" ("side",
+"triangle", "ta", "diagonal"; the result is the B buffer), "bits": 16|32|64, "layout", "ta", "tb", "m", "n", "k", "alpha", "beta",
 "a_ld", "b_ld", "c_ld", "offsets": [a, b, c], "seed": s, "low"/"high", "ab_low"/"ab_high", "batch", "strides",
 "runs": r, "sizes": [a, b, c] element counts}. Inputs are oracle.uniform(seed*3 + {0,1,2}, ...), exactly what
 tests/harness.py and the callers generate. The OpenCL host code here is a minimal ctypes binding of the
@@ -117,16 +118,27 @@ def run(spec):
     a = oracle.uniform(seed * 3 + 0, sizes[0], ab_low, ab_high, bits)
     b = oracle.uniform(seed * 3 + 1, sizes[1], ab_low, ab_high, bits)
     c = oracle.uniform(seed * 3 + 2, sizes[2], spec.get("low", -1.0), spec.get("high", 1.0), bits)
+    if spec.get("a_diagonal_boost"):  # well-conditioned triangular solves: |diagonal| >= boost (tests do the same)
+        k_diag, boost = spec["k_diag"], spec["a_diagonal_boost"]
+        positions = spec["offsets"][0] + np.arange(k_diag) * (spec["a_ld"] + 1)
+        a[positions] = a[positions] + np.where(a[positions] >= 0, boost, -boost).astype(a.dtype)
     a_buffer, b_buffer, c_buffer = opencl.buffer_from(a), opencl.buffer_from(b), opencl.buffer_from(c)
+    in_place_b = spec["routine"] in ("trmm", "trsm")  # these overwrite B; "c" is then unused
     sz, vp = ctypes.c_size_t, ctypes.c_void_p
     queue = vp(opencl.queue.value)
-    alpha, beta = scalar_argument(bits, spec["alpha"], reference), scalar_argument(bits, spec["beta"], reference)
+    alpha, beta = scalar_argument(bits, spec["alpha"], reference), scalar_argument(bits, spec.get("beta", 0.0), reference)
     offsets = spec.get("offsets", [0, 0, 0])
     m, n, k = sz(spec["m"]), sz(spec["n"]), sz(spec.get("k", 0))
 
     def call():
         event = vp(None)
-        if spec["routine"] == "symm":
+        if in_place_b:
+            function = getattr(reference, "CLBlast%s%s" % (PREFIX[bits], spec["routine"]))
+            status = function(ctypes.c_int(spec["layout"]), ctypes.c_int(spec["side"]), ctypes.c_int(spec["triangle"]),
+                              ctypes.c_int(spec["ta"]), ctypes.c_int(spec["diagonal"]), m, n, alpha, a_buffer,
+                              sz(offsets[0]), sz(spec["a_ld"]), b_buffer, sz(offsets[1]), sz(spec["b_ld"]),
+                              ctypes.byref(queue), ctypes.byref(event))
+        elif spec["routine"] == "symm":
             function = getattr(reference, "CLBlast%ssymm" % PREFIX[bits])
             status = function(ctypes.c_int(spec["layout"]), ctypes.c_int(spec["side"]), ctypes.c_int(spec["triangle"]), m,
                               n, alpha, a_buffer, sz(offsets[0]), sz(spec["a_ld"]), b_buffer, sz(offsets[1]),
@@ -154,11 +166,14 @@ def run(spec):
 
     status = call()  # first call: includes the reference's run-time kernel compilation
     opencl.finish()
-    result = np.empty_like(c)
-    opencl.read(c_buffer, result)
+    result = np.empty_like(b if in_place_b else c)
+    opencl.read(b_buffer if in_place_b else c_buffer, result)
     times = []
     for _ in range(spec.get("runs", 0)):  # the reference's client reports the minimum over runs, wall clock
-        opencl.write(c_buffer, c)
+        if in_place_b:
+            opencl.write(b_buffer, b)
+        else:
+            opencl.write(c_buffer, c)
         opencl.finish()
         begin = time.perf_counter()
         call()
@@ -190,13 +205,21 @@ def status_sweep(spec):
     alpha, beta = scalar_argument(bits, 1.0, reference), scalar_argument(bits, 0.0, reference)
     statuses = []
     for case in spec["cases"]:
-        if spec.get("symm"):  # [layout, side, triangle, m, n, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes]
+        if spec.get("triangular"):  # "trmm" or "trsm": [layout, side, triangle, ta, diagonal, m, n, a_ld, b_ld, a_bytes, b_bytes]
+            layout, side, triangle, ta, diagonal, m, n, a_ld, b_ld, a_bytes, b_bytes = case
+            c_bytes = 0
+        elif spec.get("symm"):  # [layout, side, triangle, m, n, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes]
             layout, side, triangle, m, n, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes = case
         else:
             layout, ta, tb, m, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes = case[:12]
         a, b, c = buffer_of(a_bytes, 0), buffer_of(b_bytes, 1), buffer_of(c_bytes, 2)
         event = vp(None)
-        if spec.get("symm"):
+        if spec.get("triangular"):
+            function = getattr(reference, "CLBlast%s%s" % (PREFIX[bits], spec["triangular"]))
+            status = function(ctypes.c_int(layout), ctypes.c_int(side), ctypes.c_int(triangle), ctypes.c_int(ta),
+                              ctypes.c_int(diagonal), sz(m), sz(n), alpha, a, sz(0), sz(a_ld), b, sz(0), sz(b_ld),
+                              ctypes.byref(queue), ctypes.byref(event))
+        elif spec.get("symm"):
             function = getattr(reference, "CLBlast%ssymm" % PREFIX[bits])
             status = function(ctypes.c_int(layout), ctypes.c_int(side), ctypes.c_int(triangle), sz(m), sz(n), alpha, a, sz(0),
                               sz(a_ld), b, sz(0), sz(b_ld), beta, c, sz(0), sz(c_ld), ctypes.byref(queue), ctypes.byref(event))
