@@ -36,6 +36,12 @@ def _declare(lib):
         f = getattr(lib, "CLBlast%ssymm" % prefix)
         f.argtypes = [c_int, c_int, c_int, sz, sz, scalar, vp, sz, sz, vp, sz, sz, scalar, vp, sz, sz, vp, vp]
         f.restype = c_int
+        f = getattr(lib, "CLBlast%ssyrk" % prefix)
+        f.argtypes = [c_int, c_int, c_int, sz, sz, scalar, vp, sz, sz, scalar, vp, sz, sz, vp, vp]
+        f.restype = c_int
+        f = getattr(lib, "CLBlast%ssyr2k" % prefix)
+        f.argtypes = [c_int, c_int, c_int, sz, sz, scalar, vp, sz, sz, vp, sz, sz, scalar, vp, sz, sz, vp, vp]
+        f.restype = c_int
         f = getattr(lib, "CLBlast%strmm" % prefix)
         f.argtypes = [c_int] * 5 + [sz, sz, scalar, vp, sz, sz, vp, sz, sz, vp, vp]
         f.restype = c_int
@@ -66,7 +72,8 @@ def load():
 # Every symbol the public C headers declare, for the export test.
 C_API_SYMBOLS = (
     ["CLBlast%sgemm%s" % (p, s) for p in "SDH" for s in ("", "Batched", "StridedBatched", "WithTempBuffer")] +
-    ["CLBlast%sGemmTempBufferSize" % p for p in "SDH"] + ["CLBlast%ssymm" % p for p in "SDH"] + ["CLBlast%strmm" % p for p in "SDH"] +
+    ["CLBlast%sGemmTempBufferSize" % p for p in "SDH"] + ["CLBlast%ssymm" % p for p in "SDH"] + ["CLBlast%strmm" % p for p in "SDH"] + ["CLBlast%ssyrk" % p for p in "SDH"] +
+    ["CLBlast%ssyr2k" % p for p in "SDH"] +
     ["CLBlastClearCache", "CLBlastOverrideParameters", "CLBlastFloatToHalf", "CLBlastHalfToFloat"])
 DEVICE_LAYER_SYMBOLS = [
     "clbh_gemm_launch", "clbh_gemm_workspace_bytes", "clbh_buffer_extent", "clbh_alloc_async", "clbh_free_async",

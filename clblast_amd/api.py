@@ -87,6 +87,26 @@ def raw_symm(prefix, layout, side, triangle, m, n, alpha, a_ptr, a_offset, a_ld,
                                                   _stream_ref(stream_handle), event_ref)
 
 
+def raw_syrk(prefix, layout, triangle, a_transpose, n, k, alpha, a_ptr, a_offset, a_ld, beta, c_ptr, c_offset, c_ld,
+             stream_handle=0, event_handle=None):
+    """CLBlast{S,D,H}syrk through the C ABI (reference: include/clblast_c.h:972-1001)."""
+    lib = _lib.load()
+    event_ref = None if event_handle is None else ctypes.byref(ctypes.c_void_p(event_handle))
+    return getattr(lib, "CLBlast%ssyrk" % prefix)(layout, triangle, a_transpose, n, k, _scalar(prefix, alpha), a_ptr, a_offset,
+                                                  a_ld, _scalar(prefix, beta), c_ptr, c_offset, c_ld,
+                                                  _stream_ref(stream_handle), event_ref)
+
+
+def raw_syr2k(prefix, layout, triangle, ab_transpose, n, k, alpha, a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld, beta, c_ptr,
+              c_offset, c_ld, stream_handle=0, event_handle=None):
+    """CLBlast{S,D,H}syr2k through the C ABI (reference: include/clblast_c.h:1013-1048)."""
+    lib = _lib.load()
+    event_ref = None if event_handle is None else ctypes.byref(ctypes.c_void_p(event_handle))
+    return getattr(lib, "CLBlast%ssyr2k" % prefix)(layout, triangle, ab_transpose, n, k, _scalar(prefix, alpha), a_ptr,
+                                                   a_offset, a_ld, b_ptr, b_offset, b_ld, _scalar(prefix, beta), c_ptr,
+                                                   c_offset, c_ld, _stream_ref(stream_handle), event_ref)
+
+
 def raw_trmm(prefix, layout, side, triangle, a_transpose, diagonal, m, n, alpha, a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld,
              stream_handle=0, event_handle=None):
     """CLBlast{S,D,H}trmm through the C ABI (reference: include/clblast_c.h:1062-1092)."""
@@ -185,6 +205,27 @@ def symm(queue, m, n, a, b, c, a_ld, b_ld, c_ld, alpha=1.0, beta=0.0, right_side
                       b.data_ptr(), b_offset, b_ld, beta, c.data_ptr(), c_offset, c_ld, _stream_handle(queue))
     if status != 0:
         raise CLBlastError("CLBlast%ssymm" % prefix, status)
+
+
+def syrk(queue, n, k, a, c, a_ld, c_ld, alpha=1.0, beta=0.0, lower_triangle=False, a_transp=False, a_offset=0, c_offset=0):
+    """xSYRK: Rank-K update of a symmetric matrix (row-major, like pyclblast.syrk; pyclblast.pyx:2026-2060)."""
+    prefix = _tensor_info(a, c)
+    status = raw_syrk(prefix, ROW_MAJOR, TRIANGLE_LOWER if lower_triangle else TRIANGLE_UPPER,
+                      TRANS_YES if a_transp else TRANS_NO, n, k, alpha, a.data_ptr(), a_offset, a_ld, beta, c.data_ptr(),
+                      c_offset, c_ld, _stream_handle(queue))
+    if status != 0:
+        raise CLBlastError("CLBlast%ssyrk" % prefix, status)
+
+
+def syr2k(queue, n, k, a, b, c, a_ld, b_ld, c_ld, alpha=1.0, beta=0.0, lower_triangle=False, ab_transp=False, a_offset=0,
+          b_offset=0, c_offset=0):
+    """xSYR2K: Rank-2K update of a symmetric matrix (row-major, like pyclblast.syr2k; pyclblast.pyx:2109-2146)."""
+    prefix = _tensor_info(a, b, c)
+    status = raw_syr2k(prefix, ROW_MAJOR, TRIANGLE_LOWER if lower_triangle else TRIANGLE_UPPER,
+                       TRANS_YES if ab_transp else TRANS_NO, n, k, alpha, a.data_ptr(), a_offset, a_ld, b.data_ptr(),
+                       b_offset, b_ld, beta, c.data_ptr(), c_offset, c_ld, _stream_handle(queue))
+    if status != 0:
+        raise CLBlastError("CLBlast%ssyr2k" % prefix, status)
 
 
 def trmm(queue, m, n, a, b, a_ld, b_ld, alpha=1.0, right_side=False, lower_triangle=False, a_transp=False,

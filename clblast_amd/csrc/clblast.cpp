@@ -11,6 +11,7 @@
 #include "routines/xgemm.hpp"
 #include "routines/xgemmbatched.hpp"
 #include "routines/xsymm.hpp"
+#include "routines/xsyrk.hpp"
 #include "routines/xtrmm.hpp"
 
 #define CLBLAST_HIP_PUBLIC __attribute__((visibility("default")))
@@ -45,6 +46,36 @@ StatusCode Symm(const Layout layout, const Side side, const Triangle triangle, c
     auto routine = Xsymm<T>(queue, event);
     routine.DoSymm(layout, side, triangle, m, n, alpha, Buffer<T>(a_buffer), a_offset, a_ld, Buffer<T>(b_buffer), b_offset,
                    b_ld, beta, Buffer<T>(c_buffer), c_offset, c_ld);
+    return StatusCode::kSuccess;
+  } catch (...) {
+    return DispatchException();
+  }
+}
+
+template <typename T>
+StatusCode Syrk(const Layout layout, const Triangle triangle, const Transpose a_transpose, const size_t n,
+                const size_t k, const T alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+                const T beta, void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                hipEvent_t* event) {
+  try {
+    auto routine = Xsyrk<T>(queue, event);
+    routine.DoSyrk(layout, triangle, a_transpose, n, k, alpha, Buffer<T>(a_buffer), a_offset, a_ld, beta,
+                   Buffer<T>(c_buffer), c_offset, c_ld);
+    return StatusCode::kSuccess;
+  } catch (...) {
+    return DispatchException();
+  }
+}
+
+template <typename T>
+StatusCode Syr2k(const Layout layout, const Triangle triangle, const Transpose ab_transpose, const size_t n,
+                 const size_t k, const T alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+                 const void* b_buffer, const size_t b_offset, const size_t b_ld, const T beta, void* c_buffer,
+                 const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {
+  try {
+    auto routine = Xsyr2k<T>(queue, event);
+    routine.DoSyr2k(layout, triangle, ab_transpose, n, k, alpha, Buffer<T>(a_buffer), a_offset, a_ld, Buffer<T>(b_buffer),
+                    b_offset, b_ld, beta, Buffer<T>(c_buffer), c_offset, c_ld);
     return StatusCode::kSuccess;
   } catch (...) {
     return DispatchException();
@@ -151,6 +182,14 @@ StatusCode GemmTempBufferSize(const Layout layout, const Transpose a_transpose, 
                                                  const T, const void*, const size_t, const size_t, const void*,     \
                                                  const size_t, const size_t, const T, void*, const size_t,          \
                                                  const size_t, hipStream_t*, hipEvent_t*);                          \
+  template StatusCode CLBLAST_HIP_PUBLIC Syrk<T>(const Layout, const Triangle, const Transpose, const size_t,         \
+                                                 const size_t, const T, const void*, const size_t, const size_t,    \
+                                                 const T, void*, const size_t, const size_t, hipStream_t*,          \
+                                                 hipEvent_t*);                                                      \
+  template StatusCode CLBLAST_HIP_PUBLIC Syr2k<T>(const Layout, const Triangle, const Transpose, const size_t,        \
+                                                  const size_t, const T, const void*, const size_t, const size_t,   \
+                                                  const void*, const size_t, const size_t, const T, void*,          \
+                                                  const size_t, const size_t, hipStream_t*, hipEvent_t*);           \
   template StatusCode CLBLAST_HIP_PUBLIC Trmm<T>(const Layout, const Side, const Triangle, const Transpose,         \
                                                  const Diagonal, const size_t, const size_t, const T, const void*,  \
                                                  const size_t, const size_t, void*, const size_t, const size_t,     \

@@ -295,6 +295,38 @@ CLBlastStatusCode CLBlastHsymm(const CLBlastLayout layout, const CLBlastSide sid
   });
 }
 
+// ---- SYRK, SYR2K --------------------------------------------------------------------------------
+#define CLBLAST_HIP_SYRK(NAME, CTYPE, TYPE)                                                                          \
+  CLBlastStatusCode NAME(const CLBlastLayout layout, const CLBlastTriangle triangle,                                 \
+                         const CLBlastTranspose a_transpose, const size_t n, const size_t k, const CTYPE alpha,      \
+                         const void* a_buffer, const size_t a_offset, const size_t a_ld, const CTYPE beta,           \
+                         void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,               \
+                         hipEvent_t* event) {                                                                        \
+    return Guarded([&]() {                                                                                           \
+      return clblast::Syrk<TYPE>(L(layout), static_cast<clblast::Triangle>(triangle), Tr(a_transpose), n, k, alpha,  \
+                                 a_buffer, a_offset, a_ld, beta, c_buffer, c_offset, c_ld, queue, event);            \
+    });                                                                                                              \
+  }
+CLBLAST_HIP_SYRK(CLBlastSsyrk, float, float)
+CLBLAST_HIP_SYRK(CLBlastDsyrk, double, double)
+CLBLAST_HIP_SYRK(CLBlastHsyrk, unsigned short, clblast::half)
+
+#define CLBLAST_HIP_SYR2K(NAME, CTYPE, TYPE)                                                                         \
+  CLBlastStatusCode NAME(const CLBlastLayout layout, const CLBlastTriangle triangle,                                 \
+                         const CLBlastTranspose ab_transpose, const size_t n, const size_t k, const CTYPE alpha,     \
+                         const void* a_buffer, const size_t a_offset, const size_t a_ld, const void* b_buffer,       \
+                         const size_t b_offset, const size_t b_ld, const CTYPE beta, void* c_buffer,                 \
+                         const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {          \
+    return Guarded([&]() {                                                                                           \
+      return clblast::Syr2k<TYPE>(L(layout), static_cast<clblast::Triangle>(triangle), Tr(ab_transpose), n, k,       \
+                                  alpha, a_buffer, a_offset, a_ld, b_buffer, b_offset, b_ld, beta, c_buffer,         \
+                                  c_offset, c_ld, queue, event);                                                     \
+    });                                                                                                              \
+  }
+CLBLAST_HIP_SYR2K(CLBlastSsyr2k, float, float)
+CLBLAST_HIP_SYR2K(CLBlastDsyr2k, double, double)
+CLBLAST_HIP_SYR2K(CLBlastHsyr2k, unsigned short, clblast::half)
+
 // ---- TRMM ---------------------------------------------------------------------------------------
 #define CLBLAST_HIP_TRMM(NAME, ROUTINE, CTYPE, TYPE)                                                                \
   CLBlastStatusCode NAME(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,         \

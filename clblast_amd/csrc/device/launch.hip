@@ -38,6 +38,9 @@ bool ValidDescriptor(const clbh_gemm_desc& d) {
     if (d.c_ld < d.m) { return false; }
   }
   if (d.a_offset < 0 || d.b_offset < 0 || d.c_offset < 0) { return false; }
+  if (d.c_triangle < 0 || d.c_triangle > 2 || d.operand_triangle < 0 || d.operand_triangle > 4) { return false; }
+  // the one-wavefront-per-matrix kernel knows no triangles
+  if ((d.c_triangle != 0 || d.operand_triangle != 0) && d.kernel_class == CLBH_KERNEL_SMALL_BATCHED) { return false; }
   return true;
 }
 

@@ -54,6 +54,8 @@ GemmArgs<CT> MakeArgs(const clbh_gemm_desc& d) {
   p.split_chunk = 0;
   p.split_ld = 0;
   p.split_workspace = nullptr;
+  p.c_triangle = d.c_triangle;
+  p.operand_triangle = d.operand_triangle;
   return p;
 }
 
@@ -92,7 +94,8 @@ struct SplitPlan {
 };
 inline SplitPlan PlanSplit(const clbh_gemm_desc& d) {
   SplitPlan plan{1, 0, 0};
-  if (d.split_k > 1 && d.batch_count == 1 && d.batch.alphas == nullptr && d.precision != 16) {
+  if (d.split_k > 1 && d.batch_count == 1 && d.batch.alphas == nullptr && d.precision != 16 && d.c_triangle == 0 &&
+      d.operand_triangle == 0) {
     const int chunk = ((d.k + d.split_k - 1) / d.split_k + 63) / 64 * 64;
     const int splits = (d.k + chunk - 1) / chunk;
     if (splits > 1) { plan = SplitPlan{splits, chunk, (d.m + 3) / 4 * 4}; }

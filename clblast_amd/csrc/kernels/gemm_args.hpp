@@ -35,7 +35,42 @@ struct GemmArgs {
   int split_chunk;
   int split_ld;
   void* split_workspace;
+  // Triangular variants (see clbh_gemm_desc): which part of C is written, which part of an operand is zero
+  int c_triangle;
+  int operand_triangle;
 };
+
+// True when no element of the tile [m0, m0 + tile_m) x [n0, n0 + tile_n) of C belongs to the requested triangle.
+__device__ __forceinline__ bool TileOutsideTriangle(const int c_triangle, const int m0, const int n0, const int tile_m,
+                                                    const int tile_n) {
+  return (c_triangle == 1 && m0 > n0 + tile_n - 1) || (c_triangle == 2 && m0 + tile_m - 1 < n0);
+}
+
+// True when some element of the tile lies outside the requested triangle, i.e. stores have to be masked.
+__device__ __forceinline__ bool TileCrossesDiagonal(const int c_triangle, const int m0, const int n0, const int tile_m,
+                                                    const int tile_n) {
+  return (c_triangle == 1 && m0 + tile_m - 1 > n0) || (c_triangle == 2 && m0 < n0 + tile_n - 1);
+}
+
+__device__ __forceinline__ bool InTriangle(const int c_triangle, const int i, const int j) {
+  return c_triangle == 0 || (c_triangle == 1 ? i <= j : i >= j);
+}
+
+// K range [first, first + length) of the tile at (m0, n0) that a triangular operand leaves non-zero; first is a
+// multiple of the tile extent it derives from, so operand alignment is kept.
+__device__ __forceinline__ void TriangularRange(const int operand_triangle, const int m0, const int n0, const int tile_m,
+                                                const int tile_n, const int k, int& first, int& length) {
+  first = 0;
+  int last = k;
+  switch (operand_triangle) {
+    case 1: last = min(k, m0 + tile_m); break;
+    case 2: first = min(m0, k); break;
+    case 3: last = min(k, n0 + tile_n); break;
+    case 4: first = min(n0, k); break;
+    default: break;
+  }
+  length = last - first;
+}
 
 // Resolves the operand bases and scalars of batch `batch`.
 template <typename T, typename CT>

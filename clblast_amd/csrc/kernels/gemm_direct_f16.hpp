@@ -168,6 +168,8 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
   int tile_m, tile_n;
   TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
   const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
+  if (TileOutsideTriangle(p.c_triangle, m0, n0, TILE_M, TILE_N)) { return; }  // uniform: the whole work-group leaves
+  const bool masked = TileCrossesDiagonal(p.c_triangle, m0, n0, TILE_M, TILE_N);
 
   int a_offset[FM], b_offset[FN];
 #pragma unroll
@@ -181,7 +183,13 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
     T* c;
     float alpha, beta;
     ResolveBatch<T, float>(p, batch, a, b, c, alpha, beta);
-    const int k_len = p.k;
+    int k_len = p.k;
+    if (p.operand_triangle != 0) {  // skip the K range in which a triangular operand is zero
+      int k_first;
+      TriangularRange(p.operand_triangle, m0, n0, TILE_M, TILE_N, p.k, k_first, k_len);
+      a += A_KC ? static_cast<long long>(k_first) : k_first * p.a_ld;
+      b += B_KC ? static_cast<long long>(k_first) : k_first * p.b_ld;
+    }
     const int slabs = (k_len + TILE_K - 1) / TILE_K;
     const int k_tail = k_len % TILE_K;  // valid depth of the last slab when it is partial
 
@@ -344,7 +352,8 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
       typedef _Float16 half8u_t __attribute__((ext_vector_type(8), aligned(4)));  // C needs dword alignment only
       T* stage = lds + wave * (32 * STAGE_PITCH);
       const int wave_m0 = m0 + wave_m * WAVE_M;
-      const bool vector_rows = (wave_m0 + WAVE_M <= p.m) && (p.c_ld % 2 == 0) && ((reinterpret_cast<unsigned long long>(c) & 3) == 0);
+      const bool vector_rows = (wave_m0 + WAVE_M <= p.m) && (p.c_ld % 2 == 0) && ((reinterpret_cast<unsigned long long>(c) & 3) == 0) &&
+                               !masked;
       auto wave_fence = [&]() {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -370,7 +379,7 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
             if (n_blk + row >= p.n) { break; }
 #pragma unroll
             for (int col = lane; col < WAVE_M; col += 64) {
-              if (wave_m0 + col < p.m) {
+              if (wave_m0 + col < p.m && (!masked || InTriangle(p.c_triangle, wave_m0 + col, n_blk + row))) {
                 T* global = c + (n_blk + row) * p.c_ld + wave_m0 + col;
                 if (LOAD) { stage[row * STAGE_PITCH + col] = *global; }
                 else { *global = stage[row * STAGE_PITCH + col]; }

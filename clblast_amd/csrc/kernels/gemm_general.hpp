@@ -33,6 +33,7 @@ __global__ __launch_bounds__(kGeneralThreads) void GemmGeneralKernel(
   const int ty = tid / 16;  // 4 columns of C each
   const int m0 = (blockIdx.x % tiles_m) * TM;
   const int n0 = (blockIdx.x / tiles_m) * TN;
+  if (TileOutsideTriangle(p.c_triangle, m0, n0, TM, TN)) { return; }  // uniform: the whole work-group leaves
 
   for (int batch = blockIdx.y; batch < p.batch_count; batch += gridDim.y) {
     const T* a;
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(kGeneralThreads) void GemmGeneralKernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int gm = m0 + tx * 4 + i;
-        if (gm < p.m && gn < p.n) {
+        if (gm < p.m && gn < p.n && InTriangle(p.c_triangle, gm, gn)) {
           StoreResult<T, CT>(c, gn * p.c_ld + gm, acc[j][i], alpha, beta);
         }
       }

@@ -295,6 +295,8 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
   int tile_m, tile_n;
   TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
   const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
+  if (TileOutsideTriangle(p.c_triangle, m0, n0, TILE_M, TILE_N)) { return; }  // uniform: the whole work-group leaves
+  const bool masked = TileCrossesDiagonal(p.c_triangle, m0, n0, TILE_M, TILE_N);
 
   // LDS read offsets of this lane. Aligned operands: the lane owns FM consecutive m (one vector LDS read,
   // one vector store to C). Otherwise C is stored element-wise, and the lane owns m = lane_x, lane_x + MF,
@@ -322,6 +324,11 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
       c = static_cast<T*>(p.split_workspace) + static_cast<long long>(batch) * p.split_ld * p.n;
       alpha = T(1);
       beta = T(0);
+    } else if (p.operand_triangle != 0) {  // skip the K range in which a triangular operand is zero
+      int k_first;
+      TriangularRange(p.operand_triangle, m0, n0, TILE_M, TILE_N, p.k, k_first, k_len);
+      a += A_KC ? static_cast<long long>(k_first) : k_first * p.a_ld;
+      b += B_KC ? static_cast<long long>(k_first) : k_first * p.b_ld;
     }
     const int slabs = (k_len + TILE_K - 1) / TILE_K;
 
@@ -491,7 +498,7 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
     constexpr int M_STEP = M_INTERLEAVED ? 1 : MF;  // distance in m between the lane's accumulator blocks
     // 16-byte accesses to C need dword alignment only, which every fp32/fp64 address has
     typedef T VMG __attribute__((ext_vector_type(FM > 1 ? FM : 2), aligned(sizeof(T))));
-    const bool vector_store = M_INTERLEAVED && (FM > 1) && (m_base + FM <= p.m);
+    const bool vector_store = M_INTERLEAVED && (FM > 1) && (m_base + FM <= p.m) && !masked;
 #pragma unroll
     for (int j = 0; j < FN; ++j) {
 #pragma unroll
@@ -513,7 +520,9 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
         } else {
 #pragma unroll
           for (int i = 0; i < FM; ++i) {
-            if (m_base + i * M_STEP < p.m) { StoreResult<T, T>(dst, i * M_STEP, acc[i][j][r], alpha, beta); }
+            if (m_base + i * M_STEP < p.m && (!masked || InTriangle(p.c_triangle, m_base + i * M_STEP, n))) {
+              StoreResult<T, T>(dst, i * M_STEP, acc[i][j][r], alpha, beta);
+            }
           }
         }
       }

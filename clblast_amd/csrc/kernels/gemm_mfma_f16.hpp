@@ -165,6 +165,8 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
   int tile_m, tile_n;
   TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
   const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
+  if (TileOutsideTriangle(p.c_triangle, m0, n0, TILE_M, TILE_N)) { return; }  // uniform: the whole work-group leaves
+  const bool masked = TileCrossesDiagonal(p.c_triangle, m0, n0, TILE_M, TILE_N);
   const bool interior = (m0 + TILE_M <= p.m) && (n0 + TILE_N <= p.n);
   const int full_slabs = p.k / TILE_K;
   const int slabs = (p.k + TILE_K - 1) / TILE_K;
@@ -261,7 +263,7 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
       T* stage = lds + wave * (32 * STAGE_PITCH);
       const int wave_m0 = m0 + wave_m * WAVE_M;
       const bool vector_rows = ALIGNED && (wave_m0 + WAVE_M <= p.m) && (p.c_ld % 8 == 0) &&
-                               ((reinterpret_cast<unsigned long long>(c) & 15) == 0);
+                               ((reinterpret_cast<unsigned long long>(c) & 15) == 0) && !masked;
       auto wave_fence = [&]() {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -287,7 +289,7 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
             if (n_blk + row >= p.n) { break; }
 #pragma unroll
             for (int col = lane; col < WAVE_M; col += 64) {
-              if (wave_m0 + col < p.m) {
+              if (wave_m0 + col < p.m && (!masked || InTriangle(p.c_triangle, wave_m0 + col, n_blk + row))) {
                 T* global = c + (n_blk + row) * p.c_ld + wave_m0 + col;
                 if (LOAD) { stage[row * STAGE_PITCH + col] = *global; }
                 else { *global = stage[row * STAGE_PITCH + col]; }

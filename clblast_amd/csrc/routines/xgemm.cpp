@@ -117,7 +117,8 @@ void Xgemm<T>::DoGemm(const Layout layout, const Transpose a_transpose, const Tr
                       const size_t n, const size_t k, const T alpha, const Buffer<T>& a_buffer, const size_t a_offset,
                       const size_t a_ld, const Buffer<T>& b_buffer, const size_t b_offset, const size_t b_ld,
                       const T beta, const Buffer<T>& c_buffer, const size_t c_offset, const size_t c_ld,
-                      const Buffer<T>& temp_buffer, const bool temp_buffer_provided) {
+                      const Buffer<T>& temp_buffer, const bool temp_buffer_provided, const GemmTriangles& triangles,
+                      const bool record_event) {
   // Same order as the reference: dimensions, then A (ld, size), B, C, then the temporary buffer
   const auto shape = ProcessArguments(layout, a_transpose, b_transpose, m, n, k);
   TestMatrixA(shape.a_one, shape.a_two, a_buffer, a_offset, a_ld);
@@ -134,6 +135,15 @@ void Xgemm<T>::DoGemm(const Layout layout, const Transpose a_transpose, const Tr
   desc.split_k = choice.split_k;
   desc.alpha = ScalarToDouble(alpha);
   desc.beta = ScalarToDouble(beta);
+  if (triangles.output != OutputTriangle::kFull || triangles.operand != OperandTriangle::kNone) {
+    // In the canonical problem of a row-major call A and B have changed places and C is transposed
+    const bool folded = (layout != Layout::kColMajor);
+    static constexpr int kFoldedOutput[3] = {0, 2, 1};
+    static constexpr int kFoldedOperand[5] = {0, 3, 4, 1, 2};
+    desc.c_triangle = folded ? kFoldedOutput[static_cast<int>(triangles.output)] : static_cast<int>(triangles.output);
+    desc.operand_triangle = folded ? kFoldedOperand[static_cast<int>(triangles.operand)] : static_cast<int>(triangles.operand);
+    desc.split_k = 1;  // the K ranges of a split launch and of a triangle do not combine
+  }
 
   // Temporary memory: only split-K launches want any. A caller-provided buffer must be large enough
   // (reference: xgemm.cpp:146-151), otherwise stream-ordered scratch is taken for the call.
@@ -157,7 +167,7 @@ void Xgemm<T>::DoGemm(const Layout layout, const Transpose a_transpose, const Tr
     clbh_free_async(scratch, stream());
   }
   CheckDevice(launch_status, "clbh_gemm_launch");
-  Finish();
+  if (record_event) { Finish(); }
 }
 
 template class Xgemm<half>;

@@ -24,6 +24,16 @@ struct GemmShape {
   size_t c_one, c_two;
 };
 
+// Triangular variants of a GEMM, stated for the logical matrices op(A) (m x k), op(B) (k x n) and C (m x n) of the
+// call, whatever the layout: which triangle of C is computed and written (the rest of C stays untouched), and which
+// operand is triangular, i.e. holds explicit zeros that the kernels may skip.
+enum class OutputTriangle { kFull = 0, kUpper = 1, kLower = 2 };  // upper: C(i,j) with i <= j
+enum class OperandTriangle { kNone = 0, kLowerA = 1, kUpperA = 2, kUpperB = 3, kLowerB = 4 };
+struct GemmTriangles {
+  OutputTriangle output = OutputTriangle::kFull;
+  OperandTriangle operand = OperandTriangle::kNone;
+};
+
 // Common part of the three routines: owns the stream, the optional event and the device ordinal.
 class GemmRoutineBase {
  public:
@@ -67,7 +77,8 @@ class Xgemm : public GemmRoutineBase {
               const size_t n, const size_t k, const T alpha, const Buffer<T>& a_buffer, const size_t a_offset,
               const size_t a_ld, const Buffer<T>& b_buffer, const size_t b_offset, const size_t b_ld, const T beta,
               const Buffer<T>& c_buffer, const size_t c_offset, const size_t c_ld, const Buffer<T>& temp_buffer,
-              const bool temp_buffer_provided);
+              const bool temp_buffer_provided, const GemmTriangles& triangles = GemmTriangles{},
+              const bool record_event = true);
 };
 
 // =================================================================================================

@@ -57,13 +57,18 @@ void Xtrmm<T>::DoTrmm(const Layout layout, const Side side, const Triangle trian
   const auto copy_buffer = Buffer<T>(b_copy.get(), copy_bytes);
   const auto no_temp = Buffer<T>(nullptr);
   const auto zero = ConstantZero<T>();
+  // op(A) is lower triangular for (lower, not transposed) and (upper, transposed): the GEMM skips its zero half
+  const bool op_lower = ((triangle == Triangle::kLower) == (a_transpose == Transpose::kNo));
+  auto triangles = GemmTriangles{};
   if (side == Side::kLeft) {  // B := alpha * op(A) * B
+    triangles.operand = op_lower ? OperandTriangle::kLowerA : OperandTriangle::kUpperA;
     this->DoGemm(layout, a_transpose, Transpose::kNo, m, n, k, alpha, square_buffer, 0, square_ld, copy_buffer, 0, copy_ld, zero,
-                 b_buffer, b_offset, b_ld, no_temp, false);
+                 b_buffer, b_offset, b_ld, no_temp, false, triangles);
   } else {  // B := alpha * B * op(A): the GEMM's A is the caller's B (xtrmm.cpp:104-127)
+    triangles.operand = op_lower ? OperandTriangle::kLowerB : OperandTriangle::kUpperB;
     try {
       this->DoGemm(layout, Transpose::kNo, a_transpose, m, n, k, alpha, copy_buffer, 0, copy_ld, square_buffer, 0, square_ld, zero,
-                   b_buffer, b_offset, b_ld, no_temp, false);
+                   b_buffer, b_offset, b_ld, no_temp, false, triangles);
     } catch (BLASError& e) {
       throw SwappedOperands(e);
     }

@@ -66,6 +66,10 @@ typedef struct clbh_gemm_desc_ {
   clbh_batch_arrays batch;
   void* workspace;          // optional device scratch (split-K partial sums), may be NULL
   size_t workspace_bytes;
+  // Triangular variants of the canonical problem (both 0 for a plain GEMM; neither combines with split_k > 1):
+  int c_triangle;        // 1: only C(i,j) with i <= j is computed and written, 2: only i >= j; the rest of C is untouched
+  int operand_triangle;  // the caller states that part of an operand is zero, so that the kernels may skip it:
+                         // 1: A(i,p) = 0 for p > i, 2: A(i,p) = 0 for p < i, 3: B(p,j) = 0 for p > j, 4: B(p,j) = 0 for p < j
 } clbh_gemm_desc;
 
 // Enqueues the kernel(s) for one descriptor on `stream`. Returns 0 on success, otherwise the HIP

@@ -2,7 +2,7 @@
 // C++ interface of the MI355X (gfx950) GEMM engine behind the CLBlast GEMM API.
 //
 // The argument surface is the one of CLBlast's `include/clblast.h` (reference: Gemm :427-432,
-// GemmBatched :538-543, GemmStridedBatched :547-553, Symm :459-464, Trmm :476-481, GemmTempBufferSize :558-562, StatusCode :61-129,
+// GemmBatched :538-543, GemmStridedBatched :547-553, Symm :435-439, Syrk :449-453, Syr2k :463-467, Trmm :477-481, GemmTempBufferSize :558-562, StatusCode :61-129,
 // Layout/Transpose/Precision :132-147, OverrideParameters :620-624, ClearCache :568). Only the handle
 // types differ: `cl_mem` becomes a raw device pointer (`void*`, as returned by hipMalloc or
 // `tensor.data_ptr()`), `cl_command_queue*` becomes `hipStream_t*` and `cl_event*` becomes
@@ -135,16 +135,33 @@ StatusCode GemmStridedBatched(const Layout layout, const Transpose a_transpose, 
 
 // Symmetric matrix-matrix multiplication, C = alpha * A * B + beta * C (side left, A is m x m) or
 // C = alpha * B * A + beta * C (side right, A is n x n); only the named triangle of A is read (reference:
-// include/clblast.h:459-464, src/routines/level3/xsymm.cpp:33-114). T is float, double or half.
+// include/clblast.h:435-439, src/routines/level3/xsymm.cpp:33-114). T is float, double or half.
 template <typename T>
 StatusCode Symm(const Layout layout, const Side side, const Triangle triangle, const size_t m, const size_t n,
                 const T alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld, const void* b_buffer,
                 const size_t b_offset, const size_t b_ld, const T beta, void* c_buffer, const size_t c_offset,
                 const size_t c_ld, hipStream_t* queue, hipEvent_t* event = nullptr);
 
+// Rank-k update of one triangle of a symmetric matrix, C = alpha * op(A) * op(A)^T + beta * C with op(A) n x k; the
+// other triangle of C is neither read nor written (reference: include/clblast.h:449-453,
+// src/routines/level3/xsyrk.cpp:50-166).
+template <typename T>
+StatusCode Syrk(const Layout layout, const Triangle triangle, const Transpose a_transpose, const size_t n,
+                const size_t k, const T alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+                const T beta, void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                hipEvent_t* event = nullptr);
+
+// Rank-2k update, C = alpha * op(A) * op(B)^T + alpha * op(B) * op(A)^T + beta * C (reference:
+// include/clblast.h:463-467, src/routines/level3/xsyr2k.cpp:30-48).
+template <typename T>
+StatusCode Syr2k(const Layout layout, const Triangle triangle, const Transpose ab_transpose, const size_t n,
+                 const size_t k, const T alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+                 const void* b_buffer, const size_t b_offset, const size_t b_ld, const T beta, void* c_buffer,
+                 const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event = nullptr);
+
 // Triangular matrix-matrix multiplication in place, B = alpha * op(A) * B (side left, A is m x m) or
 // B = alpha * B * op(A) (side right, A is n x n); only the named triangle of A is read, and not its diagonal when
-// that is `kUnit` (reference: include/clblast.h:476-481, src/routines/level3/xtrmm.cpp:33-130).
+// that is `kUnit` (reference: include/clblast.h:477-481, src/routines/level3/xtrmm.cpp:33-130).
 template <typename T>
 StatusCode Trmm(const Layout layout, const Side side, const Triangle triangle, const Transpose a_transpose,
                 const Diagonal diagonal, const size_t m, const size_t n, const T alpha, const void* a_buffer,

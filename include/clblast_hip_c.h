@@ -124,6 +124,45 @@ CLBlastStatusCode CLBLAST_HIP_API CLBlastHsymm(const CLBlastLayout layout, const
                                                const size_t c_offset, const size_t c_ld, hipStream_t* queue,
                                                hipEvent_t* event);
 
+// Rank-k update of a symmetric matrix: C = alpha*op(A)*op(A)^T + beta*C, one triangle of C only
+// replaces CLBlastSsyrk/CLBlastDsyrk/CLBlastHsyrk (reference: include/clblast_c.h:972-1001, src/clblast_c.cpp:2052-2140)
+CLBlastStatusCode CLBLAST_HIP_API CLBlastSsyrk(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                               const CLBlastTranspose a_transpose, const size_t n, const size_t k,
+                                               const float alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, const float beta, void* c_buffer, const size_t c_offset,
+                                               const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastDsyrk(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                               const CLBlastTranspose a_transpose, const size_t n, const size_t k,
+                                               const double alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, const double beta, void* c_buffer, const size_t c_offset,
+                                               const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastHsyrk(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                               const CLBlastTranspose a_transpose, const size_t n, const size_t k,
+                                               const unsigned short alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, const unsigned short beta, void* c_buffer, const size_t c_offset,
+                                               const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+
+// Rank-2k update of a symmetric matrix: C = alpha*op(A)*op(B)^T + alpha*op(B)*op(A)^T + beta*C, one triangle of C only
+// replaces CLBlastSsyr2k/CLBlastDsyr2k/CLBlastHsyr2k (reference: include/clblast_c.h:1013-1048, src/clblast_c.cpp:2170-2270)
+CLBlastStatusCode CLBLAST_HIP_API CLBlastSsyr2k(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                                const CLBlastTranspose ab_transpose, const size_t n, const size_t k,
+                                                const float alpha, const void* a_buffer, const size_t a_offset,
+                                                const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                                                const size_t b_ld, const float beta, void* c_buffer, const size_t c_offset,
+                                                const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastDsyr2k(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                                const CLBlastTranspose ab_transpose, const size_t n, const size_t k,
+                                                const double alpha, const void* a_buffer, const size_t a_offset,
+                                                const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                                                const size_t b_ld, const double beta, void* c_buffer, const size_t c_offset,
+                                                const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastHsyr2k(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                                const CLBlastTranspose ab_transpose, const size_t n, const size_t k,
+                                                const unsigned short alpha, const void* a_buffer, const size_t a_offset,
+                                                const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                                                const size_t b_ld, const unsigned short beta, void* c_buffer, const size_t c_offset,
+                                                const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+
 // Triangular matrix-matrix multiplication in place: B = alpha*op(A)*B (side left) or alpha*B*op(A) (side right)
 // replaces CLBlastStrmm/CLBlastDtrmm/CLBlastHtrmm (reference: include/clblast_c.h:1062-1092, src/clblast_c.cpp:2300-2400)
 CLBlastStatusCode CLBLAST_HIP_API CLBlastStrmm(const CLBlastLayout layout, const CLBlastSide side,

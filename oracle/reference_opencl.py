@@ -11,7 +11,7 @@ HIP (both runtimes in one process were seen to lose the device), hence the comma
     python -m oracle.reference_opencl --spec spec.json --out result.npz
 
 spec.json: {"routine": "gemm"|"strided"|"symm" (then "side", "triangle" instead of "ta", "tb", "k")|"trmm"|"trsm" ("side",
-"triangle", "ta", "diagonal"; the result is the B buffer), "bits": 16|32|64, "layout", "ta", "tb", "m", "n", "k", "alpha", "beta",
+"triangle", "ta", "diagonal"; the result is the B buffer)|"syrk"|"syr2k" ("triangle", "ta", "n", "k"), "bits": 16|32|64, "layout", "ta", "tb", "m", "n", "k", "alpha", "beta",
 "a_ld", "b_ld", "c_ld", "offsets": [a, b, c], "seed": s, "low"/"high", "ab_low"/"ab_high", "batch", "strides",
 "runs": r, "sizes": [a, b, c] element counts}. Inputs are oracle.uniform(seed*3 + {0,1,2}, ...), exactly what
 tests/harness.py and the callers generate. The OpenCL host code here is a minimal ctypes binding of the
@@ -128,7 +128,7 @@ def run(spec):
     queue = vp(opencl.queue.value)
     alpha, beta = scalar_argument(bits, spec["alpha"], reference), scalar_argument(bits, spec.get("beta", 0.0), reference)
     offsets = spec.get("offsets", [0, 0, 0])
-    m, n, k = sz(spec["m"]), sz(spec["n"]), sz(spec.get("k", 0))
+    m, n, k = sz(spec.get("m", 0)), sz(spec["n"]), sz(spec.get("k", 0))
 
     def call():
         event = vp(None)
@@ -138,6 +138,16 @@ def run(spec):
                               ctypes.c_int(spec["ta"]), ctypes.c_int(spec["diagonal"]), m, n, alpha, a_buffer,
                               sz(offsets[0]), sz(spec["a_ld"]), b_buffer, sz(offsets[1]), sz(spec["b_ld"]),
                               ctypes.byref(queue), ctypes.byref(event))
+        elif spec["routine"] == "syrk":
+            function = getattr(reference, "CLBlast%ssyrk" % PREFIX[bits])
+            status = function(ctypes.c_int(spec["layout"]), ctypes.c_int(spec["triangle"]), ctypes.c_int(spec["ta"]), n, k,
+                              alpha, a_buffer, sz(offsets[0]), sz(spec["a_ld"]), beta, c_buffer, sz(offsets[2]),
+                              sz(spec["c_ld"]), ctypes.byref(queue), ctypes.byref(event))
+        elif spec["routine"] == "syr2k":
+            function = getattr(reference, "CLBlast%ssyr2k" % PREFIX[bits])
+            status = function(ctypes.c_int(spec["layout"]), ctypes.c_int(spec["triangle"]), ctypes.c_int(spec["ta"]), n, k,
+                              alpha, a_buffer, sz(offsets[0]), sz(spec["a_ld"]), b_buffer, sz(offsets[1]), sz(spec["b_ld"]),
+                              beta, c_buffer, sz(offsets[2]), sz(spec["c_ld"]), ctypes.byref(queue), ctypes.byref(event))
         elif spec["routine"] == "symm":
             function = getattr(reference, "CLBlast%ssymm" % PREFIX[bits])
             status = function(ctypes.c_int(spec["layout"]), ctypes.c_int(spec["side"]), ctypes.c_int(spec["triangle"]), m,
@@ -205,7 +215,9 @@ def status_sweep(spec):
     alpha, beta = scalar_argument(bits, 1.0, reference), scalar_argument(bits, 0.0, reference)
     statuses = []
     for case in spec["cases"]:
-        if spec.get("triangular"):  # "trmm" or "trsm": [layout, side, triangle, ta, diagonal, m, n, a_ld, b_ld, a_bytes, b_bytes]
+        if spec.get("rank_update"):  # "syrk" or "syr2k": [layout, triangle, ta, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes]
+            layout, triangle, ta, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes = case
+        elif spec.get("triangular"):  # "trmm" or "trsm": [layout, side, triangle, ta, diagonal, m, n, a_ld, b_ld, a_bytes, b_bytes]
             layout, side, triangle, ta, diagonal, m, n, a_ld, b_ld, a_bytes, b_bytes = case
             c_bytes = 0
         elif spec.get("symm"):  # [layout, side, triangle, m, n, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes]
@@ -214,7 +226,15 @@ def status_sweep(spec):
             layout, ta, tb, m, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes = case[:12]
         a, b, c = buffer_of(a_bytes, 0), buffer_of(b_bytes, 1), buffer_of(c_bytes, 2)
         event = vp(None)
-        if spec.get("triangular"):
+        if spec.get("rank_update") == "syrk":
+            function = getattr(reference, "CLBlast%ssyrk" % PREFIX[bits])
+            status = function(ctypes.c_int(layout), ctypes.c_int(triangle), ctypes.c_int(ta), sz(n), sz(k), alpha, a, sz(0),
+                              sz(a_ld), beta, c, sz(0), sz(c_ld), ctypes.byref(queue), ctypes.byref(event))
+        elif spec.get("rank_update") == "syr2k":
+            function = getattr(reference, "CLBlast%ssyr2k" % PREFIX[bits])
+            status = function(ctypes.c_int(layout), ctypes.c_int(triangle), ctypes.c_int(ta), sz(n), sz(k), alpha, a, sz(0),
+                              sz(a_ld), b, sz(0), sz(b_ld), beta, c, sz(0), sz(c_ld), ctypes.byref(queue), ctypes.byref(event))
+        elif spec.get("triangular"):
             function = getattr(reference, "CLBlast%s%s" % (PREFIX[bits], spec["triangular"]))
             status = function(ctypes.c_int(layout), ctypes.c_int(side), ctypes.c_int(triangle), ctypes.c_int(ta),
                               ctypes.c_int(diagonal), sz(m), sz(n), alpha, a, sz(0), sz(a_ld), b, sz(0), sz(b_ld),
