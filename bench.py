@@ -166,6 +166,102 @@ class SymmWorkload(Workload):
         return self.full.view(self.m, self.m) if which == "a" else super().logical(which)
 
 
+class TrmmWorkload(Workload):
+    """TRMM in place, B := alpha op(A) B with A m x m triangular on the left (column-major). The unused triangle holds
+    NaN. Repeated calls multiply B by A again and again, so A is close to the identity (unit-sized diagonal,
+    off-diagonal elements uniform in +-1/m): B keeps its magnitude over hundreds of calls. `routine` "trsm" solves
+    with the same matrix instead."""
+
+    def __init__(self, name, prefix, routine, lower, transpose, m, n):
+        import torch
+        super().__init__(name, prefix, COL, YES if transpose else NO, NO, m, n, m, 1.0, 0.0)
+        self.routine, self.triangle = routine, (122 if lower else 121)
+        square = self.a.view(m, m)  # memory [r, q] holds A(q, r): the lower triangle of A is torch's upper one
+        square.mul_(1.0 / m)
+        square.diagonal().fill_(1.0)
+        mask = torch.ones(m, m, device="cuda", dtype=torch.bool)
+        self.dense = (torch.triu(square) if lower else torch.tril(square)).contiguous()
+        square[torch.tril(mask, -1) if lower else torch.triu(mask, 1)] = float("nan")
+        self.b_initial = self.b.clone()
+
+    @property
+    def flops(self):
+        return 1.0 * self.m * self.m * self.n  # the BLAS count of a triangular multiply or solve from the left
+
+    @property
+    def algorithmic_bytes(self):
+        element = BITS[self.prefix] // 8
+        return element * (self.m * self.m // 2 + 2 * self.m * self.n)
+
+    def call(self, stream_handle):
+        from clblast_amd import api
+        status = getattr(api, "raw_" + self.routine)(self.prefix, COL, 141, self.triangle, self.ta, 131, self.m, self.n, 1.0,
+                                                     self.a.data_ptr(), 0, self.m, self.b.data_ptr(), 0, self.m, stream_handle)
+        if status != 0:
+            raise RuntimeError("%s: status %d" % (self.name, status))
+
+    def freivalds_error(self):
+        """One call on the initial B, then op(A) (B0 x) against B x (TRMM) or op(A) (B x) against B0 x (TRSM)."""
+        import torch
+        self.b.copy_(self.b_initial)
+        self.call(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        x = torch.rand(self.n, 1, device="cuda", dtype=torch.float64) - 0.5
+        a = self.dense.view(self.m, self.m).double().T  # as a logical (row, column) matrix
+        if self.ta != NO:
+            a = a.T
+        shape, strides = (self.m, self.n), (1, self.m)
+        after = torch.as_strided(self.b, shape, strides).double()
+        before = torch.as_strided(self.b_initial, shape, strides).double()
+        got, expected = (after @ x, a @ (before @ x)) if self.routine == "trmm" else (a @ (after @ x), before @ x)
+        return float((got - expected).norm() / expected.norm())
+
+
+class SyrkWorkload(Workload):
+    """SYRK, the upper or lower triangle of C := alpha A A^T + beta C with A n x k (column-major); the other triangle
+    of C holds NaN and must keep it."""
+
+    def __init__(self, name, prefix, lower, n, k):
+        import torch
+        super().__init__(name, prefix, COL, NO, YES, n, n, k, 1.0, 0.0)
+        self.b = self.a  # the logical second operand is A itself
+        self.triangle = 122 if lower else 121
+        mask = torch.ones(n, n, device="cuda", dtype=torch.bool)
+        self.inside = torch.triu(mask) if lower else torch.tril(mask)  # memory [r, q] holds C(q, r)
+        self.c.view(n, n)[~self.inside] = float("nan")
+
+    @property
+    def flops(self):
+        return 1.0 * self.k * self.n * (self.n + 1)  # the BLAS count of a rank-k update
+
+    @property
+    def algorithmic_bytes(self):
+        element = BITS[self.prefix] // 8
+        return element * (self.n * self.k + self.n * (self.n + 1) // 2)
+
+    def call(self, stream_handle):
+        from clblast_amd.api import raw_syrk
+        status = raw_syrk(self.prefix, COL, self.triangle, NO, self.n, self.k, 1.0, self.a.data_ptr(), 0, self.n, 0.0,
+                          self.c.data_ptr(), 0, self.n, stream_handle)
+        if status != 0:
+            raise RuntimeError("%s: status %d" % (self.name, status))
+
+    def freivalds_error(self):
+        """The triangle against A (A^T x) with the other triangle's contribution removed: both sides are masked."""
+        import torch
+        x = torch.rand(self.n, 1, device="cuda", dtype=torch.float64) - 0.5
+        a = self.logical("a").double()
+        c = self.c.view(self.n, self.n)
+        assert torch.isnan(c[~self.inside]).all(), "SYRK wrote outside its triangle"
+        got = torch.where(self.inside, c, torch.zeros_like(c)).double().T  # logical C, zero outside the triangle
+        # exact reference for a sample of rows: row i of the triangle times x
+        rows = torch.randint(0, self.n, (64,), device="cuda")
+        full_rows = a[rows] @ a.T  # 64 x n
+        logical_inside = self.inside.T[rows]
+        expected = (torch.where(logical_inside, full_rows, torch.zeros_like(full_rows)) @ x)
+        return float(((got[rows] @ x) - expected).norm() / expected.norm())
+
+
 def time_workload(workload, steps, warmup):
     """Returns (wall seconds for `steps` calls, average device milliseconds per call from stream events)."""
     import torch
@@ -301,6 +397,10 @@ EXTRA_WORKLOADS = {
                                                         132, 8198, (11, 13, 19)),
     "next_ssymm_4096_colLeftUpper": lambda: SymmWorkload("symm_s", "S", COL, True, 4096, 4096, 1.0, 0.0),
     "next_hsymm_4096_rowLeftLower": lambda: SymmWorkload("symm_h", "H", ROW, False, 4096, 4096, 1.0, 0.0),
+    "next_strmm_4096_colLeftLower": lambda: TrmmWorkload("trmm_s", "S", "trmm", True, False, 4096, 4096),
+    "next_dtrmm_4096_colLeftUpperT": lambda: TrmmWorkload("trmm_d", "D", "trmm", False, True, 4096, 4096),
+    "next_ssyrk_4096_colLower": lambda: SyrkWorkload("syrk_s", "S", True, 4096, 4096),
+    "next_hsyrk_8192_colUpper": lambda: SyrkWorkload("syrk_h", "H", False, 8192, 8192),
 }
 
 

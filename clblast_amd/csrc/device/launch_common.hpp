@@ -60,6 +60,14 @@ GemmArgs<CT> MakeArgs(const clbh_gemm_desc& d) {
 }
 
 
+// Work-groups along x of an MFMA-class launch over tiles_m x tiles_n tiles: one per tile, or - for launches with a
+// triangle, whose kernels walk the tiles column-cyclically over the 8 XCDs (TileOfBlockCyclic) - the tile columns
+// rounded up to a multiple of 8.
+inline long long TileBlocks(const clbh_gemm_desc& d, const long long tiles_m, const long long tiles_n) {
+  if (d.c_triangle == 0 && d.operand_triangle == 0) { return tiles_m * tiles_n; }
+  return 8 * tiles_m * ((tiles_n + 7) / 8);
+}
+
 // True when every 16-byte access of the tile loaders and of the epilogue is naturally aligned.
 template <typename T>
 inline bool Aligned16(const clbh_gemm_desc& d) {

@@ -36,8 +36,8 @@ int LaunchHgemmVariant(const clbh_gemm_desc& d, hipStream_t stream) {
   const auto args = MakeArgs<float>(d);
   const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
   const long long tiles_n = (d.n + Config::TILE_N - 1) / Config::TILE_N;
-  if (tiles_m * tiles_n > INT_MAX) { return hipErrorInvalidConfiguration; }
-  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
+  if (TileBlocks(d, tiles_m, tiles_n) > INT_MAX) { return hipErrorInvalidConfiguration; }
+  const dim3 grid(static_cast<unsigned>(TileBlocks(d, tiles_m, tiles_n)), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
   constexpr size_t lds_bytes = Config::LDS_BYTES;
   auto kernel = HgemmMfmaKernel<Config, A_KC, B_KC, ALIGNED>;
   if (lds_bytes > 48 * 1024) {
@@ -66,8 +66,8 @@ int LaunchHdirectVariant(const clbh_gemm_desc& d, hipStream_t stream) {
   const auto args = MakeArgs<float>(d);
   const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
   const long long tiles_n = (d.n + Config::TILE_N - 1) / Config::TILE_N;
-  if (tiles_m * tiles_n > INT_MAX) { return hipErrorInvalidConfiguration; }
-  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
+  if (TileBlocks(d, tiles_m, tiles_n) > INT_MAX) { return hipErrorInvalidConfiguration; }
+  const dim3 grid(static_cast<unsigned>(TileBlocks(d, tiles_m, tiles_n)), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
   constexpr size_t lds_bytes = Config::LDS_BYTES;
   auto kernel = HgemmDirectKernel<Config, A_KC, B_KC>;
   if (lds_bytes > 48 * 1024) {

@@ -39,7 +39,7 @@ int LaunchMfmaVariant(const clbh_gemm_desc& d, hipStream_t stream) {
   auto args = MakeArgs<T>(d);
   const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
   const long long tiles_n = (d.n + Config::TILE_N - 1) / Config::TILE_N;
-  if (tiles_m * tiles_n > INT_MAX) { return hipErrorInvalidConfiguration; }
+  if (TileBlocks(d, tiles_m, tiles_n) > INT_MAX) { return hipErrorInvalidConfiguration; }
   const auto plan = PlanSplit(d);
   int grid_y = std::min(d.batch_count, kMaxGridY);
   if (plan.splits > 1) {
@@ -52,7 +52,7 @@ int LaunchMfmaVariant(const clbh_gemm_desc& d, hipStream_t stream) {
     args.batch_count = plan.splits;
     grid_y = plan.splits;
   }
-  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(grid_y));
+  const dim3 grid(static_cast<unsigned>(TileBlocks(d, tiles_m, tiles_n)), static_cast<unsigned>(grid_y));
   constexpr size_t lds_bytes = Config::LDS_ELEMS * sizeof(T);
   auto kernel = GemmMfmaKernel<T, Config, A_KC, B_KC, ALIGNED>;
   if (lds_bytes > 48 * 1024) {

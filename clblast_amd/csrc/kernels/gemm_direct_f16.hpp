@@ -166,7 +166,11 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
   const int wave_m = wave % Config::WM, wave_n = wave / Config::WM;
 
   int tile_m, tile_n;
-  TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
+  if ((p.c_triangle | p.operand_triangle) != 0) {
+    if (!TileOfBlockCyclic(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n)) { return; }
+  } else {
+    TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
+  }
   const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
   if (TileOutsideTriangle(p.c_triangle, m0, n0, TILE_M, TILE_N)) { return; }  // uniform: the whole work-group leaves
   const bool masked = TileCrossesDiagonal(p.c_triangle, m0, n0, TILE_M, TILE_N);

@@ -248,6 +248,27 @@ __device__ __forceinline__ void TileOfBlock(const int block, const int num_block
   tile_n = (logical % in_group) / group_rows;
 }
 
+// The walk of launches with uneven work per tile (a triangle of C: tiles outside it leave at once; a triangular
+// operand: the K range depends on the tile row or column). Work-groups are dispatched in index order and dealt to the
+// XCDs round-robin, so the XCDs stay evenly loaded only if eight consecutive work-groups carry similar work: XCD x
+// owns the tile columns x, x + 8, x + 16, ..., eight consecutive work-groups are eight neighbouring columns of one
+// tile row, and inside its columns each XCD still walks GROUP_M rows at a time (operand reuse in its L2). The grid
+// holds kNumXcd * tiles_m * ceil(tiles_n / kNumXcd) work-groups (see TriangleBlocks in the launchers); the function
+// returns false for the ones beyond the last column.
+__device__ __forceinline__ bool TileOfBlockCyclic(const int block, const int tiles_m, const int tiles_n, int& tile_m,
+                                                  int& tile_n) {
+  const int xcd = block % kNumXcd, local = block / kNumXcd;
+  constexpr int GROUP_M = 8;
+  const int columns = (tiles_n + kNumXcd - 1) / kNumXcd;  // tile columns per XCD
+  const int in_group = GROUP_M * columns;
+  const int group = local / in_group;
+  const int first_m = group * GROUP_M;
+  const int group_rows = min(tiles_m - first_m, GROUP_M);
+  tile_m = first_m + (local % in_group) % group_rows;
+  tile_n = ((local % in_group) / group_rows) * kNumXcd + xcd;
+  return tile_n < tiles_n;
+}
+
 // ---- the kernel ------------------------------------------------------------------------------------
 template <typename T, typename Config, bool A_KC, bool B_KC, bool ALIGNED>
 __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void GemmMfmaKernel(const GemmArgs<T> p, const int tiles_m,
@@ -293,7 +314,11 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
   const int lane_g = lane / MF;  // k-group of the lane inside one instruction
 
   int tile_m, tile_n;
-  TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
+  if ((p.c_triangle | p.operand_triangle) != 0) {
+    if (!TileOfBlockCyclic(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n)) { return; }
+  } else {
+    TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
+  }
   const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
   if (TileOutsideTriangle(p.c_triangle, m0, n0, TILE_M, TILE_N)) { return; }  // uniform: the whole work-group leaves
   const bool masked = TileCrossesDiagonal(p.c_triangle, m0, n0, TILE_M, TILE_N);

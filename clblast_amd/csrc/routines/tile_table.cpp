@@ -81,7 +81,7 @@ int SplitFor(const size_t tiles, const size_t k) {
 
 KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const bool b_kcontig, const size_t m,
                           const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,
-                          const size_t min_indirect_size) {
+                          const size_t min_indirect_size, const bool triangular) {
   (void)a_kcontig; (void)b_kcontig; (void)per_batch_scalars;
   // Many small fp32 matrices: one wavefront per matrix, bandwidth bound
   if (precision == Precision::kSingle && batch_count >= 16 && m <= 32 && n <= 32 && k <= 32) {
@@ -96,6 +96,22 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     const auto ranges = (precision != Precision::kHalf && batch_count == 1)
                             ? std::max<size_t>(1, std::min<size_t>(ForcedSplit(precision), k / 16)) : 1;
     return KernelChoice{CLBH_KERNEL_MFMA, static_cast<int>(forced) - 1, static_cast<int>(ranges)};
+  }
+  if (triangular) {
+    // About half of the tile work is skipped and what remains is uneven: the largest tile that still leaves four
+    // rounds of working tiles for the 256 CUs, so that the dispatcher can even the load out; never split K.
+    struct Candidate { int index; size_t tile_m, tile_n; };
+    static constexpr Candidate kHalfTiles[] = {{2, 256, 256}, {0, 128, 128}, {1, 64, 64}};
+    static constexpr Candidate kSingleTiles[] = {{3, 256, 128}, {0, 128, 128}, {7, 64, 64}};
+    static constexpr Candidate kDoubleTiles[] = {{0, 128, 128}, {1, 64, 64}, {1, 64, 64}};
+    const auto* candidates = (precision == Precision::kHalf) ? kHalfTiles
+                             : (precision == Precision::kSingle) ? kSingleTiles : kDoubleTiles;
+    auto tile = candidates[2].index;
+    for (int c = 0; c < 3; ++c) {
+      const auto working = CeilDivide(m, candidates[c].tile_m) * CeilDivide(n, candidates[c].tile_n) * batch_count / 2;
+      if (working >= 4 * 256) { tile = candidates[c].index; break; }
+    }
+    return KernelChoice{CLBH_KERNEL_MFMA, tile, 1};
   }
   if (precision == Precision::kHalf) {
     // Direct-load tiles, 0: 128 x 128, 1: 64 x 64, 2: 256 x 256 (8 wavefronts), 3: 128 x 32, 4: 32 x 128. Measured

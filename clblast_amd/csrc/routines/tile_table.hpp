@@ -31,10 +31,11 @@ size_t MinIndirectSize(const int device, const Precision precision);
 // Same decision rule as the reference (src/routines/level3/xgemm.hpp:63-69): m*n*k < threshold^3.
 bool UseDirectKernel(const size_t m, const size_t n, const size_t k, const size_t min_indirect_size);
 
-// Picks the kernel family and tile for a canonical problem (m, n, k per matrix).
+// Picks the kernel family and tile for a canonical problem (m, n, k per matrix). `triangular`: about half of the
+// tile work of the launch is skipped (a triangle of C, or a triangular operand), which calls for smaller tiles.
 KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const bool b_kcontig, const size_t m,
                           const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,
-                          const size_t min_indirect_size);
+                          const size_t min_indirect_size, const bool triangular = false);
 
 // Parameter override store behind clblast::OverrideParameters / RetrieveParameters / ClearCache.
 StatusCode OverrideRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,

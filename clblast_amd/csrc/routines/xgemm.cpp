@@ -127,15 +127,16 @@ void Xgemm<T>::DoGemm(const Layout layout, const Transpose a_transpose, const Tr
 
   auto desc = Canonicalise(shape, layout, m, n, k, a_buffer(), a_offset, a_ld, b_buffer(), b_offset, b_ld,
                            const_cast<void*>(c_buffer()), c_offset, c_ld);
+  const bool triangular = (triangles.output != OutputTriangle::kFull || triangles.operand != OperandTriangle::kNone);
   const auto choice = SelectKernel(PrecisionValue<T>(), desc.a_kcontig != 0, desc.b_kcontig != 0,
                                    static_cast<size_t>(desc.m), static_cast<size_t>(desc.n), k, 1, false,
-                                   min_indirect_size());
+                                   min_indirect_size(), triangular);
   desc.kernel_class = choice.kernel_class;
   desc.tile_variant = choice.tile_variant;
   desc.split_k = choice.split_k;
   desc.alpha = ScalarToDouble(alpha);
   desc.beta = ScalarToDouble(beta);
-  if (triangles.output != OutputTriangle::kFull || triangles.operand != OperandTriangle::kNone) {
+  if (triangular) {
     // In the canonical problem of a row-major call A and B have changed places and C is transposed
     const bool folded = (layout != Layout::kColMajor);
     static constexpr int kFoldedOutput[3] = {0, 2, 1};
