@@ -42,9 +42,10 @@ def _declare(lib):
         f = getattr(lib, "CLBlast%ssyr2k" % prefix)
         f.argtypes = [c_int, c_int, c_int, sz, sz, scalar, vp, sz, sz, vp, sz, sz, scalar, vp, sz, sz, vp, vp]
         f.restype = c_int
-        f = getattr(lib, "CLBlast%strmm" % prefix)
-        f.argtypes = [c_int] * 5 + [sz, sz, scalar, vp, sz, sz, vp, sz, sz, vp, vp]
-        f.restype = c_int
+        for routine in ("trmm", "trsm") if prefix != "H" else ("trmm",):  # there is no half-precision TRSM
+            f = getattr(lib, "CLBlast%s%s" % (prefix, routine))
+            f.argtypes = [c_int] * 5 + [sz, sz, scalar, vp, sz, sz, vp, sz, sz, vp, vp]
+            f.restype = c_int
         f = getattr(lib, "CLBlast%sGemmTempBufferSize" % prefix)
         f.argtypes = [c_int, c_int, c_int, sz, sz, sz, sz, sz, sz, sz, sz, sz, vp, POINTER(sz)]
         f.restype = c_int
@@ -72,9 +73,10 @@ def load():
 # Every symbol the public C headers declare, for the export test.
 C_API_SYMBOLS = (
     ["CLBlast%sgemm%s" % (p, s) for p in "SDH" for s in ("", "Batched", "StridedBatched", "WithTempBuffer")] +
-    ["CLBlast%sGemmTempBufferSize" % p for p in "SDH"] + ["CLBlast%ssymm" % p for p in "SDH"] + ["CLBlast%strmm" % p for p in "SDH"] + ["CLBlast%ssyrk" % p for p in "SDH"] +
+    ["CLBlast%sGemmTempBufferSize" % p for p in "SDH"] + ["CLBlast%ssymm" % p for p in "SDH"] + ["CLBlast%strmm" % p for p in "SDH"] + ["CLBlast%strsm" % p for p in "SD"] + ["CLBlast%ssyrk" % p for p in "SDH"] +
     ["CLBlast%ssyr2k" % p for p in "SDH"] +
     ["CLBlastClearCache", "CLBlastOverrideParameters", "CLBlastFloatToHalf", "CLBlastHalfToFloat"])
 DEVICE_LAYER_SYMBOLS = [
     "clbh_gemm_launch", "clbh_gemm_workspace_bytes", "clbh_buffer_extent", "clbh_alloc_async", "clbh_free_async",
-    "clbh_upload_async", "clbh_event_record", "clbh_stream_device", "clbh_error_string", "clbh_symmetric_to_square", "clbh_triangular_to_square", "clbh_copy_matrix"]
+    "clbh_upload_async", "clbh_event_record", "clbh_stream_device", "clbh_error_string", "clbh_symmetric_to_square", "clbh_triangular_to_square", "clbh_copy_matrix", "clbh_invert_block_size",
+                        "clbh_invert_diagonal_blocks"]

@@ -117,6 +117,16 @@ def raw_trmm(prefix, layout, side, triangle, a_transpose, diagonal, m, n, alpha,
                                                   event_ref)
 
 
+def raw_trsm(prefix, layout, side, triangle, a_transpose, diagonal, m, n, alpha, a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld,
+             stream_handle=0, event_handle=None):
+    """CLBlast{S,D,H}trsm through the C ABI (reference: include/clblast_c.h:1094-1124)."""
+    lib = _lib.load()
+    event_ref = None if event_handle is None else ctypes.byref(ctypes.c_void_p(event_handle))
+    return getattr(lib, "CLBlast%strsm" % prefix)(layout, side, triangle, a_transpose, diagonal, m, n, _scalar(prefix, alpha),
+                                                  a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld, _stream_ref(stream_handle),
+                                                  event_ref)
+
+
 def raw_gemm_batched(prefix, layout, a_transpose, b_transpose, m, n, k, alphas, a_ptr, a_offsets, a_ld, b_ptr,
                      b_offsets, b_ld, betas, c_ptr, c_offsets, c_ld, batch_count, stream_handle=0):
     lib = _lib.load()
@@ -238,6 +248,18 @@ def trmm(queue, m, n, a, b, a_ld, b_ld, alpha=1.0, right_side=False, lower_trian
                       b.data_ptr(), b_offset, b_ld, _stream_handle(queue))
     if status != 0:
         raise CLBlastError("CLBlast%strmm" % prefix, status)
+
+
+def trsm(queue, m, n, a, b, a_ld, b_ld, alpha=1.0, right_side=False, lower_triangle=False, a_transp=False,
+         unit_diagonal=False, a_offset=0, b_offset=0):
+    """xTRSM: Solves a triangular system of equations (row-major, like pyclblast.trsm; pyclblast.pyx:2243-2279)."""
+    prefix = _tensor_info(a, b)
+    status = raw_trsm(prefix, ROW_MAJOR, SIDE_RIGHT if right_side else SIDE_LEFT,
+                      TRIANGLE_LOWER if lower_triangle else TRIANGLE_UPPER, TRANS_YES if a_transp else TRANS_NO,
+                      DIAGONAL_UNIT if unit_diagonal else DIAGONAL_NON_UNIT, m, n, alpha, a.data_ptr(), a_offset, a_ld,
+                      b.data_ptr(), b_offset, b_ld, _stream_handle(queue))
+    if status != 0:
+        raise CLBlastError("CLBlast%strsm" % prefix, status)
 
 
 def gemmBatched(queue, m, n, k, a, b, c, alphas, betas, a_ld, b_ld, c_ld, a_offsets, b_offsets, c_offsets,

@@ -13,6 +13,7 @@
 #include "routines/xsymm.hpp"
 #include "routines/xsyrk.hpp"
 #include "routines/xtrmm.hpp"
+#include "routines/xtrsm.hpp"
 
 #define CLBLAST_HIP_PUBLIC __attribute__((visibility("default")))
 
@@ -90,6 +91,21 @@ StatusCode Trmm(const Layout layout, const Side side, const Triangle triangle, c
   try {
     auto routine = Xtrmm<T>(queue, event);
     routine.DoTrmm(layout, side, triangle, a_transpose, diagonal, m, n, alpha, Buffer<T>(a_buffer), a_offset, a_ld,
+                   Buffer<T>(b_buffer), b_offset, b_ld);
+    return StatusCode::kSuccess;
+  } catch (...) {
+    return DispatchException();
+  }
+}
+
+template <typename T>
+StatusCode Trsm(const Layout layout, const Side side, const Triangle triangle, const Transpose a_transpose,
+                const Diagonal diagonal, const size_t m, const size_t n, const T alpha, const void* a_buffer,
+                const size_t a_offset, const size_t a_ld, void* b_buffer, const size_t b_offset, const size_t b_ld,
+                hipStream_t* queue, hipEvent_t* event) {
+  try {
+    auto routine = Xtrsm<T>(queue, event);
+    routine.DoTrsm(layout, side, triangle, a_transpose, diagonal, m, n, alpha, Buffer<T>(a_buffer), a_offset, a_ld,
                    Buffer<T>(b_buffer), b_offset, b_ld);
     return StatusCode::kSuccess;
   } catch (...) {
@@ -198,6 +214,15 @@ CLBLAST_HIP_INSTANTIATE(half)
 CLBLAST_HIP_INSTANTIATE(float)
 CLBLAST_HIP_INSTANTIATE(double)
 #undef CLBLAST_HIP_INSTANTIATE
+// TRSM exists for float and double only (reference: src/clblast.cpp:1339-1346)
+template StatusCode CLBLAST_HIP_PUBLIC Trsm<float>(const Layout, const Side, const Triangle, const Transpose, const Diagonal,
+                                                   const size_t, const size_t, const float, const void*, const size_t,
+                                                   const size_t, void*, const size_t, const size_t, hipStream_t*,
+                                                   hipEvent_t*);
+template StatusCode CLBLAST_HIP_PUBLIC Trsm<double>(const Layout, const Side, const Triangle, const Transpose, const Diagonal,
+                                                    const size_t, const size_t, const double, const void*, const size_t,
+                                                    const size_t, void*, const size_t, const size_t, hipStream_t*,
+                                                    hipEvent_t*);
 
 // =================================================================================================
 

@@ -327,7 +327,7 @@ CLBLAST_HIP_SYR2K(CLBlastSsyr2k, float, float)
 CLBLAST_HIP_SYR2K(CLBlastDsyr2k, double, double)
 CLBLAST_HIP_SYR2K(CLBlastHsyr2k, unsigned short, clblast::half)
 
-// ---- TRMM ---------------------------------------------------------------------------------------
+// ---- TRMM, TRSM ---------------------------------------------------------------------------------------
 #define CLBLAST_HIP_TRMM(NAME, ROUTINE, CTYPE, TYPE)                                                                \
   CLBlastStatusCode NAME(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,         \
                          const CLBlastTranspose a_transpose, const CLBlastDiagonal diagonal, const size_t m,         \
@@ -344,5 +344,7 @@ CLBLAST_HIP_SYR2K(CLBlastHsyr2k, unsigned short, clblast::half)
 CLBLAST_HIP_TRMM(CLBlastStrmm, Trmm, float, float)
 CLBLAST_HIP_TRMM(CLBlastDtrmm, Trmm, double, double)
 CLBLAST_HIP_TRMM(CLBlastHtrmm, Trmm, unsigned short, clblast::half)
+CLBLAST_HIP_TRMM(CLBlastStrsm, Trsm, float, float)
+CLBLAST_HIP_TRMM(CLBlastDtrsm, Trsm, double, double)
 
 }  // extern "C"

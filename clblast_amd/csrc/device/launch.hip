@@ -117,21 +117,37 @@ bool MultipleOf8Bytes(const void* pointer) { return reinterpret_cast<unsigned lo
 
 template <typename T>
 int LaunchTriangularToSquare(const int upper, const int unit, const int k, const void* src, const long long src_offset,
-                             const long long src_ld, void* dst, const long long dst_ld, hipStream_t stream) {
+                             const long long src_ld, void* dst, const int extent, const long long dst_ld,
+                             hipStream_t stream) {
   const T* source = static_cast<const T*>(src) + src_offset;
   constexpr int VEC = 8 / sizeof(T);
-  const bool vector = VEC > 1 && k % VEC == 0 && src_ld % VEC == 0 && dst_ld % VEC == 0 && MultipleOf8Bytes(source) &&
-                      MultipleOf8Bytes(dst);
-  const int lanes = vector ? (k + VEC - 1) / VEC : k;
+  const bool vector = VEC > 1 && k % VEC == 0 && extent % VEC == 0 && src_ld % VEC == 0 && dst_ld % VEC == 0 &&
+                      MultipleOf8Bytes(source) && MultipleOf8Bytes(dst);
+  const int lanes = vector ? (extent + VEC - 1) / VEC : extent;
   const dim3 grid(static_cast<unsigned>((lanes + clbh::kCopyThreads - 1) / clbh::kCopyThreads),
-                  static_cast<unsigned>(std::min(k, clbh::kCopyMaxGridY)));
+                  static_cast<unsigned>(std::min(extent, clbh::kCopyMaxGridY)));
   if (vector) {
     clbh::TriangularToSquareKernel<T, VEC><<<grid, dim3(clbh::kCopyThreads), 0, stream>>>(
-        k, upper != 0, unit != 0, source, src_ld, static_cast<T*>(dst), dst_ld);
+        k, extent, upper != 0, unit != 0, source, src_ld, static_cast<T*>(dst), dst_ld);
   } else {
     clbh::TriangularToSquareKernel<T, 1><<<grid, dim3(clbh::kCopyThreads), 0, stream>>>(
-        k, upper != 0, unit != 0, source, src_ld, static_cast<T*>(dst), dst_ld);
+        k, extent, upper != 0, unit != 0, source, src_ld, static_cast<T*>(dst), dst_ld);
   }
+  return static_cast<int>(hipGetLastError());
+}
+
+template <typename T, typename CT, int BLOCK>
+int LaunchInvertDiagonalBlocks(const int upper, const int blocks, const void* src, const long long src_ld, void* dst,
+                               hipStream_t stream) {
+  constexpr size_t lds_bytes = size_t{2} * BLOCK * (BLOCK + 1) * sizeof(CT);
+  auto kernel = clbh::InvertDiagonalBlocksKernel<T, CT, BLOCK>;
+  if (lds_bytes > 48 * 1024) {
+    static const hipError_t attribute_status = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+    if (attribute_status != hipSuccess) { return static_cast<int>(attribute_status); }
+  }
+  kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), lds_bytes, stream>>>(upper != 0, static_cast<const T*>(src),
+                                                                                  src_ld, static_cast<T*>(dst));
   return static_cast<int>(hipGetLastError());
 }
 
@@ -181,12 +197,29 @@ int clbh_symmetric_to_square(int precision, int upper, int k, const void* src, l
 }
 
 int clbh_triangular_to_square(int precision, int upper, int unit_diagonal, int k, const void* src, long long src_offset,
-                              long long src_ld, void* dst, long long dst_ld, hipStream_t stream) {
-  if (k <= 0 || src == nullptr || dst == nullptr || src_ld < k || dst_ld < k || src_offset < 0) { return hipErrorInvalidValue; }
+                              long long src_ld, void* dst, int dst_extent, long long dst_ld, hipStream_t stream) {
+  if (k <= 0 || src == nullptr || dst == nullptr || src_ld < k || dst_extent < k || dst_ld < dst_extent || src_offset < 0) {
+    return hipErrorInvalidValue;
+  }
   switch (precision) {
-    case 16: return LaunchTriangularToSquare<_Float16>(upper, unit_diagonal, k, src, src_offset, src_ld, dst, dst_ld, stream);
-    case 32: return LaunchTriangularToSquare<float>(upper, unit_diagonal, k, src, src_offset, src_ld, dst, dst_ld, stream);
-    case 64: return LaunchTriangularToSquare<double>(upper, unit_diagonal, k, src, src_offset, src_ld, dst, dst_ld, stream);
+    case 16: return LaunchTriangularToSquare<_Float16>(upper, unit_diagonal, k, src, src_offset, src_ld, dst, dst_extent, dst_ld, stream);
+    case 32: return LaunchTriangularToSquare<float>(upper, unit_diagonal, k, src, src_offset, src_ld, dst, dst_extent, dst_ld, stream);
+    case 64: return LaunchTriangularToSquare<double>(upper, unit_diagonal, k, src, src_offset, src_ld, dst, dst_extent, dst_ld, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+int clbh_invert_block_size(int precision) { return (precision == 64) ? 64 : 128; }
+
+int clbh_invert_diagonal_blocks(int precision, int upper, int blocks, const void* src, long long src_ld, void* dst,
+                                hipStream_t stream) {
+  if (blocks <= 0 || src == nullptr || dst == nullptr || src_ld < static_cast<long long>(blocks) * clbh_invert_block_size(precision)) {
+    return hipErrorInvalidValue;
+  }
+  switch (precision) {
+    case 16: return LaunchInvertDiagonalBlocks<_Float16, float, 128>(upper, blocks, src, src_ld, dst, stream);
+    case 32: return LaunchInvertDiagonalBlocks<float, float, 128>(upper, blocks, src, src_ld, dst, stream);
+    case 64: return LaunchInvertDiagonalBlocks<double, double, 64>(upper, blocks, src, src_ld, dst, stream);
     default: return hipErrorInvalidValue;
   }
 }

@@ -49,8 +49,8 @@ void Xtrmm<T>::DoTrmm(const Layout layout, const Side side, const Triangle trian
   const StreamScratch square(square_bytes, this->stream(), "square copy of the triangular matrix");
   CheckDevice(clbh_triangular_to_square(precision, is_upper ? 1 : 0, (diagonal == Diagonal::kUnit) ? 1 : 0,
                                         static_cast<int>(k), a_buffer(), static_cast<long long>(a_offset),
-                                        static_cast<long long>(a_ld), square.get(), static_cast<long long>(square_ld),
-                                        this->stream()),
+                                        static_cast<long long>(a_ld), square.get(), static_cast<int>(k),
+                                        static_cast<long long>(square_ld), this->stream()),
               "clbh_triangular_to_square");
 
   const auto square_buffer = Buffer<T>(square.get(), square_bytes);

@@ -1,0 +1,144 @@
+// =================================================================================================
+// Xtrsm<T> host logic (see xtrsm.hpp).
+// =================================================================================================
+#include "routines/xtrsm.hpp"
+
+#include <climits>
+#include <functional>
+#include <utility>
+
+namespace clblast {
+// =================================================================================================
+
+template <typename T>
+Xtrsm<T>::Xtrsm(hipStream_t* queue, hipEvent_t* event) : Xgemm<T>(queue, event) {}
+
+template <typename T>
+void Xtrsm<T>::DoTrsm(const Layout layout, Side side, Triangle triangle, const Transpose a_transpose,
+                      const Diagonal diagonal, size_t m, size_t n, const T alpha, const Buffer<T>& a_buffer,
+                      const size_t a_offset, const size_t a_ld, const Buffer<T>& b_buffer, const size_t b_offset,
+                      const size_t b_ld) {
+  // A row-major problem is the column-major problem of the transposed matrices: B^T = X^T * A^T exchanges the sides,
+  // the triangles and m and n (xtrsm.cpp:44-57)
+  if (layout == Layout::kRowMajor) {
+    std::swap(m, n);
+    side = (side == Side::kLeft) ? Side::kRight : Side::kLeft;
+    triangle = (triangle == Triangle::kLower) ? Triangle::kUpper : Triangle::kLower;
+  }
+  TrsmColMajor(side, triangle, a_transpose, diagonal, m, n, alpha, a_buffer, a_offset, a_ld, b_buffer, b_offset, b_ld);
+}
+
+template <typename T>
+void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Transpose a_transpose,
+                            const Diagonal diagonal, const size_t m, const size_t n, const T alpha,
+                            const Buffer<T>& a_buffer, const size_t a_offset, const size_t a_ld,
+                            const Buffer<T>& b_buffer, const size_t b_offset, const size_t b_ld) {
+  // Same order as the reference (xtrsm.cpp:73-89): dimensions, the triangular matrix A, then B
+  if ((m == 0) || (n == 0)) {
+    throw BLASError(StatusCode::kInvalidDimension);
+  }
+  if (m > static_cast<size_t>(INT_MAX) / 2 || n > static_cast<size_t>(INT_MAX) / 2) {
+    throw BLASError(StatusCode::kInvalidDimension, "dimension exceeds 2^30");
+  }
+  const auto k = (side == Side::kLeft) ? m : n;
+  TestMatrixA(k, k, a_buffer, a_offset, a_ld);
+  TestMatrixB(m, n, b_buffer, b_offset, b_ld);
+
+  const auto precision = static_cast<int>(PrecisionValue<T>());
+  const auto stream = this->stream();
+  const auto block = static_cast<size_t>(clbh_invert_block_size(precision));
+  const auto blocks = (k + block - 1) / block;
+  const auto k_padded = blocks * block;
+  constexpr size_t kLineMultiple = 16 / sizeof(T);
+
+  // Dense copy of the triangle, padded with the identity to whole blocks: the other triangle becomes zeros, an
+  // implied diagonal ones, and no block operation below has a ragged edge on the A side
+  const auto dense_bytes = k_padded * k_padded * sizeof(T);
+  const StreamScratch dense(dense_bytes, stream, "dense copy of the triangular matrix");
+  const auto is_upper = (triangle == Triangle::kUpper);
+  CheckDevice(clbh_triangular_to_square(precision, is_upper ? 1 : 0, (diagonal == Diagonal::kUnit) ? 1 : 0,
+                                        static_cast<int>(k), a_buffer(), static_cast<long long>(a_offset),
+                                        static_cast<long long>(a_ld), dense.get(), static_cast<int>(k_padded),
+                                        static_cast<long long>(k_padded), stream),
+              "clbh_triangular_to_square");
+  // Inverses of the diagonal blocks (xtrsm.cpp:105-118 with Xinvert)
+  const auto inverse_bytes = blocks * block * block * sizeof(T);
+  const StreamScratch inverses(inverse_bytes, stream, "inverted diagonal blocks");
+  CheckDevice(clbh_invert_diagonal_blocks(precision, is_upper ? 1 : 0, static_cast<int>(blocks), dense.get(),
+                                          static_cast<long long>(k_padded), inverses.get(), stream),
+              "clbh_invert_diagonal_blocks");
+  // The solution is built in a buffer of its own and copied over B at the end: the block products read B while
+  // they write X (xtrsm.cpp:91-99, 243)
+  const auto x_ld = (m + kLineMultiple - 1) / kLineMultiple * kLineMultiple;
+  const auto x_bytes = x_ld * n * sizeof(T);
+  const StreamScratch solution(x_bytes, stream, "solution of the triangular system");
+
+  const auto dense_buffer = Buffer<T>(dense.get(), dense_bytes);
+  const auto inverse_buffer = Buffer<T>(inverses.get(), inverse_bytes);
+  const auto x_buffer = Buffer<T>(solution.get(), x_bytes);
+  const auto no_temp = Buffer<T>(nullptr);
+  const auto one = ConstantOne<T>();
+  const auto zero = ConstantZero<T>();
+  const auto minus_one = ConstantNegOne<T>();
+  const auto no = Transpose::kNo;
+  const bool transposed = (a_transpose != Transpose::kNo);
+  // op(A) is lower triangular for (lower, not transposed) and (upper, transposed)
+  const bool op_lower = (is_upper == transposed);
+
+  // Offset in the dense copy of the stored block that op(A)[rows r0.., columns c0..] is read from
+  const auto stored_at = [&](const size_t r0, const size_t c0) {
+    return transposed ? (c0 + r0 * k_padded) : (r0 + c0 * k_padded);
+  };
+  const auto gemm = [&](const Transpose ta, const Transpose tb, const size_t gm, const size_t gn, const size_t gk,
+                        const T galpha, const Buffer<T>& ga, const size_t ga_offset, const size_t ga_ld,
+                        const Buffer<T>& gb, const size_t gb_offset, const size_t gb_ld, const T gbeta,
+                        const Buffer<T>& gc, const size_t gc_offset, const size_t gc_ld) {
+    this->DoGemm(Layout::kColMajor, ta, tb, gm, gn, gk, galpha, ga, ga_offset, ga_ld, gb, gb_offset, gb_ld, gbeta, gc,
+                 gc_offset, gc_ld, no_temp, false, GemmTriangles{}, false);
+  };
+
+  // Solves for the rows (left) or columns (right) [lo, hi) of X. `scaled`: this part of B has already been multiplied by
+  // alpha (by an update); alpha multiplies every element of B exactly once, in the first product that reads it.
+  std::function<void(size_t, size_t, bool)> solve = [&](const size_t lo, const size_t hi, const bool scaled) {
+    const auto factor = scaled ? one : alpha;
+    if (hi - lo <= block) {
+      const auto size = hi - lo;
+      const auto inverse_offset = (lo / block) * block * block;
+      if (side == Side::kLeft) {  // X[lo:hi, :] = factor * op(inverse) * B[lo:hi, :]
+        gemm(a_transpose, no, size, n, size, factor, inverse_buffer, inverse_offset, block, b_buffer, b_offset + lo, b_ld, zero,
+             x_buffer, lo, x_ld);
+      } else {                    // X[:, lo:hi] = factor * B[:, lo:hi] * op(inverse)
+        gemm(no, a_transpose, m, size, size, factor, b_buffer, b_offset + lo * b_ld, b_ld, inverse_buffer, inverse_offset,
+             block, zero, x_buffer, lo * x_ld, x_ld);
+      }
+      return;
+    }
+    const auto mid = lo + ((hi - lo + block - 1) / block / 2) * block;  // a multiple of the block size inside (lo, hi)
+    // Left: a lower op(A) is solved from the top, an upper one from the bottom; right: the other way round
+    const bool first_half_first = (side == Side::kLeft) ? op_lower : !op_lower;
+    const auto done_lo = first_half_first ? lo : mid, done_hi = first_half_first ? mid : hi;  // solved first
+    const auto rest_lo = first_half_first ? mid : lo, rest_hi = first_half_first ? hi : mid;  // updated, then solved
+    solve(done_lo, done_hi, scaled);
+    if (side == Side::kLeft) {  // B[rest, :] = factor * B[rest, :] - op(A)[rest, done] * X[done, :]
+      gemm(a_transpose, no, rest_hi - rest_lo, n, done_hi - done_lo, minus_one, dense_buffer, stored_at(rest_lo, done_lo),
+           k_padded, x_buffer, done_lo, x_ld, factor, b_buffer, b_offset + rest_lo, b_ld);
+    } else {                    // B[:, rest] = factor * B[:, rest] - X[:, done] * op(A)[done, rest]
+      gemm(no, a_transpose, m, rest_hi - rest_lo, done_hi - done_lo, minus_one, x_buffer, done_lo * x_ld, x_ld, dense_buffer,
+           stored_at(done_lo, rest_lo), k_padded, factor, b_buffer, b_offset + rest_lo * b_ld, b_ld);
+    }
+    solve(rest_lo, rest_hi, true);
+  };
+  solve(0, k, false);
+
+  CheckDevice(clbh_copy_matrix(precision, static_cast<int>(m), static_cast<int>(n), solution.get(), 0,
+                               static_cast<long long>(x_ld), const_cast<void*>(b_buffer()), static_cast<long long>(b_offset),
+                               static_cast<long long>(b_ld), stream),
+              "clbh_copy_matrix");
+  this->Finish();
+}
+
+template class Xtrsm<float>;
+template class Xtrsm<double>;
+
+// =================================================================================================
+}  // namespace clblast

@@ -1,0 +1,35 @@
+// =================================================================================================
+// Xtrsm<T>: host logic of Trsm<T>, the solution X of op(A) * X = alpha * B (left) or X * op(A) = alpha * B
+// (right) written over B, with A triangular (reference: src/routines/level3/xtrsm.{hpp,cpp}).
+//
+// The reference walks the diagonal in blocks of 16: it inverts the 16 x 16 diagonal blocks, and for every block
+// runs one small GEMM with the inverse and one GEMM that updates the rest of B, synchronising with the host in
+// between. The structure here is the same - inverted diagonal blocks, everything else is GEMM - but recursive and
+// stream-ordered: the diagonal blocks are 128 x 128 (64 x 64 in fp64) and inverted by one kernel, and the triangle is
+// halved recursively, so that the bulk of the work is a few GEMMs with a long K instead of many rank-16 updates.
+// =================================================================================================
+#ifndef CLBLAST_HIP_ROUTINES_XTRSM_HPP_
+#define CLBLAST_HIP_ROUTINES_XTRSM_HPP_
+
+#include "routines/xgemm.hpp"
+
+namespace clblast {
+
+template <typename T>
+class Xtrsm : public Xgemm<T> {
+ public:
+  Xtrsm(hipStream_t* queue, hipEvent_t* event);
+  void DoTrsm(const Layout layout, Side side, Triangle triangle, const Transpose a_transpose, const Diagonal diagonal,
+              size_t m, size_t n, const T alpha, const Buffer<T>& a_buffer, const size_t a_offset, const size_t a_ld,
+              const Buffer<T>& b_buffer, const size_t b_offset, const size_t b_ld);
+
+ private:
+  // The column-major problem (xtrsm.cpp:63-246)
+  void TrsmColMajor(const Side side, const Triangle triangle, const Transpose a_transpose, const Diagonal diagonal,
+                    const size_t m, const size_t n, const T alpha, const Buffer<T>& a_buffer, const size_t a_offset,
+                    const size_t a_ld, const Buffer<T>& b_buffer, const size_t b_offset, const size_t b_ld);
+};
+
+}  // namespace clblast
+
+#endif  // CLBLAST_HIP_ROUTINES_XTRSM_HPP_

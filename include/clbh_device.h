@@ -85,11 +85,21 @@ CLBH_API size_t clbh_gemm_workspace_bytes(const clbh_gemm_desc* desc);
 CLBH_API int clbh_symmetric_to_square(int precision, int upper, int k, const void* src, long long src_offset,
                                       long long src_ld, void* dst, hipStream_t stream);
 
-// Dense k x k copy (leading dimension dst_ld >= k) of the triangular matrix at src + src_offset: the stored triangle
-// as it is, zeros in the other one, ones on the diagonal when `unit_diagonal` (the stored diagonal is then not read).
+// Dense dst_extent x dst_extent copy (dst_extent >= k, leading dimension dst_ld >= dst_extent) of the k x k triangular
+// matrix at src + src_offset: the stored triangle as it is, zeros in the other one, ones on the diagonal when
+// `unit_diagonal` (the stored diagonal is then not read), and the identity in rows and columns k .. dst_extent - 1.
 CLBH_API int clbh_triangular_to_square(int precision, int upper, int unit_diagonal, int k, const void* src,
-                                       long long src_offset, long long src_ld, void* dst, long long dst_ld,
-                                       hipStream_t stream);
+                                       long long src_offset, long long src_ld, void* dst, int dst_extent,
+                                       long long dst_ld, hipStream_t stream);
+
+// Block size of clbh_invert_diagonal_blocks for a precision (128 for 16 and 32 bits, 64 for 64 bits).
+CLBH_API int clbh_invert_block_size(int precision);
+
+// Inverts the `blocks` diagonal blocks (clbh_invert_block_size(precision) squared each) of the dense triangular matrix
+// `src` (blocks * block rows and columns, zeros in the other triangle, non-zero diagonal); block b of the result is
+// the dense block x block matrix at dst + b * block * block (leading dimension block).
+CLBH_API int clbh_invert_diagonal_blocks(int precision, int upper, int blocks, const void* src, long long src_ld,
+                                         void* dst, hipStream_t stream);
 
 // dst[dst_offset + two * dst_ld + one] = src[src_offset + two * src_ld + one] for one < one_extent, two < two_extent.
 CLBH_API int clbh_copy_matrix(int precision, int one_extent, int two_extent, const void* src, long long src_offset,

@@ -2,7 +2,7 @@
 // C++ interface of the MI355X (gfx950) GEMM engine behind the CLBlast GEMM API.
 //
 // The argument surface is the one of CLBlast's `include/clblast.h` (reference: Gemm :427-432,
-// GemmBatched :538-543, GemmStridedBatched :547-553, Symm :435-439, Syrk :449-453, Syr2k :463-467, Trmm :477-481, GemmTempBufferSize :558-562, StatusCode :61-129,
+// GemmBatched :538-543, GemmStridedBatched :547-553, Symm :435-439, Syrk :449-453, Syr2k :463-467, Trmm :477-481, Trsm :484-488, GemmTempBufferSize :558-562, StatusCode :61-129,
 // Layout/Transpose/Precision :132-147, OverrideParameters :620-624, ClearCache :568). Only the handle
 // types differ: `cl_mem` becomes a raw device pointer (`void*`, as returned by hipMalloc or
 // `tensor.data_ptr()`), `cl_command_queue*` becomes `hipStream_t*` and `cl_event*` becomes
@@ -164,6 +164,16 @@ StatusCode Syr2k(const Layout layout, const Triangle triangle, const Transpose a
 // that is `kUnit` (reference: include/clblast.h:477-481, src/routines/level3/xtrmm.cpp:33-130).
 template <typename T>
 StatusCode Trmm(const Layout layout, const Side side, const Triangle triangle, const Transpose a_transpose,
+                const Diagonal diagonal, const size_t m, const size_t n, const T alpha, const void* a_buffer,
+                const size_t a_offset, const size_t a_ld, void* b_buffer, const size_t b_offset, const size_t b_ld,
+                hipStream_t* queue, hipEvent_t* event = nullptr);
+
+// Solves a triangular system in place: B becomes the X with op(A) * X = alpha * B (side left, A is m x m) or
+// X * op(A) = alpha * B (side right, A is n x n); only the named triangle of A is read, and not its diagonal when
+// that is `kUnit`. T is float or double: like the reference this routine has no half-precision version (reference:
+// include/clblast.h:484-488, src/clblast.cpp:1339-1346, src/routines/level3/xtrsm.cpp:38-246).
+template <typename T>
+StatusCode Trsm(const Layout layout, const Side side, const Triangle triangle, const Transpose a_transpose,
                 const Diagonal diagonal, const size_t m, const size_t n, const T alpha, const void* a_buffer,
                 const size_t a_offset, const size_t a_ld, void* b_buffer, const size_t b_offset, const size_t b_ld,
                 hipStream_t* queue, hipEvent_t* event = nullptr);

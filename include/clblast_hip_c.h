@@ -184,6 +184,21 @@ CLBlastStatusCode CLBLAST_HIP_API CLBlastHtrmm(const CLBlastLayout layout, const
                                                const size_t a_ld, void* b_buffer, const size_t b_offset,
                                                const size_t b_ld, hipStream_t* queue, hipEvent_t* event);
 
+// Triangular solve in place: B becomes the X with op(A)*X = alpha*B (side left) or X*op(A) = alpha*B (side right)
+// replaces CLBlastStrsm/CLBlastDtrsm; like the reference there is no half-precision TRSM (reference: include/clblast_c.h:1094-1124, src/clblast_c.cpp:2402-2500)
+CLBlastStatusCode CLBLAST_HIP_API CLBlastStrsm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const CLBlastTranspose a_transpose,
+                                               const CLBlastDiagonal diagonal, const size_t m, const size_t n,
+                                               const float alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastDtrsm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const CLBlastTranspose a_transpose,
+                                               const CLBlastDiagonal diagonal, const size_t m, const size_t n,
+                                               const double alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, hipStream_t* queue, hipEvent_t* event);
+
 // =================================================================================================
 // Batched GEMM with per-batch alpha, beta and element offsets (host arrays of length batch_count)
 // replaces CLBlast{S,D,H}gemmBatched (reference: include/clblast_c.h:1303-1337, src/clblast_c.cpp:2723-2833)

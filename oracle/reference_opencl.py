@@ -118,8 +118,9 @@ def run(spec):
     a = oracle.uniform(seed * 3 + 0, sizes[0], ab_low, ab_high, bits)
     b = oracle.uniform(seed * 3 + 1, sizes[1], ab_low, ab_high, bits)
     c = oracle.uniform(seed * 3 + 2, sizes[2], spec.get("low", -1.0), spec.get("high", 1.0), bits)
-    if spec.get("a_diagonal_boost"):  # well-conditioned triangular solves: |diagonal| >= boost (tests do the same)
-        k_diag, boost = spec["k_diag"], spec["a_diagonal_boost"]
+    if spec.get("a_diagonal_boost"):  # well-conditioned triangular solves (tests/level3_harness.py does the same):
+        k_diag, boost = spec["k_diag"], spec["a_diagonal_boost"]  # off-diagonal row sums below 1, |diagonal| >= boost
+        a = (a.astype(np.float64) * (2.0 / k_diag)).astype(a.dtype)
         positions = spec["offsets"][0] + np.arange(k_diag) * (spec["a_ld"] + 1)
         a[positions] = a[positions] + np.where(a[positions] >= 0, boost, -boost).astype(a.dtype)
     a_buffer, b_buffer, c_buffer = opencl.buffer_from(a), opencl.buffer_from(b), opencl.buffer_from(c)

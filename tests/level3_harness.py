@@ -69,7 +69,8 @@ class TriangularProblem:
         self.a = oracle.uniform(seed * 3, self.sizes[0], ab_range[0], ab_range[1], bits)
         self.b = oracle.uniform(seed * 3 + 1, self.sizes[1], ab_range[0], ab_range[1], bits)
         diagonal_positions = offsets[0] + np.arange(self.k) * (self.a_ld + 1)
-        if routine == "trsm":  # keep the solve well conditioned
+        if routine == "trsm":  # keep the solve well conditioned: off-diagonal row sums below 1, |diagonal| >= 4
+            self.a = (self.a.astype(np.float64) * (2.0 / self.k)).astype(self.a.dtype)
             boost = np.where(self.a[diagonal_positions] >= 0, self.DIAGONAL_BOOST, -self.DIAGONAL_BOOST)
             self.a[diagonal_positions] = self.a[diagonal_positions] + boost.astype(self.a.dtype)
         self.a_clean = self.a.copy()
