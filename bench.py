@@ -358,8 +358,19 @@ def reference_on_this_gpu(runs=3):
                                                    sizes=[1024 * 8192] * 3),
              "ssymm_4096_colLeftUpper": dict(routine="symm", bits=32, layout=COL, side=141, triangle=121, m=4096, n=4096,
                                              k=4096, alpha=1.0, beta=0.0, a_ld=4096, b_ld=4096, c_ld=4096,
-                                             offsets=[0, 0, 0], seed=10, runs=5, sizes=[4096 * 4096] * 3)}
-    flops = {name: 2.0 * spec["m"] * spec["n"] * spec["k"] * spec.get("batch", 1) for name, spec in specs.items()}
+                                             offsets=[0, 0, 0], seed=10, runs=5, sizes=[4096 * 4096] * 3),
+             "ssyrk_4096_colLower": dict(routine="syrk", bits=32, layout=COL, triangle=122, ta=NO, m=4096, n=4096, k=4096,
+                                         alpha=1.0, beta=0.0, a_ld=4096, b_ld=4096, c_ld=4096, offsets=[0, 0, 0], seed=11,
+                                         runs=5, sizes=[4096 * 4096] * 3),
+             "strmm_4096_colLeftLower": dict(routine="trmm", bits=32, layout=COL, side=141, triangle=122, ta=NO, diagonal=131,
+                                             m=4096, n=4096, k=4096, alpha=1.0, a_ld=4096, b_ld=4096, offsets=[0, 0, 0],
+                                             seed=12, runs=5, sizes=[4096 * 4096] * 3),
+             "strsm_4096_colLeftLower": dict(routine="trsm", bits=32, layout=COL, side=141, triangle=122, ta=NO, diagonal=131,
+                                             m=4096, n=4096, k=4096, alpha=1.0, a_ld=4096, b_ld=4096, offsets=[0, 0, 0],
+                                             seed=13, runs=3, sizes=[4096 * 4096] * 3, a_diagonal_boost=4.0, k_diag=4096)}
+    half_count = ("ssyrk_4096_colLower", "strmm_4096_colLeftLower", "strsm_4096_colLeftLower")  # BLAS counts n*n*k, m*m*n
+    flops = {name: (1.0 if name in half_count else 2.0) * spec["m"] * spec["n"] * spec["k"] * spec.get("batch", 1)
+             for name, spec in specs.items()}
     root = os.path.dirname(os.path.abspath(__file__))
     with tempfile.TemporaryDirectory() as folder:
         spec_file, out_file = os.path.join(folder, "spec.json"), os.path.join(folder, "out.npz")
@@ -399,6 +410,8 @@ EXTRA_WORKLOADS = {
     "next_hsymm_4096_rowLeftLower": lambda: SymmWorkload("symm_h", "H", ROW, False, 4096, 4096, 1.0, 0.0),
     "next_strmm_4096_colLeftLower": lambda: TrmmWorkload("trmm_s", "S", "trmm", True, False, 4096, 4096),
     "next_dtrmm_4096_colLeftUpperT": lambda: TrmmWorkload("trmm_d", "D", "trmm", False, True, 4096, 4096),
+    "next_strsm_4096_colLeftLower": lambda: TrmmWorkload("trsm_s", "S", "trsm", True, False, 4096, 4096),
+    "next_dtrsm_4096_colLeftUpperT": lambda: TrmmWorkload("trsm_d", "D", "trsm", False, True, 4096, 4096),
     "next_ssyrk_4096_colLower": lambda: SyrkWorkload("syrk_s", "S", True, 4096, 4096),
     "next_hsyrk_8192_colUpper": lambda: SyrkWorkload("syrk_h", "H", False, 8192, 8192),
 }

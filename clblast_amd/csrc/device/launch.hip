@@ -139,15 +139,15 @@ int LaunchTriangularToSquare(const int upper, const int unit, const int k, const
 template <typename T, typename CT, int BLOCK>
 int LaunchInvertDiagonalBlocks(const int upper, const int blocks, const void* src, const long long src_ld, void* dst,
                                hipStream_t stream) {
-  constexpr size_t lds_bytes = size_t{2} * BLOCK * (BLOCK + 1) * sizeof(CT);
+  constexpr size_t lds_bytes = clbh::InvertLds<CT, BLOCK>::BYTES;
   auto kernel = clbh::InvertDiagonalBlocksKernel<T, CT, BLOCK>;
   if (lds_bytes > 48 * 1024) {
     static const hipError_t attribute_status = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (attribute_status != hipSuccess) { return static_cast<int>(attribute_status); }
   }
-  kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), lds_bytes, stream>>>(upper != 0, static_cast<const T*>(src),
-                                                                                  src_ld, static_cast<T*>(dst));
+  kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(clbh::kInvertThreads), lds_bytes, stream>>>(
+      upper != 0, static_cast<const T*>(src), src_ld, static_cast<T*>(dst));
   return static_cast<int>(hipGetLastError());
 }
 

@@ -65,49 +65,93 @@ __global__ __launch_bounds__(kCopyThreads) void CopyMatrixKernel(const int one_e
 
 // Inverts the BLOCK x BLOCK diagonal blocks of a dense triangular matrix (zeros in the other triangle; reference:
 // Xinvert, src/routines/levelx/xinvert.cpp:45-140 and src/kernels/level3/invert_diagonal_blocks_part1.opencl, which
-// invert 16 x 16 blocks and combine them by block products). One work-group per block, one thread per column of the
-// inverse: column j of the inverse of a lower triangular L is the solution of L x = e_j by forward substitution
-// (backward for an upper triangular matrix), computed in CT (fp32 for fp16 storage). The block and the growing
-// inverse live in LDS as [row][column] with one column per thread, so that no two lanes share a bank. src must
-// hold blocks * BLOCK rows and columns; block b of the result is dst[b * BLOCK * BLOCK + column * BLOCK + row].
+// invert 16 x 16 blocks and combine them by block products in several launches). One work-group of 256 threads per
+// block, everything in LDS and in CT (fp32 for fp16 storage):
+//   1. the 16 x 16 blocks on the diagonal are inverted by substitution, one thread per column of an inverse: column j
+//      of the inverse of a lower triangular L solves L x = e_j from the top (an upper triangular one from the bottom);
+//   2. the inverses are doubled in size until they fill the block: with R the rows and C the columns of the
+//      off-diagonal part of a pair of neighbouring inverted blocks, inverse(R, C) = -inverse(R, R) * A(R, C) *
+//      inverse(C, C), two small products per level in which every thread owns a few elements of the result.
+// LDS rows have an odd pitch, so that lanes walking down a column and lanes walking along a row both spread over
+// the banks. src must hold blocks * BLOCK rows and columns; block b of the result is the dense matrix at
+// dst + b * BLOCK * BLOCK with leading dimension BLOCK.
+constexpr int kInvertThreads = 256;
+constexpr int kInvertBase = 16;
+
+template <typename CT, int BLOCK>
+struct InvertLds {
+  static constexpr int PITCH = BLOCK + 1;
+  static constexpr int TEMP_PITCH = BLOCK / 2 + 1;
+  // the block, its inverse, and the intermediate product of a doubling step (at most BLOCK/2 squared per pair)
+  static constexpr size_t BYTES = (size_t{2} * BLOCK * PITCH + size_t{BLOCK / 2} * TEMP_PITCH) * sizeof(CT);
+};
+
 template <typename T, typename CT, int BLOCK>
-__global__ __launch_bounds__(BLOCK) void InvertDiagonalBlocksKernel(const bool upper, const T* __restrict__ src,
-                                                                    const long long src_ld, T* __restrict__ dst) {
-  constexpr int PITCH = BLOCK + 1;  // odd: the lanes of a row access and of a column access both spread over the banks
+__global__ __launch_bounds__(kInvertThreads) void InvertDiagonalBlocksKernel(const bool upper, const T* __restrict__ src,
+                                                                             const long long src_ld, T* __restrict__ dst) {
+  constexpr int PITCH = InvertLds<CT, BLOCK>::PITCH, TEMP_PITCH = InvertLds<CT, BLOCK>::TEMP_PITCH;
   extern __shared__ __attribute__((aligned(16))) unsigned char invert_lds[];
   CT* matrix = reinterpret_cast<CT*>(invert_lds);  // [row * PITCH + column]: element (row, column) of the block
   CT* inverse = matrix + BLOCK * PITCH;             // the same layout
-  const int j = threadIdx.x;
+  CT* temp = inverse + BLOCK * PITCH;               // [row * TEMP_PITCH + column] of the only pair of the last level,
+                                                    // smaller levels pack their pairs side by side along the columns
+  const int tid = threadIdx.x;
   const T* block = src + static_cast<long long>(blockIdx.x) * BLOCK * (src_ld + 1);
-  for (int column = 0; column < BLOCK; ++column) {  // lanes along a column of the source: contiguous addresses
-    matrix[j * PITCH + column] = static_cast<CT>(block[column * src_ld + j]);
+  for (int index = tid; index < BLOCK * BLOCK; index += kInvertThreads) {  // lanes along a column: contiguous addresses
+    const int row = index % BLOCK, column = index / BLOCK;
+    matrix[row * PITCH + column] = static_cast<CT>(block[column * src_ld + row]);
+    inverse[row * PITCH + column] = CT(0);
   }
   __syncthreads();
-  if (!upper) {
-    for (int row = 0; row < BLOCK; ++row) {
-      CT value = CT(0);
-      if (row >= j) {
+
+  // 1. substitution inside the 16 x 16 diagonal blocks
+  if (tid < BLOCK) {
+    const int first = (tid / kInvertBase) * kInvertBase, j = tid;  // the thread's base block and its column
+    if (!upper) {
+      for (int row = j; row < first + kInvertBase; ++row) {
         CT sum = (row == j) ? CT(1) : CT(0);
         for (int p = j; p < row; ++p) { sum -= matrix[row * PITCH + p] * inverse[p * PITCH + j]; }
-        value = sum / matrix[row * PITCH + row];
+        inverse[row * PITCH + j] = sum / matrix[row * PITCH + row];
       }
-      inverse[row * PITCH + j] = value;
-    }
-  } else {
-    for (int row = BLOCK - 1; row >= 0; --row) {
-      CT value = CT(0);
-      if (row <= j) {
+    } else {
+      for (int row = j; row >= first; --row) {
         CT sum = (row == j) ? CT(1) : CT(0);
         for (int p = row + 1; p <= j; ++p) { sum -= matrix[row * PITCH + p] * inverse[p * PITCH + j]; }
-        value = sum / matrix[row * PITCH + row];
+        inverse[row * PITCH + j] = sum / matrix[row * PITCH + row];
       }
-      inverse[row * PITCH + j] = value;
     }
   }
   __syncthreads();
+
+  // 2. doubling: size is the extent of the inverted diagonal blocks so far
+  for (int size = kInvertBase; size < BLOCK; size *= 2) {
+    const int elements = (BLOCK / (2 * size)) * size * size;  // off-diagonal elements of all pairs
+    // temp(R, C) = A(R, C) * inverse(C, C)
+    for (int index = tid; index < elements; index += kInvertThreads) {
+      const int pair = index / (size * size), r = index % size, c = (index / size) % size;
+      const int low = pair * 2 * size, high = low + size;
+      const int rows = upper ? low : high, columns = upper ? high : low;
+      CT sum = CT(0);
+      for (int p = 0; p < size; ++p) { sum += matrix[(rows + r) * PITCH + columns + p] * inverse[(columns + p) * PITCH + columns + c]; }
+      temp[r * TEMP_PITCH + pair * size + c] = sum;
+    }
+    __syncthreads();
+    // inverse(R, C) = -inverse(R, R) * temp(R, C)
+    for (int index = tid; index < elements; index += kInvertThreads) {
+      const int pair = index / (size * size), r = index % size, c = (index / size) % size;
+      const int low = pair * 2 * size, high = low + size;
+      const int rows = upper ? low : high, columns = upper ? high : low;
+      CT sum = CT(0);
+      for (int p = 0; p < size; ++p) { sum -= inverse[(rows + r) * PITCH + rows + p] * temp[p * TEMP_PITCH + pair * size + c]; }
+      inverse[(rows + r) * PITCH + columns + c] = sum;
+    }
+    __syncthreads();
+  }
+
   T* result = dst + static_cast<long long>(blockIdx.x) * BLOCK * BLOCK;
-  for (int column = 0; column < BLOCK; ++column) {
-    result[column * BLOCK + j] = static_cast<T>(inverse[j * PITCH + column]);
+  for (int index = tid; index < BLOCK * BLOCK; index += kInvertThreads) {
+    const int row = index % BLOCK, column = index / BLOCK;
+    result[column * BLOCK + row] = static_cast<T>(inverse[row * PITCH + column]);
   }
 }
 
