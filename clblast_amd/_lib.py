@@ -17,8 +17,22 @@ _lib = None
 _SCALAR = {"S": c_float, "D": c_double, "H": c_ushort}
 
 
+class Float2(ctypes.Structure):
+    """CLBlastFloat2: a complex scalar passed by value."""
+    _fields_ = [("x", ctypes.c_float), ("y", ctypes.c_float)]
+
+
+class Double2(ctypes.Structure):
+    """CLBlastDouble2: a complex scalar passed by value."""
+    _fields_ = [("x", ctypes.c_double), ("y", ctypes.c_double)]
+
+
 def _declare(lib):
     sz, vp = c_size_t, c_void_p
+    for prefix, scalar in (("C", Float2), ("Z", Double2)):
+        f = getattr(lib, "CLBlast%sgemm" % prefix)
+        f.argtypes = [c_int, c_int, c_int, sz, sz, sz, scalar, vp, sz, sz, vp, sz, sz, scalar, vp, sz, sz, vp, vp]
+        f.restype = c_int
     for prefix, scalar in _SCALAR.items():
         gemm_args = [c_int, c_int, c_int, sz, sz, sz, scalar, vp, sz, sz, vp, sz, sz, scalar, vp, sz, sz, vp, vp]
         f = getattr(lib, "CLBlast%sgemm" % prefix)
@@ -73,10 +87,10 @@ def load():
 # Every symbol the public C headers declare, for the export test.
 C_API_SYMBOLS = (
     ["CLBlast%sgemm%s" % (p, s) for p in "SDH" for s in ("", "Batched", "StridedBatched", "WithTempBuffer")] +
-    ["CLBlast%sGemmTempBufferSize" % p for p in "SDH"] + ["CLBlast%ssymm" % p for p in "SDH"] + ["CLBlast%strmm" % p for p in "SDH"] + ["CLBlast%strsm" % p for p in "SD"] + ["CLBlast%ssyrk" % p for p in "SDH"] +
+    ["CLBlast%sGemmTempBufferSize" % p for p in "SDH"] + ["CLBlastCgemm", "CLBlastZgemm"] + ["CLBlast%ssymm" % p for p in "SDH"] + ["CLBlast%strmm" % p for p in "SDH"] + ["CLBlast%strsm" % p for p in "SD"] + ["CLBlast%ssyrk" % p for p in "SDH"] +
     ["CLBlast%ssyr2k" % p for p in "SDH"] +
     ["CLBlastClearCache", "CLBlastOverrideParameters", "CLBlastFloatToHalf", "CLBlastHalfToFloat"])
 DEVICE_LAYER_SYMBOLS = [
     "clbh_gemm_launch", "clbh_gemm_workspace_bytes", "clbh_buffer_extent", "clbh_alloc_async", "clbh_free_async",
     "clbh_upload_async", "clbh_event_record", "clbh_stream_device", "clbh_error_string", "clbh_symmetric_to_square", "clbh_triangular_to_square", "clbh_copy_matrix", "clbh_invert_block_size",
-                        "clbh_invert_diagonal_blocks"]
+                        "clbh_invert_diagonal_blocks", "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale"]

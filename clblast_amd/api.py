@@ -50,7 +50,7 @@ def half_bits_to_float(bits):
 
 def _prefix_of(dtype_name):
     try:
-        return {"float32": "S", "float64": "D", "float16": "H"}[dtype_name]
+        return {"float32": "S", "float64": "D", "float16": "H", "complex64": "C", "complex128": "Z"}[dtype_name]
     except KeyError:
         raise ValueError("PyCLBlast: unrecognized data-type '%s'" % dtype_name)
 
@@ -75,6 +75,19 @@ def raw_gemm(prefix, layout, a_transpose, b_transpose, m, n, k, alpha, a_ptr, a_
     if temp_ptr is None:
         return getattr(lib, "CLBlast%sgemm" % prefix)(*args)
     return getattr(lib, "CLBlast%sgemmWithTempBuffer" % prefix)(*(args + [temp_ptr]))
+
+
+def raw_complex_gemm(prefix, layout, a_transpose, b_transpose, m, n, k, alpha, a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld,
+                     beta, c_ptr, c_offset, c_ld, stream_handle=0, event_handle=None):
+    """CLBlastCgemm ("C", complex64 data) / CLBlastZgemm ("Z", complex128) through the C ABI (reference:
+    include/clblast_c.h:899-912); alpha and beta are Python complex numbers."""
+    lib = _lib.load()
+    scalar = _lib.Float2 if prefix == "C" else _lib.Double2
+    alpha, beta = complex(alpha), complex(beta)
+    event_ref = None if event_handle is None else ctypes.byref(ctypes.c_void_p(event_handle))
+    return getattr(lib, "CLBlast%sgemm" % prefix)(layout, a_transpose, b_transpose, m, n, k, scalar(alpha.real, alpha.imag),
+                                                  a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld, scalar(beta.real, beta.imag),
+                                                  c_ptr, c_offset, c_ld, _stream_ref(stream_handle), event_ref)
 
 
 def raw_symm(prefix, layout, side, triangle, m, n, alpha, a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld, beta, c_ptr,
@@ -199,9 +212,10 @@ def gemm(queue, m, n, k, a, b, c, a_ld, b_ld, c_ld, alpha=1.0, beta=0.0, a_trans
          b_offset=0, c_offset=0):
     """xGEMM: General matrix-matrix multiplication (row-major, like pyclblast.gemm)."""
     prefix = _tensor_info(a, b, c)
-    status = raw_gemm(prefix, ROW_MAJOR, TRANS_YES if a_transp else TRANS_NO, TRANS_YES if b_transp else TRANS_NO, m,
-                      n, k, alpha, a.data_ptr(), a_offset, a_ld, b.data_ptr(), b_offset, b_ld, beta, c.data_ptr(),
-                      c_offset, c_ld, _stream_handle(queue))
+    call = raw_complex_gemm if prefix in "CZ" else raw_gemm
+    status = call(prefix, ROW_MAJOR, TRANS_YES if a_transp else TRANS_NO, TRANS_YES if b_transp else TRANS_NO, m,
+                  n, k, alpha, a.data_ptr(), a_offset, a_ld, b.data_ptr(), b_offset, b_ld, beta, c.data_ptr(),
+                  c_offset, c_ld, _stream_handle(queue))
     if status != 0:
         raise CLBlastError("CLBlast%sgemm" % prefix, status)
 

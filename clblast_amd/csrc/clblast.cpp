@@ -9,6 +9,7 @@
 
 #include "clblast_hip.h"
 #include "routines/xgemm.hpp"
+#include "routines/xgemm_complex.hpp"
 #include "routines/xgemmbatched.hpp"
 #include "routines/xsymm.hpp"
 #include "routines/xsyrk.hpp"
@@ -214,6 +215,45 @@ CLBLAST_HIP_INSTANTIATE(half)
 CLBLAST_HIP_INSTANTIATE(float)
 CLBLAST_HIP_INSTANTIATE(double)
 #undef CLBLAST_HIP_INSTANTIATE
+
+// CGEMM and ZGEMM (reference: src/clblast.cpp:1093-1100)
+template <typename R>
+StatusCode ComplexGemm(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
+                       const size_t n, const size_t k, const std::complex<R> alpha, const void* a_buffer,
+                       const size_t a_offset, const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                       const size_t b_ld, const std::complex<R> beta, void* c_buffer, const size_t c_offset,
+                       const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {
+  try {
+    using Complex = std::complex<R>;
+    auto routine = XgemmComplex<R>(queue, event);
+    routine.DoGemm(layout, a_transpose, b_transpose, m, n, k, alpha, Buffer<Complex>(a_buffer), a_offset, a_ld,
+                   Buffer<Complex>(b_buffer), b_offset, b_ld, beta, Buffer<Complex>(c_buffer), c_offset, c_ld);
+    return StatusCode::kSuccess;
+  } catch (...) {
+    return DispatchException();
+  }
+}
+template <>
+StatusCode CLBLAST_HIP_PUBLIC Gemm<float2>(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
+                                           const size_t m, const size_t n, const size_t k, const float2 alpha,
+                                           const void* a_buffer, const size_t a_offset, const size_t a_ld,
+                                           const void* b_buffer, const size_t b_offset, const size_t b_ld, const float2 beta,
+                                           void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                                           hipEvent_t* event, void*) {
+  return ComplexGemm<float>(layout, a_transpose, b_transpose, m, n, k, alpha, a_buffer, a_offset, a_ld, b_buffer, b_offset,
+                            b_ld, beta, c_buffer, c_offset, c_ld, queue, event);
+}
+template <>
+StatusCode CLBLAST_HIP_PUBLIC Gemm<double2>(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
+                                            const size_t m, const size_t n, const size_t k, const double2 alpha,
+                                            const void* a_buffer, const size_t a_offset, const size_t a_ld,
+                                            const void* b_buffer, const size_t b_offset, const size_t b_ld,
+                                            const double2 beta, void* c_buffer, const size_t c_offset, const size_t c_ld,
+                                            hipStream_t* queue, hipEvent_t* event, void*) {
+  return ComplexGemm<double>(layout, a_transpose, b_transpose, m, n, k, alpha, a_buffer, a_offset, a_ld, b_buffer, b_offset,
+                             b_ld, beta, c_buffer, c_offset, c_ld, queue, event);
+}
+
 // TRSM exists for float and double only (reference: src/clblast.cpp:1339-1346)
 template StatusCode CLBLAST_HIP_PUBLIC Trsm<float>(const Layout, const Side, const Triangle, const Transpose, const Diagonal,
                                                    const size_t, const size_t, const float, const void*, const size_t,

@@ -9,6 +9,7 @@
 
 #include "device/launch_common.hpp"
 #include "kernels/symmetric_to_square.hpp"
+#include "kernels/complex_helpers.hpp"
 #include "kernels/triangular_to_square.hpp"
 
 namespace clbh {
@@ -171,6 +172,41 @@ int LaunchCopyMatrix(const int one, const int two, const void* src, const long l
 }
 }  // namespace
 
+namespace {
+unsigned Blocks(const int extent, const int per_block) { return static_cast<unsigned>((extent + per_block - 1) / per_block); }
+
+template <typename R>
+int LaunchComplexExpand(const int m, const int k, const int kcontig, const int conjugate, const int conjugated_b,
+                        const double alpha_re, const double alpha_im, const void* src, const long long src_offset,
+                        const long long src_ld, void* dst, hipStream_t stream) {
+  const dim3 grid(Blocks(m, clbh::kComplexTile), Blocks(k, clbh::kComplexTile));
+  if (grid.y > 65535) { return hipErrorInvalidConfiguration; }
+  clbh::ExpandComplexKernel<R><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
+      m, k, kcontig != 0, conjugate != 0, conjugated_b != 0, static_cast<R>(alpha_re), static_cast<R>(alpha_im),
+      static_cast<const clbh::ComplexOf<R>*>(src) + src_offset, src_ld, static_cast<R*>(dst));
+  return static_cast<int>(hipGetLastError());
+}
+
+template <typename R>
+int LaunchComplexTranspose(const int k, const int n, const void* src, const long long src_offset, const long long src_ld,
+                           void* dst, hipStream_t stream) {
+  const dim3 grid(Blocks(k, clbh::kComplexTile), Blocks(n, clbh::kComplexTile));
+  if (grid.y > 65535) { return hipErrorInvalidConfiguration; }
+  clbh::TransposeComplexKernel<R><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
+      k, n, static_cast<const clbh::ComplexOf<R>*>(src) + src_offset, src_ld, static_cast<clbh::ComplexOf<R>*>(dst));
+  return static_cast<int>(hipGetLastError());
+}
+
+template <typename R>
+int LaunchComplexScale(const int m, const int n, const double beta_re, const double beta_im, void* c,
+                       const long long c_offset, const long long c_ld, hipStream_t stream) {
+  const dim3 grid(Blocks(m, clbh::kComplexThreads), static_cast<unsigned>(std::min(n, 16384)));
+  clbh::ScaleComplexKernel<R><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
+      m, n, static_cast<R>(beta_re), static_cast<R>(beta_im), static_cast<clbh::ComplexOf<R>*>(c) + c_offset, c_ld);
+  return static_cast<int>(hipGetLastError());
+}
+}  // namespace
+
 extern "C" {
 
 int clbh_gemm_launch(const clbh_gemm_desc* desc, hipStream_t stream) {
@@ -236,6 +272,37 @@ int clbh_copy_matrix(int precision, int one_extent, int two_extent, const void* 
     case 64: return LaunchCopyMatrix<double>(one_extent, two_extent, src, src_offset, src_ld, dst, dst_offset, dst_ld, stream);
     default: return hipErrorInvalidValue;
   }
+}
+
+int clbh_complex_expand(int precision, int m, int k, int kcontig, int conjugate, int conjugated_b, double alpha_re,
+                        double alpha_im, const void* src, long long src_offset, long long src_ld, void* dst,
+                        hipStream_t stream) {
+  if (m <= 0 || k <= 0 || src == nullptr || dst == nullptr || src_offset < 0 || src_ld < (kcontig ? k : m)) {
+    return hipErrorInvalidValue;
+  }
+  if (precision == 32) {
+    return LaunchComplexExpand<float>(m, k, kcontig, conjugate, conjugated_b, alpha_re, alpha_im, src, src_offset, src_ld, dst, stream);
+  }
+  if (precision == 64) {
+    return LaunchComplexExpand<double>(m, k, kcontig, conjugate, conjugated_b, alpha_re, alpha_im, src, src_offset, src_ld, dst, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+int clbh_complex_transpose(int precision, int k, int n, const void* src, long long src_offset, long long src_ld, void* dst,
+                           hipStream_t stream) {
+  if (k <= 0 || n <= 0 || src == nullptr || dst == nullptr || src_offset < 0 || src_ld < n) { return hipErrorInvalidValue; }
+  if (precision == 32) { return LaunchComplexTranspose<float>(k, n, src, src_offset, src_ld, dst, stream); }
+  if (precision == 64) { return LaunchComplexTranspose<double>(k, n, src, src_offset, src_ld, dst, stream); }
+  return hipErrorInvalidValue;
+}
+
+int clbh_complex_scale(int precision, int m, int n, double beta_re, double beta_im, void* c, long long c_offset,
+                       long long c_ld, hipStream_t stream) {
+  if (m <= 0 || n <= 0 || c == nullptr || c_offset < 0 || c_ld < m) { return hipErrorInvalidValue; }
+  if (precision == 32) { return LaunchComplexScale<float>(m, n, beta_re, beta_im, c, c_offset, c_ld, stream); }
+  if (precision == 64) { return LaunchComplexScale<double>(m, n, beta_re, beta_im, c, c_offset, c_ld, stream); }
+  return hipErrorInvalidValue;
 }
 
 int clbh_buffer_extent(const void* ptr, size_t* bytes_available) {

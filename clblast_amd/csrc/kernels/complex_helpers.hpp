@@ -1,0 +1,111 @@
+// =================================================================================================
+// Helper kernels of the complex GEMM (CGEMM/ZGEMM; reference: the complex paths of src/kernels/common.opencl:
+// 76-105, 202-251 and of the Xgemm kernels). A complex product is four real products, and the matrix cores of
+// gfx950 multiply real matrices, so the complex GEMM is run as ONE real GEMM of twice the size in m and k: with
+// interleaved (re, im) storage a column-major complex m x n matrix IS a real 2m x n matrix, a complex k x n operand
+// whose k index is contiguous IS a real 2k x n matrix, and only the first operand has to be rewritten, every
+// element a (times alpha, conjugated if asked) as the 2 x 2 block
+//     [ re(a)  -im(a) ]                               [ re(a)   im(a) ]
+//     [ im(a)   re(a) ]   or, for a conjugated B,     [ im(a)  -re(a) ]
+// so that block * (re(b), im(b))^T = (re(a b), im(a b))^T resp. (re(a conj(b)), im(a conj(b)))^T.
+//
+// ExpandComplexKernel     A (m x k complex, either orientation) -> real 2m x 2k, column-major, dense
+// TransposeComplexKernel  B (k x n complex with n contiguous) -> k x n with k contiguous, dense
+// ScaleComplexKernel      C := beta * C for a complex beta (the real GEMM's epilogue only knows real factors)
+// All three are HBM bound; the two that change orientation go through a 32 x 32 LDS tile so that reads and writes
+// both run along contiguous addresses.
+// =================================================================================================
+#ifndef CLBLAST_HIP_KERNELS_COMPLEX_HELPERS_HPP_
+#define CLBLAST_HIP_KERNELS_COMPLEX_HELPERS_HPP_
+
+#include <hip/hip_runtime.h>
+
+namespace clbh {
+
+constexpr int kComplexTile = 32;
+constexpr int kComplexThreads = 256;
+
+template <typename R>
+struct ComplexOf {
+  R re, im;
+};
+
+// src: A(i, p) at src[(kcontig ? i * src_ld + p : p * src_ld + i)], i < m, p < k. dst: real, column-major, leading
+// dimension 2 * m. grid: (ceil(m / 32), ceil(k / 32)).
+template <typename R>
+__global__ __launch_bounds__(kComplexThreads) void ExpandComplexKernel(const int m, const int k, const bool kcontig,
+                                                                       const bool conjugate, const bool conjugated_b,
+                                                                       const R alpha_re, const R alpha_im,
+                                                                       const ComplexOf<R>* __restrict__ src,
+                                                                       const long long src_ld, R* __restrict__ dst) {
+  __shared__ ComplexOf<R> tile[kComplexTile][kComplexTile + 1];  // [p][i]
+  const int i0 = blockIdx.x * kComplexTile, p0 = blockIdx.y * kComplexTile;
+  const int fast = threadIdx.x % kComplexTile, slow = threadIdx.x / kComplexTile;
+  for (int step = slow; step < kComplexTile; step += kComplexThreads / kComplexTile) {
+    // lanes run along the contiguous index of the source
+    const int i = i0 + (kcontig ? step : fast), p = p0 + (kcontig ? fast : step);
+    if (i < m && p < k) {
+      const ComplexOf<R> value = src[kcontig ? i * src_ld + p : p * src_ld + i];
+      tile[p - p0][i - i0] = value;
+    }
+  }
+  __syncthreads();
+  const long long dst_ld = 2LL * m;
+  for (int step = slow; step < kComplexTile; step += kComplexThreads / kComplexTile) {
+    const int i = i0 + fast, p = p0 + step;  // lanes run along i: contiguous in both columns of the result
+    if (i < m && p < k) {
+      ComplexOf<R> a = tile[step][fast];
+      if (conjugate) { a.im = -a.im; }
+      const R re = alpha_re * a.re - alpha_im * a.im, im = alpha_re * a.im + alpha_im * a.re;
+      typedef R Pair __attribute__((ext_vector_type(2)));
+      Pair first, second;
+      first[0] = re;
+      first[1] = im;
+      second[0] = conjugated_b ? im : -im;
+      second[1] = conjugated_b ? -re : re;
+      *reinterpret_cast<Pair*>(dst + (2LL * p) * dst_ld + 2 * i) = first;
+      *reinterpret_cast<Pair*>(dst + (2LL * p + 1) * dst_ld + 2 * i) = second;
+    }
+  }
+}
+
+// src: B(p, j) at src[p * src_ld + j] (j contiguous), p < k, j < n. dst: B(p, j) at dst[j * k + p].
+// grid: (ceil(k / 32), ceil(n / 32)).
+template <typename R>
+__global__ __launch_bounds__(kComplexThreads) void TransposeComplexKernel(const int k, const int n,
+                                                                          const ComplexOf<R>* __restrict__ src,
+                                                                          const long long src_ld,
+                                                                          ComplexOf<R>* __restrict__ dst) {
+  __shared__ ComplexOf<R> tile[kComplexTile][kComplexTile + 1];  // [p][j]
+  const int p0 = blockIdx.x * kComplexTile, j0 = blockIdx.y * kComplexTile;
+  const int fast = threadIdx.x % kComplexTile, slow = threadIdx.x / kComplexTile;
+  for (int step = slow; step < kComplexTile; step += kComplexThreads / kComplexTile) {
+    const int p = p0 + step, j = j0 + fast;
+    if (p < k && j < n) { tile[step][fast] = src[p * src_ld + j]; }
+  }
+  __syncthreads();
+  for (int step = slow; step < kComplexTile; step += kComplexThreads / kComplexTile) {
+    const int p = p0 + fast, j = j0 + step;
+    if (p < k && j < n) { dst[static_cast<long long>(j) * k + p] = tile[fast][step]; }
+  }
+}
+
+// c: C(i, j) at c[j * c_ld + i], i < m, j < n. grid: (ceil(m / 256), min(n, 16384)).
+template <typename R>
+__global__ __launch_bounds__(kComplexThreads) void ScaleComplexKernel(const int m, const int n, const R beta_re,
+                                                                      const R beta_im, ComplexOf<R>* __restrict__ c,
+                                                                      const long long c_ld) {
+  const int i = blockIdx.x * kComplexThreads + threadIdx.x;
+  if (i >= m) { return; }
+  for (int j = blockIdx.y; j < n; j += gridDim.y) {
+    const ComplexOf<R> old = c[j * c_ld + i];
+    ComplexOf<R> scaled;
+    scaled.re = beta_re * old.re - beta_im * old.im;
+    scaled.im = beta_re * old.im + beta_im * old.re;
+    c[j * c_ld + i] = scaled;
+  }
+}
+
+}  // namespace clbh
+
+#endif  // CLBLAST_HIP_KERNELS_COMPLEX_HELPERS_HPP_

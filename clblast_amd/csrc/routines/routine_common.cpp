@@ -130,6 +130,8 @@ void TestMatrixC(const size_t one, const size_t two, const Buffer<T>& buffer, co
 CLBLAST_HIP_INSTANTIATE(half)
 CLBLAST_HIP_INSTANTIATE(float)
 CLBLAST_HIP_INSTANTIATE(double)
+CLBLAST_HIP_INSTANTIATE(float2)
+CLBLAST_HIP_INSTANTIATE(double2)
 #undef CLBLAST_HIP_INSTANTIATE
 
 // =================================================================================================

@@ -1,0 +1,36 @@
+// =================================================================================================
+// XgemmComplex<R>: host logic of Gemm<std::complex<R>> (CGEMM, ZGEMM), C = alpha * op(A) * op(B) + beta * C with
+// op(X) = X, X^T or X^H (reference: the float2/double2 instantiations of src/routines/level3/xgemm.{hpp,cpp} and the
+// complex arithmetic of src/kernels/common.opencl:76-105, 202-251).
+//
+// The argument checks are those of the real GEMM with complex element sizes. The product itself runs as one real
+// GEMM of shape 2m x n x 2k on the MFMA kernels (kernels/complex_helpers.hpp explains the 2 x 2 block form): the
+// first operand of the canonical problem is expanded into a real temporary (alpha, its transpose and both
+// conjugations are folded into that pass), the second one is used in place when its k index is contiguous and
+// transposed into a temporary otherwise, and C is used in place. A beta with an imaginary part costs one more pass
+// over C.
+// =================================================================================================
+#ifndef CLBLAST_HIP_ROUTINES_XGEMM_COMPLEX_HPP_
+#define CLBLAST_HIP_ROUTINES_XGEMM_COMPLEX_HPP_
+
+#include <complex>
+
+#include "routines/xgemm.hpp"
+
+namespace clblast {
+
+template <typename R>
+class XgemmComplex : public Xgemm<R> {
+ public:
+  using Complex = std::complex<R>;
+  XgemmComplex(hipStream_t* queue, hipEvent_t* event);
+  void DoGemm(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
+              const size_t n, const size_t k, const Complex alpha, const Buffer<Complex>& a_buffer,
+              const size_t a_offset, const size_t a_ld, const Buffer<Complex>& b_buffer, const size_t b_offset,
+              const size_t b_ld, const Complex beta, const Buffer<Complex>& c_buffer, const size_t c_offset,
+              const size_t c_ld);
+};
+
+}  // namespace clblast
+
+#endif  // CLBLAST_HIP_ROUTINES_XGEMM_COMPLEX_HPP_

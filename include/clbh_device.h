@@ -105,6 +105,21 @@ CLBH_API int clbh_invert_diagonal_blocks(int precision, int upper, int blocks, c
 CLBH_API int clbh_copy_matrix(int precision, int one_extent, int two_extent, const void* src, long long src_offset,
                               long long src_ld, void* dst, long long dst_offset, long long dst_ld, hipStream_t stream);
 
+// ---- complex GEMM helpers: precision is the width of ONE component, 32 (float2 data) or 64 (double2); offsets and
+// leading dimensions count complex elements --------------------------------------------------------------------
+// dst (real, column-major 2m x 2k, dense) = alpha * A (conjugated if `conjugate`) with every element as a 2 x 2 real
+// block (the block form for a conjugated second operand if `conjugated_b`); A(i,p) at
+// src[src_offset + (kcontig ? i*src_ld + p : p*src_ld + i)].
+CLBH_API int clbh_complex_expand(int precision, int m, int k, int kcontig, int conjugate, int conjugated_b,
+                                 double alpha_re, double alpha_im, const void* src, long long src_offset,
+                                 long long src_ld, void* dst, hipStream_t stream);
+// dst[j*k + p] = src[src_offset + p*src_ld + j] for p < k, j < n (complex elements).
+CLBH_API int clbh_complex_transpose(int precision, int k, int n, const void* src, long long src_offset,
+                                    long long src_ld, void* dst, hipStream_t stream);
+// C(i,j) *= beta for i < m, j < n; C(i,j) at c[c_offset + j*c_ld + i].
+CLBH_API int clbh_complex_scale(int precision, int m, int n, double beta_re, double beta_im, void* c,
+                                long long c_offset, long long c_ld, hipStream_t stream);
+
 // Number of bytes addressable from `ptr` to the end of the device allocation that contains it.
 // Returns 0 on success, non-zero if `ptr` is not inside a device allocation.
 CLBH_API int clbh_buffer_extent(const void* ptr, size_t* bytes_available);

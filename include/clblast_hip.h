@@ -17,6 +17,7 @@
 #ifndef CLBLAST_HIP_H_
 #define CLBLAST_HIP_H_
 
+#include <complex>
 #include <cstddef>
 #include <string>
 #include <unordered_map>
@@ -105,10 +106,14 @@ enum class Precision { kHalf = 16, kSingle = 32, kDouble = 64, kComplexSingle = 
 
 // Host type of fp16 scalars and data: the IEEE binary16 bit pattern (reference: clblast_half.h:21).
 using half = unsigned short;
+// Complex scalars and data, interleaved (real, imaginary) (reference: src/utilities/utilities.hpp:33-35).
+using float2 = std::complex<float>;
+using double2 = std::complex<double>;
 
 // =================================================================================================
 
-// C = alpha * op(A) * op(B) + beta * C. T is float, double or half.
+// C = alpha * op(A) * op(B) + beta * C. T is float, double, half, float2 or double2 (the complex types take no
+// temp_buffer; the batched routines exist for the real types only).
 template <typename T>
 StatusCode Gemm(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
                 const size_t n, const size_t k, const T alpha, const void* a_buffer, const size_t a_offset,

@@ -64,6 +64,9 @@ typedef enum CLBlastTranspose_ {
   CLBlastTransposeYes = 112,
   CLBlastTransposeConjugate = 113
 } CLBlastTranspose;
+// Complex scalars by value, (real, imaginary): stand in for cl_float2 / cl_double2 of the reference's C API
+typedef struct CLBlastFloat2_ { float x; float y; } CLBlastFloat2;
+typedef struct CLBlastDouble2_ { double x; double y; } CLBlastDouble2;
 typedef enum CLBlastTriangle_ { CLBlastTriangleUpper = 121, CLBlastTriangleLower = 122 } CLBlastTriangle;
 typedef enum CLBlastDiagonal_ { CLBlastDiagonalNonUnit = 131, CLBlastDiagonalUnit = 132 } CLBlastDiagonal;
 typedef enum CLBlastSide_ { CLBlastSideLeft = 141, CLBlastSideRight = 142 } CLBlastSide;
@@ -96,6 +99,24 @@ CLBlastStatusCode CLBLAST_HIP_API CLBlastHgemm(const CLBlastLayout layout, const
                                                const size_t k, const cl_half alpha, const void* a_buffer,
                                                const size_t a_offset, const size_t a_ld, const void* b_buffer,
                                                const size_t b_offset, const size_t b_ld, const cl_half beta,
+                                               void* c_buffer, const size_t c_offset, const size_t c_ld,
+                                               hipStream_t* queue, hipEvent_t* event);
+
+// =================================================================================================
+// Complex general matrix-matrix multiplication, data interleaved (real, imaginary); CLBlastTransposeConjugate is the
+// conjugate transpose. replaces CLBlastCgemm/CLBlastZgemm (reference: include/clblast_c.h:899-912, src/clblast_c.cpp:1822-1850)
+CLBlastStatusCode CLBLAST_HIP_API CLBlastCgemm(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                               const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                               const size_t k, const CLBlastFloat2 alpha, const void* a_buffer,
+                                               const size_t a_offset, const size_t a_ld, const void* b_buffer,
+                                               const size_t b_offset, const size_t b_ld, const CLBlastFloat2 beta,
+                                               void* c_buffer, const size_t c_offset, const size_t c_ld,
+                                               hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastZgemm(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                               const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                               const size_t k, const CLBlastDouble2 alpha, const void* a_buffer,
+                                               const size_t a_offset, const size_t a_ld, const void* b_buffer,
+                                               const size_t b_offset, const size_t b_ld, const CLBlastDouble2 beta,
                                                void* c_buffer, const size_t c_offset, const size_t c_ld,
                                                hipStream_t* queue, hipEvent_t* event);
 

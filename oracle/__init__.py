@@ -63,6 +63,8 @@ def lib():
         handle.oracle_syr2k.restype = ci
         handle.oracle_syr2k_status.argtypes = [ci, ci, ci] + [sz] * 11
         handle.oracle_syr2k_status.restype = ci
+        handle.oracle_complex_gemm.argtypes = [ci, ci, ci, ci, sz, sz, sz, dbl, dbl, vp, sz, sz, vp, sz, sz, dbl, dbl, vp, sz, sz, vp]
+        handle.oracle_complex_gemm.restype = ci
         handle.oracle_process_arguments.argtypes = [ci, ci, ci, sz, sz, sz, ctypes.POINTER(Shape)]
         handle.oracle_process_arguments.restype = ci
         handle.oracle_gemm_status.argtypes = [ci, ci, ci, ci] + [sz] * 12
@@ -174,6 +176,28 @@ def symm_numpy(layout, side, triangle, m, n, alpha, a, a_offset, a_ld, b, b_offs
     c_full = c[c_offset + (q * c_ld + r if col_major else r * c_ld + q)].astype(np.float64)
     product = full @ b_full if side == LEFT else b_full @ full
     return alpha * product + (beta * c_full if beta != 0 else 0.0)
+
+
+def complex_gemm(layout, a_transpose, b_transpose, m, n, k, alpha, a, a_offset, a_ld, b, b_offset, b_ld, beta, c, c_offset,
+                 c_ld):
+    """New logical C (m x n, complex128, unrounded) of CGEMM/ZGEMM by the C oracle; a, b, c are flat complex64 or
+    complex128 numpy buffers, offsets and leading dimensions count complex elements."""
+    assert a.dtype == b.dtype == c.dtype and a.dtype in (np.complex64, np.complex128)
+    component_bits = 32 if a.dtype == np.complex64 else 64
+    a, b, c = np.ascontiguousarray(a), np.ascontiguousarray(b), np.ascontiguousarray(c)
+    result = np.empty((m, n), dtype=np.complex128)
+    alpha, beta = complex(alpha), complex(beta)
+    status = lib().oracle_complex_gemm(component_bits, layout, a_transpose, b_transpose, m, n, k, alpha.real, alpha.imag,
+                                       a.ctypes.data, a_offset, a_ld, b.ctypes.data, b_offset, b_ld, beta.real, beta.imag,
+                                       c.ctypes.data, c_offset, c_ld, result.ctypes.data)
+    if status != 0:
+        raise ValueError("oracle_complex_gemm status %d" % status)
+    return result
+
+
+def complex_uniform(seed, count, low, high, component_bits):
+    """`count` complex numbers whose 2 * count components are uniform(seed, ...) of that width, interleaved."""
+    return uniform(seed, 2 * count, low, high, component_bits).view(np.complex64 if component_bits == 32 else np.complex128)
 
 
 NON_UNIT, UNIT = 131, 132

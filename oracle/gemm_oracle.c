@@ -31,6 +31,7 @@
  *                              acc += a*b in the storage precision) and copy/transpose C back. This is
  *                              the "port" CPU baseline, parallelised over tiles with OpenMP.
  *
+ *   oracle_complex_gemm        CGEMM/ZGEMM from the definition, complex multiply-add in long double
  *   oracle_symm, oracle_trmm,  the Level-3 routines the reference builds on its GEMM (src/routines/level3/xsymm.cpp,
  *   oracle_trsm, oracle_syr2k  xtrmm.cpp, xtrsm.cpp, xsyrk.cpp, xsyr2k.cpp) stated from their definitions in long
  *   and their *_status         double arithmetic, with the check order of those files.
@@ -45,6 +46,8 @@
  *   - status functions (gemm, batched, strided-batched): against the status codes the real reference
  *     library returns for a validation sweep per precision (1000 + 455 + 430 cases), executed on an
  *     OpenCL device (tests/test_reference_opencl_gpu.py).
+ *   - oracle_complex_gemm: against numpy complex128 matmul with .T / .conj().T, and the real reference library
+ *     (CLBlastCgemm/Zgemm) on an OpenCL device (tests/test_complex_gemm.py, tests/test_complex_gemm_gpu.py).
  *   - symm/trmm/trsm/syrk/syr2k: against independent numpy statements, the BLAS routines of scipy
  *     (dsymm, dtrmm, dtrsm, dsyrk, dsyr2k), algebraic identities, and the real reference library on an OpenCL
  *     device, status codes included (tests/test_level3_oracle.py, tests/test_symm_oracle.py, tests/test_*_gpu.py).
@@ -562,6 +565,52 @@ EXPORT int oracle_syr2k_status(int bits, int layout, int transpose, size_t n, si
   status = test_matrix(one, two, b_bytes, b_offset, b_ld, eb, 1, kInvalidLeadDimB, kInsufficientMemoryB);
   if (status != kSuccess) return status;
   return test_matrix(n, n, c_bytes, c_offset, c_ld, eb, 1, kInvalidLeadDimC, kInsufficientMemoryC);
+}
+
+/* ---- complex GEMM (CGEMM, ZGEMM) ------------------------------------------------------------------ */
+
+/* C = alpha * op(A) * op(B) + beta * C for interleaved (re, im) data of `component_bits` (32 or 64) per component;
+ * op is identity, transpose or conjugate transpose (src/routines/level3/xgemm.hpp:87-107 for the indexing,
+ * src/kernels/common.opencl:202-251 for the complex multiply-add and the conjugation). Offsets and leading
+ * dimensions count complex elements. result: m x n x 2 doubles, row-major over (i, j). */
+EXPORT int oracle_complex_gemm(int component_bits, int layout, int a_transpose, int b_transpose, size_t m, size_t n,
+                               size_t k, double alpha_re, double alpha_im, const void* a, size_t a_offset, size_t a_ld,
+                               const void* b, size_t b_offset, size_t b_ld, double beta_re, double beta_im,
+                               const void* c, size_t c_offset, size_t c_ld, double* result) {
+  if (m == 0 || n == 0 || k == 0) return kInvalidDimension;
+#pragma omp parallel for schedule(static)
+  for (long long ii = 0; ii < (long long)m; ++ii) {
+    const size_t i = (size_t)ii;
+    for (size_t j = 0; j < n; ++j) {
+      long double sum_re = 0.0L, sum_im = 0.0L;
+      for (size_t p = 0; p < k; ++p) {
+        /* op(A)(i, p) = A(i, p) or A(p, i) [conjugated]; op(B)(p, j) likewise */
+        const size_t ai = (a_transpose == kNo) ? matrix_index(layout, a_offset, a_ld, i, p)
+                                               : matrix_index(layout, a_offset, a_ld, p, i);
+        const size_t bi = (b_transpose == kNo) ? matrix_index(layout, b_offset, b_ld, p, j)
+                                               : matrix_index(layout, b_offset, b_ld, j, p);
+        const long double ar = load_as_double(a, component_bits, 2 * ai);
+        long double aim = load_as_double(a, component_bits, 2 * ai + 1);
+        const long double br = load_as_double(b, component_bits, 2 * bi);
+        long double bim = load_as_double(b, component_bits, 2 * bi + 1);
+        if (a_transpose == kConjugate) aim = -aim;
+        if (b_transpose == kConjugate) bim = -bim;
+        sum_re += ar * br - aim * bim;
+        sum_im += ar * bim + aim * br;
+      }
+      double re = (double)((long double)alpha_re * sum_re - (long double)alpha_im * sum_im);
+      double im = (double)((long double)alpha_re * sum_im + (long double)alpha_im * sum_re);
+      if (beta_re != 0.0 || beta_im != 0.0) {
+        const size_t ci = matrix_index(layout, c_offset, c_ld, i, j);
+        const double cr = load_as_double(c, component_bits, 2 * ci), cim = load_as_double(c, component_bits, 2 * ci + 1);
+        re += beta_re * cr - beta_im * cim;
+        im += beta_re * cim + beta_im * cr;
+      }
+      result[2 * (i * n + j)] = re;
+      result[2 * (i * n + j) + 1] = im;
+    }
+  }
+  return kSuccess;
 }
 
 /* ---- the reference's indirect path restated on the CPU (the "port" baseline) -------------------- */

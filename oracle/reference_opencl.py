@@ -13,7 +13,8 @@ HIP (both runtimes in one process were seen to lose the device), hence the comma
 spec.json: {"routine": "gemm"|"strided"|"symm" (then "side", "triangle" instead of "ta", "tb", "k")|"trmm"|"trsm" ("side",
 "triangle", "ta", "diagonal"; the result is the B buffer)|"syrk"|"syr2k" ("triangle", "ta", "n", "k"), "bits": 16|32|64, "layout", "ta", "tb", "m", "n", "k", "alpha", "beta",
 "a_ld", "b_ld", "c_ld", "offsets": [a, b, c], "seed": s, "low"/"high", "ab_low"/"ab_high", "batch", "strides",
-"runs": r, "sizes": [a, b, c] element counts}. Inputs are oracle.uniform(seed*3 + {0,1,2}, ...), exactly what
+"runs": r, "sizes": [a, b, c] element counts, "complex": true for CLBlastCgemm/Zgemm ("bits" is then the width of one
+component, "alpha"/"beta" are [re, im] pairs)}. Inputs are oracle.uniform(seed*3 + {0,1,2}, ...), exactly what
 tests/harness.py and the callers generate. The OpenCL host code here is a minimal ctypes binding of the
 standard OpenCL 1.2 C API; nothing of the reference is copied.
 """
@@ -100,7 +101,18 @@ class OpenCL:
         self.cl.clFinish(self.queue)
 
 
-def scalar_argument(bits, value, reference):
+class Float2(ctypes.Structure):  # cl_float2 by value
+    _fields_ = [("x", ctypes.c_float), ("y", ctypes.c_float)]
+
+
+class Double2(ctypes.Structure):  # cl_double2 by value
+    _fields_ = [("x", ctypes.c_double), ("y", ctypes.c_double)]
+
+
+def scalar_argument(bits, value, reference, is_complex=False):
+    if is_complex:
+        value = complex(*value) if isinstance(value, (list, tuple)) else complex(value)
+        return (Float2 if bits == 32 else Double2)(value.real, value.imag)
     if bits == 16:  # cl_half bit pattern; the test scalars are exactly representable
         return ctypes.c_ushort(int(np.array([value], dtype=np.float32).astype(np.float16).view(np.uint16)[0]))
     return SCALAR[bits](value)
@@ -115,9 +127,11 @@ def run(spec):
     seed = spec["seed"]
     sizes = spec["sizes"]
     ab_low, ab_high = spec.get("ab_low", spec.get("low", -1.0)), spec.get("ab_high", spec.get("high", 1.0))
-    a = oracle.uniform(seed * 3 + 0, sizes[0], ab_low, ab_high, bits)
-    b = oracle.uniform(seed * 3 + 1, sizes[1], ab_low, ab_high, bits)
-    c = oracle.uniform(seed * 3 + 2, sizes[2], spec.get("low", -1.0), spec.get("high", 1.0), bits)
+    is_complex = bool(spec.get("complex"))  # then "bits" is the width of one component and sizes count complex elements
+    generate = oracle.complex_uniform if is_complex else oracle.uniform
+    a = generate(seed * 3 + 0, sizes[0], ab_low, ab_high, bits)
+    b = generate(seed * 3 + 1, sizes[1], ab_low, ab_high, bits)
+    c = generate(seed * 3 + 2, sizes[2], spec.get("low", -1.0), spec.get("high", 1.0), bits)
     if spec.get("a_diagonal_boost"):  # well-conditioned triangular solves (tests/level3_harness.py does the same):
         k_diag, boost = spec["k_diag"], spec["a_diagonal_boost"]  # off-diagonal row sums below 1, |diagonal| >= boost
         a = (a.astype(np.float64) * (2.0 / k_diag)).astype(a.dtype)
@@ -127,7 +141,9 @@ def run(spec):
     in_place_b = spec["routine"] in ("trmm", "trsm")  # these overwrite B; "c" is then unused
     sz, vp = ctypes.c_size_t, ctypes.c_void_p
     queue = vp(opencl.queue.value)
-    alpha, beta = scalar_argument(bits, spec["alpha"], reference), scalar_argument(bits, spec.get("beta", 0.0), reference)
+    alpha = scalar_argument(bits, spec["alpha"], reference, is_complex)
+    beta = scalar_argument(bits, spec.get("beta", 0.0), reference, is_complex)
+    prefix = {32: "C", 64: "Z"}[bits] if is_complex else PREFIX[bits]
     offsets = spec.get("offsets", [0, 0, 0])
     m, n, k = sz(spec.get("m", 0)), sz(spec["n"]), sz(spec.get("k", 0))
 
@@ -156,7 +172,10 @@ def run(spec):
                               sz(spec["b_ld"]), beta, c_buffer, sz(offsets[2]), sz(spec["c_ld"]), ctypes.byref(queue),
                               ctypes.byref(event))
         elif spec["routine"] == "gemm":
-            function = getattr(reference, "CLBlast%sgemm" % PREFIX[bits])
+            function = getattr(reference, "CLBlast%sgemm" % prefix)
+            if is_complex:
+                function.argtypes = [ctypes.c_int] * 3 + [sz] * 3 + [type(alpha), vp, sz, sz, vp, sz, sz, type(beta), vp, sz, sz,
+                                                                   vp, vp]
             status = function(ctypes.c_int(spec["layout"]), ctypes.c_int(spec["ta"]), ctypes.c_int(spec["tb"]), m, n, k,
                               alpha, a_buffer, sz(offsets[0]), sz(spec["a_ld"]), b_buffer, sz(offsets[1]),
                               sz(spec["b_ld"]), beta, c_buffer, sz(offsets[2]), sz(spec["c_ld"]), ctypes.byref(queue),
@@ -213,7 +232,8 @@ def status_sweep(spec):
             pool[key] = opencl.buffer_from(np.zeros(max(size_bytes, 1), dtype=np.uint8))
         return pool[key]
 
-    alpha, beta = scalar_argument(bits, 1.0, reference), scalar_argument(bits, 0.0, reference)
+    is_complex = bool(spec.get("complex"))  # plain gemm cases only; "bits" is the width of one component
+    alpha, beta = scalar_argument(bits, 1.0, reference, is_complex), scalar_argument(bits, 0.0, reference, is_complex)
     statuses = []
     for case in spec["cases"]:
         if spec.get("rank_update"):  # "syrk" or "syr2k": [layout, triangle, ta, n, k, a_ld, b_ld, c_ld, a_bytes, b_bytes, c_bytes]
@@ -261,7 +281,10 @@ def status_sweep(spec):
                               sz(a_ld), sz(a_stride), b, sz(0), sz(b_ld), sz(b_stride), beta, c, sz(0), sz(c_ld), sz(c_stride),
                               sz(batch), ctypes.byref(queue), ctypes.byref(event))
         else:
-            function = getattr(reference, "CLBlast%sgemm" % PREFIX[bits])
+            function = getattr(reference, "CLBlast%sgemm" % ({32: "C", 64: "Z"}[bits] if is_complex else PREFIX[bits]))
+            if is_complex:
+                function.argtypes = [ctypes.c_int] * 3 + [sz] * 3 + [type(alpha), vp, sz, sz, vp, sz, sz, type(beta), vp, sz, sz,
+                                                                   vp, vp]
             status = function(ctypes.c_int(layout), ctypes.c_int(ta), ctypes.c_int(tb), sz(m), sz(n), sz(k), alpha, a, sz(0),
                               sz(a_ld), b, sz(0), sz(b_ld), beta, c, sz(0), sz(c_ld), ctypes.byref(queue), ctypes.byref(event))
         if status == 0 and event.value:
