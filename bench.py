@@ -25,10 +25,10 @@ if ROOT not in sys.path:
 
 ROW, COL, NO, YES = 101, 102, 111, 112
 # MI355X datasheet peaks (dense): TFLOP/s per storage type, HBM3E TB/s
-PEAK_TFLOPS = {"S": 157.3, "D": 78.6, "H": 2516.6}
+PEAK_TFLOPS = {"S": 157.3, "D": 78.6, "H": 2516.6, "C": 157.3, "Z": 78.6}  # complex: the real MFMA peak of its components
 PEAK_HBM_GBS = 8000.0
-BITS = {"S": 32, "D": 64, "H": 16}
-DTYPE_NAME = {"S": "f32", "D": "f64", "H": "f16"}
+BITS = {"S": 32, "D": 64, "H": 16, "C": 64, "Z": 128}
+DTYPE_NAME = {"S": "f32", "D": "f64", "H": "f16", "C": "c64 (f32 arithmetic)", "Z": "c128 (f64 arithmetic)"}
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
 # the readings of a plain 1 GiB copy (profiles/<workload>.md holds the commands and the raw readings). A bench run
 # cannot collect counters itself, so these are the figures of the committed profiles.
@@ -164,6 +164,51 @@ class SymmWorkload(Workload):
 
     def logical(self, which):
         return self.full.view(self.m, self.m) if which == "a" else super().logical(which)
+
+
+class ComplexWorkload:
+    """CGEMM / ZGEMM, C := alpha op(A) op(B) + beta C on interleaved complex data (torch complex tensors are row-major:
+    a row-major call). 8 m n k real flops, priced against the real MFMA peak of the component type."""
+
+    def __init__(self, name, prefix, ta, tb, m, n, k, alpha, beta):
+        import torch
+        self.name, self.prefix, self.ta, self.tb, self.m, self.n, self.k = name, prefix, ta, tb, m, n, k
+        self.alpha, self.beta = complex(alpha), complex(beta)
+        dtype = torch.complex64 if prefix == "C" else torch.complex128
+        generator = torch.Generator(device="cuda")
+        generator.manual_seed(2024)
+        draw = lambda rows, cols: torch.view_as_complex(  # noqa: E731
+            torch.rand(rows, cols, 2, device="cuda", dtype=torch.float64, generator=generator).mul_(2).sub_(1)).to(dtype)
+        self.a = draw(m, k) if ta == NO else draw(k, m)
+        self.b = draw(k, n) if tb == NO else draw(n, k)
+        self.c = draw(m, n)
+        self.c_initial = self.c.clone() if self.beta != 0 else None
+
+    @property
+    def flops(self):
+        return 8.0 * self.m * self.n * self.k
+
+    @property
+    def algorithmic_bytes(self):
+        element = 8 if self.prefix == "C" else 16
+        return element * (self.m * self.k + self.k * self.n + (2 if self.beta != 0 else 1) * self.m * self.n)
+
+    def call(self, stream_handle):
+        from clblast_amd.api import raw_complex_gemm
+        status = raw_complex_gemm(self.prefix, ROW, self.ta, self.tb, self.m, self.n, self.k, self.alpha, self.a.data_ptr(), 0,
+                                  self.a.shape[1], self.b.data_ptr(), 0, self.b.shape[1], self.beta, self.c.data_ptr(), 0,
+                                  self.n, stream_handle)
+        if status != 0:
+            raise RuntimeError("%s: status %d" % (self.name, status))
+
+    def freivalds_error(self):
+        import torch
+        x = torch.rand(self.n, 1, device="cuda", dtype=torch.float64).sub_(0.5).to(torch.complex128)
+        op = lambda t, flag: t if flag == NO else (t.T if flag == YES else t.conj().T)  # noqa: E731
+        expected = self.alpha * (op(self.a, self.ta).to(torch.complex128) @ (op(self.b, self.tb).to(torch.complex128) @ x))
+        if self.c_initial is not None:
+            expected = expected + self.beta * (self.c_initial.to(torch.complex128) @ x)
+        return float(((self.c.to(torch.complex128) @ x) - expected).norm() / expected.norm())
 
 
 class TrmmWorkload(Workload):
@@ -359,6 +404,9 @@ def reference_on_this_gpu(runs=3):
              "ssymm_4096_colLeftUpper": dict(routine="symm", bits=32, layout=COL, side=141, triangle=121, m=4096, n=4096,
                                              k=4096, alpha=1.0, beta=0.0, a_ld=4096, b_ld=4096, c_ld=4096,
                                              offsets=[0, 0, 0], seed=10, runs=5, sizes=[4096 * 4096] * 3),
+             "cgemm_4096_rowNC": dict(routine="gemm", complex=True, bits=32, layout=ROW, ta=NO, tb=113, m=4096, n=4096, k=4096,
+                                      alpha=[1.0, -0.5], beta=[0.0, 0.0], a_ld=4096, b_ld=4096, c_ld=4096, offsets=[0, 0, 0],
+                                      seed=14, runs=3, sizes=[4096 * 4096] * 3),
              "ssyrk_4096_colLower": dict(routine="syrk", bits=32, layout=COL, triangle=122, ta=NO, m=4096, n=4096, k=4096,
                                          alpha=1.0, beta=0.0, a_ld=4096, b_ld=4096, c_ld=4096, offsets=[0, 0, 0], seed=11,
                                          runs=5, sizes=[4096 * 4096] * 3),
@@ -369,7 +417,7 @@ def reference_on_this_gpu(runs=3):
                                              m=4096, n=4096, k=4096, alpha=1.0, a_ld=4096, b_ld=4096, offsets=[0, 0, 0],
                                              seed=13, runs=3, sizes=[4096 * 4096] * 3, a_diagonal_boost=4.0, k_diag=4096)}
     half_count = ("ssyrk_4096_colLower", "strmm_4096_colLeftLower", "strsm_4096_colLeftLower")  # BLAS counts n*n*k, m*m*n
-    flops = {name: (1.0 if name in half_count else 2.0) * spec["m"] * spec["n"] * spec["k"] * spec.get("batch", 1)
+    flops = {name: (1.0 if name in half_count else 8.0 if spec.get("complex") else 2.0) * spec["m"] * spec["n"] * spec["k"] * spec.get("batch", 1)
              for name, spec in specs.items()}
     root = os.path.dirname(os.path.abspath(__file__))
     with tempfile.TemporaryDirectory() as folder:
@@ -406,6 +454,8 @@ EXTRA_WORKLOADS = {
                                                        24, (11, 13, 19)),
     "cfg5_sgemm_8191x8191x127_colNN": lambda: Workload("cfg5d", "S", COL, NO, NO, 8191, 8191, 127, -0.75, 2.0, 8194,
                                                         132, 8198, (11, 13, 19)),
+    "next_cgemm_4096_rowNC": lambda: ComplexWorkload("cgemm", "C", NO, 113, 4096, 4096, 4096, 1.0 - 0.5j, 0.0),
+    "next_zgemm_2048_rowTN": lambda: ComplexWorkload("zgemm", "Z", YES, NO, 2048, 2048, 2048, 0.5 + 1.0j, 1.0 - 0.5j),
     "next_ssymm_4096_colLeftUpper": lambda: SymmWorkload("symm_s", "S", COL, True, 4096, 4096, 1.0, 0.0),
     "next_hsymm_4096_rowLeftLower": lambda: SymmWorkload("symm_h", "H", ROW, False, 4096, 4096, 1.0, 0.0),
     "next_strmm_4096_colLeftLower": lambda: TrmmWorkload("trmm_s", "S", "trmm", True, False, 4096, 4096),
