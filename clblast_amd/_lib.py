@@ -87,10 +87,13 @@ def load():
 # Every symbol the public C headers declare, for the export test.
 C_API_SYMBOLS = (
     ["CLBlast%sgemm%s" % (p, s) for p in "SDH" for s in ("", "Batched", "StridedBatched", "WithTempBuffer")] +
-    ["CLBlast%sGemmTempBufferSize" % p for p in "SDH"] + ["CLBlastCgemm", "CLBlastZgemm"] + ["CLBlast%ssymm" % p for p in "SDH"] + ["CLBlast%strmm" % p for p in "SDH"] + ["CLBlast%strsm" % p for p in "SD"] + ["CLBlast%ssyrk" % p for p in "SDH"] +
-    ["CLBlast%ssyr2k" % p for p in "SDH"] +
+    ["CLBlast%sGemmTempBufferSize" % p for p in "SDH"] + ["CLBlastCgemm", "CLBlastZgemm"] +
+    ["CLBlast%s%s" % (p, r) for p in "SDH" for r in ("symm", "syrk", "syr2k", "trmm")] + ["CLBlastStrsm", "CLBlastDtrsm"] +
     ["CLBlastClearCache", "CLBlastOverrideParameters", "CLBlastFloatToHalf", "CLBlastHalfToFloat"])
+NETLIB_SYMBOLS = (["cblas_%sgemm" % p for p in "sdcz"] +
+                  ["cblas_%s%s" % (p, r) for p in "sd" for r in ("symm", "syrk", "syr2k", "trmm", "trsm")])
 DEVICE_LAYER_SYMBOLS = [
     "clbh_gemm_launch", "clbh_gemm_workspace_bytes", "clbh_buffer_extent", "clbh_alloc_async", "clbh_free_async",
-    "clbh_upload_async", "clbh_event_record", "clbh_stream_device", "clbh_error_string", "clbh_symmetric_to_square", "clbh_triangular_to_square", "clbh_copy_matrix", "clbh_invert_block_size",
-                        "clbh_invert_diagonal_blocks", "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale"]
+    "clbh_upload_async", "clbh_event_record", "clbh_stream_device", "clbh_error_string", "clbh_symmetric_to_square",
+    "clbh_triangular_to_square", "clbh_copy_matrix", "clbh_invert_block_size", "clbh_invert_diagonal_blocks",
+    "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale", "clbh_alloc", "clbh_free", "clbh_copy"]

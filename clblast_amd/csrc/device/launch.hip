@@ -305,6 +305,18 @@ int clbh_complex_scale(int precision, int m, int n, double beta_re, double beta_
   return hipErrorInvalidValue;
 }
 
+int clbh_alloc(void** ptr, size_t bytes) {
+  if (ptr == nullptr) { return hipErrorInvalidValue; }
+  return static_cast<int>(hipMalloc(ptr, bytes));
+}
+
+int clbh_free(void* ptr) { return static_cast<int>(hipFree(ptr)); }
+
+int clbh_copy(void* dst, const void* src, size_t bytes, int to_device) {
+  if (dst == nullptr || src == nullptr) { return hipErrorInvalidValue; }
+  return static_cast<int>(hipMemcpy(dst, src, bytes, to_device ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost));
+}
+
 int clbh_buffer_extent(const void* ptr, size_t* bytes_available) {
   if (ptr == nullptr || bytes_available == nullptr) { return hipErrorInvalidValue; }
   hipDeviceptr_t base = nullptr;

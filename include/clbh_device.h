@@ -120,6 +120,12 @@ CLBH_API int clbh_complex_transpose(int precision, int k, int n, const void* src
 CLBH_API int clbh_complex_scale(int precision, int m, int n, double beta_re, double beta_im, void* c,
                                 long long c_offset, long long c_ld, hipStream_t stream);
 
+// Plain device memory and blocking copies for callers that hold host data (the Netlib-style façade): to_device != 0
+// copies host -> device, else waits for the default stream's work and copies device -> host.
+CLBH_API int clbh_alloc(void** ptr, size_t bytes);
+CLBH_API int clbh_free(void* ptr);
+CLBH_API int clbh_copy(void* dst, const void* src, size_t bytes, int to_device);
+
 // Number of bytes addressable from `ptr` to the end of the device allocation that contains it.
 // Returns 0 on success, non-zero if `ptr` is not inside a device allocation.
 CLBH_API int clbh_buffer_extent(const void* ptr, size_t* bytes_available);

@@ -17,16 +17,17 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def declared_functions(header):
     text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"//[^\n]*", "", text)
-    return set(re.findall(r"\b(CLBlast[A-Za-z0-9]+|clbh_[a-z_]+)\s*\(", text))
+    return set(re.findall(r"\b(CLBlast[A-Za-z0-9]+|clbh_[a-z_]+|cblas_[a-z0-9]+)\s*\(", text))
 
 
 def test_library_loads_and_exports_every_declared_symbol():
     lib = _lib.load()
-    declared = declared_functions("clblast_hip_c.h") | declared_functions("clbh_device.h")
+    declared = (declared_functions("clblast_hip_c.h") | declared_functions("clbh_device.h") |
+                declared_functions("clblast_hip_netlib_c.h"))
     assert len(declared) >= 28
     missing = sorted(name for name in declared if not hasattr(lib, name))
     assert not missing, missing
-    assert declared == set(_lib.C_API_SYMBOLS) | set(_lib.DEVICE_LAYER_SYMBOLS)
+    assert declared == set(_lib.C_API_SYMBOLS) | set(_lib.DEVICE_LAYER_SYMBOLS) | set(_lib.NETLIB_SYMBOLS)
 
 
 def test_cpp_api_instantiations_are_exported():
