@@ -33,6 +33,10 @@ def _declare(lib):
         f = getattr(lib, "CLBlast%sgemm" % prefix)
         f.argtypes = [c_int, c_int, c_int, sz, sz, sz, scalar, vp, sz, sz, vp, sz, sz, scalar, vp, sz, sz, vp, vp]
         f.restype = c_int
+    for prefix in "SDH":
+        f = getattr(lib, "CLBlast%sconvgemm" % prefix)
+        f.argtypes = [c_int] + [sz] * 13 + [vp, sz, vp, sz, vp, sz, vp, vp]
+        f.restype = c_int
     for prefix, scalar in _SCALAR.items():
         gemm_args = [c_int, c_int, c_int, sz, sz, sz, scalar, vp, sz, sz, vp, sz, sz, scalar, vp, sz, sz, vp, vp]
         f = getattr(lib, "CLBlast%sgemm" % prefix)
@@ -89,6 +93,7 @@ C_API_SYMBOLS = (
     ["CLBlast%sgemm%s" % (p, s) for p in "SDH" for s in ("", "Batched", "StridedBatched", "WithTempBuffer")] +
     ["CLBlast%sGemmTempBufferSize" % p for p in "SDH"] + ["CLBlastCgemm", "CLBlastZgemm"] +
     ["CLBlast%s%s" % (p, r) for p in "SDH" for r in ("symm", "syrk", "syr2k", "trmm")] + ["CLBlastStrsm", "CLBlastDtrsm"] +
+    ["CLBlast%sconvgemm" % p for p in "SDH"] +
     ["CLBlastClearCache", "CLBlastOverrideParameters", "CLBlastFloatToHalf", "CLBlastHalfToFloat"])
 NETLIB_SYMBOLS = (["cblas_%sgemm" % p for p in "sdcz"] +
                   ["cblas_%s%s" % (p, r) for p in "sd" for r in ("symm", "syrk", "syr2k", "trmm", "trsm")])
@@ -96,4 +101,4 @@ DEVICE_LAYER_SYMBOLS = [
     "clbh_gemm_launch", "clbh_gemm_workspace_bytes", "clbh_buffer_extent", "clbh_alloc_async", "clbh_free_async",
     "clbh_upload_async", "clbh_event_record", "clbh_stream_device", "clbh_error_string", "clbh_symmetric_to_square",
     "clbh_triangular_to_square", "clbh_copy_matrix", "clbh_invert_block_size", "clbh_invert_diagonal_blocks",
-    "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale", "clbh_alloc", "clbh_free", "clbh_copy"]
+    "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale", "clbh_alloc", "clbh_free", "clbh_copy", "clbh_im2col"]

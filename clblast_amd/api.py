@@ -20,6 +20,7 @@ TRANS_NO, TRANS_YES, TRANS_CONJ = 111, 112, 113
 TRIANGLE_UPPER, TRIANGLE_LOWER = 121, 122
 SIDE_LEFT, SIDE_RIGHT = 141, 142
 DIAGONAL_NON_UNIT, DIAGONAL_UNIT = 131, 132
+CROSS_CORRELATION, CONVOLUTION = 151, 152
 
 STATUS_NAMES = {
     0: "kSuccess", -4: "kTempBufferAllocFailure", -30: "kInvalidValue", -36: "kInvalidCommandQueue",
@@ -88,6 +89,18 @@ def raw_complex_gemm(prefix, layout, a_transpose, b_transpose, m, n, k, alpha, a
     return getattr(lib, "CLBlast%sgemm" % prefix)(layout, a_transpose, b_transpose, m, n, k, scalar(alpha.real, alpha.imag),
                                                   a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld, scalar(beta.real, beta.imag),
                                                   c_ptr, c_offset, c_ld, _stream_ref(stream_handle), event_ref)
+
+
+def raw_convgemm(prefix, kernel_mode, channels, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w, dilation_h,
+                 dilation_w, num_kernels, batch_count, im_ptr, im_offset, kernel_ptr, kernel_offset, result_ptr, result_offset,
+                 stream_handle=0, event_handle=None):
+    """CLBlast{S,D,H}convgemm through the C ABI (reference: include/clblast_c.h:1252-1281)."""
+    lib = _lib.load()
+    event_ref = None if event_handle is None else ctypes.byref(ctypes.c_void_p(event_handle))
+    return getattr(lib, "CLBlast%sconvgemm" % prefix)(kernel_mode, channels, height, width, kernel_h, kernel_w, pad_h, pad_w,
+                                                      stride_h, stride_w, dilation_h, dilation_w, num_kernels, batch_count,
+                                                      im_ptr, im_offset, kernel_ptr, kernel_offset, result_ptr, result_offset,
+                                                      _stream_ref(stream_handle), event_ref)
 
 
 def raw_symm(prefix, layout, side, triangle, m, n, alpha, a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld, beta, c_ptr,

@@ -10,6 +10,7 @@
 #include "clblast_hip.h"
 #include "routines/xgemm.hpp"
 #include "routines/xgemm_complex.hpp"
+#include "routines/xconvgemm.hpp"
 #include "routines/xgemmbatched.hpp"
 #include "routines/xsymm.hpp"
 #include "routines/xsyrk.hpp"
@@ -115,6 +116,24 @@ StatusCode Trsm(const Layout layout, const Side side, const Triangle triangle, c
 }
 
 template <typename T>
+StatusCode Convgemm(const KernelMode kernel_mode, const size_t channels, const size_t height, const size_t width,
+                    const size_t kernel_h, const size_t kernel_w, const size_t pad_h, const size_t pad_w,
+                    const size_t stride_h, const size_t stride_w, const size_t dilation_h, const size_t dilation_w,
+                    const size_t num_kernels, const size_t batch_count, const void* im_buffer, const size_t im_offset,
+                    const void* kernel_buffer, const size_t kernel_offset, void* result_buffer,
+                    const size_t result_offset, hipStream_t* queue, hipEvent_t* event) {
+  try {
+    auto routine = Xconvgemm<T>(queue, event);
+    routine.DoConvgemm(kernel_mode, channels, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w, dilation_h,
+                       dilation_w, num_kernels, batch_count, Buffer<T>(im_buffer), im_offset, Buffer<T>(kernel_buffer),
+                       kernel_offset, Buffer<T>(result_buffer), result_offset);
+    return StatusCode::kSuccess;
+  } catch (...) {
+    return DispatchException();
+  }
+}
+
+template <typename T>
 StatusCode GemmBatched(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
                        const size_t n, const size_t k, const T* alphas, const void* a_buffer, const size_t* a_offsets,
                        const size_t a_ld, const void* b_buffer, const size_t* b_offsets, const size_t b_ld,
@@ -199,6 +218,10 @@ StatusCode GemmTempBufferSize(const Layout layout, const Transpose a_transpose, 
                                                  const T, const void*, const size_t, const size_t, const void*,     \
                                                  const size_t, const size_t, const T, void*, const size_t,          \
                                                  const size_t, hipStream_t*, hipEvent_t*);                          \
+  template StatusCode CLBLAST_HIP_PUBLIC Convgemm<T>(                                                               \
+      const KernelMode, const size_t, const size_t, const size_t, const size_t, const size_t, const size_t,         \
+      const size_t, const size_t, const size_t, const size_t, const size_t, const size_t, const size_t, const void*, \
+      const size_t, const void*, const size_t, void*, const size_t, hipStream_t*, hipEvent_t*);                     \
   template StatusCode CLBLAST_HIP_PUBLIC Syrk<T>(const Layout, const Triangle, const Transpose, const size_t,         \
                                                  const size_t, const T, const void*, const size_t, const size_t,    \
                                                  const T, void*, const size_t, const size_t, hipStream_t*,          \

@@ -295,6 +295,26 @@ CLBlastStatusCode CLBlastHsymm(const CLBlastLayout layout, const CLBlastSide sid
   });
 }
 
+// ---- CONVGEMM -----------------------------------------------------------------------------------
+#define CLBLAST_HIP_CONVGEMM(NAME, TYPE)                                                                             \
+  CLBlastStatusCode NAME(const CLBlastKernelMode kernel_mode, const size_t channels, const size_t height,            \
+                         const size_t width, const size_t kernel_h, const size_t kernel_w, const size_t pad_h,       \
+                         const size_t pad_w, const size_t stride_h, const size_t stride_w, const size_t dilation_h,  \
+                         const size_t dilation_w, const size_t num_kernels, const size_t batch_count,                \
+                         const void* im_buffer, const size_t im_offset, const void* kernel_buffer,                   \
+                         const size_t kernel_offset, void* result_buffer, const size_t result_offset,                \
+                         hipStream_t* queue, hipEvent_t* event) {                                                    \
+    return Guarded([&]() {                                                                                           \
+      return clblast::Convgemm<TYPE>(static_cast<clblast::KernelMode>(kernel_mode), channels, height, width, kernel_h, \
+                                     kernel_w, pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w, num_kernels, \
+                                     batch_count, im_buffer, im_offset, kernel_buffer, kernel_offset, result_buffer,  \
+                                     result_offset, queue, event);                                                   \
+    });                                                                                                              \
+  }
+CLBLAST_HIP_CONVGEMM(CLBlastSconvgemm, float)
+CLBLAST_HIP_CONVGEMM(CLBlastDconvgemm, double)
+CLBLAST_HIP_CONVGEMM(CLBlastHconvgemm, clblast::half)
+
 // ---- CGEMM, ZGEMM -------------------------------------------------------------------------------
 CLBlastStatusCode CLBlastCgemm(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
                                const CLBlastTranspose b_transpose, const size_t m, const size_t n, const size_t k,

@@ -10,6 +10,7 @@
 #include "device/launch_common.hpp"
 #include "kernels/symmetric_to_square.hpp"
 #include "kernels/complex_helpers.hpp"
+#include "kernels/im2col.hpp"
 #include "kernels/triangular_to_square.hpp"
 
 namespace clbh {
@@ -303,6 +304,36 @@ int clbh_complex_scale(int precision, int m, int n, double beta_re, double beta_
   if (precision == 32) { return LaunchComplexScale<float>(m, n, beta_re, beta_im, c, c_offset, c_ld, stream); }
   if (precision == 64) { return LaunchComplexScale<double>(m, n, beta_re, beta_im, c, c_offset, c_ld, stream); }
   return hipErrorInvalidValue;
+}
+
+int clbh_im2col(int precision, const clbh_im2col_shape* shape, int batch_count, const void* image, long long image_offset,
+                void* col, hipStream_t stream) {
+  if (shape == nullptr || image == nullptr || col == nullptr || batch_count <= 0 || image_offset < 0) { return hipErrorInvalidValue; }
+  const auto& g = *shape;
+  if (g.channels <= 0 || g.height <= 0 || g.width <= 0 || g.kernel_h <= 0 || g.kernel_w <= 0 || g.stride_h <= 0 ||
+      g.stride_w <= 0 || g.dilation_h <= 0 || g.dilation_w <= 0 || g.output_h <= 0 || g.output_w <= 0 || g.pad_h < 0 || g.pad_w < 0) {
+    return hipErrorInvalidValue;
+  }
+  const long long patches = static_cast<long long>(g.output_h) * g.output_w;
+  const long long rows = static_cast<long long>(g.channels) * g.kernel_h * g.kernel_w;
+  if (patches > INT_MAX || rows > INT_MAX) { return hipErrorInvalidConfiguration; }
+  clbh::Im2colShape s;
+  s.channels = g.channels; s.height = g.height; s.width = g.width;
+  s.kernel_h = g.kernel_h; s.kernel_w = g.kernel_w; s.pad_h = g.pad_h; s.pad_w = g.pad_w;
+  s.stride_h = g.stride_h; s.stride_w = g.stride_w; s.dilation_h = g.dilation_h; s.dilation_w = g.dilation_w;
+  s.output_h = g.output_h; s.output_w = g.output_w; s.flip = g.flip;
+  const dim3 grid(static_cast<unsigned>((patches + clbh::kIm2colThreads - 1) / clbh::kIm2colThreads),
+                  static_cast<unsigned>(std::min<long long>(rows, 65535)), static_cast<unsigned>(std::min(batch_count, 65535)));
+  switch (precision) {
+    case 16: clbh::Im2colKernel<_Float16><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(
+                 s, batch_count, static_cast<const _Float16*>(image) + image_offset, static_cast<_Float16*>(col)); break;
+    case 32: clbh::Im2colKernel<float><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(
+                 s, batch_count, static_cast<const float*>(image) + image_offset, static_cast<float*>(col)); break;
+    case 64: clbh::Im2colKernel<double><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(
+                 s, batch_count, static_cast<const double*>(image) + image_offset, static_cast<double*>(col)); break;
+    default: return hipErrorInvalidValue;
+  }
+  return static_cast<int>(hipGetLastError());
 }
 
 int clbh_alloc(void** ptr, size_t bytes) {

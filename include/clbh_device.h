@@ -120,6 +120,18 @@ CLBH_API int clbh_complex_transpose(int precision, int k, int n, const void* src
 CLBH_API int clbh_complex_scale(int precision, int m, int n, double beta_re, double beta_im, void* c,
                                 long long c_offset, long long c_ld, hipStream_t stream);
 
+// im2col of a batch of images for CONVGEMM (all arguments in elements; see kernels/im2col.hpp for the layout):
+// image + image_offset holds batch x channels x height x width, col receives batch matrices of
+// (output_h * output_w) x (channels * kernel_h * kernel_w), column-major. flip != 0 mirrors the kernel taps.
+typedef struct clbh_im2col_shape_ {
+  int channels, height, width;
+  int kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w;
+  int output_h, output_w;
+  int flip;
+} clbh_im2col_shape;
+CLBH_API int clbh_im2col(int precision, const clbh_im2col_shape* shape, int batch_count, const void* image,
+                         long long image_offset, void* col, hipStream_t stream);
+
 // Plain device memory and blocking copies for callers that hold host data (the Netlib-style façade): to_device != 0
 // copies host -> device, else waits for the default stream's work and copies device -> host.
 CLBH_API int clbh_alloc(void** ptr, size_t bytes);

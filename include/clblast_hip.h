@@ -2,7 +2,7 @@
 // C++ interface of the MI355X (gfx950) GEMM engine behind the CLBlast GEMM API.
 //
 // The argument surface is the one of CLBlast's `include/clblast.h` (reference: Gemm :427-432,
-// GemmBatched :538-543, GemmStridedBatched :547-553, Symm :435-439, Syrk :449-453, Syr2k :463-467, Trmm :477-481, Trsm :484-488, GemmTempBufferSize :558-562, StatusCode :61-129,
+// GemmBatched :538-543, GemmStridedBatched :547-553, Symm :435-439, Syrk :449-453, Syr2k :463-467, Trmm :477-481, Trsm :484-488, Convgemm :523-529, GemmTempBufferSize :558-562, StatusCode :61-129,
 // Layout/Transpose/Precision :132-147, OverrideParameters :620-624, ClearCache :568). Only the handle
 // types differ: `cl_mem` becomes a raw device pointer (`void*`, as returned by hipMalloc or
 // `tensor.data_ptr()`), `cl_command_queue*` becomes `hipStream_t*` and `cl_event*` becomes
@@ -102,6 +102,7 @@ enum class Transpose { kNo = 111, kYes = 112, kConjugate = 113 };
 enum class Triangle { kUpper = 121, kLower = 122 };
 enum class Diagonal { kNonUnit = 131, kUnit = 132 };
 enum class Side { kLeft = 141, kRight = 142 };
+enum class KernelMode { kCrossCorrelation = 151, kConvolution = 152 };
 enum class Precision { kHalf = 16, kSingle = 32, kDouble = 64, kComplexSingle = 3232, kComplexDouble = 6464, kAny = -1 };
 
 // Host type of fp16 scalars and data: the IEEE binary16 bit pattern (reference: clblast_half.h:21).
@@ -182,6 +183,19 @@ StatusCode Trsm(const Layout layout, const Side side, const Triangle triangle, c
                 const Diagonal diagonal, const size_t m, const size_t n, const T alpha, const void* a_buffer,
                 const size_t a_offset, const size_t a_ld, void* b_buffer, const size_t b_offset, const size_t b_ld,
                 hipStream_t* queue, hipEvent_t* event = nullptr);
+
+// Batched 2-D convolution as a matrix multiplication: images batch_count x channels x height x width, kernels
+// num_kernels x channels x kernel_h x kernel_w, result batch_count x num_kernels x output_h x output_w (all contiguous,
+// offsets in elements) with output_h = (height + 2 pad_h - dilation_h (kernel_h - 1) - 1) / stride_h + 1 and likewise
+// output_w; `kConvolution` mirrors the kernels, `kCrossCorrelation` does not (reference: include/clblast.h:523-529,
+// src/routines/levelx/xconvgemm.cpp:49-160). T is float, double or half.
+template <typename T>
+StatusCode Convgemm(const KernelMode kernel_mode, const size_t channels, const size_t height, const size_t width,
+                    const size_t kernel_h, const size_t kernel_w, const size_t pad_h, const size_t pad_w,
+                    const size_t stride_h, const size_t stride_w, const size_t dilation_h, const size_t dilation_w,
+                    const size_t num_kernels, const size_t batch_count, const void* im_buffer, const size_t im_offset,
+                    const void* kernel_buffer, const size_t kernel_offset, void* result_buffer,
+                    const size_t result_offset, hipStream_t* queue, hipEvent_t* event = nullptr);
 
 // Bytes this engine wants in `temp_buffer` for the given arguments (0 when none is needed).
 template <typename T>

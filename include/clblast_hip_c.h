@@ -69,6 +69,7 @@ typedef struct CLBlastFloat2_ { float x; float y; } CLBlastFloat2;
 typedef struct CLBlastDouble2_ { double x; double y; } CLBlastDouble2;
 typedef enum CLBlastTriangle_ { CLBlastTriangleUpper = 121, CLBlastTriangleLower = 122 } CLBlastTriangle;
 typedef enum CLBlastDiagonal_ { CLBlastDiagonalNonUnit = 131, CLBlastDiagonalUnit = 132 } CLBlastDiagonal;
+typedef enum CLBlastKernelMode_ { CLBlastKernelModeCrossCorrelation = 151, CLBlastKernelModeConvolution = 152 } CLBlastKernelMode;
 typedef enum CLBlastSide_ { CLBlastSideLeft = 141, CLBlastSideRight = 142 } CLBlastSide;
 typedef enum CLBlastPrecision_ {
   CLBlastPrecisionHalf = 16,
@@ -204,6 +205,36 @@ CLBlastStatusCode CLBLAST_HIP_API CLBlastHtrmm(const CLBlastLayout layout, const
                                                const unsigned short alpha, const void* a_buffer, const size_t a_offset,
                                                const size_t a_ld, void* b_buffer, const size_t b_offset,
                                                const size_t b_ld, hipStream_t* queue, hipEvent_t* event);
+
+// Batched convolution as GEMM (non-BLAS function)
+// replaces CLBlastSconvgemm/CLBlastDconvgemm/CLBlastHconvgemm (reference: include/clblast_c.h:1252-1281, src/clblast_c.cpp:2625-2700)
+CLBlastStatusCode CLBLAST_HIP_API CLBlastSconvgemm(const CLBlastKernelMode kernel_mode, const size_t channels,
+                                                   const size_t height, const size_t width, const size_t kernel_h,
+                                                   const size_t kernel_w, const size_t pad_h, const size_t pad_w,
+                                                   const size_t stride_h, const size_t stride_w, const size_t dilation_h,
+                                                   const size_t dilation_w, const size_t num_kernels,
+                                                   const size_t batch_count, const void* im_buffer, const size_t im_offset,
+                                                   const void* kernel_buffer, const size_t kernel_offset,
+                                                   void* result_buffer, const size_t result_offset, hipStream_t* queue,
+                                                   hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastDconvgemm(const CLBlastKernelMode kernel_mode, const size_t channels,
+                                                   const size_t height, const size_t width, const size_t kernel_h,
+                                                   const size_t kernel_w, const size_t pad_h, const size_t pad_w,
+                                                   const size_t stride_h, const size_t stride_w, const size_t dilation_h,
+                                                   const size_t dilation_w, const size_t num_kernels,
+                                                   const size_t batch_count, const void* im_buffer, const size_t im_offset,
+                                                   const void* kernel_buffer, const size_t kernel_offset,
+                                                   void* result_buffer, const size_t result_offset, hipStream_t* queue,
+                                                   hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastHconvgemm(const CLBlastKernelMode kernel_mode, const size_t channels,
+                                                   const size_t height, const size_t width, const size_t kernel_h,
+                                                   const size_t kernel_w, const size_t pad_h, const size_t pad_w,
+                                                   const size_t stride_h, const size_t stride_w, const size_t dilation_h,
+                                                   const size_t dilation_w, const size_t num_kernels,
+                                                   const size_t batch_count, const void* im_buffer, const size_t im_offset,
+                                                   const void* kernel_buffer, const size_t kernel_offset,
+                                                   void* result_buffer, const size_t result_offset, hipStream_t* queue,
+                                                   hipEvent_t* event);
 
 // Triangular solve in place: B becomes the X with op(A)*X = alpha*B (side left) or X*op(A) = alpha*B (side right)
 // replaces CLBlastStrsm/CLBlastDtrsm; like the reference there is no half-precision TRSM (reference: include/clblast_c.h:1094-1124, src/clblast_c.cpp:2402-2500)

@@ -65,6 +65,8 @@ def lib():
         handle.oracle_syr2k_status.restype = ci
         handle.oracle_complex_gemm.argtypes = [ci, ci, ci, ci, sz, sz, sz, dbl, dbl, vp, sz, sz, vp, sz, sz, dbl, dbl, vp, sz, sz, vp]
         handle.oracle_complex_gemm.restype = ci
+        handle.oracle_convgemm.argtypes = [ci, ci] + [sz] * 13 + [vp, sz, vp, sz, vp]
+        handle.oracle_convgemm.restype = ci
         handle.oracle_process_arguments.argtypes = [ci, ci, ci, sz, sz, sz, ctypes.POINTER(Shape)]
         handle.oracle_process_arguments.restype = ci
         handle.oracle_gemm_status.argtypes = [ci, ci, ci, ci] + [sz] * 12
@@ -198,6 +200,32 @@ def complex_gemm(layout, a_transpose, b_transpose, m, n, k, alpha, a, a_offset, 
 def complex_uniform(seed, count, low, high, component_bits):
     """`count` complex numbers whose 2 * count components are uniform(seed, ...) of that width, interleaved."""
     return uniform(seed, 2 * count, low, high, component_bits).view(np.complex64 if component_bits == 32 else np.complex128)
+
+
+CROSS_CORRELATION, CONVOLUTION = 151, 152
+
+
+def conv_output_extent(extent, kernel, pad, stride, dilation):
+    """Reference: src/routines/levelx/xconvgemm.cpp:66-72."""
+    size, padding = extent + 2 * pad, dilation * (kernel - 1) + 1
+    return (size - padding) // stride + 1 if size >= padding else 1
+
+
+def convgemm(kernel_mode, channels, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w,
+             num_kernels, batch_count, image, image_offset, kernels, kernel_offset):
+    """The result tensor (batch x num_kernels x output_h x output_w, float64) of CONVGEMM by the C oracle."""
+    bits = _bits(image)
+    assert _bits(kernels) == bits
+    image, kernels = np.ascontiguousarray(image), np.ascontiguousarray(kernels)
+    output_h = conv_output_extent(height, kernel_h, pad_h, stride_h, dilation_h)
+    output_w = conv_output_extent(width, kernel_w, pad_w, stride_w, dilation_w)
+    result = np.empty((batch_count, num_kernels, output_h, output_w), dtype=np.float64)
+    status = lib().oracle_convgemm(bits, kernel_mode, channels, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w,
+                                   dilation_h, dilation_w, num_kernels, batch_count, image.ctypes.data, image_offset,
+                                   kernels.ctypes.data, kernel_offset, result.ctypes.data)
+    if status != 0:
+        raise ValueError("oracle_convgemm status %d" % status)
+    return result
 
 
 NON_UNIT, UNIT = 131, 132

@@ -32,6 +32,8 @@
  *                              the "port" CPU baseline, parallelised over tiles with OpenMP.
  *
  *   oracle_complex_gemm        CGEMM/ZGEMM from the definition, complex multiply-add in long double
+ *   oracle_convgemm            CONVGEMM from the definition of the convolution (src/routines/levelx/xconvgemm.cpp,
+ *                              src/kernels/levelx/im2col.opencl), not through im2col
  *   oracle_symm, oracle_trmm,  the Level-3 routines the reference builds on its GEMM (src/routines/level3/xsymm.cpp,
  *   oracle_trsm, oracle_syr2k  xtrmm.cpp, xtrsm.cpp, xsyrk.cpp, xsyr2k.cpp) stated from their definitions in long
  *   and their *_status         double arithmetic, with the check order of those files.
@@ -48,6 +50,9 @@
  *     OpenCL device (tests/test_reference_opencl_gpu.py).
  *   - oracle_complex_gemm: against numpy complex128 matmul with .T / .conj().T, and the real reference library
  *     (CLBlastCgemm/Zgemm) on an OpenCL device (tests/test_complex_gemm.py, tests/test_complex_gemm_gpu.py).
+ *   - oracle_convgemm: against torch.nn.functional.conv2d on the CPU in float64 (padding, strides, dilations; the
+ *     mirrored kernel for kConvolution), hand-computed cases, and the real reference (tests/test_convgemm.py,
+ *     tests/test_convgemm_gpu.py).
  *   - symm/trmm/trsm/syrk/syr2k: against independent numpy statements, the BLAS routines of scipy
  *     (dsymm, dtrmm, dtrsm, dsyrk, dsyr2k), algebraic identities, and the real reference library on an OpenCL
  *     device, status codes included (tests/test_level3_oracle.py, tests/test_symm_oracle.py, tests/test_*_gpu.py).
@@ -608,6 +613,58 @@ EXPORT int oracle_complex_gemm(int component_bits, int layout, int a_transpose, 
       }
       result[2 * (i * n + j)] = re;
       result[2 * (i * n + j) + 1] = im;
+    }
+  }
+  return kSuccess;
+}
+
+/* ---- CONVGEMM --------------------------------------------------------------------------------------- */
+
+enum { kCrossCorrelation = 151, kConvolution = 152 };
+
+static size_t conv_output_extent(size_t input, size_t kernel, size_t pad, size_t stride, size_t dilation) {
+  /* src/routines/levelx/xconvgemm.cpp:66-72 */
+  const size_t size = input + 2 * pad, padding = dilation * (kernel - 1) + 1;
+  return (size >= padding) ? (size - padding) / stride + 1 : 1;
+}
+
+/* Batched 2-D convolution from its definition (what src/kernels/levelx/im2col.opencl:22-66 followed by the product of
+ * xconvgemm.cpp:98-100 computes): result[b][f][oh][ow] = sum over c, kh, kw of
+ *   image[b][c][oh*stride_h - pad_h + kh*dilation_h][ow*stride_w - pad_w + kw*dilation_w]  (0 outside the image)
+ *   * kernel[f][c][tap], tap = kh*kernel_w + kw, mirrored (kernel_h*kernel_w - 1 - tap) for kConvolution.
+ * result: batch x num_kernels x output_h x output_w doubles. */
+EXPORT int oracle_convgemm(int bits, int kernel_mode, size_t channels, size_t height, size_t width, size_t kernel_h,
+                           size_t kernel_w, size_t pad_h, size_t pad_w, size_t stride_h, size_t stride_w, size_t dilation_h,
+                           size_t dilation_w, size_t num_kernels, size_t batch_count, const void* image, size_t image_offset,
+                           const void* kernels, size_t kernel_offset, double* result) {
+  if (batch_count == 0) return kInvalidBatchCount;
+  if (channels == 0 || height == 0 || width == 0 || num_kernels == 0) return kInvalidDimension;
+  const size_t output_h = conv_output_extent(height, kernel_h, pad_h, stride_h, dilation_h);
+  const size_t output_w = conv_output_extent(width, kernel_w, pad_w, stride_w, dilation_w);
+  const size_t taps = kernel_h * kernel_w;
+#pragma omp parallel for schedule(static) collapse(2)
+  for (long long bb = 0; bb < (long long)batch_count; ++bb) {
+    for (long long ff = 0; ff < (long long)num_kernels; ++ff) {
+      const size_t b = (size_t)bb, f = (size_t)ff;
+      for (size_t oh = 0; oh < output_h; ++oh) {
+        for (size_t ow = 0; ow < output_w; ++ow) {
+          long double sum = 0.0L;
+          for (size_t c = 0; c < channels; ++c) {
+            for (size_t kh = 0; kh < kernel_h; ++kh) {
+              for (size_t kw = 0; kw < kernel_w; ++kw) {
+                const long long h = (long long)(oh * stride_h + kh * dilation_h) - (long long)pad_h;
+                const long long w = (long long)(ow * stride_w + kw * dilation_w) - (long long)pad_w;
+                if (h < 0 || h >= (long long)height || w < 0 || w >= (long long)width) continue;
+                const size_t tap = kh * kernel_w + kw;
+                const size_t kernel_index = (kernel_mode == kConvolution) ? (taps - 1 - tap) : tap;
+                sum += (long double)load_as_double(image, bits, image_offset + ((b * channels + c) * height + (size_t)h) * width + (size_t)w) *
+                       (long double)load_as_double(kernels, bits, kernel_offset + (f * channels + c) * taps + kernel_index);
+              }
+            }
+          }
+          result[((b * num_kernels + f) * output_h + oh) * output_w + ow] = (double)sum;
+        }
+      }
     }
   }
   return kSuccess;

@@ -11,7 +11,9 @@ HIP (both runtimes in one process were seen to lose the device), hence the comma
     python -m oracle.reference_opencl --spec spec.json --out result.npz
 
 spec.json: {"routine": "gemm"|"strided"|"symm" (then "side", "triangle" instead of "ta", "tb", "k")|"trmm"|"trsm" ("side",
-"triangle", "ta", "diagonal"; the result is the B buffer)|"syrk"|"syr2k" ("triangle", "ta", "n", "k"), "bits": 16|32|64, "layout", "ta", "tb", "m", "n", "k", "alpha", "beta",
+"triangle", "ta", "diagonal"; the result is the B buffer)|"syrk"|"syr2k" ("triangle", "ta", "n", "k")|"convgemm" ("kernel_mode",
+"conv": [channels, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w, num_kernels,
+batch_count]; buffers a, b, c are the images, the kernels and the result), "bits": 16|32|64, "layout", "ta", "tb", "m", "n", "k", "alpha", "beta",
 "a_ld", "b_ld", "c_ld", "offsets": [a, b, c], "seed": s, "low"/"high", "ab_low"/"ab_high", "batch", "strides",
 "runs": r, "sizes": [a, b, c] element counts, "complex": true for CLBlastCgemm/Zgemm ("bits" is then the width of one
 component, "alpha"/"beta" are [re, im] pairs)}. Inputs are oracle.uniform(seed*3 + {0,1,2}, ...), exactly what
@@ -141,15 +143,20 @@ def run(spec):
     in_place_b = spec["routine"] in ("trmm", "trsm")  # these overwrite B; "c" is then unused
     sz, vp = ctypes.c_size_t, ctypes.c_void_p
     queue = vp(opencl.queue.value)
-    alpha = scalar_argument(bits, spec["alpha"], reference, is_complex)
+    alpha = scalar_argument(bits, spec.get("alpha", 1.0), reference, is_complex)
     beta = scalar_argument(bits, spec.get("beta", 0.0), reference, is_complex)
     prefix = {32: "C", 64: "Z"}[bits] if is_complex else PREFIX[bits]
     offsets = spec.get("offsets", [0, 0, 0])
-    m, n, k = sz(spec.get("m", 0)), sz(spec["n"]), sz(spec.get("k", 0))
+    m, n, k = sz(spec.get("m", 0)), sz(spec.get("n", 0)), sz(spec.get("k", 0))
 
     def call():
         event = vp(None)
-        if in_place_b:
+        if spec["routine"] == "convgemm":  # a = images, b = kernels, c = result; "conv": the 13 size_t arguments in order
+            function = getattr(reference, "CLBlast%sconvgemm" % PREFIX[bits])
+            status = function(ctypes.c_int(spec["kernel_mode"]), *[sz(value) for value in spec["conv"]], a_buffer,
+                              sz(offsets[0]), b_buffer, sz(offsets[1]), c_buffer, sz(offsets[2]), ctypes.byref(queue),
+                              ctypes.byref(event))
+        elif in_place_b:
             function = getattr(reference, "CLBlast%s%s" % (PREFIX[bits], spec["routine"]))
             status = function(ctypes.c_int(spec["layout"]), ctypes.c_int(spec["side"]), ctypes.c_int(spec["triangle"]),
                               ctypes.c_int(spec["ta"]), ctypes.c_int(spec["diagonal"]), m, n, alpha, a_buffer,

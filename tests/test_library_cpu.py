@@ -17,7 +17,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def declared_functions(header):
     text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"//[^\n]*", "", text)
-    return set(re.findall(r"\b(CLBlast[A-Za-z0-9]+|clbh_[a-z_]+|cblas_[a-z0-9]+)\s*\(", text))
+    return set(re.findall(r"\b(CLBlast[A-Za-z0-9]+|clbh_[a-z0-9_]+|cblas_[a-z0-9]+)\s*\(", text))
 
 
 def test_library_loads_and_exports_every_declared_symbol():
@@ -34,7 +34,7 @@ def test_cpp_api_instantiations_are_exported():
     """The C++ templates of clblast_hip.h are exported for half, float and double."""
     import subprocess
     symbols = subprocess.run(["nm", "-D", "--defined-only", "-C", _lib.LIB_PATH], capture_output=True, text=True).stdout
-    for routine in ("Gemm", "GemmBatched", "GemmStridedBatched", "GemmTempBufferSize", "Symm", "Syrk", "Syr2k", "Trmm", "Trsm"):
+    for routine in ("Gemm", "GemmBatched", "GemmStridedBatched", "GemmTempBufferSize", "Symm", "Syrk", "Syr2k", "Trmm", "Trsm", "Convgemm"):
         for type_name in ("float", "double", "unsigned short"):
             if routine == "Trsm" and type_name == "unsigned short":
                 continue  # like the reference: no half-precision TRSM
