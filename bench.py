@@ -211,6 +211,46 @@ class ComplexWorkload:
         return float(((self.c.to(torch.complex128) @ x) - expected).norm() / expected.norm())
 
 
+class ConvWorkload:
+    """CONVGEMM: `batch` images of channels x size x size against num_kernels kernels of 3 x 3, padding 1, stride 1
+    (cross-correlation). 2 * outputs * channels * 9 flops."""
+
+    def __init__(self, name, prefix, channels, size, num_kernels, batch):
+        import torch
+        self.name, self.prefix, self.beta = name, prefix, 0.0
+        self.channels, self.size, self.num_kernels, self.batch = channels, size, num_kernels, batch
+        dtype = {"S": torch.float32, "D": torch.float64, "H": torch.float16}[prefix]
+        generator = torch.Generator(device="cuda")
+        generator.manual_seed(2024)
+        self.image = torch.rand(batch, channels, size, size, device="cuda", generator=generator).sub_(0.5).to(dtype)
+        self.weights = torch.rand(num_kernels, channels, 3, 3, device="cuda", generator=generator).sub_(0.5).to(dtype)
+        self.result = torch.empty(batch, num_kernels, size, size, device="cuda", dtype=dtype)
+        self.c_initial = None
+
+    @property
+    def flops(self):
+        return 2.0 * self.batch * self.num_kernels * self.size * self.size * self.channels * 9
+
+    @property
+    def algorithmic_bytes(self):
+        element = BITS[self.prefix] // 8
+        return element * (self.image.numel() + self.weights.numel() + self.result.numel())
+
+    def call(self, stream_handle):
+        from clblast_amd.api import raw_convgemm
+        status = raw_convgemm(self.prefix, 151, self.channels, self.size, self.size, 3, 3, 1, 1, 1, 1, 1, 1, self.num_kernels,
+                              self.batch, self.image.data_ptr(), 0, self.weights.data_ptr(), 0, self.result.data_ptr(), 0,
+                              stream_handle)
+        if status != 0:
+            raise RuntimeError("%s: status %d" % (self.name, status))
+
+    def freivalds_error(self):
+        """Against torch's conv2d in fp32 on one image (the check of a convolution is a convolution)."""
+        import torch
+        expected = torch.nn.functional.conv2d(self.image[:1].float(), self.weights.float(), None, 1, 1, 1)
+        return float((self.result[:1].float() - expected).norm() / expected.norm())
+
+
 class TrmmWorkload(Workload):
     """TRMM in place, B := alpha op(A) B with A m x m triangular on the left (column-major). The unused triangle holds
     NaN. Repeated calls multiply B by A again and again, so A is close to the identity (unit-sized diagonal,
@@ -407,6 +447,10 @@ def reference_on_this_gpu(runs=3):
              "cgemm_4096_rowNC": dict(routine="gemm", complex=True, bits=32, layout=ROW, ta=NO, tb=113, m=4096, n=4096, k=4096,
                                       alpha=[1.0, -0.5], beta=[0.0, 0.0], a_ld=4096, b_ld=4096, c_ld=4096, offsets=[0, 0, 0],
                                       seed=14, runs=3, sizes=[4096 * 4096] * 3),
+             "sconvgemm_64x112x112_k128_b8": dict(routine="convgemm", bits=32, kernel_mode=151,
+                                                  conv=[64, 112, 112, 3, 3, 1, 1, 1, 1, 1, 1, 128, 8], m=8 * 112 * 112, n=128,
+                                                  k=64 * 9, offsets=[0, 0, 0], seed=15, runs=5,
+                                                  sizes=[8 * 64 * 112 * 112, 128 * 64 * 9, 8 * 128 * 112 * 112]),
              "ssyrk_4096_colLower": dict(routine="syrk", bits=32, layout=COL, triangle=122, ta=NO, m=4096, n=4096, k=4096,
                                          alpha=1.0, beta=0.0, a_ld=4096, b_ld=4096, c_ld=4096, offsets=[0, 0, 0], seed=11,
                                          runs=5, sizes=[4096 * 4096] * 3),
@@ -456,6 +500,8 @@ EXTRA_WORKLOADS = {
                                                         132, 8198, (11, 13, 19)),
     "next_cgemm_4096_rowNC": lambda: ComplexWorkload("cgemm", "C", NO, 113, 4096, 4096, 4096, 1.0 - 0.5j, 0.0),
     "next_zgemm_2048_rowTN": lambda: ComplexWorkload("zgemm", "Z", YES, NO, 2048, 2048, 2048, 0.5 + 1.0j, 1.0 - 0.5j),
+    "next_sconvgemm_64x112x112_k128_b8": lambda: ConvWorkload("conv_s", "S", 64, 112, 128, 8),
+    "next_hconvgemm_64x112x112_k128_b8": lambda: ConvWorkload("conv_h", "H", 64, 112, 128, 8),
     "next_ssymm_4096_colLeftUpper": lambda: SymmWorkload("symm_s", "S", COL, True, 4096, 4096, 1.0, 0.0),
     "next_hsymm_4096_rowLeftLower": lambda: SymmWorkload("symm_h", "H", ROW, False, 4096, 4096, 1.0, 0.0),
     "next_strmm_4096_colLeftLower": lambda: TrmmWorkload("trmm_s", "S", "trmm", True, False, 4096, 4096),

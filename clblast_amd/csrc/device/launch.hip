@@ -208,6 +208,26 @@ int LaunchComplexScale(const int m, const int n, const double beta_re, const dou
 }
 }  // namespace
 
+namespace {
+template <typename T>
+int LaunchIm2col(const clbh::Im2colShape& s, const int batch_count, const void* image, const long long image_offset, void* col,
+                 hipStream_t stream) {
+  constexpr int VEC = 16 / sizeof(T);
+  const int patches = s.output_h * s.output_w;
+  const bool vector = patches % VEC == 0 && reinterpret_cast<unsigned long long>(col) % 16 == 0;
+  const int lanes = vector ? patches / VEC : patches;
+  const dim3 grid(static_cast<unsigned>((lanes + clbh::kIm2colThreads - 1) / clbh::kIm2colThreads),
+                  static_cast<unsigned>(std::min(s.channels, 65535)), static_cast<unsigned>(std::min(batch_count, 65535)));
+  const T* source = static_cast<const T*>(image) + image_offset;
+  if (vector) {
+    clbh::Im2colKernel<T, VEC><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(s, batch_count, source, static_cast<T*>(col));
+  } else {
+    clbh::Im2colKernel<T, 1><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(s, batch_count, source, static_cast<T*>(col));
+  }
+  return static_cast<int>(hipGetLastError());
+}
+}  // namespace
+
 extern "C" {
 
 int clbh_gemm_launch(const clbh_gemm_desc* desc, hipStream_t stream) {
@@ -322,18 +342,12 @@ int clbh_im2col(int precision, const clbh_im2col_shape* shape, int batch_count, 
   s.kernel_h = g.kernel_h; s.kernel_w = g.kernel_w; s.pad_h = g.pad_h; s.pad_w = g.pad_w;
   s.stride_h = g.stride_h; s.stride_w = g.stride_w; s.dilation_h = g.dilation_h; s.dilation_w = g.dilation_w;
   s.output_h = g.output_h; s.output_w = g.output_w; s.flip = g.flip;
-  const dim3 grid(static_cast<unsigned>((patches + clbh::kIm2colThreads - 1) / clbh::kIm2colThreads),
-                  static_cast<unsigned>(std::min<long long>(rows, 65535)), static_cast<unsigned>(std::min(batch_count, 65535)));
   switch (precision) {
-    case 16: clbh::Im2colKernel<_Float16><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(
-                 s, batch_count, static_cast<const _Float16*>(image) + image_offset, static_cast<_Float16*>(col)); break;
-    case 32: clbh::Im2colKernel<float><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(
-                 s, batch_count, static_cast<const float*>(image) + image_offset, static_cast<float*>(col)); break;
-    case 64: clbh::Im2colKernel<double><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(
-                 s, batch_count, static_cast<const double*>(image) + image_offset, static_cast<double*>(col)); break;
+    case 16: return LaunchIm2col<_Float16>(s, batch_count, image, image_offset, col, stream);
+    case 32: return LaunchIm2col<float>(s, batch_count, image, image_offset, col, stream);
+    case 64: return LaunchIm2col<double>(s, batch_count, image, image_offset, col, stream);
     default: return hipErrorInvalidValue;
   }
-  return static_cast<int>(hipGetLastError());
 }
 
 int clbh_alloc(void** ptr, size_t bytes) {

@@ -24,32 +24,43 @@ struct Im2colShape {
 
 constexpr int kIm2colThreads = 256;
 
-// grid: (ceil(output_w * output_h / 256), min(channels * kernel_h * kernel_w, 65535), min(batch, 65535)); rows and
-// batches beyond the grid are covered by grid-stride loops
-template <typename T>
+// grid: (ceil(patches / (256 * VEC)), min(channels, 65535), min(batch, 65535)); channels and batches beyond the grid
+// are covered by grid-stride loops. A thread owns VEC consecutive patches (VEC > 1 needs patches % VEC == 0 and 16-byte
+// aligned col) and walks all taps of its channel: VEC loads and one VEC-wide store per tap.
+template <typename T, int VEC>
 __global__ __launch_bounds__(kIm2colThreads) void Im2colKernel(const Im2colShape s, const int batch_count,
                                                                const T* __restrict__ image, T* __restrict__ col) {
-  const int patch = blockIdx.x * kIm2colThreads + threadIdx.x;
+  typedef T Vector __attribute__((ext_vector_type(VEC)));
+  const int patch = (blockIdx.x * kIm2colThreads + threadIdx.x) * VEC;
   const int patches = s.output_h * s.output_w;
   if (patch >= patches) { return; }
   const int taps = s.kernel_h * s.kernel_w;
-  const int rows = s.channels * taps;
-  const int oh = patch / s.output_w, ow = patch % s.output_w;
-  const long long image_size = static_cast<long long>(s.channels) * s.height * s.width;
+  int h_base[VEC], w_base[VEC];  // top-left corner of each patch in the (padded) image
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    h_base[v] = ((patch + v) / s.output_w) * s.stride_h - s.pad_h;
+    w_base[v] = ((patch + v) % s.output_w) * s.stride_w - s.pad_w;
+  }
+  const long long plane = static_cast<long long>(s.height) * s.width;
   for (int batch = blockIdx.z; batch < batch_count; batch += gridDim.z) {
-    const T* source = image + batch * image_size;
-    T* destination = col + static_cast<long long>(batch) * rows * patches;
-    for (int row = blockIdx.y; row < rows; row += gridDim.y) {
-      const int channel = row / taps, tap = row % taps;
-      const int kh = tap / s.kernel_w, kw = tap % s.kernel_w;
-      const int h = oh * s.stride_h - s.pad_h + kh * s.dilation_h;
-      const int w = ow * s.stride_w - s.pad_w + kw * s.dilation_w;
-      T value = T(0);
-      if (h >= 0 && h < s.height && w >= 0 && w < s.width) {
-        value = source[(static_cast<long long>(channel) * s.height + h) * s.width + w];
+    for (int channel = blockIdx.y; channel < s.channels; channel += gridDim.y) {
+      const T* source = image + (static_cast<long long>(batch) * s.channels + channel) * plane;
+      T* destination = col + ((static_cast<long long>(batch) * s.channels + channel) * taps) * patches + patch;
+      for (int kh = 0; kh < s.kernel_h; ++kh) {
+        for (int kw = 0; kw < s.kernel_w; ++kw) {
+          Vector value;
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            const int h = h_base[v] + kh * s.dilation_h, w = w_base[v] + kw * s.dilation_w;
+            const bool inside = (h >= 0 && h < s.height && w >= 0 && w < s.width);
+            value[v] = inside ? source[h * s.width + w] : T(0);
+          }
+          const int tap = kh * s.kernel_w + kw;
+          const int kernel_index = s.flip ? (taps - 1 - tap) : tap;
+          T* target = destination + static_cast<long long>(kernel_index) * patches;
+          if constexpr (VEC == 1) { *target = value[0]; } else { *reinterpret_cast<Vector*>(target) = value; }
+        }
       }
-      const int kernel_index = s.flip ? (taps - 1 - tap) : tap;
-      destination[(static_cast<long long>(channel) * taps + kernel_index) * patches + patch] = value;
     }
   }
 }
