@@ -101,4 +101,4 @@ DEVICE_LAYER_SYMBOLS = [
     "clbh_gemm_launch", "clbh_gemm_workspace_bytes", "clbh_buffer_extent", "clbh_alloc_async", "clbh_free_async",
     "clbh_upload_async", "clbh_event_record", "clbh_stream_device", "clbh_error_string", "clbh_symmetric_to_square",
     "clbh_triangular_to_square", "clbh_copy_matrix", "clbh_invert_block_size", "clbh_invert_diagonal_blocks",
-    "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale", "clbh_alloc", "clbh_free", "clbh_copy", "clbh_im2col"]
+    "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale", "clbh_alloc", "clbh_free", "clbh_copy", "clbh_im2col", "clbh_fill_zero"]

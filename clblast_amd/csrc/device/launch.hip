@@ -140,7 +140,7 @@ int LaunchTriangularToSquare(const int upper, const int unit, const int k, const
 
 template <typename T, typename CT, int BLOCK>
 int LaunchInvertDiagonalBlocks(const int upper, const int blocks, const void* src, const long long src_ld, void* dst,
-                               hipStream_t stream) {
+                               const long long dst_ld, hipStream_t stream) {
   constexpr size_t lds_bytes = clbh::InvertLds<CT, BLOCK>::BYTES;
   auto kernel = clbh::InvertDiagonalBlocksKernel<T, CT, BLOCK>;
   if (lds_bytes > 48 * 1024) {
@@ -149,7 +149,7 @@ int LaunchInvertDiagonalBlocks(const int upper, const int blocks, const void* sr
     if (attribute_status != hipSuccess) { return static_cast<int>(attribute_status); }
   }
   kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(clbh::kInvertThreads), lds_bytes, stream>>>(
-      upper != 0, static_cast<const T*>(src), src_ld, static_cast<T*>(dst));
+      upper != 0, static_cast<const T*>(src), src_ld, static_cast<T*>(dst), dst_ld);
   return static_cast<int>(hipGetLastError());
 }
 
@@ -269,16 +269,24 @@ int clbh_triangular_to_square(int precision, int upper, int unit_diagonal, int k
 int clbh_invert_block_size(int precision) { return (precision == 64) ? 64 : 128; }
 
 int clbh_invert_diagonal_blocks(int precision, int upper, int blocks, const void* src, long long src_ld, void* dst,
-                                hipStream_t stream) {
-  if (blocks <= 0 || src == nullptr || dst == nullptr || src_ld < static_cast<long long>(blocks) * clbh_invert_block_size(precision)) {
-    return hipErrorInvalidValue;
-  }
+                                long long dst_ld, hipStream_t stream) {
+  const long long extent = static_cast<long long>(blocks) * clbh_invert_block_size(precision);
+  if (blocks <= 0 || src == nullptr || dst == nullptr || src_ld < extent || dst_ld < extent) { return hipErrorInvalidValue; }
   switch (precision) {
-    case 16: return LaunchInvertDiagonalBlocks<_Float16, float, 128>(upper, blocks, src, src_ld, dst, stream);
-    case 32: return LaunchInvertDiagonalBlocks<float, float, 128>(upper, blocks, src, src_ld, dst, stream);
-    case 64: return LaunchInvertDiagonalBlocks<double, double, 64>(upper, blocks, src, src_ld, dst, stream);
+    case 16: return LaunchInvertDiagonalBlocks<_Float16, float, 128>(upper, blocks, src, src_ld, dst, dst_ld, stream);
+    case 32: return LaunchInvertDiagonalBlocks<float, float, 128>(upper, blocks, src, src_ld, dst, dst_ld, stream);
+    case 64: return LaunchInvertDiagonalBlocks<double, double, 64>(upper, blocks, src, src_ld, dst, dst_ld, stream);
     default: return hipErrorInvalidValue;
   }
+}
+
+int clbh_fill_zero(void* ptr, size_t bytes, hipStream_t stream) {
+  if (ptr == nullptr || bytes % 16 != 0 || reinterpret_cast<unsigned long long>(ptr) % 16 != 0) { return hipErrorInvalidValue; }
+  if (bytes == 0) { return 0; }
+  const long long words = static_cast<long long>(bytes / 16);
+  const unsigned blocks = static_cast<unsigned>(std::min<long long>((words + clbh::kCopyThreads - 1) / clbh::kCopyThreads, 8192));
+  clbh::FillZeroKernel<<<dim3(blocks), dim3(clbh::kCopyThreads), 0, stream>>>(static_cast<uint4*>(ptr), words);
+  return static_cast<int>(hipGetLastError());
 }
 
 int clbh_copy_matrix(int precision, int one_extent, int two_extent, const void* src, long long src_offset, long long src_ld,

@@ -73,8 +73,8 @@ __global__ __launch_bounds__(kCopyThreads) void CopyMatrixKernel(const int one_e
 //      off-diagonal part of a pair of neighbouring inverted blocks, inverse(R, C) = -inverse(R, R) * A(R, C) *
 //      inverse(C, C), two small products per level in which every thread owns a few elements of the result.
 // LDS rows have an odd pitch, so that lanes walking down a column and lanes walking along a row both spread over
-// the banks. src must hold blocks * BLOCK rows and columns; block b of the result is the dense matrix at
-// dst + b * BLOCK * BLOCK with leading dimension BLOCK.
+// the banks. src must hold blocks * BLOCK rows and columns; block b of the result goes to the same place of dst as
+// it has in src: dst + b * BLOCK * (dst_ld + 1) with leading dimension dst_ld.
 constexpr int kInvertThreads = 256;
 constexpr int kInvertBase = 16;
 
@@ -88,7 +88,8 @@ struct InvertLds {
 
 template <typename T, typename CT, int BLOCK>
 __global__ __launch_bounds__(kInvertThreads) void InvertDiagonalBlocksKernel(const bool upper, const T* __restrict__ src,
-                                                                             const long long src_ld, T* __restrict__ dst) {
+                                                                             const long long src_ld, T* __restrict__ dst,
+                                                                             const long long dst_ld) {
   constexpr int PITCH = InvertLds<CT, BLOCK>::PITCH, TEMP_PITCH = InvertLds<CT, BLOCK>::TEMP_PITCH;
   extern __shared__ __attribute__((aligned(16))) unsigned char invert_lds[];
   CT* matrix = reinterpret_cast<CT*>(invert_lds);  // [row * PITCH + column]: element (row, column) of the block
@@ -148,10 +149,18 @@ __global__ __launch_bounds__(kInvertThreads) void InvertDiagonalBlocksKernel(con
     __syncthreads();
   }
 
-  T* result = dst + static_cast<long long>(blockIdx.x) * BLOCK * BLOCK;
+  T* result = dst + static_cast<long long>(blockIdx.x) * BLOCK * (dst_ld + 1);
   for (int index = tid; index < BLOCK * BLOCK; index += kInvertThreads) {
     const int row = index % BLOCK, column = index / BLOCK;
-    result[column * BLOCK + row] = static_cast<T>(inverse[row * PITCH + column]);
+    result[column * dst_ld + row] = static_cast<T>(inverse[row * PITCH + column]);
+  }
+}
+
+// Fills `count` 16-byte words with zeros (a kernel rather than a memset node, so that callers may capture it).
+__global__ __launch_bounds__(kCopyThreads) void FillZeroKernel(uint4* __restrict__ words, const long long count) {
+  for (long long index = static_cast<long long>(blockIdx.x) * kCopyThreads + threadIdx.x; index < count;
+       index += static_cast<long long>(gridDim.x) * kCopyThreads) {
+    words[index] = make_uint4(0u, 0u, 0u, 0u);
   }
 }
 

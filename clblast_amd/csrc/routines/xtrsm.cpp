@@ -3,6 +3,8 @@
 // =================================================================================================
 #include "routines/xtrsm.hpp"
 
+#include "routines/xgemmbatched.hpp"
+
 #include <climits>
 #include <functional>
 #include <utility>
@@ -45,13 +47,17 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
   TestMatrixB(m, n, b_buffer, b_offset, b_ld);
 
   const auto precision = static_cast<int>(PrecisionValue<T>());
-  const auto stream = this->stream();
-  const auto block = static_cast<size_t>(clbh_invert_block_size(precision));
-  const auto blocks = (k + block - 1) / block;
-  const auto k_padded = blocks * block;
+  auto stream = this->stream();
   constexpr size_t kLineMultiple = 16 / sizeof(T);
+  // Diagonal blocks: `block` is what the inversion kernel inverts; the inverses are then doubled in size with GEMMs
+  // up to the leaf size of the recursion (at most kMaxLeaf, and no more doublings than the matrix has use for)
+  constexpr size_t kMaxLeaf = 512;
+  const auto block = static_cast<size_t>(clbh_invert_block_size(precision));
+  auto leaf = block;
+  while (leaf < kMaxLeaf && leaf < k) { leaf *= 2; }
+  const auto k_padded = (k + leaf - 1) / leaf * leaf;
 
-  // Dense copy of the triangle, padded with the identity to whole blocks: the other triangle becomes zeros, an
+  // Dense copy of the triangle, padded with the identity to whole leaves: the other triangle becomes zeros, an
   // implied diagonal ones, and no block operation below has a ragged edge on the A side
   const auto dense_bytes = k_padded * k_padded * sizeof(T);
   const StreamScratch dense(dense_bytes, stream, "dense copy of the triangular matrix");
@@ -61,20 +67,47 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
                                         static_cast<long long>(a_ld), dense.get(), static_cast<int>(k_padded),
                                         static_cast<long long>(k_padded), stream),
               "clbh_triangular_to_square");
-  // Inverses of the diagonal blocks (xtrsm.cpp:105-118 with Xinvert)
-  const auto inverse_bytes = blocks * block * block * sizeof(T);
-  const StreamScratch inverses(inverse_bytes, stream, "inverted diagonal blocks");
-  CheckDevice(clbh_invert_diagonal_blocks(precision, is_upper ? 1 : 0, static_cast<int>(blocks), dense.get(),
-                                          static_cast<long long>(k_padded), inverses.get(), stream),
+  const auto dense_buffer = Buffer<T>(dense.get(), dense_bytes);
+
+  // Inverses of the diagonal leaves (xtrsm.cpp:105-118 with Xinvert), kept in a matrix of the same shape as the dense
+  // copy, each inverse in the place of its block, zeros elsewhere
+  const StreamScratch inverses(dense_bytes, stream, "inverted diagonal blocks");
+  CheckDevice(clbh_fill_zero(inverses.get(), dense_bytes, stream), "clbh_fill_zero");
+  CheckDevice(clbh_invert_diagonal_blocks(precision, is_upper ? 1 : 0, static_cast<int>(k_padded / block), dense.get(),
+                                          static_cast<long long>(k_padded), inverses.get(),
+                                          static_cast<long long>(k_padded), stream),
               "clbh_invert_diagonal_blocks");
+  const auto inverse_buffer = Buffer<T>(inverses.get(), dense_bytes);
+  if (leaf > block) {
+    // Doubling (xinvert.cpp:103-140 does the same with dedicated kernels): for two neighbouring inverted blocks of
+    // extent `size`, with R the rows and C the columns of the off-diagonal block between them,
+    // inverse(R, C) = -inverse(R, R) * A(R, C) * inverse(C, C). All pairs of a level sit at a constant distance along
+    // the diagonal: two strided-batched GEMMs per level.
+    const auto product_bytes = (k_padded / 2) * (leaf / 2) * sizeof(T);
+    const StreamScratch products(product_bytes, stream, "block products of the inversion");
+    const auto product_buffer = Buffer<T>(products.get(), product_bytes);
+    auto batched = XgemmStridedBatched<T>(&stream, nullptr);
+    for (auto size = block; size < leaf; size *= 2) {
+      const auto pairs = k_padded / (2 * size);
+      const auto diagonal_step = 2 * size * (k_padded + 1);
+      const auto rows = is_upper ? size_t{0} : size, columns = is_upper ? size : size_t{0};
+      const auto at = [&](const size_t r, const size_t c) { return r + c * k_padded; };
+      batched.DoGemmStridedBatched(Layout::kColMajor, Transpose::kNo, Transpose::kNo, size, size, size, ConstantOne<T>(),
+                                   dense_buffer, at(rows, columns), k_padded, diagonal_step, inverse_buffer,
+                                   at(columns, columns), k_padded, diagonal_step, ConstantZero<T>(), product_buffer, 0, size,
+                                   size * size, pairs);
+      batched.DoGemmStridedBatched(Layout::kColMajor, Transpose::kNo, Transpose::kNo, size, size, size, ConstantNegOne<T>(),
+                                   inverse_buffer, at(rows, rows), k_padded, diagonal_step, product_buffer, 0, size,
+                                   size * size, ConstantZero<T>(), inverse_buffer, at(rows, columns), k_padded, diagonal_step,
+                                   pairs);
+    }
+  }
   // The solution is built in a buffer of its own and copied over B at the end: the block products read B while
   // they write X (xtrsm.cpp:91-99, 243)
   const auto x_ld = (m + kLineMultiple - 1) / kLineMultiple * kLineMultiple;
   const auto x_bytes = x_ld * n * sizeof(T);
   const StreamScratch solution(x_bytes, stream, "solution of the triangular system");
 
-  const auto dense_buffer = Buffer<T>(dense.get(), dense_bytes);
-  const auto inverse_buffer = Buffer<T>(inverses.get(), inverse_bytes);
   const auto x_buffer = Buffer<T>(solution.get(), x_bytes);
   const auto no_temp = Buffer<T>(nullptr);
   const auto one = ConstantOne<T>();
@@ -101,19 +134,19 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
   // alpha (by an update); alpha multiplies every element of B exactly once, in the first product that reads it.
   std::function<void(size_t, size_t, bool)> solve = [&](const size_t lo, const size_t hi, const bool scaled) {
     const auto factor = scaled ? one : alpha;
-    if (hi - lo <= block) {
+    if (hi - lo <= leaf) {
       const auto size = hi - lo;
-      const auto inverse_offset = (lo / block) * block * block;
+      const auto inverse_offset = lo * (k_padded + 1);
       if (side == Side::kLeft) {  // X[lo:hi, :] = factor * op(inverse) * B[lo:hi, :]
-        gemm(a_transpose, no, size, n, size, factor, inverse_buffer, inverse_offset, block, b_buffer, b_offset + lo, b_ld, zero,
+        gemm(a_transpose, no, size, n, size, factor, inverse_buffer, inverse_offset, k_padded, b_buffer, b_offset + lo, b_ld, zero,
              x_buffer, lo, x_ld);
       } else {                    // X[:, lo:hi] = factor * B[:, lo:hi] * op(inverse)
         gemm(no, a_transpose, m, size, size, factor, b_buffer, b_offset + lo * b_ld, b_ld, inverse_buffer, inverse_offset,
-             block, zero, x_buffer, lo * x_ld, x_ld);
+             k_padded, zero, x_buffer, lo * x_ld, x_ld);
       }
       return;
     }
-    const auto mid = lo + ((hi - lo + block - 1) / block / 2) * block;  // a multiple of the block size inside (lo, hi)
+    const auto mid = lo + ((hi - lo + leaf - 1) / leaf / 2) * leaf;  // a multiple of the leaf size inside (lo, hi)
     // Left: a lower op(A) is solved from the top, an upper one from the bottom; right: the other way round
     const bool first_half_first = (side == Side::kLeft) ? op_lower : !op_lower;
     const auto done_lo = first_half_first ? lo : mid, done_hi = first_half_first ? mid : hi;  // solved first

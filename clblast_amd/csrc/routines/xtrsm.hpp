@@ -5,8 +5,9 @@
 // The reference walks the diagonal in blocks of 16: it inverts the 16 x 16 diagonal blocks, and for every block
 // runs one small GEMM with the inverse and one GEMM that updates the rest of B, synchronising with the host in
 // between. The structure here is the same - inverted diagonal blocks, everything else is GEMM - but recursive and
-// stream-ordered: the diagonal blocks are 128 x 128 (64 x 64 in fp64) and inverted by one kernel, and the triangle is
-// halved recursively, so that the bulk of the work is a few GEMMs with a long K instead of many rank-16 updates.
+// stream-ordered: one kernel inverts the 128 x 128 (fp64: 64 x 64) diagonal blocks, strided-batched GEMMs double the
+// inverses up to 512 x 512 leaves, and the triangle is halved recursively, so that the bulk of the work is a few
+// GEMMs with a long K instead of many rank-16 updates.
 // =================================================================================================
 #ifndef CLBLAST_HIP_ROUTINES_XTRSM_HPP_
 #define CLBLAST_HIP_ROUTINES_XTRSM_HPP_

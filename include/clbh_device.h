@@ -97,9 +97,12 @@ CLBH_API int clbh_invert_block_size(int precision);
 
 // Inverts the `blocks` diagonal blocks (clbh_invert_block_size(precision) squared each) of the dense triangular matrix
 // `src` (blocks * block rows and columns, zeros in the other triangle, non-zero diagonal); block b of the result is
-// the dense block x block matrix at dst + b * block * block (leading dimension block).
+// written to the same place of `dst` (leading dimension dst_ld) as it has in `src`: dst + b * block * (dst_ld + 1).
 CLBH_API int clbh_invert_diagonal_blocks(int precision, int upper, int blocks, const void* src, long long src_ld,
-                                         void* dst, hipStream_t stream);
+                                         void* dst, long long dst_ld, hipStream_t stream);
+
+// Zeroes `bytes` bytes (a multiple of 16) at the 16-byte aligned `ptr` with a kernel.
+CLBH_API int clbh_fill_zero(void* ptr, size_t bytes, hipStream_t stream);
 
 // dst[dst_offset + two * dst_ld + one] = src[src_offset + two * src_ld + one] for one < one_extent, two < two_extent.
 CLBH_API int clbh_copy_matrix(int precision, int one_extent, int two_extent, const void* src, long long src_offset,
