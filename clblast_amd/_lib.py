@@ -29,9 +29,24 @@ class Double2(ctypes.Structure):
 
 def _declare(lib):
     sz, vp = c_size_t, c_void_p
-    for prefix, scalar in (("C", Float2), ("Z", Double2)):
+    for prefix, scalar, real in (("C", Float2, c_float), ("Z", Double2, c_double)):
         f = getattr(lib, "CLBlast%sgemm" % prefix)
         f.argtypes = [c_int, c_int, c_int, sz, sz, sz, scalar, vp, sz, sz, vp, sz, sz, scalar, vp, sz, sz, vp, vp]
+        f.restype = c_int
+        for routine in ("symm", "hemm"):
+            f = getattr(lib, "CLBlast%s%s" % (prefix, routine))
+            f.argtypes = [c_int, c_int, c_int, sz, sz, scalar, vp, sz, sz, vp, sz, sz, scalar, vp, sz, sz, vp, vp]
+            f.restype = c_int
+        for routine, alpha_type, beta_type in (("syrk", scalar, scalar), ("herk", real, real)):
+            f = getattr(lib, "CLBlast%s%s" % (prefix, routine))
+            f.argtypes = [c_int, c_int, c_int, sz, sz, alpha_type, vp, sz, sz, beta_type, vp, sz, sz, vp, vp]
+            f.restype = c_int
+        for routine, beta_type in (("syr2k", scalar), ("her2k", real)):
+            f = getattr(lib, "CLBlast%s%s" % (prefix, routine))
+            f.argtypes = [c_int, c_int, c_int, sz, sz, scalar, vp, sz, sz, vp, sz, sz, beta_type, vp, sz, sz, vp, vp]
+            f.restype = c_int
+        f = getattr(lib, "CLBlast%strmm" % prefix)
+        f.argtypes = [c_int] * 5 + [sz, sz, scalar, vp, sz, sz, vp, sz, sz, vp, vp]
         f.restype = c_int
     for prefix in "SDH":
         f = getattr(lib, "CLBlast%sconvgemm" % prefix)
@@ -92,6 +107,7 @@ def load():
 C_API_SYMBOLS = (
     ["CLBlast%sgemm%s" % (p, s) for p in "SDH" for s in ("", "Batched", "StridedBatched", "WithTempBuffer")] +
     ["CLBlast%sGemmTempBufferSize" % p for p in "SDH"] + ["CLBlastCgemm", "CLBlastZgemm"] +
+    ["CLBlast%s%s" % (p, r) for p in "CZ" for r in ("symm", "hemm", "syrk", "herk", "syr2k", "her2k", "trmm")] +
     ["CLBlast%s%s" % (p, r) for p in "SDH" for r in ("symm", "syrk", "syr2k", "trmm")] + ["CLBlastStrsm", "CLBlastDtrsm"] +
     ["CLBlast%sconvgemm" % p for p in "SDH"] +
     ["CLBlastClearCache", "CLBlastOverrideParameters", "CLBlastFloatToHalf", "CLBlastHalfToFloat"])
@@ -101,4 +117,5 @@ DEVICE_LAYER_SYMBOLS = [
     "clbh_gemm_launch", "clbh_gemm_workspace_bytes", "clbh_buffer_extent", "clbh_alloc_async", "clbh_free_async",
     "clbh_upload_async", "clbh_event_record", "clbh_stream_device", "clbh_error_string", "clbh_symmetric_to_square",
     "clbh_triangular_to_square", "clbh_copy_matrix", "clbh_invert_block_size", "clbh_invert_diagonal_blocks",
-    "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale", "clbh_alloc", "clbh_free", "clbh_copy", "clbh_im2col", "clbh_fill_zero"]
+    "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale", "clbh_alloc", "clbh_free", "clbh_copy", "clbh_im2col", "clbh_fill_zero", "clbh_complex_symmetric_to_square",
+    "clbh_complex_triangular_to_square", "clbh_complex_zero_diagonal_imag"]

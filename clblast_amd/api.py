@@ -103,6 +103,23 @@ def raw_convgemm(prefix, kernel_mode, channels, height, width, kernel_h, kernel_
                                                       _stream_ref(stream_handle), event_ref)
 
 
+def raw_complex_level3(routine, prefix, *arguments, stream_handle=0):
+    """CLBlast{C,Z}{symm,hemm,syrk,herk,syr2k,her2k,trmm} through the C ABI (reference: include/clblast_c.h:934-1092).
+    `arguments` are those of the C function up to the last leading dimension; Python complex numbers (or floats for the
+    real scalars of HERK and HER2K) stand for the scalars."""
+    lib = _lib.load()
+    function = getattr(lib, "CLBlast%s%s" % (prefix, routine))
+    scalar = _lib.Float2 if prefix == "C" else _lib.Double2
+    converted = []
+    for value, expected in zip(arguments, function.argtypes):
+        if expected in (_lib.Float2, _lib.Double2):
+            value = complex(value)
+            converted.append(scalar(value.real, value.imag))
+        else:
+            converted.append(value)
+    return function(*converted, _stream_ref(stream_handle), None)
+
+
 def raw_symm(prefix, layout, side, triangle, m, n, alpha, a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld, beta, c_ptr,
              c_offset, c_ld, stream_handle=0, event_handle=None):
     """CLBlast{S,D,H}symm through the C ABI (reference: include/clblast_c.h:921-945)."""

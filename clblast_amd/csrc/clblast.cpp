@@ -277,6 +277,111 @@ StatusCode CLBLAST_HIP_PUBLIC Gemm<double2>(const Layout layout, const Transpose
                              b_ld, beta, c_buffer, c_offset, c_ld, queue, event);
 }
 
+// The complex Level-3 routines (reference: src/clblast.cpp:1110-1330)
+namespace {
+template <typename R, typename Body>
+StatusCode ComplexRoutine(hipStream_t* queue, hipEvent_t* event, Body body) {
+  try {
+    auto routine = Xlevel3Complex<R>(queue, event);
+    body(routine);
+    return StatusCode::kSuccess;
+  } catch (...) {
+    return DispatchException();
+  }
+}
+}  // namespace
+
+#define CLBLAST_HIP_COMPLEX_LEVEL3(R)                                                                                  \
+  template <>                                                                                                          \
+  StatusCode CLBLAST_HIP_PUBLIC Symm<std::complex<R>>(                                                                 \
+      const Layout layout, const Side side, const Triangle triangle, const size_t m, const size_t n,                   \
+      const std::complex<R> alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld, const void* b_buffer, \
+      const size_t b_offset, const size_t b_ld, const std::complex<R> beta, void* c_buffer, const size_t c_offset,     \
+      const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {                                                      \
+    using C = std::complex<R>;                                                                                         \
+    return ComplexRoutine<R>(queue, event, [&](Xlevel3Complex<R>& routine) {                                           \
+      routine.DoSymm(false, layout, side, triangle, m, n, alpha, Buffer<C>(a_buffer), a_offset, a_ld, Buffer<C>(b_buffer), \
+                     b_offset, b_ld, beta, Buffer<C>(c_buffer), c_offset, c_ld);                                       \
+    });                                                                                                                \
+  }                                                                                                                    \
+  template <>                                                                                                          \
+  StatusCode CLBLAST_HIP_PUBLIC Hemm<std::complex<R>>(                                                                 \
+      const Layout layout, const Side side, const Triangle triangle, const size_t m, const size_t n,                   \
+      const std::complex<R> alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld, const void* b_buffer, \
+      const size_t b_offset, const size_t b_ld, const std::complex<R> beta, void* c_buffer, const size_t c_offset,     \
+      const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {                                                      \
+    using C = std::complex<R>;                                                                                         \
+    return ComplexRoutine<R>(queue, event, [&](Xlevel3Complex<R>& routine) {                                           \
+      routine.DoSymm(true, layout, side, triangle, m, n, alpha, Buffer<C>(a_buffer), a_offset, a_ld, Buffer<C>(b_buffer), \
+                     b_offset, b_ld, beta, Buffer<C>(c_buffer), c_offset, c_ld);                                       \
+    });                                                                                                                \
+  }                                                                                                                    \
+  template <>                                                                                                          \
+  StatusCode CLBLAST_HIP_PUBLIC Syrk<std::complex<R>>(                                                                 \
+      const Layout layout, const Triangle triangle, const Transpose a_transpose, const size_t n, const size_t k,       \
+      const std::complex<R> alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,                     \
+      const std::complex<R> beta, void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,        \
+      hipEvent_t* event) {                                                                                             \
+    using C = std::complex<R>;                                                                                         \
+    return ComplexRoutine<R>(queue, event, [&](Xlevel3Complex<R>& routine) {                                           \
+      routine.DoRankUpdate(false, layout, triangle, a_transpose, n, k, alpha, Buffer<C>(a_buffer), a_offset, a_ld, nullptr, \
+                           0, 0, beta, Buffer<C>(c_buffer), c_offset, c_ld);                                           \
+    });                                                                                                                \
+  }                                                                                                                    \
+  template <>                                                                                                          \
+  StatusCode CLBLAST_HIP_PUBLIC Herk<R>(const Layout layout, const Triangle triangle, const Transpose a_transpose,     \
+                                        const size_t n, const size_t k, const R alpha, const void* a_buffer,           \
+                                        const size_t a_offset, const size_t a_ld, const R beta, void* c_buffer,        \
+                                        const size_t c_offset, const size_t c_ld, hipStream_t* queue,                  \
+                                        hipEvent_t* event) {                                                           \
+    using C = std::complex<R>;                                                                                         \
+    return ComplexRoutine<R>(queue, event, [&](Xlevel3Complex<R>& routine) {                                           \
+      routine.DoRankUpdate(true, layout, triangle, a_transpose, n, k, C(alpha, R(0)), Buffer<C>(a_buffer), a_offset, a_ld, \
+                           nullptr, 0, 0, C(beta, R(0)), Buffer<C>(c_buffer), c_offset, c_ld);                         \
+    });                                                                                                                \
+  }                                                                                                                    \
+  template <>                                                                                                          \
+  StatusCode CLBLAST_HIP_PUBLIC Syr2k<std::complex<R>>(                                                                \
+      const Layout layout, const Triangle triangle, const Transpose ab_transpose, const size_t n, const size_t k,      \
+      const std::complex<R> alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld, const void* b_buffer, \
+      const size_t b_offset, const size_t b_ld, const std::complex<R> beta, void* c_buffer, const size_t c_offset,     \
+      const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {                                                      \
+    using C = std::complex<R>;                                                                                         \
+    return ComplexRoutine<R>(queue, event, [&](Xlevel3Complex<R>& routine) {                                           \
+      const auto b = Buffer<C>(b_buffer);                                                                              \
+      routine.DoRankUpdate(false, layout, triangle, ab_transpose, n, k, alpha, Buffer<C>(a_buffer), a_offset, a_ld, &b, \
+                           b_offset, b_ld, beta, Buffer<C>(c_buffer), c_offset, c_ld);                                 \
+    });                                                                                                                \
+  }                                                                                                                    \
+  template <>                                                                                                          \
+  StatusCode CLBLAST_HIP_PUBLIC Her2k<std::complex<R>, R>(                                                             \
+      const Layout layout, const Triangle triangle, const Transpose ab_transpose, const size_t n, const size_t k,      \
+      const std::complex<R> alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld, const void* b_buffer, \
+      const size_t b_offset, const size_t b_ld, const R beta, void* c_buffer, const size_t c_offset, const size_t c_ld, \
+      hipStream_t* queue, hipEvent_t* event) {                                                                         \
+    using C = std::complex<R>;                                                                                         \
+    return ComplexRoutine<R>(queue, event, [&](Xlevel3Complex<R>& routine) {                                           \
+      const auto b = Buffer<C>(b_buffer);                                                                              \
+      routine.DoRankUpdate(true, layout, triangle, ab_transpose, n, k, alpha, Buffer<C>(a_buffer), a_offset, a_ld, &b, \
+                           b_offset, b_ld, C(beta, R(0)), Buffer<C>(c_buffer), c_offset, c_ld);                        \
+    });                                                                                                                \
+  }                                                                                                                    \
+  template <>                                                                                                          \
+  StatusCode CLBLAST_HIP_PUBLIC Trmm<std::complex<R>>(                                                                 \
+      const Layout layout, const Side side, const Triangle triangle, const Transpose a_transpose,                      \
+      const Diagonal diagonal, const size_t m, const size_t n, const std::complex<R> alpha, const void* a_buffer,      \
+      const size_t a_offset, const size_t a_ld, void* b_buffer, const size_t b_offset, const size_t b_ld,              \
+      hipStream_t* queue, hipEvent_t* event) {                                                                         \
+    using C = std::complex<R>;                                                                                         \
+    return ComplexRoutine<R>(queue, event, [&](Xlevel3Complex<R>& routine) {                                           \
+      routine.DoTrmm(layout, side, triangle, a_transpose, diagonal, m, n, alpha, Buffer<C>(a_buffer), a_offset, a_ld,  \
+                     Buffer<C>(b_buffer), b_offset, b_ld);                                                             \
+    });                                                                                                                \
+  }
+CLBLAST_HIP_COMPLEX_LEVEL3(float)
+CLBLAST_HIP_COMPLEX_LEVEL3(double)
+#undef CLBLAST_HIP_COMPLEX_LEVEL3
+
 // TRSM exists for float and double only (reference: src/clblast.cpp:1339-1346)
 template StatusCode CLBLAST_HIP_PUBLIC Trsm<float>(const Layout, const Side, const Triangle, const Transpose, const Diagonal,
                                                    const size_t, const size_t, const float, const void*, const size_t,

@@ -342,6 +342,104 @@ CLBlastStatusCode CLBlastZgemm(const CLBlastLayout layout, const CLBlastTranspos
   });
 }
 
+// ---- complex Level 3 ----------------------------------------------------------------------------
+#define CLBLAST_HIP_TO_COMPLEX_float(v) clblast::float2((v).x, (v).y)
+#define CLBLAST_HIP_TO_COMPLEX_double(v) clblast::double2((v).x, (v).y)
+#define CLBLAST_HIP_COMPLEX_SYMM(NAME, ROUTINE, CTYPE, R)                                                            \
+  CLBlastStatusCode NAME(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,         \
+                         const size_t m, const size_t n, const CTYPE alpha, const void* a_buffer,                    \
+                         const size_t a_offset, const size_t a_ld, const void* b_buffer, const size_t b_offset,      \
+                         const size_t b_ld, const CTYPE beta, void* c_buffer, const size_t c_offset,                 \
+                         const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {                                 \
+    return Guarded([&]() {                                                                                           \
+      return clblast::ROUTINE<std::complex<R>>(L(layout), static_cast<clblast::Side>(side),                          \
+                                               static_cast<clblast::Triangle>(triangle), m, n,                       \
+                                               CLBLAST_HIP_TO_COMPLEX_##R(alpha), a_buffer, a_offset, a_ld, b_buffer, \
+                                               b_offset, b_ld, CLBLAST_HIP_TO_COMPLEX_##R(beta), c_buffer, c_offset, \
+                                               c_ld, queue, event);                                                  \
+    });                                                                                                              \
+  }
+CLBLAST_HIP_COMPLEX_SYMM(CLBlastCsymm, Symm, CLBlastFloat2, float)
+CLBLAST_HIP_COMPLEX_SYMM(CLBlastZsymm, Symm, CLBlastDouble2, double)
+CLBLAST_HIP_COMPLEX_SYMM(CLBlastChemm, Hemm, CLBlastFloat2, float)
+CLBLAST_HIP_COMPLEX_SYMM(CLBlastZhemm, Hemm, CLBlastDouble2, double)
+
+#define CLBLAST_HIP_COMPLEX_SYRK(NAME, CTYPE, R)                                                                     \
+  CLBlastStatusCode NAME(const CLBlastLayout layout, const CLBlastTriangle triangle,                                 \
+                         const CLBlastTranspose a_transpose, const size_t n, const size_t k, const CTYPE alpha,      \
+                         const void* a_buffer, const size_t a_offset, const size_t a_ld, const CTYPE beta,           \
+                         void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,               \
+                         hipEvent_t* event) {                                                                        \
+    return Guarded([&]() {                                                                                           \
+      return clblast::Syrk<std::complex<R>>(L(layout), static_cast<clblast::Triangle>(triangle), Tr(a_transpose), n, k, \
+                                            CLBLAST_HIP_TO_COMPLEX_##R(alpha), a_buffer, a_offset, a_ld,             \
+                                            CLBLAST_HIP_TO_COMPLEX_##R(beta), c_buffer, c_offset, c_ld, queue, event); \
+    });                                                                                                              \
+  }
+CLBLAST_HIP_COMPLEX_SYRK(CLBlastCsyrk, CLBlastFloat2, float)
+CLBLAST_HIP_COMPLEX_SYRK(CLBlastZsyrk, CLBlastDouble2, double)
+
+#define CLBLAST_HIP_HERK(NAME, R)                                                                                    \
+  CLBlastStatusCode NAME(const CLBlastLayout layout, const CLBlastTriangle triangle,                                 \
+                         const CLBlastTranspose a_transpose, const size_t n, const size_t k, const R alpha,          \
+                         const void* a_buffer, const size_t a_offset, const size_t a_ld, const R beta, void* c_buffer, \
+                         const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {          \
+    return Guarded([&]() {                                                                                           \
+      return clblast::Herk<R>(L(layout), static_cast<clblast::Triangle>(triangle), Tr(a_transpose), n, k, alpha,     \
+                              a_buffer, a_offset, a_ld, beta, c_buffer, c_offset, c_ld, queue, event);               \
+    });                                                                                                              \
+  }
+CLBLAST_HIP_HERK(CLBlastCherk, float)
+CLBLAST_HIP_HERK(CLBlastZherk, double)
+
+#define CLBLAST_HIP_COMPLEX_SYR2K(NAME, CTYPE, R)                                                                    \
+  CLBlastStatusCode NAME(const CLBlastLayout layout, const CLBlastTriangle triangle,                                 \
+                         const CLBlastTranspose ab_transpose, const size_t n, const size_t k, const CTYPE alpha,     \
+                         const void* a_buffer, const size_t a_offset, const size_t a_ld, const void* b_buffer,       \
+                         const size_t b_offset, const size_t b_ld, const CTYPE beta, void* c_buffer,                 \
+                         const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {          \
+    return Guarded([&]() {                                                                                           \
+      return clblast::Syr2k<std::complex<R>>(L(layout), static_cast<clblast::Triangle>(triangle), Tr(ab_transpose), n, k, \
+                                             CLBLAST_HIP_TO_COMPLEX_##R(alpha), a_buffer, a_offset, a_ld, b_buffer,  \
+                                             b_offset, b_ld, CLBLAST_HIP_TO_COMPLEX_##R(beta), c_buffer, c_offset,   \
+                                             c_ld, queue, event);                                                    \
+    });                                                                                                              \
+  }
+CLBLAST_HIP_COMPLEX_SYR2K(CLBlastCsyr2k, CLBlastFloat2, float)
+CLBLAST_HIP_COMPLEX_SYR2K(CLBlastZsyr2k, CLBlastDouble2, double)
+
+#define CLBLAST_HIP_HER2K(NAME, CTYPE, R)                                                                            \
+  CLBlastStatusCode NAME(const CLBlastLayout layout, const CLBlastTriangle triangle,                                 \
+                         const CLBlastTranspose ab_transpose, const size_t n, const size_t k, const CTYPE alpha,     \
+                         const void* a_buffer, const size_t a_offset, const size_t a_ld, const void* b_buffer,       \
+                         const size_t b_offset, const size_t b_ld, const R beta, void* c_buffer,                     \
+                         const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {          \
+    return Guarded([&]() {                                                                                           \
+      return clblast::Her2k<std::complex<R>, R>(L(layout), static_cast<clblast::Triangle>(triangle), Tr(ab_transpose), n, \
+                                                k, CLBLAST_HIP_TO_COMPLEX_##R(alpha), a_buffer, a_offset, a_ld, b_buffer, \
+                                                b_offset, b_ld, beta, c_buffer, c_offset, c_ld, queue, event);       \
+    });                                                                                                              \
+  }
+CLBLAST_HIP_HER2K(CLBlastCher2k, CLBlastFloat2, float)
+CLBLAST_HIP_HER2K(CLBlastZher2k, CLBlastDouble2, double)
+
+#define CLBLAST_HIP_COMPLEX_TRMM(NAME, CTYPE, R)                                                                     \
+  CLBlastStatusCode NAME(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,         \
+                         const CLBlastTranspose a_transpose, const CLBlastDiagonal diagonal, const size_t m,         \
+                         const size_t n, const CTYPE alpha, const void* a_buffer, const size_t a_offset,             \
+                         const size_t a_ld, void* b_buffer, const size_t b_offset, const size_t b_ld,                \
+                         hipStream_t* queue, hipEvent_t* event) {                                                    \
+    return Guarded([&]() {                                                                                           \
+      return clblast::Trmm<std::complex<R>>(L(layout), static_cast<clblast::Side>(side),                             \
+                                            static_cast<clblast::Triangle>(triangle), Tr(a_transpose),               \
+                                            static_cast<clblast::Diagonal>(diagonal), m, n,                          \
+                                            CLBLAST_HIP_TO_COMPLEX_##R(alpha), a_buffer, a_offset, a_ld, b_buffer,   \
+                                            b_offset, b_ld, queue, event);                                           \
+    });                                                                                                              \
+  }
+CLBLAST_HIP_COMPLEX_TRMM(CLBlastCtrmm, CLBlastFloat2, float)
+CLBLAST_HIP_COMPLEX_TRMM(CLBlastZtrmm, CLBlastDouble2, double)
+
 // ---- SYRK, SYR2K --------------------------------------------------------------------------------
 #define CLBLAST_HIP_SYRK(NAME, CTYPE, TYPE)                                                                          \
   CLBlastStatusCode NAME(const CLBlastLayout layout, const CLBlastTriangle triangle,                                 \

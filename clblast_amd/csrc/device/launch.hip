@@ -40,7 +40,7 @@ bool ValidDescriptor(const clbh_gemm_desc& d) {
     if (d.c_ld < d.m) { return false; }
   }
   if (d.a_offset < 0 || d.b_offset < 0 || d.c_offset < 0) { return false; }
-  if (d.c_triangle < 0 || d.c_triangle > 2 || d.operand_triangle < 0 || d.operand_triangle > 4) { return false; }
+  if (d.c_triangle < 0 || d.c_triangle > 4 || d.operand_triangle < 0 || d.operand_triangle > 4) { return false; }
   // the one-wavefront-per-matrix kernel knows no triangles
   if ((d.c_triangle != 0 || d.operand_triangle != 0) && d.kernel_class == CLBH_KERNEL_SMALL_BATCHED) { return false; }
   return true;
@@ -199,11 +199,11 @@ int LaunchComplexTranspose(const int k, const int n, const void* src, const long
 }
 
 template <typename R>
-int LaunchComplexScale(const int m, const int n, const double beta_re, const double beta_im, void* c,
+int LaunchComplexScale(const int m, const int n, const int triangle, const double beta_re, const double beta_im, void* c,
                        const long long c_offset, const long long c_ld, hipStream_t stream) {
   const dim3 grid(Blocks(m, clbh::kComplexThreads), static_cast<unsigned>(std::min(n, 16384)));
   clbh::ScaleComplexKernel<R><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
-      m, n, static_cast<R>(beta_re), static_cast<R>(beta_im), static_cast<clbh::ComplexOf<R>*>(c) + c_offset, c_ld);
+      m, n, triangle, static_cast<R>(beta_re), static_cast<R>(beta_im), static_cast<clbh::ComplexOf<R>*>(c) + c_offset, c_ld);
   return static_cast<int>(hipGetLastError());
 }
 }  // namespace
@@ -299,6 +299,9 @@ int clbh_copy_matrix(int precision, int one_extent, int two_extent, const void* 
     case 16: return LaunchCopyMatrix<_Float16>(one_extent, two_extent, src, src_offset, src_ld, dst, dst_offset, dst_ld, stream);
     case 32: return LaunchCopyMatrix<float>(one_extent, two_extent, src, src_offset, src_ld, dst, dst_offset, dst_ld, stream);
     case 64: return LaunchCopyMatrix<double>(one_extent, two_extent, src, src_offset, src_ld, dst, dst_offset, dst_ld, stream);
+    case 128:  // 16-byte elements: twice as many doubles along the contiguous index
+      if (one_extent > INT_MAX / 2) { return hipErrorInvalidValue; }
+      return LaunchCopyMatrix<double>(2 * one_extent, two_extent, src, 2 * src_offset, 2 * src_ld, dst, 2 * dst_offset, 2 * dst_ld, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -326,11 +329,11 @@ int clbh_complex_transpose(int precision, int k, int n, const void* src, long lo
   return hipErrorInvalidValue;
 }
 
-int clbh_complex_scale(int precision, int m, int n, double beta_re, double beta_im, void* c, long long c_offset,
+int clbh_complex_scale(int precision, int m, int n, int triangle, double beta_re, double beta_im, void* c, long long c_offset,
                        long long c_ld, hipStream_t stream) {
-  if (m <= 0 || n <= 0 || c == nullptr || c_offset < 0 || c_ld < m) { return hipErrorInvalidValue; }
-  if (precision == 32) { return LaunchComplexScale<float>(m, n, beta_re, beta_im, c, c_offset, c_ld, stream); }
-  if (precision == 64) { return LaunchComplexScale<double>(m, n, beta_re, beta_im, c, c_offset, c_ld, stream); }
+  if (m <= 0 || n <= 0 || c == nullptr || c_offset < 0 || c_ld < m || triangle < 0 || triangle > 2) { return hipErrorInvalidValue; }
+  if (precision == 32) { return LaunchComplexScale<float>(m, n, triangle, beta_re, beta_im, c, c_offset, c_ld, stream); }
+  if (precision == 64) { return LaunchComplexScale<double>(m, n, triangle, beta_re, beta_im, c, c_offset, c_ld, stream); }
   return hipErrorInvalidValue;
 }
 
@@ -368,6 +371,58 @@ int clbh_free(void* ptr) { return static_cast<int>(hipFree(ptr)); }
 int clbh_copy(void* dst, const void* src, size_t bytes, int to_device) {
   if (dst == nullptr || src == nullptr) { return hipErrorInvalidValue; }
   return static_cast<int>(hipMemcpy(dst, src, bytes, to_device ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost));
+}
+
+int clbh_complex_symmetric_to_square(int precision, int upper, int hermitian, int k, const void* src, long long src_offset,
+                                     long long src_ld, void* dst, hipStream_t stream) {
+  if (k <= 0 || src == nullptr || dst == nullptr || src_ld < k || src_offset < 0) { return hipErrorInvalidValue; }
+  const dim3 grid(Blocks(k, clbh::kComplexTile), Blocks(k, clbh::kComplexTile));
+  if (grid.y > 65535) { return hipErrorInvalidConfiguration; }
+  if (precision == 32) {
+    clbh::ComplexSymmetricToSquareKernel<float><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
+        k, upper != 0, hermitian != 0, static_cast<const clbh::ComplexOf<float>*>(src) + src_offset, src_ld,
+        static_cast<clbh::ComplexOf<float>*>(dst));
+  } else if (precision == 64) {
+    clbh::ComplexSymmetricToSquareKernel<double><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
+        k, upper != 0, hermitian != 0, static_cast<const clbh::ComplexOf<double>*>(src) + src_offset, src_ld,
+        static_cast<clbh::ComplexOf<double>*>(dst));
+  } else {
+    return hipErrorInvalidValue;
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
+int clbh_complex_triangular_to_square(int precision, int upper, int unit_diagonal, int k, const void* src, long long src_offset,
+                                      long long src_ld, void* dst, long long dst_ld, hipStream_t stream) {
+  if (k <= 0 || src == nullptr || dst == nullptr || src_ld < k || dst_ld < k || src_offset < 0) { return hipErrorInvalidValue; }
+  const dim3 grid(Blocks(k, clbh::kComplexThreads), static_cast<unsigned>(std::min(k, 16384)));
+  if (precision == 32) {
+    clbh::ComplexTriangularToSquareKernel<float><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
+        k, upper != 0, unit_diagonal != 0, static_cast<const clbh::ComplexOf<float>*>(src) + src_offset, src_ld,
+        static_cast<clbh::ComplexOf<float>*>(dst), dst_ld);
+  } else if (precision == 64) {
+    clbh::ComplexTriangularToSquareKernel<double><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
+        k, upper != 0, unit_diagonal != 0, static_cast<const clbh::ComplexOf<double>*>(src) + src_offset, src_ld,
+        static_cast<clbh::ComplexOf<double>*>(dst), dst_ld);
+  } else {
+    return hipErrorInvalidValue;
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
+int clbh_complex_zero_diagonal_imag(int precision, int n, void* c, long long c_offset, long long c_ld, hipStream_t stream) {
+  if (n <= 0 || c == nullptr || c_offset < 0 || c_ld < n) { return hipErrorInvalidValue; }
+  const dim3 grid(Blocks(n, clbh::kComplexThreads));
+  if (precision == 32) {
+    clbh::ZeroDiagonalImagKernel<float><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
+        n, static_cast<clbh::ComplexOf<float>*>(c) + c_offset, c_ld);
+  } else if (precision == 64) {
+    clbh::ZeroDiagonalImagKernel<double><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
+        n, static_cast<clbh::ComplexOf<double>*>(c) + c_offset, c_ld);
+  } else {
+    return hipErrorInvalidValue;
+  }
+  return static_cast<int>(hipGetLastError());
 }
 
 int clbh_buffer_extent(const void* ptr, size_t* bytes_available) {

@@ -90,20 +90,93 @@ __global__ __launch_bounds__(kComplexThreads) void TransposeComplexKernel(const 
   }
 }
 
-// c: C(i, j) at c[j * c_ld + i], i < m, j < n. grid: (ceil(m / 256), min(n, 16384)).
+// c: C(i, j) at c[j * c_ld + i], i < m, j < n; triangle 1: only i <= j, 2: only i >= j, 0: all.
+// grid: (ceil(m / 256), min(n, 16384)).
 template <typename R>
-__global__ __launch_bounds__(kComplexThreads) void ScaleComplexKernel(const int m, const int n, const R beta_re,
-                                                                      const R beta_im, ComplexOf<R>* __restrict__ c,
-                                                                      const long long c_ld) {
+__global__ __launch_bounds__(kComplexThreads) void ScaleComplexKernel(const int m, const int n, const int triangle,
+                                                                      const R beta_re, const R beta_im,
+                                                                      ComplexOf<R>* __restrict__ c, const long long c_ld) {
   const int i = blockIdx.x * kComplexThreads + threadIdx.x;
   if (i >= m) { return; }
   for (int j = blockIdx.y; j < n; j += gridDim.y) {
+    if ((triangle == 1 && i > j) || (triangle == 2 && i < j)) { continue; }
     const ComplexOf<R> old = c[j * c_ld + i];
     ComplexOf<R> scaled;
     scaled.re = beta_re * old.re - beta_im * old.im;
     scaled.im = beta_re * old.im + beta_im * old.re;
     c[j * c_ld + i] = scaled;
   }
+}
+
+// Dense k x k copy (leading dimension k) of a complex symmetric or Hermitian matrix of which one triangle is stored
+// (reference: src/kernels/level3/convert_symmetric.opencl, convert_hermitian.opencl:25-95); matrices are addressed as
+// [two * ld + one], "upper": the stored elements have one <= two. Hermitian: mirrored elements are conjugated and the
+// imaginary part of the diagonal is taken as zero. Reads run along the contiguous index of the stored triangle only
+// (mirror tiles are transposed in LDS). grid: (ceil(k / 32), ceil(k / 32)).
+template <typename R>
+__global__ __launch_bounds__(kComplexThreads) void ComplexSymmetricToSquareKernel(const int k, const bool upper,
+                                                                                  const bool hermitian,
+                                                                                  const ComplexOf<R>* __restrict__ src,
+                                                                                  const long long src_ld,
+                                                                                  ComplexOf<R>* __restrict__ dst) {
+  __shared__ ComplexOf<R> tile[kComplexTile][kComplexTile + 1];  // [two][one] of the stored tile
+  const int one0 = blockIdx.x * kComplexTile, two0 = blockIdx.y * kComplexTile;
+  const bool stored = upper ? (one0 <= two0) : (two0 <= one0);
+  const int s_one0 = stored ? one0 : two0, s_two0 = stored ? two0 : one0;
+  const int fast = threadIdx.x % kComplexTile, slow = threadIdx.x / kComplexTile;
+  for (int two = slow; two < kComplexTile; two += kComplexThreads / kComplexTile) {
+    const int g_one = s_one0 + fast, g_two = s_two0 + two;
+    ComplexOf<R> value;
+    value.re = R(0);
+    value.im = R(0);
+    if (g_one < k && g_two < k) { value = src[g_two * src_ld + g_one]; }
+    tile[two][fast] = value;
+  }
+  __syncthreads();
+  const bool diagonal = (one0 == two0);
+  for (int two = slow; two < kComplexTile; two += kComplexThreads / kComplexTile) {
+    const int g_one = one0 + fast, g_two = two0 + two;
+    if (g_one < k && g_two < k) {
+      const bool as_stored = diagonal ? (upper ? (fast <= two) : (two <= fast)) : stored;
+      ComplexOf<R> value = as_stored ? tile[two][fast] : tile[fast][two];
+      if (hermitian) {
+        if (!as_stored) { value.im = -value.im; }
+        if (g_one == g_two) { value.im = R(0); }
+      }
+      dst[static_cast<long long>(g_two) * k + g_one] = value;
+    }
+  }
+}
+
+// Dense k x k copy (leading dimension dst_ld) of a complex triangular matrix: zeros in the other triangle, ones on an
+// implied diagonal (reference: src/kernels/level3/convert_triangular.opencl:24-94). grid: (ceil(k / 256), min(k, 16384)).
+template <typename R>
+__global__ __launch_bounds__(kComplexThreads) void ComplexTriangularToSquareKernel(const int k, const bool upper,
+                                                                                   const bool unit,
+                                                                                   const ComplexOf<R>* __restrict__ src,
+                                                                                   const long long src_ld,
+                                                                                   ComplexOf<R>* __restrict__ dst,
+                                                                                   const long long dst_ld) {
+  const int one = blockIdx.x * kComplexThreads + threadIdx.x;
+  if (one >= k) { return; }
+  for (int two = blockIdx.y; two < k; two += gridDim.y) {
+    ComplexOf<R> value;
+    value.re = R(0);
+    value.im = R(0);
+    const bool is_stored = upper ? (one <= two) : (one >= two);
+    if (one == two && unit) { value.re = R(1); }
+    else if (is_stored) { value = src[two * src_ld + one]; }
+    dst[two * dst_ld + one] = value;
+  }
+}
+
+// Sets the imaginary part of the diagonal of the n x n matrix c (leading dimension c_ld) to zero: the last step of
+// HERK and HER2K (reference: the diagonal_imag_zero flag of src/routines/common.hpp:49-140). grid: ceil(n / 256).
+template <typename R>
+__global__ __launch_bounds__(kComplexThreads) void ZeroDiagonalImagKernel(const int n, ComplexOf<R>* __restrict__ c,
+                                                                          const long long c_ld) {
+  const int i = blockIdx.x * kComplexThreads + threadIdx.x;
+  if (i < n) { c[i * (c_ld + 1)].im = R(0); }
 }
 
 }  // namespace clbh

@@ -40,20 +40,31 @@ struct GemmArgs {
   int operand_triangle;
 };
 
+// c_triangle: 1 keeps C(i,j) with i <= j, 2 with i >= j. 3 and 4 are the same for a complex matrix stored as a real
+// one with interleaved rows (rows 2i and 2i+1 are the real and imaginary part of complex row i): i / 2 <= j resp.
+// i / 2 >= j.
+__device__ __forceinline__ int TriangleRow(const int c_triangle, const int i) { return (c_triangle >= 3) ? (i >> 1) : i; }
+
 // True when no element of the tile [m0, m0 + tile_m) x [n0, n0 + tile_n) of C belongs to the requested triangle.
 __device__ __forceinline__ bool TileOutsideTriangle(const int c_triangle, const int m0, const int n0, const int tile_m,
                                                     const int tile_n) {
-  return (c_triangle == 1 && m0 > n0 + tile_n - 1) || (c_triangle == 2 && m0 + tile_m - 1 < n0);
+  if (c_triangle == 0) { return false; }
+  const int first = TriangleRow(c_triangle, m0), last = TriangleRow(c_triangle, m0 + tile_m - 1);
+  return (c_triangle & 1) ? (first > n0 + tile_n - 1) : (last < n0);
 }
 
 // True when some element of the tile lies outside the requested triangle, i.e. stores have to be masked.
 __device__ __forceinline__ bool TileCrossesDiagonal(const int c_triangle, const int m0, const int n0, const int tile_m,
                                                     const int tile_n) {
-  return (c_triangle == 1 && m0 + tile_m - 1 > n0) || (c_triangle == 2 && m0 < n0 + tile_n - 1);
+  if (c_triangle == 0) { return false; }
+  const int first = TriangleRow(c_triangle, m0), last = TriangleRow(c_triangle, m0 + tile_m - 1);
+  return (c_triangle & 1) ? (last > n0) : (first < n0 + tile_n - 1);
 }
 
 __device__ __forceinline__ bool InTriangle(const int c_triangle, const int i, const int j) {
-  return c_triangle == 0 || (c_triangle == 1 ? i <= j : i >= j);
+  if (c_triangle == 0) { return true; }
+  const int row = TriangleRow(c_triangle, i);
+  return (c_triangle & 1) ? (row <= j) : (row >= j);
 }
 
 // K range [first, first + length) of the tile at (m0, n0) that a triangular operand leaves non-zero; first is a

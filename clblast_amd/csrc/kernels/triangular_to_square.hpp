@@ -19,6 +19,7 @@
 namespace clbh {
 
 constexpr int kCopyThreads = 256;
+
 constexpr int kCopyMaxGridY = 16384;  // values of `two` beyond that are covered by a grid-stride loop
 
 template <typename T, int VEC>

@@ -139,7 +139,7 @@ void Xgemm<T>::DoGemm(const Layout layout, const Transpose a_transpose, const Tr
   if (triangular) {
     // In the canonical problem of a row-major call A and B have changed places and C is transposed
     const bool folded = (layout != Layout::kColMajor);
-    static constexpr int kFoldedOutput[3] = {0, 2, 1};
+    static constexpr int kFoldedOutput[5] = {0, 2, 1, 3, 4};  // (the pair forms are only used column-major)
     static constexpr int kFoldedOperand[5] = {0, 3, 4, 1, 2};
     desc.c_triangle = folded ? kFoldedOutput[static_cast<int>(triangles.output)] : static_cast<int>(triangles.output);
     desc.operand_triangle = folded ? kFoldedOperand[static_cast<int>(triangles.operand)] : static_cast<int>(triangles.operand);

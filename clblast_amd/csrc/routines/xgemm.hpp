@@ -27,7 +27,9 @@ struct GemmShape {
 // Triangular variants of a GEMM, stated for the logical matrices op(A) (m x k), op(B) (k x n) and C (m x n) of the
 // call, whatever the layout: which triangle of C is computed and written (the rest of C stays untouched), and which
 // operand is triangular, i.e. holds explicit zeros that the kernels may skip.
-enum class OutputTriangle { kFull = 0, kUpper = 1, kLower = 2 };  // upper: C(i,j) with i <= j
+// upper: C(i,j) with i <= j; the "Pairs" values are for a complex C given as a column-major real matrix whose rows
+// 2i and 2i+1 hold complex row i (the real GEMM behind the complex one): i / 2 <= j resp. i / 2 >= j
+enum class OutputTriangle { kFull = 0, kUpper = 1, kLower = 2, kUpperPairs = 3, kLowerPairs = 4 };
 enum class OperandTriangle { kNone = 0, kLowerA = 1, kUpperA = 2, kUpperB = 3, kLowerB = 4 };
 struct GemmTriangles {
   OutputTriangle output = OutputTriangle::kFull;

@@ -18,7 +18,7 @@ void XgemmComplex<R>::DoGemm(const Layout layout, const Transpose a_transpose, c
                              const Buffer<Complex>& a_buffer, const size_t a_offset, const size_t a_ld,
                              const Buffer<Complex>& b_buffer, const size_t b_offset, const size_t b_ld,
                              const Complex beta, const Buffer<Complex>& c_buffer, const size_t c_offset,
-                             const size_t c_ld) {
+                             const size_t c_ld, const OutputTriangle triangle, const bool record_event) {
   // Same order as the reference (xgemm.cpp:72-83): dimensions, then A (ld, size), B, C
   const auto shape = Xgemm<R>::ProcessArguments(layout, a_transpose, b_transpose, m, n, k);
   TestMatrixA(shape.a_one, shape.a_two, a_buffer, a_offset, a_ld);
@@ -68,10 +68,13 @@ void XgemmComplex<R>::DoGemm(const Layout layout, const Transpose a_transpose, c
     right_offset = 0;
     right_ld = k;
   }
-  // beta: the real GEMM applies a real factor; an imaginary part needs a pass over C of its own
+  // A triangle of the complex C: in the canonical problem of a row-major call C is transposed (upper <-> lower)
+  const bool canonical_upper = (triangle == OutputTriangle::kUpper) == col_major;
+  const auto canonical_triangle = (triangle == OutputTriangle::kFull) ? 0 : (canonical_upper ? 1 : 2);
+  // beta: the real GEMM applies a real factor; an imaginary part needs a pass over C (or its triangle) of its own
   auto real_beta = beta.real();
   if (beta.imag() != R(0)) {
-    CheckDevice(clbh_complex_scale(precision, static_cast<int>(rows), static_cast<int>(columns),
+    CheckDevice(clbh_complex_scale(precision, static_cast<int>(rows), static_cast<int>(columns), canonical_triangle,
                                    static_cast<double>(beta.real()), static_cast<double>(beta.imag()),
                                    const_cast<void*>(c_buffer()), static_cast<long long>(c_offset),
                                    static_cast<long long>(c_ld), stream),
@@ -81,13 +84,141 @@ void XgemmComplex<R>::DoGemm(const Layout layout, const Transpose a_transpose, c
   const auto real_left = Buffer<R>(expanded.get(), expanded_bytes);
   const auto real_right = transposed ? Buffer<R>(right_pointer, right_bytes) : Buffer<R>(right_pointer);
   const auto real_c = Buffer<R>(c_buffer());
+  // the rows of the real matrix come in (re, im) pairs
+  auto triangles = GemmTriangles{};
+  if (canonical_triangle != 0) {
+    triangles.output = canonical_upper ? OutputTriangle::kUpperPairs : OutputTriangle::kLowerPairs;
+  }
   Xgemm<R>::DoGemm(Layout::kColMajor, Transpose::kNo, Transpose::kNo, 2 * rows, columns, 2 * k, R(1), real_left, 0, 2 * rows,
                    real_right, 2 * right_offset, 2 * right_ld, real_beta, real_c, 2 * c_offset, 2 * c_ld, Buffer<R>(nullptr),
-                   false);
+                   false, triangles, record_event);
+}
+
+// =================================================================================================
+
+template <typename R>
+Xlevel3Complex<R>::Xlevel3Complex(hipStream_t* queue, hipEvent_t* event) : XgemmComplex<R>(queue, event) {}
+
+template <typename R>
+void Xlevel3Complex<R>::DoSymm(const bool hermitian, const Layout layout, const Side side, const Triangle triangle,
+                               const size_t m, const size_t n, const Complex alpha, const Buffer<Complex>& a_buffer,
+                               const size_t a_offset, const size_t a_ld, const Buffer<Complex>& b_buffer,
+                               const size_t b_offset, const size_t b_ld, const Complex beta,
+                               const Buffer<Complex>& c_buffer, const size_t c_offset, const size_t c_ld) {
+  // Same order as the reference (xsymm.cpp:39-49, xhemm.cpp:39-49): dimensions, then the square matrix A
+  if ((m == 0) || (n == 0)) { throw BLASError(StatusCode::kInvalidDimension); }
+  const auto k = (side == Side::kLeft) ? m : n;
+  if (k > static_cast<size_t>(INT_MAX)) { throw BLASError(StatusCode::kInvalidDimension, "dimension exceeds 2^31-1"); }
+  TestMatrixA(k, k, a_buffer, a_offset, a_ld);
+  const auto is_upper = ((triangle == Triangle::kUpper && layout != Layout::kRowMajor) ||
+                         (triangle == Triangle::kLower && layout == Layout::kRowMajor));
+  const auto square_bytes = k * k * sizeof(Complex);
+  const StreamScratch square(square_bytes, this->stream(), "square copy of the symmetric matrix");
+  // The expansion addresses memory, not the logical matrix: for a row-major Hermitian matrix the memory image of the
+  // stored triangle is the conjugate of the column-major reading, and so is the image of the result - consistent, as
+  // every mirrored element is the conjugate of its twin in both readings
+  CheckDevice(clbh_complex_symmetric_to_square(static_cast<int>(8 * sizeof(R)), is_upper ? 1 : 0, hermitian ? 1 : 0,
+                                               static_cast<int>(k), a_buffer(), static_cast<long long>(a_offset),
+                                               static_cast<long long>(a_ld), square.get(), this->stream()),
+              "clbh_complex_symmetric_to_square");
+  const auto square_buffer = Buffer<Complex>(square.get(), square_bytes);
+  if (side == Side::kLeft) {
+    XgemmComplex<R>::DoGemm(layout, Transpose::kNo, Transpose::kNo, m, n, k, alpha, square_buffer, 0, k, b_buffer, b_offset, b_ld,
+                            beta, c_buffer, c_offset, c_ld);
+  } else {
+    try {
+      XgemmComplex<R>::DoGemm(layout, Transpose::kNo, Transpose::kNo, m, n, k, alpha, b_buffer, b_offset, b_ld, square_buffer, 0, k,
+                              beta, c_buffer, c_offset, c_ld);
+    } catch (BLASError& e) {
+      throw SwappedOperands(e);
+    }
+  }
+}
+
+template <typename R>
+void Xlevel3Complex<R>::DoRankUpdate(const bool hermitian, const Layout layout, const Triangle triangle,
+                                     const Transpose transpose, const size_t n, const size_t k, const Complex alpha,
+                                     const Buffer<Complex>& a_buffer, const size_t a_offset, const size_t a_ld,
+                                     const Buffer<Complex>* b_buffer, const size_t b_offset, const size_t b_ld,
+                                     const Complex beta, const Buffer<Complex>& c_buffer, const size_t c_offset,
+                                     const size_t c_ld) {
+  // The second operand of each product is the other matrix with the opposite transpose (xsyrk.cpp:54-60,
+  // xsyr2k.cpp:36-47); in the Hermitian routines every transpose is a conjugate transpose (xherk.cpp:77-80)
+  const bool transposed = (transpose != Transpose::kNo);
+  const auto first = hermitian ? (transposed ? Transpose::kConjugate : Transpose::kNo) : transpose;
+  const auto second = transposed ? Transpose::kNo : (hermitian ? Transpose::kConjugate : Transpose::kYes);
+  const auto output = (triangle == Triangle::kUpper) ? OutputTriangle::kUpper : OutputTriangle::kLower;
+  const bool two_sided = (b_buffer != nullptr);
+  // the complex GEMM makes the reference's checks in the reference's order: dimensions (with m = n), A, B, C
+  const auto& other = two_sided ? *b_buffer : a_buffer;
+  const auto other_offset = two_sided ? b_offset : a_offset, other_ld = two_sided ? b_ld : a_ld;
+  XgemmComplex<R>::DoGemm(layout, first, second, n, n, k, alpha, a_buffer, a_offset, a_ld, other, other_offset, other_ld, beta,
+                          c_buffer, c_offset, c_ld, output, !two_sided && !hermitian);
+  if (two_sided) {  // C += alpha' * op(B) * op(A)^T with alpha' = alpha, or conj(alpha) for HER2K (xher2k.cpp:44-47)
+    const auto second_alpha = hermitian ? std::conj(alpha) : alpha;
+    XgemmComplex<R>::DoGemm(layout, first, second, n, n, k, second_alpha, other, other_offset, other_ld, a_buffer, a_offset, a_ld,
+                            Complex(R(1), R(0)), c_buffer, c_offset, c_ld, output, !hermitian);
+  }
+  if (hermitian) {  // the diagonal of a Hermitian matrix is real (the reference's diagonal_imag_zero)
+    CheckDevice(clbh_complex_zero_diagonal_imag(static_cast<int>(8 * sizeof(R)), static_cast<int>(n),
+                                                const_cast<void*>(c_buffer()), static_cast<long long>(c_offset),
+                                                static_cast<long long>(c_ld), this->stream()),
+                "clbh_complex_zero_diagonal_imag");
+    this->Finish();
+  }
+}
+
+template <typename R>
+void Xlevel3Complex<R>::DoTrmm(const Layout layout, const Side side, const Triangle triangle, const Transpose a_transpose,
+                               const Diagonal diagonal, const size_t m, const size_t n, const Complex alpha,
+                               const Buffer<Complex>& a_buffer, const size_t a_offset, const size_t a_ld,
+                               const Buffer<Complex>& b_buffer, const size_t b_offset, const size_t b_ld) {
+  // Same order as the reference (xtrmm.cpp:38-52): dimensions, the triangular matrix A, then B
+  if ((m == 0) || (n == 0)) { throw BLASError(StatusCode::kInvalidDimension); }
+  if (m > static_cast<size_t>(INT_MAX) / 2 || n > static_cast<size_t>(INT_MAX) / 2) {
+    throw BLASError(StatusCode::kInvalidDimension, "dimension exceeds 2^30");
+  }
+  const auto k = (side == Side::kLeft) ? m : n;
+  TestMatrixA(k, k, a_buffer, a_offset, a_ld);
+  const auto b_one = (layout == Layout::kRowMajor) ? n : m;
+  const auto b_two = (layout == Layout::kRowMajor) ? m : n;
+  TestMatrixB(b_one, b_two, b_buffer, b_offset, b_ld);
+  const auto component_bits = static_cast<int>(8 * sizeof(R));
+  const auto copy_bytes = b_one * b_two * sizeof(Complex);
+  const StreamScratch b_copy(copy_bytes, this->stream(), "copy of B");
+  CheckDevice(clbh_copy_matrix(2 * component_bits, static_cast<int>(b_one), static_cast<int>(b_two), b_buffer(),
+                               static_cast<long long>(b_offset), static_cast<long long>(b_ld), b_copy.get(), 0,
+                               static_cast<long long>(b_one), this->stream()),
+              "clbh_copy_matrix");
+  const auto is_upper = ((triangle == Triangle::kUpper && layout != Layout::kRowMajor) ||
+                         (triangle == Triangle::kLower && layout == Layout::kRowMajor));
+  const auto square_bytes = k * k * sizeof(Complex);
+  const StreamScratch square(square_bytes, this->stream(), "square copy of the triangular matrix");
+  CheckDevice(clbh_complex_triangular_to_square(component_bits, is_upper ? 1 : 0, (diagonal == Diagonal::kUnit) ? 1 : 0,
+                                                static_cast<int>(k), a_buffer(), static_cast<long long>(a_offset),
+                                                static_cast<long long>(a_ld), square.get(), static_cast<long long>(k),
+                                                this->stream()),
+              "clbh_complex_triangular_to_square");
+  const auto square_buffer = Buffer<Complex>(square.get(), square_bytes);
+  const auto copy_buffer = Buffer<Complex>(b_copy.get(), copy_bytes);
+  const auto zero = Complex(R(0), R(0));
+  if (side == Side::kLeft) {
+    XgemmComplex<R>::DoGemm(layout, a_transpose, Transpose::kNo, m, n, k, alpha, square_buffer, 0, k, copy_buffer, 0, b_one, zero,
+                            b_buffer, b_offset, b_ld);
+  } else {
+    try {
+      XgemmComplex<R>::DoGemm(layout, Transpose::kNo, a_transpose, m, n, k, alpha, copy_buffer, 0, b_one, square_buffer, 0, k, zero,
+                              b_buffer, b_offset, b_ld);
+    } catch (BLASError& e) {
+      throw SwappedOperands(e);
+    }
+  }
 }
 
 template class XgemmComplex<float>;
 template class XgemmComplex<double>;
+template class Xlevel3Complex<float>;
+template class Xlevel3Complex<double>;
 
 // =================================================================================================
 }  // namespace clblast

@@ -28,7 +28,34 @@ class XgemmComplex : public Xgemm<R> {
               const size_t n, const size_t k, const Complex alpha, const Buffer<Complex>& a_buffer,
               const size_t a_offset, const size_t a_ld, const Buffer<Complex>& b_buffer, const size_t b_offset,
               const size_t b_ld, const Complex beta, const Buffer<Complex>& c_buffer, const size_t c_offset,
-              const size_t c_ld);
+              const size_t c_ld, const OutputTriangle triangle = OutputTriangle::kFull, const bool record_event = true);
+};
+
+// The Level-3 routines of the complex types on top of it (reference: the float2/double2 instantiations of
+// src/routines/level3/xsymm.cpp, xhemm.cpp, xsyrk.cpp, xherk.cpp, xsyr2k.cpp, xher2k.cpp, xtrmm.cpp). Same structure as
+// their real counterparts (routines/xsymm.cpp, xsyrk.cpp, xtrmm.cpp): expansion kernels for complex data, then the
+// complex GEMM, for SYRK ... HER2K restricted to one triangle of C.
+template <typename R>
+class Xlevel3Complex : public XgemmComplex<R> {
+ public:
+  using Complex = std::complex<R>;
+  Xlevel3Complex(hipStream_t* queue, hipEvent_t* event);
+  // SYMM (hermitian false) and HEMM (true)
+  void DoSymm(const bool hermitian, const Layout layout, const Side side, const Triangle triangle, const size_t m,
+              const size_t n, const Complex alpha, const Buffer<Complex>& a_buffer, const size_t a_offset,
+              const size_t a_ld, const Buffer<Complex>& b_buffer, const size_t b_offset, const size_t b_ld,
+              const Complex beta, const Buffer<Complex>& c_buffer, const size_t c_offset, const size_t c_ld);
+  // SYRK, SYR2K (hermitian false; any alpha, beta) and HERK, HER2K (true; HERK: real alpha; both: real beta).
+  // b_buffer == nullptr selects the rank-k update.
+  void DoRankUpdate(const bool hermitian, const Layout layout, const Triangle triangle, const Transpose transpose,
+                    const size_t n, const size_t k, const Complex alpha, const Buffer<Complex>& a_buffer,
+                    const size_t a_offset, const size_t a_ld, const Buffer<Complex>* b_buffer, const size_t b_offset,
+                    const size_t b_ld, const Complex beta, const Buffer<Complex>& c_buffer, const size_t c_offset,
+                    const size_t c_ld);
+  void DoTrmm(const Layout layout, const Side side, const Triangle triangle, const Transpose a_transpose,
+              const Diagonal diagonal, const size_t m, const size_t n, const Complex alpha,
+              const Buffer<Complex>& a_buffer, const size_t a_offset, const size_t a_ld,
+              const Buffer<Complex>& b_buffer, const size_t b_offset, const size_t b_ld);
 };
 
 }  // namespace clblast

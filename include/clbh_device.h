@@ -67,7 +67,8 @@ typedef struct clbh_gemm_desc_ {
   void* workspace;          // optional device scratch (split-K partial sums), may be NULL
   size_t workspace_bytes;
   // Triangular variants of the canonical problem (both 0 for a plain GEMM; neither combines with split_k > 1):
-  int c_triangle;        // 1: only C(i,j) with i <= j is computed and written, 2: only i >= j; the rest of C is untouched
+  int c_triangle;        // 1: only C(i,j) with i <= j is computed and written, 2: only i >= j; the rest of C is untouched.
+                         // 3, 4: the same for a complex C stored as a real matrix with interleaved rows: i/2 <= j, i/2 >= j
   int operand_triangle;  // the caller states that part of an operand is zero, so that the kernels may skip it:
                          // 1: A(i,p) = 0 for p > i, 2: A(i,p) = 0 for p < i, 3: B(p,j) = 0 for p > j, 4: B(p,j) = 0 for p < j
 } clbh_gemm_desc;
@@ -105,6 +106,7 @@ CLBH_API int clbh_invert_diagonal_blocks(int precision, int upper, int blocks, c
 CLBH_API int clbh_fill_zero(void* ptr, size_t bytes, hipStream_t stream);
 
 // dst[dst_offset + two * dst_ld + one] = src[src_offset + two * src_ld + one] for one < one_extent, two < two_extent.
+// precision: bits per element (16, 32, 64, or 128 for double-precision complex; single-precision complex copies as 64).
 CLBH_API int clbh_copy_matrix(int precision, int one_extent, int two_extent, const void* src, long long src_offset,
                               long long src_ld, void* dst, long long dst_offset, long long dst_ld, hipStream_t stream);
 
@@ -119,8 +121,8 @@ CLBH_API int clbh_complex_expand(int precision, int m, int k, int kcontig, int c
 // dst[j*k + p] = src[src_offset + p*src_ld + j] for p < k, j < n (complex elements).
 CLBH_API int clbh_complex_transpose(int precision, int k, int n, const void* src, long long src_offset,
                                     long long src_ld, void* dst, hipStream_t stream);
-// C(i,j) *= beta for i < m, j < n; C(i,j) at c[c_offset + j*c_ld + i].
-CLBH_API int clbh_complex_scale(int precision, int m, int n, double beta_re, double beta_im, void* c,
+// C(i,j) *= beta for i < m, j < n (triangle 1: only i <= j, 2: only i >= j, 0: all); C(i,j) at c[c_offset + j*c_ld + i].
+CLBH_API int clbh_complex_scale(int precision, int m, int n, int triangle, double beta_re, double beta_im, void* c,
                                 long long c_offset, long long c_ld, hipStream_t stream);
 
 // im2col of a batch of images for CONVGEMM (all arguments in elements; see kernels/im2col.hpp for the layout):
@@ -140,6 +142,18 @@ CLBH_API int clbh_im2col(int precision, const clbh_im2col_shape* shape, int batc
 CLBH_API int clbh_alloc(void** ptr, size_t bytes);
 CLBH_API int clbh_free(void* ptr);
 CLBH_API int clbh_copy(void* dst, const void* src, size_t bytes, int to_device);
+
+// Complex symmetric (hermitian == 0) or Hermitian k x k matrix with one stored triangle -> dense k x k (leading dimension k)
+CLBH_API int clbh_complex_symmetric_to_square(int precision, int upper, int hermitian, int k, const void* src,
+                                              long long src_offset, long long src_ld, void* dst, hipStream_t stream);
+// Complex triangular k x k matrix -> dense k x k (leading dimension dst_ld): zeros in the other triangle, ones on an
+// implied diagonal
+CLBH_API int clbh_complex_triangular_to_square(int precision, int upper, int unit_diagonal, int k, const void* src,
+                                               long long src_offset, long long src_ld, void* dst, long long dst_ld,
+                                               hipStream_t stream);
+// Im(C(i,i)) = 0 for i < n; C(i,j) at c[c_offset + j*c_ld + i]
+CLBH_API int clbh_complex_zero_diagonal_imag(int precision, int n, void* c, long long c_offset, long long c_ld,
+                                             hipStream_t stream);
 
 // Number of bytes addressable from `ptr` to the end of the device allocation that contains it.
 // Returns 0 on success, non-zero if `ptr` is not inside a device allocation.

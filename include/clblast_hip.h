@@ -114,7 +114,8 @@ using double2 = std::complex<double>;
 // =================================================================================================
 
 // C = alpha * op(A) * op(B) + beta * C. T is float, double, half, float2 or double2 (the complex types take no
-// temp_buffer; the batched routines exist for the real types only).
+// temp_buffer; the batched routines exist for the real types only). Symm, Syrk, Syr2k and Trmm below also exist for
+// float2 and double2; Trsm and Convgemm do not.
 template <typename T>
 StatusCode Gemm(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
                 const size_t n, const size_t k, const T alpha, const void* a_buffer, const size_t a_offset,
@@ -147,6 +148,31 @@ StatusCode Symm(const Layout layout, const Side side, const Triangle triangle, c
                 const T alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld, const void* b_buffer,
                 const size_t b_offset, const size_t b_ld, const T beta, void* c_buffer, const size_t c_offset,
                 const size_t c_ld, hipStream_t* queue, hipEvent_t* event = nullptr);
+
+// Hermitian matrix-matrix multiplication (CHEMM/ZHEMM): as Symm with A Hermitian; the imaginary part of A's diagonal is
+// taken as zero. T is float2 or double2 (reference: include/clblast.h:442-446, src/routines/level3/xhemm.cpp).
+template <typename T>
+StatusCode Hemm(const Layout layout, const Side side, const Triangle triangle, const size_t m, const size_t n,
+                const T alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld, const void* b_buffer,
+                const size_t b_offset, const size_t b_ld, const T beta, void* c_buffer, const size_t c_offset,
+                const size_t c_ld, hipStream_t* queue, hipEvent_t* event = nullptr);
+
+// Rank-k update of a Hermitian matrix (CHERK/ZHERK), C = alpha * op(A) * op(A)^H + beta * C on one triangle, the
+// diagonal made real. T is float or double - the type of alpha and beta; the data is complex of that precision
+// (reference: include/clblast.h:456-460, src/routines/level3/xherk.cpp).
+template <typename T>
+StatusCode Herk(const Layout layout, const Triangle triangle, const Transpose a_transpose, const size_t n,
+                const size_t k, const T alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+                const T beta, void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                hipEvent_t* event = nullptr);
+
+// Rank-2k update of a Hermitian matrix (CHER2K/ZHER2K), C = alpha * op(A) * op(B)^H + conj(alpha) * op(B) * op(A)^H +
+// beta * C. T is float2 or double2, U its real type (reference: include/clblast.h:470-474, xher2k.cpp).
+template <typename T, typename U>
+StatusCode Her2k(const Layout layout, const Triangle triangle, const Transpose ab_transpose, const size_t n,
+                 const size_t k, const T alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+                 const void* b_buffer, const size_t b_offset, const size_t b_ld, const U beta, void* c_buffer,
+                 const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event = nullptr);
 
 // Rank-k update of one triangle of a symmetric matrix, C = alpha * op(A) * op(A)^T + beta * C with op(A) n x k; the
 // other triangle of C is neither read nor written (reference: include/clblast.h:449-453,

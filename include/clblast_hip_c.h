@@ -206,6 +206,94 @@ CLBlastStatusCode CLBLAST_HIP_API CLBlastHtrmm(const CLBlastLayout layout, const
                                                const size_t a_ld, void* b_buffer, const size_t b_offset,
                                                const size_t b_ld, hipStream_t* queue, hipEvent_t* event);
 
+// The complex versions of the Level-3 routines above and the Hermitian ones; complex data is interleaved (real,
+// imaginary). replaces CLBlast{C,Z}symm, ...hemm, ...syrk, ...herk, ...syr2k, ...her2k, ...trmm (reference:
+// include/clblast_c.h:934-1092). HERK takes real alpha and beta, HER2K a complex alpha and a real beta.
+CLBlastStatusCode CLBLAST_HIP_API CLBlastCsymm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const size_t m, const size_t n,
+                                               const CLBlastFloat2 alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, const CLBlastFloat2 beta, void* c_buffer,
+                                               const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                                               hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastZsymm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const size_t m, const size_t n,
+                                               const CLBlastDouble2 alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, const CLBlastDouble2 beta, void* c_buffer,
+                                               const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                                               hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastChemm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const size_t m, const size_t n,
+                                               const CLBlastFloat2 alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, const CLBlastFloat2 beta, void* c_buffer,
+                                               const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                                               hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastZhemm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const size_t m, const size_t n,
+                                               const CLBlastDouble2 alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, const CLBlastDouble2 beta, void* c_buffer,
+                                               const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                                               hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastCsyrk(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                               const CLBlastTranspose a_transpose, const size_t n, const size_t k,
+                                               const CLBlastFloat2 alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, const CLBlastFloat2 beta, void* c_buffer, const size_t c_offset,
+                                               const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastZsyrk(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                               const CLBlastTranspose a_transpose, const size_t n, const size_t k,
+                                               const CLBlastDouble2 alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, const CLBlastDouble2 beta, void* c_buffer, const size_t c_offset,
+                                               const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastCherk(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                               const CLBlastTranspose a_transpose, const size_t n, const size_t k,
+                                               const float alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, const float beta, void* c_buffer, const size_t c_offset,
+                                               const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastZherk(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                               const CLBlastTranspose a_transpose, const size_t n, const size_t k,
+                                               const double alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, const double beta, void* c_buffer, const size_t c_offset,
+                                               const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastCsyr2k(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                                const CLBlastTranspose ab_transpose, const size_t n, const size_t k,
+                                                const CLBlastFloat2 alpha, const void* a_buffer, const size_t a_offset,
+                                                const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                                                const size_t b_ld, const CLBlastFloat2 beta, void* c_buffer, const size_t c_offset,
+                                                const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastZsyr2k(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                                const CLBlastTranspose ab_transpose, const size_t n, const size_t k,
+                                                const CLBlastDouble2 alpha, const void* a_buffer, const size_t a_offset,
+                                                const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                                                const size_t b_ld, const CLBlastDouble2 beta, void* c_buffer, const size_t c_offset,
+                                                const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastCher2k(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                                const CLBlastTranspose ab_transpose, const size_t n, const size_t k,
+                                                const CLBlastFloat2 alpha, const void* a_buffer, const size_t a_offset,
+                                                const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                                                const size_t b_ld, const float beta, void* c_buffer, const size_t c_offset,
+                                                const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastZher2k(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                                const CLBlastTranspose ab_transpose, const size_t n, const size_t k,
+                                                const CLBlastDouble2 alpha, const void* a_buffer, const size_t a_offset,
+                                                const size_t a_ld, const void* b_buffer, const size_t b_offset,
+                                                const size_t b_ld, const double beta, void* c_buffer, const size_t c_offset,
+                                                const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastCtrmm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const CLBlastTranspose a_transpose,
+                                               const CLBlastDiagonal diagonal, const size_t m, const size_t n,
+                                               const CLBlastFloat2 alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastZtrmm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const CLBlastTranspose a_transpose,
+                                               const CLBlastDiagonal diagonal, const size_t m, const size_t n,
+                                               const CLBlastDouble2 alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, hipStream_t* queue, hipEvent_t* event);
+
 // Batched convolution as GEMM (non-BLAS function)
 // replaces CLBlastSconvgemm/CLBlastDconvgemm/CLBlastHconvgemm (reference: include/clblast_c.h:1252-1281, src/clblast_c.cpp:2625-2700)
 CLBlastStatusCode CLBLAST_HIP_API CLBlastSconvgemm(const CLBlastKernelMode kernel_mode, const size_t channels,

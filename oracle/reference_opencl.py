@@ -151,7 +151,34 @@ def run(spec):
 
     def call():
         event = vp(None)
-        if spec["routine"] == "convgemm":  # a = images, b = kernels, c = result; "conv": the 13 size_t arguments in order
+        if is_complex and spec["routine"] in ("symm", "hemm", "syrk", "herk", "syr2k", "her2k", "trmm"):
+            # the complex Level-3 routines: "side", "triangle", "ta", "diagonal" as far as the routine has them; HERK takes
+            # real alpha and beta, HER2K a real beta ("alpha"/"beta" are [re, im] pairs, the imaginary part then unused)
+            name = spec["routine"]
+            function = getattr(reference, "CLBlast%s%s" % (prefix, name))
+            real = ctypes.c_float if bits == 32 else ctypes.c_double
+            real_alpha, real_beta = real(spec["alpha"][0]), real(spec.get("beta", [0.0, 0.0])[0])
+            ci = ctypes.c_int
+            if name in ("symm", "hemm"):
+                arguments = [ci(spec["layout"]), ci(spec["side"]), ci(spec["triangle"]), m, n, alpha, a_buffer, sz(offsets[0]),
+                             sz(spec["a_ld"]), b_buffer, sz(offsets[1]), sz(spec["b_ld"]), beta, c_buffer, sz(offsets[2]),
+                             sz(spec["c_ld"])]
+            elif name in ("syrk", "herk"):
+                arguments = [ci(spec["layout"]), ci(spec["triangle"]), ci(spec["ta"]), n, k,
+                             real_alpha if name == "herk" else alpha, a_buffer, sz(offsets[0]), sz(spec["a_ld"]),
+                             real_beta if name == "herk" else beta, c_buffer, sz(offsets[2]), sz(spec["c_ld"])]
+            elif name in ("syr2k", "her2k"):
+                arguments = [ci(spec["layout"]), ci(spec["triangle"]), ci(spec["ta"]), n, k, alpha, a_buffer, sz(offsets[0]),
+                             sz(spec["a_ld"]), b_buffer, sz(offsets[1]), sz(spec["b_ld"]),
+                             real_beta if name == "her2k" else beta, c_buffer, sz(offsets[2]), sz(spec["c_ld"])]
+            else:
+                arguments = [ci(spec["layout"]), ci(spec["side"]), ci(spec["triangle"]), ci(spec["ta"]), ci(spec["diagonal"]), m,
+                             n, alpha, a_buffer, sz(offsets[0]), sz(spec["a_ld"]), b_buffer, sz(offsets[1]), sz(spec["b_ld"])]
+            arguments += [ctypes.byref(queue), ctypes.byref(event)]
+            function.argtypes = [type(argument) if not isinstance(argument, type(ctypes.byref(queue))) else vp
+                                 for argument in arguments]
+            status = function(*arguments)
+        elif spec["routine"] == "convgemm":  # a = images, b = kernels, c = result; "conv": the 13 size_t arguments in order
             function = getattr(reference, "CLBlast%sconvgemm" % PREFIX[bits])
             status = function(ctypes.c_int(spec["kernel_mode"]), *[sz(value) for value in spec["conv"]], a_buffer,
                               sz(offsets[0]), b_buffer, sz(offsets[1]), c_buffer, sz(offsets[2]), ctypes.byref(queue),
