@@ -18,11 +18,10 @@ namespace {
 
 int LaunchTyped(const clbh_gemm_desc& d, hipStream_t stream) {
   const bool mfma = (d.kernel_class == CLBH_KERNEL_MFMA);
+  if (d.kernel_class == CLBH_KERNEL_SMALL_BATCHED) { return LaunchSmallBatched(d, stream); }
   switch (d.precision) {
     case 16: return mfma ? LaunchMfmaF16(d, stream) : LaunchGeneralF16(d, stream);
-    case 32:
-      if (d.kernel_class == CLBH_KERNEL_SMALL_BATCHED) { return LaunchSmallBatched(d, stream); }
-      return mfma ? LaunchMfmaF32(d, stream) : LaunchGeneralF32(d, stream);
+    case 32: return mfma ? LaunchMfmaF32(d, stream) : LaunchGeneralF32(d, stream);
     case 64: return mfma ? LaunchMfmaF64(d, stream) : LaunchGeneralF64(d, stream);
     default: return hipErrorInvalidValue;
   }

@@ -83,8 +83,8 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
                           const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,
                           const size_t min_indirect_size, const bool triangular) {
   (void)a_kcontig; (void)b_kcontig; (void)per_batch_scalars;
-  // Many small fp32 matrices: one wavefront per matrix, bandwidth bound
-  if (precision == Precision::kSingle && batch_count >= 16 && m <= 32 && n <= 32 && k <= 32) {
+  // Many small matrices: one wavefront per matrix, bandwidth bound
+  if (batch_count >= 16 && m <= 32 && n <= 32 && k <= 32) {
     return KernelChoice{CLBH_KERNEL_SMALL_BATCHED, 0, 1};
   }
   if (UseDirectKernel(m, n, k, min_indirect_size)) {
