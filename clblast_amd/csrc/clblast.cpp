@@ -396,7 +396,11 @@ template StatusCode CLBLAST_HIP_PUBLIC Trsm<double>(const Layout, const Side, co
 
 // Kernels are compiled ahead of time: there is no program or binary cache to drop. Parameter
 // overrides survive, as they do in the reference (api_common.cpp:25-33 leaves the database cache alone).
-CLBLAST_HIP_PUBLIC StatusCode ClearCache() { return StatusCode::kSuccess; }
+// There are no compiled programs to forget; what the library does keep between calls is its per-stream scratch memory
+CLBLAST_HIP_PUBLIC StatusCode ClearCache() {
+  ReleaseCachedScratch();
+  return StatusCode::kSuccess;
+}
 
 CLBLAST_HIP_PUBLIC StatusCode OverrideParameters(const int device, const std::string& kernel_name,
                                                  const Precision precision,

@@ -4,6 +4,10 @@
 #include "routines/routine_common.hpp"
 
 #include <cstdio>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <utility>
 
 namespace clblast {
 // =================================================================================================
@@ -44,8 +48,57 @@ BLASError SwappedOperands(const BLASError& error) {
   }
 }
 
+namespace {
+struct CachedScratch {
+  void* pointer = nullptr;
+  size_t bytes = 0;
+  std::mutex taken;  // held by the StreamScratch that uses the buffer
+};
+std::mutex scratch_cache_mutex;
+std::map<std::pair<int, hipStream_t>, std::unique_ptr<CachedScratch>> scratch_cache;
+
+// The entry of this stream with at least `bytes` bytes, locked, or nullptr (then the caller allocates on the stream)
+CachedScratch* TakeCachedScratch(const size_t bytes, hipStream_t stream) {
+  auto device = 0;
+  if (bytes == 0 || bytes > kCachedScratchBytes || clbh_stream_device(stream, &device) != 0) { return nullptr; }
+  CachedScratch* entry = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(scratch_cache_mutex);
+    const auto key = std::make_pair(device, stream);
+    auto found = scratch_cache.find(key);
+    if (found == scratch_cache.end()) {
+      if (scratch_cache.size() >= kCachedScratchStreams) { return nullptr; }
+      found = scratch_cache.emplace(key, std::unique_ptr<CachedScratch>(new CachedScratch())).first;
+    }
+    entry = found->second.get();
+    if (!entry->taken.try_lock()) { return nullptr; }
+  }
+  if (entry->bytes < bytes) {
+    // grows in powers of two from 1 MiB, so that this happens a few times per stream at most; freeing the old buffer
+    // waits for the device, which covers kernels of earlier calls that still use it
+    auto wanted = size_t{1} << 20;
+    while (wanted < bytes) { wanted *= 2; }
+    if (entry->pointer != nullptr) { clbh_free(entry->pointer); }
+    entry->pointer = nullptr;
+    entry->bytes = 0;
+    if (clbh_alloc(&entry->pointer, wanted) != 0) {
+      entry->pointer = nullptr;
+      entry->taken.unlock();
+      return nullptr;
+    }
+    entry->bytes = wanted;
+  }
+  return entry;
+}
+}  // namespace
+
 StreamScratch::StreamScratch(const size_t bytes, hipStream_t stream, const char* what)
-    : pointer_(nullptr), bytes_(bytes), stream_(stream) {
+    : pointer_(nullptr), bytes_(bytes), stream_(stream), cached_(nullptr) {
+  if (auto* entry = TakeCachedScratch(bytes, stream)) {
+    cached_ = entry;
+    pointer_ = entry->pointer;
+    return;
+  }
   if (clbh_alloc_async(&pointer_, bytes, stream) != 0) {
     pointer_ = nullptr;
     throw RuntimeErrorCode(StatusCode::kTempBufferAllocFailure, what);
@@ -53,7 +106,21 @@ StreamScratch::StreamScratch(const size_t bytes, hipStream_t stream, const char*
 }
 
 StreamScratch::~StreamScratch() {
-  if (pointer_ != nullptr) { clbh_free_async(pointer_, stream_); }
+  if (cached_ != nullptr) { static_cast<CachedScratch*>(cached_)->taken.unlock(); }
+  else if (pointer_ != nullptr) { clbh_free_async(pointer_, stream_); }
+}
+
+void ReleaseCachedScratch() {
+  std::lock_guard<std::mutex> lock(scratch_cache_mutex);
+  for (auto entry = scratch_cache.begin(); entry != scratch_cache.end();) {
+    if (entry->second->taken.try_lock()) {  // not in the hands of a running call
+      if (entry->second->pointer != nullptr) { clbh_free(entry->second->pointer); }
+      entry->second->taken.unlock();
+      entry = scratch_cache.erase(entry);
+    } else {
+      ++entry;
+    }
+  }
 }
 
 StatusCode DispatchExceptionForC() {

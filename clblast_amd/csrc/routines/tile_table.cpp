@@ -61,7 +61,7 @@ bool UseDirectKernel(const size_t m, const size_t n, const size_t k, const size_
 
 // fp32 tile table (index -> work-group tile), see device/launch.hip:
 //   0: 128 x 128 x 16   3: 256 x 128 x 16   5: 128 x 32 x 32   6: 32 x 128 x 32   7: 64 x 64 x 16
-//   9: 64 x 32 x 32 and 10: 32 x 32 x 64 on the 16x16x4 MFMA (two and more work-groups per CU for mid-sized problems)
+//   8: 32 x 64 x 32, 9: 64 x 32 x 32 and 10: 32 x 32 x 64 on the 16x16x4 MFMA (two and more work-groups per CU for mid-sized problems)
 namespace {
 struct Tile {
   int index;
@@ -69,11 +69,18 @@ struct Tile {
 };
 
 // Number of K ranges for a launch of `tiles` work-groups. Splitting costs a second launch (the reduction, about
-// 8 us) and pays only when most CUs would idle through a long K walk (about 16 ns per unit of k and work-group):
-// ranges stay >= 512 deep and bring the launch to about two work-groups per CU (four of the half-sized tiles).
+// 5 us) and pays only when most CUs would idle through a long K walk (about 16 ns per unit of k and work-group):
+// ranges stay >= 512 deep and bring the launch to about two work-groups per CU. The half- and quarter-sized tiles
+// (four work-groups per CU fit) are split up to 1024 work-groups, into ranges that may be the shorter the emptier the
+// GPU would be otherwise (measured: 128^2 x 1024 13.2 -> 9.2 us with four ranges, 768^2 x 4096 79.5 -> 54.4 us).
 int SplitFor(const size_t tiles, const size_t k, const bool small_tile = false) {
-  const size_t kWantedGroups = small_tile ? 1024 : 512;
-  if (tiles >= (small_tile ? 384u : 192u) || k < 2048) { return 1; }
+  if (small_tile) {
+    const size_t min_range = (tiles <= 64) ? 256 : (tiles <= 128) ? 512 : 1024;
+    if (tiles >= 384 || k < 2 * min_range) { return 1; }
+    return static_cast<int>(std::max<size_t>(1, std::min<size_t>({CeilDivide(1024, tiles), k / min_range, 16})));
+  }
+  constexpr size_t kWantedGroups = 512;
+  if (tiles >= 192 || k < 2048) { return 1; }
   const auto wanted = CeilDivide(kWantedGroups, tiles);
   const auto allowed = k / 512;
   return static_cast<int>(std::max<size_t>(1, std::min<size_t>({wanted, allowed, 32})));
@@ -128,18 +135,18 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   if (precision == Precision::kSingle) {
     // Measured on the MI355X (tile x split sweep over 18 shapes): 64 x 64 tiles (several work-groups per CU hide
     // each other's latencies) win up to about 3072^3 and whenever k is short (C traffic dominates); 256 x 128 needs
-    // two full rounds of tiles and a long K walk; the skinny tiles stream the one large operand. Below 1024 tiles of
+    // two full rounds of tiles and a long K walk; skinny problems take the 64 x 32 / 32 x 64 tiles with K split. Below 1024 tiles of
     // 64 x 64 (four per CU) the chip is not full: the 64 x 32 tile of the 16x16x4 MFMA doubles the work-groups
     // (1024^3: 28.5 -> 23.8 us), and up to 64 such tiles with a short k the 32 x 32 tile does so again (512^3: 16.0 -> 8.8 us).
     auto tile = Tile{7, 64, 64};
     const auto tiles64 = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;
-    if (n <= 32 && m >= 256) { tile = Tile{5, 128, 32}; }        // skinny: stream A
-    else if (m <= 32 && n >= 256) { tile = Tile{6, 32, 128}; }   // skinny: stream B
+    if (n <= 32 && m >= 256) { tile = Tile{9, 64, 32}; }         // skinny: stream A
+    else if (m <= 32 && n >= 256) { tile = Tile{8, 32, 64}; }    // skinny: stream B
     else if (CeilDivide(m, 256) * CeilDivide(n, 128) >= 512 && k >= 1024) { tile = Tile{3, 256, 128}; }
     else if (tiles64 <= 64 && k < 2048) { tile = Tile{10, 32, 32}; }
     else if (tiles64 < 1024) { tile = Tile{9, 64, 32}; }
     const auto tiles = CeilDivide(m, tile.tile_m) * CeilDivide(n, tile.tile_n) * batch_count;
-    const auto split = (batch_count == 1) ? SplitFor(tiles, k, tile.index >= 9) : 1;
+    const auto split = (batch_count == 1) ? SplitFor(tiles, k, tile.index >= 8) : 1;
     return KernelChoice{CLBH_KERNEL_MFMA, tile.index, split};
   }
   // fp64 (same sweep): 64 x 64 x 16 tiles (index 1) up to about 3072^3, 128 x 128 x 8 (index 0) beyond; for launches

@@ -3,6 +3,8 @@
 // =================================================================================================
 #include "routines/xgemm.hpp"
 
+#include <memory>
+
 #include <climits>
 
 namespace clblast {
@@ -149,25 +151,19 @@ void Xgemm<T>::DoGemm(const Layout layout, const Transpose a_transpose, const Tr
   // Temporary memory: only split-K launches want any. A caller-provided buffer must be large enough
   // (reference: xgemm.cpp:146-151), otherwise stream-ordered scratch is taken for the call.
   const auto temp_bytes = clbh_gemm_workspace_bytes(&desc);
-  void* scratch = nullptr;
+  std::unique_ptr<StreamScratch> scratch;
   if (temp_buffer_provided) {
     if (temp_bytes > 0 && temp_buffer.GetSize() < temp_bytes) {
       throw BLASError(StatusCode::kInsufficientMemoryTemp);
     }
     desc.workspace = const_cast<void*>(temp_buffer());
   } else if (temp_bytes > 0) {
-    if (clbh_alloc_async(&scratch, temp_bytes, stream()) != 0) {
-      throw RuntimeErrorCode(StatusCode::kTempBufferAllocFailure, "temporary buffer");
-    }
-    desc.workspace = scratch;
+    scratch.reset(new StreamScratch(temp_bytes, stream(), "temporary buffer"));
+    desc.workspace = scratch->get();
   }
   desc.workspace_bytes = temp_bytes;
 
-  const auto launch_status = clbh_gemm_launch(&desc, stream());
-  if (scratch != nullptr) {
-    clbh_free_async(scratch, stream());
-  }
-  CheckDevice(launch_status, "clbh_gemm_launch");
+  CheckDevice(clbh_gemm_launch(&desc, stream()), "clbh_gemm_launch");
   if (record_event) { Finish(); }
 }
 

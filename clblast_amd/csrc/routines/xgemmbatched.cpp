@@ -90,13 +90,10 @@ void XgemmBatched<T>::DoGemmBatched(const Layout layout, const Transpose a_trans
   }
   desc.batch.offset_multiple = static_cast<int>(multiple);
 
-  void* device_block = nullptr;
-  if (clbh_alloc_async(&device_block, total_bytes, stream()) != 0) {
-    throw RuntimeErrorCode(StatusCode::kTempBufferAllocFailure, "batch metadata");
-  }
-  auto status = clbh_upload_async(device_block, packed.data(), total_bytes, stream());
+  const StreamScratch device_block(total_bytes, stream(), "batch metadata");
+  auto status = clbh_upload_async(device_block.get(), packed.data(), total_bytes, stream());
   if (status == 0) {
-    const auto base = static_cast<unsigned char*>(device_block);
+    const auto base = static_cast<unsigned char*>(device_block.get());
     desc.batch.alphas = base;
     desc.batch.betas = base + scalars_block;
     desc.batch.a_offsets = reinterpret_cast<const long long*>(base + 2 * scalars_block);
@@ -104,7 +101,6 @@ void XgemmBatched<T>::DoGemmBatched(const Layout layout, const Transpose a_trans
     desc.batch.c_offsets = reinterpret_cast<const long long*>(base + 2 * scalars_block + 2 * offsets_block);
     status = clbh_gemm_launch(&desc, stream());
   }
-  clbh_free_async(device_block, stream());
   CheckDevice(status, "batched GEMM launch");
   Finish();
 }

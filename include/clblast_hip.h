@@ -232,8 +232,9 @@ StatusCode GemmTempBufferSize(const Layout layout, const Transpose a_transpose, 
 
 // =================================================================================================
 
-// Kept for source compatibility: kernels are compiled ahead of time, so there is no program cache to
-// clear. Returns kSuccess and leaves parameter overrides in place.
+// Kernels are compiled ahead of time, so there is no program cache to clear; what the library keeps between calls is
+// up to 16 MiB of scratch memory for each of up to 16 (device, stream) pairs, and this frees it. Call it with the
+// device idle. Returns kSuccess and leaves parameter overrides in place.
 StatusCode ClearCache();
 
 // Overrides engine parameters for one device ordinal and precision. Accepted kernel names:

@@ -180,3 +180,22 @@ def test_padding_and_neighbouring_memory_never_reach_the_result(gpu, bits, path)
             problem.check(c_after)
     finally:
         gpu.force_path(bits, None)
+
+
+@pytest.mark.parametrize("bits", (32, 64))
+def test_split_k_calls_share_the_streams_scratch(gpu, bits):
+    """Split-K launches take their partial-sum buffer from the scratch memory the library keeps per stream: a call
+    that needs more than the previous one (the buffer grows), one that needs less (stale partial sums of the larger
+    call lie behind its own), ClearCache between calls, and a caller-provided buffer's absence throughout."""
+    import clblast_amd
+    seed = 9900
+    for step, (m, n, k) in enumerate(((96, 96, 2048), (256, 200, 4096), (96, 96, 2048), (128, 64, 8192), (128, 128, 4096))):
+        if step == 3:
+            import torch
+            torch.cuda.synchronize()
+            assert clblast_amd.clear_cache() == 0
+        seed += 1
+        problem = gpu.Problem(bits, COL_MAJOR, NO, YES, m, n, k, 0.75, 1.5, seed=seed)
+        status, c_after = problem.run()
+        assert status == 0, problem.describe()
+        problem.check(c_after)
