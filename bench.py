@@ -168,17 +168,18 @@ class SymmWorkload(Workload):
 
 class ComplexWorkload:
     """CGEMM / ZGEMM, C := alpha op(A) op(B) + beta C on interleaved complex data (torch complex tensors are row-major:
-    a row-major call). 8 m n k real flops, priced against the real MFMA peak of the component type."""
+    a row-major call); batch > 1: that many products through the strided-batched entry point. 8 m n k real flops each,
+    priced against the real MFMA peak of the component type."""
 
-    def __init__(self, name, prefix, ta, tb, m, n, k, alpha, beta):
+    def __init__(self, name, prefix, ta, tb, m, n, k, alpha, beta, batch=1):
         import torch
-        self.name, self.prefix, self.ta, self.tb, self.m, self.n, self.k = name, prefix, ta, tb, m, n, k
+        self.name, self.prefix, self.ta, self.tb, self.m, self.n, self.k, self.batch = name, prefix, ta, tb, m, n, k, batch
         self.alpha, self.beta = complex(alpha), complex(beta)
         dtype = torch.complex64 if prefix == "C" else torch.complex128
         generator = torch.Generator(device="cuda")
         generator.manual_seed(2024)
         draw = lambda rows, cols: torch.view_as_complex(  # noqa: E731
-            torch.rand(rows, cols, 2, device="cuda", dtype=torch.float64, generator=generator).mul_(2).sub_(1)).to(dtype)
+            torch.rand(batch, rows, cols, 2, device="cuda", dtype=torch.float64, generator=generator).mul_(2).sub_(1)).to(dtype)
         self.a = draw(m, k) if ta == NO else draw(k, m)
         self.b = draw(k, n) if tb == NO else draw(n, k)
         self.c = draw(m, n)
@@ -186,25 +187,31 @@ class ComplexWorkload:
 
     @property
     def flops(self):
-        return 8.0 * self.m * self.n * self.k
+        return 8.0 * self.m * self.n * self.k * self.batch
 
     @property
     def algorithmic_bytes(self):
         element = 8 if self.prefix == "C" else 16
-        return element * (self.m * self.k + self.k * self.n + (2 if self.beta != 0 else 1) * self.m * self.n)
+        return element * self.batch * (self.m * self.k + self.k * self.n + (2 if self.beta != 0 else 1) * self.m * self.n)
 
     def call(self, stream_handle):
-        from clblast_amd.api import raw_complex_gemm
-        status = raw_complex_gemm(self.prefix, ROW, self.ta, self.tb, self.m, self.n, self.k, self.alpha, self.a.data_ptr(), 0,
-                                  self.a.shape[1], self.b.data_ptr(), 0, self.b.shape[1], self.beta, self.c.data_ptr(), 0,
-                                  self.n, stream_handle)
+        from clblast_amd.api import raw_complex_gemm, raw_gemm_strided_batched
+        a_ld, b_ld = self.a.shape[2], self.b.shape[2]
+        if self.batch == 1:
+            status = raw_complex_gemm(self.prefix, ROW, self.ta, self.tb, self.m, self.n, self.k, self.alpha, self.a.data_ptr(), 0,
+                                      a_ld, self.b.data_ptr(), 0, b_ld, self.beta, self.c.data_ptr(), 0, self.n, stream_handle)
+        else:
+            status = raw_gemm_strided_batched(self.prefix, ROW, self.ta, self.tb, self.m, self.n, self.k, self.alpha,
+                                              self.a.data_ptr(), 0, a_ld, self.a.shape[1] * a_ld, self.b.data_ptr(), 0, b_ld,
+                                              self.b.shape[1] * b_ld, self.beta, self.c.data_ptr(), 0, self.n, self.m * self.n,
+                                              self.batch, stream_handle)
         if status != 0:
             raise RuntimeError("%s: status %d" % (self.name, status))
 
     def freivalds_error(self):
         import torch
         x = torch.rand(self.n, 1, device="cuda", dtype=torch.float64).sub_(0.5).to(torch.complex128)
-        op = lambda t, flag: t if flag == NO else (t.T if flag == YES else t.conj().T)  # noqa: E731
+        op = lambda t, flag: t if flag == NO else (t.transpose(1, 2) if flag == YES else t.conj().transpose(1, 2))  # noqa: E731
         expected = self.alpha * (op(self.a, self.ta).to(torch.complex128) @ (op(self.b, self.tb).to(torch.complex128) @ x))
         if self.c_initial is not None:
             expected = expected + self.beta * (self.c_initial.to(torch.complex128) @ x)
@@ -500,6 +507,8 @@ EXTRA_WORKLOADS = {
                                                         132, 8198, (11, 13, 19)),
     "next_cgemm_4096_rowNC": lambda: ComplexWorkload("cgemm", "C", NO, 113, 4096, 4096, 4096, 1.0 - 0.5j, 0.0),
     "next_zgemm_2048_rowTN": lambda: ComplexWorkload("zgemm", "Z", YES, NO, 2048, 2048, 2048, 0.5 + 1.0j, 1.0 - 0.5j),
+    "next_cgemm_strided_batched_4096x64_rowNC": lambda: ComplexWorkload("cgemm_batched", "C", NO, 113, 64, 64, 64, 1.0 - 0.5j,
+                                                                        0.0, batch=4096),
     "next_sconvgemm_64x112x112_k128_b8": lambda: ConvWorkload("conv_s", "S", 64, 112, 128, 8),
     "next_hconvgemm_64x112x112_k128_b8": lambda: ConvWorkload("conv_h", "H", 64, 112, 128, 8),
     "next_ssymm_4096_colLeftUpper": lambda: SymmWorkload("symm_s", "S", COL, True, 4096, 4096, 1.0, 0.0),

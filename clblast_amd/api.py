@@ -57,6 +57,9 @@ def _prefix_of(dtype_name):
 
 
 def _scalar(prefix, value):
+    if prefix in "CZ":  # complex scalars travel as (re, im) structs
+        value = complex(value)
+        return (_lib.Float2 if prefix == "C" else _lib.Double2)(value.real, value.imag)
     return float_to_half_bits(value) if prefix == "H" else value
 
 
@@ -173,7 +176,7 @@ def raw_trsm(prefix, layout, side, triangle, a_transpose, diagonal, m, n, alpha,
 def raw_gemm_batched(prefix, layout, a_transpose, b_transpose, m, n, k, alphas, a_ptr, a_offsets, a_ld, b_ptr,
                      b_offsets, b_ld, betas, c_ptr, c_offsets, c_ld, batch_count, stream_handle=0):
     lib = _lib.load()
-    scalar_t = _lib._SCALAR[prefix]
+    scalar_t = {"C": _lib.Float2, "Z": _lib.Double2}.get(prefix) or _lib._SCALAR[prefix]
     count = len(alphas)
     mk_s = lambda xs: (scalar_t * max(len(xs), 1))(*[_scalar(prefix, x) for x in xs])
     mk_z = lambda xs: (ctypes.c_size_t * max(len(xs), 1))(*xs)

@@ -10,6 +10,8 @@
 #include "clblast_hip.h"
 #include "routines/xgemm.hpp"
 #include "routines/xgemm_complex.hpp"
+#include "routines/xgemmbatched_complex.hpp"
+#include "routines/xgemmbatched_complex.hpp"
 #include "routines/xconvgemm.hpp"
 #include "routines/xgemmbatched.hpp"
 #include "routines/xsymm.hpp"
@@ -276,6 +278,53 @@ StatusCode CLBLAST_HIP_PUBLIC Gemm<double2>(const Layout layout, const Transpose
   return ComplexGemm<double>(layout, a_transpose, b_transpose, m, n, k, alpha, a_buffer, a_offset, a_ld, b_buffer, b_offset,
                              b_ld, beta, c_buffer, c_offset, c_ld, queue, event);
 }
+
+// The batched GEMMs of the complex types (reference: src/clblast.cpp:1612-1621, 1660-1671)
+#define CLBLAST_HIP_COMPLEX_BATCHED(R)                                                                                 \
+  template <>                                                                                                          \
+  StatusCode CLBLAST_HIP_PUBLIC GemmBatched<std::complex<R>>(                                                          \
+      const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m, const size_t n,   \
+      const size_t k, const std::complex<R>* alphas, const void* a_buffer, const size_t* a_offsets, const size_t a_ld, \
+      const void* b_buffer, const size_t* b_offsets, const size_t b_ld, const std::complex<R>* betas, void* c_buffer,  \
+      const size_t* c_offsets, const size_t c_ld, const size_t batch_count, hipStream_t* queue, hipEvent_t* event) {   \
+    try {                                                                                                              \
+      using Complex = std::complex<R>;                                                                                 \
+      auto routine = XgemmComplexBatched<R>(queue, event);                                                             \
+      if (batch_count > 0 && (alphas == nullptr || betas == nullptr || a_offsets == nullptr || b_offsets == nullptr || \
+                              c_offsets == nullptr)) {                                                                 \
+        throw BLASError(StatusCode::kInvalidBatchCount, "null per-batch array");                                       \
+      }                                                                                                                \
+      routine.DoGemmBatched(layout, a_transpose, b_transpose, m, n, k, std::vector<Complex>(alphas, alphas + batch_count), \
+                            Buffer<Complex>(a_buffer), std::vector<size_t>(a_offsets, a_offsets + batch_count), a_ld,  \
+                            Buffer<Complex>(b_buffer), std::vector<size_t>(b_offsets, b_offsets + batch_count), b_ld,  \
+                            std::vector<Complex>(betas, betas + batch_count), Buffer<Complex>(c_buffer),               \
+                            std::vector<size_t>(c_offsets, c_offsets + batch_count), c_ld, batch_count);               \
+      return StatusCode::kSuccess;                                                                                     \
+    } catch (...) {                                                                                                    \
+      return DispatchException();                                                                                      \
+    }                                                                                                                  \
+  }                                                                                                                    \
+  template <>                                                                                                          \
+  StatusCode CLBLAST_HIP_PUBLIC GemmStridedBatched<std::complex<R>>(                                                   \
+      const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m, const size_t n,   \
+      const size_t k, const std::complex<R> alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,     \
+      const size_t a_stride, const void* b_buffer, const size_t b_offset, const size_t b_ld, const size_t b_stride,    \
+      const std::complex<R> beta, void* c_buffer, const size_t c_offset, const size_t c_ld, const size_t c_stride,     \
+      const size_t batch_count, hipStream_t* queue, hipEvent_t* event) {                                               \
+    try {                                                                                                              \
+      using Complex = std::complex<R>;                                                                                 \
+      auto routine = XgemmComplexBatched<R>(queue, event);                                                             \
+      routine.DoGemmStridedBatched(layout, a_transpose, b_transpose, m, n, k, alpha, Buffer<Complex>(a_buffer), a_offset, \
+                                   a_ld, a_stride, Buffer<Complex>(b_buffer), b_offset, b_ld, b_stride, beta,          \
+                                   Buffer<Complex>(c_buffer), c_offset, c_ld, c_stride, batch_count);                  \
+      return StatusCode::kSuccess;                                                                                     \
+    } catch (...) {                                                                                                    \
+      return DispatchException();                                                                                      \
+    }                                                                                                                  \
+  }
+CLBLAST_HIP_COMPLEX_BATCHED(float)
+CLBLAST_HIP_COMPLEX_BATCHED(double)
+#undef CLBLAST_HIP_COMPLEX_BATCHED
 
 // The complex Level-3 routines (reference: src/clblast.cpp:1110-1330)
 namespace {

@@ -342,6 +342,39 @@ CLBlastStatusCode CLBlastZgemm(const CLBlastLayout layout, const CLBlastTranspos
   });
 }
 
+// ---- batched CGEMM, ZGEMM: the C structs and std::complex share their layout -------------------------
+#define CLBLAST_HIP_COMPLEX_BATCHED(PREFIX, CTYPE, CPPTYPE)                                                          \
+  CLBlastStatusCode CLBlast##PREFIX##gemmBatched(                                                                    \
+      const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose,            \
+      const size_t m, const size_t n, const size_t k, const CTYPE* alphas, const void* a_buffer,                     \
+      const size_t* a_offsets, const size_t a_ld, const void* b_buffer, const size_t* b_offsets, const size_t b_ld,  \
+      const CTYPE* betas, void* c_buffer, const size_t* c_offsets, const size_t c_ld, const size_t batch_count,      \
+      hipStream_t* queue, hipEvent_t* event) {                                                                       \
+    static_assert(sizeof(CTYPE) == sizeof(CPPTYPE), "interleaved (re, im) layout");                                  \
+    return Guarded([&]() {                                                                                           \
+      return clblast::GemmBatched<CPPTYPE>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k,                     \
+                                           reinterpret_cast<const CPPTYPE*>(alphas), a_buffer, a_offsets, a_ld,      \
+                                           b_buffer, b_offsets, b_ld, reinterpret_cast<const CPPTYPE*>(betas),       \
+                                           c_buffer, c_offsets, c_ld, batch_count, queue, event);                    \
+    });                                                                                                              \
+  }                                                                                                                  \
+  CLBlastStatusCode CLBlast##PREFIX##gemmStridedBatched(                                                             \
+      const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose,            \
+      const size_t m, const size_t n, const size_t k, const CTYPE alpha, const void* a_buffer, const size_t a_offset, \
+      const size_t a_ld, const size_t a_stride, const void* b_buffer, const size_t b_offset, const size_t b_ld,      \
+      const size_t b_stride, const CTYPE beta, void* c_buffer, const size_t c_offset, const size_t c_ld,             \
+      const size_t c_stride, const size_t batch_count, hipStream_t* queue, hipEvent_t* event) {                      \
+    return Guarded([&]() {                                                                                           \
+      return clblast::GemmStridedBatched<CPPTYPE>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k,              \
+                                                  CPPTYPE(alpha.x, alpha.y), a_buffer, a_offset, a_ld, a_stride,     \
+                                                  b_buffer, b_offset, b_ld, b_stride, CPPTYPE(beta.x, beta.y),       \
+                                                  c_buffer, c_offset, c_ld, c_stride, batch_count, queue, event);    \
+    });                                                                                                              \
+  }
+CLBLAST_HIP_COMPLEX_BATCHED(C, CLBlastFloat2, clblast::float2)
+CLBLAST_HIP_COMPLEX_BATCHED(Z, CLBlastDouble2, clblast::double2)
+#undef CLBLAST_HIP_COMPLEX_BATCHED
+
 // ---- complex Level 3 ----------------------------------------------------------------------------
 #define CLBLAST_HIP_TO_COMPLEX_float(v) clblast::float2((v).x, (v).y)
 #define CLBLAST_HIP_TO_COMPLEX_double(v) clblast::double2((v).x, (v).y)

@@ -176,33 +176,52 @@ namespace {
 unsigned Blocks(const int extent, const int per_block) { return static_cast<unsigned>((extent + per_block - 1) / per_block); }
 
 template <typename R>
+clbh::ComplexBatches<R> MakeComplexBatches(const clbh_complex_batches* batches) {
+  clbh::ComplexBatches<R> result;
+  result.count = (batches != nullptr) ? batches->count : 1;
+  result.src_stride = (batches != nullptr) ? batches->src_stride : 0;
+  result.src_offsets = (batches != nullptr) ? batches->src_offsets : nullptr;
+  result.dst_stride = (batches != nullptr) ? batches->dst_stride : 0;
+  result.scalars = (batches != nullptr) ? static_cast<const clbh::ComplexOf<R>*>(batches->scalars) : nullptr;
+  return result;
+}
+
+template <typename R>
 int LaunchComplexExpand(const int m, const int k, const int kcontig, const int conjugate, const int conjugated_b,
                         const double alpha_re, const double alpha_im, const void* src, const long long src_offset,
-                        const long long src_ld, void* dst, hipStream_t stream) {
-  const dim3 grid(Blocks(m, clbh::kComplexTile), Blocks(k, clbh::kComplexTile));
+                        const long long src_ld, void* dst, const clbh_complex_batches* batches, hipStream_t stream) {
+  const auto walk = MakeComplexBatches<R>(batches);
+  const dim3 grid(Blocks(m, clbh::kComplexTile), Blocks(k, clbh::kComplexTile), static_cast<unsigned>(std::min(walk.count, 65535)));
   if (grid.y > 65535) { return hipErrorInvalidConfiguration; }
   clbh::ExpandComplexKernel<R><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
       m, k, kcontig != 0, conjugate != 0, conjugated_b != 0, static_cast<R>(alpha_re), static_cast<R>(alpha_im),
-      static_cast<const clbh::ComplexOf<R>*>(src) + src_offset, src_ld, static_cast<R*>(dst));
+      static_cast<const clbh::ComplexOf<R>*>(src) + src_offset, src_ld, static_cast<R*>(dst), walk);
   return static_cast<int>(hipGetLastError());
 }
 
 template <typename R>
 int LaunchComplexTranspose(const int k, const int n, const void* src, const long long src_offset, const long long src_ld,
-                           void* dst, hipStream_t stream) {
-  const dim3 grid(Blocks(k, clbh::kComplexTile), Blocks(n, clbh::kComplexTile));
+                           void* dst, const clbh_complex_batches* batches, hipStream_t stream) {
+  const auto walk = MakeComplexBatches<R>(batches);
+  const dim3 grid(Blocks(k, clbh::kComplexTile), Blocks(n, clbh::kComplexTile), static_cast<unsigned>(std::min(walk.count, 65535)));
   if (grid.y > 65535) { return hipErrorInvalidConfiguration; }
   clbh::TransposeComplexKernel<R><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
-      k, n, static_cast<const clbh::ComplexOf<R>*>(src) + src_offset, src_ld, static_cast<clbh::ComplexOf<R>*>(dst));
+      k, n, static_cast<const clbh::ComplexOf<R>*>(src) + src_offset, src_ld, static_cast<clbh::ComplexOf<R>*>(dst), walk);
   return static_cast<int>(hipGetLastError());
 }
 
 template <typename R>
 int LaunchComplexScale(const int m, const int n, const int triangle, const double beta_re, const double beta_im, void* c,
-                       const long long c_offset, const long long c_ld, hipStream_t stream) {
-  const dim3 grid(Blocks(m, clbh::kComplexThreads), static_cast<unsigned>(std::min(n, 16384)));
+                       const long long c_offset, const long long c_ld, const clbh_complex_batches* batches,
+                       hipStream_t stream) {
+  const auto walk = MakeComplexBatches<R>(batches);
+  // the columns of one matrix share the second grid dimension; large batches leave it small
+  const auto column_blocks = (walk.count > 1) ? std::min(n, 64) : std::min(n, 16384);
+  const dim3 grid(Blocks(m, clbh::kComplexThreads), static_cast<unsigned>(column_blocks),
+                  static_cast<unsigned>(std::min(walk.count, 65535)));
   clbh::ScaleComplexKernel<R><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
-      m, n, triangle, static_cast<R>(beta_re), static_cast<R>(beta_im), static_cast<clbh::ComplexOf<R>*>(c) + c_offset, c_ld);
+      m, n, triangle, static_cast<R>(beta_re), static_cast<R>(beta_im), static_cast<clbh::ComplexOf<R>*>(c) + c_offset, c_ld,
+      walk);
   return static_cast<int>(hipGetLastError());
 }
 }  // namespace
@@ -305,35 +324,67 @@ int clbh_copy_matrix(int precision, int one_extent, int two_extent, const void* 
   }
 }
 
-int clbh_complex_expand(int precision, int m, int k, int kcontig, int conjugate, int conjugated_b, double alpha_re,
-                        double alpha_im, const void* src, long long src_offset, long long src_ld, void* dst,
-                        hipStream_t stream) {
-  if (m <= 0 || k <= 0 || src == nullptr || dst == nullptr || src_offset < 0 || src_ld < (kcontig ? k : m)) {
+namespace {
+bool ValidComplexBatches(const clbh_complex_batches* batches) {
+  return batches == nullptr || (batches->count >= 1 && batches->src_stride >= 0 && batches->dst_stride >= 0);
+}
+}  // namespace
+
+int clbh_complex_expand_batched(int precision, int m, int k, int kcontig, int conjugate, int conjugated_b, double alpha_re,
+                                double alpha_im, const void* src, long long src_offset, long long src_ld, void* dst,
+                                const clbh_complex_batches* batches, hipStream_t stream) {
+  // (lines of the source may overlap, src_ld below their length: GemmBatched does not test the leading dimensions of
+  // A and B, and overlapping reads are well defined)
+  if (m <= 0 || k <= 0 || src == nullptr || dst == nullptr || src_offset < 0 || src_ld < 0 || !ValidComplexBatches(batches)) {
     return hipErrorInvalidValue;
   }
   if (precision == 32) {
-    return LaunchComplexExpand<float>(m, k, kcontig, conjugate, conjugated_b, alpha_re, alpha_im, src, src_offset, src_ld, dst, stream);
+    return LaunchComplexExpand<float>(m, k, kcontig, conjugate, conjugated_b, alpha_re, alpha_im, src, src_offset, src_ld, dst, batches, stream);
   }
   if (precision == 64) {
-    return LaunchComplexExpand<double>(m, k, kcontig, conjugate, conjugated_b, alpha_re, alpha_im, src, src_offset, src_ld, dst, stream);
+    return LaunchComplexExpand<double>(m, k, kcontig, conjugate, conjugated_b, alpha_re, alpha_im, src, src_offset, src_ld, dst, batches, stream);
   }
+  return hipErrorInvalidValue;
+}
+
+int clbh_complex_expand(int precision, int m, int k, int kcontig, int conjugate, int conjugated_b, double alpha_re,
+                        double alpha_im, const void* src, long long src_offset, long long src_ld, void* dst,
+                        hipStream_t stream) {
+  if (src_ld < (kcontig ? k : m)) { return hipErrorInvalidValue; }
+  return clbh_complex_expand_batched(precision, m, k, kcontig, conjugate, conjugated_b, alpha_re, alpha_im, src, src_offset,
+                                     src_ld, dst, nullptr, stream);
+}
+
+int clbh_complex_transpose_batched(int precision, int k, int n, const void* src, long long src_offset, long long src_ld,
+                                   void* dst, const clbh_complex_batches* batches, hipStream_t stream) {
+  if (k <= 0 || n <= 0 || src == nullptr || dst == nullptr || src_offset < 0 || src_ld < 0 || !ValidComplexBatches(batches)) {
+    return hipErrorInvalidValue;
+  }
+  if (precision == 32) { return LaunchComplexTranspose<float>(k, n, src, src_offset, src_ld, dst, batches, stream); }
+  if (precision == 64) { return LaunchComplexTranspose<double>(k, n, src, src_offset, src_ld, dst, batches, stream); }
   return hipErrorInvalidValue;
 }
 
 int clbh_complex_transpose(int precision, int k, int n, const void* src, long long src_offset, long long src_ld, void* dst,
                            hipStream_t stream) {
-  if (k <= 0 || n <= 0 || src == nullptr || dst == nullptr || src_offset < 0 || src_ld < n) { return hipErrorInvalidValue; }
-  if (precision == 32) { return LaunchComplexTranspose<float>(k, n, src, src_offset, src_ld, dst, stream); }
-  if (precision == 64) { return LaunchComplexTranspose<double>(k, n, src, src_offset, src_ld, dst, stream); }
+  if (src_ld < n) { return hipErrorInvalidValue; }
+  return clbh_complex_transpose_batched(precision, k, n, src, src_offset, src_ld, dst, nullptr, stream);
+}
+
+int clbh_complex_scale_batched(int precision, int m, int n, int triangle, double beta_re, double beta_im, void* c,
+                               long long c_offset, long long c_ld, const clbh_complex_batches* batches, hipStream_t stream) {
+  if (m <= 0 || n <= 0 || c == nullptr || c_offset < 0 || c_ld < m || triangle < 0 || triangle > 2 ||
+      !ValidComplexBatches(batches)) {
+    return hipErrorInvalidValue;
+  }
+  if (precision == 32) { return LaunchComplexScale<float>(m, n, triangle, beta_re, beta_im, c, c_offset, c_ld, batches, stream); }
+  if (precision == 64) { return LaunchComplexScale<double>(m, n, triangle, beta_re, beta_im, c, c_offset, c_ld, batches, stream); }
   return hipErrorInvalidValue;
 }
 
 int clbh_complex_scale(int precision, int m, int n, int triangle, double beta_re, double beta_im, void* c, long long c_offset,
                        long long c_ld, hipStream_t stream) {
-  if (m <= 0 || n <= 0 || c == nullptr || c_offset < 0 || c_ld < m || triangle < 0 || triangle > 2) { return hipErrorInvalidValue; }
-  if (precision == 32) { return LaunchComplexScale<float>(m, n, triangle, beta_re, beta_im, c, c_offset, c_ld, stream); }
-  if (precision == 64) { return LaunchComplexScale<double>(m, n, triangle, beta_re, beta_im, c, c_offset, c_ld, stream); }
-  return hipErrorInvalidValue;
+  return clbh_complex_scale_batched(precision, m, n, triangle, beta_re, beta_im, c, c_offset, c_ld, nullptr, stream);
 }
 
 int clbh_im2col(int precision, const clbh_im2col_shape* shape, int batch_count, const void* image, long long image_offset,

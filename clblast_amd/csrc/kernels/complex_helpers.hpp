@@ -30,81 +30,117 @@ struct ComplexOf {
   R re, im;
 };
 
+// The matrices of a batched call: matrix b of the source starts src_offsets[b] (when given) or b * src_stride complex
+// elements behind the kernel's source pointer, its result b * dst_stride elements (of the result's type) behind the
+// destination pointer; scalars (when given) holds one (re, im) pair per matrix that replaces the scalar argument.
+// The third grid dimension walks the batch.
+template <typename R>
+struct ComplexBatches {
+  int count;
+  long long src_stride;
+  const long long* src_offsets;
+  long long dst_stride;
+  const ComplexOf<R>* scalars;
+  __device__ __forceinline__ long long SourceOffset(const int b) const {
+    return (src_offsets != nullptr) ? src_offsets[b] : b * src_stride;
+  }
+};
+
 // src: A(i, p) at src[(kcontig ? i * src_ld + p : p * src_ld + i)], i < m, p < k. dst: real, column-major, leading
-// dimension 2 * m. grid: (ceil(m / 32), ceil(k / 32)).
+// dimension 2 * m. grid: (ceil(m / 32), ceil(k / 32), batches).
 template <typename R>
 __global__ __launch_bounds__(kComplexThreads) void ExpandComplexKernel(const int m, const int k, const bool kcontig,
                                                                        const bool conjugate, const bool conjugated_b,
                                                                        const R alpha_re, const R alpha_im,
-                                                                       const ComplexOf<R>* __restrict__ src,
-                                                                       const long long src_ld, R* __restrict__ dst) {
+                                                                       const ComplexOf<R>* __restrict__ src_base,
+                                                                       const long long src_ld, R* __restrict__ dst_base,
+                                                                       const ComplexBatches<R> batches) {
   __shared__ ComplexOf<R> tile[kComplexTile][kComplexTile + 1];  // [p][i]
   const int i0 = blockIdx.x * kComplexTile, p0 = blockIdx.y * kComplexTile;
   const int fast = threadIdx.x % kComplexTile, slow = threadIdx.x / kComplexTile;
-  for (int step = slow; step < kComplexTile; step += kComplexThreads / kComplexTile) {
-    // lanes run along the contiguous index of the source
-    const int i = i0 + (kcontig ? step : fast), p = p0 + (kcontig ? fast : step);
-    if (i < m && p < k) {
-      const ComplexOf<R> value = src[kcontig ? i * src_ld + p : p * src_ld + i];
-      tile[p - p0][i - i0] = value;
+  for (int batch = blockIdx.z; batch < batches.count; batch += gridDim.z) {
+    const ComplexOf<R>* __restrict__ src = src_base + batches.SourceOffset(batch);
+    R* __restrict__ dst = dst_base + batch * batches.dst_stride;
+    const R scale_re = (batches.scalars != nullptr) ? batches.scalars[batch].re : alpha_re;
+    const R scale_im = (batches.scalars != nullptr) ? batches.scalars[batch].im : alpha_im;
+    for (int step = slow; step < kComplexTile; step += kComplexThreads / kComplexTile) {
+      // lanes run along the contiguous index of the source
+      const int i = i0 + (kcontig ? step : fast), p = p0 + (kcontig ? fast : step);
+      if (i < m && p < k) {
+        const ComplexOf<R> value = src[kcontig ? i * src_ld + p : p * src_ld + i];
+        tile[p - p0][i - i0] = value;
+      }
     }
-  }
-  __syncthreads();
-  const long long dst_ld = 2LL * m;
-  for (int step = slow; step < kComplexTile; step += kComplexThreads / kComplexTile) {
-    const int i = i0 + fast, p = p0 + step;  // lanes run along i: contiguous in both columns of the result
-    if (i < m && p < k) {
-      ComplexOf<R> a = tile[step][fast];
-      if (conjugate) { a.im = -a.im; }
-      const R re = alpha_re * a.re - alpha_im * a.im, im = alpha_re * a.im + alpha_im * a.re;
-      typedef R Pair __attribute__((ext_vector_type(2)));
-      Pair first, second;
-      first[0] = re;
-      first[1] = im;
-      second[0] = conjugated_b ? im : -im;
-      second[1] = conjugated_b ? -re : re;
-      *reinterpret_cast<Pair*>(dst + (2LL * p) * dst_ld + 2 * i) = first;
-      *reinterpret_cast<Pair*>(dst + (2LL * p + 1) * dst_ld + 2 * i) = second;
+    __syncthreads();
+    const long long dst_ld = 2LL * m;
+    for (int step = slow; step < kComplexTile; step += kComplexThreads / kComplexTile) {
+      const int i = i0 + fast, p = p0 + step;  // lanes run along i: contiguous in both columns of the result
+      if (i < m && p < k) {
+        ComplexOf<R> a = tile[step][fast];
+        if (conjugate) { a.im = -a.im; }
+        const R re = scale_re * a.re - scale_im * a.im, im = scale_re * a.im + scale_im * a.re;
+        typedef R Pair __attribute__((ext_vector_type(2)));
+        Pair first, second;
+        first[0] = re;
+        first[1] = im;
+        second[0] = conjugated_b ? im : -im;
+        second[1] = conjugated_b ? -re : re;
+        *reinterpret_cast<Pair*>(dst + (2LL * p) * dst_ld + 2 * i) = first;
+        *reinterpret_cast<Pair*>(dst + (2LL * p + 1) * dst_ld + 2 * i) = second;
+      }
     }
+    __syncthreads();  // the tile is rewritten for the next matrix
   }
 }
 
 // src: B(p, j) at src[p * src_ld + j] (j contiguous), p < k, j < n. dst: B(p, j) at dst[j * k + p].
-// grid: (ceil(k / 32), ceil(n / 32)).
+// grid: (ceil(k / 32), ceil(n / 32), batches).
 template <typename R>
 __global__ __launch_bounds__(kComplexThreads) void TransposeComplexKernel(const int k, const int n,
-                                                                          const ComplexOf<R>* __restrict__ src,
+                                                                          const ComplexOf<R>* __restrict__ src_base,
                                                                           const long long src_ld,
-                                                                          ComplexOf<R>* __restrict__ dst) {
+                                                                          ComplexOf<R>* __restrict__ dst_base,
+                                                                          const ComplexBatches<R> batches) {
   __shared__ ComplexOf<R> tile[kComplexTile][kComplexTile + 1];  // [p][j]
   const int p0 = blockIdx.x * kComplexTile, j0 = blockIdx.y * kComplexTile;
   const int fast = threadIdx.x % kComplexTile, slow = threadIdx.x / kComplexTile;
-  for (int step = slow; step < kComplexTile; step += kComplexThreads / kComplexTile) {
-    const int p = p0 + step, j = j0 + fast;
-    if (p < k && j < n) { tile[step][fast] = src[p * src_ld + j]; }
-  }
-  __syncthreads();
-  for (int step = slow; step < kComplexTile; step += kComplexThreads / kComplexTile) {
-    const int p = p0 + fast, j = j0 + step;
-    if (p < k && j < n) { dst[static_cast<long long>(j) * k + p] = tile[fast][step]; }
+  for (int batch = blockIdx.z; batch < batches.count; batch += gridDim.z) {
+    const ComplexOf<R>* __restrict__ src = src_base + batches.SourceOffset(batch);
+    ComplexOf<R>* __restrict__ dst = dst_base + batch * batches.dst_stride;
+    for (int step = slow; step < kComplexTile; step += kComplexThreads / kComplexTile) {
+      const int p = p0 + step, j = j0 + fast;
+      if (p < k && j < n) { tile[step][fast] = src[p * src_ld + j]; }
+    }
+    __syncthreads();
+    for (int step = slow; step < kComplexTile; step += kComplexThreads / kComplexTile) {
+      const int p = p0 + fast, j = j0 + step;
+      if (p < k && j < n) { dst[static_cast<long long>(j) * k + p] = tile[fast][step]; }
+    }
+    __syncthreads();  // the tile is rewritten for the next matrix
   }
 }
 
 // c: C(i, j) at c[j * c_ld + i], i < m, j < n; triangle 1: only i <= j, 2: only i >= j, 0: all.
-// grid: (ceil(m / 256), min(n, 16384)).
+// grid: (ceil(m / 256), min(n, 16384), batches).
 template <typename R>
 __global__ __launch_bounds__(kComplexThreads) void ScaleComplexKernel(const int m, const int n, const int triangle,
                                                                       const R beta_re, const R beta_im,
-                                                                      ComplexOf<R>* __restrict__ c, const long long c_ld) {
+                                                                      ComplexOf<R>* __restrict__ c_base, const long long c_ld,
+                                                                      const ComplexBatches<R> batches) {
   const int i = blockIdx.x * kComplexThreads + threadIdx.x;
   if (i >= m) { return; }
-  for (int j = blockIdx.y; j < n; j += gridDim.y) {
-    if ((triangle == 1 && i > j) || (triangle == 2 && i < j)) { continue; }
-    const ComplexOf<R> old = c[j * c_ld + i];
-    ComplexOf<R> scaled;
-    scaled.re = beta_re * old.re - beta_im * old.im;
-    scaled.im = beta_re * old.im + beta_im * old.re;
-    c[j * c_ld + i] = scaled;
+  for (int batch = blockIdx.z; batch < batches.count; batch += gridDim.z) {
+    ComplexOf<R>* __restrict__ c = c_base + batches.SourceOffset(batch);
+    const R scale_re = (batches.scalars != nullptr) ? batches.scalars[batch].re : beta_re;
+    const R scale_im = (batches.scalars != nullptr) ? batches.scalars[batch].im : beta_im;
+    for (int j = blockIdx.y; j < n; j += gridDim.y) {
+      if ((triangle == 1 && i > j) || (triangle == 2 && i < j)) { continue; }
+      const ComplexOf<R> old = c[j * c_ld + i];
+      ComplexOf<R> scaled;
+      scaled.re = scale_re * old.re - scale_im * old.im;
+      scaled.im = scale_re * old.im + scale_im * old.re;
+      c[j * c_ld + i] = scaled;
+    }
   }
 }
 

@@ -125,6 +125,29 @@ CLBH_API int clbh_complex_transpose(int precision, int k, int n, const void* src
 CLBH_API int clbh_complex_scale(int precision, int m, int n, int triangle, double beta_re, double beta_im, void* c,
                                 long long c_offset, long long c_ld, hipStream_t stream);
 
+// The same three for the matrices of a batched call (batches == NULL: one matrix): matrix b of the source starts
+// src_offsets[b] (a device array, when given) or b * src_stride complex elements behind src + src_offset, its result
+// b * dst_stride elements of the result's type (real numbers for the expansion, complex ones for the transpose)
+// behind dst; scalars (a device array of (re, im) pairs of the component type, when given) replaces alpha / beta per
+// matrix. The scaling works in place and ignores dst_stride.
+typedef struct clbh_complex_batches_ {
+  int count;
+  long long src_stride;
+  const long long* src_offsets;
+  long long dst_stride;
+  const void* scalars;
+} clbh_complex_batches;
+CLBH_API int clbh_complex_expand_batched(int precision, int m, int k, int kcontig, int conjugate, int conjugated_b,
+                                         double alpha_re, double alpha_im, const void* src, long long src_offset,
+                                         long long src_ld, void* dst, const clbh_complex_batches* batches,
+                                         hipStream_t stream);
+CLBH_API int clbh_complex_transpose_batched(int precision, int k, int n, const void* src, long long src_offset,
+                                            long long src_ld, void* dst, const clbh_complex_batches* batches,
+                                            hipStream_t stream);
+CLBH_API int clbh_complex_scale_batched(int precision, int m, int n, int triangle, double beta_re, double beta_im, void* c,
+                                        long long c_offset, long long c_ld, const clbh_complex_batches* batches,
+                                        hipStream_t stream);
+
 // im2col of a batch of images for CONVGEMM (all arguments in elements; see kernels/im2col.hpp for the layout):
 // image + image_offset holds batch x channels x height x width, col receives batch matrices of
 // (output_h * output_w) x (channels * kernel_h * kernel_w), column-major. flip != 0 mirrors the kernel taps.

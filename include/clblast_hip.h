@@ -114,8 +114,8 @@ using double2 = std::complex<double>;
 // =================================================================================================
 
 // C = alpha * op(A) * op(B) + beta * C. T is float, double, half, float2 or double2 (the complex types take no
-// temp_buffer; the batched routines exist for the real types only). Symm, Syrk, Syr2k and Trmm below also exist for
-// float2 and double2; Trsm and Convgemm do not.
+// temp_buffer). GemmBatched, GemmStridedBatched, Symm, Syrk, Syr2k and Trmm below also exist for float2 and double2;
+// Trsm and Convgemm do not.
 template <typename T>
 StatusCode Gemm(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
                 const size_t n, const size_t k, const T alpha, const void* a_buffer, const size_t a_offset,

@@ -121,6 +121,34 @@ CLBlastStatusCode CLBLAST_HIP_API CLBlastZgemm(const CLBlastLayout layout, const
                                                void* c_buffer, const size_t c_offset, const size_t c_ld,
                                                hipStream_t* queue, hipEvent_t* event);
 
+// Batched and strided-batched complex GEMM: as CLBlast{S,D}gemmBatched / ...StridedBatched with complex scalars.
+// replaces CLBlastCgemmBatched/CLBlastZgemmBatched (reference: include/clblast_c.h:1317-1330, src/clblast_c.cpp:2767-2810)
+// and CLBlastCgemmStridedBatched/CLBlastZgemmStridedBatched (include/clblast_c.h:1353-1364, src/clblast_c.cpp:2869-2904)
+CLBlastStatusCode CLBLAST_HIP_API CLBlastCgemmBatched(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const CLBlastFloat2* alphas, const void* a_buffer, const size_t* a_offsets,
+    const size_t a_ld, const void* b_buffer, const size_t* b_offsets, const size_t b_ld, const CLBlastFloat2* betas,
+    void* c_buffer, const size_t* c_offsets, const size_t c_ld, const size_t batch_count, hipStream_t* queue,
+    hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastZgemmBatched(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const CLBlastDouble2* alphas, const void* a_buffer, const size_t* a_offsets,
+    const size_t a_ld, const void* b_buffer, const size_t* b_offsets, const size_t b_ld, const CLBlastDouble2* betas,
+    void* c_buffer, const size_t* c_offsets, const size_t c_ld, const size_t batch_count, hipStream_t* queue,
+    hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastCgemmStridedBatched(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const CLBlastFloat2 alpha, const void* a_buffer, const size_t a_offset,
+    const size_t a_ld, const size_t a_stride, const void* b_buffer, const size_t b_offset, const size_t b_ld,
+    const size_t b_stride, const CLBlastFloat2 beta, void* c_buffer, const size_t c_offset, const size_t c_ld,
+    const size_t c_stride, const size_t batch_count, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastZgemmStridedBatched(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const CLBlastDouble2 alpha, const void* a_buffer, const size_t a_offset,
+    const size_t a_ld, const size_t a_stride, const void* b_buffer, const size_t b_offset, const size_t b_ld,
+    const size_t b_stride, const CLBlastDouble2 beta, void* c_buffer, const size_t c_offset, const size_t c_ld,
+    const size_t c_stride, const size_t batch_count, hipStream_t* queue, hipEvent_t* event);
+
 // =================================================================================================
 // Symmetric matrix-matrix multiplication C = alpha*A*B + beta*C (side left) or alpha*B*A + beta*C (side right)
 // replaces CLBlastSsymm/CLBlastDsymm/CLBlastHsymm (reference: include/clblast_c.h:921-945, src/clblast_c.cpp:1876-1960)

@@ -10,7 +10,7 @@ HIP (both runtimes in one process were seen to lose the device), hence the comma
 
     python -m oracle.reference_opencl --spec spec.json --out result.npz
 
-spec.json: {"routine": "gemm"|"strided"|"symm" (then "side", "triangle" instead of "ta", "tb", "k")|"trmm"|"trsm" ("side",
+spec.json: {"routine": "gemm"|"strided"|"batched" (per-batch "alphas", "betas" and "batch_offsets")|"symm" (then "side", "triangle" instead of "ta", "tb", "k")|"trmm"|"trsm" ("side",
 "triangle", "ta", "diagonal"; the result is the B buffer)|"syrk"|"syr2k" ("triangle", "ta", "n", "k")|"convgemm" ("kernel_mode",
 "conv": [channels, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w, num_kernels,
 batch_count]; buffers a, b, c are the images, the kernels and the result), "bits": 16|32|64, "layout", "ta", "tb", "m", "n", "k", "alpha", "beta",
@@ -214,9 +214,25 @@ def run(spec):
                               alpha, a_buffer, sz(offsets[0]), sz(spec["a_ld"]), b_buffer, sz(offsets[1]),
                               sz(spec["b_ld"]), beta, c_buffer, sz(offsets[2]), sz(spec["c_ld"]), ctypes.byref(queue),
                               ctypes.byref(event))
+        elif spec["routine"] == "batched":  # "alphas", "betas" (complex: [re, im] pairs), "batch_offsets": three lists
+            function = getattr(reference, "CLBlast%sgemmBatched" % prefix)
+            count = len(spec["alphas"])
+            scalars = [scalar_argument(bits, value, reference, is_complex) for value in spec["alphas"] + spec["betas"]]
+            scalar_array = type(scalars[0]) * count
+            offset_arrays = [(sz * count)(*values) for values in spec["batch_offsets"]]
+            function.argtypes = [ctypes.c_int] * 3 + [sz] * 3 + [vp, vp, vp, sz, vp, vp, sz, vp, vp, vp, sz, sz, vp, vp]
+            alphas_array, betas_array = scalar_array(*scalars[:count]), scalar_array(*scalars[count:])
+            status = function(spec["layout"], spec["ta"], spec["tb"], m, n, k, ctypes.cast(alphas_array, vp), a_buffer,
+                              ctypes.cast(offset_arrays[0], vp), sz(spec["a_ld"]), b_buffer,
+                              ctypes.cast(offset_arrays[1], vp), sz(spec["b_ld"]), ctypes.cast(betas_array, vp), c_buffer,
+                              ctypes.cast(offset_arrays[2], vp), sz(spec["c_ld"]), sz(count), ctypes.byref(queue),
+                              ctypes.byref(event))
         else:
             strides = spec["strides"]
-            function = getattr(reference, "CLBlast%sgemmStridedBatched" % PREFIX[bits])
+            function = getattr(reference, "CLBlast%sgemmStridedBatched" % prefix)
+            if is_complex:
+                function.argtypes = ([ctypes.c_int] * 3 + [sz] * 3 + [type(alpha), vp, sz, sz, sz, vp, sz, sz, sz, type(beta), vp,
+                                                                     sz, sz, sz, sz, vp, vp])
             status = function(ctypes.c_int(spec["layout"]), ctypes.c_int(spec["ta"]), ctypes.c_int(spec["tb"]), m, n, k,
                               alpha, a_buffer, sz(offsets[0]), sz(spec["a_ld"]), sz(strides[0]), b_buffer,
                               sz(offsets[1]), sz(spec["b_ld"]), sz(strides[1]), beta, c_buffer, sz(offsets[2]),
