@@ -309,6 +309,54 @@ class TrmmWorkload(Workload):
         return float((got - expected).norm() / expected.norm())
 
 
+class ComplexTrsmWorkload:
+    """CTRSM / ZTRSM in place, the X with A X = B for a lower triangular m x m A (column-major). As for the real TRSM
+    workload A is close to the identity (unit diagonal, off-diagonal elements of size 1/m), so that B keeps its
+    magnitude over hundreds of calls; the unused triangle holds NaN. 4 m^2 n real flops (the BLAS count of a complex
+    triangular solve)."""
+
+    def __init__(self, name, prefix, m, n):
+        import torch
+        self.name, self.prefix, self.m, self.n, self.beta, self.c_initial = name, prefix, m, n, 0.0, None
+        dtype = torch.complex64 if prefix == "C" else torch.complex128
+        generator = torch.Generator(device="cuda")
+        generator.manual_seed(2024)
+        draw = lambda rows, cols: torch.view_as_complex(  # noqa: E731
+            torch.rand(rows, cols, 2, device="cuda", dtype=torch.float64, generator=generator).mul_(2).sub_(1)).to(dtype)
+        square = draw(m, m).mul_(1.0 / m)  # memory [r, q] holds A(q, r): the lower triangle of A is torch's upper one
+        square.diagonal().fill_(1.0)
+        self.dense = torch.triu(square).contiguous()
+        square[torch.tril(torch.ones(m, m, device="cuda", dtype=torch.bool), -1)] = complex("nan+nanj")
+        self.a, self.b = square, draw(n, m)  # B (m x n, column-major) is torch's n x m
+        self.b_initial = self.b.clone()
+
+    @property
+    def flops(self):
+        return 4.0 * self.m * self.m * self.n
+
+    @property
+    def algorithmic_bytes(self):
+        return (BITS[self.prefix] // 8) * (self.m * self.m // 2 + 2 * self.m * self.n)
+
+    def call(self, stream_handle):
+        from clblast_amd.api import raw_complex_level3
+        status = raw_complex_level3("trsm", self.prefix, COL, 141, 122, NO, 131, self.m, self.n, 1.0, self.a.data_ptr(), 0, self.m,
+                                    self.b.data_ptr(), 0, self.m, stream_handle=stream_handle)
+        if status != 0:
+            raise RuntimeError("%s: status %d" % (self.name, status))
+
+    def freivalds_error(self):
+        """One call on the initial B, then A (X x) against B0 x."""
+        import torch
+        self.b.copy_(self.b_initial)
+        self.call(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        x = torch.rand(self.n, 1, device="cuda", dtype=torch.float64).sub_(0.5).to(torch.complex128)
+        a = self.dense.to(torch.complex128).T  # as a logical (row, column) matrix
+        got, expected = a @ (self.b.to(torch.complex128).T @ x), self.b_initial.to(torch.complex128).T @ x
+        return float((got - expected).norm() / expected.norm())
+
+
 class SyrkWorkload(Workload):
     """SYRK, the upper or lower triangle of C := alpha A A^T + beta C with A n x k (column-major); the other triangle
     of C holds NaN and must keep it."""
@@ -517,6 +565,7 @@ EXTRA_WORKLOADS = {
     "next_dtrmm_4096_colLeftUpperT": lambda: TrmmWorkload("trmm_d", "D", "trmm", False, True, 4096, 4096),
     "next_strsm_4096_colLeftLower": lambda: TrmmWorkload("trsm_s", "S", "trsm", True, False, 4096, 4096),
     "next_dtrsm_4096_colLeftUpperT": lambda: TrmmWorkload("trsm_d", "D", "trsm", False, True, 4096, 4096),
+    "next_ctrsm_4096_colLeftLower": lambda: ComplexTrsmWorkload("trsm_c", "C", 4096, 4096),
     "next_ssyrk_4096_colLower": lambda: SyrkWorkload("syrk_s", "S", True, 4096, 4096),
     "next_hsyrk_8192_colUpper": lambda: SyrkWorkload("syrk_h", "H", False, 8192, 8192),
 }

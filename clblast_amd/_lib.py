@@ -45,9 +45,10 @@ def _declare(lib):
             f = getattr(lib, "CLBlast%s%s" % (prefix, routine))
             f.argtypes = [c_int, c_int, c_int, sz, sz, scalar, vp, sz, sz, vp, sz, sz, beta_type, vp, sz, sz, vp, vp]
             f.restype = c_int
-        f = getattr(lib, "CLBlast%strmm" % prefix)
-        f.argtypes = [c_int] * 5 + [sz, sz, scalar, vp, sz, sz, vp, sz, sz, vp, vp]
-        f.restype = c_int
+        for routine in ("trmm", "trsm"):
+            f = getattr(lib, "CLBlast%s%s" % (prefix, routine))
+            f.argtypes = [c_int] * 5 + [sz, sz, scalar, vp, sz, sz, vp, sz, sz, vp, vp]
+            f.restype = c_int
         f = getattr(lib, "CLBlast%sgemmBatched" % prefix)
         f.argtypes = [c_int, c_int, c_int, sz, sz, sz, POINTER(scalar), vp, POINTER(sz), sz, vp, POINTER(sz), sz,
                       POINTER(scalar), vp, POINTER(sz), sz, sz, vp, vp]
@@ -116,7 +117,7 @@ C_API_SYMBOLS = (
     ["CLBlast%sgemm%s" % (p, s) for p in "SDH" for s in ("", "Batched", "StridedBatched", "WithTempBuffer")] +
     ["CLBlast%sGemmTempBufferSize" % p for p in "SDH"] + ["CLBlastCgemm", "CLBlastZgemm"] +
     ["CLBlast%sgemm%s" % (p, s) for p in "CZ" for s in ("Batched", "StridedBatched")] +
-    ["CLBlast%s%s" % (p, r) for p in "CZ" for r in ("symm", "hemm", "syrk", "herk", "syr2k", "her2k", "trmm")] +
+    ["CLBlast%s%s" % (p, r) for p in "CZ" for r in ("symm", "hemm", "syrk", "herk", "syr2k", "her2k", "trmm", "trsm")] +
     ["CLBlast%s%s" % (p, r) for p in "SDH" for r in ("symm", "syrk", "syr2k", "trmm")] + ["CLBlastStrsm", "CLBlastDtrsm"] +
     ["CLBlast%sconvgemm" % p for p in "SDH"] +
     ["CLBlastClearCache", "CLBlastOverrideParameters", "CLBlastFloatToHalf", "CLBlastHalfToFloat"])
@@ -128,4 +129,5 @@ DEVICE_LAYER_SYMBOLS = [
     "clbh_triangular_to_square", "clbh_copy_matrix", "clbh_invert_block_size", "clbh_invert_diagonal_blocks",
     "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale", "clbh_complex_expand_batched",
     "clbh_complex_transpose_batched", "clbh_complex_scale_batched", "clbh_alloc", "clbh_free", "clbh_copy", "clbh_im2col", "clbh_fill_zero", "clbh_complex_symmetric_to_square",
-    "clbh_complex_triangular_to_square", "clbh_complex_zero_diagonal_imag"]
+    "clbh_complex_triangular_to_square", "clbh_complex_zero_diagonal_imag", "clbh_complex_invert_block_size",
+    "clbh_complex_invert_diagonal_blocks"]

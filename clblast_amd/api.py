@@ -107,7 +107,7 @@ def raw_convgemm(prefix, kernel_mode, channels, height, width, kernel_h, kernel_
 
 
 def raw_complex_level3(routine, prefix, *arguments, stream_handle=0):
-    """CLBlast{C,Z}{symm,hemm,syrk,herk,syr2k,her2k,trmm} through the C ABI (reference: include/clblast_c.h:934-1092).
+    """CLBlast{C,Z}{symm,hemm,syrk,herk,syr2k,her2k,trmm,trsm} through the C ABI (reference: include/clblast_c.h:934-1117).
     `arguments` are those of the C function up to the last leading dimension; Python complex numbers (or floats for the
     real scalars of HERK and HER2K) stand for the scalars."""
     lib = _lib.load()

@@ -431,7 +431,15 @@ CLBLAST_HIP_COMPLEX_LEVEL3(float)
 CLBLAST_HIP_COMPLEX_LEVEL3(double)
 #undef CLBLAST_HIP_COMPLEX_LEVEL3
 
-// TRSM exists for float and double only (reference: src/clblast.cpp:1339-1346)
+// TRSM exists for float, double and the complex types (reference: src/clblast.cpp:1339-1354)
+template StatusCode CLBLAST_HIP_PUBLIC Trsm<float2>(const Layout, const Side, const Triangle, const Transpose, const Diagonal,
+                                                    const size_t, const size_t, const float2, const void*, const size_t,
+                                                    const size_t, void*, const size_t, const size_t, hipStream_t*,
+                                                    hipEvent_t*);
+template StatusCode CLBLAST_HIP_PUBLIC Trsm<double2>(const Layout, const Side, const Triangle, const Transpose, const Diagonal,
+                                                     const size_t, const size_t, const double2, const void*, const size_t,
+                                                     const size_t, void*, const size_t, const size_t, hipStream_t*,
+                                                     hipEvent_t*);
 template StatusCode CLBLAST_HIP_PUBLIC Trsm<float>(const Layout, const Side, const Triangle, const Transpose, const Diagonal,
                                                    const size_t, const size_t, const float, const void*, const size_t,
                                                    const size_t, void*, const size_t, const size_t, hipStream_t*,

@@ -456,22 +456,24 @@ CLBLAST_HIP_COMPLEX_SYR2K(CLBlastZsyr2k, CLBlastDouble2, double)
 CLBLAST_HIP_HER2K(CLBlastCher2k, CLBlastFloat2, float)
 CLBLAST_HIP_HER2K(CLBlastZher2k, CLBlastDouble2, double)
 
-#define CLBLAST_HIP_COMPLEX_TRMM(NAME, CTYPE, R)                                                                     \
+#define CLBLAST_HIP_COMPLEX_TRMM(NAME, ROUTINE, CTYPE, R)                                                              \
   CLBlastStatusCode NAME(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,         \
                          const CLBlastTranspose a_transpose, const CLBlastDiagonal diagonal, const size_t m,         \
                          const size_t n, const CTYPE alpha, const void* a_buffer, const size_t a_offset,             \
                          const size_t a_ld, void* b_buffer, const size_t b_offset, const size_t b_ld,                \
                          hipStream_t* queue, hipEvent_t* event) {                                                    \
     return Guarded([&]() {                                                                                           \
-      return clblast::Trmm<std::complex<R>>(L(layout), static_cast<clblast::Side>(side),                             \
+      return clblast::ROUTINE<std::complex<R>>(L(layout), static_cast<clblast::Side>(side),                          \
                                             static_cast<clblast::Triangle>(triangle), Tr(a_transpose),               \
                                             static_cast<clblast::Diagonal>(diagonal), m, n,                          \
                                             CLBLAST_HIP_TO_COMPLEX_##R(alpha), a_buffer, a_offset, a_ld, b_buffer,   \
                                             b_offset, b_ld, queue, event);                                           \
     });                                                                                                              \
   }
-CLBLAST_HIP_COMPLEX_TRMM(CLBlastCtrmm, CLBlastFloat2, float)
-CLBLAST_HIP_COMPLEX_TRMM(CLBlastZtrmm, CLBlastDouble2, double)
+CLBLAST_HIP_COMPLEX_TRMM(CLBlastCtrmm, Trmm, CLBlastFloat2, float)
+CLBLAST_HIP_COMPLEX_TRMM(CLBlastZtrmm, Trmm, CLBlastDouble2, double)
+CLBLAST_HIP_COMPLEX_TRMM(CLBlastCtrsm, Trsm, CLBlastFloat2, float)
+CLBLAST_HIP_COMPLEX_TRMM(CLBlastZtrsm, Trsm, CLBlastDouble2, double)
 
 // ---- SYRK, SYR2K --------------------------------------------------------------------------------
 #define CLBLAST_HIP_SYRK(NAME, CTYPE, TYPE)                                                                          \

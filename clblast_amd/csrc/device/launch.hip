@@ -443,21 +443,38 @@ int clbh_complex_symmetric_to_square(int precision, int upper, int hermitian, in
 }
 
 int clbh_complex_triangular_to_square(int precision, int upper, int unit_diagonal, int k, const void* src, long long src_offset,
-                                      long long src_ld, void* dst, long long dst_ld, hipStream_t stream) {
-  if (k <= 0 || src == nullptr || dst == nullptr || src_ld < k || dst_ld < k || src_offset < 0) { return hipErrorInvalidValue; }
-  const dim3 grid(Blocks(k, clbh::kComplexThreads), static_cast<unsigned>(std::min(k, 16384)));
+                                      long long src_ld, void* dst, int dst_extent, long long dst_ld, hipStream_t stream) {
+  if (k <= 0 || src == nullptr || dst == nullptr || src_ld < k || dst_extent < k || dst_ld < dst_extent || src_offset < 0) {
+    return hipErrorInvalidValue;
+  }
+  const dim3 grid(Blocks(dst_extent, clbh::kComplexThreads), static_cast<unsigned>(std::min(dst_extent, 16384)));
   if (precision == 32) {
     clbh::ComplexTriangularToSquareKernel<float><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
-        k, upper != 0, unit_diagonal != 0, static_cast<const clbh::ComplexOf<float>*>(src) + src_offset, src_ld,
+        k, dst_extent, upper != 0, unit_diagonal != 0, static_cast<const clbh::ComplexOf<float>*>(src) + src_offset, src_ld,
         static_cast<clbh::ComplexOf<float>*>(dst), dst_ld);
   } else if (precision == 64) {
     clbh::ComplexTriangularToSquareKernel<double><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
-        k, upper != 0, unit_diagonal != 0, static_cast<const clbh::ComplexOf<double>*>(src) + src_offset, src_ld,
+        k, dst_extent, upper != 0, unit_diagonal != 0, static_cast<const clbh::ComplexOf<double>*>(src) + src_offset, src_ld,
         static_cast<clbh::ComplexOf<double>*>(dst), dst_ld);
   } else {
     return hipErrorInvalidValue;
   }
   return static_cast<int>(hipGetLastError());
+}
+
+int clbh_complex_invert_block_size(int precision) { return (precision == 64) ? 32 : 64; }
+
+int clbh_complex_invert_diagonal_blocks(int precision, int upper, int blocks, const void* src, long long src_ld, void* dst,
+                                        long long dst_ld, hipStream_t stream) {
+  const long long extent = static_cast<long long>(blocks) * clbh_complex_invert_block_size(precision);
+  if (blocks <= 0 || src == nullptr || dst == nullptr || src_ld < extent || dst_ld < extent) { return hipErrorInvalidValue; }
+  if (precision == 32) {
+    return LaunchInvertDiagonalBlocks<clbh::ComplexOf<float>, clbh::ComplexOf<float>, 64>(upper, blocks, src, src_ld, dst, dst_ld, stream);
+  }
+  if (precision == 64) {
+    return LaunchInvertDiagonalBlocks<clbh::ComplexOf<double>, clbh::ComplexOf<double>, 32>(upper, blocks, src, src_ld, dst, dst_ld, stream);
+  }
+  return hipErrorInvalidValue;
 }
 
 int clbh_complex_zero_diagonal_imag(int precision, int n, void* c, long long c_offset, long long c_ld, hipStream_t stream) {

@@ -28,7 +28,21 @@ constexpr int kComplexThreads = 256;
 template <typename R>
 struct ComplexOf {
   R re, im;
+  ComplexOf() = default;
+  __host__ __device__ constexpr ComplexOf(const R real, const R imaginary = R(0)) : re(real), im(imaginary) {}
+  __device__ __forceinline__ ComplexOf& operator+=(const ComplexOf other) { re += other.re; im += other.im; return *this; }
+  __device__ __forceinline__ ComplexOf& operator-=(const ComplexOf other) { re -= other.re; im -= other.im; return *this; }
 };
+// The arithmetic the block inversion of the complex TRSM is written in (kernels/triangular_to_square.hpp)
+template <typename R>
+__device__ __forceinline__ ComplexOf<R> operator*(const ComplexOf<R> a, const ComplexOf<R> b) {
+  return ComplexOf<R>(a.re * b.re - a.im * b.im, a.re * b.im + a.im * b.re);
+}
+template <typename R>
+__device__ __forceinline__ ComplexOf<R> operator/(const ComplexOf<R> a, const ComplexOf<R> b) {
+  const R scale = R(1) / (b.re * b.re + b.im * b.im);
+  return ComplexOf<R>((a.re * b.re + a.im * b.im) * scale, (a.im * b.re - a.re * b.im) * scale);
+}
 
 // The matrices of a batched call: matrix b of the source starts src_offsets[b] (when given) or b * src_stride complex
 // elements behind the kernel's source pointer, its result b * dst_stride elements (of the result's type) behind the
@@ -184,24 +198,26 @@ __global__ __launch_bounds__(kComplexThreads) void ComplexSymmetricToSquareKerne
   }
 }
 
-// Dense k x k copy (leading dimension dst_ld) of a complex triangular matrix: zeros in the other triangle, ones on an
-// implied diagonal (reference: src/kernels/level3/convert_triangular.opencl:24-94). grid: (ceil(k / 256), min(k, 16384)).
+// Dense extent x extent copy (extent >= k, leading dimension dst_ld) of a complex triangular k x k matrix: zeros in the
+// other triangle, ones on an implied diagonal, the identity in rows and columns k .. extent - 1 (reference:
+// src/kernels/level3/convert_triangular.opencl:24-94). grid: (ceil(extent / 256), min(extent, 16384)).
 template <typename R>
-__global__ __launch_bounds__(kComplexThreads) void ComplexTriangularToSquareKernel(const int k, const bool upper,
-                                                                                   const bool unit,
+__global__ __launch_bounds__(kComplexThreads) void ComplexTriangularToSquareKernel(const int k, const int extent,
+                                                                                   const bool upper, const bool unit,
                                                                                    const ComplexOf<R>* __restrict__ src,
                                                                                    const long long src_ld,
                                                                                    ComplexOf<R>* __restrict__ dst,
                                                                                    const long long dst_ld) {
   const int one = blockIdx.x * kComplexThreads + threadIdx.x;
-  if (one >= k) { return; }
-  for (int two = blockIdx.y; two < k; two += gridDim.y) {
+  if (one >= extent) { return; }
+  for (int two = blockIdx.y; two < extent; two += gridDim.y) {
     ComplexOf<R> value;
     value.re = R(0);
     value.im = R(0);
+    const bool inside = (one < k && two < k);
     const bool is_stored = upper ? (one <= two) : (one >= two);
-    if (one == two && unit) { value.re = R(1); }
-    else if (is_stored) { value = src[two * src_ld + one]; }
+    if (one == two && (unit || !inside)) { value.re = R(1); }
+    else if (inside && is_stored) { value = src[two * src_ld + one]; }
     dst[two * dst_ld + one] = value;
   }
 }

@@ -196,8 +196,8 @@ void Xlevel3Complex<R>::DoTrmm(const Layout layout, const Side side, const Trian
   const StreamScratch square(square_bytes, this->stream(), "square copy of the triangular matrix");
   CheckDevice(clbh_complex_triangular_to_square(component_bits, is_upper ? 1 : 0, (diagonal == Diagonal::kUnit) ? 1 : 0,
                                                 static_cast<int>(k), a_buffer(), static_cast<long long>(a_offset),
-                                                static_cast<long long>(a_ld), square.get(), static_cast<long long>(k),
-                                                this->stream()),
+                                                static_cast<long long>(a_ld), square.get(), static_cast<int>(k),
+                                                static_cast<long long>(k), this->stream()),
               "clbh_complex_triangular_to_square");
   const auto square_buffer = Buffer<Complex>(square.get(), square_bytes);
   const auto copy_buffer = Buffer<Complex>(b_copy.get(), copy_bytes);

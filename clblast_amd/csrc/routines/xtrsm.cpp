@@ -3,8 +3,6 @@
 // =================================================================================================
 #include "routines/xtrsm.hpp"
 
-#include "routines/xgemmbatched.hpp"
-
 #include <climits>
 #include <functional>
 #include <utility>
@@ -13,7 +11,7 @@ namespace clblast {
 // =================================================================================================
 
 template <typename T>
-Xtrsm<T>::Xtrsm(hipStream_t* queue, hipEvent_t* event) : Xgemm<T>(queue, event) {}
+Xtrsm<T>::Xtrsm(hipStream_t* queue, hipEvent_t* event) : TrsmEngine<T>::Gemm(queue, event) {}
 
 template <typename T>
 void Xtrsm<T>::DoTrsm(const Layout layout, Side side, Triangle triangle, const Transpose a_transpose,
@@ -46,13 +44,15 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
   TestMatrixA(k, k, a_buffer, a_offset, a_ld);
   TestMatrixB(m, n, b_buffer, b_offset, b_ld);
 
-  const auto precision = static_cast<int>(PrecisionValue<T>());
+  using Engine = TrsmEngine<T>;
+  constexpr auto precision = Engine::kComponentBits;  // what the device layer calls the precision of complex data too
   auto stream = this->stream();
   constexpr size_t kLineMultiple = 16 / sizeof(T);
   // Diagonal blocks: `block` is what the inversion kernel inverts; the inverses are then doubled in size with GEMMs
   // up to the leaf size of the recursion (at most kMaxLeaf, and no more doublings than the matrix has use for)
   constexpr size_t kMaxLeaf = 512;
-  const auto block = static_cast<size_t>(clbh_invert_block_size(precision));
+  const auto block = static_cast<size_t>(Engine::kComplex ? clbh_complex_invert_block_size(precision)
+                                                          : clbh_invert_block_size(precision));
   auto leaf = block;
   while (leaf < kMaxLeaf && leaf < k) { leaf *= 2; }
   const auto k_padded = (k + leaf - 1) / leaf * leaf;
@@ -62,10 +62,10 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
   const auto dense_bytes = k_padded * k_padded * sizeof(T);
   const StreamScratch dense(dense_bytes, stream, "dense copy of the triangular matrix");
   const auto is_upper = (triangle == Triangle::kUpper);
-  CheckDevice(clbh_triangular_to_square(precision, is_upper ? 1 : 0, (diagonal == Diagonal::kUnit) ? 1 : 0,
-                                        static_cast<int>(k), a_buffer(), static_cast<long long>(a_offset),
-                                        static_cast<long long>(a_ld), dense.get(), static_cast<int>(k_padded),
-                                        static_cast<long long>(k_padded), stream),
+  const auto to_square = Engine::kComplex ? clbh_complex_triangular_to_square : clbh_triangular_to_square;
+  CheckDevice(to_square(precision, is_upper ? 1 : 0, (diagonal == Diagonal::kUnit) ? 1 : 0, static_cast<int>(k), a_buffer(),
+                        static_cast<long long>(a_offset), static_cast<long long>(a_ld), dense.get(),
+                        static_cast<int>(k_padded), static_cast<long long>(k_padded), stream),
               "clbh_triangular_to_square");
   const auto dense_buffer = Buffer<T>(dense.get(), dense_bytes);
 
@@ -73,9 +73,9 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
   // copy, each inverse in the place of its block, zeros elsewhere
   const StreamScratch inverses(dense_bytes, stream, "inverted diagonal blocks");
   CheckDevice(clbh_fill_zero(inverses.get(), dense_bytes, stream), "clbh_fill_zero");
-  CheckDevice(clbh_invert_diagonal_blocks(precision, is_upper ? 1 : 0, static_cast<int>(k_padded / block), dense.get(),
-                                          static_cast<long long>(k_padded), inverses.get(),
-                                          static_cast<long long>(k_padded), stream),
+  const auto invert = Engine::kComplex ? clbh_complex_invert_diagonal_blocks : clbh_invert_diagonal_blocks;
+  CheckDevice(invert(precision, is_upper ? 1 : 0, static_cast<int>(k_padded / block), dense.get(),
+                     static_cast<long long>(k_padded), inverses.get(), static_cast<long long>(k_padded), stream),
               "clbh_invert_diagonal_blocks");
   const auto inverse_buffer = Buffer<T>(inverses.get(), dense_bytes);
   if (leaf > block) {
@@ -86,7 +86,7 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
     const auto product_bytes = (k_padded / 2) * (leaf / 2) * sizeof(T);
     const StreamScratch products(product_bytes, stream, "block products of the inversion");
     const auto product_buffer = Buffer<T>(products.get(), product_bytes);
-    auto batched = XgemmStridedBatched<T>(&stream, nullptr);
+    auto batched = typename Engine::StridedBatched(&stream, nullptr);
     for (auto size = block; size < leaf; size *= 2) {
       const auto pairs = k_padded / (2 * size);
       const auto diagonal_step = 2 * size * (k_padded + 1);
@@ -109,7 +109,6 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
   const StreamScratch solution(x_bytes, stream, "solution of the triangular system");
 
   const auto x_buffer = Buffer<T>(solution.get(), x_bytes);
-  const auto no_temp = Buffer<T>(nullptr);
   const auto one = ConstantOne<T>();
   const auto zero = ConstantZero<T>();
   const auto minus_one = ConstantNegOne<T>();
@@ -126,8 +125,13 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
                         const T galpha, const Buffer<T>& ga, const size_t ga_offset, const size_t ga_ld,
                         const Buffer<T>& gb, const size_t gb_offset, const size_t gb_ld, const T gbeta,
                         const Buffer<T>& gc, const size_t gc_offset, const size_t gc_ld) {
-    this->DoGemm(Layout::kColMajor, ta, tb, gm, gn, gk, galpha, ga, ga_offset, ga_ld, gb, gb_offset, gb_ld, gbeta, gc,
-                 gc_offset, gc_ld, no_temp, false, GemmTriangles{}, false);
+    if constexpr (Engine::kComplex) {
+      this->DoGemm(Layout::kColMajor, ta, tb, gm, gn, gk, galpha, ga, ga_offset, ga_ld, gb, gb_offset, gb_ld, gbeta, gc,
+                   gc_offset, gc_ld, OutputTriangle::kFull, false);
+    } else {
+      this->DoGemm(Layout::kColMajor, ta, tb, gm, gn, gk, galpha, ga, ga_offset, ga_ld, gb, gb_offset, gb_ld, gbeta, gc,
+                   gc_offset, gc_ld, Buffer<T>(nullptr), false, GemmTriangles{}, false);
+    }
   };
 
   // Solves for the rows (left) or columns (right) [lo, hi) of X. `scaled`: this part of B has already been multiplied by
@@ -163,7 +167,7 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
   };
   solve(0, k, false);
 
-  CheckDevice(clbh_copy_matrix(precision, static_cast<int>(m), static_cast<int>(n), solution.get(), 0,
+  CheckDevice(clbh_copy_matrix(static_cast<int>(8 * sizeof(T)), static_cast<int>(m), static_cast<int>(n), solution.get(), 0,
                                static_cast<long long>(x_ld), const_cast<void*>(b_buffer()), static_cast<long long>(b_offset),
                                static_cast<long long>(b_ld), stream),
               "clbh_copy_matrix");
@@ -172,6 +176,8 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
 
 template class Xtrsm<float>;
 template class Xtrsm<double>;
+template class Xtrsm<std::complex<float>>;
+template class Xtrsm<std::complex<double>>;
 
 // =================================================================================================
 }  // namespace clblast

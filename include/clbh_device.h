@@ -169,11 +169,16 @@ CLBH_API int clbh_copy(void* dst, const void* src, size_t bytes, int to_device);
 // Complex symmetric (hermitian == 0) or Hermitian k x k matrix with one stored triangle -> dense k x k (leading dimension k)
 CLBH_API int clbh_complex_symmetric_to_square(int precision, int upper, int hermitian, int k, const void* src,
                                               long long src_offset, long long src_ld, void* dst, hipStream_t stream);
-// Complex triangular k x k matrix -> dense k x k (leading dimension dst_ld): zeros in the other triangle, ones on an
-// implied diagonal
+// Complex triangular k x k matrix -> dense dst_extent x dst_extent (dst_extent >= k, leading dimension dst_ld): zeros in
+// the other triangle, ones on an implied diagonal, the identity in rows and columns k .. dst_extent - 1
 CLBH_API int clbh_complex_triangular_to_square(int precision, int upper, int unit_diagonal, int k, const void* src,
-                                               long long src_offset, long long src_ld, void* dst, long long dst_ld,
-                                               hipStream_t stream);
+                                               long long src_offset, long long src_ld, void* dst, int dst_extent,
+                                               long long dst_ld, hipStream_t stream);
+// clbh_invert_block_size and clbh_invert_diagonal_blocks for complex matrices (blocks of 64 for 32-bit components, 32
+// for 64-bit ones)
+CLBH_API int clbh_complex_invert_block_size(int precision);
+CLBH_API int clbh_complex_invert_diagonal_blocks(int precision, int upper, int blocks, const void* src, long long src_ld,
+                                                 void* dst, long long dst_ld, hipStream_t stream);
 // Im(C(i,i)) = 0 for i < n; C(i,j) at c[c_offset + j*c_ld + i]
 CLBH_API int clbh_complex_zero_diagonal_imag(int precision, int n, void* c, long long c_offset, long long c_ld,
                                              hipStream_t stream);

@@ -114,8 +114,8 @@ using double2 = std::complex<double>;
 // =================================================================================================
 
 // C = alpha * op(A) * op(B) + beta * C. T is float, double, half, float2 or double2 (the complex types take no
-// temp_buffer). GemmBatched, GemmStridedBatched, Symm, Syrk, Syr2k and Trmm below also exist for float2 and double2;
-// Trsm and Convgemm do not.
+// temp_buffer). GemmBatched, GemmStridedBatched, Symm, Syrk, Syr2k, Trmm and Trsm below also exist for float2 and
+// double2; Convgemm, like the reference's, does not.
 template <typename T>
 StatusCode Gemm(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
                 const size_t n, const size_t k, const T alpha, const void* a_buffer, const size_t a_offset,
@@ -202,8 +202,8 @@ StatusCode Trmm(const Layout layout, const Side side, const Triangle triangle, c
 
 // Solves a triangular system in place: B becomes the X with op(A) * X = alpha * B (side left, A is m x m) or
 // X * op(A) = alpha * B (side right, A is n x n); only the named triangle of A is read, and not its diagonal when
-// that is `kUnit`. T is float or double: like the reference this routine has no half-precision version (reference:
-// include/clblast.h:484-488, src/clblast.cpp:1339-1346, src/routines/level3/xtrsm.cpp:38-246).
+// that is `kUnit`. T is float, double, float2 or double2: like the reference this routine has no half-precision version
+// (reference: include/clblast.h:484-488, src/clblast.cpp:1339-1354, src/routines/level3/xtrsm.cpp:38-246).
 template <typename T>
 StatusCode Trsm(const Layout layout, const Side side, const Triangle triangle, const Transpose a_transpose,
                 const Diagonal diagonal, const size_t m, const size_t n, const T alpha, const void* a_buffer,

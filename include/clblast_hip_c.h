@@ -353,7 +353,8 @@ CLBlastStatusCode CLBLAST_HIP_API CLBlastHconvgemm(const CLBlastKernelMode kerne
                                                    hipEvent_t* event);
 
 // Triangular solve in place: B becomes the X with op(A)*X = alpha*B (side left) or X*op(A) = alpha*B (side right)
-// replaces CLBlastStrsm/CLBlastDtrsm; like the reference there is no half-precision TRSM (reference: include/clblast_c.h:1094-1124, src/clblast_c.cpp:2402-2500)
+// replaces CLBlastStrsm/CLBlastDtrsm/CLBlastCtrsm/CLBlastZtrsm; like the reference there is no half-precision TRSM
+// (reference: include/clblast_c.h:1094-1117, src/clblast_c.cpp:2265-2324)
 CLBlastStatusCode CLBLAST_HIP_API CLBlastStrsm(const CLBlastLayout layout, const CLBlastSide side,
                                                const CLBlastTriangle triangle, const CLBlastTranspose a_transpose,
                                                const CLBlastDiagonal diagonal, const size_t m, const size_t n,
@@ -364,6 +365,18 @@ CLBlastStatusCode CLBLAST_HIP_API CLBlastDtrsm(const CLBlastLayout layout, const
                                                const CLBlastTriangle triangle, const CLBlastTranspose a_transpose,
                                                const CLBlastDiagonal diagonal, const size_t m, const size_t n,
                                                const double alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastCtrsm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const CLBlastTranspose a_transpose,
+                                               const CLBlastDiagonal diagonal, const size_t m, const size_t n,
+                                               const CLBlastFloat2 alpha, const void* a_buffer, const size_t a_offset,
+                                               const size_t a_ld, void* b_buffer, const size_t b_offset,
+                                               const size_t b_ld, hipStream_t* queue, hipEvent_t* event);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastZtrsm(const CLBlastLayout layout, const CLBlastSide side,
+                                               const CLBlastTriangle triangle, const CLBlastTranspose a_transpose,
+                                               const CLBlastDiagonal diagonal, const size_t m, const size_t n,
+                                               const CLBlastDouble2 alpha, const void* a_buffer, const size_t a_offset,
                                                const size_t a_ld, void* b_buffer, const size_t b_offset,
                                                const size_t b_ld, hipStream_t* queue, hipEvent_t* event);
 

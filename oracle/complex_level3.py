@@ -76,3 +76,18 @@ def trmm(layout, side, triangle, a_transpose, diagonal, m, n, alpha, a, a_offset
     op_a = dense if a_transpose == NO else (dense.T if a_transpose == YES else dense.conj().T)
     b_matrix = matrix(layout, b, b_offset, b_ld, m, n)
     return alpha * (op_a @ b_matrix if side == LEFT else b_matrix @ op_a)
+
+
+def trsm(layout, side, triangle, a_transpose, diagonal, m, n, alpha, a, a_offset, a_ld, b, b_offset, b_ld):
+    """TRSM: the X with op(A) * X = alpha * B (left) or X * op(A) = alpha * B (right) (reference:
+    src/routines/level3/xtrsm.cpp:38-246), by a general dense solve on the matrix built from the stored triangle."""
+    k = m if side == LEFT else n
+    stored = matrix(layout, a, a_offset, a_ld, k, k)
+    dense = np.triu(stored) if triangle == UPPER else np.tril(stored)
+    if diagonal == UNIT:
+        np.fill_diagonal(dense, 1.0)
+    op_a = dense if a_transpose == NO else (dense.T if a_transpose == YES else dense.conj().T)
+    right_hand_side = alpha * matrix(layout, b, b_offset, b_ld, m, n)
+    if side == LEFT:
+        return np.linalg.solve(op_a, right_hand_side)
+    return np.linalg.solve(op_a.T, right_hand_side.T).T

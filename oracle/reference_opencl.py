@@ -136,9 +136,9 @@ def run(spec):
     c = generate(seed * 3 + 2, sizes[2], spec.get("low", -1.0), spec.get("high", 1.0), bits)
     if spec.get("a_diagonal_boost"):  # well-conditioned triangular solves (tests/level3_harness.py does the same):
         k_diag, boost = spec["k_diag"], spec["a_diagonal_boost"]  # off-diagonal row sums below 1, |diagonal| >= boost
-        a = (a.astype(np.float64) * (2.0 / k_diag)).astype(a.dtype)
+        a = (a.astype(np.complex128 if is_complex else np.float64) * (2.0 / k_diag)).astype(a.dtype)
         positions = spec["offsets"][0] + np.arange(k_diag) * (spec["a_ld"] + 1)
-        a[positions] = a[positions] + np.where(a[positions] >= 0, boost, -boost).astype(a.dtype)
+        a[positions] = a[positions] + np.where(np.real(a[positions]) >= 0, boost, -boost).astype(a.dtype)
     a_buffer, b_buffer, c_buffer = opencl.buffer_from(a), opencl.buffer_from(b), opencl.buffer_from(c)
     in_place_b = spec["routine"] in ("trmm", "trsm")  # these overwrite B; "c" is then unused
     sz, vp = ctypes.c_size_t, ctypes.c_void_p
@@ -151,7 +151,7 @@ def run(spec):
 
     def call():
         event = vp(None)
-        if is_complex and spec["routine"] in ("symm", "hemm", "syrk", "herk", "syr2k", "her2k", "trmm"):
+        if is_complex and spec["routine"] in ("symm", "hemm", "syrk", "herk", "syr2k", "her2k", "trmm", "trsm"):
             # the complex Level-3 routines: "side", "triangle", "ta", "diagonal" as far as the routine has them; HERK takes
             # real alpha and beta, HER2K a real beta ("alpha"/"beta" are [re, im] pairs, the imaginary part then unused)
             name = spec["routine"]

@@ -1,5 +1,5 @@
 """The numpy restatements of the complex Level-3 routines (oracle/complex_level3.py) pinned against the Fortran BLAS that
-scipy links: zsymm, zhemm, zsyrk, zherk, zsyr2k, zher2k, ztrmm, over sides, triangles and transposes, with NaN in every
+scipy links: zsymm, zhemm, zsyrk, zherk, zsyr2k, zher2k, ztrmm, ztrsm, over sides, triangles and transposes, with NaN in every
 element the routine must not read (the other triangle; for the Hermitian routines also the imaginary part of the
 diagonal is poisoned with a finite value that must not matter)."""
 import itertools
@@ -110,3 +110,25 @@ def test_trmm_matches_the_fortran_blas():
                           diag=int(diagonal == UNIT))
         got = complex_level3.trmm(COL_MAJOR, side, triangle, transpose, diagonal, m, n, 0.5 + 2j, a, 0, a_ld, b, 0, b_ld)
         assert np.abs(got - want).max() <= 1e-13, (side, triangle, transpose, diagonal)
+
+
+def test_trsm_matches_the_fortran_blas():
+    for side, triangle, transpose, diagonal in itertools.product((LEFT, RIGHT), (UPPER, LOWER), (NO, YES, CONJ), (NON_UNIT, UNIT)):
+        m, n = 9, 6
+        k = m if side == LEFT else n
+        stored = poisoned_triangle(k, triangle) / k
+        stored[np.diag_indices(k)] += 2.0  # well conditioned
+        if diagonal == UNIT:
+            np.fill_diagonal(stored, np.nan + 1j * np.nan)
+        b_matrix = draw(m, n)
+        a, a_ld = column_major(stored, 1)
+        b, b_ld = column_major(b_matrix, 2)
+        want = blas.ztrsm(0.5 + 2j, np.asfortranarray(np.nan_to_num(stored, nan=9.0)), np.asfortranarray(b_matrix),
+                          side=int(side == RIGHT), lower=int(triangle == LOWER), trans_a={NO: 0, YES: 1, CONJ: 2}[transpose],
+                          diag=int(diagonal == UNIT))
+        got = complex_level3.trsm(COL_MAJOR, side, triangle, transpose, diagonal, m, n, 0.5 + 2j, a, 0, a_ld, b, 0, b_ld)
+        assert np.abs(got - want).max() <= 1e-12, (side, triangle, transpose, diagonal)
+        # the row-major call on the same memory is the column-major call on the transposed problem
+        as_rows = complex_level3.trsm(ROW_MAJOR, RIGHT if side == LEFT else LEFT, LOWER if triangle == UPPER else UPPER,
+                                      transpose, diagonal, n, m, 0.5 + 2j, a, 0, a_ld, b, 0, b_ld)
+        assert np.abs(as_rows.T - want).max() <= 1e-12

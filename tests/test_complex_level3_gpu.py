@@ -1,4 +1,4 @@
-"""The complex Level-3 routines through the C ABI (CLBlast{C,Z}symm, hemm, syrk, herk, syr2k, her2k, trmm; reference:
+"""The complex Level-3 routines through the C ABI (CLBlast{C,Z}symm, hemm, syrk, herk, syr2k, her2k, trmm, trsm; reference:
 include/clblast_c.h:934-1092) against the numpy oracle (oracle/complex_level3.py, pinned against scipy's Fortran BLAS)
 and against the real reference on the same GPU. Every element a routine must not read holds NaN (the other triangle of
 A, the other triangle of C), an implied unit diagonal too; the imaginary part of a Hermitian diagonal holds a value
@@ -111,24 +111,39 @@ def run_rank_update(gpu, bits, hermitian, two_sided, layout, triangle, transpose
     return case, expected, where, inside, name
 
 
-def run_trmm(gpu, bits, layout, side, triangle, transpose, diagonal, m, n, alpha, seed, poison=True):
+DIAGONAL_BOOST = 4.0
+
+
+def run_triangular(routine, gpu, bits, layout, side, triangle, transpose, diagonal, m, n, alpha, seed, poison=True):
+    """TRMM or TRSM. For TRSM the matrix is made well conditioned the way the reference host (oracle/reference_opencl.py,
+    "a_diagonal_boost") does: off-diagonal elements scaled by 2 / k, the diagonal pushed away from zero by 4."""
     k = m if side == LEFT else n
     case = Case(bits, seed, [(k, k), (m, n), (1, 1)], layout, (seed % 3, 1, 0), ((0, 0, 0), (5, 3, 0))[seed % 2])
     a, b, _ = case.buffers
+    if routine == "trsm":
+        a = (a.astype(np.complex128) * (2.0 / k)).astype(a.dtype)
+        positions = case.offsets[0] + np.arange(k) * (case.ld[0] + 1)
+        a[positions] = a[positions] + np.where(np.real(a[positions]) >= 0, DIAGONAL_BOOST, -DIAGONAL_BOOST).astype(a.dtype)
+        case.buffers[0] = a
     clean = a.copy()
     if poison:
         poison_triangle(a, layout, triangle, k, case.offsets[0], case.ld[0], with_diagonal=(diagonal == UNIT))
-    expected = complex_level3.trmm(layout, side, triangle, transpose, diagonal, m, n, alpha, clean, case.offsets[0], case.ld[0], b,
-                                   case.offsets[1], case.ld[1])
+    restatement = complex_level3.trsm if routine == "trsm" else complex_level3.trmm
+    expected = restatement(layout, side, triangle, transpose, diagonal, m, n, alpha, clean, case.offsets[0], case.ld[0], b,
+                           case.offsets[1], case.ld[1])
     a_dev, b_dev, _ = case.device(gpu)
-    status = clblast_amd.raw_complex_level3("trmm", PREFIX[bits], layout, side, triangle, transpose, diagonal, m, n, alpha,
+    status = clblast_amd.raw_complex_level3(routine, PREFIX[bits], layout, side, triangle, transpose, diagonal, m, n, alpha,
                                             a_dev.data_ptr(), case.offsets[0], case.ld[0], b_dev.data_ptr(), case.offsets[1],
                                             case.ld[1], stream_handle=gpu.stream_handle())
     torch.cuda.synchronize()
     assert status == 0
     where = oracle.c_indices(layout, m, n, case.offsets[1], case.ld[1])
-    check_region(b_dev.cpu().numpy(), b, where, expected, bits, label=("trmm", layout, side, triangle, transpose, diagonal, m, n))
+    check_region(b_dev.cpu().numpy(), b, where, expected, bits, label=(routine, layout, side, triangle, transpose, diagonal, m, n))
     return case, expected, where
+
+
+def run_trmm(gpu, *arguments, **options):
+    return run_triangular("trmm", gpu, *arguments, **options)
 
 
 SIZES = ((7, 7), (7, 64), (64, 7), (65, 130), (200, 96), (1, 1), (129, 3))
@@ -168,6 +183,25 @@ def test_complex_trmm(gpu, bits):
         for m, n in SIZES[:5]:
             seed += 1
             run_trmm(gpu, bits, layout, side, triangle, transpose, diagonal, m, n, (1.0, 0.5 - 1.5j, -1j)[seed % 3], seed)
+
+
+@pytest.mark.parametrize("bits", (32, 64))
+def test_complex_trsm(gpu, bits):
+    seed = 22500
+    for layout, side, triangle, transpose, diagonal in itertools.product((ROW_MAJOR, COL_MAJOR), (LEFT, RIGHT), (UPPER, LOWER),
+                                                                         (NO, YES, CONJ), (NON_UNIT, UNIT)):
+        for m, n in SIZES[:5]:
+            seed += 1
+            run_triangular("trsm", gpu, bits, layout, side, triangle, transpose, diagonal, m, n, (1.0, 0.5 - 1.5j, -1j)[seed % 3], seed)
+
+
+def test_complex_trsm_large(gpu):
+    """Several inverted blocks, doubling levels and recursion levels: 64-blocks doubled to 512 leaves (complex64), 32-blocks
+    (complex128), sizes that are no multiple of either."""
+    run_triangular("trsm", gpu, 32, COL_MAJOR, LEFT, LOWER, NO, NON_UNIT, 1300, 200, 0.5 - 1.5j, 22901)
+    run_triangular("trsm", gpu, 32, ROW_MAJOR, RIGHT, UPPER, CONJ, UNIT, 300, 1100, 1.0, 22902)
+    run_triangular("trsm", gpu, 64, COL_MAJOR, RIGHT, UPPER, YES, NON_UNIT, 260, 700, -1j, 22903)
+    run_triangular("trsm", gpu, 64, ROW_MAJOR, LEFT, LOWER, CONJ, NON_UNIT, 1030, 150, 0.5 - 1.5j, 22904)
 
 
 def test_complex_level3_large(gpu):
@@ -216,6 +250,14 @@ def test_complex_level3_against_the_real_reference(gpu, tmp_path):
             spec = dict(routine="trmm", complex=True, bits=bits, layout=layout, side=side, triangle=triangle, ta=transpose,
                         diagonal=diagonal, m=m, n=n, alpha=[0.5, -1.5], a_ld=case.ld[0], b_ld=case.ld[1],
                         offsets=list(case.offsets), seed=seed, sizes=case.sizes, runs=0)
+            entries.append((spec, expected, where, None, bits))
+            seed += 1
+            case, expected, where = run_triangular("trsm", gpu, bits, layout, side, triangle, transpose, diagonal, m, n, 0.5 - 1.5j,
+                                                   seed, poison=False)
+            spec = dict(routine="trsm", complex=True, bits=bits, layout=layout, side=side, triangle=triangle, ta=transpose,
+                        diagonal=diagonal, m=m, n=n, alpha=[0.5, -1.5], a_ld=case.ld[0], b_ld=case.ld[1],
+                        offsets=list(case.offsets), seed=seed, sizes=case.sizes, runs=0, a_diagonal_boost=DIAGONAL_BOOST,
+                        k_diag=(m if side == LEFT else n))
             entries.append((spec, expected, where, None, bits))
     data, summary = run_reference([entry[0] for entry in entries], tmp_path)
     for index, (spec, expected, where, inside, bits) in enumerate(entries):
