@@ -18,6 +18,7 @@ namespace {
 
 int LaunchTyped(const clbh_gemm_desc& d, hipStream_t stream) {
   const bool mfma = (d.kernel_class == CLBH_KERNEL_MFMA);
+  if (d.conv != nullptr && !(mfma && d.precision == 32)) { return hipErrorInvalidValue; }  // only that kernel gathers
   if (d.kernel_class == CLBH_KERNEL_SMALL_BATCHED) { return LaunchSmallBatched(d, stream); }
   switch (d.precision) {
     case 16: return mfma ? LaunchMfmaF16(d, stream) : LaunchGeneralF16(d, stream);
@@ -385,6 +386,10 @@ int clbh_complex_scale_batched(int precision, int m, int n, int triangle, double
 int clbh_complex_scale(int precision, int m, int n, int triangle, double beta_re, double beta_im, void* c, long long c_offset,
                        long long c_ld, hipStream_t stream) {
   return clbh_complex_scale_batched(precision, m, n, triangle, beta_re, beta_im, c, c_offset, c_ld, nullptr, stream);
+}
+
+int clbh_conv_gather_possible(int precision, const clbh_im2col_shape* shape) {
+  return (shape != nullptr && clbh::ConvGatherPossible(precision, *shape)) ? 1 : 0;
 }
 
 int clbh_im2col(int precision, const clbh_im2col_shape* shape, int batch_count, const void* image, long long image_offset,

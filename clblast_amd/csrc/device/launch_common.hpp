@@ -56,7 +56,48 @@ GemmArgs<CT> MakeArgs(const clbh_gemm_desc& d) {
   p.split_workspace = nullptr;
   p.c_triangle = d.c_triangle;
   p.operand_triangle = d.operand_triangle;
+  p.conv = ConvGather{};
+  if (d.conv != nullptr) {
+    const auto& g = *d.conv;
+    const auto magic = [](const int divisor) {  // ceil(2^32 / divisor); unused for a divisor of 1
+      return static_cast<unsigned>(divisor > 1 ? 0xffffffffull / static_cast<unsigned>(divisor) + 1 : 0);
+    };
+    p.conv.enabled = 1;
+    p.conv.height = g.height;
+    p.conv.width = g.width;
+    p.conv.output_w = g.output_w;
+    p.conv.taps = g.kernel_h * g.kernel_w;
+    p.conv.kernel_w = g.kernel_w;
+    p.conv.taps_magic = magic(p.conv.taps);
+    p.conv.kernel_w_magic = magic(g.kernel_w);
+    p.conv.pad_h = g.pad_h;
+    p.conv.pad_w = g.pad_w;
+    p.conv.stride_h = g.stride_h;
+    p.conv.stride_w = g.stride_w;
+    p.conv.dilation_h = g.dilation_h;
+    p.conv.dilation_w = g.dilation_w;
+    p.conv.flip = g.flip;
+    p.conv.image_bytes = static_cast<unsigned>(4ll * g.channels * g.height * g.width);
+  }
   return p;
+}
+
+// True when the GEMM kernels can gather the A operand of a CONVGEMM from images of this shape (see ConvGather).
+inline bool ConvGatherPossible(const int precision, const clbh_im2col_shape& g) {
+  if (precision != 32) { return false; }
+  if (g.channels <= 0 || g.height <= 0 || g.width <= 0 || g.kernel_h <= 0 || g.kernel_w <= 0 || g.stride_h <= 0 ||
+      g.stride_w <= 0 || g.dilation_h <= 0 || g.dilation_w <= 0 || g.output_h <= 0 || g.output_w <= 0 || g.pad_h < 0 ||
+      g.pad_w < 0) {
+    return false;
+  }
+  const long long taps = static_cast<long long>(g.kernel_h) * g.kernel_w;
+  const long long rows = taps * g.channels;
+  const long long image_bytes = 4ll * g.channels * g.height * g.width;
+  // offsets inside one image and the corner coordinates of a patch stay in 31 bits; p / taps by multiplication is exact
+  const long long reach_h = static_cast<long long>(g.output_h) * g.stride_h + static_cast<long long>(g.kernel_h) * g.dilation_h + g.pad_h;
+  const long long reach_w = static_cast<long long>(g.output_w) * g.stride_w + static_cast<long long>(g.kernel_w) * g.dilation_w + g.pad_w;
+  return image_bytes < (1ll << 31) && taps < (1ll << 16) && (rows + 64) * taps < (1ll << 32) && reach_h < (1 << 27) &&
+         reach_w < (1 << 27) && reach_h * g.width < (1ll << 29);
 }
 
 

@@ -5,9 +5,26 @@
 
 namespace clbh {
 namespace {
+
+// CONVGEMM with the A operand gathered from the images (clbh_gemm_desc::conv): the kernel matrix is k-contiguous,
+// the batches are strided, K is not split; tiles of 64 x 64 x 16 (measured against 128 x 128 x 16 and depths of 32: the
+// gather's address arithmetic, not the tile shape, decides the speed)
+int LaunchConvF32(const clbh_gemm_desc& d, hipStream_t stream) {
+  const auto& g = *d.conv;
+  const long long patches = static_cast<long long>(g.output_h) * g.output_w;
+  const long long rows = static_cast<long long>(g.channels) * g.kernel_h * g.kernel_w;
+  if (!ConvGatherPossible(d.precision, g) || d.m != patches || d.k != rows || !d.b_kcontig || d.a_kcontig ||
+      d.batch.alphas != nullptr || d.split_k > 1 || d.c_triangle != 0 || d.operand_triangle != 0 ||
+      d.a_stride < static_cast<long long>(g.channels) * g.height * g.width) {
+    return hipErrorInvalidValue;
+  }
+  return LaunchMfmaVariant<float, MfmaConfig<float, 2, 2, 1, 1, 16, 4>, false, true, true, true>(d, stream);
+}
+
 }  // namespace
 
 int LaunchMfmaF32(const clbh_gemm_desc& d, hipStream_t stream) {
+  if (d.conv != nullptr) { return LaunchConvF32(d, stream); }
   if (!LeadingDimsFitTiles<float>(d)) { return LaunchGeneral<float>(d, stream); }
   switch (d.tile_variant) {
     case 1: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 1, 1, 32, 4>>(d, stream);  // 64 x 64 x 32

@@ -34,7 +34,7 @@ int LaunchGeneral(const clbh_gemm_desc& d, hipStream_t stream) {
 }
 
 // ---- MFMA kernels (fp32, fp64) ----------------------------------------------------------------------
-template <typename T, typename Config, bool A_KC, bool B_KC, bool ALIGNED>
+template <typename T, typename Config, bool A_KC, bool B_KC, bool ALIGNED, bool A_CONV = false>
 int LaunchMfmaVariant(const clbh_gemm_desc& d, hipStream_t stream) {
   auto args = MakeArgs<T>(d);
   const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
@@ -54,7 +54,7 @@ int LaunchMfmaVariant(const clbh_gemm_desc& d, hipStream_t stream) {
   }
   const dim3 grid(static_cast<unsigned>(TileBlocks(d, tiles_m, tiles_n)), static_cast<unsigned>(grid_y));
   constexpr size_t lds_bytes = Config::LDS_ELEMS * sizeof(T);
-  auto kernel = GemmMfmaKernel<T, Config, A_KC, B_KC, ALIGNED>;
+  auto kernel = GemmMfmaKernel<T, Config, A_KC, B_KC, ALIGNED, A_CONV>;
   if (lds_bytes > 48 * 1024) {
     static const hipError_t attribute_status = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));

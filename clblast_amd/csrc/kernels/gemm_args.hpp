@@ -13,6 +13,20 @@ namespace clbh {
 template <typename T> struct ComputeType { using type = T; };
 template <> struct ComputeType<_Float16> { using type = float; };
 
+// CONVGEMM without a materialised im2col matrix: the A operand of the GEMM (patches x patch_size, patch (oh, ow) along m,
+// (channel, tap) along k) is gathered from the image while the tiles are loaded. Row p of the patch matrix is channel
+// p / taps and kernel index p % taps (mirrored for a true convolution); the divisions by the uniform taps and kernel_w
+// are multiplications by ceil(2^32 / d) (exact for p * d < 2^32, which the host checks; d == 1 is special-cased).
+struct ConvGather {
+  int enabled;
+  int height, width, output_w;
+  int taps, kernel_w;
+  unsigned taps_magic, kernel_w_magic;
+  int pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w;
+  int flip;
+  unsigned image_bytes;  // bytes of one image (all channels): the range of the gather's buffer resource
+};
+
 template <typename CT>
 struct GemmArgs {
   const void* a;
@@ -38,6 +52,7 @@ struct GemmArgs {
   // Triangular variants (see clbh_gemm_desc): which part of C is written, which part of an operand is zero
   int c_triangle;
   int operand_triangle;
+  ConvGather conv;  // enabled != 0: `a` is a batch of images (a_stride apart) instead of a matrix, see ConvGather
 };
 
 // c_triangle: 1 keeps C(i,j) with i <= j, 2 with i >= j. 3 and 4 are the same for a complex matrix stored as a real

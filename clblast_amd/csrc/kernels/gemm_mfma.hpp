@@ -196,6 +196,62 @@ __device__ __forceinline__ void DirectLoad(const T* __restrict__ slab, const T* 
       (LdsPtr)(stage + group * L::GROUP_PITCH + part * L::WAVE_ELEMS), LANE_BYTES, lane_bytes, 0, 0, 0);
 }
 
+// Gathered A operand (ConvGather). Once per slab the lanes of a wavefront decompose the TILE_K rows of the slab in
+// parallel (lane l: row k0 + l of the patch matrix -> channel and kernel tap -> the offset of that tap in the image
+// plane and its distance dh, dw from the top-left corner of a patch); the loads then pick their row's values with
+// v_readlane, which keeps the per-load arithmetic to a handful of instructions.
+struct GatherRows {
+  int plane_offset, dh, dw;
+};
+
+template <int TILE_K>
+__device__ __forceinline__ GatherRows DecomposeRows(const ConvGather& g, const int k0, const int k_len, const int lane) {
+  const unsigned p = static_cast<unsigned>(k0 + lane % TILE_K);
+  const unsigned channel = (g.taps == 1) ? p : __umulhi(p, g.taps_magic);
+  const unsigned kernel_index = p - channel * g.taps;
+  const unsigned tap = g.flip ? (g.taps - 1 - kernel_index) : kernel_index;
+  const unsigned kh = (g.kernel_w == 1) ? tap : __umulhi(tap, g.kernel_w_magic);
+  const unsigned kw = tap - kh * g.kernel_w;
+  GatherRows rows;
+  const int dh = static_cast<int>(kh) * g.dilation_h;
+  rows.dw = static_cast<int>(kw) * g.dilation_w;
+  rows.plane_offset = (static_cast<int>(channel) * g.height + dh) * g.width + rows.dw;
+  rows.dh = (static_cast<int>(p) < k_len) ? dh : (1 << 28);  // a row beyond k fails every lane's bounds test
+  return rows;
+}
+
+// The direct load of a gathered operand: the same instruction as DirectLoad with 4 bytes per lane, but every lane
+// brings the offset of its own image element - or one beyond the resource's range, which reads as zero, for the
+// padding around the image, for patches beyond m and for rows beyond k. `patch_h`, `patch_w` (top-left corner of the
+// lane's patch in the padded image; -2^29 for patches beyond m) and `patch_offset` belong to the lane.
+template <typename T, int TILE_X, int TILE_K, typename Tag>
+__device__ __forceinline__ void GatherLoad(const T* __restrict__ image, const ConvGather& g, T* stage, const int wave,
+                                           const int round, const GatherRows& rows, const int* patch_h,
+                                           const int* patch_w, const int* patch_offset) {
+  using L = SlabLayout<T, TILE_X, TILE_K, true, 4>;
+  static_assert(L::R == 1 && sizeof(T) == 4 && TILE_K <= 64, "one row per load, dword elements, a lane per row");
+  static_assert(L::LOADS % 4 == 0, "every wavefront issues the same number of loads (the waits count them)");
+  const int index = wave + 4 * round;
+  const int row = index / L::PARTS, part = index % L::PARTS;
+  const int dh = __builtin_amdgcn_readlane(rows.dh, row), dw = __builtin_amdgcn_readlane(rows.dw, row);
+  const int plane_offset = __builtin_amdgcn_readlane(rows.plane_offset, row);
+  const int h = patch_h[part] + dh, w = patch_w[part] + dw;
+  const bool inside = static_cast<unsigned>(h) < static_cast<unsigned>(g.height) &&
+                      static_cast<unsigned>(w) < static_cast<unsigned>(g.width);
+  const int offset_bytes = inside ? (plane_offset + patch_offset[part]) * 4 : static_cast<int>(0x80000000u);
+  // The resource is uniform, but under register pressure the compiler keeps it in vector registers and then loops over
+  // its distinct values around every load: take it from the first lane explicitly.
+  const unsigned long long address = reinterpret_cast<unsigned long long>(image);
+  const unsigned long long low = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(address)));
+  const unsigned long long high = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(address >> 32)));
+  T* uniform_image = reinterpret_cast<T*>((high << 32) | low);
+  const int bytes = __builtin_amdgcn_readfirstlane(static_cast<int>(g.image_bytes));
+  typedef __attribute__((address_space(3))) void* LdsPtr;
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(__builtin_amdgcn_make_buffer_rsrc(uniform_image, 0, bytes, kRawBufferFlags),
+                                           (LdsPtr)(stage + row * L::GROUP_PITCH + part * L::WAVE_ELEMS), 4, offset_bytes, 0,
+                                           0, 0);
+}
+
 // Staged operand: thread t moves the pieces t, t + 256, ... of the slab (VL elements each, consecutive
 // threads along k); with LINES whole x lines per round, piece c lies c * LINES lines after piece 0.
 template <int TILE_X, int TILE_K, int VL>
@@ -284,7 +340,8 @@ __device__ __forceinline__ bool TileOfBlockCyclic(const int block, const int til
 }
 
 // ---- the kernel ------------------------------------------------------------------------------------
-template <typename T, typename Config, bool A_KC, bool B_KC, bool ALIGNED>
+// A_CONV: the A operand is gathered from a batch of images (GemmArgs::conv); needs !A_KC and fp32.
+template <typename T, typename Config, bool A_KC, bool B_KC, bool ALIGNED, bool A_CONV = false>
 __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void GemmMfmaKernel(const GemmArgs<T> p, const int tiles_m,
                                                                const int tiles_n) {
   using Traits = typename Config::Traits;
@@ -297,7 +354,9 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
   constexpr int VL = ALIGNED ? VEC : 1;         // elements per staged global access
   constexpr int LANE_BYTES = ALIGNED ? 16 : 4;  // bytes per lane of a direct load
   constexpr bool A_DIRECT = !A_KC, B_DIRECT = !B_KC;
-  using LA = SlabLayout<T, TILE_M, TILE_K, A_DIRECT, LANE_BYTES>;
+  static_assert(!A_CONV || !A_KC, "a gathered operand takes the direct path");
+  constexpr int LANE_BYTES_A = A_CONV ? 4 : LANE_BYTES;  // the gather moves single elements
+  using LA = SlabLayout<T, TILE_M, TILE_K, A_DIRECT, LANE_BYTES_A>;
   using LB = SlabLayout<T, TILE_N, TILE_K, B_DIRECT, LANE_BYTES>;
   using PA = StagedPieces<TILE_M, TILE_K, VL>;
   using PB = StagedPieces<TILE_N, TILE_K, VL>;
@@ -313,7 +372,7 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
   using VM = typename VecType<T, FM>::type;
   using VN = typename VecType<T, FN>::type;
   using VP = typename VecType<T, VL>::type;
-  using KernelTag = std::tuple<Config, std::integral_constant<int, (A_KC ? 4 : 0) | (B_KC ? 2 : 0) | (ALIGNED ? 1 : 0)>>;
+  using KernelTag = std::tuple<Config, std::integral_constant<int, (A_CONV ? 8 : 0) | (A_KC ? 4 : 0) | (B_KC ? 2 : 0) | (ALIGNED ? 1 : 0)>>;
 
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
@@ -345,6 +404,22 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
   const int b_read = wave_n * (FN * MF) + lane_x * FN;
   static_assert((KP % LA::R == 0 || LA::R % KP == 0) && (KP % LB::R == 0 || LB::R % KP == 0), "row offsets add up");
   const int a_lane_row = LA::Row(lane_g) + a_read, b_lane_row = LB::Row(lane_g) + b_read;
+
+  // Gathered A: the patches this lane loads (one per part of a tile row), as the top-left corner of the patch in the
+  // padded image and the offset of that corner in the image plane; patches beyond m never pass the bounds test
+  constexpr int GATHER_PARTS = A_CONV ? LA::PARTS : 1;
+  int patch_h[GATHER_PARTS], patch_w[GATHER_PARTS], patch_offset[GATHER_PARTS];
+  if constexpr (A_CONV) {
+#pragma unroll
+    for (int part = 0; part < GATHER_PARTS; ++part) {
+      const int patch = m0 + part * LA::WAVE_ELEMS + lane;
+      const int oh = patch / p.conv.output_w, ow = patch - oh * p.conv.output_w;
+      const int corner_h = oh * p.conv.stride_h - p.conv.pad_h;
+      patch_w[part] = ow * p.conv.stride_w - p.conv.pad_w;
+      patch_offset[part] = corner_h * p.conv.width + patch_w[part];
+      patch_h[part] = (patch < p.m) ? corner_h : -(1 << 29);
+    }
+  }
 
   for (int batch = blockIdx.y; batch < p.batch_count; batch += gridDim.y) {
     const T* a;
@@ -391,7 +466,7 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
     // behind the last element of the operand: (x = extent - 1, k = k_len - 1) + 1
     const T* a_end = a + (A_KC ? (p.m - 1) * p.a_ld + k_len : (k_len - 1) * p.a_ld + p.m);
     const T* b_end = b + (B_KC ? (p.n - 1) * p.b_ld + k_len : (k_len - 1) * p.b_ld + p.n);
-    const int a_lane_bytes = A_DIRECT ? DirectLaneBytes<T, TILE_M, TILE_K, LANE_BYTES>(p.a_ld, lane)
+    const int a_lane_bytes = A_DIRECT ? DirectLaneBytes<T, TILE_M, TILE_K, LANE_BYTES_A>(p.a_ld, lane)
                                       : static_cast<int>((PA::Line(tid) * p.a_ld + PA::K(tid)) * static_cast<long long>(sizeof(T)));
     const int b_lane_bytes = B_DIRECT ? DirectLaneBytes<T, TILE_N, TILE_K, LANE_BYTES>(p.b_ld, lane)
                                       : static_cast<int>((PB::Line(tid) * p.b_ld + PB::K(tid)) * static_cast<long long>(sizeof(T)));
@@ -419,9 +494,16 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
       constexpr int DIRECT_A = A_DIRECT ? LA::LOADS_PER_WAVE : 0, DIRECT_B = B_DIRECT ? LB::LOADS_PER_WAVE : 0;
       constexpr int DIRECT = DIRECT_A + DIRECT_B;
       constexpr int DIRECT_PER_SLOT = (DIRECT + SLOTS - 1) / SLOTS;
+      GatherRows gather_rows{};  // of the slab whose loads are being issued (gathered A only)
       auto direct_load = [&](const int load, const int k0, auto* a_dst, auto* b_dst) {
         if constexpr (DIRECT_A > 0) {
-          if (load < DIRECT_A) { DirectLoad<T, TILE_M, TILE_K, LANE_BYTES, RANGE, KernelTag>(a_slab(k0), a_end, p.a_ld, a_dst, wave_u, a_lane_bytes, load); }
+          if (load < DIRECT_A) {
+            if constexpr (A_CONV) {
+              GatherLoad<T, TILE_M, TILE_K, KernelTag>(a, p.conv, a_dst, wave_u, load, gather_rows, patch_h, patch_w, patch_offset);
+            } else {
+              DirectLoad<T, TILE_M, TILE_K, LANE_BYTES, RANGE, KernelTag>(a_slab(k0), a_end, p.a_ld, a_dst, wave_u, a_lane_bytes, load);
+            }
+          }
         }
         if constexpr (DIRECT_B > 0) {
           if (load >= DIRECT_A) { DirectLoad<T, TILE_N, TILE_K, LANE_BYTES, RANGE, KernelTag>(b_slab(k0), b_end, p.b_ld, b_dst, wave_u, b_lane_bytes, load - DIRECT_A); }
@@ -444,6 +526,7 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
 
       // Prologue: slab 0 lands in buffer 0 (the staged registers' wait also covers the older direct loads),
       // slab 1 is requested.
+      if constexpr (A_CONV) { gather_rows = DecomposeRows<TILE_K>(p.conv, 0, k_len, lane); }
 #pragma unroll
       for (int load = 0; load < DIRECT; ++load) { direct_load(load, 0, a_stages, b_stages); }
 #pragma unroll
@@ -452,6 +535,7 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
       for (int piece = 0; piece < STAGED; ++piece) { store_piece(piece, a_stages, b_stages, 0, std::true_type{}); }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       if (slabs > 1) {
+        if constexpr (A_CONV) { gather_rows = DecomposeRows<TILE_K>(p.conv, TILE_K, k_len, lane); }
 #pragma unroll
         for (int load = 0; load < DIRECT; ++load) { direct_load(load, TILE_K, a_stages + LA::ELEMS, b_stages + LB::ELEMS); }
 #pragma unroll
@@ -477,6 +561,7 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
         T* a_prv = a_stages + prv * LA::ELEMS;
         T* b_prv = b_stages + prv * LB::ELEMS;
         const int k_store = (slab + 1) * TILE_K, k_load = (slab + 2) * TILE_K;
+        if constexpr (A_CONV && LOAD) { gather_rows = DecomposeRows<TILE_K>(p.conv, k_load, k_len, lane); }
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
           const int set = ks % 2;

@@ -59,8 +59,6 @@ void Xconvgemm<T>::DoConvgemm(const KernelMode kernel_mode, const size_t channel
   TestMatrixA(width, height * channels * batch_count, im_buffer, im_offset, width);
 
   const auto precision = static_cast<int>(PrecisionValue<T>());
-  const auto col_bytes = col_stride * batch_count * sizeof(T);
-  const StreamScratch col(col_bytes, this->stream(), "im2col matrices");
   auto shape = clbh_im2col_shape{};
   shape.channels = static_cast<int>(channels);
   shape.height = static_cast<int>(height);
@@ -76,6 +74,44 @@ void Xconvgemm<T>::DoConvgemm(const KernelMode kernel_mode, const size_t channel
   shape.output_h = static_cast<int>(output_h);
   shape.output_w = static_cast<int>(output_w);
   shape.flip = (kernel_mode == KernelMode::kConvolution) ? 1 : 0;
+
+  // The reference's single-kernel method (xconvgemm.cpp:121-160, doc/details_conv.md): no im2col matrix; the GEMM kernel
+  // gathers the patches from the images while it loads its tiles. fp32, all batches in one launch.
+  if (clbh_conv_gather_possible(precision, &shape) != 0) {
+    auto desc = clbh_gemm_desc{};
+    desc.precision = precision;
+    desc.kernel_class = CLBH_KERNEL_MFMA;
+    desc.tile_variant = 7;  // 64 x 64 x 16, the one tile the gathering kernel is built for
+    desc.split_k = 1;
+    desc.a_kcontig = 0;
+    desc.b_kcontig = 1;
+    desc.m = static_cast<int>(num_patches);
+    desc.n = static_cast<int>(num_kernels);
+    desc.k = static_cast<int>(patch_size);
+    desc.batch_count = static_cast<int>(batch_count);
+    desc.a = im_buffer();
+    desc.a_offset = static_cast<long long>(im_offset);
+    desc.a_ld = static_cast<long long>(num_patches);  // of the patch matrix that is never stored
+    desc.a_stride = static_cast<long long>(channels * height * width);
+    desc.b = kernel_buffer();
+    desc.b_offset = static_cast<long long>(kernel_offset);
+    desc.b_ld = static_cast<long long>(patch_size);
+    desc.b_stride = 0;  // the kernel matrix is shared by the batches
+    desc.c = const_cast<void*>(result_buffer());
+    desc.c_offset = static_cast<long long>(result_offset);
+    desc.c_ld = static_cast<long long>(num_patches);
+    desc.c_stride = static_cast<long long>(result_stride);
+    desc.alpha = 1.0;
+    desc.beta = 0.0;
+    desc.conv = &shape;
+    CheckDevice(clbh_gemm_launch(&desc, this->stream()), "clbh_gemm_launch (gathered convolution)");
+    this->Finish();
+    return;
+  }
+
+  // Otherwise "im2col + GEMM" (xconvgemm.cpp:78-119): one launch unfolds all images
+  const auto col_bytes = col_stride * batch_count * sizeof(T);
+  const StreamScratch col(col_bytes, this->stream(), "im2col matrices");
   CheckDevice(clbh_im2col(precision, &shape, static_cast<int>(batch_count), im_buffer(), static_cast<long long>(im_offset),
                           col.get(), this->stream()),
               "clbh_im2col");

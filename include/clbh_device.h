@@ -47,6 +47,8 @@ typedef struct clbh_batch_arrays_ {
   int offset_multiple;          // every entry of the three offset arrays is a multiple of this (0 or 1: unknown)
 } clbh_batch_arrays;
 
+struct clbh_im2col_shape_;  // defined below (clbh_im2col)
+
 typedef struct clbh_gemm_desc_ {
   int precision;      // 16, 32 or 64 (bits of the storage type)
   int kernel_class;   // enum clbh_kernel_class
@@ -71,6 +73,11 @@ typedef struct clbh_gemm_desc_ {
                          // 3, 4: the same for a complex C stored as a real matrix with interleaved rows: i/2 <= j, i/2 >= j
   int operand_triangle;  // the caller states that part of an operand is zero, so that the kernels may skip it:
                          // 1: A(i,p) = 0 for p > i, 2: A(i,p) = 0 for p < i, 3: B(p,j) = 0 for p > j, 4: B(p,j) = 0 for p < j
+  // CONVGEMM without an im2col matrix (NULL for every other launch; see clbh_conv_gather_possible): `a` + a_offset holds
+  // batch_count images, a_stride elements apart, and A(i,p) is element i of row p of the im2col matrix that clbh_im2col
+  // would write for this shape, gathered from the image while the tiles are loaded. Needs m = output_h * output_w,
+  // k = channels * kernel_h * kernel_w, precision 32, the MFMA class (one tile: 64 x 64 x 16), b_kcontig, strided batches.
+  const struct clbh_im2col_shape_* conv;
 } clbh_gemm_desc;
 
 // Enqueues the kernel(s) for one descriptor on `stream`. Returns 0 on success, otherwise the HIP
@@ -159,6 +166,9 @@ typedef struct clbh_im2col_shape_ {
 } clbh_im2col_shape;
 CLBH_API int clbh_im2col(int precision, const clbh_im2col_shape* shape, int batch_count, const void* image,
                          long long image_offset, void* col, hipStream_t stream);
+// Non-zero when a GEMM launch can gather its A operand from images of this shape itself (clbh_gemm_desc::conv): fp32
+// only, one image below 2 GiB, and row indices small enough for the kernel's division by multiplication.
+CLBH_API int clbh_conv_gather_possible(int precision, const clbh_im2col_shape* shape);
 
 // Plain device memory and blocking copies for callers that hold host data (the Netlib-style façade): to_device != 0
 // copies host -> device, else waits for the default stream's work and copies device -> host.

@@ -23,7 +23,7 @@ CASES = [  # channels, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h
     (16, 32, 32, 3, 3, 1, 1, 1, 1, 1, 1, 32, 4),
     (8, 30, 17, 3, 3, 0, 1, 2, 2, 1, 1, 20, 20),   # small patches x kernels, 20 batches
     (3, 64, 64, 7, 7, 3, 3, 2, 2, 1, 1, 64, 2),
-    (4, 4, 4, 3, 3, 0, 0, 1, 1, 1, 1, 2, 40),      # 2 x 2 outputs: the one-wavefront-per-matrix kernel in fp32
+    (4, 4, 4, 3, 3, 0, 0, 1, 1, 1, 1, 2, 40),      # 2 x 2 outputs, many batches
 ]
 
 
