@@ -258,7 +258,8 @@ size_t clbh_gemm_workspace_bytes(const clbh_gemm_desc* desc) {
   if (desc == nullptr || desc->kernel_class != CLBH_KERNEL_MFMA) { return 0; }
   const auto plan = clbh::PlanSplit(*desc);
   if (plan.splits <= 1) { return 0; }
-  return static_cast<size_t>(desc->precision / 8) * plan.splits * plan.ld * static_cast<size_t>(desc->n);
+  const auto element_bytes = static_cast<size_t>(desc->precision == 16 ? 4 : desc->precision / 8);  // fp16 sums in fp32
+  return element_bytes * plan.splits * plan.ld * static_cast<size_t>(desc->n);
 }
 
 int clbh_symmetric_to_square(int precision, int upper, int k, const void* src, long long src_offset, long long src_ld,

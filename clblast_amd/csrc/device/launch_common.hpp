@@ -143,8 +143,9 @@ struct SplitPlan {
 };
 inline SplitPlan PlanSplit(const clbh_gemm_desc& d) {
   SplitPlan plan{1, 0, 0};
-  if (d.split_k > 1 && d.batch_count == 1 && d.batch.alphas == nullptr && d.precision != 16 && d.c_triangle == 0 &&
-      d.operand_triangle == 0) {
+  // (the reduction's second grid dimension walks n; fp16 partial sums are kept in fp32)
+  if (d.split_k > 1 && d.batch_count == 1 && d.batch.alphas == nullptr && d.c_triangle == 0 && d.operand_triangle == 0 &&
+      d.n <= 65535 && d.conv == nullptr) {
     const int chunk = ((d.k + d.split_k - 1) / d.split_k + 63) / 64 * 64;
     const int splits = (d.k + chunk - 1) / chunk;
     if (splits > 1) { plan = SplitPlan{splits, chunk, (d.m + 3) / 4 * 4}; }

@@ -63,11 +63,23 @@ int LaunchHgemmConfig(const clbh_gemm_desc& d, hipStream_t stream) {
 // ---- direct-load MFMA kernel, fp16 (dword-aligned operands) ---------------------------------------
 template <typename Config, bool A_KC, bool B_KC>
 int LaunchHdirectVariant(const clbh_gemm_desc& d, hipStream_t stream) {
-  const auto args = MakeArgs<float>(d);
+  auto args = MakeArgs<float>(d);
   const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
   const long long tiles_n = (d.n + Config::TILE_N - 1) / Config::TILE_N;
   if (TileBlocks(d, tiles_m, tiles_n) > INT_MAX) { return hipErrorInvalidConfiguration; }
-  const dim3 grid(static_cast<unsigned>(TileBlocks(d, tiles_m, tiles_n)), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
+  const auto plan = PlanSplit(d);
+  int grid_y = std::min(d.batch_count, kMaxGridY);
+  if (plan.splits > 1) {  // K ranges as batch entries into the fp32 workspace, then the reduction
+    if (d.workspace == nullptr || d.workspace_bytes < sizeof(float) * plan.splits * plan.ld * static_cast<size_t>(d.n)) {
+      return hipErrorInvalidValue;
+    }
+    args.split_chunk = plan.chunk;
+    args.split_ld = plan.ld;
+    args.split_workspace = d.workspace;
+    args.batch_count = plan.splits;
+    grid_y = plan.splits;
+  }
+  const dim3 grid(static_cast<unsigned>(TileBlocks(d, tiles_m, tiles_n)), static_cast<unsigned>(grid_y));
   constexpr size_t lds_bytes = Config::LDS_BYTES;
   auto kernel = HgemmDirectKernel<Config, A_KC, B_KC>;
   if (lds_bytes > 48 * 1024) {
@@ -76,6 +88,12 @@ int LaunchHdirectVariant(const clbh_gemm_desc& d, hipStream_t stream) {
     if (attribute_status != hipSuccess) { return static_cast<int>(attribute_status); }
   }
   kernel<<<grid, dim3(Config::THREADS), lds_bytes, stream>>>(args, static_cast<int>(tiles_m), static_cast<int>(tiles_n));
+  if (plan.splits > 1) {
+    const dim3 reduce_grid(static_cast<unsigned>((d.m + 255) / 256), static_cast<unsigned>(d.n));
+    HgemmSplitReduceKernel<<<reduce_grid, dim3(256), 0, stream>>>(
+        static_cast<const float*>(d.workspace), plan.splits, plan.ld, static_cast<_Float16*>(d.c) + d.c_offset, d.c_ld, d.m, d.n,
+        static_cast<float>(d.alpha), static_cast<float>(d.beta));
+  }
   return static_cast<int>(hipGetLastError());
 }
 

@@ -188,7 +188,12 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
     float alpha, beta;
     ResolveBatch<T, float>(p, batch, a, b, c, alpha, beta);
     int k_len = p.k;
-    if (p.operand_triangle != 0) {  // skip the K range in which a triangular operand is zero
+    if (p.split_chunk > 0) {  // this "batch" is one K range of a single problem (ranges are multiples of 64 deep)
+      const int k_begin = batch * p.split_chunk;
+      k_len = min(p.split_chunk, p.k - k_begin);
+      a = static_cast<const T*>(p.a) + p.a_offset + (A_KC ? static_cast<long long>(k_begin) : k_begin * p.a_ld);
+      b = static_cast<const T*>(p.b) + p.b_offset + (B_KC ? static_cast<long long>(k_begin) : k_begin * p.b_ld);
+    } else if (p.operand_triangle != 0) {  // skip the K range in which a triangular operand is zero
       int k_first;
       TriangularRange(p.operand_triangle, m0, n0, TILE_M, TILE_N, p.k, k_first, k_len);
       a += A_KC ? static_cast<long long>(k_first) : k_first * p.a_ld;
@@ -350,7 +355,30 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
     // with 16-byte accesses along m, every lane combines its four consecutive m in fp32 and rounds once, and
     // the finished rows leave with 16-byte stores. Only wavefront-local ordering is needed (LDS operations of
     // a wavefront complete in order).
-    {
+    if (p.split_chunk > 0) {
+      // Split-K: the fp32 partial sums go to slab `batch` of the workspace (column-major, leading dimension split_ld,
+      // a multiple of 4 >= m), four consecutive m per store; a second kernel adds the slabs and applies alpha and beta.
+      float* partial = static_cast<float*>(p.split_workspace) + static_cast<long long>(batch) * p.split_ld * p.n;
+      typedef float float4u_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+        const int n_index = n0 + (wave_n * FN + j) * 32 + lane % 32;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int m_index = m0 + (wave_m * FM + i) * 32 + 8 * g + 4 * (lane / 32);
+            if (n_index < p.n && m_index < p.split_ld) {
+              float4u_t out;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) { out[e] = acc[i][j][4 * g + e]; }
+              *reinterpret_cast<float4u_t*>(partial + static_cast<long long>(n_index) * p.split_ld + m_index) = out;
+            }
+          }
+        }
+      }
+      __syncthreads();  // the next K range refills the slab buffers
+    } else {
       constexpr int WAVE_M = FM * 32, STAGE_PITCH = WAVE_M + 8;
       constexpr int LANES_PER_ROW = WAVE_M / 8, ROWS_PER_PASS = 64 / LANES_PER_ROW, PASSES = 32 / ROWS_PER_PASS;
       typedef _Float16 half8u_t __attribute__((ext_vector_type(8), aligned(4)));  // C needs dword alignment only
@@ -426,6 +454,22 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
       __syncthreads();  // the next batch entry refills the slab buffers
     }
   }
+}
+
+// Second pass of a split-K launch: C = alpha * (sum of the fp32 workspace slabs) + beta * C, rounded to fp16 once.
+// grid: (ceil(m / 256), n).
+__global__ __launch_bounds__(256) void HgemmSplitReduceKernel(const float* __restrict__ workspace, const int splits,
+                                                              const int split_ld, _Float16* __restrict__ c,
+                                                              const long long c_ld, const int m, const int n,
+                                                              const float alpha, const float beta) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int j = blockIdx.y;
+  if (i >= m || j >= n) { return; }
+  const long long slab = static_cast<long long>(split_ld) * n;
+  const float* src = workspace + static_cast<long long>(j) * split_ld + i;
+  float sum = 0.0f;
+  for (int s = 0; s < splits; ++s) { sum += src[s * slab]; }
+  StoreResult<_Float16, float>(c, j * c_ld + i, sum, alpha, beta);
 }
 
 }  // namespace clbh

@@ -100,9 +100,8 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   }
   const auto forced = ForcedTileVariant(precision);
   if (forced != 0) {
-    // a forced tile takes the forced number of K ranges (fp32/fp64, unbatched calls only), never more than k / 16
-    const auto ranges = (precision != Precision::kHalf && batch_count == 1)
-                            ? std::max<size_t>(1, std::min<size_t>(ForcedSplit(precision), k / 16)) : 1;
+    // a forced tile takes the forced number of K ranges (unbatched calls only), never more than k / 16
+    const auto ranges = (batch_count == 1) ? std::max<size_t>(1, std::min<size_t>(ForcedSplit(precision), k / 16)) : 1;
     return KernelChoice{CLBH_KERNEL_MFMA, static_cast<int>(forced) - 1, static_cast<int>(ranges)};
   }
   if (triangular) {
@@ -124,13 +123,23 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   if (precision == Precision::kHalf) {
     // Direct-load tiles, 0: 128 x 128, 1: 64 x 64, 2: 256 x 256 (8 wavefronts), 3: 128 x 32, 4: 32 x 128. Measured
     // (tile sweep over 15 shapes): 256 x 256 when its tiles fill whole rounds of the 256 CUs, 128 x 128 from 256
-    // tiles on, else 64 x 64 - also for skinny shapes (there is no split-K for fp16, occupancy does the hiding).
+    // tiles on, else 64 x 64 - also for skinny shapes.
     const auto big = CeilDivide(m, 256) * CeilDivide(n, 256) * batch_count;
     const auto rounds = CeilDivide(big, 256);
     int tile = 1;
     if (5 * big >= 4 * rounds * 256 && k >= 512) { tile = 2; }
     else if (CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count >= 256) { tile = 0; }
-    return KernelChoice{CLBH_KERNEL_MFMA, tile, 1};
+    // K ranges (fp32 partial sums, then a reduction) when the 64 x 64 tiles would leave the GPU mostly idle through a
+    // long K walk: up to 512 work-groups, ranges at least 512 deep - 2048 when there are 192 tiles or more, which by
+    // themselves keep most CUs busy (measured: 256^2 x 8192 33.6 -> 13.4 us, 4099 x 17 x 4096 33.9 -> 14.1 us,
+    // 1024^2 x 8192 54.4 -> 42.3 us; 1024^2 x 2048 is faster unsplit)
+    auto split = size_t{1};
+    const auto tiles = CeilDivide(m, 64) * CeilDivide(n, 64);
+    if (tile == 1 && batch_count == 1 && tiles < 512 && k >= 2048) {
+      const auto min_range = (tiles >= 192) ? size_t{2048} : size_t{512};
+      split = std::max<size_t>(1, std::min<size_t>({CeilDivide(512, tiles), k / min_range, 16}));
+    }
+    return KernelChoice{CLBH_KERNEL_MFMA, tile, static_cast<int>(split)};
   }
   if (precision == Precision::kSingle) {
     // Measured on the MI355X (tile x split sweep over 18 shapes): 64 x 64 tiles (several work-groups per CU hide

@@ -148,6 +148,15 @@ def test_every_tile_variant(gpu, bits):
                     status, c_after = problem.run()
                     assert status == 0, (variant, problem.describe())
                     problem.check(c_after)
+            # the same tile with K split into three ranges (192, 192 and 116 deep: the last one has a K tail)
+            clblast_amd.override_parameters(0, "Xgemm", bits, {"TILE_VARIANT": variant, "SPLIT_K": 3})
+            for (ta, tb) in itertools.product(TRANSPOSES, TRANSPOSES):
+                seed += 1
+                problem = gpu.Problem(bits, COL_MAJOR, ta, tb, 300, 270, 500, 0.5, 2.0 if seed % 2 else 0.0, a_offset=8, b_offset=16,
+                                      c_offset=3, seed=seed, extra_ld=(8, 8, 5))
+                status, c_after = problem.run()
+                assert status == 0, (variant, "split", problem.describe())
+                problem.check(c_after)
     finally:
         import clblast_amd
         clblast_amd.override_parameters(0, "Xgemm", bits, {"TILE_VARIANT": 0})
