@@ -68,6 +68,14 @@ struct Tile {
   size_t tile_m, tile_n;
 };
 
+// True when `tiles` large tiles (one work-group per CU at a time) keep the 256 CUs busy: two rounds or more, or at
+// least 90 % of the last round (4096 x 2048 x 4096, 256 tiles: 564 -> 505 us against 64 x 64 tiles; 2560^3, 200 tiles,
+// and 3584^3, 392 tiles, are faster with 64 x 64)
+bool FillsRounds(const size_t tiles) {
+  const auto rounds = CeilDivide(tiles, 256);
+  return tiles >= 512 || 10 * tiles >= 9 * rounds * 256;
+}
+
 // Number of K ranges for a launch of `tiles` work-groups. Splitting costs a second launch (the reduction, about
 // 5 us) and pays only when most CUs would idle through a long K walk (about 16 ns per unit of k and work-group):
 // ranges stay >= 512 deep and bring the launch to about two work-groups per CU. The half- and quarter-sized tiles
@@ -151,7 +159,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     const auto tiles64 = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;
     if (n <= 32 && m >= 256) { tile = Tile{9, 64, 32}; }         // skinny: stream A
     else if (m <= 32 && n >= 256) { tile = Tile{8, 32, 64}; }    // skinny: stream B
-    else if (CeilDivide(m, 256) * CeilDivide(n, 128) >= 512 && k >= 1024) { tile = Tile{3, 256, 128}; }
+    else if (k >= 1024 && FillsRounds(CeilDivide(m, 256) * CeilDivide(n, 128) * batch_count)) { tile = Tile{3, 256, 128}; }
     else if (tiles64 <= 64 && k < 2048) { tile = Tile{10, 32, 32}; }
     else if (tiles64 < 1024) { tile = Tile{9, 64, 32}; }
     const auto tiles = CeilDivide(m, tile.tile_m) * CeilDivide(n, tile.tile_n) * batch_count;
