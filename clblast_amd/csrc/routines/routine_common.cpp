@@ -3,6 +3,7 @@
 // =================================================================================================
 #include "routines/routine_common.hpp"
 
+#include <algorithm>
 #include <cstdio>
 #include <map>
 #include <memory>
@@ -49,16 +50,25 @@ BLASError SwappedOperands(const BLASError& error) {
 }
 
 namespace {
+// The buffer kept for one (device, stream). A call may hold several pieces of it at once (a routine with several
+// temporaries, a GEMM called from inside such a routine): pieces are cut off its front in the order they are asked for
+// and given back in the opposite order, as the scopes of the StreamScratch objects of one call nest. The mutex is held
+// by the calling thread from its first piece to the return of its last one.
 struct CachedScratch {
   void* pointer = nullptr;
   size_t bytes = 0;
-  std::mutex taken;  // held by the StreamScratch that uses the buffer
+  size_t used = 0;   // offset of the first free byte
+  size_t live = 0;   // pieces handed out and not yet returned
+  size_t demand = 0; // what a call would have needed while the buffer could not grow
+  std::recursive_mutex taken;
 };
+constexpr size_t kScratchAlignment = 256;
 std::mutex scratch_cache_mutex;
 std::map<std::pair<int, hipStream_t>, std::unique_ptr<CachedScratch>> scratch_cache;
 
-// The entry of this stream with at least `bytes` bytes, locked, or nullptr (then the caller allocates on the stream)
-CachedScratch* TakeCachedScratch(const size_t bytes, hipStream_t stream) {
+// A piece of `bytes` bytes of this stream's buffer (its entry then stays locked by this thread until the piece is
+// returned), or nullptr: then the caller allocates on the stream.
+CachedScratch* TakeCachedScratch(const size_t bytes, hipStream_t stream, size_t& offset) {
   auto device = 0;
   if (bytes == 0 || bytes > kCachedScratchBytes || clbh_stream_device(stream, &device) != 0) { return nullptr; }
   CachedScratch* entry = nullptr;
@@ -71,13 +81,22 @@ CachedScratch* TakeCachedScratch(const size_t bytes, hipStream_t stream) {
       found = scratch_cache.emplace(key, std::unique_ptr<CachedScratch>(new CachedScratch())).first;
     }
     entry = found->second.get();
-    if (!entry->taken.try_lock()) { return nullptr; }
+    if (!entry->taken.try_lock()) { return nullptr; }  // another host thread is inside a call on this stream
   }
-  if (entry->bytes < bytes) {
-    // grows in powers of two from 1 MiB, so that this happens a few times per stream at most; freeing the old buffer
-    // waits for the device, which covers kernels of earlier calls that still use it
+  offset = (entry->used + kScratchAlignment - 1) / kScratchAlignment * kScratchAlignment;
+  if (offset + bytes > entry->bytes || (entry->live == 0 && entry->demand > entry->bytes)) {
+    // Too small: grow - in powers of two from 1 MiB, so that this happens a few times per stream at most - unless
+    // pieces of the buffer are in use: then the size that would have done is remembered, and the next call's first
+    // request grows the buffer to it. Freeing the old buffer waits for the device, which covers kernels of earlier
+    // calls that still use it.
     auto wanted = size_t{1} << 20;
-    while (wanted < bytes) { wanted *= 2; }
+    while (wanted < std::max(offset + bytes, entry->demand)) { wanted *= 2; }
+    if (wanted > kCachedScratchBytes) { wanted = kCachedScratchBytes; }
+    if (entry->live > 0 || offset + bytes > wanted) {
+      entry->demand = std::max(entry->demand, std::min(offset + bytes, kCachedScratchBytes));
+      entry->taken.unlock();
+      return nullptr;
+    }
     if (entry->pointer != nullptr) { clbh_free(entry->pointer); }
     entry->pointer = nullptr;
     entry->bytes = 0;
@@ -88,15 +107,24 @@ CachedScratch* TakeCachedScratch(const size_t bytes, hipStream_t stream) {
     }
     entry->bytes = wanted;
   }
+  entry->used = offset + bytes;
+  entry->live += 1;
   return entry;
+}
+
+void ReturnCachedScratch(CachedScratch* entry, const size_t offset, const size_t bytes) {
+  entry->live -= 1;
+  if (entry->live == 0) { entry->used = 0; }
+  else if (entry->used == offset + bytes) { entry->used = offset; }  // the last piece taken: its space is free again
+  entry->taken.unlock();
 }
 }  // namespace
 
 StreamScratch::StreamScratch(const size_t bytes, hipStream_t stream, const char* what)
-    : pointer_(nullptr), bytes_(bytes), stream_(stream), cached_(nullptr) {
-  if (auto* entry = TakeCachedScratch(bytes, stream)) {
+    : pointer_(nullptr), bytes_(bytes), stream_(stream), cached_(nullptr), cached_offset_(0) {
+  if (auto* entry = TakeCachedScratch(bytes, stream, cached_offset_)) {
     cached_ = entry;
-    pointer_ = entry->pointer;
+    pointer_ = static_cast<unsigned char*>(entry->pointer) + cached_offset_;
     return;
   }
   if (clbh_alloc_async(&pointer_, bytes, stream) != 0) {
@@ -106,20 +134,20 @@ StreamScratch::StreamScratch(const size_t bytes, hipStream_t stream, const char*
 }
 
 StreamScratch::~StreamScratch() {
-  if (cached_ != nullptr) { static_cast<CachedScratch*>(cached_)->taken.unlock(); }
+  if (cached_ != nullptr) { ReturnCachedScratch(static_cast<CachedScratch*>(cached_), cached_offset_, bytes_); }
   else if (pointer_ != nullptr) { clbh_free_async(pointer_, stream_); }
 }
 
 void ReleaseCachedScratch() {
   std::lock_guard<std::mutex> lock(scratch_cache_mutex);
   for (auto entry = scratch_cache.begin(); entry != scratch_cache.end();) {
-    if (entry->second->taken.try_lock()) {  // not in the hands of a running call
-      if (entry->second->pointer != nullptr) { clbh_free(entry->second->pointer); }
+    if (entry->second->taken.try_lock()) {
+      const bool idle = (entry->second->live == 0);  // not in the hands of a running call (of this thread either)
+      if (idle && entry->second->pointer != nullptr) { clbh_free(entry->second->pointer); }
       entry->second->taken.unlock();
-      entry = scratch_cache.erase(entry);
-    } else {
-      ++entry;
+      if (idle) { entry = scratch_cache.erase(entry); continue; }
     }
+    ++entry;
   }
 }
 

@@ -137,13 +137,15 @@ class Buffer {
 // src/routines/level3/xsymm.cpp:92-109, xtrmm.cpp:110-127).
 BLASError SwappedOperands(const BLASError& error);
 
-// Scratch memory of one call, valid for kernels enqueued on `stream` while the object lives. Requests up to
-// kCachedScratchBytes are served from a buffer the library keeps per (device, stream) - stream order makes its reuse
-// by the next call on that stream safe, and nothing is allocated or freed on the way (a stream-ordered free costs
-// about 8 us of host time, more than many a small GEMM). Larger requests, requests while that buffer is taken (a
-// routine holding several buffers, another host thread on the same stream) and streams beyond kCachedScratchStreams
-// get stream-ordered memory that is freed on the stream when the object goes out of scope, also when an error unwinds
-// the call. ReleaseCachedScratch (ClearCache calls it) frees the kept buffers; the caller must have synchronised.
+// Scratch memory of one call, valid for kernels enqueued on `stream` while the object lives. Requests are served from a
+// buffer of up to kCachedScratchBytes that the library keeps per (device, stream) - stream order makes its reuse by the
+// next call on that stream safe, and nothing is allocated or freed on the way (a stream-ordered free costs about 8 us of
+// host time, more than many a small GEMM). The objects of one call share the buffer as a stack: they are expected to be
+// destroyed in the opposite order of their construction (anything else only delays the reuse of their space). Requests
+// that do not fit, requests while another host thread is inside a call on the same stream, and streams beyond
+// kCachedScratchStreams get stream-ordered memory that is freed on the stream when the object goes out of scope, also
+// when an error unwinds the call. ReleaseCachedScratch (ClearCache calls it) frees the kept buffers; the caller must
+// have synchronised.
 constexpr size_t kCachedScratchBytes = size_t{16} << 20;
 constexpr size_t kCachedScratchStreams = 16;
 class StreamScratch {
@@ -159,7 +161,8 @@ class StreamScratch {
   void* pointer_;
   size_t bytes_;
   hipStream_t stream_;
-  void* cached_;  // the cache entry this object holds, or nullptr for stream-ordered memory
+  void* cached_;          // the cache entry this object holds a piece of, or nullptr for stream-ordered memory
+  size_t cached_offset_;  // where in the entry's buffer the piece starts
 };
 void ReleaseCachedScratch();
 
