@@ -286,15 +286,15 @@ int clbh_triangular_to_square(int precision, int upper, int unit_diagonal, int k
   }
 }
 
-int clbh_invert_block_size(int precision) { return (precision == 64) ? 64 : 128; }
+int clbh_invert_block_size(int precision) { (void)precision; return 64; }
 
 int clbh_invert_diagonal_blocks(int precision, int upper, int blocks, const void* src, long long src_ld, void* dst,
                                 long long dst_ld, hipStream_t stream) {
   const long long extent = static_cast<long long>(blocks) * clbh_invert_block_size(precision);
   if (blocks <= 0 || src == nullptr || dst == nullptr || src_ld < extent || dst_ld < extent) { return hipErrorInvalidValue; }
   switch (precision) {
-    case 16: return LaunchInvertDiagonalBlocks<_Float16, float, 128>(upper, blocks, src, src_ld, dst, dst_ld, stream);
-    case 32: return LaunchInvertDiagonalBlocks<float, float, 128>(upper, blocks, src, src_ld, dst, dst_ld, stream);
+    case 16: return LaunchInvertDiagonalBlocks<_Float16, float, 64>(upper, blocks, src, src_ld, dst, dst_ld, stream);
+    case 32: return LaunchInvertDiagonalBlocks<float, float, 64>(upper, blocks, src, src_ld, dst, dst_ld, stream);
     case 64: return LaunchInvertDiagonalBlocks<double, double, 64>(upper, blocks, src, src_ld, dst, dst_ld, stream);
     default: return hipErrorInvalidValue;
   }

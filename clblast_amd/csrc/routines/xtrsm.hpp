@@ -5,9 +5,9 @@
 // The reference walks the diagonal in blocks of 16: it inverts the 16 x 16 diagonal blocks, and for every block
 // runs one small GEMM with the inverse and one GEMM that updates the rest of B, synchronising with the host in
 // between. The structure here is the same - inverted diagonal blocks, everything else is GEMM - but recursive and
-// stream-ordered: one kernel inverts the 128 x 128 (fp64: 64 x 64) diagonal blocks, strided-batched GEMMs double the
-// inverses up to 512 x 512 leaves, and the triangle is halved recursively, so that the bulk of the work is a few
-// GEMMs with a long K instead of many rank-16 updates.
+// stream-ordered: one kernel inverts the 64 x 64 diagonal blocks (32 x 32 for double complex), strided-batched GEMMs
+// double the inverses up to 512 x 512 leaves, and the triangle is halved recursively, so that the bulk of the work is
+// a few GEMMs with a long K instead of many rank-16 updates.
 //
 // T is float, double, std::complex<float> or std::complex<double> (the reference has no half-precision TRSM); the
 // complex types run the same recursion on the complex GEMM (routines/xgemm_complex.hpp) with complex versions of the

@@ -100,7 +100,8 @@ CLBH_API int clbh_triangular_to_square(int precision, int upper, int unit_diagon
                                        long long src_offset, long long src_ld, void* dst, int dst_extent,
                                        long long dst_ld, hipStream_t stream);
 
-// Block size of clbh_invert_diagonal_blocks for a precision (128 for 16 and 32 bits, 64 for 64 bits).
+// Block size of clbh_invert_diagonal_blocks for a precision (64 for all three: larger blocks are cheaper to build by
+// doubling with GEMMs than inside the inversion kernel).
 CLBH_API int clbh_invert_block_size(int precision);
 
 // Inverts the `blocks` diagonal blocks (clbh_invert_block_size(precision) squared each) of the dense triangular matrix
