@@ -389,6 +389,33 @@ int clbh_complex_scale(int precision, int m, int n, int triangle, double beta_re
   return clbh_complex_scale_batched(precision, m, n, triangle, beta_re, beta_im, c, c_offset, c_ld, nullptr, stream);
 }
 
+int clbh_pad_image(int precision, int planes, int height, int width, int pad_h, int pad_w, const void* src,
+                   long long src_offset, void* dst, hipStream_t stream) {
+  const long long padded = static_cast<long long>(height + 2ll * pad_h) * (width + 2ll * pad_w);
+  if (planes <= 0 || height <= 0 || width <= 0 || pad_h < 0 || pad_w < 0 || src == nullptr || dst == nullptr || src_offset < 0 ||
+      padded > INT_MAX) {
+    return hipErrorInvalidValue;
+  }
+  const dim3 grid(static_cast<unsigned>((padded + clbh::kIm2colThreads - 1) / clbh::kIm2colThreads),
+                  static_cast<unsigned>(std::min(planes, 65535)));
+  switch (precision) {
+    case 16:
+      clbh::PadImageKernel<_Float16><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(
+          planes, height, width, pad_h, pad_w, static_cast<const _Float16*>(src) + src_offset, static_cast<_Float16*>(dst));
+      break;
+    case 32:
+      clbh::PadImageKernel<float><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(
+          planes, height, width, pad_h, pad_w, static_cast<const float*>(src) + src_offset, static_cast<float*>(dst));
+      break;
+    case 64:
+      clbh::PadImageKernel<double><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(
+          planes, height, width, pad_h, pad_w, static_cast<const double*>(src) + src_offset, static_cast<double*>(dst));
+      break;
+    default: return hipErrorInvalidValue;
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
 int clbh_conv_gather_possible(int precision, const clbh_im2col_shape* shape) {
   return (shape != nullptr && clbh::ConvGatherPossible(precision, *shape)) ? 1 : 0;
 }

@@ -18,7 +18,12 @@ int LaunchConvF32(const clbh_gemm_desc& d, hipStream_t stream) {
       d.a_stride < static_cast<long long>(g.channels) * g.height * g.width) {
     return hipErrorInvalidValue;
   }
-  return LaunchMfmaVariant<float, MfmaConfig<float, 2, 2, 1, 1, 16, 4>, false, true, true, true>(d, stream);
+  // without padding, with unit stride along the width and whole groups of four patches per output row a lane can
+  // fetch four patches at once (GatherLoadVector)
+  if (g.pad_h == 0 && g.pad_w == 0 && g.stride_w == 1 && g.output_w % 4 == 0) {
+    return LaunchMfmaVariant<float, MfmaConfig<float, 2, 2, 1, 1, 16, 4>, false, true, true, 2>(d, stream);
+  }
+  return LaunchMfmaVariant<float, MfmaConfig<float, 2, 2, 1, 1, 16, 4>, false, true, true, 1>(d, stream);
 }
 
 }  // namespace

@@ -34,7 +34,7 @@ int LaunchGeneral(const clbh_gemm_desc& d, hipStream_t stream) {
 }
 
 // ---- MFMA kernels (fp32, fp64) ----------------------------------------------------------------------
-template <typename T, typename Config, bool A_KC, bool B_KC, bool ALIGNED, bool A_CONV = false>
+template <typename T, typename Config, bool A_KC, bool B_KC, bool ALIGNED, int A_CONV = 0>
 int LaunchMfmaVariant(const clbh_gemm_desc& d, hipStream_t stream) {
   auto args = MakeArgs<T>(d);
   const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;

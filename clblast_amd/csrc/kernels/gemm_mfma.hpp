@@ -252,6 +252,40 @@ __device__ __forceinline__ void GatherLoad(const T* __restrict__ image, const Co
                                            0, 0);
 }
 
+// Gathered operand, 16 bytes per lane: for images without padding, unit stride along the width and an output width
+// that is a multiple of 4, four consecutive patches of an output row are four consecutive image elements for every
+// tap, so a lane can fetch them in one piece and a wavefront needs ONE load per slab (64 patches x 16 rows: lanes
+// 0..15 bring row 4 * wave of the slab, lanes 16..31 the next one, ...). Each lane decomposes its own row; the row a
+// lane serves advances by TILE_K per slab. `patch_offset` is the lane's offset of its first patch in the image plane,
+// or negative for patches beyond m.
+template <typename T, int TILE_X, int TILE_K, typename Tag>
+__device__ __forceinline__ void GatherLoadVector(const T* __restrict__ image, const ConvGather& g, T* stage, const int wave,
+                                                 const int round, const int k0, const int k_len, const int lane,
+                                                 const int patch_offset) {
+  using L = SlabLayout<T, TILE_X, TILE_K, true, 16>;
+  static_assert(L::PARTS == 1 && sizeof(T) == 4, "whole rows per load, dword elements");
+  static_assert(L::LOADS % 4 == 0, "every wavefront issues the same number of loads (the waits count them)");
+  const int group = wave + 4 * round;
+  const unsigned p = static_cast<unsigned>(k0 + group * L::R + (lane * 16) / L::ROW_BYTES);
+  const unsigned channel = (g.taps == 1) ? p : __umulhi(p, g.taps_magic);
+  const unsigned kernel_index = p - channel * g.taps;
+  const unsigned tap = g.flip ? (g.taps - 1 - kernel_index) : kernel_index;
+  const unsigned kh = (g.kernel_w == 1) ? tap : __umulhi(tap, g.kernel_w_magic);
+  const unsigned kw = tap - kh * g.kernel_w;
+  const int plane_offset = (static_cast<int>(channel) * g.height + static_cast<int>(kh) * g.dilation_h) * g.width +
+                           static_cast<int>(kw) * g.dilation_w;
+  const bool inside = static_cast<int>(p) < k_len && patch_offset >= 0;
+  const int offset_bytes = inside ? (plane_offset + patch_offset) * 4 : static_cast<int>(0x80000000u);
+  const unsigned long long address = reinterpret_cast<unsigned long long>(image);
+  const unsigned long long low = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(address)));
+  const unsigned long long high = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(address >> 32)));
+  T* uniform_image = reinterpret_cast<T*>((high << 32) | low);
+  const int bytes = __builtin_amdgcn_readfirstlane(static_cast<int>(g.image_bytes));
+  typedef __attribute__((address_space(3))) void* LdsPtr;
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(__builtin_amdgcn_make_buffer_rsrc(uniform_image, 0, bytes, kRawBufferFlags),
+                                           (LdsPtr)(stage + group * L::GROUP_PITCH), 16, offset_bytes, 0, 0, 0);
+}
+
 // Staged operand: thread t moves the pieces t, t + 256, ... of the slab (VL elements each, consecutive
 // threads along k); with LINES whole x lines per round, piece c lies c * LINES lines after piece 0.
 template <int TILE_X, int TILE_K, int VL>
@@ -340,8 +374,9 @@ __device__ __forceinline__ bool TileOfBlockCyclic(const int block, const int til
 }
 
 // ---- the kernel ------------------------------------------------------------------------------------
-// A_CONV: the A operand is gathered from a batch of images (GemmArgs::conv); needs !A_KC and fp32.
-template <typename T, typename Config, bool A_KC, bool B_KC, bool ALIGNED, bool A_CONV = false>
+// A_CONV != 0: the A operand is gathered from a batch of images (GemmArgs::conv); needs !A_KC and fp32. 1: one element
+// per lane, any convolution; 2: four per lane (GatherLoadVector names the conditions).
+template <typename T, typename Config, bool A_KC, bool B_KC, bool ALIGNED, int A_CONV = 0>
 __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void GemmMfmaKernel(const GemmArgs<T> p, const int tiles_m,
                                                                const int tiles_n) {
   using Traits = typename Config::Traits;
@@ -354,8 +389,8 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
   constexpr int VL = ALIGNED ? VEC : 1;         // elements per staged global access
   constexpr int LANE_BYTES = ALIGNED ? 16 : 4;  // bytes per lane of a direct load
   constexpr bool A_DIRECT = !A_KC, B_DIRECT = !B_KC;
-  static_assert(!A_CONV || !A_KC, "a gathered operand takes the direct path");
-  constexpr int LANE_BYTES_A = A_CONV ? 4 : LANE_BYTES;  // the gather moves single elements
+  static_assert(A_CONV == 0 || !A_KC, "a gathered operand takes the direct path");
+  constexpr int LANE_BYTES_A = (A_CONV == 1) ? 4 : LANE_BYTES;  // the general gather moves single elements
   using LA = SlabLayout<T, TILE_M, TILE_K, A_DIRECT, LANE_BYTES_A>;
   using LB = SlabLayout<T, TILE_N, TILE_K, B_DIRECT, LANE_BYTES>;
   using PA = StagedPieces<TILE_M, TILE_K, VL>;
@@ -372,7 +407,7 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
   using VM = typename VecType<T, FM>::type;
   using VN = typename VecType<T, FN>::type;
   using VP = typename VecType<T, VL>::type;
-  using KernelTag = std::tuple<Config, std::integral_constant<int, (A_CONV ? 8 : 0) | (A_KC ? 4 : 0) | (B_KC ? 2 : 0) | (ALIGNED ? 1 : 0)>>;
+  using KernelTag = std::tuple<Config, std::integral_constant<int, A_CONV * 8 + (A_KC ? 4 : 0) | (B_KC ? 2 : 0) | (ALIGNED ? 1 : 0)>>;
 
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
@@ -407,9 +442,15 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
 
   // Gathered A: the patches this lane loads (one per part of a tile row), as the top-left corner of the patch in the
   // padded image and the offset of that corner in the image plane; patches beyond m never pass the bounds test
-  constexpr int GATHER_PARTS = A_CONV ? LA::PARTS : 1;
+  constexpr int GATHER_PARTS = (A_CONV == 1) ? LA::PARTS : 1;
   int patch_h[GATHER_PARTS], patch_w[GATHER_PARTS], patch_offset[GATHER_PARTS];
-  if constexpr (A_CONV) {
+  if constexpr (A_CONV == 2) {  // the lane's four patches: first one at 4 * (lane % 16) of the tile row
+    const int patch = m0 + (lane * 4) % TILE_M;
+    const int oh = patch / p.conv.output_w, ow = patch - oh * p.conv.output_w;
+    patch_offset[0] = (patch < p.m) ? oh * p.conv.stride_h * p.conv.width + ow : -1;
+    patch_h[0] = patch_w[0] = 0;
+  }
+  if constexpr (A_CONV == 1) {
 #pragma unroll
     for (int part = 0; part < GATHER_PARTS; ++part) {
       const int patch = m0 + part * LA::WAVE_ELEMS + lane;
@@ -498,8 +539,10 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
       auto direct_load = [&](const int load, const int k0, auto* a_dst, auto* b_dst) {
         if constexpr (DIRECT_A > 0) {
           if (load < DIRECT_A) {
-            if constexpr (A_CONV) {
+            if constexpr (A_CONV == 1) {
               GatherLoad<T, TILE_M, TILE_K, KernelTag>(a, p.conv, a_dst, wave_u, load, gather_rows, patch_h, patch_w, patch_offset);
+            } else if constexpr (A_CONV == 2) {
+              GatherLoadVector<T, TILE_M, TILE_K, KernelTag>(a, p.conv, a_dst, wave_u, load, k0, k_len, lane, patch_offset[0]);
             } else {
               DirectLoad<T, TILE_M, TILE_K, LANE_BYTES, RANGE, KernelTag>(a_slab(k0), a_end, p.a_ld, a_dst, wave_u, a_lane_bytes, load);
             }
@@ -526,7 +569,7 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
 
       // Prologue: slab 0 lands in buffer 0 (the staged registers' wait also covers the older direct loads),
       // slab 1 is requested.
-      if constexpr (A_CONV) { gather_rows = DecomposeRows<TILE_K>(p.conv, 0, k_len, lane); }
+      if constexpr (A_CONV == 1) { gather_rows = DecomposeRows<TILE_K>(p.conv, 0, k_len, lane); }
 #pragma unroll
       for (int load = 0; load < DIRECT; ++load) { direct_load(load, 0, a_stages, b_stages); }
 #pragma unroll
@@ -535,7 +578,7 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
       for (int piece = 0; piece < STAGED; ++piece) { store_piece(piece, a_stages, b_stages, 0, std::true_type{}); }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       if (slabs > 1) {
-        if constexpr (A_CONV) { gather_rows = DecomposeRows<TILE_K>(p.conv, TILE_K, k_len, lane); }
+        if constexpr (A_CONV == 1) { gather_rows = DecomposeRows<TILE_K>(p.conv, TILE_K, k_len, lane); }
 #pragma unroll
         for (int load = 0; load < DIRECT; ++load) { direct_load(load, TILE_K, a_stages + LA::ELEMS, b_stages + LB::ELEMS); }
 #pragma unroll
@@ -561,7 +604,7 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
         T* a_prv = a_stages + prv * LA::ELEMS;
         T* b_prv = b_stages + prv * LB::ELEMS;
         const int k_store = (slab + 1) * TILE_K, k_load = (slab + 2) * TILE_K;
-        if constexpr (A_CONV && LOAD) { gather_rows = DecomposeRows<TILE_K>(p.conv, k_load, k_len, lane); }
+        if constexpr (A_CONV == 1 && LOAD) { gather_rows = DecomposeRows<TILE_K>(p.conv, k_load, k_len, lane); }
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
           const int set = ks % 2;

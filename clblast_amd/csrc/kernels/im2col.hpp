@@ -65,6 +65,24 @@ __global__ __launch_bounds__(kIm2colThreads) void Im2colKernel(const Im2colShape
   }
 }
 
+// Copies `planes` image planes of height x width into planes of (height + 2 pad_h) x (width + 2 pad_w) with a border of
+// zeros, for the convolution kernels that want every patch element to exist. grid: (ceil(padded plane / 256),
+// min(planes, 65535)).
+template <typename T>
+__global__ __launch_bounds__(kIm2colThreads) void PadImageKernel(const int planes, const int height, const int width,
+                                                                 const int pad_h, const int pad_w,
+                                                                 const T* __restrict__ src, T* __restrict__ dst) {
+  const int padded_w = width + 2 * pad_w, padded_h = height + 2 * pad_h;
+  const int index = blockIdx.x * kIm2colThreads + threadIdx.x;
+  if (index >= padded_h * padded_w) { return; }
+  const int row = index / padded_w - pad_h, col = index % padded_w - pad_w;
+  const bool inside = (row >= 0 && row < height && col >= 0 && col < width);
+  for (int plane = blockIdx.y; plane < planes; plane += gridDim.y) {
+    dst[static_cast<long long>(plane) * padded_h * padded_w + index] =
+        inside ? src[(static_cast<long long>(plane) * height + row) * width + col] : T(0);
+  }
+}
+
 }  // namespace clbh
 
 #endif  // CLBLAST_HIP_KERNELS_IM2COL_HPP_

@@ -4,6 +4,7 @@
 #include "routines/xconvgemm.hpp"
 
 #include <climits>
+#include <memory>
 
 namespace clblast {
 // =================================================================================================
@@ -78,6 +79,33 @@ void Xconvgemm<T>::DoConvgemm(const KernelMode kernel_mode, const size_t channel
   // The reference's single-kernel method (xconvgemm.cpp:121-160, doc/details_conv.md): no im2col matrix; the GEMM kernel
   // gathers the patches from the images while it loads its tiles. fp32, all batches in one launch.
   if (clbh_conv_gather_possible(precision, &shape) != 0) {
+    // With unit stride along the width and whole groups of four patches per output row the kernel fetches four patches
+    // per lane - if no patch element lies in the padding: then the images are copied into a zero border first (one
+    // pass over the images instead of a nine times larger im2col matrix), and the kernel sees images without padding.
+    auto gather_shape = shape;
+    const void* images = im_buffer();
+    auto images_offset = static_cast<long long>(im_offset);
+    std::unique_ptr<StreamScratch> padded;
+    if ((pad_h > 0 || pad_w > 0) && stride_w == 1 && output_w % 4 == 0) {
+      auto padded_shape = shape;
+      padded_shape.height = static_cast<int>(height + 2 * pad_h);
+      padded_shape.width = static_cast<int>(width + 2 * pad_w);
+      padded_shape.pad_h = 0;
+      padded_shape.pad_w = 0;
+      if (clbh_conv_gather_possible(precision, &padded_shape) != 0) {
+        const auto planes = batch_count * channels;
+        const auto padded_bytes = planes * (height + 2 * pad_h) * (width + 2 * pad_w) * sizeof(T);
+        if (planes <= kLimit) {
+          padded.reset(new StreamScratch(padded_bytes, this->stream(), "images with a border of zeros"));
+          CheckDevice(clbh_pad_image(precision, static_cast<int>(planes), shape.height, shape.width, shape.pad_h, shape.pad_w,
+                                     im_buffer(), images_offset, padded->get(), this->stream()),
+                      "clbh_pad_image");
+          gather_shape = padded_shape;
+          images = padded->get();
+          images_offset = 0;
+        }
+      }
+    }
     auto desc = clbh_gemm_desc{};
     desc.precision = precision;
     desc.kernel_class = CLBH_KERNEL_MFMA;
@@ -89,10 +117,10 @@ void Xconvgemm<T>::DoConvgemm(const KernelMode kernel_mode, const size_t channel
     desc.n = static_cast<int>(num_kernels);
     desc.k = static_cast<int>(patch_size);
     desc.batch_count = static_cast<int>(batch_count);
-    desc.a = im_buffer();
-    desc.a_offset = static_cast<long long>(im_offset);
+    desc.a = images;
+    desc.a_offset = images_offset;
     desc.a_ld = static_cast<long long>(num_patches);  // of the patch matrix that is never stored
-    desc.a_stride = static_cast<long long>(channels * height * width);
+    desc.a_stride = static_cast<long long>(channels) * gather_shape.height * gather_shape.width;
     desc.b = kernel_buffer();
     desc.b_offset = static_cast<long long>(kernel_offset);
     desc.b_ld = static_cast<long long>(patch_size);
@@ -103,7 +131,7 @@ void Xconvgemm<T>::DoConvgemm(const KernelMode kernel_mode, const size_t channel
     desc.c_stride = static_cast<long long>(result_stride);
     desc.alpha = 1.0;
     desc.beta = 0.0;
-    desc.conv = &shape;
+    desc.conv = &gather_shape;
     CheckDevice(clbh_gemm_launch(&desc, this->stream()), "clbh_gemm_launch (gathered convolution)");
     this->Finish();
     return;

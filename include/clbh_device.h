@@ -167,6 +167,10 @@ typedef struct clbh_im2col_shape_ {
 } clbh_im2col_shape;
 CLBH_API int clbh_im2col(int precision, const clbh_im2col_shape* shape, int batch_count, const void* image,
                          long long image_offset, void* col, hipStream_t stream);
+// dst = `planes` planes of (height + 2 pad_h) x (width + 2 pad_w): the planes of height x width at src + src_offset
+// inside a border of zeros.
+CLBH_API int clbh_pad_image(int precision, int planes, int height, int width, int pad_h, int pad_w, const void* src,
+                            long long src_offset, void* dst, hipStream_t stream);
 // Non-zero when a GEMM launch can gather its A operand from images of this shape itself (clbh_gemm_desc::conv): fp32
 // only, one image below 2 GiB, and row indices small enough for the kernel's division by multiplication.
 CLBH_API int clbh_conv_gather_possible(int precision, const clbh_im2col_shape* shape);

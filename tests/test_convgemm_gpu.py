@@ -24,6 +24,9 @@ CASES = [  # channels, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h
     (8, 30, 17, 3, 3, 0, 1, 2, 2, 1, 1, 20, 20),   # small patches x kernels, 20 batches
     (3, 64, 64, 7, 7, 3, 3, 2, 2, 1, 1, 64, 2),
     (4, 4, 4, 3, 3, 0, 0, 1, 1, 1, 1, 2, 40),      # 2 x 2 outputs, many batches
+    (5, 12, 16, 3, 5, 1, 2, 2, 1, 1, 1, 7, 3),     # unit stride along the width, output width 16: four patches per lane (fp32)
+    (3, 10, 20, 3, 3, 0, 2, 1, 1, 2, 2, 9, 2),     # the same with dilation, padding along the width only
+    (6, 9, 12, 2, 1, 0, 0, 1, 1, 1, 1, 70, 2),     # no padding at all (no padded copy), kernel width 1, 70 kernels
 ]
 
 
@@ -132,7 +135,7 @@ def test_convgemm_against_the_real_reference(gpu, tmp_path):
     problems = []
     seed = 19000
     for bits in (32, 64, 16):
-        for case in CASES[:9]:
+        for case in CASES[:9] + CASES[10:]:
             for mode in (CROSS_CORRELATION, CONVOLUTION):
                 seed += 1
                 problems.append(ConvProblem(bits, mode, case, seed, ((0, 0, 0), (10, 6, 14))[seed % 2]))
