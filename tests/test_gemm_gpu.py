@@ -208,3 +208,20 @@ def test_split_k_calls_share_the_streams_scratch(gpu, bits):
         status, c_after = problem.run()
         assert status == 0, problem.describe()
         problem.check(c_after)
+
+
+@pytest.mark.parametrize("bits", BITS)
+def test_long_k_with_few_tiles(gpu, bits):
+    """Shapes the tile table splits along K by itself (few tiles, a long K walk), in all three precisions - fp16 keeps
+    its partial sums in fp32 - with a K that is no multiple of the range size, padded leading dimensions and offsets
+    (odd ones: fp16 operands are then copied into aligned temporaries first)."""
+    seed = 9950
+    for (m, n, k), (ta, tb) in itertools.product(((256, 256, 4096), (130, 70, 8200), (1030, 17, 4100), (17, 1030, 2048)),
+                                                 ((NO, NO), (YES, NO), (NO, YES))):
+        seed += 1
+        extra, offsets = (((0, 0, 0), (0, 0, 0)), ((3, 1, 5), (11, 13, 19)), ((8, 8, 8), (16, 8, 24)))[seed % 3]
+        problem = gpu.Problem(bits, (COL_MAJOR, ROW_MAJOR)[seed % 2], ta, tb, m, n, k, -0.75, (2.0, 0.0)[seed % 2],
+                              a_offset=offsets[0], b_offset=offsets[1], c_offset=offsets[2], seed=seed, extra_ld=extra)
+        status, c_after = problem.run()
+        assert status == 0, problem.describe()
+        problem.check(c_after)
