@@ -70,7 +70,9 @@ struct Tile {
 
 // Share of the tiles' area that the m x n matrix fills (tiles of tile_m x tile_n), in per cent
 size_t TileUse(const size_t m, const size_t n, const size_t tile_m, const size_t tile_n) {
-  return 100 * m * n / (CeilDivide(m, tile_m) * tile_m * CeilDivide(n, tile_n) * tile_n);
+  const auto along_m = static_cast<double>(m) / static_cast<double>(CeilDivide(m, tile_m) * tile_m);
+  const auto along_n = static_cast<double>(n) / static_cast<double>(CeilDivide(n, tile_n) * tile_n);
+  return static_cast<size_t>(100.0 * along_m * along_n + 0.5);
 }
 
 // True when `tiles` large tiles (one work-group per CU at a time) keep the 256 CUs busy: two rounds or more, or at
