@@ -18,7 +18,7 @@ namespace {
 
 int LaunchTyped(const clbh_gemm_desc& d, hipStream_t stream) {
   const bool mfma = (d.kernel_class == CLBH_KERNEL_MFMA);
-  if (d.conv != nullptr && !(mfma && d.precision == 32)) { return hipErrorInvalidValue; }  // only that kernel gathers
+  if (d.conv != nullptr && !(mfma && (d.precision == 32 || d.precision == 16))) { return hipErrorInvalidValue; }  // only those kernels gather
   if (d.kernel_class == CLBH_KERNEL_SMALL_BATCHED) { return LaunchSmallBatched(d, stream); }
   switch (d.precision) {
     case 16: return mfma ? LaunchMfmaF16(d, stream) : LaunchGeneralF16(d, stream);
@@ -389,27 +389,39 @@ int clbh_complex_scale(int precision, int m, int n, int triangle, double beta_re
   return clbh_complex_scale_batched(precision, m, n, triangle, beta_re, beta_im, c, c_offset, c_ld, nullptr, stream);
 }
 
-int clbh_pad_image(int precision, int planes, int height, int width, int pad_h, int pad_w, const void* src,
-                   long long src_offset, void* dst, hipStream_t stream) {
-  const long long padded = static_cast<long long>(height + 2ll * pad_h) * (width + 2ll * pad_w);
-  if (planes <= 0 || height <= 0 || width <= 0 || pad_h < 0 || pad_w < 0 || src == nullptr || dst == nullptr || src_offset < 0 ||
-      padded > INT_MAX) {
+int clbh_pad_image(int precision, int images, int channels, int height, int width, int pad_h, int pad_w, int extra_w,
+                   const void* src, long long src_offset, void* dst, long long image_stride, long long copy_stride,
+                   hipStream_t stream) {
+  const long long padded = static_cast<long long>(height + 2ll * pad_h) * (width + 2ll * pad_w + extra_w);
+  const long long planes = static_cast<long long>(images) * channels;
+  if (images <= 0 || channels <= 0 || height <= 0 || width <= 0 || pad_h < 0 || pad_w < 0 || extra_w < 0 || src == nullptr ||
+      dst == nullptr || src_offset < 0 || padded > INT_MAX || planes > INT_MAX || copy_stride < 0 ||
+      (copy_stride > 0 && copy_stride < channels * padded) || image_stride < (copy_stride > 0 ? copy_stride : 0) + channels * padded) {
     return hipErrorInvalidValue;
   }
-  const dim3 grid(static_cast<unsigned>((padded + clbh::kIm2colThreads - 1) / clbh::kIm2colThreads),
-                  static_cast<unsigned>(std::min(planes, 65535)));
+  const long long total = channels * padded;
+  const auto launch = [&](auto element, auto vec_tag) {
+    using T = decltype(element);
+    constexpr int VEC = decltype(vec_tag)::value;
+    const long long threads = (total + VEC - 1) / VEC;
+    const dim3 grid(static_cast<unsigned>((threads + clbh::kIm2colThreads - 1) / clbh::kIm2colThreads),
+                    static_cast<unsigned>(std::min(images, 65535)));
+    clbh::PadImageKernel<T, VEC><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(
+        images, channels, height, width, pad_h, pad_w, extra_w, static_cast<const T*>(src) + src_offset, static_cast<T*>(dst),
+        image_stride, copy_stride);
+  };
+  const auto vector_ok = [&](const long long vec) {
+    return total % vec == 0 && image_stride % vec == 0 && copy_stride % vec == 0 && reinterpret_cast<unsigned long long>(dst) % 16 == 0;
+  };
   switch (precision) {
     case 16:
-      clbh::PadImageKernel<_Float16><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(
-          planes, height, width, pad_h, pad_w, static_cast<const _Float16*>(src) + src_offset, static_cast<_Float16*>(dst));
+      if (vector_ok(8)) { launch(_Float16(0), std::integral_constant<int, 8>{}); } else { launch(_Float16(0), std::integral_constant<int, 1>{}); }
       break;
     case 32:
-      clbh::PadImageKernel<float><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(
-          planes, height, width, pad_h, pad_w, static_cast<const float*>(src) + src_offset, static_cast<float*>(dst));
+      if (vector_ok(4)) { launch(0.0f, std::integral_constant<int, 4>{}); } else { launch(0.0f, std::integral_constant<int, 1>{}); }
       break;
     case 64:
-      clbh::PadImageKernel<double><<<grid, dim3(clbh::kIm2colThreads), 0, stream>>>(
-          planes, height, width, pad_h, pad_w, static_cast<const double*>(src) + src_offset, static_cast<double*>(dst));
+      if (vector_ok(2)) { launch(0.0, std::integral_constant<int, 2>{}); } else { launch(0.0, std::integral_constant<int, 1>{}); }
       break;
     default: return hipErrorInvalidValue;
   }

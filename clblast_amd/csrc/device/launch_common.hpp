@@ -77,14 +77,18 @@ GemmArgs<CT> MakeArgs(const clbh_gemm_desc& d) {
     p.conv.dilation_h = g.dilation_h;
     p.conv.dilation_w = g.dilation_w;
     p.conv.flip = g.flip;
-    p.conv.image_bytes = static_cast<unsigned>(4ll * g.channels * g.height * g.width);
+    const long long image_elements = static_cast<long long>(g.channels) * g.height * g.width;
+    p.conv.image_bytes = static_cast<unsigned>(d.precision == 16 ? 2 * (d.conv_copy_stride + image_elements) : 4 * image_elements);
+    p.conv.copy_stride = static_cast<int>(d.precision == 16 ? d.conv_copy_stride : 0);
   }
   return p;
 }
 
 // True when the GEMM kernels can gather the A operand of a CONVGEMM from images of this shape (see ConvGather).
 inline bool ConvGatherPossible(const int precision, const clbh_im2col_shape& g) {
-  if (precision != 32) { return false; }
+  if (precision != 32 && precision != 16) { return false; }
+  // fp16: eight patches per lane from images without padding, dword-aligned through the second copy
+  if (precision == 16 && (g.pad_h != 0 || g.pad_w != 0 || g.stride_w != 1 || g.width % 2 != 0 || g.output_w % 8 != 0)) { return false; }
   if (g.channels <= 0 || g.height <= 0 || g.width <= 0 || g.kernel_h <= 0 || g.kernel_w <= 0 || g.stride_h <= 0 ||
       g.stride_w <= 0 || g.dilation_h <= 0 || g.dilation_w <= 0 || g.output_h <= 0 || g.output_w <= 0 || g.pad_h < 0 ||
       g.pad_w < 0) {

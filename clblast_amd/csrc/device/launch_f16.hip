@@ -61,7 +61,7 @@ int LaunchHgemmConfig(const clbh_gemm_desc& d, hipStream_t stream) {
 }
 
 // ---- direct-load MFMA kernel, fp16 (dword-aligned operands) ---------------------------------------
-template <typename Config, bool A_KC, bool B_KC>
+template <typename Config, bool A_KC, bool B_KC, bool A_CONV = false>
 int LaunchHdirectVariant(const clbh_gemm_desc& d, hipStream_t stream) {
   auto args = MakeArgs<float>(d);
   const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
@@ -81,7 +81,7 @@ int LaunchHdirectVariant(const clbh_gemm_desc& d, hipStream_t stream) {
   }
   const dim3 grid(static_cast<unsigned>(TileBlocks(d, tiles_m, tiles_n)), static_cast<unsigned>(grid_y));
   constexpr size_t lds_bytes = Config::LDS_BYTES;
-  auto kernel = HgemmDirectKernel<Config, A_KC, B_KC>;
+  auto kernel = HgemmDirectKernel<Config, A_KC, B_KC, A_CONV>;
   if (lds_bytes > 48 * 1024) {
     static const hipError_t attribute_status = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
@@ -125,9 +125,30 @@ bool DwordAlignedHalf(const clbh_gemm_desc& d) {
   return true;
 }
 
+// CONVGEMM with the A operand gathered from the images (clbh_gemm_desc::conv; HGatherPiece names the conditions): the
+// kernel matrix is k-contiguous and dword aligned, the batches are strided, K is not split
+int LaunchConvF16(const clbh_gemm_desc& d, hipStream_t stream) {
+  const auto& g = *d.conv;
+  const long long patches = static_cast<long long>(g.output_h) * g.output_w;
+  const long long rows = static_cast<long long>(g.channels) * g.kernel_h * g.kernel_w;
+  const long long image_elements = static_cast<long long>(g.channels) * g.height * g.width;
+  const auto b_address = reinterpret_cast<unsigned long long>(d.b) + 2ull * static_cast<unsigned long long>(d.b_offset);
+  const auto a_address = reinterpret_cast<unsigned long long>(d.a) + 2ull * static_cast<unsigned long long>(d.a_offset);
+  if (!ConvGatherPossible(d.precision, g) || d.m != patches || d.k != rows || !d.b_kcontig || d.a_kcontig ||
+      d.batch.alphas != nullptr || d.split_k > 1 || d.c_triangle != 0 || d.operand_triangle != 0 ||
+      d.conv_copy_stride < image_elements || d.conv_copy_stride % 2 != 0 || d.a_stride < d.conv_copy_stride + image_elements ||
+      d.a_stride % 2 != 0 || a_address % 4 != 0 || b_address % 4 != 0 || d.b_ld % 2 != 0 || d.b_stride % 2 != 0 ||
+      2 * (d.conv_copy_stride + image_elements) >= (1ll << 31)) {
+    return hipErrorInvalidValue;
+  }
+  if (d.tile_variant == 1) { return LaunchHdirectVariant<HdirectConfig<2, 2, 1, 1, 4>, false, true, true>(d, stream); }  // 64 x 64
+  return LaunchHdirectVariant<HdirectConfig<2, 2, 2, 2, 2>, false, true, true>(d, stream);                               // 128 x 128
+}
+
 }  // namespace
 
 int LaunchMfmaF16(const clbh_gemm_desc& d, hipStream_t stream) {
+  if (d.conv != nullptr) { return LaunchConvF16(d, stream); }
   if (!LeadingDimsFitTiles<_Float16>(d)) { return LaunchGeneral<_Float16>(d, stream); }
   // operands at odd element offsets or with odd leading dimensions: element-wise 128 x 128 kernel
   if (!DwordAlignedHalf(d)) { return LaunchHgemmConfig<HgemmConfig<2, 2, 2, 2, 32, 2>, false>(d, stream); }

@@ -25,6 +25,7 @@ struct ConvGather {
   int pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w;
   int flip;
   unsigned image_bytes;  // bytes of one image (all channels): the range of the gather's buffer resource
+  int copy_stride;       // fp16: elements from an image to its copy shifted by one element (see HGatherPiece), else 0
 };
 
 template <typename CT>

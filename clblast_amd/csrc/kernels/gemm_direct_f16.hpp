@@ -87,6 +87,40 @@ __device__ __forceinline__ void HRequestPiece(const _Float16* __restrict__ sourc
       (LdsPtr)(destination), 16, lane_bytes, 0, 0, 0);
 }
 
+// The request of a lane for a piece of a gathered A operand (CONVGEMM without an im2col matrix, see ConvGather): the
+// lane's 16 bytes are eight consecutive patches of one output row in row `p` of the patch matrix - eight consecutive
+// image elements, for images without padding, unit stride along the width and an output width that is a multiple of
+// 8. The loads move dwords, so an odd element offset cannot be fetched from the image itself: the host keeps a second
+// copy of the images shifted by one element, copy_stride elements behind the first (copy[j] = image[j + 1]), and odd
+// offsets read that one. With an even image width the parity is that of the tap's column offset. `patch_offset` is
+// the offset of the lane's first patch in the image plane (even), or negative for patches beyond m; rows beyond k and
+// those patches get an offset beyond the resource's range, which reads as zero.
+template <typename Tag>
+__device__ __forceinline__ void HGatherPiece(const _Float16* __restrict__ image, const ConvGather& g, _Float16* destination,
+                                             const int p_row, const int k_len, const int patch_offset) {
+  const unsigned p = static_cast<unsigned>(p_row);
+  const unsigned channel = (g.taps == 1) ? p : __umulhi(p, g.taps_magic);
+  const unsigned kernel_index = p - channel * g.taps;
+  const unsigned tap = g.flip ? (g.taps - 1 - kernel_index) : kernel_index;
+  const unsigned kh = (g.kernel_w == 1) ? tap : __umulhi(tap, g.kernel_w_magic);
+  const unsigned kw = tap - kh * g.kernel_w;
+  const int element = (static_cast<int>(channel) * g.height + static_cast<int>(kh) * g.dilation_h) * g.width +
+                      static_cast<int>(kw) * g.dilation_w + patch_offset;
+  const int aligned = (element & 1) ? element - 1 + g.copy_stride : element;
+  const bool inside = p_row < k_len && patch_offset >= 0;
+  const int offset_bytes = inside ? aligned * 2 : static_cast<int>(0x80000000u);
+  // (the resource is taken from the first lane explicitly: under register pressure the compiler keeps it in vector
+  // registers otherwise and loops over its distinct values around every load)
+  const unsigned long long address = reinterpret_cast<unsigned long long>(image);
+  const unsigned long long low = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(address)));
+  const unsigned long long high = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(address >> 32)));
+  _Float16* uniform_image = reinterpret_cast<_Float16*>((high << 32) | low);
+  const int bytes = __builtin_amdgcn_readfirstlane(static_cast<int>(g.image_bytes));
+  typedef __attribute__((address_space(3))) void* LdsPtr;
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(__builtin_amdgcn_make_buffer_rsrc(uniform_image, 0, bytes, kRawBufferFlags),
+                                           (LdsPtr)(destination), 16, offset_bytes, 0, 0, 0);
+}
+
 // Byte offset of a lane's 16 bytes from the first row of piece `piece`. KC: the piece is x rows
 // 16*piece..+15 of 32 halfs; XC: k rows (512/W)*piece.. of W halfs. The lane's LDS position is fixed
 // (16 * lane), the chunk it fetches carries the swizzle.
@@ -144,7 +178,8 @@ __device__ __forceinline__ half8_t HFragment(const _Float16* __restrict__ stage,
 }
 
 // ---- the kernel ------------------------------------------------------------------------------------
-template <typename Config, bool A_KC, bool B_KC>
+// A_CONV: the A operand is gathered from a batch of images (GemmArgs::conv, HGatherPiece); needs !A_KC.
+template <typename Config, bool A_KC, bool B_KC, bool A_CONV = false>
 __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirectKernel(const GemmArgs<float> p, const int tiles_m,
                                                                   const int tiles_n) {
   using T = _Float16;
@@ -152,7 +187,8 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
   constexpr int FM = Config::FM, FN = Config::FN, WAVES = Config::WAVES, STAGES = Config::STAGES, ROUNDS = Config::ROUNDS;
   constexpr int KSTEPS = TILE_K / 16;
   static_assert(KSTEPS == 2 && STAGES == 3, "schedule below: one barrier after the first of two k-steps, ring of three");
-  using KernelTag = std::tuple<Config, std::integral_constant<int, (A_KC ? 2 : 0) | (B_KC ? 1 : 0)>>;
+  static_assert(!A_CONV || !A_KC, "a gathered operand is x-contiguous in LDS");
+  using KernelTag = std::tuple<Config, std::integral_constant<int, (A_CONV ? 4 : 0) | (A_KC ? 2 : 0) | (B_KC ? 1 : 0)>>;
 
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
@@ -227,6 +263,8 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
       const long long b_step = B_KC ? static_cast<long long>(TILE_K) : TILE_K * p.b_ld;
       long long piece_start[ROUNDS];
       int piece_lane_bytes[ROUNDS], piece_place[ROUNDS];
+      int gather_row[A_CONV ? ROUNDS : 1];  // gathered A: the row of the slab a lane serves in a round
+      int request_k = 0;                    // first row of the slab to be requested next
 #pragma unroll
       for (int round = 0; round < ROUNDS; ++round) {
         const int piece = wave_u + WAVES * round;
@@ -234,6 +272,17 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
           piece_start[round] = static_cast<long long>((A_KC ? 16 : 512 / TILE_M) * piece) * p.a_ld;
           piece_lane_bytes[round] = HPieceLaneBytes<TILE_M, A_KC>(p.a_ld, piece, lane);
           piece_place[round] = piece * 512;
+          if constexpr (A_CONV) {
+            // the lane's row of the piece and its (swizzled) chunk of eight patches, as in HPieceLaneBytes; in place of
+            // the byte offset the offset of the first of these patches in the image plane, or -1 beyond m
+            constexpr int ROWS = 512 / TILE_M, CHUNKS = TILE_M / 8;
+            const int row = ROWS * piece + lane / CHUNKS;
+            const int chunk = (lane % CHUNKS) ^ HSwizzle<TILE_M>(row);
+            const int patch = m0 + 8 * chunk;
+            const int oh = patch / p.conv.output_w, ow = patch - oh * p.conv.output_w;
+            gather_row[round] = row;
+            piece_lane_bytes[round] = (patch < p.m) ? oh * p.conv.stride_h * p.conv.width + ow : -1;
+          }
         } else {
           const int b_piece = piece - Config::PIECES_A;
           piece_start[round] = static_cast<long long>((B_KC ? 16 : 512 / TILE_N) * b_piece) * p.b_ld;
@@ -250,8 +299,13 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
       auto request = [&](const int round, const int buffer) {
         const int piece = wave_u + WAVES * round;
         if (is_a(round, piece)) {
-          HRequestPiece<RANGE, KernelTag>(a_request + piece_start[round], a_end,
-                                          a_ring + buffer * Config::A_ELEMS + piece_place[round], piece_lane_bytes[round]);
+          if constexpr (A_CONV) {
+            HGatherPiece<KernelTag>(a, p.conv, a_ring + buffer * Config::A_ELEMS + piece_place[round],
+                                    request_k + gather_row[round], k_len, piece_lane_bytes[round]);
+          } else {
+            HRequestPiece<RANGE, KernelTag>(a_request + piece_start[round], a_end,
+                                            a_ring + buffer * Config::A_ELEMS + piece_place[round], piece_lane_bytes[round]);
+          }
         } else if (!Config::DUMMY || piece < Config::PIECES_A + Config::PIECES_B) {
           HRequestPiece<RANGE, KernelTag>(b_request + piece_start[round], b_end,
                                           b_ring + buffer * Config::B_ELEMS + piece_place[round], piece_lane_bytes[round]);
@@ -263,7 +317,7 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
                                                    (LdsPtr)(scratch_piece), 16, lane * 16, 0, 0, 0);
         }
       };
-      auto next_request_slab = [&]() { a_request += a_step; b_request += b_step; };
+      auto next_request_slab = [&]() { a_request += a_step; b_request += b_step; request_k += TILE_K; };
       // zeroes the K tail of the k-contiguous pieces this wavefront requested for the slab in `buffer`
       auto zero_tail = [&](const int buffer) {
         if (!RANGE || k_tail == 0 || !(A_KC || B_KC)) { return; }

@@ -65,21 +65,53 @@ __global__ __launch_bounds__(kIm2colThreads) void Im2colKernel(const Im2colShape
   }
 }
 
-// Copies `planes` image planes of height x width into planes of (height + 2 pad_h) x (width + 2 pad_w) with a border of
-// zeros, for the convolution kernels that want every patch element to exist. grid: (ceil(padded plane / 256),
-// min(planes, 65535)).
-template <typename T>
-__global__ __launch_bounds__(kIm2colThreads) void PadImageKernel(const int planes, const int height, const int width,
-                                                                 const int pad_h, const int pad_w,
-                                                                 const T* __restrict__ src, T* __restrict__ dst) {
-  const int padded_w = width + 2 * pad_w, padded_h = height + 2 * pad_h;
-  const int index = blockIdx.x * kIm2colThreads + threadIdx.x;
-  if (index >= padded_h * padded_w) { return; }
-  const int row = index / padded_w - pad_h, col = index % padded_w - pad_w;
-  const bool inside = (row >= 0 && row < height && col >= 0 && col < width);
-  for (int plane = blockIdx.y; plane < planes; plane += gridDim.y) {
-    dst[static_cast<long long>(plane) * padded_h * padded_w + index] =
-        inside ? src[(static_cast<long long>(plane) * height + row) * width + col] : T(0);
+// Copies `images` images of `channels` planes of height x width into planes of (height + 2 pad_h) x (width + 2 pad_w +
+// extra_w) with a border of zeros (extra_w more columns of zeros on the right), for the convolution kernels that want
+// every patch element to exist; image i of the result starts i * image_stride elements behind dst. With copy_stride
+// > 0 every image is written a second time, copy_stride elements behind its first copy and shifted by one element
+// (copy[j] = image[j + 1], a zero at the end): the fp16 gather fetches odd
+// element offsets from there (HGatherPiece).
+// A thread owns VEC consecutive elements of the padded image (all channels of an image form one array; VEC > 1 needs the
+// padded image size, image_stride and copy_stride to be multiples of VEC and 16-byte aligned dst) and writes them - and
+// the VEC elements one further on for the shifted copy - with one store each.
+// grid: (ceil(channels * padded plane / (256 * VEC)), min(images, 65535)).
+template <typename T, int VEC>
+__global__ __launch_bounds__(kIm2colThreads) void PadImageKernel(const int images, const int channels, const int height,
+                                                                 const int width, const int pad_h, const int pad_w,
+                                                                 const int extra_w, const T* __restrict__ src,
+                                                                 T* __restrict__ dst, const long long image_stride,
+                                                                 const long long copy_stride) {
+  typedef T Vector __attribute__((ext_vector_type(VEC)));
+  const int padded_w = width + 2 * pad_w + extra_w, padded_h = height + 2 * pad_h;
+  const int plane = padded_h * padded_w;
+  const long long total = static_cast<long long>(channels) * plane;
+  const long long first = (static_cast<long long>(blockIdx.x) * kIm2colThreads + threadIdx.x) * VEC;
+  if (first >= total) { return; }
+  // position of the first element; the following ones are reached by stepping
+  int channel = static_cast<int>(first / plane);
+  int row = static_cast<int>(first % plane) / padded_w, col = static_cast<int>(first % plane) % padded_w;
+  for (int image = blockIdx.y; image < images; image += gridDim.y) {
+    const T* source = src + static_cast<long long>(image) * channels * height * width;
+    T value[VEC + 1];
+    int c = channel, r = row, x = col;
+#pragma unroll
+    for (int v = 0; v <= VEC; ++v) {
+      const int in_row = r - pad_h, in_col = x - pad_w;
+      const bool inside = (c < channels && in_row >= 0 && in_row < height && in_col >= 0 && in_col < width);
+      value[v] = inside ? source[(static_cast<long long>(c) * height + in_row) * width + in_col] : T(0);
+      if (++x == padded_w) { x = 0; if (++r == padded_h) { r = 0; ++c; } }
+    }
+    T* target = dst + image * image_stride + first;
+    if constexpr (VEC == 1) {
+      target[0] = value[0];
+      if (copy_stride > 0) { target[copy_stride] = value[1]; }
+    } else {
+      Vector out, shifted;
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) { out[v] = value[v]; shifted[v] = value[v + 1]; }
+      *reinterpret_cast<Vector*>(target) = out;
+      if (copy_stride > 0) { *reinterpret_cast<Vector*>(target + copy_stride) = shifted; }
+    }
   }
 }
 

@@ -77,39 +77,55 @@ void Xconvgemm<T>::DoConvgemm(const KernelMode kernel_mode, const size_t channel
   shape.flip = (kernel_mode == KernelMode::kConvolution) ? 1 : 0;
 
   // The reference's single-kernel method (xconvgemm.cpp:121-160, doc/details_conv.md): no im2col matrix; the GEMM kernel
-  // gathers the patches from the images while it loads its tiles. fp32, all batches in one launch.
-  if (clbh_conv_gather_possible(precision, &shape) != 0) {
-    // With unit stride along the width and whole groups of four patches per output row the kernel fetches four patches
-    // per lane - if no patch element lies in the padding: then the images are copied into a zero border first (one
-    // pass over the images instead of a nine times larger im2col matrix), and the kernel sees images without padding.
+  // gathers the patches from the images while it loads its tiles. fp32 and (with restrictions) fp16, all batches in one
+  // launch.
+  // Both element types: images whose patches never reach into padding are what the gathering kernels take without
+  // (fp32) or only with (fp16) restrictions; an image with padding is first copied into a border of zeros - one pass
+  // over the images instead of a nine times larger im2col matrix.
+  auto padded_shape = shape;
+  const auto extra_w = (precision == 16) ? (width + 2 * pad_w) % 2 : size_t{0};  // fp16 wants an even image width
+  padded_shape.height = static_cast<int>(height + 2 * pad_h);
+  padded_shape.width = static_cast<int>(width + 2 * pad_w + extra_w);
+  padded_shape.pad_h = 0;
+  padded_shape.pad_w = 0;
+  const auto padded_elements = channels * (height + 2 * pad_h) * (width + 2 * pad_w + extra_w);
+  const bool needs_copy = (pad_h > 0 || pad_w > 0 || extra_w > 0);
+  // fp16: the kernel matrix must be fetched in dwords as well
+  const bool half_kernels_aligned =
+      (reinterpret_cast<unsigned long long>(kernel_buffer()) + 2 * kernel_offset) % 4 == 0 && patch_size % 2 == 0;
+  const bool half_images_aligned = (reinterpret_cast<unsigned long long>(im_buffer()) + 2 * im_offset) % 4 == 0;
+  const bool vector_gather =  // four (fp32) or eight (fp16) patches per lane
+      stride_w == 1 && output_w % (precision == 16 ? 8 : 4) == 0 && batch_count * channels <= kLimit &&
+      clbh_conv_gather_possible(precision, &padded_shape) != 0 &&
+      (precision == 32 || (precision == 16 && half_kernels_aligned && (needs_copy || half_images_aligned)));
+  if (vector_gather || (precision == 32 && clbh_conv_gather_possible(precision, &shape) != 0)) {
     auto gather_shape = shape;
     const void* images = im_buffer();
     auto images_offset = static_cast<long long>(im_offset);
+    auto images_stride = static_cast<long long>(channels * height * width);
+    auto copy_stride = static_cast<long long>(0);
     std::unique_ptr<StreamScratch> padded;
-    if ((pad_h > 0 || pad_w > 0) && stride_w == 1 && output_w % 4 == 0) {
-      auto padded_shape = shape;
-      padded_shape.height = static_cast<int>(height + 2 * pad_h);
-      padded_shape.width = static_cast<int>(width + 2 * pad_w);
-      padded_shape.pad_h = 0;
-      padded_shape.pad_w = 0;
-      if (clbh_conv_gather_possible(precision, &padded_shape) != 0) {
-        const auto planes = batch_count * channels;
-        const auto padded_bytes = planes * (height + 2 * pad_h) * (width + 2 * pad_w) * sizeof(T);
-        if (planes <= kLimit) {
-          padded.reset(new StreamScratch(padded_bytes, this->stream(), "images with a border of zeros"));
-          CheckDevice(clbh_pad_image(precision, static_cast<int>(planes), shape.height, shape.width, shape.pad_h, shape.pad_w,
-                                     im_buffer(), images_offset, padded->get(), this->stream()),
-                      "clbh_pad_image");
-          gather_shape = padded_shape;
-          images = padded->get();
-          images_offset = 0;
-        }
-      }
+    if (vector_gather && (needs_copy || precision == 16)) {
+      // fp16 always copies: its kernel reads odd element offsets from a second copy of every image, shifted by one element
+      copy_stride = (precision == 16) ? static_cast<long long>((padded_elements + 7) / 8 * 8) : 0;
+      images_stride = (precision == 16) ? 2 * copy_stride : static_cast<long long>(padded_elements);
+      padded.reset(new StreamScratch(batch_count * static_cast<size_t>(images_stride) * sizeof(T), this->stream(),
+                                     "images with a border of zeros"));
+      CheckDevice(clbh_pad_image(precision, static_cast<int>(batch_count), shape.channels, shape.height, shape.width, shape.pad_h,
+                                 shape.pad_w, static_cast<int>(extra_w), im_buffer(), images_offset, padded->get(),
+                                 images_stride, copy_stride, this->stream()),
+                  "clbh_pad_image");
+      gather_shape = padded_shape;
+      images = padded->get();
+      images_offset = 0;
+    } else if (vector_gather) {
+      gather_shape = padded_shape;  // fp32 without padding: the images as they are
     }
     auto desc = clbh_gemm_desc{};
     desc.precision = precision;
     desc.kernel_class = CLBH_KERNEL_MFMA;
-    desc.tile_variant = 7;  // 64 x 64 x 16, the one tile the gathering kernel is built for
+    // fp32: 64 x 64 x 16, the one tile its gathering kernel is built for; fp16: 128 x 128, 64 x 64 for up to 64 kernels
+    desc.tile_variant = (precision == 16) ? (num_kernels <= 64 ? 1 : 0) : 7;
     desc.split_k = 1;
     desc.a_kcontig = 0;
     desc.b_kcontig = 1;
@@ -120,7 +136,7 @@ void Xconvgemm<T>::DoConvgemm(const KernelMode kernel_mode, const size_t channel
     desc.a = images;
     desc.a_offset = images_offset;
     desc.a_ld = static_cast<long long>(num_patches);  // of the patch matrix that is never stored
-    desc.a_stride = static_cast<long long>(channels) * gather_shape.height * gather_shape.width;
+    desc.a_stride = images_stride;
     desc.b = kernel_buffer();
     desc.b_offset = static_cast<long long>(kernel_offset);
     desc.b_ld = static_cast<long long>(patch_size);
@@ -132,6 +148,7 @@ void Xconvgemm<T>::DoConvgemm(const KernelMode kernel_mode, const size_t channel
     desc.alpha = 1.0;
     desc.beta = 0.0;
     desc.conv = &gather_shape;
+    desc.conv_copy_stride = copy_stride;
     CheckDevice(clbh_gemm_launch(&desc, this->stream()), "clbh_gemm_launch (gathered convolution)");
     this->Finish();
     return;

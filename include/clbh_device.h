@@ -76,8 +76,11 @@ typedef struct clbh_gemm_desc_ {
   // CONVGEMM without an im2col matrix (NULL for every other launch; see clbh_conv_gather_possible): `a` + a_offset holds
   // batch_count images, a_stride elements apart, and A(i,p) is element i of row p of the im2col matrix that clbh_im2col
   // would write for this shape, gathered from the image while the tiles are loaded. Needs m = output_h * output_w,
-  // k = channels * kernel_h * kernel_w, precision 32, the MFMA class (one tile: 64 x 64 x 16), b_kcontig, strided batches.
+  // k = channels * kernel_h * kernel_w, precision 32 or 16, the MFMA class, b_kcontig, strided batches. fp16: every
+  // image is followed, conv_copy_stride elements (even) behind its start, by a copy of itself shifted by one element
+  // (clbh_pad_image writes both), and a_offset and a_stride are even.
   const struct clbh_im2col_shape_* conv;
+  long long conv_copy_stride;
 } clbh_gemm_desc;
 
 // Enqueues the kernel(s) for one descriptor on `stream`. Returns 0 on success, otherwise the HIP
@@ -167,12 +170,18 @@ typedef struct clbh_im2col_shape_ {
 } clbh_im2col_shape;
 CLBH_API int clbh_im2col(int precision, const clbh_im2col_shape* shape, int batch_count, const void* image,
                          long long image_offset, void* col, hipStream_t stream);
-// dst = `planes` planes of (height + 2 pad_h) x (width + 2 pad_w): the planes of height x width at src + src_offset
-// inside a border of zeros.
-CLBH_API int clbh_pad_image(int precision, int planes, int height, int width, int pad_h, int pad_w, const void* src,
-                            long long src_offset, void* dst, hipStream_t stream);
-// Non-zero when a GEMM launch can gather its A operand from images of this shape itself (clbh_gemm_desc::conv): fp32
-// only, one image below 2 GiB, and row indices small enough for the kernel's division by multiplication.
+// Copies `images` images of `channels` planes of height x width (at src + src_offset) into planes of (height + 2 pad_h)
+// x (width + 2 pad_w + extra_w) inside a border of zeros, with extra_w more columns of zeros on the right; image i of
+// the result starts i * image_stride elements behind dst. copy_stride > 0: every image is written a second time,
+// copy_stride elements behind its first copy and shifted by one element (copy[j] = image[j + 1]), for the fp16 gather
+// of clbh_gemm_desc::conv.
+CLBH_API int clbh_pad_image(int precision, int images, int channels, int height, int width, int pad_h, int pad_w,
+                            int extra_w, const void* src, long long src_offset, void* dst, long long image_stride,
+                            long long copy_stride, hipStream_t stream);
+// Non-zero when a GEMM launch can gather its A operand from images of this shape itself (clbh_gemm_desc::conv): one
+// image below 2 GiB (1 GiB together with its second copy for fp16) and row indices small enough for the kernel's
+// division by multiplication; fp32 for any convolution, fp16 only without padding, with unit stride along the width,
+// an even image width and an output width that is a multiple of 8; not for fp64.
 CLBH_API int clbh_conv_gather_possible(int precision, const clbh_im2col_shape* shape);
 
 // Plain device memory and blocking copies for callers that hold host data (the Netlib-style façade): to_device != 0

@@ -27,6 +27,10 @@ CASES = [  # channels, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h
     (5, 12, 16, 3, 5, 1, 2, 2, 1, 1, 1, 7, 3),     # unit stride along the width, output width 16: four patches per lane (fp32)
     (3, 10, 20, 3, 3, 0, 2, 1, 1, 2, 2, 9, 2),     # the same with dilation, padding along the width only
     (6, 9, 12, 2, 1, 0, 0, 1, 1, 1, 1, 70, 2),     # no padding at all (no padded copy), kernel width 1, 70 kernels
+    (4, 10, 24, 3, 3, 1, 1, 1, 1, 1, 1, 10, 3),    # output width 24, even patch size: eight patches per lane in fp16
+    (6, 9, 15, 3, 2, 0, 1, 2, 1, 1, 1, 70, 2),     # odd padded width (one more column of zeros in fp16), output width 16
+    (2, 12, 24, 3, 3, 2, 2, 1, 1, 2, 2, 33, 2),    # dilation 2: even tap offsets only; (next) 130 kernels, two tile columns
+    (8, 6, 8, 3, 3, 1, 1, 1, 1, 1, 1, 130, 5),
 ]
 
 
