@@ -264,6 +264,48 @@ def symm(queue, m, n, a, b, c, a_ld, b_ld, c_ld, alpha=1.0, beta=0.0, right_side
         raise CLBlastError("CLBlast%ssymm" % prefix, status)
 
 
+def hemm(queue, m, n, a, b, c, a_ld, b_ld, c_ld, alpha=1.0, beta=0.0, right_side=False, lower_triangle=False, a_offset=0,
+         b_offset=0, c_offset=0):
+    """xHEMM: Hermitian matrix-matrix multiplication (row-major, like pyclblast.hemm; pyclblast.pyx:1984-2019); complex
+    tensors only."""
+    prefix = _tensor_info(a, b, c)
+    if prefix not in "CZ":
+        raise ValueError("PyCLBlast: Unrecognized data-type '%s'" % a.dtype)
+    status = raw_complex_level3("hemm", prefix, ROW_MAJOR, SIDE_RIGHT if right_side else SIDE_LEFT,
+                                TRIANGLE_LOWER if lower_triangle else TRIANGLE_UPPER, m, n, alpha, a.data_ptr(), a_offset, a_ld,
+                                b.data_ptr(), b_offset, b_ld, beta, c.data_ptr(), c_offset, c_ld,
+                                stream_handle=_stream_handle(queue))
+    if status != 0:
+        raise CLBlastError("CLBlast%shemm" % prefix, status)
+
+
+def herk(queue, n, k, a, c, a_ld, c_ld, alpha=1.0, beta=0.0, lower_triangle=False, a_transp=False, a_offset=0, c_offset=0):
+    """xHERK: Rank-K update of a hermitian matrix (row-major, like pyclblast.herk; pyclblast.pyx:2069-2102): real alpha
+    and beta, a_transp means the conjugate transpose."""
+    prefix = _tensor_info(a, c)
+    if prefix not in "CZ":
+        raise ValueError("PyCLBlast: Unrecognized data-type '%s'" % a.dtype)
+    status = raw_complex_level3("herk", prefix, ROW_MAJOR, TRIANGLE_LOWER if lower_triangle else TRIANGLE_UPPER,
+                                TRANS_CONJ if a_transp else TRANS_NO, n, k, float(alpha), a.data_ptr(), a_offset, a_ld,
+                                float(beta), c.data_ptr(), c_offset, c_ld, stream_handle=_stream_handle(queue))
+    if status != 0:
+        raise CLBlastError("CLBlast%sherk" % prefix, status)
+
+
+def her2k(queue, n, k, a, b, c, a_ld, b_ld, c_ld, alpha=1.0, beta=0.0, lower_triangle=False, ab_transp=False, a_offset=0,
+          b_offset=0, c_offset=0):
+    """xHER2K: Rank-2K update of a hermitian matrix (row-major, like pyclblast.her2k; pyclblast.pyx:2154-2189): complex
+    alpha, real beta, ab_transp means the conjugate transpose."""
+    prefix = _tensor_info(a, b, c)
+    if prefix not in "CZ":
+        raise ValueError("PyCLBlast: Unrecognized data-type '%s'" % a.dtype)
+    status = raw_complex_level3("her2k", prefix, ROW_MAJOR, TRIANGLE_LOWER if lower_triangle else TRIANGLE_UPPER,
+                                TRANS_CONJ if ab_transp else TRANS_NO, n, k, alpha, a.data_ptr(), a_offset, a_ld, b.data_ptr(),
+                                b_offset, b_ld, float(beta), c.data_ptr(), c_offset, c_ld, stream_handle=_stream_handle(queue))
+    if status != 0:
+        raise CLBlastError("CLBlast%sher2k" % prefix, status)
+
+
 def syrk(queue, n, k, a, c, a_ld, c_ld, alpha=1.0, beta=0.0, lower_triangle=False, a_transp=False, a_offset=0, c_offset=0):
     """xSYRK: Rank-K update of a symmetric matrix (row-major, like pyclblast.syrk; pyclblast.pyx:2026-2060)."""
     prefix = _tensor_info(a, c)
