@@ -122,7 +122,8 @@ C_API_SYMBOLS = (
     ["CLBlast%sconvgemm" % p for p in "SDH"] +
     ["CLBlastClearCache", "CLBlastOverrideParameters", "CLBlastFloatToHalf", "CLBlastHalfToFloat"])
 NETLIB_SYMBOLS = (["cblas_%sgemm" % p for p in "sdcz"] +
-                  ["cblas_%s%s" % (p, r) for p in "sd" for r in ("symm", "syrk", "syr2k", "trmm", "trsm")])
+                  ["cblas_%s%s" % (p, r) for p in "sdcz" for r in ("symm", "syrk", "syr2k", "trmm", "trsm")] +
+                  ["cblas_%s%s" % (p, r) for p in "cz" for r in ("hemm", "herk", "her2k")])
 DEVICE_LAYER_SYMBOLS = [
     "clbh_gemm_launch", "clbh_gemm_workspace_bytes", "clbh_buffer_extent", "clbh_alloc_async", "clbh_free_async",
     "clbh_upload_async", "clbh_event_record", "clbh_stream_device", "clbh_error_string", "clbh_symmetric_to_square",

@@ -60,6 +60,14 @@ clblast::Triangle Tri(const CLBlastTriangle v) { return static_cast<clblast::Tri
 clblast::Side Sd(const CLBlastSide v) { return static_cast<clblast::Side>(v); }
 clblast::Diagonal Dg(const CLBlastDiagonal v) { return static_cast<clblast::Diagonal>(v); }
 
+// HEMM exists for the complex types only; the real instantiations of SymmOnHost never ask for it
+template <typename T> struct IsComplex { static constexpr bool value = false; };
+template <typename R> struct IsComplex<std::complex<R>> { static constexpr bool value = true; };
+template <typename T>
+auto HemmRoutine() -> decltype(&clblast::Symm<T>) {
+  if constexpr (IsComplex<T>::value) { return clblast::Hemm<T>; } else { return clblast::Symm<T>; }
+}
+
 // T: element type of the buffers, S: scalar type of the routine (the same, or std::complex for void* data)
 template <typename T>
 void GemmOnHost(const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose,
@@ -75,24 +83,26 @@ void GemmOnHost(const CLBlastLayout layout, const CLBlastTranspose a_transpose, 
   c_buffer.Read(c);
 }
 
+// hermitian: HEMM instead of SYMM (complex T only)
 template <typename T>
-void SymmOnHost(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle, const int m,
-                const int n, const T alpha, const T* a, const int a_ld, const T* b, const int b_ld, const T beta, T* c,
-                const int c_ld) {
+void SymmOnHost(const bool hermitian, const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,
+                const int m, const int n, const T alpha, const void* a, const int a_ld, const void* b, const int b_ld,
+                const T beta, void* c, const int c_ld) {
   const auto lines = (layout == CLBlastLayoutRowMajor) ? m : n;
   const DeviceCopy<T> a_buffer(a, Count(side == CLBlastSideLeft ? m : n, a_ld));
   const DeviceCopy<T> b_buffer(b, Count(lines, b_ld));
   const DeviceCopy<T> c_buffer(c, Count(lines, c_ld));
   hipStream_t stream = nullptr;
-  Check(clblast::Symm<T>(L(layout), Sd(side), Tri(triangle), Dim(m), Dim(n), alpha, a_buffer.get(), 0, Dim(a_ld),
-                         b_buffer.get(), 0, Dim(b_ld), beta, c_buffer.get(), 0, Dim(c_ld), &stream));
+  const auto routine = hermitian ? HemmRoutine<T>() : clblast::Symm<T>;
+  Check(routine(L(layout), Sd(side), Tri(triangle), Dim(m), Dim(n), alpha, a_buffer.get(), 0, Dim(a_ld), b_buffer.get(), 0,
+                Dim(b_ld), beta, c_buffer.get(), 0, Dim(c_ld), &stream, nullptr));
   c_buffer.Read(c);
 }
 
 template <typename T>
 void Syr2kOnHost(const bool two_sided, const CLBlastLayout layout, const CLBlastTriangle triangle,
-                 const CLBlastTranspose transpose, const int n, const int k, const T alpha, const T* a, const int a_ld,
-                 const T* b, const int b_ld, const T beta, T* c, const int c_ld) {
+                 const CLBlastTranspose transpose, const int n, const int k, const T alpha, const void* a, const int a_ld,
+                 const void* b, const int b_ld, const T beta, void* c, const int c_ld) {
   const auto lines = Rotated(layout, transpose) ? n : k;
   const DeviceCopy<T> a_buffer(a, Count(lines, a_ld));
   const DeviceCopy<T> c_buffer(c, Count(n, c_ld));
@@ -112,7 +122,7 @@ void Syr2kOnHost(const bool two_sided, const CLBlastLayout layout, const CLBlast
 template <typename T>
 void TriangularOnHost(const bool solve, const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,
                       const CLBlastTranspose a_transpose, const CLBlastDiagonal diagonal, const int m, const int n,
-                      const T alpha, const T* a, const int a_ld, T* b, const int b_ld) {
+                      const T alpha, const void* a, const int a_ld, void* b, const int b_ld) {
   const DeviceCopy<T> a_buffer(a, Count(side == CLBlastSideLeft ? m : n, a_ld));
   const DeviceCopy<T> b_buffer(b, Count(layout == CLBlastLayoutRowMajor ? m : n, b_ld));
   hipStream_t stream = nullptr;
@@ -120,6 +130,28 @@ void TriangularOnHost(const bool solve, const CLBlastLayout layout, const CLBlas
   Check(routine(L(layout), Sd(side), Tri(triangle), Tr(a_transpose), Dg(diagonal), Dim(m), Dim(n), alpha, a_buffer.get(), 0,
                 Dim(a_ld), b_buffer.get(), 0, Dim(b_ld), &stream, nullptr));
   b_buffer.Read(b);
+}
+
+// HERK (b == nullptr; alpha real) and HER2K (alpha complex); beta is real in both
+template <typename R>
+void HerkOnHost(const CLBlastLayout layout, const CLBlastTriangle triangle, const CLBlastTranspose transpose, const int n,
+                const int k, const std::complex<R> alpha, const void* a, const int a_ld, const void* b, const int b_ld,
+                const R beta, void* c, const int c_ld) {
+  using T = std::complex<R>;
+  const auto lines = Rotated(layout, transpose) ? n : k;
+  const DeviceCopy<T> a_buffer(a, Count(lines, a_ld));
+  const DeviceCopy<T> c_buffer(c, Count(n, c_ld));
+  hipStream_t stream = nullptr;
+  if (b != nullptr) {
+    const DeviceCopy<T> b_buffer(b, Count(lines, b_ld));
+    Check(clblast::Her2k<T, R>(L(layout), Tri(triangle), Tr(transpose), Dim(n), Dim(k), alpha, a_buffer.get(), 0, Dim(a_ld),
+                               b_buffer.get(), 0, Dim(b_ld), beta, c_buffer.get(), 0, Dim(c_ld), &stream));
+    c_buffer.Read(c);  // before b_buffer goes away: the copy waits for the routine
+  } else {
+    Check(clblast::Herk<R>(L(layout), Tri(triangle), Tr(transpose), Dim(n), Dim(k), alpha.real(), a_buffer.get(), 0, Dim(a_ld),
+                           beta, c_buffer.get(), 0, Dim(c_ld), &stream));
+    c_buffer.Read(c);
+  }
 }
 
 template <typename R>
@@ -157,12 +189,12 @@ void cblas_zgemm(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
 void cblas_ssymm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle, const int m,
                  const int n, const float alpha, const float* a, const int a_ld, const float* b, const int b_ld,
                  const float beta, float* c, const int c_ld) {
-  SymmOnHost<float>(layout, side, triangle, m, n, alpha, a, a_ld, b, b_ld, beta, c, c_ld);
+  SymmOnHost<float>(false, layout, side, triangle, m, n, alpha, a, a_ld, b, b_ld, beta, c, c_ld);
 }
 void cblas_dsymm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle, const int m,
                  const int n, const double alpha, const double* a, const int a_ld, const double* b, const int b_ld,
                  const double beta, double* c, const int c_ld) {
-  SymmOnHost<double>(layout, side, triangle, m, n, alpha, a, a_ld, b, b_ld, beta, c, c_ld);
+  SymmOnHost<double>(false, layout, side, triangle, m, n, alpha, a, a_ld, b, b_ld, beta, c, c_ld);
 }
 
 void cblas_ssyrk(const CLBlastLayout layout, const CLBlastTriangle triangle, const CLBlastTranspose a_transpose,
@@ -206,5 +238,57 @@ void cblas_dtrsm(const CLBlastLayout layout, const CLBlastSide side, const CLBla
                  const double alpha, const double* a, const int a_ld, double* b, const int b_ld) {
   TriangularOnHost<double>(true, layout, side, triangle, a_transpose, diagonal, m, n, alpha, a, a_ld, b, b_ld);
 }
+
+// ---- the complex Level-3 routines (reference: include/clblast_netlib_c.h:427-515) -----------------------
+#define CLBH_NETLIB_COMPLEX(P, R)                                                                                       \
+  void cblas_##P##symm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle, const int m, \
+                       const int n, const void* alpha, const void* a, const int a_ld, const void* b, const int b_ld,    \
+                       const void* beta, void* c, const int c_ld) {                                                     \
+    SymmOnHost<std::complex<R>>(false, layout, side, triangle, m, n, Scalar<R>(alpha), a, a_ld, b, b_ld, Scalar<R>(beta), \
+                                c, c_ld);                                                                               \
+  }                                                                                                                     \
+  void cblas_##P##hemm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle, const int m, \
+                       const int n, const void* alpha, const void* a, const int a_ld, const void* b, const int b_ld,    \
+                       const void* beta, void* c, const int c_ld) {                                                     \
+    SymmOnHost<std::complex<R>>(true, layout, side, triangle, m, n, Scalar<R>(alpha), a, a_ld, b, b_ld, Scalar<R>(beta), \
+                                c, c_ld);                                                                               \
+  }                                                                                                                     \
+  void cblas_##P##syrk(const CLBlastLayout layout, const CLBlastTriangle triangle, const CLBlastTranspose a_transpose,  \
+                       const int n, const int k, const void* alpha, const void* a, const int a_ld, const void* beta,    \
+                       void* c, const int c_ld) {                                                                       \
+    Syr2kOnHost<std::complex<R>>(false, layout, triangle, a_transpose, n, k, Scalar<R>(alpha), a, a_ld, nullptr, 0,     \
+                                 Scalar<R>(beta), c, c_ld);                                                             \
+  }                                                                                                                     \
+  void cblas_##P##syr2k(const CLBlastLayout layout, const CLBlastTriangle triangle, const CLBlastTranspose ab_transpose, \
+                        const int n, const int k, const void* alpha, const void* a, const int a_ld, const void* b,      \
+                        const int b_ld, const void* beta, void* c, const int c_ld) {                                    \
+    Syr2kOnHost<std::complex<R>>(true, layout, triangle, ab_transpose, n, k, Scalar<R>(alpha), a, a_ld, b, b_ld,        \
+                                 Scalar<R>(beta), c, c_ld);                                                             \
+  }                                                                                                                     \
+  void cblas_##P##herk(const CLBlastLayout layout, const CLBlastTriangle triangle, const CLBlastTranspose a_transpose,  \
+                       const int n, const int k, const R alpha, const void* a, const int a_ld, const R beta, void* c,   \
+                       const int c_ld) {                                                                                \
+    HerkOnHost<R>(layout, triangle, a_transpose, n, k, std::complex<R>(alpha, R(0)), a, a_ld, nullptr, 0, beta, c, c_ld); \
+  }                                                                                                                     \
+  void cblas_##P##her2k(const CLBlastLayout layout, const CLBlastTriangle triangle, const CLBlastTranspose ab_transpose, \
+                        const int n, const int k, const void* alpha, const void* a, const int a_ld, const void* b,      \
+                        const int b_ld, const R beta, void* c, const int c_ld) {                                        \
+    HerkOnHost<R>(layout, triangle, ab_transpose, n, k, Scalar<R>(alpha), a, a_ld, b, b_ld, beta, c, c_ld);             \
+  }                                                                                                                     \
+  void cblas_##P##trmm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,              \
+                       const CLBlastTranspose a_transpose, const CLBlastDiagonal diagonal, const int m, const int n,    \
+                       const void* alpha, const void* a, const int a_ld, void* b, const int b_ld) {                     \
+    TriangularOnHost<std::complex<R>>(false, layout, side, triangle, a_transpose, diagonal, m, n, Scalar<R>(alpha), a,  \
+                                      a_ld, b, b_ld);                                                                   \
+  }                                                                                                                     \
+  void cblas_##P##trsm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,              \
+                       const CLBlastTranspose a_transpose, const CLBlastDiagonal diagonal, const int m, const int n,    \
+                       const void* alpha, const void* a, const int a_ld, void* b, const int b_ld) {                     \
+    TriangularOnHost<std::complex<R>>(true, layout, side, triangle, a_transpose, diagonal, m, n, Scalar<R>(alpha), a,   \
+                                      a_ld, b, b_ld);                                                                   \
+  }
+CLBH_NETLIB_COMPLEX(c, float)
+CLBH_NETLIB_COMPLEX(z, double)
+#undef CLBH_NETLIB_COMPLEX
 
 }  // extern "C"

@@ -88,6 +88,65 @@ void CLBLAST_HIP_API cblas_dtrsm(const CLBlastLayout layout, const CLBlastSide s
                                  const int n, const double alpha, const double* a, const int a_ld, double* b,
                                  const int b_ld);
 
+// The same routines on interleaved complex data (scalars by pointer to (re, im); HERK takes real alpha and beta, HER2K
+// a real beta), and the Hermitian ones (reference: :427-440, :449-462, :473-490, :499-515)
+void CLBLAST_HIP_API cblas_csymm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,
+                                 const int m, const int n, const void* alpha, const void* a, const int a_ld,
+                                 const void* b, const int b_ld, const void* beta, void* c, const int c_ld);
+void CLBLAST_HIP_API cblas_chemm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,
+                                 const int m, const int n, const void* alpha, const void* a, const int a_ld,
+                                 const void* b, const int b_ld, const void* beta, void* c, const int c_ld);
+void CLBLAST_HIP_API cblas_csyrk(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                 const CLBlastTranspose a_transpose, const int n, const int k, const void* alpha,
+                                 const void* a, const int a_ld, const void* beta, void* c, const int c_ld);
+void CLBLAST_HIP_API cblas_cherk(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                 const CLBlastTranspose a_transpose, const int n, const int k, const float alpha,
+                                 const void* a, const int a_ld, const float beta, void* c, const int c_ld);
+void CLBLAST_HIP_API cblas_csyr2k(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                  const CLBlastTranspose ab_transpose, const int n, const int k, const void* alpha,
+                                  const void* a, const int a_ld, const void* b, const int b_ld, const void* beta,
+                                  void* c, const int c_ld);
+void CLBLAST_HIP_API cblas_cher2k(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                  const CLBlastTranspose ab_transpose, const int n, const int k, const void* alpha,
+                                  const void* a, const int a_ld, const void* b, const int b_ld, const float beta,
+                                  void* c, const int c_ld);
+void CLBLAST_HIP_API cblas_ctrmm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,
+                                 const CLBlastTranspose a_transpose, const CLBlastDiagonal diagonal, const int m,
+                                 const int n, const void* alpha, const void* a, const int a_ld, void* b,
+                                 const int b_ld);
+void CLBLAST_HIP_API cblas_ctrsm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,
+                                 const CLBlastTranspose a_transpose, const CLBlastDiagonal diagonal, const int m,
+                                 const int n, const void* alpha, const void* a, const int a_ld, void* b,
+                                 const int b_ld);
+void CLBLAST_HIP_API cblas_zsymm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,
+                                 const int m, const int n, const void* alpha, const void* a, const int a_ld,
+                                 const void* b, const int b_ld, const void* beta, void* c, const int c_ld);
+void CLBLAST_HIP_API cblas_zhemm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,
+                                 const int m, const int n, const void* alpha, const void* a, const int a_ld,
+                                 const void* b, const int b_ld, const void* beta, void* c, const int c_ld);
+void CLBLAST_HIP_API cblas_zsyrk(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                 const CLBlastTranspose a_transpose, const int n, const int k, const void* alpha,
+                                 const void* a, const int a_ld, const void* beta, void* c, const int c_ld);
+void CLBLAST_HIP_API cblas_zherk(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                 const CLBlastTranspose a_transpose, const int n, const int k, const double alpha,
+                                 const void* a, const int a_ld, const double beta, void* c, const int c_ld);
+void CLBLAST_HIP_API cblas_zsyr2k(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                  const CLBlastTranspose ab_transpose, const int n, const int k, const void* alpha,
+                                  const void* a, const int a_ld, const void* b, const int b_ld, const void* beta,
+                                  void* c, const int c_ld);
+void CLBLAST_HIP_API cblas_zher2k(const CLBlastLayout layout, const CLBlastTriangle triangle,
+                                  const CLBlastTranspose ab_transpose, const int n, const int k, const void* alpha,
+                                  const void* a, const int a_ld, const void* b, const int b_ld, const double beta,
+                                  void* c, const int c_ld);
+void CLBLAST_HIP_API cblas_ztrmm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,
+                                 const CLBlastTranspose a_transpose, const CLBlastDiagonal diagonal, const int m,
+                                 const int n, const void* alpha, const void* a, const int a_ld, void* b,
+                                 const int b_ld);
+void CLBLAST_HIP_API cblas_ztrsm(const CLBlastLayout layout, const CLBlastSide side, const CLBlastTriangle triangle,
+                                 const CLBlastTranspose a_transpose, const CLBlastDiagonal diagonal, const int m,
+                                 const int n, const void* alpha, const void* a, const int a_ld, void* b,
+                                 const int b_ld);
+
 #ifdef __cplusplus
 }  // extern "C"
 #endif

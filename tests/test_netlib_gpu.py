@@ -1,4 +1,4 @@
-"""The Netlib-style façade on host pointers (cblas_sgemm ... cblas_dtrsm in include/clblast_hip_netlib_c.h; reference:
+"""The Netlib-style façade on host pointers (cblas_sgemm ... cblas_ztrsm in include/clblast_hip_netlib_c.h; reference:
 include/clblast_netlib_c.h:402-515, src/clblast_netlib_c.cpp:2718-3500) against the CPU oracle: numpy buffers in,
 result in the same numpy buffer, nothing outside the logical result changed."""
 import itertools
@@ -8,7 +8,7 @@ import pytest
 
 import oracle
 from clblast_amd import netlib
-from oracle import COL_MAJOR, CONJ, LEFT, LOWER, NO, NON_UNIT, RIGHT, ROW_MAJOR, UNIT, UPPER, YES
+from oracle import COL_MAJOR, CONJ, LEFT, LOWER, NO, NON_UNIT, RIGHT, ROW_MAJOR, UNIT, UPPER, YES, complex_level3
 
 pytestmark = pytest.mark.gpu
 
@@ -100,3 +100,74 @@ def test_level3_on_host_pointers(gpu, dtype):
         expected = oracle.syr2k(layout, triangle, transpose, n, k, 0.5, a, 0, a_ld, b, 0, b_ld, 2.0, c_in, 0, c_ld)
         netlib.syr2k(layout, triangle, transpose, n, k, 0.5, a, a_ld, b, b_ld, 2.0, c_in, c_ld)
         assert relative_error(c_in[where], expected) <= TOL[dtype], ("syr2k", layout, triangle, transpose)
+
+
+@pytest.mark.parametrize("dtype", (np.complex64, np.complex128))
+def test_complex_level3_on_host_pointers(gpu, dtype):
+    """cblas_{c,z}{symm,hemm,syrk,herk,syr2k,her2k,trmm,trsm} against the numpy restatement of the complex routines."""
+    dtype = np.dtype(dtype)
+    bits = 32 if dtype == np.complex64 else 64
+    alpha, beta = 0.5 - 1.5j, 2.0 + 0.25j
+    seed = 18000
+    for layout, side, triangle in itertools.product((ROW_MAJOR, COL_MAJOR), (LEFT, RIGHT), (UPPER, LOWER)):
+        seed += 1
+        m, n = ((33, 17), (64, 64), (20, 130))[seed % 3]
+        k = m if side == LEFT else n
+        one, two = (n, m) if layout == ROW_MAJOR else (m, n)
+        a_ld, b_ld, c_ld = k + 1, one + 2, one + 3
+        a = oracle.complex_uniform(seed * 3, k * a_ld, -1.0, 1.0, bits)
+        b = oracle.complex_uniform(seed * 3 + 1, two * b_ld, -1.0, 1.0, bits)
+        c = oracle.complex_uniform(seed * 3 + 2, two * c_ld, -1.0, 1.0, bits)
+        where = oracle.c_indices(layout, m, n, 0, c_ld)
+        for hermitian in (False, True):
+            c_in = c.copy()
+            expected = complex_level3.symm(hermitian, layout, side, triangle, m, n, alpha, a, 0, a_ld, b, 0, b_ld, beta, c_in, 0,
+                                           c_ld)
+            (netlib.hemm if hermitian else netlib.symm)(layout, side, triangle, m, n, alpha, a, a_ld, b, b_ld, beta, c_in, c_ld)
+            assert relative_error(c_in[where], expected) <= TOL[dtype], ("symm", hermitian, layout, side, triangle)
+            untouched = np.ones(c.size, dtype=bool)
+            untouched[where.ravel()] = False
+            assert np.array_equal(c_in[untouched].view(np.uint8), c[untouched].view(np.uint8))
+        where_b = oracle.c_indices(layout, m, n, 0, b_ld)
+        a_solve = (a.astype(np.complex128) * (2.0 / k)).astype(dtype)
+        positions = np.arange(k) * (a_ld + 1)
+        a_solve[positions] = a_solve[positions] + np.where(a_solve[positions].real >= 0, 4.0, -4.0).astype(dtype)
+        for transpose, diagonal in ((NO, NON_UNIT), (YES, UNIT), (CONJ, NON_UNIT)):
+            b_in = b.copy()
+            expected = complex_level3.trmm(layout, side, triangle, transpose, diagonal, m, n, alpha, a, 0, a_ld, b_in, 0, b_ld)
+            netlib.trmm(layout, side, triangle, transpose, diagonal, m, n, alpha, a, a_ld, b_in, b_ld)
+            assert relative_error(b_in[where_b], expected) <= TOL[dtype], ("trmm", layout, side, triangle, transpose)
+            b_in = b.copy()
+            expected = complex_level3.trsm(layout, side, triangle, transpose, diagonal, m, n, alpha, a_solve, 0, a_ld, b_in, 0,
+                                           b_ld)
+            netlib.trsm(layout, side, triangle, transpose, diagonal, m, n, alpha, a_solve, a_ld, b_in, b_ld)
+            assert relative_error(b_in[where_b], expected) <= 2 * TOL[dtype], ("trsm", layout, side, triangle, transpose)
+    for layout, triangle, transpose in itertools.product((ROW_MAJOR, COL_MAJOR), (UPPER, LOWER), (NO, YES)):
+        seed += 1
+        n, k = ((33, 17), (64, 64), (20, 130))[seed % 3]
+        i, j = np.arange(n)[:, None], np.arange(n)[None, :]
+        inside = (i <= j) if triangle == UPPER else (i >= j)
+        where = oracle.c_indices(layout, n, n, 0, n + 3)
+        for hermitian, two_sided in itertools.product((False, True), (False, True)):
+            # the Hermitian routines take "conjugate transpose" where the symmetric ones take "transpose"
+            trans = CONJ if (hermitian and transpose == YES) else transpose
+            rows, cols = (n, k) if transpose == NO else (k, n)
+            one, two = (cols, rows) if layout == ROW_MAJOR else (rows, cols)
+            a_ld, b_ld, c_ld = one + 1, one + 2, n + 3
+            a = oracle.complex_uniform(seed * 3, two * a_ld, -1.0, 1.0, bits)
+            b = oracle.complex_uniform(seed * 3 + 1, two * b_ld, -1.0, 1.0, bits)
+            c = oracle.complex_uniform(seed * 3 + 2, n * c_ld, -1.0, 1.0, bits)
+            c_in = c.copy()
+            # HERK takes real alpha and beta, HER2K a real beta
+            alpha_used = alpha.real if (hermitian and not two_sided) else alpha
+            beta_used = beta.real if hermitian else beta
+            expected = complex_level3.rank_update(hermitian, layout, triangle, trans, n, k, alpha_used, a, 0, a_ld,
+                                                  b if two_sided else None, 0, b_ld, beta_used, c_in, 0, c_ld)
+            if two_sided:
+                (netlib.her2k if hermitian else netlib.syr2k)(layout, triangle, trans, n, k, alpha_used, a, a_ld, b, b_ld, beta_used,
+                                                              c_in, c_ld)
+            else:
+                (netlib.herk if hermitian else netlib.syrk)(layout, triangle, trans, n, k, alpha_used, a, a_ld, beta_used, c_in, c_ld)
+            label = ("rank update", hermitian, two_sided, layout, triangle, trans)
+            assert relative_error(c_in[where][inside], expected[inside]) <= TOL[dtype], label
+            assert np.array_equal(c_in[where][~inside].view(np.uint8), c[where][~inside].view(np.uint8)), label
