@@ -389,6 +389,16 @@ int clbh_complex_scale(int precision, int m, int n, int triangle, double beta_re
   return clbh_complex_scale_batched(precision, m, n, triangle, beta_re, beta_im, c, c_offset, c_ld, nullptr, stream);
 }
 
+int clbh_complex_gemm_small_batched(const clbh_complex_small_desc* desc, hipStream_t stream) {
+  if (desc == nullptr) { return hipErrorInvalidValue; }
+  for (const auto* operand : {&desc->left, &desc->right, &desc->c}) {
+    if (operand->offset < 0 || operand->ld < 1 || (operand->offsets == nullptr && operand->stride < 0)) {
+      return hipErrorInvalidValue;
+    }
+  }
+  return clbh::LaunchComplexSmall(*desc, stream);
+}
+
 int clbh_pad_image(int precision, int images, int channels, int height, int width, int pad_h, int pad_w, int extra_w,
                    const void* src, long long src_offset, void* dst, long long image_stride, long long copy_stride,
                    hipStream_t stream) {

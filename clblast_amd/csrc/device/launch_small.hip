@@ -2,6 +2,7 @@
 // Small-matrix batched kernel instantiations (fp32, fp64, fp16).
 // =================================================================================================
 #include "device/launch_common.hpp"
+#include "kernels/gemm_complex_small.hpp"
 #include "kernels/gemm_small_batched.hpp"
 
 namespace clbh {
@@ -35,7 +36,71 @@ int LaunchSmallBatchedTyped(const clbh_gemm_desc& d, hipStream_t stream) {
   }
 }
 
+ComplexSmallOperand Operand(const clbh_complex_small_operand& o) {
+  return ComplexSmallOperand{o.pointer, o.offset, o.ld, o.stride, o.offsets, o.conjugate};
+}
+
+template <typename R, int BLOCKS, bool LEFT_KC, bool RIGHT_KC>
+int LaunchComplexSmallVariant(const ComplexSmallArgs<R>& args, const unsigned groups, hipStream_t stream) {
+  GemmComplexSmallKernel<R, BLOCKS, LEFT_KC, RIGHT_KC><<<dim3(groups), dim3(kComplexSmallThreads), 0, stream>>>(args);
+  return static_cast<int>(hipGetLastError());
+}
+
+template <typename R, int BLOCKS>
+int LaunchComplexSmallTiled(const clbh_complex_small_desc& d, hipStream_t stream) {
+  constexpr int TILE = ComplexSmallTile<BLOCKS>::TILE;
+  auto args = ComplexSmallArgs<R>{};
+  args.rows = d.rows;
+  args.columns = d.columns;
+  args.k = d.k;
+  args.tiles_r = (d.rows + TILE - 1) / TILE;
+  args.tiles_c = (d.columns + TILE - 1) / TILE;
+  args.left = Operand(d.left);
+  args.right = Operand(d.right);
+  args.c = Operand(d.c);
+  args.alpha_re = static_cast<R>(d.alpha_re);
+  args.alpha_im = static_cast<R>(d.alpha_im);
+  args.beta_re = static_cast<R>(d.beta_re);
+  args.beta_im = static_cast<R>(d.beta_im);
+  args.alphas = static_cast<const R*>(d.alphas);
+  args.betas = static_cast<const R*>(d.betas);
+  const auto groups = static_cast<long long>(args.tiles_r) * args.tiles_c * d.batch_count;
+  if (groups > 0x7fffffffll) { return hipErrorInvalidValue; }
+  const auto count = static_cast<unsigned>(groups);
+  switch ((d.left.kcontig ? 2 : 0) | (d.right.kcontig ? 1 : 0)) {
+    case 0: return LaunchComplexSmallVariant<R, BLOCKS, false, false>(args, count, stream);
+    case 1: return LaunchComplexSmallVariant<R, BLOCKS, false, true>(args, count, stream);
+    case 2: return LaunchComplexSmallVariant<R, BLOCKS, true, false>(args, count, stream);
+    default: return LaunchComplexSmallVariant<R, BLOCKS, true, true>(args, count, stream);
+  }
+}
+
+// Tiles of 32 x 32 when those waste less of the matrix cores' work than tiles of 64 x 64 (matrices of up to 32 rows
+// or columns, or 65..96 of both)
+template <typename R>
+int LaunchComplexSmallTyped(const clbh_complex_small_desc& d, hipStream_t stream) {
+  const auto padded = [&d](const long long tile) {
+    return ((d.rows + tile - 1) / tile) * ((d.columns + tile - 1) / tile) * tile * tile;
+  };
+  return (4 * padded(32) <= 3 * padded(64)) ? LaunchComplexSmallTiled<R, 1>(d, stream)
+                                            : LaunchComplexSmallTiled<R, 2>(d, stream);
+}
+
 }  // namespace
+
+int LaunchComplexSmall(const clbh_complex_small_desc& d, hipStream_t stream) {
+  if (d.rows < 1 || d.columns < 1 || d.k < 0 || d.batch_count < 1) { return hipErrorInvalidValue; }
+  if (d.left.pointer == nullptr || d.right.pointer == nullptr || d.c.pointer == nullptr) { return hipErrorInvalidValue; }
+  const auto element_bytes = static_cast<uintptr_t>(d.precision / 4);  // one complex number
+  for (const auto* operand : {&d.left, &d.right, &d.c}) {  // the kernel moves whole complex numbers
+    if (reinterpret_cast<uintptr_t>(operand->pointer) % element_bytes != 0) { return hipErrorInvalidValue; }
+  }
+  switch (d.precision) {
+    case 32: return LaunchComplexSmallTyped<float>(d, stream);
+    case 64: return LaunchComplexSmallTyped<double>(d, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
 
 int LaunchSmallBatched(const clbh_gemm_desc& d, hipStream_t stream) {
   if (d.m > kSmallDim || d.n > kSmallDim || d.k > kSmallDim) { return hipErrorInvalidValue; }

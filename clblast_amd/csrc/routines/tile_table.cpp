@@ -18,12 +18,6 @@ std::map<std::tuple<int, int>, size_t> min_indirect_overrides;  // (device, prec
 std::map<int, size_t> tile_variant_overrides;                   // precision bits -> forced MFMA tile (0 = automatic)
 std::map<int, size_t> split_overrides;                          // precision bits -> K ranges of a forced tile
 
-size_t ForcedTileVariant(const Precision precision) {
-  std::lock_guard<std::mutex> lock(override_mutex);
-  const auto found = tile_variant_overrides.find(static_cast<int>(precision));
-  return (found != tile_variant_overrides.end()) ? found->second : 0;
-}
-
 size_t ForcedSplit(const Precision precision) {
   std::lock_guard<std::mutex> lock(override_mutex);
   const auto found = split_overrides.find(static_cast<int>(precision));
@@ -31,6 +25,12 @@ size_t ForcedSplit(const Precision precision) {
 }
 
 }  // namespace
+
+size_t ForcedTileVariant(const Precision precision) {
+  std::lock_guard<std::mutex> lock(override_mutex);
+  const auto found = tile_variant_overrides.find(static_cast<int>(precision));
+  return (found != tile_variant_overrides.end()) ? found->second : 0;
+}
 
 // The MFMA kernels predicate their edge tiles, so they are correct for every shape; the threshold only
 // marks where a 128x128 (or larger) macro tile stops paying for itself against the 64x64 FMA kernel.

@@ -37,6 +37,9 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
                           const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,
                           const size_t min_indirect_size, const bool triangular = false);
 
+// Tile forced for a precision through OverrideParameters("Xgemm", {"TILE_VARIANT": 1 + index}); 0 = automatic.
+size_t ForcedTileVariant(const Precision precision);
+
 // Parameter override store behind clblast::OverrideParameters / RetrieveParameters / ClearCache.
 StatusCode OverrideRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,
                                      const std::unordered_map<std::string, size_t>& parameters);

@@ -13,6 +13,7 @@ namespace clblast {
 
 namespace {
 constexpr size_t kMaxRealExtent = static_cast<size_t>(INT_MAX) / 2;
+constexpr size_t kSmallExtent = 128;
 
 // One operand of the canonical column-major problems C' = A' * B' (for a row-major call the operands change places)
 struct BatchedOperand {
@@ -21,6 +22,24 @@ struct BatchedOperand {
   const std::vector<size_t>* offsets;  // per-batch offsets (GemmBatched) or nullptr (strided)
   bool kcontig, conjugate;
 };
+
+// The kernel that works on the interleaved data itself reads and writes every matrix once; the real form moves the
+// first operand three more times but runs on the large-tile real kernels. The former wins while a matrix is a few
+// tiles of 64 x 64.
+// A tile forced through OverrideParameters asks for the real kernels.
+bool UseSmallKernel(const size_t rows, const size_t columns, const size_t k, const size_t batch_count,
+                    const Precision precision) {
+  if (rows > kSmallExtent || columns > kSmallExtent || ForcedTileVariant(precision) != 0) { return false; }
+  // a few work-groups walking a long k alone are slower than the real kernels, which split such a k
+  const auto groups = CeilDiv(rows, size_t{64}) * CeilDiv(columns, size_t{64}) * batch_count;
+  return groups >= 512 || k <= 256;
+}
+
+clbh_complex_small_operand SmallOperand(const BatchedOperand& operand, const long long* device_offsets) {
+  return clbh_complex_small_operand{operand.pointer, static_cast<long long>(operand.offset),
+                                    static_cast<long long>(operand.ld), static_cast<long long>(operand.stride),
+                                    device_offsets, operand.kcontig ? 1 : 0, operand.conjugate ? 1 : 0};
+}
 }  // namespace
 
 template <typename R>
@@ -60,6 +79,26 @@ void XgemmComplexBatched<R>::DoGemmStridedBatched(
   const auto rows = col_major ? m : n, columns = col_major ? n : m;
   const auto precision = static_cast<int>(8 * sizeof(R));
   const auto batches = static_cast<int>(batch_count);
+
+  if (UseSmallKernel(rows, columns, k, batch_count, PrecisionValue<R>())) {
+    auto desc = clbh_complex_small_desc{};
+    desc.precision = precision;
+    desc.rows = static_cast<int>(rows);
+    desc.columns = static_cast<int>(columns);
+    desc.k = static_cast<int>(k);
+    desc.batch_count = batches;
+    desc.left = SmallOperand(left, nullptr);
+    desc.right = SmallOperand(right, nullptr);
+    desc.c = clbh_complex_small_operand{c_buffer(), static_cast<long long>(c_offset), static_cast<long long>(c_ld),
+                                        static_cast<long long>(c_stride), nullptr, 0, 0};
+    desc.alpha_re = static_cast<double>(alpha.real());
+    desc.alpha_im = static_cast<double>(alpha.imag());
+    desc.beta_re = static_cast<double>(beta.real());
+    desc.beta_im = static_cast<double>(beta.imag());
+    CheckDevice(clbh_complex_gemm_small_batched(&desc, stream()), "clbh_complex_gemm_small_batched");
+    Finish();  // records the caller's event
+    return;
+  }
 
   // left operands -> real 2 rows x 2k each, densely behind one another
   const auto expanded_elements = 4 * rows * k;
@@ -176,6 +215,23 @@ void XgemmComplexBatched<R>::DoGemmBatched(const Layout layout, const Transpose 
   const auto device_left = reinterpret_cast<const long long*>(base + 2 * scalars_block);
   const auto device_right = reinterpret_cast<const long long*>(base + 2 * scalars_block + offsets_block);
   const auto device_c = reinterpret_cast<const long long*>(base + 2 * scalars_block + 2 * offsets_block);
+
+  if (UseSmallKernel(rows, columns, k, batch_count, PrecisionValue<R>())) {
+    auto desc = clbh_complex_small_desc{};
+    desc.precision = precision;
+    desc.rows = static_cast<int>(rows);
+    desc.columns = static_cast<int>(columns);
+    desc.k = static_cast<int>(k);
+    desc.batch_count = batches;
+    desc.left = SmallOperand(left, device_left);
+    desc.right = SmallOperand(right, device_right);
+    desc.c = clbh_complex_small_operand{c_buffer(), 0, static_cast<long long>(c_ld), 0, device_c, 0, 0};
+    desc.alphas = device_alphas;
+    desc.betas = device_betas;
+    CheckDevice(clbh_complex_gemm_small_batched(&desc, stream()), "clbh_complex_gemm_small_batched");
+    Finish();  // records the caller's event
+    return;
+  }
 
   // left operands -> real 2 rows x 2k each (times their alpha), densely behind one another
   const auto expanded_elements = 4 * rows * k;

@@ -159,6 +159,29 @@ CLBH_API int clbh_complex_scale_batched(int precision, int m, int n, int triangl
                                         long long c_offset, long long c_ld, const clbh_complex_batches* batches,
                                         hipStream_t stream);
 
+// Batched complex GEMM on the interleaved data itself, for matrices so small that the real forms above would be most
+// of the traffic. Canonical column-major problem per matrix b of the batch:
+//   C'(rows x columns) = alpha * L(rows x k) * R(k x columns) + beta * C'
+// Matrix b of an operand starts at pointer + offset + (offsets ? offsets[b] : b * stride), in complex elements
+// (offsets: device array); element (x, p) of L or R lies at kcontig ? x * ld + p : p * ld + x, element (i, j) of C'
+// at j * ld + i. conjugate != 0 conjugates L or R. alphas / betas (device arrays of (re, im) pairs of the component
+// type), when given, replace alpha / beta per matrix. C' is not read when beta is zero.
+typedef struct clbh_complex_small_operand_ {
+  const void* pointer;
+  long long offset, ld, stride;
+  const long long* offsets;
+  int kcontig, conjugate;
+} clbh_complex_small_operand;
+typedef struct clbh_complex_small_desc_ {
+  int precision;  // 32 or 64: bits of a component
+  int rows, columns, k, batch_count;
+  clbh_complex_small_operand left, right, c;
+  double alpha_re, alpha_im, beta_re, beta_im;
+  const void* alphas;
+  const void* betas;
+} clbh_complex_small_desc;
+CLBH_API int clbh_complex_gemm_small_batched(const clbh_complex_small_desc* desc, hipStream_t stream);
+
 // im2col of a batch of images for CONVGEMM (all arguments in elements; see kernels/im2col.hpp for the layout):
 // image + image_offset holds batch x channels x height x width, col receives batch matrices of
 // (output_h * output_w) x (channels * kernel_h * kernel_w), column-major. flip != 0 mirrors the kernel taps.
