@@ -1,7 +1,7 @@
 """CLBlast{C,Z}gemmBatched and CLBlast{C,Z}gemmStridedBatched through the C ABI (reference: include/clblast_c.h:1317-1330,
 1353-1364) against the CPU oracle applied matrix by matrix, and against the real reference on the same GPU. All
 2 x 3 x 3 combinations of layout, op(A) and op(B); padded leading dimensions, offsets and strides; shared operands
-(stride 0); per-batch complex alphas and betas; matrices on both sides of 128 rows and columns, where the routine changes
+(stride 0); per-batch complex alphas and betas; matrices on both sides of 384 rows and columns, where the routine changes
 from the kernel that works on the interleaved data to the real form of the problem. Everything of C outside the
 batch's logical matrices must keep its bits.
 Tolerance: relative Frobenius error 1e-5 (complex64) and 1e-12 (complex128), as for the real types."""
@@ -143,7 +143,7 @@ def test_complex_strided_batched_sweep(gpu, bits):
     seed = 21000
     for layout, ta, tb in MODES:
         for (m, n, k), batch in (((7, 7, 7), 3), ((33, 17, 20), 4), ((64, 64, 64), 2), ((32, 32, 32), 17), ((1, 5, 130), 3),
-                                  ((100, 128, 33), 2), ((150, 70, 40), 2), ((60, 131, 17), 3)):
+                                  ((100, 128, 33), 2), ((150, 70, 40), 2), ((60, 131, 17), 3), ((390, 20, 33), 2)):
             seed += 1
             extra, base, slack = (((0, 0, 0), (0, 0, 0), (0, 0, 0)), ((3, 1, 2), (10, 10, 10), (5, 0, 9)),
                                   ((1, 0, 5), (1, 3, 7), (0, 4, 1)))[seed % 3]
@@ -160,7 +160,7 @@ def test_complex_batched_sweep(gpu, bits):
     seed = 22000
     for layout, ta, tb in MODES:
         for (m, n, k), batch in (((7, 7, 7), 3), ((33, 17, 20), 5), ((64, 64, 64), 2), ((32, 32, 32), 19),
-                                  ((128, 90, 35), 2), ((129, 70, 40), 2), ((20, 140, 8), 3)):
+                                  ((128, 90, 35), 2), ((129, 70, 40), 2), ((20, 140, 8), 3), ((30, 400, 20), 2)):
             seed += 1
             problem = scattered_problem(bits, layout, ta, tb, m, n, k, batch, seed, ((0, 0, 0), (2, 3, 1))[seed % 2],
                                         real_betas=(seed % 3 == 0))
