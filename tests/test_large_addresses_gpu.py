@@ -163,3 +163,74 @@ def test_leading_dimension_beyond_the_tile_window(gpu, prefix, kcontig):
     assert relative_error(c.t(), want) <= TOL[prefix]
     del a, a_view, a_matrix
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("prefix", ("C", "Z"))
+@pytest.mark.parametrize("shape", ((60, 50, 40), (300, 200, 300)))
+def test_complex_offsets_beyond_4_gib(gpu, prefix, shape):
+    """CGEMM / ZGEMM on matrices behind more than 4 GiB of one buffer (row-major, B conjugate-transposed): the small
+    shape takes the kernel on interleaved data, the large one the real form with its helper kernels."""
+    dtype = torch.complex64 if prefix == "C" else torch.complex128
+    element = 8 if prefix == "C" else 16
+    m, n, k = shape
+    first = (5 << 30) // element + 3
+    a_offset, b_offset, c_offset = first, first + m * k + 5, first + m * k + n * k + 9
+    buffer = torch.empty(c_offset + m * n + 16, device="cuda:0", dtype=dtype)
+    tail = torch.view_as_real(buffer[first:])
+    tail.copy_(torch.rand(tail.shape, device="cuda:0").sub_(0.5))
+    before = buffer[first:].clone()
+    a = before[:m * k].view(m, k).to(torch.complex128)
+    b = before[b_offset - first:b_offset - first + n * k].view(n, k).to(torch.complex128)
+    c = before[c_offset - first:c_offset - first + m * n].view(m, n).to(torch.complex128)
+    alpha, beta = 0.5 - 1.5j, 2.0 + 0.25j
+    want = alpha * (a @ b.conj().t()) + beta * c
+    status = clblast_amd.raw_complex_gemm(prefix, ROW_MAJOR, NO, 113, m, n, k, alpha, buffer.data_ptr(), a_offset, k,
+                                          buffer.data_ptr(), b_offset, k, beta, buffer.data_ptr(), c_offset, n,
+                                          gpu.stream_handle())
+    torch.cuda.synchronize()
+    assert status == 0
+    after = buffer[first:]
+    got = after[c_offset - first:c_offset - first + m * n].view(m, n).to(torch.complex128)
+    assert float((got - want).norm() / want.norm()) <= (1e-5 if prefix == "C" else 1e-12)
+    assert torch.equal(torch.view_as_real(after[:c_offset - first]), torch.view_as_real(before[:c_offset - first]))
+    del buffer, tail, after
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("prefix", ("S", "D"))
+def test_symm_and_trsm_offsets_beyond_4_gib(gpu, prefix):
+    """The routines that prepare an operand with a kernel of their own (SYMM: the mirrored square; TRSM: the padded
+    triangle and its inverted diagonal blocks) on matrices behind more than 4 GiB of one buffer."""
+    dtype = DTYPE[prefix]
+    element = torch.empty(0, dtype=dtype).element_size()
+    m, n = 200, 150
+    first = (5 << 30) // element + 7
+    a_offset, b_offset, c_offset = first, first + m * m + 3, first + m * m + m * n + 9
+    buffer = torch.empty(c_offset + m * n + 16, device="cuda:0", dtype=dtype)
+    tail = buffer[first:]
+    tail.copy_(torch.rand(tail.numel(), device="cuda:0").sub_(0.5))
+    # a diagonally dominant A (row-major m x m) so that the solve is well conditioned
+    a_view = buffer[a_offset:a_offset + m * m].view(m, m)
+    a_view.mul_(2.0 / m).add_(4.0 * torch.eye(m, device="cuda:0", dtype=dtype))
+    a = a_view.double().clone()
+    b = buffer[b_offset:b_offset + m * n].view(m, n).double().clone()
+    c = buffer[c_offset:c_offset + m * n].view(m, n).double().clone()
+    lower = torch.tril(a)
+    symmetric = lower + torch.tril(a, -1).t()
+    # SYMM: row-major, left, lower (141 / 122): C = 0.5 A B + 2 C
+    status = clblast_amd.raw_symm(prefix, ROW_MAJOR, 141, 122, m, n, 0.5, buffer.data_ptr(), a_offset, m, buffer.data_ptr(),
+                                  b_offset, n, 2.0, buffer.data_ptr(), c_offset, n, gpu.stream_handle())
+    torch.cuda.synchronize()
+    assert status == 0
+    got = buffer[c_offset:c_offset + m * n].view(m, n)
+    assert relative_error(got, 0.5 * symmetric @ b + 2.0 * c) <= TOL[prefix]
+    # TRSM: row-major, left, lower, no transpose, non-unit diagonal (131): solves A X = 1.5 B in place
+    status = clblast_amd.raw_trsm(prefix, ROW_MAJOR, 141, 122, NO, 131, m, n, 1.5, buffer.data_ptr(), a_offset, m,
+                                  buffer.data_ptr(), b_offset, n, gpu.stream_handle())
+    torch.cuda.synchronize()
+    assert status == 0
+    got = buffer[b_offset:b_offset + m * n].view(m, n)
+    want = torch.linalg.solve_triangular(lower, 1.5 * b, upper=False)
+    assert relative_error(got, want) <= 2 * TOL[prefix]
+    del buffer, tail, a_view, got
+    torch.cuda.empty_cache()
