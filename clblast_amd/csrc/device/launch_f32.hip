@@ -42,6 +42,7 @@ int LaunchMfmaF32(const clbh_gemm_desc& d, hipStream_t stream) {
     case 8: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 1, 2, 32, 4, MfmaTraitsF32Small>>(d, stream);  // 32 x 64 x 32
     case 9: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 1, 32, 4, MfmaTraitsF32Small>>(d, stream);  // 64 x 32 x 32
     case 10: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 1, 1, 64, 4, MfmaTraitsF32Small>>(d, stream);  // 32 x 32 x 64
+    case 11: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 4, 2, 32, 2, MfmaTraitsF32Small>>(d, stream);  // 128 x 64 x 32
     default: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16, 2>>(d, stream);  // 128 x 128 x 16
   }
 }

@@ -68,6 +68,12 @@ struct Tile {
   size_t tile_m, tile_n;
 };
 
+// Tiles of which two share a CU: the launch runs in rounds of 512, and the last round should be at least 90 % full
+bool FillsPairs(const size_t tiles) {
+  const auto rounds = CeilDivide(tiles, 512);
+  return tiles >= 460 && 10 * tiles >= 9 * rounds * 512;
+}
+
 // Share of the tiles' area that the m x n matrix fills (tiles of tile_m x tile_n), in per cent
 size_t TileUse(const size_t m, const size_t n, const size_t tile_m, const size_t tile_n) {
   const auto along_m = static_cast<double>(m) / static_cast<double>(CeilDivide(m, tile_m) * tile_m);
@@ -176,6 +182,9 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
              TileUse(m, n, 256, 128) >= 80) { tile = Tile{3, 256, 128}; }  // (batches: 256 x 256^3 96 -> 80 us)
     else if (batch_count > 1 && TileUse(m, n, 128, 128) >= 90 && CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count >= 512) {
       tile = Tile{0, 128, 128};  // batches of matrices that fill 128 x 128 tiles (1024 x 128^3: 66 -> 57 us)
+    }
+    else if (batch_count == 1 && k >= 256 && TileUse(m, n, 128, 64) >= 90 && FillsPairs(CeilDivide(m, 128) * CeilDivide(n, 64))) {
+      tile = Tile{11, 128, 64};  // whole rounds of two work-groups per CU (2048^3: 140 -> 131 us, 4096 x 3072 x 2048: 396 -> 385)
     }
     else if (tiles64 <= 64 && k < 2048) { tile = Tile{10, 32, 32}; }
     else if (tiles64 < 1024 && (batch_count == 1 || n > 64)) { tile = Tile{9, 64, 32}; }  // (batches of matrices one tile
