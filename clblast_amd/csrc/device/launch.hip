@@ -309,6 +309,36 @@ int clbh_fill_zero(void* ptr, size_t bytes, hipStream_t stream) {
   return static_cast<int>(hipGetLastError());
 }
 
+int clbh_copy_matrix_batched(int precision, int one_extent, int two_extent, int batch_count, const void* src,
+                             long long src_offset, long long src_ld, long long src_stride, const long long* src_offsets,
+                             void* dst, long long dst_ld, long long dst_stride, hipStream_t stream) {
+  if (one_extent <= 0 || two_extent <= 0 || batch_count <= 0 || src == nullptr || dst == nullptr || dst_ld < one_extent ||
+      src_ld < 1 || src_offset < 0 || src_stride < 0 || dst_stride < dst_ld * two_extent) {
+    return hipErrorInvalidValue;
+  }
+  const long long blocks = (static_cast<long long>(one_extent) * two_extent + clbh::kCopyThreads - 1) / clbh::kCopyThreads;
+  const dim3 grid(static_cast<unsigned>(std::min<long long>(blocks, 4096)), static_cast<unsigned>(std::min(batch_count, 65535)));
+  switch (precision) {
+    case 16:
+      clbh::CopyMatrixBatchedKernel<_Float16><<<grid, dim3(clbh::kCopyThreads), 0, stream>>>(
+          one_extent, two_extent, batch_count, static_cast<const _Float16*>(src) + src_offset, src_ld, src_stride, src_offsets,
+          static_cast<_Float16*>(dst), dst_ld, dst_stride);
+      break;
+    case 32:
+      clbh::CopyMatrixBatchedKernel<float><<<grid, dim3(clbh::kCopyThreads), 0, stream>>>(
+          one_extent, two_extent, batch_count, static_cast<const float*>(src) + src_offset, src_ld, src_stride, src_offsets,
+          static_cast<float*>(dst), dst_ld, dst_stride);
+      break;
+    case 64:
+      clbh::CopyMatrixBatchedKernel<double><<<grid, dim3(clbh::kCopyThreads), 0, stream>>>(
+          one_extent, two_extent, batch_count, static_cast<const double*>(src) + src_offset, src_ld, src_stride, src_offsets,
+          static_cast<double*>(dst), dst_ld, dst_stride);
+      break;
+    default: return hipErrorInvalidValue;
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
 int clbh_copy_matrix(int precision, int one_extent, int two_extent, const void* src, long long src_offset, long long src_ld,
                      void* dst, long long dst_offset, long long dst_ld, hipStream_t stream) {
   if (one_extent <= 0 || two_extent <= 0 || src == nullptr || dst == nullptr || src_ld < one_extent || dst_ld < one_extent ||

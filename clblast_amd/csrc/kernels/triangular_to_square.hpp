@@ -64,6 +64,28 @@ __global__ __launch_bounds__(kCopyThreads) void CopyMatrixKernel(const int one_e
   }
 }
 
+// The same for the matrices of a batch: matrix b starts at src + (offsets ? offsets[b] : b * src_stride) and goes to
+// dst + b * dst_stride. Element-wise, for sources whose alignment allows nothing wider.
+template <typename T>
+__global__ __launch_bounds__(kCopyThreads) void CopyMatrixBatchedKernel(const int one_extent, const int two_extent,
+                                                                        const int batch_count, const T* __restrict__ src,
+                                                                        const long long src_ld, const long long src_stride,
+                                                                        const long long* __restrict__ src_offsets,
+                                                                        T* __restrict__ dst, const long long dst_ld,
+                                                                        const long long dst_stride) {
+  // consecutive threads walk the elements of a matrix in storage order, whatever the length of a line
+  const long long elements = static_cast<long long>(one_extent) * two_extent;
+  for (int batch = blockIdx.y; batch < batch_count; batch += gridDim.y) {
+    const T* from = src + (src_offsets != nullptr ? src_offsets[batch] : batch * src_stride);
+    T* to = dst + batch * dst_stride;
+    for (long long element = blockIdx.x * kCopyThreads + threadIdx.x; element < elements;
+         element += static_cast<long long>(gridDim.x) * kCopyThreads) {
+      const long long two = element / one_extent, one = element - two * one_extent;
+      to[two * dst_ld + one] = from[two * src_ld + one];
+    }
+  }
+}
+
 // Inverts the BLOCK x BLOCK diagonal blocks of a dense triangular matrix (zeros in the other triangle; reference:
 // Xinvert, src/routines/levelx/xinvert.cpp:45-140 and src/kernels/level3/invert_diagonal_blocks_part1.opencl, which
 // invert 16 x 16 blocks and combine them by block products in several launches). One work-group of 256 threads per

@@ -120,6 +120,13 @@ CLBH_API int clbh_fill_zero(void* ptr, size_t bytes, hipStream_t stream);
 // precision: bits per element (16, 32, 64, or 128 for double-precision complex; single-precision complex copies as 64).
 CLBH_API int clbh_copy_matrix(int precision, int one_extent, int two_extent, const void* src, long long src_offset,
                               long long src_ld, void* dst, long long dst_offset, long long dst_ld, hipStream_t stream);
+// The same for a batch: matrix b is read at src + src_offset + (src_offsets ? src_offsets[b] : b * src_stride)
+// (src_offsets: device array) and written densely at dst + b * dst_stride with leading dimension dst_ld. Element-wise:
+// for sources at addresses or with leading dimensions that allow no wider access (the aligned copies of fp16 operands).
+CLBH_API int clbh_copy_matrix_batched(int precision, int one_extent, int two_extent, int batch_count, const void* src,
+                                      long long src_offset, long long src_ld, long long src_stride,
+                                      const long long* src_offsets, void* dst, long long dst_ld, long long dst_stride,
+                                      hipStream_t stream);
 
 // ---- complex GEMM helpers: precision is the width of ONE component, 32 (float2 data) or 64 (double2); offsets and
 // leading dimensions count complex elements --------------------------------------------------------------------

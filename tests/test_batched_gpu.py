@@ -62,6 +62,21 @@ def test_strided_batched_reference_sweep(gpu, bits):
                             offsets=((0, 0, 0), (10, 10, 10))[seed % 2], extra_ld=((0, 0, 0), (1, 2, 3))[(seed // 2) % 2])
 
 
+@pytest.mark.parametrize("bits", [16, 32])
+def test_strided_batched_with_odd_offsets_leading_dimensions_and_strides(gpu, bits):
+    """Matrices at odd elements, with odd leading dimensions and odd strides, large enough for the tiled kernels: the
+    fp16 kernels fetch dwords and get aligned copies of such operands; a shared operand (stride 0) is copied once."""
+    seed = 300
+    for layout, ta, tb in itertools.product((ROW_MAJOR, COL_MAJOR), (NO, YES), (NO, YES)):
+        for (m, n, k), offsets, extra, strides in (((33, 65, 40), (1, 3, 5), (0, 0, 0), (None, None)),
+                                                   ((33, 65, 40), (0, 0, 1), (1, 0, 0), (None, None)),
+                                                   ((64, 48, 72), (2, 1, 0), (0, 1, 1), (64 * 72 + 1, None)),
+                                                   ((40, 33, 65), (1, 1, 1), (1, 1, 1), (0, None)),
+                                                   ((40, 33, 65), (0, 0, 0), (0, 0, 0), (None, 0))):
+            seed += 3
+            run_strided(gpu, bits, layout, ta, tb, m, n, k, 0.75, -1.5, 50, strides[0], strides[1], offsets, extra, seed)
+
+
 @pytest.mark.parametrize("layout", [ROW_MAJOR, COL_MAJOR])
 def test_strided_batched_small_matrix_kernel(gpu, layout):
     """m, n, k <= 32 with many batches takes the one-wavefront-per-matrix kernel: dense 32^3 (16-byte loads)
@@ -83,7 +98,7 @@ def test_strided_batched_small_matrix_kernel(gpu, layout):
 def test_batched_with_per_batch_scalars_and_offsets(gpu, bits):
     seed = 500
     for layout, ta, tb in itertools.product((ROW_MAJOR, COL_MAJOR), (NO, YES), (NO, YES)):
-        for (m, n, k), batch in (((7, 64, 7), 3), ((64, 7, 64), 1), ((32, 32, 32), 40), ((9, 5, 33), 17)):
+        for (m, n, k), batch in (((7, 64, 7), 3), ((64, 7, 64), 1), ((32, 32, 32), 40), ((9, 5, 33), 17), ((33, 65, 40), 50)):
             seed += 3
             _, shape = oracle.process_arguments(layout, ta, tb, m, n, k)
             a_ld, b_ld, c_ld = shape.a_one + 1, shape.b_one, shape.c_one + 2
