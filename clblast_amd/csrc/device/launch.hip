@@ -20,6 +20,7 @@ int LaunchTyped(const clbh_gemm_desc& d, hipStream_t stream) {
   const bool mfma = (d.kernel_class == CLBH_KERNEL_MFMA);
   if (d.conv != nullptr && !(mfma && (d.precision == 32 || d.precision == 16))) { return hipErrorInvalidValue; }  // only those kernels gather
   if (d.kernel_class == CLBH_KERNEL_SMALL_BATCHED) { return LaunchSmallBatched(d, stream); }
+  if (d.kernel_class == CLBH_KERNEL_SMALL_TILED) { return LaunchSmallTiled(d, stream); }
   switch (d.precision) {
     case 16: return mfma ? LaunchMfmaF16(d, stream) : LaunchGeneralF16(d, stream);
     case 32: return mfma ? LaunchMfmaF32(d, stream) : LaunchGeneralF32(d, stream);
@@ -42,7 +43,10 @@ bool ValidDescriptor(const clbh_gemm_desc& d) {
   if (d.a_offset < 0 || d.b_offset < 0 || d.c_offset < 0) { return false; }
   if (d.c_triangle < 0 || d.c_triangle > 4 || d.operand_triangle < 0 || d.operand_triangle > 4) { return false; }
   // the one-wavefront-per-matrix kernel knows no triangles
-  if ((d.c_triangle != 0 || d.operand_triangle != 0) && d.kernel_class == CLBH_KERNEL_SMALL_BATCHED) { return false; }
+  if ((d.c_triangle != 0 || d.operand_triangle != 0) &&
+      (d.kernel_class == CLBH_KERNEL_SMALL_BATCHED || d.kernel_class == CLBH_KERNEL_SMALL_TILED)) {
+    return false;
+  }
   return true;
 }
 

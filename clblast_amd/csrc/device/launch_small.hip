@@ -86,7 +86,44 @@ int LaunchComplexSmallTyped(const clbh_complex_small_desc& d, hipStream_t stream
                                             : LaunchComplexSmallTiled<R, 2>(d, stream);
 }
 
+template <typename T, int BLOCKS, bool A_KC, bool B_KC>
+int LaunchSmallTiledVariant(const clbh_gemm_desc& d, hipStream_t stream) {
+  constexpr int TILE = ComplexSmallTile<BLOCKS>::TILE;
+  const auto args = MakeArgs<T>(d);
+  const long long tiles_m = (d.m + TILE - 1) / TILE, tiles_n = (d.n + TILE - 1) / TILE;
+  if (tiles_m * tiles_n > INT_MAX) { return hipErrorInvalidConfiguration; }
+  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
+  GemmSmallTiledKernel<T, BLOCKS, A_KC, B_KC><<<grid, dim3(kComplexSmallThreads), 0, stream>>>(
+      args, static_cast<int>(tiles_m), static_cast<int>(tiles_n));
+  return static_cast<int>(hipGetLastError());
+}
+
+template <typename T, int BLOCKS>
+int LaunchSmallTiledBlocks(const clbh_gemm_desc& d, hipStream_t stream) {
+  switch ((d.a_kcontig ? 2 : 0) | (d.b_kcontig ? 1 : 0)) {
+    case 0: return LaunchSmallTiledVariant<T, BLOCKS, false, false>(d, stream);
+    case 1: return LaunchSmallTiledVariant<T, BLOCKS, false, true>(d, stream);
+    case 2: return LaunchSmallTiledVariant<T, BLOCKS, true, false>(d, stream);
+    default: return LaunchSmallTiledVariant<T, BLOCKS, true, true>(d, stream);
+  }
+}
+
+// tile_variant 1: tiles of 32 x 32, else 64 x 64
+template <typename T>
+int LaunchSmallTiledTyped(const clbh_gemm_desc& d, hipStream_t stream) {
+  return d.tile_variant == 1 ? LaunchSmallTiledBlocks<T, 1>(d, stream) : LaunchSmallTiledBlocks<T, 2>(d, stream);
+}
+
 }  // namespace
+
+int LaunchSmallTiled(const clbh_gemm_desc& d, hipStream_t stream) {
+  if (d.c_triangle != 0 || d.operand_triangle != 0 || d.conv != nullptr || d.k < 1) { return hipErrorInvalidValue; }
+  switch (d.precision) {
+    case 32: return LaunchSmallTiledTyped<float>(d, stream);
+    case 64: return LaunchSmallTiledTyped<double>(d, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
 
 int LaunchComplexSmall(const clbh_complex_small_desc& d, hipStream_t stream) {
   if (d.rows < 1 || d.columns < 1 || d.k < 0 || d.batch_count < 1) { return hipErrorInvalidValue; }

@@ -239,6 +239,127 @@ __global__ __launch_bounds__(kComplexSmallThreads, (sizeof(R) == 8 && BLOCKS == 
   }
 }
 
+// ---- the same scheme for batches of small REAL matrices (fp32, fp64) -------------------------------------------
+// Batches of matrices of a few tiles with a short k are bound by HBM and by latency: the ring of three slabs of the
+// large-tile kernel costs LDS (three work-groups per CU) and a long prologue. Here a work-group keeps one slab per
+// operand in LDS (two planes of 16 x (TILE + 4)), loads the next one into registers while it multiplies, and eight
+// or more work-groups share a CU. Arguments as for the other GEMM kernels (column-major canonical problem).
+template <typename T, int BLOCKS, bool KC>
+struct RealSlabLoader {
+  using Tile = ComplexSmallTile<BLOCKS>;
+  const T* src;
+  long long first, piece_step, slab_step;
+  int x_valid, p_first, p_end;
+
+  __device__ __forceinline__ RealSlabLoader(const T* src_, const long long ld, const int x0, const int x_end,
+                                            const int p_end_, const int thread)
+      : src(src_), p_end(p_end_) {
+    const int x = x0 + Tile::template X<KC>(thread, 0), p = Tile::template P<KC>(thread, 0);
+    first = KC ? x * ld + p : p * ld + x;
+    piece_step = KC ? (kComplexSmallThreads / kComplexSmallSlab) * ld : (kComplexSmallThreads / Tile::TILE) * ld;
+    slab_step = KC ? kComplexSmallSlab : kComplexSmallSlab * ld;
+    p_first = p;
+    x_valid = 0;
+#pragma unroll
+    for (int q = 0; q < Tile::PIECES; ++q) {
+      if (x0 + Tile::template X<KC>(thread, q) < x_end) { x_valid |= 1 << q; }
+    }
+  }
+
+  // branch-free like ComplexSlabLoader::Load: a piece outside the matrix reads its first element
+  __device__ __forceinline__ int Load(T (&values)[Tile::PIECES], const int slab) const {
+    int valid = 0;
+#pragma unroll
+    for (int q = 0; q < Tile::PIECES; ++q) {
+      const int p = slab * kComplexSmallSlab + p_first + (KC ? 0 : (kComplexSmallThreads / Tile::TILE) * q);
+      const bool inside = ((x_valid >> q) & 1) != 0 && p < p_end;
+      const long long index = inside ? first + q * piece_step + slab * slab_step : 0;
+      values[q] = src[index];
+      valid |= inside ? 1 << q : 0;
+    }
+    return valid;
+  }
+};
+
+template <typename T, int BLOCKS, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kComplexSmallThreads) void GemmSmallTiledKernel(const GemmArgs<T> p, const int tiles_m,
+                                                                             const int tiles_n) {
+  using Traits = typename ComplexSmallTraits<T>::Mfma;
+  using Acc = typename Traits::Acc;
+  using Tile = ComplexSmallTile<BLOCKS>;
+  constexpr int PLANE = kComplexSmallSlab * Tile::PITCH;
+  __shared__ T planes[2 * PLANE];
+  T* const a_plane = planes;
+  T* const b_plane = planes + PLANE;
+
+  const int thread = threadIdx.x, wave = thread / 64, lane = thread % 64;
+  const int m0 = (blockIdx.x % tiles_m) * Tile::TILE, n0 = (blockIdx.x / tiles_m) * Tile::TILE;
+  const int wave_m = 16 * BLOCKS * (wave % 2), wave_n = 16 * BLOCKS * (wave / 2);
+  const int in_block = lane % 16, k_group = lane / 16;
+  const int slabs = (p.k + kComplexSmallSlab - 1) / kComplexSmallSlab;
+
+  for (int batch = blockIdx.y; batch < p.batch_count; batch += gridDim.y) {
+    const T* a;
+    const T* b;
+    T* c;
+    T alpha, beta;
+    ResolveBatch<T, T>(p, batch, a, b, c, alpha, beta);
+    Acc acc[BLOCKS][BLOCKS];
+#pragma unroll
+    for (int i = 0; i < BLOCKS; ++i) {
+#pragma unroll
+      for (int j = 0; j < BLOCKS; ++j) { acc[i][j] = Traits::Zero(); }
+    }
+    const RealSlabLoader<T, BLOCKS, A_KC> a_loader(a, p.a_ld, m0, p.m, p.k, thread);
+    const RealSlabLoader<T, BLOCKS, B_KC> b_loader(b, p.b_ld, n0, p.n, p.k, thread);
+    T a_values[Tile::PIECES], b_values[Tile::PIECES];
+    int a_valid = a_loader.Load(a_values, 0), b_valid = b_loader.Load(b_values, 0);  // the host guarantees k > 0
+    for (int slab = 0; slab < slabs; ++slab) {
+      __syncthreads();  // the previous slab (or matrix) has been consumed
+#pragma unroll
+      for (int q = 0; q < Tile::PIECES; ++q) {
+        a_plane[Tile::template P<A_KC>(thread, q) * Tile::PITCH + Tile::template X<A_KC>(thread, q)] =
+            ((a_valid >> q) & 1) != 0 ? a_values[q] : T(0);
+        b_plane[Tile::template P<B_KC>(thread, q) * Tile::PITCH + Tile::template X<B_KC>(thread, q)] =
+            ((b_valid >> q) & 1) != 0 ? b_values[q] : T(0);
+      }
+      __syncthreads();
+      if (slab + 1 < slabs) {
+        a_valid = a_loader.Load(a_values, slab + 1);
+        b_valid = b_loader.Load(b_values, slab + 1);
+      }
+#pragma unroll
+      for (int step = 0; step < kComplexSmallSlab / 4; ++step) {
+        const int line = (4 * step + k_group) * Tile::PITCH + in_block;
+        T a_fragment[BLOCKS], b_fragment[BLOCKS];
+#pragma unroll
+        for (int i = 0; i < BLOCKS; ++i) {
+          a_fragment[i] = a_plane[line + wave_m + 16 * i];
+          b_fragment[i] = b_plane[line + wave_n + 16 * i];
+        }
+        // B's fragment goes first: the lanes of a result register then run along m, the contiguous index of C
+#pragma unroll
+        for (int i = 0; i < BLOCKS; ++i) {
+#pragma unroll
+          for (int j = 0; j < BLOCKS; ++j) { acc[i][j] = Traits::Mfma(b_fragment[j], a_fragment[i], acc[i][j]); }
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < BLOCKS; ++i) {
+#pragma unroll
+      for (int j = 0; j < BLOCKS; ++j) {
+        const int row = m0 + wave_m + 16 * i + in_block;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int column = n0 + wave_n + 16 * j + Traits::Row(r, k_group);
+          if (row < p.m && column < p.n) { StoreResult<T, T>(c, column * p.c_ld + row, acc[i][j][r], alpha, beta); }
+        }
+      }
+    }
+  }
+}
+
 }  // namespace clbh
 
 #endif  // CLBLAST_HIP_KERNELS_GEMM_COMPLEX_SMALL_HPP_

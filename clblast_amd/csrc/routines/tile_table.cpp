@@ -123,6 +123,15 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     return KernelChoice{CLBH_KERNEL_GENERAL, 0, 1};
   }
   const auto forced = ForcedTileVariant(precision);
+  // Batches of fp32 / fp64 matrices of a few tiles with a short k are bound by HBM and latency, not by the matrix
+  // cores: the kernel that keeps one slab per operand in LDS runs eight work-groups or more per CU (fp32 4096 x 64^3:
+  // 49 -> 42 us, 1024 x 96^3: 53 -> 43 us with tiles of 32 x 32; fp64 2048 x 128 x 64 x 64: 123 -> 75 us). With a
+  // longer k (fp32 1024 x 128^3: 57 against 70 us) the ring of three slabs of the large-tile kernels wins.
+  if (forced == 0 && batch_count > 1 && !triangular && precision != Precision::kHalf && m <= 256 && n <= 256 &&
+      k <= (precision == Precision::kSingle ? 96u : 64u) && CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count >= 512) {
+    const auto padded = [m, n](const size_t tile) { return CeilDivide(m, tile) * CeilDivide(n, tile) * tile * tile; };
+    return KernelChoice{CLBH_KERNEL_SMALL_TILED, (4 * padded(32) < 3 * padded(64)) ? 1 : 0, 1};
+  }
   if (forced != 0) {
     // a forced tile takes the forced number of K ranges (unbatched calls only), never more than k / 16
     const auto ranges = (batch_count == 1) ? std::max<size_t>(1, std::min<size_t>(ForcedSplit(precision), k / 16)) : 1;

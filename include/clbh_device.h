@@ -34,7 +34,9 @@ enum clbh_kernel_class {
   CLBH_KERNEL_GENERAL = 0,  // bounds-checked LDS-tiled FMA kernel, any shape (reference analogue: XgemmDirect)
   CLBH_KERNEL_MFMA = 1,     // large-tile MFMA kernel with LDS double buffering (analogue: Xgemm indirect)
   CLBH_KERNEL_SMALL_BATCHED = 2,  // one wavefront per small matrix, bandwidth bound
-  CLBH_KERNEL_SKINNY = 3          // split-K streaming kernel for problems with a tiny m or n
+  CLBH_KERNEL_SKINNY = 3,         // split-K streaming kernel for problems with a tiny m or n
+  CLBH_KERNEL_SMALL_TILED = 4     // fp32 / fp64 batches of matrices of a few tiles: one slab per operand in LDS, many
+                                  // work-groups per CU (tile_variant 1: tiles of 32 x 32, else 64 x 64)
 };
 
 // Per-batch metadata of GemmBatched, all device pointers (NULL for plain and strided launches).

@@ -77,6 +77,20 @@ def test_strided_batched_with_odd_offsets_leading_dimensions_and_strides(gpu, bi
             run_strided(gpu, bits, layout, ta, tb, m, n, k, 0.75, -1.5, 50, strides[0], strides[1], offsets, extra, seed)
 
 
+@pytest.mark.parametrize("bits", [32, 64])
+def test_batches_of_matrices_of_a_few_tiles_with_a_short_k(gpu, bits):
+    """At least 512 tiles of 64 x 64 over the batch, m and n up to 256, k up to 64: the kernel with one slab per operand
+    in LDS, with tiles of 64 x 64 or of 32 x 32; ragged edges, padded leading dimensions, offsets, a shared operand."""
+    seed = 400
+    for layout, ta, tb in itertools.product((ROW_MAJOR, COL_MAJOR), (NO, YES), (NO, YES)):
+        for (m, n, k), batch, offsets, extra, strides in (((33, 65, 40), 300, (1, 3, 5), (1, 0, 2), (None, None)),
+                                                          ((90, 30, 64), 600, (0, 0, 0), (0, 0, 0), (None, None)),
+                                                          ((100, 200, 17), 130, (4, 0, 8), (0, 3, 0), (0, None)),
+                                                          ((64, 64, 1), 520, (0, 0, 0), (0, 0, 0), (None, 0))):
+            seed += 3
+            run_strided(gpu, bits, layout, ta, tb, m, n, k, -0.5, 1.25, batch, strides[0], strides[1], offsets, extra, seed)
+
+
 @pytest.mark.parametrize("layout", [ROW_MAJOR, COL_MAJOR])
 def test_strided_batched_small_matrix_kernel(gpu, layout):
     """m, n, k <= 32 with many batches takes the one-wavefront-per-matrix kernel: dense 32^3 (16-byte loads)
@@ -98,7 +112,7 @@ def test_strided_batched_small_matrix_kernel(gpu, layout):
 def test_batched_with_per_batch_scalars_and_offsets(gpu, bits):
     seed = 500
     for layout, ta, tb in itertools.product((ROW_MAJOR, COL_MAJOR), (NO, YES), (NO, YES)):
-        for (m, n, k), batch in (((7, 64, 7), 3), ((64, 7, 64), 1), ((32, 32, 32), 40), ((9, 5, 33), 17), ((33, 65, 40), 50)):
+        for (m, n, k), batch in (((7, 64, 7), 3), ((64, 7, 64), 1), ((32, 32, 32), 40), ((9, 5, 33), 17), ((33, 65, 40), 50), ((70, 33, 24), 300)):
             seed += 3
             _, shape = oracle.process_arguments(layout, ta, tb, m, n, k)
             a_ld, b_ld, c_ld = shape.a_one + 1, shape.b_one, shape.c_one + 2
