@@ -553,6 +553,9 @@ EXTRA_WORKLOADS = {
                                                        24, (11, 13, 19)),
     "cfg5_sgemm_8191x8191x127_colNN": lambda: Workload("cfg5d", "S", COL, NO, NO, 8191, 8191, 127, -0.75, 2.0, 8194,
                                                         132, 8198, (11, 13, 19)),
+    "next_sgemm_strided_batched_4096x64": lambda: Workload("sbat64", "S", ROW, NO, NO, 64, 64, 64, 1.0, 0.0, batch=4096),
+    "next_dgemm_strided_batched_2048x128x64x64": lambda: Workload("dbat128", "D", ROW, NO, YES, 128, 64, 64, 1.0, 0.0,
+                                                                  batch=2048),
     "next_cgemm_4096_rowNC": lambda: ComplexWorkload("cgemm", "C", NO, 113, 4096, 4096, 4096, 1.0 - 0.5j, 0.0),
     "next_zgemm_2048_rowTN": lambda: ComplexWorkload("zgemm", "Z", YES, NO, 2048, 2048, 2048, 0.5 + 1.0j, 1.0 - 0.5j),
     "next_cgemm_strided_batched_4096x64_rowNC": lambda: ComplexWorkload("cgemm_batched", "C", NO, 113, 64, 64, 64, 1.0 - 0.5j,
