@@ -281,8 +281,10 @@ struct RealSlabLoader {
   }
 };
 
+// (the register budget is set for many wavefronts per SIMD: what hides the latencies here is other work-groups)
 template <typename T, int BLOCKS, bool A_KC, bool B_KC>
-__global__ __launch_bounds__(kComplexSmallThreads) void GemmSmallTiledKernel(const GemmArgs<T> p, const int tiles_m,
+__global__ __launch_bounds__(kComplexSmallThreads, sizeof(T) == 8 ? (BLOCKS == 2 ? 3 : 6) : (BLOCKS == 2 ? 4 : 8))
+void GemmSmallTiledKernel(const GemmArgs<T> p, const int tiles_m,
                                                                              const int tiles_n) {
   using Traits = typename ComplexSmallTraits<T>::Mfma;
   using Acc = typename Traits::Acc;
