@@ -32,7 +32,7 @@ bool UseSmallKernel(const size_t rows, const size_t columns, const size_t k, con
   if (rows > kSmallExtent || columns > kSmallExtent || ForcedTileVariant(precision) != 0) { return false; }
   // a few work-groups walking a long k alone are slower than the real kernels, which split such a k
   const auto groups = CeilDiv(rows, size_t{64}) * CeilDiv(columns, size_t{64}) * batch_count;
-  return groups >= 512 || k <= 256;
+  return groups >= 512 || k <= 64;
 }
 
 clbh_complex_small_operand SmallOperand(const BatchedOperand& operand, const long long* device_offsets) {

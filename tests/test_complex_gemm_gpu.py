@@ -88,7 +88,7 @@ SCALARS = ((1.0, 0.0), (0.5 - 1.5j, 2.0 + 0.25j), (-1j, 1.0), (2.0, -0.5), (0.0,
 def test_complex_gemm_sweep(gpu, bits):
     seed = 13000
     for layout, ta, tb in MODES:
-        for m, n, k in ((7, 7, 7), (7, 64, 7), (64, 7, 64), (64, 64, 64), (33, 17, 65), (130, 65, 129), (1, 1, 1), (200, 3, 40)):
+        for m, n, k in ((7, 7, 7), (7, 64, 7), (64, 7, 64), (64, 64, 64), (33, 17, 65), (130, 65, 129), (1, 1, 1), (200, 3, 40), (100, 90, 30)):
             seed += 1
             extra, offsets = (((0, 0, 0), (0, 0, 0)), ((3, 1, 2), (10, 10, 10)), ((1, 0, 5), (1, 3, 7)))[seed % 3]
             alpha, beta = SCALARS[seed % len(SCALARS)]
