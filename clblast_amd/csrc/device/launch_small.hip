@@ -2,7 +2,7 @@
 // Small-matrix batched kernel instantiations (fp32, fp64, fp16).
 // =================================================================================================
 #include "device/launch_common.hpp"
-#include "kernels/gemm_complex_small.hpp"
+#include "kernels/gemm_small_tiled.hpp"
 #include "kernels/gemm_small_batched.hpp"
 
 namespace clbh {

@@ -1,5 +1,10 @@
 // =================================================================================================
-// Batched complex GEMM of small matrices on gfx950, on interleaved (re, im) data as it lies in memory. It serves the
+// Batched GEMMs of matrices of a few tiles on gfx950: GemmComplexSmallKernel (complex64 / complex128, below) and
+// GemmSmallTiledKernel (fp32 / fp64, at the end of the file). Both keep ONE slab of k = 16 per operand in LDS, so that
+// many work-groups share a CU and hide each other's latencies, load the next slab into registers under the products of
+// the current one, and use the 16 x 16 x 4 matrix instructions.
+//
+// Batched complex GEMM of small matrices, on interleaved (re, im) data as it lies in memory. It serves the
 // shapes for which the reference launches XgemmDirectBatched / XgemmDirectStridedBatched on float2 / double2
 // (src/kernels/level3/xgemm_direct_batched.opencl:24-212 with the complex MultiplyAdd of
 // src/kernels/common.opencl:244-251). Such a batch is bound by HBM bandwidth, so every operand is read once and C is
@@ -10,8 +15,8 @@
 // (the minus sign and the conjugations are applied to the imaginary plane when it is read or stored).
 // The canonical problem is column-major: C'(rows x columns) = alpha * L(rows x k) * R(k x columns) + beta * C'.
 // =================================================================================================
-#ifndef CLBLAST_HIP_KERNELS_GEMM_COMPLEX_SMALL_HPP_
-#define CLBLAST_HIP_KERNELS_GEMM_COMPLEX_SMALL_HPP_
+#ifndef CLBLAST_HIP_KERNELS_GEMM_SMALL_TILED_HPP_
+#define CLBLAST_HIP_KERNELS_GEMM_SMALL_TILED_HPP_
 
 #include "kernels/gemm_mfma.hpp"
 
@@ -364,4 +369,4 @@ void GemmSmallTiledKernel(const GemmArgs<T> p, const int tiles_m,
 
 }  // namespace clbh
 
-#endif  // CLBLAST_HIP_KERNELS_GEMM_COMPLEX_SMALL_HPP_
+#endif  // CLBLAST_HIP_KERNELS_GEMM_SMALL_TILED_HPP_
