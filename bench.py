@@ -32,7 +32,8 @@ DTYPE_NAME = {"S": "f32", "D": "f64", "H": "f16", "C": "c64 (f32 arithmetic)", "
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
 # the readings of a plain 1 GiB copy (profiles/<workload>.md holds the commands and the raw readings). A bench run
 # cannot collect counters itself, so these are the figures of the committed profiles.
-MEASURED_TRAFFIC_BYTES = {"cfg2s": 5.602e9, "cfg2d": 1.0697e10, "cfg3": 1.888e9, "cfg4": 1.007e8, "cfg5d": 6.319e8}
+MEASURED_TRAFFIC_BYTES = {"cfg2s": 5.602e9, "cfg2d": 1.0697e10, "cfg3": 1.888e9, "cfg4": 1.007e8, "cfg5d": 6.319e8, "sbat64": 2.014e8,
+                          "cgemm_batched": 4.028e8}
 
 
 def parse_args():
