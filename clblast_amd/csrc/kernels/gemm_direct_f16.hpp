@@ -5,11 +5,13 @@
 // src/kernels/level3/xgemm_part1-4.opencl) and its direct kernels (xgemm_direct_part1-3.opencl) with
 // one launch that reads the caller's operands in place. Unlike the reference, which accumulates in
 // fp16 (src/kernels/common.opencl:44-45), products are accumulated in fp32 by
-// v_mfma_f32_32x32x16_f16 and rounded to fp16 once, in the epilogue.
+// v_mfma_f32_16x16x32_f16 and rounded to fp16 once, in the epilogue. (Of the two fp16 shapes of gfx950 this one
+// draws less power per flop: on uniform random operands a loop of nothing but MFMAs sustains 1.97 PFLOP/s with
+// 16x16x32 and 1.71 PFLOP/s with 32x32x16 under the same power cap, and large HGEMMs run against that cap.)
 //
 // Structure:
-//   * work-group tile (32*WM*FM) x (32*WN*FN), one wavefront per FM x FN blocks of 32 x 32; K is walked
-//     in slabs of 32 that live in a ring of three LDS buffers;
+//   * work-group tile (32*WM*FM) x (32*WN*FN), one wavefront per 2FM x 2FN blocks of 16 x 16; K is walked
+//     in slabs of 32 - one MFMA deep - that live in a ring of LDS buffers;
 //   * every slab goes global -> LDS directly (`buffer_load_dwordx4 ... lds`: lane l's 16 bytes land at
 //     base + 16 * l, so LDS is filled in 1 KiB pieces whose inner order is fixed, while which 16 bytes of
 //     global memory a lane fetches is free - that freedom carries the bank swizzles). The resources
@@ -17,16 +19,19 @@
 //     tiles and the K tail of an x-contiguous operand need nothing special; the K tail of a
 //     k-contiguous operand (whose out-of-range elements are the next line's data) is zeroed in LDS by
 //     the wavefront that requested the piece;
-//   * the MFMA wants 8 consecutive k per lane. A k-contiguous operand is kept as [x][32] (16-byte chunk c
-//     of row x at position c ^ ((x >> 2) & 3): the 16-byte reads of 16 consecutive rows cover all 64 banks
-//     once) and read with one ds_read_b128 per fragment. An x-contiguous operand is kept as [k][W] (chunk t
-//     of row k at t ^ swizzle(k)) and read with the CDNA4 transposing LDS read ds_read_b64_tr_b16. LDS
-//     serves 32 lanes of such a read per cycle: rows k..k+3, 64 bytes each, which the swizzle spreads
-//     over four different 16-dword bank windows;
-//   * explicit schedule, fenced for the compiler: per quarter of a k-step "LDS reads of the fragments of
-//     the next k-step (other register set), FN MFMAs, a share of the requests for slab t+2"; one barrier
-//     per slab, before its last k-step, so that the last k-step already fetches the first fragments of
-//     slab t+1 and the matrix pipe never drains at a slab boundary;
+//   * the MFMA wants 8 consecutive k per lane (lane l: row l % 16, k = 8 * (l / 16) ..). A k-contiguous
+//     operand is kept as [x][32] (16-byte chunk c of row x at position c ^ ((x >> 2) & 3): the 16-byte reads
+//     of 16 consecutive rows cover all 64 banks once) and read with one ds_read_b128 per fragment. An
+//     x-contiguous operand is kept as [k][W] (chunk t of row k at t ^ swizzle(k)) and read with the CDNA4
+//     transposing LDS read ds_read_b64_tr_b16. LDS serves 32 lanes of such a read per cycle: rows k..k+3 and
+//     k+8..k+11, 32 bytes each, which the swizzle spreads over eight different 8-dword bank windows;
+//   * explicit schedule, fenced for the compiler. The wavefront's blocks form four quadrants (halves of
+//     its A blocks x halves of its B blocks) that are multiplied in the order (A0,B0) (A0,B1) (A1,B0) (A1,B1);
+//     under the MFMAs of a quadrant the fragments that the next one lacks are read - B1, A1, then A0 and B0
+//     of the next slab - so every fragment register is refilled right after its last use and no second
+//     register set is needed. One barrier per slab, after the second quadrant, when all reads of the slab
+//     have been issued: the second half of a slab already fetches the first fragments of the next one and
+//     the matrix pipe never drains at a slab boundary;
 //   * the m-indexed fragment is the MFMA's A operand, so a lane holds runs of four consecutive m; the
 //     epilogue stages each block column through LDS and moves C in 16-byte pieces along m.
 // =================================================================================================
@@ -42,12 +47,14 @@
 namespace clbh {
 
 // WM x WN wavefronts per work-group, each owning FM x FN MFMA blocks of 32 x 32 (FM >= FN). MIN_WAVES is the
-// number of wavefronts per SIMD the register budget must allow.
-template <int WM_, int WN_, int FM_, int FN_, int MIN_WAVES_>
+// number of wavefronts per SIMD the register budget must allow. STAGES slab buffers form the LDS ring: the slab
+// STAGES - 1 ahead of the one being multiplied is on its way from memory.
+template <int WM_, int WN_, int FM_, int FN_, int MIN_WAVES_, int STAGES_ = 3, bool STAGGER_ = false>
 struct HdirectConfig {
+  static constexpr bool STAGGER = STAGGER_;
   static constexpr int WM = WM_, WN = WN_, FM = FM_, FN = FN_, MIN_WAVES = MIN_WAVES_;
   static constexpr int WAVES = WM * WN, THREADS = 64 * WAVES;
-  static constexpr int TILE_M = WM * FM * 32, TILE_N = WN * FN * 32, TILE_K = 32, STAGES = 3;
+  static constexpr int TILE_M = WM * FM * 32, TILE_N = WN * FN * 32, TILE_K = 32, STAGES = STAGES_;
   static constexpr int PIECES_A = TILE_M / 16, PIECES_B = TILE_N / 16;  // 1 KiB pieces of a slab
   static constexpr int ROUNDS = (PIECES_A + PIECES_B + WAVES - 1) / WAVES;  // requests per wavefront and slab
   static constexpr bool DUMMY = (PIECES_A + PIECES_B) % WAVES != 0;  // some requests go to a scratch piece
@@ -58,11 +65,12 @@ struct HdirectConfig {
   static_assert(FM >= FN, "the quarters of a k-step run over the m blocks");
 };
 
-// Chunk swizzle of row k of an x-contiguous slab [k][W]: rows k..k+3 must fall into different 16-dword
-// bank windows for a 64-byte read per row.
+// Chunk swizzle of row k of an x-contiguous slab [k][W]: one cycle of a transposing read takes 32 bytes from each
+// of the rows k..k+3 and k+8..k+11 (k a multiple of 4), which must fall into eight different 8-dword bank windows.
 template <int W>
 __device__ __forceinline__ int HSwizzle(const int k) {
-  return (W >= 128) ? 4 * (k & 3) : (W == 64) ? 4 * ((k >> 1) & 1) : 0;
+  const int by_octet = 2 * ((k >> 3) & 1);
+  return by_octet ^ ((W >= 128) ? 4 * (k & 3) : (W == 64) ? 4 * ((k >> 1) & 1) : 0);
 }
 
 // Byte count from `from` to `end`, rounded up to whole dwords (the range check works per dword; the last
@@ -144,31 +152,33 @@ __device__ __forceinline__ void HZeroTail(_Float16* stage, const int piece, cons
   }
 }
 
-// Offset (halfs) of a lane's fragment data for the block starting at x32 (a multiple of 32), k-step 0.
+// Offset (halfs) of a lane's fragment data for the block starting at x16 (a multiple of 16): the lane feeds row
+// x16 + lane % 16 with k = 8 * (lane / 16) .. + 7.
 template <int W, bool KC>
-__device__ __forceinline__ int HFragmentOffset(const int lane, const int x32) {
+__device__ __forceinline__ int HFragmentOffset(const int lane, const int x16) {
   if (KC) {
-    const int x = x32 + lane % 32;
-    return x * 32 + 8 * ((lane / 32) ^ ((x >> 2) & 3));
+    const int x = x16 + lane % 16;
+    return x * 32 + 8 * ((lane / 16) ^ ((x >> 2) & 3));
   } else {
+    // a group of 16 lanes reads a 4 (k) x 16 (x) block, four consecutive x per lane, and gets it back transposed:
+    // lane q of the group then holds four consecutive k of column q
     const int group = lane / 16, q = lane % 16;
-    const int k = 8 * (group / 2) + q / 4;
-    const int x = x32 + 16 * (group % 2) + 4 * (q % 4);
+    const int k = 8 * group + q / 4;
+    const int x = x16 + 4 * (q % 4);
     return k * W + 8 * ((x / 8) ^ HSwizzle<W>(k)) + x % 8;
   }
 }
 
-// Fragment of k-step ks (0 or 1) of a stage.
+// Fragment of a stage.
 template <int W, bool KC>
-__device__ __forceinline__ half8_t HFragment(const _Float16* __restrict__ stage, const int offset, const int ks) {
+__device__ __forceinline__ half8_t HFragment(const _Float16* __restrict__ stage, const int offset) {
   if (KC) {
-    // chunk index of the k-step is 2*ks + lane/32; the swizzle is an XOR, so k-step 1 flips bit 1 of it
-    return *reinterpret_cast<const half8_t*>(&stage[offset ^ (ks * 16)]);
+    return *reinterpret_cast<const half8_t*>(&stage[offset]);
   } else {
     typedef __attribute__((address_space(3))) short4_t* LdsPtr;
-    const _Float16* src = stage + ks * 16 * W + offset;  // rows k + 16 * ks: the swizzle depends on k % 4 only
+    const _Float16* src = stage + offset;
     const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(src));
-    const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(src + 4 * W));
+    const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(src + 4 * W));  // rows k + 4: the same swizzle
     half8_t out;
     const half4_t lo_h = __builtin_bit_cast(half4_t, lo), hi_h = __builtin_bit_cast(half4_t, hi);
 #pragma unroll
@@ -185,8 +195,10 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
   using T = _Float16;
   constexpr int TILE_M = Config::TILE_M, TILE_N = Config::TILE_N, TILE_K = Config::TILE_K;
   constexpr int FM = Config::FM, FN = Config::FN, WAVES = Config::WAVES, STAGES = Config::STAGES, ROUNDS = Config::ROUNDS;
-  constexpr int KSTEPS = TILE_K / 16;
-  static_assert(KSTEPS == 2 && STAGES == 3, "schedule below: one barrier after the first of two k-steps, ring of three");
+  constexpr int BM = 2 * FM, BN = 2 * FN;  // the wavefront's blocks of 16 x 16
+  constexpr int AHEAD = STAGES - 1;        // slabs on their way or landed beyond the current one, in the steady state
+  static_assert(TILE_K == 32 && (STAGES == 3 || STAGES == 4), "a slab is one MFMA deep; the waits below count up to three slabs");
+  typedef float float4_t __attribute__((ext_vector_type(4)));
   static_assert(!A_CONV || !A_KC, "a gathered operand is x-contiguous in LDS");
   using KernelTag = std::tuple<Config, std::integral_constant<int, (A_CONV ? 4 : 0) | (A_KC ? 2 : 0) | (B_KC ? 1 : 0)>>;
 
@@ -211,11 +223,11 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
   if (TileOutsideTriangle(p.c_triangle, m0, n0, TILE_M, TILE_N)) { return; }  // uniform: the whole work-group leaves
   const bool masked = TileCrossesDiagonal(p.c_triangle, m0, n0, TILE_M, TILE_N);
 
-  int a_offset[FM], b_offset[FN];
+  int a_offset[BM], b_offset[BN];
 #pragma unroll
-  for (int q = 0; q < FM; ++q) { a_offset[q] = HFragmentOffset<TILE_M, A_KC>(lane, (wave_m * FM + q) * 32); }
+  for (int q = 0; q < BM; ++q) { a_offset[q] = HFragmentOffset<TILE_M, A_KC>(lane, (wave_m * BM + q) * 16); }
 #pragma unroll
-  for (int q = 0; q < FN; ++q) { b_offset[q] = HFragmentOffset<TILE_N, B_KC>(lane, (wave_n * FN + q) * 32); }
+  for (int q = 0; q < BN; ++q) { b_offset[q] = HFragmentOffset<TILE_N, B_KC>(lane, (wave_n * BN + q) * 16); }
 
   for (int batch = blockIdx.y; batch < p.batch_count; batch += gridDim.y) {
     const T* a;
@@ -238,11 +250,11 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
     const int slabs = (k_len + TILE_K - 1) / TILE_K;
     const int k_tail = k_len % TILE_K;  // valid depth of the last slab when it is partial
 
-    float16_t acc[FM][FN];
+    float4_t acc[BM][BN];
 #pragma unroll
-    for (int i = 0; i < FM; ++i) {
+    for (int i = 0; i < BM; ++i) {
 #pragma unroll
-      for (int j = 0; j < FN; ++j) { acc[i][j] = float16_t(0.0f); }
+      for (int j = 0; j < BN; ++j) { acc[i][j] = float4_t(0.0f); }
     }
 
     const T* a_tile0 = a + (A_KC ? m0 * p.a_ld : static_cast<long long>(m0));  // element (m0, k = 0), uniform
@@ -332,80 +344,117 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
         }
       };
 
-      // Prologue: slab 0 lands in ring position 0, slab 1 is requested.
+      // Prologue: the first AHEAD slabs are requested into ring positions 0, 1, ...; slab 0 must have landed.
+      const int first_slabs = min(slabs, AHEAD);
 #pragma unroll
-      for (int round = 0; round < ROUNDS; ++round) { request(round, 0); }
-      next_request_slab();
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      if (slabs == 1) { zero_tail(0); }
-      if (slabs > 1) {
+      for (int s = 0; s < AHEAD; ++s) {
+        if (s < first_slabs) {
 #pragma unroll
-        for (int round = 0; round < ROUNDS; ++round) { request(round, 1); }
-        next_request_slab();
+          for (int round = 0; round < ROUNDS; ++round) { request(round, s); }
+          next_request_slab();
+        }
       }
+      if (first_slabs == 1) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+      else if (first_slabs == 2) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(ROUNDS) : "memory"); }
+      else { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * ROUNDS) : "memory"); }
+      if (slabs == 1) { zero_tail(0); }
       __syncthreads();
+      // Fragments: the halves A0, A1 of the wavefront's A blocks and B0, B1 of its B blocks, one register set each
       half8_t a_frag[2][FM], b_frag[2][FN];
 #pragma unroll
-      for (int q = 0; q < FM; ++q) { a_frag[0][q] = HFragment<TILE_M, A_KC>(a_ring, a_offset[q], 0); }
+      for (int q = 0; q < FM; ++q) { a_frag[0][q] = HFragment<TILE_M, A_KC>(a_ring, a_offset[q]); }
 #pragma unroll
-      for (int q = 0; q < FN; ++q) { b_frag[0][q] = HFragment<TILE_N, B_KC>(b_ring, b_offset[q], 0); }
-      int cur = 0;  // ring position of the current slab; slab + 1 is in the next one, slab + 2 goes into the one before
-      // One slab. NEXT: slab + 1 exists; LOAD: slab + 2 exists and is requested into the buffer that the barrier of
-      // the previous slab released. Compile-time, so that the steady state has no branches.
-      constexpr int PER_QUARTER = (ROUNDS + FM - 1) / FM;
-      auto slab_body = [&](const int slab, auto next_tag, auto load_tag) {
-        constexpr bool NEXT = decltype(next_tag)::value, LOAD = decltype(load_tag)::value;
+      for (int q = 0; q < FN; ++q) { b_frag[0][q] = HFragment<TILE_N, B_KC>(b_ring, b_offset[q]); }
+      int cur = 0;  // ring position of the current slab; slab + s is s positions on, slab + AHEAD goes into the one before
+      // One slab. LATER (compile-time, so that the steady state has no branches): how many slabs follow this one, capped
+      // at AHEAD. LATER == AHEAD: slab + AHEAD exists and is requested into the buffer that the barrier of the previous
+      // slab released.
+      // Ring of three: slab + 2 is requested under the first two quadrants, into the buffer whose reads everybody had
+      // finished (waited for) at the previous barrier. Ring of four: slab + 3 is requested under the last two quadrants,
+      // after this slab's barrier, into the buffer of slab - 1 - every wavefront has consumed its last fragments of that
+      // slab before it reached this barrier, so the barrier need not wait for LDS reads and their latency stays hidden.
+      constexpr int REQUEST_QUADRANT = (STAGES == 4) ? 2 : 0;
+      // STAGGER: the two halves of the work-group issue their requests under different quadrants. (Wavefronts issue in
+      // order and a 1 KiB request occupies the memory pipeline's front end for 16 cycles: when all wavefronts reach a
+      // request in the same cycles, the last one in the queue cannot issue its next MFMAs for 100 cycles.)
+      constexpr int REQUEST_SLOTS = Config::STAGGER ? FM : 2 * FM;  // MFMA groups that carry a share of the requests each
+      constexpr int PER_SLOT = (ROUNDS + REQUEST_SLOTS - 1) / REQUEST_SLOTS;
+      auto slab_body = [&](auto later_tag, auto phase_tag) {
+        constexpr int LATER = decltype(later_tag)::value;
+        constexpr int PHASE = decltype(phase_tag)::value;
+        constexpr bool LOAD = LATER == AHEAD;
         const int nxt = (cur == STAGES - 1) ? 0 : cur + 1, prv = (cur == 0) ? STAGES - 1 : cur - 1;
         const T* a_cur = a_ring + cur * Config::A_ELEMS;
         const T* b_cur = b_ring + cur * Config::B_ELEMS;
         const T* a_nxt = a_ring + nxt * Config::A_ELEMS;
         const T* b_nxt = b_ring + nxt * Config::B_ELEMS;
+        // quadrant (A half ha, B half hb); under its MFMAs the fragments the next quadrant lacks are read: B1, A1 (this
+        // slab), then A0, B0 (next slab)
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          const int set = ks % 2;
-          const T* a_src = (ks + 1 < KSTEPS) ? a_cur : a_nxt;
-          const T* b_src = (ks + 1 < KSTEPS) ? b_cur : b_nxt;
-          const int ks_src = (ks + 1 < KSTEPS) ? ks + 1 : 0;
+        for (int quadrant = 0; quadrant < 4; ++quadrant) {
+          const int ha = quadrant / 2, hb = quadrant % 2;
 #pragma unroll
           for (int q = 0; q < FM; ++q) {
-            a_frag[set ^ 1][q] = HFragment<TILE_M, A_KC>(a_src, a_offset[q], ks_src);
-            if (q < FN) { b_frag[set ^ 1][q] = HFragment<TILE_N, B_KC>(b_src, b_offset[q], ks_src); }
+            // the reads of a quadrant go with its first groups of MFMAs, one fragment each
+            if (quadrant == 0 || quadrant == 3) {
+              if (q < FN) {
+                if (quadrant == 0) { b_frag[1][q] = HFragment<TILE_N, B_KC>(b_cur, b_offset[FN + q]); }
+                else { b_frag[0][q] = HFragment<TILE_N, B_KC>(b_nxt, b_offset[q]); }
+              }
+            } else if (quadrant == 1) {
+              a_frag[1][q] = HFragment<TILE_M, A_KC>(a_cur, a_offset[FM + q]);
+            } else {
+              a_frag[0][q] = HFragment<TILE_M, A_KC>(a_nxt, a_offset[q]);
+            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
-              acc[q][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag[set][q], b_frag[set][j], acc[q][j], 0, 0, 0);
+              acc[ha * FM + q][hb * FN + j] =
+                  __builtin_amdgcn_mfma_f32_16x16x32_f16(a_frag[ha][q], b_frag[hb][j], acc[ha * FM + q][hb * FN + j], 0, 0, 0);
             }
-            // spread over the quarters: a burst of identical requests from all work-groups defeats the L2
-            if (LOAD && ks == 0) {
+            // spread over the groups: a burst of identical requests from all work-groups defeats the L2
+            if (LOAD && (Config::STAGGER ? quadrant == REQUEST_QUADRANT + PHASE
+                                         : (quadrant >= REQUEST_QUADRANT && quadrant < REQUEST_QUADRANT + 2))) {
 #pragma unroll
-              for (int u = 0; u < PER_QUARTER; ++u) {
-                if (q * PER_QUARTER + u < ROUNDS) { request(q * PER_QUARTER + u, prv); }
+              for (int u = 0; u < PER_SLOT; ++u) {
+                const int round = ((Config::STAGGER ? 0 : quadrant - REQUEST_QUADRANT) * FM + q) * PER_SLOT + u;
+                if (round < ROUNDS) { request(round, prv); }
               }
             }
             __builtin_amdgcn_sched_barrier(0);
           }
-          if (ks == KSTEPS - 2) {
-            // slab + 1 must have landed for everybody; this slab's own requests (slab + 2) may stay in flight
-            if (LOAD) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(ROUNDS) : "memory"); }
-            else { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-            if (NEXT && !LOAD) { zero_tail(nxt); }  // slab + 1 is the last one
-            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+          if (quadrant == 1) {
+            // slab + 1 must have landed for everybody; the requests for the slab behind it may stay in flight
+            constexpr int IN_FLIGHT = (LATER >= 2) ? ROUNDS : 0;
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IN_FLIGHT) : "memory");
+            if (LATER == 1) { zero_tail(nxt); }  // slab + 1 is the last one
+            // (the zeroed tail must be in LDS, not on its way, when the others pass the barrier)
+            if (STAGES == 4 && LATER != 1) { asm volatile("s_barrier" ::: "memory"); }
+            else { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
           }
         }
         cur = nxt;
         if (LOAD) { next_request_slab(); }
       };
       int slab = 0;
-      for (; slab + 2 < slabs; ++slab) { slab_body(slab, std::true_type{}, std::true_type{}); }
-      if (slab + 1 < slabs) { slab_body(slab, std::true_type{}, std::false_type{}); ++slab; }
-      slab_body(slab, std::false_type{}, std::false_type{});
+      using Phase0 = std::integral_constant<int, 0>;
+      if (Config::STAGGER && wave_u >= WAVES / 2) {
+        for (; slab + AHEAD < slabs; ++slab) { slab_body(std::integral_constant<int, AHEAD>{}, std::integral_constant<int, 1>{}); }
+      } else {
+        for (; slab + AHEAD < slabs; ++slab) { slab_body(std::integral_constant<int, AHEAD>{}, Phase0{}); }
+      }
+      if constexpr (AHEAD >= 3) {
+        if (slab + 2 < slabs) { slab_body(std::integral_constant<int, 2>{}, Phase0{}); ++slab; }
+      }
+      if (slab + 1 < slabs) { slab_body(std::integral_constant<int, 1>{}, Phase0{}); ++slab; }
+      slab_body(std::integral_constant<int, 0>{}, Phase0{});
     };
     if (m0 + TILE_M <= p.m && n0 + TILE_N <= p.n && k_tail == 0) { walk(std::false_type{}); }
     else { walk(std::true_type{}); }
 
-    // Epilogue, staged through LDS so that global memory sees whole lines. Accumulator elements 4g..4g+3 of a
-    // lane are the rows m = 8g + 4*(lane/32) + 0..3 of column n = lane%32 of the 32 x 32 block. Per block
-    // column j a wavefront owns a [32 n][WAVE_M m] fp16 staging tile of its own: C (when beta != 0) comes in
+    // Epilogue, staged through LDS so that global memory sees whole lines. The four accumulator elements of a
+    // lane are the rows m = 4*(lane/16) + 0..3 of column n = lane%16 of a 16 x 16 block. Per pair j of block
+    // columns a wavefront owns a [32 n][WAVE_M m] fp16 staging tile of its own: C (when beta != 0) comes in
     // with 16-byte accesses along m, every lane combines its four consecutive m in fp32 and rounds once, and
     // the finished rows leave with 16-byte stores. Only wavefront-local ordering is needed (LDS operations of
     // a wavefront complete in order).
@@ -415,19 +464,16 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
       float* partial = static_cast<float*>(p.split_workspace) + static_cast<long long>(batch) * p.split_ld * p.n;
       typedef float float4u_t __attribute__((ext_vector_type(4)));
 #pragma unroll
-      for (int j = 0; j < FN; ++j) {
-        const int n_index = n0 + (wave_n * FN + j) * 32 + lane % 32;
+      for (int j = 0; j < BN; ++j) {
+        const int n_index = n0 + (wave_n * BN + j) * 16 + lane % 16;
 #pragma unroll
-        for (int i = 0; i < FM; ++i) {
+        for (int i = 0; i < BM; ++i) {
+          const int m_index = m0 + (wave_m * BM + i) * 16 + 4 * (lane / 16);
+          if (n_index < p.n && m_index < p.split_ld) {
+            float4u_t out;
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const int m_index = m0 + (wave_m * FM + i) * 32 + 8 * g + 4 * (lane / 32);
-            if (n_index < p.n && m_index < p.split_ld) {
-              float4u_t out;
-#pragma unroll
-              for (int e = 0; e < 4; ++e) { out[e] = acc[i][j][4 * g + e]; }
-              *reinterpret_cast<float4u_t*>(partial + static_cast<long long>(n_index) * p.split_ld + m_index) = out;
-            }
+            for (int e = 0; e < 4; ++e) { out[e] = acc[i][j][e]; }
+            *reinterpret_cast<float4u_t*>(partial + static_cast<long long>(n_index) * p.split_ld + m_index) = out;
           }
         }
       }
@@ -484,18 +530,18 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
             wave_fence();
           }
 #pragma unroll
-          for (int i = 0; i < FM; ++i) {
+          for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-              half4_t* cell = reinterpret_cast<half4_t*>(&stage[(lane % 32) * STAGE_PITCH + 32 * i + 8 * g + 4 * (lane / 32)]);
+            for (int i = 0; i < BM; ++i) {
+              half4_t* cell = reinterpret_cast<half4_t*>(&stage[(16 * jj + lane % 16) * STAGE_PITCH + 16 * i + 4 * (lane / 16)]);
               half4_t out;
               if (beta != 0.0f) {
                 const half4_t old = *cell;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { out[e] = static_cast<T>(alpha * acc[i][j][4 * g + e] + beta * static_cast<float>(old[e])); }
+                for (int e = 0; e < 4; ++e) { out[e] = static_cast<T>(alpha * acc[i][2 * j + jj][e] + beta * static_cast<float>(old[e])); }
               } else {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { out[e] = static_cast<T>(alpha * acc[i][j][4 * g + e]); }
+                for (int e = 0; e < 4; ++e) { out[e] = static_cast<T>(alpha * acc[i][2 * j + jj][e]); }
               }
               *cell = out;
             }

@@ -247,6 +247,12 @@ CLBH_API int clbh_buffer_extent(const void* ptr, size_t* bytes_available);
 CLBH_API int clbh_alloc_async(void** ptr, size_t bytes, hipStream_t stream);
 CLBH_API int clbh_free_async(void* ptr, hipStream_t stream);
 
+// Scratch memory that needs no allocation: every GPU holds one array of clbh_static_scratch_bytes() bytes (256-byte
+// aligned) from the loading of the library's code object on. The first call for a device asks the runtime for the
+// address of that device's copy. All callers on one GPU share it; its contents survive from call to call.
+CLBH_API size_t clbh_static_scratch_bytes(void);
+CLBH_API int clbh_static_scratch(int device, void** pointer);
+
 // Stream-ordered host-to-device copy of a small array; the host memory may be reused on return.
 CLBH_API int clbh_upload_async(void* dst_device, const void* src_host, size_t bytes, hipStream_t stream);
 
