@@ -3,4 +3,4 @@ from .api import (CLBlastError, COL_MAJOR, CONVOLUTION, CROSS_CORRELATION, DIAGO
                   TRIANGLE_LOWER, TRIANGLE_UPPER, clear_cache,
                   float_to_half_bits, gemm, gemmBatched, gemmStridedBatched, half_bits_to_float, hemm, her2k, herk,
                   override_parameters, raw_complex_gemm, raw_complex_level3, raw_convgemm, raw_gemm, raw_gemm_batched, raw_gemm_strided_batched,
-                  raw_gemm_temp_buffer_size, raw_symm, raw_syr2k, raw_syrk, raw_trmm, raw_trsm, symm, syr2k, syrk, trmm, trsm)
+                  raw_gemm_temp_buffer_size, raw_sgemm_no_alloc, raw_symm, raw_syr2k, raw_syrk, raw_trmm, raw_trsm, symm, syr2k, syrk, trmm, trsm)

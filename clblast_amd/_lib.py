@@ -67,6 +67,8 @@ def _declare(lib):
         f.argtypes, f.restype = gemm_args, c_int
         f = getattr(lib, "CLBlast%sgemmWithTempBuffer" % prefix)
         f.argtypes, f.restype = gemm_args + [vp], c_int
+        if prefix == "S":
+            lib.CLBlastSgemmNoAlloc.argtypes, lib.CLBlastSgemmNoAlloc.restype = gemm_args, c_int
         f = getattr(lib, "CLBlast%sgemmBatched" % prefix)
         f.argtypes = [c_int, c_int, c_int, sz, sz, sz, POINTER(scalar), vp, POINTER(sz), sz, vp, POINTER(sz), sz,
                       POINTER(scalar), vp, POINTER(sz), sz, sz, vp, vp]
@@ -120,7 +122,7 @@ C_API_SYMBOLS = (
     ["CLBlast%s%s" % (p, r) for p in "CZ" for r in ("symm", "hemm", "syrk", "herk", "syr2k", "her2k", "trmm", "trsm")] +
     ["CLBlast%s%s" % (p, r) for p in "SDH" for r in ("symm", "syrk", "syr2k", "trmm")] + ["CLBlastStrsm", "CLBlastDtrsm"] +
     ["CLBlast%sconvgemm" % p for p in "SDH"] +
-    ["CLBlastClearCache", "CLBlastOverrideParameters", "CLBlastFloatToHalf", "CLBlastHalfToFloat"])
+    ["CLBlastSgemmNoAlloc", "CLBlastClearCache", "CLBlastOverrideParameters", "CLBlastFloatToHalf", "CLBlastHalfToFloat"])
 NETLIB_SYMBOLS = (["cblas_%sgemm" % p for p in "sdcz"] +
                   ["cblas_%s%s" % (p, r) for p in "sdcz" for r in ("symm", "syrk", "syr2k", "trmm", "trsm")] +
                   ["cblas_%s%s" % (p, r) for p in "cz" for r in ("hemm", "herk", "her2k")])
@@ -131,4 +133,4 @@ DEVICE_LAYER_SYMBOLS = [
     "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale", "clbh_complex_expand_batched",
     "clbh_complex_transpose_batched", "clbh_complex_scale_batched", "clbh_complex_gemm_small_batched", "clbh_copy_matrix_batched", "clbh_alloc", "clbh_free", "clbh_copy", "clbh_im2col", "clbh_conv_gather_possible", "clbh_pad_image", "clbh_fill_zero", "clbh_complex_symmetric_to_square",
     "clbh_complex_triangular_to_square", "clbh_complex_zero_diagonal_imag", "clbh_complex_invert_block_size",
-    "clbh_complex_invert_diagonal_blocks"]
+    "clbh_complex_invert_diagonal_blocks", "clbh_static_scratch", "clbh_static_scratch_bytes"]

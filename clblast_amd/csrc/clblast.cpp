@@ -5,6 +5,7 @@
 // :1630-1647 (GemmStridedBatched), :1682-1708 (GemmTempBufferSize) and src/api_common.cpp:25-33,
 // 140-221 (ClearCache, RetrieveParameters, OverrideParameters).
 // =================================================================================================
+#include <string>
 #include <vector>
 
 #include "clblast_hip.h"
@@ -36,6 +37,38 @@ StatusCode Gemm(const Layout layout, const Transpose a_transpose, const Transpos
     routine.DoGemm(layout, a_transpose, b_transpose, m, n, k, alpha, Buffer<T>(a_buffer), a_offset, a_ld,
                    Buffer<T>(b_buffer), b_offset, b_ld, beta, Buffer<T>(c_buffer), c_offset, c_ld,
                    Buffer<T>(temp_buffer), temp_buffer_provided);
+    return StatusCode::kSuccess;
+  } catch (...) {
+    return DispatchException();
+  }
+}
+
+// fp32 GEMM that allocates nothing: the temporary buffer is the static scratch array of the stream's GPU, and a problem
+// whose split-K workspace does not fit it is refused.
+CLBLAST_HIP_PUBLIC StatusCode GemmNoAlloc(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
+                       const size_t n, const size_t k, const float alpha, const void* a_buffer, const size_t a_offset,
+                       const size_t a_ld, const void* b_buffer, const size_t b_offset, const size_t b_ld,
+                       const float beta, void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                       hipEvent_t* event) {
+  try {
+    auto routine = Xgemm<float>(queue, event);
+    auto device = 0;
+    CheckDevice(clbh_stream_device(*queue, &device), "clbh_stream_device");
+    void* scratch = nullptr;
+    CheckDevice(clbh_static_scratch(device, &scratch), "clbh_static_scratch");
+    const auto scratch_bytes = clbh_static_scratch_bytes();
+    try {
+      routine.DoGemm(layout, a_transpose, b_transpose, m, n, k, alpha, Buffer<float>(a_buffer), a_offset, a_ld,
+                     Buffer<float>(b_buffer), b_offset, b_ld, beta, Buffer<float>(c_buffer), c_offset, c_ld,
+                     Buffer<float>(scratch, scratch_bytes), true);
+    } catch (const BLASError& e) {
+      if (e.status() == StatusCode::kInsufficientMemoryTemp) {
+        throw RuntimeErrorCode(StatusCode::kInsufficientMemoryTemp,
+                               "SgemmNoAlloc: this problem's split-K workspace exceeds the static scratch array of " +
+                                   std::to_string(scratch_bytes) + " bytes; call Sgemm or SgemmWithTempBuffer instead");
+      }
+      throw;
+    }
     return StatusCode::kSuccess;
   } catch (...) {
     return DispatchException();

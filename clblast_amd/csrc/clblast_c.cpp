@@ -53,6 +53,20 @@ CLBlastStatusCode CLBlastSgemmWithTempBuffer(const CLBlastLayout layout, const C
   });
 }
 
+// SGEMM for callers that cannot allocate: the split-K workspace, the only scratch memory an fp32 GEMM can want, is this
+// GPU's static scratch array (device/static_scratch.hip). Nothing here calls hipMalloc, hipFree or a routine that does.
+CLBlastStatusCode CLBlastSgemmNoAlloc(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                      const CLBlastTranspose b_transpose, const size_t m, const size_t n, const size_t k,
+                                      const float alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+                                      const void* b_buffer, const size_t b_offset, const size_t b_ld, const float beta,
+                                      void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                                      hipEvent_t* event) {
+  return Guarded([&]() {
+    return clblast::GemmNoAlloc(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, alpha, a_buffer, a_offset, a_ld,
+                                b_buffer, b_offset, b_ld, beta, c_buffer, c_offset, c_ld, queue, event);
+  });
+}
+
 CLBlastStatusCode CLBlastSgemmBatched(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
                                       const CLBlastTranspose b_transpose, const size_t m, const size_t n,
                                       const size_t k, const float* alphas, const void* a_buffer,

@@ -444,6 +444,18 @@ CLBlastStatusCode CLBLAST_HIP_API CLBlastHgemmWithTempBuffer(
     const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event, void* temp_buffer);
 
 // =================================================================================================
+// SGEMM that allocates nothing. No counterpart in the reference: it is for callers that cannot allocate device memory
+// (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). Same arguments and results as
+// CLBlastSgemm; the split-K workspace is a static device array of 8 MiB per GPU instead of stream scratch, and a problem
+// that would need more returns CLBlastInsufficientMemoryTemp (-2050) with a message on stderr. All calls on one GPU
+// share that array: calls that overlap on one GPU (different streams) race.
+CLBlastStatusCode CLBLAST_HIP_API CLBlastSgemmNoAlloc(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const float alpha, const void* a_buffer, const size_t a_offset, const size_t a_ld,
+    const void* b_buffer, const size_t b_offset, const size_t b_ld, const float beta, void* c_buffer,
+    const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event);
+
+// =================================================================================================
 // Bytes wanted in temp_buffer for these arguments (0 when none is needed)
 // replaces CLBlast{S,D,H}GemmTempBufferSize (reference: include/clblast_c.h:1412-1445, src/clblast_c.cpp:3011-3084)
 CLBlastStatusCode CLBLAST_HIP_API CLBlastSGemmTempBufferSize(
