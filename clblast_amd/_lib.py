@@ -33,6 +33,12 @@ def _declare(lib):
         f = getattr(lib, "CLBlast%sgemm" % prefix)
         f.argtypes = [c_int, c_int, c_int, sz, sz, sz, scalar, vp, sz, sz, vp, sz, sz, scalar, vp, sz, sz, vp, vp]
         f.restype = c_int
+        f = getattr(lib, "CLBlast%sgemmWithTempBuffer" % prefix)
+        f.argtypes = [c_int, c_int, c_int, sz, sz, sz, scalar, vp, sz, sz, vp, sz, sz, scalar, vp, sz, sz, vp, vp, vp]
+        f.restype = c_int
+        f = getattr(lib, "CLBlast%sGemmTempBufferSize" % prefix)
+        f.argtypes = [c_int, c_int, c_int, sz, sz, sz, sz, sz, sz, sz, sz, sz, vp, POINTER(sz)]
+        f.restype = c_int
         for routine in ("symm", "hemm"):
             f = getattr(lib, "CLBlast%s%s" % (prefix, routine))
             f.argtypes = [c_int, c_int, c_int, sz, sz, scalar, vp, sz, sz, vp, sz, sz, scalar, vp, sz, sz, vp, vp]
@@ -117,7 +123,8 @@ def load():
 # Every symbol the public C headers declare, for the export test.
 C_API_SYMBOLS = (
     ["CLBlast%sgemm%s" % (p, s) for p in "SDH" for s in ("", "Batched", "StridedBatched", "WithTempBuffer")] +
-    ["CLBlast%sGemmTempBufferSize" % p for p in "SDH"] + ["CLBlastCgemm", "CLBlastZgemm"] +
+    ["CLBlast%sGemmTempBufferSize" % p for p in "SDHCZ"] + ["CLBlastCgemm", "CLBlastZgemm"] +
+    ["CLBlastCgemmWithTempBuffer", "CLBlastZgemmWithTempBuffer"] +
     ["CLBlast%sgemm%s" % (p, s) for p in "CZ" for s in ("Batched", "StridedBatched")] +
     ["CLBlast%s%s" % (p, r) for p in "CZ" for r in ("symm", "hemm", "syrk", "herk", "syr2k", "her2k", "trmm", "trsm")] +
     ["CLBlast%s%s" % (p, r) for p in "SDH" for r in ("symm", "syrk", "syr2k", "trmm")] + ["CLBlastStrsm", "CLBlastDtrsm"] +
@@ -133,4 +140,5 @@ DEVICE_LAYER_SYMBOLS = [
     "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale", "clbh_complex_expand_batched",
     "clbh_complex_transpose_batched", "clbh_complex_scale_batched", "clbh_complex_gemm_small_batched", "clbh_copy_matrix_batched", "clbh_alloc", "clbh_free", "clbh_copy", "clbh_im2col", "clbh_conv_gather_possible", "clbh_pad_image", "clbh_fill_zero", "clbh_complex_symmetric_to_square",
     "clbh_complex_triangular_to_square", "clbh_complex_zero_diagonal_imag", "clbh_complex_invert_block_size",
-    "clbh_complex_invert_diagonal_blocks", "clbh_static_scratch", "clbh_static_scratch_bytes"]
+    "clbh_complex_invert_diagonal_blocks", "clbh_static_scratch", "clbh_static_scratch_bytes", "clbh_stream_capturing",
+    "clbh_stream_is_alias"]

@@ -92,16 +92,18 @@ def raw_sgemm_no_alloc(layout, a_transpose, b_transpose, m, n, k, alpha, a_ptr, 
 
 
 def raw_complex_gemm(prefix, layout, a_transpose, b_transpose, m, n, k, alpha, a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld,
-                     beta, c_ptr, c_offset, c_ld, stream_handle=0, event_handle=None):
+                     beta, c_ptr, c_offset, c_ld, stream_handle=0, event_handle=None, temp_ptr=None):
     """CLBlastCgemm ("C", complex64 data) / CLBlastZgemm ("Z", complex128) through the C ABI (reference:
     include/clblast_c.h:899-912); alpha and beta are Python complex numbers."""
     lib = _lib.load()
     scalar = _lib.Float2 if prefix == "C" else _lib.Double2
     alpha, beta = complex(alpha), complex(beta)
     event_ref = None if event_handle is None else ctypes.byref(ctypes.c_void_p(event_handle))
-    return getattr(lib, "CLBlast%sgemm" % prefix)(layout, a_transpose, b_transpose, m, n, k, scalar(alpha.real, alpha.imag),
-                                                  a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld, scalar(beta.real, beta.imag),
-                                                  c_ptr, c_offset, c_ld, _stream_ref(stream_handle), event_ref)
+    arguments = [layout, a_transpose, b_transpose, m, n, k, scalar(alpha.real, alpha.imag), a_ptr, a_offset, a_ld, b_ptr,
+                 b_offset, b_ld, scalar(beta.real, beta.imag), c_ptr, c_offset, c_ld, _stream_ref(stream_handle), event_ref]
+    if temp_ptr is None:
+        return getattr(lib, "CLBlast%sgemm" % prefix)(*arguments)
+    return getattr(lib, "CLBlast%sgemmWithTempBuffer" % prefix)(*(arguments + [temp_ptr]))
 
 
 def raw_convgemm(prefix, kernel_mode, channels, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w, dilation_h,

@@ -280,12 +280,14 @@ StatusCode ComplexGemm(const Layout layout, const Transpose a_transpose, const T
                        const size_t n, const size_t k, const std::complex<R> alpha, const void* a_buffer,
                        const size_t a_offset, const size_t a_ld, const void* b_buffer, const size_t b_offset,
                        const size_t b_ld, const std::complex<R> beta, void* c_buffer, const size_t c_offset,
-                       const size_t c_ld, hipStream_t* queue, hipEvent_t* event) {
+                       const size_t c_ld, hipStream_t* queue, hipEvent_t* event, void* temp_buffer) {
   try {
     using Complex = std::complex<R>;
     auto routine = XgemmComplex<R>(queue, event);
+    const auto temp = Buffer<Complex>(temp_buffer);
     routine.DoGemm(layout, a_transpose, b_transpose, m, n, k, alpha, Buffer<Complex>(a_buffer), a_offset, a_ld,
-                   Buffer<Complex>(b_buffer), b_offset, b_ld, beta, Buffer<Complex>(c_buffer), c_offset, c_ld);
+                   Buffer<Complex>(b_buffer), b_offset, b_ld, beta, Buffer<Complex>(c_buffer), c_offset, c_ld,
+                   OutputTriangle::kFull, true, (temp_buffer != nullptr) ? &temp : nullptr);
     return StatusCode::kSuccess;
   } catch (...) {
     return DispatchException();
@@ -297,9 +299,9 @@ StatusCode CLBLAST_HIP_PUBLIC Gemm<float2>(const Layout layout, const Transpose 
                                            const void* a_buffer, const size_t a_offset, const size_t a_ld,
                                            const void* b_buffer, const size_t b_offset, const size_t b_ld, const float2 beta,
                                            void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
-                                           hipEvent_t* event, void*) {
+                                           hipEvent_t* event, void* temp_buffer) {
   return ComplexGemm<float>(layout, a_transpose, b_transpose, m, n, k, alpha, a_buffer, a_offset, a_ld, b_buffer, b_offset,
-                            b_ld, beta, c_buffer, c_offset, c_ld, queue, event);
+                            b_ld, beta, c_buffer, c_offset, c_ld, queue, event, temp_buffer);
 }
 template <>
 StatusCode CLBLAST_HIP_PUBLIC Gemm<double2>(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
@@ -307,9 +309,42 @@ StatusCode CLBLAST_HIP_PUBLIC Gemm<double2>(const Layout layout, const Transpose
                                             const void* a_buffer, const size_t a_offset, const size_t a_ld,
                                             const void* b_buffer, const size_t b_offset, const size_t b_ld,
                                             const double2 beta, void* c_buffer, const size_t c_offset, const size_t c_ld,
-                                            hipStream_t* queue, hipEvent_t* event, void*) {
+                                            hipStream_t* queue, hipEvent_t* event, void* temp_buffer) {
   return ComplexGemm<double>(layout, a_transpose, b_transpose, m, n, k, alpha, a_buffer, a_offset, a_ld, b_buffer, b_offset,
-                             b_ld, beta, c_buffer, c_offset, c_ld, queue, event);
+                             b_ld, beta, c_buffer, c_offset, c_ld, queue, event, temp_buffer);
+}
+
+// Bytes the complex GEMM wants in temp_buffer (reference: GemmTempBufferSize<float2/double2>, src/clblast.cpp:1717-1724)
+template <typename R>
+StatusCode ComplexGemmTempBufferSize(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
+                                     const size_t m, const size_t n, const size_t k, hipStream_t* queue,
+                                     size_t& temp_buffer_size) {
+  try {
+    if (queue == nullptr) { throw RuntimeErrorCode(StatusCode::kInvalidCommandQueue, "queue is a null pointer"); }
+    auto device = 0;
+    CheckDevice(clbh_stream_device(*queue, &device), "clbh_stream_device");
+    temp_buffer_size = XgemmComplex<R>::TempBytes(layout, a_transpose, b_transpose, m, n, k,
+                                                  MinIndirectSize(device, PrecisionValue<R>()));
+    return StatusCode::kSuccess;
+  } catch (...) {
+    return DispatchException();
+  }
+}
+template <>
+StatusCode CLBLAST_HIP_PUBLIC GemmTempBufferSize<float2>(const Layout layout, const Transpose a_transpose,
+                                                         const Transpose b_transpose, const size_t m, const size_t n,
+                                                         const size_t k, const size_t, const size_t, const size_t,
+                                                         const size_t, const size_t, const size_t, hipStream_t* queue,
+                                                         size_t& temp_buffer_size) {
+  return ComplexGemmTempBufferSize<float>(layout, a_transpose, b_transpose, m, n, k, queue, temp_buffer_size);
+}
+template <>
+StatusCode CLBLAST_HIP_PUBLIC GemmTempBufferSize<double2>(const Layout layout, const Transpose a_transpose,
+                                                          const Transpose b_transpose, const size_t m, const size_t n,
+                                                          const size_t k, const size_t, const size_t, const size_t,
+                                                          const size_t, const size_t, const size_t, hipStream_t* queue,
+                                                          size_t& temp_buffer_size) {
+  return ComplexGemmTempBufferSize<double>(layout, a_transpose, b_transpose, m, n, k, queue, temp_buffer_size);
 }
 
 // The batched GEMMs of the complex types (reference: src/clblast.cpp:1612-1621, 1660-1671)

@@ -356,6 +356,60 @@ CLBlastStatusCode CLBlastZgemm(const CLBlastLayout layout, const CLBlastTranspos
   });
 }
 
+CLBlastStatusCode CLBlastCgemmWithTempBuffer(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                             const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                             const size_t k, const CLBlastFloat2 alpha, const void* a_buffer,
+                                             const size_t a_offset, const size_t a_ld, const void* b_buffer,
+                                             const size_t b_offset, const size_t b_ld, const CLBlastFloat2 beta,
+                                             void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                                             hipEvent_t* event, void* temp_buffer) {
+  return Guarded([&]() {
+    return clblast::Gemm<clblast::float2>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k,
+                                          clblast::float2(alpha.x, alpha.y), a_buffer, a_offset, a_ld, b_buffer, b_offset,
+                                          b_ld, clblast::float2(beta.x, beta.y), c_buffer, c_offset, c_ld, queue, event,
+                                          temp_buffer);
+  });
+}
+
+CLBlastStatusCode CLBlastZgemmWithTempBuffer(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                             const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                             const size_t k, const CLBlastDouble2 alpha, const void* a_buffer,
+                                             const size_t a_offset, const size_t a_ld, const void* b_buffer,
+                                             const size_t b_offset, const size_t b_ld, const CLBlastDouble2 beta,
+                                             void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                                             hipEvent_t* event, void* temp_buffer) {
+  return Guarded([&]() {
+    return clblast::Gemm<clblast::double2>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k,
+                                           clblast::double2(alpha.x, alpha.y), a_buffer, a_offset, a_ld, b_buffer, b_offset,
+                                           b_ld, clblast::double2(beta.x, beta.y), c_buffer, c_offset, c_ld, queue, event,
+                                           temp_buffer);
+  });
+}
+
+CLBlastStatusCode CLBlastCGemmTempBufferSize(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                             const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                             const size_t k, const size_t a_offset, const size_t a_ld, const size_t b_offset,
+                                             const size_t b_ld, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                                             size_t* temp_buffer_size) {
+  return Guarded([&]() {
+    if (temp_buffer_size == nullptr) { return clblast::StatusCode::kInvalidValue; }
+    return clblast::GemmTempBufferSize<clblast::float2>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, a_offset, a_ld,
+                                                        b_offset, b_ld, c_offset, c_ld, queue, *temp_buffer_size);
+  });
+}
+
+CLBlastStatusCode CLBlastZGemmTempBufferSize(const CLBlastLayout layout, const CLBlastTranspose a_transpose,
+                                             const CLBlastTranspose b_transpose, const size_t m, const size_t n,
+                                             const size_t k, const size_t a_offset, const size_t a_ld, const size_t b_offset,
+                                             const size_t b_ld, const size_t c_offset, const size_t c_ld, hipStream_t* queue,
+                                             size_t* temp_buffer_size) {
+  return Guarded([&]() {
+    if (temp_buffer_size == nullptr) { return clblast::StatusCode::kInvalidValue; }
+    return clblast::GemmTempBufferSize<clblast::double2>(L(layout), Tr(a_transpose), Tr(b_transpose), m, n, k, a_offset, a_ld,
+                                                         b_offset, b_ld, c_offset, c_ld, queue, *temp_buffer_size);
+  });
+}
+
 // ---- batched CGEMM, ZGEMM: the C structs and std::complex share their layout -------------------------
 #define CLBLAST_HIP_COMPLEX_BATCHED(PREFIX, CTYPE, CPPTYPE)                                                          \
   CLBlastStatusCode CLBlast##PREFIX##gemmBatched(                                                                    \

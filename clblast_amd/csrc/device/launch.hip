@@ -610,6 +610,24 @@ int clbh_upload_async(void* dst_device, const void* src_host, size_t bytes, hipS
   return clbh::StagedUpload(dst_device, src_host, bytes, stream, device);
 }
 
+int clbh_stream_capturing(hipStream_t stream, int* capturing) {
+  if (capturing == nullptr) { return hipErrorInvalidValue; }
+  *capturing = 0;
+  if (stream == nullptr) { return 0; }  // the legacy null stream cannot be captured
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  const auto result = hipStreamIsCapturing(stream, &status);
+  if (result != hipSuccess) {
+    (void)hipGetLastError();
+    return static_cast<int>(result);
+  }
+  *capturing = (status != hipStreamCaptureStatusNone) ? 1 : 0;
+  return 0;
+}
+
+int clbh_stream_is_alias(hipStream_t stream) {
+  return (stream == hipStreamPerThread || stream == hipStreamLegacy) ? 1 : 0;
+}
+
 int clbh_event_record(hipEvent_t event, hipStream_t stream) {
   return static_cast<int>(hipEventRecord(event, stream));
 }

@@ -91,6 +91,9 @@ inline bool ConvGatherPossible(const int precision, const clbh_im2col_shape& g) 
   if (precision != 32 && precision != 16) { return false; }
   // fp16: eight patches per lane from images without padding, dword-aligned through the second copy
   if (precision == 16 && (g.pad_h != 0 || g.pad_w != 0 || g.stride_w != 1 || g.width % 2 != 0 || g.output_w % 8 != 0)) { return false; }
+  // (... whose kernel window fits into the image: that gather tests no tap against the image bounds)
+  if (precision == 16 && (static_cast<long long>(g.dilation_h) * (g.kernel_h - 1) + 1 > g.height ||
+                          static_cast<long long>(g.dilation_w) * (g.kernel_w - 1) + 1 > g.width)) { return false; }
   if (g.channels <= 0 || g.height <= 0 || g.width <= 0 || g.kernel_h <= 0 || g.kernel_w <= 0 || g.stride_h <= 0 ||
       g.stride_w <= 0 || g.dilation_h <= 0 || g.dilation_w <= 0 || g.output_h <= 0 || g.output_w <= 0 || g.pad_h < 0 ||
       g.pad_w < 0) {

@@ -20,7 +20,11 @@ int LaunchConvF32(const clbh_gemm_desc& d, hipStream_t stream) {
   }
   // without padding, with unit stride along the width and whole groups of four patches per output row a lane can
   // fetch four patches at once (GatherLoadVector)
-  if (g.pad_h == 0 && g.pad_w == 0 && g.stride_w == 1 && g.output_w % 4 == 0) {
+  // (and every tap of every patch inside the image: a kernel window larger than the image - the output extent is then
+  // clamped to 1 - has taps that count as zeros, which only the element-wise gather tests for)
+  const bool window_fits = static_cast<long long>(g.dilation_h) * (g.kernel_h - 1) + 1 <= g.height &&
+                           static_cast<long long>(g.dilation_w) * (g.kernel_w - 1) + 1 <= g.width;
+  if (g.pad_h == 0 && g.pad_w == 0 && g.stride_w == 1 && g.output_w % 4 == 0 && window_fits) {
     return LaunchMfmaVariant<float, MfmaConfig<float, 2, 2, 1, 1, 16, 4>, false, true, true, 2>(d, stream);
   }
   return LaunchMfmaVariant<float, MfmaConfig<float, 2, 2, 1, 1, 16, 4>, false, true, true, 1>(d, stream);

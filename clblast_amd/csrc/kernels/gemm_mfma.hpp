@@ -655,40 +655,104 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
       slab_body(slab, std::false_type{}, std::false_type{});
       __syncthreads();
     };
-    if (m0 + TILE_M <= p.m && n0 + TILE_N <= p.n && k_len % TILE_K == 0) { walk(std::false_type{}); }
-    else { walk(std::true_type{}); }
-
-    // Epilogue. Lane owns m = m_base + i (i < FM); accumulator element r of block (i, j) is the
-    // column n = n_base + FN * Row(r) + j.
+    // Lane owns m = m_base + i * M_STEP (i < FM); accumulator element r of block (i, j) is the column
+    // n = n_base + FN * Row(r) + j.
     const int m_base = m0 + a_read;
     const int n_base = n0 + wave_n * (FN * MF);
     constexpr int M_STEP = M_INTERLEAVED ? 1 : MF;  // distance in m between the lane's accumulator blocks
     // 16-byte accesses to C need dword alignment only, which every fp32/fp64 address has
     typedef T VMG __attribute__((ext_vector_type(FM > 1 ? FM : 2), aligned(sizeof(T))));
     const bool vector_store = M_INTERLEAVED && (FM > 1) && (m_base + FM <= p.m) && !masked;
+    auto writes = [&](const int i, const int n) {  // element i of the lane's piece of column n belongs to the result
+      return n < p.n && m_base + i * M_STEP < p.m && (!masked || InTriangle(p.c_triangle, m_base + i * M_STEP, n));
+    };
+    // Small tiles (at most 16 registers of old C per lane) fetch the old C before the K walk when beta != 0: with a
+    // short k the launch is a stream over C, and a work-group that asked for its C only after its last product would
+    // wait out a second memory latency with nothing else to do (8191 x 8191 x 127: 0.27 -> 0.14 ms). The loads are the
+    // oldest in the queue, so the first wait of the walk covers them.
+    constexpr bool PREFETCH_C = FM * FN * ACC * sizeof(T) <= 64;
+    T old_c[PREFETCH_C ? FM * FN * ACC : 1];
+    if constexpr (PREFETCH_C) {
+      if (beta != T(0)) {
 #pragma unroll
-    for (int j = 0; j < FN; ++j) {
+        for (int j = 0; j < FN; ++j) {
 #pragma unroll
-      for (int r = 0; r < ACC; ++r) {
-        const int n = n_base + FN * Traits::Row(r, lane_g) + j;
-        if (n >= p.n) { continue; }
-        T* dst = c + n * c_ld + m_base;
-        if (vector_store) {
-          VMG out;
-          if (beta == T(0)) {
+          for (int r = 0; r < ACC; ++r) {
+            const int n = n_base + FN * Traits::Row(r, lane_g) + j;
 #pragma unroll
-            for (int i = 0; i < FM; ++i) { out[i] = alpha * acc[i][j][r]; }
-          } else {
-            const VMG old = *reinterpret_cast<const VMG*>(dst);
-#pragma unroll
-            for (int i = 0; i < FM; ++i) { out[i] = alpha * acc[i][j][r] + beta * old[i]; }
+            for (int i = 0; i < FM; ++i) {
+              old_c[(j * ACC + r) * FM + i] = writes(i, n) ? c[n * c_ld + m_base + i * M_STEP] : T(0);
+            }
           }
-          *reinterpret_cast<VMG*>(dst) = out;
-        } else {
+        }
+      }
+    }
+
+    if (m0 + TILE_M <= p.m && n0 + TILE_N <= p.n && k_len % TILE_K == 0) { walk(std::false_type{}); }
+    else { walk(std::true_type{}); }
+
+    // Epilogue.
+    if constexpr (PREFETCH_C) {
 #pragma unroll
-          for (int i = 0; i < FM; ++i) {
-            if (m_base + i * M_STEP < p.m && (!masked || InTriangle(p.c_triangle, m_base + i * M_STEP, n))) {
-              StoreResult<T, T>(dst, i * M_STEP, acc[i][j][r], alpha, beta);
+      for (int j = 0; j < FN; ++j) {
+#pragma unroll
+        for (int r = 0; r < ACC; ++r) {
+          const int n = n_base + FN * Traits::Row(r, lane_g) + j;
+          T* dst = c + n * c_ld + m_base;
+          if (vector_store && n < p.n) {
+            VMG out;
+#pragma unroll
+            for (int i = 0; i < FM; ++i) {
+              out[i] = (beta == T(0)) ? alpha * acc[i][j][r] : alpha * acc[i][j][r] + beta * old_c[(j * ACC + r) * FM + i];
+            }
+            *reinterpret_cast<VMG*>(dst) = out;
+          } else {
+#pragma unroll
+            for (int i = 0; i < FM; ++i) {
+              if (writes(i, n)) {
+                dst[i * M_STEP] = (beta == T(0)) ? alpha * acc[i][j][r] : alpha * acc[i][j][r] + beta * old_c[(j * ACC + r) * FM + i];
+              }
+            }
+          }
+        }
+      }
+    } else {
+      // Large tiles: the old C of four columns at a time is fetched before the first of them is combined and stored
+      // (a load behind a store to memory that may alias it cannot be hoisted by the compiler).
+      constexpr int BATCH = (ACC % 4 == 0) ? 4 : 1;
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+#pragma unroll
+        for (int r0 = 0; r0 < ACC; r0 += BATCH) {
+          VMG old[BATCH];
+          if (vector_store && beta != T(0)) {
+#pragma unroll
+            for (int rr = 0; rr < BATCH; ++rr) {
+              const int n = n_base + FN * Traits::Row(r0 + rr, lane_g) + j;
+              if (n < p.n) { old[rr] = *reinterpret_cast<const VMG*>(c + n * c_ld + m_base); }
+            }
+          }
+#pragma unroll
+          for (int rr = 0; rr < BATCH; ++rr) {
+            const int r = r0 + rr;
+            const int n = n_base + FN * Traits::Row(r, lane_g) + j;
+            if (n >= p.n) { continue; }
+            T* dst = c + n * c_ld + m_base;
+            if (vector_store) {
+              VMG out;
+              if (beta == T(0)) {
+#pragma unroll
+                for (int i = 0; i < FM; ++i) { out[i] = alpha * acc[i][j][r]; }
+              } else {
+#pragma unroll
+                for (int i = 0; i < FM; ++i) { out[i] = alpha * acc[i][j][r] + beta * old[rr][i]; }
+              }
+              *reinterpret_cast<VMG*>(dst) = out;
+            } else {
+#pragma unroll
+              for (int i = 0; i < FM; ++i) {
+                if (writes(i, n)) { StoreResult<T, T>(dst, i * M_STEP, acc[i][j][r], alpha, beta); }
+              }
             }
           }
         }

@@ -60,44 +60,78 @@ struct CachedScratch {
   size_t used = 0;   // offset of the first free byte
   size_t live = 0;   // pieces handed out and not yet returned
   size_t demand = 0; // what a call would have needed while the buffer could not grow
+  bool pinned = false;          // a captured graph holds the buffer's address: it is never freed or replaced again
+  unsigned long long last_use = 0;
   std::recursive_mutex taken;
 };
 constexpr size_t kScratchAlignment = 256;
 std::mutex scratch_cache_mutex;
 std::map<std::pair<int, hipStream_t>, std::unique_ptr<CachedScratch>> scratch_cache;
+unsigned long long scratch_clock = 0;
+
+void FreeScratchBuffer(void* pointer) {
+  // (hipFree waits for the device, which covers kernels of earlier calls that still use the buffer)
+  const auto status = clbh_free(pointer);
+  if (status != 0) { fprintf(stderr, "CLBlast: freeing a scratch buffer failed: %s\n", clbh_error_string(status)); }
+}
+
+// With the table full, the idle entry that was used least recently makes room (streams come and go in long-running
+// programs). Called with scratch_cache_mutex held.
+bool EvictIdleScratch() {
+  auto victim = scratch_cache.end();
+  for (auto entry = scratch_cache.begin(); entry != scratch_cache.end(); ++entry) {
+    auto& cached = *entry->second;
+    if (cached.pinned || !cached.taken.try_lock()) { continue; }
+    const bool idle = (cached.live == 0);
+    cached.taken.unlock();
+    if (idle && (victim == scratch_cache.end() || cached.last_use < victim->second->last_use)) { victim = entry; }
+  }
+  if (victim == scratch_cache.end()) { return false; }
+  if (victim->second->pointer != nullptr) { FreeScratchBuffer(victim->second->pointer); }
+  scratch_cache.erase(victim);
+  return true;
+}
 
 // A piece of `bytes` bytes of this stream's buffer (its entry then stays locked by this thread until the piece is
 // returned), or nullptr: then the caller allocates on the stream.
 CachedScratch* TakeCachedScratch(const size_t bytes, hipStream_t stream, size_t& offset) {
   auto device = 0;
   if (bytes == 0 || bytes > kCachedScratchBytes || clbh_stream_device(stream, &device) != 0) { return nullptr; }
+  // hipStreamPerThread is one handle value for a different stream in every host thread: a buffer keyed by it would be
+  // shared by streams that nothing orders against each other.
+  if (clbh_stream_is_alias(stream) != 0) { return nullptr; }
+  // While the stream is being captured into a graph nothing may be allocated or freed with the blocking calls, and the
+  // address a captured kernel gets must stay valid for every later replay.
+  auto capturing = 0;
+  if (clbh_stream_capturing(stream, &capturing) != 0) { return nullptr; }
   CachedScratch* entry = nullptr;
   {
     std::lock_guard<std::mutex> lock(scratch_cache_mutex);
     const auto key = std::make_pair(device, stream);
     auto found = scratch_cache.find(key);
     if (found == scratch_cache.end()) {
-      if (scratch_cache.size() >= kCachedScratchStreams) { return nullptr; }
+      if (capturing != 0) { return nullptr; }  // no buffer in place: the captured call allocates on the stream
+      if (scratch_cache.size() >= kCachedScratchStreams && !EvictIdleScratch()) { return nullptr; }
       found = scratch_cache.emplace(key, std::unique_ptr<CachedScratch>(new CachedScratch())).first;
     }
     entry = found->second.get();
     if (!entry->taken.try_lock()) { return nullptr; }  // another host thread is inside a call on this stream
+    entry->last_use = ++scratch_clock;
   }
   offset = (entry->used + kScratchAlignment - 1) / kScratchAlignment * kScratchAlignment;
-  if (offset + bytes > entry->bytes || (entry->live == 0 && entry->demand > entry->bytes)) {
+  if (offset + bytes > entry->bytes || (entry->live == 0 && entry->demand > entry->bytes && !entry->pinned && capturing == 0)) {
     // Too small: grow - in powers of two from 1 MiB, so that this happens a few times per stream at most - unless
-    // pieces of the buffer are in use: then the size that would have done is remembered, and the next call's first
-    // request grows the buffer to it. Freeing the old buffer waits for the device, which covers kernels of earlier
-    // calls that still use it.
+    // pieces of the buffer are in use (then the size that would have done is remembered, and the next call's first
+    // request grows the buffer to it), the stream is being captured, or a captured graph knows the buffer's address.
     auto wanted = size_t{1} << 20;
     while (wanted < std::max(offset + bytes, entry->demand)) { wanted *= 2; }
     if (wanted > kCachedScratchBytes) { wanted = kCachedScratchBytes; }
-    if (entry->live > 0 || offset + bytes > wanted) {
-      entry->demand = std::max(entry->demand, std::min(offset + bytes, kCachedScratchBytes));
+    if (entry->live > 0 || offset + bytes > wanted || entry->pinned || capturing != 0) {
+      if (!entry->pinned) { entry->demand = std::max(entry->demand, std::min(offset + bytes, kCachedScratchBytes)); }
       entry->taken.unlock();
       return nullptr;
     }
-    if (entry->pointer != nullptr) { clbh_free(entry->pointer); }
+    if (entry->pointer != nullptr) { FreeScratchBuffer(entry->pointer); }
     entry->pointer = nullptr;
     entry->bytes = 0;
     if (clbh_alloc(&entry->pointer, wanted) != 0) {
@@ -107,6 +141,7 @@ CachedScratch* TakeCachedScratch(const size_t bytes, hipStream_t stream, size_t&
     }
     entry->bytes = wanted;
   }
+  if (capturing != 0) { entry->pinned = true; }
   entry->used = offset + bytes;
   entry->live += 1;
   return entry;
@@ -141,9 +176,9 @@ StreamScratch::~StreamScratch() {
 void ReleaseCachedScratch() {
   std::lock_guard<std::mutex> lock(scratch_cache_mutex);
   for (auto entry = scratch_cache.begin(); entry != scratch_cache.end();) {
-    if (entry->second->taken.try_lock()) {
+    if (!entry->second->pinned && entry->second->taken.try_lock()) {
       const bool idle = (entry->second->live == 0);  // not in the hands of a running call (of this thread either)
-      if (idle && entry->second->pointer != nullptr) { clbh_free(entry->second->pointer); }
+      if (idle && entry->second->pointer != nullptr) { FreeScratchBuffer(entry->second->pointer); }
       entry->second->taken.unlock();
       if (idle) { entry = scratch_cache.erase(entry); continue; }
     }

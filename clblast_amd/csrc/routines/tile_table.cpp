@@ -112,8 +112,8 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
                           const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,
                           const size_t min_indirect_size, const bool triangular) {
   (void)a_kcontig; (void)b_kcontig; (void)per_batch_scalars;
-  // Many small matrices: one wavefront per matrix, bandwidth bound
-  if (batch_count >= 16 && m <= 32 && n <= 32 && k <= 32) {
+  // Many small matrices: one wavefront per matrix, bandwidth bound (that kernel knows no triangles)
+  if (!triangular && batch_count >= 16 && m <= 32 && n <= 32 && k <= 32) {
     return KernelChoice{CLBH_KERNEL_SMALL_BATCHED, 0, 1};
   }
   // The reference's threshold is on the volume of one matrix product; here the general kernel only wins when the whole

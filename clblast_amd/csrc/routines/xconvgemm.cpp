@@ -94,8 +94,11 @@ void Xconvgemm<T>::DoConvgemm(const KernelMode kernel_mode, const size_t channel
   const bool half_kernels_aligned =
       (reinterpret_cast<unsigned long long>(kernel_buffer()) + 2 * kernel_offset) % 4 == 0 && patch_size % 2 == 0;
   const bool half_images_aligned = (reinterpret_cast<unsigned long long>(im_buffer()) + 2 * im_offset) % 4 == 0;
+  // (a kernel window larger than the padded image - the output extent is then clamped to 1 - has taps beyond the image
+  // that read as zero; only the element-wise gather and im2col test every tap against the image bounds)
   const bool vector_gather =  // four (fp32) or eight (fp16) patches per lane
       stride_w == 1 && output_w % (precision == 16 ? 8 : 4) == 0 && batch_count * channels <= kLimit &&
+      size_h >= padding_h && size_w >= padding_w &&
       clbh_conv_gather_possible(precision, &padded_shape) != 0 &&
       (precision == 32 || (precision == 16 && half_kernels_aligned && (needs_copy || half_images_aligned)));
   if (vector_gather || (precision == 32 && clbh_conv_gather_possible(precision, &shape) != 0)) {

@@ -13,12 +13,50 @@ template <typename R>
 XgemmComplex<R>::XgemmComplex(hipStream_t* queue, hipEvent_t* event) : Xgemm<R>(queue, event) {}
 
 template <typename R>
+typename XgemmComplex<R>::TempLayout XgemmComplex<R>::PlanTemp(const size_t rows, const size_t columns, const size_t k,
+                                                               const bool right_kcontig, const bool full,
+                                                               const size_t min_indirect_size) {
+  auto plan = TempLayout{};
+  // A small product in one launch on the interleaved data itself (the kernel of the small batched products): the real
+  // form takes three to four launches, which is most of the time at these sizes. Only for a short k: a single
+  // work-group per tile walks its slabs at the latency of one load each (128^3: 15.9 us against 10.1 below, complex128
+  // 64^3: 14.0 against 11).
+  plan.small_kernel = full && rows <= 128 && columns <= 128 && k <= 32 && ForcedTileVariant(PrecisionValue<R>()) == 0;
+  if (plan.small_kernel) { return plan; }
+  const auto aligned = [](const size_t bytes) { return (bytes + 255) / 256 * 256; };
+  plan.expanded_bytes = 4 * rows * k * sizeof(R);                           // real 2 rows x 2k
+  plan.transposed_bytes = right_kcontig ? 0 : 2 * k * columns * sizeof(R);  // complex columns x k, k contiguous
+  // the real GEMM of a full product is a plain column-major 2 rows x columns x 2k call (triangles never split K)
+  plan.workspace_bytes = full ? Xgemm<R>::TempBytes(Layout::kColMajor, Transpose::kNo, Transpose::kNo, 2 * rows, columns,
+                                                    2 * k, min_indirect_size)
+                              : 0;
+  plan.transposed_at = aligned(plan.expanded_bytes);
+  plan.workspace_at = plan.transposed_at + aligned(plan.transposed_bytes);
+  plan.total = plan.workspace_at + plan.workspace_bytes;
+  return plan;
+}
+
+template <typename R>
+size_t XgemmComplex<R>::TempBytes(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
+                                  const size_t m, const size_t n, const size_t k, const size_t min_indirect_size) {
+  const auto shape = Xgemm<R>::ProcessArguments(layout, a_transpose, b_transpose, m, n, k);
+  if (m > static_cast<size_t>(INT_MAX) / 2 || n > static_cast<size_t>(INT_MAX) / 2 || k > static_cast<size_t>(INT_MAX) / 2) {
+    throw BLASError(StatusCode::kInvalidDimension, "dimension exceeds 2^30");
+  }
+  const bool col_major = (layout == Layout::kColMajor);
+  // (the canonical second operand is B for a column-major call and A for a row-major one, see DoGemm)
+  const bool right_kcontig = col_major ? !shape.b_rotated : shape.a_rotated;
+  return PlanTemp(col_major ? m : n, col_major ? n : m, k, right_kcontig, true, min_indirect_size).total;
+}
+
+template <typename R>
 void XgemmComplex<R>::DoGemm(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
                              const size_t m, const size_t n, const size_t k, const Complex alpha,
                              const Buffer<Complex>& a_buffer, const size_t a_offset, const size_t a_ld,
                              const Buffer<Complex>& b_buffer, const size_t b_offset, const size_t b_ld,
                              const Complex beta, const Buffer<Complex>& c_buffer, const size_t c_offset,
-                             const size_t c_ld, const OutputTriangle triangle, const bool record_event) {
+                             const size_t c_ld, const OutputTriangle triangle, const bool record_event,
+                             const Buffer<Complex>* temp_buffer) {
   // Same order as the reference (xgemm.cpp:72-83): dimensions, then A (ld, size), B, C
   const auto shape = Xgemm<R>::ProcessArguments(layout, a_transpose, b_transpose, m, n, k);
   TestMatrixA(shape.a_one, shape.a_two, a_buffer, a_offset, a_ld);
@@ -45,12 +83,14 @@ void XgemmComplex<R>::DoGemm(const Layout layout, const Transpose a_transpose, c
 
   const auto precision = static_cast<int>(8 * sizeof(R));
   const auto stream = this->stream();
-  // A small product in one launch on the interleaved data itself (the kernel of the small batched products): the real
-  // form below takes three to four launches, which is most of the time at these sizes. Only for a short k: a single
-  // work-group per tile walks its slabs at the latency of one load each (128^3: 15.9 us against 10.1 below, complex128
-  // 64^3: 14.0 against 11).
-  if (triangle == OutputTriangle::kFull && rows <= 128 && columns <= 128 && k <= 32 &&
-      ForcedTileVariant(PrecisionValue<R>()) == 0) {
+  // The temporaries, in the caller's buffer when one is given (reference: xgemm.cpp:146-151 - too small is an error)
+  const auto plan = PlanTemp(rows, columns, k, right.kcontig, triangle == OutputTriangle::kFull, this->min_indirect_size());
+  unsigned char* provided = nullptr;
+  if (temp_buffer != nullptr) {
+    if (plan.total > 0 && temp_buffer->GetSize() < plan.total) { throw BLASError(StatusCode::kInsufficientMemoryTemp); }
+    provided = static_cast<unsigned char*>(const_cast<void*>((*temp_buffer)()));
+  }
+  if (plan.small_kernel) {
     auto desc = clbh_complex_small_desc{};
     desc.precision = precision;
     desc.rows = static_cast<int>(rows);
@@ -73,25 +113,29 @@ void XgemmComplex<R>::DoGemm(const Layout layout, const Transpose a_transpose, c
     return;
   }
   // left operand -> real 2 rows x 2k
-  const auto expanded_bytes = 4 * rows * k * sizeof(R);
-  const StreamScratch expanded(expanded_bytes, stream, "real form of the first operand");
+  const auto expanded_bytes = plan.expanded_bytes;
+  std::unique_ptr<StreamScratch> expanded_scratch;
+  if (provided == nullptr) { expanded_scratch.reset(new StreamScratch(expanded_bytes, stream, "real form of the first operand")); }
+  void* const expanded = (provided != nullptr) ? static_cast<void*>(provided) : expanded_scratch->get();
   CheckDevice(clbh_complex_expand(precision, static_cast<int>(rows), static_cast<int>(k), left.kcontig ? 1 : 0,
                                   left.conjugate ? 1 : 0, right.conjugate ? 1 : 0, static_cast<double>(alpha.real()),
                                   static_cast<double>(alpha.imag()), left.pointer, static_cast<long long>(left.offset),
-                                  static_cast<long long>(left.ld), expanded.get(), stream),
+                                  static_cast<long long>(left.ld), expanded, stream),
               "clbh_complex_expand");
   // right operand: in place as a real 2k x columns matrix when its k index is contiguous, else transposed first
   const void* right_pointer = right.pointer;
   size_t right_offset = right.offset, right_ld = right.ld, right_bytes = 0;
-  std::unique_ptr<StreamScratch> transposed;
-  if (!right.kcontig) {
-    right_bytes = 2 * k * columns * sizeof(R);
-    transposed.reset(new StreamScratch(right_bytes, stream, "transposed second operand"));
+  std::unique_ptr<StreamScratch> transposed_scratch;
+  const bool transposed = !right.kcontig;
+  if (transposed) {
+    right_bytes = plan.transposed_bytes;
+    if (provided == nullptr) { transposed_scratch.reset(new StreamScratch(right_bytes, stream, "transposed second operand")); }
+    void* const target = (provided != nullptr) ? static_cast<void*>(provided + plan.transposed_at) : transposed_scratch->get();
     CheckDevice(clbh_complex_transpose(precision, static_cast<int>(k), static_cast<int>(columns), right.pointer,
-                                       static_cast<long long>(right.offset), static_cast<long long>(right.ld),
-                                       transposed->get(), stream),
+                                       static_cast<long long>(right.offset), static_cast<long long>(right.ld), target,
+                                       stream),
                 "clbh_complex_transpose");
-    right_pointer = transposed->get();
+    right_pointer = target;
     right_offset = 0;
     right_ld = k;
   }
@@ -108,7 +152,7 @@ void XgemmComplex<R>::DoGemm(const Layout layout, const Transpose a_transpose, c
                 "clbh_complex_scale");
     real_beta = R(1);
   }
-  const auto real_left = Buffer<R>(expanded.get(), expanded_bytes);
+  const auto real_left = Buffer<R>(expanded, expanded_bytes);
   const auto real_right = transposed ? Buffer<R>(right_pointer, right_bytes) : Buffer<R>(right_pointer);
   const auto real_c = Buffer<R>(c_buffer());
   // the rows of the real matrix come in (re, im) pairs
@@ -116,9 +160,11 @@ void XgemmComplex<R>::DoGemm(const Layout layout, const Transpose a_transpose, c
   if (canonical_triangle != 0) {
     triangles.output = canonical_upper ? OutputTriangle::kUpperPairs : OutputTriangle::kLowerPairs;
   }
+  // (with a caller's buffer the real GEMM's split-K workspace is its third piece; the size test above covered it)
+  const auto real_temp = (provided != nullptr) ? Buffer<R>(provided + plan.workspace_at, plan.workspace_bytes) : Buffer<R>(nullptr);
   Xgemm<R>::DoGemm(Layout::kColMajor, Transpose::kNo, Transpose::kNo, 2 * rows, columns, 2 * k, R(1), real_left, 0, 2 * rows,
-                   real_right, 2 * right_offset, 2 * right_ld, real_beta, real_c, 2 * c_offset, 2 * c_ld, Buffer<R>(nullptr),
-                   false, triangles, record_event);
+                   real_right, 2 * right_offset, 2 * right_ld, real_beta, real_c, 2 * c_offset, 2 * c_ld, real_temp,
+                   provided != nullptr, triangles, record_event);
 }
 
 // =================================================================================================

@@ -24,11 +24,30 @@ class XgemmComplex : public Xgemm<R> {
  public:
   using Complex = std::complex<R>;
   XgemmComplex(hipStream_t* queue, hipEvent_t* event);
+  // temp_buffer: the caller's temporary memory (reference: the temp_buffer of Gemm<float2/double2>,
+  // src/clblast.cpp:1093-1100), or nullptr: then the routine takes stream scratch. Smaller than TempBytes says:
+  // kInsufficientMemoryTemp.
   void DoGemm(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
               const size_t n, const size_t k, const Complex alpha, const Buffer<Complex>& a_buffer,
               const size_t a_offset, const size_t a_ld, const Buffer<Complex>& b_buffer, const size_t b_offset,
               const size_t b_ld, const Complex beta, const Buffer<Complex>& c_buffer, const size_t c_offset,
-              const size_t c_ld, const OutputTriangle triangle = OutputTriangle::kFull, const bool record_event = true);
+              const size_t c_ld, const OutputTriangle triangle = OutputTriangle::kFull, const bool record_event = true,
+              const Buffer<Complex>* temp_buffer = nullptr);
+
+  // Bytes of temporary memory the full (no triangle) product wants: the real form of the first operand, the transposed
+  // second operand when its k index is not contiguous, the real GEMM's own split-K workspace - each piece at a multiple
+  // of 256 bytes, in that order - or 0 for the products small enough for the kernel on interleaved data.
+  static size_t TempBytes(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
+                          const size_t n, const size_t k, const size_t min_indirect_size);
+
+ private:
+  struct TempLayout {
+    bool small_kernel;  // one launch on the interleaved data, no temporaries
+    size_t expanded_bytes, transposed_bytes, workspace_bytes;
+    size_t transposed_at, workspace_at, total;
+  };
+  static TempLayout PlanTemp(const size_t rows, const size_t columns, const size_t k, const bool right_kcontig,
+                             const bool full, const size_t min_indirect_size);
 };
 
 // The Level-3 routines of the complex types on top of it (reference: the float2/double2 instantiations of

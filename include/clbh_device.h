@@ -258,6 +258,12 @@ CLBH_API int clbh_upload_async(void* dst_device, const void* src_host, size_t by
 
 CLBH_API int clbh_event_record(hipEvent_t event, hipStream_t stream);
 
+// *capturing = 1 while work enqueued on `stream` is being recorded into a HIP graph instead of executed.
+CLBH_API int clbh_stream_capturing(hipStream_t stream, int* capturing);
+// Non-zero for the handle values that do not name one stream: hipStreamPerThread (a different stream in every host
+// thread) and hipStreamLegacy.
+CLBH_API int clbh_stream_is_alias(hipStream_t stream);
+
 // Ordinal of the device `stream` belongs to (the current device for the null stream).
 CLBH_API int clbh_stream_device(hipStream_t stream, int* device);
 

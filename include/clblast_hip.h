@@ -113,8 +113,7 @@ using double2 = std::complex<double>;
 
 // =================================================================================================
 
-// C = alpha * op(A) * op(B) + beta * C. T is float, double, half, float2 or double2 (the complex types take no
-// temp_buffer). GemmBatched, GemmStridedBatched, Symm, Syrk, Syr2k, Trmm and Trsm below also exist for float2 and
+// C = alpha * op(A) * op(B) + beta * C. T is float, double, half, float2 or double2. GemmBatched, GemmStridedBatched, Symm, Syrk, Syr2k, Trmm and Trsm below also exist for float2 and
 // double2; Convgemm, like the reference's, does not.
 template <typename T>
 StatusCode Gemm(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
@@ -232,7 +231,7 @@ StatusCode Convgemm(const KernelMode kernel_mode, const size_t channels, const s
                     const void* kernel_buffer, const size_t kernel_offset, void* result_buffer,
                     const size_t result_offset, hipStream_t* queue, hipEvent_t* event = nullptr);
 
-// Bytes this engine wants in `temp_buffer` for the given arguments (0 when none is needed).
+// Bytes this engine wants in `temp_buffer` for the given arguments (0 when none is needed). T as for Gemm.
 template <typename T>
 StatusCode GemmTempBufferSize(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
                               const size_t m, const size_t n, const size_t k, const size_t a_offset, const size_t a_ld,

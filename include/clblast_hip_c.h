@@ -443,6 +443,28 @@ CLBlastStatusCode CLBLAST_HIP_API CLBlastHgemmWithTempBuffer(
     const void* b_buffer, const size_t b_offset, const size_t b_ld, const cl_half beta, void* c_buffer,
     const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event, void* temp_buffer);
 
+// The complex forms. replaces CLBlast{C,Z}gemmWithTempBuffer and CLBlast{C,Z}GemmTempBufferSize (reference:
+// include/clblast_c.h:1385-1400, 1426-1439): the temporary buffer holds the real form of the first operand, the
+// transposed second operand when needed, and the real GEMM's split-K workspace.
+CLBlastStatusCode CLBLAST_HIP_API CLBlastCgemmWithTempBuffer(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const CLBlastFloat2 alpha, const void* a_buffer, const size_t a_offset,
+    const size_t a_ld, const void* b_buffer, const size_t b_offset, const size_t b_ld, const CLBlastFloat2 beta,
+    void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event, void* temp_buffer);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastZgemmWithTempBuffer(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const CLBlastDouble2 alpha, const void* a_buffer, const size_t a_offset,
+    const size_t a_ld, const void* b_buffer, const size_t b_offset, const size_t b_ld, const CLBlastDouble2 beta,
+    void* c_buffer, const size_t c_offset, const size_t c_ld, hipStream_t* queue, hipEvent_t* event, void* temp_buffer);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastCGemmTempBufferSize(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const size_t a_offset, const size_t a_ld, const size_t b_offset, const size_t b_ld,
+    const size_t c_offset, const size_t c_ld, hipStream_t* queue, size_t* temp_buffer_size);
+CLBlastStatusCode CLBLAST_HIP_API CLBlastZGemmTempBufferSize(
+    const CLBlastLayout layout, const CLBlastTranspose a_transpose, const CLBlastTranspose b_transpose, const size_t m,
+    const size_t n, const size_t k, const size_t a_offset, const size_t a_ld, const size_t b_offset, const size_t b_ld,
+    const size_t c_offset, const size_t c_ld, hipStream_t* queue, size_t* temp_buffer_size);
+
 // =================================================================================================
 // SGEMM that allocates nothing. No counterpart in the reference: it is for callers that cannot allocate device memory
 // (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). Same arguments and results as

@@ -91,21 +91,27 @@ def test_batches_of_matrices_of_a_few_tiles_with_a_short_k(gpu, bits):
             run_strided(gpu, bits, layout, ta, tb, m, n, k, -0.5, 1.25, batch, strides[0], strides[1], offsets, extra, seed)
 
 
+@pytest.mark.parametrize("bits", [16, 32, 64])
 @pytest.mark.parametrize("layout", [ROW_MAJOR, COL_MAJOR])
-def test_strided_batched_small_matrix_kernel(gpu, layout):
-    """m, n, k <= 32 with many batches takes the one-wavefront-per-matrix kernel: dense 32^3 (16-byte loads)
-    and ragged / padded / offset variants (element-wise loads)."""
+def test_strided_batched_small_matrix_kernel(gpu, layout, bits):
+    """m, n, k <= 32 with many batches takes the one-wavefront-per-matrix kernel, which has its own LDS tiles and MFMA
+    per precision (fp16: [x][k] tiles of pitch 40 and fp32 accumulation; fp64: two wavefronts per work-group, 2 x 2
+    blocks): dense 32^3 at 16-byte aligned addresses (the 16-byte loads of every precision), the same at offsets that
+    are not, ragged / padded / offset variants (element-wise loads), broadcast operands (stride 0). Reference sweep:
+    test/routines/levelx/xgemmstridedbatched.hpp:21-194."""
     seed = 100
     for ta, tb in itertools.product((NO, YES), (NO, YES)):
         for (m, n, k), extra, offsets, strides in [((32, 32, 32), (0, 0, 0), (0, 0, 0), (1024, 1024)),
+                                                   ((32, 32, 32), (0, 0, 0), (8, 16, 24), (1024, 1024)),
                                                    ((32, 32, 32), (0, 0, 0), (4, 8, 12), (1024, 1024)),
                                                    ((32, 32, 32), (1, 0, 2), (3, 1, 5), (None, None)),
                                                    ((17, 31, 9), (0, 0, 0), (0, 0, 0), (None, None)),
                                                    ((1, 32, 32), (2, 2, 2), (1, 1, 1), (None, None)),
+                                                   ((32, 16, 24), (0, 0, 0), (0, 0, 0), (32 * 24, 24 * 16)),  # dense, not 32^3
                                                    ((32, 32, 32), (0, 0, 0), (0, 0, 0), (0, 0))]:  # broadcast A and B
             for alpha, beta in ((1.0, 0.0), (-0.75, 2.0)):
                 seed += 3
-                run_strided(gpu, 32, layout, ta, tb, m, n, k, alpha, beta, 67, strides[0], strides[1], offsets, extra, seed)
+                run_strided(gpu, bits, layout, ta, tb, m, n, k, alpha, beta, 67, strides[0], strides[1], offsets, extra, seed)
 
 
 @pytest.mark.parametrize("bits", [32, 64, 16])

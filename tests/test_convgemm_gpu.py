@@ -31,6 +31,10 @@ CASES = [  # channels, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h
     (6, 9, 15, 3, 2, 0, 1, 2, 1, 1, 1, 70, 2),     # odd padded width (one more column of zeros in fp16), output width 16
     (2, 12, 24, 3, 3, 2, 2, 1, 1, 2, 2, 33, 2),    # dilation 2: even tap offsets only; (next) 130 kernels, two tile columns
     (8, 6, 8, 3, 3, 1, 1, 1, 1, 1, 1, 130, 5),
+    # kernel windows taller / wider than the padded image: the output extent is clamped to 1 and the taps beyond the
+    # image count as zeros (output widths 8 and 1: the first would otherwise qualify for the gather of whole vectors)
+    (3, 2, 10, 3, 3, 0, 0, 1, 1, 1, 1, 5, 2),
+    (2, 6, 2, 3, 5, 1, 0, 1, 1, 1, 1, 4, 2),
 ]
 
 

@@ -38,7 +38,18 @@ def test_replays_match_eager_calls(gpu):
     with torch.cuda.graph(graph, stream=side):
         calls(a, b, c, torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
+    big_a, big_b, big_c = draw(640 * 16384), draw(640 * 16384), draw(640 * 640)
     for replay in range(3):
+        if replay == 1:
+            # An eager call on the captured stream that wants a larger workspace than the buffer the graph knows: the
+            # buffer must stay where it is (the call takes stream-ordered memory instead), or the next replay would
+            # write its partial sums into freed memory.
+            with torch.cuda.stream(side):
+                status = clblast_amd.raw_gemm("S", COL_MAJOR, NO, NO, 640, 640, 16384, 1.0, big_a.data_ptr(), 0, 640,
+                                              big_b.data_ptr(), 0, 16384, 0.0, big_c.data_ptr(), 0, 640, side.cuda_stream)
+                assert status == 0
+            side.synchronize()
+            assert clblast_amd.clear_cache() == 0  # must leave the captured buffer alone, too
         a.copy_(draw(a.numel()))  # the program's own eager work between replays
         b.copy_(draw(b.numel()))
         for target, source in zip(c, initial):
