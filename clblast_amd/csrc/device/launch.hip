@@ -21,6 +21,9 @@ int LaunchTyped(const clbh_gemm_desc& d, hipStream_t stream) {
   if (d.conv != nullptr && !(mfma && (d.precision == 32 || d.precision == 16))) { return hipErrorInvalidValue; }  // only those kernels gather
   if (d.kernel_class == CLBH_KERNEL_SMALL_BATCHED) { return LaunchSmallBatched(d, stream); }
   if (d.kernel_class == CLBH_KERNEL_SMALL_TILED) { return LaunchSmallTiled(d, stream); }
+  if (d.kernel_class == CLBH_KERNEL_STREAM) {
+    return d.precision == 32 ? LaunchStreamF32(d, stream) : d.precision == 64 ? LaunchStreamF64(d, stream) : hipErrorInvalidValue;
+  }
   switch (d.precision) {
     case 16: return mfma ? LaunchMfmaF16(d, stream) : LaunchGeneralF16(d, stream);
     case 32: return mfma ? LaunchMfmaF32(d, stream) : LaunchGeneralF32(d, stream);
@@ -44,7 +47,8 @@ bool ValidDescriptor(const clbh_gemm_desc& d) {
   if (d.c_triangle < 0 || d.c_triangle > 4 || d.operand_triangle < 0 || d.operand_triangle > 4) { return false; }
   // the one-wavefront-per-matrix kernel knows no triangles
   if ((d.c_triangle != 0 || d.operand_triangle != 0) &&
-      (d.kernel_class == CLBH_KERNEL_SMALL_BATCHED || d.kernel_class == CLBH_KERNEL_SMALL_TILED)) {
+      (d.kernel_class == CLBH_KERNEL_SMALL_BATCHED || d.kernel_class == CLBH_KERNEL_SMALL_TILED ||
+       d.kernel_class == CLBH_KERNEL_STREAM)) {
     return false;
   }
   return true;

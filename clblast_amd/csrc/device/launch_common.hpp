@@ -24,6 +24,8 @@ int LaunchMfmaF64(const clbh_gemm_desc& d, hipStream_t stream);
 int LaunchSmallBatched(const clbh_gemm_desc& d, hipStream_t stream);
 int LaunchComplexSmall(const clbh_complex_small_desc& d, hipStream_t stream);
 int LaunchSmallTiled(const clbh_gemm_desc& d, hipStream_t stream);
+int LaunchStreamF32(const clbh_gemm_desc& d, hipStream_t stream);
+int LaunchStreamF64(const clbh_gemm_desc& d, hipStream_t stream);
 
 constexpr int kMaxGridY = 65535;
 

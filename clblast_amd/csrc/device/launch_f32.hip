@@ -52,6 +52,12 @@ int LaunchMfmaF32(const clbh_gemm_desc& d, hipStream_t stream) {
 }
 
 
+int LaunchStreamF32(const clbh_gemm_desc& d, hipStream_t stream) {
+  // tile_variant 1: tiles of 128 x 128 x 16 (for launches that read no old C: that tile has no registers to spare for it)
+  if (d.tile_variant == 1) { return LaunchStreamConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16, 2>>(d, stream); }
+  return LaunchStreamConfig<float, MfmaConfig<float, 2, 2, 1, 1, 16, 4>>(d, stream);  // 64 x 64 x 16
+}
+
 int LaunchGeneralF32(const clbh_gemm_desc& d, hipStream_t stream) { return LaunchGeneral<float>(d, stream); }
 
 }  // namespace clbh

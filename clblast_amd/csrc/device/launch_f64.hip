@@ -21,6 +21,10 @@ int LaunchMfmaF64(const clbh_gemm_desc& d, hipStream_t stream) {
 }
 
 
+int LaunchStreamF64(const clbh_gemm_desc& d, hipStream_t stream) {
+  return LaunchStreamConfig<double, MfmaConfig<double, 2, 2, 2, 2, 16, 3>>(d, stream);  // 64 x 64 x 16
+}
+
 int LaunchGeneralF64(const clbh_gemm_desc& d, hipStream_t stream) { return LaunchGeneral<double>(d, stream); }
 
 }  // namespace clbh

@@ -8,6 +8,7 @@
 #include "device/launch_common.hpp"
 #include "kernels/gemm_general.hpp"
 #include "kernels/gemm_mfma.hpp"
+#include "kernels/gemm_stream.hpp"
 
 namespace clbh {
 namespace {
@@ -68,6 +69,61 @@ int LaunchMfmaVariant(const clbh_gemm_desc& d, hipStream_t stream) {
         static_cast<T>(d.alpha), static_cast<T>(d.beta));
   }
   return static_cast<int>(hipGetLastError());
+}
+
+// ---- persistent kernel for many tiles with a short K walk ---------------------------------------------
+template <typename T, typename Config, bool A_KC, bool B_KC, bool USE_C>
+int LaunchStreamVariant(const clbh_gemm_desc& d, hipStream_t stream) {
+  const auto args = MakeArgs<T>(d);
+  const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
+  const long long tiles_n = (d.n + Config::TILE_N - 1) / Config::TILE_N;
+  const long long items = tiles_m * tiles_n * d.batch_count;
+  if (items > INT_MAX / 2) { return hipErrorInvalidConfiguration; }
+  constexpr size_t lds_bytes = Config::LDS_ELEMS * sizeof(T);
+  auto kernel = GemmStreamKernel<T, Config, A_KC, B_KC, USE_C>;
+  // as many work-groups as the GPU holds at once (a multiple of 8: work-group g runs on XCD g % 8, and the walk over
+  // the items relies on item i going to XCD i % 8)
+  struct Residency { hipError_t status; int groups; };
+  static const Residency residency = [&]() {
+    Residency r{hipSuccess, 0};
+    if (lds_bytes > 48 * 1024) {
+      r.status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     static_cast<int>(lds_bytes));
+      if (r.status != hipSuccess) { return r; }
+    }
+    int device = 0, units = 0, per_unit = 0;
+    r.status = hipGetDevice(&device);
+    if (r.status == hipSuccess) { r.status = hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device); }
+    if (r.status == hipSuccess) {
+      r.status = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_unit, reinterpret_cast<const void*>(kernel), kMfmaThreads, lds_bytes);
+    }
+    r.groups = std::max(8, units * std::max(1, per_unit) / 8 * 8);
+    return r;
+  }();
+  if (residency.status != hipSuccess) { return static_cast<int>(residency.status); }
+  const auto groups = static_cast<unsigned>(std::min<long long>(residency.groups, (items + 7) / 8 * 8));
+  kernel<<<dim3(groups), dim3(kMfmaThreads), lds_bytes, stream>>>(args, static_cast<int>(tiles_m), static_cast<int>(tiles_n),
+                                                                  static_cast<int>(items));
+  return static_cast<int>(hipGetLastError());
+}
+
+template <typename T, typename Config>
+int LaunchStreamConfig(const clbh_gemm_desc& d, hipStream_t stream) {
+  if (d.c_triangle != 0 || d.operand_triangle != 0 || d.conv != nullptr || d.k <= 3 * Config::TILE_K || d.m < Config::FM || !LeadingDimsFitTiles<T>(d)) {
+    return hipErrorInvalidValue;
+  }
+  const bool use_c = (d.batch.alphas != nullptr) || d.beta != 0.0;  // per-matrix betas: some may be non-zero
+  const int variant = (d.a_kcontig ? 4 : 0) | (d.b_kcontig ? 2 : 0) | (use_c ? 1 : 0);
+  switch (variant) {
+    case 0: return LaunchStreamVariant<T, Config, false, false, false>(d, stream);
+    case 1: return LaunchStreamVariant<T, Config, false, false, true>(d, stream);
+    case 2: return LaunchStreamVariant<T, Config, false, true, false>(d, stream);
+    case 3: return LaunchStreamVariant<T, Config, false, true, true>(d, stream);
+    case 4: return LaunchStreamVariant<T, Config, true, false, false>(d, stream);
+    case 5: return LaunchStreamVariant<T, Config, true, false, true>(d, stream);
+    case 6: return LaunchStreamVariant<T, Config, true, true, false>(d, stream);
+    default: return LaunchStreamVariant<T, Config, true, true, true>(d, stream);
+  }
 }
 
 template <typename T, typename Config>

@@ -125,12 +125,23 @@ __device__ __forceinline__ void ResolveBatch(const GemmArgs<CT>& p, const int ba
 // Epilogue rule of the reference kernels: with beta == 0 the old C is never read, so NaN/Inf in it do
 // not propagate (reference: src/kernels/level3/xgemm_part2.opencl:84-165,
 // xgemm_direct_part1.opencl:178-187). alpha == 0 is not special-cased.
+// alpha * acc + beta * old with one fixed sequence of roundings - the product alpha * acc, then one fused
+// multiply-add - wherever an epilogue combines its sum with the old C: left to the compiler, the contraction of
+// `alpha * acc + beta * old` comes out differently in different code paths, and the same element would get different
+// last bits depending on the path that stored it (a masked tile on a triangle's diagonal against a full tile).
+__device__ __forceinline__ float Combine(const float alpha, const float acc, const float beta, const float old) {
+  return __builtin_fmaf(beta, old, alpha * acc);
+}
+__device__ __forceinline__ double Combine(const double alpha, const double acc, const double beta, const double old) {
+  return __builtin_fma(beta, old, alpha * acc);
+}
+
 template <typename T, typename CT>
 __device__ __forceinline__ void StoreResult(T* c, const long long index, const CT acc, const CT alpha, const CT beta) {
   if (beta == CT(0)) {
     c[index] = static_cast<T>(alpha * acc);
   } else {
-    c[index] = static_cast<T>(alpha * acc + beta * static_cast<CT>(c[index]));
+    c[index] = static_cast<T>(Combine(alpha, acc, beta, static_cast<CT>(c[index])));
   }
 }
 

@@ -703,14 +703,14 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
             VMG out;
 #pragma unroll
             for (int i = 0; i < FM; ++i) {
-              out[i] = (beta == T(0)) ? alpha * acc[i][j][r] : alpha * acc[i][j][r] + beta * old_c[(j * ACC + r) * FM + i];
+              out[i] = (beta == T(0)) ? alpha * acc[i][j][r] : Combine(alpha, acc[i][j][r], beta, old_c[(j * ACC + r) * FM + i]);
             }
             *reinterpret_cast<VMG*>(dst) = out;
           } else {
 #pragma unroll
             for (int i = 0; i < FM; ++i) {
               if (writes(i, n)) {
-                dst[i * M_STEP] = (beta == T(0)) ? alpha * acc[i][j][r] : alpha * acc[i][j][r] + beta * old_c[(j * ACC + r) * FM + i];
+                dst[i * M_STEP] = (beta == T(0)) ? alpha * acc[i][j][r] : Combine(alpha, acc[i][j][r], beta, old_c[(j * ACC + r) * FM + i]);
               }
             }
           }
@@ -745,7 +745,7 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
                 for (int i = 0; i < FM; ++i) { out[i] = alpha * acc[i][j][r]; }
               } else {
 #pragma unroll
-                for (int i = 0; i < FM; ++i) { out[i] = alpha * acc[i][j][r] + beta * old[rr][i]; }
+                for (int i = 0; i < FM; ++i) { out[i] = Combine(alpha, acc[i][j][r], beta, old[rr][i]); }
               }
               *reinterpret_cast<VMG*>(dst) = out;
             } else {

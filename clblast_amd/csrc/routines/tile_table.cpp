@@ -110,7 +110,7 @@ int SplitFor(const size_t tiles, const size_t k, const bool small_tile = false) 
 
 KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const bool b_kcontig, const size_t m,
                           const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,
-                          const size_t min_indirect_size, const bool triangular) {
+                          const size_t min_indirect_size, const bool triangular, const bool beta_zero) {
   (void)a_kcontig; (void)b_kcontig; (void)per_batch_scalars;
   // Many small matrices: one wavefront per matrix, bandwidth bound (that kernel knows no triangles)
   if (!triangular && batch_count >= 16 && m <= 32 && n <= 32 && k <= 32) {
@@ -123,6 +123,23 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     return KernelChoice{CLBH_KERNEL_GENERAL, 0, 1};
   }
   const auto forced = ForcedTileVariant(precision);
+  // Thousands of tiles with a short K walk: the launch is a stream over C, and work-groups that stay resident and
+  // overlap one tile's C traffic with the products of the next beat one work-group per tile. Tiles of 64 x 64 -
+  // fp32 8191 x 8191 x 127: 271 -> 225 us, 4096 x 4096 x 128: 63 -> 55 us, 512 x 256 x 256 x 64: 106 -> 79 us (no gain
+  // is left from k = 256 on); fp64 512 x 256 x 256 x 64: 209 -> 150 us, 64 x 512 x 512 x 128: 107 -> 92 us. fp32 tiles of
+  // 128 x 128 (a quarter of the operand traffic per flop, but no registers to spare: the old C of a tile comes in one
+  // burst) where no old C is read - 8191 x 8191 x 127: 219 -> 166 us, x 511: 608 -> 519 us - or where its columns lie
+  // close together in memory (matrices of up to 1024 rows: 512 x 256 x 256 x 64 106 -> 67 us, 1024 x 128^3 60 -> 54 us; at
+  // 8191 rows the 128 column pieces of a tile are 32 KB apart and their reads take longer than the products).
+  if (forced == 0 && !triangular && precision != Precision::kHalf && k > 48) {
+    const auto tiles128 = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
+    if (precision == Precision::kSingle && tiles128 >= 1024 && TileUse(m, n, 128, 128) >= 90 &&
+        (beta_zero ? k <= 512 : (k <= 256 && m <= 1024))) {
+      return KernelChoice{CLBH_KERNEL_STREAM, 1, 1};
+    }
+    const auto tiles64 = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;
+    if (k <= 192 && tiles64 >= 4096 && TileUse(m, n, 64, 64) >= 80) { return KernelChoice{CLBH_KERNEL_STREAM, 2, 1}; }
+  }
   // Batches of fp32 / fp64 matrices of a few tiles with a short k are bound by HBM and latency, not by the matrix
   // cores: the kernel that keeps one slab per operand in LDS runs eight work-groups or more per CU (fp32 4096 x 64^3:
   // 49 -> 42 us, 1024 x 96^3: 53 -> 43 us with tiles of 32 x 32; fp64 2048 x 128 x 64 x 64: 123 -> 75 us). With a
@@ -131,6 +148,13 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       k <= (precision == Precision::kSingle ? 96u : 64u) && CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count >= 512) {
     const auto padded = [m, n](const size_t tile) { return CeilDivide(m, tile) * CeilDivide(n, tile) * tile * tile; };
     return KernelChoice{CLBH_KERNEL_SMALL_TILED, (4 * padded(32) < 3 * padded(64)) ? 1 : 0, 1};
+  }
+  if ((forced == 101 || forced == 102) && !triangular && precision != Precision::kHalf) {
+    return KernelChoice{CLBH_KERNEL_SMALL_TILED, static_cast<int>(forced) - 101, 1};  // one-slab kernel, 64 x 64 / 32 x 32 tiles
+  }
+  if ((forced == 103 || forced == 104) && !triangular && precision != Precision::kHalf && k > 48) {
+    // persistent work-groups over tiles of 64 x 64, or (fp32) 128 x 128
+    return KernelChoice{CLBH_KERNEL_STREAM, (forced == 104 && precision == Precision::kSingle) ? 1 : 2, 1};
   }
   if (forced != 0) {
     // a forced tile takes the forced number of K ranges (unbatched calls only), never more than k / 16

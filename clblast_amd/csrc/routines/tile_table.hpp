@@ -33,9 +33,10 @@ bool UseDirectKernel(const size_t m, const size_t n, const size_t k, const size_
 
 // Picks the kernel family and tile for a canonical problem (m, n, k per matrix). `triangular`: about half of the
 // tile work of the launch is skipped (a triangle of C, or a triangular operand), which calls for smaller tiles.
+// `beta_zero`: the old C is not read (the choice never changes the workspace a problem needs).
 KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const bool b_kcontig, const size_t m,
                           const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,
-                          const size_t min_indirect_size, const bool triangular = false);
+                          const size_t min_indirect_size, const bool triangular = false, const bool beta_zero = false);
 
 // Tile forced for a precision through OverrideParameters("Xgemm", {"TILE_VARIANT": 1 + index}); 0 = automatic.
 size_t ForcedTileVariant(const Precision precision);
