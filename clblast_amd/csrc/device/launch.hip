@@ -24,6 +24,7 @@ int LaunchTyped(const clbh_gemm_desc& d, hipStream_t stream) {
   if (d.kernel_class == CLBH_KERNEL_STREAM) {
     return d.precision == 32 ? LaunchStreamF32(d, stream) : d.precision == 64 ? LaunchStreamF64(d, stream) : hipErrorInvalidValue;
   }
+  if (d.kernel_class == CLBH_KERNEL_SKINNY) { return LaunchSkinnyF32(d, stream); }
   switch (d.precision) {
     case 16: return mfma ? LaunchMfmaF16(d, stream) : LaunchGeneralF16(d, stream);
     case 32: return mfma ? LaunchMfmaF32(d, stream) : LaunchGeneralF32(d, stream);
@@ -48,7 +49,7 @@ bool ValidDescriptor(const clbh_gemm_desc& d) {
   // the one-wavefront-per-matrix kernel knows no triangles
   if ((d.c_triangle != 0 || d.operand_triangle != 0) &&
       (d.kernel_class == CLBH_KERNEL_SMALL_BATCHED || d.kernel_class == CLBH_KERNEL_SMALL_TILED ||
-       d.kernel_class == CLBH_KERNEL_STREAM)) {
+       d.kernel_class == CLBH_KERNEL_STREAM || d.kernel_class == CLBH_KERNEL_SKINNY)) {
     return false;
   }
   return true;
@@ -263,7 +264,8 @@ int clbh_gemm_launch(const clbh_gemm_desc* desc, hipStream_t stream) {
 }
 
 size_t clbh_gemm_workspace_bytes(const clbh_gemm_desc* desc) {
-  if (desc == nullptr || desc->kernel_class != CLBH_KERNEL_MFMA) { return 0; }
+  if (desc == nullptr || (desc->kernel_class != CLBH_KERNEL_MFMA && desc->kernel_class != CLBH_KERNEL_SKINNY)) { return 0; }
+  if (desc->kernel_class == CLBH_KERNEL_SKINNY) { return clbh::SkinnyWorkspaceBytes(*desc); }
   const auto plan = clbh::PlanSplit(*desc);
   if (plan.splits <= 1) { return 0; }
   const auto element_bytes = static_cast<size_t>(desc->precision == 16 ? 4 : desc->precision / 8);  // fp16 sums in fp32

@@ -26,6 +26,7 @@ int LaunchComplexSmall(const clbh_complex_small_desc& d, hipStream_t stream);
 int LaunchSmallTiled(const clbh_gemm_desc& d, hipStream_t stream);
 int LaunchStreamF32(const clbh_gemm_desc& d, hipStream_t stream);
 int LaunchStreamF64(const clbh_gemm_desc& d, hipStream_t stream);
+int LaunchSkinnyF32(const clbh_gemm_desc& d, hipStream_t stream);
 
 constexpr int kMaxGridY = 65535;
 
@@ -163,6 +164,11 @@ inline SplitPlan PlanSplit(const clbh_gemm_desc& d) {
   }
   return plan;
 }
+
+// K ranges of a launch of the kernel for skinny problems (launch_skinny.hip): `chunk` is the range of a work-group.
+SplitPlan PlanSkinny(const clbh_gemm_desc& d);
+// Workspace bytes of such a launch: the slabs of its K ranges, or (tile_variant 2) a k-contiguous copy of the small operand
+size_t SkinnyWorkspaceBytes(const clbh_gemm_desc& d);
 
 }  // namespace clbh
 

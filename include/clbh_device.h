@@ -34,12 +34,17 @@ enum clbh_kernel_class {
   CLBH_KERNEL_GENERAL = 0,  // bounds-checked LDS-tiled FMA kernel, any shape (reference analogue: XgemmDirect)
   CLBH_KERNEL_MFMA = 1,     // large-tile MFMA kernel with LDS double buffering (analogue: Xgemm indirect)
   CLBH_KERNEL_SMALL_BATCHED = 2,  // one wavefront per small matrix, bandwidth bound
-  CLBH_KERNEL_SKINNY = 3,         // split-K streaming kernel for problems with a tiny m or n
+  CLBH_KERNEL_SKINNY = 3,         // fp32, m or n at most 32, unbatched, no triangles: streams the large operand through
+                                  // registers, K split over the wavefronts of a work-group (tile_variant 1: four,
+                                  // else eight) and over split_k work-groups; leading dimensions below
+                                  // CLBH_SKINNY_MAX_LD
   CLBH_KERNEL_SMALL_TILED = 4,    // fp32 / fp64 batches of matrices of a few tiles: one slab per operand in LDS, many
                                   // work-groups per CU (tile_variant 1: tiles of 32 x 32, else 64 x 64)
   CLBH_KERNEL_STREAM = 5          // fp32 / fp64 launches of many 64 x 64 tiles with a short K walk (k > 48): persistent
                                   // work-groups that overlap an item's C traffic with the products of its neighbours
 };
+
+#define CLBH_SKINNY_MAX_LD (1ll << 21)
 
 // Per-batch metadata of GemmBatched, all device pointers (NULL for plain and strided launches).
 typedef struct clbh_batch_arrays_ {

@@ -262,3 +262,46 @@ def test_persistent_kernel_for_many_tiles_with_a_short_k(gpu, bits):
         torch.cuda.synchronize()
     finally:
         clblast_amd.override_parameters(0, "Xgemm", bits, {"TILE_VARIANT": 0})
+
+
+def test_register_streaming_kernel_for_skinny_problems(gpu):
+    """The fp32 kernel for a C of at most 32 rows or columns (it streams the large operand through registers and splits
+    K over wavefronts and work-groups): picked by the tile table for the first shapes, forced - with one and with several
+    K ranges - on the others; every operand orientation and both layouts, the small extent from 1 to 32, large extents
+    that end inside a tile of 128, K tails that are no multiple of 4, 32 or the range, K shorter than one work-group's
+    share, padded leading dimensions, offsets, NaNs in C under beta zero and NaNs in every element of the A and B buffers
+    outside the logical matrices."""
+    import clblast_amd
+    import torch
+    seed = 8800
+    shapes = ((4099, 17, 4096), (17, 4099, 4096), (1030, 32, 1000), (1, 700, 513), (600, 1, 300), (2000, 5, 131),
+              (31, 515, 258), (128, 32, 128), (129, 3, 33))
+    try:
+        for (m, n, k), (ta, tb) in itertools.product(shapes, itertools.product(TRANSPOSES, TRANSPOSES)):
+            for forced_split in ((0,) if m * n >= 17 * 4099 else (1, 3, 64)):
+                seed += 1
+                if forced_split:  # (eight wavefronts per work-group, or four, or - where the large operand is
+                    # k-contiguous, else the choice is automatic - the kernel with its lanes along k)
+                    clblast_amd.override_parameters(0, "Xgemm", 32, {"TILE_VARIANT": 105 + seed % 3, "SPLIT_K": forced_split})
+                else:
+                    clblast_amd.override_parameters(0, "Xgemm", 32, {"TILE_VARIANT": 0})
+                extra, offsets = (((0, 0, 0), (0, 0, 0)), ((3, 1, 5), (11, 13, 19)), ((8, 8, 8), (16, 8, 24)))[seed % 3]
+                beta = (2.0, 0.0)[(seed // 3) % 2]
+                problem = gpu.Problem(32, (COL_MAJOR, ROW_MAJOR)[(seed // 6) % 2], ta, tb, m, n, k, -0.75, beta,
+                                      a_offset=offsets[0], b_offset=offsets[1], c_offset=offsets[2], seed=seed, extra_ld=extra)
+                for buffer, transpose, rows, cols, offset, ld in ((problem.a, ta, m, k, problem.a_offset, problem.a_ld),
+                                                                  (problem.b, tb, k, n, problem.b_offset, problem.b_ld)):
+                    keep = np.zeros(buffer.size, dtype=bool)
+                    keep[oracle.operand_indices(problem.layout, transpose, rows, cols, offset, ld).ravel()] = True
+                    buffer[~keep] = np.nan
+                if beta == 0.0:
+                    problem.c[:] = np.nan  # beta == 0 never reads C
+                status, c_after = problem.run()
+                assert status == 0, problem.describe()
+                if beta == 0.0:
+                    index = oracle.c_indices(problem.layout, m, n, problem.c_offset, problem.c_ld)
+                    problem.c[index.ravel()] = 0.0
+                problem.check(c_after)
+        torch.cuda.synchronize()
+    finally:
+        clblast_amd.override_parameters(0, "Xgemm", 32, {"TILE_VARIANT": 0})
