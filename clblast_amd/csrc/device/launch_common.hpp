@@ -165,9 +165,8 @@ inline SplitPlan PlanSplit(const clbh_gemm_desc& d) {
   return plan;
 }
 
-// K ranges of a launch of the kernel for skinny problems (launch_skinny.hip): `chunk` is the range of a work-group.
-SplitPlan PlanSkinny(const clbh_gemm_desc& d);
-// Workspace bytes of such a launch: the slabs of its K ranges, or (tile_variant 2) a k-contiguous copy of the small operand
+// Workspace bytes of a launch of the kernel for skinny problems (launch_skinny.hip): a k-contiguous copy of the small
+// operand, where that is not k-contiguous already
 size_t SkinnyWorkspaceBytes(const clbh_gemm_desc& d);
 
 }  // namespace clbh

@@ -34,10 +34,9 @@ enum clbh_kernel_class {
   CLBH_KERNEL_GENERAL = 0,  // bounds-checked LDS-tiled FMA kernel, any shape (reference analogue: XgemmDirect)
   CLBH_KERNEL_MFMA = 1,     // large-tile MFMA kernel with LDS double buffering (analogue: Xgemm indirect)
   CLBH_KERNEL_SMALL_BATCHED = 2,  // one wavefront per small matrix, bandwidth bound
-  CLBH_KERNEL_SKINNY = 3,         // fp32, m or n at most 32, unbatched, no triangles: streams the large operand through
-                                  // registers, K split over the wavefronts of a work-group (tile_variant 1: four,
-                                  // else eight) and over split_k work-groups; leading dimensions below
-                                  // CLBH_SKINNY_MAX_LD
+  CLBH_KERNEL_SKINNY = 3,         // fp32, m or n at most 32, unbatched, no triangles, the large operand k-contiguous
+                                  // (n <= 32: a_kcontig, else b_kcontig), leading dimensions below CLBH_SKINNY_MAX_LD:
+                                  // lanes along k, a work-group owns a few rows of the large operand and all of K
   CLBH_KERNEL_SMALL_TILED = 4,    // fp32 / fp64 batches of matrices of a few tiles: one slab per operand in LDS, many
                                   // work-groups per CU (tile_variant 1: tiles of 32 x 32, else 64 x 64)
   CLBH_KERNEL_STREAM = 5          // fp32 / fp64 launches of many 64 x 64 tiles with a short K walk (k > 48): persistent

@@ -264,27 +264,24 @@ def test_persistent_kernel_for_many_tiles_with_a_short_k(gpu, bits):
         clblast_amd.override_parameters(0, "Xgemm", bits, {"TILE_VARIANT": 0})
 
 
-def test_register_streaming_kernel_for_skinny_problems(gpu):
-    """The fp32 kernel for a C of at most 32 rows or columns (it streams the large operand through registers and splits
-    K over wavefronts and work-groups): picked by the tile table for the first shapes, forced - with one and with several
-    K ranges - on the others; every operand orientation and both layouts, the small extent from 1 to 32, large extents
-    that end inside a tile of 128, K tails that are no multiple of 4, 32 or the range, K shorter than one work-group's
-    share, padded leading dimensions, offsets, NaNs in C under beta zero and NaNs in every element of the A and B buffers
-    outside the logical matrices."""
+def test_kernel_for_skinny_problems_with_a_k_contiguous_large_operand(gpu):
+    """The fp32 kernel for a C of at most 32 rows or columns whose large operand is k-contiguous (its lanes run along
+    k, a work-group owns a few rows of that operand and all of K): picked by the tile table for the first shapes, forced
+    on the others (where the large operand is not k-contiguous the choice stays automatic); every operand orientation
+    and both layouts, the small extent from 1 to 32, large extents that end inside a group of four rows, K tails that are
+    no multiple of 4 or 64, K shorter than one wavefront's share, a small operand that needs the k-contiguous copy, padded
+    leading dimensions, offsets, NaNs in C under beta zero and NaNs in every element of the A and B buffers outside
+    the logical matrices."""
     import clblast_amd
     import torch
     seed = 8800
     shapes = ((4099, 17, 4096), (17, 4099, 4096), (1030, 32, 1000), (1, 700, 513), (600, 1, 300), (2000, 5, 131),
-              (31, 515, 258), (128, 32, 128), (129, 3, 33))
+              (31, 515, 258), (128, 32, 128), (129, 3, 33), (2051, 20, 70), (8, 3000, 1027))
     try:
         for (m, n, k), (ta, tb) in itertools.product(shapes, itertools.product(TRANSPOSES, TRANSPOSES)):
-            for forced_split in ((0,) if m * n >= 17 * 4099 else (1, 3, 64)):
+            for forced in ((0,) if m * n >= 17 * 4099 else (105, 0)):
                 seed += 1
-                if forced_split:  # (eight wavefronts per work-group, or four, or - where the large operand is
-                    # k-contiguous, else the choice is automatic - the kernel with its lanes along k)
-                    clblast_amd.override_parameters(0, "Xgemm", 32, {"TILE_VARIANT": 105 + seed % 3, "SPLIT_K": forced_split})
-                else:
-                    clblast_amd.override_parameters(0, "Xgemm", 32, {"TILE_VARIANT": 0})
+                clblast_amd.override_parameters(0, "Xgemm", 32, {"TILE_VARIANT": forced})
                 extra, offsets = (((0, 0, 0), (0, 0, 0)), ((3, 1, 5), (11, 13, 19)), ((8, 8, 8), (16, 8, 24)))[seed % 3]
                 beta = (2.0, 0.0)[(seed // 3) % 2]
                 problem = gpu.Problem(32, (COL_MAJOR, ROW_MAJOR)[(seed // 6) % 2], ta, tb, m, n, k, -0.75, beta,
