@@ -264,8 +264,7 @@ int clbh_gemm_launch(const clbh_gemm_desc* desc, hipStream_t stream) {
 }
 
 size_t clbh_gemm_workspace_bytes(const clbh_gemm_desc* desc) {
-  if (desc == nullptr || (desc->kernel_class != CLBH_KERNEL_MFMA && desc->kernel_class != CLBH_KERNEL_SKINNY)) { return 0; }
-  if (desc->kernel_class == CLBH_KERNEL_SKINNY) { return clbh::SkinnyWorkspaceBytes(*desc); }
+  if (desc == nullptr || desc->kernel_class != CLBH_KERNEL_MFMA) { return 0; }
   const auto plan = clbh::PlanSplit(*desc);
   if (plan.splits <= 1) { return 0; }
   const auto element_bytes = static_cast<size_t>(desc->precision == 16 ? 4 : desc->precision / 8);  // fp16 sums in fp32

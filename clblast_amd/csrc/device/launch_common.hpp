@@ -165,10 +165,6 @@ inline SplitPlan PlanSplit(const clbh_gemm_desc& d) {
   return plan;
 }
 
-// Workspace bytes of a launch of the kernel for skinny problems (launch_skinny.hip): a k-contiguous copy of the small
-// operand, where that is not k-contiguous already
-size_t SkinnyWorkspaceBytes(const clbh_gemm_desc& d);
-
 }  // namespace clbh
 
 #endif  // CLBLAST_HIP_DEVICE_LAUNCH_COMMON_HPP_

@@ -12,13 +12,18 @@ namespace {
 constexpr int kRowsWaves = 4, kRowsDepth = 2;
 
 template <int GROUPS, int ROW_GROUPS>
-int LaunchSkinnyRows(SkinnyArgs args, const bool x_is_a, hipStream_t stream) {
+int LaunchSkinnyRows(SkinnyArgs args, const bool x_is_a, const bool s_kc, hipStream_t stream) {
   constexpr size_t lds_bytes = sizeof(float) * SkinnyRowsLdsFloats(kRowsWaves, GROUPS, ROW_GROUPS);
   static_assert(lds_bytes <= 48 * 1024, "more LDS than a kernel gets without asking");
   args.k_per_wave = ((args.k + kRowsWaves - 1) / kRowsWaves + kSkinnyRowsStep - 1) / kSkinnyRowsStep * kSkinnyRowsStep;
   const dim3 grid(static_cast<unsigned>((args.extent + 4 * ROW_GROUPS - 1) / (4 * ROW_GROUPS)));
-  if (x_is_a) { GemmSkinnyRowsKernel<kRowsWaves, GROUPS, ROW_GROUPS, kRowsDepth, true><<<grid, dim3(64 * kRowsWaves), lds_bytes, stream>>>(args); }
-  else { GemmSkinnyRowsKernel<kRowsWaves, GROUPS, ROW_GROUPS, kRowsDepth, false><<<grid, dim3(64 * kRowsWaves), lds_bytes, stream>>>(args); }
+  const dim3 block(64 * kRowsWaves);
+  switch ((x_is_a ? 2 : 0) | (s_kc ? 1 : 0)) {
+    case 0: GemmSkinnyRowsKernel<kRowsWaves, GROUPS, ROW_GROUPS, kRowsDepth, false, false><<<grid, block, lds_bytes, stream>>>(args); break;
+    case 1: GemmSkinnyRowsKernel<kRowsWaves, GROUPS, ROW_GROUPS, kRowsDepth, false, true><<<grid, block, lds_bytes, stream>>>(args); break;
+    case 2: GemmSkinnyRowsKernel<kRowsWaves, GROUPS, ROW_GROUPS, kRowsDepth, true, false><<<grid, block, lds_bytes, stream>>>(args); break;
+    default: GemmSkinnyRowsKernel<kRowsWaves, GROUPS, ROW_GROUPS, kRowsDepth, true, true><<<grid, block, lds_bytes, stream>>>(args); break;
+  }
   return static_cast<int>(hipGetLastError());
 }
 
@@ -26,7 +31,7 @@ int LaunchSkinnyRows(SkinnyArgs args, const bool x_is_a, hipStream_t stream) {
 // takes as long as the CU with the most rows. 4099 rows: 257 work-groups of 16 rows leave one CU with two of them (32
 // rows, 23 us); 205 work-groups of 20 rows take 17 us.
 template <int GROUPS, int MAX_ROW_GROUPS>
-int LaunchSkinnyRowsBalanced(const SkinnyArgs& args, const bool x_is_a, hipStream_t stream) {
+int LaunchSkinnyRowsBalanced(const SkinnyArgs& args, const bool x_is_a, const bool s_kc, hipStream_t stream) {
   int units = 256;
   int device = 0;
   if (hipGetDevice(&device) == hipSuccess) { (void)hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device); }
@@ -38,26 +43,20 @@ int LaunchSkinnyRowsBalanced(const SkinnyArgs& args, const bool x_is_a, hipStrea
     if (best_rows < 0 || busiest <= best_rows) { best = row_groups; best_rows = busiest; }  // (ties: fewer reads of S)
   }
   switch (best) {
-    case 2: return LaunchSkinnyRows<GROUPS, 2>(args, x_is_a, stream);
-    case 3: return LaunchSkinnyRows<GROUPS, 3>(args, x_is_a, stream);
-    case 4: return LaunchSkinnyRows<GROUPS, (MAX_ROW_GROUPS >= 4 ? 4 : MAX_ROW_GROUPS)>(args, x_is_a, stream);
-    default: return LaunchSkinnyRows<GROUPS, (MAX_ROW_GROUPS >= 5 ? 5 : MAX_ROW_GROUPS)>(args, x_is_a, stream);
+    case 2: return LaunchSkinnyRows<GROUPS, 2>(args, x_is_a, s_kc, stream);
+    case 3: return LaunchSkinnyRows<GROUPS, 3>(args, x_is_a, s_kc, stream);
+    case 4: return LaunchSkinnyRows<GROUPS, (MAX_ROW_GROUPS >= 4 ? 4 : MAX_ROW_GROUPS)>(args, x_is_a, s_kc, stream);
+    default: return LaunchSkinnyRows<GROUPS, (MAX_ROW_GROUPS >= 5 ? 5 : MAX_ROW_GROUPS)>(args, x_is_a, s_kc, stream);
   }
 }
 
 bool SkinnyXIsA(const clbh_gemm_desc& d) { return d.n <= 32; }
 bool SkinnySKcontig(const clbh_gemm_desc& d) { return SkinnyXIsA(d) ? (d.b_kcontig != 0) : (d.a_kcontig != 0); }
-long long SkinnyCopyLd(const clbh_gemm_desc& d) { return (static_cast<long long>(d.k) + 3) / 4 * 4; }
-
 }  // namespace
-
-size_t SkinnyWorkspaceBytes(const clbh_gemm_desc& d) {  // a k-contiguous copy of the small operand, where it is not
-  return SkinnySKcontig(d) ? 0 : sizeof(float) * static_cast<size_t>(SkinnyCopyLd(d)) * static_cast<size_t>(std::min(d.m, d.n));
-}
 
 int LaunchSkinnyF32(const clbh_gemm_desc& d, hipStream_t stream) {
   if (d.precision != 32 || d.batch_count != 1 || d.batch.alphas != nullptr || d.c_triangle != 0 || d.operand_triangle != 0 ||
-      d.conv != nullptr || std::min(d.m, d.n) > 32 || d.a_ld >= CLBH_SKINNY_MAX_LD || d.b_ld >= CLBH_SKINNY_MAX_LD) {
+      d.conv != nullptr || std::min(d.m, d.n) > 32 || d.k >= (1 << 28) || d.a_ld >= CLBH_SKINNY_MAX_LD || d.b_ld >= CLBH_SKINNY_MAX_LD) {
     return hipErrorInvalidValue;
   }
   const bool x_is_a = SkinnyXIsA(d);
@@ -76,17 +75,11 @@ int LaunchSkinnyF32(const clbh_gemm_desc& d, hipStream_t stream) {
   args.k = d.k;
   args.alpha = static_cast<float>(d.alpha);
   args.beta = static_cast<float>(d.beta);
-  if (!SkinnySKcontig(d)) {
-    if (d.workspace == nullptr || d.workspace_bytes < SkinnyWorkspaceBytes(d)) { return hipErrorInvalidValue; }
-    SkinnyTransposeKernel<<<dim3(static_cast<unsigned>((d.k + 31) / 32)), dim3(256), 0, stream>>>(
-        args.s, args.s_ld, d.k, args.small, static_cast<float*>(d.workspace), SkinnyCopyLd(d));
-    args.s = static_cast<const float*>(d.workspace);
-    args.s_ld = SkinnyCopyLd(d);
-  }
+  const bool s_kc = SkinnySKcontig(d);
   // (column groups, and the most row groups whose sums fit the registers beside them)
-  if (args.small <= 8) { return LaunchSkinnyRowsBalanced<2, 5>(args, x_is_a, stream); }
-  if (args.small <= 20) { return LaunchSkinnyRowsBalanced<5, 5>(args, x_is_a, stream); }
-  return LaunchSkinnyRowsBalanced<8, 3>(args, x_is_a, stream);
+  if (args.small <= 8) { return LaunchSkinnyRowsBalanced<2, 5>(args, x_is_a, s_kc, stream); }
+  if (args.small <= 20) { return LaunchSkinnyRowsBalanced<5, 5>(args, x_is_a, s_kc, stream); }
+  return LaunchSkinnyRowsBalanced<8, 3>(args, x_is_a, s_kc, stream);
 }
 
 }  // namespace clbh

@@ -49,16 +49,18 @@ struct SkinnyArgs {
 // wavefronts: no second pass, no workspace. A lane's sums cover its share of k only; they meet at the end - first the
 // four lanes of a 16-lane row that hold the same row of X (two rotations), then rows and wavefronts through LDS, added
 // in a fixed order.
-// S must be k-contiguous as well (element (k, col) at s[col * s_ld + k]): a lane loads the four k of its block for
-// column 4g + lane % 4 in one piece, which is the A operand of its block as it stands. Both operands are requested
-// DEPTH steps (of 64 k) ahead: the counter of outstanding loads completes in order, a wait for a late request of S
-// would wait for every earlier request of X too.
+// S comes straight from memory (L2 holds all of it) in the layout of the A operand. S_KC, element (k, col) at
+// s[col * s_ld + k]: a lane loads the four k of its block for column 4g + lane % 4 in one piece. Otherwise, element at
+// s[k * s_ld + col]: lane % 4 = i takes the GROUPS consecutive columns from i * GROUPS on, one piece per k (which
+// column a result register stands for is a matter of the epilogue only). Both operands are requested DEPTH steps (of
+// 64 k) ahead: the counter of outstanding loads completes in order, a wait for a late request of S would wait for every
+// earlier request of X too.
 // =================================================================================================
 constexpr int kSkinnyRowsStep = 64;  // k per step and wavefront
 
 constexpr int SkinnyRowsLdsFloats(const int waves, const int groups, const int rg) { return waves * 4 * (4 * rg) * (4 * groups); }
 
-template <int WAVES, int GROUPS, int RG, int DEPTH, bool X_IS_A, int WAVES_PER_SIMD = 2>
+template <int WAVES, int GROUPS, int RG, int DEPTH, bool X_IS_A, bool S_KC, int WAVES_PER_SIMD = 2>
 __global__ __launch_bounds__(64 * WAVES, WAVES_PER_SIMD) void GemmSkinnyRowsKernel(const SkinnyArgs p) {
   typedef float float4_t __attribute__((ext_vector_type(4)));
   extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -111,9 +113,10 @@ __global__ __launch_bounds__(64 * WAVES, WAVES_PER_SIMD) void GemmSkinnyRowsKern
   // straddles the end reads what lies there (the next row, padding; zeros behind the operand) and is cleaned below.
   // Rows of X beyond its extent and columns of S beyond p.small read the last valid one (their results are not stored).
   const float* x_base = p.x + static_cast<long long>(row0) * p.x_ld + k_begin;
-  const float* s_base = p.s + k_begin;
+  const float* s_base = p.s + (S_KC ? k_begin : k_begin * p.s_ld);
   const long long x_valid = static_cast<long long>(rows - 1) * p.x_ld + p.k - k_begin;
-  const long long s_valid = static_cast<long long>(p.small - 1) * p.s_ld + p.k - k_begin;
+  const long long s_valid = S_KC ? static_cast<long long>(p.small - 1) * p.s_ld + p.k - k_begin
+                                 : static_cast<long long>(p.k - k_begin - 1) * p.s_ld + p.small;
   constexpr int kOutside = 0x7fffff00;  // (an offset no resource reaches)
   const int x_records = static_cast<int>(min(max(x_valid, 0ll) * 4, static_cast<long long>(kOutside)));
   const int s_records = static_cast<int>(min(max(s_valid, 0ll) * 4, static_cast<long long>(kOutside)));
@@ -122,20 +125,49 @@ __global__ __launch_bounds__(64 * WAVES, WAVES_PER_SIMD) void GemmSkinnyRowsKern
   for (int r = 0; r < RG; ++r) { x_offset[r] = static_cast<int>((min(4 * r + quad_lane, rows - 1) * p.x_ld + 4 * slot) * 4); }
 #pragma unroll
   for (int g = 0; g < GROUPS; ++g) { s_offset[g] = static_cast<int>((min(4 * g + quad_lane, p.small - 1) * p.s_ld + 4 * slot) * 4); }
+  const int s_row_bytes = static_cast<int>(p.s_ld * 4);                                     // (column-contiguous S)
+  const int s_lane_bytes = static_cast<int>((4 * slot * p.s_ld + quad_lane * GROUPS) * 4);  // (k = 4 * slot, column i * GROUPS)
 
-  float4_t x_ring[DEPTH][RG], s_ring[DEPTH][GROUPS];
+  float4_t x_ring[DEPTH][RG], s_ring[DEPTH][S_KC ? GROUPS : 1];
+  float s_pieces[DEPTH][4][S_KC ? 1 : GROUPS];  // (column-contiguous S: [t][g])
   auto request = [&](const int d, const int position) {
     const int step = rotated(position);
     // (the offsets go through an empty asm statement: the compiler would otherwise turn each select into a branch
     // around two loads, and could no longer count the loads in flight)
     const int step_bytes = (step * kSkinnyRowsStep < lane_length) ? step * kSkinnyRowsStep * 4 : kOutside;
     const auto x_resource = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(x_base), 0, x_records, kRawBufferFlags);
-    const auto s_resource = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(s_base), 0, s_records, kRawBufferFlags);
+    // (a column-contiguous S advances by whole rows of it per step: the resource moves along, the lane's offset stays small)
+    const long long s_step = S_KC ? 0 : static_cast<long long>(step) * kSkinnyRowsStep * p.s_ld;
+    const int s_step_records = static_cast<int>(min(max(s_valid - s_step, 0ll) * 4, static_cast<long long>(kOutside)));
+    const auto s_resource = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(s_base + s_step), 0,
+                                                              S_KC ? s_records : s_step_records, kRawBufferFlags);
+    if constexpr (S_KC) {
 #pragma unroll
-    for (int g = 0; g < GROUPS; ++g) {
-      int offset = s_offset[g] + step_bytes;
-      asm volatile("" : "+v"(offset));
-      s_ring[d][g] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(s_resource, offset, 0, 0));
+      for (int g = 0; g < GROUPS; ++g) {
+        int offset = s_offset[g] + step_bytes;
+        asm volatile("" : "+v"(offset));
+        s_ring[d][g] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(s_resource, offset, 0, 0));
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {  // k = 64 * step + 4 * slot + t: valid while inside the lane's range. (The column
+        // offsets of the pieces are part of the lane's offset, which is what the resource's range is checked against.)
+        int offset = (step * kSkinnyRowsStep + t < lane_length) ? s_lane_bytes + t * s_row_bytes : kOutside;
+        asm volatile("" : "+v"(offset));
+        int g = 0;
+#pragma unroll
+        for (; g + 4 <= GROUPS; g += 4) {
+          const float4_t piece = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(s_resource, offset + 4 * g, 0, 0));
+          s_pieces[d][t][g] = piece[0]; s_pieces[d][t][g + 1] = piece[1]; s_pieces[d][t][g + 2] = piece[2]; s_pieces[d][t][g + 3] = piece[3];
+        }
+        if (g + 2 <= GROUPS) {
+          typedef float float2_t __attribute__((ext_vector_type(2)));
+          const float2_t piece = __builtin_bit_cast(float2_t, __builtin_amdgcn_raw_buffer_load_b64(s_resource, offset + 4 * g, 0, 0));
+          s_pieces[d][t][g] = piece[0]; s_pieces[d][t][g + 1] = piece[1];
+          g += 2;
+        }
+        if (g < GROUPS) { s_pieces[d][t][g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(s_resource, offset + 4 * g, 0, 0)); }
+      }
     }
 #pragma unroll
     for (int r = 0; r < RG; ++r) {
@@ -158,8 +190,10 @@ __global__ __launch_bounds__(64 * WAVES, WAVES_PER_SIMD) void GemmSkinnyRowsKern
         for (int t = 1; t < 4; ++t) {
 #pragma unroll
           for (int r = 0; r < RG; ++r) { x_ring[d][r][t] = (t < left) ? x_ring[d][r][t] : 0.0f; }
+          if constexpr (S_KC) {
 #pragma unroll
-          for (int g = 0; g < GROUPS; ++g) { s_ring[d][g][t] = (t < left) ? s_ring[d][g][t] : 0.0f; }
+            for (int g = 0; g < GROUPS; ++g) { s_ring[d][g][t] = (t < left) ? s_ring[d][g][t] : 0.0f; }
+          }
         }
       }
 #pragma unroll
@@ -168,7 +202,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES_PER_SIMD) void GemmSkinnyRowsKern
         for (int r = 0; r < RG; ++r) {
 #pragma unroll
           for (int g = 0; g < GROUPS; ++g) {
-            acc[r][g] = __builtin_amdgcn_mfma_f32_4x4x1f32(s_ring[d][g][t], x_ring[d][r][t], acc[r][g], 0, 0, 0);
+            const float s_value = S_KC ? s_ring[d][g][t] : s_pieces[d][t][g];
+            acc[r][g] = __builtin_amdgcn_mfma_f32_4x4x1f32(s_value, x_ring[d][r][t], acc[r][g], 0, 0, 0);
           }
         }
       }
@@ -204,7 +239,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES_PER_SIMD) void GemmSkinnyRowsKern
 #pragma unroll
       for (int g = 0; g < GROUPS; ++g) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { mine[element(4 * r + quad_lane, 4 * g + i)] = acc[r][g][i]; }
+        for (int i = 0; i < 4; ++i) { mine[element(4 * r + quad_lane, S_KC ? 4 * g + i : i * GROUPS + g)] = acc[r][g][i]; }
       }
     }
   }
@@ -220,22 +255,6 @@ __global__ __launch_bounds__(64 * WAVES, WAVES_PER_SIMD) void GemmSkinnyRowsKern
       for (int part = 0; part < 4 * WAVES; ++part) { sum += lds[part * ELEMENTS + e]; }
       p.c[index] = (p.beta != 0.0f) ? Combine(p.alpha, sum, p.beta, old_c[q]) : p.alpha * sum;
     }
-  }
-}
-
-// Copies S (element (k, col) at s[k * s_ld + col]) into a k-contiguous one (at target[col * target_ld + k]) for
-// GemmSkinnyRowsKernel: 32 x 32 tiles through LDS.
-__global__ __launch_bounds__(256) void SkinnyTransposeKernel(const float* __restrict__ s, const long long s_ld, const int k,
-                                                             const int columns, float* __restrict__ target,
-                                                             const long long target_ld) {
-  __shared__ float tile[32][33];
-  const int k0 = blockIdx.x * 32, lane_x = threadIdx.x % 32, lane_y = threadIdx.x / 32;
-  for (int kk = lane_y; kk < 32; kk += 8) {
-    tile[kk][lane_x] = (k0 + kk < k && lane_x < columns) ? s[(k0 + kk) * s_ld + lane_x] : 0.0f;
-  }
-  __syncthreads();
-  for (int col = lane_y; col < columns; col += 8) {
-    if (k0 + lane_x < k) { target[col * target_ld + k0 + lane_x] = tile[lane_x][col]; }
   }
 }
 

@@ -157,7 +157,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     // persistent work-groups over tiles of 64 x 64, or (fp32) 128 x 128
     return KernelChoice{CLBH_KERNEL_STREAM, (forced == 104 && precision == Precision::kSingle) ? 1 : 2, 1};
   }
-  if (forced == 105 && precision == Precision::kSingle && !triangular && batch_count == 1 && std::min(m, n) <= 32 &&
+  if (forced == 105 && precision == Precision::kSingle && !triangular && batch_count == 1 && std::min(m, n) <= 32 && k < (size_t{1} << 28) &&
       largest_ld < static_cast<size_t>(CLBH_SKINNY_MAX_LD) && (n <= 32 ? a_kcontig : b_kcontig)) {
     return KernelChoice{CLBH_KERNEL_SKINNY, 0, 1};  // the lanes-along-k kernel for a k-contiguous large operand
   }
@@ -214,9 +214,9 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     // (1024^3: 28.5 -> 23.8 us), and up to 64 such tiles with a short k the 32 x 32 tile does so again (512^3: 16.0 -> 8.8 us).
     // A C of at most 32 rows or columns with a long k is a stream over the large operand. Where that operand is
     // k-contiguous, the kernel that puts its lanes along k and gives a work-group 8 to 20 rows and all of K does it in one
-    // launch (4099 x 17 x 4096 with a transposed A: 27.5 us on 64 x 32 tiles with K split, 16.4 us here; 17 x 4099 x 4096,
-    // whose small operand is copied into a k-contiguous one first: 27.5 -> 19.3 us)
-    if (batch_count == 1 && std::min(m, n) <= 32 && std::max(m, n) >= 1024 && k >= 512 && (n <= 32 ? a_kcontig : b_kcontig) &&
+    // launch (4099 x 17 x 4096 with a transposed A: 27.5 us on 64 x 32 tiles with K split, 16.4 us here; 17 x 4099 x 4096:
+    // 27.5 -> 17.7 us)
+    if (batch_count == 1 && std::min(m, n) <= 32 && std::max(m, n) >= 1024 && k >= 512 && k < (size_t{1} << 28) && (n <= 32 ? a_kcontig : b_kcontig) &&
         largest_ld < static_cast<size_t>(CLBH_SKINNY_MAX_LD)) {
       return KernelChoice{CLBH_KERNEL_SKINNY, 0, 1};
     }
