@@ -30,10 +30,28 @@ PEAK_HBM_GBS = 8000.0
 BITS = {"S": 32, "D": 64, "H": 16, "C": 64, "Z": 128}
 DTYPE_NAME = {"S": "f32", "D": "f64", "H": "f16", "C": "c64 (f32 arithmetic)", "Z": "c128 (f64 arithmetic)"}
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
-# the readings of a plain 1 GiB copy (profiles/<workload>.md holds the commands and the raw readings). A bench run
-# cannot collect counters itself, so these are the figures of the committed profiles.
-MEASURED_TRAFFIC_BYTES = {"cfg2s": 5.602e9, "cfg2d": 1.0697e10, "cfg3": 1.888e9, "cfg4": 1.007e8, "cfg5d": 6.319e8, "sbat64": 2.014e8,
-                          "cgemm_batched": 4.028e8}
+# the readings of a plain 1 GiB copy. A bench run cannot collect counters itself, so these are the figures of the
+# committed profiles: workload -> (bytes, the profile that holds the commands and the raw readings, the kernel they
+# were read for). The roofline object names both, and tests/test_bench_contract.py checks each entry against its file.
+MEASURED_TRAFFIC = {
+    "cfg2s": (5.680e9, "profiles/sgemm_8192_rowTN.md", "clbh::GemmMfmaKernel<float, clbh::MfmaConfig<float, 2, 2, 4, 2, 16, 2"),
+    "cfg2d": (1.2002e10, "profiles/dgemm_8192_rowTN.md", "clbh::GemmMfmaKernel<double, clbh::MfmaConfig<double, 2, 2, 4, 4, 8, 2"),
+    "cfg3": (1.900e9, "profiles/hgemm_8192_colNT.md", "clbh::HgemmDirectKernel<clbh::HdirectConfig<2, 4, 4, 2, 2, 3, false>"),
+    "cfg4": (1.007e8, "profiles/sgemm_strided_batched_8192x32.md", "clbh::GemmSmallBatchedKernel"),
+    "cfg5c": (7.465e7, "profiles/sgemm_17x4099x4096_colNN.md", "clbh::GemmSkinnyRowsKernel<4, 5, 5, 2, false, false, 2>"),
+    "cfg5d": (6.389e8, "profiles/sgemm_8191x8191x127_colNN.md", "clbh::GemmStreamKernel<float, clbh::MfmaConfig<float, 2, 2, 1, 1, 16, 4"),
+    "cfg5e": (7.367e7, "profiles/sgemm_4099x17x4096_colTN.md", "clbh::GemmSkinnyRowsKernel<4, 5, 5, 2, true, true, 2>"),
+    "sbat64": (2.019e8, "profiles/sgemm_strided_batched_4096x64.md", "clbh::GemmStreamKernel<float, clbh::MfmaConfig<float, 2, 2, 1, 1, 16, 4"),
+    "cgemm_batched": (4.028e8, "profiles/cgemm_strided_batched_4096x64_rowNC.md", "clbh::GemmComplexSmallKernel<float, 2, true, true>"),
+}
+
+
+def traffic_of(workload_name):
+    """The `traffic` and `traffic_source` members of a roofline object (null where no counter run is committed)."""
+    entry = MEASURED_TRAFFIC.get(workload_name)
+    if entry is None:
+        return {"traffic": None}
+    return {"traffic": entry[0], "traffic_source": "%s (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of %s)" % (entry[1], entry[2])}
 
 
 def parse_args():
@@ -439,11 +457,11 @@ def roofline_of(workload, device_ms):
     if intensity >= ridge:
         achieved = workload.flops / seconds / 1e12
         peak = PEAK_TFLOPS[workload.prefix]
-        return {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(workload.name)}
+        return dict({"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(achieved / peak, 4)}, **traffic_of(workload.name))
     achieved = workload.algorithmic_bytes / seconds / 1e9
-    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-            "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(workload.name)}
+    return dict({"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                 "frac": round(achieved / PEAK_HBM_GBS, 4)}, **traffic_of(workload.name))
 
 
 def cpu_baseline(target_seconds=15.0):
@@ -552,6 +570,8 @@ EXTRA_WORKLOADS = {
                                                        4106, (11, 13, 19)),
     "cfg5_sgemm_17x4099x4096_colNN": lambda: Workload("cfg5c", "S", COL, NO, NO, 17, 4099, 4096, -0.75, 2.0, 20, 4101,
                                                        24, (11, 13, 19)),
+    "cfg5_sgemm_4099x17x4096_colTN": lambda: Workload("cfg5e", "S", COL, YES, NO, 4099, 17, 4096, -0.75, 2.0, 4099, 4101,
+                                                       4106, (11, 13, 19)),
     "cfg5_sgemm_8191x8191x127_colNN": lambda: Workload("cfg5d", "S", COL, NO, NO, 8191, 8191, 127, -0.75, 2.0, 8194,
                                                         132, 8198, (11, 13, 19)),
     "next_sgemm_strided_batched_4096x64": lambda: Workload("sbat64", "S", ROW, NO, NO, 64, 64, 64, 1.0, 0.0, batch=4096),
@@ -596,6 +616,49 @@ def run_extra(name, steps, warmup):
     return entry
 
 
+def run_mfma_ceiling(steps):
+    """The matrix pipe's sustained fp16 rate on the operands of the cfg3 workload: the library's measurement kernel runs
+    nothing but v_mfma_f32_16x16x32_f16 on fragments taken from the same A and B (two wavefronts per SIMD, about 1 ms
+    per launch). The HGEMM line is read against this ceiling: the pipe's clock under load depends on the data."""
+    import ctypes
+    import torch
+    from clblast_amd import _lib
+    lib = _lib.load()
+    workload = EXTRA_WORKLOADS["cfg3_hgemm_8192_colNT"]()
+    lib.clbh_probe_mfma_f16_out_bytes.restype = ctypes.c_size_t
+    lib.clbh_probe_mfma_f16_out_bytes.argtypes = [ctypes.c_int]
+    lib.clbh_probe_mfma_f16_flops.restype = ctypes.c_double
+    lib.clbh_probe_mfma_f16_flops.argtypes = [ctypes.c_int, ctypes.c_int]
+    lib.clbh_probe_mfma_f16.restype = ctypes.c_int
+    lib.clbh_probe_mfma_f16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int, ctypes.c_int,
+                                        ctypes.c_void_p, ctypes.c_void_p]
+    groups, iterations = 256, 1000
+    out = torch.empty(lib.clbh_probe_mfma_f16_out_bytes(groups) // 4, dtype=torch.float32, device="cuda")
+    elements = min(workload.a.numel(), workload.b.numel()) // 8 * 8
+    stream = torch.cuda.Stream()
+
+    def launch():
+        status = lib.clbh_probe_mfma_f16(workload.a.data_ptr(), workload.b.data_ptr(), elements, groups, iterations,
+                                         out.data_ptr(), stream.cuda_stream)
+        if status != 0:
+            sys.exit("bench.py: clbh_probe_mfma_f16 failed with %d" % status)
+    with torch.cuda.stream(stream):
+        for _ in range(20):
+            launch()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record(stream)
+        for _ in range(max(steps, 100)):
+            launch()
+        stop.record(stream)
+        torch.cuda.synchronize()
+    ms = start.elapsed_time(stop) / max(steps, 100)
+    tflops = lib.clbh_probe_mfma_f16_flops(groups, iterations) / (ms * 1e-3) / 1e12
+    return {"ms": round(ms, 4), "tflops": round(tflops, 1), "frac_of_peak": round(tflops / PEAK_TFLOPS["H"], 4),
+            "instruction": "v_mfma_f32_16x16x32_f16", "data": "operands of cfg3_hgemm_8192_colNT",
+            "hgemm_flop_at_this_rate_ms": round(2.0 * 8192 ** 3 / (tflops * 1e12) * 1e3, 4)}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -614,6 +677,9 @@ def main():
         del source, target
         torch.cuda.empty_cache()
 
+    if args.only == "probe_hgemm_mfma_ceiling":
+        print(json.dumps({args.only: run_mfma_ceiling(args.steps)}))
+        return
     if args.only is not None:
         print(json.dumps({args.only: run_extra(args.only, args.steps, args.warmup)}))
         return
