@@ -7,11 +7,13 @@
 //
 // Structure (one work-group = 256 threads = 4 wavefronts):
 //   * the work-group owns a TILE_M x TILE_N block of C; K is walked in slabs of TILE_K;
-//   * global -> registers -> LDS staging with two LDS buffers, so that the loads of slab t+1 are in
-//     flight while slab t feeds the matrix cores, with one barrier per slab;
+//   * a ring of three LDS slab buffers: while slab t feeds the matrix cores, slab t+1 has landed or is
+//     landing and slab t+2 is being requested into the buffer that the previous barrier released; one
+//     barrier per slab;
 //   * both operands sit in LDS as [k][x] (x = m for A, n for B; x contiguous) whatever their layout in
-//     memory: x-contiguous operands are copied with 16-byte loads and stores, k-contiguous ones are
-//     loaded with 16-byte loads along k and scattered into LDS (a transpose on the fly);
+//     memory: x-contiguous operands go from global memory straight into LDS (buffer loads with the LDS
+//     as destination, 16 bytes per lane), k-contiguous ones are loaded into registers with 16-byte
+//     loads along k and scattered into LDS (a transpose on the fly);
 //   * each wavefront computes a (MF*FM) x (MF*FN) block with v_mfma_f32_32x32x2_f32 (MF = 32) or
 //     v_mfma_f64_16x16x4_f64 (MF = 16). The n-indexed values are fed as the MFMA's A operand and the
 //     m-indexed ones as its B operand, so the lanes of a result register run along m: stores to the

@@ -2,9 +2,11 @@
 // Xconvgemm<T>: host logic of Convgemm<T>, batched 2-D convolution as matrix multiplication (reference:
 // src/routines/levelx/xconvgemm.{hpp,cpp}, doc/details_conv.md). Images are batch x channels x height x width,
 // kernels num_kernels x channels x kernel_h x kernel_w, the result batch x num_kernels x output_h x output_w, all
-// contiguous. Of the reference's two methods this is "im2col + batched GEMM" (xconvgemm.cpp:78-100), with one im2col
-// launch for the whole batch instead of one per image and the strided-batched GEMM of this engine (the kernel matrix
-// has batch stride 0) instead of a dedicated kernel.
+// contiguous. The reference has two methods (xconvgemm.cpp:78-100): "im2col + batched GEMM" and a GEMM kernel that
+// gathers its patches itself. Both exist here: fp32 and - for images without padding whose kernel window fits, unit
+// width stride and suitable widths - fp16 run ONE strided-batched GEMM launch whose A loader gathers the patches from
+// the images (no im2col matrix); fp64 and the remaining fp16 shapes materialise the im2col matrix with one launch for
+// the whole batch and then run the strided-batched GEMM of this engine (the kernel matrix has batch stride 0).
 // =================================================================================================
 #ifndef CLBLAST_HIP_ROUTINES_XCONVGEMM_HPP_
 #define CLBLAST_HIP_ROUTINES_XCONVGEMM_HPP_
