@@ -167,20 +167,30 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     return KernelChoice{CLBH_KERNEL_MFMA, static_cast<int>(forced) - 1, static_cast<int>(ranges)};
   }
   if (triangular) {
-    // About half of the tile work is skipped and what remains is uneven: the largest tile that still leaves four
-    // rounds of working tiles for the 256 CUs, so that the dispatcher can even the load out; never split K.
-    struct Candidate { int index; size_t tile_m, tile_n; };
-    static constexpr Candidate kHalfTiles[] = {{2, 256, 256}, {0, 128, 128}, {1, 64, 64}};
-    static constexpr Candidate kSingleTiles[] = {{3, 256, 128}, {0, 128, 128}, {7, 64, 64}};
-    static constexpr Candidate kDoubleTiles[] = {{0, 128, 128}, {1, 64, 64}, {1, 64, 64}};
-    const auto* candidates = (precision == Precision::kHalf) ? kHalfTiles
-                             : (precision == Precision::kSingle) ? kSingleTiles : kDoubleTiles;
-    auto tile = candidates[2].index;
-    for (int c = 0; c < 3; ++c) {
-      const auto working = CeilDivide(m, candidates[c].tile_m) * CeilDivide(n, candidates[c].tile_n) * batch_count / 2;
-      if (working >= 4 * 256) { tile = candidates[c].index; break; }
+    // About half of the tile work is skipped and what remains is uneven, so the dispatcher needs spare tiles to even
+    // the load out; never split K. Working tiles: about half of the grid.
+    const auto working = [&](const size_t tile_m, const size_t tile_n) {
+      return CeilDivide(m, tile_m) * CeilDivide(n, tile_n) * batch_count / 2;
+    };
+    if (precision == Precision::kHalf) {
+      // The large tiles run at a much higher rate than the small ones in fp16 (256 x 256: 50 % of the peak, 64 x 64:
+      // 30 %), which outweighs rounds that stay partly empty. Measured (SYRK, lower triangle, n = k): 4096 142 us on
+      // 64 x 64, 100 us on 128 x 128; 8192 853 us on 128 x 128, 559 us on 256 x 256; 8192 x 1024 (short k) 89 us on
+      // 128 x 128, 104 us on 256 x 256; 2048 and below are fastest on 64 x 64.
+      if (working(256, 256) >= 512 && k >= 2048) { return KernelChoice{CLBH_KERNEL_MFMA, 2, 1}; }
+      if (working(128, 128) >= 256) { return KernelChoice{CLBH_KERNEL_MFMA, 0, 1}; }
+      return KernelChoice{CLBH_KERNEL_MFMA, 1, 1};
     }
-    return KernelChoice{CLBH_KERNEL_MFMA, tile, 1};
+    if (precision == Precision::kSingle) {
+      // From about 6000 rows on the 128 x 64 tile of the 16x16x4 MFMA (two work-groups per CU) beats 128 x 128 and
+      // 256 x 128 (SYRK n = k = 8192: 4.65 -> 4.08 ms, 6144: 2.09 -> 1.81 ms); below, the largest tile that still leaves
+      // four rounds of working tiles for the 256 CUs.
+      if (working(128, 64) >= 2048) { return KernelChoice{CLBH_KERNEL_MFMA, 11, 1}; }
+      if (working(256, 128) >= 4 * 256) { return KernelChoice{CLBH_KERNEL_MFMA, 3, 1}; }
+      if (working(128, 128) >= 4 * 256) { return KernelChoice{CLBH_KERNEL_MFMA, 0, 1}; }
+      return KernelChoice{CLBH_KERNEL_MFMA, 7, 1};
+    }
+    return KernelChoice{CLBH_KERNEL_MFMA, (working(128, 128) >= 4 * 256) ? 0 : 1, 1};
   }
   if (precision == Precision::kHalf) {
     // Direct-load tiles, 0: 128 x 128, 1: 64 x 64, 2: 256 x 256 (8 wavefronts), 3: 128 x 32, 4: 32 x 128. Measured
