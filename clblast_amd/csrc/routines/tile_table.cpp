@@ -235,7 +235,16 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     if (n <= 32 && m >= 256) { tile = Tile{9, 64, 32}; }         // skinny: stream A
     else if (m <= 32 && n >= 256) { tile = Tile{8, 32, 64}; }    // skinny: stream B
     else if (k >= (batch_count > 1 ? 256u : 1024u) && FillsRounds(CeilDivide(m, 256) * CeilDivide(n, 128) * batch_count) &&
-             TileUse(m, n, 256, 128) >= 80) { tile = Tile{3, 256, 128}; }  // (batches: 256 x 256^3 96 -> 80 us)
+             TileUse(m, n, 256, 128) >= 80) {
+      tile = Tile{3, 256, 128};  // (batches: 256 x 256^3 96 -> 80 us)
+      // ... unless its last round stays emptier than that of 128 x 128 tiles, two of which share a CU (6144^3: four and
+      // a half rounds of 256 x 128 take 3.54 ms, nine of 128 x 128 3.20 ms; at whole rounds 256 x 128 is 1-2 % ahead)
+      const auto big = CeilDivide(m, 256) * CeilDivide(n, 128) * batch_count, half = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
+      const auto fill = [](const size_t tiles, const size_t slots) { return 100 * tiles / (CeilDivide(tiles, slots) * slots); };
+      if (batch_count == 1 && fill(big, 256) < 95 && fill(half, 256) >= fill(big, 256) + 5 && TileUse(m, n, 128, 128) >= 80) {
+        tile = Tile{0, 128, 128};
+      }
+    }
     else if (batch_count > 1 && TileUse(m, n, 128, 128) >= 90 && CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count >= 512) {
       tile = Tile{0, 128, 128};  // batches of matrices that fill 128 x 128 tiles (1024 x 128^3: 66 -> 57 us)
     }
@@ -261,10 +270,19 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   if (batch_count > 1 && m <= 128 && n <= 128 && TileUse(m, n, 128, 128) >= 50 && batch_count >= 512) {
     return KernelChoice{CLBH_KERNEL_MFMA, 0, 1};  // batches of matrices of about one 128 x 128 tile (1024 x 96^3: 92 -> 74 us)
   }
-  const bool large = CeilDivide(m, 128) * CeilDivide(n, 128) >= 1024 && k >= 1024;
-  const auto tile_size = large ? size_t{128} : size_t{64};
-  const auto tiles = CeilDivide(m, tile_size) * CeilDivide(n, tile_size) * batch_count;
-  return KernelChoice{CLBH_KERNEL_MFMA, large ? 0 : 1, (batch_count == 1) ? SplitFor(tiles, k) : 1};
+  const auto tiles128 = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
+  if (tiles128 >= 1024 && k >= 1024 && batch_count == 1) {
+    return KernelChoice{CLBH_KERNEL_MFMA, 0, SplitFor(tiles128, k)};
+  }
+  // Between one and four rounds of 128 x 128 tiles the 128 x 64 x 16 tile (two work-groups per CU) wins where its
+  // work-groups come in whole rounds of 512 - 2048^3 301 -> 249 us, 2048^2 x 8192 1.38 -> 0.98 ms, 4096 x 1024 x 4096
+  // 685 -> 496 us - and loses where they do not (3072^3: 963 against 798 us on 64 x 64)
+  const auto pairs = 2 * tiles128;
+  if (batch_count == 1 && k >= 1024 && tiles128 >= 256 && 10 * pairs >= 9 * CeilDivide(pairs, 512) * 512 && TileUse(m, n, 128, 64) >= 90) {
+    return KernelChoice{CLBH_KERNEL_MFMA, 2, 1};
+  }
+  const auto tiles = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;
+  return KernelChoice{CLBH_KERNEL_MFMA, 1, (batch_count == 1) ? SplitFor(tiles, k) : 1};
 }
 
 StatusCode OverrideRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,
