@@ -193,17 +193,24 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     return KernelChoice{CLBH_KERNEL_MFMA, (working(128, 128) >= 4 * 256) ? 0 : 1, 1};
   }
   if (precision == Precision::kHalf) {
-    // Direct-load tiles, 0: 128 x 128, 1: 64 x 64, 2: 256 x 256 (8 wavefronts), 3: 128 x 32, 4: 32 x 128. Measured
-    // (tile sweep over 15 shapes): 256 x 256 when its tiles fill whole rounds of the 256 CUs, 128 x 128 from 256
-    // tiles on, else 64 x 64 - also for skinny shapes.
-    const auto big = CeilDivide(m, 256) * CeilDivide(n, 256) * batch_count;
-    const auto rounds = CeilDivide(big, 256);
-    // A large tile must also be filled by the matrix: batches of small matrices (4096 x 64^3: 32 us on 128 x 128
-    // tiles, 19 us on 64 x 64) count many tiles that are mostly empty.
+    // Direct-load tiles, 0: 128 x 128, 1: 64 x 64, 2: 256 x 256 (8 wavefronts), 3: 128 x 32, 4: 32 x 128 (the last two
+    // lose to 64 x 64 on skinny shapes too). The tile is chosen by a cost estimate: rounds of work-groups (256 x 256: one per CU, 128 x 128: two, 64 x 64: four)
+    // times what a CU spends on a round, tile area over the rate that tile's kernel reaches (relative to 256 x 256: 128 x
+    // 128 0.85, 64 x 64 0.5). Padded tiles count in full, so a matrix that fills a large tile badly pays for it. Checked
+    // against forced tiles on 25 shapes: 5000^3 297 us (64 x 64, the choice of an earlier rule: 672 us), 3500^3 117 us
+    // (215), 7000^3 844 us on 128 x 128 (256 x 256: 889), 1024 x 8192 x 1024 25 us on 128 x 128, 1500^3 38 us on 64 x 64.
+    const auto cost = [&](const size_t tile, const size_t per_cu, const size_t rate_percent) {
+      const auto tiles = CeilDivide(m, tile) * CeilDivide(n, tile) * batch_count;
+      return static_cast<double>(CeilDivide(tiles, 256 * per_cu) * per_cu * tile * tile) * 100.0 / static_cast<double>(rate_percent);
+    };
+    // (with a long k the 64 x 64 kernel stays at 550 TFLOP/s while 128 x 128 climbs to 800: 2048^2 x 8192 takes 125 us
+    // on 64 x 64 tiles and 90 us on 128 x 128 - but only where the latter fill the CUs; below that the 64 x 64 tiles win
+    // with K split)
+    const bool long_k = k >= 4096 && CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count >= 256;
+    const auto cost256 = (k >= 512) ? cost(256, 1, 100) : 1e300, cost128 = cost(128, 2, 85), cost64 = cost(64, 4, long_k ? 38 : 50);
     int tile = 1;
-    if (5 * big >= 4 * rounds * 256 && k >= 512 && TileUse(m, n, 256, 256) + 10 >= TileUse(m, n, 128, 128)) { tile = 2; }
-    else if (CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count >= 256 &&
-             TileUse(m, n, 128, 128) >= TileUse(m, n, 64, 64)) { tile = 0; }
+    if (cost256 <= cost128 && cost256 <= cost64) { tile = 2; }
+    else if (cost128 <= cost64) { tile = 0; }
     // K ranges (fp32 partial sums, then a reduction) when the 64 x 64 tiles would leave the GPU mostly idle through a
     // long K walk: up to 512 work-groups, ranges at least 512 deep - 2048 when there are 192 tiles or more, which by
     // themselves keep most CUs busy (measured: 256^2 x 8192 33.6 -> 13.4 us, 4099 x 17 x 4096 33.9 -> 14.1 us,
@@ -271,7 +278,9 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     return KernelChoice{CLBH_KERNEL_MFMA, 0, 1};  // batches of matrices of about one 128 x 128 tile (1024 x 96^3: 92 -> 74 us)
   }
   const auto tiles128 = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
-  if (tiles128 >= 1024 && k >= 1024 && batch_count == 1) {
+  // (... whose last round is at least 90 % full: 5000^3, 1600 tiles in 6.25 rounds, takes 4.05 ms on them and 3.67 ms
+  // on 64 x 64)
+  if (tiles128 >= 1024 && k >= 1024 && batch_count == 1 && 10 * tiles128 >= 9 * CeilDivide(tiles128, 256) * 256) {
     return KernelChoice{CLBH_KERNEL_MFMA, 0, SplitFor(tiles128, k)};
   }
   // Between one and four rounds of 128 x 128 tiles the 128 x 64 x 16 tile (two work-groups per CU) wins where its
