@@ -292,7 +292,12 @@ __global__ __launch_bounds__(kMfmaThreads, Config::MIN_WAVES) void GemmStreamKer
             *reinterpret_cast<OldC*>(dst) = out;
           }
         }
-      } else {  // a tile on an edge of the matrix reads its old C here, element by element
+      } else {
+        // A tile on an edge of the matrix: element-wise stores under bounds tests (their number is not counted: the next
+        // item's first wait lets them all retire). Its old C has come with the others - fetch_old_c moved a lane's piece
+        // back into the matrix where it would have reached beyond m or n, so the lane's element i is element i + shift of
+        // the piece it holds, whenever that element exists.
+        const int shift = mb - max(min(mb, p.m - FM), 0);
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
 #pragma unroll
@@ -301,7 +306,18 @@ __global__ __launch_bounds__(kMfmaThreads, Config::MIN_WAVES) void GemmStreamKer
             T* dst = current.c + n * p.c_ld + mb;
 #pragma unroll
             for (int i = 0; i < FM; ++i) {
-              if (n < p.n && mb + i < p.m) { StoreResult<T, T>(dst, i, acc[i][j][r], current.alpha, current.beta); }
+              if (n < p.n && mb + i < p.m) {
+                T value = current.alpha * acc[i][j][r];
+                if constexpr (USE_C) {
+                  if (current.beta != T(0)) {
+                    T old = VecGet<OldC, T, FM>(old_c[j * ACC + r], FM - 1);
+#pragma unroll
+                    for (int e = 0; e < FM - 1; ++e) { if (i + shift == e) { old = VecGet<OldC, T, FM>(old_c[j * ACC + r], e); } }
+                    value = Combine(current.alpha, acc[i][j][r], current.beta, old);
+                  }
+                }
+                dst[i] = value;
+              }
             }
           }
         }

@@ -125,17 +125,16 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   }
   const auto forced = ForcedTileVariant(precision);
   // Thousands of tiles with a short K walk: the launch is a stream over C, and work-groups that stay resident and
-  // overlap one tile's C traffic with the products of the next beat one work-group per tile. Tiles of 64 x 64 -
-  // fp32 8191 x 8191 x 127: 271 -> 225 us, 4096 x 4096 x 128: 63 -> 55 us, 512 x 256 x 256 x 64: 106 -> 79 us (no gain
-  // is left from k = 256 on); fp64 512 x 256 x 256 x 64: 209 -> 150 us, 64 x 512 x 512 x 128: 107 -> 92 us. fp32 tiles of
-  // 128 x 128 (a quarter of the operand traffic per flop, but no registers to spare: the old C of a tile comes in one
-  // burst) where no old C is read - 8191 x 8191 x 127: 219 -> 166 us, x 511: 608 -> 519 us - or where its columns lie
-  // close together in memory (matrices of up to 1024 rows: 512 x 256 x 256 x 64 106 -> 67 us, 1024 x 128^3 60 -> 54 us; at
-  // 8191 rows the 128 column pieces of a tile are 32 KB apart and their reads take longer than the products).
+  // overlap one tile's C traffic with the products of the next beat one work-group per tile. fp32 tiles of 128 x 128 (a
+  // quarter of the operand traffic per flop of 64 x 64) where they fill the matrix - 8191 x 8191 x 127 with beta = 2:
+  // 271 us with one work-group per 64 x 64 tile, 230 us with resident work-groups on 64 x 64 tiles, 201 us on 128 x 128
+  // tiles; with beta = 0: 219 -> 159 us; 8192^2 x 256: 367 -> 323 us; no gain is left from k = 512 on - else tiles of
+  // 64 x 64 (4096 x 4096 x 128: 63 -> 55 us, 512 x 256 x 256 x 64: 106 -> 79 us; fp64 512 x 256 x 256 x 64: 209 -> 150 us,
+  // 64 x 512 x 512 x 128: 107 -> 92 us).
   if (forced == 0 && !triangular && precision != Precision::kHalf && k > 48) {
     const auto tiles128 = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
     if (precision == Precision::kSingle && tiles128 >= 1024 && TileUse(m, n, 128, 128) >= 90 &&
-        (beta_zero ? k <= 512 : (k <= 256 && m <= 1024))) {
+        k <= (beta_zero ? 512u : 256u)) {
       return KernelChoice{CLBH_KERNEL_STREAM, 1, 1};
     }
     const auto tiles64 = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;
