@@ -138,7 +138,13 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       return KernelChoice{CLBH_KERNEL_STREAM, 1, 1};
     }
     const auto tiles64 = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;
-    if (k <= 192 && tiles64 >= 4096 && TileUse(m, n, 64, 64) >= 80) { return KernelChoice{CLBH_KERNEL_STREAM, 2, 1}; }
+    // (batches: from 2048 tiles on, and fp64 up to k = 400 - fp64 256 x 256^3 164 -> 153 us, 256 x 200 x 300 x 400
+    // 296 -> 275 us, 128 x 384^3 266 -> 245 us; at k = 512 the tiled kernel is ahead again)
+    const bool batched = batch_count > 1;
+    if (k <= ((batched && precision == Precision::kDouble) ? 400u : 192u) && tiles64 >= (batched ? 2048u : 4096u) &&
+        TileUse(m, n, 64, 64) >= (batched ? 70u : 80u)) {
+      return KernelChoice{CLBH_KERNEL_STREAM, 2, 1};
+    }
   }
   // Batches of fp32 / fp64 matrices of a few tiles with a short k are bound by HBM and latency, not by the matrix
   // cores: the kernel that keeps one slab per operand in LDS runs eight work-groups or more per CU (fp32 4096 x 64^3:
@@ -206,7 +212,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     // on 64 x 64 tiles and 90 us on 128 x 128 - but only where the latter fill the CUs; below that the 64 x 64 tiles win
     // with K split)
     const bool long_k = k >= 4096 && CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count >= 256;
-    const auto cost256 = (k >= 512) ? cost(256, 1, 100) : 1e300, cost128 = cost(128, 2, 85), cost64 = cost(64, 4, long_k ? 38 : 50);
+    const auto cost256 = (k >= 256) ? cost(256, 1, 100) : 1e300, cost128 = cost(128, 2, 85), cost64 = cost(64, 4, long_k ? 38 : 50);
     int tile = 1;
     if (cost256 <= cost128 && cost256 <= cost64) { tile = 2; }
     else if (cost128 <= cost64) { tile = 0; }
