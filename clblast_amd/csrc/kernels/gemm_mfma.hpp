@@ -569,20 +569,25 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
         return *reinterpret_cast<const VN*>(stage + LB::Row(ks * KP) + b_lane_row);
       };
 
-      // Prologue: slab 0 lands in buffer 0 (the staged registers' wait also covers the older direct loads),
-      // slab 1 is requested.
+      // Prologue: slab 0 lands in buffer 0 and slab 1 is requested - its direct loads before the wait for slab 0, so that
+      // the two memory latencies overlap (loads complete in order: when at most the direct loads of slab 1 are
+      // outstanding, everything of slab 0 has arrived); its staged pieces once slab 0 has left the staging registers.
       if constexpr (A_CONV == 1) { gather_rows = DecomposeRows<TILE_K>(p.conv, 0, k_len, lane); }
 #pragma unroll
       for (int load = 0; load < DIRECT; ++load) { direct_load(load, 0, a_stages, b_stages); }
 #pragma unroll
       for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, 0); }
-#pragma unroll
-      for (int piece = 0; piece < STAGED; ++piece) { store_piece(piece, a_stages, b_stages, 0, std::true_type{}); }
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       if (slabs > 1) {
         if constexpr (A_CONV == 1) { gather_rows = DecomposeRows<TILE_K>(p.conv, TILE_K, k_len, lane); }
 #pragma unroll
         for (int load = 0; load < DIRECT; ++load) { direct_load(load, TILE_K, a_stages + LA::ELEMS, b_stages + LB::ELEMS); }
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DIRECT) : "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+#pragma unroll
+      for (int piece = 0; piece < STAGED; ++piece) { store_piece(piece, a_stages, b_stages, 0, std::true_type{}); }
+      if (slabs > 1) {
 #pragma unroll
         for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, TILE_K); }
       }
