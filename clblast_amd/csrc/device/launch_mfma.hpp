@@ -109,7 +109,8 @@ int LaunchStreamVariant(const clbh_gemm_desc& d, hipStream_t stream) {
 
 template <typename T, typename Config>
 int LaunchStreamConfig(const clbh_gemm_desc& d, hipStream_t stream) {
-  if (d.c_triangle != 0 || d.operand_triangle != 0 || d.conv != nullptr || d.k <= 3 * Config::TILE_K || d.m < Config::FM || !LeadingDimsFitTiles<T>(d)) {
+  if (d.c_triangle != 0 || d.operand_triangle != 0 || d.conv != nullptr || d.k <= 3 * Config::TILE_K || d.m < Config::FM || !LeadingDimsFitTiles<T>(d) ||
+      d.c_ld >= CLBH_STREAM_MAX_LD) {
     return hipErrorInvalidValue;
   }
   const bool use_c = (d.batch.alphas != nullptr) || d.beta != 0.0;  // per-matrix betas: some may be non-zero

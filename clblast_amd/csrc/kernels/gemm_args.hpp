@@ -99,6 +99,15 @@ __device__ __forceinline__ void TriangularRange(const int operand_triangle, cons
   length = last - first;
 }
 
+// Read of a per-batch value through the constant address space: where the address is the same for the whole wavefront
+// (a batch index derived from the work-group index) this is a scalar load, which the counter of vector memory operations
+// does not see - a persistent kernel can look up its next batch while its own loads and stores stay in flight. The arrays
+// are complete before the kernel starts and no kernel writes them.
+template <typename V>
+__device__ __forceinline__ V UniformRead(const V* ptr) {
+  return *(const __attribute__((address_space(4))) V*)(ptr);
+}
+
 // Resolves the operand bases and scalars of batch `batch`.
 template <typename T, typename CT>
 __device__ __forceinline__ void ResolveBatch(const GemmArgs<CT>& p, const int batch, const T*& a, const T*& b, T*& c,
@@ -107,11 +116,11 @@ __device__ __forceinline__ void ResolveBatch(const GemmArgs<CT>& p, const int ba
   alpha = p.alpha;
   beta = p.beta;
   if (p.alphas != nullptr) {
-    a_off += p.a_offsets[batch];
-    b_off += p.b_offsets[batch];
-    c_off += p.c_offsets[batch];
-    alpha = p.alphas[batch];
-    beta = p.betas[batch];
+    a_off += UniformRead(p.a_offsets + batch);
+    b_off += UniformRead(p.b_offsets + batch);
+    c_off += UniformRead(p.c_offsets + batch);
+    alpha = UniformRead(p.alphas + batch);
+    beta = UniformRead(p.betas + batch);
   } else {
     a_off += p.a_stride * batch;
     b_off += p.b_stride * batch;

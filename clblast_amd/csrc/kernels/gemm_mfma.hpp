@@ -300,13 +300,27 @@ struct StagedPieces {
   static __device__ __forceinline__ int K(const int tid) { return (tid % ALONG) * VL; }
 };
 
+// `offset`: the lane's byte offset, the one the resource's range check looks at; `uniform_offset`: a byte offset common to
+// the wavefront, added behind that check (it travels in a scalar register: no vector arithmetic per access).
 template <typename T, int VL, typename Resource>
-__device__ __forceinline__ typename VecType<T, VL>::type BufferLoad(const Resource resource, const int offset) {
+__device__ __forceinline__ typename VecType<T, VL>::type BufferLoad(const Resource resource, const int offset,
+                                                                    const int uniform_offset = 0) {
   using V = typename VecType<T, VL>::type;
   constexpr int BYTES = VL * sizeof(T);
-  if constexpr (BYTES == 4) { return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b32(resource, offset, 0, 0)); }
-  else if constexpr (BYTES == 8) { return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b64(resource, offset, 0, 0)); }
-  else { static_assert(BYTES == 16, "piece size"); return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b128(resource, offset, 0, 0)); }
+  if constexpr (BYTES == 4) { return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b32(resource, offset, uniform_offset, 0)); }
+  else if constexpr (BYTES == 8) { return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b64(resource, offset, uniform_offset, 0)); }
+  else { static_assert(BYTES == 16, "piece size"); return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b128(resource, offset, uniform_offset, 0)); }
+}
+
+template <typename T, int VL, typename V, typename Resource>
+__device__ __forceinline__ void BufferStore(const V value, const Resource resource, const int offset, const int uniform_offset = 0) {
+  typedef unsigned Dwords2 __attribute__((ext_vector_type(2)));
+  typedef unsigned Dwords4 __attribute__((ext_vector_type(4)));
+  constexpr int BYTES = VL * sizeof(T);
+  static_assert(sizeof(V) == BYTES, "value type");
+  if constexpr (BYTES == 4) { __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, value), resource, offset, uniform_offset, 0); }
+  else if constexpr (BYTES == 8) { __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(Dwords2, value), resource, offset, uniform_offset, 0); }
+  else { static_assert(BYTES == 16, "piece size"); __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(Dwords4, value), resource, offset, uniform_offset, 0); }
 }
 
 // Piece c of this thread for the slab at `slab` (element (x0, k0), uniform).

@@ -20,6 +20,8 @@
 
 namespace clbh {
 
+constexpr int kStreamOutside = 0x7fffff00;  // byte count of the view of a tile's C, and the offset of a store that is to move nothing
+
 // USE_C: the old C is read (some beta is not zero). Needs at least four slabs per item (k > 3 * TILE_K) and tiles whose
 // accumulators are few enough for a second register set of the same size (the old C).
 template <typename T, typename Config, bool A_KC, bool B_KC, bool USE_C>
@@ -170,20 +172,39 @@ __global__ __launch_bounds__(kMfmaThreads, Config::MIN_WAVES) void GemmStreamKer
   using OldC = typename std::conditional<(FM > 1), VMG, T>::type;
   OldC old_c[USE_C ? OLD_C : 1];
 
-  // Position of the lane's accumulators in C: m = m_base + i (i < FM), column n = n_base + FN * Row(r) + j of block j
+  // Position of the lane's accumulators in C: m = m_base + i (i < FM); column n0 + lane_n + u of block j and accumulator
+  // element r, with u = FN * Row(r, 0) + j known at compile time. The C of an item is addressed through a range-checked
+  // view that starts at the item's first column: the lane's byte offset holds its own column and row - or lies outside
+  // the view for a piece that is not to move, which then touches no memory (a load delivers zero) - and the u columns
+  // travel as the access's uniform offset, so a piece costs a comparison and a select, not a 64-bit address.
   auto m_base = [&](const Item& item) { return item.m0 + a_read; };
-  auto n_of = [&](const Item& item, const int j, const int r) { return item.n0 + wave_n * (FN * MF) + FN * Traits::Row(r, lane_g) + j; };
-  // The old C of an item: one load per column piece, none of them under a branch (the waits below count them). A tile
-  // that reaches beyond the matrix reads some piece inside the matrix instead; its epilogue does not use these values.
+  const int c_ld = static_cast<int>(p.c_ld);  // (the host admits leading dimensions whose tile offsets fit 31 bits)
+  const int lane_n = wave_n * (FN * MF) + FN * Traits::Row(0, lane_g);
+  const int lane_columns = lane_n * c_ld;
+  auto c_view = [&](const Item& item) {
+    return __builtin_amdgcn_make_buffer_rsrc(item.c + static_cast<long long>(item.n0) * p.c_ld, 0, kStreamOutside, kRawBufferFlags);
+  };
+  auto columns_of = [](const int j, const int r) { return FN * Traits::Row(r, 0) + j; };
+  // the lane's offset for piece (j, r): `lane_offset` while the piece's column is one of the `columns_left` of the matrix
+  auto piece_offset = [&](const int lane_offset, const int columns, const int columns_left) {
+    int offset = (lane_n + columns < columns_left) ? lane_offset : kStreamOutside;
+    asm volatile("" : "+v"(offset));  // (a plain value: no branch around the access)
+    return offset;
+  };
+  // The old C of an item: one load per column piece, none of them under a branch (the waits below count them). A lane
+  // whose piece would reach beyond the last row reads the piece FM rows up from the last row instead (the epilogue
+  // picks its elements out of it).
   auto fetch_old_c = [&](const Item& item) {
     if constexpr (USE_C) {
-      const int m = max(min(m_base(item), p.m - FM), 0);
+      const auto view = c_view(item);
+      const int lane_offset = static_cast<int>((lane_columns + max(min(m_base(item), p.m - FM), 0)) * sizeof(T));
+      const int columns_left = p.n - item.n0;
 #pragma unroll
       for (int j = 0; j < FN; ++j) {
 #pragma unroll
         for (int r = 0; r < ACC; ++r) {
-          const int n = min(n_of(item, j, r), p.n - 1);
-          old_c[j * ACC + r] = *reinterpret_cast<const OldC*>(item.c + n * p.c_ld + m);
+          old_c[j * ACC + r] = __builtin_bit_cast(OldC, BufferLoad<T, FM>(view, piece_offset(lane_offset, columns_of(j, r), columns_left),
+                                                                        static_cast<int>(columns_of(j, r) * c_ld * sizeof(T))));
         }
       }
     }
@@ -254,75 +275,84 @@ __global__ __launch_bounds__(kMfmaThreads, Config::MIN_WAVES) void GemmStreamKer
   using NoFetch = std::false_type;
   using NoExtra = std::integral_constant<int, 0>;
   using OldCInFlight = std::integral_constant<int, USE_C ? OLD_C : 0>;
-  constexpr int INTERIOR_STORES = OLD_C;  // store instructions of the epilogue of a tile inside the matrix
+  constexpr int INTERIOR_STORES = OLD_C;  // store instructions of every epilogue (a tile cut by the last row issues more)
   using StoresInFlight = std::integral_constant<int, INTERIOR_STORES>;
 
-  bool counted_stores = false;  // the previous item's epilogue issued exactly INTERIOR_STORES stores per thread
+  // What the prologue requested has landed (a wait the compiler knows of, unlike the waits written as text: it counts
+  // the operations in flight to place its own waits for the staging registers, and where the start of the stream joins
+  // the loop it would otherwise have to assume the smallest count on either path).
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), the other counters at their maximum
   while (true) {
     // The slabs of the item (at least four). Every slab requests the slab two ahead: of the same item, then the first two
-    // of the next item. The old C is fetched under the third slab from the end, two slabs before the epilogue needs it.
-    if (counted_stores) { slab_body(TILE_K, current, 2 * TILE_K, NoFetch{}, StoresInFlight{}); }
-    else { slab_body(TILE_K, current, 2 * TILE_K, NoFetch{}, NoExtra{}); }
+    // of the next item. The old C is fetched under the third slab from the end. The first slab's wait lets the stores of
+    // the previous item's epilogue fly on (the first item has none, and nothing its wait is about is outstanding either).
+    slab_body(TILE_K, current, 2 * TILE_K, NoFetch{}, StoresInFlight{});
     for (int s = 1; s + 3 < slabs; ++s) { slab_body((s + 1) * TILE_K, current, (s + 2) * TILE_K, NoFetch{}, NoExtra{}); }
     slab_body((slabs - 2) * TILE_K, current, (slabs - 1) * TILE_K, Fetch{}, NoExtra{});
     slab_body((slabs - 1) * TILE_K, next, 0, NoFetch{}, OldCInFlight{});
     slab_body(0, next, TILE_K, NoFetch{}, NoExtra{});
 
-    // Epilogue of the item; its stores drain under the products of the next item.
+    // Epilogue of the item; its stores drain under the products of the next item. Every tile issues the same store
+    // instructions, none of them under a branch, through a range-checked view of the tile's part of C: a lane whose piece
+    // is not wholly inside the matrix stores at an offset outside that view, which moves nothing. So the number of stores
+    // in flight behind an epilogue is fixed (INTERIOR_STORES, more for the rare tile below), and the waits of the next
+    // item's first slab - the one written here and the ones the compiler places for the staging registers - can let
+    // them fly on. (Stores under bounds tests would come in a number nobody knows: where such a path joins the loop, the
+    // compiler's waits have to assume that no store was issued and drain the memory pipe at every item.)
     {
       const int mb = m_base(current);
-      const bool interior = current.m0 + TILE_M <= p.m && current.n0 + TILE_N <= p.n;
-      if (interior) {  // exactly one store per column piece: the next item's first wait counts them
+      const auto view = c_view(current);
+      const int columns_left = p.n - current.n0;
+      const int row_offset = static_cast<int>((lane_columns + mb) * sizeof(T));
+      const int whole_offset = (mb + FM <= p.m) ? row_offset : kStreamOutside;
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+#pragma unroll
+        for (int r = 0; r < ACC; ++r) {
+          OldC out;
+#pragma unroll
+          for (int i = 0; i < FM; ++i) {
+            T value = current.alpha * acc[i][j][r];
+            if constexpr (USE_C) {
+              if (current.beta != T(0)) {
+                value = Combine(current.alpha, acc[i][j][r], current.beta, VecGet<OldC, T, FM>(old_c[j * ACC + r], i));
+              }
+            }
+            out = VecWith<OldC, T, FM>(out, i, value);
+          }
+          BufferStore<T, FM>(out, view, piece_offset(whole_offset, columns_of(j, r), columns_left),
+                             static_cast<int>(columns_of(j, r) * c_ld * sizeof(T)));
+        }
+      }
+      if (FM > 1 && current.m0 + TILE_M > p.m) {
+        // A tile that the last row of the matrix cuts: a piece that straddles the edge stores its elements one by one.
+        // Its old C has come with the others - fetch_old_c moved the lane's piece back into the matrix, so the lane's
+        // element i is element i + shift of the piece it holds, whenever that element exists.
+        const int shift = mb - max(min(mb, p.m - FM), 0);
+        const int straddling_offset = (mb < p.m && mb + FM > p.m) ? row_offset : kStreamOutside;
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
 #pragma unroll
           for (int r = 0; r < ACC; ++r) {
-            T* dst = current.c + n_of(current, j, r) * p.c_ld + mb;
-            OldC out;
+            const int offset = piece_offset(straddling_offset, columns_of(j, r), columns_left);
 #pragma unroll
-            for (int i = 0; i < FM; ++i) {
+            for (int i = 0; i < FM - 1; ++i) {  // (the last element of a straddling piece is never inside)
               T value = current.alpha * acc[i][j][r];
               if constexpr (USE_C) {
                 if (current.beta != T(0)) {
-                  value = Combine(current.alpha, acc[i][j][r], current.beta, VecGet<OldC, T, FM>(old_c[j * ACC + r], i));
+                  T old = VecGet<OldC, T, FM>(old_c[j * ACC + r], FM - 1);
+#pragma unroll
+                  for (int e = 0; e < FM - 1; ++e) { if (i + shift == e) { old = VecGet<OldC, T, FM>(old_c[j * ACC + r], e); } }
+                  value = Combine(current.alpha, acc[i][j][r], current.beta, old);
                 }
               }
-              out = VecWith<OldC, T, FM>(out, i, value);
-            }
-            *reinterpret_cast<OldC*>(dst) = out;
-          }
-        }
-      } else {
-        // A tile on an edge of the matrix: element-wise stores under bounds tests (their number is not counted: the next
-        // item's first wait lets them all retire). Its old C has come with the others - fetch_old_c moved a lane's piece
-        // back into the matrix where it would have reached beyond m or n, so the lane's element i is element i + shift of
-        // the piece it holds, whenever that element exists.
-        const int shift = mb - max(min(mb, p.m - FM), 0);
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-#pragma unroll
-          for (int r = 0; r < ACC; ++r) {
-            const int n = n_of(current, j, r);
-            T* dst = current.c + n * p.c_ld + mb;
-#pragma unroll
-            for (int i = 0; i < FM; ++i) {
-              if (n < p.n && mb + i < p.m) {
-                T value = current.alpha * acc[i][j][r];
-                if constexpr (USE_C) {
-                  if (current.beta != T(0)) {
-                    T old = VecGet<OldC, T, FM>(old_c[j * ACC + r], FM - 1);
-#pragma unroll
-                    for (int e = 0; e < FM - 1; ++e) { if (i + shift == e) { old = VecGet<OldC, T, FM>(old_c[j * ACC + r], e); } }
-                    value = Combine(current.alpha, acc[i][j][r], current.beta, old);
-                  }
-                }
-                dst[i] = value;
-              }
+              int element = (mb + i < p.m) ? offset + i * static_cast<int>(sizeof(T)) : kStreamOutside;
+              asm volatile("" : "+v"(element));
+              BufferStore<T, 1>(value, view, element, static_cast<int>(columns_of(j, r) * c_ld * sizeof(T)));
             }
           }
         }
       }
-      counted_stores = interior;
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
 #pragma unroll

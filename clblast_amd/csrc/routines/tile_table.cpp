@@ -131,7 +131,8 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   // tiles; with beta = 0: 219 -> 159 us; 8192^2 x 256: 367 -> 323 us; no gain is left from k = 512 on - else tiles of
   // 64 x 64 (4096 x 4096 x 128: 63 -> 55 us, 512 x 256 x 256 x 64: 106 -> 79 us; fp64 512 x 256 x 256 x 64: 209 -> 150 us,
   // 64 x 512 x 512 x 128: 107 -> 92 us).
-  if (forced == 0 && !triangular && precision != Precision::kHalf && k > 48) {
+  if (forced == 0 && !triangular && precision != Precision::kHalf && k > 48 &&
+      largest_ld < static_cast<size_t>(CLBH_STREAM_MAX_LD)) {
     const auto tiles128 = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
     if (precision == Precision::kSingle && tiles128 >= 1024 && TileUse(m, n, 128, 128) >= 90 &&
         k <= (beta_zero ? 512u : 256u)) {
@@ -158,7 +159,8 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   if ((forced == 101 || forced == 102) && !triangular && precision != Precision::kHalf) {
     return KernelChoice{CLBH_KERNEL_SMALL_TILED, static_cast<int>(forced) - 101, 1};  // one-slab kernel, 64 x 64 / 32 x 32 tiles
   }
-  if ((forced == 103 || forced == 104) && !triangular && precision != Precision::kHalf && k > 48) {
+  if ((forced == 103 || forced == 104) && !triangular && precision != Precision::kHalf && k > 48 &&
+      largest_ld < static_cast<size_t>(CLBH_STREAM_MAX_LD)) {
     // persistent work-groups over tiles of 64 x 64, or (fp32) 128 x 128
     return KernelChoice{CLBH_KERNEL_STREAM, (forced == 104 && precision == Precision::kSingle) ? 1 : 2, 1};
   }

@@ -33,7 +33,7 @@ bool UseDirectKernel(const size_t m, const size_t n, const size_t k, const size_
 
 // Picks the kernel family and tile for a canonical problem (m, n, k per matrix). `triangular`: about half of the
 // tile work of the launch is skipped (a triangle of C, or a triangular operand), which calls for smaller tiles.
-// `beta_zero`: the old C is not read. `largest_ld`: the larger leading dimension of A and B. (Neither of the two ever
+// `beta_zero`: the old C is not read. `largest_ld`: the largest leading dimension of A, B and C. (Neither of the two ever
 // makes a problem need more workspace than it needs with the default values.)
 KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const bool b_kcontig, const size_t m,
                           const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,

@@ -133,7 +133,7 @@ void Xgemm<T>::DoGemm(const Layout layout, const Transpose a_transpose, const Tr
   const bool triangular = (triangles.output != OutputTriangle::kFull || triangles.operand != OperandTriangle::kNone);
   const auto choice = SelectKernel(PrecisionValue<T>(), desc.a_kcontig != 0, desc.b_kcontig != 0,
                                    static_cast<size_t>(desc.m), static_cast<size_t>(desc.n), k, 1, false,
-                                   min_indirect_size(), triangular, ScalarToDouble(beta) == 0.0, std::max(a_ld, b_ld));
+                                   min_indirect_size(), triangular, ScalarToDouble(beta) == 0.0, std::max({a_ld, b_ld, c_ld}));
   desc.kernel_class = choice.kernel_class;
   desc.tile_variant = choice.tile_variant;
   desc.split_k = choice.split_k;

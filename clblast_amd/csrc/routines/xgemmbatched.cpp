@@ -47,7 +47,7 @@ void XgemmBatched<T>::DoGemmBatched(const Layout layout, const Transpose a_trans
                                      const_cast<void*>(c_buffer()), 0, c_ld);
   const auto choice = SelectKernel(PrecisionValue<T>(), desc.a_kcontig != 0, desc.b_kcontig != 0,
                                    static_cast<size_t>(desc.m), static_cast<size_t>(desc.n), k, batch_count, true,
-                                   min_indirect_size());
+                                   min_indirect_size(), false, false, std::max({a_ld, b_ld, c_ld}));
   desc.kernel_class = choice.kernel_class;
   desc.tile_variant = choice.tile_variant;
   desc.split_k = choice.split_k;
@@ -201,7 +201,7 @@ void XgemmStridedBatched<T>::DoGemmStridedBatched(
   desc.beta = ScalarToDouble(beta);
   const auto choice = SelectKernel(PrecisionValue<T>(), desc.a_kcontig != 0, desc.b_kcontig != 0,
                                    static_cast<size_t>(desc.m), static_cast<size_t>(desc.n), k, batch_count, false,
-                                   min_indirect_size(), false, desc.beta == 0.0);
+                                   min_indirect_size(), false, desc.beta == 0.0, std::max({a_ld, b_ld, c_ld}));
   desc.kernel_class = choice.kernel_class;
   desc.tile_variant = choice.tile_variant;
   desc.split_k = choice.split_k;

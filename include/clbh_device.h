@@ -40,10 +40,12 @@ enum clbh_kernel_class {
   CLBH_KERNEL_SMALL_TILED = 4,    // fp32 / fp64 batches of matrices of a few tiles: one slab per operand in LDS, many
                                   // work-groups per CU (tile_variant 1: tiles of 32 x 32, else 64 x 64)
   CLBH_KERNEL_STREAM = 5          // fp32 / fp64 launches of many 64 x 64 tiles with a short K walk (k > 48): persistent
-                                  // work-groups that overlap an item's C traffic with the products of its neighbours
+                                  // work-groups that overlap an item's C traffic with the products of its neighbours;
+                                  // the leading dimension of C below CLBH_STREAM_MAX_LD
 };
 
 #define CLBH_SKINNY_MAX_LD (1ll << 21)
+#define CLBH_STREAM_MAX_LD (1ll << 20)  // (a tile's offsets into C stay below 2^31 bytes)
 
 // Per-batch metadata of GemmBatched, all device pointers (NULL for plain and strided launches).
 typedef struct clbh_batch_arrays_ {

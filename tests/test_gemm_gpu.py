@@ -230,35 +230,41 @@ def test_long_k_with_few_tiles(gpu, bits):
 
 @pytest.mark.parametrize("bits", (32, 64))
 def test_persistent_kernel_for_many_tiles_with_a_short_k(gpu, bits):
-    """The kernel whose work-groups stay resident and walk many 64 x 64 tiles (normally picked for launches of thousands
-    of tiles with a short k), forced on shapes with fewer and with more tiles than resident work-groups, ragged edges, a K
-    tail, four slabs only, beta zero and non-zero, all four operand orientations; then on strided batches."""
+    """The kernel whose work-groups stay resident and walk many 64 x 64 tiles, or in fp32 128 x 128 tiles (normally picked
+    for launches of thousands of tiles with a short k), forced on shapes with fewer and with more tiles than resident
+    work-groups, ragged edges (odd extents too: a lane's pair of rows then straddles the last row), a K tail, four slabs
+    only, beta zero and non-zero, all four operand orientations; then on strided batches. A store that reached beyond the
+    matrix would show in the padding of C, which the check compares too."""
     import clblast_amd
     import torch
     from tests.test_batched_gpu import run_strided
     try:
-        clblast_amd.override_parameters(0, "Xgemm", bits, {"TILE_VARIANT": 103})
         seed = 7600
-        for (ta, tb) in itertools.product(TRANSPOSES, TRANSPOSES):
-            for (m, n, k), extra, offsets in (((520, 264, 200), (8, 8, 8), (8, 16, 24)),
-                                              ((300, 270, 100), (3, 5, 7), (11, 13, 19)),
-                                              ((64, 64, 49), (0, 0, 0), (0, 0, 0)),
-                                              ((130, 1000, 65), (1, 0, 2), (5, 0, 3)),
-                                              ((2100, 2600, 50), (3, 5, 7), (11, 13, 19))):
-                for beta in (2.0, 0.0):
-                    seed += 1
-                    problem = gpu.Problem(bits, (COL_MAJOR, ROW_MAJOR)[seed % 2], ta, tb, m, n, k, -0.75, beta,
-                                          a_offset=offsets[0], b_offset=offsets[1], c_offset=offsets[2], seed=seed, extra_ld=extra)
-                    if beta == 0.0:
-                        problem.c[:] = np.nan  # beta == 0 never reads C
-                    status, c_after = problem.run()
-                    assert status == 0, problem.describe()
-                    if beta == 0.0:
-                        index = oracle.c_indices(problem.layout, m, n, problem.c_offset, problem.c_ld)
-                        problem.c[index.ravel()] = 0.0
-                    problem.check(c_after)
-            run_strided(gpu, bits, COL_MAJOR, ta, tb, 100, 70, 60, 0.5, 1.5, 300, None, None, (1, 2, 3), (1, 0, 2), seed)
-            run_strided(gpu, bits, ROW_MAJOR, ta, tb, 64, 128, 64, 0.5, 0.0, 150, 0, None, (0, 0, 0), (0, 0, 0), seed + 1)
+        for variant in ((103, 104) if bits == 32 else (103,)):  # 64 x 64 tiles; fp32 also 128 x 128
+            clblast_amd.override_parameters(0, "Xgemm", bits, {"TILE_VARIANT": variant})
+            for (ta, tb) in itertools.product(TRANSPOSES, TRANSPOSES):
+                for (m, n, k), extra, offsets in (((520, 264, 200), (8, 8, 8), (8, 16, 24)),
+                                                  ((300, 270, 100), (3, 5, 7), (11, 13, 19)),
+                                                  ((64, 64, 49), (0, 0, 0), (0, 0, 0)),
+                                                  ((130, 1000, 65), (1, 0, 2), (5, 0, 3)),
+                                                  ((301, 271, 100), (3, 5, 7), (11, 13, 19)),  # odd: a lane's pair of rows straddles the edge
+                                                  ((1027, 643, 77), (0, 0, 0), (1, 2, 3)),
+                                                  ((2100, 2600, 50), (3, 5, 7), (11, 13, 19))):
+                    for beta in (2.0, 0.0):
+                        seed += 1
+                        problem = gpu.Problem(bits, (COL_MAJOR, ROW_MAJOR)[seed % 2], ta, tb, m, n, k, -0.75, beta,
+                                              a_offset=offsets[0], b_offset=offsets[1], c_offset=offsets[2], seed=seed, extra_ld=extra)
+                        if beta == 0.0:
+                            problem.c[:] = np.nan  # beta == 0 never reads C
+                        status, c_after = problem.run()
+                        assert status == 0, problem.describe()
+                        if beta == 0.0:
+                            index = oracle.c_indices(problem.layout, m, n, problem.c_offset, problem.c_ld)
+                            problem.c[index.ravel()] = 0.0
+                        problem.check(c_after)
+                run_strided(gpu, bits, COL_MAJOR, ta, tb, 100, 70, 60, 0.5, 1.5, 300, None, None, (1, 2, 3), (1, 0, 2), seed)
+                run_strided(gpu, bits, COL_MAJOR, ta, tb, 131, 67, 60, 0.5, 1.5, 150, None, None, (0, 0, 0), (1, 0, 2), seed + 2)
+                run_strided(gpu, bits, ROW_MAJOR, ta, tb, 64, 128, 64, 0.5, 0.0, 150, 0, None, (0, 0, 0), (0, 0, 0), seed + 1)
         torch.cuda.synchronize()
     finally:
         clblast_amd.override_parameters(0, "Xgemm", bits, {"TILE_VARIANT": 0})
