@@ -128,22 +128,27 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   // overlap one tile's C traffic with the products of the next beat one work-group per tile. fp32 tiles of 128 x 128 (a
   // quarter of the operand traffic per flop of 64 x 64) where they fill the matrix - 8191 x 8191 x 127 with beta = 2:
   // 271 us with one work-group per 64 x 64 tile, 230 us with resident work-groups on 64 x 64 tiles, 201 us on 128 x 128
-  // tiles; with beta = 0: 219 -> 159 us; 8192^2 x 256: 367 -> 323 us; no gain is left from k = 512 on - else tiles of
-  // 64 x 64 (4096 x 4096 x 128: 63 -> 55 us, 512 x 256 x 256 x 64: 106 -> 79 us; fp64 512 x 256 x 256 x 64: 209 -> 150 us,
-  // 64 x 512 x 512 x 128: 107 -> 92 us).
+  // tiles; 8192^2 x 384: 477 -> 407 us, x 768: 837 -> 747 us, 4096^2 x 640: 180 -> 161 us, 16384 x 4096 x 640: 722 -> 637 us;
+  // at k = 1024 the gain is down to 2 % and stays there - else tiles of 64 x 64 (4096 x 4096 x 128: 63 -> 55 us,
+  // 100352 x 128 x 200: 60 -> 50 us, 30000 x 256 x 400: 66 -> 57 us, 6000 x 1000 x 300: 41 -> 36 us, at k = 800 nothing is
+  // left; 512 x 256 x 256 x 64: 106 -> 79 us; fp64 8192^2 x 256: 605 -> 543 us, 100352 x 128 x 300: 155 -> 135 us,
+  // x 576: 253 -> 237 us, 512 x 256 x 256 x 64: 209 -> 150 us, 64 x 512 x 512 x 128: 107 -> 92 us).
   if (forced == 0 && !triangular && precision != Precision::kHalf && k > 48 &&
       largest_ld < static_cast<size_t>(CLBH_STREAM_MAX_LD)) {
     const auto tiles128 = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
+    // (two k-contiguous operands go through the staging registers: 4096^2 x 1000 is 6 % behind the 256 x 128 tiles then)
     if (precision == Precision::kSingle && tiles128 >= 1024 && TileUse(m, n, 128, 128) >= 90 &&
-        k <= (beta_zero ? 512u : 256u)) {
+        k <= ((a_kcontig && b_kcontig) ? 640u : 1024u)) {
       return KernelChoice{CLBH_KERNEL_STREAM, 1, 1};
     }
     const auto tiles64 = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;
     // (batches: from 2048 tiles on, and fp64 up to k = 400 - fp64 256 x 256^3 164 -> 153 us, 256 x 200 x 300 x 400
     // 296 -> 275 us, 128 x 384^3 266 -> 245 us; at k = 512 the tiled kernel is ahead again)
     const bool batched = batch_count > 1;
-    if (k <= ((batched && precision == Precision::kDouble) ? 400u : 192u) && tiles64 >= (batched ? 2048u : 4096u) &&
-        TileUse(m, n, 64, 64) >= (batched ? 70u : 80u)) {
+    const bool fp64 = (precision == Precision::kDouble);
+    const size_t k_limit = batched ? (fp64 ? 400 : 192) : (fp64 ? 640 : 448);
+    const size_t tiles_floor = batched ? 2048 : (fp64 ? 2048 : 1500);
+    if (k <= k_limit && tiles64 >= tiles_floor && TileUse(m, n, 64, 64) >= (batched ? 70u : 80u)) {
       return KernelChoice{CLBH_KERNEL_STREAM, 2, 1};
     }
   }
