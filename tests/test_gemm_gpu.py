@@ -249,6 +249,7 @@ def test_persistent_kernel_for_many_tiles_with_a_short_k(gpu, bits):
                                                   ((130, 1000, 65), (1, 0, 2), (5, 0, 3)),
                                                   ((301, 271, 100), (3, 5, 7), (11, 13, 19)),  # odd: a lane's pair of rows straddles the edge
                                                   ((1027, 643, 77), (0, 0, 0), (1, 2, 3)),
+                                                  ((261, 390, 1000), (5, 3, 1), (0, 7, 2)),  # a long walk: 63 slabs per item
                                                   ((2100, 2600, 50), (3, 5, 7), (11, 13, 19))):
                     for beta in (2.0, 0.0):
                         seed += 1
