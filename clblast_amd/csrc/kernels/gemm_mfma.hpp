@@ -320,7 +320,18 @@ __device__ __forceinline__ void BufferStore(const V value, const Resource resour
   static_assert(sizeof(V) == BYTES, "value type");
   if constexpr (BYTES == 4) { __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, value), resource, offset, uniform_offset, 0); }
   else if constexpr (BYTES == 8) { __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(Dwords2, value), resource, offset, uniform_offset, 0); }
-  else { static_assert(BYTES == 16, "piece size"); __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(Dwords4, value), resource, offset, uniform_offset, 0); }
+  else {
+    static_assert(BYTES == 16, "piece size");
+    const Dwords4 data = __builtin_bit_cast(Dwords4, value);
+    __builtin_amdgcn_raw_buffer_store_b128(data, resource, offset, uniform_offset, 0);
+    // A store of more than 64 bits reads its data registers over several cycles, and a vector instruction that
+    // overwrites them right behind it can get there first: with the uniform offset in a scalar register the compiler
+    // places no wait state between the two (it does for the other forms of the instruction), and on gfx950 the lanes
+    // 12..15 of every row of 16 then stored the new contents of the upper two registers now and then (fp64 results of
+    // the persistent kernel, one piece in fifty tiles). The wait states below read the data registers, so whatever
+    // overwrites them comes behind.
+    asm volatile("s_nop 1" ::"v"(data) : "memory");
+  }
 }
 
 // Piece c of this thread for the slab at `slab` (element (x0, k0), uniform).

@@ -250,7 +250,8 @@ def test_persistent_kernel_for_many_tiles_with_a_short_k(gpu, bits):
                                                   ((301, 271, 100), (3, 5, 7), (11, 13, 19)),  # odd: a lane's pair of rows straddles the edge
                                                   ((1027, 643, 77), (0, 0, 0), (1, 2, 3)),
                                                   ((261, 390, 1000), (5, 3, 1), (0, 7, 2)),  # a long walk: 63 slabs per item
-                                                  ((2100, 2600, 50), (3, 5, 7), (11, 13, 19))):
+                                                  ((2100, 2600, 50), (3, 5, 7), (11, 13, 19)),
+                                                  ((3000, 2900, 60), (1, 2, 3), (3, 2, 1))):  # more 128 x 128 tiles than resident work-groups
                     for beta in (2.0, 0.0):
                         seed += 1
                         problem = gpu.Problem(bits, (COL_MAJOR, ROW_MAJOR)[seed % 2], ta, tb, m, n, k, -0.75, beta,
