@@ -59,10 +59,11 @@ int LaunchStreamF32(const clbh_gemm_desc& d, hipStream_t stream) {
   // address unit of the vector memory path was full for 10 % of the cycles; 8192^2 x 128: 187 -> 177 us, from k = 384
   // on 0-2 % - the wavefronts read a quarter more from LDS this way, which fp32 has to spare).
   if (d.tile_variant == 1) { return LaunchStreamConfig<float, MfmaConfig<float, 1, 4, 4, 1, 16, 2>>(d, stream); }
-  // tiles of 64 x 64 x 16 on the 16x16x4 instruction: a lane owns two consecutive m of 2 x 2 blocks and moves C in 8-byte
-  // pieces, 8 loads and 8 stores per item (on the 32x32x2 instruction: 16 of 4 bytes; 100352 x 128 x 200: 52.9 -> 50.9 us,
-  // 8191 x 8191 x 127 on these tiles: 194 -> 186 us, 4096 x 64^3: 35.2 -> 34.4 us)
-  return LaunchStreamConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16, 4, MfmaTraitsF32Small>>(d, stream);
+  // tiles of 64 x 64 x 16 on the 16x16x4 instruction, the wavefronts side by side along n (64 x 16 each): a lane owns
+  // four consecutive m and moves C in 16-byte pieces, 4 loads and 4 stores per item (on the 32x32x2 instruction with
+  // 2 x 2 wavefronts: 16 of 4 bytes; 100352 x 128 x 200: 52.9 -> 49.7 us, 8191 x 8191 x 127 on these tiles: 194 -> 182 us,
+  // 4096 x 64^3: 35.2 -> 33.5 us)
+  return LaunchStreamConfig<float, MfmaConfig<float, 1, 4, 4, 1, 16, 4, MfmaTraitsF32Small>>(d, stream);
 }
 
 int LaunchGeneralF32(const clbh_gemm_desc& d, hipStream_t stream) { return LaunchGeneral<float>(d, stream); }
