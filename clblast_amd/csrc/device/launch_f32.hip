@@ -47,6 +47,9 @@ int LaunchMfmaF32(const clbh_gemm_desc& d, hipStream_t stream) {
     case 9: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 1, 32, 4, MfmaTraitsF32Small>>(d, stream);  // 64 x 32 x 32
     case 10: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 1, 1, 64, 4, MfmaTraitsF32Small>>(d, stream);  // 32 x 32 x 64
     case 11: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 4, 2, 32, 2, MfmaTraitsF32Small>>(d, stream);  // 128 x 64 x 32
+    // 64 x 64 x 16 as four wavefronts of 64 x 16 on the 16x16x4 instruction: a lane owns four consecutive m, C moves in
+    // 16-byte pieces (index 7 moves it in 4-byte pieces: 3000^3 433 -> 415 us, 3072^3 N/N 490 -> 444 us)
+    case 12: return LaunchMfmaConfig<float, MfmaConfig<float, 1, 4, 4, 1, 16, 4, MfmaTraitsF32Small>>(d, stream);
     default: return LaunchMfmaConfig<float, MfmaConfig<float, 2, 2, 2, 2, 16, 2>>(d, stream);  // 128 x 128 x 16
   }
 }

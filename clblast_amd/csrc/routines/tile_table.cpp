@@ -249,7 +249,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
         largest_ld < static_cast<size_t>(CLBH_SKINNY_MAX_LD)) {
       return KernelChoice{CLBH_KERNEL_SKINNY, 0, 1};
     }
-    auto tile = Tile{7, 64, 64};
+    auto tile = Tile{12, 64, 64};  // (the 64 x 64 tile that moves C in 16-byte pieces; index 7 is the one on 32x32x2)
     const auto tiles64 = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;
     if (n <= 32 && m >= 256) { tile = Tile{9, 64, 32}; }         // skinny: stream A
     else if (m <= 32 && n >= 256) { tile = Tile{8, 32, 64}; }    // skinny: stream B
@@ -274,7 +274,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     else if (tiles64 < 1024 && (batch_count == 1 || n > 64)) { tile = Tile{9, 64, 32}; }  // (batches of matrices one tile
                                                                                          // wide keep 64 x 64: 87 -> 62 us)
     const auto tiles = CeilDivide(m, tile.tile_m) * CeilDivide(n, tile.tile_n) * batch_count;
-    const auto split = (batch_count == 1) ? SplitFor(tiles, k, tile.index >= 8) : 1;
+    const auto split = (batch_count == 1) ? SplitFor(tiles, k, tile.index >= 8 && tile.index != 12) : 1;
     return KernelChoice{CLBH_KERNEL_MFMA, tile.index, split};
   }
   // fp64 (same sweep): 64 x 64 x 16 tiles (index 1) up to about 3072^3, 128 x 128 x 8 (index 0) beyond; for launches
