@@ -7,8 +7,10 @@ namespace clbh {
 namespace {
 
 // CONVGEMM with the A operand gathered from the images (clbh_gemm_desc::conv): the kernel matrix is k-contiguous,
-// the batches are strided, K is not split; tiles of 64 x 64 x 16 (measured against 128 x 128 x 16 and depths of 32: the
-// gather's address arithmetic, not the tile shape, decides the speed)
+// the batches are strided, K is not split; tiles of 64 x 64 x 16 (measured against 128 x 128 x 16 and depths of 32: no
+// better; neither is a table of the rows' image offsets in LDS in place of the gather's address arithmetic), four
+// wavefronts of 64 x 16 on the 16x16x4 instruction so that C leaves in 16-byte pieces (8 x 64 x 112 x 112 images, 128
+// kernels of 3 x 3: 167 -> 159 us against 2 x 2 wavefronts on 32x32x2 with 4-byte pieces)
 int LaunchConvF32(const clbh_gemm_desc& d, hipStream_t stream) {
   const auto& g = *d.conv;
   const long long patches = static_cast<long long>(g.output_h) * g.output_w;
@@ -25,9 +27,9 @@ int LaunchConvF32(const clbh_gemm_desc& d, hipStream_t stream) {
   const bool window_fits = static_cast<long long>(g.dilation_h) * (g.kernel_h - 1) + 1 <= g.height &&
                            static_cast<long long>(g.dilation_w) * (g.kernel_w - 1) + 1 <= g.width;
   if (g.pad_h == 0 && g.pad_w == 0 && g.stride_w == 1 && g.output_w % 4 == 0 && window_fits) {
-    return LaunchMfmaVariant<float, MfmaConfig<float, 2, 2, 1, 1, 16, 4>, false, true, true, 2>(d, stream);
+    return LaunchMfmaVariant<float, MfmaConfig<float, 1, 4, 4, 1, 16, 4, MfmaTraitsF32Small>, false, true, true, 2>(d, stream);
   }
-  return LaunchMfmaVariant<float, MfmaConfig<float, 2, 2, 1, 1, 16, 4>, false, true, true, 1>(d, stream);
+  return LaunchMfmaVariant<float, MfmaConfig<float, 1, 4, 4, 1, 16, 4, MfmaTraitsF32Small>, false, true, true, 1>(d, stream);
 }
 
 }  // namespace
