@@ -271,8 +271,13 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       tile = Tile{11, 128, 64};  // whole rounds of two work-groups per CU (2048^3: 140 -> 131 us, 4096 x 3072 x 2048: 396 -> 385)
     }
     else if (tiles64 <= 64 && k < 2048) { tile = Tile{10, 32, 32}; }
-    else if (tiles64 < 1024 && (batch_count == 1 || n > 64)) { tile = Tile{9, 64, 32}; }  // (batches of matrices one tile
-                                                                                         // wide keep 64 x 64: 87 -> 62 us)
+    else if (tiles64 < 1024 && (batch_count == 1 || n > 64) &&
+             !(a_kcontig && b_kcontig && tiles64 >= 512 && k >= 1024 && batch_count == 1)) {
+      // (batches of matrices one tile wide keep 64 x 64: 87 -> 62 us; so do two k-contiguous operands from two tiles per
+      // CU on, where the narrow tile's staging costs more than it gains: 2048 x 1024 x 4096 T/N 163 -> 149 us, x 8192
+      // 321 -> 287 us; with 384 tiles the 64 x 32 tile is still 14 % ahead)
+      tile = Tile{9, 64, 32};
+    }
     const auto tiles = CeilDivide(m, tile.tile_m) * CeilDivide(n, tile.tile_n) * batch_count;
     const auto split = (batch_count == 1) ? SplitFor(tiles, k, tile.index >= 8 && tile.index != 12) : 1;
     return KernelChoice{CLBH_KERNEL_MFMA, tile.index, split};
