@@ -96,7 +96,9 @@ bool FillsRounds(const size_t tiles) {
 // GPU would be otherwise (measured: 128^2 x 1024 13.2 -> 9.2 us with four ranges, 768^2 x 4096 79.5 -> 54.4 us).
 int SplitFor(const size_t tiles, const size_t k, const bool small_tile = false) {
   if (small_tile) {
-    const size_t min_range = (tiles <= 64) ? 256 : (tiles <= 128) ? 512 : 1024;
+    // (129 to 192 work-groups with 2048 <= k < 4096: ranges of 512 too - 8200 x 9 x 2048 27.9 -> 22.9 us,
+    // 3000 x 128 x 2048 T/N 30.0 -> 24.8 us, 640 x 600 x 2048 27.1 -> 22.8 us; from k = 4096 on ranges of 1024 do as well)
+    const size_t min_range = (tiles <= 64) ? 256 : (tiles <= 128 || (tiles <= 192 && k >= 2048 && k < 4096)) ? 512 : 1024;
     if (tiles >= 384 || k < 2 * min_range) { return 1; }
     return static_cast<int>(std::max<size_t>(1, std::min<size_t>({CeilDivide(1024, tiles), k / min_range, 16})));
   }
