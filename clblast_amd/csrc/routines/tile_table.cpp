@@ -4,6 +4,7 @@
 #include "routines/tile_table.hpp"
 
 #include <algorithm>
+#include <cmath>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -279,6 +280,32 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       // CU on, where the narrow tile's staging costs more than it gains: 2048 x 1024 x 4096 T/N 163 -> 149 us, x 8192
       // 321 -> 287 us; with 384 tiles the 64 x 32 tile is still 14 % ahead)
       tile = Tile{9, 64, 32};
+    }
+    // Large single products with a long k: the four tiles that matter there by a cost estimate. A tile's work-groups
+    // run in rounds (256 x 128: one per CU, 128 x 128 and 128 x 64: two, 64 x 64: four); a whole round costs the tile area
+    // over the rate that tile's kernel sustains (145, 142, 134 and 136 TFLOP/s; 64 x 64 with two k-contiguous operands,
+    // which pass through staging registers: 128), and in the last round a CU with c of its p work-groups runs at
+    // (c / p)^0.4 of that rate. The small tiles lose 6 % of the rate and waste far less on a last round that stays partly
+    // empty. Rates and exponent are fitted to 77 measured shapes (mean loss against the best of the four tiles 0.4 %,
+    // worst 7 %): 5120^3 2167 us on 128 x 128 (the choice of the rules above), 1976 us on 64 x 64; 6000 x 3000 x 4000
+    // 1235 -> 1103 us on 128 x 64; 3029 x 6403 x 2752 T/N 987 -> 860 us on 64 x 64; 4096^3 and 8192^3 keep 256 x 128, 7000^3
+    // keeps 128 x 128.
+    if (batch_count == 1 && k >= 1024 && tiles64 >= 1024) {
+      struct Candidate { Tile tile; size_t per_cu; double rate; };
+      const Candidate candidates[] = {{Tile{3, 256, 128}, 1, 145.0}, {Tile{0, 128, 128}, 2, 142.0}, {Tile{11, 128, 64}, 2, 134.0},
+                                      {Tile{12, 64, 64}, 4, (a_kcontig && b_kcontig) ? 128.0 : 136.0}};
+      auto lowest = 1e300;
+      for (const auto& candidate : candidates) {
+        const auto count = CeilDivide(m, candidate.tile.tile_m) * CeilDivide(n, candidate.tile.tile_n);
+        const auto slots = 256 * candidate.per_cu;
+        auto rounds = static_cast<double>((count / slots) * candidate.per_cu);
+        if (count % slots != 0) {
+          const auto together = static_cast<double>(CeilDivide(count % slots, 256));
+          rounds += together / std::pow(together / static_cast<double>(candidate.per_cu), 0.4);
+        }
+        const auto cost = rounds * static_cast<double>(candidate.tile.tile_m * candidate.tile.tile_n) / candidate.rate;
+        if (cost < lowest) { lowest = cost; tile = candidate.tile; }
+      }
     }
     const auto tiles = CeilDivide(m, tile.tile_m) * CeilDivide(n, tile.tile_n) * batch_count;
     const auto split = (batch_count == 1) ? SplitFor(tiles, k, tile.index >= 8 && tile.index != 12) : 1;
