@@ -109,6 +109,26 @@ int SplitFor(const size_t tiles, const size_t k, const bool small_tile = false) 
   const auto allowed = k / 512;
   return static_cast<int>(std::max<size_t>(1, std::min<size_t>({wanted, allowed, 32})));
 }
+
+// Cost estimate of a launch of `count` work-groups of tile_m x tile_n, of which per_cu share a CU: the work-groups run in
+// rounds of 256 * per_cu; a whole round costs per_cu tile areas over the rate the tile's kernel sustains, and in the last
+// round a CU with c of its per_cu work-groups runs at (c / per_cu)^tail of that rate (tail = 1: a partly empty round
+// costs a whole one; tail = 0: it costs its share).
+struct TileCandidate {
+  Tile tile;
+  size_t per_cu;
+  double rate;
+};
+double LaunchCost(const TileCandidate& candidate, const size_t m, const size_t n, const double tail) {
+  const auto count = CeilDivide(m, candidate.tile.tile_m) * CeilDivide(n, candidate.tile.tile_n);
+  const auto slots = 256 * candidate.per_cu;
+  auto rounds = static_cast<double>((count / slots) * candidate.per_cu);
+  if (count % slots != 0) {
+    const auto together = static_cast<double>(CeilDivide(count % slots, 256));
+    rounds += together / std::pow(together / static_cast<double>(candidate.per_cu), tail);
+  }
+  return rounds * static_cast<double>(candidate.tile.tile_m * candidate.tile.tile_n) / candidate.rate;
+}
 }  // namespace
 
 KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const bool b_kcontig, const size_t m,
@@ -291,19 +311,11 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     // 1235 -> 1103 us on 128 x 64; 3029 x 6403 x 2752 T/N 987 -> 860 us on 64 x 64; 4096^3 and 8192^3 keep 256 x 128, 7000^3
     // keeps 128 x 128.
     if (batch_count == 1 && k >= 1024 && tiles64 >= 1024) {
-      struct Candidate { Tile tile; size_t per_cu; double rate; };
-      const Candidate candidates[] = {{Tile{3, 256, 128}, 1, 145.0}, {Tile{0, 128, 128}, 2, 142.0}, {Tile{11, 128, 64}, 2, 134.0},
-                                      {Tile{12, 64, 64}, 4, (a_kcontig && b_kcontig) ? 128.0 : 136.0}};
+      const TileCandidate candidates[] = {{Tile{3, 256, 128}, 1, 145.0}, {Tile{0, 128, 128}, 2, 142.0}, {Tile{11, 128, 64}, 2, 134.0},
+                                          {Tile{12, 64, 64}, 4, (a_kcontig && b_kcontig) ? 128.0 : 136.0}};
       auto lowest = 1e300;
       for (const auto& candidate : candidates) {
-        const auto count = CeilDivide(m, candidate.tile.tile_m) * CeilDivide(n, candidate.tile.tile_n);
-        const auto slots = 256 * candidate.per_cu;
-        auto rounds = static_cast<double>((count / slots) * candidate.per_cu);
-        if (count % slots != 0) {
-          const auto together = static_cast<double>(CeilDivide(count % slots, 256));
-          rounds += together / std::pow(together / static_cast<double>(candidate.per_cu), 0.4);
-        }
-        const auto cost = rounds * static_cast<double>(candidate.tile.tile_m * candidate.tile.tile_n) / candidate.rate;
+        const auto cost = LaunchCost(candidate, m, n, 0.4);
         if (cost < lowest) { lowest = cost; tile = candidate.tile; }
       }
     }
@@ -323,18 +335,18 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   if (batch_count > 1 && m <= 128 && n <= 128 && TileUse(m, n, 128, 128) >= 50 && batch_count >= 512) {
     return KernelChoice{CLBH_KERNEL_MFMA, 0, 1};  // batches of matrices of about one 128 x 128 tile (1024 x 96^3: 92 -> 74 us)
   }
-  const auto tiles128 = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
-  // (... whose last round is at least 90 % full: 5000^3, 1600 tiles in 6.25 rounds, takes 4.05 ms on them and 3.67 ms
-  // on 64 x 64)
-  if (tiles128 >= 1024 && k >= 1024 && batch_count == 1 && 10 * tiles128 >= 9 * CeilDivide(tiles128, 256) * 256) {
-    return KernelChoice{CLBH_KERNEL_MFMA, 0, SplitFor(tiles128, k)};
-  }
-  // Between one and four rounds of 128 x 128 tiles the 128 x 64 x 16 tile (two work-groups per CU) wins where its
-  // work-groups come in whole rounds of 512 - 2048^3 301 -> 249 us, 2048^2 x 8192 1.38 -> 0.98 ms, 4096 x 1024 x 4096
-  // 685 -> 496 us - and loses where they do not (3072^3: 963 against 798 us on 64 x 64)
-  const auto pairs = 2 * tiles128;
-  if (batch_count == 1 && k >= 1024 && tiles128 >= 256 && 10 * pairs >= 9 * CeilDivide(pairs, 512) * 512 && TileUse(m, n, 128, 64) >= 90) {
-    return KernelChoice{CLBH_KERNEL_MFMA, 2, 1};
+  // Single products with a long k: 128 x 128 x 8 or 64 x 64 x 16 by the cost estimate of the fp32 table (rates 70 and 69
+  // TFLOP/s, two and three work-groups per CU, a partly empty round at (c / p)^0.2 of the rate; fitted to 50 measured
+  // shapes: the choice is within 1 % of the better tile on all of them). 128 x 128 wins on whole tiles in whole rounds
+  // (8192^3, 4096^3: 1 %, 7000^3: 3 %, 3328 x 2304 x 2712: 8 %), 64 x 64 elsewhere (5120^3: 13 %). Against the rules this
+  // replaces (128 x 128 from 1024 tiles on with a last round 90 % full, 128 x 64 x 16 between one and four rounds of
+  // 128 x 128 tiles): 6016 x 2560 x 5793 3234 -> 2707 us, 3029 x 6403 x 2752 1745 -> 1634 us, 7680 x 2560 x 2133
+  // 1381 -> 1285 us, 3328 x 2304 x 2712 716 -> 646 us; the 128 x 64 x 16 tile (index 2) is no longer ahead anywhere.
+  if (batch_count == 1 && k >= 1024) {
+    const TileCandidate large{Tile{0, 128, 128}, 2, 70.0}, small{Tile{1, 64, 64}, 3, 69.0};
+    if (LaunchCost(large, m, n, 0.2) < LaunchCost(small, m, n, 0.2)) {
+      return KernelChoice{CLBH_KERNEL_MFMA, 0, SplitFor(CeilDivide(m, 128) * CeilDivide(n, 128), k)};
+    }
   }
   const auto tiles = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;
   return KernelChoice{CLBH_KERNEL_MFMA, 1, (batch_count == 1) ? SplitFor(tiles, k) : 1};
