@@ -73,6 +73,10 @@ __device__ __forceinline__ int HSwizzle(const int k) {
   return by_octet ^ ((W >= 128) ? 4 * (k & 3) : (W == 64) ? 4 * ((k >> 1) & 1) : 0);
 }
 
+// Byte offset that lies outside every buffer view of C (views are this long): loads from there deliver zero, stores
+// to there move nothing
+constexpr int kHOutside = 0x7fffff00;
+
 // Byte count from `from` to `end`, rounded up to whole dwords (the range check works per dword; the last
 // one may hold a single valid half) and clamped to what a resource can hold.
 __device__ __forceinline__ int HRecordsUpTo(const void* from, const void* end) {
@@ -481,28 +485,75 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
     } else {
       constexpr int WAVE_M = FM * 32, STAGE_PITCH = WAVE_M + 8;
       constexpr int LANES_PER_ROW = WAVE_M / 8, ROWS_PER_PASS = 64 / LANES_PER_ROW, PASSES = 32 / ROWS_PER_PASS;
-      typedef _Float16 half8u_t __attribute__((ext_vector_type(8), aligned(4)));  // C needs dword alignment only
       T* stage = lds + wave * (32 * STAGE_PITCH);
       const int wave_m0 = m0 + wave_m * WAVE_M;
-      const bool vector_rows = (wave_m0 + WAVE_M <= p.m) && (p.c_ld % 2 == 0) && ((reinterpret_cast<unsigned long long>(c) & 3) == 0) &&
-                               !masked;
+      // (the pieces of a block column are addressed by 32-bit byte offsets from its first element)
+      const bool vector_rows = (p.c_ld % 2 == 0) && ((reinterpret_cast<unsigned long long>(c) & 3) == 0) && !masked &&
+                               p.c_ld < (1 << 24);
       auto wave_fence = [&]() {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
       };
+      // (the lane number once more, opaque: what the epilogue derives from it is then computed here and not ahead of the
+      // K walk, where it would sit in registers that the walk has none to spare of - the 256 x 256 tile spilled 150)
+      int late_lane = lane;
+      asm volatile("" : "+v"(late_lane));
       // moves the staging tile's rows from (LOAD) or to (!LOAD) the block column starting at n_blk
       auto rows = [&](const int n_blk, auto load_tag) {
         constexpr bool LOAD = decltype(load_tag)::value;
         if (vector_rows) {
+          // C through a buffer view of the block column, every piece at an offset that lies outside the view where the
+          // piece does (rows from n on, m from the matrix's last row on): such loads deliver zeros and such stores move
+          // nothing, so no branch stands between the passes and all loads of a block column are in flight together
+          // (with a branch per pass each load was waited for before the next one left).
+          const auto view = __builtin_amdgcn_make_buffer_rsrc(c + n_blk * p.c_ld + wave_m0, 0, kHOutside, kRawBufferFlags);
+          const int rows_left = p.n - n_blk;
+          const int first_row = late_lane / LANES_PER_ROW, col = 8 * (late_lane % LANES_PER_ROW);
+          const int inside = p.m - (wave_m0 + col);  // how many of the lane's eight m lie inside the matrix
+          const int lane_offset = (first_row * static_cast<int>(p.c_ld) + col) * 2;
+          const int pass_step = ROWS_PER_PASS * static_cast<int>(p.c_ld) * 2;
+          T* cells = &stage[first_row * STAGE_PITCH + col];
+          // (four passes at a time: more pieces in flight cost the 256 x 256 tile, whose accumulators fill half of the
+          // registers, spills)
+          constexpr int GROUP = PASSES < 4 ? PASSES : 4;
+          const auto offset_of = [&](const int pass) {
+            const bool there = pass * ROWS_PER_PASS + first_row < rows_left && inside >= 8;
+            return there ? lane_offset + pass * pass_step : kHOutside;
+          };
 #pragma unroll
-          for (int pass = 0; pass < PASSES; ++pass) {
-            const int row = pass * ROWS_PER_PASS + lane / LANES_PER_ROW, col = 8 * (lane % LANES_PER_ROW);
-            if (n_blk + row < p.n) {
-              T* global = c + (n_blk + row) * p.c_ld + wave_m0 + col;
-              half8_t* local = reinterpret_cast<half8_t*>(&stage[row * STAGE_PITCH + col]);
-              if (LOAD) { *local = *reinterpret_cast<const half8u_t*>(global); }
-              else { *reinterpret_cast<half8u_t*>(global) = *local; }
+          for (int group = 0; group < PASSES; group += GROUP) {
+            half8_t pieces[GROUP];
+            if (LOAD) {
+#pragma unroll
+              for (int g = 0; g < GROUP; ++g) { pieces[g] = BufferLoad<T, 8>(view, offset_of(group + g)); }
+            }
+#pragma unroll
+            for (int g = 0; g < GROUP; ++g) {
+              half8_t* local = reinterpret_cast<half8_t*>(cells + (group + g) * ROWS_PER_PASS * STAGE_PITCH);
+              if (LOAD) { *local = pieces[g]; }
+              else { BufferStore<T, 8>(*local, view, offset_of(group + g)); }
+            }
+          }
+          // A wavefront on the m edge of the matrix: the one piece per row that straddles the last row of C moves
+          // element by element, in the same way (the pieces before it above, as whole pieces).
+          if (wave_m0 + WAVE_M > p.m) {
+            const bool straddles = inside > 0 && inside < 8;
+#pragma unroll
+            for (int pass = 0; pass < PASSES; ++pass) {
+              const bool there = pass * ROWS_PER_PASS + first_row < rows_left && straddles;
+              T* row_cells = cells + pass * ROWS_PER_PASS * STAGE_PITCH;
+              unsigned short values[7];
+#pragma unroll
+              for (int e = 0; e < 7; ++e) {
+                const int element = (there && e < inside) ? lane_offset + pass * pass_step + 2 * e : kHOutside;
+                if (LOAD) { values[e] = __builtin_amdgcn_raw_buffer_load_b16(view, element, 0, 0); }
+                else { __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, row_cells[e]), view, element, 0, 0); }
+              }
+              if (LOAD && straddles) {
+#pragma unroll
+                for (int e = 0; e < 7; ++e) { row_cells[e] = __builtin_bit_cast(T, values[e]); }
+              }
             }
           }
         } else {

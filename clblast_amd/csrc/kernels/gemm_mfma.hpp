@@ -167,6 +167,11 @@ __device__ __forceinline__ int RecordsUpTo(const void* from, const void* end) {
 }
 
 constexpr int kRawBufferFlags = 0x00020000;  // untyped raw buffer (stride 0), range-checked against its byte count
+// A buffer view of a tile of C is this many bytes long, so that a piece at this offset lies outside it (loads deliver
+// zero, stores move nothing); leading dimensions below kViewMaxLd keep every piece of a tile (up to 128 columns of
+// 8-byte elements) at a 32-bit offset inside.
+constexpr int kViewOutside = 0x7fffff00;
+constexpr long long kViewMaxLd = 1ll << 20;
 
 // Byte offset of this lane inside the chunk a direct load moves.
 template <typename T, int TILE_X, int TILE_K, int LANE_BYTES>
@@ -309,7 +314,15 @@ __device__ __forceinline__ typename VecType<T, VL>::type BufferLoad(const Resour
   constexpr int BYTES = VL * sizeof(T);
   if constexpr (BYTES == 4) { return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b32(resource, offset, uniform_offset, 0)); }
   else if constexpr (BYTES == 8) { return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b64(resource, offset, uniform_offset, 0)); }
-  else { static_assert(BYTES == 16, "piece size"); return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b128(resource, offset, uniform_offset, 0)); }
+  else if constexpr (BYTES == 16) { return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b128(resource, offset, uniform_offset, 0)); }
+  else {
+    static_assert(BYTES == 32, "piece size");  // two halves (an offset outside the resource stays outside: it is far from the end of the range)
+    struct Halves { decltype(__builtin_amdgcn_raw_buffer_load_b128(resource, 0, 0, 0)) low, high; };
+    Halves halves;
+    halves.low = __builtin_amdgcn_raw_buffer_load_b128(resource, offset, uniform_offset, 0);
+    halves.high = __builtin_amdgcn_raw_buffer_load_b128(resource, offset + 16, uniform_offset, 0);
+    return __builtin_bit_cast(V, halves);
+  }
 }
 
 template <typename T, int VL, typename V, typename Resource>
@@ -320,7 +333,12 @@ __device__ __forceinline__ void BufferStore(const V value, const Resource resour
   static_assert(sizeof(V) == BYTES, "value type");
   if constexpr (BYTES == 4) { __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, value), resource, offset, uniform_offset, 0); }
   else if constexpr (BYTES == 8) { __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(Dwords2, value), resource, offset, uniform_offset, 0); }
-  else {
+  else if constexpr (BYTES == 32) {
+    struct Halves { Dwords4 low, high; };
+    const Halves halves = __builtin_bit_cast(Halves, value);
+    BufferStore<unsigned, 4>(halves.low, resource, offset, uniform_offset);
+    BufferStore<unsigned, 4>(halves.high, resource, offset + 16, uniform_offset);
+  } else {
     static_assert(BYTES == 16, "piece size");
     const Dwords4 data = __builtin_bit_cast(Dwords4, value);
     __builtin_amdgcn_raw_buffer_store_b128(data, resource, offset, uniform_offset, 0);
@@ -743,6 +761,68 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
             for (int i = 0; i < FM; ++i) {
               if (writes(i, n)) {
                 dst[i * M_STEP] = (beta == T(0)) ? alpha * acc[i][j][r] : Combine(alpha, acc[i][j][r], beta, old_c[(j * ACC + r) * FM + i]);
+              }
+            }
+          }
+        }
+      }
+    } else if (M_INTERLEAVED && FM > 1 && c_ld < kViewMaxLd) {
+      // Large tiles whose lanes own runs of FM consecutive m: C through a buffer view of the tile, every piece at an
+      // offset that lies outside the view where the piece does (columns from n on, lanes at or beyond the last row): such
+      // loads deliver zeros and such stores move nothing. No branch stands between the pieces then, and the old C of
+      // four columns is in flight together before the first of them is combined and stored (with one branch per piece
+      // every load was waited for before the next one left). Lanes whose run straddles the last row, and tiles on the
+      // diagonal of a triangle, move their elements one by one afterwards.
+      // (64 bytes of old C per lane in flight)
+      constexpr int WANTED = 64 / static_cast<int>(sizeof(VMG)) > 0 ? 64 / static_cast<int>(sizeof(VMG)) : 1;
+      constexpr int BATCH = (ACC % WANTED == 0) ? WANTED : (ACC % 4 == 0) ? 4 : 1;
+      // (the lane's place once more, opaque: what the epilogue derives from it is then computed here and not ahead of
+      // the K walk, where it would occupy registers that the large tiles have none to spare of)
+      int late_read = a_read, late_g = lane_g;
+      asm volatile("" : "+v"(late_read), "+v"(late_g));
+      const int late_m = m0 + late_read;
+      const bool whole_run = (late_m + FM <= p.m) && !masked;
+      const auto view = __builtin_amdgcn_make_buffer_rsrc(c + n0 * c_ld + m0, 0, kViewOutside, kRawBufferFlags);
+      const int column_bytes = static_cast<int>(c_ld) * static_cast<int>(sizeof(T));
+      const int lane_bytes = (n_base - n0) * column_bytes + late_read * static_cast<int>(sizeof(T));
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+#pragma unroll
+        for (int r0 = 0; r0 < ACC; r0 += BATCH) {
+          int offset[BATCH];
+          VMG old[BATCH];
+#pragma unroll
+          for (int rr = 0; rr < BATCH; ++rr) {
+            const int column = FN * Traits::Row(r0 + rr, late_g) + j;
+            offset[rr] = (whole_run && n_base + column < p.n) ? lane_bytes + column * column_bytes : kViewOutside;
+          }
+          if (beta != T(0)) {
+#pragma unroll
+            for (int rr = 0; rr < BATCH; ++rr) { old[rr] = BufferLoad<T, FM>(view, offset[rr]); }
+          }
+#pragma unroll
+          for (int rr = 0; rr < BATCH; ++rr) {
+            const int r = r0 + rr;
+            VMG out;
+            if (beta == T(0)) {
+#pragma unroll
+              for (int i = 0; i < FM; ++i) { out[i] = alpha * acc[i][j][r]; }
+            } else {
+#pragma unroll
+              for (int i = 0; i < FM; ++i) { out[i] = Combine(alpha, acc[i][j][r], beta, old[rr][i]); }
+            }
+            BufferStore<T, FM>(out, view, offset[rr]);
+          }
+          if (!whole_run) {
+#pragma unroll
+            for (int rr = 0; rr < BATCH; ++rr) {
+              const int r = r0 + rr;
+              const int n = n_base + FN * Traits::Row(r, late_g) + j;
+#pragma unroll
+              for (int i = 0; i < FM; ++i) {
+                if (n < p.n && late_m + i < p.m && (!masked || InTriangle(p.c_triangle, late_m + i, n))) {
+                  StoreResult<T, T>(c + n * c_ld + late_m, i, acc[i][j][r], alpha, beta);
+                }
               }
             }
           }
