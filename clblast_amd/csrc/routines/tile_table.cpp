@@ -119,8 +119,9 @@ struct TileCandidate {
   size_t per_cu;
   double rate;
 };
-double LaunchCost(const TileCandidate& candidate, const size_t m, const size_t n, const double tail) {
-  const auto count = CeilDivide(m, candidate.tile.tile_m) * CeilDivide(n, candidate.tile.tile_n);
+double LaunchCost(const TileCandidate& candidate, const size_t m, const size_t n, const double tail,
+                  const size_t batch_count = 1) {
+  const auto count = CeilDivide(m, candidate.tile.tile_m) * CeilDivide(n, candidate.tile.tile_n) * batch_count;
   const auto slots = 256 * candidate.per_cu;
   auto rounds = static_cast<double>((count / slots) * candidate.per_cu);
   if (count % slots != 0) {
@@ -229,20 +230,22 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   }
   if (precision == Precision::kHalf) {
     // Direct-load tiles, 0: 128 x 128, 1: 64 x 64, 2: 256 x 256 (8 wavefronts), 3: 128 x 32, 4: 32 x 128 (the last two
-    // lose to 64 x 64 on skinny shapes too). The tile is chosen by a cost estimate: rounds of work-groups (256 x 256: one per CU, 128 x 128: two, 64 x 64: four)
-    // times what a CU spends on a round, tile area over the rate that tile's kernel reaches (relative to 256 x 256: 128 x
-    // 128 0.85, 64 x 64 0.5). Padded tiles count in full, so a matrix that fills a large tile badly pays for it. Checked
-    // against forced tiles on 25 shapes: 5000^3 297 us (64 x 64, the choice of an earlier rule: 672 us), 3500^3 117 us
-    // (215), 7000^3 844 us on 128 x 128 (256 x 256: 889), 1024 x 8192 x 1024 25 us on 128 x 128, 1500^3 38 us on 64 x 64.
-    const auto cost = [&](const size_t tile, const size_t per_cu, const size_t rate_percent) {
-      const auto tiles = CeilDivide(m, tile) * CeilDivide(n, tile) * batch_count;
-      return static_cast<double>(CeilDivide(tiles, 256 * per_cu) * per_cu * tile * tile) * 100.0 / static_cast<double>(rate_percent);
+    // lose to 64 x 64 on skinny shapes too). The tile is chosen by the cost estimate of LaunchCost - rounds of
+    // work-groups (256 x 256: one per CU, 128 x 128: two, 64 x 64: four), a partly empty last round at (c / p)^0.25 of
+    // the rate - times k + k0 over the tile's rate: a tile costs what k0 more slabs would, its prologue and epilogue
+    // (256 x 256: 1480 TFLOP/s and k0 = 630, 128 x 128: 940 and 290, 64 x 64: 490 and 40). Padded tiles count in full, so
+    // a matrix that fills a large tile badly pays for it. Fitted to the times of all three tiles on 107 shapes; the
+    // choice loses 1 % on average against the best of the three (the rule before it, whole rounds at fixed rates: 3-5 %;
+    // 1792 x 1536 x 6334 86 -> 71 us, 9728 x 2432 x 4512 263 -> 220 us, 6272 x 5760 x 3560 399 -> 321 us).
+    const auto cost = [&](const size_t tile, const size_t per_cu, const double rate, const double k0) {
+      return LaunchCost(TileCandidate{Tile{0, tile, tile}, per_cu, rate}, m, n, 0.25, batch_count) * (static_cast<double>(k) + k0);
     };
-    // (with a long k the 64 x 64 kernel stays at 550 TFLOP/s while 128 x 128 climbs to 800: 2048^2 x 8192 takes 125 us
-    // on 64 x 64 tiles and 90 us on 128 x 128 - but only where the latter fill the CUs; below that the 64 x 64 tiles win
-    // with K split)
+    // (with a long k the 64 x 64 kernel falls back to 450 TFLOP/s while 128 x 128 stays at 1000: 2048^2 x 8192 takes
+    // 125 us on 64 x 64 tiles and 90 us on 128 x 128 - but only where the latter fill the CUs; below that the 64 x 64
+    // tiles win with K split)
     const bool long_k = k >= 4096 && CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count >= 256;
-    const auto cost256 = (k >= 256) ? cost(256, 1, 100) : 1e300, cost128 = cost(128, 2, 85), cost64 = cost(64, 4, long_k ? 38 : 50);
+    const auto cost256 = (k >= 256) ? cost(256, 1, 1484.0, 627.0) : 1e300, cost128 = cost(128, 2, 936.0, 293.0),
+               cost64 = cost(64, 4, long_k ? 371.0 : 488.0, 44.0);
     int tile = 1;
     if (cost256 <= cost128 && cost256 <= cost64) { tile = 2; }
     else if (cost128 <= cost64) { tile = 0; }
