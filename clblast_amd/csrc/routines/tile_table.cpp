@@ -297,12 +297,18 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       tile = Tile{11, 128, 64};  // whole rounds of two work-groups per CU (2048^3: 140 -> 131 us, 4096 x 3072 x 2048: 396 -> 385)
     }
     else if (tiles64 <= 64 && k < 2048) { tile = Tile{10, 32, 32}; }
-    else if (tiles64 < 1024 && (batch_count == 1 || n > 64) &&
+    else if (tiles64 < (batch_count > 1 ? 1024u : (k >= 4096 ? 704u : 600u)) && (batch_count == 1 || n > 64) &&
              !(a_kcontig && b_kcontig && tiles64 >= 512 && k >= 1024 && batch_count == 1)) {
       // (batches of matrices one tile wide keep 64 x 64: 87 -> 62 us; so do two k-contiguous operands from two tiles per
       // CU on, where the narrow tile's staging costs more than it gains: 2048 x 1024 x 4096 T/N 163 -> 149 us, x 8192
       // 321 -> 287 us; with 384 tiles the 64 x 32 tile is still 14 % ahead)
+      // (from 600 tiles on - 704 with k >= 4096 - a single product stays on 64 x 64 tiles, which move C in 16-byte
+      // pieces: 439 x 6743 x 746 53 -> 49 us, 1572 x 2291 x 179 26 -> 23 us, 576 x 7123 x 3145 233 -> 214 us,
+      // 896 x 2944 x 1733 100 -> 93 us; 1728 x 1472 x 5895 keeps 64 x 32: 273 against 300 us)
       tile = Tile{9, 64, 32};
+      // ... or 32 x 64 where that pads the matrix less (455 x 3908 x 5312: 211 -> 195 us, 128 x 2603 x 708: 16 -> 14 us)
+      const auto padded = [&](const size_t tile_m, const size_t tile_n) { return CeilDivide(m, tile_m) * tile_m * CeilDivide(n, tile_n) * tile_n; };
+      if (batch_count == 1 && (padded(32, 64) < padded(64, 32) || (padded(32, 64) == padded(64, 32) && n > m))) { tile = Tile{8, 32, 64}; }
     }
     // Large single products with a long k: the four tiles that matter there by a cost estimate. A tile's work-groups
     // run in rounds (256 x 128: one per CU, 128 x 128 and 128 x 64: two, 64 x 64: four); a whole round costs the tile area
@@ -313,7 +319,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     // worst 7 %): 5120^3 2167 us on 128 x 128 (the choice of the rules above), 1976 us on 64 x 64; 6000 x 3000 x 4000
     // 1235 -> 1103 us on 128 x 64; 3029 x 6403 x 2752 T/N 987 -> 860 us on 64 x 64; 4096^3 and 8192^3 keep 256 x 128, 7000^3
     // keeps 128 x 128.
-    if (batch_count == 1 && k >= 1024 && tiles64 >= 1024) {
+    if (batch_count == 1 && k >= 1024 && tiles64 >= 704) {
       const TileCandidate candidates[] = {{Tile{3, 256, 128}, 1, 145.0}, {Tile{0, 128, 128}, 2, 142.0}, {Tile{11, 128, 64}, 2, 134.0},
                                           {Tile{12, 64, 64}, 4, (a_kcontig && b_kcontig) ? 128.0 : 136.0}};
       auto lowest = 1e300;
