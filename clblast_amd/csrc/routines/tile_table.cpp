@@ -333,10 +333,12 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     return KernelChoice{CLBH_KERNEL_MFMA, tile.index, split};
   }
   // fp64 (same sweep): 64 x 64 x 16 tiles (index 1) up to about 3072^3, 128 x 128 x 8 (index 0) beyond; for launches
-  // that leave CUs idle 64 x 32 x 16 (index 5, up to 256 tiles of 64 x 64) and 32 x 32 x 32 (index 6, up to 144 such
+  // that leave CUs idle 64 x 32 x 16 (index 5, up to 256 tiles of 64 x 64 in a batch, 420 otherwise) and 32 x 32 x 32 (index 6, up to 144 such
   // tiles and a short k: 512^3 22.7 -> 10.4 us)
+  // (single products up to 420 tiles: 1587 x 886 x 211 26 -> 21 us, 320 x 3937 x 1920 132 -> 103 us, 960 x 1123 x 5062
+  // 339 -> 276 us on 64 x 32; from 424 tiles on the two are level)
   const auto tiles64 = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;
-  if (tiles64 <= 256) {
+  if (tiles64 <= (batch_count == 1 ? 420u : 256u)) {
     const bool smallest = (tiles64 <= 144 && k < 2048);
     const auto tiles = CeilDivide(m, smallest ? 32 : 64) * CeilDivide(n, 32) * batch_count;
     return KernelChoice{CLBH_KERNEL_MFMA, smallest ? 6 : 5, (batch_count == 1) ? SplitFor(tiles, k, true) : 1};
@@ -355,6 +357,16 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     const TileCandidate large{Tile{0, 128, 128}, 2, 70.0}, small{Tile{1, 64, 64}, 3, 69.0};
     if (LaunchCost(large, m, n, 0.2) < LaunchCost(small, m, n, 0.2)) {
       return KernelChoice{CLBH_KERNEL_MFMA, 0, SplitFor(CeilDivide(m, 128) * CeilDivide(n, 128), k)};
+    }
+  }
+  // Up to 2000 tiles of 64 x 64 (three share a CU) their last round can stay emptier than that of the 64 x 32 tiles (five
+  // per CU, 87 % of the rate): the same estimate, with a partly empty round at (c / p)^0.8 of the rate, picks between the
+  // two (fitted to 26 shapes: 4616 x 760 x 448 80 -> 67 us, 8002 x 448 x 5254 723 -> 661 us, 1792 x 2033 x 1216
+  // 173 -> 152 us; 576 x 7123 x 3145 stays on 64 x 64: 394 against 436 us)
+  if (batch_count == 1 && tiles64 <= 2000) {
+    const TileCandidate square{Tile{1, 64, 64}, 3, 69.0}, narrow{Tile{5, 64, 32}, 5, 60.0};
+    if (LaunchCost(narrow, m, n, 0.8) < LaunchCost(square, m, n, 0.8)) {
+      return KernelChoice{CLBH_KERNEL_MFMA, 5, SplitFor(CeilDivide(m, 64) * CeilDivide(n, 32), k, true)};
     }
   }
   const auto tiles = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;
