@@ -165,6 +165,50 @@ def test_every_tile_variant(gpu, bits):
 
 
 @pytest.mark.parametrize("bits", BITS)
+def test_pieces_of_c_that_straddle_the_last_row(gpu, bits):
+    """The tiles move C in pieces of several consecutive rows per lane (eight in fp16, two or four in fp32 and
+    fp64) at offsets into a buffer view of the tile; the piece that straddles the last row of C moves element by
+    element and the pieces beyond it not at all. Shapes whose m leaves every remainder of a piece, with an even
+    leading dimension and offset (the fp16 kernel's vector path), for every tile, beta zero and non-zero; the
+    check covers the memory around C too."""
+    import clblast_amd
+    gpu.force_path(bits, "indirect")
+    try:
+        seed = 7600
+        for variant in TILE_VARIANTS[bits]:
+            clblast_amd.override_parameters(0, "Xgemm", bits, {"TILE_VARIANT": variant})
+            for m, (ta, tb) in zip((257, 258, 259, 261, 262, 263, 385, 390), itertools.cycle(itertools.product(TRANSPOSES, TRANSPOSES))):
+                seed += 1
+                extra_c = 8 - m % 2  # m + extra_c is even
+                problem = gpu.Problem(bits, COL_MAJOR, ta, tb, m, 150, 96, 0.5, 2.0 if seed % 2 else 0.0, a_offset=8,
+                                      b_offset=16, c_offset=24, seed=seed, extra_ld=(8, 8, extra_c))
+                status, c_after = problem.run()
+                assert status == 0, (variant, problem.describe())
+                problem.check(c_after)
+    finally:
+        clblast_amd.override_parameters(0, "Xgemm", bits, {"TILE_VARIANT": 0})
+        gpu.force_path(bits, None)
+
+
+def test_leading_dimension_of_c_beyond_the_buffer_views(gpu):
+    """From a leading dimension of 2^20 elements on the offsets of a tile's pieces no longer fit the 32-bit offsets
+    of a buffer view, and the large fp32 tiles address C through pointers again."""
+    import clblast_amd
+    gpu.force_path(32, "indirect")
+    try:
+        for variant, seed in ((4, 7700), (1, 7701), (12, 7702)):
+            clblast_amd.override_parameters(0, "Xgemm", 32, {"TILE_VARIANT": variant})
+            problem = gpu.Problem(32, COL_MAJOR, NO, YES, 301, 20, 64, 0.5, 2.0, seed=seed, extra_ld=(0, 0, (1 << 20) + 3 - 301))
+            assert problem.c_ld == (1 << 20) + 3
+            status, c_after = problem.run()
+            assert status == 0, (variant, problem.describe())
+            problem.check(c_after)
+    finally:
+        clblast_amd.override_parameters(0, "Xgemm", 32, {"TILE_VARIANT": 0})
+        gpu.force_path(32, None)
+
+
+@pytest.mark.parametrize("bits", BITS)
 def test_padding_and_neighbouring_memory_never_reach_the_result(gpu, bits, path):
     """Every element of the A and B buffers outside the logical matrices (leading-dimension padding, the
     offset prefix, the tail) is NaN: edge tiles and the K tail may read such memory but must not let it
