@@ -34,14 +34,14 @@ DTYPE_NAME = {"S": "f32", "D": "f64", "H": "f16", "C": "c64 (f32 arithmetic)", "
 # committed profiles: workload -> (bytes, the profile that holds the commands and the raw readings, the kernel they
 # were read for). The roofline object names both, and tests/test_bench_contract.py checks each entry against its file.
 MEASURED_TRAFFIC = {
-    "cfg2s": (5.614e9, "profiles/sgemm_8192_rowTN.md", "clbh::GemmMfmaKernel<float, clbh::MfmaConfig<float, 2, 2, 4, 2, 16, 2"),
-    "cfg2d": (1.2041e10, "profiles/dgemm_8192_rowTN.md", "clbh::GemmMfmaKernel<double, clbh::MfmaConfig<double, 2, 2, 4, 4, 8, 2"),
-    "cfg3": (1.892e9, "profiles/hgemm_8192_colNT.md", "clbh::HgemmDirectKernel<clbh::HdirectConfig<2, 4, 4, 2, 2, 3, false>"),
+    "cfg2s": (5.196e9, "profiles/sgemm_8192_rowTN.md", "clbh::GemmMfmaKernel<float, clbh::MfmaConfig<float, 2, 2, 4, 2, 16, 2"),
+    "cfg2d": (1.3193e10, "profiles/dgemm_8192_rowTN.md", "clbh::GemmMfmaKernel<double, clbh::MfmaConfig<double, 2, 2, 4, 4, 8, 2"),
+    "cfg3": (1.932e9, "profiles/hgemm_8192_colNT.md", "clbh::HgemmDirectKernel<clbh::HdirectConfig<2, 4, 4, 2, 2, 3, false>"),
     "cfg4": (1.007e8, "profiles/sgemm_strided_batched_8192x32.md", "clbh::GemmSmallBatchedKernel"),
-    "cfg5c": (7.464e7, "profiles/sgemm_17x4099x4096_colNN.md", "clbh::GemmSkinnyRowsKernel<4, 5, 5, 2, false, false, 2>"),
-    "cfg5d": (6.271e8, "profiles/sgemm_8191x8191x127_colNN.md", "clbh::GemmStreamKernel<float, clbh::MfmaConfig<float, 1, 4, 4, 1, 16, 2"),
-    "cfg5e": (7.369e7, "profiles/sgemm_4099x17x4096_colTN.md", "clbh::GemmSkinnyRowsKernel<4, 5, 5, 2, true, true, 2>"),
-    "sbat64": (2.027e8, "profiles/sgemm_strided_batched_4096x64.md", "clbh::GemmStreamKernel<float, clbh::MfmaConfig<float, 1, 4, 4, 1, 16, 4"),
+    "cfg5c": (7.461e7, "profiles/sgemm_17x4099x4096_colNN.md", "clbh::GemmSkinnyRowsKernel<4, 5, 5, 2, false, false, 2>"),
+    "cfg5d": (6.225e8, "profiles/sgemm_8191x8191x127_colNN.md", "clbh::GemmStreamKernel<float, clbh::MfmaConfig<float, 1, 4, 4, 1, 16, 2"),
+    "cfg5e": (7.371e7, "profiles/sgemm_4099x17x4096_colTN.md", "clbh::GemmSkinnyRowsKernel<4, 5, 5, 2, true, true, 2>"),
+    "sbat64": (2.036e8, "profiles/sgemm_strided_batched_4096x64.md", "clbh::GemmStreamKernel<float, clbh::MfmaConfig<float, 1, 4, 4, 1, 16, 4"),
     "cgemm_batched": (4.028e8, "profiles/cgemm_strided_batched_4096x64_rowNC.md", "clbh::GemmComplexSmallKernel<float, 2, true, true>"),
 }
 
