@@ -160,15 +160,32 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   if (forced == 0 && !triangular && precision != Precision::kHalf && k > 48 &&
       largest_ld < static_cast<size_t>(CLBH_STREAM_MAX_LD)) {
     const auto tiles128 = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
-    // (two k-contiguous operands go through the staging registers: 4096^2 x 1000 is 6 % behind the 256 x 128 tiles then)
-    if (precision == Precision::kSingle && tiles128 >= 1024 && TileUse(m, n, 128, 128) >= 90 &&
+    // (two k-contiguous operands go through the staging registers: 4096^2 x 1000 is 6 % behind the 256 x 128 tiles then;
+    // batches also where these tiles fill 70 % of the matrices and pad them no more than 64 x 64 tiles would:
+    // 224 x 128 x 102 x 1525 203 -> 145 us)
+    const bool batched = batch_count > 1;
+    const auto use128 = TileUse(m, n, 128, 128), use64 = TileUse(m, n, 64, 64);
+    if (precision == Precision::kSingle && (use128 >= 90 ? tiles128 >= 1024 : (batched && tiles128 >= 512 && use128 >= 70 && use128 >= use64)) &&
         k <= ((a_kcontig && b_kcontig) ? 640u : 1024u)) {
       return KernelChoice{CLBH_KERNEL_STREAM, 1, 1};
     }
     const auto tiles64 = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;
+    // Batches (forced-kernel sweeps over 76 random batched shapes per precision, m, n <= 1024, k <= 2048): the persistent
+    // kernel on 64 x 64 tiles is the fastest or within 5 % of it on five shapes in six, also with a long k and with as few
+    // as 400 tiles - fp32 64 x 928 x 188 x 28 15 -> 11 us, 349 x 974 x 540 x 7 39 -> 31 us, 979 x 580 x 608 x 20 155 -> 132 us,
+    // 224 x 251 x 1515 x 93 197 -> 171 us; fp64 33 x 480 x 96 x 776 157 -> 111 us, 129 x 892 x 186 x 1139 1533 -> 1383 us - unless
+    // its tiles pad the matrices badly (fp32 424 x 78 x 1137 x 1033: 1368 against 1260 us on 64 x 32 tiles). Before it:
+    // where 128 x 128 tiles pad the matrices no more than 64 x 64 tiles do (n or m just below 128), k is not short and
+    // the batch fills four rounds of them, the tiled kernel on 128 x 128 - fp32 251 x 98 x 373 x 1656 607 -> 424 us,
+    // 199 x 79 x 571 x 3380 1439 -> 1165 us (the persistent kernel: 613 and 1536), fp64 251 x 98 x 373 x 1656 1011 -> 789 us.
+    if (batched) {
+      if (k >= 320 && tiles128 >= 2048 && use128 >= use64) { return KernelChoice{CLBH_KERNEL_MFMA, 0, 1}; }
+      // (with k up to 512 whatever the padding: fp32 192 x 34 x 266 x 218 21 -> 18 us, fp64 33 x 160 x 96 x 555 44 -> 32 us)
+      const bool fills = k <= 512 || use64 >= (precision == Precision::kSingle ? 60u : 68u);
+      if (tiles64 >= 400 && k <= 2048 && fills) { return KernelChoice{CLBH_KERNEL_STREAM, 2, 1}; }
+    }
     // (batches: from 2048 tiles on, and fp64 up to k = 400 - fp64 256 x 256^3 164 -> 153 us, 256 x 200 x 300 x 400
     // 296 -> 275 us, 128 x 384^3 266 -> 245 us; at k = 512 the tiled kernel is ahead again)
-    const bool batched = batch_count > 1;
     const bool fp64 = (precision == Precision::kDouble);
     const size_t k_limit = batched ? (fp64 ? 400 : 192) : (fp64 ? 640 : 448);
     const size_t tiles_floor = batched ? 2048 : (fp64 ? 2048 : 1500);
@@ -182,8 +199,10 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   // longer k (fp32 1024 x 128^3: 57 against 70 us) the ring of three slabs of the large-tile kernels wins.
   if (forced == 0 && batch_count > 1 && !triangular && precision != Precision::kHalf && m <= 256 && n <= 256 &&
       k <= (precision == Precision::kSingle ? 96u : 64u) && CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count >= 512) {
+    // (only where its 32 x 32 tiles pad the matrices a quarter less than 64 x 64 tiles: on 64 x 64 tiles the kernels with
+    // the ring of slabs have caught up - 2491 x 256 x 64 x 32 fp32 92 against 84 us, fp64 182 against 162 us)
     const auto padded = [m, n](const size_t tile) { return CeilDivide(m, tile) * CeilDivide(n, tile) * tile * tile; };
-    return KernelChoice{CLBH_KERNEL_SMALL_TILED, (4 * padded(32) < 3 * padded(64)) ? 1 : 0, 1};
+    if (4 * padded(32) < 3 * padded(64)) { return KernelChoice{CLBH_KERNEL_SMALL_TILED, 1, 1}; }
   }
   if ((forced == 101 || forced == 102) && !triangular && precision != Precision::kHalf) {
     return KernelChoice{CLBH_KERNEL_SMALL_TILED, static_cast<int>(forced) - 101, 1};  // one-slab kernel, 64 x 64 / 32 x 32 tiles
@@ -290,8 +309,10 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
         tile = Tile{0, 128, 128};
       }
     }
-    else if (batch_count > 1 && TileUse(m, n, 128, 128) >= 90 && CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count >= 512) {
-      tile = Tile{0, 128, 128};  // batches of matrices that fill 128 x 128 tiles (1024 x 128^3: 66 -> 57 us)
+    else if (batch_count > 1 && k >= 96 && TileUse(m, n, 128, 128) >= 90 && CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count >= 512) {
+      // batches of matrices that fill 128 x 128 tiles (1024 x 128^3: 66 -> 57 us), but for the shortest k, where C's
+      // 16-byte pieces of the 64 x 64 tile count for more (497 x 960 x 32 x 466: 676 -> 500 us, 961 x 67 x 20 x 348: 107 -> 72 us)
+      tile = Tile{0, 128, 128};
     }
     else if (batch_count == 1 && k >= 256 && TileUse(m, n, 128, 64) >= 90 && FillsPairs(CeilDivide(m, 128) * CeilDivide(n, 64))) {
       tile = Tile{11, 128, 64};  // whole rounds of two work-groups per CU (2048^3: 140 -> 131 us, 4096 x 3072 x 2048: 396 -> 385)
@@ -342,6 +363,12 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     const bool smallest = (tiles64 <= 144 && k < 2048);
     const auto tiles = CeilDivide(m, smallest ? 32 : 64) * CeilDivide(n, 32) * batch_count;
     return KernelChoice{CLBH_KERNEL_MFMA, smallest ? 6 : 5, (batch_count == 1) ? SplitFor(tiles, k, true) : 1};
+  }
+  // (batches of matrices that 64 x 64 tiles fill badly and 32 x 32 tiles one and a half times better, k not short:
+  // 224 x 96 x 800 x 133 161 -> 120 us, 199 x 79 x 571 x 3380 2453 -> 2196 us; at 1.4 times - 515 x 96 x 544 x 1641 - the 64 x 64
+  // tiles are ahead, 2090 against 2329 us)
+  if (batch_count > 1 && tiles64 >= 400 && k >= 256 && TileUse(m, n, 64, 64) < 68 && 2 * TileUse(m, n, 32, 32) >= 3 * TileUse(m, n, 64, 64)) {
+    return KernelChoice{CLBH_KERNEL_MFMA, 6, 1};
   }
   if (batch_count > 1 && m <= 128 && n <= 128 && TileUse(m, n, 128, 128) >= 50 && batch_count >= 512) {
     return KernelChoice{CLBH_KERNEL_MFMA, 0, 1};  // batches of matrices of about one 128 x 128 tile (1024 x 96^3: 92 -> 74 us)
