@@ -183,3 +183,29 @@ def test_python_binding_mirrors_pyclblast(gpu):
     with pytest.raises(clblast_amd.CLBlastError) as info:
         clblast_amd.gemm(None, 0, 4, 4, a_dev, b_dev, c_dev.float(), 4, 4, 4)
     assert info.value.status == -1017
+
+
+@pytest.mark.parametrize("bits", [32, 64, 16])
+def test_random_batched_shapes_through_the_automatic_choice(gpu, bits):
+    """Seeded random strided-batched calls - shapes up to 300 x 300 x 400, batches of 2 to 60, all layouts and
+    transposes, odd and even offsets and paddings - through whatever kernel the library picks for them (the
+    persistent kernel, the tiled kernels with small and large tiles, the one-slab and one-wavefront kernels)."""
+    rng = np.random.default_rng(4200 + bits)
+    for case in range(40):
+        m, n = (int(v) for v in rng.integers(1, 300, size=2))
+        k = int(rng.integers(1, 400))
+        batch = int(rng.integers(2, 60))
+        layout = (ROW_MAJOR, COL_MAJOR)[int(rng.integers(2))]
+        ta, tb = ((NO, YES)[int(rng.integers(2))] for _ in range(2))
+        even = bool(rng.integers(2))
+        offsets = tuple(int(v) * (2 if even else 1) for v in rng.integers(0, 9, size=3))
+        extra = tuple(int(v) * (2 if even else 1) for v in rng.integers(0, 5, size=3))
+        if even:  # even leading dimensions too: the fp16 kernels' dword path
+            _, shape = oracle.process_arguments(layout, ta, tb, m, n, k)
+            extra = tuple(e + (one % 2) for e, one in zip(extra, (shape.a_one, shape.b_one, shape.c_one)))
+        alpha, beta = float(rng.choice([1.0, -0.5, 2.0])), float(rng.choice([0.0, 1.0, 0.75]))
+        try:
+            run_strided(gpu, bits, layout, ta, tb, m, n, k, alpha, beta, batch, offsets=offsets, extra_ld=extra, seed=9000 + 3 * case)
+        except AssertionError as failure:
+            raise AssertionError("case %d: layout=%d ta=%d tb=%d m=%d n=%d k=%d batch=%d offsets=%s extra=%s alpha=%g beta=%g: %s" %
+                                 (case, layout, ta, tb, m, n, k, batch, offsets, extra, alpha, beta, failure))

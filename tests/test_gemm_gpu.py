@@ -190,6 +190,32 @@ def test_pieces_of_c_that_straddle_the_last_row(gpu, bits):
         gpu.force_path(bits, None)
 
 
+@pytest.mark.parametrize("bits", BITS)
+def test_random_shapes_through_the_automatic_choice(gpu, bits):
+    """Seeded random calls - shapes up to 1500 x 1500 x 1200 (most of them smaller), all layouts and transposes, odd
+    and even offsets and paddings, beta zero and non-zero - through whatever tile and K split the library's cost
+    estimates pick for them."""
+    rng = np.random.default_rng(5200 + bits)
+    for case in range(36):
+        large = case % 6 == 0
+        m, n = (int(v) for v in rng.integers(1, 1500 if large else 500, size=2))
+        k = int(rng.integers(1, 1200 if large else 700))
+        layout = LAYOUTS[int(rng.integers(2))]
+        ta, tb = (TRANSPOSES[int(rng.integers(2))] for _ in range(2))
+        even = bool(rng.integers(2))
+        offsets = [int(v) * (2 if even else 1) for v in rng.integers(0, 9, size=3)]
+        extra = [int(v) * (2 if even else 1) for v in rng.integers(0, 5, size=3)]
+        if even:  # even leading dimensions too: the fp16 kernels' dword path
+            _, shape = oracle.process_arguments(layout, ta, tb, m, n, k)
+            extra = [e + (one % 2) for e, one in zip(extra, (shape.a_one, shape.b_one, shape.c_one))]
+        alpha, beta = float(rng.choice([1.0, -0.5, 2.0])), float(rng.choice([0.0, 1.0, 0.75]))
+        problem = gpu.Problem(bits, layout, ta, tb, m, n, k, alpha, beta, a_offset=offsets[0], b_offset=offsets[1],
+                              c_offset=offsets[2], seed=5300 + case, extra_ld=tuple(extra))
+        status, c_after = problem.run()
+        assert status == 0, (case, problem.describe())
+        problem.check(c_after)
+
+
 def test_leading_dimension_of_c_beyond_the_buffer_views(gpu):
     """From a leading dimension of 2^20 elements on the offsets of a tile's pieces no longer fit the 32-bit offsets
     of a buffer view, and the large fp32 tiles address C through pointers again."""
