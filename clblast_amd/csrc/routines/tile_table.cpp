@@ -409,6 +409,32 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   // fp64 (same sweep): 64 x 64 x 16 tiles (index 1) up to about 3072^3, 128 x 128 x 8 (index 0) beyond; for launches
   // that leave CUs idle 64 x 32 x 16 (index 5, up to 256 tiles of 64 x 64 in a batch, 420 otherwise) and 32 x 32 x 32 (index 6, up to 144 such
   // tiles and a short k: 512^3 22.7 -> 10.4 us)
+  // Single products with a long k and at most one round of 128 x 128 tiles: tile and number of K ranges together, as in
+  // the fp32 table (128 x 128 x 8: 70.6 TFLOP/s and k0 = 43, two per CU; 64 x 64: 70.6 and 91, three; 64 x 32: 67.9 and 81,
+  // five; 32 x 32: 61 and 101, eight; two k-contiguous operands 0.94 of the rate; a partly empty round at (c / p)^0.18;
+  // the reduction 3.3 us and 0.6 us per range). Fitted to 360 timings (24 shapes, four tiles, four splits): the choice
+  // loses 3 % on average against the best of them, the rules it replaces 13 % - 384 x 2048 x 11674 415 -> 289 us,
+  // 1600 x 704 x 9315 T/N 496 -> 361 us, 658 x 2109 x 18036 995 -> 815 us.
+  if (batch_count == 1 && k >= 2048 && std::min(m, n) >= 256 && CeilDivide(m, 128) * CeilDivide(n, 128) <= 256) {
+    struct Option { Tile tile; size_t per_cu; double rate, k0; };
+    const Option options[] = {{Tile{0, 128, 128}, 2, 70.6, 43.0}, {Tile{1, 64, 64}, 3, 70.6, 91.0}, {Tile{5, 64, 32}, 5, 67.9, 81.0},
+                              {Tile{6, 32, 32}, 8, 61.0, 101.0}};
+    auto lowest = 1e300;
+    auto chosen = KernelChoice{CLBH_KERNEL_MFMA, 1, 1};
+    for (const auto& option : options) {
+      const auto rate = option.rate * ((a_kcontig && b_kcontig) ? 0.936 : 1.0);
+      for (size_t ranges = 1; ranges <= 16; ranges *= 2) {
+        const auto range = CeilDivide(CeilDivide(k, ranges), 64) * 64;
+        if (ranges > 1 && range < 512) { break; }
+        const auto launched = CeilDivide(k, range);
+        auto time = LaunchCost(TileCandidate{option.tile, option.per_cu, rate}, m, n, 0.178, launched) *
+                    (static_cast<double>(range) + option.k0) * 512e-6;
+        if (launched > 1) { time += 3.3 + 0.6 * static_cast<double>(launched); }
+        if (time < lowest) { lowest = time; chosen = KernelChoice{CLBH_KERNEL_MFMA, option.tile.index, static_cast<int>(launched)}; }
+      }
+    }
+    return chosen;
+  }
   // (single products up to 420 tiles: 1587 x 886 x 211 26 -> 21 us, 320 x 3937 x 1920 132 -> 103 us, 960 x 1123 x 5062
   // 339 -> 276 us on 64 x 32; from 424 tiles on the two are level)
   const auto tiles64 = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;
