@@ -317,9 +317,16 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     // k-contiguous, the kernel that puts its lanes along k and gives a work-group 8 to 20 rows and all of K does it in one
     // launch (4099 x 17 x 4096 with a transposed A: 27.5 us on 64 x 32 tiles with K split, 16.4 us here; 17 x 4099 x 4096:
     // 27.5 -> 17.7 us)
-    if (batch_count == 1 && std::min(m, n) <= 32 && std::max(m, n) >= 1024 && k >= 512 && k < (size_t{1} << 28) && (n <= 32 ? a_kcontig : b_kcontig) &&
+    // Its products run on the vector ALUs, about 17e6 of them per microsecond, so with more than a dozen columns and a large
+    // operand it falls behind the 64 x 32 / 32 x 64 tiles with K split, which stream at 5.2 TB/s after 10 us: the kernel is
+    // taken where 4 us + max(bytes / 5.8 TB/s, products / 17e6) is the shorter time (4 x 16384 x 16384: 182 against 205 us;
+    // 17 x 16384 x 4096: 63 against 52 us, 32 x 16384 x 16384: 565 against 217 us - those two take the tiles now).
+    if (batch_count == 1 && std::min(m, n) <= 32 && std::max(m, n) >= 256 && k >= 256 && k < (size_t{1} << 28) && (n <= 32 ? a_kcontig : b_kcontig) &&
         largest_ld < static_cast<size_t>(CLBH_SKINNY_MAX_LD)) {
-      return KernelChoice{CLBH_KERNEL_SKINNY, 0, 1};
+      const auto elements = static_cast<double>(std::max(m, n)) * static_cast<double>(k);
+      const auto skinny_time = 4.0 + std::max(elements * 4.0 / 5.8e6, elements * static_cast<double>(std::min(m, n)) / 17e6);
+      const auto tiled_time = 10.0 + elements * 4.0 / 5.2e6;
+      if (skinny_time < tiled_time) { return KernelChoice{CLBH_KERNEL_SKINNY, 0, 1}; }
     }
     auto tile = Tile{12, 64, 64};  // (the 64 x 64 tile that moves C in 16-byte pieces; index 7 is the one on 32x32x2)
     const auto tiles64 = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;
@@ -386,10 +393,13 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     // Fitted to 870 timings (62 shapes, four tiles, up to four splits each); the choice loses 1.6 % on average against
     // the best of them, the rules it replaces 8 %: 1024^2 x 8192 T/N 176 -> 137 us, 1536^2 x 4096 180 -> 161 us,
     // 1024^2 x 4096 T/N 91 -> 76 us, 768^2 x 16384 T/N 210 -> 178 us.
-    if (batch_count == 1 && k >= 2048 && std::min(m, n) >= 256 && CeilDivide(m, 128) * CeilDivide(n, 128) <= 256) {
+    // (also for matrices with 33 to 255 rows or columns, with the 32 x 64 tile at the rates of its mirror image:
+    // 13311 x 58 x 5185 125 -> 110 us, 8917 x 183 x 7358 303 -> 261 us)
+    if (batch_count == 1 && k >= 2048 && std::min(m, n) > 32 && CeilDivide(m, 128) * CeilDivide(n, 128) <= 256) {
       struct Option { Tile tile; size_t per_cu; double rate, k0, both_kcontig; };
       const Option options[] = {{Tile{0, 128, 128}, 2, 157.6, 172.0, 0.984}, {Tile{11, 128, 64}, 2, 140.4, 103.0, 0.984},
-                                {Tile{12, 64, 64}, 4, 142.6, 110.0, 0.935}, {Tile{9, 64, 32}, 4, 123.8, 92.0, 0.935}};
+                                {Tile{12, 64, 64}, 4, 142.6, 110.0, 0.935}, {Tile{9, 64, 32}, 4, 123.8, 92.0, 0.935},
+                                {Tile{8, 32, 64}, 4, 123.8, 92.0, 0.935}};
       auto lowest = 1e300;
       for (const auto& option : options) {
         const auto rate = option.rate * ((a_kcontig && b_kcontig) ? option.both_kcontig : 1.0);
