@@ -424,7 +424,9 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   // the reduction 3.3 us and 0.6 us per range). Fitted to 360 timings (24 shapes, four tiles, four splits): the choice
   // loses 3 % on average against the best of them, the rules it replaces 13 % - 384 x 2048 x 11674 415 -> 289 us,
   // 1600 x 704 x 9315 T/N 496 -> 361 us, 658 x 2109 x 18036 995 -> 815 us.
-  if (batch_count == 1 && k >= 2048 && std::min(m, n) >= 256 && CeilDivide(m, 128) * CeilDivide(n, 128) <= 256) {
+  // (from k = 700 and 33 rows and columns on, ranges from 256: on 78 shapes the choice loses 3 % against the best forced
+  // pair, the rules it replaces 9 % - 128 x 2944 x 1761 T/N 48 -> 35 us, 256 x 1088 x 1158 31 -> 25 us)
+  if (batch_count == 1 && k >= 700 && std::min(m, n) > 32 && CeilDivide(m, 128) * CeilDivide(n, 128) <= 256) {
     struct Option { Tile tile; size_t per_cu; double rate, k0; };
     const Option options[] = {{Tile{0, 128, 128}, 2, 70.6, 43.0}, {Tile{1, 64, 64}, 3, 70.6, 91.0}, {Tile{5, 64, 32}, 5, 67.9, 81.0},
                               {Tile{6, 32, 32}, 8, 61.0, 101.0}};
@@ -434,7 +436,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       const auto rate = option.rate * ((a_kcontig && b_kcontig) ? 0.936 : 1.0);
       for (size_t ranges = 1; ranges <= 16; ranges *= 2) {
         const auto range = CeilDivide(CeilDivide(k, ranges), 64) * 64;
-        if (ranges > 1 && range < 512) { break; }
+        if (ranges > 1 && range < 256) { break; }
         const auto launched = CeilDivide(k, range);
         auto time = LaunchCost(TileCandidate{option.tile, option.per_cu, rate}, m, n, 0.178, launched) *
                     (static_cast<double>(range) + option.k0) * 512e-6;
