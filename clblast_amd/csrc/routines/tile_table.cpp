@@ -288,14 +288,15 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     // 4 us and 0.4 us per MB of partial sums for the reduction. 1024^2 x 8192 on 128 x 128 tiles in four ranges: 41.7 ->
     // 34.5 us (64 x 64 in two ranges before), 768^2 x 16384 T/N 56.9 -> 52.8 us; 512^2 x 8192 (64 x 64, eight ranges) and
     // 2048^2 x 8192 (128 x 128, unsplit) keep what they had.
-    if (batch_count == 1 && k >= 2048 && CeilDivide(m, 128) * CeilDivide(n, 128) < 512) {
+    // (from k = 1024 on, ranges from 256: 204 x 612 x 1804 16 -> 12 us, 930 x 178 x 1654 15 -> 12 us)
+    if (batch_count == 1 && k >= 1024 && CeilDivide(m, 128) * CeilDivide(n, 128) < 512) {
       struct Option { int tile; size_t extent, per_cu; double rate, k0; };
       const Option options[] = {{0, 128, 2, 936.0, 293.0}, {1, 64, 4, 488.0, 44.0}, {2, 256, 1, 1484.0, 627.0}};
       auto lowest = 1e300;
       for (const auto& option : options) {
         for (size_t ranges = 1; ranges <= 16; ranges *= 2) {
           const auto range = CeilDivide(CeilDivide(k, ranges), 64) * 64;
-          if (ranges > 1 && range < 512) { break; }
+          if (ranges > 1 && range < 256) { break; }
           const auto launched = CeilDivide(k, range);
           const auto slow = option.tile == 1 && range >= 4096 && CeilDivide(m, 128) * CeilDivide(n, 128) * launched >= 256;
           auto time = LaunchCost(TileCandidate{Tile{0, option.extent, option.extent}, option.per_cu, slow ? 371.0 : option.rate}, m, n, 0.25, launched) *
