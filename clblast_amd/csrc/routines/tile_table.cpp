@@ -240,10 +240,36 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       // From about 6000 rows on the 128 x 64 tile of the 16x16x4 MFMA (two work-groups per CU) beats 128 x 128 and
       // 256 x 128 (SYRK n = k = 8192: 4.65 -> 4.08 ms, 6144: 2.09 -> 1.81 ms); below, the largest tile that still leaves
       // four rounds of working tiles for the 256 CUs.
-      if (working(128, 64) >= 2048) { return KernelChoice{CLBH_KERNEL_MFMA, 11, 1}; }
-      if (working(256, 128) >= 4 * 256) { return KernelChoice{CLBH_KERNEL_MFMA, 3, 1}; }
-      if (working(128, 128) >= 4 * 256) { return KernelChoice{CLBH_KERNEL_MFMA, 0, 1}; }
-      return KernelChoice{CLBH_KERNEL_MFMA, 7, 1};
+      // That rule's choices lost 30 % on average against the best forced tile on 24 random SYRK shapes (up to 1.7 times:
+      // n = 1106, k = 4092 141 us on the 64 x 64 tile of the 32x32x2 instruction, 83 us on 64 x 32 tiles). Now the cost
+      // estimate of the GEMM table - the tiles that touch the triangle of a square C, or all tiles and half of k for a
+      // triangular operand - with the rates the tiles reach on SYRK (0.76 to 0.93 of their GEMM rates): 1.7 % on the
+      // same shapes.
+      const bool square = (m == n);
+      const auto touching = [&](const size_t tile_m, const size_t tile_n) {
+        if (!square) { return CeilDivide(m, tile_m) * CeilDivide(n, tile_n) * batch_count; }
+        size_t count = 0;  // lower triangle: tile column j holds the tile rows from (j * tile_n) / tile_m on
+        for (size_t j = 0; j < CeilDivide(n, tile_n); ++j) { count += CeilDivide(m, tile_m) - (j * tile_n) / tile_m; }
+        return count * batch_count;
+      };
+      const auto depth = static_cast<double>(square ? k : (k + 1) / 2);
+      struct Option { int index; size_t tile_m, tile_n, per_cu; double rate, k0; };
+      const Option options[] = {{3, 256, 128, 1, 0.762 * 150.0, 150.0}, {0, 128, 128, 2, 0.843 * 153.7, 136.0}, {11, 128, 64, 2, 0.863 * 137.6, 96.0},
+                                {12, 64, 64, 4, 0.870 * 140.0, 85.0}, {9, 64, 32, 4, 0.926 * 122.6, 110.0}};
+      auto lowest = 1e300;
+      int chosen = 12;
+      for (const auto& option : options) {
+        const auto count = touching(option.tile_m, option.tile_n);
+        const auto slots = 256 * option.per_cu;
+        auto rounds = static_cast<double>((count / slots) * option.per_cu);
+        if (count % slots != 0) {
+          const auto together = static_cast<double>(CeilDivide(count % slots, 256));
+          rounds += together / std::pow(together / static_cast<double>(option.per_cu), 0.226);
+        }
+        const auto time = rounds * static_cast<double>(option.tile_m * option.tile_n) * (depth + option.k0) / option.rate;
+        if (time < lowest) { lowest = time; chosen = option.index; }
+      }
+      return KernelChoice{CLBH_KERNEL_MFMA, chosen, 1};
     }
     return KernelChoice{CLBH_KERNEL_MFMA, (working(128, 128) >= 4 * 256) ? 0 : 1, 1};
   }
