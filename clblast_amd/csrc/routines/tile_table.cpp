@@ -134,7 +134,7 @@ double LaunchCost(const TileCandidate& candidate, const size_t m, const size_t n
 
 KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const bool b_kcontig, const size_t m,
                           const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,
-                          const size_t min_indirect_size, const bool triangular, const bool beta_zero,
+                          const size_t min_indirect_size, const int triangular, const bool beta_zero,
                           const size_t largest_ld) {
   (void)per_batch_scalars;
   // Many small matrices: one wavefront per matrix, bandwidth bound (that kernel knows no triangles)
@@ -242,10 +242,17 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       // four rounds of working tiles for the 256 CUs.
       // That rule's choices lost 30 % on average against the best forced tile on 24 random SYRK shapes (up to 1.7 times:
       // n = 1106, k = 4092 141 us on the 64 x 64 tile of the 32x32x2 instruction, 83 us on 64 x 32 tiles). Now the cost
-      // estimate of the GEMM table - the tiles that touch the triangle of a square C, or all tiles and half of k for a
-      // triangular operand - with the rates the tiles reach on SYRK (0.76 to 0.93 of their GEMM rates): 1.7 % on the
+      // estimate of the GEMM table over the tiles that touch the triangle of C, with the rates the tiles reach on SYRK (0.76 to 0.93 of their GEMM rates): 1.7 % on the
       // same shapes.
-      const bool square = (m == n);
+      // A triangular operand (TRMM, the products inside TRSM) keeps the rule above: its tiles walk K ranges of very
+      // different lengths, which the estimate does not see (STRMM 4096^2: 0.64 ms by the rule, 0.68 ms by the estimate).
+      if (triangular == 2) {
+        if (working(128, 64) >= 2048) { return KernelChoice{CLBH_KERNEL_MFMA, 11, 1}; }
+        if (working(256, 128) >= 4 * 256) { return KernelChoice{CLBH_KERNEL_MFMA, 3, 1}; }
+        if (working(128, 128) >= 4 * 256) { return KernelChoice{CLBH_KERNEL_MFMA, 0, 1}; }
+        return KernelChoice{CLBH_KERNEL_MFMA, 7, 1};
+      }
+      const bool square = true;
       const auto touching = [&](const size_t tile_m, const size_t tile_n) {
         if (!square) { return CeilDivide(m, tile_m) * CeilDivide(n, tile_n) * batch_count; }
         size_t count = 0;  // lower triangle: tile column j holds the tile rows from (j * tile_n) / tile_m on
@@ -267,6 +274,43 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
           rounds += together / std::pow(together / static_cast<double>(option.per_cu), 0.226);
         }
         const auto time = rounds * static_cast<double>(option.tile_m * option.tile_n) * (depth + option.k0) / option.rate;
+        if (time < lowest) { lowest = time; chosen = option.index; }
+      }
+      return KernelChoice{CLBH_KERNEL_MFMA, chosen, 1};
+    }
+    if (precision == Precision::kDouble) {
+      // fp64: the same estimate (the rule before it - 128 x 128 with four rounds of working tiles, else 64 x 64 - lost 55 %
+      // on average against the best forced tile on 24 random SYRK shapes, up to 3 times: n = 473, k = 3907 184 us on
+      // 64 x 64 tiles, 61 us on 32 x 32). Rates on SYRK: 128 x 128 x 8 73 TFLOP/s with k0 = 149, 64 x 64 67 and 84, 64 x 32
+      // 64 and 74, 32 x 32 57 and 121; two k-contiguous operands 0.86 to 0.93 of that, and no 128 x 128 x 8 tiles then
+      // (n = 3756, k = 4935: 1900 us on them, 1252 us on 64 x 32).
+      // (a triangular operand keeps the rule of old, as in the fp32 table: DTRMM 4096^2 1.31 against 1.45 ms)
+      if (triangular == 2) { return KernelChoice{CLBH_KERNEL_MFMA, (working(128, 128) >= 4 * 256) ? 0 : 1, 1}; }
+      const bool square = true;
+      const auto touching = [&](const size_t tile_m, const size_t tile_n) {
+        if (!square) { return CeilDivide(m, tile_m) * CeilDivide(n, tile_n) * batch_count; }
+        size_t count = 0;
+        for (size_t j = 0; j < CeilDivide(n, tile_n); ++j) { count += CeilDivide(m, tile_m) - (j * tile_n) / tile_m; }
+        return count * batch_count;
+      };
+      const auto depth = static_cast<double>(square ? k : (k + 1) / 2);
+      const bool both_kcontig = a_kcontig && b_kcontig;
+      struct Option { int index; size_t tile_m, tile_n, per_cu; double rate, k0, both; };
+      const Option options[] = {{0, 128, 128, 2, 73.2, 149.0, 0.925}, {1, 64, 64, 3, 66.7, 84.0, 0.862}, {5, 64, 32, 5, 64.0, 74.0, 0.903},
+                                {6, 32, 32, 8, 57.2, 121.0, 0.870}};
+      auto lowest = 1e300;
+      int chosen = 1;
+      for (const auto& option : options) {
+        if (both_kcontig && option.index == 0) { continue; }
+        const auto count = touching(option.tile_m, option.tile_n);
+        const auto slots = 256 * option.per_cu;
+        auto rounds = static_cast<double>((count / slots) * option.per_cu);
+        if (count % slots != 0) {
+          const auto together = static_cast<double>(CeilDivide(count % slots, 256));
+          rounds += together / std::pow(together / static_cast<double>(option.per_cu), 0.178);
+        }
+        const auto time = rounds * static_cast<double>(option.tile_m * option.tile_n) * (depth + option.k0) /
+                          (option.rate * (both_kcontig ? option.both : 1.0));
         if (time < lowest) { lowest = time; chosen = option.index; }
       }
       return KernelChoice{CLBH_KERNEL_MFMA, chosen, 1};
@@ -390,7 +434,9 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       tile = Tile{9, 64, 32};
       // ... or 32 x 64 where that pads the matrix less (455 x 3908 x 5312: 211 -> 195 us, 128 x 2603 x 708: 16 -> 14 us)
       const auto padded = [&](const size_t tile_m, const size_t tile_n) { return CeilDivide(m, tile_m) * tile_m * CeilDivide(n, tile_n) * tile_n; };
-      if (batch_count == 1 && (padded(32, 64) < padded(64, 32) || (padded(32, 64) == padded(64, 32) && n > m))) { tile = Tile{8, 32, 64}; }
+      // (on equal padding the tile whose longer side runs along an operand that is contiguous in it: 576^2 x 1255 T/T 23 -> 20 us
+      // on 32 x 64, 512 x 4096 x 512 N/N 25.3 -> 23.6 us on 64 x 32)
+      if (batch_count == 1 && (padded(32, 64) < padded(64, 32) || (padded(32, 64) == padded(64, 32) && a_kcontig && !b_kcontig))) { tile = Tile{8, 32, 64}; }
     }
     // Large single products with a long k: the four tiles that matter there by a cost estimate. A tile's work-groups
     // run in rounds (256 x 128: one per CU, 128 x 128 and 128 x 64: two, 64 x 64: four); a whole round costs the tile area
@@ -446,7 +492,8 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   // that leave CUs idle 64 x 32 x 16 (index 5, up to 256 tiles of 64 x 64 in a batch, 420 otherwise) and 32 x 32 x 32 (index 6, up to 144 such
   // tiles and a short k: 512^3 22.7 -> 10.4 us)
   // Single products with a long k and at most one round of 128 x 128 tiles: tile and number of K ranges together, as in
-  // the fp32 table (128 x 128 x 8: 70.6 TFLOP/s and k0 = 43, two per CU; 64 x 64: 70.6 and 91, three; 64 x 32: 67.9 and 81,
+  // the fp32 table (128 x 128 x 8: 70.6 TFLOP/s and k0 = 150 - the random shapes of the fit do not pin it, 1024 x 4096 x 1024
+  // in one range and in two does -, two per CU; 64 x 64: 70.6 and 91, three; 64 x 32: 67.9 and 81,
   // five; 32 x 32: 61 and 101, eight; two k-contiguous operands 0.94 of the rate; a partly empty round at (c / p)^0.18;
   // the reduction 3.3 us and 0.6 us per range). Fitted to 360 timings (24 shapes, four tiles, four splits): the choice
   // loses 3 % on average against the best of them, the rules it replaces 13 % - 384 x 2048 x 11674 415 -> 289 us,
@@ -455,7 +502,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   // pair, the rules it replaces 9 % - 128 x 2944 x 1761 T/N 48 -> 35 us, 256 x 1088 x 1158 31 -> 25 us)
   if (batch_count == 1 && k >= 700 && std::min(m, n) > 32 && CeilDivide(m, 128) * CeilDivide(n, 128) <= 256) {
     struct Option { Tile tile; size_t per_cu; double rate, k0; };
-    const Option options[] = {{Tile{0, 128, 128}, 2, 70.6, 43.0}, {Tile{1, 64, 64}, 3, 70.6, 91.0}, {Tile{5, 64, 32}, 5, 67.9, 81.0},
+    const Option options[] = {{Tile{0, 128, 128}, 2, 70.6, 150.0}, {Tile{1, 64, 64}, 3, 70.6, 91.0}, {Tile{5, 64, 32}, 5, 67.9, 81.0},
                               {Tile{6, 32, 32}, 8, 61.0, 101.0}};
     auto lowest = 1e300;
     auto chosen = KernelChoice{CLBH_KERNEL_MFMA, 1, 1};

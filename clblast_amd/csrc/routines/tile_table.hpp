@@ -32,12 +32,13 @@ size_t MinIndirectSize(const int device, const Precision precision);
 bool UseDirectKernel(const size_t m, const size_t n, const size_t k, const size_t min_indirect_size);
 
 // Picks the kernel family and tile for a canonical problem (m, n, k per matrix). `triangular`: about half of the
-// tile work of the launch is skipped (a triangle of C, or a triangular operand), which calls for smaller tiles.
+// tile work of the launch is skipped (1: only a triangle of C is computed, 2: a triangular operand whose zero half of K is
+// skipped), which calls for smaller tiles.
 // `beta_zero`: the old C is not read. `largest_ld`: the largest leading dimension of A, B and C. (Neither of the two ever
 // makes a problem need more workspace than it needs with the default values.)
 KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const bool b_kcontig, const size_t m,
                           const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,
-                          const size_t min_indirect_size, const bool triangular = false, const bool beta_zero = false,
+                          const size_t min_indirect_size, const int triangular = 0, const bool beta_zero = false,
                           const size_t largest_ld = 0);
 
 // Tile forced for a precision through OverrideParameters("Xgemm", {"TILE_VARIANT": 1 + index}); 0 = automatic.

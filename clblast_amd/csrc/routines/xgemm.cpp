@@ -130,7 +130,8 @@ void Xgemm<T>::DoGemm(const Layout layout, const Transpose a_transpose, const Tr
 
   auto desc = Canonicalise(shape, layout, m, n, k, a_buffer(), a_offset, a_ld, b_buffer(), b_offset, b_ld,
                            const_cast<void*>(c_buffer()), c_offset, c_ld);
-  const bool triangular = (triangles.output != OutputTriangle::kFull || triangles.operand != OperandTriangle::kNone);
+  // (1: only a triangle of C is computed, 2: an operand is triangular and its zero half of K is skipped)
+  const int triangular = (triangles.output != OutputTriangle::kFull) ? 1 : (triangles.operand != OperandTriangle::kNone) ? 2 : 0;
   const auto choice = SelectKernel(PrecisionValue<T>(), desc.a_kcontig != 0, desc.b_kcontig != 0,
                                    static_cast<size_t>(desc.m), static_cast<size_t>(desc.n), k, 1, false,
                                    min_indirect_size(), triangular, ScalarToDouble(beta) == 0.0, std::max({a_ld, b_ld, c_ld}));
