@@ -84,7 +84,7 @@ def raw_gemm(prefix, layout, a_transpose, b_transpose, m, n, k, alpha, a_ptr, a_
 def raw_sgemm_no_alloc(layout, a_transpose, b_transpose, m, n, k, alpha, a_ptr, a_offset, a_ld, b_ptr, b_offset, b_ld, beta,
                        c_ptr, c_offset, c_ld, stream_handle=0, event_handle=None):
     """CLBlastSgemmNoAlloc through the C ABI: CLBlastSgemm's arguments; the library allocates nothing (its split-K
-    workspace is a static device array of 8 MiB per GPU; larger needs return -2050)."""
+    workspace is a static device array of 64 MiB per GPU; larger needs return -2050)."""
     event_ref = None if event_handle is None else ctypes.byref(ctypes.c_void_p(event_handle))
     return _lib.load().CLBlastSgemmNoAlloc(layout, a_transpose, b_transpose, m, n, k, _scalar("S", alpha), a_ptr, a_offset,
                                            a_ld, b_ptr, b_offset, b_ld, _scalar("S", beta), c_ptr, c_offset, c_ld,

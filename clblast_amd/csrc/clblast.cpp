@@ -5,6 +5,7 @@
 // :1630-1647 (GemmStridedBatched), :1682-1708 (GemmTempBufferSize) and src/api_common.cpp:25-33,
 // 140-221 (ClearCache, RetrieveParameters, OverrideParameters).
 // =================================================================================================
+#include <algorithm>
 #include <string>
 #include <vector>
 
@@ -218,14 +219,16 @@ StatusCode GemmTempBufferSize(const Layout layout, const Transpose a_transpose, 
                               const size_t b_offset, const size_t b_ld, const size_t c_offset, const size_t c_ld,
                               hipStream_t* queue, size_t& temp_buffer_size) {
   try {
-    (void)a_offset; (void)a_ld; (void)b_offset; (void)b_ld; (void)c_offset; (void)c_ld;  // operands are read in place
+    (void)a_offset; (void)b_offset; (void)c_offset;  // operands are read in place
     if (queue == nullptr) {
       throw RuntimeErrorCode(StatusCode::kInvalidCommandQueue, "queue is a null pointer");
     }
     auto device = 0;
     CheckDevice(clbh_stream_device(*queue, &device), "clbh_stream_device");
+    // (the leading dimensions only matter through their maximum: beyond 2^20 elements some kernels are not available
+    // and the one that runs instead may split K)
     temp_buffer_size = Xgemm<T>::TempBytes(layout, a_transpose, b_transpose, m, n, k,
-                                           MinIndirectSize(device, PrecisionValue<T>()));
+                                           MinIndirectSize(device, PrecisionValue<T>()), std::max({a_ld, b_ld, c_ld}));
     return StatusCode::kSuccess;
   } catch (...) {
     return DispatchException();

@@ -13,7 +13,7 @@
 
 namespace {
 
-constexpr size_t kStaticScratchBytes = size_t{8} << 20;
+constexpr size_t kStaticScratchBytes = size_t{64} << 20;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 // In host code `scratch` is a stand-in for the symbol, not an address: the address of each GPU's copy is asked for

@@ -100,13 +100,14 @@ clbh_gemm_desc Xgemm<T>::Canonicalise(const GemmShape& shape, const Layout layou
 
 template <typename T>
 size_t Xgemm<T>::TempBytes(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
-                           const size_t m, const size_t n, const size_t k, const size_t min_indirect_size) {
+                           const size_t m, const size_t n, const size_t k, const size_t min_indirect_size,
+                           const size_t largest_ld) {
   const auto shape = ProcessArguments(layout, a_transpose, b_transpose, m, n, k);
   auto desc = Canonicalise(shape, layout, m, n, k, nullptr, 0, shape.a_one, nullptr, 0, shape.b_one, nullptr, 0,
                            shape.c_one);
   const auto choice = SelectKernel(PrecisionValue<T>(), desc.a_kcontig != 0, desc.b_kcontig != 0,
                                    static_cast<size_t>(desc.m), static_cast<size_t>(desc.n), k, 1, false,
-                                   min_indirect_size);
+                                   min_indirect_size, 0, false, std::max({largest_ld, shape.a_one, shape.b_one, shape.c_one}));
   desc.kernel_class = choice.kernel_class;
   desc.tile_variant = choice.tile_variant;
   desc.split_k = choice.split_k;

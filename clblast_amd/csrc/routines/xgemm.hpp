@@ -69,9 +69,11 @@ class Xgemm : public GemmRoutineBase {
                                      const void* b, const size_t b_offset, const size_t b_ld, void* c,
                                      const size_t c_offset, const size_t c_ld);
 
-  // Bytes of temporary device memory the engine wants for this problem (split-K partial sums; usually 0)
+  // Bytes of temporary device memory the engine wants for this problem (split-K partial sums; usually 0). `largest_ld`:
+  // the largest leading dimension of the call, which decides between some kernels as it does in DoGemm.
   static size_t TempBytes(const Layout layout, const Transpose a_transpose, const Transpose b_transpose,
-                          const size_t m, const size_t n, const size_t k, const size_t min_indirect_size);
+                          const size_t m, const size_t n, const size_t k, const size_t min_indirect_size,
+                          const size_t largest_ld = 0);
 
   Xgemm(hipStream_t* queue, hipEvent_t* event);
 

@@ -123,7 +123,7 @@ StatusCode Gemm(const Layout layout, const Transpose a_transpose, const Transpos
                 hipEvent_t* event = nullptr, void* temp_buffer = nullptr);
 
 // Gemm<float> for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
-// harnesses that forbid hipMalloc): the split-K workspace is a static array of 8 MiB that every GPU holds; problems
+// harnesses that forbid hipMalloc): the split-K workspace is a static array of 64 MiB that every GPU holds; problems
 // that would need more return kInsufficientMemoryTemp. Calls that overlap on one GPU share the array and race.
 StatusCode GemmNoAlloc(const Layout layout, const Transpose a_transpose, const Transpose b_transpose, const size_t m,
                        const size_t n, const size_t k, const float alpha, const void* a_buffer, const size_t a_offset,

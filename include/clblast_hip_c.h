@@ -468,7 +468,7 @@ CLBlastStatusCode CLBLAST_HIP_API CLBlastZGemmTempBufferSize(
 // =================================================================================================
 // SGEMM that allocates nothing. No counterpart in the reference: it is for callers that cannot allocate device memory
 // (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). Same arguments and results as
-// CLBlastSgemm; the split-K workspace is a static device array of 8 MiB per GPU instead of stream scratch, and a problem
+// CLBlastSgemm; the split-K workspace is a static device array of 64 MiB per GPU instead of stream scratch, and a problem
 // that would need more returns CLBlastInsufficientMemoryTemp (-2050) with a message on stderr. All calls on one GPU
 // share that array: calls that overlap on one GPU (different streams) race.
 CLBlastStatusCode CLBLAST_HIP_API CLBlastSgemmNoAlloc(

@@ -44,13 +44,13 @@ def test_workspace_beyond_the_static_array_is_refused(gpu):
                                                 gpu.stream_handle())
     assert lib_status == -1017
     found = None
-    for m, n, k in ((768, 768, 65536), (1024, 512, 131072), (512, 512, 262144)):
+    for m, n, k in ((2048, 2048, 65536), (1536, 1536, 131072), (1024, 1024, 262144)):
         needed = clblast_amd.raw_gemm_temp_buffer_size("S", COL_MAJOR, NO, YES, m, n, k, 0, m, 0, n, 0, m, gpu.stream_handle())
-        if needed[0] == 0 and needed[1] > (8 << 20):
+        if needed[0] == 0 and needed[1] > (64 << 20):
             found = (m, n, k)
             break
     if found is None:
-        pytest.skip("no probed shape wants more than 8 MiB of workspace")
+        pytest.skip("no probed shape wants more than 64 MiB of workspace")
     m, n, k = found
     a = torch.zeros(m * k, dtype=torch.float32, device="cuda")
     b = torch.zeros(n * k, dtype=torch.float32, device="cuda")
