@@ -514,6 +514,15 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   // fp64 (same sweep): 64 x 64 x 16 tiles (index 1) up to about 3072^3, 128 x 128 x 8 (index 0) beyond; for launches
   // that leave CUs idle 64 x 32 x 16 (index 5, up to 256 tiles of 64 x 64 in a batch, 420 otherwise) and 32 x 32 x 32 (index 6, up to 144 such
   // tiles and a short k: 512^3 22.7 -> 10.4 us)
+  // One whole round of 128 x 64 x 16 tiles (two per CU, 460 to 512 of them) that the matrix fills: that tile - 2048^3 301 ->
+  // 250 us, 1024 x 4096 x 2048 300 -> 246 us, 2048^2 x 1024 140 -> 131 us against the estimate below, which has no term
+  // for a round that comes out even. (With 936 of them, not quite two rounds, it is the slowest of the tiles.)
+  {
+    const auto pairs = CeilDivide(m, 128) * CeilDivide(n, 64);
+    if (batch_count == 1 && k >= 1024 && pairs >= 460 && pairs <= 512 && TileUse(m, n, 128, 64) >= 95) {
+      return KernelChoice{CLBH_KERNEL_MFMA, 2, 1};
+    }
+  }
   // Single products with a long k and at most one round of 128 x 128 tiles: tile and number of K ranges together, as in
   // the fp32 table (128 x 128 x 8: 70.6 TFLOP/s and k0 = 150 - the random shapes of the fit do not pin it, 1024 x 4096 x 1024
   // in one range and in two does -, two per CU; 64 x 64: 70.6 and 91, three; 64 x 32: 67.9 and 81,
