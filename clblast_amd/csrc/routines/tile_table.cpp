@@ -483,18 +483,20 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     auto split = (batch_count == 1) ? SplitFor(tiles, k, tile.index >= 8 && tile.index != 12) : 1;
     // Single products with k from 700 on and at most one round of 128 x 128 tiles (more than 32 rows and columns): tile and
     // number of K ranges together, by an estimate in microseconds - the launch of tiles x ranges work-groups on ranges of
-    // k / ranges (rounded up to 64, at least 256), each tile costing k0 more than its range (128 x 128: 154 TFLOP/s and
-    // k0 = 136, 128 x 64: 138 and 96, 64 x 64: 140 and 85, 64 x 32 and 32 x 64: 123 and 110, 32 x 32: 97 and 188; two
-    // k-contiguous operands: 0.99 of the rate on the first two, 0.92 on the others; a partly empty round at (c / p)^0.23),
-    // plus, for the reduction, 1.3 us, 0.3 us per range and 0.14 us per MB of partial sums. Fitted to 2300 timings (162
-    // shapes - mid-sized with a long k, with 700 <= k < 2048, skinny - on up to six tiles and four splits each); the
-    // choice loses 2 % on average against the best of them, the rules it replaces 8-10 %: 1024^2 x 8192 T/N 176 -> 137 us,
+    // k / ranges (rounded up to 64, at least 256), each tile costing k0 more than its range (128 x 128: 138 TFLOP/s and
+    // k0 = 136, 128 x 64: 138 and 106, 64 x 64: 133 and 77, 64 x 32 and 32 x 64: 123 and 99, 32 x 32: 105 and 188; two
+    // k-contiguous operands: 0.94 of the rate on the first two, 0.92 on the others; a partly empty round at (c / p)^0.23),
+    // plus, for the reduction, 1.4 us, 0.3 us per range and 0.14 us per MB of partial sums. Fitted by least squares to 2300
+    // timings (162 random shapes - mid-sized with a long k, with 700 <= k < 2048, skinny - on up to six tiles and four
+    // splits each), then adjusted coordinate by coordinate for the loss of the choice itself on those and on 60 shapes of
+    // powers of two and their multiples; the choice loses 1.4 % (powers of two) and 1.8 % (random) on average against the
+    // best of them, the rules it replaces 8-10 %: 1024^2 x 8192 T/N 176 -> 137 us,
     // 1536^2 x 4096 180 -> 161 us, 1024^2 x 4096 T/N 91 -> 76 us, 13311 x 58 x 5185 125 -> 110 us, 205 x 613 x 1804 22 -> 18 us.
     if (batch_count == 1 && k >= 700 && std::min(m, n) > 32 && CeilDivide(m, 128) * CeilDivide(n, 128) <= 256) {
       struct Option { Tile tile; size_t per_cu; double rate, k0, both_kcontig; };
-      const Option options[] = {{Tile{0, 128, 128}, 2, 153.7, 136.0, 0.992}, {Tile{11, 128, 64}, 2, 137.6, 96.0, 0.992},
-                                {Tile{12, 64, 64}, 4, 140.0, 85.0, 0.916}, {Tile{9, 64, 32}, 4, 122.6, 110.0, 0.916},
-                                {Tile{8, 32, 64}, 4, 122.6, 110.0, 0.916}, {Tile{10, 32, 32}, 8, 97.2, 188.0, 0.916}};
+      const Option options[] = {{Tile{0, 128, 128}, 2, 138.3, 136.0, 0.942}, {Tile{11, 128, 64}, 2, 137.6, 106.0, 0.942},
+                                {Tile{12, 64, 64}, 4, 133.0, 76.5, 0.916}, {Tile{9, 64, 32}, 4, 122.6, 99.0, 0.916},
+                                {Tile{8, 32, 64}, 4, 122.6, 99.0, 0.916}, {Tile{10, 32, 32}, 8, 105.0, 188.0, 0.916}};
       auto lowest = 1e300;
       for (const auto& option : options) {
         const auto rate = option.rate * ((a_kcontig && b_kcontig) ? option.both_kcontig : 1.0);
@@ -504,7 +506,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
           const auto launched = CeilDivide(k, range);
           auto time = LaunchCost(TileCandidate{option.tile, option.per_cu, rate}, m, n, 0.226, launched) *
                       (static_cast<double>(range) + option.k0) * 512e-6;
-          if (launched > 1) { time += 1.3 + 0.3 * static_cast<double>(launched) + 0.135 * 4e-6 * static_cast<double>(m * n * launched); }
+          if (launched > 1) { time += 1.37 + 0.27 * static_cast<double>(launched) + 0.135 * 4e-6 * static_cast<double>(m * n * launched); }
           if (time < lowest) { lowest = time; tile = option.tile; split = static_cast<int>(launched); }
         }
       }
