@@ -42,6 +42,7 @@ MEASURED_TRAFFIC = {
     "cfg5d": (6.225e8, "profiles/sgemm_8191x8191x127_colNN.md", "clbh::GemmStreamKernel<float, clbh::MfmaConfig<float, 1, 4, 4, 1, 16, 2"),
     "cfg5e": (7.371e7, "profiles/sgemm_4099x17x4096_colTN.md", "clbh::GemmSkinnyRowsKernel<4, 5, 5, 2, true, true, 2>"),
     "sbat64": (2.036e8, "profiles/sgemm_strided_batched_4096x64.md", "clbh::GemmStreamKernel<float, clbh::MfmaConfig<float, 1, 4, 4, 1, 16, 4"),
+    "hbat_short_k": (2.939e8, "profiles/hgemm_strided_batched_8x4096x4096x64.md", "clbh::HgemmDirectKernel<clbh::HdirectConfig<2, 2, 2, 2, 3"),
     "cgemm_batched": (4.028e8, "profiles/cgemm_strided_batched_4096x64_rowNC.md", "clbh::GemmComplexSmallKernel<float, 2, true, true>"),
 }
 
@@ -577,6 +578,7 @@ EXTRA_WORKLOADS = {
     "next_sgemm_strided_batched_4096x64": lambda: Workload("sbat64", "S", ROW, NO, NO, 64, 64, 64, 1.0, 0.0, batch=4096),
     "next_dgemm_strided_batched_2048x128x64x64": lambda: Workload("dbat128", "D", ROW, NO, YES, 128, 64, 64, 1.0, 0.0,
                                                                   batch=2048),
+    "next_hgemm_strided_batched_8x4096x4096x64": lambda: Workload("hbat_short_k", "H", COL, NO, YES, 4096, 4096, 64, 1.0, 0.0, batch=8),
     "next_cgemm_4096_rowNC": lambda: ComplexWorkload("cgemm", "C", NO, 113, 4096, 4096, 4096, 1.0 - 0.5j, 0.0),
     "next_zgemm_2048_rowTN": lambda: ComplexWorkload("zgemm", "Z", YES, NO, 2048, 2048, 2048, 0.5 + 1.0j, 1.0 - 0.5j),
     "next_cgemm_strided_batched_4096x64_rowNC": lambda: ComplexWorkload("cgemm_batched", "C", NO, 113, 64, 64, 64, 1.0 - 0.5j,

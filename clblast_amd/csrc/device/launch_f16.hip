@@ -157,6 +157,9 @@ int LaunchMfmaF16(const clbh_gemm_desc& d, hipStream_t stream) {
     case 2: return LaunchHdirectConfig<HdirectConfig<2, 4, 4, 2, 2>>(d, stream);  // 256 x 256, 8 wavefronts
     case 3: return LaunchHdirectConfig<HdirectConfig<4, 1, 1, 1, 4>>(d, stream);  // 128 x 32 (skinny n)
     case 4: return LaunchHdirectConfig<HdirectConfig<1, 4, 1, 1, 4>>(d, stream);  // 32 x 128 (skinny m)
+    // 128 x 128 held to 168 registers (a few of them spilled), three work-groups per CU: for short k, where the
+    // work-groups mostly wait - for their first slabs and for their stores - and a third one fills the gaps
+    case 5: return LaunchHdirectConfig<HdirectConfig<2, 2, 2, 2, 3>>(d, stream);
     default: return LaunchHdirectConfig<HdirectConfig<2, 2, 2, 2, 2>>(d, stream);  // 128 x 128, 4 wavefronts
   }
 }

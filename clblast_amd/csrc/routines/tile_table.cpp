@@ -342,7 +342,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   }
   if (precision == Precision::kHalf) {
     // Direct-load tiles, 0: 128 x 128, 1: 64 x 64, 2: 256 x 256 (8 wavefronts), 3: 128 x 32, 4: 32 x 128 (the last two
-    // lose to 64 x 64 on skinny shapes too). The tile is chosen by the cost estimate of LaunchCost - rounds of
+    // lose to 64 x 64 on skinny shapes too), 5: 128 x 128 with three work-groups per CU. The tile is chosen by the cost estimate of LaunchCost - rounds of
     // work-groups (256 x 256: one per CU, 128 x 128: two, 64 x 64: four), a partly empty last round at (c / p)^0.25 of
     // the rate - times k + k0 over the tile's rate: a tile costs what k0 more slabs would, its prologue and epilogue
     // (256 x 256: 1480 TFLOP/s and k0 = 630, 128 x 128: 940 and 290, 64 x 64: 490 and 40). Padded tiles count in full, so
@@ -366,6 +366,18 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     int tile = 1;
     if (cost256 <= cost128 && cost256 <= cost64) { tile = 2; }
     else if (cost128 <= cost64) { tile = 0; }
+    // A short k with many tiles is a stream over C, and latency decides it: a work-group waits for its first slabs,
+    // walks the few there are and waits for its stores. The estimate above, fitted to longer walks, takes the 64 x 64
+    // tiles there, which fetch the operand tiles twice as often; the 128 x 128 tiles are faster up to k = 128 (4096^2 x 64
+    // 18 -> 15 us, 8 x 4096^2 x 64 100 -> 83 us), and from 2048 tiles on, up to k = 320, three work-groups of them per CU
+    // (index 5: the same kernel held to 168 registers) hide more of each other's waits than two (8192^2 x 128: 48 ->
+    // 41 us, 96 x 2048^2 x 128 N/T 350 -> 292 us, 8 x 4096^2 x 64 83 -> 67 us; at 1024 tiles and at k = 512 no gain)
+    {
+      const auto tiles128 = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
+      const bool fills = 10 * TileUse(m, n, 128, 128) >= 9 * TileUse(m, n, 64, 64);
+      if (k <= 320 && tiles128 >= 2048 && fills) { tile = 5; }
+      else if (k <= 128 && tiles128 >= 512 && fills) { tile = 0; }
+    }
     // K ranges (fp32 partial sums, then a reduction) when the 64 x 64 tiles would leave the GPU mostly idle through a
     // long K walk: up to 512 work-groups, ranges at least 512 deep - 2048 when there are 192 tiles or more, which by
     // themselves keep most CUs busy (measured: 256^2 x 8192 33.6 -> 13.4 us, 4099 x 17 x 4096 33.9 -> 14.1 us,

@@ -231,6 +231,15 @@ void XgemmStridedBatched<T>::DoGemmStridedBatched(
     align(desc.a, desc.a_offset, desc.a_ld, desc.a_stride, desc.a_kcontig != 0, desc.m, aligned_a);
     align(desc.b, desc.b_offset, desc.b_ld, desc.b_stride, desc.b_kcontig != 0, desc.n, aligned_b);
   }
+  // A batch of one matrix gets the tile table's choice for a single product, which may split a long k: the K ranges
+  // sum in stream-ordered scratch, as in Xgemm::DoGemm
+  const auto temp_bytes = clbh_gemm_workspace_bytes(&desc);
+  std::unique_ptr<StreamScratch> scratch;
+  if (temp_bytes > 0) {
+    scratch.reset(new StreamScratch(temp_bytes, stream(), "temporary buffer"));
+    desc.workspace = scratch->get();
+  }
+  desc.workspace_bytes = temp_bytes;
   CheckDevice(clbh_gemm_launch(&desc, stream()), "strided-batched GEMM launch");
   Finish();
 }

@@ -209,3 +209,20 @@ def test_random_batched_shapes_through_the_automatic_choice(gpu, bits):
         except AssertionError as failure:
             raise AssertionError("case %d: layout=%d ta=%d tb=%d m=%d n=%d k=%d batch=%d offsets=%s extra=%s alpha=%g beta=%g: %s" %
                                  (case, layout, ta, tb, m, n, k, batch, offsets, extra, alpha, beta, failure))
+
+
+@pytest.mark.parametrize("bits", [32, 64, 16])
+def test_a_batch_of_one_matrix_with_a_long_k(gpu, bits):
+    """A strided batch of one matrix gets the tile choice of a single product, which splits a long k into ranges
+    that sum in temporary memory: the strided-batched routine has to bring that memory along."""
+    for (m, n, k) in ((256, 192, 6144), (64, 64, 8192), (512, 512, 4096)):
+        run_strided(gpu, bits, COL_MAJOR, NO, YES, m, n, k, 1.0, 0.5, 1, seed=77 + m)
+        run_strided(gpu, bits, ROW_MAJOR, YES, NO, m, n, k, -0.5, 0.0, 1, seed=78 + m)
+
+
+def test_half_precision_short_k_with_thousands_of_tiles(gpu):
+    """From 2048 tiles of 128 x 128 on and up to k = 320 the fp16 tile table runs three work-groups per CU (a kernel
+    instance held to fewer registers): the automatic choice on such shapes, with edges in m and n, against the oracle."""
+    run_strided(gpu, 16, COL_MAJOR, NO, YES, 2040, 2048, 72, 1.0, 0.0, 8, seed=501)
+    run_strided(gpu, 16, COL_MAJOR, YES, NO, 2048, 2030, 300, -0.5, 0.75, 8, seed=502)
+    run_strided(gpu, 16, ROW_MAJOR, NO, NO, 5800, 5790, 64, 2.0, 1.0, 1, seed=503)
