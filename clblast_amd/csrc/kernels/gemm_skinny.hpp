@@ -18,7 +18,12 @@
 // for about 1 us), the epilogue 2.6 us. An x-contiguous X (a plain A) stays with the tiled kernel: there the lanes must
 // run along the rows of X, K has to be split over work-groups again, and the variant of this kernel built that way
 // (register streaming, wavefront-private LDS tiles of S, tree of partial sums) was no faster than the tiled one (25.9
-// against 25.6 us; its epilogue and the reduction launch took 10 us of that).
+// against 25.6 us; its epilogue and the reduction launch took 10 us of that). Nor does it help to give a work-group
+// a few such rows and all of K, which needs no second launch: with sixteen rows per work-group (runs of 64 bytes, half
+// a cache line) X streams at 3 TB/s (4099 x 17 x 4096: 46 us, 16384 x 4 x 16384: 345 against 176 us), with 32 rows
+// per work-group, the two halves of the lines fetched by two wavefronts side by side, at 3.5 TB/s (34 and 307 us) -
+// every load of a wavefront touches sixteen lines, one per k. Only below about 8 MB of X is that ahead (4099 x 17 x 512:
+// 9.8 against 11.0 us).
 // =================================================================================================
 #ifndef CLBLAST_HIP_KERNELS_GEMM_SKINNY_HPP_
 #define CLBLAST_HIP_KERNELS_GEMM_SKINNY_HPP_
