@@ -180,6 +180,14 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     // 199 x 79 x 571 x 3380 1439 -> 1165 us (the persistent kernel: 613 and 1536), fp64 251 x 98 x 373 x 1656 1011 -> 789 us.
     if (batched) {
       if (k >= 320 && tiles128 >= 2048 && use128 >= use64) { return KernelChoice{CLBH_KERNEL_MFMA, 0, 1}; }
+      // (k from 1024 on and matrices that the larger tiles fill: those tiles - fp32 128 x 64: 96 x 2048 x 128 x 2048 933 ->
+      // 822 us, 96 x 2048 x 64 x 1536 374 -> 318 us, 200 x 512 x 128 x 2048 503 -> 475 us; fp64 128 x 128: 96 x 2048 x 128 x 2048
+      // 1643 -> 1511 us, 64 x 1024 x 256 x 1280 683 -> 641 us, while with n = 64 the persistent kernel is level with the best)
+      if (k >= 1024 && precision == Precision::kSingle && TileUse(m, n, 128, 64) >= 95 &&
+          CeilDivide(m, 128) * CeilDivide(n, 64) * batch_count >= 1024) {
+        return KernelChoice{CLBH_KERNEL_MFMA, 11, 1};
+      }
+      if (k >= 1024 && precision == Precision::kDouble && use128 >= 95 && tiles128 >= 1024) { return KernelChoice{CLBH_KERNEL_MFMA, 0, 1}; }
       // (with k up to 512 whatever the padding: fp32 192 x 34 x 266 x 218 21 -> 18 us, fp64 33 x 160 x 96 x 555 44 -> 32 us)
       const bool fills = k <= 512 || use64 >= (precision == Precision::kSingle ? 60u : 68u);
       if (tiles64 >= 400 && k <= 2048 && fills) { return KernelChoice{CLBH_KERNEL_STREAM, 2, 1}; }

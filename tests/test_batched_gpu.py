@@ -226,3 +226,11 @@ def test_half_precision_short_k_with_thousands_of_tiles(gpu):
     run_strided(gpu, 16, COL_MAJOR, NO, YES, 2040, 2048, 72, 1.0, 0.0, 8, seed=501)
     run_strided(gpu, 16, COL_MAJOR, YES, NO, 2048, 2030, 300, -0.5, 0.75, 8, seed=502)
     run_strided(gpu, 16, ROW_MAJOR, NO, NO, 5800, 5790, 64, 2.0, 1.0, 1, seed=503)
+
+
+@pytest.mark.parametrize("bits,batch", [(32, 32), (64, 64)])
+def test_batches_with_a_long_k_that_the_large_tiles_fill(gpu, bits, batch):
+    """Batches with k >= 1024 whose matrices the 128 x 64 (fp32) or 128 x 128 (fp64) tiles fill, 1024 tiles or more of
+    them: the tile table takes those tiles in place of the persistent kernel."""
+    run_strided(gpu, bits, COL_MAJOR, NO, YES, 512, 512, 1024, 1.0, 0.5, batch, seed=880 + bits)
+    run_strided(gpu, bits, ROW_MAJOR, YES, NO, 512, 508, 1100, -0.5, 0.0, batch, seed=881 + bits)
