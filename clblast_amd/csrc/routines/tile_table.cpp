@@ -350,7 +350,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   }
   if (precision == Precision::kHalf) {
     // Direct-load tiles, 0: 128 x 128, 1: 64 x 64, 2: 256 x 256 (8 wavefronts), 3: 128 x 32, 4: 32 x 128 (the last two
-    // lose to 64 x 64 on skinny shapes too), 5: 128 x 128 with three work-groups per CU. The tile is chosen by the cost estimate of LaunchCost - rounds of
+    // lose to 64 x 64 on skinny shapes too), 5: 128 x 128 with three work-groups per CU, 6: 256 x 128 (4 wavefronts). The tile is chosen by the cost estimate of LaunchCost - rounds of
     // work-groups (256 x 256: one per CU, 128 x 128: two, 64 x 64: four), a partly empty last round at (c / p)^0.25 of
     // the rate - times k + k0 over the tile's rate: a tile costs what k0 more slabs would, its prologue and epilogue
     // (256 x 256: 1480 TFLOP/s and k0 = 630, 128 x 128: 940 and 290, 64 x 64: 490 and 40). Padded tiles count in full, so
@@ -385,6 +385,16 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       const bool fills = 10 * TileUse(m, n, 128, 128) >= 9 * TileUse(m, n, 64, 64);
       if (k <= 320 && tiles128 >= 2048 && fills) { tile = 5; }
       else if (k <= 128 && tiles128 >= 512 && fills) { tile = 0; }
+    }
+    // One column of tiles (64 <= n <= 128) under a long k and a tall A with contiguous columns: every tile streams its
+    // rows of A once, nothing of A is shared, and the 256 x 128 tile (index 6, four wavefronts of 128 x 64, two
+    // work-groups per CU) fetches B half as often per row of A as 128 x 128 does - from a full round of such tiles on
+    // (96 x 2048 x 128 x 2048 N/N 224 -> 193 us, N/T 203 -> 186 us, 16 x 8192 x 128 x 8192 N/N 485 -> 401 us, 96 x 2048 x 64 x 2048
+    // 180 -> 168 us; with a k-contiguous A it loses, 219 -> 239 us, and on square products it lies between 128 x 128 and
+    // 256 x 256: 4096^3 125 against 142 and 115 us)
+    if (!a_kcontig && n >= 64 && n <= 128 && k >= 1024 && CeilDivide(m, 256) * batch_count >= 512 &&
+        10 * m >= 9 * CeilDivide(m, 256) * 256) {
+      tile = 6;
     }
     // K ranges (fp32 partial sums, then a reduction) when the 64 x 64 tiles would leave the GPU mostly idle through a
     // long K walk: up to 512 work-groups, ranges at least 512 deep - 2048 when there are 192 tiles or more, which by

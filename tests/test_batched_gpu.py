@@ -234,3 +234,10 @@ def test_batches_with_a_long_k_that_the_large_tiles_fill(gpu, bits, batch):
     them: the tile table takes those tiles in place of the persistent kernel."""
     run_strided(gpu, bits, COL_MAJOR, NO, YES, 512, 512, 1024, 1.0, 0.5, batch, seed=880 + bits)
     run_strided(gpu, bits, ROW_MAJOR, YES, NO, 512, 508, 1100, -0.5, 0.0, batch, seed=881 + bits)
+
+
+def test_half_precision_tall_products_with_one_column_of_tiles(gpu):
+    """fp16 with 64 <= n <= 128, a long k, an A with contiguous columns and a full round of 256 x 128 tiles: the tile
+    table takes that tile (a kernel instance of its own); with an edge in m and in n."""
+    run_strided(gpu, 16, COL_MAJOR, NO, NO, 2040, 100, 1024, 1.0, 0.5, 64, seed=611)
+    run_strided(gpu, 16, COL_MAJOR, NO, YES, 2048, 128, 1056, -0.5, 0.0, 64, seed=612)
