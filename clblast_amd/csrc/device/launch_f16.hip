@@ -160,6 +160,7 @@ int LaunchMfmaF16(const clbh_gemm_desc& d, hipStream_t stream) {
     // 128 x 128 held to 168 registers (a few of them spilled), three work-groups per CU: for short k, where the
     // work-groups mostly wait - for their first slabs and for their stores - and a third one fills the gaps
     case 5: return LaunchHdirectConfig<HdirectConfig<2, 2, 2, 2, 3>>(d, stream);
+    case 7: return LaunchHdirectConfig<HdirectConfig<1, 4, 4, 2, 2>>(d, stream);  // 128 x 256, 4 wavefronts of 128 x 64 side by side (wide products with one row of tiles)
     case 6: return LaunchHdirectConfig<HdirectConfig<2, 2, 4, 2, 2>>(d, stream);  // 256 x 128, 4 wavefronts of 128 x 64 (tall products with one column of tiles)
     default: return LaunchHdirectConfig<HdirectConfig<2, 2, 2, 2, 2>>(d, stream);  // 128 x 128, 4 wavefronts
   }

@@ -350,7 +350,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   }
   if (precision == Precision::kHalf) {
     // Direct-load tiles, 0: 128 x 128, 1: 64 x 64, 2: 256 x 256 (8 wavefronts), 3: 128 x 32, 4: 32 x 128 (the last two
-    // lose to 64 x 64 on skinny shapes too), 5: 128 x 128 with three work-groups per CU, 6: 256 x 128 (4 wavefronts). The tile is chosen by the cost estimate of LaunchCost - rounds of
+    // lose to 64 x 64 on skinny shapes too), 5: 128 x 128 with three work-groups per CU, 6: 256 x 128, 7: 128 x 256 (4 wavefronts). The tile is chosen by the cost estimate of LaunchCost - rounds of
     // work-groups (256 x 256: one per CU, 128 x 128: two, 64 x 64: four), a partly empty last round at (c / p)^0.25 of
     // the rate - times k + k0 over the tile's rate: a tile costs what k0 more slabs would, its prologue and epilogue
     // (256 x 256: 1480 TFLOP/s and k0 = 630, 128 x 128: 940 and 290, 64 x 64: 490 and 40). Padded tiles count in full, so
@@ -395,6 +395,13 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     if (!a_kcontig && n >= 64 && n <= 128 && k >= 1024 && CeilDivide(m, 256) * batch_count >= 512 &&
         10 * m >= 9 * CeilDivide(m, 256) * 256) {
       tile = 6;
+    }
+    // (the mirror image, one row of tiles under a wide B with contiguous rows: 128 x 256, index 7, the four wavefronts
+    // side by side - 96 x 128 x 2048 x 2048 N/T 203 -> 183 us, T/T 220 -> 189 us, 16 x 128 x 8192 x 8192 T/T 488 -> 414 us; with
+    // m = 64 nothing is gained)
+    if (!b_kcontig && m >= 96 && m <= 128 && k >= 1024 && CeilDivide(n, 256) * batch_count >= 512 &&
+        10 * n >= 9 * CeilDivide(n, 256) * 256) {
+      tile = 7;
     }
     // K ranges (fp32 partial sums, then a reduction) when the 64 x 64 tiles would leave the GPU mostly idle through a
     // long K walk: up to 512 work-groups, ranges at least 512 deep - 2048 when there are 192 tiles or more, which by

@@ -241,3 +241,5 @@ def test_half_precision_tall_products_with_one_column_of_tiles(gpu):
     table takes that tile (a kernel instance of its own); with an edge in m and in n."""
     run_strided(gpu, 16, COL_MAJOR, NO, NO, 2040, 100, 1024, 1.0, 0.5, 64, seed=611)
     run_strided(gpu, 16, COL_MAJOR, NO, YES, 2048, 128, 1056, -0.5, 0.0, 64, seed=612)
+    # (the mirror image: one row of 128 x 256 tiles under a wide B with contiguous rows)
+    run_strided(gpu, 16, COL_MAJOR, YES, YES, 100, 2040, 1024, 1.0, 0.5, 64, seed=613)

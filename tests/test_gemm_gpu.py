@@ -124,7 +124,7 @@ def test_alpha_zero_is_not_special(gpu, bits, path):
         gpu.force_path(bits, None)
 
 
-TILE_VARIANTS = {32: range(1, 14), 64: range(1, 8), 16: range(1, 8)}  # override value = tile index + 1
+TILE_VARIANTS = {32: range(1, 14), 64: range(1, 8), 16: range(1, 9)}  # override value = tile index + 1
 
 
 @pytest.mark.parametrize("bits", BITS)
