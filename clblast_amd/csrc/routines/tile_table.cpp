@@ -374,6 +374,18 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     int tile = 1;
     if (cost256 <= cost128 && cost256 <= cost64) { tile = 2; }
     else if (cost128 <= cost64) { tile = 0; }
+    // (single products with an A of contiguous columns: the 256 x 128 tile as a fourth candidate, 1250 TFLOP/s and
+    // k0 = 500, two per CU - it has finer rounds than 256 x 256 and fetches less than 128 x 128; 6126 x 3116 x 3448 191 ->
+    // 172 us, 7012 x 2798 x 3854 220 -> 197 us, 4068 x 4866 x 2530 145 -> 135 us; with a k-contiguous A the tile loses 30 %)
+    // (and 128 x 256 under a B of contiguous rows: 5678 x 5926 x 4356 N/T 341 -> 325 us, 4412 x 5082 x 5264 N/T 252 -> 244 us)
+    if (batch_count == 1 && k >= 256) {
+      auto lowest = std::min({cost256, cost128, cost64});
+      const auto half_cost = [&](const size_t tile_m, const size_t tile_n) {
+        return LaunchCost(TileCandidate{Tile{0, tile_m, tile_n}, 2, 1250.0}, m, n, 0.25, 1) * (static_cast<double>(k) + 500.0);
+      };
+      if (!a_kcontig && half_cost(256, 128) < lowest) { tile = 6; lowest = half_cost(256, 128); }
+      if (!b_kcontig && half_cost(128, 256) < lowest) { tile = 7; }
+    }
     // A short k with many tiles is a stream over C, and latency decides it: a work-group waits for its first slabs,
     // walks the few there are and waits for its stores. The estimate above, fitted to longer walks, takes the 64 x 64
     // tiles there, which fetch the operand tiles twice as often; the 128 x 128 tiles are faster up to k = 128 (4096^2 x 64
