@@ -4,6 +4,7 @@
 #include "device/launch_common.hpp"
 #include "kernels/gemm_general.hpp"
 #include "kernels/gemm_direct_f16.hpp"
+#include "kernels/gemm_wide_f16.hpp"
 #include "kernels/gemm_mfma_f16.hpp"
 
 namespace clbh {
@@ -125,6 +126,47 @@ bool DwordAlignedHalf(const clbh_gemm_desc& d) {
   return true;
 }
 
+// ---- 256 x 256 tiles with one wavefront per SIMD (kernels/gemm_wide_f16.hpp) ---------------------------
+template <bool A_KC, bool B_KC, bool RANGE>
+int LaunchHwideVariant(const clbh_gemm_desc& d, hipStream_t stream) {
+  const auto args = MakeArgs<float>(d);
+  const long long tiles_m = (d.m + HwideConfig::TILE_M - 1) / HwideConfig::TILE_M;
+  const long long tiles_n = (d.n + HwideConfig::TILE_N - 1) / HwideConfig::TILE_N;
+  if (tiles_m * tiles_n > INT_MAX) { return hipErrorInvalidConfiguration; }
+  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
+  HgemmWideKernel<A_KC, B_KC, RANGE><<<grid, dim3(HwideConfig::THREADS), 0, stream>>>(args, static_cast<int>(tiles_m), static_cast<int>(tiles_n));
+  return static_cast<int>(hipGetLastError());
+}
+
+template <bool RANGE>
+int LaunchHwide(const clbh_gemm_desc& d, hipStream_t stream) {
+  const int variant = (d.a_kcontig ? 2 : 0) | (d.b_kcontig ? 1 : 0);
+  switch (variant) {
+    case 0: return LaunchHwideVariant<false, false, RANGE>(d, stream);
+    case 1: return LaunchHwideVariant<false, true, RANGE>(d, stream);
+    case 2: return LaunchHwideVariant<true, false, RANGE>(d, stream);
+    default: return LaunchHwideVariant<true, true, RANGE>(d, stream);
+  }
+}
+
+// Which form of the 256 x 256 tile a launch takes: 0 the eight-wavefront kernel, 1 the wide kernel without range
+// checks (whole tiles, K a multiple of 128), 2 the wide kernel with them. The wide kernel moves C in 16-byte pieces
+// only and addresses with 32-bit byte offsets; measured against the eight-wavefront kernel it gains 5 to 10 % on whole
+// tiles from k = 256 on (8192^2 x 256 88 -> 82 us, 8192^3 N/T 0.832 -> 0.764 ms, 4096^3 116 -> 108 us), with range checks
+// only under a long K walk of two x-contiguous operands (5000^3 N/T 272 -> 246 us; 8192^2 x 1312, whose K it pads to
+// 1408, 180 -> 191 us; with a k-contiguous operand it loses 20 to 40 %).
+int WideForm(const clbh_gemm_desc& d) {
+  if (d.conv != nullptr || d.c_triangle != 0 || d.operand_triangle != 0 || PlanSplit(d).splits > 1) { return 0; }
+  constexpr long long kMaxLd = 1ll << 21;
+  if (d.a_ld >= kMaxLd || d.b_ld >= kMaxLd || d.c_ld >= kMaxLd || d.c_ld % 2 != 0) { return 0; }
+  const auto c_address = reinterpret_cast<unsigned long long>(d.c) + 2ull * static_cast<unsigned long long>(d.c_offset);
+  if (c_address % 4 != 0) { return 0; }
+  if (d.batch_count > 1 && (d.batch.alphas != nullptr || d.c_stride % 2 != 0)) { return 0; }
+  if ((d.a_kcontig || d.b_kcontig) && d.k % 8 != 0) { return 0; }
+  if (d.m % HwideConfig::TILE_M == 0 && d.n % HwideConfig::TILE_N == 0 && d.k % (HwideConfig::TILE_K * HwideConfig::STAGES) == 0) { return 1; }
+  return (!d.a_kcontig && !d.b_kcontig && d.k >= 2048) ? 2 : 0;
+}
+
 // CONVGEMM with the A operand gathered from the images (clbh_gemm_desc::conv; HGatherPiece names the conditions): the
 // kernel matrix is k-contiguous and dword aligned, the batches are strided, K is not split
 int LaunchConvF16(const clbh_gemm_desc& d, hipStream_t stream) {
@@ -154,7 +196,13 @@ int LaunchMfmaF16(const clbh_gemm_desc& d, hipStream_t stream) {
   if (!DwordAlignedHalf(d)) { return LaunchHgemmConfig<HgemmConfig<2, 2, 2, 2, 32, 2>, false>(d, stream); }
   switch (d.tile_variant) {
     case 1: return LaunchHdirectConfig<HdirectConfig<2, 2, 1, 1, 4>>(d, stream);  // 64 x 64, 4 wavefronts
-    case 2: return LaunchHdirectConfig<HdirectConfig<2, 4, 4, 2, 2>>(d, stream);  // 256 x 256, 8 wavefronts
+    case 2:  // 256 x 256: four wavefronts of 128 x 128 where that kernel applies, else eight of 128 x 64
+      switch (WideForm(d)) {
+        case 1: return LaunchHwide<false>(d, stream);
+        case 2: return LaunchHwide<true>(d, stream);
+        default: return LaunchHdirectConfig<HdirectConfig<2, 4, 4, 2, 2>>(d, stream);
+      }
+    case 12: return LaunchHdirectConfig<HdirectConfig<2, 4, 4, 2, 2>>(d, stream);  // 256 x 256, 8 wavefronts, for comparisons
     case 3: return LaunchHdirectConfig<HdirectConfig<4, 1, 1, 1, 4>>(d, stream);  // 128 x 32 (skinny n)
     case 4: return LaunchHdirectConfig<HdirectConfig<1, 4, 1, 1, 4>>(d, stream);  // 32 x 128 (skinny m)
     // 128 x 128 held to 168 registers (a few of them spilled), three work-groups per CU: for short k, where the

@@ -1,0 +1,104 @@
+"""The 256 x 256 fp16 tile exists in two implementations: eight wavefronts of 128 x 64 (tile index 2 wherever the wide
+kernel does not apply, and index 12 always) and four wavefronts of 128 x 128 (kernels/gemm_wide_f16.hpp), without
+range checks on whole tiles with K a multiple of 128 and with them under a long K walk of two x-contiguous operands.
+Both accumulate the same products in the same order, so besides the comparison with the oracle the wide kernel has to
+reproduce the eight-wavefront kernel bit for bit."""
+import itertools
+
+import numpy as np
+import pytest
+
+import clblast_amd
+from tests import harness as gpu_harness
+from tests.harness import COL_MAJOR, NO, ROW_MAJOR, YES
+
+pytestmark = pytest.mark.gpu
+
+WIDE_OR_NOT, EIGHT_WAVES = 3, 13  # override value = tile index + 1
+
+
+def run_with(variant, problem):
+    clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": variant})
+    status, c_after = problem.run()
+    assert status == 0, (variant, problem.describe())
+    return c_after
+
+
+@pytest.fixture
+def forced():
+    gpu_harness.check_library_loaded()
+    gpu_harness.force_path(16, "indirect")
+    yield
+    clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": 0})
+    gpu_harness.force_path(16, None)
+
+
+def both_ways(problem):
+    wide = run_with(WIDE_OR_NOT, problem)
+    problem.check(wide)
+    eight = run_with(EIGHT_WAVES, problem)
+    assert np.array_equal(wide.view(np.uint16), eight.view(np.uint16)), problem.describe()
+
+
+def test_whole_tiles(forced):
+    """m, n multiples of 256 and k a multiple of 128: the instance without range checks, every orientation and both
+    layouts, one to three turns of the ring of slab buffers, beta zero and not, padded leading dimensions and even
+    offsets."""
+    seed = 9100
+    for layout, (ta, tb), (m, n, k) in itertools.product((COL_MAJOR, ROW_MAJOR), itertools.product((NO, YES), (NO, YES)),
+                                                         ((256, 256, 128), (512, 768, 384), (768, 256, 1024))):
+        seed += 1
+        problem = gpu_harness.Problem(16, layout, ta, tb, m, n, k, 0.75, 0.0 if seed % 3 == 0 else -1.5, a_offset=8,
+                                      b_offset=16, c_offset=24, seed=seed, extra_ld=(8, 16, 24), ab_low=-0.5, ab_high=0.5)
+        both_ways(problem)
+
+
+def test_edges_under_a_long_k(forced):
+    """Two x-contiguous operands (column-major N/T, row-major T/N) and k >= 2048: the instance with range checks - edge
+    tiles in m and n, a K that is no multiple of the slab, of eight or of two, rows of C that straddle the last row."""
+    seed = 9200
+    for (layout, ta, tb), (m, n, k) in itertools.product(((COL_MAJOR, NO, YES), (ROW_MAJOR, YES, NO)),
+                                                         ((300, 520, 2056), (257, 255, 2051), (515, 262, 2176), (1000, 300, 2500))):
+        seed += 1
+        problem = gpu_harness.Problem(16, layout, ta, tb, m, n, k, -0.75, 0.0 if seed % 2 else 2.0, a_offset=2, b_offset=4,
+                                      c_offset=6, seed=seed, extra_ld=(2, 4, 6), ab_low=-0.5, ab_high=0.5)
+        both_ways(problem)
+
+
+def test_what_the_wide_kernel_leaves_to_the_other(forced):
+    """Odd leading dimension or offset of C, a k-contiguous operand with k not a multiple of 8: the launch takes the
+    eight-wavefront kernel and stays correct."""
+    seed = 9300
+    for (ta, tb), extra_c, c_offset, k in (((NO, YES), 1, 0, 2048), ((NO, YES), 0, 3, 2048), ((YES, NO), 0, 0, 2052), ((NO, NO), 2, 2, 132)):
+        seed += 1
+        problem = gpu_harness.Problem(16, COL_MAJOR, ta, tb, 512, 256, k, 1.0, 1.0, c_offset=c_offset, seed=seed,
+                                      extra_ld=(0, 0, extra_c), ab_low=-0.5, ab_high=0.5)
+        both_ways(problem)
+
+
+def test_strided_batches_of_whole_tiles(forced):
+    """blockIdx.y walks the matrices of a strided batch; the slab buffers are refilled per matrix."""
+    import torch
+    from clblast_amd import _lib
+    rng = np.random.default_rng(9400)
+    m, n, k, batch = 256, 512, 256, 5
+    import oracle
+    a = rng.uniform(-0.5, 0.5, batch * k * m).astype(np.float16)   # column-major m x k each
+    b = rng.uniform(-0.5, 0.5, batch * k * n).astype(np.float16)   # column-major n x k each (used transposed)
+    c = rng.uniform(-1.0, 1.0, batch * n * m).astype(np.float16)   # column-major m x n each
+    expected = [oracle.gemm(COL_MAJOR, NO, YES, m, n, k, 0.5, a, i * m * k, m, b, i * n * k, n, 1.25, c, i * m * n, m)
+                for i in range(batch)]
+    results = []
+    for variant in (WIDE_OR_NOT, EIGHT_WAVES):
+        clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": variant})
+        a_dev, b_dev, c_dev = (torch.from_numpy(x).to("cuda:0") for x in (a, b, c))
+        status = clblast_amd.raw_gemm_strided_batched("H", COL_MAJOR, NO, YES, m, n, k, 0.5, a_dev.data_ptr(), 0, m, m * k,
+                                                      b_dev.data_ptr(), 0, n, n * k, 1.25, c_dev.data_ptr(), 0, m, m * n, batch,
+                                                      gpu_harness.stream_handle())
+        torch.cuda.synchronize()
+        assert status == 0
+        results.append(c_dev.cpu().numpy())
+    for i in range(batch):
+        where = oracle.c_indices(COL_MAJOR, m, n, i * m * n, m)
+        assert oracle.rel_frobenius(results[0][where], expected[i]) <= 1e-2, i
+    assert np.array_equal(results[0].view(np.uint16), results[1].view(np.uint16))
