@@ -465,7 +465,7 @@ def roofline_of(workload, device_ms):
                  "frac": round(achieved / PEAK_HBM_GBS, 4)}, **traffic_of(workload.name))
 
 
-def cpu_baseline(target_seconds=15.0):
+def cpu_baseline(target_seconds=5.0):
     """The reference's indirect path restated on the CPU (oracle/gemm_oracle.c: xgemm_port_f32), timed on a
     row slab of the headline problem sized to take about `target_seconds` on this host."""
     import numpy as np
@@ -483,14 +483,16 @@ def cpu_baseline(target_seconds=15.0):
         return time.perf_counter() - begin
 
     probe_m = 256
-    probe_seconds = run(probe_m)
+    probe_seconds = run(probe_m)  # also the warm-up run
     rate = 2.0 * probe_m * n * k / probe_seconds
     m = int(min(8192, max(256, (rate * target_seconds / (2.0 * n * k)) // 256 * 256)))
-    seconds = run(m) if m != probe_m else probe_seconds
+    times = [run(m) for _ in range(3)]
+    seconds = min(times)
     return {"value": round(2.0 * m * n * k / seconds / 1e9, 1), "unit": "GFLOPS", "cores": threads, "kind": "port",
-            "sample": "rows 0..%d of C of the same SGEMM (m=%d, n=k=8192, row-major, A^T): %.1f s; CPU restatement "
-                      "of the reference's Xgemm indirect path with its default 32x32x32 tiles, OpenMP over tiles, not "
-                      "CLBlast on PoCL (no CPU OpenCL device on this host)" % (m - 1, m, seconds)}
+            "sample": "rows 0..%d of C of the same SGEMM (m=%d, n=k=8192, row-major, A^T): one warm-up run, then the "
+                      "minimum of three runs (%s s); CPU restatement of the reference's Xgemm indirect path with its "
+                      "default 32x32x32 tiles, OpenMP over tiles, not CLBlast on PoCL (no CPU OpenCL device on this "
+                      "host)" % (m - 1, m, ", ".join("%.1f" % t for t in times))}
 
 
 def reference_on_this_gpu(runs=3):
@@ -598,16 +600,18 @@ EXTRA_WORKLOADS = {
 
 
 def run_extra(name, steps, warmup):
-    """One of the other BASELINE workloads. Short kernels are repeated until about 0.1 s is timed (at least
-    `steps` calls): a 1 ms kernel timed over ten calls mostly measures how fast the clocks ramp."""
+    """One of the other workloads. The GPU's clocks settle only after some tens of milliseconds of work (the first
+    twenty launches of an 0.8 ms kernel after an idle phase run 8 % slower than the sustained rate), so the kernel
+    is first run for about 50 ms untimed and then timed over about 0.3 s (at least `steps` calls)."""
     import torch
     workload = EXTRA_WORKLOADS[name]()
     error = verified_error(workload)
     _, probe_ms = time_workload(workload, 3, warmup)
-    steps = int(min(500, max(steps, 100.0 / max(probe_ms, 1e-3))))
+    settle = int(min(2000, max(warmup, 50.0 / max(probe_ms, 1e-3))))
+    steps = int(min(2000, max(steps, 300.0 / max(probe_ms, 1e-3))))
     if abs(workload.beta) > 1:
-        steps = min(steps, 60)  # C is scaled by beta on every call: stay far inside the fp32 range
-    _, device_ms = time_workload(workload, steps, 1)
+        settle, steps = min(settle, 20), min(steps, 60)  # C is scaled by beta on every call: stay far inside the fp32 range
+    _, device_ms = time_workload(workload, steps, settle)
     roofline = roofline_of(workload, device_ms)
     entry = {"ms": round(device_ms, 4), "steps": steps, "gflops": round(workload.flops / (device_ms * 1e-3) / 1e9, 1),
              "gbs": round(workload.algorithmic_bytes / (device_ms * 1e-3) / 1e9, 1), "dtype": DTYPE_NAME[workload.prefix],
@@ -618,47 +622,11 @@ def run_extra(name, steps, warmup):
     return entry
 
 
-def run_mfma_ceiling(steps):
-    """The matrix pipe's sustained fp16 rate on the operands of the cfg3 workload: the library's measurement kernel runs
-    nothing but v_mfma_f32_16x16x32_f16 on fragments taken from the same A and B (two wavefronts per SIMD, about 1 ms
-    per launch). The HGEMM line is read against this ceiling: the pipe's clock under load depends on the data."""
-    import ctypes
-    import torch
-    from clblast_amd import _lib
-    lib = _lib.load()
-    workload = EXTRA_WORKLOADS["cfg3_hgemm_8192_colNT"]()
-    lib.clbh_probe_mfma_f16_out_bytes.restype = ctypes.c_size_t
-    lib.clbh_probe_mfma_f16_out_bytes.argtypes = [ctypes.c_int]
-    lib.clbh_probe_mfma_f16_flops.restype = ctypes.c_double
-    lib.clbh_probe_mfma_f16_flops.argtypes = [ctypes.c_int, ctypes.c_int]
-    lib.clbh_probe_mfma_f16.restype = ctypes.c_int
-    lib.clbh_probe_mfma_f16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int, ctypes.c_int,
-                                        ctypes.c_void_p, ctypes.c_void_p]
-    groups, iterations = 256, 1000
-    out = torch.empty(lib.clbh_probe_mfma_f16_out_bytes(groups) // 4, dtype=torch.float32, device="cuda")
-    elements = min(workload.a.numel(), workload.b.numel()) // 8 * 8
-    stream = torch.cuda.Stream()
-
-    def launch():
-        status = lib.clbh_probe_mfma_f16(workload.a.data_ptr(), workload.b.data_ptr(), elements, groups, iterations,
-                                         out.data_ptr(), stream.cuda_stream)
-        if status != 0:
-            sys.exit("bench.py: clbh_probe_mfma_f16 failed with %d" % status)
-    with torch.cuda.stream(stream):
-        for _ in range(20):
-            launch()
-        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        start.record(stream)
-        for _ in range(max(steps, 100)):
-            launch()
-        stop.record(stream)
-        torch.cuda.synchronize()
-    ms = start.elapsed_time(stop) / max(steps, 100)
-    tflops = lib.clbh_probe_mfma_f16_flops(groups, iterations) / (ms * 1e-3) / 1e12
-    return {"ms": round(ms, 4), "tflops": round(tflops, 1), "frac_of_peak": round(tflops / PEAK_TFLOPS["H"], 4),
-            "instruction": "v_mfma_f32_16x16x32_f16", "data": "operands of cfg3_hgemm_8192_colNT",
-            "hgemm_flop_at_this_rate_ms": round(2.0 * 8192 ** 3 / (tflops * 1e12) * 1e3, 4)}
+def compact(entry):
+    """What config.baseline keeps of a workload's entry: numbers only."""
+    roofline = entry["roofline"]
+    return {"ms": entry["ms"], "tflops": round(entry["gflops"] / 1e3, 2), "gbs": entry["gbs"], "bound": roofline["bound"],
+            "frac": roofline["frac"]}
 
 
 def main():
@@ -679,9 +647,6 @@ def main():
         del source, target
         torch.cuda.empty_cache()
 
-    if args.only == "probe_hgemm_mfma_ceiling":
-        print(json.dumps({args.only: run_mfma_ceiling(args.steps)}))
-        return
     if args.only is not None:
         print(json.dumps({args.only: run_extra(args.only, args.steps, args.warmup)}))
         return
@@ -691,7 +656,7 @@ def main():
     wall, device_ms = time_workload(headline, args.steps, args.warmup)
     gflops = headline.flops * args.steps / wall / 1e9
     result = {
-        "metric": "SGEMM 8192^3 GFLOPS (2*m*n*k/s)", "value": round(gflops, 1), "unit": "GFLOPS", "n_gpus": 1,
+        "metric": "SGEMM 8192^3 GFLOPS (2*m*n*k/s); the HGEMM 8192^3 leg is config.hgemm_8192_gflops, every BASELINE configuration config.baseline", "value": round(gflops, 1), "unit": "GFLOPS", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall / args.steps * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "BASELINE configs[1] fp32: SGEMM row-major, A transposed, B not, m=n=k=8192, "
@@ -700,13 +665,27 @@ def main():
         "freivalds_rel_error": float("%.3g" % error),
         "roofline": roofline_of(headline, device_ms),
     }
+    headline_entry = {"ms": round(device_ms, 4), "gflops": round(headline.flops / (device_ms * 1e-3) / 1e9, 1),
+                      "gbs": round(headline.algorithmic_bytes / (device_ms * 1e-3) / 1e9, 1), "roofline": result["roofline"]}
     del headline
     torch.cuda.empty_cache()
-    if not args.no_extras:
-        extras = {}
-        for name in EXTRA_WORKLOADS:
+    # Every BASELINE configuration, where the driver keeps it: config.baseline holds one compact entry per
+    # configuration (milliseconds per call, TFLOP/s, algorithmic GB/s, the bound and the fraction of that bound's
+    # peak), the way the reference's client prints one row per configuration (test/performance/client.cpp:437-468).
+    # --no-extras leaves out only the workloads beyond BASELINE.json's configurations.
+    extras = {}
+    baseline = {"cfg2_sgemm_8192_rowTN": compact(headline_entry)}
+    for name in EXTRA_WORKLOADS:
+        if name.startswith("cfg"):
             extras[name] = run_extra(name, max(3, args.steps // 2), args.warmup)
-        result["other_configs"] = extras
+            baseline[name] = compact(extras[name])
+        elif not args.no_extras:
+            extras[name] = run_extra(name, max(3, args.steps // 2), args.warmup)
+    result["config"]["baseline"] = baseline
+    hgemm = extras["cfg3_hgemm_8192_colNT"]
+    result["config"]["hgemm_8192_gflops"] = hgemm["gflops"]
+    result["config"]["frac_of_fp16_peak"] = hgemm["frac_of_peak"]
+    result["other_configs"] = extras
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
         result["cpu_baseline"]["reference_opencl_on_this_gpu"] = reference_on_this_gpu()

@@ -255,15 +255,6 @@ CLBH_API int clbh_buffer_extent(const void* ptr, size_t* bytes_available);
 CLBH_API int clbh_alloc_async(void** ptr, size_t bytes, hipStream_t stream);
 CLBH_API int clbh_free_async(void* ptr, hipStream_t stream);
 
-// Measurement aid: runs nothing but v_mfma_f32_16x16x32_f16 on fragments taken from the fp16 operands a and b (`elements`
-// halves each, 16-byte aligned) - `groups` work-groups of eight wavefronts, `iterations` rounds of 64 instructions per
-// wavefront - and writes one float per thread to out (clbh_probe_mfma_f16_out_bytes(groups) bytes). The rate it reaches,
-// clbh_probe_mfma_f16_flops(groups, iterations) over its duration, is the matrix pipe's ceiling on that data.
-CLBH_API size_t clbh_probe_mfma_f16_out_bytes(int groups);
-CLBH_API double clbh_probe_mfma_f16_flops(int groups, int iterations);
-CLBH_API int clbh_probe_mfma_f16(const void* a, const void* b, long long elements, int groups, int iterations, void* out,
-                                 hipStream_t stream);
-
 // Scratch memory that needs no allocation: every GPU holds one array of clbh_static_scratch_bytes() bytes (256-byte
 // aligned) from the loading of the library's code object on. The first call for a device asks the runtime for the
 // address of that device's copy. All callers on one GPU share it; its contents survive from call to call.
