@@ -637,6 +637,14 @@ int clbh_event_record(hipEvent_t event, hipStream_t stream) {
   return static_cast<int>(hipEventRecord(event, stream));
 }
 
+int clbh_compute_units(int* units) {
+  if (units == nullptr) { return static_cast<int>(hipErrorInvalidValue); }
+  int device = 0;
+  auto status = hipGetDevice(&device);
+  if (status == hipSuccess) { status = hipDeviceGetAttribute(units, hipDeviceAttributeMultiprocessorCount, device); }
+  return static_cast<int>(status);
+}
+
 int clbh_stream_device(hipStream_t stream, int* device) {
   if (device == nullptr) { return hipErrorInvalidValue; }
   if (stream == nullptr) { return static_cast<int>(hipGetDevice(device)); }

@@ -51,6 +51,17 @@ size_t MinIndirectSize(const int device, const Precision precision) {
 
 namespace {
 size_t CeilDivide(const size_t x, const size_t y) { return (x + y - 1) / y; }
+
+// Compute units of the current device, asked once from the device layer (256 on an MI355X in its default partition
+// mode; a partition of the GPU shows fewer). The rounds of work-groups in the estimates below are counted in these; the
+// fitted thresholds next to them were measured on 256.
+size_t Units() {
+  static const size_t units = [] {
+    int count = 0;
+    return (clbh_compute_units(&count) == 0 && count > 0) ? static_cast<size_t>(count) : size_t{256};
+  }();
+  return units;
+}
 }  // namespace
 
 bool UseDirectKernel(const size_t m, const size_t n, const size_t k, const size_t min_indirect_size) {
@@ -71,8 +82,8 @@ struct Tile {
 
 // Tiles of which two share a CU: the launch runs in rounds of 512, and the last round should be at least 90 % full
 bool FillsPairs(const size_t tiles) {
-  const auto rounds = CeilDivide(tiles, 512);
-  return tiles >= 460 && 10 * tiles >= 9 * rounds * 512;
+  const auto rounds = CeilDivide(tiles, 2 * Units());
+  return tiles >= 9 * 2 * Units() / 10 && 10 * tiles >= 9 * rounds * 2 * Units();
 }
 
 // Share of the tiles' area that the m x n matrix fills (tiles of tile_m x tile_n), in per cent
@@ -86,8 +97,8 @@ size_t TileUse(const size_t m, const size_t n, const size_t tile_m, const size_t
 // least 90 % of the last round (4096 x 2048 x 4096, 256 tiles: 564 -> 505 us against 64 x 64 tiles; 2560^3, 200 tiles,
 // and 3584^3, 392 tiles, are faster with 64 x 64)
 bool FillsRounds(const size_t tiles) {
-  const auto rounds = CeilDivide(tiles, 256);
-  return tiles >= 512 || 10 * tiles >= 9 * rounds * 256;
+  const auto rounds = CeilDivide(tiles, Units());
+  return tiles >= 2 * Units() || 10 * tiles >= 9 * rounds * Units();
 }
 
 // Number of K ranges for a launch of `tiles` work-groups. Splitting costs a second launch (the reduction, about
@@ -122,10 +133,10 @@ struct TileCandidate {
 double LaunchCost(const TileCandidate& candidate, const size_t m, const size_t n, const double tail,
                   const size_t batch_count = 1) {
   const auto count = CeilDivide(m, candidate.tile.tile_m) * CeilDivide(n, candidate.tile.tile_n) * batch_count;
-  const auto slots = 256 * candidate.per_cu;
+  const auto slots = Units() * candidate.per_cu;
   auto rounds = static_cast<double>((count / slots) * candidate.per_cu);
   if (count % slots != 0) {
-    const auto together = static_cast<double>(CeilDivide(count % slots, 256));
+    const auto together = static_cast<double>(CeilDivide(count % slots, Units()));
     rounds += together / std::pow(together / static_cast<double>(candidate.per_cu), tail);
   }
   return rounds * static_cast<double>(candidate.tile.tile_m * candidate.tile.tile_n) / candidate.rate;
@@ -136,7 +147,6 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
                           const size_t n, const size_t k, const size_t batch_count, const bool per_batch_scalars,
                           const size_t min_indirect_size, const int triangular, const bool beta_zero,
                           const size_t largest_ld) {
-  (void)per_batch_scalars;
   // Many small matrices: one wavefront per matrix, bandwidth bound (that kernel knows no triangles)
   if (!triangular && batch_count >= 16 && m <= 32 && n <= 32 && k <= 32) {
     return KernelChoice{CLBH_KERNEL_SMALL_BATCHED, 0, 1};
@@ -157,7 +167,9 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   // 100352 x 128 x 200: 60 -> 50 us, 30000 x 256 x 400: 66 -> 57 us, 6000 x 1000 x 300: 41 -> 36 us, at k = 800 nothing is
   // left; 512 x 256 x 256 x 64: 106 -> 79 us; fp64 8192^2 x 256: 605 -> 543 us, 100352 x 128 x 300: 155 -> 135 us,
   // x 576: 253 -> 237 us, 512 x 256 x 256 x 64: 209 -> 150 us, 64 x 512 x 512 x 128: 107 -> 92 us).
-  if (forced == 0 && !triangular && precision != Precision::kHalf && k > 48 &&
+  // (the persistent kernel's lanes own four consecutive rows in fp32 and two in fp64: it takes no problem with fewer)
+  const size_t stream_min_m = (precision == Precision::kSingle) ? 4 : 2;
+  if (forced == 0 && !triangular && precision != Precision::kHalf && k > 48 && m >= stream_min_m &&
       largest_ld < static_cast<size_t>(CLBH_STREAM_MAX_LD)) {
     const auto tiles128 = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
     // (two k-contiguous operands go through the staging registers: 4096^2 x 1000 is 6 % behind the 256 x 128 tiles then;
@@ -215,12 +227,12 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   if ((forced == 101 || forced == 102) && !triangular && precision != Precision::kHalf) {
     return KernelChoice{CLBH_KERNEL_SMALL_TILED, static_cast<int>(forced) - 101, 1};  // one-slab kernel, 64 x 64 / 32 x 32 tiles
   }
-  if ((forced == 103 || forced == 104) && !triangular && precision != Precision::kHalf && k > 48 &&
+  if ((forced == 103 || forced == 104) && !triangular && precision != Precision::kHalf && k > 48 && m >= stream_min_m &&
       largest_ld < static_cast<size_t>(CLBH_STREAM_MAX_LD)) {
     // persistent work-groups over tiles of 64 x 64, or (fp32) 128 x 128
     return KernelChoice{CLBH_KERNEL_STREAM, (forced == 104 && precision == Precision::kSingle) ? 1 : 2, 1};
   }
-  if (forced == 105 && precision == Precision::kSingle && !triangular && batch_count == 1 && std::min(m, n) <= 32 && k < (size_t{1} << 28) &&
+  if (forced == 105 && precision == Precision::kSingle && !triangular && batch_count == 1 && !per_batch_scalars && std::min(m, n) <= 32 && k < (size_t{1} << 28) &&
       largest_ld < static_cast<size_t>(CLBH_SKINNY_MAX_LD) && (n <= 32 ? a_kcontig : b_kcontig)) {
     return KernelChoice{CLBH_KERNEL_SKINNY, 0, 1};  // the lanes-along-k kernel for a k-contiguous large operand
   }
@@ -252,10 +264,10 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
           if (option.index == 2 && k < 256) { continue; }
           const auto along = CeilDivide(n, option.extent);
           const auto count = along * (along + 1) / 2 * batch_count;
-          const auto slots = 256 * option.per_cu;
+          const auto slots = Units() * option.per_cu;
           auto rounds = static_cast<double>((count / slots) * option.per_cu);
           if (count % slots != 0) {
-            const auto together = static_cast<double>(CeilDivide(count % slots, 256));
+            const auto together = static_cast<double>(CeilDivide(count % slots, Units()));
             rounds += together / std::pow(together / static_cast<double>(option.per_cu), 0.25);
           }
           const auto time = rounds * static_cast<double>(option.extent * option.extent) * (static_cast<double>(k) + option.k0) / option.rate;
@@ -298,10 +310,10 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       int chosen = 12;
       for (const auto& option : options) {
         const auto count = touching(option.tile_m, option.tile_n);
-        const auto slots = 256 * option.per_cu;
+        const auto slots = Units() * option.per_cu;
         auto rounds = static_cast<double>((count / slots) * option.per_cu);
         if (count % slots != 0) {
-          const auto together = static_cast<double>(CeilDivide(count % slots, 256));
+          const auto together = static_cast<double>(CeilDivide(count % slots, Units()));
           rounds += together / std::pow(together / static_cast<double>(option.per_cu), 0.226);
         }
         const auto time = rounds * static_cast<double>(option.tile_m * option.tile_n) * (depth + option.k0) / option.rate;
@@ -334,10 +346,10 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       for (const auto& option : options) {
         if (both_kcontig && option.index == 0) { continue; }
         const auto count = touching(option.tile_m, option.tile_n);
-        const auto slots = 256 * option.per_cu;
+        const auto slots = Units() * option.per_cu;
         auto rounds = static_cast<double>((count / slots) * option.per_cu);
         if (count % slots != 0) {
-          const auto together = static_cast<double>(CeilDivide(count % slots, 256));
+          const auto together = static_cast<double>(CeilDivide(count % slots, Units()));
           rounds += together / std::pow(together / static_cast<double>(option.per_cu), 0.178);
         }
         const auto time = rounds * static_cast<double>(option.tile_m * option.tile_n) * (depth + option.k0) /
@@ -464,7 +476,8 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     // operand it falls behind the 64 x 32 / 32 x 64 tiles with K split, which stream at 5.2 TB/s after 10 us: the kernel is
     // taken where 4 us + max(bytes / 5.8 TB/s, products / 17e6) is the shorter time (4 x 16384 x 16384: 182 against 205 us;
     // 17 x 16384 x 4096: 63 against 52 us, 32 x 16384 x 16384: 565 against 217 us - those two take the tiles now).
-    if (batch_count == 1 && std::min(m, n) <= 32 && std::max(m, n) >= 256 && k >= 256 && k < (size_t{1} << 28) && (n <= 32 ? a_kcontig : b_kcontig) &&
+    // (a GemmBatched call of one matrix carries its scalars and offsets in device arrays, which that kernel does not read)
+    if (batch_count == 1 && !per_batch_scalars && std::min(m, n) <= 32 && std::max(m, n) >= 256 && k >= 256 && k < (size_t{1} << 28) && (n <= 32 ? a_kcontig : b_kcontig) &&
         largest_ld < static_cast<size_t>(CLBH_SKINNY_MAX_LD)) {
       const auto elements = static_cast<double>(std::max(m, n)) * static_cast<double>(k);
       const auto skinny_time = 4.0 + std::max(elements * 4.0 / 5.8e6, elements * static_cast<double>(std::min(m, n)) / 17e6);

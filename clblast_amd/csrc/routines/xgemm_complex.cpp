@@ -3,8 +3,11 @@
 // =================================================================================================
 #include "routines/xgemm_complex.hpp"
 
+#include <algorithm>
 #include <climits>
 #include <memory>
+
+#include "clbh_device.h"
 
 namespace clblast {
 // =================================================================================================
@@ -27,9 +30,16 @@ typename XgemmComplex<R>::TempLayout XgemmComplex<R>::PlanTemp(const size_t rows
   plan.expanded_bytes = 4 * rows * k * sizeof(R);                           // real 2 rows x 2k
   plan.transposed_bytes = right_kcontig ? 0 : 2 * k * columns * sizeof(R);  // complex columns x k, k contiguous
   // the real GEMM of a full product is a plain column-major 2 rows x columns x 2k call (triangles never split K)
-  plan.workspace_bytes = full ? Xgemm<R>::TempBytes(Layout::kColMajor, Transpose::kNo, Transpose::kNo, 2 * rows, columns,
-                                                    2 * k, min_indirect_size)
-                              : 0;
+  // (which kernel that call takes, and with it whether K is split, depends on the leading dimensions through two limits
+  // of the device layer; the plan holds the largest of the three possible sizes, so the size reported for a call never
+  // depends on leading dimensions the query does not know)
+  plan.workspace_bytes = 0;
+  if (full) {
+    for (const auto largest_ld : {size_t{0}, static_cast<size_t>(CLBH_STREAM_MAX_LD), static_cast<size_t>(CLBH_SKINNY_MAX_LD)}) {
+      plan.workspace_bytes = std::max(plan.workspace_bytes, Xgemm<R>::TempBytes(Layout::kColMajor, Transpose::kNo, Transpose::kNo, 2 * rows,
+                                                                                columns, 2 * k, min_indirect_size, largest_ld));
+    }
+  }
   plan.transposed_at = aligned(plan.expanded_bytes);
   plan.workspace_at = plan.transposed_at + aligned(plan.transposed_bytes);
   plan.total = plan.workspace_at + plan.workspace_bytes;

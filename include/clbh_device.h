@@ -275,6 +275,9 @@ CLBH_API int clbh_stream_is_alias(hipStream_t stream);
 // Ordinal of the device `stream` belongs to (the current device for the null stream).
 CLBH_API int clbh_stream_device(hipStream_t stream, int* device);
 
+// Number of compute units of the current device (the tile table counts its rounds of work-groups in these).
+CLBH_API int clbh_compute_units(int* units);
+
 // Human-readable text for a code returned by the functions above.
 CLBH_API const char* clbh_error_string(int code);
 

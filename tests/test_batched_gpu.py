@@ -243,3 +243,40 @@ def test_half_precision_tall_products_with_one_column_of_tiles(gpu):
     run_strided(gpu, 16, COL_MAJOR, NO, YES, 2048, 128, 1056, -0.5, 0.0, 64, seed=612)
     # (the mirror image: one row of 128 x 256 tiles under a wide B with contiguous rows)
     run_strided(gpu, 16, COL_MAJOR, YES, YES, 100, 2040, 1024, 1.0, 0.5, 64, seed=613)
+
+
+@pytest.mark.parametrize("bits", [32, 64])
+def test_batches_of_matrices_with_one_to_three_rows(gpu, bits):
+    """Hundreds of tiles with a short k call for the persistent kernel, whose lanes own four (fp32) or two (fp64)
+    consecutive rows of the canonical problem: matrices with fewer rows (column-major m, row-major n) must get another
+    kernel, not an error."""
+    seed = 900
+    for layout, (m, n) in itertools.product((COL_MAJOR, ROW_MAJOR), ((1, 1000), (2, 512), (3, 640), (512, 2), (1000, 1))):
+        for k, batch in ((64, 100), (100, 400), (300, 128)):
+            seed += 3
+            run_strided(gpu, bits, layout, NO, YES if seed % 2 else NO, m, n, k, 0.75, -1.5 if seed % 3 else 0.0, batch, seed=seed)
+
+
+def test_batched_call_of_one_skinny_matrix(gpu):
+    """GemmBatched with batch_count = 1 carries its scalars and offsets in device arrays; the lanes-along-k kernel that a
+    plain Gemm of 4099 x 17 x 4096 (transposed A) or 17 x 4099 x 4096 takes does not read those."""
+    seed = 950
+    for ta, tb, (m, n, k) in ((YES, NO, (4099, 17, 4096)), (NO, NO, (17, 4099, 4096)), (YES, NO, (4099, 17, 512))):
+        seed += 3
+        _, shape = oracle.process_arguments(COL_MAJOR, ta, tb, m, n, k)
+        a_ld, b_ld, c_ld = shape.a_one + 3, shape.b_one + 5, shape.c_one + 7
+        a_need = oracle.required_elements(shape.a_one, shape.a_two, a_ld, 11)
+        b_need = oracle.required_elements(shape.b_one, shape.b_two, b_ld, 13)
+        c_need = oracle.required_elements(shape.c_one, shape.c_two, c_ld, 19)
+        a = oracle.uniform(seed, a_need + gpu.CANARY, -1, 1, 32)
+        b = oracle.uniform(seed + 1, b_need + gpu.CANARY, -1, 1, 32)
+        c = oracle.uniform(seed + 2, c_need + gpu.CANARY, -1, 1, 32)
+        a_dev, b_dev, c_dev = gpu.to_device(a), gpu.to_device(b), gpu.to_device(c)
+        status = clblast_amd.raw_gemm_batched("S", COL_MAJOR, ta, tb, m, n, k, [-0.75], a_dev.data_ptr(), [11], a_ld,
+                                              b_dev.data_ptr(), [13], b_ld, [2.0], c_dev.data_ptr(), [19], c_ld, 1,
+                                              gpu.stream_handle())
+        torch.cuda.synchronize()
+        assert status == 0, (ta, tb, m, n, k)
+        expected = oracle.gemm(COL_MAJOR, ta, tb, m, n, k, -0.75, a, 11, a_ld, b, 13, b_ld, 2.0, c, 19, c_ld)
+        where = oracle.c_indices(COL_MAJOR, m, n, 19, c_ld)
+        assert oracle.rel_frobenius(c_dev.cpu().numpy()[where], expected) <= TOL[32]

@@ -63,3 +63,37 @@ def test_complex_temp_buffer_contract(gpu, prefix):
             assert status == -2050
             assert np.array_equal(untouched.view(np.uint8), c.view(np.uint8))
             short.free()
+
+
+def test_reported_size_suffices_under_a_very_large_leading_dimension(gpu):
+    """Which kernel the real GEMM inside takes, and with it whether K is split into ranges that need workspace, depends
+    on the leading dimensions through limits of the device layer; the size query does not take them into account, so
+    the size it reports must suffice for any of them. A C whose leading dimension is 2^19 + 8 complex elements (beyond
+    2^20 as a real matrix), skinny enough for a long-K split: the call with a buffer of exactly the reported size
+    succeeds and matches the call without a buffer bit for bit."""
+    m, n, k, c_ld = 2050, 12, 2048, (1 << 19) + 8
+    a = oracle.complex_uniform(7801, m * k, -1.0, 1.0, 32)
+    b = oracle.complex_uniform(7802, k * n, -1.0, 1.0, 32)
+    c = oracle.complex_uniform(7803, c_ld * n, -1.0, 1.0, 32)
+    alpha, beta = complex(0.5, 0.25), complex(1.0, -0.5)
+    a_dev, b_dev = gpu.to_device(a), gpu.to_device(b)
+    status, needed = clblast_amd.raw_gemm_temp_buffer_size("C", COL_MAJOR, NO, NO, m, n, k, 0, m, 0, k, 0, c_ld, gpu.stream_handle())
+    assert status == 0 and needed > 0
+
+    def call(temp_ptr):
+        c_dev = gpu.to_device(c)
+        result = clblast_amd.raw_complex_gemm("C", COL_MAJOR, NO, NO, m, n, k, alpha, a_dev.data_ptr(), 0, m, b_dev.data_ptr(), 0, k,
+                                              beta, c_dev.data_ptr(), 0, c_ld, gpu.stream_handle(), None, temp_ptr)
+        torch.cuda.synchronize()
+        return result, c_dev.cpu().numpy()
+
+    status, plain = call(None)
+    assert status == 0
+    expected = oracle.complex_gemm(COL_MAJOR, NO, NO, m, n, k, alpha, a, 0, m, b, 0, k, beta, c, 0, c_ld)
+    where = oracle.c_indices(COL_MAJOR, m, n, 0, c_ld)
+    assert np.linalg.norm(plain[where].astype(np.complex128) - expected) / np.linalg.norm(expected) <= TOL["C"]
+    exact = DeviceBuffer(needed)
+    status, with_temp = call(exact.pointer.value)
+    assert status == 0
+    assert np.array_equal(with_temp.view(np.uint8), plain.view(np.uint8))
+    exact.free()

@@ -1,0 +1,26 @@
+"""The tile table picks a kernel per problem and nothing falls back when that kernel's launcher refuses the problem,
+so every choice has to satisfy the launcher's preconditions. The table is plain host code: it is compiled here with a
+sweep over small and skinny shapes, both precisions' corner cases and batches with and without per-matrix scalars."""
+import os
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_every_choice_is_one_its_launcher_accepts(tmp_path):
+    compiler = shutil.which("g++")
+    if compiler is None:
+        pytest.skip("no g++ here")
+    binary = tmp_path / "sweep"
+    sources = [os.path.join(ROOT, "tests", "host", "select_kernel_sweep.cpp"),
+               os.path.join(ROOT, "clblast_amd", "csrc", "routines", "tile_table.cpp")]
+    done = subprocess.run([compiler, "-std=c++17", "-O1", "-I" + os.path.join(ROOT, "include"),
+                           "-I" + os.path.join(ROOT, "clblast_amd", "csrc")] + sources + ["-o", str(binary)],
+                          capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr[-3000:]
+    run = subprocess.run([str(binary)], capture_output=True, text=True)
+    assert run.returncode == 0, run.stdout[-3000:]
+    assert "violations 0" in run.stdout

@@ -49,8 +49,7 @@ def test_workspace_beyond_the_static_array_is_refused(gpu):
         if needed[0] == 0 and needed[1] > (64 << 20):
             found = (m, n, k)
             break
-    if found is None:
-        pytest.skip("no probed shape wants more than 64 MiB of workspace")
+    assert found is not None, "no probed shape wants more than 64 MiB of workspace: the refusal can no longer be shown"
     m, n, k = found
     a = torch.zeros(m * k, dtype=torch.float32, device="cuda")
     b = torch.zeros(n * k, dtype=torch.float32, device="cuda")
@@ -60,3 +59,23 @@ def test_workspace_beyond_the_static_array_is_refused(gpu):
     torch.cuda.synchronize()
     assert status == -2050
     assert bool((c == 3.0).all())
+
+
+def test_the_call_leaves_the_free_device_memory_as_it_was(gpu):
+    """With the library's cached scratch buffers dropped first, a call whose K is split (it needs a workspace) must not
+    change what the driver reports as free device memory: the partial sums live in the static array."""
+    m, n, k = 4099, 17, 4096
+    a = torch.rand(m * k, dtype=torch.float32, device="cuda")
+    b = torch.rand(k * n, dtype=torch.float32, device="cuda")
+    c = torch.rand(m * n, dtype=torch.float32, device="cuda")
+    needed = clblast_amd.raw_gemm_temp_buffer_size("S", COL_MAJOR, NO, NO, m, n, k, 0, m, 0, k, 0, m, gpu.stream_handle())
+    assert needed[0] == 0 and needed[1] > 0, "this shape no longer splits K: pick one that does"
+    assert clblast_amd.clear_cache() == 0
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        status = clblast_amd.raw_sgemm_no_alloc(COL_MAJOR, NO, NO, m, n, k, 1.0, a.data_ptr(), 0, m, b.data_ptr(), 0, k, 0.0,
+                                                c.data_ptr(), 0, m, gpu.stream_handle())
+        assert status == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
