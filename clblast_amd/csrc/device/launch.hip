@@ -264,6 +264,9 @@ int clbh_gemm_launch(const clbh_gemm_desc* desc, hipStream_t stream) {
 }
 
 size_t clbh_gemm_workspace_bytes(const clbh_gemm_desc* desc) {
+  if (desc != nullptr && desc->kernel_class == CLBH_KERNEL_SKINNY && desc->tile_variant == 1) {
+    return clbh::PlanSkinnyCols(*desc).workspace_bytes;
+  }
   if (desc == nullptr || desc->kernel_class != CLBH_KERNEL_MFMA) { return 0; }
   const auto plan = clbh::PlanSplit(*desc);
   if (plan.splits <= 1) { return 0; }

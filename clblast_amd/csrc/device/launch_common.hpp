@@ -165,6 +165,40 @@ inline SplitPlan PlanSplit(const clbh_gemm_desc& d) {
   return plan;
 }
 
+// Geometry of a launch of the kernel for skinny products with an x-contiguous large operand
+// (kernels/gemm_skinny_cols.hpp; kernel class CLBH_KERNEL_SKINNY, tile_variant 1): strips of 64 rows of the large
+// operand, per strip as many work-groups (K ranges) as fit one round on four fifths of the compute units while
+// every wavefront keeps at least two runs of 16 k, and the workspace: the ranges' partial sums, then one counter per
+// strip (used when the stream has no counters of its own, see clbh_tickets).
+struct SkinnyColsPlan {
+  int blocks, extra, strips, ranges, k_per_group, partial_ld;  // (blocks of 16 columns on the matrix pipe, columns beside them)
+  size_t partial_bytes, workspace_bytes;
+};
+inline SkinnyColsPlan PlanSkinnyCols(const clbh_gemm_desc& d) {
+  SkinnyColsPlan plan{};
+  const int extent = (d.n <= 32) ? d.m : d.n, small = (d.n <= 32) ? d.n : d.m;
+  if (small > 32 || extent <= 0) { return plan; }
+  plan.blocks = (small <= 20) ? 1 : 2;  // (up to four columns beyond a block go to the vector ALUs)
+  plan.extra = (small > 16 && small <= 20) ? small - 16 : 0;
+  plan.strips = (extent + 63) / 64;
+  int units = 256;
+  if (clbh_compute_units(&units) != 0 || units <= 0) { units = 256; }
+  const int wave_runs = 8 * 16;                                  // k of a run of each of the eight wavefronts
+  const int most = std::max(1, d.k / (2 * wave_runs));          // ranges that leave two runs per wavefront
+  // (one round of work-groups that leaves a fifth of the compute units free: 4099 x 17 x 4096 takes 20 us with 3 ranges,
+  // 195 work-groups, and 26 us with 4, which is 4 more work-groups than compute units)
+  plan.ranges = std::max(1, std::min({4 * units / (5 * plan.strips), most, 32}));
+  if (d.split_k > 1) { plan.ranges = std::min(d.split_k, std::max(1, d.k / wave_runs)); }  // a number of ranges asked for
+  plan.k_per_group = ((d.k + plan.ranges - 1) / plan.ranges + wave_runs - 1) / wave_runs * wave_runs;
+  plan.ranges = (d.k + plan.k_per_group - 1) / plan.k_per_group;
+  plan.partial_ld = plan.strips * 64;
+  if (plan.ranges > 1) {
+    plan.partial_bytes = sizeof(float) * static_cast<size_t>(plan.ranges) * (16 * plan.blocks + plan.extra) * plan.partial_ld;
+    plan.workspace_bytes = plan.partial_bytes + (static_cast<size_t>(plan.strips) * sizeof(unsigned int) + 255) / 256 * 256;
+  }
+  return plan;
+}
+
 }  // namespace clbh
 
 #endif  // CLBLAST_HIP_DEVICE_LAUNCH_COMMON_HPP_

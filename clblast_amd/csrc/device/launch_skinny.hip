@@ -3,6 +3,7 @@
 // =================================================================================================
 #include "device/launch_common.hpp"
 #include "kernels/gemm_skinny.hpp"
+#include "kernels/gemm_skinny_cols.hpp"
 
 namespace clbh {
 namespace {
@@ -54,8 +55,80 @@ bool SkinnyXIsA(const clbh_gemm_desc& d) { return d.n <= 32; }
 bool SkinnySKcontig(const clbh_gemm_desc& d) { return SkinnyXIsA(d) ? (d.b_kcontig != 0) : (d.a_kcontig != 0); }
 }  // namespace
 
+// ---- x-contiguous large operand (kernels/gemm_skinny_cols.hpp) ---------------------------------------------
+template <int BLOCKS, int EXTRA>
+int LaunchSkinnyColsBlocks(const SkinnyColsArgs& args, const bool s_kc, const unsigned groups, hipStream_t stream) {
+  constexpr int kDepth = 3;
+  constexpr size_t lds_bytes = SkinnyColsLdsBytes(BLOCKS, EXTRA);
+  const auto launch = [&](auto kernel) {
+    if (lds_bytes > 48 * 1024) {
+      static const hipError_t attribute_status = hipFuncSetAttribute(
+          reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+      if (attribute_status != hipSuccess) { return static_cast<int>(attribute_status); }
+    }
+    kernel<<<dim3(groups), dim3(64 * kSkinnyColsWaves), lds_bytes, stream>>>(args);
+    return static_cast<int>(hipGetLastError());
+  };
+  return s_kc ? launch(GemmSkinnyColsKernel<BLOCKS, EXTRA, kDepth, true>) : launch(GemmSkinnyColsKernel<BLOCKS, EXTRA, kDepth, false>);
+}
+
+int LaunchSkinnyColsF32(const clbh_gemm_desc& d, hipStream_t stream) {
+  const auto plan = PlanSkinnyCols(d);
+  const bool x_is_a = SkinnyXIsA(d);
+  if ((x_is_a ? d.a_kcontig : d.b_kcontig) != 0 || plan.strips <= 0) { return hipErrorInvalidValue; }
+  SkinnyColsArgs args{};
+  const float* a = static_cast<const float*>(d.a) + d.a_offset;
+  const float* b = static_cast<const float*>(d.b) + d.b_offset;
+  args.x = x_is_a ? a : b;
+  args.s = x_is_a ? b : a;
+  args.c = static_cast<float*>(d.c) + d.c_offset;
+  args.x_ld = x_is_a ? d.a_ld : d.b_ld;
+  // S as (k, col): B is k x n (k contiguous, or n contiguous), A is m x k (k contiguous, or m contiguous)
+  const bool s_kc = x_is_a ? (d.b_kcontig != 0) : (d.a_kcontig != 0);
+  const long long s_ld = x_is_a ? d.b_ld : d.a_ld;
+  args.s_k_stride = s_kc ? 1 : s_ld;
+  args.s_col_stride = s_kc ? s_ld : 1;
+  args.c_row_stride = x_is_a ? 1 : d.c_ld;   // rows of X are rows of C (X = A) or its columns (X = B)
+  args.c_col_stride = x_is_a ? d.c_ld : 1;
+  args.extent = x_is_a ? d.m : d.n;
+  args.small = x_is_a ? d.n : d.m;
+  args.k = d.k;
+  args.ranges = plan.ranges;
+  args.k_per_group = plan.k_per_group;
+  args.partial_ld = plan.partial_ld;
+  args.alpha = static_cast<float>(d.alpha);
+  args.beta = static_cast<float>(d.beta);
+  if (plan.ranges > 1) {
+    if (d.workspace == nullptr || d.workspace_bytes < plan.workspace_bytes) { return hipErrorInvalidValue; }
+    args.partials = static_cast<float*>(d.workspace);
+    // counters: the stream's slot of counters that are zero between launches, or, where the stream has none, the
+    // counters at the end of the workspace behind a launch that clears them
+    unsigned int* tickets = nullptr;
+    if (plan.strips > CLBH_TICKETS_PER_STREAM || clbh_tickets(stream, &tickets) != 0 || tickets == nullptr) {
+      tickets = reinterpret_cast<unsigned int*>(static_cast<unsigned char*>(d.workspace) + plan.partial_bytes);
+      const auto status = clbh_fill_zero(tickets, plan.workspace_bytes - plan.partial_bytes, stream);
+      if (status != 0) { return status; }
+    }
+    args.tickets = tickets;
+  }
+  const auto groups = static_cast<unsigned>(plan.strips * plan.ranges);
+  if (plan.blocks == 2) { return LaunchSkinnyColsBlocks<2, 0>(args, s_kc, groups, stream); }
+  switch (plan.extra) {
+    case 0: return LaunchSkinnyColsBlocks<1, 0>(args, s_kc, groups, stream);
+    case 1: return LaunchSkinnyColsBlocks<1, 1>(args, s_kc, groups, stream);
+    case 2: return LaunchSkinnyColsBlocks<1, 2>(args, s_kc, groups, stream);
+    case 3: return LaunchSkinnyColsBlocks<1, 3>(args, s_kc, groups, stream);
+    default: return LaunchSkinnyColsBlocks<1, 4>(args, s_kc, groups, stream);
+  }
+}
+
 int LaunchSkinnyF32(const clbh_gemm_desc& d, hipStream_t stream) {
-  if (d.precision != 32 || d.batch_count != 1 || d.batch.alphas != nullptr || d.c_triangle != 0 || d.operand_triangle != 0 ||
+  if (d.precision == 32 && d.tile_variant == 1 && d.batch_count == 1 && d.batch.alphas == nullptr && d.c_triangle == 0 &&
+      d.operand_triangle == 0 && d.conv == nullptr && std::min(d.m, d.n) <= 32 && d.k < (1 << 28) && d.a_ld < CLBH_SKINNY_MAX_LD &&
+      d.b_ld < CLBH_SKINNY_MAX_LD && d.c_ld < CLBH_SKINNY_MAX_LD) {
+    return LaunchSkinnyColsF32(d, stream);
+  }
+  if (d.precision != 32 || d.tile_variant != 0 || d.batch_count != 1 || d.batch.alphas != nullptr || d.c_triangle != 0 || d.operand_triangle != 0 ||
       d.conv != nullptr || std::min(d.m, d.n) > 32 || d.k >= (1 << 28) || d.a_ld >= CLBH_SKINNY_MAX_LD || d.b_ld >= CLBH_SKINNY_MAX_LD) {
     return hipErrorInvalidValue;
   }

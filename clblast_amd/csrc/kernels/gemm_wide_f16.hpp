@@ -150,7 +150,7 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
     // strip 0 comes in under the first three slabs of the last turn (3, 3 and 2 loads), strip 1 under the fourth, whose
     // MFMAs need no fragments of a next slab any more
     constexpr int EARLY_STRIPS = 2;
-    constexpr int kEarlyBefore[STAGES] = {0, 3, 6, 8};  // loads of old C issued before slab ST of the last turn
+    constexpr int kEarlyBefore[STAGES + 1] = {0, 3, 6, 8, 8};  // loads of old C issued before slab ST of the last turn
 
     const T* a_tile0 = a + (A_KC ? m0 * p.a_ld : static_cast<long long>(m0));  // element (m0, k = 0), uniform
     const T* b_tile0 = b + (B_KC ? n0 * p.b_ld : static_cast<long long>(n0));

@@ -236,6 +236,11 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       largest_ld < static_cast<size_t>(CLBH_SKINNY_MAX_LD) && (n <= 32 ? a_kcontig : b_kcontig)) {
     return KernelChoice{CLBH_KERNEL_SKINNY, 0, 1};  // the lanes-along-k kernel for a k-contiguous large operand
   }
+  if (forced == 106 && precision == Precision::kSingle && !triangular && batch_count == 1 && !per_batch_scalars && std::min(m, n) <= 32 && k < (size_t{1} << 28) &&
+      largest_ld < static_cast<size_t>(CLBH_SKINNY_MAX_LD) && !(n <= 32 ? a_kcontig : b_kcontig)) {
+    // the lanes-along-the-rows kernel for an x-contiguous large operand; a forced number of K ranges is passed on
+    return KernelChoice{CLBH_KERNEL_SKINNY, 1, static_cast<int>(ForcedSplit(precision))};
+  }
   if (forced != 0 && forced < 100) {
     // a forced tile takes the forced number of K ranges (unbatched calls only), never more than k / 16
     const auto ranges = (batch_count == 1) ? std::max<size_t>(1, std::min<size_t>(ForcedSplit(precision), k / 16)) : 1;
@@ -483,6 +488,12 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       const auto skinny_time = 4.0 + std::max(elements * 4.0 / 5.8e6, elements * static_cast<double>(std::min(m, n)) / 17e6);
       const auto tiled_time = 10.0 + elements * 4.0 / 5.2e6;
       if (skinny_time < tiled_time) { return KernelChoice{CLBH_KERNEL_SKINNY, 0, 1}; }
+    }
+    // Where the large operand is x-contiguous, the kernel that puts its lanes along the rows of that operand, 64 rows per
+    // work-group, and splits K over work-groups that meet in memory within the one launch.
+    if (batch_count == 1 && !per_batch_scalars && std::min(m, n) <= 32 && std::max(m, n) >= 256 && k >= 256 && k < (size_t{1} << 28) &&
+        !(n <= 32 ? a_kcontig : b_kcontig) && largest_ld < static_cast<size_t>(CLBH_SKINNY_MAX_LD)) {
+      return KernelChoice{CLBH_KERNEL_SKINNY, 1, 1};
     }
     auto tile = Tile{12, 64, 64};  // (the 64 x 64 tile that moves C in 16-byte pieces; index 7 is the one on 32x32x2)
     const auto tiles64 = CeilDivide(m, 64) * CeilDivide(n, 64) * batch_count;

@@ -34,9 +34,12 @@ enum clbh_kernel_class {
   CLBH_KERNEL_GENERAL = 0,  // bounds-checked LDS-tiled FMA kernel, any shape (reference analogue: XgemmDirect)
   CLBH_KERNEL_MFMA = 1,     // large-tile MFMA kernel with LDS double buffering (analogue: Xgemm indirect)
   CLBH_KERNEL_SMALL_BATCHED = 2,  // one wavefront per small matrix, bandwidth bound
-  CLBH_KERNEL_SKINNY = 3,         // fp32, m or n at most 32, unbatched, no triangles, the large operand k-contiguous
-                                  // (n <= 32: a_kcontig, else b_kcontig), leading dimensions below CLBH_SKINNY_MAX_LD:
-                                  // lanes along k, a work-group owns a few rows of the large operand and all of K
+  CLBH_KERNEL_SKINNY = 3,         // fp32, m or n at most 32, unbatched, no triangles, leading dimensions below
+                                  // CLBH_SKINNY_MAX_LD. tile_variant 0: the large operand k-contiguous (n <= 32:
+                                  // a_kcontig, else b_kcontig) - lanes along k, a work-group owns a few rows of the
+                                  // large operand and all of K. tile_variant 1: the large operand x-contiguous - lanes
+                                  // along its rows, K split over work-groups that meet in the workspace (see
+                                  // clbh_gemm_workspace_bytes) within the one launch
   CLBH_KERNEL_SMALL_TILED = 4,    // fp32 / fp64 batches of matrices of a few tiles: one slab per operand in LDS, many
                                   // work-groups per CU (tile_variant 1: tiles of 32 x 32, else 64 x 64)
   CLBH_KERNEL_STREAM = 5          // fp32 / fp64 launches of many 64 x 64 tiles with a short K walk (k > 48): persistent
@@ -274,6 +277,13 @@ CLBH_API int clbh_stream_is_alias(hipStream_t stream);
 
 // Ordinal of the device `stream` belongs to (the current device for the null stream).
 CLBH_API int clbh_stream_device(hipStream_t stream, int* device);
+
+// CLBH_TICKETS_PER_STREAM counters for kernels whose work-groups meet in memory: zero when handed out and left at zero by
+// every kernel that uses them. Launches on `stream` may share them (they are ordered); other streams get others.
+// Non-zero when this stream gets none (the per-thread stream, or more stream handles than the library has slots): the
+// caller then clears counters of its own.
+#define CLBH_TICKETS_PER_STREAM 1024
+CLBH_API int clbh_tickets(hipStream_t stream, unsigned int** pointer);
 
 // Number of compute units of the current device (the tile table counts its rounds of work-groups in these).
 CLBH_API int clbh_compute_units(int* units);
