@@ -33,9 +33,14 @@ int main() {
             else if (m < (precision == Precision::kSingle ? 4u : 2u)) { broken = "stream kernel with fewer rows than a lane owns"; }
             else if (k <= 48) { broken = "stream kernel with k <= 48"; }
             break;
-          case CLBH_KERNEL_SKINNY:  // LaunchSkinnyF32
-            if (precision != Precision::kSingle || batch != 1 || per_batch || (m < n ? m : n) > 32 || !(n <= 32 ? a_kc : b_kc)) { broken = "skinny kernel outside its conditions"; }
+          case CLBH_KERNEL_SKINNY: {  // LaunchSkinnyF32: variant 0 wants the large operand k-contiguous, variant 1 x-contiguous
+            const bool large_kc = (n <= 32) ? a_kc : b_kc;
+            if (precision != Precision::kSingle || batch != 1 || per_batch || (m < n ? m : n) > 32 || choice.tile_variant < 0 ||
+                choice.tile_variant > 1 || large_kc != (choice.tile_variant == 0)) {
+              broken = "skinny kernel outside its conditions";
+            }
             break;
+          }
           case CLBH_KERNEL_SMALL_BATCHED:
             if (m > 32 || n > 32 || k > 32 || batch < 16) { broken = "one-wavefront-per-matrix kernel outside its conditions"; }
             break;
