@@ -132,8 +132,12 @@ int LaunchHwideVariant(const clbh_gemm_desc& d, hipStream_t stream) {
   const auto args = MakeArgs<float>(d);
   const long long tiles_m = (d.m + HwideConfig::TILE_M - 1) / HwideConfig::TILE_M;
   const long long tiles_n = (d.n + HwideConfig::TILE_N - 1) / HwideConfig::TILE_N;
-  if (tiles_m * tiles_n > INT_MAX) { return hipErrorInvalidConfiguration; }
-  const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n), static_cast<unsigned>(std::min(d.batch_count, kMaxGridY)));
+  if (tiles_m * tiles_n * d.batch_count > INT_MAX) { return hipErrorInvalidConfiguration; }
+  // persistent work-groups, one per compute unit (a multiple of the eight XCDs, which the tile order counts on)
+  int units = 0;
+  if (clbh_compute_units(&units) != 0 || units < 8) { units = 256; }
+  const long long items = tiles_m * tiles_n * d.batch_count;
+  const dim3 grid(static_cast<unsigned>(std::min<long long>(items, units - units % 8)));
   HgemmWideKernel<A_KC, B_KC, RANGE><<<grid, dim3(HwideConfig::THREADS), 0, stream>>>(args, static_cast<int>(tiles_m), static_cast<int>(tiles_n));
   return static_cast<int>(hipGetLastError());
 }
@@ -152,9 +156,9 @@ int LaunchHwide(const clbh_gemm_desc& d, hipStream_t stream) {
 // Which form of the 256 x 256 tile a launch takes: 0 the eight-wavefront kernel, 1 the wide kernel without range
 // checks (whole tiles, K a multiple of 128), 2 the wide kernel with them. The wide kernel moves C in 16-byte pieces
 // only and addresses with 32-bit byte offsets; measured against the eight-wavefront kernel it gains 5 to 10 % on whole
-// tiles from k = 256 on (8192^2 x 256 88 -> 82 us, 8192^3 N/T 0.832 -> 0.764 ms, 4096^3 116 -> 108 us), with range checks
-// only under a long K walk of two x-contiguous operands (5000^3 N/T 272 -> 246 us; 8192^2 x 1312, whose K it pads to
-// 1408, 180 -> 191 us; with a k-contiguous operand it loses 20 to 40 %).
+// tiles from k = 256 on (8192^2 x 256 85 -> 79 us, 8192^3 N/T 0.815 -> 0.747 ms, 4096^3 115 -> 108 us), with range checks
+// only under a long K walk of two x-contiguous operands (5000^3 N/T 272 -> 253 us; 8192^2 x 1312, whose K it pads to
+// 1408, 177 -> 208 us; with a k-contiguous operand it loses 5 to 40 %).
 int WideForm(const clbh_gemm_desc& d) {
   if (d.conv != nullptr || d.c_triangle != 0 || d.operand_triangle != 0 || PlanSplit(d).splits > 1) { return 0; }
   constexpr long long kMaxLd = 1ll << 21;

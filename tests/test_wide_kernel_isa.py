@@ -55,8 +55,8 @@ def test_no_accumulator_copies_inside_the_walk(assembly):
                 assert "v_accvgpr" not in line, (name, line)
                 mfmas += "v_mfma_f32_16x16x32_f16" in line
         assert walks == 1 and not inside, name
-        # first turn of one slab, first turn, steady turn, start of the last turn, rest of the last turn: 64 MFMAs per slab
-        assert mfmas == 64 * (1 + 4 + 4 + 1 + 3), (name, mfmas)
+        # a walk of one turn, else first turn, steady turn, last turn: four slabs each, 64 MFMAs per slab
+        assert mfmas == 64 * (4 + 4 + 4 + 4), (name, mfmas)
 
 
 def test_the_walk_of_whole_tiles_spills_nothing(assembly):
@@ -72,6 +72,21 @@ def test_the_walk_of_whole_tiles_spills_nothing(assembly):
                 inside = False
             elif inside:
                 assert "scratch_" not in line, (name, line)
+
+
+def test_requests_run_once_per_wavefront(assembly):
+    """The buffer resources of the slab requests are kept in scalar registers; were they vector values, every request
+    would sit in a loop over the values the lanes hold (its end: a jump while lanes are left in exec)."""
+    for name, lines in kernels_of(assembly).items():
+        for at, line in enumerate(lines):
+            if "buffer_load_dwordx4" in line and " lds" in line:
+                assert not any("s_cbranch_execnz" in later for later in lines[at + 1:at + 4]), (name, at)
+
+
+def test_the_instances_for_whole_tiles_use_no_scratch_memory(assembly):
+    for name, lines in kernels_of(assembly).items():
+        if name.endswith("Lb0EEEvNS_8GemmArgsIfEEii"):
+            assert not any("scratch_" in line for line in lines), name
 
 
 def test_only_the_store_helper_issues_16_byte_buffer_stores():
