@@ -36,8 +36,9 @@ DTYPE_NAME = {"S": "f32", "D": "f64", "H": "f16", "C": "c64 (f32 arithmetic)", "
 MEASURED_TRAFFIC = {
     "cfg2s": (5.196e9, "profiles/sgemm_8192_rowTN.md", "clbh::GemmMfmaKernel<float, clbh::MfmaConfig<float, 2, 2, 4, 2, 16, 2"),
     "cfg2d": (1.3193e10, "profiles/dgemm_8192_rowTN.md", "clbh::GemmMfmaKernel<double, clbh::MfmaConfig<double, 2, 2, 4, 4, 8, 2"),
-    "cfg3": (1.932e9, "profiles/hgemm_8192_colNT.md", "clbh::HgemmDirectKernel<clbh::HdirectConfig<2, 4, 4, 2, 2, 3, false>"),
+    "cfg3": (1.884e9, "profiles/hgemm_8192_colNT.md", "clbh::HgemmWideKernel<false, false, false>"),
     "cfg4": (1.007e8, "profiles/sgemm_strided_batched_8192x32.md", "clbh::GemmSmallBatchedKernel"),
+    "cfg5b": (7.704e7, "profiles/sgemm_4099x17x4096_colNN.md", "clbh::GemmSkinnyColsKernel<1, 1, 3, true>"),
     "cfg5c": (7.461e7, "profiles/sgemm_17x4099x4096_colNN.md", "clbh::GemmSkinnyRowsKernel<4, 5, 5, 2, false, false, 2>"),
     "cfg5d": (6.225e8, "profiles/sgemm_8191x8191x127_colNN.md", "clbh::GemmStreamKernel<float, clbh::MfmaConfig<float, 1, 4, 4, 1, 16, 2"),
     "cfg5e": (7.371e7, "profiles/sgemm_4099x17x4096_colTN.md", "clbh::GemmSkinnyRowsKernel<4, 5, 5, 2, true, true, 2>"),
@@ -63,6 +64,9 @@ def parse_args():
     parser.add_argument("--no-extras", action="store_true", help="only the headline workload")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     parser.add_argument("--only", default=None, help="run a single extra workload by name and exit (for profiling)")
+    parser.add_argument("--quick", action="store_true",
+                        help="with --only: exactly --warmup and --steps calls, no settling of the clocks (for counter "
+                             "runs, in which the profiler serialises every launch)")
     parser.add_argument("--copy-calibration", action="store_true",
                         help="also run one plain 1 GiB device-to-device copy (reads 2^30 bytes, writes 2^30 bytes): the "
                              "known-size kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -599,7 +603,7 @@ EXTRA_WORKLOADS = {
 }
 
 
-def run_extra(name, steps, warmup):
+def run_extra(name, steps, warmup, quick=False):
     """One of the other workloads. The GPU's clocks settle only after some tens of milliseconds of work (the first
     twenty launches of an 0.8 ms kernel after an idle phase run 8 % slower than the sustained rate), so the kernel
     is first run for about 50 ms untimed and then timed over about 0.3 s (at least `steps` calls)."""
@@ -607,8 +611,11 @@ def run_extra(name, steps, warmup):
     workload = EXTRA_WORKLOADS[name]()
     error = verified_error(workload)
     _, probe_ms = time_workload(workload, 3, warmup)
-    settle = int(min(2000, max(warmup, 50.0 / max(probe_ms, 1e-3))))
-    steps = int(min(2000, max(steps, 300.0 / max(probe_ms, 1e-3))))
+    if quick:
+        settle, steps = warmup, max(1, steps)
+    else:
+        settle = int(min(2000, max(warmup, 50.0 / max(probe_ms, 1e-3))))
+        steps = int(min(2000, max(steps, 300.0 / max(probe_ms, 1e-3))))
     if abs(workload.beta) > 1:
         settle, steps = min(settle, 20), min(steps, 60)  # C is scaled by beta on every call: stay far inside the fp32 range
     _, device_ms = time_workload(workload, steps, settle)
@@ -648,7 +655,7 @@ def main():
         torch.cuda.empty_cache()
 
     if args.only is not None:
-        print(json.dumps({args.only: run_extra(args.only, args.steps, args.warmup)}))
+        print(json.dumps({args.only: run_extra(args.only, args.steps, args.warmup, args.quick)}))
         return
 
     headline = Workload("cfg2s", "S", ROW, YES, NO, 8192, 8192, 8192, 1.0, 0.0)

@@ -184,10 +184,12 @@ inline SkinnyColsPlan PlanSkinnyCols(const clbh_gemm_desc& d) {
   int units = 256;
   if (clbh_compute_units(&units) != 0 || units <= 0) { units = 256; }
   const int wave_runs = 8 * 16;                                  // k of a run of each of the eight wavefronts
-  const int most = std::max(1, d.k / (2 * wave_runs));          // ranges that leave two runs per wavefront
-  // (one round of work-groups that leaves a fifth of the compute units free: 4099 x 17 x 4096 takes 20 us with 3 ranges,
-  // 195 work-groups, and 26 us with 4, which is 4 more work-groups than compute units)
-  plan.ranges = std::max(1, std::min({4 * units / (5 * plan.strips), most, 32}));
+  // As many ranges as keep the launch within one work-group per compute unit, each at least 640 deep. More work-groups
+  // than compute units cost 4 to 5 us at once (4099 x 17 x 4096: 195 work-groups 18.1 us, 260 work-groups 22.5 us;
+  // 3000 x 17 x 16384: 235 work-groups 36.7 us, 282 work-groups 51.7 us), shallower ranges pay more for the meeting of
+  // the sums than they gain (1024 x 16 x 8192: 8 ranges 12.9 us, 16 ranges 14.0 us).
+  const int most = std::max(1, d.k / 640);
+  plan.ranges = std::max(1, std::min({units / plan.strips, most, 32}));
   if (d.split_k > 1) { plan.ranges = std::min(d.split_k, std::max(1, d.k / wave_runs)); }  // a number of ranges asked for
   plan.k_per_group = ((d.k + plan.ranges - 1) / plan.ranges + wave_runs - 1) / wave_runs * wave_runs;
   plan.ranges = (d.k + plan.k_per_group - 1) / plan.k_per_group;

@@ -378,15 +378,19 @@ __device__ __forceinline__ void StorePiece(T* __restrict__ tile, const int tid, 
 }
 
 // ---- blockIdx -> tile ------------------------------------------------------------------------------
-__device__ __forceinline__ void TileOfBlock(const int block, const int num_blocks, const int tiles_m,
-                                            const int tiles_n, int& tile_m, int& tile_n) {
-  // (1) work-groups are dealt to the XCDs round-robin: give each XCD a contiguous logical range
+// Work-groups are dealt to the XCDs round-robin; this index gives each XCD a contiguous range of 0 .. num_blocks - 1
+__device__ __forceinline__ int XcdContiguousIndex(const int block, const int num_blocks) {
   const int per_xcd = (num_blocks + kNumXcd - 1) / kNumXcd;
   const int remainder = num_blocks % kNumXcd;
   const int tall = (remainder == 0) ? kNumXcd : remainder;  // XCDs that own per_xcd blocks
   const int xcd = block % kNumXcd, local = block / kNumXcd;
-  const int logical = (xcd < tall) ? xcd * per_xcd + local
-                                   : tall * per_xcd + (xcd - tall) * (per_xcd - 1) + local;
+  return (xcd < tall) ? xcd * per_xcd + local : tall * per_xcd + (xcd - tall) * (per_xcd - 1) + local;
+}
+
+__device__ __forceinline__ void TileOfBlock(const int block, const int num_blocks, const int tiles_m,
+                                            const int tiles_n, int& tile_m, int& tile_n) {
+  // (1) a contiguous logical range per XCD
+  const int logical = XcdContiguousIndex(block, num_blocks);
   // (2) grouped walk: GROUP_M tile rows at a time, column by column inside a group
   constexpr int GROUP_M = 8;
   const int in_group = GROUP_M * tiles_n;

@@ -62,7 +62,7 @@ constexpr size_t SkinnyColsLdsBytes(const int blocks, const int extra) {
   return sizeof(float) * kSkinnyColsWaves * (16 * blocks + 4 * extra) * kSkinnyColsPitch;
 }
 
-// grid: strips * ranges work-groups of 512 threads; work-group g serves strip g % strips and range g / strips.
+// grid: strips * ranges work-groups of 512 threads (which strip and range a work-group serves: see below).
 template <int BLOCKS, int EXTRA, int DEPTH, bool S_KC>
 __global__ __launch_bounds__(64 * kSkinnyColsWaves, 2) void GemmSkinnyColsKernel(const SkinnyColsArgs p) {
   constexpr int WAVES = kSkinnyColsWaves, RUN = kSkinnyColsRun, PITCH = kSkinnyColsPitch;
@@ -75,10 +75,14 @@ __global__ __launch_bounds__(64 * kSkinnyColsWaves, 2) void GemmSkinnyColsKernel
 
   const int tid = threadIdx.x, lane = tid % 64;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
-  // (neighbouring work-groups take neighbouring strips of the same K range: they start together and walk K at the
-  // same pace, so the 256-byte runs they fetch from a row of k are asked of the memory at about the same time)
+  // Neighbouring strips go to the same XCD (work-groups are dealt to the XCDs in turn, each XCD has its own L2): a
+  // strip's 256-byte runs start wherever the leading dimension puts them, so a run shares its first and last 128-byte
+  // line with the neighbours' runs, and the work-groups of an XCD walk K at the same pace - one of them fetches such a
+  // line, the other finds it in the L2. (Strip after strip dealt across the XCDs, 4099 x 17 x 4096 with a leading
+  // dimension of 4102 read 1.56 times the bytes of X from memory.)
   const int strips = gridDim.x / p.ranges;
-  const int strip = blockIdx.x % strips, range = blockIdx.x / strips;
+  const int logical = XcdContiguousIndex(blockIdx.x, gridDim.x);
+  const int strip = logical / p.ranges, range = logical % p.ranges;
   const int row0 = strip * kSkinnyColsRows;
   const int lane_row = 4 * (lane % 16), lane_g = lane / 16;
 
@@ -114,6 +118,30 @@ __global__ __launch_bounds__(64 * kSkinnyColsWaves, 2) void GemmSkinnyColsKernel
   for (int b = 0; b < BLOCKS; ++b) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) { acc[b][j] = float4_t(0.0f); }
+  }
+
+  // At the end thread t holds the piece (col, rows 4 q .. 4 q + 3) of the strip's sums, t = 16 col + q; with two blocks
+  // of columns every thread has a piece, with one block the first half of the threads. The old values of C that such
+  // a piece is combined with are fetched here, ahead of the walk over K, by every work-group of the strip (only the
+  // one that finishes the strip uses them, and only that one writes C, after all others have come by): the fetch
+  // would otherwise stand at the end of a chain of memory round trips - partial sums, ticket, partial sums, C.
+  const int col = tid / 16, q = tid % 16;
+  const bool has_piece = col < COLS;
+  const int row = row0 + 4 * q;
+  const bool stores = has_piece && col < p.small && row < p.extent;
+  const bool whole_piece = p.c_row_stride == 1 && row + 3 < p.extent;
+  typedef float float4u_t __attribute__((ext_vector_type(4), aligned(4)));
+  float* const c_piece = p.c + row * p.c_row_stride + col * p.c_col_stride;
+  float4_t old_c = float4_t(0.0f);
+  if (stores && p.beta != 0.0f) {
+    if (whole_piece) {
+      old_c = *reinterpret_cast<const float4u_t*>(c_piece);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (row + e < p.extent) { old_c[e] = c_piece[e * p.c_row_stride]; }
+      }
+    }
   }
 
   // One run of 16 k: the lane's four pieces of X (steps s = 0..3) and its values of S per block
@@ -228,11 +256,7 @@ __global__ __launch_bounds__(64 * kSkinnyColsWaves, 2) void GemmSkinnyColsKernel
     *reinterpret_cast<float4_t*>(&extra_sums[((wave * 4 + lane_g) * EXTRA + c) * PITCH + lane_row]) = extra_acc[c];
   }
   __syncthreads();
-  // thread t adds the piece (col, rows 4 q .. 4 q + 3), t = 16 col + q, of all wavefronts in their order; with two
-  // blocks of columns every thread has a piece, with one block the first half of the threads
-  const int col = tid / 16, q = tid % 16;
-  const bool has_piece = col < COLS;
-  const int row = row0 + 4 * q;
+  // thread t adds its piece of all wavefronts in their order
   float4_t total = float4_t(0.0f);
   if (has_piece && col < BLOCK_COLS) {
 #pragma unroll
@@ -241,28 +265,16 @@ __global__ __launch_bounds__(64 * kSkinnyColsWaves, 2) void GemmSkinnyColsKernel
 #pragma unroll
     for (int w = 0; w < WAVES * 4; ++w) { total += *reinterpret_cast<const float4_t*>(&extra_sums[(w * EXTRA + col - BLOCK_COLS) * PITCH + 4 * q]); }
   }
-  const bool stores = has_piece && col < p.small && row < p.extent;
   auto finish = [&](const float4_t sum) {  // C = alpha * sum + beta * C for the thread's piece
-    float* target = p.c + row * p.c_row_stride + col * p.c_col_stride;
-    if (p.c_row_stride == 1 && row + 3 < p.extent) {
-      typedef float float4u_t __attribute__((ext_vector_type(4), aligned(4)));
-      float4u_t out;
-      if (p.beta != 0.0f) {
-        const float4u_t old = *reinterpret_cast<const float4u_t*>(target);
+    float4_t out;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { out[e] = Combine(p.alpha, sum[e], p.beta, old[e]); }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) { out[e] = p.alpha * sum[e]; }
-      }
-      *reinterpret_cast<float4u_t*>(target) = out;
+    for (int e = 0; e < 4; ++e) { out[e] = (p.beta != 0.0f) ? Combine(p.alpha, sum[e], p.beta, old_c[e]) : p.alpha * sum[e]; }
+    if (whole_piece) {
+      *reinterpret_cast<float4u_t*>(c_piece) = out;
     } else {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        if (row + e < p.extent) {
-          float* element = target + e * p.c_row_stride;
-          *element = (p.beta != 0.0f) ? Combine(p.alpha, sum[e], p.beta, *element) : p.alpha * sum[e];
-        }
+        if (row + e < p.extent) { c_piece[e * p.c_row_stride] = out[e]; }
       }
     }
   };
