@@ -13,7 +13,12 @@ int LaunchSmallBatchedVariant(const clbh_gemm_desc& d, hipStream_t stream) {
   using CT = typename ComputeType<T>::type;
   const auto args = MakeArgs<CT>(d);
   constexpr int WAVES = SmallTraits<T>::WAVES;
-  const int groups = (d.batch_count + WAVES - 1) / WAVES;
+  // (no more work-groups than stay resident together, four per compute unit: their wavefronts walk the batch.
+  // 8192 x 32^3 fp32: 17.6 us with a work-group per four matrices, 16.7 us with 1024 work-groups, 17.3 us with 512;
+  // requesting a wavefront's next matrix under the products of the current one made it slower, 18.2 us)
+  int units = 256;
+  if (clbh_compute_units(&units) != 0 || units <= 0) { units = 256; }
+  const int groups = std::min((d.batch_count + WAVES - 1) / WAVES, 4 * units);
   GemmSmallBatchedKernel<T, A_KC, B_KC, FAST><<<dim3(static_cast<unsigned>(groups)), dim3(64 * WAVES), 0, stream>>>(args);
   return static_cast<int>(hipGetLastError());
 }
