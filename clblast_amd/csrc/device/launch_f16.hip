@@ -154,11 +154,12 @@ int LaunchHwide(const clbh_gemm_desc& d, hipStream_t stream) {
 }
 
 // Which form of the 256 x 256 tile a launch takes: 0 the eight-wavefront kernel, 1 the wide kernel without range
-// checks (whole tiles, K a multiple of 128), 2 the wide kernel with them. The wide kernel moves C in 16-byte pieces
-// only and addresses with 32-bit byte offsets; measured against the eight-wavefront kernel it gains 5 to 10 % on whole
-// tiles from k = 256 on (8192^2 x 256 85 -> 79 us, 8192^3 N/T 0.815 -> 0.747 ms, 4096^3 115 -> 108 us), with range checks
-// only under a long K walk of two x-contiguous operands (5000^3 N/T 272 -> 253 us; 8192^2 x 1312, whose K it pads to
-// 1408, 177 -> 208 us; with a k-contiguous operand it loses 5 to 40 %).
+// checks (whole tiles, K a multiple of 128), 2 the wide kernel with them. The wide kernel moves C in 16-byte pieces of
+// eight rows and addresses with 32-bit byte offsets. Measured against the eight-wavefront kernel (same box, us): whole
+// tiles 8192^2 x 256 67 / 85, x 1024 130 / 157, 8192^3 N/T 755 / 832, 4096^3 106 / 118, with a k-contiguous operand
+// 8192^2 x 256 71 / 85; with range checks and two x-contiguous operands 4096^2 x 1000 38 / 44, 5000^3 222 / 267,
+// 8192^2 x 1312 163 / 174 (K padded to 1408); with range checks and a k-contiguous operand it loses (5000^3 T/N 311 /
+// 289).
 int WideForm(const clbh_gemm_desc& d) {
   if (d.conv != nullptr || d.c_triangle != 0 || d.operand_triangle != 0 || PlanSplit(d).splits > 1) { return 0; }
   constexpr long long kMaxLd = 1ll << 21;
@@ -167,8 +168,9 @@ int WideForm(const clbh_gemm_desc& d) {
   if (c_address % 4 != 0) { return 0; }
   if (d.batch_count > 1 && (d.batch.alphas != nullptr || d.c_stride % 2 != 0)) { return 0; }
   if ((d.a_kcontig || d.b_kcontig) && d.k % 8 != 0) { return 0; }
+  if (d.m % 8 != 0) { return 0; }  // (C moves in pieces of eight rows)
   if (d.m % HwideConfig::TILE_M == 0 && d.n % HwideConfig::TILE_N == 0 && d.k % (HwideConfig::TILE_K * HwideConfig::STAGES) == 0) { return 1; }
-  return (!d.a_kcontig && !d.b_kcontig && d.k >= 2048) ? 2 : 0;
+  return (!d.a_kcontig && !d.b_kcontig && d.k >= 1000) ? 2 : 0;
 }
 
 // CONVGEMM with the A operand gathered from the images (clbh_gemm_desc::conv; HGatherPiece names the conditions): the

@@ -145,12 +145,21 @@ __device__ __forceinline__ double Combine(const double alpha, const double acc, 
   return __builtin_fma(beta, old, alpha * acc);
 }
 
+// An epilogue's result in the storage type. A narrowing conversion (fp32 sums, fp16 storage) first hides the value
+// from the compiler: it would otherwise fuse the last multiply-add with the conversion in some code paths (one
+// rounding) and not in others (two), and an element's last bit would depend on the kernel that stored it.
+template <typename T, typename CT>
+__device__ __forceinline__ T Narrow(CT value) {
+  if constexpr (sizeof(T) < sizeof(CT)) { asm("" : "+v"(value)); }
+  return static_cast<T>(value);
+}
+
 template <typename T, typename CT>
 __device__ __forceinline__ void StoreResult(T* c, const long long index, const CT acc, const CT alpha, const CT beta) {
   if (beta == CT(0)) {
-    c[index] = static_cast<T>(alpha * acc);
+    c[index] = Narrow<T, CT>(alpha * acc);
   } else {
-    c[index] = static_cast<T>(Combine(alpha, acc, beta, static_cast<CT>(c[index])));
+    c[index] = Narrow<T, CT>(Combine(alpha, acc, beta, static_cast<CT>(c[index])));
   }
 }
 

@@ -589,10 +589,10 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmDirec
               if (beta != 0.0f) {
                 const half4_t old = *cell;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { out[e] = static_cast<T>(Combine(alpha, acc[i][2 * j + jj][e], beta, static_cast<float>(old[e]))); }
+                for (int e = 0; e < 4; ++e) { out[e] = Narrow<T, float>(Combine(alpha, acc[i][2 * j + jj][e], beta, static_cast<float>(old[e]))); }
               } else {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { out[e] = static_cast<T>(alpha * acc[i][2 * j + jj][e]); }
+                for (int e = 0; e < 4; ++e) { out[e] = Narrow<T, float>(alpha * acc[i][2 * j + jj][e]); }
               }
               *cell = out;
             }

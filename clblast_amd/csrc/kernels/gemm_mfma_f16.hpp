@@ -320,10 +320,10 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
               if (beta != 0.0f) {
                 const half4_t old = *cell;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { out[e] = static_cast<T>(Combine(alpha, acc[i][j][4 * g + e], beta, static_cast<float>(old[e]))); }
+                for (int e = 0; e < 4; ++e) { out[e] = Narrow<T, float>(Combine(alpha, acc[i][j][4 * g + e], beta, static_cast<float>(old[e]))); }
               } else {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { out[e] = static_cast<T>(alpha * acc[i][j][4 * g + e]); }
+                for (int e = 0; e < 4; ++e) { out[e] = Narrow<T, float>(alpha * acc[i][j][4 * g + e]); }
               }
               *cell = out;
             }

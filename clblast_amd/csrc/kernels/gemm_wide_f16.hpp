@@ -24,10 +24,13 @@
 //     immediates) and K is padded to a multiple of 128 with slabs beyond the operand, which the range check of
 //     the buffer loads turns into zeros without touching memory;
 //   * every MFMA is followed by at most one LDS read or one request: with a single wavefront per SIMD nothing
-//     else fills the issue slots.
+//     else fills the issue slots;
+//   * C moves straight between memory and the accumulators' values in 16-byte pieces (v_permlane16_swap gathers eight
+//     consecutive rows of a column in one lane): for the length of the epilogue the matrix pipe stands still, and an
+//     epilogue staged through LDS - thirteen, later three LDS round trips per 16 columns - took 11 us of a tile's 187.
 // Requirements (the launcher checks them): dword-aligned operands, no triangles, no split-K, no gathered
 // operand; a k-contiguous operand needs k % 8 == 0 (its K tail is cut by giving whole 16-byte chunks an
-// offset outside the buffer's range).
+// offset outside the buffer's range); m % 8 == 0 (C moves in pieces of eight rows, each inside the matrix or not).
 // =================================================================================================
 #ifndef CLBLAST_HIP_KERNELS_GEMM_WIDE_F16_HPP_
 #define CLBLAST_HIP_KERNELS_GEMM_WIDE_F16_HPP_
@@ -46,9 +49,9 @@ struct HwideConfig {
   static constexpr int ROUNDS = 2 * PIECES / WAVES;  // requests per wavefront and slab: four for A, then four for B
   static constexpr int OPERAND_ELEMS = 256 * 32;    // halfs of one operand's slab
   static constexpr int RING_BYTES = STAGES * 2 * OPERAND_ELEMS * 2;
-  static constexpr int WAVE_M = 128, STAGE_PITCH = WAVE_M + 8;
-  static constexpr int STAGING_BYTES = WAVES * 16 * STAGE_PITCH * 2;  // the epilogue's tiles of 16 columns, one per wavefront
-  static constexpr int LDS_BYTES = RING_BYTES + STAGING_BYTES;        // beside the ring: it is refilled under the epilogue
+  static constexpr int WAVE_M = 128;
+  static constexpr int OLD_C_BYTES = WAVES * 8 * 1024;  // one strip of old C per wavefront (eight pieces of 16 bytes per lane)
+  static constexpr int LDS_BYTES = RING_BYTES + OLD_C_BYTES;
   static constexpr int STORES = 32;                                   // 16-byte stores per wavefront and tile
 };
 
@@ -77,6 +80,24 @@ __device__ __forceinline__ void WideMfmaDrain(wide_acc_t (&acc)[8][8]) {
   }
 }
 
+// v_permlane16_swap: of two registers, the odd rows of 16 lanes of the first change places with the even rows of the
+// second (rows 0..3 of `first` become first.0, second.0, first.2, second.2; of `second`: first.1, second.1, first.3,
+// second.3). Four pairs at once, written as instructions (their inputs come from instructions the compiler does not
+// know either) between the wait states that the compiler places for the builtin: two between a vector instruction's
+// result and this instruction's read of it, two between its results and a vector instruction that reads them.
+__device__ __forceinline__ void WidePermlane16Swap(float (&first)[4], float (&second)[4]) {
+  asm volatile(
+      "s_nop 1\n\tv_permlane16_swap_b32 %0, %4\n\tv_permlane16_swap_b32 %1, %5\n\tv_permlane16_swap_b32 %2, %6\n\t"
+      "v_permlane16_swap_b32 %3, %7\n\ts_nop 1"
+      : "+v"(first[0]), "+v"(first[1]), "+v"(first[2]), "+v"(first[3]), "+v"(second[0]), "+v"(second[1]), "+v"(second[2]), "+v"(second[3]));
+}
+
+#ifdef WIDE_TIMELINE
+__device__ long long wide_timeline[256 * 64];
+#define WIDE_MARK(i) { asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(marks[i]) :: "memory"); }
+#else
+#define WIDE_MARK(i)
+#endif
 // RANGE: range-checked requests (some tile touches an edge of the matrix, or K is not a multiple of 128); without,
 // every tile is whole and the byte count per slab and operand is saved.
 //
@@ -103,11 +124,11 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
   T* lds = reinterpret_cast<T*>(lds_raw);
   T* a_ring = lds;                         // [STAGES][ELEMS]
   T* b_ring = lds + STAGES * ELEMS;        // [STAGES][ELEMS]
-  T* staging = lds + 2 * STAGES * ELEMS;   // [WAVES][16][STAGE_PITCH]
 
   const int tid = threadIdx.x;
   const int lane = tid % 64, wave = tid / 64;
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  T* old_c_lds = lds + 2 * STAGES * ELEMS + wave_u * 4096;  // [8 pieces][64 lanes][8]: the last strip of old C of this wavefront
   const int wave_m = wave_u % Config::WM, wave_n = wave_u / Config::WM;  // (uniform: C is addressed through a buffer view per wavefront)
   const int tiles = tiles_m * tiles_n, items = tiles * p.batch_count;
 
@@ -182,46 +203,71 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
     request_k += TILE_K;
     refresh_resources();
   };
-  // The first turn of the ring of `item` (without the range check K is a multiple of 128: all four slabs exist)
-  auto request_first_turn = [&](const int wanted) {
-    request_open = (wanted < items) ? -1 : 0;
-    const int item = (wanted < items) ? wanted : 0;
-    const int batch = item / tiles;
+  // The slabs of all items of a work-group form ONE stream through the ring: the last turn of an item's walk requests
+  // the first four slabs of the next item (without the range check K is a multiple of 128: they all exist) at the usual
+  // pace, one request per eight MFMAs - requested in one go between walk and epilogue, those 128 KiB per CU kept the
+  // vector memory pipe of the CU busy for 1.8 us with nothing to multiply. Where the next item's operands lie is worked
+  // out ahead of the walk (scalar arithmetic with a few divisions and, for batches, loads of pointers).
+  const T* planned_a = nullptr;
+  const T* planned_b = nullptr;
+  const T* planned_a_end = nullptr;
+  const T* planned_b_end = nullptr;
+  int planned_open = 0;
+  auto plan_first_turn = [&](const int wanted) {
+    planned_open = (wanted < items) ? -1 : 0;
+    const int planned_item = (wanted < items) ? wanted : 0;
+    const int batch = planned_item / tiles;
     int tile_m, tile_n;
-    TileOfBlock(item - batch * tiles, tiles, tiles_m, tiles_n, tile_m, tile_n);
+    TileOfBlock(planned_item - batch * tiles, tiles, tiles_m, tiles_n, tile_m, tile_n);
     const T* a;
     const T* b;
     T* c;
     float alpha, beta;
     ResolveBatch<T, float>(p, batch, a, b, c, alpha, beta);
-    a_request = a + (A_KC ? tile_m * TILE_M * p.a_ld : static_cast<long long>(tile_m * TILE_M));  // element (m0, k = 0), uniform
-    b_request = b + (B_KC ? tile_n * TILE_N * p.b_ld : static_cast<long long>(tile_n * TILE_N));
-    a_end = a + (A_KC ? (p.m - 1) * p.a_ld + k_len : (k_len - 1) * p.a_ld + p.m);
-    b_end = b + (B_KC ? (p.n - 1) * p.b_ld + k_len : (k_len - 1) * p.b_ld + p.n);
+    planned_a = a + (A_KC ? tile_m * TILE_M * p.a_ld : static_cast<long long>(tile_m * TILE_M));  // element (m0, k = 0), uniform
+    planned_b = b + (B_KC ? tile_n * TILE_N * p.b_ld : static_cast<long long>(tile_n * TILE_N));
+    planned_a_end = a + (A_KC ? (p.m - 1) * p.a_ld + k_len : (k_len - 1) * p.a_ld + p.m);
+    planned_b_end = b + (B_KC ? (p.n - 1) * p.b_ld + k_len : (k_len - 1) * p.b_ld + p.n);
+  };
+  auto switch_requests = [&]() {  // from here on the requests fetch the planned item, from its slab 0 on
+    request_open = planned_open;
+    a_request = planned_a;
+    b_request = planned_b;
+    a_end = planned_a_end;
+    b_end = planned_b_end;
     request_k = 0;
     refresh_resources();
-#pragma unroll
-    for (int s = 0; s < STAGES; ++s) {
-#pragma unroll
-      for (int round = 0; round < ROUNDS; ++round) { request(round, s); }
-      next_request_slab();
-    }
   };
 
-  constexpr int WAVE_M = Config::WAVE_M, STAGE_PITCH = Config::STAGE_PITCH;
-  constexpr int LANES_PER_ROW = WAVE_M / 8, ROWS_PER_PASS = 64 / LANES_PER_ROW, PASSES = 32 / ROWS_PER_PASS, STRIPS = BN / 2;
-  static_assert(STRIPS * PASSES == Config::STORES, "stores per wavefront and tile");
-  const int c_first_row = lane / LANES_PER_ROW, c_col = 8 * (lane % LANES_PER_ROW);
-  const int c_lane_offset = (c_first_row * static_cast<int>(p.c_ld) + c_col) * 2;
-  const int c_pass_bytes = ROWS_PER_PASS * static_cast<int>(p.c_ld) * 2;
-  // strip 0 of old C comes in under the first three slabs of the last turn (3, 3 and 2 loads), strip 1 under the fourth,
-  // whose MFMAs need no fragments of a next slab any more
-  constexpr int EARLY_STRIPS = 2;
-  constexpr int kEarlyBefore[STAGES + 1] = {0, 3, 6, 8, 8};  // loads of old C issued before slab ST of the last turn
+  // C moves in pieces of 16 bytes, eight consecutive m of one column, straight between memory and the accumulators' values:
+  // of two blocks of rows, 2 q and 2 q + 1, a lane holds rows 4 g + r (g = lane / 16, r = 0..3) of each; one
+  // v_permlane16_swap per register exchanges the odd rows of 16 lanes of the one with the even rows of the other, and
+  // the lane then holds the eight rows 16 (g % 2) + 8 (g / 2) + 0..7 of the pair's 32, all of column lane % 16. A
+  // wavefront's 128 x 128 part is four strips of 32 columns; a strip is eight pieces per lane (piece: block of 16
+  // columns pass / 4 of the strip, pair of row blocks pass % 4).
+  constexpr int WAVE_M = Config::WAVE_M;
+  constexpr int PASSES = 8, STRIPS = BN / 2;
+  static_assert(STRIPS * PASSES == Config::STORES && BM == 8, "stores per wavefront and tile");
+  const int c_lane_m = 16 * ((lane / 16) % 2) + 8 * (lane / 32);
+  const int c_lane_offset = ((lane % 16) * static_cast<int>(p.c_ld) + c_lane_m) * 2;
+  const int c_block_bytes = 16 * static_cast<int>(p.c_ld) * 2;  // from one block of 16 columns to the next
+  // All of old C is asked for under the last turn of the walk, two microseconds (a load's latency under this load)
+  // before the epilogue wants it: strip 0 under the first three slabs (3, 3 and 2 loads) into registers the walk leaves
+  // free, strips 1 and 2 under the fourth, whose MFMAs need no fragments of a next slab any more (one set of fragment
+  // registers is idle there), strip 3 under the second and third slab straight into LDS (four loads each).
+  constexpr int kEarlyStrip0[STAGES + 1] = {0, 3, 6, 8, 8};      // loads of strip 0 issued before slab ST of the last turn
+  constexpr int kEarlyBefore[STAGES + 1] = {0, 3, 10, 16, 16};   // all loads of old C issued before slab ST of the last turn
 
   int item = blockIdx.x;
   if (item >= items) { return; }
-  request_first_turn(item);
+  plan_first_turn(item);
+  switch_requests();
+#pragma unroll
+  for (int slab = 0; slab < STAGES; ++slab) {
+#pragma unroll
+    for (int round = 0; round < ROUNDS; ++round) { request(round, slab); }
+    next_request_slab();
+  }
   {
     // as many stores as an epilogue issues, into a view of no bytes: they move nothing and take their places in the queue
     const auto nothing = __builtin_amdgcn_make_buffer_rsrc(static_cast<T*>(p.c), 0, 0, kRawBufferFlags);
@@ -232,7 +278,15 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
     for (int i = 0; i < Config::STORES; ++i) { BufferStore<T, 8>(zeros, nothing, 0); }
   }
 
+#ifdef WIDE_TIMELINE
+  int ordinal = -1;
+#endif
   for (; item < items; item += gridDim.x) {
+#ifdef WIDE_TIMELINE
+    ++ordinal;
+    long long marks[6];
+#endif
+    WIDE_MARK(0);
     // the tile of C of this item
     const int batch = item / tiles;
     int tile_m, tile_n;
@@ -246,80 +300,93 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
       ResolveBatch<T, float>(p, batch, a, b, c, alpha, beta);
     }
     wide_acc_t acc[BM][BN];  // written by the first slab
+    plan_first_turn(item + gridDim.x);
 
-    // Old C. The wavefront's 128 x 128 part of the tile is handled as four strips of 32 columns; a strip moves in eight
-    // passes of 16 bytes per lane (lane: 8 consecutive m, pass g: columns 4 g + lane / 16 of the strip). The first two
-    // strips are fetched under the MFMAs of the last turn of the K walk, into registers the walk leaves free, the other
-    // two right behind the walk into the registers of the fragments. With beta == 0 the same loads run with an offset
-    // outside the view (no memory is touched), so the code and the count of loads in flight do not depend on beta.
+    // Old C. The first two strips are fetched under the MFMAs of the last turn of the K walk, into registers the walk
+    // leaves free, the other two right behind the walk into the registers of the fragments. With beta == 0 the same
+    // loads run with an offset outside the view (no memory is touched), so the code and the count of loads in flight
+    // do not depend on beta.
     const int wave_m0 = m0 + wave_m * WAVE_M, wave_n0 = n0 + wave_n * (BN * 16);
     const auto c_view = __builtin_amdgcn_make_buffer_rsrc(c + wave_n0 * p.c_ld + wave_m0, 0, kHOutside, kRawBufferFlags);
-    const int c_inside = p.m - (wave_m0 + c_col);   // how many of the lane's eight m lie inside the matrix
-    const int c_rows_left = p.n - wave_n0;          // columns of C from the wavefront's first one to the matrix's edge
-    const auto c_piece_there = [&](const int strip, const int pass) {
-      return !RANGE || ((32 * strip + pass * ROWS_PER_PASS + c_first_row < c_rows_left) && c_inside >= 8);
+    const int c_inside = p.m - (wave_m0 + c_lane_m);   // rows of C from the lane's first one (of pair 0) to the matrix's edge
+    const int c_cols_left = p.n - wave_n0 - lane % 16; // columns of C from the lane's first one to the matrix's edge
+    const auto c_uniform = [&](const int strip, const int pass) { return (2 * strip + pass / 4) * c_block_bytes + 64 * (pass % 4); };
+    const auto c_piece_there = [&](const int strip, const int pass) {  // all eight rows of the piece inside the matrix
+      return !RANGE || (16 * (2 * strip + pass / 4) < c_cols_left && c_inside - 32 * (pass % 4) >= 8);
     };
     const auto c_load = [&](const int strip, const int pass) {
-      const int uniform = (strip * PASSES + pass) * c_pass_bytes;
-      if (RANGE) { return BufferLoad<T, 8>(c_view, (beta != 0.0f && c_piece_there(strip, pass)) ? c_lane_offset + uniform : kHOutside); }
-      return BufferLoad<T, 8>(c_view, (beta != 0.0f) ? c_lane_offset : kHOutside, uniform);
+      if (RANGE) { return BufferLoad<T, 8>(c_view, (beta != 0.0f && c_piece_there(strip, pass)) ? c_lane_offset + c_uniform(strip, pass) : kHOutside); }
+      return BufferLoad<T, 8>(c_view, (beta != 0.0f) ? c_lane_offset : kHOutside, c_uniform(strip, pass));
     };
-    half8_t old_c[STRIPS][PASSES];
+    const auto c_load_to_lds = [&](const int pass) {  // piece `pass` of strip 3: lane l's 16 bytes land at old_c_lds[pass][l]
+      // (every operand of the load worked out beforehand: with a call among the load's own arguments the host pass of
+      // the compiler drops this kernel's launch stub without a word)
+      const bool wanted = beta != 0.0f && c_piece_there(STRIPS - 1, pass);
+      const int piece_offset = c_lane_offset + c_uniform(STRIPS - 1, pass);
+      const int offset = wanted ? piece_offset : kHOutside;
+      LdsPtr place = (LdsPtr)(old_c_lds + pass * 512);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(c_view, place, 16, offset, 0, 0, 0);
+    };
+    half8_t old_c[STRIPS - 1][PASSES];
 
     {
-      // slab 0 of this item has landed (behind it in the queue: three slabs and the stores of the previous epilogue)
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 1) * ROUNDS + PENDING) : "memory");
-      __syncthreads();
+      // the first four slabs of this item have landed: the youngest operations in the queue are the stores of the
+      // previous epilogue (or the stores that stand in for them ahead of the first item), all requests are older
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PENDING) : "memory");
+      WIDE_MARK(1);
       half8_t a_frag[2][BM], b_frag[2][BN];
 #pragma unroll
       for (int q = 0; q < BM; ++q) { a_frag[0][q] = HFragment<TILE_M, A_KC>(a_read[q], 0); }
 #pragma unroll
       for (int q = 0; q < BN; ++q) { b_frag[0][q] = HFragment<TILE_N, B_KC>(b_read[q], 0); }
 
-      // One slab in ring position ST (compile time). LAST: the final turn of the ring - nothing is requested any more
-      // and the waits count what is still in flight. TURN1: the first turn - the stores of the previous epilogue stand
-      // in the queue behind the requests of this turn's slabs.
+      // One slab in ring position ST (compile time): wait and barrier, 64 MFMAs with the fragment reads of the next slab,
+      // the requests for the slab four further on (in the last turn: of the next item) and, in the last turn, the first
+      // loads of old C between them. TURN1: the first turn of an item - its slabs have landed, but what it requests
+      // stands behind the previous epilogue's stores in the queue.
       auto slab_body = [&](auto stage_tag, auto last_tag, auto first_tag, auto turn1_tag) {
         constexpr int ST = decltype(stage_tag)::value;
         constexpr bool LAST = decltype(last_tag)::value;
         constexpr bool FIRST = decltype(first_tag)::value;  // the very first slab: the accumulators start here
         constexpr bool TURN1 = decltype(turn1_tag)::value;
         constexpr int CUR = ST % 2, NXT = 1 - CUR, NEXT_ST = (ST + 1) % STAGES;
-        // my requests for the next slab have landed (two later slabs may stay in flight), my reads of this slab are done
-        // (in the last turn the loads of old C issued under its earlier slabs stand behind the requests in the queue)
-        constexpr int IN_FLIGHT = (LAST ? (ST + 2 < STAGES ? (STAGES - 2 - ST) * ROUNDS : 0) + kEarlyBefore[ST] : 2 * ROUNDS) +
-                                  ((TURN1 && ST + 1 < STAGES) ? PENDING : 0);
+        constexpr bool READS_NEXT = !(LAST && ST == STAGES - 1);  // (the next item's first fragments are read at its top)
+        // My requests for the next slab have landed - the requests of two later slabs may stay in flight, and so may the
+        // loads of old C issued since (last turn) -, my reads of this slab are done. Nothing to wait for where the next
+        // slab is one of the item's first four, or is not read here.
+        constexpr int IN_FLIGHT = ((TURN1 && ST + 1 < STAGES) || !READS_NEXT) ? 63 : 2 * ROUNDS + (LAST ? kEarlyBefore[ST] : 0);
         static_assert(IN_FLIGHT < 64, "the counter of memory operations holds six bits");
-        if (!(LAST && ST == STAGES - 1)) {
-          asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::"n"(IN_FLIGHT) : "memory");
-        }
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::"n"(IN_FLIGHT) : "memory");
 #pragma unroll
         for (int i = 0; i < BM; ++i) {
 #pragma unroll
           for (int j = 0; j < BN; ++j) {
             const int n = i * BN + j;
             WideMfma<FIRST>(acc[i][j], a_frag[CUR][i], b_frag[CUR][j]);
-            if (!(LAST && ST == STAGES - 1) && n % 4 == 1) {  // one fragment of the next slab per four MFMAs: B first
+            if (READS_NEXT && n % 4 == 1) {  // one fragment of the next slab per four MFMAs: B first
               const int f = n / 4;
               if (f < BN) { b_frag[NXT][f] = HFragment<TILE_N, B_KC>(b_read[f], NEXT_ST * ELEMS); }
               else { a_frag[NXT][f - BN] = HFragment<TILE_M, A_KC>(a_read[f - BN], NEXT_ST * ELEMS); }
             }
-            if (!LAST && n % 8 == 7) { request(n / 8, ST); }
-            if (LAST && ST < STAGES - 1 && n % 16 == 11 && kEarlyBefore[ST] + n / 16 < kEarlyBefore[ST + 1]) {
-              const int piece = kEarlyBefore[ST] + n / 16;
+            if (n % 8 == 7) { request(n / 8, ST); }
+            if (LAST && ST < STAGES - 1 && n % 16 == 11 && kEarlyStrip0[ST] + n / 16 < kEarlyStrip0[ST + 1]) {
+              const int piece = kEarlyStrip0[ST] + n / 16;
               old_c[0][piece] = c_load(0, piece);
             }
+            if (LAST && (ST == 1 || ST == 2) && n % 16 == 3) { c_load_to_lds(4 * (ST - 1) + n / 16); }
             if (LAST && ST == STAGES - 1 && n % 8 == 3) { old_c[1][n / 8] = c_load(1, n / 8); }
+            if (LAST && ST == STAGES - 1 && n % 8 == 5) { old_c[2][n / 8] = c_load(2, n / 8); }  // (into the idle set of fragment registers)
             __builtin_amdgcn_sched_barrier(0);
           }
         }
-        if (!LAST) { next_request_slab(); }
+        next_request_slab();
       };
       using std::integral_constant;
       using std::false_type;
       using std::true_type;
       asm volatile("; WIDE_WALK_BEGIN" ::: "memory");
       if (groups == 1) {
+        switch_requests();
         slab_body(integral_constant<int, 0>{}, true_type{}, true_type{}, true_type{});
         slab_body(integral_constant<int, 1>{}, true_type{}, false_type{}, true_type{});
         slab_body(integral_constant<int, 2>{}, true_type{}, false_type{}, true_type{});
@@ -335,6 +402,7 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
           slab_body(integral_constant<int, 2>{}, false_type{}, false_type{}, false_type{});
           slab_body(integral_constant<int, 3>{}, false_type{}, false_type{}, false_type{});
         }
+        switch_requests();
         slab_body(integral_constant<int, 0>{}, true_type{}, false_type{}, false_type{});
         slab_body(integral_constant<int, 1>{}, true_type{}, false_type{}, false_type{});
         slab_body(integral_constant<int, 2>{}, true_type{}, false_type{}, false_type{});
@@ -342,118 +410,62 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
       }
       asm volatile("; WIDE_WALK_END" ::: "memory");
       WideMfmaDrain(acc);
+      WIDE_MARK(2);
     }
 
-    // Epilogue, staged through LDS so that global memory sees whole lines: per half strip (16 columns) a wavefront fills
-    // its [16 n][128 m] fp16 staging tile; old C goes in with 16 bytes per lane, every lane combines its four consecutive
-    // m per block in fp32 and rounds once, the finished rows leave with 16-byte stores. Only wavefront-local ordering is
-    // needed (the LDS operations of a wavefront complete in order).
+    // Epilogue: piece by piece the accumulators' values are exchanged between the rows of lanes (see above), combined
+    // with the old values in fp32, rounded once and stored; no LDS, no dependence between pieces.
     {
-      auto wave_fence = [&]() {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      WIDE_MARK(3);
+      WIDE_MARK(4);
+      auto combine = [&](auto use_c_tag) {
+        constexpr bool USE_C = decltype(use_c_tag)::value;
+#pragma unroll
+        for (int strip = 0; strip < STRIPS; ++strip) {
+#pragma unroll
+          for (int pass = 0; pass < PASSES; ++pass) {
+            const int j = 2 * strip + pass / 4, pair = pass % 4;
+            if (pass % 2 == 0) { __builtin_amdgcn_sched_barrier(0); }  // (the accumulators leave their registers two pieces at a time, not all at once)
+            // (copied to vector registers here, and from nowhere else: with a copy per use the compiler fetches all 256
+            // accumulators at the top of the epilogue and spills what else lives there)
+            float even[4], odd[4];  // rows 4 g + r of the pair's two blocks, then rows 0..3 and 4..7 of the lane's eight
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(even[r]) : "a"(acc[2 * pair][j][r]));
+              asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(odd[r]) : "a"(acc[2 * pair + 1][j][r]));
+            }
+            WidePermlane16Swap(even, odd);
+            float values[8];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { values[r] = even[r]; values[4 + r] = odd[r]; }
+            half8_t old = half8_t(T(0));
+            if (USE_C) {
+              if (strip < STRIPS - 1) {
+                old = old_c[strip][pass];
+              } else {
+                // (its loads into LDS are older than every store: all but the stores of the strips before have completed)
+                if (pass == 0) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STRIPS - 1) * PASSES) : "memory"); }
+                old = *reinterpret_cast<const half8_t*>(old_c_lds + pass * 512 + lane * 8);
+              }
+            }
+            half8_t out;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              if constexpr (USE_C) { out[e] = Narrow<T, float>(Combine(alpha, values[e], beta, static_cast<float>(old[e]))); }
+              else { out[e] = Narrow<T, float>(alpha * values[e]); }
+            }
+            if (RANGE) { BufferStore<T, 8>(out, c_view, c_piece_there(strip, pass) ? c_lane_offset + c_uniform(strip, pass) : kHOutside); }
+            else { BufferStore<T, 8>(out, c_view, c_lane_offset, c_uniform(strip, pass)); }
+          }
+        }
       };
-#pragma unroll
-      for (int strip = EARLY_STRIPS; strip < STRIPS; ++strip) {
-#pragma unroll
-        for (int g = 0; g < PASSES; ++g) { old_c[strip][g] = c_load(strip, g); }
+      if (beta != 0.0f) { combine(std::true_type{}); } else { combine(std::false_type{}); }
+      WIDE_MARK(5);
+#ifdef WIDE_TIMELINE
+      if (threadIdx.x == 0 && ordinal < 8) {
+        for (int i = 0; i < 6; ++i) { wide_timeline[blockIdx.x * 64 + ordinal * 8 + i] = marks[i]; }
       }
-      __syncthreads();  // every wavefront is done with the slab buffers
-      // the next item's first slabs are requested now, ahead of this item's stores
-      request_first_turn(item + gridDim.x);
-      const bool wave_has_rows = wave_m0 < p.m;
-      // (the lane number once more, opaque: the LDS addresses the epilogue derives from it are then computed here and
-      // not ahead of the K walk, where they would sit in registers all through it)
-      int late_lane = lane;
-      asm volatile("" : "+v"(late_lane));
-      const int late_first_row = late_lane / LANES_PER_ROW, late_col = 8 * (late_lane % LANES_PER_ROW);
-      // RANGE: the piece per row that straddles the last row of C moves element by element
-      const bool straddles = RANGE && c_inside > 0 && c_inside < 8;
-      T* stage = staging + wave_u * (16 * STAGE_PITCH);
-      T* cells = &stage[late_first_row * STAGE_PITCH + late_col];
-      constexpr int HALF_PASSES = PASSES / 2;
-#pragma unroll
-      for (int half_strip = 0; half_strip < 2 * STRIPS; ++half_strip) {
-        const int strip = half_strip / 2, half = half_strip % 2;
-        if (RANGE && !(16 * half_strip < c_rows_left && wave_has_rows)) {  // (uniform) nothing of C here: the stores alone
-          half8_t nothing;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) { nothing[e] = T(0); }
-#pragma unroll
-          for (int g = 0; g < HALF_PASSES; ++g) { BufferStore<T, 8>(nothing, c_view, kHOutside); }
-          continue;
-        }
-        __builtin_amdgcn_sched_barrier(0);  // (the accumulators leave their registers half strip by half strip, not all at once)
-        if (beta != 0.0f) {
-#pragma unroll
-          for (int g = 0; g < HALF_PASSES; ++g) {
-            *reinterpret_cast<half8_t*>(cells + g * ROWS_PER_PASS * STAGE_PITCH) = old_c[strip][half * HALF_PASSES + g];
-          }
-          if (RANGE && wave_m0 + WAVE_M > p.m) {
-#pragma unroll 1
-            for (int g = 0; g < HALF_PASSES; ++g) {
-              const int pass = half * HALF_PASSES + g;
-              const bool there = 32 * strip + pass * ROWS_PER_PASS + c_first_row < c_rows_left && straddles;
-              unsigned short values[7];
-#pragma unroll
-              for (int e = 0; e < 7; ++e) {
-                const int element = (there && e < c_inside) ? c_lane_offset + (strip * PASSES + pass) * c_pass_bytes + 2 * e : kHOutside;
-                values[e] = __builtin_amdgcn_raw_buffer_load_b16(c_view, element, 0, 0);
-              }
-              if (straddles) {
-#pragma unroll
-                for (int e = 0; e < 7; ++e) { cells[g * ROWS_PER_PASS * STAGE_PITCH + e] = __builtin_bit_cast(T, values[e]); }
-              }
-            }
-          }
-          wave_fence();
-        }
-        // (the half strip's accumulators are copied to vector registers here, and from nowhere else: with a copy per
-        // use the compiler fetches all 256 of them at the top of the epilogue and spills what else lives there)
-        float values[BM][4];
-#pragma unroll
-        for (int i = 0; i < BM; ++i) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) { asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(values[i][e]) : "a"(acc[i][half_strip][e])); }
-        }
-#pragma unroll
-        for (int i = 0; i < BM; ++i) {
-          half4_t* cell = reinterpret_cast<half4_t*>(&stage[(late_lane % 16) * STAGE_PITCH + 16 * i + 4 * (late_lane / 16)]);
-          half4_t out;
-          if (beta != 0.0f) {
-            const half4_t old = *cell;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) { out[e] = static_cast<T>(Combine(alpha, values[i][e], beta, static_cast<float>(old[e]))); }
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) { out[e] = static_cast<T>(alpha * values[i][e]); }
-          }
-          *cell = out;
-        }
-        wave_fence();
-#pragma unroll
-        for (int g = 0; g < HALF_PASSES; ++g) {
-          const int pass = half * HALF_PASSES + g;
-          const half8_t row = *reinterpret_cast<const half8_t*>(cells + g * ROWS_PER_PASS * STAGE_PITCH);
-          const int uniform = (strip * PASSES + pass) * c_pass_bytes;
-          if (RANGE) { BufferStore<T, 8>(row, c_view, c_piece_there(strip, pass) ? c_lane_offset + uniform : kHOutside); }
-          else { BufferStore<T, 8>(row, c_view, c_lane_offset, uniform); }
-        }
-        if (RANGE && wave_m0 + WAVE_M > p.m) {
-#pragma unroll 1
-          for (int g = 0; g < HALF_PASSES; ++g) {
-            const int pass = half * HALF_PASSES + g;
-            const bool there = 32 * strip + pass * ROWS_PER_PASS + c_first_row < c_rows_left && straddles;
-#pragma unroll
-            for (int e = 0; e < 7; ++e) {
-              const int element = (there && e < c_inside) ? c_lane_offset + (strip * PASSES + pass) * c_pass_bytes + 2 * e : kHOutside;
-              __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, cells[g * ROWS_PER_PASS * STAGE_PITCH + e]), c_view, element, 0, 0);
-            }
-          }
-        }
-        wave_fence();
-      }
+#endif
     }
   }
 }

@@ -386,7 +386,12 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     // the 64 x 64 tiles 1.6 times there - fitted to 40 random batched shapes, mean loss against the best tile 3.7 % -> 0.9 %;
     // 160 x 178 x 496 x 1355: 364 us on 64 x 64 tiles, 208 us with one 256 x 256 tile per matrix)
     const double batch_128 = (batch_count > 1) ? 1.2 : 1.0, batch_64 = (batch_count > 1) ? 1.6 : 1.0;
-    const auto cost256 = (k >= 256) ? cost(256, 1, 1484.0, 627.0) : 1e300, cost128 = batch_128 * cost(128, 2, 936.0, 293.0),
+    // (where the 256 x 256 tile runs on four wavefronts of 128 x 128 with persistent work-groups - whole tiles with k a
+    // multiple of 128, or two x-contiguous operands from k = 1000 on, rows a multiple of 8; the device layer decides
+    // the same way - it costs less: fitted to 8192^2 x k, k = 256 .. 8192, 1608 TFLOP/s and k0 = 467)
+    const bool wide = triangular == 0 && m % 8 == 0 &&
+                      ((m % 256 == 0 && n % 256 == 0 && k % 128 == 0) || (!a_kcontig && !b_kcontig && k >= 1000));
+    const auto cost256 = (k >= 256) ? cost(256, 1, wide ? 1608.0 : 1484.0, wide ? 467.0 : 627.0) : 1e300, cost128 = batch_128 * cost(128, 2, 936.0, 293.0),
                cost64 = batch_64 * cost(64, 4, long_k ? 371.0 : 488.0, 44.0);
     int tile = 1;
     if (cost256 <= cost128 && cost256 <= cost64) { tile = 2; }
@@ -412,7 +417,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     {
       const auto tiles128 = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
       const bool fills = 10 * TileUse(m, n, 128, 128) >= 9 * TileUse(m, n, 64, 64);
-      if (k <= 320 && tiles128 >= 2048 && fills) { tile = 5; }
+      if (k <= 320 && tiles128 >= 2048 && fills && !(wide && tile == 2)) { tile = 5; }  // (8192^2 x 256 T/N: 69 us that way, 61 us on the wide tile)
       else if (k <= 128 && tiles128 >= 512 && fills) { tile = 0; }
     }
     // One column of tiles (64 <= n <= 128) under a long k and a tall A with contiguous columns: every tile streams its
