@@ -136,7 +136,7 @@ NETLIB_SYMBOLS = (["cblas_%sgemm" % p for p in "sdcz"] +
 DEVICE_LAYER_SYMBOLS = [
     "clbh_gemm_launch", "clbh_gemm_workspace_bytes", "clbh_buffer_extent", "clbh_alloc_async", "clbh_free_async",
     "clbh_upload_async", "clbh_event_record", "clbh_stream_device", "clbh_error_string", "clbh_symmetric_to_square",
-    "clbh_triangular_to_square", "clbh_copy_matrix", "clbh_invert_block_size", "clbh_invert_diagonal_blocks",
+    "clbh_triangular_to_square", "clbh_triangular_to_band", "clbh_complex_triangular_to_band", "clbh_copy_matrix", "clbh_invert_block_size", "clbh_invert_diagonal_blocks",
     "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale", "clbh_complex_expand_batched",
     "clbh_complex_transpose_batched", "clbh_complex_scale_batched", "clbh_complex_gemm_small_batched", "clbh_copy_matrix_batched", "clbh_alloc", "clbh_free", "clbh_copy", "clbh_im2col", "clbh_conv_gather_possible", "clbh_pad_image", "clbh_fill_zero", "clbh_complex_symmetric_to_square",
     "clbh_complex_triangular_to_square", "clbh_complex_zero_diagonal_imag", "clbh_complex_invert_block_size",

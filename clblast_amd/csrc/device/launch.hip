@@ -129,14 +129,14 @@ bool MultipleOf8Bytes(const void* pointer) { return reinterpret_cast<unsigned lo
 template <typename T>
 int LaunchTriangularToSquare(const int upper, const int unit, const int k, const void* src, const long long src_offset,
                              const long long src_ld, void* dst, const int extent, const long long dst_ld,
-                             hipStream_t stream) {
+                             hipStream_t stream, const int leaves = 1) {
   const T* source = static_cast<const T*>(src) + src_offset;
   constexpr int VEC = 8 / sizeof(T);
   const bool vector = VEC > 1 && k % VEC == 0 && extent % VEC == 0 && src_ld % VEC == 0 && dst_ld % VEC == 0 &&
                       MultipleOf8Bytes(source) && MultipleOf8Bytes(dst);
   const int lanes = vector ? (extent + VEC - 1) / VEC : extent;
   const dim3 grid(static_cast<unsigned>((lanes + clbh::kCopyThreads - 1) / clbh::kCopyThreads),
-                  static_cast<unsigned>(std::min(extent, clbh::kCopyMaxGridY)));
+                  static_cast<unsigned>(std::min(extent, clbh::kCopyMaxGridY)), static_cast<unsigned>(leaves));
   if (vector) {
     clbh::TriangularToSquareKernel<T, VEC><<<grid, dim3(clbh::kCopyThreads), 0, stream>>>(
         k, extent, upper != 0, unit != 0, source, src_ld, static_cast<T*>(dst), dst_ld);
@@ -298,12 +298,25 @@ int clbh_triangular_to_square(int precision, int upper, int unit_diagonal, int k
   }
 }
 
+int clbh_triangular_to_band(int precision, int upper, int unit_diagonal, int k, int leaf, const void* src, long long src_offset,
+                            long long src_ld, void* dst, hipStream_t stream) {
+  if (k <= 0 || leaf <= 0 || src == nullptr || dst == nullptr || src_ld < k || src_offset < 0) { return hipErrorInvalidValue; }
+  const int leaves = (k + leaf - 1) / leaf;
+  if (leaves > 65535) { return hipErrorInvalidValue; }
+  switch (precision) {
+    case 16: return LaunchTriangularToSquare<_Float16>(upper, unit_diagonal, k, src, src_offset, src_ld, dst, leaf, leaf, stream, leaves);
+    case 32: return LaunchTriangularToSquare<float>(upper, unit_diagonal, k, src, src_offset, src_ld, dst, leaf, leaf, stream, leaves);
+    case 64: return LaunchTriangularToSquare<double>(upper, unit_diagonal, k, src, src_offset, src_ld, dst, leaf, leaf, stream, leaves);
+    default: return hipErrorInvalidValue;
+  }
+}
+
 int clbh_invert_block_size(int precision) { (void)precision; return 64; }
 
 int clbh_invert_diagonal_blocks(int precision, int upper, int blocks, const void* src, long long src_ld, void* dst,
                                 long long dst_ld, hipStream_t stream) {
-  const long long extent = static_cast<long long>(blocks) * clbh_invert_block_size(precision);
-  if (blocks <= 0 || src == nullptr || dst == nullptr || src_ld < extent || dst_ld < extent) { return hipErrorInvalidValue; }
+  const long long block = clbh_invert_block_size(precision);
+  if (blocks <= 0 || src == nullptr || dst == nullptr || src_ld < block || dst_ld < block) { return hipErrorInvalidValue; }
   switch (precision) {
     case 16: return LaunchInvertDiagonalBlocks<_Float16, float, 64>(upper, blocks, src, src_ld, dst, dst_ld, stream);
     case 32: return LaunchInvertDiagonalBlocks<float, float, 64>(upper, blocks, src, src_ld, dst, dst_ld, stream);
@@ -539,12 +552,11 @@ int clbh_complex_symmetric_to_square(int precision, int upper, int hermitian, in
   return static_cast<int>(hipGetLastError());
 }
 
-int clbh_complex_triangular_to_square(int precision, int upper, int unit_diagonal, int k, const void* src, long long src_offset,
-                                      long long src_ld, void* dst, int dst_extent, long long dst_ld, hipStream_t stream) {
-  if (k <= 0 || src == nullptr || dst == nullptr || src_ld < k || dst_extent < k || dst_ld < dst_extent || src_offset < 0) {
-    return hipErrorInvalidValue;
-  }
-  const dim3 grid(Blocks(dst_extent, clbh::kComplexThreads), static_cast<unsigned>(std::min(dst_extent, 16384)));
+static int LaunchComplexTriangularToSquare(int precision, int upper, int unit_diagonal, int k, const void* src, long long src_offset,
+                                           long long src_ld, void* dst, int dst_extent, long long dst_ld, int leaves,
+                                           hipStream_t stream) {
+  const dim3 grid(Blocks(dst_extent, clbh::kComplexThreads), static_cast<unsigned>(std::min(dst_extent, 16384)),
+                  static_cast<unsigned>(leaves));
   if (precision == 32) {
     clbh::ComplexTriangularToSquareKernel<float><<<grid, dim3(clbh::kComplexThreads), 0, stream>>>(
         k, dst_extent, upper != 0, unit_diagonal != 0, static_cast<const clbh::ComplexOf<float>*>(src) + src_offset, src_ld,
@@ -559,12 +571,28 @@ int clbh_complex_triangular_to_square(int precision, int upper, int unit_diagona
   return static_cast<int>(hipGetLastError());
 }
 
+int clbh_complex_triangular_to_square(int precision, int upper, int unit_diagonal, int k, const void* src, long long src_offset,
+                                      long long src_ld, void* dst, int dst_extent, long long dst_ld, hipStream_t stream) {
+  if (k <= 0 || src == nullptr || dst == nullptr || src_ld < k || dst_extent < k || dst_ld < dst_extent || src_offset < 0) {
+    return hipErrorInvalidValue;
+  }
+  return LaunchComplexTriangularToSquare(precision, upper, unit_diagonal, k, src, src_offset, src_ld, dst, dst_extent, dst_ld, 1, stream);
+}
+
+int clbh_complex_triangular_to_band(int precision, int upper, int unit_diagonal, int k, int leaf, const void* src,
+                                    long long src_offset, long long src_ld, void* dst, hipStream_t stream) {
+  if (k <= 0 || leaf <= 0 || src == nullptr || dst == nullptr || src_ld < k || src_offset < 0) { return hipErrorInvalidValue; }
+  const int leaves = (k + leaf - 1) / leaf;
+  if (leaves > 65535) { return hipErrorInvalidValue; }
+  return LaunchComplexTriangularToSquare(precision, upper, unit_diagonal, k, src, src_offset, src_ld, dst, leaf, leaf, leaves, stream);
+}
+
 int clbh_complex_invert_block_size(int precision) { return (precision == 64) ? 32 : 64; }
 
 int clbh_complex_invert_diagonal_blocks(int precision, int upper, int blocks, const void* src, long long src_ld, void* dst,
                                         long long dst_ld, hipStream_t stream) {
-  const long long extent = static_cast<long long>(blocks) * clbh_complex_invert_block_size(precision);
-  if (blocks <= 0 || src == nullptr || dst == nullptr || src_ld < extent || dst_ld < extent) { return hipErrorInvalidValue; }
+  const long long block = clbh_complex_invert_block_size(precision);
+  if (blocks <= 0 || src == nullptr || dst == nullptr || src_ld < block || dst_ld < block) { return hipErrorInvalidValue; }
   if (precision == 32) {
     return LaunchInvertDiagonalBlocks<clbh::ComplexOf<float>, clbh::ComplexOf<float>, 64>(upper, blocks, src, src_ld, dst, dst_ld, stream);
   }

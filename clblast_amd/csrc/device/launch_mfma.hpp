@@ -40,7 +40,11 @@ int LaunchMfmaVariant(const clbh_gemm_desc& d, hipStream_t stream) {
   auto args = MakeArgs<T>(d);
   const long long tiles_m = (d.m + Config::TILE_M - 1) / Config::TILE_M;
   const long long tiles_n = (d.n + Config::TILE_N - 1) / Config::TILE_N;
-  if (TileBlocks(d, tiles_m, tiles_n) > INT_MAX) { return hipErrorInvalidConfiguration; }
+  // (a triangular operand: the kernel folds the tile rows, or columns, in two - one work-group per pair of tiles)
+  const bool fold_rows = d.c_triangle == 0 && (d.operand_triangle == 1 || d.operand_triangle == 2);
+  const bool fold_columns = d.c_triangle == 0 && d.operand_triangle >= 3;
+  const long long walk_m = fold_rows ? (tiles_m + 1) / 2 : tiles_m, walk_n = fold_columns ? (tiles_n + 1) / 2 : tiles_n;
+  if (TileBlocks(d, walk_m, walk_n) > INT_MAX) { return hipErrorInvalidConfiguration; }
   const auto plan = PlanSplit(d);
   int grid_y = std::min(d.batch_count, kMaxGridY);
   if (plan.splits > 1) {
@@ -53,7 +57,7 @@ int LaunchMfmaVariant(const clbh_gemm_desc& d, hipStream_t stream) {
     args.batch_count = plan.splits;
     grid_y = plan.splits;
   }
-  const dim3 grid(static_cast<unsigned>(TileBlocks(d, tiles_m, tiles_n)), static_cast<unsigned>(grid_y));
+  const dim3 grid(static_cast<unsigned>(TileBlocks(d, walk_m, walk_n)), static_cast<unsigned>(grid_y));
   constexpr size_t lds_bytes = Config::LDS_ELEMS * sizeof(T);
   auto kernel = GemmMfmaKernel<T, Config, A_KC, B_KC, ALIGNED, A_CONV>;
   if (lds_bytes > 48 * 1024) {

@@ -200,16 +200,21 @@ __global__ __launch_bounds__(kComplexThreads) void ComplexSymmetricToSquareKerne
 
 // Dense extent x extent copy (extent >= k, leading dimension dst_ld) of a complex triangular k x k matrix: zeros in the
 // other triangle, ones on an implied diagonal, the identity in rows and columns k .. extent - 1 (reference:
-// src/kernels/level3/convert_triangular.opencl:24-94). grid: (ceil(extent / 256), min(extent, 16384)).
+// src/kernels/level3/convert_triangular.opencl:24-94). grid: (ceil(extent / 256), min(extent, 16384), leaves): layer b
+// of the grid does the same for the rows and columns from b * extent on and writes to dst + b * extent * (dst_ld + 1).
 template <typename R>
-__global__ __launch_bounds__(kComplexThreads) void ComplexTriangularToSquareKernel(const int k, const int extent,
+__global__ __launch_bounds__(kComplexThreads) void ComplexTriangularToSquareKernel(const int k_all, const int extent,
                                                                                    const bool upper, const bool unit,
-                                                                                   const ComplexOf<R>* __restrict__ src,
+                                                                                   const ComplexOf<R>* __restrict__ src_all,
                                                                                    const long long src_ld,
-                                                                                   ComplexOf<R>* __restrict__ dst,
+                                                                                   ComplexOf<R>* __restrict__ dst_all,
                                                                                    const long long dst_ld) {
   const int one = blockIdx.x * kComplexThreads + threadIdx.x;
   if (one >= extent) { return; }
+  const long long first = static_cast<long long>(blockIdx.z) * extent;
+  const int k = static_cast<int>(min(static_cast<long long>(extent), max(0ll, k_all - first)));
+  const ComplexOf<R>* __restrict__ src = src_all + first * (src_ld + 1);
+  ComplexOf<R>* __restrict__ dst = dst_all + first * (dst_ld + 1);
   for (int two = blockIdx.y; two < extent; two += gridDim.y) {
     ComplexOf<R> value;
     value.re = R(0);

@@ -407,9 +407,12 @@ __device__ __forceinline__ void TileOfBlock(const int block, const int num_block
 // owns the tile columns x, x + 8, x + 16, ..., eight consecutive work-groups are eight neighbouring columns of one
 // tile row, and inside its columns each XCD still walks GROUP_M rows at a time (operand reuse in its L2). The grid
 // holds kNumXcd * tiles_m * ceil(tiles_n / kNumXcd) work-groups (see TriangleBlocks in the launchers); the function
-// returns false for the ones beyond the last column.
+// returns false for the ones beyond the last column. `operand_triangle` (kernels that give every tile a work-group of
+// its own pass it): the tiles with the longest K range come first (TriangularRange: the last tile rows for 1, the last
+// tile columns for 3, the first ones for 2 and 4), so that work-groups which start late fill the time the early ones
+// leave instead of ending the launch on the longest tiles.
 __device__ __forceinline__ bool TileOfBlockCyclic(const int block, const int tiles_m, const int tiles_n, int& tile_m,
-                                                  int& tile_n) {
+                                                  int& tile_n, const int operand_triangle = 0) {
   const int xcd = block % kNumXcd, local = block / kNumXcd;
   constexpr int GROUP_M = 8;
   const int columns = (tiles_n + kNumXcd - 1) / kNumXcd;  // tile columns per XCD
@@ -418,8 +421,10 @@ __device__ __forceinline__ bool TileOfBlockCyclic(const int block, const int til
   const int first_m = group * GROUP_M;
   const int group_rows = min(tiles_m - first_m, GROUP_M);
   tile_m = first_m + (local % in_group) % group_rows;
-  tile_n = ((local % in_group) / group_rows) * kNumXcd + xcd;
-  return tile_n < tiles_n;
+  const int column = ((local % in_group) / group_rows) * kNumXcd + xcd;
+  tile_m = (operand_triangle == 1) ? tiles_m - 1 - tile_m : tile_m;
+  tile_n = (operand_triangle == 3) ? tiles_n - 1 - column : column;
+  return column < tiles_n;
 }
 
 // ---- the kernel ------------------------------------------------------------------------------------
@@ -470,391 +475,361 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
   const int lane_x = lane % MF;  // position along the lane dimension of the MFMA block
   const int lane_g = lane / MF;  // k-group of the lane inside one instruction
 
+  // The tile, or the two tiles, of this work-group. With a triangular operand the K range of a tile grows or shrinks
+  // with its row (its column, for the second operand): a launch of one work-group per tile leaves the compute units
+  // that drew short tiles idle (two work-groups that share a compute unit are placed there by their index, so no order
+  // of the walk evens that out). Such launches are folded instead: a work-group takes a tile of the first half of the
+  // rows and then its mirror image in the second half, the two K ranges add up to the same length for every work-group.
   int tile_m, tile_n;
+  int partner_m = -1, partner_n = -1;
   if ((p.c_triangle | p.operand_triangle) != 0) {
-    if (!TileOfBlockCyclic(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n)) { return; }
+    const bool fold_rows = p.c_triangle == 0 && (p.operand_triangle == 1 || p.operand_triangle == 2);
+    const bool fold_columns = p.c_triangle == 0 && p.operand_triangle >= 3;
+    const int walk_m = fold_rows ? (tiles_m + 1) / 2 : tiles_m, walk_n = fold_columns ? (tiles_n + 1) / 2 : tiles_n;
+    if (!TileOfBlockCyclic(blockIdx.x, walk_m, walk_n, tile_m, tile_n)) { return; }
+    if (fold_rows && tiles_m - 1 - tile_m != tile_m) { partner_m = tiles_m - 1 - tile_m; partner_n = tile_n; }
+    if (fold_columns && tiles_n - 1 - tile_n != tile_n) { partner_m = tile_m; partner_n = tiles_n - 1 - tile_n; }
   } else {
     TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
   }
-  const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
-  if (TileOutsideTriangle(p.c_triangle, m0, n0, TILE_M, TILE_N)) { return; }  // uniform: the whole work-group leaves
-  const bool masked = TileCrossesDiagonal(p.c_triangle, m0, n0, TILE_M, TILE_N);
+  for (int pass = 0; pass < 2; ++pass) {
+    if (pass == 1) {
+      if (partner_m < 0) { break; }
+      tile_m = partner_m;
+      tile_n = partner_n;
+      __syncthreads();  // every wavefront has left the LDS buffers of the first tile
+    }
+    const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
+    if (TileOutsideTriangle(p.c_triangle, m0, n0, TILE_M, TILE_N)) { continue; }  // uniform: the whole work-group leaves
+    const bool masked = TileCrossesDiagonal(p.c_triangle, m0, n0, TILE_M, TILE_N);
 
-  // LDS read offsets of this lane. Aligned operands: the lane owns FM consecutive m (one vector LDS read,
-  // one vector store to C). Otherwise C is stored element-wise, and the lane owns m = lane_x, lane_x + MF,
-  // ... so that the lanes of each scalar store cover consecutive addresses.
-  constexpr bool M_INTERLEAVED = ALIGNED;
-  const int a_read = wave_m * (FM * MF) + (M_INTERLEAVED ? lane_x * FM : lane_x);
-  const int b_read = wave_n * (FN * MF) + lane_x * FN;
-  static_assert((KP % LA::R == 0 || LA::R % KP == 0) && (KP % LB::R == 0 || LB::R % KP == 0), "row offsets add up");
-  const int a_lane_row = LA::Row(lane_g) + a_read, b_lane_row = LB::Row(lane_g) + b_read;
+    // LDS read offsets of this lane. Aligned operands: the lane owns FM consecutive m (one vector LDS read,
+    // one vector store to C). Otherwise C is stored element-wise, and the lane owns m = lane_x, lane_x + MF,
+    // ... so that the lanes of each scalar store cover consecutive addresses.
+    constexpr bool M_INTERLEAVED = ALIGNED;
+    const int a_read = wave_m * (FM * MF) + (M_INTERLEAVED ? lane_x * FM : lane_x);
+    const int b_read = wave_n * (FN * MF) + lane_x * FN;
+    static_assert((KP % LA::R == 0 || LA::R % KP == 0) && (KP % LB::R == 0 || LB::R % KP == 0), "row offsets add up");
+    const int a_lane_row = LA::Row(lane_g) + a_read, b_lane_row = LB::Row(lane_g) + b_read;
 
-  // Gathered A: the patches this lane loads (one per part of a tile row), as the top-left corner of the patch in the
-  // padded image and the offset of that corner in the image plane; patches beyond m never pass the bounds test
-  constexpr int GATHER_PARTS = (A_CONV == 1) ? LA::PARTS : 1;
-  int patch_h[GATHER_PARTS], patch_w[GATHER_PARTS], patch_offset[GATHER_PARTS];
-  if constexpr (A_CONV == 2) {  // the lane's four patches: first one at 4 * (lane % 16) of the tile row
-    const int patch = m0 + (lane * 4) % TILE_M;
-    const int oh = patch / p.conv.output_w, ow = patch - oh * p.conv.output_w;
-    patch_offset[0] = (patch < p.m) ? oh * p.conv.stride_h * p.conv.width + ow : -1;
-    patch_h[0] = patch_w[0] = 0;
-  }
-  if constexpr (A_CONV == 1) {
-#pragma unroll
-    for (int part = 0; part < GATHER_PARTS; ++part) {
-      const int patch = m0 + part * LA::WAVE_ELEMS + lane;
+    // Gathered A: the patches this lane loads (one per part of a tile row), as the top-left corner of the patch in the
+    // padded image and the offset of that corner in the image plane; patches beyond m never pass the bounds test
+    constexpr int GATHER_PARTS = (A_CONV == 1) ? LA::PARTS : 1;
+    int patch_h[GATHER_PARTS], patch_w[GATHER_PARTS], patch_offset[GATHER_PARTS];
+    if constexpr (A_CONV == 2) {  // the lane's four patches: first one at 4 * (lane % 16) of the tile row
+      const int patch = m0 + (lane * 4) % TILE_M;
       const int oh = patch / p.conv.output_w, ow = patch - oh * p.conv.output_w;
-      const int corner_h = oh * p.conv.stride_h - p.conv.pad_h;
-      patch_w[part] = ow * p.conv.stride_w - p.conv.pad_w;
-      patch_offset[part] = corner_h * p.conv.width + patch_w[part];
-      patch_h[part] = (patch < p.m) ? corner_h : -(1 << 29);
+      patch_offset[0] = (patch < p.m) ? oh * p.conv.stride_h * p.conv.width + ow : -1;
+      patch_h[0] = patch_w[0] = 0;
     }
-  }
-
-  for (int batch = blockIdx.y; batch < p.batch_count; batch += gridDim.y) {
-    const T* a;
-    const T* b;
-    T* c;
-    T alpha, beta;
-    ResolveBatch<T, T>(p, batch, a, b, c, alpha, beta);
-    int k_len = p.k;
-    long long c_ld = p.c_ld;
-    if (p.split_chunk > 0) {  // this "batch" is one K range of a single problem
-      const int k_begin = batch * p.split_chunk;
-      k_len = min(p.split_chunk, p.k - k_begin);
-      a = static_cast<const T*>(p.a) + p.a_offset + (A_KC ? k_begin : k_begin * p.a_ld);
-      b = static_cast<const T*>(p.b) + p.b_offset + (B_KC ? k_begin : k_begin * p.b_ld);
-      c_ld = p.split_ld;
-      c = static_cast<T*>(p.split_workspace) + static_cast<long long>(batch) * p.split_ld * p.n;
-      alpha = T(1);
-      beta = T(0);
-    } else if (p.operand_triangle != 0) {  // skip the K range in which a triangular operand is zero
-      int k_first;
-      TriangularRange(p.operand_triangle, m0, n0, TILE_M, TILE_N, p.k, k_first, k_len);
-      a += A_KC ? static_cast<long long>(k_first) : k_first * p.a_ld;
-      b += B_KC ? static_cast<long long>(k_first) : k_first * p.b_ld;
-    }
-    const int slabs = (k_len + TILE_K - 1) / TILE_K;
-
-    Acc acc[FM][FN];
+    if constexpr (A_CONV == 1) {
 #pragma unroll
-    for (int i = 0; i < FM; ++i) {
-#pragma unroll
-      for (int j = 0; j < FN; ++j) { acc[i][j] = Traits::Zero(); }
-    }
-
-    // Walk over the slabs, explicitly scheduled so that the matrix pipe never waits at a slab boundary even
-    // with one wavefront per SIMD. Per k-step: LDS reads of the fragments of the NEXT k-step (other
-    // register set), the FM x FN MFMAs of this k-step, then a share of the data movement for the coming
-    // slabs: a direct operand's slab t+1 is requested in the first k-step of slab t; a staged operand
-    // stores its slab t+1 into the other LDS buffer and refills the staging registers with slab t+2. One
-    // barrier per slab, before its last k-step: by then every wavefront has finished its reads of the
-    // current buffer and its writes to the other one, so the last k-step already fetches the first
-    // fragments of slab t+1.
-    const T* a_tile0 = a + (A_KC ? m0 * p.a_ld : static_cast<long long>(m0));  // element (m0, k = 0), uniform
-    const T* b_tile0 = b + (B_KC ? n0 * p.b_ld : static_cast<long long>(n0));
-    // behind the last element of the operand: (x = extent - 1, k = k_len - 1) + 1
-    const T* a_end = a + (A_KC ? (p.m - 1) * p.a_ld + k_len : (k_len - 1) * p.a_ld + p.m);
-    const T* b_end = b + (B_KC ? (p.n - 1) * p.b_ld + k_len : (k_len - 1) * p.b_ld + p.n);
-    const int a_lane_bytes = A_DIRECT ? DirectLaneBytes<T, TILE_M, TILE_K, LANE_BYTES_A>(p.a_ld, lane)
-                                      : static_cast<int>((PA::Line(tid) * p.a_ld + PA::K(tid)) * static_cast<long long>(sizeof(T)));
-    const int b_lane_bytes = B_DIRECT ? DirectLaneBytes<T, TILE_N, TILE_K, LANE_BYTES>(p.b_ld, lane)
-                                      : static_cast<int>((PB::Line(tid) * p.b_ld + PB::K(tid)) * static_cast<long long>(sizeof(T)));
-    auto a_slab = [&](const int k0) { return a_tile0 + (A_KC ? static_cast<long long>(k0) : k0 * p.a_ld); };
-    auto b_slab = [&](const int k0) { return b_tile0 + (B_KC ? static_cast<long long>(k0) : k0 * p.b_ld); };
-    // The walk exists twice: with range-checked loads (tiles that touch an edge of the matrix, or a K
-    // tail), and without (the resources then cover "everything", which saves the scalar arithmetic of one
-    // byte count per load).
-    auto walk = [&](auto range_tag) {
-      constexpr bool RANGE = decltype(range_tag)::value;
-      VP a_stage[STAGED_A > 0 ? STAGED_A : 1], b_stage[STAGED_B > 0 ? STAGED_B : 1];
-      auto load_piece = [&](const int piece, const int k0) {
-        if (piece < STAGED_A) { a_stage[piece] = LoadPiece<T, TILE_M, TILE_K, VL, RANGE>(a_slab(k0), a_end, p.a_ld, a_lane_bytes, piece); }
-        else { b_stage[piece - STAGED_A] = LoadPiece<T, TILE_N, TILE_K, VL, RANGE>(b_slab(k0), b_end, p.b_ld, b_lane_bytes, piece - STAGED_A); }
-      };
-      auto store_piece = [&](const int piece, T* a_dst, T* b_dst, const int k0, auto check_tag) {
-        constexpr bool CHECK = RANGE && decltype(check_tag)::value;
-        if (piece < STAGED_A) {
-          StorePiece<T, TILE_M, TILE_K, LA::GROUP_PITCH, VL, CHECK>(a_dst, tid, piece, a_stage[piece], k_len - k0);
-        } else {
-          StorePiece<T, TILE_N, TILE_K, LB::GROUP_PITCH, VL, CHECK>(b_dst, tid, piece - STAGED_A, b_stage[piece - STAGED_A], k_len - k0);
-        }
-      };
-      // direct loads of one slab, numbered over both operands: A's rounds first
-      constexpr int DIRECT_A = A_DIRECT ? LA::LOADS_PER_WAVE : 0, DIRECT_B = B_DIRECT ? LB::LOADS_PER_WAVE : 0;
-      constexpr int DIRECT = DIRECT_A + DIRECT_B;
-      constexpr int DIRECT_PER_SLOT = (DIRECT + SLOTS - 1) / SLOTS;
-      GatherRows gather_rows{};  // of the slab whose loads are being issued (gathered A only)
-      auto direct_load = [&](const int load, const int k0, auto* a_dst, auto* b_dst) {
-        if constexpr (DIRECT_A > 0) {
-          if (load < DIRECT_A) {
-            if constexpr (A_CONV == 1) {
-              GatherLoad<T, TILE_M, TILE_K, KernelTag>(a, p.conv, a_dst, wave_u, load, gather_rows, patch_h, patch_w, patch_offset);
-            } else if constexpr (A_CONV == 2) {
-              GatherLoadVector<T, TILE_M, TILE_K, KernelTag>(a, p.conv, a_dst, wave_u, load, k0, k_len, lane, patch_offset[0]);
-            } else {
-              DirectLoad<T, TILE_M, TILE_K, LANE_BYTES, RANGE, KernelTag>(a_slab(k0), a_end, p.a_ld, a_dst, wave_u, a_lane_bytes, load);
-            }
-          }
-        }
-        if constexpr (DIRECT_B > 0) {
-          if (load >= DIRECT_A) { DirectLoad<T, TILE_N, TILE_K, LANE_BYTES, RANGE, KernelTag>(b_slab(k0), b_end, p.b_ld, b_dst, wave_u, b_lane_bytes, load - DIRECT_A); }
-        }
-      };
-      auto read_a = [&](const T* stage, const int ks) {
-        const T* src = stage + LA::Row(ks * KP) + a_lane_row;
-        VM av;
-        if constexpr (M_INTERLEAVED) {
-          av = *reinterpret_cast<const VM*>(src);
-        } else {
-#pragma unroll
-          for (int i = 0; i < FM; ++i) { av = VecWith<VM, T, FM>(av, i, src[i * MF]); }
-        }
-        return av;
-      };
-      auto read_b = [&](const T* stage, const int ks) {
-        return *reinterpret_cast<const VN*>(stage + LB::Row(ks * KP) + b_lane_row);
-      };
-
-      // Prologue: slab 0 lands in buffer 0 and slab 1 is requested - its direct loads before the wait for slab 0, so that
-      // the two memory latencies overlap (loads complete in order: when at most the direct loads of slab 1 are
-      // outstanding, everything of slab 0 has arrived); its staged pieces once slab 0 has left the staging registers.
-      if constexpr (A_CONV == 1) { gather_rows = DecomposeRows<TILE_K>(p.conv, 0, k_len, lane); }
-#pragma unroll
-      for (int load = 0; load < DIRECT; ++load) { direct_load(load, 0, a_stages, b_stages); }
-#pragma unroll
-      for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, 0); }
-      if (slabs > 1) {
-        if constexpr (A_CONV == 1) { gather_rows = DecomposeRows<TILE_K>(p.conv, TILE_K, k_len, lane); }
-#pragma unroll
-        for (int load = 0; load < DIRECT; ++load) { direct_load(load, TILE_K, a_stages + LA::ELEMS, b_stages + LB::ELEMS); }
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DIRECT) : "memory");
-      } else {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      for (int part = 0; part < GATHER_PARTS; ++part) {
+        const int patch = m0 + part * LA::WAVE_ELEMS + lane;
+        const int oh = patch / p.conv.output_w, ow = patch - oh * p.conv.output_w;
+        const int corner_h = oh * p.conv.stride_h - p.conv.pad_h;
+        patch_w[part] = ow * p.conv.stride_w - p.conv.pad_w;
+        patch_offset[part] = corner_h * p.conv.width + patch_w[part];
+        patch_h[part] = (patch < p.m) ? corner_h : -(1 << 29);
       }
-#pragma unroll
-      for (int piece = 0; piece < STAGED; ++piece) { store_piece(piece, a_stages, b_stages, 0, std::true_type{}); }
-      if (slabs > 1) {
-#pragma unroll
-        for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, TILE_K); }
+    }
+
+    for (int batch = blockIdx.y; batch < p.batch_count; batch += gridDim.y) {
+      const T* a;
+      const T* b;
+      T* c;
+      T alpha, beta;
+      ResolveBatch<T, T>(p, batch, a, b, c, alpha, beta);
+      int k_len = p.k;
+      long long c_ld = p.c_ld;
+      if (p.split_chunk > 0) {  // this "batch" is one K range of a single problem
+        const int k_begin = batch * p.split_chunk;
+        k_len = min(p.split_chunk, p.k - k_begin);
+        a = static_cast<const T*>(p.a) + p.a_offset + (A_KC ? k_begin : k_begin * p.a_ld);
+        b = static_cast<const T*>(p.b) + p.b_offset + (B_KC ? k_begin : k_begin * p.b_ld);
+        c_ld = p.split_ld;
+        c = static_cast<T*>(p.split_workspace) + static_cast<long long>(batch) * p.split_ld * p.n;
+        alpha = T(1);
+        beta = T(0);
+      } else if (p.operand_triangle != 0) {  // skip the K range in which a triangular operand is zero
+        int k_first;
+        TriangularRange(p.operand_triangle, m0, n0, TILE_M, TILE_N, p.k, k_first, k_len);
+        a += A_KC ? static_cast<long long>(k_first) : k_first * p.a_ld;
+        b += B_KC ? static_cast<long long>(k_first) : k_first * p.b_ld;
       }
-      __syncthreads();
-      VM av[2];
-      VN bv[2];
-      av[0] = read_a(a_stages, 0);
-      bv[0] = read_b(b_stages, 0);
-      int cur = 0;  // ring position of the current slab; slab + 1 is in the next buffer, slab + 2 goes into the one before
-      // One slab. STORE: slab + 1 exists (staged operands store it); LOAD: slab + 2 exists (direct operands
-      // request it into the buffer that the barrier of the previous slab released, staged operands fetch it
-      // into registers). Compile-time, so that the steady state has no branches; the slab stored without a
-      // following load is the last one, the only one that can hold a K tail.
-      auto slab_body = [&](const int slab, auto store_tag, auto load_tag) {
-        constexpr bool STORE = decltype(store_tag)::value, LOAD = decltype(load_tag)::value;
-        const int nxt = (cur == STAGES - 1) ? 0 : cur + 1, prv = (cur == 0) ? STAGES - 1 : cur - 1;
-        const T* a_cur = a_stages + cur * LA::ELEMS;
-        const T* b_cur = b_stages + cur * LB::ELEMS;
-        T* a_nxt = a_stages + nxt * LA::ELEMS;
-        T* b_nxt = b_stages + nxt * LB::ELEMS;
-        T* a_prv = a_stages + prv * LA::ELEMS;
-        T* b_prv = b_stages + prv * LB::ELEMS;
-        const int k_store = (slab + 1) * TILE_K, k_load = (slab + 2) * TILE_K;
-        if constexpr (A_CONV == 1 && LOAD) { gather_rows = DecomposeRows<TILE_K>(p.conv, k_load, k_len, lane); }
+      const int slabs = (k_len + TILE_K - 1) / TILE_K;
+
+      Acc acc[FM][FN];
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          const int set = ks % 2;
-          if (ks + 1 < KSTEPS) {
-            av[set ^ 1] = read_a(a_cur, ks + 1);
-            bv[set ^ 1] = read_b(b_cur, ks + 1);
+      for (int i = 0; i < FM; ++i) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) { acc[i][j] = Traits::Zero(); }
+      }
+
+      // Walk over the slabs, explicitly scheduled so that the matrix pipe never waits at a slab boundary even
+      // with one wavefront per SIMD. Per k-step: LDS reads of the fragments of the NEXT k-step (other
+      // register set), the FM x FN MFMAs of this k-step, then a share of the data movement for the coming
+      // slabs: a direct operand's slab t+1 is requested in the first k-step of slab t; a staged operand
+      // stores its slab t+1 into the other LDS buffer and refills the staging registers with slab t+2. One
+      // barrier per slab, before its last k-step: by then every wavefront has finished its reads of the
+      // current buffer and its writes to the other one, so the last k-step already fetches the first
+      // fragments of slab t+1.
+      const T* a_tile0 = a + (A_KC ? m0 * p.a_ld : static_cast<long long>(m0));  // element (m0, k = 0), uniform
+      const T* b_tile0 = b + (B_KC ? n0 * p.b_ld : static_cast<long long>(n0));
+      // behind the last element of the operand: (x = extent - 1, k = k_len - 1) + 1
+      const T* a_end = a + (A_KC ? (p.m - 1) * p.a_ld + k_len : (k_len - 1) * p.a_ld + p.m);
+      const T* b_end = b + (B_KC ? (p.n - 1) * p.b_ld + k_len : (k_len - 1) * p.b_ld + p.n);
+      const int a_lane_bytes = A_DIRECT ? DirectLaneBytes<T, TILE_M, TILE_K, LANE_BYTES_A>(p.a_ld, lane)
+                                        : static_cast<int>((PA::Line(tid) * p.a_ld + PA::K(tid)) * static_cast<long long>(sizeof(T)));
+      const int b_lane_bytes = B_DIRECT ? DirectLaneBytes<T, TILE_N, TILE_K, LANE_BYTES>(p.b_ld, lane)
+                                        : static_cast<int>((PB::Line(tid) * p.b_ld + PB::K(tid)) * static_cast<long long>(sizeof(T)));
+      auto a_slab = [&](const int k0) { return a_tile0 + (A_KC ? static_cast<long long>(k0) : k0 * p.a_ld); };
+      auto b_slab = [&](const int k0) { return b_tile0 + (B_KC ? static_cast<long long>(k0) : k0 * p.b_ld); };
+      // The walk exists twice: with range-checked loads (tiles that touch an edge of the matrix, or a K
+      // tail), and without (the resources then cover "everything", which saves the scalar arithmetic of one
+      // byte count per load).
+      auto walk = [&](auto range_tag) {
+        constexpr bool RANGE = decltype(range_tag)::value;
+        VP a_stage[STAGED_A > 0 ? STAGED_A : 1], b_stage[STAGED_B > 0 ? STAGED_B : 1];
+        auto load_piece = [&](const int piece, const int k0) {
+          if (piece < STAGED_A) { a_stage[piece] = LoadPiece<T, TILE_M, TILE_K, VL, RANGE>(a_slab(k0), a_end, p.a_ld, a_lane_bytes, piece); }
+          else { b_stage[piece - STAGED_A] = LoadPiece<T, TILE_N, TILE_K, VL, RANGE>(b_slab(k0), b_end, p.b_ld, b_lane_bytes, piece - STAGED_A); }
+        };
+        auto store_piece = [&](const int piece, T* a_dst, T* b_dst, const int k0, auto check_tag) {
+          constexpr bool CHECK = RANGE && decltype(check_tag)::value;
+          if (piece < STAGED_A) {
+            StorePiece<T, TILE_M, TILE_K, LA::GROUP_PITCH, VL, CHECK>(a_dst, tid, piece, a_stage[piece], k_len - k0);
           } else {
-            av[set ^ 1] = read_a(a_nxt, 0);
-            bv[set ^ 1] = read_b(b_nxt, 0);
+            StorePiece<T, TILE_N, TILE_K, LB::GROUP_PITCH, VL, CHECK>(b_dst, tid, piece - STAGED_A, b_stage[piece - STAGED_A], k_len - k0);
           }
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int i = 0; i < FM; ++i) {
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-              acc[i][j] = Traits::Mfma(VecGet<VN, T, FN>(bv[set], j), VecGet<VM, T, FM>(av[set], i), acc[i][j]);
-            }
-          }
-          if (ks < KSTEPS - 1) {
-#pragma unroll
-            for (int u = 0; u < PER_SLOT; ++u) {
-              const int piece = ks * PER_SLOT + u;
-              if (piece < STAGED) {
-                if (STORE) { store_piece(piece, a_nxt, b_nxt, k_store, std::integral_constant<bool, !LOAD>{}); }
-                if (LOAD) { load_piece(piece, k_load); }
+        };
+        // direct loads of one slab, numbered over both operands: A's rounds first
+        constexpr int DIRECT_A = A_DIRECT ? LA::LOADS_PER_WAVE : 0, DIRECT_B = B_DIRECT ? LB::LOADS_PER_WAVE : 0;
+        constexpr int DIRECT = DIRECT_A + DIRECT_B;
+        constexpr int DIRECT_PER_SLOT = (DIRECT + SLOTS - 1) / SLOTS;
+        GatherRows gather_rows{};  // of the slab whose loads are being issued (gathered A only)
+        auto direct_load = [&](const int load, const int k0, auto* a_dst, auto* b_dst) {
+          if constexpr (DIRECT_A > 0) {
+            if (load < DIRECT_A) {
+              if constexpr (A_CONV == 1) {
+                GatherLoad<T, TILE_M, TILE_K, KernelTag>(a, p.conv, a_dst, wave_u, load, gather_rows, patch_h, patch_w, patch_offset);
+              } else if constexpr (A_CONV == 2) {
+                GatherLoadVector<T, TILE_M, TILE_K, KernelTag>(a, p.conv, a_dst, wave_u, load, k0, k_len, lane, patch_offset[0]);
+              } else {
+                DirectLoad<T, TILE_M, TILE_K, LANE_BYTES, RANGE, KernelTag>(a_slab(k0), a_end, p.a_ld, a_dst, wave_u, a_lane_bytes, load);
               }
             }
+          }
+          if constexpr (DIRECT_B > 0) {
+            if (load >= DIRECT_A) { DirectLoad<T, TILE_N, TILE_K, LANE_BYTES, RANGE, KernelTag>(b_slab(k0), b_end, p.b_ld, b_dst, wave_u, b_lane_bytes, load - DIRECT_A); }
+          }
+        };
+        auto read_a = [&](const T* stage, const int ks) {
+          const T* src = stage + LA::Row(ks * KP) + a_lane_row;
+          VM av;
+          if constexpr (M_INTERLEAVED) {
+            av = *reinterpret_cast<const VM*>(src);
+          } else {
 #pragma unroll
-            for (int u = 0; u < DIRECT_PER_SLOT; ++u) {
-              const int load = ks * DIRECT_PER_SLOT + u;
-              if (LOAD && load < DIRECT) { direct_load(load, k_load, a_prv, b_prv); }
+            for (int i = 0; i < FM; ++i) { av = VecWith<VM, T, FM>(av, i, src[i * MF]); }
+          }
+          return av;
+        };
+        auto read_b = [&](const T* stage, const int ks) {
+          return *reinterpret_cast<const VN*>(stage + LB::Row(ks * KP) + b_lane_row);
+        };
+
+        // Prologue: slab 0 lands in buffer 0 and slab 1 is requested - its direct loads before the wait for slab 0, so that
+        // the two memory latencies overlap (loads complete in order: when at most the direct loads of slab 1 are
+        // outstanding, everything of slab 0 has arrived); its staged pieces once slab 0 has left the staging registers.
+        if constexpr (A_CONV == 1) { gather_rows = DecomposeRows<TILE_K>(p.conv, 0, k_len, lane); }
+#pragma unroll
+        for (int load = 0; load < DIRECT; ++load) { direct_load(load, 0, a_stages, b_stages); }
+#pragma unroll
+        for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, 0); }
+        if (slabs > 1) {
+          if constexpr (A_CONV == 1) { gather_rows = DecomposeRows<TILE_K>(p.conv, TILE_K, k_len, lane); }
+#pragma unroll
+          for (int load = 0; load < DIRECT; ++load) { direct_load(load, TILE_K, a_stages + LA::ELEMS, b_stages + LB::ELEMS); }
+          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DIRECT) : "memory");
+        } else {
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+#pragma unroll
+        for (int piece = 0; piece < STAGED; ++piece) { store_piece(piece, a_stages, b_stages, 0, std::true_type{}); }
+        if (slabs > 1) {
+#pragma unroll
+          for (int piece = 0; piece < STAGED; ++piece) { load_piece(piece, TILE_K); }
+        }
+        __syncthreads();
+        VM av[2];
+        VN bv[2];
+        av[0] = read_a(a_stages, 0);
+        bv[0] = read_b(b_stages, 0);
+        int cur = 0;  // ring position of the current slab; slab + 1 is in the next buffer, slab + 2 goes into the one before
+        // One slab. STORE: slab + 1 exists (staged operands store it); LOAD: slab + 2 exists (direct operands
+        // request it into the buffer that the barrier of the previous slab released, staged operands fetch it
+        // into registers). Compile-time, so that the steady state has no branches; the slab stored without a
+        // following load is the last one, the only one that can hold a K tail.
+        auto slab_body = [&](const int slab, auto store_tag, auto load_tag) {
+          constexpr bool STORE = decltype(store_tag)::value, LOAD = decltype(load_tag)::value;
+          const int nxt = (cur == STAGES - 1) ? 0 : cur + 1, prv = (cur == 0) ? STAGES - 1 : cur - 1;
+          const T* a_cur = a_stages + cur * LA::ELEMS;
+          const T* b_cur = b_stages + cur * LB::ELEMS;
+          T* a_nxt = a_stages + nxt * LA::ELEMS;
+          T* b_nxt = b_stages + nxt * LB::ELEMS;
+          T* a_prv = a_stages + prv * LA::ELEMS;
+          T* b_prv = b_stages + prv * LB::ELEMS;
+          const int k_store = (slab + 1) * TILE_K, k_load = (slab + 2) * TILE_K;
+          if constexpr (A_CONV == 1 && LOAD) { gather_rows = DecomposeRows<TILE_K>(p.conv, k_load, k_len, lane); }
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) {
+            const int set = ks % 2;
+            if (ks + 1 < KSTEPS) {
+              av[set ^ 1] = read_a(a_cur, ks + 1);
+              bv[set ^ 1] = read_b(b_cur, ks + 1);
+            } else {
+              av[set ^ 1] = read_a(a_nxt, 0);
+              bv[set ^ 1] = read_b(b_nxt, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < FM; ++i) {
+#pragma unroll
+              for (int j = 0; j < FN; ++j) {
+                acc[i][j] = Traits::Mfma(VecGet<VN, T, FN>(bv[set], j), VecGet<VM, T, FM>(av[set], i), acc[i][j]);
+              }
+            }
+            if (ks < KSTEPS - 1) {
+#pragma unroll
+              for (int u = 0; u < PER_SLOT; ++u) {
+                const int piece = ks * PER_SLOT + u;
+                if (piece < STAGED) {
+                  if (STORE) { store_piece(piece, a_nxt, b_nxt, k_store, std::integral_constant<bool, !LOAD>{}); }
+                  if (LOAD) { load_piece(piece, k_load); }
+                }
+              }
+#pragma unroll
+              for (int u = 0; u < DIRECT_PER_SLOT; ++u) {
+                const int load = ks * DIRECT_PER_SLOT + u;
+                if (LOAD && load < DIRECT) { direct_load(load, k_load, a_prv, b_prv); }
+              }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (ks == KSTEPS - 2) {
+              // slab + 1 must have landed for everybody: everything requested before this slab has to be
+              // complete, this slab's own requests (slab + 2) may stay in flight (loads complete in order)
+              if (LOAD) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DIRECT + STAGED) : "memory"); }
+              else { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+              asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
             }
           }
-          __builtin_amdgcn_sched_barrier(0);
-          if (ks == KSTEPS - 2) {
-            // slab + 1 must have landed for everybody: everything requested before this slab has to be
-            // complete, this slab's own requests (slab + 2) may stay in flight (loads complete in order)
-            if (LOAD) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DIRECT + STAGED) : "memory"); }
-            else { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+          cur = nxt;
+        };
+        int slab = 0;
+        for (; slab + 2 < slabs; ++slab) { slab_body(slab, std::true_type{}, std::true_type{}); }
+        if (slab + 1 < slabs) { slab_body(slab, std::true_type{}, std::false_type{}); ++slab; }
+        slab_body(slab, std::false_type{}, std::false_type{});
+        __syncthreads();
+      };
+      // Lane owns m = m_base + i * M_STEP (i < FM); accumulator element r of block (i, j) is the column
+      // n = n_base + FN * Row(r) + j.
+      const int m_base = m0 + a_read;
+      const int n_base = n0 + wave_n * (FN * MF);
+      constexpr int M_STEP = M_INTERLEAVED ? 1 : MF;  // distance in m between the lane's accumulator blocks
+      // 16-byte accesses to C need dword alignment only, which every fp32/fp64 address has
+      typedef T VMG __attribute__((ext_vector_type(FM > 1 ? FM : 2), aligned(sizeof(T))));
+      const bool vector_store = M_INTERLEAVED && (FM > 1) && (m_base + FM <= p.m) && !masked;
+      auto writes = [&](const int i, const int n) {  // element i of the lane's piece of column n belongs to the result
+        return n < p.n && m_base + i * M_STEP < p.m && (!masked || InTriangle(p.c_triangle, m_base + i * M_STEP, n));
+      };
+      // Small tiles (at most 16 registers of old C per lane) fetch the old C before the K walk when beta != 0: with a
+      // short k the launch is a stream over C, and a work-group that asked for its C only after its last product would
+      // wait out a second memory latency with nothing else to do (8191 x 8191 x 127: 0.27 -> 0.14 ms). The loads are the
+      // oldest in the queue, so the first wait of the walk covers them.
+      constexpr bool PREFETCH_C = FM * FN * ACC * sizeof(T) <= 64;
+      T old_c[PREFETCH_C ? FM * FN * ACC : 1];
+      if constexpr (PREFETCH_C) {
+        if (beta != T(0)) {
+#pragma unroll
+          for (int j = 0; j < FN; ++j) {
+#pragma unroll
+            for (int r = 0; r < ACC; ++r) {
+              const int n = n_base + FN * Traits::Row(r, lane_g) + j;
+#pragma unroll
+              for (int i = 0; i < FM; ++i) {
+                old_c[(j * ACC + r) * FM + i] = writes(i, n) ? c[n * c_ld + m_base + i * M_STEP] : T(0);
+              }
+            }
           }
         }
-        cur = nxt;
-      };
-      int slab = 0;
-      for (; slab + 2 < slabs; ++slab) { slab_body(slab, std::true_type{}, std::true_type{}); }
-      if (slab + 1 < slabs) { slab_body(slab, std::true_type{}, std::false_type{}); ++slab; }
-      slab_body(slab, std::false_type{}, std::false_type{});
-      __syncthreads();
-    };
-    // Lane owns m = m_base + i * M_STEP (i < FM); accumulator element r of block (i, j) is the column
-    // n = n_base + FN * Row(r) + j.
-    const int m_base = m0 + a_read;
-    const int n_base = n0 + wave_n * (FN * MF);
-    constexpr int M_STEP = M_INTERLEAVED ? 1 : MF;  // distance in m between the lane's accumulator blocks
-    // 16-byte accesses to C need dword alignment only, which every fp32/fp64 address has
-    typedef T VMG __attribute__((ext_vector_type(FM > 1 ? FM : 2), aligned(sizeof(T))));
-    const bool vector_store = M_INTERLEAVED && (FM > 1) && (m_base + FM <= p.m) && !masked;
-    auto writes = [&](const int i, const int n) {  // element i of the lane's piece of column n belongs to the result
-      return n < p.n && m_base + i * M_STEP < p.m && (!masked || InTriangle(p.c_triangle, m_base + i * M_STEP, n));
-    };
-    // Small tiles (at most 16 registers of old C per lane) fetch the old C before the K walk when beta != 0: with a
-    // short k the launch is a stream over C, and a work-group that asked for its C only after its last product would
-    // wait out a second memory latency with nothing else to do (8191 x 8191 x 127: 0.27 -> 0.14 ms). The loads are the
-    // oldest in the queue, so the first wait of the walk covers them.
-    constexpr bool PREFETCH_C = FM * FN * ACC * sizeof(T) <= 64;
-    T old_c[PREFETCH_C ? FM * FN * ACC : 1];
-    if constexpr (PREFETCH_C) {
-      if (beta != T(0)) {
+      }
+
+      if (m0 + TILE_M <= p.m && n0 + TILE_N <= p.n && k_len % TILE_K == 0) { walk(std::false_type{}); }
+      else { walk(std::true_type{}); }
+
+      // Epilogue.
+      if constexpr (PREFETCH_C) {
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
 #pragma unroll
           for (int r = 0; r < ACC; ++r) {
             const int n = n_base + FN * Traits::Row(r, lane_g) + j;
-#pragma unroll
-            for (int i = 0; i < FM; ++i) {
-              old_c[(j * ACC + r) * FM + i] = writes(i, n) ? c[n * c_ld + m_base + i * M_STEP] : T(0);
-            }
-          }
-        }
-      }
-    }
-
-    if (m0 + TILE_M <= p.m && n0 + TILE_N <= p.n && k_len % TILE_K == 0) { walk(std::false_type{}); }
-    else { walk(std::true_type{}); }
-
-    // Epilogue.
-    if constexpr (PREFETCH_C) {
-#pragma unroll
-      for (int j = 0; j < FN; ++j) {
-#pragma unroll
-        for (int r = 0; r < ACC; ++r) {
-          const int n = n_base + FN * Traits::Row(r, lane_g) + j;
-          T* dst = c + n * c_ld + m_base;
-          if (vector_store && n < p.n) {
-            VMG out;
-#pragma unroll
-            for (int i = 0; i < FM; ++i) {
-              out[i] = (beta == T(0)) ? alpha * acc[i][j][r] : Combine(alpha, acc[i][j][r], beta, old_c[(j * ACC + r) * FM + i]);
-            }
-            *reinterpret_cast<VMG*>(dst) = out;
-          } else {
-#pragma unroll
-            for (int i = 0; i < FM; ++i) {
-              if (writes(i, n)) {
-                dst[i * M_STEP] = (beta == T(0)) ? alpha * acc[i][j][r] : Combine(alpha, acc[i][j][r], beta, old_c[(j * ACC + r) * FM + i]);
-              }
-            }
-          }
-        }
-      }
-    } else if (M_INTERLEAVED && FM > 1 && c_ld < kViewMaxLd) {
-      // Large tiles whose lanes own runs of FM consecutive m: C through a buffer view of the tile, every piece at an
-      // offset that lies outside the view where the piece does (columns from n on, lanes at or beyond the last row): such
-      // loads deliver zeros and such stores move nothing. No branch stands between the pieces then, and the old C of
-      // four columns is in flight together before the first of them is combined and stored (with one branch per piece
-      // every load was waited for before the next one left). Lanes whose run straddles the last row, and tiles on the
-      // diagonal of a triangle, move their elements one by one afterwards.
-      // (64 bytes of old C per lane in flight)
-      constexpr int WANTED = 64 / static_cast<int>(sizeof(VMG)) > 0 ? 64 / static_cast<int>(sizeof(VMG)) : 1;
-      constexpr int BATCH = (ACC % WANTED == 0) ? WANTED : (ACC % 4 == 0) ? 4 : 1;
-      // (the lane's place once more, opaque: what the epilogue derives from it is then computed here and not ahead of
-      // the K walk, where it would occupy registers that the large tiles have none to spare of)
-      int late_read = a_read, late_g = lane_g;
-      asm volatile("" : "+v"(late_read), "+v"(late_g));
-      const int late_m = m0 + late_read;
-      const bool whole_run = (late_m + FM <= p.m) && !masked;
-      const auto view = __builtin_amdgcn_make_buffer_rsrc(c + n0 * c_ld + m0, 0, kViewOutside, kRawBufferFlags);
-      const int column_bytes = static_cast<int>(c_ld) * static_cast<int>(sizeof(T));
-      const int lane_bytes = (n_base - n0) * column_bytes + late_read * static_cast<int>(sizeof(T));
-#pragma unroll
-      for (int j = 0; j < FN; ++j) {
-#pragma unroll
-        for (int r0 = 0; r0 < ACC; r0 += BATCH) {
-          int offset[BATCH];
-          VMG old[BATCH];
-#pragma unroll
-          for (int rr = 0; rr < BATCH; ++rr) {
-            const int column = FN * Traits::Row(r0 + rr, late_g) + j;
-            offset[rr] = (whole_run && n_base + column < p.n) ? lane_bytes + column * column_bytes : kViewOutside;
-          }
-          if (beta != T(0)) {
-#pragma unroll
-            for (int rr = 0; rr < BATCH; ++rr) { old[rr] = BufferLoad<T, FM>(view, offset[rr]); }
-          }
-#pragma unroll
-          for (int rr = 0; rr < BATCH; ++rr) {
-            const int r = r0 + rr;
-            VMG out;
-            if (beta == T(0)) {
-#pragma unroll
-              for (int i = 0; i < FM; ++i) { out[i] = alpha * acc[i][j][r]; }
-            } else {
-#pragma unroll
-              for (int i = 0; i < FM; ++i) { out[i] = Combine(alpha, acc[i][j][r], beta, old[rr][i]); }
-            }
-            BufferStore<T, FM>(out, view, offset[rr]);
-          }
-          if (!whole_run) {
-#pragma unroll
-            for (int rr = 0; rr < BATCH; ++rr) {
-              const int r = r0 + rr;
-              const int n = n_base + FN * Traits::Row(r, late_g) + j;
+            T* dst = c + n * c_ld + m_base;
+            if (vector_store && n < p.n) {
+              VMG out;
 #pragma unroll
               for (int i = 0; i < FM; ++i) {
-                if (n < p.n && late_m + i < p.m && (!masked || InTriangle(p.c_triangle, late_m + i, n))) {
-                  StoreResult<T, T>(c + n * c_ld + late_m, i, acc[i][j][r], alpha, beta);
+                out[i] = (beta == T(0)) ? alpha * acc[i][j][r] : Combine(alpha, acc[i][j][r], beta, old_c[(j * ACC + r) * FM + i]);
+              }
+              *reinterpret_cast<VMG*>(dst) = out;
+            } else {
+#pragma unroll
+              for (int i = 0; i < FM; ++i) {
+                if (writes(i, n)) {
+                  dst[i * M_STEP] = (beta == T(0)) ? alpha * acc[i][j][r] : Combine(alpha, acc[i][j][r], beta, old_c[(j * ACC + r) * FM + i]);
                 }
               }
             }
           }
         }
-      }
-    } else {
-      // Large tiles: the old C of four columns at a time is fetched before the first of them is combined and stored
-      // (a load behind a store to memory that may alias it cannot be hoisted by the compiler).
-      constexpr int BATCH = (ACC % 4 == 0) ? 4 : 1;
+      } else if (M_INTERLEAVED && FM > 1 && c_ld < kViewMaxLd) {
+        // Large tiles whose lanes own runs of FM consecutive m: C through a buffer view of the tile, every piece at an
+        // offset that lies outside the view where the piece does (columns from n on, lanes at or beyond the last row): such
+        // loads deliver zeros and such stores move nothing. No branch stands between the pieces then, and the old C of
+        // four columns is in flight together before the first of them is combined and stored (with one branch per piece
+        // every load was waited for before the next one left). Lanes whose run straddles the last row, and tiles on the
+        // diagonal of a triangle, move their elements one by one afterwards.
+        // (64 bytes of old C per lane in flight)
+        constexpr int WANTED = 64 / static_cast<int>(sizeof(VMG)) > 0 ? 64 / static_cast<int>(sizeof(VMG)) : 1;
+        constexpr int BATCH = (ACC % WANTED == 0) ? WANTED : (ACC % 4 == 0) ? 4 : 1;
+        // (the lane's place once more, opaque: what the epilogue derives from it is then computed here and not ahead of
+        // the K walk, where it would occupy registers that the large tiles have none to spare of)
+        int late_read = a_read, late_g = lane_g;
+        asm volatile("" : "+v"(late_read), "+v"(late_g));
+        const int late_m = m0 + late_read;
+        const bool whole_run = (late_m + FM <= p.m) && !masked;
+        const auto view = __builtin_amdgcn_make_buffer_rsrc(c + n0 * c_ld + m0, 0, kViewOutside, kRawBufferFlags);
+        const int column_bytes = static_cast<int>(c_ld) * static_cast<int>(sizeof(T));
+        const int lane_bytes = (n_base - n0) * column_bytes + late_read * static_cast<int>(sizeof(T));
 #pragma unroll
-      for (int j = 0; j < FN; ++j) {
+        for (int j = 0; j < FN; ++j) {
 #pragma unroll
-        for (int r0 = 0; r0 < ACC; r0 += BATCH) {
-          VMG old[BATCH];
-          if (vector_store && beta != T(0)) {
+          for (int r0 = 0; r0 < ACC; r0 += BATCH) {
+            int offset[BATCH];
+            VMG old[BATCH];
 #pragma unroll
             for (int rr = 0; rr < BATCH; ++rr) {
-              const int n = n_base + FN * Traits::Row(r0 + rr, lane_g) + j;
-              if (n < p.n) { old[rr] = *reinterpret_cast<const VMG*>(c + n * c_ld + m_base); }
+              const int column = FN * Traits::Row(r0 + rr, late_g) + j;
+              offset[rr] = (whole_run && n_base + column < p.n) ? lane_bytes + column * column_bytes : kViewOutside;
             }
-          }
+            if (beta != T(0)) {
 #pragma unroll
-          for (int rr = 0; rr < BATCH; ++rr) {
-            const int r = r0 + rr;
-            const int n = n_base + FN * Traits::Row(r, lane_g) + j;
-            if (n >= p.n) { continue; }
-            T* dst = c + n * c_ld + m_base;
-            if (vector_store) {
+              for (int rr = 0; rr < BATCH; ++rr) { old[rr] = BufferLoad<T, FM>(view, offset[rr]); }
+            }
+#pragma unroll
+            for (int rr = 0; rr < BATCH; ++rr) {
+              const int r = r0 + rr;
               VMG out;
               if (beta == T(0)) {
 #pragma unroll
@@ -863,11 +838,60 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
 #pragma unroll
                 for (int i = 0; i < FM; ++i) { out[i] = Combine(alpha, acc[i][j][r], beta, old[rr][i]); }
               }
-              *reinterpret_cast<VMG*>(dst) = out;
-            } else {
+              BufferStore<T, FM>(out, view, offset[rr]);
+            }
+            if (!whole_run) {
 #pragma unroll
-              for (int i = 0; i < FM; ++i) {
-                if (writes(i, n)) { StoreResult<T, T>(dst, i * M_STEP, acc[i][j][r], alpha, beta); }
+              for (int rr = 0; rr < BATCH; ++rr) {
+                const int r = r0 + rr;
+                const int n = n_base + FN * Traits::Row(r, late_g) + j;
+#pragma unroll
+                for (int i = 0; i < FM; ++i) {
+                  if (n < p.n && late_m + i < p.m && (!masked || InTriangle(p.c_triangle, late_m + i, n))) {
+                    StoreResult<T, T>(c + n * c_ld + late_m, i, acc[i][j][r], alpha, beta);
+                  }
+                }
+              }
+            }
+          }
+        }
+      } else {
+        // Large tiles: the old C of four columns at a time is fetched before the first of them is combined and stored
+        // (a load behind a store to memory that may alias it cannot be hoisted by the compiler).
+        constexpr int BATCH = (ACC % 4 == 0) ? 4 : 1;
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+#pragma unroll
+          for (int r0 = 0; r0 < ACC; r0 += BATCH) {
+            VMG old[BATCH];
+            if (vector_store && beta != T(0)) {
+#pragma unroll
+              for (int rr = 0; rr < BATCH; ++rr) {
+                const int n = n_base + FN * Traits::Row(r0 + rr, lane_g) + j;
+                if (n < p.n) { old[rr] = *reinterpret_cast<const VMG*>(c + n * c_ld + m_base); }
+              }
+            }
+#pragma unroll
+            for (int rr = 0; rr < BATCH; ++rr) {
+              const int r = r0 + rr;
+              const int n = n_base + FN * Traits::Row(r, lane_g) + j;
+              if (n >= p.n) { continue; }
+              T* dst = c + n * c_ld + m_base;
+              if (vector_store) {
+                VMG out;
+                if (beta == T(0)) {
+#pragma unroll
+                  for (int i = 0; i < FM; ++i) { out[i] = alpha * acc[i][j][r]; }
+                } else {
+#pragma unroll
+                  for (int i = 0; i < FM; ++i) { out[i] = Combine(alpha, acc[i][j][r], beta, old[rr][i]); }
+                }
+                *reinterpret_cast<VMG*>(dst) = out;
+              } else {
+#pragma unroll
+                for (int i = 0; i < FM; ++i) {
+                  if (writes(i, n)) { StoreResult<T, T>(dst, i * M_STEP, acc[i][j][r], alpha, beta); }
+                }
               }
             }
           }

@@ -164,7 +164,7 @@ __global__ __launch_bounds__(Config::THREADS, Config::MIN_WAVES) void HgemmMfmaK
 
   int tile_m, tile_n;
   if ((p.c_triangle | p.operand_triangle) != 0) {
-    if (!TileOfBlockCyclic(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n)) { return; }
+    if (!TileOfBlockCyclic(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n, p.operand_triangle)) { return; }
   } else {
     TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
   }

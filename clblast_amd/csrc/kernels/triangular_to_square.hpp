@@ -6,7 +6,9 @@
 // TriangularToSquareKernel: dense extent x extent copy (extent >= k) of a k x k triangular matrix: the stored
 // triangle as it is, zeros in the other one (which is never read), ones on the diagonal when it is implied
 // ("unit"), and the identity in the rows and columns from k on. "upper" means the stored elements are those with
-// one <= two.
+// one <= two. With a grid of several layers (blockIdx.z) the same is done for the diagonal leaves of the matrix: layer b
+// takes the rows and columns from b * extent on (k - b * extent of them, at most extent) and writes its extent x extent
+// copy to dst + b * extent * (dst_ld + 1).
 // CopyMatrixKernel: dst[two * dst_ld + one] = src[two * src_ld + one] for a one x two matrix.
 // Both are HBM bound and move VEC consecutive elements per lane and access; VEC > 1 needs every extent, leading
 // dimension and base address involved to be a multiple of VEC elements.
@@ -23,13 +25,17 @@ constexpr int kCopyThreads = 256;
 constexpr int kCopyMaxGridY = 16384;  // values of `two` beyond that are covered by a grid-stride loop
 
 template <typename T, int VEC>
-__global__ __launch_bounds__(kCopyThreads) void TriangularToSquareKernel(const int k, const int extent, const bool upper,
-                                                                         const bool unit, const T* __restrict__ src,
-                                                                         const long long src_ld, T* __restrict__ dst,
+__global__ __launch_bounds__(kCopyThreads) void TriangularToSquareKernel(const int k_all, const int extent, const bool upper,
+                                                                         const bool unit, const T* __restrict__ src_all,
+                                                                         const long long src_ld, T* __restrict__ dst_all,
                                                                          const long long dst_ld) {
   typedef T Vector __attribute__((ext_vector_type(VEC)));
   const int one = (blockIdx.x * kCopyThreads + threadIdx.x) * VEC;
   if (one >= extent) { return; }
+  const long long first = static_cast<long long>(blockIdx.z) * extent;
+  const int k = static_cast<int>(min(static_cast<long long>(extent), max(0ll, k_all - first)));
+  const T* __restrict__ src = src_all + first * (src_ld + 1);
+  T* __restrict__ dst = dst_all + first * (dst_ld + 1);
   for (int two = blockIdx.y; two < extent; two += gridDim.y) {
     // the lane's elements one .. one + VEC - 1: read only when at least one of them is stored (k is a multiple of
     // VEC on the vector path, so a lane lies entirely inside or outside the source)

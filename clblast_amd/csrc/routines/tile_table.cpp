@@ -292,14 +292,12 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       // n = 1106, k = 4092 141 us on the 64 x 64 tile of the 32x32x2 instruction, 83 us on 64 x 32 tiles). Now the cost
       // estimate of the GEMM table over the tiles that touch the triangle of C, with the rates the tiles reach on SYRK (0.76 to 0.93 of their GEMM rates): 1.7 % on the
       // same shapes.
-      // A triangular operand (TRMM, the products inside TRSM) keeps the rule above: its tiles walk K ranges of very
-      // different lengths, which the estimate does not see (STRMM 4096^2: 0.64 ms by the rule, 0.68 ms by the estimate).
-      if (triangular == 2) {
-        if (working(128, 64) >= 2048) { return KernelChoice{CLBH_KERNEL_MFMA, 11, 1}; }
-        if (working(256, 128) >= 4 * 256) { return KernelChoice{CLBH_KERNEL_MFMA, 3, 1}; }
-        if (working(128, 128) >= 4 * 256) { return KernelChoice{CLBH_KERNEL_MFMA, 0, 1}; }
-        return KernelChoice{CLBH_KERNEL_MFMA, 7, 1};
-      }
+      // A triangular operand (TRMM, the products inside TRSM): the kernel folds the tile rows (or columns) in two, every
+      // work-group walks a long and a short K range, so the launch is as even as a full product of half the tiles.
+      // 128 x 128 tiles from two rounds of such pairs on, else 64 x 64 tiles on the 16x16x4 instruction (STRMM from the
+      // left, lower, n = 4096, by tile: m = 4096 566 us on 128 x 128, 581 on 128 x 64, 586 on 64 x 64, 603 on 256 x 128;
+      // m = 2048, n = 2048 98 us on 64 x 64, 100 on 128 x 64, 172 on 128 x 128; m = 1024 61 us and m = 512 29 us on 64 x 64).
+      if (triangular == 2) { return KernelChoice{CLBH_KERNEL_MFMA, (working(128, 128) >= 2 * Units()) ? 0 : 12, 1}; }
       const bool square = true;
       const auto touching = [&](const size_t tile_m, const size_t tile_n) {
         if (!square) { return CeilDivide(m, tile_m) * CeilDivide(n, tile_n) * batch_count; }
@@ -332,8 +330,9 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
       // 64 x 64 tiles, 61 us on 32 x 32). Rates on SYRK: 128 x 128 x 8 73 TFLOP/s with k0 = 149, 64 x 64 67 and 84, 64 x 32
       // 64 and 74, 32 x 32 57 and 121; two k-contiguous operands 0.86 to 0.93 of that, and no 128 x 128 x 8 tiles then
       // (n = 3756, k = 4935: 1900 us on them, 1252 us on 64 x 32).
-      // (a triangular operand keeps the rule of old, as in the fp32 table: DTRMM 4096^2 1.31 against 1.45 ms)
-      if (triangular == 2) { return KernelChoice{CLBH_KERNEL_MFMA, (working(128, 128) >= 4 * 256) ? 0 : 1, 1}; }
+      // (a triangular operand: folded tile rows as in the fp32 table; 128 x 128 x 8 from two rounds of pairs on - DTRMM
+      // 4096^2 1.18 against 1.20 ms on 128 x 64 - else 128 x 64)
+      if (triangular == 2) { return KernelChoice{CLBH_KERNEL_MFMA, (working(128, 128) >= 2 * Units()) ? 0 : 1, 1}; }
       const bool square = true;
       const auto touching = [&](const size_t tile_m, const size_t tile_n) {
         if (!square) { return CeilDivide(m, tile_m) * CeilDivide(n, tile_n) * batch_count; }

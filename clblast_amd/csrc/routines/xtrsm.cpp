@@ -50,34 +50,39 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
   constexpr size_t kLineMultiple = 16 / sizeof(T);
   // Diagonal blocks: `block` is what the inversion kernel inverts; the inverses are then doubled in size with GEMMs
   // up to the leaf size of the recursion (at most kMaxLeaf, and no more doublings than the matrix has use for)
-  constexpr size_t kMaxLeaf = 512;
+  // (real matrices: the leaf products skip the zero half of their triangular inverse, which makes wider leaves worth
+  // their flops - STRSM 4096^2: leaves of 512 0.78 ms, of 1024 0.75 ms; the complex engine multiplies them as dense)
+  constexpr size_t kMaxLeaf = Engine::kComplex ? 512 : 1024;
   const auto block = static_cast<size_t>(Engine::kComplex ? clbh_complex_invert_block_size(precision)
                                                           : clbh_invert_block_size(precision));
   auto leaf = block;
   while (leaf < kMaxLeaf && leaf < k) { leaf *= 2; }
   const auto k_padded = (k + leaf - 1) / leaf * leaf;
 
-  // Dense copy of the triangle, padded with the identity to whole leaves: the other triangle becomes zeros, an
-  // implied diagonal ones, and no block operation below has a ragged edge on the A side
-  const auto dense_bytes = k_padded * k_padded * sizeof(T);
-  const StreamScratch dense(dense_bytes, stream, "dense copy of the triangular matrix");
+  // Dense copies of the diagonal leaves, padded with the identity to whole leaves (the other triangle becomes zeros, an
+  // implied diagonal ones, and no block operation on them has a ragged edge), kept as a band: leaf b at b * leaf *
+  // (leaf + 1) with leading dimension `leaf`, so that the diagonal blocks of one size lie at a constant stride. The
+  // blocks off the diagonal are read from the caller's matrix where they are.
+  const auto band_ld = leaf;
+  const auto band_bytes = (k_padded / leaf) * leaf * (leaf + 1) * sizeof(T);
+  const StreamScratch dense(band_bytes, stream, "dense copies of the diagonal leaves");
   const auto is_upper = (triangle == Triangle::kUpper);
-  const auto to_square = Engine::kComplex ? clbh_complex_triangular_to_square : clbh_triangular_to_square;
-  CheckDevice(to_square(precision, is_upper ? 1 : 0, (diagonal == Diagonal::kUnit) ? 1 : 0, static_cast<int>(k), a_buffer(),
-                        static_cast<long long>(a_offset), static_cast<long long>(a_ld), dense.get(),
-                        static_cast<int>(k_padded), static_cast<long long>(k_padded), stream),
-              "clbh_triangular_to_square");
-  const auto dense_buffer = Buffer<T>(dense.get(), dense_bytes);
+  const auto to_band = Engine::kComplex ? clbh_complex_triangular_to_band : clbh_triangular_to_band;
+  CheckDevice(to_band(precision, is_upper ? 1 : 0, (diagonal == Diagonal::kUnit) ? 1 : 0, static_cast<int>(k),
+                      static_cast<int>(leaf), a_buffer(), static_cast<long long>(a_offset), static_cast<long long>(a_ld),
+                      dense.get(), stream),
+              "clbh_triangular_to_band");
+  const auto dense_buffer = Buffer<T>(dense.get(), band_bytes);
 
-  // Inverses of the diagonal leaves (xtrsm.cpp:105-118 with Xinvert), kept in a matrix of the same shape as the dense
-  // copy, each inverse in the place of its block, zeros elsewhere
-  const StreamScratch inverses(dense_bytes, stream, "inverted diagonal blocks");
-  CheckDevice(clbh_fill_zero(inverses.get(), dense_bytes, stream), "clbh_fill_zero");
+  // Inverses of the diagonal leaves (xtrsm.cpp:105-118 with Xinvert), kept in a band of the same shape, each inverse in
+  // the place of its leaf
+  const StreamScratch inverses(band_bytes, stream, "inverted diagonal blocks");
+  CheckDevice(clbh_fill_zero(inverses.get(), band_bytes, stream), "clbh_fill_zero");
   const auto invert = Engine::kComplex ? clbh_complex_invert_diagonal_blocks : clbh_invert_diagonal_blocks;
   CheckDevice(invert(precision, is_upper ? 1 : 0, static_cast<int>(k_padded / block), dense.get(),
-                     static_cast<long long>(k_padded), inverses.get(), static_cast<long long>(k_padded), stream),
+                     static_cast<long long>(band_ld), inverses.get(), static_cast<long long>(band_ld), stream),
               "clbh_invert_diagonal_blocks");
-  const auto inverse_buffer = Buffer<T>(inverses.get(), dense_bytes);
+  const auto inverse_buffer = Buffer<T>(inverses.get(), band_bytes);
   if (leaf > block) {
     // Doubling (xinvert.cpp:103-140 does the same with dedicated kernels): for two neighbouring inverted blocks of
     // extent `size`, with R the rows and C the columns of the off-diagonal block between them,
@@ -89,16 +94,16 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
     auto batched = typename Engine::StridedBatched(&stream, nullptr);
     for (auto size = block; size < leaf; size *= 2) {
       const auto pairs = k_padded / (2 * size);
-      const auto diagonal_step = 2 * size * (k_padded + 1);
+      const auto diagonal_step = 2 * size * (band_ld + 1);
       const auto rows = is_upper ? size_t{0} : size, columns = is_upper ? size : size_t{0};
-      const auto at = [&](const size_t r, const size_t c) { return r + c * k_padded; };
+      const auto at = [&](const size_t r, const size_t c) { return r + c * band_ld; };
       batched.DoGemmStridedBatched(Layout::kColMajor, Transpose::kNo, Transpose::kNo, size, size, size, ConstantOne<T>(),
-                                   dense_buffer, at(rows, columns), k_padded, diagonal_step, inverse_buffer,
-                                   at(columns, columns), k_padded, diagonal_step, ConstantZero<T>(), product_buffer, 0, size,
+                                   dense_buffer, at(rows, columns), band_ld, diagonal_step, inverse_buffer,
+                                   at(columns, columns), band_ld, diagonal_step, ConstantZero<T>(), product_buffer, 0, size,
                                    size * size, pairs);
       batched.DoGemmStridedBatched(Layout::kColMajor, Transpose::kNo, Transpose::kNo, size, size, size, ConstantNegOne<T>(),
-                                   inverse_buffer, at(rows, rows), k_padded, diagonal_step, product_buffer, 0, size,
-                                   size * size, ConstantZero<T>(), inverse_buffer, at(rows, columns), k_padded, diagonal_step,
+                                   inverse_buffer, at(rows, rows), band_ld, diagonal_step, product_buffer, 0, size,
+                                   size * size, ConstantZero<T>(), inverse_buffer, at(rows, columns), band_ld, diagonal_step,
                                    pairs);
     }
   }
@@ -117,20 +122,22 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
   // op(A) is lower triangular for (lower, not transposed) and (upper, transposed)
   const bool op_lower = (is_upper == transposed);
 
-  // Offset in the dense copy of the stored block that op(A)[rows r0.., columns c0..] is read from
+  // Offset in the caller's matrix of the stored block that op(A)[rows r0.., columns c0..] is read from (only blocks
+  // off the diagonal, which lie inside the stored triangle as a whole)
   const auto stored_at = [&](const size_t r0, const size_t c0) {
-    return transposed ? (c0 + r0 * k_padded) : (r0 + c0 * k_padded);
+    return a_offset + (transposed ? (c0 + r0 * a_ld) : (r0 + c0 * a_ld));
   };
   const auto gemm = [&](const Transpose ta, const Transpose tb, const size_t gm, const size_t gn, const size_t gk,
                         const T galpha, const Buffer<T>& ga, const size_t ga_offset, const size_t ga_ld,
                         const Buffer<T>& gb, const size_t gb_offset, const size_t gb_ld, const T gbeta,
-                        const Buffer<T>& gc, const size_t gc_offset, const size_t gc_ld) {
+                        const Buffer<T>& gc, const size_t gc_offset, const size_t gc_ld,
+                        const OperandTriangle operand = OperandTriangle::kNone) {
     if constexpr (Engine::kComplex) {
       this->DoGemm(Layout::kColMajor, ta, tb, gm, gn, gk, galpha, ga, ga_offset, ga_ld, gb, gb_offset, gb_ld, gbeta, gc,
                    gc_offset, gc_ld, OutputTriangle::kFull, false);
     } else {
       this->DoGemm(Layout::kColMajor, ta, tb, gm, gn, gk, galpha, ga, ga_offset, ga_ld, gb, gb_offset, gb_ld, gbeta, gc,
-                   gc_offset, gc_ld, Buffer<T>(nullptr), false, GemmTriangles{}, false);
+                   gc_offset, gc_ld, Buffer<T>(nullptr), false, GemmTriangles{OutputTriangle::kFull, operand}, false);
     }
   };
 
@@ -140,13 +147,15 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
     const auto factor = scaled ? one : alpha;
     if (hi - lo <= leaf) {
       const auto size = hi - lo;
-      const auto inverse_offset = lo * (k_padded + 1);
+      const auto inverse_offset = lo * (band_ld + 1);
+      // (the inverse of a triangular block is triangular the same way: the product skips its zero half; the complex
+      // engine, which multiplies a rewritten copy of its first operand, takes the block as a dense one)
       if (side == Side::kLeft) {  // X[lo:hi, :] = factor * op(inverse) * B[lo:hi, :]
-        gemm(a_transpose, no, size, n, size, factor, inverse_buffer, inverse_offset, k_padded, b_buffer, b_offset + lo, b_ld, zero,
-             x_buffer, lo, x_ld);
+        gemm(a_transpose, no, size, n, size, factor, inverse_buffer, inverse_offset, band_ld, b_buffer, b_offset + lo, b_ld, zero,
+             x_buffer, lo, x_ld, op_lower ? OperandTriangle::kLowerA : OperandTriangle::kUpperA);
       } else {                    // X[:, lo:hi] = factor * B[:, lo:hi] * op(inverse)
         gemm(no, a_transpose, m, size, size, factor, b_buffer, b_offset + lo * b_ld, b_ld, inverse_buffer, inverse_offset,
-             k_padded, zero, x_buffer, lo * x_ld, x_ld);
+             band_ld, zero, x_buffer, lo * x_ld, x_ld, op_lower ? OperandTriangle::kLowerB : OperandTriangle::kUpperB);
       }
       return;
     }
@@ -157,11 +166,11 @@ void Xtrsm<T>::TrsmColMajor(const Side side, const Triangle triangle, const Tran
     const auto rest_lo = first_half_first ? mid : lo, rest_hi = first_half_first ? hi : mid;  // updated, then solved
     solve(done_lo, done_hi, scaled);
     if (side == Side::kLeft) {  // B[rest, :] = factor * B[rest, :] - op(A)[rest, done] * X[done, :]
-      gemm(a_transpose, no, rest_hi - rest_lo, n, done_hi - done_lo, minus_one, dense_buffer, stored_at(rest_lo, done_lo),
-           k_padded, x_buffer, done_lo, x_ld, factor, b_buffer, b_offset + rest_lo, b_ld);
+      gemm(a_transpose, no, rest_hi - rest_lo, n, done_hi - done_lo, minus_one, a_buffer, stored_at(rest_lo, done_lo),
+           a_ld, x_buffer, done_lo, x_ld, factor, b_buffer, b_offset + rest_lo, b_ld);
     } else {                    // B[:, rest] = factor * B[:, rest] - X[:, done] * op(A)[done, rest]
-      gemm(no, a_transpose, m, rest_hi - rest_lo, done_hi - done_lo, minus_one, x_buffer, done_lo * x_ld, x_ld, dense_buffer,
-           stored_at(done_lo, rest_lo), k_padded, factor, b_buffer, b_offset + rest_lo * b_ld, b_ld);
+      gemm(no, a_transpose, m, rest_hi - rest_lo, done_hi - done_lo, minus_one, x_buffer, done_lo * x_ld, x_ld, a_buffer,
+           stored_at(done_lo, rest_lo), a_ld, factor, b_buffer, b_offset + rest_lo * b_ld, b_ld);
     }
     solve(rest_lo, rest_hi, true);
   };

@@ -116,13 +116,22 @@ CLBH_API int clbh_triangular_to_square(int precision, int upper, int unit_diagon
                                        long long src_offset, long long src_ld, void* dst, int dst_extent,
                                        long long dst_ld, hipStream_t stream);
 
+// The diagonal of that matrix in leaves, as a band: for b = 0 .. ceil(k / leaf) - 1 the dense leaf x leaf copy (made as
+// above, the identity beyond k) of the rows and columns from b * leaf on goes to dst + b * leaf * (leaf + 1) with leading
+// dimension `leaf`. The leaves follow each other down the diagonal of a matrix of `leaf` rows, so diagonal blocks of
+// equal size lie at a constant stride, leaf boundaries included; dst holds ceil(k / leaf) * leaf * (leaf + 1) elements,
+// the `leaf` elements between two leaves are not written.
+CLBH_API int clbh_triangular_to_band(int precision, int upper, int unit_diagonal, int k, int leaf, const void* src,
+                                     long long src_offset, long long src_ld, void* dst, hipStream_t stream);
+
 // Block size of clbh_invert_diagonal_blocks for a precision (64 for all three: larger blocks are cheaper to build by
 // doubling with GEMMs than inside the inversion kernel).
 CLBH_API int clbh_invert_block_size(int precision);
 
 // Inverts the `blocks` diagonal blocks (clbh_invert_block_size(precision) squared each) of the dense triangular matrix
-// `src` (blocks * block rows and columns, zeros in the other triangle, non-zero diagonal); block b of the result is
-// written to the same place of `dst` (leading dimension dst_ld) as it has in `src`: dst + b * block * (dst_ld + 1).
+// `src` (zeros in the other triangle, non-zero diagonal; block b at src + b * block * (src_ld + 1): a matrix of blocks *
+// block rows and columns, or a band as clbh_triangular_to_band writes it); block b of the result is written to the same
+// place of `dst` (leading dimension dst_ld) as it has in `src`: dst + b * block * (dst_ld + 1).
 CLBH_API int clbh_invert_diagonal_blocks(int precision, int upper, int blocks, const void* src, long long src_ld,
                                          void* dst, long long dst_ld, hipStream_t stream);
 
@@ -241,6 +250,9 @@ CLBH_API int clbh_complex_symmetric_to_square(int precision, int upper, int herm
 CLBH_API int clbh_complex_triangular_to_square(int precision, int upper, int unit_diagonal, int k, const void* src,
                                                long long src_offset, long long src_ld, void* dst, int dst_extent,
                                                long long dst_ld, hipStream_t stream);
+// clbh_triangular_to_band for complex matrices
+CLBH_API int clbh_complex_triangular_to_band(int precision, int upper, int unit_diagonal, int k, int leaf, const void* src,
+                                             long long src_offset, long long src_ld, void* dst, hipStream_t stream);
 // clbh_invert_block_size and clbh_invert_diagonal_blocks for complex matrices (blocks of 64 for 32-bit components, 32
 // for 64-bit ones)
 CLBH_API int clbh_complex_invert_block_size(int precision);

@@ -36,7 +36,8 @@ def test_trsm_sweep(gpu, bits):
             problem.check(b_after, TRSM_TOL[bits])
 
 
-@pytest.mark.parametrize("bits,m,n", [(32, 1024, 768), (64, 517, 1030), (32, 1536, 512), (32, 300, 2049), (64, 1300, 70)])
+@pytest.mark.parametrize("bits,m,n", [(32, 1024, 768), (64, 517, 1030), (32, 1536, 512), (32, 300, 2049), (64, 1300, 70),
+                                      (32, 2500, 260), (64, 2100, 130)])
 def test_trsm_large(gpu, bits, m, n):
     seed = 11000
     for layout, side, triangle, transpose, diagonal in MODES[::3]:
