@@ -390,7 +390,10 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     // the same way - it costs less: fitted to 8192^2 x k, k = 256 .. 8192, 1608 TFLOP/s and k0 = 467)
     const bool wide = triangular == 0 && m % 8 == 0 &&
                       ((m % 256 == 0 && n % 256 == 0 && k % 128 == 0) || (!a_kcontig && !b_kcontig && k >= 1000));
-    const auto cost256 = (k >= 256) ? cost(256, 1, wide ? 1608.0 : 1484.0, wide ? 467.0 : 627.0) : 1e300, cost128 = batch_128 * cost(128, 2, 936.0, 293.0),
+    // (whole tiles with k = 128 take it too: 8 x 4096^2 x 128 with beta = 0 67 us against 81 us on three 128 x 128
+    // work-groups per CU, 96 x 2048^2 x 128 267 against 296 us; with beta = 1 the two are level)
+    const bool whole_wide = wide && m % 256 == 0 && n % 256 == 0 && k % 128 == 0;
+    const auto cost256 = (k >= 256 || whole_wide) ? cost(256, 1, wide ? 1608.0 : 1484.0, wide ? 467.0 : 627.0) : 1e300, cost128 = batch_128 * cost(128, 2, 936.0, 293.0),
                cost64 = batch_64 * cost(64, 4, long_k ? 371.0 : 488.0, 44.0);
     int tile = 1;
     if (cost256 <= cost128 && cost256 <= cost64) { tile = 2; }

@@ -54,11 +54,13 @@ def test_whole_tiles(forced):
 
 
 def test_edges_under_a_long_k(forced):
-    """Two x-contiguous operands (column-major N/T, row-major T/N) and k >= 2048: the instance with range checks - edge
-    tiles in m and n, a K that is no multiple of the slab, of eight or of two, rows of C that straddle the last row."""
+    """Two x-contiguous operands (column-major N/T, row-major T/N) and k >= 1000: the instance with range checks where the
+    rows are a multiple of 8 - edge tiles in m and n, a K that is no multiple of the slab, of eight or of two - and the
+    eight-wavefront kernel for the other row counts."""
     seed = 9200
     for (layout, ta, tb), (m, n, k) in itertools.product(((COL_MAJOR, NO, YES), (ROW_MAJOR, YES, NO)),
-                                                         ((300, 520, 2056), (257, 255, 2051), (515, 262, 2176), (1000, 300, 2500))):
+                                                         ((300, 520, 2056), (257, 255, 2051), (515, 262, 2176), (1000, 300, 2500),
+                                                          (520, 300, 2056), (264, 255, 1003), (1016, 262, 2176), (8, 700, 1000))):
         seed += 1
         problem = gpu_harness.Problem(16, layout, ta, tb, m, n, k, -0.75, 0.0 if seed % 2 else 2.0, a_offset=2, b_offset=4,
                                       c_offset=6, seed=seed, extra_ld=(2, 4, 6), ab_low=-0.5, ab_high=0.5)
@@ -101,4 +103,31 @@ def test_strided_batches_of_whole_tiles(forced):
     for i in range(batch):
         where = oracle.c_indices(COL_MAJOR, m, n, i * m * n, m)
         assert oracle.rel_frobenius(results[0][where], expected[i]) <= 1e-2, i
+    assert np.array_equal(results[0].view(np.uint16), results[1].view(np.uint16))
+
+
+@pytest.mark.parametrize("m,n,k,batch", [(512, 512, 256, 70), (520, 264, 1000, 67)])
+def test_more_items_than_work_groups(forced, m, n, k, batch):
+    """More tiles than compute units: the persistent work-groups walk several (tile, matrix) items each, the slabs of
+    one item following those of the last through the ring; whole tiles without and ragged ones with range checks."""
+    import torch
+    import oracle
+    rng = np.random.default_rng(9500 + m)
+    a = rng.uniform(-0.5, 0.5, batch * k * m).astype(np.float16)
+    b = rng.uniform(-0.5, 0.5, batch * k * n).astype(np.float16)
+    c = rng.uniform(-1.0, 1.0, batch * n * m).astype(np.float16)
+    results = []
+    for variant in (WIDE_OR_NOT, EIGHT_WAVES):
+        clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": variant})
+        a_dev, b_dev, c_dev = (torch.from_numpy(x).to("cuda:0") for x in (a, b, c))
+        status = clblast_amd.raw_gemm_strided_batched("H", COL_MAJOR, NO, YES, m, n, k, -0.5, a_dev.data_ptr(), 0, m, m * k,
+                                                      b_dev.data_ptr(), 0, n, n * k, 0.75, c_dev.data_ptr(), 0, m, m * n, batch,
+                                                      gpu_harness.stream_handle())
+        torch.cuda.synchronize()
+        assert status == 0
+        results.append(c_dev.cpu().numpy())
+    for i in (0, batch // 2, batch - 1):
+        expected = oracle.gemm(COL_MAJOR, NO, YES, m, n, k, -0.5, a, i * m * k, m, b, i * n * k, n, 0.75, c, i * m * n, m)
+        where = oracle.c_indices(COL_MAJOR, m, n, i * m * n, m)
+        assert oracle.rel_frobenius(results[0][where], expected) <= 1e-2, i
     assert np.array_equal(results[0].view(np.uint16), results[1].view(np.uint16))
