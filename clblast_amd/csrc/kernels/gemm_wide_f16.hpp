@@ -92,23 +92,16 @@ __device__ __forceinline__ void WidePermlane16Swap(float (&first)[4], float (&se
       : "+v"(first[0]), "+v"(first[1]), "+v"(first[2]), "+v"(first[3]), "+v"(second[0]), "+v"(second[1]), "+v"(second[2]), "+v"(second[3]));
 }
 
-#ifdef WIDE_TIMELINE
-__device__ long long wide_timeline[256 * 64];
-#define WIDE_MARK(i) { asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(marks[i]) :: "memory"); }
-#else
-#define WIDE_MARK(i)
-#endif
 // RANGE: range-checked requests (some tile touches an edge of the matrix, or K is not a multiple of 128); without,
 // every tile is whole and the byte count per slab and operand is saved.
 //
 // The work-groups are persistent: grid.x of them (one per compute unit) take the items - tiles of all matrices of the
-// batch - g, g + grid.x, ... Behind the K walk of an item the first turn of the ring of the NEXT item is requested
-// before the epilogue starts, so the epilogue's stores and the next walk's first slabs overlap; the queue of memory
-// operations then holds, oldest first: the next item's four slabs, the stores. The waits of a walk's first turn count
-// those stores: every epilogue issues at least HwideConfig::STORES of them per wavefront (pieces outside the matrix go
-// to offsets outside the view of C and move nothing; tiles on the last rows of C add element-wise stores, which only
-// makes the waits stricter than needed), and at the very start as many stores that move nothing are issued, so that
-// the first item sees the same queue.
+// batch - g, g + grid.x, ... Under the last turn of the K walk of an item the first turn of the ring of the NEXT item
+// is requested, so the epilogue's stores and the next walk's first slabs overlap; the queue of memory operations
+// then holds, oldest first: the next item's four slabs, the stores. The waits of a walk's first turn count
+// those stores: every epilogue issues exactly HwideConfig::STORES of them per wavefront (pieces outside the matrix go
+// to offsets outside the view of C and move nothing), and at the very start as many stores that move nothing are
+// issued, so that the first item sees the same queue.
 template <bool A_KC, bool B_KC, bool RANGE>
 __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const GemmArgs<float> p, const int tiles_m,
                                                                            const int tiles_n) {
@@ -278,15 +271,7 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
     for (int i = 0; i < Config::STORES; ++i) { BufferStore<T, 8>(zeros, nothing, 0); }
   }
 
-#ifdef WIDE_TIMELINE
-  int ordinal = -1;
-#endif
   for (; item < items; item += gridDim.x) {
-#ifdef WIDE_TIMELINE
-    ++ordinal;
-    long long marks[6];
-#endif
-    WIDE_MARK(0);
     // the tile of C of this item
     const int batch = item / tiles;
     int tile_m, tile_n;
@@ -302,10 +287,9 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
     wide_acc_t acc[BM][BN];  // written by the first slab
     plan_first_turn(item + gridDim.x);
 
-    // Old C. The first two strips are fetched under the MFMAs of the last turn of the K walk, into registers the walk
-    // leaves free, the other two right behind the walk into the registers of the fragments. With beta == 0 the same
-    // loads run with an offset outside the view (no memory is touched), so the code and the count of loads in flight
-    // do not depend on beta.
+    // Old C, fetched under the MFMAs of the last turn of the K walk (see kEarlyStrip0). With beta == 0 the same loads run
+    // with an offset outside the view (no memory is touched), so the code and the count of loads in flight do not
+    // depend on beta.
     const int wave_m0 = m0 + wave_m * WAVE_M, wave_n0 = n0 + wave_n * (BN * 16);
     const auto c_view = __builtin_amdgcn_make_buffer_rsrc(c + wave_n0 * p.c_ld + wave_m0, 0, kHOutside, kRawBufferFlags);
     const int c_inside = p.m - (wave_m0 + c_lane_m);   // rows of C from the lane's first one (of pair 0) to the matrix's edge
@@ -333,7 +317,6 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
       // the first four slabs of this item have landed: the youngest operations in the queue are the stores of the
       // previous epilogue (or the stores that stand in for them ahead of the first item), all requests are older
       asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PENDING) : "memory");
-      WIDE_MARK(1);
       half8_t a_frag[2][BM], b_frag[2][BN];
 #pragma unroll
       for (int q = 0; q < BM; ++q) { a_frag[0][q] = HFragment<TILE_M, A_KC>(a_read[q], 0); }
@@ -410,14 +393,11 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
       }
       asm volatile("; WIDE_WALK_END" ::: "memory");
       WideMfmaDrain(acc);
-      WIDE_MARK(2);
     }
 
     // Epilogue: piece by piece the accumulators' values are exchanged between the rows of lanes (see above), combined
     // with the old values in fp32, rounded once and stored; no LDS, no dependence between pieces.
     {
-      WIDE_MARK(3);
-      WIDE_MARK(4);
       auto combine = [&](auto use_c_tag) {
         constexpr bool USE_C = decltype(use_c_tag)::value;
 #pragma unroll
@@ -460,12 +440,6 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
         }
       };
       if (beta != 0.0f) { combine(std::true_type{}); } else { combine(std::false_type{}); }
-      WIDE_MARK(5);
-#ifdef WIDE_TIMELINE
-      if (threadIdx.x == 0 && ordinal < 8) {
-        for (int i = 0; i < 6; ++i) { wide_timeline[blockIdx.x * 64 + ordinal * 8 + i] = marks[i]; }
-      }
-#endif
     }
   }
 }
