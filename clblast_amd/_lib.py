@@ -134,7 +134,7 @@ NETLIB_SYMBOLS = (["cblas_%sgemm" % p for p in "sdcz"] +
                   ["cblas_%s%s" % (p, r) for p in "sdcz" for r in ("symm", "syrk", "syr2k", "trmm", "trsm")] +
                   ["cblas_%s%s" % (p, r) for p in "cz" for r in ("hemm", "herk", "her2k")])
 DEVICE_LAYER_SYMBOLS = [
-    "clbh_gemm_launch", "clbh_gemm_workspace_bytes", "clbh_buffer_extent", "clbh_alloc_async", "clbh_free_async",
+    "clbh_gemm_launch", "clbh_gemm_workspace_bytes", "clbh_gemm_workspace_optional", "clbh_buffer_extent", "clbh_alloc_async", "clbh_free_async",
     "clbh_upload_async", "clbh_event_record", "clbh_stream_device", "clbh_error_string", "clbh_symmetric_to_square",
     "clbh_triangular_to_square", "clbh_triangular_to_band", "clbh_complex_triangular_to_band", "clbh_copy_matrix", "clbh_invert_block_size", "clbh_invert_diagonal_blocks",
     "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale", "clbh_complex_expand_batched",

@@ -268,10 +268,16 @@ size_t clbh_gemm_workspace_bytes(const clbh_gemm_desc* desc) {
     return clbh::PlanSkinnyCols(*desc).workspace_bytes;
   }
   if (desc == nullptr || desc->kernel_class != CLBH_KERNEL_MFMA) { return 0; }
+  const auto wide = clbh::PlanWide(*desc);
+  if (wide.form != 0) { return wide.workspace_bytes; }  // (never together with K ranges as batch entries)
   const auto plan = clbh::PlanSplit(*desc);
   if (plan.splits <= 1) { return 0; }
   const auto element_bytes = static_cast<size_t>(desc->precision == 16 ? 4 : desc->precision / 8);  // fp16 sums in fp32
   return element_bytes * plan.splits * plan.ld * static_cast<size_t>(desc->n);
+}
+
+int clbh_gemm_workspace_optional(const clbh_gemm_desc* desc) {
+  return (desc != nullptr && desc->kernel_class == CLBH_KERNEL_MFMA && clbh::PlanWide(*desc).form != 0) ? 1 : 0;
 }
 
 int clbh_symmetric_to_square(int precision, int upper, int k, const void* src, long long src_offset, long long src_ld,

@@ -129,16 +129,33 @@ bool DwordAlignedHalf(const clbh_gemm_desc& d) {
 // ---- 256 x 256 tiles with one wavefront per SIMD (kernels/gemm_wide_f16.hpp) ---------------------------
 template <bool A_KC, bool B_KC, bool RANGE>
 int LaunchHwideVariant(const clbh_gemm_desc& d, hipStream_t stream) {
-  const auto args = MakeArgs<float>(d);
-  const long long tiles_m = (d.m + HwideConfig::TILE_M - 1) / HwideConfig::TILE_M;
-  const long long tiles_n = (d.n + HwideConfig::TILE_N - 1) / HwideConfig::TILE_N;
-  if (tiles_m * tiles_n * d.batch_count > INT_MAX) { return hipErrorInvalidConfiguration; }
+  auto args = MakeArgs<float>(d);
+  const auto plan = PlanWide(d);
+  if (plan.form == 0 || plan.items > INT_MAX) { return hipErrorInvalidConfiguration; }
+  const int tiles_m = static_cast<int>(plan.tiles_m), tiles_n = static_cast<int>(plan.tiles_n);
   // persistent work-groups, one per compute unit (a multiple of the eight XCDs, which the tile order counts on)
-  int units = 0;
-  if (clbh_compute_units(&units) != 0 || units < 8) { units = 256; }
-  const long long items = tiles_m * tiles_n * d.batch_count;
-  const dim3 grid(static_cast<unsigned>(std::min<long long>(items, units - units % 8)));
-  HgemmWideKernel<A_KC, B_KC, RANGE><<<grid, dim3(HwideConfig::THREADS), 0, stream>>>(args, static_cast<int>(tiles_m), static_cast<int>(tiles_n));
+  const dim3 grid(static_cast<unsigned>(plan.grid));
+  const bool split = plan.parts > 1 && d.workspace != nullptr && d.workspace_bytes >= plan.workspace_bytes;
+  if (!split && d.c_triangle == 0) {
+    HgemmWideKernel<A_KC, B_KC, RANGE, false><<<grid, dim3(HwideConfig::THREADS), 0, stream>>>(args, tiles_m, tiles_n,
+                                                                                              static_cast<int>(plan.tiles));
+    return static_cast<int>(hipGetLastError());
+  }
+  // a triangle of C, or a last round of tiles split into K ranges whose sums a second kernel adds up
+  long long items = plan.tiles;
+  if (split) {
+    args.tail_first = static_cast<int>(plan.tail_first);
+    args.tail_parts = plan.parts;
+    args.tail_groups = plan.groups_per_part;
+    args.tail_partials = static_cast<float*>(d.workspace);
+    items = plan.items;
+  }
+  HgemmWideKernel<A_KC, B_KC, RANGE, true><<<grid, dim3(HwideConfig::THREADS), 0, stream>>>(args, tiles_m, tiles_n,
+                                                                                           static_cast<int>(items));
+  if (split) {
+    HgemmWideFixupKernel<<<dim3(static_cast<unsigned>((plan.tiles - plan.tail_first) * kWideFixupGroupsPerTile)), dim3(256), 0, stream>>>(
+        args, tiles_m, tiles_n, plan.all_groups);
+  }
   return static_cast<int>(hipGetLastError());
 }
 
@@ -151,26 +168,6 @@ int LaunchHwide(const clbh_gemm_desc& d, hipStream_t stream) {
     case 2: return LaunchHwideVariant<true, false, RANGE>(d, stream);
     default: return LaunchHwideVariant<true, true, RANGE>(d, stream);
   }
-}
-
-// Which form of the 256 x 256 tile a launch takes: 0 the eight-wavefront kernel, 1 the wide kernel without range
-// checks (whole tiles, K a multiple of 128), 2 the wide kernel with them. The wide kernel moves C in 16-byte pieces of
-// eight rows and addresses with 32-bit byte offsets. Measured against the eight-wavefront kernel (same box, us): whole
-// tiles 8192^2 x 256 67 / 85, x 1024 130 / 157, 8192^3 N/T 755 / 832, 4096^3 106 / 118, with a k-contiguous operand
-// 8192^2 x 256 71 / 85; with range checks and two x-contiguous operands 4096^2 x 1000 38 / 44, 5000^3 222 / 267,
-// 8192^2 x 1312 163 / 174 (K padded to 1408); with range checks and a k-contiguous operand it loses (5000^3 T/N 311 /
-// 289).
-int WideForm(const clbh_gemm_desc& d) {
-  if (d.conv != nullptr || d.c_triangle != 0 || d.operand_triangle != 0 || PlanSplit(d).splits > 1) { return 0; }
-  constexpr long long kMaxLd = 1ll << 21;
-  if (d.a_ld >= kMaxLd || d.b_ld >= kMaxLd || d.c_ld >= kMaxLd || d.c_ld % 2 != 0) { return 0; }
-  const auto c_address = reinterpret_cast<unsigned long long>(d.c) + 2ull * static_cast<unsigned long long>(d.c_offset);
-  if (c_address % 4 != 0) { return 0; }
-  if (d.batch_count > 1 && (d.batch.alphas != nullptr || d.c_stride % 2 != 0)) { return 0; }
-  if ((d.a_kcontig || d.b_kcontig) && d.k % 8 != 0) { return 0; }
-  if (d.m % 8 != 0) { return 0; }  // (C moves in pieces of eight rows)
-  if (d.m % HwideConfig::TILE_M == 0 && d.n % HwideConfig::TILE_N == 0 && d.k % (HwideConfig::TILE_K * HwideConfig::STAGES) == 0) { return 1; }
-  return (!d.a_kcontig && !d.b_kcontig && d.k >= 1000) ? 2 : 0;
 }
 
 // CONVGEMM with the A operand gathered from the images (clbh_gemm_desc::conv; HGatherPiece names the conditions): the
@@ -203,7 +200,7 @@ int LaunchMfmaF16(const clbh_gemm_desc& d, hipStream_t stream) {
   switch (d.tile_variant) {
     case 1: return LaunchHdirectConfig<HdirectConfig<2, 2, 1, 1, 4>>(d, stream);  // 64 x 64, 4 wavefronts
     case 2:  // 256 x 256: four wavefronts of 128 x 128 where that kernel applies, else eight of 128 x 64
-      switch (WideForm(d)) {
+      switch (PlanWide(d).form) {
         case 1: return LaunchHwide<false>(d, stream);
         case 2: return LaunchHwide<true>(d, stream);
         default: return LaunchHdirectConfig<HdirectConfig<2, 4, 4, 2, 2>>(d, stream);

@@ -54,6 +54,12 @@ struct GemmArgs {
   int c_triangle;
   int operand_triangle;
   ConvGather conv;  // enabled != 0: `a` is a batch of images (a_stride apart) instead of a matrix, see ConvGather
+  // The persistent fp16 kernel (kernels/gemm_wide_f16.hpp) when the last round of its tiles would fill few of the
+  // work-groups: the tiles from number tail_first on are split into tail_parts K ranges of tail_groups * 128 each, one
+  // item per range, whose sums go to tail_partials ([item - tail_first][256 x 256], column-major) and are added up,
+  // scaled and stored by a second kernel. tail_parts == 0: nothing is split.
+  int tail_first, tail_parts, tail_groups;
+  float* tail_partials;
 };
 
 // c_triangle: 1 keeps C(i,j) with i <= j, 2 with i >= j. 3 and 4 are the same for a complex matrix stored as a real

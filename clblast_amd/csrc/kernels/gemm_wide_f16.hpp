@@ -28,9 +28,14 @@
 //   * C moves straight between memory and the accumulators' values in 16-byte pieces (v_permlane16_swap gathers eight
 //     consecutive rows of a column in one lane): for the length of the epilogue the matrix pipe stands still, and an
 //     epilogue staged through LDS - thirteen, later three LDS round trips per 16 columns - took 11 us of a tile's 187.
-// Requirements (the launcher checks them): dword-aligned operands, no triangles, no split-K, no gathered
-// operand; a k-contiguous operand needs k % 8 == 0 (its K tail is cut by giving whole 16-byte chunks an
-// offset outside the buffer's range); m % 8 == 0 (C moves in pieces of eight rows, each inside the matrix or not).
+//   * the GENERAL instances also walk the tiles of a triangle of a square C (tiles on the diagonal store under a mask:
+//     the other triangle's elements go back as they were read) and split the tiles of a last round that would fill at
+//     most half of the work-groups into K ranges, one item each, whose sums a second kernel adds up
+//     (HgemmWideFixupKernel) - 528 tiles on 256 work-groups then cost two rounds and a short one instead of three.
+// Requirements (the launcher checks them): dword-aligned operands, no triangular operand, no K ranges as batch
+// entries, no gathered operand; a k-contiguous operand needs k % 8 == 0 (its K tail is cut by giving whole 16-byte
+// chunks an offset outside the buffer's range); m % 8 == 0 (C moves in pieces of eight rows, each inside the matrix or
+// not); a triangle of C needs m == n.
 // =================================================================================================
 #ifndef CLBLAST_HIP_KERNELS_GEMM_WIDE_F16_HPP_
 #define CLBLAST_HIP_KERNELS_GEMM_WIDE_F16_HPP_
@@ -92,6 +97,73 @@ __device__ __forceinline__ void WidePermlane16Swap(float (&first)[4], float (&se
       : "+v"(first[0]), "+v"(first[1]), "+v"(first[2]), "+v"(first[3]), "+v"(second[0]), "+v"(second[1]), "+v"(second[2]), "+v"(second[3]));
 }
 
+// The tiles of a triangle of a square C of `along` x `along` tiles in an order with the locality of TileOfBlock: groups of
+// eight tile rows, column by column inside a group (upper triangle, tile row <= tile column: a group holds the
+// triangle on its own eight columns, then whole columns of eight), a contiguous range of that order per XCD. The
+// lower triangle is the mirror image. `index` counts 0 .. TriangleTiles(along) - 1.
+__device__ __host__ __forceinline__ int TriangleTiles(const int along) { return along * (along + 1) / 2; }
+__device__ __forceinline__ void TriangleTileOfBlock(const int index, const int along, const bool upper, int& tile_m, int& tile_n) {
+  int rest = XcdContiguousIndex(index, TriangleTiles(along));
+  int first = 0, rows = min(8, along);
+  while (first + rows < along) {  // (at most along / 8 turns, scalar; the last group takes what is left)
+    const int in_group = rows * (rows + 1) / 2 + rows * (along - first - rows);
+    if (rest < in_group) { break; }
+    rest -= in_group;
+    first += rows;
+    rows = min(8, along - first);
+  }
+  int row, column;
+  const int corner = rows * (rows + 1) / 2;
+  if (rest < corner) {  // column first + c of the group's own triangle holds the rows first .. first + c
+    int c = 0;
+    while (rest >= (c + 1) * (c + 2) / 2) { ++c; }
+    column = first + c;
+    row = first + rest - c * (c + 1) / 2;
+  } else {
+    column = first + rows + (rest - corner) / rows;
+    row = first + (rest - corner) % rows;
+  }
+  tile_m = upper ? row : column;
+  tile_n = upper ? column : row;
+}
+
+// What an item of a launch is: a tile of a matrix of the batch, the turns of the ring (128 k each) it walks, and where
+// its sums go - into C (slot < 0) or, for one K range of a split tile, into a slot of partial sums.
+struct WideItem {
+  int tile_m, tile_n, batch, first_group, groups, slot;
+};
+// GENERAL: launches over a triangle of C, and launches that split the tiles from p.tail_first on into K ranges.
+template <bool GENERAL>
+__device__ __forceinline__ WideItem WideItemOf(const GemmArgs<float>& p, const int tiles_m, const int tiles_n, const int item,
+                                              const int all_groups) {
+  WideItem w;
+  const int tiles = tiles_m * tiles_n;
+  if constexpr (!GENERAL) {
+    w.batch = item / tiles;
+    TileOfBlock(item - w.batch * tiles, tiles, tiles_m, tiles_n, w.tile_m, w.tile_n);
+    w.first_group = 0;
+    w.groups = all_groups;
+    w.slot = -1;
+  } else {
+    int logical = item;
+    w.first_group = 0;
+    w.groups = all_groups;
+    w.slot = -1;
+    if (p.tail_parts > 0 && item >= p.tail_first) {
+      w.slot = item - p.tail_first;
+      logical = p.tail_first + w.slot / p.tail_parts;
+      w.first_group = (w.slot % p.tail_parts) * p.tail_groups;
+      w.groups = min(p.tail_groups, all_groups - w.first_group);
+    }
+    const int per_matrix = (p.c_triangle != 0) ? TriangleTiles(tiles_m) : tiles;
+    w.batch = logical / per_matrix;
+    const int index = logical - w.batch * per_matrix;
+    if (p.c_triangle != 0) { TriangleTileOfBlock(index, tiles_m, p.c_triangle == 1, w.tile_m, w.tile_n); }
+    else { TileOfBlock(index, tiles, tiles_m, tiles_n, w.tile_m, w.tile_n); }
+  }
+  return w;
+}
+
 // RANGE: range-checked requests (some tile touches an edge of the matrix, or K is not a multiple of 128); without,
 // every tile is whole and the byte count per slab and operand is saved.
 //
@@ -102,9 +174,9 @@ __device__ __forceinline__ void WidePermlane16Swap(float (&first)[4], float (&se
 // those stores: every epilogue issues exactly HwideConfig::STORES of them per wavefront (pieces outside the matrix go
 // to offsets outside the view of C and move nothing), and at the very start as many stores that move nothing are
 // issued, so that the first item sees the same queue.
-template <bool A_KC, bool B_KC, bool RANGE>
+template <bool A_KC, bool B_KC, bool RANGE, bool GENERAL = false>
 __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const GemmArgs<float> p, const int tiles_m,
-                                                                           const int tiles_n) {
+                                                                           const int tiles_n, const int items) {
   using T = _Float16;
   using Config = HwideConfig;
   constexpr int TILE_M = Config::TILE_M, TILE_N = Config::TILE_N, TILE_K = Config::TILE_K, STAGES = Config::STAGES;
@@ -123,7 +195,6 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   T* old_c_lds = lds + 2 * STAGES * ELEMS + wave_u * 4096;  // [8 pieces][64 lanes][8]: the last strip of old C of this wavefront
   const int wave_m = wave_u % Config::WM, wave_n = wave_u / Config::WM;  // (uniform: C is addressed through a buffer view per wavefront)
-  const int tiles = tiles_m * tiles_n, items = tiles * p.batch_count;
 
   // LDS positions of the lane's fragments inside a slab buffer
   const T* a_read[BM];
@@ -135,7 +206,7 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
 
   const int k_len = p.k;
   const int slabs = (k_len + TILE_K - 1) / TILE_K;
-  const int groups = (slabs + STAGES - 1) / STAGES;  // the walk runs whole turns of the ring
+  const int all_groups = (slabs + STAGES - 1) / STAGES;  // the walk runs whole turns of the ring (of an item's K range: WideItem)
 
   // A request of this wavefront: round r < 4 fetches piece wave + 4 r of A, round 4 + r that piece of B. The lane's byte
   // offset from the slab's first row is kept per round (the range check of a buffer load looks at the vector offset
@@ -159,6 +230,7 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
   const T* a_end = nullptr;
   const T* b_end = nullptr;
   int request_k = 0;
+  int request_k_len = k_len;  // extent of the K range whose slabs are being requested
   int request_open = -1;  // 0 behind the last item: the requests of a next item's first turn are issued all the same, and move nothing
   auto a_resource = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a_request), 0, 0, kRawBufferFlags);
   auto b_resource = a_resource;
@@ -182,11 +254,11 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
     const int place = (wave_u + WAVES * r) * 512;
     if (round < ROUNDS / 2) {
       int offset = a_bytes[r];
-      if (A_KC && RANGE) { offset = (request_k + a_lane_k < k_len) ? offset : static_cast<int>(0x80000000u); }
+      if (A_KC && RANGE) { offset = (request_k + a_lane_k < (GENERAL ? request_k_len : k_len)) ? offset : static_cast<int>(0x80000000u); }
       __builtin_amdgcn_raw_ptr_buffer_load_lds(a_resource, (LdsPtr)(a_ring + buffer * ELEMS + place), 16, offset, 0, 0, 0);
     } else {
       int offset = b_bytes[r];
-      if (B_KC && RANGE) { offset = (request_k + b_lane_k < k_len) ? offset : static_cast<int>(0x80000000u); }
+      if (B_KC && RANGE) { offset = (request_k + b_lane_k < (GENERAL ? request_k_len : k_len)) ? offset : static_cast<int>(0x80000000u); }
       __builtin_amdgcn_raw_ptr_buffer_load_lds(b_resource, (LdsPtr)(b_ring + buffer * ELEMS + place), 16, offset, 0, 0, 0);
     }
   };
@@ -206,29 +278,33 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
   const T* planned_a_end = nullptr;
   const T* planned_b_end = nullptr;
   int planned_open = 0;
+  int planned_k_len = k_len;
   auto plan_first_turn = [&](const int wanted) {
     planned_open = (wanted < items) ? -1 : 0;
-    const int planned_item = (wanted < items) ? wanted : 0;
-    const int batch = planned_item / tiles;
-    int tile_m, tile_n;
-    TileOfBlock(planned_item - batch * tiles, tiles, tiles_m, tiles_n, tile_m, tile_n);
+    const WideItem planned = WideItemOf<GENERAL>(p, tiles_m, tiles_n, (wanted < items) ? wanted : 0, all_groups);
     const T* a;
     const T* b;
     T* c;
     float alpha, beta;
-    ResolveBatch<T, float>(p, batch, a, b, c, alpha, beta);
-    planned_a = a + (A_KC ? tile_m * TILE_M * p.a_ld : static_cast<long long>(tile_m * TILE_M));  // element (m0, k = 0), uniform
-    planned_b = b + (B_KC ? tile_n * TILE_N * p.b_ld : static_cast<long long>(tile_n * TILE_N));
-    planned_a_end = a + (A_KC ? (p.m - 1) * p.a_ld + k_len : (k_len - 1) * p.a_ld + p.m);
-    planned_b_end = b + (B_KC ? (p.n - 1) * p.b_ld + k_len : (k_len - 1) * p.b_ld + p.n);
+    ResolveBatch<T, float>(p, planned.batch, a, b, c, alpha, beta);
+    // the item's K range [k_first, k_last): all of K unless the tile is split
+    const int k_first = planned.first_group * (STAGES * TILE_K);
+    const int k_last = GENERAL ? min(k_len, k_first + planned.groups * (STAGES * TILE_K)) : k_len;
+    planned_k_len = k_last - k_first;
+    // element (m0, k_first), uniform
+    planned_a = a + (A_KC ? planned.tile_m * TILE_M * p.a_ld + k_first : k_first * p.a_ld + planned.tile_m * TILE_M);
+    planned_b = b + (B_KC ? planned.tile_n * TILE_N * p.b_ld + k_first : k_first * p.b_ld + planned.tile_n * TILE_N);
+    planned_a_end = a + (A_KC ? (p.m - 1) * p.a_ld + k_last : (k_last - 1) * p.a_ld + p.m);
+    planned_b_end = b + (B_KC ? (p.n - 1) * p.b_ld + k_last : (k_last - 1) * p.b_ld + p.n);
   };
-  auto switch_requests = [&]() {  // from here on the requests fetch the planned item, from its slab 0 on
+  auto switch_requests = [&]() {  // from here on the requests fetch the planned item, from its first slab on
     request_open = planned_open;
     a_request = planned_a;
     b_request = planned_b;
     a_end = planned_a_end;
     b_end = planned_b_end;
     request_k = 0;
+    request_k_len = planned_k_len;
     refresh_resources();
   };
 
@@ -273,17 +349,21 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
 
   for (; item < items; item += gridDim.x) {
     // the tile of C of this item
-    const int batch = item / tiles;
-    int tile_m, tile_n;
-    TileOfBlock(item - batch * tiles, tiles, tiles_m, tiles_n, tile_m, tile_n);
-    const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
+    const WideItem here = WideItemOf<GENERAL>(p, tiles_m, tiles_n, item, all_groups);
+    const int groups = here.groups;
+    const int m0 = here.tile_m * TILE_M, n0 = here.tile_n * TILE_N;
     T* c;
     float alpha, beta;
     {
       const T* a;
       const T* b;
-      ResolveBatch<T, float>(p, batch, a, b, c, alpha, beta);
+      ResolveBatch<T, float>(p, here.batch, a, b, c, alpha, beta);
     }
+    // GENERAL: a tile on the diagonal of a triangle of C keeps the old values of the other triangle's elements (they are
+    // stored back as they were read); the sums of one K range of a split tile go to their slot as they are
+    const bool masked = GENERAL && p.c_triangle != 0 && here.tile_m == here.tile_n;
+    const bool to_slot = GENERAL && here.slot >= 0;
+    const bool fetch_c = !to_slot && (beta != 0.0f || masked);
     wide_acc_t acc[BM][BN];  // written by the first slab
     plan_first_turn(item + gridDim.x);
 
@@ -299,13 +379,13 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
       return !RANGE || (16 * (2 * strip + pass / 4) < c_cols_left && c_inside - 32 * (pass % 4) >= 8);
     };
     const auto c_load = [&](const int strip, const int pass) {
-      if (RANGE) { return BufferLoad<T, 8>(c_view, (beta != 0.0f && c_piece_there(strip, pass)) ? c_lane_offset + c_uniform(strip, pass) : kHOutside); }
-      return BufferLoad<T, 8>(c_view, (beta != 0.0f) ? c_lane_offset : kHOutside, c_uniform(strip, pass));
+      if (RANGE) { return BufferLoad<T, 8>(c_view, (fetch_c && c_piece_there(strip, pass)) ? c_lane_offset + c_uniform(strip, pass) : kHOutside); }
+      return BufferLoad<T, 8>(c_view, fetch_c ? c_lane_offset : kHOutside, c_uniform(strip, pass));
     };
     const auto c_load_to_lds = [&](const int pass) {  // piece `pass` of strip 3: lane l's 16 bytes land at old_c_lds[pass][l]
       // (every operand of the load worked out beforehand: with a call among the load's own arguments the host pass of
       // the compiler drops this kernel's launch stub without a word)
-      const bool wanted = beta != 0.0f && c_piece_there(STRIPS - 1, pass);
+      const bool wanted = fetch_c && c_piece_there(STRIPS - 1, pass);
       const int piece_offset = c_lane_offset + c_uniform(STRIPS - 1, pass);
       const int offset = wanted ? piece_offset : kHOutside;
       LdsPtr place = (LdsPtr)(old_c_lds + pass * 512);
@@ -398,8 +478,10 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
     // Epilogue: piece by piece the accumulators' values are exchanged between the rows of lanes (see above), combined
     // with the old values in fp32, rounded once and stored; no LDS, no dependence between pieces.
     {
-      auto combine = [&](auto use_c_tag) {
+      auto combine = [&](auto use_c_tag, auto masked_tag) {
         constexpr bool USE_C = decltype(use_c_tag)::value;
+        constexpr bool MASKED = decltype(masked_tag)::value;  // a tile on the diagonal of a triangle of C (reads old C)
+        static_assert(USE_C || !MASKED, "the elements outside the triangle are stored back as they were read");
 #pragma unroll
         for (int strip = 0; strip < STRIPS; ++strip) {
 #pragma unroll
@@ -431,17 +513,97 @@ __global__ __launch_bounds__(HwideConfig::THREADS, 1) void HgemmWideKernel(const
             half8_t out;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-              if constexpr (USE_C) { out[e] = Narrow<T, float>(Combine(alpha, values[e], beta, static_cast<float>(old[e]))); }
-              else { out[e] = Narrow<T, float>(alpha * values[e]); }
+              if constexpr (MASKED) {
+                const float fresh = (beta != 0.0f) ? Combine(alpha, values[e], beta, static_cast<float>(old[e])) : alpha * values[e];
+                const bool kept = InTriangle(p.c_triangle, wave_m0 + c_lane_m + 32 * pair + e, wave_n0 + 16 * j + lane % 16);
+                out[e] = kept ? Narrow<T, float>(fresh) : old[e];
+              } else if constexpr (USE_C) {
+                out[e] = Narrow<T, float>(Combine(alpha, values[e], beta, static_cast<float>(old[e])));
+              } else {
+                out[e] = Narrow<T, float>(alpha * values[e]);
+              }
             }
             if (RANGE) { BufferStore<T, 8>(out, c_view, c_piece_there(strip, pass) ? c_lane_offset + c_uniform(strip, pass) : kHOutside); }
             else { BufferStore<T, 8>(out, c_view, c_lane_offset, c_uniform(strip, pass)); }
           }
         }
       };
-      if (beta != 0.0f) { combine(std::true_type{}); } else { combine(std::false_type{}); }
+      // The sums of one K range of a split tile: sixteen bytes per lane and block of 16 x 16 (four consecutive rows of a
+      // column) into the item's slot, a column-major 256 x 256 matrix of floats. (More stores than the epilogues that the
+      // waits of the next walk count on: those waits then wait for more than they need to, never for less.)
+      auto store_sums = [&]() {
+        float* slot = p.tail_partials + static_cast<long long>(here.slot) * (TILE_M * TILE_N) + wave_n * (BN * 16) * TILE_M + wave_m * WAVE_M;
+        const int slot_bytes = (TILE_N - wave_n * (BN * 16)) * TILE_M * 4;
+        const auto slot_view = __builtin_amdgcn_make_buffer_rsrc(slot, 0, slot_bytes, kRawBufferFlags);
+        const int lane_bytes = ((lane % 16) * TILE_M + 4 * (lane / 16)) * 4;
+        typedef float float4_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int j = 0; j < BN; ++j) {
+#pragma unroll
+          for (int i = 0; i < BM; ++i) {
+            if (i % 2 == 0) { __builtin_amdgcn_sched_barrier(0); }
+            float4_t sums;
+            float part[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(part[r]) : "a"(acc[i][j][r])); }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { sums[r] = part[r]; }
+            BufferStore<float, 4>(sums, slot_view, lane_bytes, (16 * j * TILE_M + 16 * i) * 4);
+          }
+        }
+      };
+      if (GENERAL && to_slot) { store_sums(); }
+      else if (GENERAL && masked) { combine(std::true_type{}, std::true_type{}); }
+      else if (beta != 0.0f) { combine(std::true_type{}, std::false_type{}); }
+      else { combine(std::false_type{}, std::false_type{}); }
     }
   }
+}
+
+// Second kernel of a launch with split tiles (GemmArgs::tail_parts > 0): the 32 work-groups t * 32 .. t * 32 + 31 add the
+// sums of the K ranges of tile tail_first + t in the order of the ranges, eight columns each, apply alpha and beta and
+// store - what lies inside the matrix, and on the diagonal of a triangle of C the triangle's elements. A thread owns
+// eight rows of a column (the rows of C are a multiple of 8: such a piece lies inside the matrix or outside).
+constexpr int kWideFixupGroupsPerTile = 32;
+__global__ __launch_bounds__(256) void HgemmWideFixupKernel(const GemmArgs<float> p, const int tiles_m, const int tiles_n,
+                                                            const int all_groups) {
+  using T = _Float16;
+  constexpr int TILE = 256;
+  const int tile = static_cast<int>(blockIdx.x) / kWideFixupGroupsPerTile;
+  const WideItem first = WideItemOf<true>(p, tiles_m, tiles_n, p.tail_first + tile * p.tail_parts, all_groups);
+  const T* a;
+  const T* b;
+  T* c;
+  float alpha, beta;
+  ResolveBatch<T, float>(p, first.batch, a, b, c, alpha, beta);
+  const int m0 = first.tile_m * TILE, n0 = first.tile_n * TILE;
+  const bool masked = p.c_triangle != 0 && first.tile_m == first.tile_n;
+  const float* sums = p.tail_partials + static_cast<long long>(tile) * p.tail_parts * (TILE * TILE);
+  const auto c_view = __builtin_amdgcn_make_buffer_rsrc(c + n0 * p.c_ld + m0, 0, kHOutside, kRawBufferFlags);
+  typedef float float4_t __attribute__((ext_vector_type(4)));
+  const int row = 8 * (threadIdx.x % 32);
+  const int column = 8 * (static_cast<int>(blockIdx.x) % kWideFixupGroupsPerTile) + threadIdx.x / 32;
+  if (m0 + row >= p.m || n0 + column >= p.n) { return; }
+  float total[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) { total[e] = 0.0f; }
+  for (int part = 0; part < p.tail_parts; ++part) {
+    const float4_t* piece = reinterpret_cast<const float4_t*>(sums + static_cast<long long>(part) * (TILE * TILE) + column * TILE + row);
+    const float4_t low = piece[0], high = piece[1];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { total[e] += low[e]; total[4 + e] += high[e]; }
+  }
+  const int offset = (column * static_cast<int>(p.c_ld) + row) * 2;
+  half8_t old = half8_t(T(0));
+  if (beta != 0.0f || masked) { old = BufferLoad<T, 8>(c_view, offset); }
+  half8_t out;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float fresh = (beta != 0.0f) ? Combine(alpha, total[e], beta, static_cast<float>(old[e])) : alpha * total[e];
+    const bool kept = !masked || InTriangle(p.c_triangle, m0 + row + e, n0 + column);
+    out[e] = kept ? Narrow<T, float>(fresh) : old[e];
+  }
+  BufferStore<T, 8>(out, c_view, offset);
 }
 
 }  // namespace clbh

@@ -141,6 +141,27 @@ double LaunchCost(const TileCandidate& candidate, const size_t m, const size_t n
   }
   return rounds * static_cast<double>(candidate.tile.tile_m * candidate.tile.tile_n) / candidate.rate;
 }
+
+// The same estimate, k included, for `count` 256 x 256 tiles of the persistent fp16 kernel (one work-group per CU,
+// 1608 TFLOP/s, a tile costs what 467 more of k would). A last round that fills at most half of the work-groups is
+// split along K the way the device layer does it (PlanWide in device/launch_common.hpp): it then costs the walk of one
+// K range plus what 2000 of k would - the sums' way through memory and the second kernel (HSYRK 8192, 528 tiles: two
+// rounds of 186 us, then 54 us for 16 tiles in 16 ranges of 512).
+double WideTileCost(const size_t count, const size_t k) {
+  const auto grid = Units() - Units() % 8;
+  const auto groups = CeilDivide(k, 128);
+  const auto whole = static_cast<double>(count / grid) * (static_cast<double>(k) + 467.0);
+  const auto tail = count % grid;
+  auto last = (tail > 0) ? static_cast<double>(k) + 467.0 : 0.0;
+  if (tail > 0 && count > grid && 2 * tail <= grid && groups >= 4) {
+    const auto most = std::min<size_t>({grid / tail, 16, groups / 2});
+    if (most >= 2) {
+      const auto groups_per_part = CeilDivide(groups, most);
+      if (CeilDivide(groups, groups_per_part) >= 2) { last = static_cast<double>(groups_per_part * 128) + 2000.0; }
+    }
+  }
+  return (whole + last) * 256.0 * 256.0 / 1608.0;
+}
 }  // namespace
 
 KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const bool b_kcontig, const size_t m,
@@ -265,10 +286,18 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
         const Option options[] = {{2, 256, 1, 1484.0, 627.0}, {0, 128, 2, 936.0, 293.0}, {1, 64, 4, 488.0, 44.0}};
         auto lowest = 1e300;
         int chosen = 1;
+        // (the 256 x 256 tiles of a triangle run in the persistent kernel where it applies, as below for the full product)
+        const bool wide = m == n && m % 8 == 0 &&
+                          ((m % 256 == 0 && k % 128 == 0) || (!a_kcontig && !b_kcontig && k >= 1000));
         for (const auto& option : options) {
           if (option.index == 2 && k < 256) { continue; }
           const auto along = CeilDivide(n, option.extent);
           const auto count = along * (along + 1) / 2 * batch_count;
+          if (option.index == 2 && wide) {
+            const auto time = WideTileCost(count, k);
+            if (time < lowest) { lowest = time; chosen = option.index; }
+            continue;
+          }
           const auto slots = Units() * option.per_cu;
           auto rounds = static_cast<double>((count / slots) * option.per_cu);
           if (count % slots != 0) {
@@ -393,7 +422,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     // (whole tiles with k = 128 take it too: 8 x 4096^2 x 128 with beta = 0 67 us against 81 us on three 128 x 128
     // work-groups per CU, 96 x 2048^2 x 128 267 against 296 us; with beta = 1 the two are level)
     const bool whole_wide = wide && m % 256 == 0 && n % 256 == 0 && k % 128 == 0;
-    const auto cost256 = (k >= 256 || whole_wide) ? cost(256, 1, wide ? 1608.0 : 1484.0, wide ? 467.0 : 627.0) : 1e300, cost128 = batch_128 * cost(128, 2, 936.0, 293.0),
+    const auto cost256 = (k >= 256 || whole_wide) ? (wide ? WideTileCost(CeilDivide(m, 256) * CeilDivide(n, 256) * batch_count, k) : cost(256, 1, 1484.0, 627.0)) : 1e300, cost128 = batch_128 * cost(128, 2, 936.0, 293.0),
                cost64 = batch_64 * cost(64, 4, long_k ? 371.0 : 488.0, 44.0);
     int tile = 1;
     if (cost256 <= cost128 && cost256 <= cost64) { tile = 2; }

@@ -175,20 +175,22 @@ void Xgemm<T>::DoGemm(const Layout layout, const Transpose a_transpose, const Tr
     align(desc.b, desc.b_offset, desc.b_ld, desc.b_kcontig != 0, desc.n, aligned_b, "aligned copy of an operand");
   }
 
-  // Temporary memory: only split-K launches want any. A caller-provided buffer must be large enough
-  // (reference: xgemm.cpp:146-151), otherwise stream-ordered scratch is taken for the call.
+  // Temporary memory: only launches that split K want any. A caller-provided buffer must be large enough
+  // (reference: xgemm.cpp:146-151) unless the launch can do with less, otherwise stream-ordered scratch is taken for
+  // the call.
   const auto temp_bytes = clbh_gemm_workspace_bytes(&desc);
   std::unique_ptr<StreamScratch> scratch;
+  desc.workspace_bytes = temp_bytes;
   if (temp_buffer_provided) {
     if (temp_bytes > 0 && temp_buffer.GetSize() < temp_bytes) {
-      throw BLASError(StatusCode::kInsufficientMemoryTemp);
+      if (clbh_gemm_workspace_optional(&desc) == 0) { throw BLASError(StatusCode::kInsufficientMemoryTemp); }
+      desc.workspace_bytes = temp_buffer.GetSize();
     }
     desc.workspace = const_cast<void*>(temp_buffer());
   } else if (temp_bytes > 0) {
     scratch.reset(new StreamScratch(temp_bytes, stream(), "temporary buffer"));
     desc.workspace = scratch->get();
   }
-  desc.workspace_bytes = temp_bytes;
 
   CheckDevice(clbh_gemm_launch(&desc, stream()), "clbh_gemm_launch");
   if (record_event) { Finish(); }

@@ -79,7 +79,7 @@ typedef struct clbh_gemm_desc_ {
   long long a_stride, b_stride, c_stride;  // elements; used when batch.alphas == NULL
   double alpha, beta;                      // used when batch.alphas == NULL
   clbh_batch_arrays batch;
-  void* workspace;          // optional device scratch (split-K partial sums), may be NULL
+  void* workspace;          // device scratch (partial sums of K ranges), may be NULL where clbh_gemm_workspace_bytes is 0
   size_t workspace_bytes;
   // Triangular variants of the canonical problem (both 0 for a plain GEMM; neither combines with split_k > 1):
   int c_triangle;        // 1: only C(i,j) with i <= j is computed and written, 2: only i >= j; the rest of C is untouched.
@@ -102,6 +102,9 @@ CLBH_API int clbh_gemm_launch(const clbh_gemm_desc* desc, hipStream_t stream);
 
 // Bytes of device scratch the given descriptor needs in `workspace` (0 for most launches).
 CLBH_API size_t clbh_gemm_workspace_bytes(const clbh_gemm_desc* desc);
+// 1 when the launch only uses that scratch to go faster (the persistent fp16 kernel splits the tiles of a sparsely
+// filled last round along K) and runs without it, or with less, as well; 0 when it cannot do without.
+CLBH_API int clbh_gemm_workspace_optional(const clbh_gemm_desc* desc);
 
 // Expands the symmetric k x k matrix at src + src_offset (elements; one triangle stored, addressed as
 // [two * src_ld + one], `upper`: the stored elements have one <= two) into the dense k x k matrix `dst`

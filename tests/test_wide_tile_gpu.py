@@ -106,10 +106,11 @@ def test_strided_batches_of_whole_tiles(forced):
     assert np.array_equal(results[0].view(np.uint16), results[1].view(np.uint16))
 
 
-@pytest.mark.parametrize("m,n,k,batch", [(512, 512, 256, 70), (520, 264, 1000, 67)])
+@pytest.mark.parametrize("m,n,k,batch", [(512, 512, 256, 100), (520, 264, 1000, 67)])
 def test_more_items_than_work_groups(forced, m, n, k, batch):
     """More tiles than compute units: the persistent work-groups walk several (tile, matrix) items each, the slabs of
-    one item following those of the last through the ring; whole tiles without and ragged ones with range checks."""
+    one item following those of the last through the ring; whole tiles without and ragged ones with range checks.
+    (400 and 402 tiles: the last round fills more than half of the 256 work-groups and is not split.)"""
     import torch
     import oracle
     rng = np.random.default_rng(9500 + m)
@@ -131,3 +132,77 @@ def test_more_items_than_work_groups(forced, m, n, k, batch):
         where = oracle.c_indices(COL_MAJOR, m, n, i * m * n, m)
         assert oracle.rel_frobenius(results[0][where], expected) <= 1e-2, i
     assert np.array_equal(results[0].view(np.uint16), results[1].view(np.uint16))
+
+
+def _forced_gemm(variant, m, n, k, batch, alpha, beta, a, b, c):
+    import torch
+    clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": variant})
+    a_dev, b_dev, c_dev = (torch.from_numpy(x).to("cuda:0") for x in (a, b, c))
+    status = clblast_amd.raw_gemm_strided_batched("H", COL_MAJOR, NO, YES, m, n, k, alpha, a_dev.data_ptr(), 0, m, m * k,
+                                                  b_dev.data_ptr(), 0, n, n * k, beta, c_dev.data_ptr(), 0, m, m * n, batch,
+                                                  gpu_harness.stream_handle())
+    torch.cuda.synchronize()
+    assert status == 0
+    return c_dev.cpu().numpy()
+
+
+@pytest.mark.parametrize("m,n,k,batch,beta", [(4352, 4352, 1024, 1, 0.0), (4360, 4300, 1000, 1, -0.75), (512, 512, 512, 70, 1.5),
+                                              (768, 512, 640, 44, 0.0)])
+def test_a_sparsely_filled_last_round_is_split_along_k(forced, m, n, k, batch, beta):
+    """289, 306, 280 and 264 tiles on 256 work-groups: the tiles of the last round become several items each, one per K
+    range, and a second kernel adds their sums. Against the eight-wavefront kernel (another order of additions, so
+    not bit for bit) and, element by element, against dot products in double precision."""
+    rng = np.random.default_rng(9600 + m + batch)
+    a = rng.uniform(-0.5, 0.5, batch * k * m).astype(np.float16)
+    b = rng.uniform(-0.5, 0.5, batch * k * n).astype(np.float16)
+    c = rng.uniform(-1.0, 1.0, batch * n * m).astype(np.float16)
+    wide = _forced_gemm(WIDE_OR_NOT, m, n, k, batch, 0.5, beta, a, b, c)
+    eight = _forced_gemm(EIGHT_WAVES, m, n, k, batch, 0.5, beta, a, b, c)
+    difference = wide.astype(np.float64) - eight.astype(np.float64)
+    assert np.linalg.norm(difference) <= 2e-3 * np.linalg.norm(eight.astype(np.float64))
+    assert np.max(np.abs(difference)) <= 0.05
+    for _ in range(400):  # (elements of the last tiles, which are the split ones, and of the others)
+        i, j, matrix = (int(rng.integers(m)), int(rng.integers(n)), int(rng.integers(batch)))
+        row = a[matrix * m * k + i + m * np.arange(k)].astype(np.float64)
+        column = b[matrix * n * k + j + n * np.arange(k)].astype(np.float64)
+        expected = 0.5 * float(row @ column) + beta * float(c[matrix * m * n + j * m + i])
+        assert abs(float(wide[matrix * m * n + j * m + i]) - expected) <= 2e-2 * max(1.0, abs(expected)), (i, j, matrix)
+
+
+def test_a_triangle_of_c_on_the_wide_tile(gpu, forced):
+    """SYRK with the 256 x 256 tile forced: the wide kernel walks the tiles of the triangle and stores the tiles on the
+    diagonal under a mask (the other triangle holds NaN and keeps its bits); whole tiles in every mode, ragged ones
+    where both operands are x-contiguous, the eight-wavefront kernel elsewhere."""
+    from tests.test_syrk_gpu import MODES, RankUpdateProblem
+    clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": WIDE_OR_NOT})
+    seed = 9700
+    for (layout, triangle, transpose), (n, k, beta) in itertools.product(MODES, ((512, 256, 0.0), (768, 128, 1.25), (520, 1000, -0.5))):
+        seed += 1
+        problem = RankUpdateProblem("syrk", 16, layout, triangle, transpose, n, k, 0.75, beta, seed, extra=(0, 0, 8),
+                                    offsets=(0, 0, 16), ab_range=(-0.5, 0.5))
+        status, c_after = problem.run(gpu)
+        assert status == 0, problem.describe()
+        problem.check(c_after)
+
+
+@pytest.mark.parametrize("triangle_name,k,beta", [("upper", 512, 0.0), ("lower", 640, 0.5)])
+def test_a_triangle_with_a_split_last_round(gpu, forced, triangle_name, k, beta):
+    """276 tiles in the triangle of 23 x 23: the last 20, tiles on the diagonal among them, are split along K. Against the
+    eight-wavefront kernel; the other triangle keeps its NaN."""
+    from oracle import LOWER, UPPER
+    from tests.test_syrk_gpu import RankUpdateProblem
+    n = 5888
+    triangle = UPPER if triangle_name == "upper" else LOWER
+    problem = RankUpdateProblem("syrk", 16, COL_MAJOR, triangle, NO, n, k, 0.5, beta, 9800 + k, ab_range=(-0.5, 0.5))
+    results = []
+    for variant in (WIDE_OR_NOT, EIGHT_WAVES):
+        clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": variant})
+        status, c_after = problem.run(gpu)
+        assert status == 0
+        results.append(c_after)
+    wide, eight = (r[problem.where].astype(np.float64) for r in results)
+    assert np.all(np.isfinite(wide[problem.inside]))
+    assert np.linalg.norm(wide[problem.inside] - eight[problem.inside]) <= 2e-3 * np.linalg.norm(eight[problem.inside])
+    untouched = np.ones(results[0].size, dtype=bool)
+    untouched[problem.where[problem.inside]] = False
+    assert np.array_equal(results[0][untouched].view(np.uint8), problem.c[untouched].view(np.uint8))
