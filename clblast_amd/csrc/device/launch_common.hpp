@@ -193,9 +193,10 @@ inline int WideForm(const clbh_gemm_desc& d) {
 
 // Geometry of a launch of the persistent fp16 kernel (kernels/gemm_wide_f16.hpp): its tiles - of the triangle, for a
 // triangle of C -, the work-groups (one per compute unit, a multiple of 8), and what becomes of a last round that
-// fills at most half of them: its tiles are split into `parts` K ranges of groups_per_part * 128 each (at most 16, at
-// least 256 deep, as many as keep that round within the work-groups), one item per range, whose sums meet in the
-// workspace (256 KiB per item). form 0: the launch is not for this kernel.
+// fills at most half of them (or of the only round there is): its tiles are split into `parts` K ranges of
+// groups_per_part * 128 each (at most 8, at least 256 deep, as many as keep that round within the work-groups), one
+// item per range, whose sums meet in the workspace (256 KiB per item) - where the shorter walk outweighs that detour.
+// form 0: the launch is not for this kernel.
 struct WidePlan {
   int form;
   long long tiles_m, tiles_n, tiles, grid, items, tail_first;
@@ -212,21 +213,27 @@ inline WidePlan PlanWide(const clbh_gemm_desc& d) {
   plan.tiles = per_matrix * d.batch_count;
   int units = 0;
   if (clbh_compute_units(&units) != 0 || units < 8) { units = 256; }
-  plan.grid = std::min<long long>(plan.tiles, units - units % 8);
+  const long long most_groups = units - units % 8;
+  plan.grid = std::min<long long>(plan.tiles, most_groups);
   plan.all_groups = (d.k + 127) / 128;
   plan.items = plan.tiles;
   plan.tail_first = plan.tiles;
-  const long long tail = plan.tiles % plan.grid;
-  if (tail > 0 && 2 * tail <= plan.grid && plan.all_groups >= 4) {
-    const int most = static_cast<int>(std::min<long long>({plan.grid / tail, 16, plan.all_groups / 2}));
+  const long long tail = plan.tiles % most_groups;  // (all tiles, when they are fewer than the work-groups)
+  if (d.split_k >= 0 && tail > 0 && 2 * tail <= most_groups && plan.all_groups >= 4) {  // (split_k < 0: told to split nothing)
+    const int most = static_cast<int>(std::min<long long>({most_groups / tail, 8, plan.all_groups / 2}));
     if (most >= 2) {
       const int groups_per_part = (plan.all_groups + most - 1) / most;
       const int parts = (plan.all_groups + groups_per_part - 1) / groups_per_part;
-      if (parts >= 2) {
+      // (the sums' way through memory and the second kernel cost what about 2000 more of k would, a tile's own
+      // prologue and epilogue what 467 would: 2048^2 x 2048, 64 tiles, 30 us whole and 48 us in four ranges; 2048^2 x 8192
+      // 88 and 80 us)
+      const bool pays = 10 * (groups_per_part * 128 + 2000) < 9 * (d.k + 467);
+      if (parts >= 2 && pays) {
         plan.parts = parts;
         plan.groups_per_part = groups_per_part;
         plan.tail_first = plan.tiles - tail;
         plan.items = plan.tail_first + tail * parts;
+        plan.grid = std::min<long long>(plan.items, most_groups);
         plan.workspace_bytes = static_cast<size_t>(tail) * parts * 256 * 256 * sizeof(float);
       }
     }

@@ -24,6 +24,13 @@ size_t ForcedSplit(const Precision precision) {
   const auto found = split_overrides.find(static_cast<int>(precision));
   return (found != split_overrides.end() && found->second > 0) ? found->second : 1;
 }
+// True when the override names one K range ("SPLIT_K": 1) rather than none: the launch then splits nothing at all, not
+// even a sparsely filled last round of the persistent fp16 kernel (which is otherwise the device layer's own decision).
+bool ForcedSingleRange(const Precision precision) {
+  std::lock_guard<std::mutex> lock(override_mutex);
+  const auto found = split_overrides.find(static_cast<int>(precision));
+  return found != split_overrides.end() && found->second == 1;
+}
 
 }  // namespace
 
@@ -146,18 +153,24 @@ double LaunchCost(const TileCandidate& candidate, const size_t m, const size_t n
 // 1608 TFLOP/s, a tile costs what 467 more of k would). A last round that fills at most half of the work-groups is
 // split along K the way the device layer does it (PlanWide in device/launch_common.hpp): it then costs the walk of one
 // K range plus what 2000 of k would - the sums' way through memory and the second kernel (HSYRK 8192, 528 tiles: two
-// rounds of 186 us, then 54 us for 16 tiles in 16 ranges of 512).
+// rounds of 186 us, then 54 us for 16 tiles in 16 ranges of 512; in eight ranges the same) - where that is less than the whole walk.
 double WideTileCost(const size_t count, const size_t k) {
   const auto grid = Units() - Units() % 8;
   const auto groups = CeilDivide(k, 128);
   const auto whole = static_cast<double>(count / grid) * (static_cast<double>(k) + 467.0);
   const auto tail = count % grid;
   auto last = (tail > 0) ? static_cast<double>(k) + 467.0 : 0.0;
-  if (tail > 0 && count > grid && 2 * tail <= grid && groups >= 4) {
-    const auto most = std::min<size_t>({grid / tail, 16, groups / 2});
+  if (tail > 0 && 2 * tail <= grid && groups >= 4) {
+    const auto most = std::min<size_t>({grid / tail, 8, groups / 2});
     if (most >= 2) {
       const auto groups_per_part = CeilDivide(groups, most);
-      if (CeilDivide(groups, groups_per_part) >= 2) { last = static_cast<double>(groups_per_part * 128) + 2000.0; }
+      const auto parts = CeilDivide(groups, groups_per_part);
+      const auto split = static_cast<double>(groups_per_part * 128) + 2000.0;
+      // (a single round of very few tiles stays with the small tiles and their K ranges: 512^2 x 8192, 4 tiles, 36 us in
+      // ranges here against 20 us there; from half a round of items on the two are level or this one wins - 2048^2 x
+      // 8192 80 against 89 us, 8 x 1024^2 x 4096 84 against 101 us, 1024^2 x 16384 56 against 53 us)
+      const bool enough = count > grid || 2 * tail * parts >= grid;
+      if (parts >= 2 && 10.0 * split < 9.0 * last && enough) { last = split; }
     }
   }
   return (whole + last) * 256.0 * 256.0 / 1608.0;
@@ -265,7 +278,7 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   if (forced != 0 && forced < 100) {
     // a forced tile takes the forced number of K ranges (unbatched calls only), never more than k / 16
     const auto ranges = (batch_count == 1) ? std::max<size_t>(1, std::min<size_t>(ForcedSplit(precision), k / 16)) : 1;
-    return KernelChoice{CLBH_KERNEL_MFMA, static_cast<int>(forced) - 1, static_cast<int>(ranges)};
+    return KernelChoice{CLBH_KERNEL_MFMA, static_cast<int>(forced) - 1, ForcedSingleRange(precision) ? -1 : static_cast<int>(ranges)};
   }
   if (triangular) {
     // About half of the tile work is skipped and what remains is uneven, so the dispatcher needs spare tiles to even
@@ -448,7 +461,8 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
     {
       const auto tiles128 = CeilDivide(m, 128) * CeilDivide(n, 128) * batch_count;
       const bool fills = 10 * TileUse(m, n, 128, 128) >= 9 * TileUse(m, n, 64, 64);
-      if (k <= 320 && tiles128 >= 2048 && fills && !(wide && tile == 2)) { tile = 5; }  // (8192^2 x 256 T/N: 69 us that way, 61 us on the wide tile)
+      if (wide && tile == 2) {}  // (8192^2 x 256 T/N: 69 us on three 128 x 128 work-groups per CU, 61 us on the wide tile)
+      else if (k <= 320 && tiles128 >= 2048 && fills) { tile = 5; }
       else if (k <= 128 && tiles128 >= 512 && fills) { tile = 0; }
     }
     // One column of tiles (64 <= n <= 128) under a long k and a tall A with contiguous columns: every tile streams its
@@ -496,6 +510,8 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
           const auto slow = option.tile == 1 && range >= 4096 && CeilDivide(m, 128) * CeilDivide(n, 128) * launched >= 256;
           auto time = LaunchCost(TileCandidate{Tile{0, option.extent, option.extent}, option.per_cu, slow ? 371.0 : option.rate}, m, n, 0.25, launched) *
                       (static_cast<double>(range) + option.k0) * 512e-6;
+          // (the persistent kernel's own estimate where it runs: it splits its one sparsely filled round by itself)
+          if (option.tile == 2 && wide && launched == 1) { time = WideTileCost(CeilDivide(m, 256) * CeilDivide(n, 256), k) * 512e-6; }
           if (launched > 1) { time += 4.0 + 0.4 * 4e-6 * static_cast<double>(m * n * launched); }
           if (time < lowest) { lowest = time; tile = option.tile; split = launched; }
         }
@@ -717,7 +733,7 @@ StatusCode OverrideRoutineParameters(const int device, const std::string& kernel
     const auto split = parameters.find("SPLIT_K");
     std::lock_guard<std::mutex> lock(override_mutex);
     tile_variant_overrides[static_cast<int>(precision)] = variant->second;
-    split_overrides[static_cast<int>(precision)] = (split != parameters.end()) ? split->second : 1;
+    split_overrides[static_cast<int>(precision)] = (split != parameters.end()) ? split->second : 0;
     return StatusCode::kSuccess;
   }
   if (kernel_name != "GemmRoutine") {

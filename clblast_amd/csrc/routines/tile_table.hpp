@@ -19,7 +19,8 @@ namespace clblast {
 struct KernelChoice {
   int kernel_class;  // enum clbh_kernel_class
   int tile_variant;  // index into the variant list of that class
-  int split_k;       // number of K ranges to spread over extra work-groups (1 = none)
+  int split_k;       // number of K ranges to spread over extra work-groups (1 = none; -1 = none, and the device layer
+                     // is not to split a last round of tiles either: a forced tile with "SPLIT_K": 1)
 };
 
 // Default direct/indirect thresholds per precision (see tile_table.cpp for the reasoning).

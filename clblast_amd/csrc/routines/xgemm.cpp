@@ -148,7 +148,7 @@ void Xgemm<T>::DoGemm(const Layout layout, const Transpose a_transpose, const Tr
     static constexpr int kFoldedOperand[5] = {0, 3, 4, 1, 2};
     desc.c_triangle = folded ? kFoldedOutput[static_cast<int>(triangles.output)] : static_cast<int>(triangles.output);
     desc.operand_triangle = folded ? kFoldedOperand[static_cast<int>(triangles.operand)] : static_cast<int>(triangles.operand);
-    desc.split_k = 1;  // the K ranges of a split launch and of a triangle do not combine
+    desc.split_k = std::min(desc.split_k, 1);  // the K ranges of a split launch and of a triangle do not combine
   }
 
   // fp16 operands of the tiled kernels are fetched in dwords: an operand that starts at an odd element or has an odd

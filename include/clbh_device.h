@@ -66,7 +66,8 @@ typedef struct clbh_gemm_desc_ {
   int precision;      // 16, 32 or 64 (bits of the storage type)
   int kernel_class;   // enum clbh_kernel_class
   int tile_variant;   // index into the tile table of that class (0 = default)
-  int split_k;        // > 1: split the K range over that many work-group rows (MFMA class, fp32/fp64, unbatched)
+  int split_k;        // > 1: split the K range over that many work-group rows (MFMA class, unbatched); < 0: split nothing,
+                      // not even the last round of tiles of the persistent fp16 kernel (else the device layer's decision)
   int a_kcontig;      // see header comment
   int b_kcontig;
   int m, n, k;

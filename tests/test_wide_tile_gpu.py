@@ -18,7 +18,8 @@ WIDE_OR_NOT, EIGHT_WAVES = 3, 13  # override value = tile index + 1
 
 
 def run_with(variant, problem):
-    clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": variant})
+    # ("SPLIT_K": 1 - one K range, no split of a sparsely filled round of tiles either: the comparisons are bit for bit)
+    clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": variant, "SPLIT_K": 1})
     status, c_after = problem.run()
     assert status == 0, (variant, problem.describe())
     return c_after
@@ -92,7 +93,7 @@ def test_strided_batches_of_whole_tiles(forced):
                 for i in range(batch)]
     results = []
     for variant in (WIDE_OR_NOT, EIGHT_WAVES):
-        clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": variant})
+        clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": variant, "SPLIT_K": 1})
         a_dev, b_dev, c_dev = (torch.from_numpy(x).to("cuda:0") for x in (a, b, c))
         status = clblast_amd.raw_gemm_strided_batched("H", COL_MAJOR, NO, YES, m, n, k, 0.5, a_dev.data_ptr(), 0, m, m * k,
                                                       b_dev.data_ptr(), 0, n, n * k, 1.25, c_dev.data_ptr(), 0, m, m * n, batch,
@@ -119,7 +120,7 @@ def test_more_items_than_work_groups(forced, m, n, k, batch):
     c = rng.uniform(-1.0, 1.0, batch * n * m).astype(np.float16)
     results = []
     for variant in (WIDE_OR_NOT, EIGHT_WAVES):
-        clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": variant})
+        clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": variant, "SPLIT_K": 1})
         a_dev, b_dev, c_dev = (torch.from_numpy(x).to("cuda:0") for x in (a, b, c))
         status = clblast_amd.raw_gemm_strided_batched("H", COL_MAJOR, NO, YES, m, n, k, -0.5, a_dev.data_ptr(), 0, m, m * k,
                                                       b_dev.data_ptr(), 0, n, n * k, 0.75, c_dev.data_ptr(), 0, m, m * n, batch,
@@ -146,11 +147,11 @@ def _forced_gemm(variant, m, n, k, batch, alpha, beta, a, b, c):
     return c_dev.cpu().numpy()
 
 
-@pytest.mark.parametrize("m,n,k,batch,beta", [(4352, 4352, 1024, 1, 0.0), (4360, 4300, 1000, 1, -0.75), (512, 512, 512, 70, 1.5),
-                                              (768, 512, 640, 44, 0.0)])
+@pytest.mark.parametrize("m,n,k,batch,beta", [(4352, 4352, 4096, 1, 0.0), (4360, 4300, 3000, 1, -0.75), (512, 512, 4096, 70, 1.5),
+                                              (768, 512, 3200, 44, 0.0), (1024, 768, 8192, 1, 1.0)])
 def test_a_sparsely_filled_last_round_is_split_along_k(forced, m, n, k, batch, beta):
-    """289, 306, 280 and 264 tiles on 256 work-groups: the tiles of the last round become several items each, one per K
-    range, and a second kernel adds their sums. Against the eight-wavefront kernel (another order of additions, so
+    """289, 306, 280 and 264 tiles on 256 work-groups, and 12 tiles alone: the tiles of the last round become several items
+    each, one per K range, and a second kernel adds their sums (K is long enough for that to pay). Against the eight-wavefront kernel (another order of additions, so
     not bit for bit) and, element by element, against dot products in double precision."""
     rng = np.random.default_rng(9600 + m + batch)
     a = rng.uniform(-0.5, 0.5, batch * k * m).astype(np.float16)
@@ -185,7 +186,7 @@ def test_a_triangle_of_c_on_the_wide_tile(gpu, forced):
         problem.check(c_after)
 
 
-@pytest.mark.parametrize("triangle_name,k,beta", [("upper", 512, 0.0), ("lower", 640, 0.5)])
+@pytest.mark.parametrize("triangle_name,k,beta", [("upper", 3072, 0.0), ("lower", 3200, 0.5)])
 def test_a_triangle_with_a_split_last_round(gpu, forced, triangle_name, k, beta):
     """276 tiles in the triangle of 23 x 23: the last 20, tiles on the diagonal among them, are split along K. Against the
     eight-wavefront kernel; the other triangle keeps its NaN."""
