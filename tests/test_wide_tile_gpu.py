@@ -186,15 +186,16 @@ def test_a_triangle_of_c_on_the_wide_tile(gpu, forced):
         problem.check(c_after)
 
 
-@pytest.mark.parametrize("triangle_name,k,beta", [("upper", 3072, 0.0), ("lower", 3200, 0.5)])
-def test_a_triangle_with_a_split_last_round(gpu, forced, triangle_name, k, beta):
-    """276 tiles in the triangle of 23 x 23: the last 20, tiles on the diagonal among them, are split along K. Against the
-    eight-wavefront kernel; the other triangle keeps its NaN."""
+@pytest.mark.parametrize("routine,triangle_name,n,k,beta", [("syrk", "upper", 5888, 3072, 0.0), ("syrk", "lower", 5888, 3200, 0.5),
+                                                            ("syrk", "lower", 5896, 3000, -1.0), ("syr2k", "upper", 5888, 2048, 0.25)])
+def test_a_triangle_with_a_split_last_round(gpu, forced, routine, triangle_name, n, k, beta):
+    """276 tiles in the triangle of 23 x 23 (300 in that of 24 x 24, with ragged tiles on two edges): the last 20 (44),
+    tiles on the diagonal among them, are split along K. SYRK and both launches of SYR2K against the eight-wavefront
+    kernel; the other triangle keeps its NaN."""
     from oracle import LOWER, UPPER
     from tests.test_syrk_gpu import RankUpdateProblem
-    n = 5888
     triangle = UPPER if triangle_name == "upper" else LOWER
-    problem = RankUpdateProblem("syrk", 16, COL_MAJOR, triangle, NO, n, k, 0.5, beta, 9800 + k, ab_range=(-0.5, 0.5))
+    problem = RankUpdateProblem(routine, 16, COL_MAJOR, triangle, NO, n, k, 0.5, beta, 9800 + k, ab_range=(-0.5, 0.5))
     results = []
     for variant in (WIDE_OR_NOT, EIGHT_WAVES):
         clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": variant})
@@ -207,3 +208,31 @@ def test_a_triangle_with_a_split_last_round(gpu, forced, triangle_name, k, beta)
     untouched = np.ones(results[0].size, dtype=bool)
     untouched[problem.where[problem.inside]] = False
     assert np.array_equal(results[0][untouched].view(np.uint8), problem.c[untouched].view(np.uint8))
+
+
+def test_a_temporary_buffer_too_small_for_the_split(forced):
+    """GemmTempBufferSize names the space for the partial sums of a split round; a caller's buffer that is smaller is
+    accepted and the product runs unsplit (bit for bit what the launch gives when told to split nothing)."""
+    import torch
+    from tests.level3_harness import DeviceBuffer
+    m, n, k = 4352, 4352, 4096
+    clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": WIDE_OR_NOT})
+    status, wanted = clblast_amd.raw_gemm_temp_buffer_size("H", COL_MAJOR, NO, YES, m, n, k, 0, m, 0, n, 0, m,
+                                                           gpu_harness.stream_handle())
+    assert status == 0 and wanted >= 33 * 2 * 256 * 256 * 4, wanted
+    rng = np.random.default_rng(9900)
+    a, b = (rng.uniform(-0.5, 0.5, k * extent).astype(np.float16) for extent in (m, n))
+    c = rng.uniform(-1.0, 1.0, m * n).astype(np.float16)
+    results = []
+    for small_buffer in (True, False):
+        a_dev, b_dev, c_dev = (torch.from_numpy(x).to("cuda:0") for x in (a, b, c))
+        temp = DeviceBuffer(1024 if small_buffer else wanted)  # (an allocation of exactly that size)
+        if not small_buffer:
+            clblast_amd.override_parameters(0, "Xgemm", 16, {"TILE_VARIANT": WIDE_OR_NOT, "SPLIT_K": 1})
+        status = clblast_amd.raw_gemm("H", COL_MAJOR, NO, YES, m, n, k, 1.0, a_dev.data_ptr(), 0, m, b_dev.data_ptr(), 0, n, 0.5,
+                                      c_dev.data_ptr(), 0, m, gpu_harness.stream_handle(), None, temp.pointer.value)
+        torch.cuda.synchronize()
+        temp.free()
+        assert status == 0, small_buffer
+        results.append(c_dev.cpu().numpy())
+    assert np.array_equal(results[0].view(np.uint16), results[1].view(np.uint16))
