@@ -387,12 +387,12 @@ __device__ __forceinline__ int XcdContiguousIndex(const int block, const int num
   return (xcd < tall) ? xcd * per_xcd + local : tall * per_xcd + (xcd - tall) * (per_xcd - 1) + local;
 }
 
+template <int GROUP_M = 8>
 __device__ __forceinline__ void TileOfBlock(const int block, const int num_blocks, const int tiles_m,
                                             const int tiles_n, int& tile_m, int& tile_n) {
   // (1) a contiguous logical range per XCD
   const int logical = XcdContiguousIndex(block, num_blocks);
   // (2) grouped walk: GROUP_M tile rows at a time, column by column inside a group
-  constexpr int GROUP_M = 8;
   const int in_group = GROUP_M * tiles_n;
   const int group = logical / in_group;
   const int first_m = group * GROUP_M;
@@ -490,7 +490,9 @@ __global__ __launch_bounds__(kMfmaThreads, ALIGNED ? Config::MIN_WAVES : 2) void
     if (fold_rows && tiles_m - 1 - tile_m != tile_m) { partner_m = tiles_m - 1 - tile_m; partner_n = tile_n; }
     if (fold_columns && tiles_n - 1 - tile_n != tile_n) { partner_m = tile_m; partner_n = tiles_n - 1 - tile_n; }
   } else {
-    TileOfBlock(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
+    // (the 32 tiles that an XCD's CUs hold at a time form GROUP_M rows of 32 / GROUP_M columns: as square a piece of C
+    // as the tile's shape allows, so that the fewest operand panels pass through that XCD's L2)
+    TileOfBlock<(TILE_M >= 2 * TILE_N) ? 4 : 8>(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
   }
   for (int pass = 0; pass < 2; ++pass) {
     if (pass == 1) {

@@ -40,4 +40,5 @@ def test_the_bench_line_keeps_every_baseline_configuration_in_config():
     entry = bench.compact({"ms": 0.75, "gflops": 1466000.0, "gbs": 716.0, "roofline": {"bound": "mfma", "frac": 0.58}})
     assert entry == {"ms": 0.75, "tflops": 1466.0, "gbs": 716.0, "bound": "mfma", "frac": 0.58}
     source = open(os.path.join(ROOT, "bench.py")).read()
-    assert 'result["config"]["baseline"] = baseline' in source and '"cfg2_sgemm_8192_rowTN": compact(headline_entry)' in source
+    assert 'result["config"]["baseline"] = baseline' in source and 'HEADLINE_NAME: compact(headline_entry)' in source
+    assert bench.HEADLINE_NAME == "cfg2_sgemm_8192_rowTN"
