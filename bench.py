@@ -38,7 +38,7 @@ MEASURED_TRAFFIC = {
     "cfg2d": (1.1247e10, "profiles/dgemm_8192_rowTN.md", "clbh::GemmMfmaKernel<double, clbh::MfmaConfig<double, 2, 2, 4, 4, 8, 2"),
     "cfg1": (3.373e7, "profiles/sgemm_1024_colNN.md", "clbh::GemmMfmaKernel<float, clbh::MfmaConfig<float, 2, 2, 2, 1, 32, 4"),
     "cfg5a": (3.390e7, "profiles/sgemm_1000_colNN.md", "clbh::GemmMfmaKernel<float, clbh::MfmaConfig<float, 2, 2, 2, 1, 32, 4"),
-    "cfg3": (1.880e9, "profiles/hgemm_8192_colNT.md", "clbh::HgemmWideKernel<false, false, false>"),
+    "cfg3": (1.880e9, "profiles/hgemm_8192_colNT.md", "clbh::HgemmWideKernel<false, false, false, false>"),
     "cfg4": (1.007e8, "profiles/sgemm_strided_batched_8192x32.md", "clbh::GemmSmallBatchedKernel"),
     "cfg5b": (7.704e7, "profiles/sgemm_4099x17x4096_colNN.md", "clbh::GemmSkinnyColsKernel<1, 1, 3, true>"),
     "cfg5c": (7.461e7, "profiles/sgemm_17x4099x4096_colNN.md", "clbh::GemmSkinnyRowsKernel<4, 5, 5, 2, false, false, 2>"),
