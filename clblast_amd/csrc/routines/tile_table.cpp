@@ -151,7 +151,7 @@ double LaunchCost(const TileCandidate& candidate, const size_t m, const size_t n
 
 // The same estimate, k included, for `count` 256 x 256 tiles of the persistent fp16 kernel (one work-group per CU,
 // 1608 TFLOP/s, a tile costs what 467 more of k would). A last round that fills at most half of the work-groups is
-// split along K the way the device layer does it (PlanWide in device/launch_common.hpp): it then costs the walk of one
+// split along K the way the device layer does it (PlanWide in device/launch_plans.hpp): it then costs the walk of one
 // K range plus what 2000 of k would - the sums' way through memory and the second kernel (HSYRK 8192, 528 tiles: two
 // rounds of 186 us, then 54 us for 16 tiles in 16 ranges of 512; in eight ranges the same) - where that is less than the whole walk.
 double WideTileCost(const size_t count, const size_t k) {

@@ -24,3 +24,22 @@ def test_every_choice_is_one_its_launcher_accepts(tmp_path):
     run = subprocess.run([str(binary)], capture_output=True, text=True)
     assert run.returncode == 0, run.stdout[-3000:]
     assert "violations 0" in run.stdout
+
+
+def test_the_plan_of_the_persistent_fp16_kernel(tmp_path):
+    """The device layer's plan of a launch of the wide fp16 kernel (which tiles, which of them split into how many K
+    ranges, how much workspace) is host code without HIP: its invariants, and its agreement with the tile table about
+    where that kernel runs, over a sweep of shapes."""
+    compiler = shutil.which("g++")
+    if compiler is None:
+        pytest.skip("no g++ here")
+    binary = tmp_path / "plan"
+    sources = [os.path.join(ROOT, "tests", "host", "wide_plan_sweep.cpp"),
+               os.path.join(ROOT, "clblast_amd", "csrc", "routines", "tile_table.cpp")]
+    done = subprocess.run([compiler, "-std=c++17", "-O1", "-I" + os.path.join(ROOT, "include"),
+                           "-I" + os.path.join(ROOT, "clblast_amd", "csrc")] + sources + ["-o", str(binary)],
+                          capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr[-3000:]
+    run = subprocess.run([str(binary)], capture_output=True, text=True)
+    assert run.returncode == 0, run.stdout[-3000:]
+    assert "violations 0" in run.stdout
