@@ -1,0 +1,343 @@
+// =================================================================================================
+// fp16 CONVGEMM with unit strides and no dilation on gfx950, without an im2col matrix and without a padded copy of
+// the images (the reference's single-kernel method, src/routines/levelx/xconvgemm.cpp:121-160 with
+// src/kernels/levelx/xconvgemm_part1.opencl / xconvgemm_part2.opencl, gathers every patch element from memory; its
+// two-kernel method writes the kernel_h * kernel_w times larger im2col matrix first, xconvgemm.cpp:78-119).
+//
+// A work-group owns `rows` whole output rows of one image (at most 448 output pixels) and 128 kernels. The channels
+// are walked in chunks of 16. For a chunk, the part of the image that the tile's patches touch - (rows + kernel_h - 1)
+// x (width + 2 pad_w) pixels, zeros outside the image - is staged in LDS with the CHANNEL as the contiguous index
+// ([row][column][channel], pitch 24 halves): 16-byte loads along the image rows of two channels at a time, their halves
+// interleaved in registers, eight 4-byte LDS writes (the lanes of a wavefront take pieces of eight different slab rows,
+// which keeps the 64 dwords of a write on 64 banks). Every tap (kh, kw) of the kernel is then one k-step of
+// v_mfma_f32_32x32x16_f16 whose pixel operand is a 16-byte LDS read at the tile pixel's address plus the tap's uniform
+// offset: the image is read from memory once per chunk, not once per tap, and no address arithmetic stands between the
+// matrix instructions. Two slabs alternate, so that the next chunk is requested before and written after the products
+// of the current one (one barrier per chunk). A single wavefront per SIMD hides only what stands between its matrix
+// instructions, so the reads of the next tap and the writes of the next chunk's pieces are placed there one by one.
+//
+// The kernel matrix is read through a copy in k-step order, [chunk][tap][kernel][16 channels] (HconvPermuteKernel; taps
+// mirrored there for a true convolution): the tile's 128 kernels of a chunk are taps contiguous pieces of 4 KiB, which
+// go straight from memory into LDS next to the slab (two chunks alternate as the slabs do), and a lane's eight k values
+// are one 16-byte LDS read. The K walk itself therefore issues no memory instruction that its products wait for: the
+// next chunk's image pieces and kernels are requested at the top of a chunk and waited for at its end. Two sets of
+// operand registers alternate from tap to tap, so that the reads of the next tap stand under the products of this one.
+//
+// Wavefront (wm, wn) of the four owns pixels [224 wm, 224 wm + 224) x kernels [64 wn, 64 wn + 64): 7 x 2 blocks of
+// 32 x 32, 224 accumulator registers. The pixels are the FIRST operand, so that a lane's four consecutive result
+// registers are four consecutive pixels of one kernel: after the walk they go to LDS as [kernel][pixel] with 8-byte
+// writes (the slabs are no longer needed) and leave with 16-byte stores along the result's rows.
+// =================================================================================================
+#ifndef CLBLAST_HIP_KERNELS_CONV_SLAB_F16_HPP_
+#define CLBLAST_HIP_KERNELS_CONV_SLAB_F16_HPP_
+
+#include <hip/hip_runtime.h>
+
+#include <type_traits>
+
+#include "kernels/gemm_mfma.hpp"
+#include "kernels/gemm_mfma_f16.hpp"
+
+namespace clbh {
+
+constexpr int kConvSlabThreads = 256;
+constexpr int kConvSlabChunk = 16;         // channels per chunk = k of one matrix instruction
+constexpr int kConvSlabPitch = 24;         // halves from a pixel to the next in a slab (16 channels + 8: no bank conflicts)
+constexpr int kConvSlabBlocks = 7;         // 32-pixel blocks per wavefront
+constexpr int kConvSlabPixels = 2 * kConvSlabBlocks * 32;  // 448 per work-group
+constexpr int kConvSlabKernels = 128;      // per work-group
+constexpr int kConvSlabResultPitch = kConvSlabPixels + 8;  // halves from a kernel to the next in the epilogue's tile
+constexpr int kConvSlabResultBytes = kConvSlabKernels * kConvSlabResultPitch * 2;
+
+struct ConvSlabArgs {
+  const _Float16* images;   // batch x channels x height x width
+  const _Float16* weights;  // [channels / 16][taps][kernels][16] (HconvPermuteKernel)
+  _Float16* result;         // batch x kernels x output_h x output_w
+  int channels, height, width;
+  int kernel_h, kernel_w, pad_h, pad_w;
+  int output_h, output_w;
+  int kernels;
+  int rows;          // output rows per tile; rows * output_w <= kConvSlabPixels
+  int row_tiles;     // ceil(output_h / rows)
+  int kernel_tiles;  // ceil(kernels / kConvSlabKernels)
+  int slab_rows, slab_width;  // rows + kernel_h - 1, width + 2 pad_w
+  int slab_halves;            // (slab_rows * slab_width + 8) * kConvSlabPitch
+  int spare_at;               // halves from a slab's start to its last 8 pixels, a strip that no product reads
+};
+
+// x / d for 0 <= x, d < 2^10, with inverse = 1.0f / d (exact: (x + 0.5) / d is at least 2^-11 away from an integer)
+__device__ __forceinline__ int SmallQuotient(const int x, const float inverse) {
+  return static_cast<int>((static_cast<float>(x) + 0.5f) * inverse);
+}
+
+// out[((chunk * taps + tap) * kernels + n) * 16 + i] = weights[n][(16 chunk + i) * taps + (flip ? taps - 1 - tap : tap)],
+// one thread per eight consecutive i
+__global__ __launch_bounds__(256) void HconvPermuteKernel(const _Float16* __restrict__ weights, _Float16* __restrict__ out,
+                                                          const int kernels, const int channels, const int taps,
+                                                          const int flip) {
+  const int index = blockIdx.x * 256 + threadIdx.x;
+  if (index >= kernels * (channels / 8) * taps) { return; }
+  const int part = index % 2;
+  const int n = (index / 2) % kernels;
+  const int step = index / (2 * kernels);
+  const int chunk = step / taps, tap = step % taps;
+  const int stored_tap = flip ? (taps - 1 - tap) : tap;
+  const _Float16* from = weights + (static_cast<long long>(n) * channels + chunk * kConvSlabChunk + 8 * part) * taps + stored_tap;
+  half8_t eight;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) { eight[i] = from[i * taps]; }
+  *reinterpret_cast<half8_t*>(out + static_cast<long long>(index) * 8) = eight;
+}
+
+// grid: batch x row_tiles x kernel_tiles work-groups of 256 threads; dynamic LDS: two slabs and two chunks of the kernel
+// matrix, or kConvSlabResultBytes where that is more.
+// TASKS: 16-byte pieces of the slab (of two channels each) a thread stages per chunk, at least
+// ceil(8 * slab_rows * (width / 8) / 256). TAPS: kernel_h * kernel_w as a constant (the walk over the taps is then
+// straight-line code), or 0 for any number of taps.
+template <int TASKS, int TAPS>
+__global__ __launch_bounds__(kConvSlabThreads, 1) void HconvSlabKernel(const ConvSlabArgs p) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  _Float16* lds = reinterpret_cast<_Float16*>(lds_raw);
+  typedef unsigned Dwords4 __attribute__((ext_vector_type(4)));
+  constexpr int PITCH = kConvSlabPitch, BLOCKS = kConvSlabBlocks;
+  constexpr int TAP_HALVES = kConvSlabKernels * kConvSlabChunk;  // the tile's part of the kernel matrix for one tap
+
+  const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const int wave_m = wave % 2, wave_n = wave / 2;
+  int block = blockIdx.x;
+  const int kernel_tile = block % p.kernel_tiles;
+  block /= p.kernel_tiles;
+  const int row_tile = block % p.row_tiles;
+  const int batch = block / p.row_tiles;
+  const int row0 = row_tile * p.rows;
+  const int valid_pixels = min(p.rows, p.output_h - row0) * p.output_w;
+  const int n0 = kernel_tile * kConvSlabKernels;
+  const int plane = p.height * p.width;
+  const int taps = TAPS > 0 ? TAPS : p.kernel_h * p.kernel_w;
+  const int chunks = p.channels / kConvSlabChunk;
+  _Float16* const ordered = lds + 2 * p.slab_halves;  // two chunks of the kernel matrix, taps * TAP_HALVES each
+
+  // The pieces this thread stages, the same for every chunk: channel pair, slab row, 8 columns. Eight neighbouring
+  // lanes hold the eight channel pairs of one piece, the eight groups of a wavefront the pieces of eight consecutive
+  // slab rows in the same columns. A pixel is 12 banks from the next and a slab row 8 x (an odd number) banks from
+  // the next (the host pads the slab's width to 2 mod 4 pixels), so the 64 dwords of one write instruction fall on 64
+  // different banks. A piece that does not exist (a row outside the image, a task beyond the slab) is loaded from the
+  // first row of the planes and written to a spare strip behind the slab: no branches, the slab keeps its zeros.
+  int piece_source[TASKS], piece_target[TASKS];  // element offsets in the chunk's planes and in LDS
+  {
+    const int row_vectors = p.width / 8;
+    const float rows_inverse = 1.0f / static_cast<float>(p.slab_rows);
+#pragma unroll
+    for (int j = 0; j < TASKS; ++j) {
+      const int t = tid + kConvSlabThreads * j;
+      const int pair = t % (kConvSlabChunk / 2), rest = t / (kConvSlabChunk / 2);
+      const int v = SmallQuotient(rest, rows_inverse), h = rest - v * p.slab_rows;
+      const int image_row = row0 + h - p.pad_h;
+      const bool exists = v < row_vectors && image_row >= 0 && image_row < p.height;
+      piece_source[j] = exists ? (2 * pair * p.height + image_row) * p.width + 8 * v : 2 * pair * plane;
+      piece_target[j] = (exists ? (h * p.slab_width + p.pad_w + 8 * v) * PITCH : p.spare_at) + 2 * pair;
+    }
+  }
+  Dwords4 even_channel[TASKS], odd_channel[TASKS];
+  const _Float16* image = p.images + static_cast<long long>(batch) * p.channels * plane;
+  auto request = [&](const int chunk) {
+    const _Float16* planes = image + static_cast<long long>(chunk) * kConvSlabChunk * plane;
+#pragma unroll
+    for (int j = 0; j < TASKS; ++j) {
+      even_channel[j] = *reinterpret_cast<const Dwords4*>(planes + piece_source[j]);
+      odd_channel[j] = *reinterpret_cast<const Dwords4*>(planes + piece_source[j] + plane);
+    }
+  };
+  auto deposit = [&](_Float16* slab) {
+#pragma unroll
+    for (int j = 0; j < TASKS; ++j) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {  // pixel i of the piece: (even channel, odd channel) as one dword
+        const unsigned pair = __builtin_amdgcn_perm(odd_channel[j][i / 2], even_channel[j][i / 2],
+                                                    (i % 2) ? 0x07060302u : 0x05040100u);
+        *reinterpret_cast<unsigned*>(slab + piece_target[j] + i * PITCH) = pair;
+      }
+    }
+  };
+  // The tile's 128 kernels of a chunk, tap by tap, straight from memory into LDS: wavefront w moves kernels
+  // [32 w, 32 w + 32) of every tap (1 KiB, contiguous on both sides). Kernels beyond the matrix read what follows them
+  // (zeros behind the end of the copy); their results are not stored.
+  const int ordered_bytes_left = (p.channels * taps * p.kernels - n0 * kConvSlabChunk) * 2;
+  const int tap_bytes = p.kernels * kConvSlabChunk * 2;
+  auto request_kernels = [&](const int chunk) {
+    typedef __attribute__((address_space(3))) void* LdsPtr;
+    const _Float16* from = p.weights + n0 * kConvSlabChunk;
+    const auto view = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(from), 0, ordered_bytes_left, kRawBufferFlags);
+    _Float16* to = ordered + (chunk & 1) * taps * TAP_HALVES + wave * 512;
+    int lane_bytes = chunk * taps * tap_bytes + wave * 1024 + lane * 16;  // (the range check covers this offset only)
+    for (int tap = 0; tap < taps; ++tap) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(view, (LdsPtr)(to), 16, lane_bytes, 0, 0, 0);
+      to += TAP_HALVES;
+      lane_bytes += tap_bytes;
+    }
+  };
+
+  request_kernels(0);
+  request(0);
+  // Zeros in both slabs: what no piece covers (the border columns, rows outside the image) stays zero
+  for (int i = tid; i < 2 * p.slab_halves / 8; i += kConvSlabThreads) { reinterpret_cast<Dwords4*>(lds)[i] = Dwords4(0u); }
+
+  // Where this lane's pixel of each block sits in a slab (tap (0, 0)), plus its half of the 16 channels
+  int pixel_at[BLOCKS];
+  const float width_inverse = 1.0f / static_cast<float>(p.output_w);
+#pragma unroll
+  for (int i = 0; i < BLOCKS; ++i) {
+    int pixel = (wave_m * BLOCKS + i) * 32 + lane % 32;
+    if (pixel >= valid_pixels) { pixel = 0; }
+    const int row = SmallQuotient(pixel, width_inverse);
+    pixel_at[i] = (row * p.slab_width + (pixel - row * p.output_w)) * PITCH + 8 * (lane / 32);
+  }
+  // This lane's kernels in a tap's part of the ordered kernel matrix
+  int kernel_at[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) { kernel_at[j] = (wave_n * 64 + j * 32 + lane % 32) * kConvSlabChunk + 8 * (lane / 32); }
+
+  // (with TAPS known the first tap of the first chunk takes 0 as its addend instead: 224 register writes less)
+  float16_t acc[BLOCKS][2];
+  if (TAPS == 0) {
+#pragma unroll
+    for (int i = 0; i < BLOCKS; ++i) {
+      acc[i][0] = float16_t(0.0f);
+      acc[i][1] = float16_t(0.0f);
+    }
+  }
+
+  __syncthreads();  // the zeros are in place
+  deposit(lds);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's part of the kernels has arrived
+  __syncthreads();
+
+  // One set of operands: the pixels' 16 channels at a tap and the kernels' 16 channels at that tap
+  struct Operands {
+    half8_t pixels[BLOCKS], kernels[2];
+  };
+  auto fetch = [&](const _Float16* slab_at_tap, const _Float16* kernels_at_tap, Operands& set) {
+    // (in the order of their first use: the reads are spread over the products of the tap before)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) { set.kernels[j] = *reinterpret_cast<const half8_t*>(kernels_at_tap + kernel_at[j]); }
+#pragma unroll
+    for (int i = 0; i < BLOCKS; ++i) { set.pixels[i] = *reinterpret_cast<const half8_t*>(slab_at_tap + pixel_at[i]); }
+  };
+  auto products = [&](const Operands& set, auto from_zero) {
+#pragma unroll
+    for (int i = 0; i < BLOCKS; ++i) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(set.pixels[i], set.kernels[j],
+                                                          decltype(from_zero)::value ? float16_t(0.0f) : acc[i][j], 0, 0, 0);
+      }
+    }
+  };
+
+  // The walk over one chunk; `first`: the chunk that starts the sums (a type, so that chunk 0 is code of its own)
+  auto walk = [&](const int chunk, auto first) {
+    constexpr bool FIRST = decltype(first)::value && TAPS > 0;
+    const _Float16* slab = lds + (chunk & 1) * p.slab_halves;
+    const _Float16* kernels_now = ordered + (chunk & 1) * taps * TAP_HALVES;
+    if (chunk + 1 < chunks) {
+      request_kernels(chunk + 1);
+      request(chunk + 1);
+    }
+    Operands set[2];
+    fetch(slab, kernels_now, set[0]);
+    int kh = 0, kw = 0;
+    auto next_tap = [&]() {  // the slab's offset of the tap after (kh, kw)
+      if (++kw == p.kernel_w) {
+        kw = 0;
+        ++kh;
+      }
+      return (kh * p.slab_width + kw) * PITCH;
+    };
+    // (the scheduler is held to an order: left alone it moves every read down to its first use, and the products then
+    // wait for the LDS read by read)
+    if (TAPS > 0) {
+#pragma unroll
+      for (int tap = 0; tap + 1 < TAPS; ++tap) {
+        fetch(slab + next_tap(), kernels_now + (tap + 1) * TAP_HALVES, set[(tap + 1) % 2]);
+        if (tap == 0) { products(set[0], std::integral_constant<bool, FIRST>{}); } else { products(set[tap % 2], std::false_type{}); }
+        // one read after every matrix instruction: nine reads in a row wait for room in the LDS queue, and the
+        // wavefront issues nothing else meanwhile
+#pragma unroll
+        for (int i = 0; i < BLOCKS + 2; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one matrix instruction,
+          __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);  // the address of
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * BLOCKS - (BLOCKS + 2), 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // The last tap has nothing to fetch: the next chunk's pieces go to their slab between its products (a wavefront
+      // alone on its SIMD hides nothing that does not stand between matrix instructions). Without a test of the chunk,
+      // which would end the scheduling region: after the last chunk the writes repeat the pieces of that chunk in the
+      // slab that nothing reads any more.
+      deposit(lds + ((chunk + 1) & 1) * p.slab_halves);
+      products(set[(TAPS - 1) % 2], std::integral_constant<bool, FIRST && TAPS == 1>{});
+#pragma unroll
+      for (int i = 0; i < 2 * BLOCKS; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one matrix instruction,
+        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);  // two vector ALU instructions,
+        __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);  // two LDS writes
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    } else {
+      for (int tap = 0; tap < taps; tap += 2) {
+        if (tap + 1 < taps) { fetch(slab + next_tap(), kernels_now + (tap + 1) * TAP_HALVES, set[1]); }
+        __builtin_amdgcn_sched_barrier(0);
+        products(set[0], std::false_type{});
+        __builtin_amdgcn_sched_barrier(0);
+        if (tap + 1 < taps) {
+          if (tap + 2 < taps) { fetch(slab + next_tap(), kernels_now + (tap + 2) * TAP_HALVES, set[0]); }
+          __builtin_amdgcn_sched_barrier(0);
+          products(set[1], std::false_type{});
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+    if (TAPS == 0 && chunk + 1 < chunks) { deposit(lds + ((chunk + 1) & 1) * p.slab_halves); }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  };
+  walk(0, std::true_type{});
+  for (int chunk = 1; chunk < chunks; ++chunk) { walk(chunk, std::false_type{}); }
+
+  // Epilogue: [kernel][pixel] in LDS (every wavefront its own part), then 16-byte stores along the result's rows.
+  // Register r of block (i, j): pixel 32 i + 8 (r / 4) + 4 (lane / 32) + r % 4, kernel 32 j + lane % 32.
+  constexpr int RP = kConvSlabResultPitch;
+#pragma unroll
+  for (int i = 0; i < BLOCKS; ++i) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        half4_t four;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { four[e] = static_cast<_Float16>(acc[i][j][4 * g + e]); }
+        const int pixel = (wave_m * BLOCKS + i) * 32 + 8 * g + 4 * (lane / 32);
+        const int n = wave_n * 64 + j * 32 + lane % 32;
+        *reinterpret_cast<half4_t*>(lds + n * RP + pixel) = four;
+      }
+    }
+  }
+  __syncthreads();
+  constexpr int ROW_VECTORS = BLOCKS * 32 / 8;  // 16-byte pieces of a kernel's row in this wavefront's part
+  const long long pixels = static_cast<long long>(p.output_h) * p.output_w;
+  _Float16* result = p.result + static_cast<long long>(batch) * p.kernels * pixels + static_cast<long long>(row0) * p.output_w;
+#pragma unroll 14
+  for (int t = 0; t < ROW_VECTORS; ++t) {
+    const int q = lane + 64 * t;
+    const int n = wave_n * 64 + q / ROW_VECTORS, pixel = wave_m * BLOCKS * 32 + (q % ROW_VECTORS) * 8;
+    if (n0 + n < p.kernels && pixel < valid_pixels) {
+      const Dwords4 value = *reinterpret_cast<const Dwords4*>(lds + n * RP + pixel);
+      *reinterpret_cast<Dwords4*>(result + (n0 + n) * pixels + pixel) = value;
+    }
+  }
+}
+
+}  // namespace clbh
+
+#endif  // CLBLAST_HIP_KERNELS_CONV_SLAB_F16_HPP_

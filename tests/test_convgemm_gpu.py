@@ -89,6 +89,55 @@ def test_convgemm_sweep(gpu, bits):
             problem.check(after)
 
 
+SLAB_CASES = [  # fp16 shapes for the kernel that stages image slabs in LDS: unit strides, 16 | channels, 8 | widths
+    (16, 32, 32, 3, 3, 1, 1, 1, 1, 1, 1, 32, 4),    # three row tiles of 11 rows, the last with 10
+    (32, 20, 24, 3, 3, 1, 1, 1, 1, 1, 1, 130, 3),   # two chunks of channels, two tile columns of kernels (the second: 2)
+    (16, 9, 40, 5, 1, 2, 0, 1, 1, 1, 1, 20, 2),     # a 5 x 1 window, padding along the height only, one tile per image
+    (48, 16, 16, 1, 1, 0, 0, 1, 1, 1, 1, 64, 5),    # 1 x 1: one tap per chunk, three k-steps in all
+    (16, 37, 16, 3, 3, 1, 1, 1, 1, 1, 1, 8, 2),     # rows of 16 pixels: tiles of 19 and 18 rows
+    (16, 16, 16, 3, 5, 1, 2, 1, 1, 1, 1, 33, 2),    # a 3 x 5 window: 15 taps (any number of taps: a loop, not straight-line code)
+    (16, 15, 24, 4, 3, 2, 1, 1, 1, 1, 1, 5, 1),     # an even window height: 16 output rows, an even number of taps
+    (32, 3, 232, 3, 3, 1, 1, 1, 1, 1, 1, 40, 2),    # one output row per tile
+]
+
+
+def slab_scratch_bytes(case):
+    """What the device layer reports for the case: non-zero when the slab kernel takes it."""
+    import ctypes
+    from clblast_amd import _lib
+
+    class Shape(ctypes.Structure):
+        _fields_ = [(name, ctypes.c_int) for name in (
+            "channels", "height", "width", "kernel_h", "kernel_w", "pad_h", "pad_w", "stride_h", "stride_w", "dilation_h",
+            "dilation_w", "output_h", "output_w", "flip")]
+    channels, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w, kernels, batch = case
+    shape = Shape(channels, height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w,
+                  oracle.conv_output_extent(height, kernel_h, pad_h, stride_h, dilation_h),
+                  oracle.conv_output_extent(width, kernel_w, pad_w, stride_w, dilation_w), 0)
+    function = _lib.load().clbh_conv_slab_scratch_bytes
+    function.restype = ctypes.c_size_t
+    function.argtypes = [ctypes.POINTER(Shape), ctypes.c_int, ctypes.c_int]
+    return function(ctypes.byref(shape), kernels, batch)
+
+
+def test_convgemm_fp16_slab_kernel(gpu):
+    """The shapes the slab kernel takes (asserted), both modes, with 16-byte aligned offsets (the kernel) and with odd
+    ones (the gathering GEMM on the same shape) against the oracle."""
+    seed = 18500
+    for case in SLAB_CASES:
+        assert slab_scratch_bytes(case) == 2 * case[0] * case[3] * case[4] * case[11], case
+        for mode in (CROSS_CORRELATION, CONVOLUTION):
+            for offsets in ((0, 0, 0), (16, 7, 24), (10, 6, 14)):
+                seed += 1
+                problem = ConvProblem(16, mode, case, seed, offsets)
+                status, after = problem.run(gpu)
+                assert status == 0, (status, case)
+                problem.check(after)
+    for case in CASES:
+        if case != SLAB_CASES[0]:
+            assert slab_scratch_bytes(case) == 0, case
+
+
 @pytest.mark.parametrize("bits", (32, 16))
 def test_convgemm_matches_torch_at_size(gpu, bits):
     """64 channels of 112 x 112, 128 kernels of 3 x 3, 8 images: against torch's conv2d (the vendor library) in fp32."""
