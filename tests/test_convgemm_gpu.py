@@ -98,6 +98,8 @@ SLAB_CASES = [  # fp16 shapes for the kernel that stages image slabs in LDS: uni
     (16, 16, 16, 3, 5, 1, 2, 1, 1, 1, 1, 33, 2),    # a 3 x 5 window: 15 taps (any number of taps: a loop, not straight-line code)
     (16, 15, 24, 4, 3, 2, 1, 1, 1, 1, 1, 5, 1),     # an even window height: 16 output rows, an even number of taps
     (32, 3, 232, 3, 3, 1, 1, 1, 1, 1, 1, 40, 2),    # one output row per tile
+    (16, 10, 224, 3, 3, 1, 1, 1, 1, 1, 1, 8, 1),    # two rows of 224 per tile: four staging pieces per thread
+    (16, 6, 160, 5, 1, 2, 0, 1, 1, 1, 1, 12, 2),    # the same with a loop over five taps; a slab wider than the image (162)
 ]
 
 
