@@ -239,12 +239,17 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void HconvSlabKernel(const Con
     constexpr bool FIRST = decltype(first)::value && TAPS > 0;
     const _Float16* slab = lds + (chunk & 1) * p.slab_halves;
     const _Float16* kernels_now = ordered + (chunk & 1) * taps * TAP_HALVES;
-    if (chunk + 1 < chunks) {
-      request_kernels(chunk + 1);
-      request(chunk + 1);
+    // The next chunk's kernels and pieces are asked for between the products of the first tap (TAPS known) - without a
+    // test of the chunk, which would end the scheduling region: the last chunk asks for itself again, into the slab and
+    // the kernel buffer that nothing reads any more, and the wait at its end keeps these loads out of the epilogue's LDS.
+    const int chunk_ahead = min(chunk + 1, chunks - 1);
+    if (TAPS == 0 && chunk + 1 < chunks) {
+      request_kernels(chunk_ahead);
+      request(chunk_ahead);
     }
     Operands set[2];
     fetch(slab, kernels_now, set[0]);
+    __builtin_amdgcn_sched_barrier(0);
     int kh = 0, kw = 0;
     auto next_tap = [&]() {  // the slab's offset of the tap after (kh, kw)
       if (++kw == p.kernel_w) {
@@ -256,8 +261,16 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void HconvSlabKernel(const Con
     // (the scheduler is held to an order: left alone it moves every read down to its first use, and the products then
     // wait for the LDS read by read)
     if (TAPS > 0) {
+      if (TAPS == 1) {
+        request_kernels(chunk_ahead);
+        request(chunk_ahead);
+      }
 #pragma unroll
       for (int tap = 0; tap + 1 < TAPS; ++tap) {
+        if (tap == 0) {
+          request_kernels(chunk_ahead);
+          request(chunk_ahead);
+        }
         fetch(slab + next_tap(), kernels_now + (tap + 1) * TAP_HALVES, set[(tap + 1) % 2]);
         if (tap == 0) { products(set[0], std::integral_constant<bool, FIRST>{}); } else { products(set[tap % 2], std::false_type{}); }
         // one read after every matrix instruction: nine reads in a row wait for room in the LDS queue, and the
@@ -266,9 +279,20 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void HconvSlabKernel(const Con
         for (int i = 0; i < BLOCKS + 2; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one matrix instruction,
           __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);  // the address of
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read,
+          if (tap == 0) {
+            __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);  // (first tap: the addresses of)
+            __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);  // two loads of the next chunk
+          }
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, 2 * BLOCKS - (BLOCKS + 2), 0);
+#pragma unroll
+        for (int i = BLOCKS + 2; i < 2 * BLOCKS; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (tap == 0) {
+            __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+          }
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
       // The last tap has nothing to fetch: the next chunk's pieces go to their slab between its products (a wavefront
