@@ -138,7 +138,7 @@ DEVICE_LAYER_SYMBOLS = [
     "clbh_upload_async", "clbh_event_record", "clbh_stream_device", "clbh_error_string", "clbh_symmetric_to_square",
     "clbh_triangular_to_square", "clbh_triangular_to_band", "clbh_complex_triangular_to_band", "clbh_copy_matrix", "clbh_invert_block_size", "clbh_invert_diagonal_blocks",
     "clbh_complex_expand", "clbh_complex_transpose", "clbh_complex_scale", "clbh_complex_expand_batched",
-    "clbh_complex_transpose_batched", "clbh_complex_scale_batched", "clbh_complex_gemm_small_batched", "clbh_copy_matrix_batched", "clbh_alloc", "clbh_free", "clbh_copy", "clbh_im2col", "clbh_conv_gather_possible", "clbh_conv_slab_scratch_bytes", "clbh_conv_slab_f16", "clbh_pad_image", "clbh_fill_zero", "clbh_complex_symmetric_to_square",
+    "clbh_complex_transpose_batched", "clbh_complex_scale_batched", "clbh_complex_gemm_small_batched", "clbh_copy_matrix_batched", "clbh_alloc", "clbh_free", "clbh_copy", "clbh_im2col", "clbh_conv_gather_possible", "clbh_conv_slab_scratch_bytes", "clbh_conv_slab", "clbh_pad_image", "clbh_fill_zero", "clbh_complex_symmetric_to_square",
     "clbh_complex_triangular_to_square", "clbh_complex_zero_diagonal_imag", "clbh_complex_invert_block_size",
     "clbh_complex_invert_diagonal_blocks", "clbh_static_scratch", "clbh_static_scratch_bytes", "clbh_stream_capturing",
     "clbh_stream_is_alias", "clbh_compute_units", "clbh_tickets"]

@@ -1,8 +1,12 @@
 // =================================================================================================
-// fp16 CONVGEMM with unit strides and no dilation on gfx950, without an im2col matrix and without a padded copy of
+// fp16 and fp32 CONVGEMM with unit strides and no dilation on gfx950, without an im2col matrix and without a padded copy of
 // the images (the reference's single-kernel method, src/routines/levelx/xconvgemm.cpp:121-160 with
 // src/kernels/levelx/xconvgemm_part1.opencl / xconvgemm_part2.opencl, gathers every patch element from memory; its
 // two-kernel method writes the kernel_h * kernel_w times larger im2col matrix first, xconvgemm.cpp:78-119).
+//
+// (Written out for fp16; fp32 is the same with half as many channels per step: a chunk of 8 channels, 16-byte pieces of
+// four pixels of ONE channel, v_mfma_f32_32x32x2_f32 - four of them per 16-byte operand pair, lane group g of the two
+// supplying channels 4 g .. 4 g + 3 - and a result that leaves the registers directly, 16 bytes of four pixels per lane.)
 //
 // A work-group owns `rows` whole output rows of one image (at most 448 output pixels) and 128 kernels. The channels
 // are walked in chunks of 16. For a chunk, the part of the image that the tile's patches touch - (rows + kernel_h - 1)
@@ -28,8 +32,8 @@
 // registers are four consecutive pixels of one kernel: after the walk they go to LDS as [kernel][pixel] with 8-byte
 // writes (the slabs are no longer needed) and leave with 16-byte stores along the result's rows.
 // =================================================================================================
-#ifndef CLBLAST_HIP_KERNELS_CONV_SLAB_F16_HPP_
-#define CLBLAST_HIP_KERNELS_CONV_SLAB_F16_HPP_
+#ifndef CLBLAST_HIP_KERNELS_CONV_SLAB_HPP_
+#define CLBLAST_HIP_KERNELS_CONV_SLAB_HPP_
 
 #include <hip/hip_runtime.h>
 
@@ -41,18 +45,27 @@
 namespace clbh {
 
 constexpr int kConvSlabThreads = 256;
-constexpr int kConvSlabChunk = 16;         // channels per chunk = k of one matrix instruction
-constexpr int kConvSlabPitch = 24;         // halves from a pixel to the next in a slab (16 channels + 8: no bank conflicts)
+constexpr int kConvSlabPixelBytes = 48;    // from a pixel to the next in a slab (32 bytes of channels + 16: no bank conflicts)
+template <typename T>
+struct ConvSlabType {
+  static constexpr int CHUNK = 32 / sizeof(T);                   // channels per chunk: 32 bytes per pixel (16 halves, 8 floats)
+  static constexpr int PITCH = kConvSlabPixelBytes / sizeof(T);  // elements from a pixel to the next
+  static constexpr int PIECE = 16 / sizeof(T);                   // pixels of a 16-byte piece of an image row (8, 4)
+  static constexpr int PLANES = sizeof(T) == 2 ? 2 : 1;          // channels a staged piece covers (fp16: a pair, one dword per pixel)
+  typedef T Vector __attribute__((ext_vector_type(16 / sizeof(T))));  // a 16-byte operand
+};
 constexpr int kConvSlabBlocks = 7;         // 32-pixel blocks per wavefront
 constexpr int kConvSlabPixels = 2 * kConvSlabBlocks * 32;  // 448 per work-group
 constexpr int kConvSlabKernels = 128;      // per work-group
-constexpr int kConvSlabResultPitch = kConvSlabPixels + 8;  // halves from a kernel to the next in the epilogue's tile
+constexpr int kConvSlabResultPitch = kConvSlabPixels + 8;  // halves from a kernel to the next in the fp16 epilogue's tile
 constexpr int kConvSlabResultBytes = kConvSlabKernels * kConvSlabResultPitch * 2;
+constexpr int kConvSlabResultBytesF32 = (kConvSlabKernels / 2) * (kConvSlabPixels + 4) * 4;  // half of the tile at a time
 
+template <typename T>
 struct ConvSlabArgs {
-  const _Float16* images;   // batch x channels x height x width
-  const _Float16* weights;  // [channels / 16][taps][kernels][16] (HconvPermuteKernel)
-  _Float16* result;         // batch x kernels x output_h x output_w
+  const T* images;   // batch x channels x height x width
+  const T* weights;  // [channels / CHUNK][taps][kernels][CHUNK] (ConvPermuteKernel)
+  T* result;         // batch x kernels x output_h x output_w
   int channels, height, width;
   int kernel_h, kernel_w, pad_h, pad_w;
   int output_h, output_w;
@@ -61,8 +74,8 @@ struct ConvSlabArgs {
   int row_tiles;     // ceil(output_h / rows)
   int kernel_tiles;  // ceil(kernels / kConvSlabKernels)
   int slab_rows, slab_width;  // rows + kernel_h - 1, width + 2 pad_w
-  int slab_halves;            // (slab_rows * slab_width + 8) * kConvSlabPitch
-  int spare_at;               // halves from a slab's start to its last 8 pixels, a strip that no product reads
+  int slab_elements;          // (slab_rows * slab_width + 8) * PITCH
+  int spare_at;               // elements from a slab's start to its last 8 pixels, a strip that no product reads
 };
 
 // x / d for 0 <= x, d < 2^10, with inverse = 1.0f / d (exact: (x + 0.5) / d is at least 2^-11 away from an integer)
@@ -70,37 +83,41 @@ __device__ __forceinline__ int SmallQuotient(const int x, const float inverse) {
   return static_cast<int>((static_cast<float>(x) + 0.5f) * inverse);
 }
 
-// out[((chunk * taps + tap) * kernels + n) * 16 + i] = weights[n][(16 chunk + i) * taps + (flip ? taps - 1 - tap : tap)],
-// one thread per eight consecutive i
-__global__ __launch_bounds__(256) void HconvPermuteKernel(const _Float16* __restrict__ weights, _Float16* __restrict__ out,
-                                                          const int kernels, const int channels, const int taps,
-                                                          const int flip) {
+// out[((chunk * taps + tap) * kernels + n) * CHUNK + i] = weights[n][(CHUNK chunk + i) * taps + (flip ? taps - 1 - tap : tap)],
+// one thread per 16 bytes (half of a kernel's chunk)
+template <typename T>
+__global__ __launch_bounds__(256) void ConvPermuteKernel(const T* __restrict__ weights, T* __restrict__ out, const int kernels,
+                                                         const int channels, const int taps, const int flip) {
+  using Type = ConvSlabType<T>;
   const int index = blockIdx.x * 256 + threadIdx.x;
-  if (index >= kernels * (channels / 8) * taps) { return; }
+  if (index >= kernels * (channels / Type::PIECE) * taps) { return; }
   const int part = index % 2;
   const int n = (index / 2) % kernels;
   const int step = index / (2 * kernels);
   const int chunk = step / taps, tap = step % taps;
   const int stored_tap = flip ? (taps - 1 - tap) : tap;
-  const _Float16* from = weights + (static_cast<long long>(n) * channels + chunk * kConvSlabChunk + 8 * part) * taps + stored_tap;
-  half8_t eight;
+  const T* from = weights + (static_cast<long long>(n) * channels + chunk * Type::CHUNK + Type::PIECE * part) * taps + stored_tap;
+  typename Type::Vector values;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) { eight[i] = from[i * taps]; }
-  *reinterpret_cast<half8_t*>(out + static_cast<long long>(index) * 8) = eight;
+  for (int i = 0; i < Type::PIECE; ++i) { values[i] = from[i * taps]; }
+  *reinterpret_cast<typename Type::Vector*>(out + static_cast<long long>(index) * Type::PIECE) = values;
 }
 
 // grid: batch x row_tiles x kernel_tiles work-groups of 256 threads; dynamic LDS: two slabs and two chunks of the kernel
 // matrix, or kConvSlabResultBytes where that is more.
-// TASKS: 16-byte pieces of the slab (of two channels each) a thread stages per chunk, at least
-// ceil(8 * slab_rows * (width / 8) / 256). TAPS: kernel_h * kernel_w as a constant (the walk over the taps is then
+// TASKS: 16-byte pieces of the slab (fp16: of two channels each) a thread stages per chunk, at least
+// ceil(8 * slab_rows * (width / PIECE) / 256). TAPS: kernel_h * kernel_w as a constant (the walk over the taps is then
 // straight-line code), or 0 for any number of taps.
-template <int TASKS, int TAPS>
-__global__ __launch_bounds__(kConvSlabThreads, 1) void HconvSlabKernel(const ConvSlabArgs p) {
+template <typename T, int TASKS, int TAPS>
+__global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const ConvSlabArgs<T> p) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
-  _Float16* lds = reinterpret_cast<_Float16*>(lds_raw);
+  T* lds = reinterpret_cast<T*>(lds_raw);
   typedef unsigned Dwords4 __attribute__((ext_vector_type(4)));
-  constexpr int PITCH = kConvSlabPitch, BLOCKS = kConvSlabBlocks;
-  constexpr int TAP_HALVES = kConvSlabKernels * kConvSlabChunk;  // the tile's part of the kernel matrix for one tap
+  using Type = ConvSlabType<T>;
+  using Vector = typename Type::Vector;
+  constexpr bool HALF = sizeof(T) == 2;
+  constexpr int CHUNK = Type::CHUNK, PITCH = Type::PITCH, PIECE = Type::PIECE, PLANES = Type::PLANES, BLOCKS = kConvSlabBlocks;
+  constexpr int TAP_ELEMENTS = kConvSlabKernels * CHUNK;  // the tile's part of the kernel matrix for one tap (4 KiB)
 
   const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int wave_m = wave % 2, wave_n = wave / 2;
@@ -114,65 +131,73 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void HconvSlabKernel(const Con
   const int n0 = kernel_tile * kConvSlabKernels;
   const int plane = p.height * p.width;
   const int taps = TAPS > 0 ? TAPS : p.kernel_h * p.kernel_w;
-  const int chunks = p.channels / kConvSlabChunk;
-  _Float16* const ordered = lds + 2 * p.slab_halves;  // two chunks of the kernel matrix, taps * TAP_HALVES each
+  const int chunks = p.channels / CHUNK;
+  T* const ordered = lds + 2 * p.slab_elements;  // two chunks of the kernel matrix, taps * TAP_ELEMENTS each
 
-  // The pieces this thread stages, the same for every chunk: channel pair, slab row, 8 columns. Eight neighbouring
-  // lanes hold the eight channel pairs of one piece, the eight groups of a wavefront the pieces of eight consecutive
+  // The pieces this thread stages, the same for every chunk: channel pair (fp32: channel), slab row, 8 (4) columns. Eight
+  // neighbouring lanes hold the eight channel pairs (channels) of one piece, the eight groups of a wavefront the pieces of eight consecutive
   // slab rows in the same columns. A pixel is 12 banks from the next and a slab row 8 x (an odd number) banks from
   // the next (the host pads the slab's width to 2 mod 4 pixels), so the 64 dwords of one write instruction fall on 64
   // different banks. A piece that does not exist (a row outside the image, a task beyond the slab) is loaded from the
   // first row of the planes and written to a spare strip behind the slab: no branches, the slab keeps its zeros.
   int piece_source[TASKS], piece_target[TASKS];  // element offsets in the chunk's planes and in LDS
   {
-    const int row_vectors = p.width / 8;
+    const int row_vectors = p.width / PIECE;
     const float rows_inverse = 1.0f / static_cast<float>(p.slab_rows);
 #pragma unroll
     for (int j = 0; j < TASKS; ++j) {
       const int t = tid + kConvSlabThreads * j;
-      const int pair = t % (kConvSlabChunk / 2), rest = t / (kConvSlabChunk / 2);
+      const int pair = t % 8, rest = t / 8;
       const int v = SmallQuotient(rest, rows_inverse), h = rest - v * p.slab_rows;
       const int image_row = row0 + h - p.pad_h;
       const bool exists = v < row_vectors && image_row >= 0 && image_row < p.height;
-      piece_source[j] = exists ? (2 * pair * p.height + image_row) * p.width + 8 * v : 2 * pair * plane;
-      piece_target[j] = (exists ? (h * p.slab_width + p.pad_w + 8 * v) * PITCH : p.spare_at) + 2 * pair;
+      piece_source[j] = exists ? (PLANES * pair * p.height + image_row) * p.width + PIECE * v : PLANES * pair * plane;
+      piece_target[j] = (exists ? (h * p.slab_width + p.pad_w + PIECE * v) * PITCH : p.spare_at) + PLANES * pair;
     }
   }
-  Dwords4 even_channel[TASKS], odd_channel[TASKS];
-  const _Float16* image = p.images + static_cast<long long>(batch) * p.channels * plane;
+  Dwords4 even_channel[TASKS], odd_channel[HALF ? TASKS : 1];  // (fp32: the piece's only channel in even_channel)
+  const T* image = p.images + static_cast<long long>(batch) * p.channels * plane;
   auto request = [&](const int chunk) {
-    const _Float16* planes = image + static_cast<long long>(chunk) * kConvSlabChunk * plane;
+    const T* planes = image + static_cast<long long>(chunk) * CHUNK * plane;
 #pragma unroll
     for (int j = 0; j < TASKS; ++j) {
       even_channel[j] = *reinterpret_cast<const Dwords4*>(planes + piece_source[j]);
-      odd_channel[j] = *reinterpret_cast<const Dwords4*>(planes + piece_source[j] + plane);
+      if constexpr (HALF) { odd_channel[j] = *reinterpret_cast<const Dwords4*>(planes + piece_source[j] + plane); }
     }
   };
-  auto deposit = [&](_Float16* slab) {
+  auto deposit = [&](T* slab) {
 #pragma unroll
     for (int j = 0; j < TASKS; ++j) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {  // pixel i of the piece: (even channel, odd channel) as one dword
-        const unsigned pair = __builtin_amdgcn_perm(odd_channel[j][i / 2], even_channel[j][i / 2],
-                                                    (i % 2) ? 0x07060302u : 0x05040100u);
-        *reinterpret_cast<unsigned*>(slab + piece_target[j] + i * PITCH) = pair;
+      for (int i = 0; i < PIECE; ++i) {  // pixel i of the piece as one dword: fp16 (even channel, odd channel)
+        unsigned pixel;
+        if constexpr (HALF) {
+          pixel = __builtin_amdgcn_perm(odd_channel[j][i / 2], even_channel[j][i / 2], (i % 2) ? 0x07060302u : 0x05040100u);
+        } else {
+          pixel = even_channel[j][i];
+        }
+        *reinterpret_cast<unsigned*>(slab + piece_target[j] + i * PITCH) = pixel;
       }
     }
   };
   // The tile's 128 kernels of a chunk, tap by tap, straight from memory into LDS: wavefront w moves kernels
   // [32 w, 32 w + 32) of every tap (1 KiB, contiguous on both sides). Kernels beyond the matrix read what follows them
   // (zeros behind the end of the copy); their results are not stored.
-  const int ordered_bytes_left = (p.channels * taps * p.kernels - n0 * kConvSlabChunk) * 2;
-  const int tap_bytes = p.kernels * kConvSlabChunk * 2;
+  const int ordered_bytes_left = (p.channels * taps * p.kernels - n0 * CHUNK) * static_cast<int>(sizeof(T));
+  const int tap_bytes = p.kernels * CHUNK * static_cast<int>(sizeof(T));
   auto request_kernels = [&](const int chunk) {
     typedef __attribute__((address_space(3))) void* LdsPtr;
-    const _Float16* from = p.weights + n0 * kConvSlabChunk;
-    const auto view = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(from), 0, ordered_bytes_left, kRawBufferFlags);
-    _Float16* to = ordered + (chunk & 1) * taps * TAP_HALVES + wave * 512;
+    const T* from = p.weights + n0 * CHUNK;
+    const auto view = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(from), 0, ordered_bytes_left, kRawBufferFlags);
+    T* to = ordered + (chunk & 1) * taps * TAP_ELEMENTS + wave * (TAP_ELEMENTS / 4);
     int lane_bytes = chunk * taps * tap_bytes + wave * 1024 + lane * 16;  // (the range check covers this offset only)
     for (int tap = 0; tap < taps; ++tap) {
+      // (device pass only: with a pointer of a dependent type here, hipcc's host pass drops the kernel's launch stub
+      // without a diagnostic and the library fails to link)
+#if defined(__HIP_DEVICE_COMPILE__)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(view, (LdsPtr)(to), 16, lane_bytes, 0, 0, 0);
-      to += TAP_HALVES;
+#endif
+      to += TAP_ELEMENTS;
       lane_bytes += tap_bytes;
     }
   };
@@ -180,7 +205,7 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void HconvSlabKernel(const Con
   request_kernels(0);
   request(0);
   // Zeros in both slabs: what no piece covers (the border columns, rows outside the image) stays zero
-  for (int i = tid; i < 2 * p.slab_halves / 8; i += kConvSlabThreads) { reinterpret_cast<Dwords4*>(lds)[i] = Dwords4(0u); }
+  for (int i = tid; i < 2 * p.slab_elements / PIECE; i += kConvSlabThreads) { reinterpret_cast<Dwords4*>(lds)[i] = Dwords4(0u); }
 
   // Where this lane's pixel of each block sits in a slab (tap (0, 0)), plus its half of the 16 channels
   int pixel_at[BLOCKS];
@@ -190,12 +215,12 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void HconvSlabKernel(const Con
     int pixel = (wave_m * BLOCKS + i) * 32 + lane % 32;
     if (pixel >= valid_pixels) { pixel = 0; }
     const int row = SmallQuotient(pixel, width_inverse);
-    pixel_at[i] = (row * p.slab_width + (pixel - row * p.output_w)) * PITCH + 8 * (lane / 32);
+    pixel_at[i] = (row * p.slab_width + (pixel - row * p.output_w)) * PITCH + PIECE * (lane / 32);
   }
   // This lane's kernels in a tap's part of the ordered kernel matrix
   int kernel_at[2];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) { kernel_at[j] = (wave_n * 64 + j * 32 + lane % 32) * kConvSlabChunk + 8 * (lane / 32); }
+  for (int j = 0; j < 2; ++j) { kernel_at[j] = (wave_n * 64 + j * 32 + lane % 32) * CHUNK + PIECE * (lane / 32); }
 
   // (with TAPS known the first tap of the first chunk takes 0 as its addend instead: 224 register writes less)
   float16_t acc[BLOCKS][2];
@@ -214,22 +239,36 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void HconvSlabKernel(const Con
 
   // One set of operands: the pixels' 16 channels at a tap and the kernels' 16 channels at that tap
   struct Operands {
-    half8_t pixels[BLOCKS], kernels[2];
+    Vector pixels[BLOCKS], kernels[2];
   };
-  auto fetch = [&](const _Float16* slab_at_tap, const _Float16* kernels_at_tap, Operands& set) {
+  auto fetch = [&](const T* slab_at_tap, const T* kernels_at_tap, Operands& set) {
     // (in the order of their first use: the reads are spread over the products of the tap before)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) { set.kernels[j] = *reinterpret_cast<const half8_t*>(kernels_at_tap + kernel_at[j]); }
+    for (int j = 0; j < 2; ++j) { set.kernels[j] = *reinterpret_cast<const Vector*>(kernels_at_tap + kernel_at[j]); }
 #pragma unroll
-    for (int i = 0; i < BLOCKS; ++i) { set.pixels[i] = *reinterpret_cast<const half8_t*>(slab_at_tap + pixel_at[i]); }
+    for (int i = 0; i < BLOCKS; ++i) { set.pixels[i] = *reinterpret_cast<const Vector*>(slab_at_tap + pixel_at[i]); }
   };
   auto products = [&](const Operands& set, auto from_zero) {
+    if constexpr (HALF) {
 #pragma unroll
-    for (int i = 0; i < BLOCKS; ++i) {
+      for (int i = 0; i < BLOCKS; ++i) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(set.pixels[i], set.kernels[j],
-                                                          decltype(from_zero)::value ? float16_t(0.0f) : acc[i][j], 0, 0, 0);
+        for (int j = 0; j < 2; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(set.pixels[i], set.kernels[j],
+                                                            decltype(from_zero)::value ? float16_t(0.0f) : acc[i][j], 0, 0, 0);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {  // channels (e, 4 + e) of the chunk; all blocks between two sums into the same registers
+#pragma unroll
+        for (int i = 0; i < BLOCKS; ++i) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(set.pixels[i][e], set.kernels[j][e],
+                                                            (decltype(from_zero)::value && e == 0) ? float16_t(0.0f) : acc[i][j], 0, 0, 0);
+          }
+        }
       }
     }
   };
@@ -237,8 +276,9 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void HconvSlabKernel(const Con
   // The walk over one chunk; `first`: the chunk that starts the sums (a type, so that chunk 0 is code of its own)
   auto walk = [&](const int chunk, auto first) {
     constexpr bool FIRST = decltype(first)::value && TAPS > 0;
-    const _Float16* slab = lds + (chunk & 1) * p.slab_halves;
-    const _Float16* kernels_now = ordered + (chunk & 1) * taps * TAP_HALVES;
+    constexpr int PER = HALF ? 1 : 4;  // matrix instructions per pair of 16-byte operands
+    const T* slab = lds + (chunk & 1) * p.slab_elements;
+    const T* kernels_now = ordered + (chunk & 1) * taps * TAP_ELEMENTS;
     // The next chunk's kernels and pieces are asked for between the products of the first tap (TAPS known) - without a
     // test of the chunk, which would end the scheduling region: the last chunk asks for itself again, into the slab and
     // the kernel buffer that nothing reads any more, and the wait at its end keeps these loads out of the epilogue's LDS.
@@ -271,13 +311,13 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void HconvSlabKernel(const Con
           request_kernels(chunk_ahead);
           request(chunk_ahead);
         }
-        fetch(slab + next_tap(), kernels_now + (tap + 1) * TAP_HALVES, set[(tap + 1) % 2]);
+        fetch(slab + next_tap(), kernels_now + (tap + 1) * TAP_ELEMENTS, set[(tap + 1) % 2]);
         if (tap == 0) { products(set[0], std::integral_constant<bool, FIRST>{}); } else { products(set[tap % 2], std::false_type{}); }
         // one read after every matrix instruction: nine reads in a row wait for room in the LDS queue, and the
         // wavefront issues nothing else meanwhile
 #pragma unroll
         for (int i = 0; i < BLOCKS + 2; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one matrix instruction,
+          __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);  // one matrix instruction (fp32: the four of a block),
           __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);  // the address of
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read,
           if (tap == 0) {
@@ -287,7 +327,7 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void HconvSlabKernel(const Con
         }
 #pragma unroll
         for (int i = BLOCKS + 2; i < 2 * BLOCKS; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
           if (tap == 0) {
             __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
             __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
@@ -299,69 +339,100 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void HconvSlabKernel(const Con
       // alone on its SIMD hides nothing that does not stand between matrix instructions). Without a test of the chunk,
       // which would end the scheduling region: after the last chunk the writes repeat the pieces of that chunk in the
       // slab that nothing reads any more.
-      deposit(lds + ((chunk + 1) & 1) * p.slab_halves);
+      deposit(lds + ((chunk + 1) & 1) * p.slab_elements);
       products(set[(TAPS - 1) % 2], std::integral_constant<bool, FIRST && TAPS == 1>{});
 #pragma unroll
       for (int i = 0; i < 2 * BLOCKS; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one matrix instruction,
+        __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);  // one matrix instruction (fp32: four),
         __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);  // two vector ALU instructions,
         __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);  // two LDS writes
       }
       __builtin_amdgcn_sched_barrier(0);
     } else {
       for (int tap = 0; tap < taps; tap += 2) {
-        if (tap + 1 < taps) { fetch(slab + next_tap(), kernels_now + (tap + 1) * TAP_HALVES, set[1]); }
+        if (tap + 1 < taps) { fetch(slab + next_tap(), kernels_now + (tap + 1) * TAP_ELEMENTS, set[1]); }
         __builtin_amdgcn_sched_barrier(0);
         products(set[0], std::false_type{});
         __builtin_amdgcn_sched_barrier(0);
         if (tap + 1 < taps) {
-          if (tap + 2 < taps) { fetch(slab + next_tap(), kernels_now + (tap + 2) * TAP_HALVES, set[0]); }
+          if (tap + 2 < taps) { fetch(slab + next_tap(), kernels_now + (tap + 2) * TAP_ELEMENTS, set[0]); }
           __builtin_amdgcn_sched_barrier(0);
           products(set[1], std::false_type{});
           __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
-    if (TAPS == 0 && chunk + 1 < chunks) { deposit(lds + ((chunk + 1) & 1) * p.slab_halves); }
+    if (TAPS == 0 && chunk + 1 < chunks) { deposit(lds + ((chunk + 1) & 1) * p.slab_elements); }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   };
   walk(0, std::true_type{});
   for (int chunk = 1; chunk < chunks; ++chunk) { walk(chunk, std::false_type{}); }
 
-  // Epilogue: [kernel][pixel] in LDS (every wavefront its own part), then 16-byte stores along the result's rows.
+  const long long pixels = static_cast<long long>(p.output_h) * p.output_w;
+  T* result = p.result + static_cast<long long>(batch) * p.kernels * pixels + static_cast<long long>(row0) * p.output_w;
   // Register r of block (i, j): pixel 32 i + 8 (r / 4) + 4 (lane / 32) + r % 4, kernel 32 j + lane % 32.
-  constexpr int RP = kConvSlabResultPitch;
+  if constexpr (HALF) {
+    // fp16 epilogue: [kernel][pixel] in LDS (every wavefront its own part), then 16-byte stores along the result's rows
+    constexpr int RP = kConvSlabResultPitch;
 #pragma unroll
-  for (int i = 0; i < BLOCKS; ++i) {
+    for (int i = 0; i < BLOCKS; ++i) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          half4_t four;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { four[e] = static_cast<_Float16>(acc[i][j][4 * g + e]); }
+          const int pixel = (wave_m * BLOCKS + i) * 32 + 8 * g + 4 * (lane / 32);
+          const int n = wave_n * 64 + j * 32 + lane % 32;
+          *reinterpret_cast<half4_t*>(lds + n * RP + pixel) = four;
+        }
+      }
+    }
+    __syncthreads();
+    constexpr int ROW_VECTORS = BLOCKS * 32 / 8;  // 16-byte pieces of a kernel's row in this wavefront's part
+#pragma unroll 14
+    for (int t = 0; t < ROW_VECTORS; ++t) {
+      const int q = lane + 64 * t;
+      const int n = wave_n * 64 + q / ROW_VECTORS, pixel = wave_m * BLOCKS * 32 + (q % ROW_VECTORS) * 8;
+      if (n0 + n < p.kernels && pixel < valid_pixels) {
+        const Dwords4 value = *reinterpret_cast<const Dwords4*>(lds + n * RP + pixel);
+        *reinterpret_cast<Dwords4*>(result + (n0 + n) * pixels + pixel) = value;
+      }
+    }
+  } else {
+    // fp32 epilogue: the same in two halves (the kernels of a wavefront's first block of 32, then of its second: 64 rows
+    // of the tile at a time fit LDS). A wavefront writes and reads its own part only.
+    constexpr int RP = kConvSlabPixels + 4;       // floats from a kernel to the next
+    constexpr int ROW_VECTORS = BLOCKS * 32 / 4;  // 16-byte pieces of a kernel's row in this wavefront's part
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        half4_t four;
+      for (int i = 0; i < BLOCKS; ++i) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { four[e] = static_cast<_Float16>(acc[i][j][4 * g + e]); }
-        const int pixel = (wave_m * BLOCKS + i) * 32 + 8 * g + 4 * (lane / 32);
-        const int n = wave_n * 64 + j * 32 + lane % 32;
-        *reinterpret_cast<half4_t*>(lds + n * RP + pixel) = four;
+        for (int g = 0; g < 4; ++g) {
+          Vector four;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { four[e] = acc[i][j][4 * g + e]; }
+          const int pixel = (wave_m * BLOCKS + i) * 32 + 8 * g + 4 * (lane / 32);
+          *reinterpret_cast<Vector*>(lds + (wave_n * 32 + lane % 32) * RP + pixel) = four;
+        }
       }
-    }
-  }
-  __syncthreads();
-  constexpr int ROW_VECTORS = BLOCKS * 32 / 8;  // 16-byte pieces of a kernel's row in this wavefront's part
-  const long long pixels = static_cast<long long>(p.output_h) * p.output_w;
-  _Float16* result = p.result + static_cast<long long>(batch) * p.kernels * pixels + static_cast<long long>(row0) * p.output_w;
 #pragma unroll 14
-  for (int t = 0; t < ROW_VECTORS; ++t) {
-    const int q = lane + 64 * t;
-    const int n = wave_n * 64 + q / ROW_VECTORS, pixel = wave_m * BLOCKS * 32 + (q % ROW_VECTORS) * 8;
-    if (n0 + n < p.kernels && pixel < valid_pixels) {
-      const Dwords4 value = *reinterpret_cast<const Dwords4*>(lds + n * RP + pixel);
-      *reinterpret_cast<Dwords4*>(result + (n0 + n) * pixels + pixel) = value;
+      for (int t = 0; t < ROW_VECTORS / 2; ++t) {
+        const int q = lane + 64 * t;
+        const int row = q / ROW_VECTORS, pixel = wave_m * BLOCKS * 32 + (q % ROW_VECTORS) * 4;
+        const int n = n0 + wave_n * 64 + j * 32 + row;
+        if (n < p.kernels && pixel < valid_pixels) {
+          const Vector value = *reinterpret_cast<const Vector*>(lds + (wave_n * 32 + row) * RP + pixel);
+          *reinterpret_cast<Vector*>(result + n * pixels + pixel) = value;
+        }
+      }
     }
   }
 }
 
 }  // namespace clbh
 
-#endif  // CLBLAST_HIP_KERNELS_CONV_SLAB_F16_HPP_
+#endif  // CLBLAST_HIP_KERNELS_CONV_SLAB_HPP_

@@ -82,19 +82,20 @@ void Xconvgemm<T>::DoConvgemm(const KernelMode kernel_mode, const size_t channel
   // Both element types: images whose patches never reach into padding are what the gathering kernels take without
   // (fp32) or only with (fp16) restrictions; an image with padding is first copied into a border of zeros - one pass
   // over the images instead of a nine times larger im2col matrix.
-  // fp16 with unit strides and no dilation (what the device layer's slab kernel takes): the images as they are, the
-  // padding as zeros in LDS, the kernel matrix through a small copy in the order the kernel reads it
-  if (precision == 16) {
-    const auto scratch_bytes = clbh_conv_slab_scratch_bytes(&shape, static_cast<int>(num_kernels), static_cast<int>(batch_count));
-    const bool aligned = (reinterpret_cast<unsigned long long>(im_buffer()) + 2 * im_offset) % 16 == 0 &&
-                         (reinterpret_cast<unsigned long long>(result_buffer()) + 2 * result_offset) % 16 == 0;
+  // fp16 and fp32 with unit strides and no dilation (what the device layer's slab kernel takes): the images as they
+  // are, the padding as zeros in LDS, the kernel matrix through a small copy in the order the kernel reads it
+  if (precision == 16 || precision == 32) {
+    const auto scratch_bytes =
+        clbh_conv_slab_scratch_bytes(precision, &shape, static_cast<int>(num_kernels), static_cast<int>(batch_count));
+    const bool aligned = (reinterpret_cast<unsigned long long>(im_buffer()) + sizeof(T) * im_offset) % 16 == 0 &&
+                         (reinterpret_cast<unsigned long long>(result_buffer()) + sizeof(T) * result_offset) % 16 == 0;
     if (scratch_bytes > 0 && aligned) {
       const StreamScratch ordered(scratch_bytes, this->stream(), "kernel matrix in k-step order");
-      CheckDevice(clbh_conv_slab_f16(&shape, static_cast<int>(num_kernels), static_cast<int>(batch_count), im_buffer(),
-                                     static_cast<long long>(im_offset), kernel_buffer(), static_cast<long long>(kernel_offset),
-                                     const_cast<void*>(result_buffer()), static_cast<long long>(result_offset), ordered.get(),
-                                     this->stream()),
-                  "clbh_conv_slab_f16");
+      CheckDevice(clbh_conv_slab(precision, &shape, static_cast<int>(num_kernels), static_cast<int>(batch_count), im_buffer(),
+                                 static_cast<long long>(im_offset), kernel_buffer(), static_cast<long long>(kernel_offset),
+                                 const_cast<void*>(result_buffer()), static_cast<long long>(result_offset), ordered.get(),
+                                 this->stream()),
+                  "clbh_conv_slab");
       this->Finish();
       return;
     }

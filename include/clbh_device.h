@@ -240,19 +240,20 @@ CLBH_API int clbh_pad_image(int precision, int images, int channels, int height,
 // an even image width and an output width that is a multiple of 8; not for fp64.
 CLBH_API int clbh_conv_gather_possible(int precision, const clbh_im2col_shape* shape);
 
-// fp16 CONVGEMM without an im2col matrix and without a padded copy of the images (kernels/conv_slab_f16.hpp): a work-group
-// stages the part of an image its output rows touch in LDS, 16 channels at a time, and every kernel tap is a matrix
-// instruction on a shifted view of it. Taken for unit strides, no dilation, a kernel window inside the padded image,
-// channels a multiple of 16, image width and output width multiples of 8, an output width of at most 448, and whole
-// output rows that fill at least half of a 448-pixel tile; images + images_offset, result + result_offset and scratch
-// 16-byte aligned. clbh_conv_slab_scratch_bytes returns 0 for a shape it does not take, else the size of the scratch
-// that receives the kernel matrix in the order the kernel reads it. shape->flip mirrors the taps. Images: batch_count x
-// channels x height x width; weights: kernels x (channels * kernel_h * kernel_w); result: batch_count x kernels x
-// output_h x output_w.
-CLBH_API size_t clbh_conv_slab_scratch_bytes(const clbh_im2col_shape* shape, int kernels, int batch_count);
-CLBH_API int clbh_conv_slab_f16(const clbh_im2col_shape* shape, int kernels, int batch_count, const void* images,
-                                long long images_offset, const void* weights, long long weights_offset, void* result,
-                                long long result_offset, void* scratch, hipStream_t stream);
+// fp16 (precision 16) and fp32 (32) CONVGEMM without an im2col matrix and without a padded copy of the images
+// (kernels/conv_slab.hpp): a work-group stages the part of an image its output rows touch in LDS, 32 bytes of channels
+// per pixel at a time (a chunk: 16 halves, 8 floats), and every kernel tap is a matrix instruction on a shifted view of
+// it. Taken for unit strides, no dilation, a kernel window inside the padded image, channels a multiple of the chunk,
+// image width and output width multiples of 8 (fp32: 4), an output width of at most 448, whole output rows that fill at
+// least half of a 448-pixel tile, and as many taps as fit LDS next to two slabs (4 KiB per tap, twice); images +
+// images_offset, result + result_offset and scratch 16-byte aligned. clbh_conv_slab_scratch_bytes returns 0 for a
+// shape it does not take, else the size of the scratch that receives the kernel matrix in the order the kernel reads it.
+// shape->flip mirrors the taps. Images: batch_count x channels x height x width; weights: kernels x (channels *
+// kernel_h * kernel_w); result: batch_count x kernels x output_h x output_w.
+CLBH_API size_t clbh_conv_slab_scratch_bytes(int precision, const clbh_im2col_shape* shape, int kernels, int batch_count);
+CLBH_API int clbh_conv_slab(int precision, const clbh_im2col_shape* shape, int kernels, int batch_count, const void* images,
+                            long long images_offset, const void* weights, long long weights_offset, void* result,
+                            long long result_offset, void* scratch, hipStream_t stream);
 
 // Plain device memory and blocking copies for callers that hold host data (the Netlib-style façade): to_device != 0
 // copies host -> device, else waits for the default stream's work and copies device -> host.

@@ -89,7 +89,7 @@ def test_convgemm_sweep(gpu, bits):
             problem.check(after)
 
 
-SLAB_CASES = [  # fp16 shapes for the kernel that stages image slabs in LDS: unit strides, 16 | channels, 8 | widths
+SLAB_CASES = [  # shapes for the kernel that stages image slabs in LDS (fp16 and fp32): unit strides, 16 | channels, 8 | widths
     (16, 32, 32, 3, 3, 1, 1, 1, 1, 1, 1, 32, 4),    # three row tiles of 11 rows, the last with 10
     (32, 20, 24, 3, 3, 1, 1, 1, 1, 1, 1, 130, 3),   # two chunks of channels, two tile columns of kernels (the second: 2)
     (16, 9, 40, 5, 1, 2, 0, 1, 1, 1, 1, 20, 2),     # a 5 x 1 window, padding along the height only, one tile per image
@@ -103,7 +103,7 @@ SLAB_CASES = [  # fp16 shapes for the kernel that stages image slabs in LDS: uni
 ]
 
 
-def slab_scratch_bytes(case):
+def slab_scratch_bytes(case, bits=16):
     """What the device layer reports for the case: non-zero when the slab kernel takes it."""
     import ctypes
     from clblast_amd import _lib
@@ -118,26 +118,46 @@ def slab_scratch_bytes(case):
                   oracle.conv_output_extent(width, kernel_w, pad_w, stride_w, dilation_w), 0)
     function = _lib.load().clbh_conv_slab_scratch_bytes
     function.restype = ctypes.c_size_t
-    function.argtypes = [ctypes.POINTER(Shape), ctypes.c_int, ctypes.c_int]
-    return function(ctypes.byref(shape), kernels, batch)
+    function.argtypes = [ctypes.c_int, ctypes.POINTER(Shape), ctypes.c_int, ctypes.c_int]
+    return function(bits, ctypes.byref(shape), kernels, batch)
 
 
-def test_convgemm_fp16_slab_kernel(gpu):
+@pytest.mark.parametrize("bits", (16, 32))
+def test_convgemm_slab_kernel(gpu, bits):
     """The shapes the slab kernel takes (asserted), both modes, with 16-byte aligned offsets (the kernel) and with odd
     ones (the gathering GEMM on the same shape) against the oracle."""
-    seed = 18500
+    seed = 18500 + bits
     for case in SLAB_CASES:
-        assert slab_scratch_bytes(case) == 2 * case[0] * case[3] * case[4] * case[11], case
+        # (fp32 stages twice as many pieces per chunk: the widest of these slabs is beyond what its threads take)
+        expected = 0 if (bits == 32 and case[2] == 160) else (bits // 8) * case[0] * case[3] * case[4] * case[11]
+        assert slab_scratch_bytes(case, bits) == expected, case
         for mode in (CROSS_CORRELATION, CONVOLUTION):
             for offsets in ((0, 0, 0), (16, 7, 24), (10, 6, 14)):
                 seed += 1
-                problem = ConvProblem(16, mode, case, seed, offsets)
+                problem = ConvProblem(bits, mode, case, seed, offsets)
                 status, after = problem.run(gpu)
                 assert status == 0, (status, case)
                 problem.check(after)
     for case in CASES:
         if case != SLAB_CASES[0]:
-            assert slab_scratch_bytes(case) == 0, case
+            assert slab_scratch_bytes(case, 16) == 0, case
+    assert slab_scratch_bytes(SLAB_CASES[0], 64) == 0
+    assert slab_scratch_bytes((8, 12, 20, 3, 3, 1, 1, 1, 1, 1, 1, 9, 2), 32) > 0      # fp32: chunks of 8 channels, widths in fours
+    assert slab_scratch_bytes((8, 12, 20, 3, 3, 1, 1, 1, 1, 1, 1, 9, 2), 16) == 0
+
+
+def test_convgemm_fp32_slab_kernel_shapes_of_its_own(gpu):
+    """fp32 takes chunks of 8 channels and widths that are multiples of 4."""
+    seed = 18700
+    for case in ((8, 12, 20, 3, 3, 1, 1, 1, 1, 1, 1, 9, 2), (24, 20, 28, 3, 3, 1, 1, 1, 1, 1, 1, 130, 2),
+                 (8, 9, 36, 1, 1, 0, 0, 1, 1, 1, 1, 40, 3), (8, 10, 44, 2, 3, 1, 1, 1, 1, 1, 1, 5, 2)):
+        assert slab_scratch_bytes(case, 32) > 0, case
+        for mode in (CROSS_CORRELATION, CONVOLUTION):
+            seed += 1
+            problem = ConvProblem(32, mode, case, seed, ((0, 0, 0), (16, 7, 24))[seed % 2])
+            status, after = problem.run(gpu)
+            assert status == 0, (status, case)
+            problem.check(after)
 
 
 @pytest.mark.parametrize("bits", (32, 16))
