@@ -132,8 +132,13 @@ int LaunchConvSlabTyped(const clbh_im2col_shape& g, const ConvSlabPlan& plan, co
 
 extern "C" {
 
-size_t clbh_conv_slab_scratch_bytes(int precision, const clbh_im2col_shape* shape, int kernels, int batch_count) {
-  if (shape == nullptr || !clbh::PlanConvSlab(precision, *shape, kernels, batch_count).possible) { return 0; }
+size_t clbh_conv_slab_scratch_bytes(int precision, const clbh_im2col_shape* shape, int kernels, int batch_count, int* work_groups,
+                                    int* tile_pixels) {
+  if (shape == nullptr) { return 0; }
+  const auto plan = clbh::PlanConvSlab(precision, *shape, kernels, batch_count);
+  if (!plan.possible) { return 0; }
+  if (work_groups != nullptr) { *work_groups = batch_count * plan.row_tiles * plan.kernel_tiles; }
+  if (tile_pixels != nullptr) { *tile_pixels = plan.rows * shape->output_w; }
   return static_cast<size_t>(shape->channels) * shape->kernel_h * shape->kernel_w * kernels * (precision / 8);
 }
 

@@ -18,6 +18,7 @@ std::mutex override_mutex;
 std::map<std::tuple<int, int>, size_t> min_indirect_overrides;  // (device, precision bits) -> threshold
 std::map<int, size_t> tile_variant_overrides;                   // precision bits -> forced MFMA tile (0 = automatic)
 std::map<int, size_t> split_overrides;                          // precision bits -> K ranges of a forced tile
+std::map<int, size_t> conv_slab_overrides;                      // precision bits -> 1: CONVGEMM's slab kernel whenever possible, 2: never
 
 size_t ForcedSplit(const Precision precision) {
   std::lock_guard<std::mutex> lock(override_mutex);
@@ -723,8 +724,42 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
   return KernelChoice{CLBH_KERNEL_MFMA, 1, (batch_count == 1) ? SplitFor(tiles, k) : 1};
 }
 
+// Measured on 8 images against the GEMM that gathers its patches (fp16 / fp32, slab kernel against that, in us):
+// 128 channels of 56 x 56, 128 kernels of 3 x 3: 28 / 34 and 250 / 98 (56 work-groups); 64 x 224 x 224, 64 kernels, 2
+// images: 27 / 39 and 133 / 96 (half of a tile's kernels); 256 x 56 x 56, 256 kernels of 1 x 1: 31 / 29 and 90 / 43;
+// 512 x 16 x 16, 512 kernels: 83 / 74 (fp16; 256 of a tile's 448 pixels); 64 x 112 x 112, 128 kernels: 23 / 46 and
+// 134 / 160. fp32, where the gathering GEMM runs at 0.6 of the peak, wants a launch that fills the device; fp16, where
+// that GEMM is bound by its address arithmetic, only tiles that are mostly full; one tap leaves a barrier per k-step.
+bool UseConvSlab(const Precision precision, const size_t taps, const size_t kernels, const size_t work_groups,
+                 const size_t tile_pixels, const size_t compute_units) {
+  size_t forced = 0;
+  {
+    std::lock_guard<std::mutex> lock(override_mutex);
+    const auto found = conv_slab_overrides.find(static_cast<int>(precision));
+    if (found != conv_slab_overrides.end()) { forced = found->second; }
+  }
+  if (forced == 1) { return true; }
+  if (forced == 2 || taps < 2 || work_groups == 0 || compute_units == 0) { return false; }
+  const auto fill = static_cast<double>(tile_pixels) / 448.0;
+  if (precision == Precision::kHalf) { return fill >= 0.75; }
+  const auto rounds = CeilDivide(work_groups, compute_units);
+  const auto kernel_tiles = CeilDivide(kernels, 128);
+  const auto use = static_cast<double>(work_groups) / static_cast<double>(rounds * compute_units) * fill *
+                   static_cast<double>(kernels) / static_cast<double>(kernel_tiles * 128);
+  return use >= 0.7;
+}
+
 StatusCode OverrideRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,
                                      const std::unordered_map<std::string, size_t>& parameters) {
+  if (kernel_name == "Xconvgemm") {  // SLAB: 0 = by rule, 1 = the slab kernel whenever it can run, 2 = never
+    const auto slab = parameters.find("SLAB");
+    if (slab == parameters.end()) {
+      return StatusCode::kMissingOverrideParameter;
+    }
+    std::lock_guard<std::mutex> lock(override_mutex);
+    conv_slab_overrides[static_cast<int>(precision)] = slab->second;
+    return StatusCode::kSuccess;
+  }
   if (kernel_name == "Xgemm") {  // forces one tile of the MFMA family: TILE_VARIANT = 1 + index, 0 = automatic
     const auto variant = parameters.find("TILE_VARIANT");
     if (variant == parameters.end()) {
@@ -750,6 +785,12 @@ StatusCode OverrideRoutineParameters(const int device, const std::string& kernel
 
 StatusCode RetrieveRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,
                                      std::unordered_map<std::string, size_t>& parameters) {
+  if (kernel_name == "Xconvgemm") {
+    std::lock_guard<std::mutex> lock(override_mutex);
+    const auto found = conv_slab_overrides.find(static_cast<int>(precision));
+    parameters["SLAB"] = (found != conv_slab_overrides.end()) ? found->second : 0;
+    return StatusCode::kSuccess;
+  }
   if (kernel_name == "Xgemm") {
     parameters["TILE_VARIANT"] = ForcedTileVariant(precision);
     parameters["SPLIT_K"] = ForcedSplit(precision);
@@ -767,6 +808,7 @@ void ClearOverrides() {
   min_indirect_overrides.clear();
   tile_variant_overrides.clear();
   split_overrides.clear();
+  conv_slab_overrides.clear();
 }
 
 }  // namespace clblast

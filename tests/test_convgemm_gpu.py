@@ -118,8 +118,8 @@ def slab_scratch_bytes(case, bits=16):
                   oracle.conv_output_extent(width, kernel_w, pad_w, stride_w, dilation_w), 0)
     function = _lib.load().clbh_conv_slab_scratch_bytes
     function.restype = ctypes.c_size_t
-    function.argtypes = [ctypes.c_int, ctypes.POINTER(Shape), ctypes.c_int, ctypes.c_int]
-    return function(bits, ctypes.byref(shape), kernels, batch)
+    function.argtypes = [ctypes.c_int, ctypes.POINTER(Shape), ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    return function(bits, ctypes.byref(shape), kernels, batch, None, None)
 
 
 @pytest.mark.parametrize("bits", (16, 32))
@@ -127,6 +127,20 @@ def test_convgemm_slab_kernel(gpu, bits):
     """The shapes the slab kernel takes (asserted), both modes, with 16-byte aligned offsets (the kernel) and with odd
     ones (the gathering GEMM on the same shape) against the oracle."""
     seed = 18500 + bits
+    clblast_amd.override_parameters(0, "Xconvgemm", bits, {"SLAB": 1})  # whenever it can run (small shapes would not take it)
+    try:
+        _slab_cases(gpu, bits, seed)
+    finally:
+        clblast_amd.override_parameters(0, "Xconvgemm", bits, {"SLAB": 0})
+    for case in CASES:
+        if case != SLAB_CASES[0]:
+            assert slab_scratch_bytes(case, 16) == 0, case
+    assert slab_scratch_bytes(SLAB_CASES[0], 64) == 0
+    assert slab_scratch_bytes((8, 12, 20, 3, 3, 1, 1, 1, 1, 1, 1, 9, 2), 32) > 0      # fp32: chunks of 8 channels, widths in fours
+    assert slab_scratch_bytes((8, 12, 20, 3, 3, 1, 1, 1, 1, 1, 1, 9, 2), 16) == 0
+
+
+def _slab_cases(gpu, bits, seed):
     for case in SLAB_CASES:
         # (fp32 stages twice as many pieces per chunk: the widest of these slabs is beyond what its threads take)
         expected = 0 if (bits == 32 and case[2] == 160) else (bits // 8) * case[0] * case[3] * case[4] * case[11]
@@ -138,16 +152,37 @@ def test_convgemm_slab_kernel(gpu, bits):
                 status, after = problem.run(gpu)
                 assert status == 0, (status, case)
                 problem.check(after)
-    for case in CASES:
-        if case != SLAB_CASES[0]:
-            assert slab_scratch_bytes(case, 16) == 0, case
-    assert slab_scratch_bytes(SLAB_CASES[0], 64) == 0
-    assert slab_scratch_bytes((8, 12, 20, 3, 3, 1, 1, 1, 1, 1, 1, 9, 2), 32) > 0      # fp32: chunks of 8 channels, widths in fours
-    assert slab_scratch_bytes((8, 12, 20, 3, 3, 1, 1, 1, 1, 1, 1, 9, 2), 16) == 0
 
 
 def test_convgemm_fp32_slab_kernel_shapes_of_its_own(gpu):
     """fp32 takes chunks of 8 channels and widths that are multiples of 4."""
+    clblast_amd.override_parameters(0, "Xconvgemm", 32, {"SLAB": 1})
+    try:
+        _fp32_cases(gpu)
+    finally:
+        clblast_amd.override_parameters(0, "Xconvgemm", 32, {"SLAB": 0})
+
+
+def test_convgemm_slab_rule_and_override(gpu):
+    """The rule takes the slab kernel for the shape of the bench and not for a launch of few work-groups in fp32; SLAB = 2
+    switches it off: both paths give the convolution, bit-identical results are not asked of them."""
+    case = (16, 32, 32, 3, 3, 1, 1, 1, 1, 1, 1, 32, 4)
+    for bits in (16, 32):
+        for setting in (2, 1, 0):
+            clblast_amd.override_parameters(0, "Xconvgemm", bits, {"SLAB": setting})
+            try:
+                problem = ConvProblem(bits, CROSS_CORRELATION, case, 18800 + setting, (0, 0, 0))
+                status, after = problem.run(gpu)
+                assert status == 0
+                problem.check(after)
+            finally:
+                clblast_amd.override_parameters(0, "Xconvgemm", bits, {"SLAB": 0})
+    with pytest.raises(clblast_amd.CLBlastError) as missing:
+        clblast_amd.override_parameters(0, "Xconvgemm", 32, {"OTHER": 1})
+    assert missing.value.status == -2047  # kMissingOverrideParameter
+
+
+def _fp32_cases(gpu):
     seed = 18700
     for case in ((8, 12, 20, 3, 3, 1, 1, 1, 1, 1, 1, 9, 2), (24, 20, 28, 3, 3, 1, 1, 1, 1, 1, 1, 130, 2),
                  (8, 9, 36, 1, 1, 0, 0, 1, 1, 1, 1, 40, 3), (8, 10, 44, 2, 3, 1, 1, 1, 1, 1, 1, 5, 2)):
