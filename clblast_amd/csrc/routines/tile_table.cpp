@@ -729,7 +729,8 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
 // images: 27 / 39 and 133 / 96 (half of a tile's kernels); 256 x 56 x 56, 256 kernels of 1 x 1: 31 / 29 and 90 / 43;
 // 512 x 16 x 16, 512 kernels: 83 / 74 (fp16; 256 of a tile's 448 pixels); 64 x 112 x 112, 128 kernels: 23 / 46 and
 // 134 / 160. fp32, where the gathering GEMM runs at 0.6 of the peak, wants a launch that fills the device; fp16, where
-// that GEMM is bound by its address arithmetic, only tiles that are mostly full; one tap leaves a barrier per k-step.
+// that GEMM is bound by its address arithmetic, tiles that are mostly full and a launch that is not tiny; one tap leaves a
+// barrier per k-step.
 bool UseConvSlab(const Precision precision, const size_t taps, const size_t kernels, const size_t work_groups,
                  const size_t tile_pixels, const size_t compute_units) {
   size_t forced = 0;
@@ -741,11 +742,14 @@ bool UseConvSlab(const Precision precision, const size_t taps, const size_t kern
   if (forced == 1) { return true; }
   if (forced == 2 || taps < 2 || work_groups == 0 || compute_units == 0) { return false; }
   const auto fill = static_cast<double>(tile_pixels) / 448.0;
-  if (precision == Precision::kHalf) { return fill >= 0.75; }
   const auto rounds = CeilDivide(work_groups, compute_units);
   const auto kernel_tiles = CeilDivide(kernels, 128);
   const auto use = static_cast<double>(work_groups) / static_cast<double>(rounds * compute_units) * fill *
                    static_cast<double>(kernels) / static_cast<double>(kernel_tiles * 128);
+  // (fp16 on few work-groups: 64 x 56 x 56, 64 kernels, 2 images - 14 work-groups, half of a tile's kernels - 18 against
+  // 13 us; 256 x 56 x 56, 64 kernels, 4 images 45 against 34 us; from 0.2 on the slab kernel is ahead: 2 images of
+  // 64 x 112 x 112 with 128 kernels 19 against 21 us, 4 images 21 against 28 us)
+  if (precision == Precision::kHalf) { return fill >= 0.75 && use >= 0.15; }
   return use >= 0.7;
 }
 
