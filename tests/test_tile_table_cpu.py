@@ -43,3 +43,20 @@ def test_the_plan_of_the_persistent_fp16_kernel(tmp_path):
     run = subprocess.run([str(binary)], capture_output=True, text=True)
     assert run.returncode == 0, run.stdout[-3000:]
     assert "violations 0" in run.stdout
+
+
+def test_the_rule_for_the_slab_kernel_of_convgemm(tmp_path):
+    """Which CONVGEMM calls go to the kernel that stages image slabs in LDS: the measured shapes and the override."""
+    compiler = shutil.which("g++")
+    if compiler is None:
+        pytest.skip("no g++ here")
+    binary = tmp_path / "rule"
+    sources = [os.path.join(ROOT, "tests", "host", "conv_slab_rule.cpp"),
+               os.path.join(ROOT, "clblast_amd", "csrc", "routines", "tile_table.cpp")]
+    done = subprocess.run([compiler, "-std=c++17", "-O1", "-I" + os.path.join(ROOT, "include"),
+                           "-I" + os.path.join(ROOT, "clblast_amd", "csrc")] + sources + ["-o", str(binary)],
+                          capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr[-3000:]
+    run = subprocess.run([str(binary)], capture_output=True, text=True)
+    assert run.returncode == 0, run.stdout[-3000:]
+    assert "violations 0" in run.stdout
