@@ -7,6 +7,7 @@
 #define CLBLAST_HIP_DEVICE_LAUNCH_PLANS_HPP_
 
 #include <algorithm>
+#include <climits>
 #include <cstddef>
 
 #include "clbh_device.h"
@@ -98,6 +99,69 @@ inline WidePlan PlanWide(const clbh_gemm_desc& d) {
       }
     }
   }
+  return plan;
+}
+
+// ---- CONVGEMM: the kernel that stages image slabs in LDS (kernels/conv_slab.hpp) -------------------------------
+// Its tile: 448 output pixels (whole output rows of one image) x 128 kernels on four wavefronts of 224 x 64.
+constexpr int kConvSlabThreads = 256;
+constexpr int kConvSlabPixelBytes = 48;    // from a pixel to the next in a slab (32 bytes of channels + 16: no bank conflicts)
+constexpr int kConvSlabBlocks = 7;         // 32-pixel blocks per wavefront
+constexpr int kConvSlabPixels = 2 * kConvSlabBlocks * 32;  // 448 per work-group
+constexpr int kConvSlabKernels = 128;      // per work-group
+constexpr int kConvSlabResultPitch = kConvSlabPixels + 8;  // halves from a kernel to the next in the fp16 epilogue's tile
+constexpr int kConvSlabResultBytes = kConvSlabKernels * kConvSlabResultPitch * 2;
+constexpr int kConvSlabResultBytesF32 = (kConvSlabKernels / 2) * (kConvSlabPixels + 4) * 4;  // half of the tile at a time
+constexpr int kConvSlabLdsBytes = 160 * 1024;
+
+struct ConvSlabPlan {
+  bool possible;
+  int rows, row_tiles, kernel_tiles, slab_rows, slab_width, slab_elements, spare_at, tasks;
+  size_t lds_bytes;
+};
+
+// Unit strides, no dilation, the kernel window inside the padded image, 16 channels per chunk, image rows and result
+// rows in 16-byte pieces, a tile of whole output rows that fills at least half of the 448 pixels, two slabs in LDS.
+inline ConvSlabPlan PlanConvSlab(const int precision, const clbh_im2col_shape& g, const int kernels, const int batch_count) {
+  if (precision != 16 && precision != 32) { return ConvSlabPlan{}; }
+  const int element = precision / 8, chunk = 32 / element, piece = 16 / element, pitch = kConvSlabPixelBytes / element;
+  ConvSlabPlan plan = {};
+  if (g.channels <= 0 || g.height <= 0 || g.width <= 0 || g.kernel_h <= 0 || g.kernel_w <= 0 || g.pad_h < 0 || g.pad_w < 0 ||
+      g.output_h <= 0 || g.output_w <= 0 || kernels <= 0 || batch_count <= 0) {
+    return plan;
+  }
+  if (g.stride_h != 1 || g.stride_w != 1 || g.dilation_h != 1 || g.dilation_w != 1) { return plan; }
+  if (g.channels % chunk != 0 || g.width % piece != 0 || g.output_w % piece != 0 || g.output_w > kConvSlabPixels) { return plan; }
+  // the output extents as the routine computes them, without its clamp to 1
+  if (g.output_h != g.height + 2ll * g.pad_h - g.kernel_h + 1 || g.output_w != g.width + 2ll * g.pad_w - g.kernel_w + 1) { return plan; }
+  const long long pixels = static_cast<long long>(g.output_h) * g.output_w;
+  const long long plane = static_cast<long long>(g.height) * g.width;
+  const long long taps = static_cast<long long>(g.kernel_h) * g.kernel_w;
+  if (pixels * kernels >= INT_MAX || plane * chunk >= INT_MAX || taps * g.channels * kernels >= INT_MAX / 4) { return plan; }
+  const int most_rows = std::min(g.output_h, kConvSlabPixels / g.output_w);
+  plan.row_tiles = (g.output_h + most_rows - 1) / most_rows;
+  plan.rows = (g.output_h + plan.row_tiles - 1) / plan.row_tiles;
+  if (2 * plan.rows * g.output_w < kConvSlabPixels) { return plan; }
+  plan.kernel_tiles = (kernels + kConvSlabKernels - 1) / kConvSlabKernels;
+  if (static_cast<long long>(batch_count) * plan.row_tiles * plan.kernel_tiles > INT_MAX) { return plan; }
+  plan.slab_rows = plan.rows + g.kernel_h - 1;
+  // (a slab row 8 x (an odd number) banks of LDS from the next: the kernel's writes of a chunk's pieces then fall on
+  // different banks)
+  long long slab_width = g.width + 2ll * g.pad_w;
+  while (slab_width % 4 != 2) { ++slab_width; }
+  const long long slab_elements = (plan.slab_rows * slab_width + 8) * pitch;  // and a spare strip of 8 pixels
+  // the furthest LDS read: the last tile pixel at the last tap, inside the slab by construction; two slabs and two
+  // chunks of the tile's kernels (taps x 128 kernels x 16 channels each) must fit
+  const long long walk_bytes = 2 * slab_elements * element + 2ll * taps * kConvSlabKernels * 32;
+  if (walk_bytes > kConvSlabLdsBytes) { return plan; }
+  plan.slab_width = static_cast<int>(slab_width);
+  plan.slab_elements = static_cast<int>(slab_elements);
+  plan.spare_at = static_cast<int>(plan.slab_rows * slab_width * pitch);
+  const int pieces = 8 * plan.slab_rows * (g.width / piece);
+  plan.tasks = (pieces + kConvSlabThreads - 1) / kConvSlabThreads;
+  if (plan.tasks > 7) { return plan; }
+  plan.lds_bytes = std::max<size_t>(static_cast<size_t>(walk_bytes), precision == 16 ? kConvSlabResultBytes : kConvSlabResultBytesF32);
+  plan.possible = true;
   return plan;
 }
 

@@ -39,13 +39,12 @@
 
 #include <type_traits>
 
+#include "device/launch_plans.hpp"
 #include "kernels/gemm_mfma.hpp"
 #include "kernels/gemm_mfma_f16.hpp"
 
 namespace clbh {
 
-constexpr int kConvSlabThreads = 256;
-constexpr int kConvSlabPixelBytes = 48;    // from a pixel to the next in a slab (32 bytes of channels + 16: no bank conflicts)
 template <typename T>
 struct ConvSlabType {
   static constexpr int CHUNK = 32 / sizeof(T);                   // channels per chunk: 32 bytes per pixel (16 halves, 8 floats)
@@ -54,12 +53,6 @@ struct ConvSlabType {
   static constexpr int PLANES = sizeof(T) == 2 ? 2 : 1;          // channels a staged piece covers (fp16: a pair, one dword per pixel)
   typedef T Vector __attribute__((ext_vector_type(16 / sizeof(T))));  // a 16-byte operand
 };
-constexpr int kConvSlabBlocks = 7;         // 32-pixel blocks per wavefront
-constexpr int kConvSlabPixels = 2 * kConvSlabBlocks * 32;  // 448 per work-group
-constexpr int kConvSlabKernels = 128;      // per work-group
-constexpr int kConvSlabResultPitch = kConvSlabPixels + 8;  // halves from a kernel to the next in the fp16 epilogue's tile
-constexpr int kConvSlabResultBytes = kConvSlabKernels * kConvSlabResultPitch * 2;
-constexpr int kConvSlabResultBytesF32 = (kConvSlabKernels / 2) * (kConvSlabPixels + 4) * 4;  // half of the tile at a time
 
 template <typename T>
 struct ConvSlabArgs {

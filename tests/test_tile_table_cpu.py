@@ -60,3 +60,19 @@ def test_the_rule_for_the_slab_kernel_of_convgemm(tmp_path):
     run = subprocess.run([str(binary)], capture_output=True, text=True)
     assert run.returncode == 0, run.stdout[-3000:]
     assert "violations 0" in run.stdout
+
+
+def test_the_plan_of_the_slab_kernel_of_convgemm(tmp_path):
+    """The launch plan of CONVGEMM's slab kernel is host code without HIP: over a sweep of shapes, what the kernel reads and
+    writes in LDS lies inside the allocation, the tiles cover the output rows once, the staging fits the kernel's instances."""
+    compiler = shutil.which("g++")
+    if compiler is None:
+        pytest.skip("no g++ here")
+    binary = tmp_path / "convplan"
+    done = subprocess.run([compiler, "-std=c++17", "-O1", "-I" + os.path.join(ROOT, "include"),
+                           "-I" + os.path.join(ROOT, "clblast_amd", "csrc"), os.path.join(ROOT, "tests", "host", "conv_slab_plan_sweep.cpp"),
+                           "-o", str(binary)], capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr[-3000:]
+    run = subprocess.run([str(binary)], capture_output=True, text=True)
+    assert run.returncode == 0, run.stdout[-3000:]
+    assert "violations 0" in run.stdout
