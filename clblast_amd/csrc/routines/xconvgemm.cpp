@@ -76,14 +76,12 @@ void Xconvgemm<T>::DoConvgemm(const KernelMode kernel_mode, const size_t channel
   shape.output_w = static_cast<int>(output_w);
   shape.flip = (kernel_mode == KernelMode::kConvolution) ? 1 : 0;
 
-  // The reference's single-kernel method (xconvgemm.cpp:121-160, doc/details_conv.md): no im2col matrix; the GEMM kernel
-  // gathers the patches from the images while it loads its tiles. fp32 and (with restrictions) fp16, all batches in one
-  // launch.
-  // Both element types: images whose patches never reach into padding are what the gathering kernels take without
-  // (fp32) or only with (fp16) restrictions; an image with padding is first copied into a border of zeros - one pass
-  // over the images instead of a nine times larger im2col matrix.
-  // fp16 and fp32 with unit strides and no dilation (what the device layer's slab kernel takes): the images as they
-  // are, the padding as zeros in LDS, the kernel matrix through a small copy in the order the kernel reads it
+  // The reference's single-kernel method (xconvgemm.cpp:121-160, doc/details_conv.md) computes the convolution without an
+  // im2col matrix. Two forms of it here, all batches in one launch each.
+  //
+  // First form, fp16 and fp32 with unit strides and no dilation (what the device layer's slab kernel can run), where the
+  // tile table's rule finds the launch worthwhile (UseConvSlab): the images as they are, the padding as zeros in LDS,
+  // the kernel matrix through a small copy in the order the kernel reads it.
   if (precision == 16 || precision == 32) {
     int work_groups = 0, tile_pixels = 0, compute_units = 0;
     const auto scratch_bytes = clbh_conv_slab_scratch_bytes(precision, &shape, static_cast<int>(num_kernels),
@@ -105,6 +103,10 @@ void Xconvgemm<T>::DoConvgemm(const KernelMode kernel_mode, const size_t channel
     }
   }
 
+  // Second form: the GEMM kernel gathers the patches from the images while it loads its tiles. Images whose patches never
+  // reach into padding are what the gathering kernels take without (fp32) or only with (fp16) restrictions; an image
+  // with padding is first copied into a border of zeros - one pass over the images instead of a nine times larger
+  // im2col matrix.
   auto padded_shape = shape;
   const auto extra_w = (precision == 16) ? (width + 2 * pad_w) % 2 : size_t{0};  // fp16 wants an even image width
   padded_shape.height = static_cast<int>(height + 2 * pad_h);
