@@ -14,9 +14,9 @@
 namespace clbh {
 namespace {
 
-template <typename T, int TASKS, int TAPS>
+template <typename T, int TASKS, int TAPS, int J>
 int LaunchConvSlab(const ConvSlabArgs<T>& args, const unsigned blocks, const size_t lds_bytes, hipStream_t stream) {
-  auto kernel = ConvSlabKernel<T, TASKS, TAPS>;
+  auto kernel = ConvSlabKernel<T, TASKS, TAPS, J>;
   static const hipError_t attribute_status =
       hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kConvSlabLdsBytes);
   if (attribute_status != hipSuccess) { return static_cast<int>(attribute_status); }
@@ -63,15 +63,20 @@ int LaunchConvSlabTyped(const clbh_im2col_shape& g, const ConvSlabPlan& plan, co
   args.slab_elements = plan.slab_elements;
   args.spare_at = plan.spare_at;
   const auto blocks = static_cast<unsigned>(batch_count * plan.row_tiles * plan.kernel_tiles);
-  const auto launch = [&](auto tasks_tag) {
-    constexpr int TASKS = decltype(tasks_tag)::value;
+  const auto launch = [&](auto tasks_tag, auto blocks_tag) {
+    constexpr int TASKS = decltype(tasks_tag)::value, J = decltype(blocks_tag)::value;
     switch (taps) {
-      case 1: return LaunchConvSlab<T, TASKS, 1>(args, blocks, plan.lds_bytes, stream);
-      case 9: return LaunchConvSlab<T, TASKS, 9>(args, blocks, plan.lds_bytes, stream);
-      default: return LaunchConvSlab<T, TASKS, 0>(args, blocks, plan.lds_bytes, stream);
+      case 1: return LaunchConvSlab<T, TASKS, 1, J>(args, blocks, plan.lds_bytes, stream);
+      case 9: return LaunchConvSlab<T, TASKS, 9, J>(args, blocks, plan.lds_bytes, stream);
+      default: return LaunchConvSlab<T, TASKS, 0, J>(args, blocks, plan.lds_bytes, stream);
     }
   };
-  return (plan.tasks <= 3) ? launch(std::integral_constant<int, 3>{}) : launch(std::integral_constant<int, 7>{});
+  if (plan.kernel_blocks == 1) {
+    return (plan.tasks <= 3) ? launch(std::integral_constant<int, 3>{}, std::integral_constant<int, 1>{})
+                             : launch(std::integral_constant<int, 7>{}, std::integral_constant<int, 1>{});
+  }
+  return (plan.tasks <= 3) ? launch(std::integral_constant<int, 3>{}, std::integral_constant<int, 2>{})
+                           : launch(std::integral_constant<int, 7>{}, std::integral_constant<int, 2>{});
 }
 
 }  // namespace
@@ -80,11 +85,12 @@ int LaunchConvSlabTyped(const clbh_im2col_shape& g, const ConvSlabPlan& plan, co
 extern "C" {
 
 size_t clbh_conv_slab_scratch_bytes(int precision, const clbh_im2col_shape* shape, int kernels, int batch_count, int* work_groups,
-                                    int* tile_pixels) {
+                                    int* tile_pixels, int* tile_kernels) {
   if (shape == nullptr) { return 0; }
   const auto plan = clbh::PlanConvSlab(precision, *shape, kernels, batch_count);
   if (!plan.possible) { return 0; }
   if (work_groups != nullptr) { *work_groups = batch_count * plan.row_tiles * plan.kernel_tiles; }
+  if (tile_kernels != nullptr) { *tile_kernels = 64 * plan.kernel_blocks; }
   if (tile_pixels != nullptr) { *tile_pixels = plan.rows * shape->output_w; }
   return static_cast<size_t>(shape->channels) * shape->kernel_h * shape->kernel_w * kernels * (precision / 8);
 }

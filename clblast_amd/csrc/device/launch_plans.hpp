@@ -108,7 +108,7 @@ constexpr int kConvSlabThreads = 256;
 constexpr int kConvSlabPixelBytes = 48;    // from a pixel to the next in a slab (32 bytes of channels + 16: no bank conflicts)
 constexpr int kConvSlabBlocks = 7;         // 32-pixel blocks per wavefront
 constexpr int kConvSlabPixels = 2 * kConvSlabBlocks * 32;  // 448 per work-group
-constexpr int kConvSlabKernels = 128;      // per work-group
+constexpr int kConvSlabKernels = 128;      // per work-group (64 for calls with at most 64 kernels: ConvSlabPlan::kernel_blocks = 1)
 constexpr int kConvSlabResultPitch = kConvSlabPixels + 8;  // halves from a kernel to the next in the fp16 epilogue's tile
 constexpr int kConvSlabResultBytes = kConvSlabKernels * kConvSlabResultPitch * 2;
 constexpr int kConvSlabResultBytesF32 = (kConvSlabKernels / 2) * (kConvSlabPixels + 4) * 4;  // half of the tile at a time
@@ -117,6 +117,7 @@ constexpr int kConvSlabLdsBytes = 160 * 1024;
 struct ConvSlabPlan {
   bool possible;
   int rows, row_tiles, kernel_tiles, slab_rows, slab_width, slab_elements, spare_at, tasks;
+  int kernel_blocks;  // blocks of 32 kernels per wavefront: 2 (tiles of 128 kernels), or 1 (64) for at most 64 kernels
   size_t lds_bytes;
 };
 
@@ -142,7 +143,9 @@ inline ConvSlabPlan PlanConvSlab(const int precision, const clbh_im2col_shape& g
   plan.row_tiles = (g.output_h + most_rows - 1) / most_rows;
   plan.rows = (g.output_h + plan.row_tiles - 1) / plan.row_tiles;
   if (2 * plan.rows * g.output_w < kConvSlabPixels) { return plan; }
-  plan.kernel_tiles = (kernels + kConvSlabKernels - 1) / kConvSlabKernels;
+  plan.kernel_blocks = (kernels <= kConvSlabKernels / 2) ? 1 : 2;
+  const int tile_kernels = 64 * plan.kernel_blocks;
+  plan.kernel_tiles = (kernels + tile_kernels - 1) / tile_kernels;
   if (static_cast<long long>(batch_count) * plan.row_tiles * plan.kernel_tiles > INT_MAX) { return plan; }
   plan.slab_rows = plan.rows + g.kernel_h - 1;
   // (a slab row 8 x (an odd number) banks of LDS from the next: the kernel's writes of a chunk's pieces then fall on
@@ -152,7 +155,7 @@ inline ConvSlabPlan PlanConvSlab(const int precision, const clbh_im2col_shape& g
   const long long slab_elements = (plan.slab_rows * slab_width + 8) * pitch;  // and a spare strip of 8 pixels
   // the furthest LDS read: the last tile pixel at the last tap, inside the slab by construction; two slabs and two
   // chunks of the tile's kernels (taps x 128 kernels x 16 channels each) must fit
-  const long long walk_bytes = 2 * slab_elements * element + 2ll * taps * kConvSlabKernels * 32;
+  const long long walk_bytes = 2 * slab_elements * element + 2ll * taps * tile_kernels * 32;
   if (walk_bytes > kConvSlabLdsBytes) { return plan; }
   plan.slab_width = static_cast<int>(slab_width);
   plan.slab_elements = static_cast<int>(slab_elements);

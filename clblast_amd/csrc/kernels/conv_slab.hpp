@@ -65,7 +65,7 @@ struct ConvSlabArgs {
   int kernels;
   int rows;          // output rows per tile; rows * output_w <= kConvSlabPixels
   int row_tiles;     // ceil(output_h / rows)
-  int kernel_tiles;  // ceil(kernels / kConvSlabKernels)
+  int kernel_tiles;  // ceil(kernels / (64 J))
   int slab_rows, slab_width;  // rows + kernel_h - 1, width + 2 pad_w
   int slab_elements;          // (slab_rows * slab_width + 8) * PITCH
   int spare_at;               // elements from a slab's start to its last 8 pixels, a strip that no product reads
@@ -100,8 +100,10 @@ __global__ __launch_bounds__(256) void ConvPermuteKernel(const T* __restrict__ w
 // matrix, or kConvSlabResultBytes where that is more.
 // TASKS: 16-byte pieces of the slab (fp16: of two channels each) a thread stages per chunk, at least
 // ceil(8 * slab_rows * (width / PIECE) / 256). TAPS: kernel_h * kernel_w as a constant (the walk over the taps is then
-// straight-line code), or 0 for any number of taps.
-template <typename T, int TASKS, int TAPS>
+// straight-line code), or 0 for any number of taps. J: blocks of 32 kernels per wavefront - 2: the tile of 128 kernels
+// described above; 1: a tile of 64 kernels (wavefronts of 224 pixels x 32 kernels) for calls with at most 64 kernels,
+// which would leave half of the large tile's matrix instructions without use.
+template <typename T, int TASKS, int TAPS, int J>
 __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const ConvSlabArgs<T> p) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
@@ -110,7 +112,8 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const Conv
   using Vector = typename Type::Vector;
   constexpr bool HALF = sizeof(T) == 2;
   constexpr int CHUNK = Type::CHUNK, PITCH = Type::PITCH, PIECE = Type::PIECE, PLANES = Type::PLANES, BLOCKS = kConvSlabBlocks;
-  constexpr int TAP_ELEMENTS = kConvSlabKernels * CHUNK;  // the tile's part of the kernel matrix for one tap (4 KiB)
+  constexpr int KERNELS = 64 * J;                // of the tile
+  constexpr int TAP_ELEMENTS = KERNELS * CHUNK;  // the tile's part of the kernel matrix for one tap (2 or 4 KiB)
 
   const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int wave_m = wave % 2, wave_n = wave / 2;
@@ -121,7 +124,7 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const Conv
   const int batch = block / p.row_tiles;
   const int row0 = row_tile * p.rows;
   const int valid_pixels = min(p.rows, p.output_h - row0) * p.output_w;
-  const int n0 = kernel_tile * kConvSlabKernels;
+  const int n0 = kernel_tile * KERNELS;
   const int plane = p.height * p.width;
   const int taps = TAPS > 0 ? TAPS : p.kernel_h * p.kernel_w;
   const int chunks = p.channels / CHUNK;
@@ -182,13 +185,13 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const Conv
     typedef __attribute__((address_space(3))) void* LdsPtr;
     const T* from = p.weights + n0 * CHUNK;
     const auto view = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(from), 0, ordered_bytes_left, kRawBufferFlags);
-    T* to = ordered + (chunk & 1) * taps * TAP_ELEMENTS + wave * (TAP_ELEMENTS / 4);
+    T* to = ordered + (chunk & 1) * taps * TAP_ELEMENTS + wave * (1024 / static_cast<int>(sizeof(T)));
     int lane_bytes = chunk * taps * tap_bytes + wave * 1024 + lane * 16;  // (the range check covers this offset only)
     for (int tap = 0; tap < taps; ++tap) {
       // (device pass only: with a pointer of a dependent type here, hipcc's host pass drops the kernel's launch stub
       // without a diagnostic and the library fails to link)
 #if defined(__HIP_DEVICE_COMPILE__)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(view, (LdsPtr)(to), 16, lane_bytes, 0, 0, 0);
+      if (wave < 2 * J) { __builtin_amdgcn_raw_ptr_buffer_load_lds(view, (LdsPtr)(to), 16, lane_bytes, 0, 0, 0); }  // (1 KiB = 32 kernels each)
 #endif
       to += TAP_ELEMENTS;
       lane_bytes += tap_bytes;
@@ -211,17 +214,17 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const Conv
     pixel_at[i] = (row * p.slab_width + (pixel - row * p.output_w)) * PITCH + PIECE * (lane / 32);
   }
   // This lane's kernels in a tap's part of the ordered kernel matrix
-  int kernel_at[2];
+  int kernel_at[J];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) { kernel_at[j] = (wave_n * 64 + j * 32 + lane % 32) * CHUNK + PIECE * (lane / 32); }
+  for (int j = 0; j < J; ++j) { kernel_at[j] = (wave_n * 32 * J + j * 32 + lane % 32) * CHUNK + PIECE * (lane / 32); }
 
   // (with TAPS known the first tap of the first chunk takes 0 as its addend instead: 224 register writes less)
-  float16_t acc[BLOCKS][2];
+  float16_t acc[BLOCKS][J];
   if (TAPS == 0) {
 #pragma unroll
     for (int i = 0; i < BLOCKS; ++i) {
-      acc[i][0] = float16_t(0.0f);
-      acc[i][1] = float16_t(0.0f);
+#pragma unroll
+      for (int j = 0; j < J; ++j) { acc[i][j] = float16_t(0.0f); }
     }
   }
 
@@ -232,12 +235,12 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const Conv
 
   // One set of operands: the pixels' 16 channels at a tap and the kernels' 16 channels at that tap
   struct Operands {
-    Vector pixels[BLOCKS], kernels[2];
+    Vector pixels[BLOCKS], kernels[J];
   };
   auto fetch = [&](const T* slab_at_tap, const T* kernels_at_tap, Operands& set) {
     // (in the order of their first use: the reads are spread over the products of the tap before)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) { set.kernels[j] = *reinterpret_cast<const Vector*>(kernels_at_tap + kernel_at[j]); }
+    for (int j = 0; j < J; ++j) { set.kernels[j] = *reinterpret_cast<const Vector*>(kernels_at_tap + kernel_at[j]); }
 #pragma unroll
     for (int i = 0; i < BLOCKS; ++i) { set.pixels[i] = *reinterpret_cast<const Vector*>(slab_at_tap + pixel_at[i]); }
   };
@@ -246,7 +249,7 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const Conv
 #pragma unroll
       for (int i = 0; i < BLOCKS; ++i) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < J; ++j) {
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(set.pixels[i], set.kernels[j],
                                                             decltype(from_zero)::value ? float16_t(0.0f) : acc[i][j], 0, 0, 0);
         }
@@ -257,7 +260,7 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const Conv
 #pragma unroll
         for (int i = 0; i < BLOCKS; ++i) {
 #pragma unroll
-          for (int j = 0; j < 2; ++j) {
+          for (int j = 0; j < J; ++j) {
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(set.pixels[i][e], set.kernels[j][e],
                                                             (decltype(from_zero)::value && e == 0) ? float16_t(0.0f) : acc[i][j], 0, 0, 0);
           }
@@ -309,7 +312,7 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const Conv
         // one read after every matrix instruction: nine reads in a row wait for room in the LDS queue, and the
         // wavefront issues nothing else meanwhile
 #pragma unroll
-        for (int i = 0; i < BLOCKS + 2; ++i) {
+        for (int i = 0; i < (BLOCKS + J < BLOCKS * J ? BLOCKS + J : BLOCKS * J); ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);  // one matrix instruction (fp32: the four of a block),
           __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);  // the address of
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read,
@@ -319,7 +322,7 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const Conv
           }
         }
 #pragma unroll
-        for (int i = BLOCKS + 2; i < 2 * BLOCKS; ++i) {
+        for (int i = BLOCKS + J; i < BLOCKS * J; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
           if (tap == 0) {
             __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
@@ -335,7 +338,7 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const Conv
       deposit(lds + ((chunk + 1) & 1) * p.slab_elements);
       products(set[(TAPS - 1) % 2], std::integral_constant<bool, FIRST && TAPS == 1>{});
 #pragma unroll
-      for (int i = 0; i < 2 * BLOCKS; ++i) {
+      for (int i = 0; i < BLOCKS * J; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);  // one matrix instruction (fp32: four),
         __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);  // two vector ALU instructions,
         __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);  // two LDS writes
@@ -371,14 +374,14 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const Conv
 #pragma unroll
     for (int i = 0; i < BLOCKS; ++i) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < J; ++j) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           half4_t four;
 #pragma unroll
           for (int e = 0; e < 4; ++e) { four[e] = static_cast<_Float16>(acc[i][j][4 * g + e]); }
           const int pixel = (wave_m * BLOCKS + i) * 32 + 8 * g + 4 * (lane / 32);
-          const int n = wave_n * 64 + j * 32 + lane % 32;
+          const int n = wave_n * 32 * J + j * 32 + lane % 32;
           *reinterpret_cast<half4_t*>(lds + n * RP + pixel) = four;
         }
       }
@@ -386,9 +389,9 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const Conv
     __syncthreads();
     constexpr int ROW_VECTORS = BLOCKS * 32 / 8;  // 16-byte pieces of a kernel's row in this wavefront's part
 #pragma unroll 14
-    for (int t = 0; t < ROW_VECTORS; ++t) {
+    for (int t = 0; t < ROW_VECTORS * J / 2; ++t) {  // 32 J rows of ROW_VECTORS pieces, 64 at a time
       const int q = lane + 64 * t;
-      const int n = wave_n * 64 + q / ROW_VECTORS, pixel = wave_m * BLOCKS * 32 + (q % ROW_VECTORS) * 8;
+      const int n = wave_n * 32 * J + q / ROW_VECTORS, pixel = wave_m * BLOCKS * 32 + (q % ROW_VECTORS) * 8;
       if (n0 + n < p.kernels && pixel < valid_pixels) {
         const Dwords4 value = *reinterpret_cast<const Dwords4*>(lds + n * RP + pixel);
         *reinterpret_cast<Dwords4*>(result + (n0 + n) * pixels + pixel) = value;
@@ -400,7 +403,7 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const Conv
     constexpr int RP = kConvSlabPixels + 4;       // floats from a kernel to the next
     constexpr int ROW_VECTORS = BLOCKS * 32 / 4;  // 16-byte pieces of a kernel's row in this wavefront's part
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < J; ++j) {
 #pragma unroll
       for (int i = 0; i < BLOCKS; ++i) {
 #pragma unroll
@@ -416,7 +419,7 @@ __global__ __launch_bounds__(kConvSlabThreads, 1) void ConvSlabKernel(const Conv
       for (int t = 0; t < ROW_VECTORS / 2; ++t) {
         const int q = lane + 64 * t;
         const int row = q / ROW_VECTORS, pixel = wave_m * BLOCKS * 32 + (q % ROW_VECTORS) * 4;
-        const int n = n0 + wave_n * 64 + j * 32 + row;
+        const int n = n0 + wave_n * 32 * J + j * 32 + row;
         if (n < p.kernels && pixel < valid_pixels) {
           const Vector value = *reinterpret_cast<const Vector*>(lds + (wave_n * 32 + row) * RP + pixel);
           *reinterpret_cast<Vector*>(result + n * pixels + pixel) = value;

@@ -726,13 +726,13 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
 
 // Measured on 8 images against the GEMM that gathers its patches (fp16 / fp32, slab kernel against that, in us):
 // 128 channels of 56 x 56, 128 kernels of 3 x 3: 28 / 34 and 250 / 98 (56 work-groups); 64 x 224 x 224, 64 kernels, 2
-// images: 27 / 39 and 133 / 96 (half of a tile's kernels); 256 x 56 x 56, 256 kernels of 1 x 1: 31 / 29 and 90 / 43;
+// images: 22 / 40 and 74 / 96 (on the tile of 64 kernels; on the one of 128: 27 and 133); 256 x 56 x 56, 256 kernels of 1 x 1: 31 / 29 and 90 / 43;
 // 512 x 16 x 16, 512 kernels: 83 / 74 (fp16; 256 of a tile's 448 pixels); 64 x 112 x 112, 128 kernels: 23 / 46 and
 // 134 / 160. fp32, where the gathering GEMM runs at 0.6 of the peak, wants a launch that fills the device; fp16, where
 // that GEMM is bound by its address arithmetic, tiles that are mostly full and a launch that is not tiny; one tap leaves a
 // barrier per k-step.
 bool UseConvSlab(const Precision precision, const size_t taps, const size_t kernels, const size_t work_groups,
-                 const size_t tile_pixels, const size_t compute_units) {
+                 const size_t tile_pixels, const size_t tile_kernels, const size_t compute_units) {
   size_t forced = 0;
   {
     std::lock_guard<std::mutex> lock(override_mutex);
@@ -740,17 +740,19 @@ bool UseConvSlab(const Precision precision, const size_t taps, const size_t kern
     if (found != conv_slab_overrides.end()) { forced = found->second; }
   }
   if (forced == 1) { return true; }
-  if (forced == 2 || taps < 2 || work_groups == 0 || compute_units == 0) { return false; }
+  if (forced == 2 || taps < 2 || work_groups == 0 || compute_units == 0 || tile_kernels == 0) { return false; }
   const auto fill = static_cast<double>(tile_pixels) / 448.0;
   const auto rounds = CeilDivide(work_groups, compute_units);
-  const auto kernel_tiles = CeilDivide(kernels, 128);
+  const auto kernel_tiles = CeilDivide(kernels, tile_kernels);
   const auto use = static_cast<double>(work_groups) / static_cast<double>(rounds * compute_units) * fill *
-                   static_cast<double>(kernels) / static_cast<double>(kernel_tiles * 128);
-  // (fp16 on few work-groups: 64 x 56 x 56, 64 kernels, 2 images - 14 work-groups, half of a tile's kernels - 18 against
-  // 13 us; 256 x 56 x 56, 64 kernels, 4 images 45 against 34 us; from 0.2 on the slab kernel is ahead: 2 images of
-  // 64 x 112 x 112 with 128 kernels 19 against 21 us, 4 images 21 against 28 us)
-  if (precision == Precision::kHalf) { return fill >= 0.75 && use >= 0.15; }
-  return use >= 0.7;
+                   static_cast<double>(kernels) / static_cast<double>(kernel_tiles * tile_kernels);
+  // (fp16 on few work-groups, tile of 128 kernels: 1 image of 64 x 112 x 112 with 128 kernels - use 0.11 - 19 against
+  // 18 us, 2 images 19 against 21 us, 4 images 21 against 28 us. Tile of 64 kernels, 64 x 56 x 56 with 64 kernels: 2 images
+  // - use 0.055 - 13.8 against 12.5 us, 4 images 13.8 against 14.5 us, 8 images 14 against 17 us, 32 images 17 against 39 us.
+  // fp32, tile of 64 kernels, same shape: 8 images - use 0.22 - 71 against 36 us, 16 images 72 against 58 us, 24 images
+  // - 0.66 - 73 against 74 us; 6 images of 64 x 112 x 112 - 0.66 - 73 against 75 us; 2 images of 64 x 224 x 224 74 against 96 us)
+  if (precision == Precision::kHalf) { return fill >= 0.75 && use >= (tile_kernels <= 64 ? 0.1 : 0.15); }
+  return use >= 0.65;
 }
 
 StatusCode OverrideRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,

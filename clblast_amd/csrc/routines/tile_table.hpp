@@ -46,10 +46,10 @@ KernelChoice SelectKernel(const Precision precision, const bool a_kcontig, const
 size_t ForcedTileVariant(const Precision precision);
 
 // CONVGEMM: whether the kernel that stages image slabs in LDS (one work-group per 448 output pixels x 128 kernels) is
-// taken for a shape that it can run. `work_groups` and `tile_pixels` as the device layer reports them, `compute_units`
-// of the device. OverrideParameters("Xconvgemm", {"SLAB": 1}) takes it whenever it can run, {"SLAB": 2} never, 0 is this rule.
+// taken for a shape that it can run. `work_groups`, `tile_pixels` and `tile_kernels` as the device layer reports them,
+// `compute_units` of the device. OverrideParameters("Xconvgemm", {"SLAB": 1}) takes it whenever it can run, {"SLAB": 2} never, 0 is this rule.
 bool UseConvSlab(const Precision precision, const size_t taps, const size_t kernels, const size_t work_groups,
-                 const size_t tile_pixels, const size_t compute_units);
+                 const size_t tile_pixels, const size_t tile_kernels, const size_t compute_units);
 
 // Parameter override store behind clblast::OverrideParameters / RetrieveParameters / ClearCache.
 StatusCode OverrideRoutineParameters(const int device, const std::string& kernel_name, const Precision precision,

@@ -83,14 +83,15 @@ void Xconvgemm<T>::DoConvgemm(const KernelMode kernel_mode, const size_t channel
   // tile table's rule finds the launch worthwhile (UseConvSlab): the images as they are, the padding as zeros in LDS,
   // the kernel matrix through a small copy in the order the kernel reads it.
   if (precision == 16 || precision == 32) {
-    int work_groups = 0, tile_pixels = 0, compute_units = 0;
+    int work_groups = 0, tile_pixels = 0, tile_kernels = 0, compute_units = 0;
     const auto scratch_bytes = clbh_conv_slab_scratch_bytes(precision, &shape, static_cast<int>(num_kernels),
-                                                            static_cast<int>(batch_count), &work_groups, &tile_pixels);
+                                                            static_cast<int>(batch_count), &work_groups, &tile_pixels, &tile_kernels);
     const bool aligned = (reinterpret_cast<unsigned long long>(im_buffer()) + sizeof(T) * im_offset) % 16 == 0 &&
                          (reinterpret_cast<unsigned long long>(result_buffer()) + sizeof(T) * result_offset) % 16 == 0;
     const bool worthwhile = scratch_bytes > 0 && aligned && clbh_compute_units(&compute_units) == 0 &&
                             UseConvSlab(PrecisionValue<T>(), kernel_h * kernel_w, num_kernels, static_cast<size_t>(work_groups),
-                                        static_cast<size_t>(tile_pixels), static_cast<size_t>(compute_units));
+                                        static_cast<size_t>(tile_pixels), static_cast<size_t>(tile_kernels),
+                                        static_cast<size_t>(compute_units));
     if (worthwhile) {
       const StreamScratch ordered(scratch_bytes, this->stream(), "kernel matrix in k-step order");
       CheckDevice(clbh_conv_slab(precision, &shape, static_cast<int>(num_kernels), static_cast<int>(batch_count), im_buffer(),

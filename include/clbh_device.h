@@ -248,12 +248,13 @@ CLBH_API int clbh_conv_gather_possible(int precision, const clbh_im2col_shape* s
 // least half of a 448-pixel tile, and as many taps as fit LDS next to two slabs (4 KiB per tap, twice); images +
 // images_offset, result + result_offset and scratch 16-byte aligned. clbh_conv_slab_scratch_bytes returns 0 for a
 // shape it does not take, else the size of the scratch that receives the kernel matrix in the order the kernel reads it,
-// and then also (where the pointers are not NULL) the number of work-groups of the launch and the output pixels of a
-// full tile of 448 - what a caller needs to judge how well the launch fills the device.
+// and then also (where the pointers are not NULL) the number of work-groups of the launch, the output pixels of a
+// full tile of 448 and the kernels of a tile (128, or 64 for calls with at most 64 kernels) - what a caller needs to judge
+// how well the launch fills the device.
 // shape->flip mirrors the taps. Images: batch_count x channels x height x width; weights: kernels x (channels *
 // kernel_h * kernel_w); result: batch_count x kernels x output_h x output_w.
 CLBH_API size_t clbh_conv_slab_scratch_bytes(int precision, const clbh_im2col_shape* shape, int kernels, int batch_count,
-                                             int* work_groups, int* tile_pixels);
+                                             int* work_groups, int* tile_pixels, int* tile_kernels);
 CLBH_API int clbh_conv_slab(int precision, const clbh_im2col_shape* shape, int kernels, int batch_count, const void* images,
                             long long images_offset, const void* weights, long long weights_offset, void* result,
                             long long result_offset, void* scratch, hipStream_t stream);

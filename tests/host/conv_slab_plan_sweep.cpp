@@ -48,7 +48,9 @@ int main() {
           plan.row_tiles * plan.rows < g.output_h || (plan.row_tiles - 1) * plan.rows >= g.output_h) {
         Violation("rows per tile", precision, g, kernels, batch);
       }
-      if (plan.kernel_tiles * clbh::kConvSlabKernels < kernels || (plan.kernel_tiles - 1) * clbh::kConvSlabKernels >= kernels) {
+      const int tile_kernels = 64 * plan.kernel_blocks;
+      if ((plan.kernel_blocks != 1 && plan.kernel_blocks != 2) || (plan.kernel_blocks == 1) != (kernels <= 64) ||
+          plan.kernel_tiles * tile_kernels < kernels || (plan.kernel_tiles - 1) * tile_kernels >= kernels) {
         Violation("tiles of kernels", precision, g, kernels, batch);
       }
       // the slab: rows the tile's patches touch, the image row inside its padding, a width of 2 mod 4 pixels
@@ -65,8 +67,8 @@ int main() {
       // the furthest staged pixel: the last column of the image in the last slab row
       const long long last_staged = static_cast<long long>(plan.slab_rows - 1) * plan.slab_width + pad_w + width - 1;
       if ((last_staged + 1) * pitch > plan.spare_at) { Violation("a staged piece lies beyond the slab", precision, g, kernels, batch); }
-      // LDS: two slabs, two chunks of kernels (4 KiB per tap), or the epilogue's tile
-      const long long walk_bytes = 2ll * plan.slab_elements * element + 2 * taps * 4096;
+      // LDS: two slabs, two chunks of kernels (32 bytes per kernel and tap), or the epilogue's tile
+      const long long walk_bytes = 2ll * plan.slab_elements * element + 2 * taps * tile_kernels * 32;
       const long long result_bytes = precision == 16 ? clbh::kConvSlabResultBytes : clbh::kConvSlabResultBytesF32;
       if (static_cast<long long>(plan.lds_bytes) > clbh::kConvSlabLdsBytes || static_cast<long long>(plan.lds_bytes) < walk_bytes ||
           static_cast<long long>(plan.lds_bytes) < result_bytes) {

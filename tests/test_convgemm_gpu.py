@@ -89,7 +89,8 @@ def test_convgemm_sweep(gpu, bits):
             problem.check(after)
 
 
-SLAB_CASES = [  # shapes for the kernel that stages image slabs in LDS (fp16 and fp32): unit strides, 16 | channels, 8 | widths
+SLAB_CASES = [  # shapes for the kernel that stages image slabs in LDS (fp16 and fp32): unit strides, 16 | channels, 8 | widths;
+               # up to 64 kernels on the tile of 64 kernels, more on the one of 128
     (16, 32, 32, 3, 3, 1, 1, 1, 1, 1, 1, 32, 4),    # three row tiles of 11 rows, the last with 10
     (32, 20, 24, 3, 3, 1, 1, 1, 1, 1, 1, 130, 3),   # two chunks of channels, two tile columns of kernels (the second: 2)
     (16, 9, 40, 5, 1, 2, 0, 1, 1, 1, 1, 20, 2),     # a 5 x 1 window, padding along the height only, one tile per image
@@ -118,8 +119,8 @@ def slab_scratch_bytes(case, bits=16):
                   oracle.conv_output_extent(width, kernel_w, pad_w, stride_w, dilation_w), 0)
     function = _lib.load().clbh_conv_slab_scratch_bytes
     function.restype = ctypes.c_size_t
-    function.argtypes = [ctypes.c_int, ctypes.POINTER(Shape), ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
-    return function(bits, ctypes.byref(shape), kernels, batch, None, None)
+    function.argtypes = [ctypes.c_int, ctypes.POINTER(Shape), ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    return function(bits, ctypes.byref(shape), kernels, batch, None, None, None)
 
 
 @pytest.mark.parametrize("bits", (16, 32))
