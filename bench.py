@@ -46,8 +46,8 @@ MEASURED_TRAFFIC = {
     "cfg5e": (7.371e7, "profiles/sgemm_4099x17x4096_colTN.md", "clbh::GemmSkinnyRowsKernel<4, 5, 5, 2, true, true, 2>"),
     "sbat64": (2.036e8, "profiles/sgemm_strided_batched_4096x64.md", "clbh::GemmStreamKernel<float, clbh::MfmaConfig<float, 1, 4, 4, 1, 16, 4"),
     "hbat_short_k": (2.939e8, "profiles/hgemm_strided_batched_8x4096x4096x64.md", "clbh::HgemmDirectKernel<clbh::HdirectConfig<2, 2, 2, 2, 3"),
-    "conv_h": (4.75e7, "profiles/hconvgemm_64x112x112_k128_b8.md", "ConvSlabKernelIDF16_Li3ELi9E"),
-    "conv_s": (9.44e7, "profiles/sconvgemm_64x112x112_k128_b8.md", "clbh::ConvSlabKernel<float, 7, 9>"),
+    "conv_h": (4.75e7, "profiles/hconvgemm_64x112x112_k128_b8.md", "ConvSlabKernelIDF16_Li3ELi9ELi2E"),
+    "conv_s": (9.44e7, "profiles/sconvgemm_64x112x112_k128_b8.md", "clbh::ConvSlabKernel<float, 7, 9, 2>"),
     "cgemm_batched": (4.028e8, "profiles/cgemm_strided_batched_4096x64_rowNC.md", "clbh::GemmComplexSmallKernel<float, 2, true, true>"),
 }
 
