@@ -87,7 +87,9 @@ extern "C" {
 size_t clbh_conv_slab_scratch_bytes(int precision, const clbh_im2col_shape* shape, int kernels, int batch_count, int* work_groups,
                                     int* tile_pixels, int* tile_kernels) {
   if (shape == nullptr) { return 0; }
-  const auto plan = clbh::PlanConvSlab(precision, *shape, kernels, batch_count);
+  int compute_units = 0;
+  if (clbh_compute_units(&compute_units) != 0) { compute_units = 0; }
+  const auto plan = clbh::PlanConvSlab(precision, *shape, kernels, batch_count, compute_units);
   if (!plan.possible) { return 0; }
   if (work_groups != nullptr) { *work_groups = batch_count * plan.row_tiles * plan.kernel_tiles; }
   if (tile_kernels != nullptr) { *tile_kernels = 64 * plan.kernel_blocks; }
@@ -102,7 +104,9 @@ int clbh_conv_slab(int precision, const clbh_im2col_shape* shape, int kernels, i
       images_offset < 0 || weights_offset < 0 || result_offset < 0) {
     return hipErrorInvalidValue;
   }
-  const auto plan = clbh::PlanConvSlab(precision, *shape, kernels, batch_count);
+  int compute_units = 0;
+  if (clbh_compute_units(&compute_units) != 0) { compute_units = 0; }
+  const auto plan = clbh::PlanConvSlab(precision, *shape, kernels, batch_count, compute_units);
   if (!plan.possible) { return hipErrorInvalidValue; }
   if (precision == 16) {
     return clbh::LaunchConvSlabTyped<_Float16>(*shape, plan, kernels, batch_count, images, images_offset, weights, weights_offset,

@@ -123,7 +123,8 @@ struct ConvSlabPlan {
 
 // Unit strides, no dilation, the kernel window inside the padded image, 16 channels per chunk, image rows and result
 // rows in 16-byte pieces, a tile of whole output rows that fills at least half of the 448 pixels, two slabs in LDS.
-inline ConvSlabPlan PlanConvSlab(const int precision, const clbh_im2col_shape& g, const int kernels, const int batch_count) {
+inline ConvSlabPlan PlanConvSlab(const int precision, const clbh_im2col_shape& g, const int kernels, const int batch_count,
+                                 const int compute_units) {
   if (precision != 16 && precision != 32) { return ConvSlabPlan{}; }
   const int element = precision / 8, chunk = 32 / element, piece = 16 / element, pitch = kConvSlabPixelBytes / element;
   ConvSlabPlan plan = {};
@@ -143,7 +144,9 @@ inline ConvSlabPlan PlanConvSlab(const int precision, const clbh_im2col_shape& g
   plan.row_tiles = (g.output_h + most_rows - 1) / most_rows;
   plan.rows = (g.output_h + plan.row_tiles - 1) / plan.row_tiles;
   if (2 * plan.rows * g.output_w < kConvSlabPixels) { return plan; }
-  plan.kernel_blocks = (kernels <= kConvSlabKernels / 2) ? 1 : 2;
+  // tiles of 64 kernels where 128 would be half empty, and where twice as many work-groups still fit one round of CUs
+  const long long large_tiles = static_cast<long long>(batch_count) * plan.row_tiles * ((kernels + kConvSlabKernels - 1) / kConvSlabKernels);
+  plan.kernel_blocks = (kernels <= kConvSlabKernels / 2 || 2 * large_tiles <= compute_units) ? 1 : 2;
   const int tile_kernels = 64 * plan.kernel_blocks;
   plan.kernel_tiles = (kernels + tile_kernels - 1) / tile_kernels;
   if (static_cast<long long>(batch_count) * plan.row_tiles * plan.kernel_tiles > INT_MAX) { return plan; }

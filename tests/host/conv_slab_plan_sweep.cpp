@@ -35,7 +35,7 @@ int main() {
       g.output_w = width + 2 * pad_w - kernel_w + 1;
       if (height + 2 * pad_h < kernel_h || g.output_w < 1) { continue; }
       ++cases;
-      const auto plan = clbh::PlanConvSlab(precision, g, kernels, batch);
+      const auto plan = clbh::PlanConvSlab(precision, g, kernels, batch, 256);
       if (!plan.possible) { continue; }
       ++taken;
       if (precision == 64 || stride != 1 || channels % chunk != 0 || width % piece != 0 || g.output_w % piece != 0) {
@@ -49,7 +49,8 @@ int main() {
         Violation("rows per tile", precision, g, kernels, batch);
       }
       const int tile_kernels = 64 * plan.kernel_blocks;
-      if ((plan.kernel_blocks != 1 && plan.kernel_blocks != 2) || (plan.kernel_blocks == 1) != (kernels <= 64) ||
+      if ((plan.kernel_blocks != 1 && plan.kernel_blocks != 2) || (kernels <= 64 && plan.kernel_blocks != 1) ||
+          (plan.kernel_blocks == 1 && kernels > 64 && static_cast<long long>(batch) * plan.row_tiles * plan.kernel_tiles > 256) ||
           plan.kernel_tiles * tile_kernels < kernels || (plan.kernel_tiles - 1) * tile_kernels >= kernels) {
         Violation("tiles of kernels", precision, g, kernels, batch);
       }
